@@ -1,0 +1,111 @@
+/* C ABI of the MI355X (gfx950) MX low-precision 3-D U-Net forward kernels.
+ *
+ * Drop-in for the forward subset of the reference's internal kernel interface src/nn_lp.h: same entry-point names,
+ * argument order, dtype codes, by-value descriptors and tensor / scale layouts. Every declaration cites the reference
+ * declaration it replaces. All pointers named x / y / w / b / gamma ... are DEVICE pointers unless stated otherwise;
+ * all work is issued on the HIP null stream, asynchronously, in stream order (as the reference on the default stream).
+ *
+ * dtype codes (src/lp_f4fwd.cuh:1224): 0 fp32 planes [n][C][S], 1 bf16 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4.
+ * MX tensor of N x C x S (src/lp_common.cuh:100-106, :132-134): bw = 8 / 16 / 32 for C <= 8 / <= 16 / else,
+ * nb = ceil(C / bw); data[n][blk][voxel][bw] e4m3 bytes (fp4: bw/2 bytes, channel k = nibble k&1 of byte k/2) followed by
+ * the scale plane sc[n][blk][voxel] of E8M0 bytes.
+ */
+#ifndef MI_LP_H
+#define MI_LP_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- descriptors, passed by value (layouts identical to the reference's) ---- */
+typedef struct { int n, c, d, h, w; } shape5;                                   /* src/nn.h:21 */
+typedef struct { const float *gamma, *beta, *mean, *rstd; int G; int zs, zo, ns, zhw; } gnp_t;   /* src/nn_lp.h:15; G == 0: no transform */
+typedef struct {                                                                 /* src/nn_lp.h:32 */
+    const void *x2; int c_split; void *y2; int o_split; int accum; gnp_t gp2; int16_t up, yD; unsigned sr; unsigned wkey;
+    int zlo, zhi; int stored_stats; unsigned osr; int16_t zi0, Di, o_pad, zw0, zw1, yzo;
+} split_t;
+/* Fields honoured by this build: x2, c_split, gp2, up, wkey, stored_stats, zlo, zhi. Training / slab fields (y2, o_split, accum,
+   sr, osr, yD, zi0, Di, o_pad, zw0, zw1, yzo) must be zero: a call that sets one prints a message and aborts, as the reference
+   does for combinations it does not support (src/lp_f8fwd.cu:28). Slab-local GroupNorm (gnp_t.ns > 0) likewise. */
+
+/* GroupNorm sum slots (src/gnacc.cuh:8-9): `osum` / `sums` buffers are arrays of 3 x uint64 fixed-point slots (24 bytes each:
+   fraction in units of 2^-64, signed integer part, count of non-finite contributions), two per (sample, group): sum, sum of squares */
+#define MI_GN_SLOT_BYTES 24
+
+/* ---- convolutions ---- */
+/* 3x3x3, stride 1, pad 1; MX-fp8 (e4m3) compute. Replaces src/nn_lp.h:53 (lp_conv_fwd_f8, src/lp_f8fwd.cu:26-52). Returns 0. */
+int lp_conv_fwd_f8(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp);
+/* the same with MX-fp4 (e2m1) compute. Replaces src/nn_lp.h:54 (src/lp_f4fwd.cu:30-51). */
+int lp_conv_fwd_f4(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp);
+/* 3x3x3, stride 2, pad 1 (ys = output shape). Replaces src/nn_lp.h:104 (src/lp_s2.cu:647-754). Returns 0, or 3 when fp4 compute ran. */
+int lp_conv_fwd_s2_f8(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, shape5 ys, gnp_t gp);
+/* prepared-weight memo (src/nn_lp.h:56-57): a conv called with sp.wkey != 0 reuses its quantised weights until the next step / clear */
+void lp_wmemo_step(unsigned step);
+void lp_wmemo_clear(void);
+gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean, const float *rstd, int G);   /* src/nn_lp.h:19 */
+int lp_gn_slab_any(void);                                                                         /* src/nn_lp.h:20: always 0 here */
+
+/* ---- MX tensor conversions (src/nn_lp.h:111-118, :126; src/lp_mx_cvt.cu:6-79, :429-447) ---- */
+size_t lp_mx8_bytes(int N, int C, size_t S);
+size_t lp_mx4_bytes(int N, int C, size_t S);
+void lp_f32_to_mx8(const float *x, int N, int C, size_t S, void *y);
+void lp_f32_to_mx4(const float *x, int N, int C, size_t S, void *y);
+void lp_h16_to_mx8(const void *x, int dt, int N, int C, size_t S, void *y);   /* dt 1 bf16, 2 fp16 */
+void lp_h16_to_mx4(const void *x, int dt, int N, int C, size_t S, void *y);
+void lp_mx8_to_f32(const void *x, int N, int C, size_t S, float *y);
+void lp_mx4_to_f32(const void *x, int N, int C, size_t S, float *y);
+/* network input rows from a uint8 CT window (src/nn_lp.h:164-165; src/lp_mx_cvt.cu:29-55) */
+void lp_pred_input_mx(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits);
+void lp_pred_input_mx8(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd);
+
+/* ---- MX elementwise ops (src/nn_lp.h:134-137, :175-176) ---- */
+void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, const float *gamma, const float *beta, const float *mean, const float *rstd, void *y, int ydt);
+void lp_add_mx(void *y, const void *x, shape5 s, int dt, unsigned sr);   /* sr must be 0 (round to nearest) */
+void lp_up2_fwd_mx(const void *x, int xdt, shape5 xs, void *y, int ydt, gnp_t gp);
+void lp_up2_fwd_mx_blocks(const void *x, int xdt, shape5 xs, int b0, int nbk, void *y, int ydt);
+int lp_gn_sums_mx(const void *x, int xdt, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1);
+int lp_gn_sums_mx_n(const void *x, int xdt, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1, int n0, int cnt);
+
+/* ---- 1x1x1 head (src/nn_lp.h:138-141; src/lp_mx_conv1.cu:370-445) ---- */
+void lp_conv1_fwd_mx(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, float *y, gnp_t gp);
+void lp_conv1_fwd_mx_h16(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, void *y, gnp_t gp);
+void lp_conv1_fwd_mx_h16_r(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, void *y, gnp_t gp, size_t vb, size_t nv);
+int lp_conv1_fwd_mx_r(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, float *y, gnp_t gp, size_t vb, size_t nv, size_t ly);
+
+/* ---- error latch (src/nn_lp.h:172; src/lp_common.cuh:35-38): message of the first HIP error since the last call, else NULL ---- */
+const char *lp_check(void);
+
+/* ---- what the reference's lp_* units pull from its op layer, provided here so the library stands alone ----
+   (the reference side: nn_malloc / nn_free / nn_zero / nn_h2d / nn_d2h / nn_sync, src/nn.h:34-48; gn_finalize_k, src/nn_elem.cu:5-11;
+   nn_ws, src/nn_core.cu:751). In an integration these stay the reference's own. */
+int mi_init(int device);                       /* selects the device, 0 on success; fails (non-zero) when no gfx950 device is present */
+int mi_device_count(void);
+void *mi_malloc(size_t bytes);                 /* device memory; aborts with a message when it cannot be had */
+void mi_free(void *p);
+void mi_zero(void *p, size_t bytes);
+void mi_h2d(void *dst, const void *src, size_t bytes);
+void mi_d2h(void *dst, const void *src, size_t bytes);
+void mi_d2d(void *dst, const void *src, size_t bytes);
+void mi_sync(void);
+void mi_ws_release(void);                      /* frees the per-device scratch (prepared weights, staged operands) */
+/* GroupNorm finalize from sum slots: mean, rstd of NG = N * G groups of `len` elements each (src/nn_elem.cu:5-11) */
+void mi_gn_finalize(const double *sums, int NG, size_t len, float eps, float *mean, float *rstd);
+void mi_gn_sums_zero(double *sums, int nslots);          /* clear slots with a kernel (safe inside graph capture) */
+void mi_gn_sums_get(const double *sums, int nslots, double *out);   /* slots -> doubles (device to device), src/gnacc.cuh:21-25 */
+/* timing on the stream the kernels run on */
+void *mi_event_create(void);
+void mi_event_record(void *ev);
+float mi_event_elapsed_ms(void *ev0, void *ev1);   /* synchronises on ev1 */
+void mi_event_destroy(void *ev);
+/* extension with no counterpart in the reference: the same conv with a fused epilogue affine + activation before the MX
+   re-quantisation (frozen GroupNorm statistics folded into per-channel a, b): v = act(a[co] * (conv + bias) + b[co]);
+   act 0 none, 1 SiLU, 2 GELU (erf), 3 ReLU. bits 8 / 4 selects the compute format. */
+int mi_conv_fwd_fused(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
+                      const float *ep_a, const float *ep_b, int act, gnp_t gp, double *osum, int Go, split_t sp);
+/* name of the conv kernel variant the last conv call on this thread launched (diagnostics / tests), "" if none */
+const char *mi_last_kernel(void);
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,554 @@
+/* CPU oracle: see mx_oracle.h. Test infrastructure, never linked into the shipped GPU library.
+   Build: gcc -O3 -march=native -ffp-contract=off -fopenmp -shared -fPIC (no fast-math: the quantiser is bit-exact). */
+#include "mx_oracle.h"
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+int orc_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ---------- block geometry (src/lp_common.cuh:132-134) ---------- */
+int orc_mx_bw(int C) { return C <= 8 ? 8 : C <= 16 ? 16 : 32; }
+int orc_mx_nb(int C) { int bw = orc_mx_bw(C); return (C + bw - 1) / bw; }
+static int rowbytes(int bw, int bits) { return bw * bits / 8; }
+size_t orc_mx_bytes(int bits, int N, int C, size_t S) { return (size_t)N * orc_mx_nb(C) * S * (rowbytes(orc_mx_bw(C), bits) + 1); }
+
+/* ---------- scale selection (src/lp_common.cuh:492-501): the product with the rounded reciprocal, exponent rounded up ---------- */
+int orc_mx_exp(float amax, float inv_qmax) {
+    const uint32_t u = f2u(amax * inv_qmax) & 0x7fffffffu;
+    if (u >= 0x7f800000u) return 128;                       /* NaN, inf, or the product overflowed */
+    int e = (int)(u >> 23) - 127 + ((u & 0x7fffffu) ? 1 : 0);
+    return e < -126 ? -126 : e > 126 ? 126 : e;
+}
+float orc_exp2i(int e) { return u2f((uint32_t)(127 + e) << 23); }   /* e = -128 gives the bits of -inf, as the reference's shift does */
+float orc_mx_scale(unsigned sbyte) { return u2f((uint32_t)(sbyte & 255u) << 23); }   /* 0xFF -> +inf (src/lp_common.cuh:186) */
+static const float INVQ8 = 1.f / 448.f, INVQ4 = 1.f / 6.f;
+
+/* ---------- element decode (src/mx_sw.cuh:78-87) ---------- */
+float orc_dec_e4m3(unsigned b) {
+    const unsigned e = (b >> 3) & 15u, m = b & 7u;
+    if ((b & 0x7fu) == 0x7fu) return u2f(0x7fc00000u | ((b & 0x80u) << 24));
+    const float v = e ? ldexpf((float)(8u + m), (int)e - 10) : ldexpf((float)m, -9);
+    return (b & 0x80u) ? -v : v;
+}
+static const float E2M1_GRID[8] = {0.f, 0.5f, 1.f, 1.5f, 2.f, 3.f, 4.f, 6.f};
+float orc_dec_e2m1(unsigned n) { const float v = E2M1_GRID[n & 7u]; return (n & 8u) ? -v : v; }
+
+/* ---------- element encode: round to nearest, ties to even code, saturating (semantics of src/mx_sw.cuh:1-12) ----------
+   e4m3: arithmetic formulation. The quantum of the binade holding |x| is 2^(max(E, -6) - 3); |x| / quantum is an exact
+   power-of-two scaling, rintf rounds it to nearest-even (default rounding mode), and the rounded multiple maps to a code. */
+unsigned orc_enc_e4m3(float x) {
+    const uint32_t u = f2u(x), s = (u >> 24) & 0x80u, a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return 0x7fu;                      /* NaN of either sign */
+    const float ax = u2f(a);
+    if (ax >= 448.f) return s | 0x7eu;                      /* 448..464 would round to 448 anyway, the rest saturates */
+    if (ax < 0x1p-11f) return s;                            /* below half the subnormal step 2^-9 (2^-10 itself ties to even 0) */
+    int ex; (void)frexpf(ax, &ex);                          /* ax = f 2^ex, f in [0.5, 1): binade exponent ex - 1 */
+    int E = ex - 1; if (E < -6) E = -6;
+    const float k = rintf(ldexpf(ax, 3 - E));               /* multiple of the quantum, 0..16 */
+    if (E == -6 && k < 8.f) return s | (unsigned)k;         /* subnormal codes 0..7 */
+    unsigned ki = (unsigned)k;
+    if (ki == 16u) { ki = 8u; E++; }                        /* rounded up into the next binade */
+    return s | (((unsigned)(E + 7) << 3) | (ki - 8u));
+}
+/* e2m1: threshold formulation on the midpoints of {0, .5, 1, 1.5, 2, 3, 4, 6}; a tie goes to the even code */
+unsigned orc_enc_e2m1(float x) {
+    const uint32_t u = f2u(x), s = (u >> 28) & 8u, a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return 7u;                         /* NaN -> +6 */
+    const float ax = u2f(a);
+    unsigned c;
+    if (ax <= 0.25f) c = 0; else if (ax < 0.75f) c = 1; else if (ax <= 1.25f) c = 2; else if (ax < 1.75f) c = 3;
+    else if (ax <= 2.5f) c = 4; else if (ax < 3.5f) c = 5; else if (ax <= 5.f) c = 6; else c = 7;
+    return s | c;
+}
+/* the pins: nearest grid point by exhaustive scan of the code values; exact-midpoint ties to the even code; no arithmetic on x
+   beyond exact differences in double */
+unsigned orc_ref_e4m3(float x) {
+    const uint32_t u = f2u(x), s = (u >> 24) & 0x80u;
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fu;
+    const double a = fabs((double)x);
+    if (a >= 448.0) return s | 0x7eu;                       /* saturation: beyond the largest grid value (also keeps the differences below exact) */
+    unsigned best = 0; double bd = INFINITY;
+    for (unsigned c = 0; c <= 0x7eu; c++) {
+        const double d = fabs((double)orc_dec_e4m3(c) - a);
+        if (d < bd || (d == bd && !(c & 1u))) { bd = d; best = c; }
+    }
+    return s | best;
+}
+unsigned orc_ref_e2m1(float x) {
+    const uint32_t u = f2u(x), s = (u >> 28) & 8u;
+    if ((u & 0x7fffffffu) > 0x7f800000u) return 7u;
+    const double a = fabs((double)x);
+    if (a >= 6.0) return s | 7u;
+    unsigned best = 0; double bd = INFINITY;
+    for (unsigned c = 0; c < 8u; c++) {
+        const double d = fabs((double)E2M1_GRID[c] - a);
+        if (d < bd || (d == bd && !(c & 1u))) { bd = d; best = c; }
+    }
+    return s | best;
+}
+uint64_t orc_enc_sweep(uint32_t first, uint64_t count, uint32_t stride, uint32_t *bad) {
+    uint64_t nbad = 0; uint32_t firstbad = 0; int have = 0;
+    if (!stride) stride = 1;
+    const uint64_t n = (count + stride - 1) / stride;
+#pragma omp parallel for schedule(static) reduction(+ : nbad)
+    for (uint64_t i = 0; i < n; i++) {
+        const uint32_t u = first + (uint32_t)(i * stride);
+        const float x = u2f(u);
+        if (orc_enc_e4m3(x) != orc_ref_e4m3(x) || orc_enc_e2m1(x) != orc_ref_e2m1(x)) {
+            nbad++;
+#pragma omp critical
+            { if (!have || u < firstbad) { firstbad = u; have = 1; } }
+        }
+    }
+    if (bad) *bad = firstbad;
+    return nbad;
+}
+
+/* ---------- fp16 (IEEE binary16) conversions, round to nearest even ---------- */
+uint16_t orc_f32_to_h16(float f) {
+    const uint32_t u = f2u(f), s = (u >> 16) & 0x8000u, a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(s | 0x7e00u);
+    if (a >= 0x477ff000u) return (uint16_t)(s | 0x7c00u);   /* >= 65520 rounds to inf */
+    if (a < 0x33000001u) return (uint16_t)s;                /* <= 2^-25: rounds to zero (2^-25 ties to even 0) */
+    const int e = (int)(a >> 23) - 127;
+    if (e < -14) {                                          /* subnormal half: units of 2^-24 */
+        const float r = rintf(ldexpf(u2f(a), 24));
+        return (uint16_t)(s | (unsigned)r);
+    }
+    const uint32_t m = a & 0x7fffffu, keep = m >> 13, rem = m & 0x1fffu;
+    uint32_t h = ((uint32_t)(e + 15) << 10) | keep;
+    if (rem > 0x1000u || (rem == 0x1000u && (keep & 1u))) h++;
+    return (uint16_t)(s | h);
+}
+float orc_h16_to_f32(uint16_t h) {
+    const uint32_t s = (uint32_t)(h & 0x8000u) << 16, e = (h >> 10) & 31u, m = h & 0x3ffu;
+    if (e == 31u) return u2f(s | 0x7f800000u | (m << 13));
+    if (!e) { const float v = ldexpf((float)m, -24); return s ? -v : v; }
+    return u2f(s | ((e + 112u) << 23) | (m << 13));
+}
+
+/* ---------- one block row (src/lp_mxops.cuh:45-65 for the NaN-propagating amax; src/lp_f8fwd.cuh:90-103 for fmaxf) ---------- */
+static void enc_codes(int bits, const float *v, int bw, float m, uint8_t *codes) {
+    if (bits == 8) for (int k = 0; k < bw; k++) codes[k] = (uint8_t)orc_enc_e4m3(v[k] * m);
+    else for (int k = 0; k < bw; k += 2) codes[k >> 1] = (uint8_t)(orc_enc_e2m1(v[k] * m) | (orc_enc_e2m1(v[k + 1] * m) << 4));   /* low nibble first */
+}
+uint8_t orc_store_row(int bits, const float *v, int bw, uint8_t *codes, int nanprop) {
+    float amax;
+    if (nanprop) { uint32_t am = 0; for (int k = 0; k < bw; k++) { const uint32_t a = f2u(v[k]) & 0x7fffffffu; if (a > am) am = a; } amax = u2f(am); }
+    else { amax = 0.f; for (int k = 0; k < bw; k++) amax = fmaxf(amax, fabsf(v[k])); }
+    const int e = orc_mx_exp(amax, bits == 8 ? INVQ8 : INVQ4);
+    enc_codes(bits, v, bw, orc_exp2i(-e), codes);
+    return (uint8_t)(e + 127);
+}
+void orc_load_row(int bits, const uint8_t *codes, uint8_t sbyte, int bw, float *v) {
+    const float s = orc_mx_scale(sbyte);
+    if (bits == 8) for (int k = 0; k < bw; k++) v[k] = orc_dec_e4m3(codes[k]) * s;
+    else for (int k = 0; k < bw; k++) v[k] = orc_dec_e2m1((codes[k >> 1] >> (4 * (k & 1))) & 15u) * s;
+}
+
+/* ---------- tensor layout (src/lp_common.cuh:100-106, src/lp_mxops.cuh:69-70) ---------- */
+typedef struct { const uint8_t *q, *sc; int bits, bw, nb, rb, N, C; size_t S; } mxt_t;
+static mxt_t mxt(const void *p, int bits, int N, int C, size_t S) {
+    mxt_t t; t.q = (const uint8_t *)p; t.bits = bits; t.bw = orc_mx_bw(C); t.nb = orc_mx_nb(C); t.rb = rowbytes(t.bw, bits);
+    t.N = N; t.C = C; t.S = S; t.sc = t.q + (size_t)N * t.nb * S * t.rb; return t;
+}
+static inline size_t mxrow(const mxt_t *t, int n, int blk, size_t v) { return ((size_t)n * t->nb + blk) * t->S + v; }
+/* decoded 32 channels of block blk at voxel v (channels past bw are zero) */
+static void mx_row32(const mxt_t *t, int n, int blk, size_t v, float *r) {
+    for (int k = 0; k < 32; k++) r[k] = 0.f;
+    if (blk >= t->nb) return;
+    const size_t ri = mxrow(t, n, blk, v);
+    orc_load_row(t->bits, t->q + ri * t->rb, t->sc[ri], t->bw, r);
+}
+
+void orc_f32_to_mx(int bits, const float *x, int N, int C, size_t S, uint8_t *y) {
+    const mxt_t t = mxt(y, bits, N, C, S);
+    uint8_t *q = y, *sc = y + (size_t)N * t.nb * S * t.rb;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)((size_t)N * t.nb * S); i++) {
+        const size_t v = (size_t)i % S; const int blk = (int)(((size_t)i / S) % t.nb), n = (int)((size_t)i / (S * t.nb));
+        float r[32];
+        for (int k = 0; k < t.bw; k++) { const int c = blk * t.bw + k; r[k] = c < C ? x[((size_t)n * C + c) * S + v] : 0.f; }
+        sc[i] = orc_store_row(bits, r, t.bw, q + (size_t)i * t.rb, 1);
+    }
+}
+void orc_h16_to_mx(int bits, const uint16_t *x, int N, int C, size_t S, uint8_t *y) {
+    const mxt_t t = mxt(y, bits, N, C, S);
+    uint8_t *q = y, *sc = y + (size_t)N * t.nb * S * t.rb;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)((size_t)N * t.nb * S); i++) {
+        const size_t v = (size_t)i % S; const int blk = (int)(((size_t)i / S) % t.nb), n = (int)((size_t)i / (S * t.nb));
+        float r[32];
+        for (int k = 0; k < t.bw; k++) { const int c = blk * t.bw + k; r[k] = c < C ? orc_h16_to_f32(x[((size_t)n * C + c) * S + v]) : 0.f; }
+        sc[i] = orc_store_row(bits, r, t.bw, q + (size_t)i * t.rb, 1);
+    }
+}
+void orc_mx_to_f32(int bits, const uint8_t *x, int N, int C, size_t S, float *y) {
+    const mxt_t t = mxt(x, bits, N, C, S);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)((size_t)N * t.nb * S); i++) {
+        const size_t v = (size_t)i % S; const int blk = (int)(((size_t)i / S) % t.nb), n = (int)((size_t)i / (S * t.nb));
+        float r[32];
+        orc_load_row(bits, t.q + (size_t)i * t.rb, t.sc[i], t.bw, r);
+        for (int k = 0; k < t.bw; k++) { const int c = blk * t.bw + k; if (c < C) y[((size_t)n * C + c) * S + v] = r[k]; }
+    }
+}
+/* src/lp_mx_cvt.cu:29-41 */
+void orc_pred_input_mx(int bits, const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis,
+                       int z0, int nz, uint8_t *y, int hd) {
+    const size_t S = (size_t)nz * W * W; const int rb = rowbytes(8, bits);
+    uint8_t *sc = y + S * rb;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)S; i++) {
+        const int xx = (int)(i % W), yy = (int)((i / W) % W), z = z0 + (int)(i / ((int64_t)W * W));
+        const float dy = dyo[z] + (float)yy, dx = dxo[z] + (float)xx, inv = axis ? (float)axis / (sqrtf(dy * dy + dx * dx) + 1e-6f) : 0.f;
+        float r[8] = {0};
+        r[0] = ((float)ct[(size_t)z * W * W + (size_t)yy * W + xx] - mean) * isd; r[2] = dy * inv; r[3] = dx * inv;
+        if (hd == 2) for (int k = 0; k < 4; k++) r[k] = orc_h16_to_f32(orc_f32_to_h16(r[k]));
+        sc[i] = orc_store_row(bits, r, 8, y + (size_t)i * rb, 1);
+    }
+}
+
+/* ---------- weights (src/lp_f8fwd.cu:54-71; src/lp_f4fwd.cu:53-66): one block = the 32 ci of one (tap, co) ----------
+   padded input channel cp -> real channel (src/lp_common.cuh:235): MX inputs pad each of the two segments to 32 */
+static int seg_ci(int cp, int Ci, int Cx, int CxP) { if (cp < CxP) return cp < Cx ? cp : -1; const int c = Cx + cp - CxP; return c < Ci ? c : -1; }
+void orc_prep_w(int bits, const float *w, int Co, int Ci, int Cx, int CxP, int Cip, float *wv, uint8_t *ws, uint8_t *wcodes) {
+    const int nch = Cip / 32;
+#pragma omp parallel for schedule(static)
+    for (int i = 0; i < 27 * Co * nch; i++) {
+        const int ch = i % nch, co = (i / nch) % Co, t = i / (nch * Co);
+        float v[32]; uint8_t codes[32];
+        for (int k = 0; k < 32; k++) { const int ci = seg_ci(ch * 32 + k, Ci, Cx, CxP); v[k] = ci >= 0 ? w[((size_t)co * Ci + ci) * 27 + t] : 0.f; }
+        const uint8_t sb = orc_store_row(bits, v, 32, codes, 0);
+        ws[i] = sb;
+        if (wcodes) memcpy(wcodes + (size_t)i * rowbytes(32, bits), codes, rowbytes(32, bits));
+        float *dst = wv + ((size_t)t * Co + co) * Cip + ch * 32;
+        for (int k = 0; k < 32; k++) dst[k] = bits == 8 ? orc_dec_e4m3(codes[k]) : orc_dec_e2m1((codes[k >> 1] >> (4 * (k & 1))) & 15u);
+    }
+}
+
+/* ---------- GN + SiLU of the conv staging (src/lp_common.cuh:258, :474-482): u = fma(x, a, b), h = u / 2, h + h tanh(h) ---------- */
+float orc_act_ab(float v, float a, float b) {
+    /* the reference's h + h tanh(h), h = u / 2, is u sigmoid(u); its tanh is NVIDIA's tanh.approx (about 2^-11), so the oracle takes
+       the exact value of the same function, correctly rounded: any faithful evaluation is inside the reference's own error */
+    const float u = fmaf(v, a, b);
+    return (float)((double)u / (1.0 + exp(-(double)u)));
+}
+static void gn_ab(const orc_gn_t *g, int n, int cc, int Cg, float *a, float *b) {
+    const int ng = n * g->G + cc / (Cg / g->G);
+    *a = g->rstd[ng] * g->gamma[cc];
+    *b = fmaf(-g->mean[ng], *a, g->beta[cc]);               /* tests/test_mx4_wide.c:119 */
+}
+/* per padded-channel (a, b, has_gn) table of sample n */
+typedef struct { float a, b; int g, ci; } chab_t;
+static void chan_table(const orc_conv_t *c, int n, int Cx, int CxP, int Cip, chab_t *tab) {
+    const int s2g = c->x2 && c->gp2.G;
+    for (int cp = 0; cp < Cip; cp++) {
+        const int mxin = c->xdt >= 3;
+        const int ci = mxin ? seg_ci(cp, c->Ci, Cx, CxP) : (cp < c->Ci ? cp : -1);
+        chab_t t = {1.f, 0.f, 0, ci};
+        if (ci >= 0) {
+            const orc_gn_t *q = s2g && ci >= Cx ? &c->gp2 : &c->gp;
+            const int cc = s2g && ci >= Cx ? ci - Cx : ci, Cg = s2g ? (ci >= Cx ? c->Ci - Cx : Cx) : c->Ci;
+            if (q->G) { gn_ab(q, n, cc, Cg, &t.a, &t.b); t.g = 1; }
+        }
+        tab[cp] = t;
+    }
+}
+
+/* ---------- staging (src/lp_f8fwd.cuh:66-113): per (n, 32-channel chunk, input voxel) the compute-format codes and scale ----------
+   Returned as decoded code values sv[n][chunk][voxel][32] and scale sf[n][chunk][voxel] (fp32 power of two).
+   Staged geometry = the input's own grid (stride 1: D x H x W; stride 2: the input dims). */
+typedef struct { float *sv; float *sf; int nch, Cip, Cx, CxP; size_t S; } staged_t;
+static void quant_row(int cbits, const float *v, float *sv, float *sf) {
+    uint8_t codes[32];
+    const uint8_t sb = orc_store_row(cbits, v, 32, codes, 0);
+    *sf = orc_mx_scale(sb);
+    for (int k = 0; k < 32; k++) sv[k] = cbits == 8 ? orc_dec_e4m3(codes[k]) : orc_dec_e2m1((codes[k >> 1] >> (4 * (k & 1))) & 15u);
+}
+/* decoder up segment (src/lp_common.cuh:618-670): coarse rows -> GN + SiLU -> e4m3 rows with a row scale (amax ignoring NaN) */
+static void coarse_rows(const orc_conv_t *c, int n, int blk, int Cx, const chab_t *tab, int Dc, int Hc, int Wc, float *cv /* [Sc][32 codes + scale] */) {
+    const size_t Sc = (size_t)Dc * Hc * Wc;
+    const mxt_t t = mxt(c->x, c->xdt == 3 ? 8 : 4, c->N, Cx, Sc);
+    for (size_t v = 0; v < Sc; v++) {
+        float r[32];
+        mx_row32(&t, n, blk, v, r);
+        for (int k = 0; k < 32; k++) if (tab[blk * 32 + k].g) r[k] = orc_act_ab(r[k], tab[blk * 32 + k].a, tab[blk * 32 + k].b);
+        uint32_t am = 0; for (int k = 0; k < 32; k++) { const uint32_t u = f2u(fabsf(r[k])); if (u <= 0x7f800000u && u > am) am = u; }
+        const int e = orc_mx_exp(u2f(am), INVQ8); const float m = orc_exp2i(-e), s = orc_mx_scale((unsigned)(e + 127));
+        /* stored as code and scale; the blend multiplies the weight by the scale first (stage_up_smem) */
+        for (int k = 0; k < 32; k++) cv[v * 33 + k] = orc_dec_e4m3(orc_enc_e4m3(r[k] * m));
+        cv[v * 33 + 32] = s;
+    }
+}
+static int build_staged(const orc_conv_t *c, staged_t *st) {
+    const int mxin = c->xdt >= 3, xbits = c->xdt == 3 ? 8 : 4;
+    const int Cx = c->x2 ? c->c_split : c->Ci, CxP = (Cx + 31) / 32 * 32;
+    const int Cip = mxin ? CxP + (c->Ci - Cx + 31) / 32 * 32 : (c->Ci + 31) / 32 * 32;
+    const size_t S = (size_t)c->D * c->H * c->W;
+    st->nch = Cip / 32; st->Cip = Cip; st->Cx = Cx; st->CxP = CxP; st->S = S;
+    st->sv = (float *)malloc((size_t)c->N * st->nch * S * 32 * sizeof(float));
+    st->sf = (float *)malloc((size_t)c->N * st->nch * S * sizeof(float));
+    if (!st->sv || !st->sf) return -1;
+    const int G = c->gp.G || c->gp2.G;
+    const int Dc = c->D >> 1, Hc = c->H >> 1, Wc = c->W >> 1;
+    for (int n = 0; n < c->N; n++) {
+        chab_t *tab = (chab_t *)malloc((size_t)Cip * sizeof(chab_t));
+        chan_table(c, n, Cx, CxP, Cip, tab);
+        for (int ch = 0; ch < st->nch; ch++) {
+            const int upc = mxin && c->up && ch * 32 < CxP;
+            const int sec = mxin && ch * 32 >= CxP;       /* chunk of the x2 segment */
+            float *cv = NULL;
+            if (upc) { cv = (float *)malloc((size_t)Dc * Hc * Wc * 33 * sizeof(float)); coarse_rows(c, n, ch, Cx, tab, Dc, Hc, Wc, cv); }
+            mxt_t t;
+            if (mxin) t = sec ? mxt(c->x2, xbits, c->N, c->Ci - Cx, S) : mxt(c->x, xbits, c->N, Cx, S);
+            const int blk = sec ? ch - CxP / 32 : ch;
+#pragma omp parallel for schedule(static)
+            for (int64_t vi = 0; vi < (int64_t)S; vi++) {
+                const size_t v = (size_t)vi;
+                float *sv = st->sv + (((size_t)n * st->nch + ch) * S + v) * 32, *sf = st->sf + ((size_t)n * st->nch + ch) * S + v;
+                float r[32];
+                if (upc) {   /* 8-term blend, fma order a (z), b (y), c (x) (stage_up_smem) */
+                    const int gz = (int)(v / ((size_t)c->H * c->W)), gy = (int)(v / c->W % c->H), gx = (int)(v % c->W);
+                    int mz[2], my[2], mx[2];
+                    mz[0] = gz >> 1; mz[1] = mz[0] + ((gz & 1) ? 1 : -1); if (mz[1] < 0) mz[1] = 0; if (mz[1] > Dc - 1) mz[1] = Dc - 1;
+                    my[0] = gy >> 1; my[1] = my[0] + ((gy & 1) ? 1 : -1); if (my[1] < 0) my[1] = 0; if (my[1] > Hc - 1) my[1] = Hc - 1;
+                    mx[0] = gx >> 1; mx[1] = mx[0] + ((gx & 1) ? 1 : -1); if (mx[1] < 0) mx[1] = 0; if (mx[1] > Wc - 1) mx[1] = Wc - 1;
+                    for (int k = 0; k < 32; k++) r[k] = 0.f;
+                    for (int a = 0; a < 2; a++) for (int b = 0; b < 2; b++) for (int cc = 0; cc < 2; cc++) {
+                        const float *row = cv + (((size_t)mz[a] * Hc + my[b]) * Wc + mx[cc]) * 33;
+                        const float w3 = (a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (cc ? 0.25f : 0.75f) * row[32];
+                        for (int k = 0; k < 32; k++) r[k] = fmaf(w3, row[k], r[k]);
+                    }
+                    quant_row(c->cbits, r, sv, sf);
+                } else if (mxin) {
+                    const int copy = !G && ((c->xdt == 3 && c->cbits == 8) || (c->xdt == 4 && c->cbits == 4));
+                    if (copy) {   /* stored block used as is (src/lp_f8fwd.cuh:68-87) */
+                        for (int k = 0; k < 32; k++) sv[k] = 0.f;
+                        *sf = orc_mx_scale(1);
+                        if (blk < t.nb) {
+                            const size_t ri = mxrow(&t, n, blk, v);
+                            for (int k = 0; k < t.bw; k++) sv[k] = xbits == 8 ? orc_dec_e4m3(t.q[ri * t.rb + k]) : orc_dec_e2m1((t.q[ri * t.rb + (k >> 1)] >> (4 * (k & 1))) & 15u);
+                            *sf = orc_mx_scale(t.sc[ri]);
+                        }
+                    } else {
+                        mx_row32(&t, n, blk, v, r);
+                        for (int k = 0; k < 32; k++) { const chab_t *q = &tab[ch * 32 + k]; r[k] = q->ci < 0 ? 0.f : q->g ? orc_act_ab(r[k], q->a, q->b) : r[k]; }
+                        quant_row(c->cbits, r, sv, sf);
+                    }
+                } else {     /* plane-major fp32 / fp16 input, quantised per (voxel, 32 channels) */
+                    for (int k = 0; k < 32; k++) {
+                        const chab_t *q = &tab[ch * 32 + k];
+                        float xv = 0.f;
+                        if (q->ci >= 0) {
+                            const int sec2 = c->x2 && q->ci >= Cx;
+                            const size_t idx = sec2 ? ((size_t)n * (c->Ci - Cx) + q->ci - Cx) * S + v : ((size_t)n * Cx + q->ci) * S + v;
+                            const void *src = sec2 ? c->x2 : c->x;
+                            xv = c->xdt == 2 ? orc_h16_to_f32(((const uint16_t *)src)[idx]) : ((const float *)src)[idx];
+                            if (q->g) xv = orc_act_ab(xv, q->a, q->b);
+                        }
+                        r[k] = xv;
+                    }
+                    quant_row(c->cbits, r, sv, sf);
+                }
+            }
+            free(cv);
+        }
+        free(tab);
+    }
+    /* tap-packed stem (src/lp_f8fwd.cuh:374-380): one scale per staged tile of 4 x 10 x 18 positions around a 2 x 8 x 16 output tile.
+       The per-position rows above are replaced by rows quantised with the tile's scale at conv time (see orc_conv3). */
+    return 0;
+}
+int orc_conv3_staged(const orc_conv_t *c, float *out) {
+    staged_t st;
+    if (build_staged(c, &st)) return -1;
+    const size_t n = (size_t)c->N * st.nch * st.S;
+    for (size_t i = 0; i < n; i++) for (int k = 0; k < 32; k++) out[i * 32 + k] = st.sv[i * 32 + k] * st.sf[i];
+    free(st.sv); free(st.sf);
+    return st.Cip;
+}
+
+static float gelu_f(float x) { return 0.5f * x * (1.f + (float)erf((double)x * 0.70710678118654752440)); }
+static float silu_f(float x) { return (float)((double)x / (1.0 + exp(-(double)x))); }
+
+/* ---------- the convolution (src/lp_f8fwd.cuh:52, :114-148; src/lp_common.cuh:1465-1597) ---------- */
+int orc_conv3(const orc_conv_t *c) {
+    staged_t st;
+    if (c->cbits != 8 && c->cbits != 4) return -2;
+    if (build_staged(c, &st)) return -1;
+    const int Co = c->Co, nch = st.nch, Cip = st.Cip, s = c->stride == 2 ? 2 : 1;
+    const int Do = s == 2 ? (c->D - 1) / 2 + 1 : c->D, Ho = s == 2 ? (c->H - 1) / 2 + 1 : c->H, Wo = s == 2 ? (c->W - 1) / 2 + 1 : c->W;   /* src/nn_bwd.cu:132-135 */
+    const size_t So = (size_t)Do * Ho * Wo;
+    float *wv = (float *)malloc((size_t)27 * Co * Cip * sizeof(float));
+    uint8_t *ws = (uint8_t *)malloc((size_t)27 * Co * nch);
+    orc_prep_w(c->cbits, c->w, Co, c->Ci, c->xdt >= 3 ? st.Cx : c->Ci, c->xdt >= 3 ? st.CxP : (c->Ci + 31) / 32 * 32, Cip, wv, ws, NULL);
+    float *wsf = (float *)malloc((size_t)27 * Co * nch * sizeof(float));
+    for (size_t i = 0; i < (size_t)27 * Co * nch; i++) wsf[i] = orc_mx_scale(ws[i]);
+    const int ybits = c->ydt == 3 ? 8 : 4, ybw = orc_mx_bw(Co), ynb = orc_mx_nb(Co), yrb = rowbytes(ybw, ybits);
+    uint8_t *yq = (uint8_t *)c->y, *ysc = yq + (size_t)c->N * ynb * So * yrb;
+    const int z0 = c->z1 ? c->z0 : 0, z1 = c->z1 ? c->z1 : Do;
+    const int cpg = c->Go ? Co / c->Go : 1;
+    for (int n = 0; n < c->N; n++) {
+        double *gs = c->osum ? (double *)calloc((size_t)2 * c->Go, sizeof(double)) : NULL;
+#pragma omp parallel
+        {
+            float *acc = (float *)malloc((size_t)Co * sizeof(float));
+            double *acc64 = (double *)malloc((size_t)Co * sizeof(double));
+            double *ls = gs ? (double *)calloc((size_t)2 * c->Go, sizeof(double)) : NULL;
+#pragma omp for schedule(dynamic, 64)
+            for (int64_t vi = (int64_t)z0 * Ho * Wo; vi < (int64_t)z1 * Ho * Wo; vi++) {
+                const int oz = (int)(vi / ((int64_t)Ho * Wo)), oy = (int)(vi / Wo % Ho), ox = (int)(vi % Wo);
+                for (int co = 0; co < Co; co++) { acc[co] = 0.f; acc64[co] = 0.0; }
+                for (int ch = 0; ch < nch; ch++)                       /* chunk-major, tap-minor (src/lp_f8fwd.cuh:52) */
+                    for (int t = 0; t < 27; t++) {
+                        const int iz = s * oz - 1 + t / 9, iy = s * oy - 1 + (t / 3) % 3, ix = s * ox - 1 + t % 3;
+                        if (iz < 0 || iz >= c->D || iy < 0 || iy >= c->H || ix < 0 || ix >= c->W) continue;   /* stored zeros contribute +0 */
+                        const size_t iv = ((size_t)iz * c->H + iy) * c->W + ix;
+                        const float *xv = st.sv + (((size_t)n * nch + ch) * st.S + iv) * 32;
+                        const float xs = st.sf[((size_t)n * nch + ch) * st.S + iv];
+                        for (int co = 0; co < Co; co++) {
+                            const float *wr = wv + ((size_t)t * Co + co) * Cip + ch * 32;
+                            double d = 0.0;                              /* exact: products of code values, 32 terms */
+                            for (int k = 0; k < 32; k++) d += (double)wr[k] * (double)xv[k];
+                            const double blk = d * (double)wsf[((size_t)t * Co + co) * nch + ch] * (double)xs;
+                            if (c->acc64) acc64[co] += blk; else acc[co] += (float)blk;
+                        }
+                    }
+                /* epilogue (src/lp_common.cuh:1492-1535) */
+                for (int co = 0; co < Co; co++) {
+                    float v = c->acc64 ? (float)(acc64[co] + (c->b ? (double)c->b[co] : 0.0)) : acc[co] + (c->b ? c->b[co] : 0.f);
+                    if (c->fused_act) {
+                        if (c->ep_a) v = fmaf(v, c->ep_a[co], c->ep_b[co]);
+                        v = c->fused_act == 1 ? silu_f(v) : c->fused_act == 2 ? gelu_f(v) : c->fused_act == 3 ? fmaxf(v, 0.f) : v;
+                    }
+                    acc[co] = v;
+                }
+                const size_t ov = (size_t)vi;
+                if (c->ydt >= 3) {
+                    for (int blk = 0; blk < ynb; blk++) {
+                        float r[32]; uint8_t codes[32];
+                        for (int k = 0; k < ybw; k++) { const int co = blk * ybw + k; r[k] = co < Co ? acc[co] : 0.f; }
+                        const size_t ri = ((size_t)n * ynb + blk) * So + ov;
+                        const uint8_t sb = orc_store_row(ybits, r, ybw, codes, 0);
+                        memcpy(yq + ri * yrb, codes, (size_t)yrb); ysc[ri] = sb;
+                        if (ls && c->stored_stats) { float d[32]; orc_load_row(ybits, codes, sb, ybw, d); for (int k = 0; k < ybw; k++) { const int co = blk * ybw + k; if (co < Co) acc[co] = d[k]; } }
+                    }
+                } else if (c->ydt == 2) {
+                    for (int co = 0; co < Co; co++) {
+                        float v = acc[co];
+                        if (c->Go > 0 && fabsf(v) > 65504.f) v = copysignf(65504.f, v);   /* sat_h16 (src/lp_common.cuh:465, :1567-1569) */
+                        ((uint16_t *)c->y)[((size_t)n * Co + co) * So + ov] = orc_f32_to_h16(v);
+                        acc[co] = v;
+                    }
+                } else for (int co = 0; co < Co; co++) ((float *)c->y)[((size_t)n * Co + co) * So + ov] = acc[co];
+                if (ls) for (int co = 0; co < Co; co++) { const double v = acc[co]; ls[2 * (co / cpg)] += v; ls[2 * (co / cpg) + 1] += v * v; }
+            }
+            if (ls) {
+#pragma omp critical
+                for (int i = 0; i < 2 * c->Go; i++) gs[i] += ls[i];
+                free(ls);
+            }
+            free(acc); free(acc64);
+        }
+        if (gs) { for (int i = 0; i < 2 * c->Go; i++) c->osum[(size_t)n * 2 * c->Go + i] += gs[i]; free(gs); }
+    }
+    free(wv); free(ws); free(wsf); free(st.sv); free(st.sf);
+    return 0;
+}
+
+/* ---------- GroupNorm ---------- */
+void orc_gn_finalize(const double *sums, int NG, size_t len, float eps, float *mean, float *rstd) {   /* src/nn_elem.cu:5-11 */
+    for (int i = 0; i < NG; i++) {
+        const double m = sums[2 * i] / (double)len, v = sums[2 * i + 1] / (double)len - m * m;
+        mean[i] = (float)m; rstd[i] = (float)(1.0 / sqrt((v > 0 ? v : 0) + (double)eps));
+    }
+}
+void orc_gn_sums_mx(int bits, const uint8_t *x, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1) {
+    const mxt_t t = mxt(x, bits, N, C, S); const int cpg = C / G;
+    for (int n = 0; n < N; n++) for (int blk = 0; blk < t.nb; blk++)
+        for (size_t v = v0; v < v1; v++) {
+            float r[32]; mx_row32(&t, n, blk, v, r);
+            for (int k = 0; k < t.bw; k++) { const int c = blk * t.bw + k; if (c < C) { const double d = r[k]; sums[2 * ((size_t)n * G + c / cpg)] += d; sums[2 * ((size_t)n * G + c / cpg) + 1] += d * d; } }
+        }
+}
+/* src/lp_mx_gn.cu:17: v = (x - mean) rstd gamma + beta (left to right, the last multiply-add contracted), v / (1 + exp(-v)) */
+static float apply_silu(float x, float mean, float rstd, float gamma, float beta) {
+    const float v = fmaf((x - mean) * rstd, gamma, beta);
+    return (float)((double)v / (1.0 + exp(-(double)v)));
+}
+void orc_gn_silu_apply_mx(const void *x, int xdt, int N, int C, size_t S, orc_gn_t gp, uint8_t *y, int ybits) {
+    const int bw = orc_mx_bw(C), nb = orc_mx_nb(C), yrb = rowbytes(bw, ybits), cpg = C / gp.G;
+    uint8_t *ysc = y + (size_t)N * nb * S * yrb;
+    mxt_t t; if (xdt >= 3) t = mxt(x, xdt == 3 ? 8 : 4, N, C, S);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)((size_t)N * nb * S); i++) {
+        const size_t v = (size_t)i % S; const int blk = (int)(((size_t)i / S) % nb), n = (int)((size_t)i / (S * nb));
+        float r[32] = {0};
+        if (xdt >= 3) mx_row32(&t, n, blk, v, r);
+        else for (int k = 0; k < bw; k++) { const int c = blk * bw + k; if (c < C) r[k] = ((const float *)x)[((size_t)n * C + c) * S + v]; }
+        for (int k = 0; k < bw; k++) {
+            const int c = blk * bw + k; if (c >= C) { r[k] = 0.f; continue; }
+            const int ng = n * gp.G + c / cpg;
+            r[k] = apply_silu(r[k], gp.mean[ng], gp.rstd[ng], gp.gamma[c], gp.beta[c]);
+        }
+        ysc[i] = orc_store_row(ybits, r, bw, y + (size_t)i * yrb, 1);
+    }
+}
+/* src/lp_mx_gn.cu:34-73: fine (z, y, x) <- 8 coarse rows, weights .75 / .25 per axis, edge clamp, fma order z, y, x */
+void orc_up2_mx(int xbits, const uint8_t *x, int N, int C, int D, int H, int W, orc_gn_t gp, uint8_t *y, int ybits) {
+    const size_t Sc = (size_t)D * H * W, Sf = Sc * 8; const int Hf = 2 * H, Wf = 2 * W;
+    const mxt_t t = mxt(x, xbits, N, C, Sc);
+    const int bw = t.bw, nb = t.nb, yrb = rowbytes(bw, ybits), cpg = gp.G ? C / gp.G : 1;
+    uint8_t *ysc = y + (size_t)N * nb * Sf * yrb;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)((size_t)N * nb * Sf); i++) {
+        const size_t v = (size_t)i % Sf; const int blk = (int)(((size_t)i / Sf) % nb), n = (int)((size_t)i / (Sf * nb));
+        const int gz = (int)(v / ((size_t)Hf * Wf)), gy = (int)(v / Wf % Hf), gx = (int)(v % Wf);
+        int mz[2], my[2], mx[2];
+        mz[0] = gz >> 1; mz[1] = mz[0] + ((gz & 1) ? 1 : -1); if (mz[1] < 0) mz[1] = 0; if (mz[1] > D - 1) mz[1] = D - 1;
+        my[0] = gy >> 1; my[1] = my[0] + ((gy & 1) ? 1 : -1); if (my[1] < 0) my[1] = 0; if (my[1] > H - 1) my[1] = H - 1;
+        mx[0] = gx >> 1; mx[1] = mx[0] + ((gx & 1) ? 1 : -1); if (mx[1] < 0) mx[1] = 0; if (mx[1] > W - 1) mx[1] = W - 1;
+        float o[32] = {0};
+        for (int a = 0; a < 2; a++) for (int b = 0; b < 2; b++) for (int c = 0; c < 2; c++) {
+            float r[32]; mx_row32(&t, n, blk, ((size_t)mz[a] * H + my[b]) * W + mx[c], r);
+            if (gp.G) for (int k = 0; k < bw; k++) {
+                const int ch = blk * bw + k; if (ch >= C) continue;
+                const int ng = n * gp.G + ch / cpg; const float aa = gp.rstd[ng] * gp.gamma[ch], bb = fmaf(-gp.mean[ng], aa, gp.beta[ch]);
+                r[k] = orc_act_ab(r[k], aa, bb);   /* src/lp_mx_gn.cu:66-67: the staging form of GN + SiLU */
+            }
+            const float w3 = (a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f);
+            for (int k = 0; k < bw; k++) o[k] = fmaf(w3, r[k], o[k]);
+        }
+        ysc[i] = orc_store_row(ybits, o, bw, y + (size_t)i * yrb, 1);
+    }
+}
+/* src/lp_mx_conv1.cu:5-21: fp32 FMA in ci order, bias first */
+void orc_conv1_mx(int xbits, const uint8_t *x, int N, int Ci, size_t S, const float *w, const float *b, int Co, orc_gn_t gp, float *y) {
+    const mxt_t t = mxt(x, xbits, N, Ci, S); const int cpg = gp.G ? Ci / gp.G : 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)((size_t)N * S); i++) {
+        const size_t v = (size_t)i % S; const int n = (int)((size_t)i / S);
+        float xin[1024];
+        for (int blk = 0; blk < t.nb; blk++) mx_row32(&t, n, blk, v, xin + blk * t.bw);
+        if (gp.G) for (int ci = 0; ci < Ci; ci++) { const int ng = n * gp.G + ci / cpg; const float a = gp.rstd[ng] * gp.gamma[ci], bb = fmaf(-gp.mean[ng], a, gp.beta[ci]); xin[ci] = orc_act_ab(xin[ci], a, bb); }
+        for (int co = 0; co < Co; co++) {
+            float acc = b ? b[co] : 0.f;
+            for (int ci = 0; ci < Ci; ci++) acc = fmaf(w[(size_t)co * Ci + ci], xin[ci], acc);
+            y[((size_t)n * Co + co) * S + v] = acc;
+        }
+    }
+}

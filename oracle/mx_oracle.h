@@ -1,0 +1,108 @@
+/* CPU oracle of the MX (fp8 e4m3 / fp4 e2m1, E8M0 block scale) 3-D U-Net forward arithmetic.
+ *
+ * TEST INFRASTRUCTURE ONLY. This is a plain-C restatement of the reference's algorithm, used as the checker by the
+ * tests, by the smoke test and as the timed "cpu_baseline" leg of the benchmark. Nothing in the shipped GPU path may
+ * call it. Every function names the reference lines it follows (paths relative to the reference checkout).
+ *
+ * Pinning status (what holds each function to the reference without running the reference):
+ *   orc_enc_e4m3 / orc_enc_e2m1   pinned: == independent nearest-grid-point search (orc_ref_*) over all 2^32 floats
+ *   orc_mx_exp                    pinned: closed form "smallest e with amax * fl(1/qmax) <= 2^e", cross-checked
+ *                                 against the ceil(log2(amax/qmax)) form of tests/test_mx4.c:51
+ *   orc_store_row / orc_f32_to_mx pinned: decoded output == host_mx4 / q_rn style quantiser written from the format
+ *   orc_conv3 (copy staging)      pinned: exact-operand construction (tests/test_mx4_wide.c:81-98) == fp64 direct conv
+ *   orc_conv3 epilogue requant    pinned: == block quantiser of the exact conv (cmp_mx, tests/test_mx4_wide.c:252-265)
+ *   GroupNorm sums / finalize     pinned: independent fp64 statistics; constant group => rstd = 1/sqrt(eps)
+ *   trilinear staging, up2        pinned: closed form 0.75/0.25 separable weights with edge clamp, grid data exact
+ *   1x1x1 head                    pinned: plain dot product (GEMM special case)
+ *   SiLU in GN staging            PARITY UNPINNED to the bit: the reference evaluates tanh with NVIDIA's
+ *                                 tanh.approx.f32 (src/lp_common.cuh:469-473), not reproducible off that hardware;
+ *                                 checked to floor/ceil code neighbours as tests/test_mx4_wide.c:165-175 does
+ *   stem tile scale (Ci <= 8)     PARITY UNPINNED to the bit: one scale per staged tile depends on the reference's tile
+ *                                 geometry (src/lp_f8fwd.cuh:374-380); restated with that geometry, tolerance only
+ */
+#ifndef MX_ORACLE_H
+#define MX_ORACLE_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- scalar format arithmetic ---- */
+int orc_mx_bw(int C);                                 /* src/lp_common.cuh:132 */
+int orc_mx_nb(int C);                                 /* src/lp_common.cuh:133 */
+size_t orc_mx_bytes(int bits, int N, int C, size_t S);/* src/lp_mx_cvt.cu:6-7 */
+int orc_mx_exp(float amax, float inv_qmax);           /* src/lp_common.cuh:492-500 */
+float orc_exp2i(int e);                               /* src/lp_common.cuh:501 */
+float orc_mx_scale(unsigned sbyte);                   /* src/lp_common.cuh:186 */
+unsigned orc_enc_e4m3(float x);                       /* src/mx_sw.cuh:14-36 (semantics), own formulation */
+unsigned orc_enc_e2m1(float x);                       /* src/mx_sw.cuh:37-56 */
+float orc_dec_e4m3(unsigned b);                       /* src/mx_sw.cuh:78-83 */
+float orc_dec_e2m1(unsigned n);                       /* src/mx_sw.cuh:84-87 */
+unsigned orc_ref_e4m3(float x);                       /* nearest-grid search, the pin of orc_enc_e4m3 */
+unsigned orc_ref_e2m1(float x);
+/* sweep [first, first + count) of fp32 bit patterns: number of inputs where enc != ref (either format); first bad in *bad */
+uint64_t orc_enc_sweep(uint32_t first, uint64_t count, uint32_t stride, uint32_t *bad);
+
+/* one block row: v[bw] -> codes (bw bytes fp8 / bw/2 bytes fp4) + scale byte. nanprop: NaN-propagating amax
+   (src/lp_mxops.cuh:45-65) else fmaxf amax (src/lp_f8fwd.cuh:91) */
+uint8_t orc_store_row(int bits, const float *v, int bw, uint8_t *codes, int nanprop);
+void orc_load_row(int bits, const uint8_t *codes, uint8_t sbyte, int bw, float *v);   /* src/lp_common.cuh:189-232 */
+
+/* ---- tensor converters (src/lp_mx_cvt.cu:9-19, 429-447) ---- */
+void orc_f32_to_mx(int bits, const float *x, int N, int C, size_t S, uint8_t *y);
+void orc_h16_to_mx(int bits, const uint16_t *x, int N, int C, size_t S, uint8_t *y);   /* fp16 source */
+void orc_mx_to_f32(int bits, const uint8_t *x, int N, int C, size_t S, float *y);
+/* network input (src/lp_mx_cvt.cu:29-41): hd 2 = fp16 rounding, 0 none */
+void orc_pred_input_mx(int bits, const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis,
+                       int z0, int nz, uint8_t *y, int hd);
+
+/* ---- weights (src/lp_f8fwd.cu:54-71, src/lp_f4fwd.cu:53-66): w[co][ci][27] -> decoded block values wv[t][co][Cip] (code
+   values, not yet scaled) and scale bytes ws[t][co][Cip/32]; Cip = padded input channels of the (split) input ---- */
+void orc_prep_w(int bits, const float *w, int Co, int Ci, int Cx, int CxP, int Cip, float *wv, uint8_t *ws, uint8_t *wcodes);
+
+/* ---- GroupNorm descriptor of an input segment (src/nn_lp.h:15) ---- */
+typedef struct { const float *gamma, *beta, *mean, *rstd; int G; } orc_gn_t;
+
+typedef struct {
+    /* input */
+    const void *x; int xdt;            /* 0 fp32 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4 */
+    int N, Ci, D, H, W;                /* output-resolution input dims for stride 1; the input's dims for stride 2 */
+    const void *x2; int c_split;       /* channels >= c_split come from x2 (same dtype) */
+    int up;                            /* the x segment is stored at D/2 x H/2 x W/2 and read trilinearly upsampled */
+    orc_gn_t gp, gp2;                  /* GN + SiLU of x (or of all channels when gp2.G == 0) and of x2 */
+    /* weights */
+    const float *w, *b; int Co; int stride;   /* 3x3x3, pad 1, stride 1 or 2 */
+    int cbits;                         /* compute format: 8 (e4m3) or 4 (e2m1) */
+    /* output */
+    void *y; int ydt;                  /* 0 fp32 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4 */
+    double *osum; int Go; int stored_stats;   /* plain doubles [N][Go][2] (sum, sum of squares), accumulated */
+    int acc64;                         /* 1: accumulate in fp64 (exact-operand checks) */
+    int fused_act; const float *ep_a, *ep_b;   /* extension: epilogue affine + activation (1 SiLU, 2 GELU, 3 ReLU) before requant */
+    int z0, z1;                        /* output z planes [z0, z1) only (z1 0: all): the bounded CPU-baseline slab */
+    int stem_tile;                     /* 1: one activation scale per staged 4x10x18 tile (Ci <= 8 tap-packed stem) */
+} orc_conv_t;
+/* 3x3x3 forward conv with MX operands (src/lp_f8fwd.cuh:19-151, src/lp_common.cuh:1465-1597, src/lp_s2.cu:4-9) */
+int orc_conv3(const orc_conv_t *c);
+/* staged (quantised) operand of a conv's input only: values = decoded code * scale per (n, padded channel, voxel) */
+int orc_conv3_staged(const orc_conv_t *c, float *staged);
+
+/* GroupNorm finalize (src/nn_elem.cu:5-11) */
+void orc_gn_finalize(const double *sums, int NG, size_t len, float eps, float *mean, float *rstd);
+/* (sum, sumsq) per (n, group) of a stored MX tensor over voxels [v0, v1) (src/lp_mx_gnsums.cu:8-80) */
+void orc_gn_sums_mx(int bits, const uint8_t *x, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1);
+/* y = MX(silu(gn(x))) (src/lp_mx_gn.cu:5-21; exp form v / (1 + exp(-v))) */
+void orc_gn_silu_apply_mx(const void *x, int xdt, int N, int C, size_t S, orc_gn_t gp, uint8_t *y, int ybits);
+/* trilinear 2x upsample of an MX tensor, optional GN + SiLU of the coarse values (src/lp_mx_gn.cu:34-73) */
+void orc_up2_mx(int xbits, const uint8_t *x, int N, int C, int D, int H, int W, orc_gn_t gp, uint8_t *y, int ybits);
+/* 1x1x1 head (src/lp_mx_conv1.cu:5-21): y[n][co][v] fp32 */
+void orc_conv1_mx(int xbits, const uint8_t *x, int N, int Ci, size_t S, const float *w, const float *b, int Co, orc_gn_t gp, float *y);
+/* GN affine + SiLU of the conv staging (src/lp_common.cuh:474-482): u = fma(v, a, b), u sigmoid(u) correctly rounded */
+float orc_act_ab(float v, float a, float b);
+uint16_t orc_f32_to_h16(float f);
+float orc_h16_to_f32(uint16_t h);
+int orc_threads(void);
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,119 @@
+"""ctypes binding of the CPU oracle (oracle/liboracle.so). Test infrastructure only."""
+import ctypes as C
+import os
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(ROOT, "oracle", "liboracle.so")
+
+
+class orc_gn_t(C.Structure):
+    _fields_ = [("gamma", C.c_void_p), ("beta", C.c_void_p), ("mean", C.c_void_p), ("rstd", C.c_void_p), ("G", C.c_int)]
+
+
+class orc_conv_t(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("xdt", C.c_int), ("N", C.c_int), ("Ci", C.c_int), ("D", C.c_int), ("H", C.c_int), ("W", C.c_int),
+                ("x2", C.c_void_p), ("c_split", C.c_int), ("up", C.c_int), ("gp", orc_gn_t), ("gp2", orc_gn_t),
+                ("w", C.c_void_p), ("b", C.c_void_p), ("Co", C.c_int), ("stride", C.c_int), ("cbits", C.c_int),
+                ("y", C.c_void_p), ("ydt", C.c_int), ("osum", C.c_void_p), ("Go", C.c_int), ("stored_stats", C.c_int),
+                ("acc64", C.c_int), ("fused_act", C.c_int), ("ep_a", C.c_void_p), ("ep_b", C.c_void_p),
+                ("z0", C.c_int), ("z1", C.c_int), ("stem_tile", C.c_int)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            import subprocess
+            subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "liboracle.so"])
+        L = C.CDLL(LIB_PATH)
+        L.orc_mx_exp.restype = C.c_int; L.orc_mx_exp.argtypes = [C.c_float, C.c_float]
+        L.orc_exp2i.restype = C.c_float; L.orc_exp2i.argtypes = [C.c_int]
+        L.orc_mx_scale.restype = C.c_float; L.orc_mx_scale.argtypes = [C.c_uint]
+        for n in ("orc_enc_e4m3", "orc_enc_e2m1", "orc_ref_e4m3", "orc_ref_e2m1"):
+            getattr(L, n).restype = C.c_uint; getattr(L, n).argtypes = [C.c_float]
+        for n in ("orc_dec_e4m3", "orc_dec_e2m1"):
+            getattr(L, n).restype = C.c_float; getattr(L, n).argtypes = [C.c_uint]
+        L.orc_enc_sweep.restype = C.c_uint64; L.orc_enc_sweep.argtypes = [C.c_uint32, C.c_uint64, C.c_uint32, C.POINTER(C.c_uint32)]
+        L.orc_mx_bytes.restype = C.c_size_t; L.orc_mx_bytes.argtypes = [C.c_int, C.c_int, C.c_int, C.c_size_t]
+        L.orc_store_row.restype = C.c_uint8; L.orc_store_row.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_void_p, C.c_int]
+        L.orc_load_row.restype = None; L.orc_load_row.argtypes = [C.c_int, C.c_void_p, C.c_uint8, C.c_int, C.c_void_p]
+        L.orc_f32_to_mx.restype = None; L.orc_f32_to_mx.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_void_p]
+        L.orc_h16_to_mx.restype = None; L.orc_h16_to_mx.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_void_p]
+        L.orc_mx_to_f32.restype = None; L.orc_mx_to_f32.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_void_p]
+        L.orc_pred_input_mx.restype = None
+        L.orc_pred_input_mx.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_float, C.c_float, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int]
+        L.orc_prep_w.restype = None
+        L.orc_prep_w.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.orc_conv3.restype = C.c_int; L.orc_conv3.argtypes = [C.POINTER(orc_conv_t)]
+        L.orc_conv3_staged.restype = C.c_int; L.orc_conv3_staged.argtypes = [C.POINTER(orc_conv_t), C.c_void_p]
+        L.orc_gn_finalize.restype = None; L.orc_gn_finalize.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_void_p, C.c_void_p]
+        L.orc_gn_sums_mx.restype = None; L.orc_gn_sums_mx.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t]
+        L.orc_gn_silu_apply_mx.restype = None; L.orc_gn_silu_apply_mx.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_size_t, orc_gn_t, C.c_void_p, C.c_int]
+        L.orc_up2_mx.restype = None; L.orc_up2_mx.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, orc_gn_t, C.c_void_p, C.c_int]
+        L.orc_conv1_mx.restype = None; L.orc_conv1_mx.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_size_t, C.c_void_p, C.c_void_p, C.c_int, orc_gn_t, C.c_void_p]
+        L.orc_act_ab.restype = C.c_float; L.orc_act_ab.argtypes = [C.c_float, C.c_float, C.c_float]
+        L.orc_f32_to_h16.restype = C.c_uint16; L.orc_f32_to_h16.argtypes = [C.c_float]
+        L.orc_h16_to_f32.restype = C.c_float; L.orc_h16_to_f32.argtypes = [C.c_uint16]
+        L.orc_threads.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def ptr(a):
+    return a.ctypes.data if a is not None else None
+
+
+def gn(gamma=None, beta=None, mean=None, rstd=None, G=0):
+    g = orc_gn_t()
+    if G:
+        g.gamma, g.beta, g.mean, g.rstd, g.G = ptr(gamma), ptr(beta), ptr(mean), ptr(rstd), G
+    return g
+
+
+def mx_bytes(bits, N, C, S):
+    return lib().orc_mx_bytes(bits, N, C, S)
+
+
+def f32_to_mx(bits, x, N, C, S):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.zeros(mx_bytes(bits, N, C, S), dtype=np.uint8)
+    lib().orc_f32_to_mx(bits, ptr(x), N, C, S, ptr(y))
+    return y
+
+
+def mx_to_f32(bits, q, N, C, S):
+    q = np.ascontiguousarray(q, dtype=np.uint8)
+    y = np.zeros((N, C, S), dtype=np.float32)
+    lib().orc_mx_to_f32(bits, ptr(q), N, C, S, ptr(y))
+    return y
+
+
+def conv3(x, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=8, stride=1, x2=None, c_split=0, up=0, gp=None, gp2=None, Go=0, want_stats=False,
+          stored_stats=0, acc64=0, fused_act=0, ep_a=None, ep_b=None, z0=0, z1=0):
+    """Runs the oracle conv; returns (y, sums or None). y: uint8 MX bytes, float32 or uint16 (fp16 bits) planes [N][Co][So]."""
+    c = orc_conv_t()
+    keep = [x, x2, w, b, ep_a, ep_b]
+    c.x, c.xdt, c.N, c.Ci, c.D, c.H, c.W = ptr(x), xdt, N, Ci, D, H, W
+    c.x2, c.c_split, c.up = ptr(x2), c_split, up
+    c.gp = gp if gp is not None else orc_gn_t(); c.gp2 = gp2 if gp2 is not None else orc_gn_t()
+    c.w, c.b, c.Co, c.stride, c.cbits = ptr(w), ptr(b), Co, stride, cbits
+    Do, Ho, Wo = ((D - 1) // 2 + 1, (H - 1) // 2 + 1, (W - 1) // 2 + 1) if stride == 2 else (D, H, W)
+    So = Do * Ho * Wo
+    if ydt >= 3:
+        y = np.zeros(mx_bytes(8 if ydt == 3 else 4, N, Co, So), dtype=np.uint8)
+    elif ydt == 2:
+        y = np.zeros((N, Co, So), dtype=np.uint16)
+    else:
+        y = np.zeros((N, Co, So), dtype=np.float32)
+    sums = np.zeros((N, max(Go, 1), 2), dtype=np.float64) if want_stats else None
+    c.y, c.ydt, c.osum, c.Go, c.stored_stats = ptr(y), ydt, ptr(sums), Go, stored_stats
+    c.acc64, c.fused_act, c.ep_a, c.ep_b, c.z0, c.z1 = acc64, fused_act, ptr(ep_a), ptr(ep_b), z0, z1
+    rc = lib().orc_conv3(C.byref(c))
+    assert rc == 0, rc
+    del keep
+    return y, sums

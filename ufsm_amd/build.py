@@ -1,0 +1,55 @@
+"""Builds the HIP library (gfx950) and the CPU oracle in-tree. Used by __graft_entry__.build(); tests and the bench only load what is built."""
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "ufsm_amd", "csrc")
+LIB = os.path.join(ROOT, "ufsm_amd", "libufsm_lp.so")
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
+HIP_SOURCES = ["rt.hip", "mx_elem.hip", "conv3.hip"]
+HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wno-unused-value",
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _run(cmd, cwd=None):
+    r = subprocess.run(cmd, cwd=cwd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in r.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_hip(verbose=False):
+    objs = []
+    procs = []
+    for src in HIP_SOURCES:
+        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        cmd = ["hipcc"] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+    for cmd, p in procs:
+        out, _ = p.communicate()
+        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l)
+        if p.returncode != 0:
+            raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+        if verbose and out.strip():
+            print(out)
+    _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    return LIB
+
+
+def build_oracle():
+    _run(["make", "-B", "liboracle.so"], cwd=ORACLE_DIR)
+    return ORACLE_LIB
+
+
+def build_all(verbose=False):
+    build_oracle()
+    build_hip(verbose)
+
+
+if __name__ == "__main__":
+    build_all(verbose=True)
+    print("built", LIB, "and", ORACLE_LIB)

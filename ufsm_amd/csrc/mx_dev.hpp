@@ -1,0 +1,165 @@
+// Device-side MX arithmetic for gfx950: E8M0 scale selection, e4m3 / e2m1 element encode / decode, block-row helpers.
+// Semantics follow the reference's conversion routines (src/lp_common.cuh:484-555, src/mx_sw.cuh:1-56); the formulations are this
+// build's own (magic-number rounding for e4m3, midpoint thresholds for e2m1) and are checked bit for bit on the device.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/mi_lp.h"
+
+#define MI_INVQ8 (1.f / 448.f)
+#define MI_INVQ4 (1.f / 6.f)
+
+__host__ __device__ __forceinline__ int mx_bw(int C) { return C <= 8 ? 8 : C <= 16 ? 16 : 32; }       // src/lp_common.cuh:132
+__host__ __device__ __forceinline__ int mx_nb(int C) { const int bw = mx_bw(C); return (C + bw - 1) / bw; }
+__host__ __device__ __forceinline__ int mx_rb(int bw, int bits) { return bw * bits / 8; }
+
+// scale exponent: smallest e with amax * fl(1 / qmax) <= 2^e, clamped; NaN / inf (or an overflowing product) -> 128 (src/lp_common.cuh:492-500)
+__device__ __forceinline__ int d_mx_exp(float amax, float inv_qmax) {
+    const unsigned u = __float_as_uint(amax * inv_qmax) & 0x7fffffffu;
+    const int e = (int)(u >> 23) - 127 + ((u & 0x7fffffu) ? 1 : 0);
+    const int ec = e < -126 ? -126 : e > 126 ? 126 : e;
+    return u >= 0x7f800000u ? 128 : ec;
+}
+__device__ __forceinline__ float d_exp2i(int e) { return __uint_as_float((unsigned)(127 + e) << 23); }   // e = -128: the bits of -inf, as the reference (src/lp_common.cuh:501)
+__device__ __forceinline__ float d_mx_scale(unsigned sbyte) { return __uint_as_float((sbyte & 255u) << 23); }   // 0xFF -> +inf
+
+// NaN-propagating |v| max on the bit patterns (src/lp_common.cuh:487)
+__device__ __forceinline__ unsigned d_amax_u(unsigned a, float v) { const unsigned b = __float_as_uint(v) & 0x7fffffffu; return b > a ? b : a; }
+
+// e4m3 (OCP FN: max 448, 0x7f NaN), round to nearest even, saturating. For |x| < 448 the value is rounded to a multiple of the
+// binade's quantum 2^(E-3) (E >= -6) by adding and subtracting 1.5 * 2^(E+20), whose ulp is that quantum; the rounded value is
+// exactly representable, so its code is a re-biased bit field (normal) or value * 2^9 (subnormal).
+__device__ __forceinline__ unsigned d_enc_e4m3(float x) {
+    const unsigned u = __float_as_uint(x), a = u & 0x7fffffffu;
+    unsigned ef = a >> 23; ef = ef < 121u ? 121u : ef; ef = ef > 136u ? 136u : ef;
+    const float M = __uint_as_float(((ef + 20u) << 23) | 0x400000u);
+    const float ax = __uint_as_float(a);
+    float r = ax + M;
+    asm volatile("" : "+v"(r));            // keep (ax + M) - M as two rounded operations
+    r -= M;
+    const unsigned rb = __float_as_uint(r);
+    unsigned code = rb >= 0x3c800000u ? (rb >> 20) - 0x3c0u : (unsigned)(r * 512.f);
+    code = a >= 0x43e00000u ? 0x7eu : code;             // >= 448 (incl. inf) saturates
+    code |= (u >> 24) & 0x80u;
+    return a > 0x7f800000u ? 0x7fu : code;              // NaN of either sign
+}
+__device__ __forceinline__ unsigned d_enc_e4m3x4(float a, float b, float c, float d) {
+    return d_enc_e4m3(a) | (d_enc_e4m3(b) << 8) | (d_enc_e4m3(c) << 16) | (d_enc_e4m3(d) << 24);
+}
+// e2m1: grid {0, .5, 1, 1.5, 2, 3, 4, 6}; the code is the number of midpoints passed, ties to the even code; > 6 -> 6; NaN -> +6
+__device__ __forceinline__ unsigned d_enc_e2m1(float x) {
+    const unsigned u = __float_as_uint(x), a = u & 0x7fffffffu;
+    const float ax = __uint_as_float(a);
+    unsigned c = (unsigned)(ax > 0.25f) + (unsigned)(ax >= 0.75f) + (unsigned)(ax > 1.25f) + (unsigned)(ax >= 1.75f) +
+                 (unsigned)(ax > 2.5f) + (unsigned)(ax >= 3.5f) + (unsigned)(ax > 5.f);
+    c |= (u >> 28) & 8u;
+    return a > 0x7f800000u ? 7u : c;
+}
+__device__ __forceinline__ unsigned d_enc_e2m1x8(const float *v, float m) {   // 8 values -> 8 nibbles, v[0] lowest
+    unsigned w = 0u;
+#pragma unroll
+    for (int k = 0; k < 8; k++) w |= d_enc_e2m1(v[k] * m) << (4 * k);
+    return w;
+}
+// decoders (exact): e4m3 byte, e2m1 nibble -> fp32
+__device__ __forceinline__ float d_dec_e4m3(unsigned b) {
+    const unsigned em = b & 0x7fu, e = em >> 3, m = em & 7u;
+    // normal: 1.m * 2^(e-7) -> fp32 field; subnormal: m * 2^-9 as an exact int -> float product
+    const float nv = __uint_as_float(((e + 120u) << 23) | (m << 20));
+    float v = e ? nv : (float)m * 0.001953125f;
+    v = em == 0x7fu ? __uint_as_float(0x7fc00000u) : v;
+    return __uint_as_float(__float_as_uint(v) | ((b & 0x80u) << 24));
+}
+__device__ __forceinline__ float d_dec_e2m1(unsigned n) {
+    const unsigned c = n & 7u;
+    // {0, .5, 1, 1.5, 2, 3, 4, 6} = mantissa bit c & 1, exponent (c >> 1): c < 2 is the subnormal pair {0, .5}
+    const float v = c < 2u ? 0.5f * (float)c : __uint_as_float(((126u + (c >> 1)) << 23) | ((c & 1u) << 22));
+    return (n & 8u) ? -v : v;
+}
+
+// one block row of bw values -> codes + scale byte. NANPROP: the NaN-propagating amax of the converters and elementwise ops
+// (src/lp_mxops.cuh:45-65), else fmaxf (conv staging, src/lp_f8fwd.cuh:91). codes: 8 words (fp8) / 4 words (fp4), zero past bw.
+template <int BITS, bool NANPROP>
+__device__ __forceinline__ unsigned d_quant_row(const float *v, int bw, unsigned *codes) {
+    float amax;
+    if (NANPROP) {
+        unsigned am = 0u;
+#pragma unroll
+        for (int k = 0; k < 32; k++) if (k < bw) am = d_amax_u(am, v[k]);
+        amax = __uint_as_float(am);
+    } else {
+        amax = 0.f;
+#pragma unroll
+        for (int k = 0; k < 32; k++) if (k < bw) amax = fmaxf(amax, fabsf(v[k]));
+    }
+    const int e = d_mx_exp(amax, BITS == 8 ? MI_INVQ8 : MI_INVQ4);
+    const float m = d_exp2i(-e);
+    if (BITS == 8) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) codes[j] = 4 * j < bw ? d_enc_e4m3x4(v[4 * j] * m, v[4 * j + 1] * m, v[4 * j + 2] * m, v[4 * j + 3] * m) : 0u;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) codes[j] = 8 * j < bw ? d_enc_e2m1x8(v + 8 * j, m) : 0u;
+    }
+    return (unsigned)(e + 127);
+}
+// decode a row held in words (8 words fp8 / 4 words fp4) times the scale
+template <int BITS>
+__device__ __forceinline__ void d_dequant_row(const unsigned *codes, unsigned sbyte, float *v) {
+    const float s = d_mx_scale(sbyte);
+    if (BITS == 8) {
+#pragma unroll
+        for (int k = 0; k < 32; k++) v[k] = d_dec_e4m3(codes[k >> 2] >> (8 * (k & 3))) * s;
+    } else {
+#pragma unroll
+        for (int k = 0; k < 32; k++) v[k] = d_dec_e2m1(codes[k >> 3] >> (4 * (k & 7))) * s;
+    }
+}
+// load the words of a stored row of bw channels (zero past the row)
+template <int BITS>
+__device__ __forceinline__ void d_load_row_words(const uint8_t *p, int bw, unsigned *w) {
+    constexpr int NW = BITS == 8 ? 8 : 4;
+#pragma unroll
+    for (int j = 0; j < NW; j++) w[j] = 0u;
+    const int nbytes = mx_rb(bw, BITS);
+    if (nbytes == 32) { const uint4 a = *(const uint4 *)p, b = *(const uint4 *)(p + 16); w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; if (NW == 8) { w[4] = b.x; w[5] = b.y; w[6] = b.z; w[7] = b.w; } }
+    else if (nbytes == 16) { const uint4 a = *(const uint4 *)p; w[0] = a.x; w[1] = a.y; w[2] = a.z; w[3] = a.w; }
+    else if (nbytes == 8) { const uint2 a = *(const uint2 *)p; w[0] = a.x; w[1] = a.y; }
+    else w[0] = *(const unsigned *)p;
+}
+template <int BITS>
+__device__ __forceinline__ void d_store_row_words(uint8_t *p, int bw, const unsigned *w) {
+    const int nbytes = mx_rb(bw, BITS);
+    if (nbytes == 32) { *(uint4 *)p = make_uint4(w[0], w[1], w[2], w[3]); *(uint4 *)(p + 16) = make_uint4(w[BITS == 8 ? 4 : 0], w[BITS == 8 ? 5 : 0], w[BITS == 8 ? 6 : 0], w[BITS == 8 ? 7 : 0]); }
+    else if (nbytes == 16) *(uint4 *)p = make_uint4(w[0], w[1], w[2], w[3]);
+    else if (nbytes == 8) *(uint2 *)p = make_uint2(w[0], w[1]);
+    else *(unsigned *)p = w[0];
+}
+// GN + SiLU of the conv staging (src/lp_common.cuh:474-482): u = fma(x, a, b), then u * sigmoid(u) (= h + h tanh(h), h = u / 2)
+__device__ __forceinline__ float d_act_ab(float v, float a, float b) {
+    const float u = fmaf(v, a, b);
+    return __fdividef(u, 1.f + __expf(-u));     // u -> -inf: exp overflows to inf and the quotient is -0
+}
+
+// exact fixed-point GroupNorm sum slot add (src/gnacc.cuh:12-20): slot = [fraction, 2^-64 units][integer part][non-finite count];
+// integer atomics, so the sums do not depend on the order of the adds
+__device__ __forceinline__ void gn_acc_add(double *b, size_t i, double v) {
+    unsigned long long *w = (unsigned long long *)b + 3 * i;
+    if (!(fabs(v) < 4.611686018427387904e18)) { atomicAdd(&w[2], 1ull); return; }
+    const double f = floor(v);
+    const long long hi = (long long)f;
+    const unsigned long long lo = (unsigned long long)((v - f) * 18446744073709551616.0);
+    if (lo) { const unsigned long long o = atomicAdd(&w[0], lo); if (o + lo < o) atomicAdd(&w[1], 1ull); }
+    if (hi) atomicAdd(&w[1], (unsigned long long)hi);
+}
+
+// ---- host-side shared declarations of the library's units ----
+void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits);
+void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits);
+void mi_post_error(hipError_t e, const char *file, int line);
+#define MICK() do { hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)
+#define MIRT(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)
+void *mi_ws(int slot, size_t bytes);        // per-device grow-on-demand scratch (the reference's nn_ws, src/nn_core.cu:751)
+enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_NSLOTS = 8 };
+static inline unsigned nblk_(size_t n, unsigned b) { return (unsigned)((n + b - 1) / b); }
+[[noreturn]] void mi_die(const char *fmt, ...);

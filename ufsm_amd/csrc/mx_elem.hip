@@ -1,0 +1,447 @@
+// MX tensor conversions and elementwise / pointwise ops (HBM-bound): fp32 / fp16 <-> MX, network input rows, GN + SiLU apply,
+// trilinear 2x upsample, add, GroupNorm sums, 1x1x1 head, and the operand re-staging used by the conv dispatch.
+// One thread owns one (n, block, voxel) row, so the per-row amax that defines the output scale is thread-local
+// (the reference's arrangement, src/lp_mxops.cuh:5-7); consecutive threads walk consecutive voxels, so both the plane-major
+// reads (one coalesced run per channel) and the 8..32-byte row writes are contiguous across a wavefront.
+#include "mx_dev.hpp"
+#include <hip/hip_fp16.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+extern "C" size_t lp_mx8_bytes(int N, int C, size_t S) { return (size_t)N * mx_nb(C) * S * (mx_bw(C) + 1); }       // src/lp_mx_cvt.cu:6
+extern "C" size_t lp_mx4_bytes(int N, int C, size_t S) { return (size_t)N * mx_nb(C) * S * (mx_bw(C) / 2 + 1); }   // src/lp_mx_cvt.cu:7
+
+template <typename T> __device__ __forceinline__ float ldx(const T *p, size_t i);
+template <> __device__ __forceinline__ float ldx<float>(const float *p, size_t i) { return p[i]; }
+template <> __device__ __forceinline__ float ldx<__half>(const __half *p, size_t i) { return __half2float(p[i]); }
+struct bf16_t { unsigned short v; };
+template <> __device__ __forceinline__ float ldx<bf16_t>(const bf16_t *p, size_t i) { return __uint_as_float((unsigned)p[i].v << 16); }
+
+template <int B> __device__ __forceinline__ uint8_t *mx_scp(uint8_t *q, int N, int C, size_t S) { return q + (size_t)N * mx_nb(C) * S * mx_rb(mx_bw(C), B); }
+template <int B> __device__ __forceinline__ const uint8_t *mx_scp(const uint8_t *q, int N, int C, size_t S) { return q + (size_t)N * mx_nb(C) * S * mx_rb(mx_bw(C), B); }
+
+// row i of an MX tensor -> 32 floats (zero past bw)
+template <int B> __device__ __forceinline__ void load_row(const uint8_t *x, const uint8_t *sc, size_t i, int bw, float *r) {
+    unsigned w[8];
+    d_load_row_words<B>(x + i * mx_rb(bw, B), bw, w);
+    if (B == 4) { w[4] = w[5] = w[6] = w[7] = 0u; }
+    d_dequant_row<B>(w, sc[i], r);
+}
+template <int B, bool NANPROP> __device__ __forceinline__ void store_row(uint8_t *y, uint8_t *sc, size_t i, int bw, const float *r) {
+    unsigned w[8];
+    const unsigned sb = d_quant_row<B, NANPROP>(r, bw, w);
+    d_store_row_words<B>(y + i * mx_rb(bw, B), bw, w);
+    sc[i] = (uint8_t)sb;
+}
+
+// ---- fp32 / 16-bit planes [n][C][S] -> MX (src/lp_mx_cvt.cu:9-19) ----
+template <int B, typename TI>
+__global__ void __launch_bounds__(256) f32_to_mx_k(const TI *x, uint8_t *y, int N, int C, size_t S) {
+    const int bw = mx_bw(C), nb = mx_nb(C);
+    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (i >= (size_t)N * nb * S) return;
+    const size_t v = i % S; const int blk = (int)((i / S) % nb), n = (int)(i / (S * nb));
+    float r[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) { const int c = blk * bw + k; r[k] = k < bw && c < C ? ldx(x, ((size_t)n * C + c) * S + v) : 0.f; }
+    store_row<B, true>(y, mx_scp<B>(y, N, C, S), i, bw, r);
+}
+template <int B> static void f32_to_mx(const float *x, int N, int C, size_t S, void *y) {
+    const size_t n = (size_t)N * mx_nb(C) * S;
+    if (!n) return;
+    f32_to_mx_k<B, float><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, N, C, S); MICK();
+}
+extern "C" void lp_f32_to_mx8(const float *x, int N, int C, size_t S, void *y) { f32_to_mx<8>(x, N, C, S, y); }
+extern "C" void lp_f32_to_mx4(const float *x, int N, int C, size_t S, void *y) { f32_to_mx<4>(x, N, C, S, y); }
+template <int B> static void h16_to_mx(const void *x, int dt, int N, int C, size_t S, void *y) {
+    const size_t n = (size_t)N * mx_nb(C) * S;
+    if (!n) return;
+    if (dt == 2) f32_to_mx_k<B, __half><<<nblk_(n, 256), 256>>>((const __half *)x, (uint8_t *)y, N, C, S);
+    else if (dt == 1) f32_to_mx_k<B, bf16_t><<<nblk_(n, 256), 256>>>((const bf16_t *)x, (uint8_t *)y, N, C, S);
+    else mi_die("lp_h16_to_mx%d: dtype %d is not 16-bit (1 bf16, 2 fp16)", B, dt);
+    MICK();
+}
+extern "C" void lp_h16_to_mx8(const void *x, int dt, int N, int C, size_t S, void *y) { h16_to_mx<8>(x, dt, N, C, S, y); }
+extern "C" void lp_h16_to_mx4(const void *x, int dt, int N, int C, size_t S, void *y) { h16_to_mx<4>(x, dt, N, C, S, y); }
+
+// ---- MX -> fp32 planes (src/lp_mx_cvt.cu:429-447) ----
+template <int B>
+__global__ void __launch_bounds__(256) mx_to_f32_k(const uint8_t *x, float *y, int N, int C, size_t S) {
+    const int bw = mx_bw(C), nb = mx_nb(C);
+    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (i >= (size_t)N * nb * S) return;
+    const size_t v = i % S; const int blk = (int)((i / S) % nb), n = (int)(i / (S * nb));
+    float r[32];
+    load_row<B>(x, mx_scp<B>(x, N, C, S), i, bw, r);
+#pragma unroll
+    for (int k = 0; k < 32; k++) { const int c = blk * bw + k; if (k < bw && c < C) y[((size_t)n * C + c) * S + v] = r[k]; }
+}
+extern "C" void lp_mx8_to_f32(const void *x, int N, int C, size_t S, float *y) {
+    const size_t n = (size_t)N * mx_nb(C) * S; if (!n) return;
+    mx_to_f32_k<8><<<nblk_(n, 256), 256>>>((const uint8_t *)x, y, N, C, S); MICK();
+}
+extern "C" void lp_mx4_to_f32(const void *x, int N, int C, size_t S, float *y) {
+    const size_t n = (size_t)N * mx_nb(C) * S; if (!n) return;
+    mx_to_f32_k<4><<<nblk_(n, 256), 256>>>((const uint8_t *)x, y, N, C, S); MICK();
+}
+
+// ---- network input rows (src/lp_mx_cvt.cu:29-55): z-scored CT, 0, unit direction away from the axis -> one 8-wide row per voxel ----
+template <int HD> __device__ __forceinline__ float in_round(float v) {
+    if (HD == 2) return __half2float(__float2half(v));
+    if (HD == 1) { unsigned u = __float_as_uint(v); if ((u & 0x7fffffffu) > 0x7f800000u) return v; u += 0x7fffu + ((u >> 16) & 1u); return __uint_as_float(u & 0xffff0000u); }
+    return v;
+}
+template <int B, int HD>
+__global__ void __launch_bounds__(256) pred_in_mx_k(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, uint8_t *y) {
+    const size_t S = (size_t)nz * W * W, i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (i >= S) return;
+    const int xx = (int)(i % W), yy = (int)((i / W) % W), z = z0 + (int)(i / ((size_t)W * W));
+    const float dy = dyo[z] + (float)yy, dx = dxo[z] + (float)xx, inv = axis ? (float)axis / (sqrtf(dy * dy + dx * dx) + 1e-6f) : 0.f;
+    float r[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) r[k] = 0.f;
+    r[0] = in_round<HD>(((float)ct[(size_t)z * W * W + (size_t)yy * W + xx] - mean) * isd); r[1] = in_round<HD>(0.f);
+    r[2] = in_round<HD>(dy * inv); r[3] = in_round<HD>(dx * inv);
+    store_row<B, true>(y, mx_scp<B>(y, 1, 4, S), i, 8, r);
+}
+extern "C" void lp_pred_input_mx(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits) {
+    const size_t S = (size_t)nz * W * W; if (!S) return;
+    uint8_t *yy = (uint8_t *)y;
+#define PIN(B, HD) pred_in_mx_k<B, HD><<<nblk_(S, 256), 256>>>(ct, W, mean, isd, dyo, dxo, axis, z0, nz, yy)
+    if (bits == 4) { if (hd == 2) PIN(4, 2); else if (hd == 1) PIN(4, 1); else PIN(4, 0); }
+    else { if (hd == 2) PIN(8, 2); else if (hd == 1) PIN(8, 1); else PIN(8, 0); }
+#undef PIN
+    MICK();
+}
+extern "C" void lp_pred_input_mx8(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd) {
+    lp_pred_input_mx(ct, W, mean, isd, dyo, dxo, axis, z0, nz, y, hd, 8);
+}
+
+// ---- y = MX(silu(gn(x))) (src/lp_mx_gn.cu:5-31): v = (x - mean) rstd gamma + beta, v / (1 + exp(-v)) ----
+template <int BX, int BY, typename TI>
+__global__ void __launch_bounds__(256) gn_silu_apply_mx_k(const void *xv, uint8_t *y, int N, int C, int G, size_t S, const float *gamma, const float *beta, const float *mean, const float *rstd) {
+    const int bw = mx_bw(C), nb = mx_nb(C), cpg = C / G;
+    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (i >= (size_t)N * nb * S) return;
+    const size_t v = i % S; const int blk = (int)((i / S) % nb), n = (int)(i / (S * nb));
+    float r[32];
+    if (BX != 0) { const uint8_t *x = (const uint8_t *)xv; load_row<BX ? BX : 8>(x, mx_scp<BX ? BX : 8>(x, N, C, S), i, bw, r); }
+    else {
+#pragma unroll
+        for (int k = 0; k < 32; k++) { const int c = blk * bw + k; r[k] = k < bw && c < C ? ldx((const TI *)xv, ((size_t)n * C + c) * S + v) : 0.f; }
+    }
+#pragma unroll
+    for (int k = 0; k < 32; k++) {
+        const int c = blk * bw + k;
+        if (k < bw && c < C) { const int ng = n * G + c / cpg; const float u = fmaf((r[k] - mean[ng]) * rstd[ng], gamma[c], beta[c]); r[k] = __fdividef(u, 1.f + __expf(-u)); }
+        else r[k] = 0.f;
+    }
+    store_row<BY, true>(y, mx_scp<BY>(y, N, C, S), i, bw, r);
+}
+extern "C" void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, const float *gamma, const float *beta, const float *mean, const float *rstd, void *y, int ydt) {
+    const size_t S = (size_t)s.d * s.h * s.w, n = (size_t)s.n * mx_nb(s.c) * S;
+    if (ydt != 3 && ydt != 4) mi_die("lp_gn_silu_apply_mx: output dtype %d is not MX", ydt);
+    if (G <= 0 || s.c % G) mi_die("lp_gn_silu_apply_mx: %d channels in %d groups", s.c, G);
+    if (!n) return;
+#define GSA(BX, BY, TI) gn_silu_apply_mx_k<BX, BY, TI><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, s.n, s.c, G, S, gamma, beta, mean, rstd)
+#define GSA_Y(BX, TI) do { if (ydt == 4) GSA(BX, 4, TI); else GSA(BX, 8, TI); } while (0)
+    if (xdt == 4) GSA_Y(4, float); else if (xdt == 3) GSA_Y(8, float); else if (xdt == 2) GSA_Y(0, __half); else if (xdt == 1) GSA_Y(0, bf16_t); else GSA_Y(0, float);
+#undef GSA_Y
+#undef GSA
+    MICK();
+}
+
+// ---- trilinear 2x upsample (src/lp_mx_gn.cu:34-73, :151-186): out[o] = .75 in[o/2] + .25 in[o/2 -+ 1] per axis, edge clamp ----
+template <int BX, int BY>
+__global__ void __launch_bounds__(256) up2_mx_k(const uint8_t *x, uint8_t *y, int N, int Cx, int b0, int Cy, int D, int H, int W, gnp_t gp) {
+    // x: Cx channels, blocks b0.. feed y's blocks 0..; y: Cy channels
+    const int bwx = mx_bw(Cx), nbx = mx_nb(Cx), bwy = mx_bw(Cy), nby = mx_nb(Cy), Do = 2 * D, Ho = 2 * H, Wo = 2 * W;
+    const size_t S = (size_t)D * H * W, So = (size_t)Do * Ho * Wo;
+    const int nbk = blockIdx.y, n = nbk / nby, blk = nbk % nby;
+    __shared__ float ca[32], cb[32];
+    if (threadIdx.x < 32) {
+        const int k = threadIdx.x, ci = blk * bwy + k;
+        float a = 1.f, b = 0.f;
+        if (gp.G && k < bwy && ci < Cy) { const int ng = n * gp.G + ci / (Cy / gp.G); a = gp.rstd[ng] * gp.gamma[ci]; b = fmaf(-gp.mean[ng], a, gp.beta[ci]); }
+        ca[k] = a; cb[k] = b;
+    }
+    __syncthreads();
+    const size_t vo = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (vo >= So) return;
+    const int ox = (int)(vo % Wo), oy = (int)((vo / Wo) % Ho), oz = (int)(vo / ((size_t)Wo * Ho));
+    const int mz[2] = {oz >> 1, min(max((oz >> 1) + ((oz & 1) ? 1 : -1), 0), D - 1)}, my[2] = {oy >> 1, min(max((oy >> 1) + ((oy & 1) ? 1 : -1), 0), H - 1)},
+              mx[2] = {ox >> 1, min(max((ox >> 1) + ((ox & 1) ? 1 : -1), 0), W - 1)};
+    const uint8_t *sc = mx_scp<BX>(x, N, Cx, S);
+    const int kmax = min(bwy, Cy - blk * bwy);
+    float acc[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) acc[k] = 0.f;
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                float r[32];
+                const float w3 = (a ? 0.25f : 0.75f) * (bb ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f);
+                load_row<BX>(x, sc, ((size_t)n * nbx + b0 + blk) * S + ((size_t)mz[a] * H + my[bb]) * W + mx[c], bwx, r);
+                if (gp.G) {
+#pragma unroll
+                    for (int k = 0; k < 32; k++) if (k < kmax) r[k] = d_act_ab(r[k], ca[k], cb[k]);
+                }
+#pragma unroll
+                for (int k = 0; k < 32; k++) acc[k] = fmaf(w3, r[k], acc[k]);
+            }
+    store_row<BY, true>(y, mx_scp<BY>(y, N, Cy, So), (size_t)nbk * So + vo, bwy, acc);
+}
+static void up2_launch(const void *x, int xdt, shape5 xs, int b0, int Cy, void *y, int ydt, gnp_t gp, const char *who) {
+    if ((xdt != 3 && xdt != 4) || (ydt != 3 && ydt != 4)) mi_die("%s: dtypes %d -> %d are not MX", who, xdt, ydt);
+    if (gp.G && (gp.ns || xs.c % gp.G)) mi_die("%s: GroupNorm of %d channels in %d groups (slab-local statistics are not supported)", who, xs.c, gp.G);
+    const size_t So = 8 * (size_t)xs.d * xs.h * xs.w;
+    if (!So || !xs.n) return;
+    const dim3 grid(nblk_(So, 256), (unsigned)(xs.n * mx_nb(Cy)));
+    const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
+#define U2(BX, BY) up2_mx_k<BX, BY><<<grid, 256>>>(xq, yq, xs.n, xs.c, b0, Cy, xs.d, xs.h, xs.w, gp)
+    if (xdt == 4) { if (ydt == 4) U2(4, 4); else U2(4, 8); } else { if (ydt == 4) U2(8, 4); else U2(8, 8); }
+#undef U2
+    MICK();
+}
+extern "C" void lp_up2_fwd_mx(const void *x, int xdt, shape5 xs, void *y, int ydt, gnp_t gp) { up2_launch(x, xdt, xs, 0, xs.c, y, ydt, gp, "lp_up2_fwd_mx"); }
+extern "C" void lp_up2_fwd_mx_blocks(const void *x, int xdt, shape5 xs, int b0, int nbk, void *y, int ydt) {
+    if (mx_bw(xs.c) != 32 || b0 < 0 || b0 + nbk > mx_nb(xs.c)) mi_die("lp_up2_fwd_mx_blocks: blocks %d + %d of %d channels", b0, nbk, xs.c);
+    gnp_t g0 = gnp_mk(nullptr, nullptr, nullptr, nullptr, 0);
+    up2_launch(x, xdt, xs, b0, 32 * nbk, y, ydt, g0, "lp_up2_fwd_mx_blocks");
+}
+
+// ---- y += x (src/lp_mx_gn.cu:134-150) ----
+template <int B> __global__ void __launch_bounds__(256) add_mx_k(uint8_t *y, const uint8_t *x, int N, int C, size_t S) {
+    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (i >= (size_t)N * mx_nb(C) * S) return;
+    const int bw = mx_bw(C);
+    float a[32], b[32];
+    load_row<B>(y, mx_scp<B>(y, N, C, S), i, bw, a); load_row<B>(x, mx_scp<B>(x, N, C, S), i, bw, b);
+#pragma unroll
+    for (int k = 0; k < 32; k++) a[k] += b[k];
+    store_row<B, true>(y, mx_scp<B>(y, N, C, S), i, bw, a);
+}
+extern "C" void lp_add_mx(void *y, const void *x, shape5 s, int dt, unsigned sr) {
+    if (sr) mi_die("lp_add_mx: stochastic rounding (sr %u) belongs to training and is not built here", sr);
+    const size_t rows = (size_t)s.n * mx_nb(s.c) * s.d * s.h * s.w; if (!rows) return;
+    if (dt == 4) add_mx_k<4><<<nblk_(rows, 256), 256>>>((uint8_t *)y, (const uint8_t *)x, s.n, s.c, (size_t)s.d * s.h * s.w);
+    else add_mx_k<8><<<nblk_(rows, 256), 256>>>((uint8_t *)y, (const uint8_t *)x, s.n, s.c, (size_t)s.d * s.h * s.w);
+    MICK();
+}
+
+// ---- GroupNorm (sum, sum of squares) of a stored MX tensor into fixed-point slots (src/lp_mx_gnsums.cu:8-101) ----
+// A block reduces a slab of voxels of one (n, channel block): per-thread fp64 partials per channel, a tree over the block in LDS
+// (fixed order: deterministic), one slot add per channel group touched.
+template <int B>
+__global__ void __launch_bounds__(256) gn_sums_mx_k(const uint8_t *x, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1, int n0) {
+    const int bw = mx_bw(C), nb = mx_nb(C), cpg = C / G, blk = blockIdx.y, n = n0 + (int)blockIdx.z, nsl = gridDim.x;
+    size_t q0 = v0 + (v1 - v0) * blockIdx.x / nsl, q1 = v0 + (v1 - v0) * (blockIdx.x + 1) / nsl;
+    const uint8_t *sc = mx_scp<B>(x, N, C, S);
+    double s1[32], s2[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) { s1[k] = 0.0; s2[k] = 0.0; }
+    for (size_t q = q0 + threadIdx.x; q < q1; q += 256) {
+        float r[32];
+        load_row<B>(x, sc, ((size_t)n * nb + blk) * S + q, bw, r);
+#pragma unroll
+        for (int k = 0; k < 32; k++) { const double d = (double)r[k]; s1[k] += d; s2[k] += d * d; }
+    }
+    __shared__ double red[256];
+    for (int k = 0; k < bw; k++) {
+        const int c = blk * bw + k; if (c >= C) break;
+        for (int pass = 0; pass < 2; pass++) {
+            red[threadIdx.x] = pass ? s2[k] : s1[k];
+            __syncthreads();
+            for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) red[threadIdx.x] += red[threadIdx.x + st]; __syncthreads(); }
+            if (threadIdx.x == 0) gn_acc_add(sums, 2 * ((size_t)n * G + c / cpg) + pass, red[0]);
+            __syncthreads();
+        }
+    }
+}
+extern "C" int lp_gn_sums_mx_n(const void *x, int xdt, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1, int n0, int cnt) {
+    if ((xdt != 3 && xdt != 4) || G <= 0 || C % G) return -1;
+    if (v1 <= v0 || cnt <= 0) return 0;
+    size_t nsl = (v1 - v0 + 4095) / 4096; if (nsl > 1024) nsl = 1024;
+    const dim3 grid((unsigned)nsl, (unsigned)mx_nb(C), (unsigned)cnt);
+    if (xdt == 4) gn_sums_mx_k<4><<<grid, 256>>>((const uint8_t *)x, N, C, G, S, sums, v0, v1, n0);
+    else gn_sums_mx_k<8><<<grid, 256>>>((const uint8_t *)x, N, C, G, S, sums, v0, v1, n0);
+    MICK();
+    return 0;
+}
+extern "C" int lp_gn_sums_mx(const void *x, int xdt, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1) {
+    return lp_gn_sums_mx_n(x, xdt, N, C, G, S, sums, v0, v1, 0, N);
+}
+
+// ---- 1x1x1 head (src/lp_mx_conv1.cu:5-21): y[n][co][v] = b[co] + sum_ci w[co][ci] act(x[ci][v]), fp32 FMA in ci order ----
+// Thread per voxel; weights, bias and the GN coefficients of the sample staged in LDS once per block; CO outputs per pass in registers.
+template <int B, int CO, typename YT>
+__global__ void __launch_bounds__(256) conv1_mx_k(const uint8_t *x, const float *w, const float *b, YT *y, int N, int Ci, size_t S, gnp_t gp, int Co, int co0,
+                                                  size_t vb, size_t nv, size_t ly) {
+    extern __shared__ float c1s[];          // [CO][Ci] weights, [CO] bias, [Ci] a, [Ci] b
+    float *sw = c1s, *sb = sw + CO * Ci, *sa = sb + CO, *sbb = sa + Ci;
+    const int n = blockIdx.y, bw = mx_bw(Ci), nb = mx_nb(Ci);
+    for (int i = threadIdx.x; i < CO * Ci; i += 256) { const int co = co0 + i / Ci; sw[i] = co < Co ? w[(size_t)co * Ci + i % Ci] : 0.f; }
+    for (int i = threadIdx.x; i < CO; i += 256) sb[i] = b && co0 + i < Co ? b[co0 + i] : 0.f;
+    for (int i = threadIdx.x; i < Ci; i += 256) {
+        float a = 1.f, bb = 0.f;
+        if (gp.G) { const int ng = n * gp.G + i / (Ci / gp.G); a = gp.rstd[ng] * gp.gamma[i]; bb = fmaf(-gp.mean[ng], a, gp.beta[i]); }
+        sa[i] = a; sbb[i] = bb;
+    }
+    __syncthreads();
+    const size_t vi = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (vi >= nv) return;
+    const size_t v = vb + vi;
+    float acc[CO];
+#pragma unroll
+    for (int co = 0; co < CO; co++) acc[co] = sb[co];
+    const uint8_t *sc = mx_scp<B>(x, N, Ci, S);
+    for (int blk = 0; blk < nb; blk++) {
+        float r[32];
+        load_row<B>(x, sc, ((size_t)n * nb + blk) * S + v, bw, r);
+#pragma unroll
+        for (int k = 0; k < 32; k++) {
+            const int ci = blk * bw + k;
+            if (k < bw && ci < Ci) {
+                const float xv = gp.G ? d_act_ab(r[k], sa[ci], sbb[ci]) : r[k];
+#pragma unroll
+                for (int co = 0; co < CO; co++) acc[co] = fmaf(sw[co * Ci + ci], xv, acc[co]);
+            }
+        }
+    }
+#pragma unroll
+    for (int co = 0; co < CO; co++) if (co0 + co < Co) {
+        const size_t o = ((size_t)n * Co + co0 + co) * ly + vi;
+        if (sizeof(YT) == 2) ((__half *)y)[o] = __float2half(acc[co]); else ((float *)y)[o] = acc[co];
+    }
+}
+template <typename YT>
+static void conv1_launch(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, YT *y, gnp_t gp, size_t vb, size_t nv, size_t ly, const char *who) {
+    if (xdt != 3 && xdt != 4) mi_die("%s: input dtype %d is not MX", who, xdt);
+    if (gp.G && (gp.ns || xs.c % gp.G)) mi_die("%s: GroupNorm of %d channels in %d groups (slab-local statistics are not supported)", who, xs.c, gp.G);
+    if (xs.c > 1024) mi_die("%s: %d input channels (at most 1024)", who, xs.c);
+    const size_t S = (size_t)xs.d * xs.h * xs.w;
+    if (!nv || !xs.n) return;
+    const dim3 grid(nblk_(nv, 256), (unsigned)xs.n);
+    const uint8_t *xq = (const uint8_t *)x;
+    for (int co0 = 0; co0 < cout; co0 += 8) {
+        const int rem = cout - co0;
+        const size_t sm = ((size_t)8 * xs.c + 8 + 2 * (size_t)xs.c) * sizeof(float);
+#define C1(B, CO) conv1_mx_k<B, CO, YT><<<grid, 256, sm>>>(xq, w, b, y, xs.n, xs.c, S, gp, cout, co0, vb, nv, ly)
+        if (xdt == 4) { if (rem >= 8) C1(4, 8); else if (rem >= 4) { C1(4, 4); co0 -= 4; } else if (rem >= 2) { C1(4, 2); co0 -= 6; } else { C1(4, 1); co0 -= 7; } }
+        else { if (rem >= 8) C1(8, 8); else if (rem >= 4) { C1(8, 4); co0 -= 4; } else if (rem >= 2) { C1(8, 2); co0 -= 6; } else { C1(8, 1); co0 -= 7; } }
+#undef C1
+    }
+    MICK();
+}
+extern "C" void lp_conv1_fwd_mx(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, float *y, gnp_t gp) {
+    const size_t S = (size_t)xs.d * xs.h * xs.w; conv1_launch<float>(x, xdt, xs, w, b, cout, y, gp, 0, S, S, "lp_conv1_fwd_mx");
+}
+extern "C" void lp_conv1_fwd_mx_h16(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, void *y, gnp_t gp) {
+    const size_t S = (size_t)xs.d * xs.h * xs.w; conv1_launch<__half>(x, xdt, xs, w, b, cout, (__half *)y, gp, 0, S, S, "lp_conv1_fwd_mx_h16");
+}
+extern "C" void lp_conv1_fwd_mx_h16_r(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, void *y, gnp_t gp, size_t vb, size_t nv) {
+    conv1_launch<__half>(x, xdt, xs, w, b, cout, (__half *)y, gp, vb, nv, nv, "lp_conv1_fwd_mx_h16_r");
+}
+extern "C" int lp_conv1_fwd_mx_r(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, float *y, gnp_t gp, size_t vb, size_t nv, size_t ly) {
+    conv1_launch<float>(x, xdt, xs, w, b, cout, y, gp, vb, nv, ly ? ly : nv, "lp_conv1_fwd_mx_r");
+    return 1;
+}
+
+// ---- operand re-staging for the conv dispatch (the arithmetic of src/lp_f8fwd.cuh:88-113 applied once per tensor instead of once per
+// staged halo position): any source (planes or MX) -> optional GN + SiLU (staging form) -> rows in the compute format, blocks of 32 ----
+template <int BX, int BY, typename TI>
+__global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0) {
+    // y: an MX tensor of nbo * 32 channels (bw 32). gp over Cg channels of which this tensor holds [cg0, cg0 + C) (whole-input GroupNorm of a split input)
+    const int nbo = (C + 31) / 32, bwx = mx_bw(C), Cy = nbo * 32;
+    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (i >= (size_t)N * nbo * S) return;
+    const size_t v = i % S; const int blk = (int)((i / S) % nbo), n = (int)(i / (S * nbo));
+    float r[32];
+    if (BX != 0) {
+        const uint8_t *x = (const uint8_t *)xv; const uint8_t *sc = mx_scp<BX ? BX : 8>(x, N, C, S);
+        if (bwx == 32) load_row<BX ? BX : 8>(x, sc, ((size_t)n * mx_nb(C) + blk) * S + v, 32, r);
+        else load_row<BX ? BX : 8>(x, sc, (size_t)n * S + v, bwx, r);           // C <= 16: one narrow block, zero-extended
+    } else {
+#pragma unroll
+        for (int k = 0; k < 32; k++) { const int c = blk * 32 + k; r[k] = c < C ? ldx((const TI *)xv, ((size_t)n * C + c) * S + v) : 0.f; }
+    }
+    if (gp.G) {
+        const int cpg = Cg / gp.G;
+#pragma unroll
+        for (int k = 0; k < 32; k++) {
+            const int c = blk * 32 + k;
+            if (c < C) { const int ng = n * gp.G + (cg0 + c) / cpg; const float a = gp.rstd[ng] * gp.gamma[cg0 + c], b = fmaf(-gp.mean[ng], a, gp.beta[cg0 + c]); r[k] = d_act_ab(r[k], a, b); }
+            else r[k] = 0.f;
+        }
+    }
+    store_row<BY, false>(y, mx_scp<BY>(y, N, Cy, S), i, 32, r);
+}
+void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits) {
+    const size_t n = (size_t)N * ((C + 31) / 32) * S; if (!n) return;
+#define RS(BX, BY, TI) restage_k<BX, BY, TI><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, N, C, S, gp, Cg, cg0)
+#define RS_Y(BX, TI) do { if (ybits == 4) RS(BX, 4, TI); else RS(BX, 8, TI); } while (0)
+    if (xdt == 4) RS_Y(4, float); else if (xdt == 3) RS_Y(8, float); else if (xdt == 2) RS_Y(0, __half); else if (xdt == 1) RS_Y(0, bf16_t); else RS_Y(0, float);
+#undef RS_Y
+#undef RS
+    MICK();
+}
+// decoder up segment (src/lp_common.cuh:618-670): coarse rows -> GN + SiLU -> e4m3 rows with a row scale (amax ignoring NaN) -> 8-term fp32
+// blend (weights .75 / .25, fma order z, y, x, the row scale folded into the weight) -> rows in the compute format at the fine resolution
+template <int BX, int BY>
+__global__ void __launch_bounds__(256) restage_up_k(const uint8_t *x, uint8_t *y, int N, int C, int D, int H, int W, gnp_t gp, int Cg) {
+    // x: C channels at (D/2, H/2, W/2); y: nbo * 32 channels at (D, H, W)
+    const int nbo = (C + 31) / 32, bwx = mx_bw(C), Cy = nbo * 32, Dc = D >> 1, Hc = H >> 1, Wc = W >> 1;
+    const size_t S = (size_t)D * H * W, Sc = (size_t)Dc * Hc * Wc;
+    const int nbk = blockIdx.y, n = nbk / nbo, blk = nbk % nbo;
+    __shared__ float ca[32], cb[32]; __shared__ int cg[32];
+    if (threadIdx.x < 32) {
+        const int k = threadIdx.x, c = blk * 32 + k;
+        float a = 1.f, b = 0.f; int g = 0;
+        if (gp.G && c < C) { const int ng = n * gp.G + c / (Cg / gp.G); a = gp.rstd[ng] * gp.gamma[c]; b = fmaf(-gp.mean[ng], a, gp.beta[c]); g = 1; }
+        ca[k] = a; cb[k] = b; cg[k] = g;
+    }
+    __syncthreads();
+    const size_t vo = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
+    if (vo >= S) return;
+    const int gx = (int)(vo % W), gy = (int)((vo / W) % H), gz = (int)(vo / ((size_t)W * H));
+    const int mz[2] = {gz >> 1, min(max((gz >> 1) + ((gz & 1) ? 1 : -1), 0), Dc - 1)}, my[2] = {gy >> 1, min(max((gy >> 1) + ((gy & 1) ? 1 : -1), 0), Hc - 1)},
+              mx[2] = {gx >> 1, min(max((gx >> 1) + ((gx & 1) ? 1 : -1), 0), Wc - 1)};
+    const uint8_t *sc = mx_scp<BX>(x, N, C, Sc);
+    float acc[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) acc[k] = 0.f;
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int bb = 0; bb < 2; bb++)
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                float r[32];
+                const size_t cv = ((size_t)mz[a] * Hc + my[bb]) * Wc + mx[c];
+                if (bwx == 32) load_row<BX>(x, sc, ((size_t)n * mx_nb(C) + blk) * Sc + cv, 32, r); else load_row<BX>(x, sc, (size_t)n * Sc + cv, bwx, r);
+#pragma unroll
+                for (int k = 0; k < 32; k++) if (cg[k]) r[k] = d_act_ab(r[k], ca[k], cb[k]);
+                unsigned am = 0u;
+#pragma unroll
+                for (int k = 0; k < 32; k++) { const unsigned u = __float_as_uint(fabsf(r[k])); am = u <= 0x7f800000u && u > am ? u : am; }
+                const int e = d_mx_exp(__uint_as_float(am), MI_INVQ8);
+                const float m = d_exp2i(-e);
+                const float w3 = (a ? 0.25f : 0.75f) * (bb ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f) * d_mx_scale((unsigned)(e + 127));
+#pragma unroll
+                for (int k = 0; k < 32; k++) acc[k] = fmaf(w3, d_dec_e4m3(d_enc_e4m3(r[k] * m)), acc[k]);
+            }
+    store_row<BY, false>(y, mx_scp<BY>(y, N, Cy, S), (size_t)nbk * S + vo, 32, acc);
+}
+void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits) {
+    const size_t S = (size_t)D * H * W; if (!S || !N) return;
+    const dim3 grid(nblk_(S, 256), (unsigned)(N * ((C + 31) / 32)));
+    const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
+#define RU(BX, BY) restage_up_k<BX, BY><<<grid, 256>>>(xq, yq, N, C, D, H, W, gp, Cg)
+    if (xdt == 4) { if (ybits == 4) RU(4, 4); else RU(4, 8); } else if (xdt == 3) { if (ybits == 4) RU(8, 4); else RU(8, 8); }
+    else mi_die("fused-upsample input must be an MX tensor (dtype %d)", xdt);
+#undef RU
+    MICK();
+}

@@ -1,0 +1,101 @@
+// Runtime shim of the library: device selection, memory, error latch, per-device scratch, events, GroupNorm finalize.
+// These stand in for what the reference's lp_* units take from its op layer (src/nn.h:34-48, src/nn_core.cu:244-290, :751).
+#include "mx_dev.hpp"
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+static thread_local hipError_t g_err = hipSuccess;      // first error since the last lp_check (src/lp_common.cuh:35-38)
+static thread_local char g_errmsg[256];
+void mi_post_error(hipError_t e, const char *file, int line) {
+    if (g_err != hipSuccess) return;
+    g_err = e;
+    snprintf(g_errmsg, sizeof g_errmsg, "%s (%s:%d)", hipGetErrorString(e), file, line);
+}
+[[noreturn]] void mi_die(const char *fmt, ...) {
+    va_list ap; va_start(ap, fmt); vfprintf(stderr, fmt, ap); va_end(ap); fputc('\n', stderr); fflush(stderr);
+    abort();
+}
+extern "C" const char *lp_check(void) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) mi_post_error(e, __FILE__, __LINE__);
+    if (g_err == hipSuccess) return nullptr;
+    g_err = hipSuccess;
+    return g_errmsg;
+}
+extern "C" int mi_device_count(void) { int n = 0; if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; } return n; }
+extern "C" int mi_init(int device) {
+    int n = mi_device_count();
+    if (device < 0 || device >= n) { fprintf(stderr, "mi_init: no HIP device %d (%d visible): the MX kernels need a gfx950 GPU\n", device, n); return 1; }
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, device) != hipSuccess) return 2;
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0) { fprintf(stderr, "mi_init: device %d is %s, this library is built for gfx950 only\n", device, p.gcnArchName); return 3; }
+    return hipSetDevice(device) == hipSuccess ? 0 : 4;
+}
+extern "C" void *mi_malloc(size_t bytes) {
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    if (e != hipSuccess) mi_die("mi_malloc: %zu bytes: %s", bytes, hipGetErrorString(e));
+    return p;
+}
+extern "C" void mi_free(void *p) { if (p) MIRT(hipFree(p)); }
+__global__ void fill_u32_k(unsigned *p, size_t n, unsigned v) { size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; if (i < n) p[i] = v; }
+extern "C" void mi_zero(void *p, size_t bytes) { MIRT(hipMemsetAsync(p, 0, bytes, 0)); }
+extern "C" void mi_h2d(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice)); }
+extern "C" void mi_d2h(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost)); }
+extern "C" void mi_d2d(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, 0)); }
+extern "C" void mi_sync(void) { MIRT(hipDeviceSynchronize()); }
+
+// per-device scratch: grow on demand, contents valid until the next request of the same slot on the same device
+static void *g_ws[8][MI_WS_NSLOTS]; static size_t g_wscap[8][MI_WS_NSLOTS];
+void *mi_ws(int slot, size_t bytes) {
+    int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
+    if (bytes > g_wscap[d][slot]) {
+        if (g_ws[d][slot]) { MIRT(hipDeviceSynchronize()); MIRT(hipFree(g_ws[d][slot])); }
+        const size_t cap = bytes + bytes / 8 + 4096;
+        hipError_t e = hipMalloc(&g_ws[d][slot], cap);
+        if (e != hipSuccess) mi_die("mi_ws: slot %d, %zu bytes: %s", slot, cap, hipGetErrorString(e));
+        g_wscap[d][slot] = cap;
+    }
+    return g_ws[d][slot];
+}
+extern "C" void mi_ws_release(void) {
+    int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
+    MIRT(hipDeviceSynchronize());
+    for (int s = 0; s < MI_WS_NSLOTS; s++) { if (g_ws[d][s]) MIRT(hipFree(g_ws[d][s])); g_ws[d][s] = nullptr; g_wscap[d][s] = 0; }
+    lp_wmemo_clear();
+}
+
+// events on the null stream
+extern "C" void *mi_event_create(void) { hipEvent_t e; if (hipEventCreate(&e) != hipSuccess) return nullptr; return (void *)e; }
+extern "C" void mi_event_record(void *ev) { MIRT(hipEventRecord((hipEvent_t)ev, 0)); }
+extern "C" float mi_event_elapsed_ms(void *ev0, void *ev1) { float ms = 0.f; MIRT(hipEventSynchronize((hipEvent_t)ev1)); MIRT(hipEventElapsedTime(&ms, (hipEvent_t)ev0, (hipEvent_t)ev1)); return ms; }
+extern "C" void mi_event_destroy(void *ev) { if (ev) MIRT(hipEventDestroy((hipEvent_t)ev)); }
+
+// ---- GroupNorm sum slots (src/gnacc.cuh): [lo: 2^-64 units][hi: integer part, two's complement][count of non-finite adds] ----
+__device__ __forceinline__ double gn_slot_get(const double *b, size_t i) {
+    const unsigned long long *w = (const unsigned long long *)b + 3 * i;
+    if (w[2]) return __longlong_as_double(0x7ff8000000000000ll);
+    return (double)(long long)w[1] + (double)w[0] * 5.42101086242752217e-20;
+}
+__global__ void gn_finalize_k(const double *sums, int NG, size_t len, float eps, float *mean, float *rstd) {   // src/nn_elem.cu:5-11
+    const int ng = blockIdx.x * blockDim.x + threadIdx.x;
+    if (ng >= NG) return;
+    const double m = gn_slot_get(sums, 2 * ng) / (double)len, v = gn_slot_get(sums, 2 * ng + 1) / (double)len - m * m;
+    mean[ng] = (float)m;
+    rstd[ng] = (float)(1.0 / sqrt((v > 0 ? v : 0) + (double)eps));
+}
+extern "C" void mi_gn_finalize(const double *sums, int NG, size_t len, float eps, float *mean, float *rstd) {
+    gn_finalize_k<<<nblk_(NG, 64), 64>>>(sums, NG, len, eps, mean, rstd); MICK();
+}
+__global__ void gn_get_k(const double *sums, int n, double *out) { const int i = blockIdx.x * blockDim.x + threadIdx.x; if (i < n) out[i] = gn_slot_get(sums, i); }
+extern "C" void mi_gn_sums_get(const double *sums, int nslots, double *out) { gn_get_k<<<nblk_(nslots, 64), 64>>>(sums, nslots, out); MICK(); }
+extern "C" void mi_gn_sums_zero(double *sums, int nslots) {
+    const size_t n = (size_t)nslots * 6;   // 24 bytes = 6 words
+    fill_u32_k<<<nblk_(n, 256), 256>>>((unsigned *)sums, n, 0u); MICK();
+}
+extern "C" gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean, const float *rstd, int G) {   // src/nn_lp.h:19
+    gnp_t g; memset(&g, 0, sizeof g); g.gamma = gamma; g.beta = beta; g.mean = mean; g.rstd = rstd; g.G = G; return g;
+}
+extern "C" int lp_gn_slab_any(void) { return 0; }

@@ -1,0 +1,162 @@
+"""ctypes mirror of include/mi_lp.h (the forward subset of the reference's src/nn_lp.h).
+
+Everything here is plumbing: argument marshalling and device-buffer helpers. All arithmetic happens in the HIP library.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libufsm_lp.so")
+MI_GN_SLOT_BYTES = 24
+
+
+class shape5(C.Structure):  # src/nn.h:21
+    _fields_ = [("n", C.c_int), ("c", C.c_int), ("d", C.c_int), ("h", C.c_int), ("w", C.c_int)]
+
+
+class gnp_t(C.Structure):  # src/nn_lp.h:15
+    _fields_ = [("gamma", C.c_void_p), ("beta", C.c_void_p), ("mean", C.c_void_p), ("rstd", C.c_void_p),
+                ("G", C.c_int), ("zs", C.c_int), ("zo", C.c_int), ("ns", C.c_int), ("zhw", C.c_int)]
+
+
+class split_t(C.Structure):  # src/nn_lp.h:32
+    _fields_ = [("x2", C.c_void_p), ("c_split", C.c_int), ("y2", C.c_void_p), ("o_split", C.c_int), ("accum", C.c_int),
+                ("gp2", gnp_t), ("up", C.c_int16), ("yD", C.c_int16), ("sr", C.c_uint), ("wkey", C.c_uint),
+                ("zlo", C.c_int), ("zhi", C.c_int), ("stored_stats", C.c_int), ("osr", C.c_uint),
+                ("zi0", C.c_int16), ("Di", C.c_int16), ("o_pad", C.c_int16), ("zw0", C.c_int16), ("zw1", C.c_int16), ("yzo", C.c_int16)]
+
+
+assert C.sizeof(split_t) <= 128  # src/nn_lp.h:41
+
+_P, _I, _Z, _F = C.c_void_p, C.c_int, C.c_size_t, C.c_float
+_PROTOS = {
+    "lp_conv_fwd_f8": (_I, [_P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t]),
+    "lp_conv_fwd_f4": (_I, [_P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t]),
+    "lp_conv_fwd_s2_f8": (_I, [_P, _I, shape5, _P, _P, _I, _P, _I, shape5, gnp_t]),
+    "lp_wmemo_step": (None, [C.c_uint]),
+    "lp_wmemo_clear": (None, []),
+    "gnp_mk": (gnp_t, [_P, _P, _P, _P, _I]),
+    "lp_gn_slab_any": (_I, []),
+    "lp_mx8_bytes": (_Z, [_I, _I, _Z]),
+    "lp_mx4_bytes": (_Z, [_I, _I, _Z]),
+    "lp_f32_to_mx8": (None, [_P, _I, _I, _Z, _P]),
+    "lp_f32_to_mx4": (None, [_P, _I, _I, _Z, _P]),
+    "lp_h16_to_mx8": (None, [_P, _I, _I, _I, _Z, _P]),
+    "lp_h16_to_mx4": (None, [_P, _I, _I, _I, _Z, _P]),
+    "lp_mx8_to_f32": (None, [_P, _I, _I, _Z, _P]),
+    "lp_mx4_to_f32": (None, [_P, _I, _I, _Z, _P]),
+    "lp_pred_input_mx": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I, _I]),
+    "lp_pred_input_mx8": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I]),
+    "lp_gn_silu_apply_mx": (None, [_P, _I, shape5, _I, _P, _P, _P, _P, _P, _I]),
+    "lp_add_mx": (None, [_P, _P, shape5, _I, C.c_uint]),
+    "lp_up2_fwd_mx": (None, [_P, _I, shape5, _P, _I, gnp_t]),
+    "lp_up2_fwd_mx_blocks": (None, [_P, _I, shape5, _I, _I, _P, _I]),
+    "lp_gn_sums_mx": (_I, [_P, _I, _I, _I, _I, _Z, _P, _Z, _Z]),
+    "lp_gn_sums_mx_n": (_I, [_P, _I, _I, _I, _I, _Z, _P, _Z, _Z, _I, _I]),
+    "lp_conv1_fwd_mx": (None, [_P, _I, shape5, _P, _P, _I, _P, gnp_t]),
+    "lp_conv1_fwd_mx_h16": (None, [_P, _I, shape5, _P, _P, _I, _P, gnp_t]),
+    "lp_conv1_fwd_mx_h16_r": (None, [_P, _I, shape5, _P, _P, _I, _P, gnp_t, _Z, _Z]),
+    "lp_conv1_fwd_mx_r": (_I, [_P, _I, shape5, _P, _P, _I, _P, gnp_t, _Z, _Z, _Z]),
+    "lp_check": (C.c_char_p, []),
+    "mi_init": (_I, [_I]),
+    "mi_device_count": (_I, []),
+    "mi_malloc": (_P, [_Z]),
+    "mi_free": (None, [_P]),
+    "mi_zero": (None, [_P, _Z]),
+    "mi_h2d": (None, [_P, _P, _Z]),
+    "mi_d2h": (None, [_P, _P, _Z]),
+    "mi_d2d": (None, [_P, _P, _Z]),
+    "mi_sync": (None, []),
+    "mi_ws_release": (None, []),
+    "mi_gn_finalize": (None, [_P, _I, _Z, _F, _P, _P]),
+    "mi_gn_sums_zero": (None, [_P, _I]),
+    "mi_gn_sums_get": (None, [_P, _I, _P]),
+    "mi_event_create": (_P, []),
+    "mi_event_record": (None, [_P]),
+    "mi_event_elapsed_ms": (_F, [_P, _P]),
+    "mi_event_destroy": (None, [_P]),
+    "mi_conv_fwd_fused": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, _P, _P, _I, gnp_t, _P, _I, split_t]),
+    "mi_last_kernel": (C.c_char_p, []),
+}
+EXPORTS = tuple(_PROTOS)
+_lib = None
+
+
+def load():
+    """Load libufsm_lp.so and set the prototypes. Raises if the library is not built: there is no fallback path."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError("%s is not built: run `python -c 'import __graft_entry__ as g; g.build()'` (hipcc, gfx950)" % LIB_PATH)
+    L = C.CDLL(LIB_PATH)
+    for name, (res, args) in _PROTOS.items():
+        f = getattr(L, name)  # AttributeError names the missing symbol
+        f.restype = res
+        f.argtypes = args
+    _lib = L
+    return L
+
+
+class _Lazy:
+    def __getattr__(self, k):
+        return getattr(load(), k)
+
+
+lib = _Lazy()
+
+
+class DevBuf:
+    """A device allocation owned by the caller (mi_malloc / mi_free), with numpy copies in and out."""
+
+    def __init__(self, nbytes, zero=True):
+        self.nbytes = int(nbytes)
+        self.ptr = lib.mi_malloc(max(self.nbytes, 1))
+        if zero and self.nbytes:
+            lib.mi_zero(self.ptr, self.nbytes)
+
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.ascontiguousarray(a)
+        b = cls(a.nbytes, zero=False)
+        if a.nbytes:
+            lib.mi_h2d(b.ptr, a.ctypes.data, a.nbytes)
+        return b
+
+    def to_numpy(self, dtype, shape=None):
+        lib.mi_sync()
+        out = np.empty(self.nbytes // np.dtype(dtype).itemsize, dtype=dtype)
+        if self.nbytes:
+            lib.mi_d2h(out.ctypes.data, self.ptr, out.nbytes)
+        return out.reshape(shape) if shape is not None else out
+
+    def free(self):
+        if self.ptr:
+            lib.mi_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class LP:
+    """Thin Python mirror of the lp_* entry points (argument meaning as in src/nn_lp.h)."""
+
+    @staticmethod
+    def gn(gamma=None, beta=None, mean=None, rstd=None, G=0):
+        g = gnp_t()
+        if G:
+            g.gamma, g.beta, g.mean, g.rstd, g.G = gamma.ptr, beta.ptr, mean.ptr, rstd.ptr, G
+        return g
+
+    @staticmethod
+    def check():
+        lib.mi_sync()
+        e = lib.lp_check()
+        if e:
+            raise RuntimeError("HIP error: " + e.decode())
