@@ -13,8 +13,8 @@
 //     ds_read_b128 per K block at a per-lane address (position of the lane's voxel + the tap's offset): no im2col.
 //   * Each wavefront owns NT voxel tiles of 32 (2 rows x 16 x) and all MT channel tiles of 32 of the workgroup: MT x NT
 //     accumulators of 32x32 (16 VGPRs each), every weight fragment reused NT times and every input fragment MT times.
-//   * Weights are prepared once per call (or memoised) in fragment order, streamed L2 -> LDS through a 3-slot ring, one
-//     barrier per K pair; the fragments of pair q+1 are fetched from LDS while the MFMAs of pair q run.
+//   * Weights are prepared once per call (or memoised) in fragment order, streamed L2 -> LDS through a 2-slot ring, one
+//     barrier per K pair; two workgroups share a CU, so one's MFMAs cover the other's LDS latency, staging and epilogue.
 //   * Epilogue (src/lp_common.cuh:1465-1597): bias -> optional affine + activation -> per (voxel, 32-channel block) amax across
 //     the lane pair (l, l^32) -> E8M0 exponent -> e4m3 / e2m1 codes -> 16-byte row halves stored coalesced along x,
 //     GroupNorm (sum, sum of squares) reduced in a fixed order and added to exact fixed-point slots.
@@ -43,7 +43,7 @@ struct conv_args {
     const uint8_t *wq, *wsc; int nmt_all;
     const float *bias; int Co;
     void *y; int ydt;
-    double *osum; int Go, stored_stats, zs0, zs1;
+    double *osum; float *part; int Go, stored_stats, zs0, zs1;   // part: per tile and channel quad (sum, sum of squares)
     const float *ep_a, *ep_b; int act;
     int ntx, nty, ntz, ncs; unsigned ntiles;
 };
@@ -55,21 +55,21 @@ template <> struct fmt_t<4> { static constexpr int RB = 16, NH = 1, WTILE = 1024
 __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678f)); }
 
 template <int FMT, int STRIDE, int MT, int NT>
-__global__ void __launch_bounds__(256, 1) conv3_mx_k(const conv_args a) {
+__global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     constexpr int TZ = NT == 2 ? 2 : 4;
     constexpr int HZ = STRIDE * (TZ - 1) + 3, HY = STRIDE * 7 + 3, HX = STRIDE * 15 + 3, TT = HZ * HY * HX;
-    constexpr int RB = fmt_t<FMT>::RB, NH = fmt_t<FMT>::NH, WTILE = fmt_t<FMT>::WTILE;
-    constexpr int STG = MT * (WTILE + 64);
+    constexpr int NH = fmt_t<FMT>::NH, WTILE = fmt_t<FMT>::WTILE;
+    constexpr int STG = MT * (WTILE + 256);              // one weight stage: MT tiles of codes, then MT x 64 scale words
+    constexpr int UPT = (MT * WTILE / 16 + 255) / 256;   // 16-byte weight units per thread and stage
     extern __shared__ __align__(16) unsigned char lds[];
-    // LDS: [3 weight slots][act data CB * NH * TT * 16][act scales CB * TT]
-    unsigned char *wring = lds;
-    unsigned char *act = lds + 3 * STG;
-    unsigned char *asc = act + (size_t)a.CB * NH * TT * 16;
+    // LDS: [2 weight stages][pair table (npairs + 2) x 2 x 16 B][halo rows CB * NH * TT * 16 B][halo scales CB * TT words]
+    const int tab_bytes = (((27 * a.CB + 1) >> 1) + 2) * 32;
+    const unsigned wring_o = 0, tab_o = 2 * STG, act_o = tab_o + tab_bytes, asc_o = act_o + a.CB * NH * TT * 16;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
 
     // XCD-aware tile order: consecutive workgroup ids land on different XCDs (8, round robin), so give each XCD a contiguous
     // range of tiles: neighbouring tiles (shared halo, same weights) then share one L2
-    unsigned tile = blockIdx.x;
+    unsigned tile;
     {
         const unsigned per = (a.ntiles + 7u) / 8u;
         tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
@@ -86,9 +86,15 @@ __global__ void __launch_bounds__(256, 1) conv3_mx_k(const conv_args a) {
     // the lane's voxel in each of its NT tiles: wave -> (z, y half) for TZ 2, z for TZ 4; tile j -> rows 2j, 2j+1; r -> (row, x)
     int lz, ly0;
     if (NT == 2) { lz = wave >> 1; ly0 = (wave & 1) * 4; } else { lz = wave; ly0 = 0; }
-    int p0[NT];
+    unsigned ab[NT], sbse[NT];     // LDS byte addresses of the lane's halo row (its 16-byte half) and scale word for tap (0, 0, 0) of block 0
 #pragma unroll
-    for (int j = 0; j < NT; j++) p0[j] = ((STRIDE * lz) * HY + STRIDE * (ly0 + 2 * j + (r >> 4))) * HX + STRIDE * (r & 15);
+    for (int j = 0; j < NT; j++) {
+        const int p0 = ((STRIDE * lz) * HY + STRIDE * (ly0 + 2 * j + (r >> 4))) * HX + STRIDE * (r & 15);
+        ab[j] = act_o + ((NH == 2 ? h * TT : 0) + p0) * 16;
+        sbse[j] = asc_o + p0 * 4;
+    }
+    const unsigned wfa = wring_o + lane * 16, wfs = wring_o + MT * WTILE + lane * 4;    // the lane's weight fragment / scale word in stage slot 0, tile 0
+    const unsigned wcp = wring_o + (tid * UPT * 16) % (MT * WTILE), wcs = wring_o + MT * WTILE + (tid * 4) % (MT * 256);   // the thread's part of a stage copy
 
     v16f acc[MT][NT];
 #pragma unroll
@@ -99,117 +105,145 @@ __global__ void __launch_bounds__(256, 1) conv3_mx_k(const conv_args a) {
             for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
 
     const size_t Sin = (size_t)a.D * a.H * a.W;
-    const uint8_t *wq_cs = a.wq + (size_t)cs * MT * WTILE, *wsc_cs = a.wsc + (size_t)cs * MT * 64;
-    const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 64;
-    constexpr int NLD = (MT * WTILE / 16 + 255) / 256;   // 16-byte weight units per thread and stage
+    const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 256;
     int pair0 = 0;                                       // global pair index of the chunk's first pair
 
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) {
         const int nbc = min(a.CB, a.nbt - b0), nunits = 27 * nbc, npairs = (nunits + 1) >> 1;
         __syncthreads();                                 // the previous chunk's readers are done with the halo
-        // ---- stage the halo of blocks [b0, b0 + nbc): rows copied as stored, zero rows (scale byte 1) outside the tensor ----
-        for (int i = tid; i < nbc * TT * NH; i += 256) {
-            const int bl = i / (TT * NH), rem = i - bl * (TT * NH), pos = rem / NH, hf = rem - pos * NH;
-            const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
-            const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
-            const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
-            v4i val = {0, 0, 0, 0};
-            if (gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && blk < a.nbs[seg]) {
-                const int rb = a.bws[seg] * FMT / 8;     // stored row bytes (32-wide blocks: RB)
-                const size_t row = ((size_t)n * a.nbs[seg] + blk) * Sin + ((size_t)gz * a.H + gy) * a.W + gx;
-                const uint8_t *src = a.xq[seg] + row * rb + hf * 16;
-                if (rb >= (hf + 1) * 16) val = *(const v4i *)src;
-                else if (rb - hf * 16 == 8) { const int2 t = *(const int2 *)src; val[0] = t.x; val[1] = t.y; }
-                else if (rb - hf * 16 == 4) val[0] = *(const int *)src;
+        // ---- pair table: per pair and lane half, the byte offsets of the pair's two units (fp8: both; fp4: the half's own) and of
+        // the half's scale word. unit u = (tap u / nbc, local block u % nbc); the odd padding unit (zero weights) re-reads unit A ----
+        for (int i = tid; i < (npairs + 2) * 2; i += 256) {
+            const int q = min(i >> 1, npairs - 1), hh = i & 1;
+            const int uA = 2 * q, uB = 2 * q + 1 < nunits ? 2 * q + 1 : 2 * q;
+            const int tA = uA / nbc, bA = uA - tA * nbc, tB = uB / nbc, bB = uB - tB * nbc;
+            const int pA = ((tA / 9) * HY + (tA / 3) % 3) * HX + tA % 3, pB = ((tB / 9) * HY + (tB / 3) % 3) * HX + tB % 3;
+            const int dA = (bA * NH * TT + pA) * 16, dB = (bB * NH * TT + pB) * 16, sA = (bA * TT + pA) * 4, sB = (bB * TT + pB) * 4;
+            *(v4i *)(lds + tab_o + i * 16) = (v4i){NH == 2 ? dA : (hh ? dB : dA), dB, hh ? sB : sA, 0};
+        }
+#ifndef DBG_NOSTAGE
+        // ---- stage the halo of blocks [b0, b0 + nbc): rows copied as stored, zero rows (scale byte 1) outside the tensor.
+        // Branch-free: every load reads a clamped in-tensor address and is zeroed afterwards when the position is outside;
+        // four independent loads are in flight per thread ----
+        {
+            constexpr int NB = 4;
+            const int E = nbc * TT * NH;
+            for (int i0 = tid; i0 < E; i0 += 256 * NB) {
+                v4i val[NB]; unsigned dst[NB]; bool inb[NB];
+#pragma unroll
+                for (int k = 0; k < NB; k++) {
+                    const int i = min(i0 + k * 256, E - 1);
+                    const int bl = i / (TT * NH), rem = i - bl * (TT * NH), pos = rem / NH, hf = rem - pos * NH;
+                    const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
+                    const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
+                    const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
+                    const int rb = a.bws[seg] * FMT / 8;     // stored row bytes (16 NH for 32-wide blocks)
+                    const bool pos_ok = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && blk < a.nbs[seg];
+                    const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1), cb = min(blk, a.nbs[seg] - 1);
+                    const size_t row = ((size_t)n * a.nbs[seg] + cb) * Sin + ((size_t)cz * a.H + cy) * a.W + cx;
+                    dst[k] = act_o + ((bl * NH + hf) * TT + pos) * 16;
+                    if (rb >= 16) {
+                        const bool have = rb >= (hf + 1) * 16;
+                        val[k] = *(const v4i *)(a.xq[seg] + row * rb + (have ? hf * 16 : 0));
+                        inb[k] = pos_ok && have;
+                    } else {                                 // 8- or 4-byte rows of a <= 8 / <= 16 channel tensor: only half 0 holds data
+                        val[k] = (v4i){0, 0, 0, 0};
+                        if (rb == 8) { const int2 t = *(const int2 *)(a.xq[seg] + row * 8); val[k][0] = t.x; val[k][1] = t.y; }
+                        else val[k][0] = *(const int *)(a.xq[seg] + row * 4);
+                        inb[k] = pos_ok && hf == 0;
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < NB; k++) *(v4i *)(lds + dst[k]) = inb[k] ? val[k] : (v4i){0, 0, 0, 0};
             }
-            *(v4i *)(act + ((size_t)(bl * NH + hf) * TT + pos) * 16) = val;
-        }
-        for (int i = tid; i < nbc * TT; i += 256) {
-            const int bl = i / TT, pos = i - bl * TT;
-            const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
-            const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
-            const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
-            unsigned char s = 1;
-            if (gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && blk < a.nbs[seg])
-                s = a.xsc[seg][((size_t)n * a.nbs[seg] + blk) * Sin + ((size_t)gz * a.H + gy) * a.W + gx];
-            asc[i] = s;
-        }
-        // ---- weight stages 0 and 1 of this chunk into ring slots 0 and 1; stage 2 into registers ----
-        v4i g[NLD]; int gs = 0;
-        auto wload = [&](int q) {       // global -> registers: stage q of this chunk
-            const uint8_t *src = wq_cs + (size_t)(pair0 + q) * wq_ps;
+            const int E2 = nbc * TT;
+            for (int i0 = tid; i0 < E2; i0 += 256 * NB) {
+                unsigned sv[NB]; unsigned dst[NB];
 #pragma unroll
-            for (int k = 0; k < NLD; k++) { const int u = tid + k * 256; if (u < MT * WTILE / 16) g[k] = *(const v4i *)(src + (size_t)u * 16); }
-            if (tid < MT * 16) gs = *(const int *)(wsc_cs + (size_t)(pair0 + q) * wsc_ps + tid * 4);
-        };
-        auto wstore = [&](int slot) {   // registers -> LDS ring slot
-            unsigned char *dst = wring + slot * STG;
+                for (int k = 0; k < NB; k++) {
+                    const int i = min(i0 + k * 256, E2 - 1);
+                    const int bl = i / TT, pos = i - bl * TT;
+                    const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
+                    const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
+                    const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
+                    const bool ok = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && blk < a.nbs[seg];
+                    const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1), cb = min(blk, a.nbs[seg] - 1);
+                    const unsigned s = a.xsc[seg][((size_t)n * a.nbs[seg] + cb) * Sin + ((size_t)cz * a.H + cy) * a.W + cx];
+                    sv[k] = ok ? s : 1u; dst[k] = asc_o + i * 4;
+                }
 #pragma unroll
-            for (int k = 0; k < NLD; k++) { const int u = tid + k * 256; if (u < MT * WTILE / 16) *(v4i *)(dst + (size_t)u * 16) = g[k]; }
-            if (tid < MT * 16) *(int *)(dst + MT * WTILE + tid * 4) = gs;
+                for (int k = 0; k < NB; k++) *(unsigned *)(lds + dst[k]) = sv[k];
+            }
+        }
+#endif
+        // ---- weight stages: global -> registers -> ring slot. Every thread moves UPT contiguous 16-byte units and one scale word per
+        // stage; offsets wrap instead of being guarded (duplicates store the same value). The prepared-weight buffers carry four
+        // stages of padding, so the loads that run ahead of the last pair stay inside them ----
+        const uint8_t *wgp = a.wq + (size_t)pair0 * wq_ps + (size_t)cs * MT * WTILE + (tid * UPT * 16) % (MT * WTILE);
+        const uint8_t *wgs = a.wsc + (size_t)pair0 * wsc_ps + (size_t)cs * MT * 256 + (tid * 4) % (MT * 256);
+        v4i g[UPT]; unsigned gs = 0;
+        auto wload = [&]() {            // the next stage in sequence
+#ifndef DBG_NOWLOAD
+#pragma unroll
+            for (int k = 0; k < UPT; k++) g[k] = *(const v4i *)(wgp + k * 16);
+            gs = *(const unsigned *)wgs;
+            wgp += wq_ps; wgs += wsc_ps;
+#endif
         };
-        wload(0); wstore(0);
-        if (npairs > 1) { wload(1); wstore(1); }
-        if (npairs > 2) wload(2);
+        auto wstore = [&](int slot) {
+#pragma unroll
+            for (int k = 0; k < UPT; k++) *(v4i *)(lds + wcp + slot * STG + k * 16) = g[k];
+            *(unsigned *)(lds + wcs + slot * STG) = gs;
+        };
+        wload(); wstore(0);
+        wload();
         __syncthreads();
 
-        // ---- K loop over unit pairs ----
-        // unit u of the chunk = (tap u / nbc, local block u % nbc); its staged rows start at position (kz HY + ky) HX + kx of block bl
-        struct uit { int kz, ky, kx, bl, u; };
-        uit it = {0, 0, 0, 0, 0};
-        auto unit_next = [&](uit &s) { s.u++; if (++s.bl == nbc) { s.bl = 0; if (++s.kx == 3) { s.kx = 0; if (++s.ky == 3) { s.ky = 0; s.kz++; } } } };
-        v8i fb[2][NT], fa[2][MT]; int sb[2][NT], sa[2][MT];
-        auto fetch = [&](int buf, int q) {      // operand fragments of pair q (units 2q, 2q + 1) into buffer buf
-            const uit A = it; unit_next(it);
-            const uit B = it.u < nunits ? it : A; unit_next(it);      // odd unit count: the padding unit (zero weights) re-reads unit A
-            const int tA = (A.kz * HY + A.ky) * HX + A.kx, tB = (B.kz * HY + B.ky) * HX + B.kx;
-            const int offS = h ? B.bl * TT + tB : A.bl * TT + tA;      // the lane's scale (and fp4 data) row: K block h
+        // ---- K loop over unit pairs, unrolled by 2 so that the ring slot (pair & 1) is static. Step of pair q: fetch its fragments
+        // from LDS (halo rows at the table's offsets, weights from ring slot q & 1), run its MFMAs, move stage q + 1 into the other
+        // slot and start loading stage q + 2 from L2. A second workgroup on the CU covers this one's LDS latency and barriers ----
+        v8i fb[NT], fa[MT]; int sb[NT], sa[MT];
+        v4i T;
+        unsigned tabp = tab_o + (lane >> 5) * 16;          // this half's entry of pair 0
+        auto fetch = [&](int slot) {
+            const v4i t = T;
 #pragma unroll
             for (int j = 0; j < NT; j++) {
+                const v4i lo = *(const v4i *)(lds + ab[j] + t[0]);
                 if (FMT == 8) {
-                    const v4i lo = *(const v4i *)(act + ((size_t)((A.bl * 2 + h) * TT) + tA + p0[j]) * 16);
-                    const v4i hi = *(const v4i *)(act + ((size_t)((B.bl * 2 + h) * TT) + tB + p0[j]) * 16);
-                    fb[buf][j] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                } else {
-                    const v4i lo = *(const v4i *)(act + ((size_t)offS + p0[j]) * 16);
-                    fb[buf][j] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                }
-                sb[buf][j] = asc[offS + p0[j]];
+                    const v4i hi = *(const v4i *)(lds + ab[j] + t[1]);
+                    fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                } else fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+                sb[j] = *(const int *)(lds + sbse[j] + t[2]);
             }
-            const unsigned char *ws = wring + (q % 3) * STG;
 #pragma unroll
             for (int m = 0; m < MT; m++) {
+                const v4i lo = *(const v4i *)(lds + wfa + slot * STG + m * WTILE);
                 if (FMT == 8) {
-                    const v4i lo = *(const v4i *)(ws + m * WTILE + lane * 16), hi = *(const v4i *)(ws + m * WTILE + 1024 + lane * 16);
-                    fa[buf][m] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                } else {
-                    const v4i lo = *(const v4i *)(ws + m * WTILE + lane * 16);
-                    fa[buf][m] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                }
-                sa[buf][m] = ws[MT * WTILE + m * 64 + lane];
+                    const v4i hi = *(const v4i *)(lds + wfa + slot * STG + m * WTILE + 1024);
+                    fa[m] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                } else fa[m] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+                sa[m] = *(const int *)(lds + wfs + slot * STG + m * 256);
             }
+            T = *(const v4i *)(lds + tabp + 32); tabp += 32;      // the next pair's table entry
         };
-        auto mma = [&](int buf) {
+        auto mma = [&]() {
+#ifndef DBG_NOMMA
 #pragma unroll
             for (int m = 0; m < MT; m++)
 #pragma unroll
                 for (int j = 0; j < NT; j++)
-                    acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[buf][m], fb[buf][j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sa[buf][m], 0, sb[buf][j]);
+                    acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[m], fb[j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sa[m], 0, sb[j]);
+#else
+            for (int m = 0; m < MT; m++) for (int j = 0; j < NT; j++) acc[m][j][0] += (float)(fa[m][0] + fb[j][0] + sa[m] + sb[j]);
+#endif
         };
-        fetch(0, 0);
+        T = *(const v4i *)(lds + tabp);
         for (int q = 0; q < npairs; q += 2) {
-            // even step: buffer 0 holds pair q
-            if (q + 1 < npairs) fetch(1, q + 1);
-            mma(0);
-            if (q + 2 < npairs) wstore((q + 2) % 3);
-            if (q + 3 < npairs) wload(q + 3);
+            fetch(0); mma(); wstore(1); wload();
             __syncthreads();
             if (q + 1 >= npairs) break;
-            // odd step: buffer 1 holds pair q + 1
-            if (q + 2 < npairs) fetch(0, q + 2);
-            mma(1);
-            if (q + 3 < npairs) wstore((q + 3) % 3);
-            if (q + 4 < npairs) wload(q + 4);
+            fetch(1); mma(); wstore(0); wload();
             __syncthreads();
         }
         pair0 += npairs;
@@ -219,7 +253,7 @@ __global__ void __launch_bounds__(256, 1) conv3_mx_k(const conv_args a) {
     // accumulator layout of the 32x32 MFMA: lane (r = voxel within the tile, h), register i -> channel (i & 3) + 4 h + 8 (i >> 2)
     const size_t So = (size_t)a.Do * a.Ho * a.Wo;
     const int co_base = cs * MT * 32;
-    float *red = (float *)lds;                      // stats scratch [4 waves][MT][8 quads][2] floats (the halo is dead now)
+    float *red = (float *)lds;                      // stats scratch [4 waves][MT][8 quads][2] floats (the ring and halo are dead now)
     const bool stats = a.osum != nullptr;
     if (stats) __syncthreads();
     float qs[MT][4], qss[MT][4];                    // per lane: sums over its voxels of the 4-channel quads (m, i >> 2)
@@ -335,17 +369,36 @@ __global__ void __launch_bounds__(256, 1) conv3_mx_k(const conv_args a) {
             }
         __syncthreads();
         if (tid < MT * 8) {
-            const int m = tid >> 3, q8 = tid & 7;                       // q8 = q4 * 2 + h
-            const int co = co_base + m * 32 + 8 * (q8 >> 1) + 4 * (q8 & 1);
-            if (co < a.Co) {
-                float s = 0.f, ss = 0.f;
-                for (int w = 0; w < 4; w++) { s += red[((w * MT + m) * 8 + q8) * 2]; ss += red[((w * MT + m) * 8 + q8) * 2 + 1]; }
-                const size_t ng = (size_t)n * a.Go + co / cpg;
-                gn_acc_add(a.osum, 2 * ng, (double)s);
-                gn_acc_add(a.osum, 2 * ng + 1, (double)ss);
-            }
+            // per tile and channel quad, the sums over the tile's voxels in wave order; a second kernel adds the tiles of a sample
+            // in a fixed order into the exact sum slots, so the statistics do not depend on the order workgroups finish in
+            const int m = tid >> 3, q8 = tid & 7;                       // q8 = q4 * 2 + h: channels co_base + 32 m + 8 q4 + 4 h .. + 3
+            float s = 0.f, ss = 0.f;
+            for (int w = 0; w < 4; w++) { s += red[((w * MT + m) * 8 + q8) * 2]; ss += red[((w * MT + m) * 8 + q8) * 2 + 1]; }
+            a.part[((size_t)tile * MT * 8 + tid) * 2] = s;
+            a.part[((size_t)tile * MT * 8 + tid) * 2 + 1] = ss;
         }
     }
+}
+
+// (sum, sum of squares) partials of the tiles -> exact GroupNorm sum slots: one block per (sample, group), double accumulation over
+// the sample's tiles in index order, a fixed tree over the block, one slot add per sum (src/lp_common.cuh:1575-1597 does the same with
+// one fixed-point atomic per block and channel)
+__global__ void __launch_bounds__(256) gn_part_reduce_k(const float *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum) {
+    const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, cpg = Co / Go, nq = MT * 8;
+    double s = 0.0, ss = 0.0;
+    for (int i = threadIdx.x; i < tiles_per_n * nq; i += 256) {
+        const int t = i / nq, qd = i - t * nq, cs = t % ncs, m = qd >> 3, q8 = qd & 7;
+        const int co = (cs * MT + m) * 32 + 8 * (q8 >> 1) + 4 * (q8 & 1);
+        if (co < Co && co / cpg == gidx) {
+            const float *p = part + ((size_t)(n * tiles_per_n + t) * nq + qd) * 2;
+            s += (double)p[0]; ss += (double)p[1];
+        }
+    }
+    __shared__ double r1[256], r2[256];
+    r1[threadIdx.x] = s; r2[threadIdx.x] = ss;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) { r1[threadIdx.x] += r1[threadIdx.x + st]; r2[threadIdx.x] += r2[threadIdx.x + st]; } __syncthreads(); }
+    if (threadIdx.x == 0) { gn_acc_add(osum, 2 * (size_t)blockIdx.x, r1[0]); gn_acc_add(osum, 2 * (size_t)blockIdx.x + 1, r2[0]); }
 }
 
 // ---- weights: fp32 w[co][ci][27] -> per (chunk, unit pair, 32-row channel tile) fragment-ordered codes + scale bytes ----
@@ -353,7 +406,7 @@ __global__ void __launch_bounds__(256, 1) conv3_mx_k(const conv_args a) {
 // padding unit are zero codes with scale byte 1
 __host__ __device__ __forceinline__ int seg_ci(int cp, int Ci, int Cx, int CxP) { if (cp < CxP) return cp < Cx ? cp : -1; const int c = Cx + cp - CxP; return c < Ci ? c : -1; }
 template <int FMT>
-__global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uint8_t *__restrict__ wq, uint8_t *__restrict__ wsc, int Co, int Ci, int Cx, int CxP,
+__global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uint8_t *__restrict__ wq, unsigned *__restrict__ wsc, int Co, int Ci, int Cx, int CxP,
                                                int nbt, int CB, int nmt_all, int npairs_all) {
     constexpr int WTILE = fmt_t<FMT>::WTILE;
     const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
@@ -364,7 +417,7 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
     for (;; b0 += CB) { nbc = min(CB, nbt - b0); const int np = (27 * nbc + 1) >> 1; if (gp < pb + np) break; pb += np; }
     const int q = gp - pb, m = cop >> 5, r = cop & 31;
     uint8_t *tile = wq + ((size_t)gp * nmt_all + m) * WTILE;
-    uint8_t *tsc = wsc + ((size_t)gp * nmt_all + m) * 64;
+    unsigned *tsc = wsc + ((size_t)gp * nmt_all + m) * 64;      // one word per lane: the byte the MFMA reads is the low one
 #pragma unroll
     for (int side = 0; side < 2; side++) {
         const int u = 2 * q + side;
@@ -390,7 +443,7 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
             for (int j = 0; j < 4; j++) c[j] = d_enc_e2m1x8(v + 8 * j, mult);
             *(uint4 *)(tile + ((size_t)(r + 32 * side) * 16)) = make_uint4(c[0], c[1], c[2], c[3]);            // lane (r, side): the unit's 32 nibbles
         }
-        tsc[r + 32 * side] = (uint8_t)(e + 127);
+        tsc[r + 32 * side] = (unsigned)(e + 127);
     }
 }
 
@@ -488,12 +541,19 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const int TZ = NT == 2 ? 2 : 4;
     const int HZ = stride * (TZ - 1) + 3, HY = stride * 7 + 3, HX = stride * 15 + 3, TT = HZ * HY * HX;
     const int RB = fmt == 8 ? 32 : 16, WTILE = fmt == 8 ? 2048 : 1024;
-    const size_t wbytes = (size_t)3 * MT * (WTILE + 64), budget = 160 * 1024 - 512;
-    int cbmax = (int)((budget - wbytes) / ((size_t)TT * (RB + 1)));
+    // LDS of a workgroup holding CB input blocks: weight ring, pair table, halo rows and scale words. Prefer the largest CB that
+    // still lets two workgroups share a CU (160 KB): the second one computes while the first stages its halo or runs its epilogue
+    auto lds_bytes = [&](int cb) { return (size_t)2 * MT * (WTILE + 256) + (size_t)(((27 * cb + 1) >> 1) + 2) * 32 + (size_t)cb * TT * (RB + 4); };
+    int cb2 = 0, cb1 = 0;
+    for (int cb = 1; cb <= a.nbt; cb++) { if (lds_bytes(cb) <= 80 * 1024) cb2 = cb; if (lds_bytes(cb) <= 160 * 1024 - 256) cb1 = cb; }
+    int cbmax = cb2 ? cb2 : cb1;
+    static int cb_env = -1;
+    if (cb_env < 0) cb_env = getenv("MI_CONV_CB") ? atoi(getenv("MI_CONV_CB")) : 0;      // tuning knob: blocks per chunk
+    if (cb_env > 0 && cb_env <= cb1) cbmax = cb_env;
     if (cbmax < 1) mi_die("%s: tile does not fit LDS", who);
     const int nchunks = (a.nbt + cbmax - 1) / cbmax;
     a.CB = (a.nbt + nchunks - 1) / nchunks;
-    size_t smem = wbytes + (size_t)a.CB * TT * (RB + 1);
+    size_t smem = lds_bytes(a.CB);
     const size_t red_bytes = (size_t)4 * MT * 8 * 2 * sizeof(float);
     if (smem < red_bytes) smem = red_bytes;
     smem = (smem + 15) & ~(size_t)15;
@@ -503,7 +563,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // ---- weights ----
     int npairs_all = 0;
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) npairs_all += (27 * (a.nbt - b0 < a.CB ? a.nbt - b0 : a.CB) + 1) >> 1;
-    const size_t wq_bytes = (size_t)npairs_all * nmt_all * WTILE, wsc_bytes = (size_t)npairs_all * nmt_all * 64;
+    // (four stages of padding: the kernel's weight loads run up to three pairs ahead of the last one)
+    const size_t wq_bytes = (size_t)(npairs_all + 4) * nmt_all * WTILE, wsc_bytes = (size_t)(npairs_all + 4) * nmt_all * 256;
     const int CxP = (Cx + 31) / 32 * 32;
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
@@ -513,18 +574,24 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         if (!have) {
             MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes));
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
+            MIRT(hipMemsetAsync(wq, 0, wq_bytes, 0)); MIRT(hipMemsetAsync(wsc, 0, wsc_bytes, 0));
             g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, a.CB, nmt_all, dev, wq, wsc});
         }
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) {
         const size_t nt = (size_t)npairs_all * nmt_all * 32;
-        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all);
-        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all);
+        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all);
+        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all);
         MICK();
     }
     a.wq = wq; a.wsc = wsc;
+    if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * MT * 8 * 2 * sizeof(float));
     if (fmt == 8) { if (stride == 1) launch_mt<8, 1>(MT, NT, a, smem); else launch_mt<8, 2>(MT, NT, a, smem); }
     else { if (stride == 1) launch_mt<4, 1>(MT, NT, a, smem); else launch_mt<4, 2>(MT, NT, a, smem); }
+    if (osum) {
+        gn_part_reduce_k<<<N * Go, 256>>>(a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum);
+        MICK();
+    }
     return 0;
 }
 
