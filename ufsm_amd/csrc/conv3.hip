@@ -1,398 +1,19 @@
-// 3x3x3 (stride 1 / 2, pad 1) implicit-GEMM convolution on MX operands for gfx950 (CDNA4), fp32 accumulate.
-//
-// Mapping (one workgroup = 4 wavefronts = one output tile of TZ x 8 x 16 voxels x up to 128 output channels):
-//   * GEMM view: M = output channels (A operand = prepared weights), N = output voxels (B operand = staged input halo),
-//     K = (tap, 32-channel input block) "units". One v_mfma_scale_f32_32x32x64_f8f6f4 consumes two units (K = 64): each
-//     32-element K block carries its own E8M0 scale, supplied per lane: lanes 0-31 give the scale of K block 0 of their row,
-//     lanes 32-63 that of K block 1. That is exactly the reference's "one scale per (voxel, 32 channels)" for the input and
-//     "per (tap, co, 32 ci)" for the weights (src/lp_common.cuh:16-19).
-//   * fp8 operand registers: lane (r, h) holds bytes [16h, 16h+16) of K block 0 in v0-3 and of K block 1 in v4-7;
-//     fp4: lane (r, h) holds the 32 nibbles of K block h in v0-3.
-//   * The input halo of the tile ((S(TZ-1)+3) x (7S+3) x (15S+3) positions, S = stride) for up to CB 32-channel blocks is
-//     staged once into LDS as [block][16-byte half][position]; a wavefront's operand read for any tap is then one
-//     ds_read_b128 per K block at a per-lane address (position of the lane's voxel + the tap's offset): no im2col.
-//   * Each wavefront owns NT voxel tiles of 32 (2 rows x 16 x) and all MT channel tiles of 32 of the workgroup: MT x NT
-//     accumulators of 32x32 (16 VGPRs each), every weight fragment reused NT times and every input fragment MT times.
-//   * Weights are prepared once per call (or memoised) in fragment order, streamed L2 -> LDS through a 2-slot ring, one
-//     barrier per K pair; two workgroups share a CU, so one's MFMAs cover the other's LDS latency, staging and epilogue.
-//   * Epilogue (src/lp_common.cuh:1465-1597): bias -> optional affine + activation -> per (voxel, 32-channel block) amax across
-//     the lane pair (l, l^32) -> E8M0 exponent -> e4m3 / e2m1 codes -> 16-byte row halves stored coalesced along x,
-//     GroupNorm (sum, sum of squares) reduced in a fixed order and added to exact fixed-point slots.
-#include "mx_dev.hpp"
-#include <hip/hip_fp16.h>
-#include <stdio.h>
-#include <stdlib.h>
-#include <string.h>
-#include <utility>
-#include <vector>
-
-// compile-time loops: accumulator tiles must be indexed with constants to stay in registers
-template <int... Is, typename F> __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>) { (f(std::integral_constant<int, Is>{}), ...); }
-template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
-
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-
-struct conv_args {
-    const uint8_t *xq[2], *xsc[2];     // input segments (compute-format MX tensors): data, scale plane
-    int nbs[2], bws[2];                // blocks per sample and block width of each segment's tensor
-    int nb0p;                          // padded blocks of segment 0 (staged blocks [0, nb0p) come from segment 0)
-    int nbt, CB;                       // staged 32-channel blocks in total, blocks per LDS chunk
-    int N, D, H, W, Do, Ho, Wo;
-    const uint8_t *wq, *wsc; int nmt_all;
-    const float *bias; int Co;
-    void *y; int ydt;
-    double *osum; float *part; int Go, stored_stats, zs0, zs1;   // part: per tile and channel quad (sum, sum of squares)
-    const float *ep_a, *ep_b; int act;
-    int ntx, nty, ntz, ncs; unsigned ntiles;
-};
-
-template <int FMT> struct fmt_t;
-template <> struct fmt_t<8> { static constexpr int RB = 32, NH = 2, WTILE = 2048; };
-template <> struct fmt_t<4> { static constexpr int RB = 16, NH = 1, WTILE = 1024; };
-
-__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678f)); }
-
-template <int FMT, int STRIDE, int MT, int NT>
-__global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
-    constexpr int TZ = NT == 2 ? 2 : 4;
-    constexpr int HZ = STRIDE * (TZ - 1) + 3, HY = STRIDE * 7 + 3, HX = STRIDE * 15 + 3, TT = HZ * HY * HX;
-    constexpr int NH = fmt_t<FMT>::NH, WTILE = fmt_t<FMT>::WTILE;
-    constexpr int STG = MT * (WTILE + 256);              // one weight stage: MT tiles of codes, then MT x 64 scale words
-    constexpr int UPT = (MT * WTILE / 16 + 255) / 256;   // 16-byte weight units per thread and stage
-    extern __shared__ __align__(16) unsigned char lds[];
-    // LDS: [2 weight stages][pair table (npairs + 2) x 2 x 16 B][halo rows CB * NH * TT * 16 B][halo scales CB * TT words]
-    const int tab_bytes = (((27 * a.CB + 1) >> 1) + 2) * 32;
-    const unsigned wring_o = 0, tab_o = 2 * STG, act_o = tab_o + tab_bytes, asc_o = act_o + a.CB * NH * TT * 16;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
-
-    // XCD-aware tile order: consecutive workgroup ids land on different XCDs (8, round robin), so give each XCD a contiguous
-    // range of tiles: neighbouring tiles (shared halo, same weights) then share one L2
-    unsigned tile;
-    {
-        const unsigned per = (a.ntiles + 7u) / 8u;
-        tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
-        if (tile >= a.ntiles) return;
-    }
-    int tt = (int)tile;
-    const int cs = tt % a.ncs; tt /= a.ncs;
-    const int tx = tt % a.ntx; tt /= a.ntx;
-    const int ty = tt % a.nty; tt /= a.nty;
-    const int tz = tt % a.ntz; const int n = tt / a.ntz;
-    const int ox0 = tx * 16, oy0 = ty * 8, oz0 = tz * TZ;
-    const int ix0 = STRIDE * ox0 - 1, iy0 = STRIDE * oy0 - 1, iz0 = STRIDE * oz0 - 1;
-
-    // the lane's voxel in each of its NT tiles: wave -> (z, y half) for TZ 2, z for TZ 4; tile j -> rows 2j, 2j+1; r -> (row, x)
-    int lz, ly0;
-    if (NT == 2) { lz = wave >> 1; ly0 = (wave & 1) * 4; } else { lz = wave; ly0 = 0; }
-    unsigned ab[NT], sbse[NT];     // LDS byte addresses of the lane's halo row (its 16-byte half) and scale word for tap (0, 0, 0) of block 0
-#pragma unroll
-    for (int j = 0; j < NT; j++) {
-        const int p0 = ((STRIDE * lz) * HY + STRIDE * (ly0 + 2 * j + (r >> 4))) * HX + STRIDE * (r & 15);
-        ab[j] = act_o + ((NH == 2 ? h * TT : 0) + p0) * 16;
-        sbse[j] = asc_o + p0 * 4;
-    }
-    const unsigned wfa = wring_o + lane * 16, wfs = wring_o + MT * WTILE + lane * 4;    // the lane's weight fragment / scale word in stage slot 0, tile 0
-    const unsigned wcp = wring_o + (tid * UPT * 16) % (MT * WTILE), wcs = wring_o + MT * WTILE + (tid * 4) % (MT * 256);   // the thread's part of a stage copy
-
-    v16f acc[MT][NT];
-#pragma unroll
-    for (int m = 0; m < MT; m++)
-#pragma unroll
-        for (int j = 0; j < NT; j++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
-
-    const size_t Sin = (size_t)a.D * a.H * a.W;
-    const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 256;
-    int pair0 = 0;                                       // global pair index of the chunk's first pair
-
-    for (int b0 = 0; b0 < a.nbt; b0 += a.CB) {
-        const int nbc = min(a.CB, a.nbt - b0), nunits = 27 * nbc, npairs = (nunits + 1) >> 1;
-        __syncthreads();                                 // the previous chunk's readers are done with the halo
-        // ---- pair table: per pair and lane half, the byte offsets of the pair's two units (fp8: both; fp4: the half's own) and of
-        // the half's scale word. unit u = (tap u / nbc, local block u % nbc); the odd padding unit (zero weights) re-reads unit A ----
-        for (int i = tid; i < (npairs + 2) * 2; i += 256) {
-            const int q = min(i >> 1, npairs - 1), hh = i & 1;
-            const int uA = 2 * q, uB = 2 * q + 1 < nunits ? 2 * q + 1 : 2 * q;
-            const int tA = uA / nbc, bA = uA - tA * nbc, tB = uB / nbc, bB = uB - tB * nbc;
-            const int pA = ((tA / 9) * HY + (tA / 3) % 3) * HX + tA % 3, pB = ((tB / 9) * HY + (tB / 3) % 3) * HX + tB % 3;
-            const int dA = (bA * NH * TT + pA) * 16, dB = (bB * NH * TT + pB) * 16, sA = (bA * TT + pA) * 4, sB = (bB * TT + pB) * 4;
-            *(v4i *)(lds + tab_o + i * 16) = (v4i){NH == 2 ? dA : (hh ? dB : dA), dB, hh ? sB : sA, 0};
-        }
-#ifndef DBG_NOSTAGE
-        // ---- stage the halo of blocks [b0, b0 + nbc): rows copied as stored, zero rows (scale byte 1) outside the tensor.
-        // Branch-free: every load reads a clamped in-tensor address and is zeroed afterwards when the position is outside;
-        // four independent loads are in flight per thread ----
-        {
-            constexpr int NB = 4;
-            const int E = nbc * TT * NH;
-            for (int i0 = tid; i0 < E; i0 += 256 * NB) {
-                v4i val[NB]; unsigned dst[NB]; bool inb[NB];
-#pragma unroll
-                for (int k = 0; k < NB; k++) {
-                    const int i = min(i0 + k * 256, E - 1);
-                    const int bl = i / (TT * NH), rem = i - bl * (TT * NH), pos = rem / NH, hf = rem - pos * NH;
-                    const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
-                    const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
-                    const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
-                    const int rb = a.bws[seg] * FMT / 8;     // stored row bytes (16 NH for 32-wide blocks)
-                    const bool pos_ok = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && blk < a.nbs[seg];
-                    const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1), cb = min(blk, a.nbs[seg] - 1);
-                    const size_t row = ((size_t)n * a.nbs[seg] + cb) * Sin + ((size_t)cz * a.H + cy) * a.W + cx;
-                    dst[k] = act_o + ((bl * NH + hf) * TT + pos) * 16;
-                    if (rb >= 16) {
-                        const bool have = rb >= (hf + 1) * 16;
-                        val[k] = *(const v4i *)(a.xq[seg] + row * rb + (have ? hf * 16 : 0));
-                        inb[k] = pos_ok && have;
-                    } else {                                 // 8- or 4-byte rows of a <= 8 / <= 16 channel tensor: only half 0 holds data
-                        val[k] = (v4i){0, 0, 0, 0};
-                        if (rb == 8) { const int2 t = *(const int2 *)(a.xq[seg] + row * 8); val[k][0] = t.x; val[k][1] = t.y; }
-                        else val[k][0] = *(const int *)(a.xq[seg] + row * 4);
-                        inb[k] = pos_ok && hf == 0;
-                    }
-                }
-#pragma unroll
-                for (int k = 0; k < NB; k++) *(v4i *)(lds + dst[k]) = inb[k] ? val[k] : (v4i){0, 0, 0, 0};
-            }
-            const int E2 = nbc * TT;
-            for (int i0 = tid; i0 < E2; i0 += 256 * NB) {
-                unsigned sv[NB]; unsigned dst[NB];
-#pragma unroll
-                for (int k = 0; k < NB; k++) {
-                    const int i = min(i0 + k * 256, E2 - 1);
-                    const int bl = i / TT, pos = i - bl * TT;
-                    const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
-                    const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
-                    const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
-                    const bool ok = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W && blk < a.nbs[seg];
-                    const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1), cb = min(blk, a.nbs[seg] - 1);
-                    const unsigned s = a.xsc[seg][((size_t)n * a.nbs[seg] + cb) * Sin + ((size_t)cz * a.H + cy) * a.W + cx];
-                    sv[k] = ok ? s : 1u; dst[k] = asc_o + i * 4;
-                }
-#pragma unroll
-                for (int k = 0; k < NB; k++) *(unsigned *)(lds + dst[k]) = sv[k];
-            }
-        }
-#endif
-        // ---- weight stages: global -> registers -> ring slot. Every thread moves UPT contiguous 16-byte units and one scale word per
-        // stage; offsets wrap instead of being guarded (duplicates store the same value). The prepared-weight buffers carry four
-        // stages of padding, so the loads that run ahead of the last pair stay inside them ----
-        const uint8_t *wgp = a.wq + (size_t)pair0 * wq_ps + (size_t)cs * MT * WTILE + (tid * UPT * 16) % (MT * WTILE);
-        const uint8_t *wgs = a.wsc + (size_t)pair0 * wsc_ps + (size_t)cs * MT * 256 + (tid * 4) % (MT * 256);
-        v4i g[UPT]; unsigned gs = 0;
-        auto wload = [&]() {            // the next stage in sequence
-#ifndef DBG_NOWLOAD
-#pragma unroll
-            for (int k = 0; k < UPT; k++) g[k] = *(const v4i *)(wgp + k * 16);
-            gs = *(const unsigned *)wgs;
-            wgp += wq_ps; wgs += wsc_ps;
-#endif
-        };
-        auto wstore = [&](int slot) {
-#pragma unroll
-            for (int k = 0; k < UPT; k++) *(v4i *)(lds + wcp + slot * STG + k * 16) = g[k];
-            *(unsigned *)(lds + wcs + slot * STG) = gs;
-        };
-        wload(); wstore(0);
-        wload();
-        __syncthreads();
-
-        // ---- K loop over unit pairs, unrolled by 2 so that the ring slot (pair & 1) is static. Step of pair q: fetch its fragments
-        // from LDS (halo rows at the table's offsets, weights from ring slot q & 1), run its MFMAs, move stage q + 1 into the other
-        // slot and start loading stage q + 2 from L2. A second workgroup on the CU covers this one's LDS latency and barriers ----
-        v8i fb[NT], fa[MT]; int sb[NT], sa[MT];
-        v4i T;
-        unsigned tabp = tab_o + (lane >> 5) * 16;          // this half's entry of pair 0
-        auto fetch = [&](int slot) {
-            const v4i t = T;
-#pragma unroll
-            for (int j = 0; j < NT; j++) {
-                const v4i lo = *(const v4i *)(lds + ab[j] + t[0]);
-                if (FMT == 8) {
-                    const v4i hi = *(const v4i *)(lds + ab[j] + t[1]);
-                    fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                } else fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                sb[j] = *(const int *)(lds + sbse[j] + t[2]);
-            }
-#pragma unroll
-            for (int m = 0; m < MT; m++) {
-                const v4i lo = *(const v4i *)(lds + wfa + slot * STG + m * WTILE);
-                if (FMT == 8) {
-                    const v4i hi = *(const v4i *)(lds + wfa + slot * STG + m * WTILE + 1024);
-                    fa[m] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                } else fa[m] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                sa[m] = *(const int *)(lds + wfs + slot * STG + m * 256);
-            }
-            T = *(const v4i *)(lds + tabp + 32); tabp += 32;      // the next pair's table entry
-        };
-        auto mma = [&]() {
-#ifndef DBG_NOMMA
-#pragma unroll
-            for (int m = 0; m < MT; m++)
-#pragma unroll
-                for (int j = 0; j < NT; j++)
-                    acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[m], fb[j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sa[m], 0, sb[j]);
-#else
-            for (int m = 0; m < MT; m++) for (int j = 0; j < NT; j++) acc[m][j][0] += (float)(fa[m][0] + fb[j][0] + sa[m] + sb[j]);
-#endif
-        };
-        T = *(const v4i *)(lds + tabp);
-        for (int q = 0; q < npairs; q += 2) {
-            fetch(0); mma(); wstore(1); wload();
-            __syncthreads();
-            if (q + 1 >= npairs) break;
-            fetch(1); mma(); wstore(0); wload();
-            __syncthreads();
-        }
-        pair0 += npairs;
-    }
-
-    // ================= epilogue =================
-    // accumulator layout of the 32x32 MFMA: lane (r = voxel within the tile, h), register i -> channel (i & 3) + 4 h + 8 (i >> 2)
-    const size_t So = (size_t)a.Do * a.Ho * a.Wo;
-    const int co_base = cs * MT * 32;
-    float *red = (float *)lds;                      // stats scratch [4 waves][MT][8 quads][2] floats (the ring and halo are dead now)
-    const bool stats = a.osum != nullptr;
-    if (stats) __syncthreads();
-    float qs[MT][4], qss[MT][4];                    // per lane: sums over its voxels of the 4-channel quads (m, i >> 2)
-#pragma unroll
-    for (int m = 0; m < MT; m++)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) { qs[m][q4] = 0.f; qss[m][q4] = 0.f; }
-    const int cpg = a.Go > 0 ? a.Co / a.Go : 1;
-    static_for<NT>([&](auto J) {
-        constexpr int j = J;
-        const int oz = oz0 + lz, oy = oy0 + ly0 + 2 * j + (r >> 4), ox = ox0 + (r & 15);
-        const bool ok = oz < a.Do && oy < a.Ho && ox < a.Wo;
-        const size_t ov = ((size_t)oz * a.Ho + oy) * a.Wo + ox;
-        const bool zst = ok && oz >= a.zs0 && oz < a.zs1;
-        static_for<MT>([&](auto M) {
-            constexpr int m = M;
-            float v[16];
-            float am = 0.f;
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int co = co_base + m * 32 + (i & 3) + 4 * h + 8 * (i >> 2);
-                float t = acc[m][j][i];
-                if (co < a.Co) {
-                    if (a.bias) t += a.bias[co];
-                    if (a.act) {
-                        if (a.ep_a) t = fmaf(t, a.ep_a[co], a.ep_b[co]);
-                        t = a.act == 1 ? __fdividef(t, 1.f + __expf(-t)) : a.act == 2 ? gelu_erf(t) : fmaxf(t, 0.f);
-                    }
-                } else t = 0.f;
-                v[i] = t; am = fmaxf(am, fabsf(t));
-            }
-            if (a.ydt >= 3) {
-                const int ybits = a.ydt == 3 ? 8 : 4;
-                am = fmaxf(am, __shfl_xor(am, 32));
-                const int e = d_mx_exp(am, ybits == 8 ? MI_INVQ8 : MI_INVQ4);
-                const float mult = d_exp2i(-e);
-                const int bwo = mx_bw(a.Co), nbo = mx_nb(a.Co);
-                uint8_t *yq = (uint8_t *)a.y, *ysc = yq + (size_t)a.N * nbo * So * mx_rb(bwo, ybits);
-                const int blk = (co_base + m * 32) / bwo;                  // bwo < 32 only when Co <= 16: one tile, block 0
-                const size_t row = ((size_t)n * nbo + blk) * So + ov;
-                if (ybits == 8) {
-                    unsigned d[4];
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc_e4m3x4(v[4 * q4] * mult, v[4 * q4 + 1] * mult, v[4 * q4 + 2] * mult, v[4 * q4 + 3] * mult);
-                    if (a.stored_stats) {
-                        const float sc = d_exp2i(e);
-#pragma unroll
-                        for (int i = 0; i < 16; i++) v[i] = d_dec_e4m3(d[i >> 2] >> (8 * (i & 3))) * sc;
-                    }
-                    // lane h = 0 holds bytes {0-3, 8-11, 16-19, 24-27}, its partner {4-7, 12-15, 20-23, 28-31}: swap so each stores 16 contiguous bytes
-                    const unsigned s0 = h ? d[0] : d[2], s1 = h ? d[1] : d[3];
-                    const unsigned r0 = __shfl_xor(s0, 32), r1 = __shfl_xor(s1, 32);
-                    const uint4 out = h ? make_uint4(r0, d[2], r1, d[3]) : make_uint4(d[0], r0, d[1], r1);
-                    if (ok && co_base + m * 32 < a.Co) {
-                        if (bwo == 32) *(uint4 *)(yq + row * 32 + 16 * h) = out;
-                        else if (bwo == 16) { if (!h) *(uint4 *)(yq + row * 16) = out; }
-                        else if (!h) *(uint2 *)(yq + row * 8) = make_uint2(out.x, out.y);
-                    }
-                } else {
-                    unsigned hw[4];   // 4 channels -> 16 bits each
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        hw[q4] = 0u;
-#pragma unroll
-                        for (int k = 0; k < 4; k++) hw[q4] |= d_enc_e2m1(v[4 * q4 + k] * mult) << (4 * k);
-                    }
-                    if (a.stored_stats) {
-                        const float sc = d_exp2i(e);
-#pragma unroll
-                        for (int i = 0; i < 16; i++) v[i] = d_dec_e2m1(hw[i >> 2] >> (4 * (i & 3))) * sc;
-                    }
-                    // halfword q4 of lane h sits at byte 4 q4 + 2 h of the 16-byte row: lane 0 assembles words 0-1, lane 1 words 2-3
-                    const unsigned mine01 = hw[0] | (hw[1] << 16), mine23 = hw[2] | (hw[3] << 16);
-                    const unsigned send = h ? mine01 : mine23, recv = __shfl_xor(send, 32);
-                    uint2 out;
-                    if (!h) out = make_uint2((hw[0] & 0xffffu) | ((recv & 0xffffu) << 16), (hw[1] & 0xffffu) | (recv & 0xffff0000u));
-                    else out = make_uint2((recv & 0xffffu) | ((hw[2] & 0xffffu) << 16), (recv >> 16) | ((hw[3] & 0xffffu) << 16));
-                    if (ok && co_base + m * 32 < a.Co) {
-                        if (bwo == 32) *(uint2 *)(yq + row * 16 + 8 * h) = out;
-                        else if (bwo == 16) { if (!h) *(uint2 *)(yq + row * 8) = out; }
-                        else if (!h) *(unsigned *)(yq + row * 4) = out.x;
-                    }
-                }
-                if (ok && !h && co_base + m * 32 < a.Co) ysc[row] = (uint8_t)(e + 127);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int co = co_base + m * 32 + (i & 3) + 4 * h + 8 * (i >> 2);
-                    if (a.ydt == 2) {
-                        if (a.Go > 0) v[i] = fabsf(v[i]) > 65504.f ? copysignf(65504.f, v[i]) : v[i];     // src/lp_common.cuh:465, :1567-1569
-                        if (ok && co < a.Co) ((__half *)a.y)[((size_t)n * a.Co + co) * So + ov] = __float2half(v[i]);
-                    } else if (ok && co < a.Co) ((float *)a.y)[((size_t)n * a.Co + co) * So + ov] = v[i];
-                }
-            }
-            if (stats && zst) {
-#pragma unroll
-                for (int i = 0; i < 16; i++) { qs[m][i >> 2] += v[i]; qss[m][i >> 2] += v[i] * v[i]; }
-            }
-        });
-    });
-    if (stats) {
-        // channels per group a multiple of 4: a quad (m, q4, h) = channels co_base + 32 m + 8 q4 + 4 h .. +3 lies in one group.
-        // Sum over the 32 voxel lanes of each half (butterfly, fixed order), then over the 4 waves in wave order, then one
-        // exact slot add per quad.
-#pragma unroll
-        for (int m = 0; m < MT; m++)
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                float s = qs[m][q4], ss = qss[m][q4];
-#pragma unroll
-                for (int d = 1; d < 32; d <<= 1) { s += __shfl_xor(s, d); ss += __shfl_xor(ss, d); }
-                if (r == 0) { red[((wave * MT + m) * 8 + q4 * 2 + h) * 2] = s; red[((wave * MT + m) * 8 + q4 * 2 + h) * 2 + 1] = ss; }
-            }
-        __syncthreads();
-        if (tid < MT * 8) {
-            // per tile and channel quad, the sums over the tile's voxels in wave order; a second kernel adds the tiles of a sample
-            // in a fixed order into the exact sum slots, so the statistics do not depend on the order workgroups finish in
-            const int m = tid >> 3, q8 = tid & 7;                       // q8 = q4 * 2 + h: channels co_base + 32 m + 8 q4 + 4 h .. + 3
-            float s = 0.f, ss = 0.f;
-            for (int w = 0; w < 4; w++) { s += red[((w * MT + m) * 8 + q8) * 2]; ss += red[((w * MT + m) * 8 + q8) * 2 + 1]; }
-            a.part[((size_t)tile * MT * 8 + tid) * 2] = s;
-            a.part[((size_t)tile * MT * 8 + tid) * 2 + 1] = ss;
-        }
-    }
-}
+// Host side of the 3x3x3 MX convolutions: entry points, operand re-staging, weight preparation and memo, tile-shape selection,
+// GroupNorm partial-sum reduction. The kernel itself is conv3_kernel.hpp, instantiated per (compute format, output kind) in
+// conv3_f*_o*.hip.
+#include "conv3_kernel.hpp"
 
 // (sum, sum of squares) partials of the tiles -> exact GroupNorm sum slots: one block per (sample, group), double accumulation over
 // the sample's tiles in index order, a fixed tree over the block, one slot add per sum (src/lp_common.cuh:1575-1597 does the same with
 // one fixed-point atomic per block and channel)
-__global__ void __launch_bounds__(256) gn_part_reduce_k(const float *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum) {
-    const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, cpg = Co / Go, nq = MT * 8;
+__global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum) {
+    // the group's channel quads are consecutive: quad Q = co / 4 lives in channel slice Q / (8 MT), slot Q % (8 MT) of its tile's record
+    const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, qpg = Co / Go / 4, nq = MT * 8, nst = tiles_per_n / ncs;
     double s = 0.0, ss = 0.0;
-    for (int i = threadIdx.x; i < tiles_per_n * nq; i += 256) {
-        const int t = i / nq, qd = i - t * nq, cs = t % ncs, m = qd >> 3, q8 = qd & 7;
-        const int co = (cs * MT + m) * 32 + 8 * (q8 >> 1) + 4 * (q8 & 1);
-        if (co < Co && co / cpg == gidx) {
-            const float *p = part + ((size_t)(n * tiles_per_n + t) * nq + qd) * 2;
-            s += (double)p[0]; ss += (double)p[1];
-        }
+    for (int i = threadIdx.x; i < nst * qpg; i += 256) {
+        const int st = i / qpg, Q = gidx * qpg + i % qpg, cs = Q / nq, qd = Q - cs * nq;
+        const float2 p = part[(size_t)(n * tiles_per_n + st * ncs + cs) * nq + qd];
+        s += (double)p.x; ss += (double)p.y;
     }
     __shared__ double r1[256], r2[256];
     r1[threadIdx.x] = s; r2[threadIdx.x] = ss;
@@ -459,31 +80,8 @@ extern "C" void lp_wmemo_clear(void) {
 }
 extern "C" void lp_wmemo_step(unsigned step) { if (step != g_wstep) { g_wstep = step; lp_wmemo_clear(); } }
 
-static thread_local char g_last_kernel[96] = "";
+thread_local char g_last_kernel[128] = "";
 extern "C" const char *mi_last_kernel(void) { return g_last_kernel; }
-
-template <int FMT, int STRIDE, int MT, int NT>
-static void launch_conv(const conv_args &a, size_t smem) {
-    static bool attr[8];
-    int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
-    if (!attr[d]) { MIRT(hipFuncSetAttribute((const void *)conv3_mx_k<FMT, STRIDE, MT, NT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); attr[d] = true; }
-    const unsigned per = (a.ntiles + 7u) / 8u;
-    conv3_mx_k<FMT, STRIDE, MT, NT><<<per * 8u, 256, smem>>>(a);
-    MICK();
-    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_mx_k<fmt %d, stride %d, MT %d, NT %d> CB %d tiles %u", FMT, STRIDE, MT, NT, a.CB, a.ntiles);
-}
-template <int FMT, int STRIDE>
-static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
-    switch (MT * 10 + NT) {
-    case 12: launch_conv<FMT, STRIDE, 1, 2>(a, smem); break;
-    case 14: if (STRIDE == 1) { launch_conv<FMT, 1, 1, 4>(a, smem); break; }
-    case 22: launch_conv<FMT, STRIDE, 2, 2>(a, smem); break;
-    case 24: if (STRIDE == 1) { launch_conv<FMT, 1, 2, 4>(a, smem); break; }
-    case 32: launch_conv<FMT, STRIDE, 3, 2>(a, smem); break;
-    case 42: launch_conv<FMT, STRIDE, 4, 2>(a, smem); break;
-    default: mi_die("conv3: no kernel for MT %d NT %d", MT, NT);
-    }
-}
 
 // the conv of every entry point: fmt 8 / 4 = compute format, stride 1 / 2
 static int conv_dispatch(const char *who, int fmt, int stride, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
@@ -586,10 +184,12 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     }
     a.wq = wq; a.wsc = wsc;
     if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * MT * 8 * 2 * sizeof(float));
-    if (fmt == 8) { if (stride == 1) launch_mt<8, 1>(MT, NT, a, smem); else launch_mt<8, 2>(MT, NT, a, smem); }
-    else { if (stride == 1) launch_mt<4, 1>(MT, NT, a, smem); else launch_mt<4, 2>(MT, NT, a, smem); }
+    const bool epi = act != 0;
+    const int out = ybf == 3 ? 8 : ybf == 4 ? 4 : 0;
+    if (fmt == 8) { if (out == 8) conv3_launch_f8_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f8_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f8_o0(stride, epi, MT, NT, a, smem); }
+    else { if (out == 8) conv3_launch_f4_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f4_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f4_o0(stride, epi, MT, NT, a, smem); }
     if (osum) {
-        gn_part_reduce_k<<<N * Go, 256>>>(a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum);
+        gn_part_reduce_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum);
         MICK();
     }
     return 0;

@@ -1,0 +1,3 @@
+// kernels of the 3x3x3 MX convolution with e2m1 compute and MX-fp4 output
+#include "conv3_kernel.hpp"
+CONV3_LAUNCH_DECL(4, 4) { launch_out<4, 4>(stride, epi, MT, NT, a, smem); }

@@ -1,0 +1,3 @@
+// kernels of the 3x3x3 MX convolution with e4m3 compute and MX-fp8 output
+#include "conv3_kernel.hpp"
+CONV3_LAUNCH_DECL(8, 8) { launch_out<8, 8>(stride, epi, MT, NT, a, smem); }
