@@ -214,7 +214,7 @@ void orc_pred_input_mx(int bits, const uint8_t *ct, int W, float mean, float isd
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < (int64_t)S; i++) {
         const int xx = (int)(i % W), yy = (int)((i / W) % W), z = z0 + (int)(i / ((int64_t)W * W));
-        const float dy = dyo[z] + (float)yy, dx = dxo[z] + (float)xx, inv = axis ? (float)axis / (sqrtf(dy * dy + dx * dx) + 1e-6f) : 0.f;
+        const float dy = dyo[z] + (float)yy, dx = dxo[z] + (float)xx, inv = axis ? (float)axis / (sqrtf(fmaf(dy, dy, dx * dx)) + 1e-6f) : 0.f;   /* (the reference builds with fused multiply-add contraction) */
         float r[8] = {0};
         r[0] = ((float)ct[(size_t)z * W * W + (size_t)yy * W + xx] - mean) * isd; r[2] = dy * inv; r[3] = dx * inv;
         if (hd == 2) for (int k = 0; k < 4; k++) r[k] = orc_h16_to_f32(orc_f32_to_h16(r[k]));

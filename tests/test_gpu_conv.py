@@ -1,0 +1,246 @@
+"""GPU parity of the 3x3x3 MX convolutions through the C ABI (lp_conv_fwd_f8 / _f4 / _s2_f8) against the oracle.
+
+Bars: exact-operand cases (tests/test_mx4_wide.c:81-98) are bit-exact / byte-identical; random data within 1e-3 max-abs-rel of the
+oracle's fp32-accumulated result (the north-star tolerance; measured about 2e-5), MX outputs byte-identical except rounding flips to a
+neighbouring code caused by the last bits of the fp32 sum; GroupNorm sums within 1e-5 relative (the reference accepts 1e-4,
+tests/test_mx4.c:293-318). Shapes follow the reference's own test matrix (tests/test_mx.c, tests/test_mx4.c, tests/test_mx4_wide.c)."""
+import numpy as np
+import pytest
+
+import orc
+import refnp
+from gpuutil import gpu_conv, dev_gn, code_mismatch_fraction, out_dims, lib, LP, DevBuf, to_mx, shape5, gnp_t, split_t
+
+pytestmark = pytest.mark.gpu
+GRID = np.array([0, .5, 1, 1.5, 2, 3, 4, 6], np.float32)
+
+
+def rand_case(rng, N, Ci, Co, S):
+    x = rng.standard_normal((N, Ci, S)).astype(np.float32)
+    w = (rng.standard_normal((Co, Ci, 27)) * np.sqrt(2.0 / (Ci * 27))).astype(np.float32)       # Kaiming normal (src/unet.c:588-607)
+    b = (rng.standard_normal(Co) * 0.1).astype(np.float32)
+    return x, w, b
+
+
+def exact_case(rng, N, Ci, Co, S):
+    return refnp.gen_exact(rng, (N, Ci, S)), refnp.gen_exact(rng, (Co, Ci, 27)), (GRID[rng.integers(0, 8, Co)] * 0.25).astype(np.float32)
+
+
+# (bits, N, Ci, Co, D, H, W, stride): ragged W = 20 (tests/test_mx.c:34-45), partial tiles (tests/test_mx4.c:727-760), wide channel
+# counts with odd block counts (tests/test_mx4_wide.c:741-745), stride-2 odd dims (tests/test_mx.c:159-199)
+EXACT_SHAPES = [
+    (8, 1, 32, 32, 2, 8, 16, 1), (8, 2, 32, 32, 5, 9, 18, 1), (8, 1, 64, 64, 8, 12, 20, 1), (8, 2, 128, 128, 4, 12, 20, 1), (8, 1, 96, 32, 6, 12, 20, 1),
+    (8, 1, 160, 96, 3, 8, 16, 1), (8, 1, 256, 320, 4, 8, 16, 1), (8, 1, 32, 16, 5, 9, 18, 1), (8, 1, 48, 40, 4, 7, 9, 1),
+    (4, 1, 32, 32, 16, 12, 16, 1), (4, 1, 32, 64, 8, 12, 16, 1), (4, 1, 256, 256, 6, 10, 14, 1), (4, 1, 288, 288, 6, 6, 6, 1), (4, 2, 64, 64, 4, 8, 16, 1),
+    (8, 1, 32, 32, 16, 16, 16, 2), (8, 1, 64, 64, 13, 10, 17, 2), (8, 2, 128, 128, 8, 16, 32, 2), (4, 1, 32, 32, 16, 16, 16, 2), (8, 1, 96, 96, 12, 10, 14, 2),
+]
+
+
+@pytest.mark.parametrize("bits,N,Ci,Co,D,H,W,stride", EXACT_SHAPES)
+def test_exact_operand_conv(gpu, bits, N, Ci, Co, D, H, W, stride):
+    rng = np.random.default_rng(Ci * 131 + Co * 7 + D + stride)
+    S = D * H * W
+    x, w, b = exact_case(rng, N, Ci, Co, S)
+    xdt = 3 if bits == 8 else 4
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    want, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, stride=stride, acc64=1)
+    got, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, stride=stride)
+    assert np.array_equal(got, want)                              # fp32 output == exact host conv, whatever the MFMA's summation order
+    got16, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 2, cbits=bits, stride=stride)
+    want16, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 2, cbits=bits, stride=stride, acc64=1)
+    assert np.array_equal(got16, want16)
+    for ydt in (3, 4):                                            # MX outputs of either format: byte-identical to the host quantiser
+        if stride == 2 and ydt != xdt:
+            continue
+        wq, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=bits, stride=stride, acc64=1)
+        gq, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=bits, stride=stride)
+        assert np.array_equal(gq, wq)
+
+
+RANDOM_SHAPES = [(8, 2, 32, 32, 8, 16, 16, 1), (8, 1, 128, 128, 6, 12, 20, 1), (8, 1, 64, 64, 8, 8, 24, 1), (4, 1, 256, 256, 4, 8, 16, 1), (4, 1, 32, 32, 8, 16, 16, 1),
+                 (8, 1, 64, 64, 12, 10, 14, 2), (8, 1, 80, 48, 5, 9, 18, 1)]
+
+
+@pytest.mark.parametrize("bits,N,Ci,Co,D,H,W,stride", RANDOM_SHAPES)
+def test_random_conv_tolerance_and_stats(gpu, bits, N, Ci, Co, D, H, W, stride):
+    rng = np.random.default_rng(Ci + Co * 3 + bits)
+    S = D * H * W
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    xdt = 3 if bits == 8 else 4
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    G = 8
+    stats = stride == 1 and (Co // G) % 4 == 0
+    want, ws = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, stride=stride, Go=G, want_stats=stats)
+    got, gs = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, stride=stride, Go=G, stats=stats)
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-3          # north-star tolerance on the fp32-accumulated result
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-4          # what the block-scaled MFMA actually delivers
+    if stats:
+        assert np.abs(gs - ws).max() / np.abs(ws).max() < 1e-5
+    Do, Ho, Wo = out_dims(D, H, W, stride)
+    wq, ws2 = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, stride=stride, Go=G, want_stats=stats, stored_stats=1)
+    gq, gs2 = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, stride=stride, Go=G, stats=stats, stored_stats=1)
+    frac, near = code_mismatch_fraction(bits, gq, wq, N, Co, Do * Ho * Wo)
+    assert frac < 5e-3 and near
+    if stats:                                                     # statistics of the decoded stored tensor (tests/test_gn_contract.c)
+        dec = orc.mx_to_f32(bits, gq, N, Co, Do * Ho * Wo).astype(np.float64).reshape(N, G, -1)
+        assert np.allclose(gs2[:, :, 0], dec.sum(-1), rtol=1e-5, atol=1e-3) and np.allclose(gs2[:, :, 1], (dec * dec).sum(-1), rtol=1e-5)
+    # run to run: byte-identical outputs and identical statistics (deterministic reduction order)
+    gq2, gs3 = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, stride=stride, Go=G, stats=stats, stored_stats=1)
+    assert np.array_equal(gq, gq2) and (not stats or np.array_equal(gs2, gs3))
+
+
+@pytest.mark.parametrize("bits,xdt", [(8, 3), (4, 4), (4, 3), (8, 4), (8, 0), (8, 2)])
+def test_gn_silu_input_staging(gpu, bits, xdt):
+    """The consumer applies GroupNorm + SiLU while staging (src/lp_common.cuh:413-431); any stored format feeds either compute format."""
+    rng = np.random.default_rng(20 + bits + xdt)
+    N, Ci, Co, D, H, W, G = 2, 64, 32, 4, 8, 16, 8
+    S = D * H * W
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    gam = rng.uniform(0.5, 1.5, Ci).astype(np.float32); bet = rng.uniform(-.5, .5, Ci).astype(np.float32)
+    mean = rng.uniform(-.2, .2, N * G).astype(np.float32); rstd = rng.uniform(.8, 1.2, N * G).astype(np.float32)
+    if xdt >= 3:
+        xin = orc.f32_to_mx(8 if xdt == 3 else 4, x, N, Ci, S)
+    elif xdt == 2:
+        xin = np.ascontiguousarray(x.astype(np.float16).view(np.uint16))
+    else:
+        xin = x
+    want, _ = orc.conv3(xin, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, gp=orc.gn(gam, bet, mean, rstd, G))
+    got, _ = gpu_conv(xin, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, gp=dev_gn(gam, bet, mean, rstd, G))
+    # the sigmoid runs on the hardware's fast exponential: a few staged codes land on the neighbour (the reference's own acceptance,
+    # tests/test_mx4_wide.c:165-175); measured at the conv output that is a small relative error, larger for the 8-value fp4 grid
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err < (3e-3 if bits == 8 else 3e-2)
+
+
+def test_plain_input_without_gn_is_bit_exact_vs_converter(gpu):
+    rng = np.random.default_rng(31)
+    N, Ci, Co, D, H, W = 1, 64, 32, 4, 8, 16
+    S = D * H * W
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    g0, _ = gpu_conv(x, 0, N, Ci, D, H, W, w, b, Co, 3)
+    g1, _ = gpu_conv(orc.f32_to_mx(8, x, N, Ci, S), 3, N, Ci, D, H, W, w, b, Co, 3)
+    assert np.array_equal(g0, g1)
+
+
+@pytest.mark.parametrize("bits,Cu,Cs,Co,dims,gn", [(8, 32, 32, 32, (4, 8, 16), False), (8, 64, 32, 32, (4, 8, 16), True), (8, 80, 64, 64, (8, 8, 12), True),
+                                                   (4, 64, 32, 32, (4, 8, 16), False), (8, 32, 16, 16, (12, 12, 16), True)])
+def test_decoder_conv_split_input(gpu, bits, Cu, Cs, Co, dims, gn):
+    """Decoder conv1: channels [0, Cu) from x, the rest from x2, each with its own GroupNorm (tests/test_mx.c:138-156)."""
+    rng = np.random.default_rng(40 + Cu + Cs)
+    D, H, W = dims
+    N, S, G = 1, D * H * W, 8
+    xa = rng.standard_normal((N, Cu, S)).astype(np.float32); xb = rng.standard_normal((N, Cs, S)).astype(np.float32)
+    w = (rng.standard_normal((Co, Cu + Cs, 27)) * np.sqrt(2.0 / ((Cu + Cs) * 27))).astype(np.float32); b = (rng.standard_normal(Co) * 0.1).astype(np.float32)
+    xdt = 3 if bits == 8 else 4
+    qa, qb = orc.f32_to_mx(bits, xa, N, Cu, S), orc.f32_to_mx(bits, xb, N, Cs, S)
+    p = [rng.uniform(0.5, 1.5, Cu).astype(np.float32), rng.uniform(-.5, .5, Cu).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    p2 = [rng.uniform(0.5, 1.5, Cs).astype(np.float32), rng.uniform(-.5, .5, Cs).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    want, _ = orc.conv3(qa, xdt, N, Cu + Cs, D, H, W, w, b, Co, 0, cbits=bits, x2=qb, c_split=Cu, gp=orc.gn(*p, G) if gn else None, gp2=orc.gn(*p2, G) if gn else None)
+    got, _ = gpu_conv(qa, xdt, N, Cu + Cs, D, H, W, w, b, Co, 0, cbits=bits, x2=qb, c_split=Cu, gp=dev_gn(*p, G) if gn else None, gp2=dev_gn(*p2, G) if gn else None)
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err < (2e-4 if not gn else 3e-3 if bits == 8 else 3e-2)
+
+
+@pytest.mark.parametrize("Cu,Cs,Co,dims,gn", [(32, 32, 32, (4, 8, 16), False), (64, 32, 32, (8, 8, 16), True), (32, 16, 16, (12, 12, 16), True)])
+def test_decoder_conv_fused_upsample(gpu, Cu, Cs, Co, dims, gn):
+    """Decoder conv1 reading [up2(silu(gn(coarse))) | silu(gn(skip))] without materialising the upsample (tests/test_mx.c:319+)."""
+    rng = np.random.default_rng(50 + Cu)
+    D, H, W = dims
+    N, S, Sc, G = 1, D * H * W, (D // 2) * (H // 2) * (W // 2), 8
+    exact = not gn
+    xa = refnp.gen_exact(rng, (N, Cu, Sc)) if exact else rng.standard_normal((N, Cu, Sc)).astype(np.float32)
+    if exact:
+        xa[:, 5, :] = 6.0
+    xb = refnp.gen_exact(rng, (N, Cs, S)) if exact else rng.standard_normal((N, Cs, S)).astype(np.float32)
+    w = refnp.gen_exact(rng, (Co, Cu + Cs, 27)) if exact else (rng.standard_normal((Co, Cu + Cs, 27)) * 0.05).astype(np.float32)
+    qa, qb = orc.f32_to_mx(8, xa, N, Cu, Sc), orc.f32_to_mx(8, xb, N, Cs, S)
+    p = [rng.uniform(0.5, 1.5, Cu).astype(np.float32), rng.uniform(-.5, .5, Cu).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    p2 = [rng.uniform(0.5, 1.5, Cs).astype(np.float32), rng.uniform(-.5, .5, Cs).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    want, _ = orc.conv3(qa, 3, N, Cu + Cs, D, H, W, w, None, Co, 0, x2=qb, c_split=Cu, up=1, gp=orc.gn(*p, G) if gn else None, gp2=orc.gn(*p2, G) if gn else None)
+    got, _ = gpu_conv(qa, 3, N, Cu + Cs, D, H, W, w, None, Co, 0, x2=qb, c_split=Cu, up=1, gp=dev_gn(*p, G) if gn else None, gp2=dev_gn(*p2, G) if gn else None)
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err < (1e-5 if exact else 3e-3)
+
+
+def test_fused_activation_epilogue(gpu):
+    """Extension (no reference counterpart): per-channel affine + SiLU / GELU / ReLU before the MX re-quantisation, pinned by fp64 closed forms."""
+    rng = np.random.default_rng(60)
+    N, Ci, Co, D, H, W = 1, 64, 64, 4, 8, 16
+    S = D * H * W
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    ea = rng.uniform(0.5, 1.5, Co).astype(np.float32); eb = rng.uniform(-.5, .5, Co).astype(np.float32)
+    xq = orc.f32_to_mx(8, x, N, Ci, S)
+    lin, _ = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 0)
+    for act in (1, 2, 3):
+        want, _ = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 0, fused_act=act, ep_a=ea, ep_b=eb)
+        got, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 0, fused=(act, ea, eb))
+        assert np.abs(got - want).max() / np.abs(want).max() < 1e-4
+        u = lin.astype(np.float64) * ea[None, :, None] + eb[None, :, None]
+        from math import erf
+        closed = {1: u / (1 + np.exp(-u)), 2: 0.5 * u * (1 + np.vectorize(erf)(u / np.sqrt(2))), 3: np.maximum(u, 0)}[act]
+        assert np.abs(want - closed).max() / np.abs(closed).max() < 1e-5
+        wq, _ = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 3, fused_act=act, ep_a=ea, ep_b=eb)
+        gq, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 3, fused=(act, ea, eb))
+        frac, near = code_mismatch_fraction(8, gq, wq, N, Co, S)
+        assert frac < 5e-3 and near
+
+
+def test_weight_memo(gpu):
+    rng = np.random.default_rng(70)
+    N, Ci, Co, D, H, W = 1, 32, 32, 4, 8, 16
+    S = D * H * W
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(8, x, N, Ci, S)
+    dxq, dw, db = DevBuf.from_numpy(xq), DevBuf.from_numpy(w), DevBuf.from_numpy(b)
+    dy = DevBuf(lib.lp_mx8_bytes(N, Co, S))
+    sp = split_t(); sp.wkey = 1234
+    outs = []
+    w2 = np.ascontiguousarray(2 * w)
+    for step in (0, 0, 1):
+        if step:                                                  # weights changed: a new step drops the memo (src/nn_lp.h:56)
+            lib.mi_h2d(dw.ptr, w2.ctypes.data, w2.nbytes); lib.lp_wmemo_step(1)
+        lib.lp_conv_fwd_f8(dxq.ptr, 3, shape5(N, Ci, D, H, W), dw.ptr, db.ptr, Co, dy.ptr, 3, gnp_t(), None, 0, sp)
+        LP.check()
+        outs.append(dy.to_numpy(np.uint8))
+    assert np.array_equal(outs[0], outs[1]) and not np.array_equal(outs[0], outs[2])
+    want, _ = orc.conv3(xq, 3, N, Ci, D, H, W, w2, b, Co, 3)
+    assert code_mismatch_fraction(8, outs[2], want, N, Co, S)[0] < 5e-3
+    lib.lp_wmemo_clear()
+
+
+def test_nonfinite_input_propagates(gpu):
+    """A NaN block (scale byte 0xFF) reaches every output voxel whose taps touch it and nothing else (tests/test_mx4.c:139-168)."""
+    rng = np.random.default_rng(80)
+    N, Ci, Co, D, H, W = 1, 32, 32, 4, 8, 16
+    S = D * H * W
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    x[0, 3, (2 * H + 4) * W + 8] = np.nan
+    xq = orc.f32_to_mx(8, x, N, Ci, S)
+    got, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 0)
+    bad = ~np.isfinite(got[0, 0].reshape(D, H, W))
+    exp = np.zeros((D, H, W), bool); exp[1:4, 3:6, 7:10] = True
+    assert np.array_equal(bad, exp)
+
+
+@pytest.mark.parametrize("bits", [8, 4])
+def test_full_size_properties(gpu, bits):
+    """BASELINE-size layer (128 -> 128, 64^3, N 2; fp4: 256 -> 256, 32^3, N 2): exact-operand output compared on sampled planes with the
+    oracle restricted to those planes, and byte-equal reruns."""
+    rng = np.random.default_rng(90 + bits)
+    N, Ci, Co, D = (2, 128, 128, 64) if bits == 8 else (2, 256, 256, 32)
+    H = W = D
+    S = D * H * W
+    xdt = 3 if bits == 8 else 4
+    x, w, b = exact_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    gq, gs = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, Go=8, stats=True)
+    gq2, gs2 = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, Go=8, stats=True, wkey=99)
+    assert np.array_equal(gq, gq2) and np.array_equal(gs, gs2)
+    lib.lp_wmemo_clear()
+    dec = orc.mx_to_f32(bits, gq, N, Co, S).reshape(N, Co, D, H, W)
+    for (z0, z1) in [(0, 1), (D // 2, D // 2 + 1), (D - 1, D)]:
+        want, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, z0=z0, z1=z1, acc64=1)
+        wdec = orc.mx_to_f32(bits, want, N, Co, S).reshape(N, Co, D, H, W)
+        assert np.array_equal(dec[:, :, z0:z1], wdec[:, :, z0:z1])
+    # statistics == fp64 sums of the exact pre-quantisation values is checked at small sizes; here: sum of the sums is finite and stable
+    assert np.isfinite(gs).all()

@@ -96,12 +96,12 @@ __global__ void __launch_bounds__(256) pred_in_mx_k(const uint8_t *ct, int W, fl
     const size_t S = (size_t)nz * W * W, i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     if (i >= S) return;
     const int xx = (int)(i % W), yy = (int)((i / W) % W), z = z0 + (int)(i / ((size_t)W * W));
-    const float dy = dyo[z] + (float)yy, dx = dxo[z] + (float)xx, inv = axis ? (float)axis / (sqrtf(dy * dy + dx * dx) + 1e-6f) : 0.f;
+    const float dy = dyo[z] + (float)yy, dx = dxo[z] + (float)xx, inv = axis ? (float)axis / (sqrtf(fmaf(dy, dy, dx * dx)) + 1e-6f) : 0.f;
     float r[32];
 #pragma unroll
     for (int k = 0; k < 32; k++) r[k] = 0.f;
     r[0] = in_round<HD>(((float)ct[(size_t)z * W * W + (size_t)yy * W + xx] - mean) * isd); r[1] = in_round<HD>(0.f);
-    r[2] = in_round<HD>(dy * inv); r[3] = in_round<HD>(dx * inv);
+    r[2] = in_round<HD>(__fmul_rn(dy, inv)); r[3] = in_round<HD>(__fmul_rn(dx, inv));     // (axis 0: the products are signed zeros, kept as such)
     store_row<B, true>(y, mx_scp<B>(y, 1, 4, S), i, 8, r);
 }
 extern "C" void lp_pred_input_mx(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits) {
