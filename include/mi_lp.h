@@ -103,6 +103,10 @@ void mi_event_destroy(void *ev);
    act 0 none, 1 SiLU, 2 GELU (erf), 3 ReLU. bits 8 / 4 selects the compute format. */
 int mi_conv_fwd_fused(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                       const float *ep_a, const float *ep_b, int act, gnp_t gp, double *osum, int Go, split_t sp);
+/* timing of the 3x3x3 conv kernel launches alone (benchmarks): on != 0 starts recording an event pair around every launch on the
+   stream it runs on and clears the totals; read returns the total milliseconds so far and the number of launches (synchronises) */
+void mi_kernel_timing(int on);
+double mi_kernel_timing_read(long *launches);
 /* name of the conv kernel variant the last conv call on this thread launched (diagnostics / tests), "" if none */
 const char *mi_last_kernel(void);
 #ifdef __cplusplus

@@ -81,6 +81,26 @@ extern "C" void lp_wmemo_clear(void) {
 extern "C" void lp_wmemo_step(unsigned step) { if (step != g_wstep) { g_wstep = step; lp_wmemo_clear(); } }
 
 thread_local char g_last_kernel[128] = "";
+
+// optional timing of the conv kernel launches alone (benchmarks): event pairs on the stream the kernel runs on
+static bool g_ktime = false;
+static std::vector<std::pair<hipEvent_t, hipEvent_t>> g_kev;
+static double g_kms = 0.0; static long g_kn = 0;
+extern "C" void mi_kernel_timing(int on) {
+    for (auto &e : g_kev) { MIRT(hipEventDestroy(e.first)); MIRT(hipEventDestroy(e.second)); }
+    g_kev.clear(); g_kms = 0.0; g_kn = 0; g_ktime = on != 0;
+}
+extern "C" double mi_kernel_timing_read(long *launches) {       // total milliseconds of the timed launches so far (synchronises)
+    for (auto &e : g_kev) {
+        float ms = 0.f;
+        MIRT(hipEventSynchronize(e.second)); MIRT(hipEventElapsedTime(&ms, e.first, e.second));
+        g_kms += ms; g_kn++;
+        MIRT(hipEventDestroy(e.first)); MIRT(hipEventDestroy(e.second));
+    }
+    g_kev.clear();
+    if (launches) *launches = g_kn;
+    return g_kms;
+}
 extern "C" const char *mi_last_kernel(void) { return g_last_kernel; }
 
 // the conv of every entry point: fmt 8 / 4 = compute format, stride 1 / 2
@@ -186,8 +206,11 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * MT * 8 * 2 * sizeof(float));
     const bool epi = act != 0;
     const int out = ybf == 3 ? 8 : ybf == 4 ? 4 : 0;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    if (g_ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
     if (fmt == 8) { if (out == 8) conv3_launch_f8_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f8_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f8_o0(stride, epi, MT, NT, a, smem); }
     else { if (out == 8) conv3_launch_f4_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f4_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f4_o0(stride, epi, MT, NT, a, smem); }
+    if (g_ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
     if (osum) {
         gn_part_reduce_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum);
         MICK();
