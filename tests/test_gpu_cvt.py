@@ -24,11 +24,12 @@ def test_f32_to_mx_bit_exact(gpu, bits, N, Cc, S):
     got = dq.to_numpy(np.uint8)
     want = orc.f32_to_mx(bits, x, N, Cc, S)
     assert np.array_equal(got, want)
-    # decode on the device == decode of the oracle, bit for bit (NaN payloads included)
+    # decode on the device == decode of the oracle, bit for bit (signed zeros and infinities included)
     dz = DevBuf(x.nbytes)
     (lib.lp_mx8_to_f32 if bits == 8 else lib.lp_mx4_to_f32)(dq.ptr, N, Cc, S, dz.ptr)
     back = dz.to_numpy(np.float32, x.shape)
-    assert np.array_equal(back.view(np.uint32), orc.mx_to_f32(bits, want, N, Cc, S).view(np.uint32))
+    ref = orc.mx_to_f32(bits, want, N, Cc, S)
+    assert ((back.view(np.uint32) == ref.view(np.uint32)) | (np.isnan(back) & np.isnan(ref))).all()     # (NaN payloads are not part of the format)
 
 
 @pytest.mark.parametrize("bits", [8, 4])

@@ -304,17 +304,18 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
             if (OUT != 0) {
                 am = fmaxf(am, __shfl_xor(am, 32));
                 const int e = d_mx_exp(am, YB == 8 ? MI_INVQ8 : MI_INVQ4);
-                const float mult = d_exp2i(-e);
                 const int blk = (co_base + m * 32) / bwo;                  // bwo < 32 only when Co <= 16: one tile, block 0
                 const size_t row = ((size_t)n * nbo + blk) * So + ov;
                 if (OUT == 8) {
                     unsigned d[4];
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc_e4m3x4(v[4 * q4] * mult, v[4 * q4 + 1] * mult, v[4 * q4 + 2] * mult, v[4 * q4 + 3] * mult);
+                    for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc4_e4m3(v[4 * q4], v[4 * q4 + 1], v[4 * q4 + 2], v[4 * q4 + 3], e);
                     if (a.stored_stats) {
                         const float sc = d_exp2i(e);
 #pragma unroll
-                        for (int i = 0; i < 16; i++) v[i] = d_dec_e4m3(d[i >> 2] >> (8 * (i & 3))) * sc;
+                        for (int q4 = 0; q4 < 4; q4++) d_dec4_e4m3(d[q4], v + 4 * q4);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) v[i] *= sc;
                     }
                     // lane h = 0 holds bytes {0-3, 8-11, 16-19, 24-27}, its partner {4-7, 12-15, 20-23, 28-31}: swap so each stores 16 contiguous bytes
                     const unsigned s0 = h ? d[0] : d[2], s1 = h ? d[1] : d[3];
@@ -327,16 +328,15 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
                     }
                 } else {
                     unsigned hw[4];   // 4 channels -> 16 bits each
+                    {
+                        const unsigned w01 = d_enc8_e2m1(v, e), w23 = d_enc8_e2m1(v + 8, e);
+                        hw[0] = w01 & 0xffffu; hw[1] = w01 >> 16; hw[2] = w23 & 0xffffu; hw[3] = w23 >> 16;
+                        if (a.stored_stats) {
+                            const float sc = d_exp2i(e);
+                            d_dec8_e2m1(w01, v); d_dec8_e2m1(w23, v + 8);
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) {
-                        hw[q4] = 0u;
-#pragma unroll
-                        for (int k = 0; k < 4; k++) hw[q4] |= d_enc_e2m1(v[4 * q4 + k] * mult) << (4 * k);
-                    }
-                    if (a.stored_stats) {
-                        const float sc = d_exp2i(e);
-#pragma unroll
-                        for (int i = 0; i < 16; i++) v[i] = d_dec_e2m1(hw[i >> 2] >> (4 * (i & 3))) * sc;
+                            for (int i = 0; i < 16; i++) v[i] *= sc;
+                        }
                     }
                     // halfword q4 of lane h sits at byte 4 q4 + 2 h of the 16-byte row: lane 0 assembles words 0-1, lane 1 words 2-3
                     const unsigned mine01 = hw[0] | (hw[1] << 16), mine23 = hw[2] | (hw[3] << 16);

@@ -379,8 +379,64 @@ __global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int
     }
     store_row<BY, false>(y, mx_scp<BY>(y, N, Cy, S), i, 32, r);
 }
+// the same for an MX source with 32-wide blocks, two lanes per row: each lane moves one 16-channel half (16 or 8 contiguous bytes in,
+// 16 or 8 out), so a wavefront reads and writes contiguous memory; the halves' amaxes meet through one lane exchange. The (a, b)
+// coefficients of the block's 32 channels are formed once per workgroup in LDS. HBM-bound: (bits_in + bits_out) / 8 + 2/32 bytes per element.
+template <int BX, int BY>
+__global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0) {
+    const int nb = C / 32, blk = blockIdx.y, n = blockIdx.z;
+    __shared__ float sa[32], sb[32];
+    if (threadIdx.x < 32) {
+        float a = 1.f, b = 0.f;
+        if (gp.G) { const int c = cg0 + blk * 32 + threadIdx.x, ng = n * gp.G + c / (Cg / gp.G); a = gp.rstd[ng] * gp.gamma[c]; b = fmaf(-gp.mean[ng], a, gp.beta[c]); }
+        sa[threadIdx.x] = a; sb[threadIdx.x] = b;
+    }
+    __syncthreads();
+    const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;       // (voxel, half)
+    const size_t v = t >> 1; const int hf = (int)(t & 1);
+    if (v >= S) return;                                            // (S even or odd: the pair of lanes of a row leaves together)
+    constexpr int IB = BX * 2, OB = BY * 2;                        // bytes of a 16-channel half row
+    const size_t row = ((size_t)n * nb + blk) * S + v;
+    const uint8_t *xs = x + (size_t)N * nb * S * (IB * 2);
+    uint8_t *ys = y + (size_t)N * nb * S * (OB * 2);
+    unsigned w[4] = {0u, 0u, 0u, 0u};
+    if (BX == 8) { const uint4 q = *(const uint4 *)(x + row * 32 + hf * 16); w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w; }
+    else { const uint2 q = *(const uint2 *)(x + row * 16 + hf * 8); w[0] = q.x; w[1] = q.y; }
+    const float sc = d_mx_scale(xs[row]);
+    float r[16];
+    if (BX == 8) { d_dec4_e4m3(w[0], r); d_dec4_e4m3(w[1], r + 4); d_dec4_e4m3(w[2], r + 8); d_dec4_e4m3(w[3], r + 12); }
+    else { d_dec8_e2m1(w[0], r); d_dec8_e2m1(w[1], r + 8); }
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        const float xv = r[k] * sc;
+        r[k] = gp.G ? d_act_ab(xv, sa[hf * 16 + k], sb[hf * 16 + k]) : xv;
+    }
+    float am = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(r[k]));
+    am = fmaxf(am, __shfl_xor(am, 1));
+    const int e = d_mx_exp(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
+    if (BY == 8) {
+        uint4 o;
+        o.x = d_enc4_e4m3(r[0], r[1], r[2], r[3], e); o.y = d_enc4_e4m3(r[4], r[5], r[6], r[7], e);
+        o.z = d_enc4_e4m3(r[8], r[9], r[10], r[11], e); o.w = d_enc4_e4m3(r[12], r[13], r[14], r[15], e);
+        *(uint4 *)(y + row * 32 + hf * 16) = o;
+    } else {
+        uint2 o; o.x = d_enc8_e2m1(r, e); o.y = d_enc8_e2m1(r + 8, e);
+        *(uint2 *)(y + row * 16 + hf * 8) = o;
+    }
+    if (!hf) ys[row] = (uint8_t)(e + 127);
+}
 void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits) {
     const size_t n = (size_t)N * ((C + 31) / 32) * S; if (!n) return;
+    if (xdt >= 3 && C % 32 == 0) {
+        const dim3 grid(nblk_(2 * S, 256), (unsigned)(C / 32), (unsigned)N);
+        const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
+        if (xdt == 3) { if (ybits == 8) restage32_k<8, 8><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0); else restage32_k<8, 4><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0); }
+        else { if (ybits == 8) restage32_k<4, 8><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0); else restage32_k<4, 4><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0); }
+        MICK();
+        return;
+    }
 #define RS(BX, BY, TI) restage_k<BX, BY, TI><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, N, C, S, gp, Cg, cg0)
 #define RS_Y(BX, TI) do { if (ybits == 4) RS(BX, 4, TI); else RS(BX, 8, TI); } while (0)
     if (xdt == 4) RS_Y(4, float); else if (xdt == 3) RS_Y(8, float); else if (xdt == 2) RS_Y(0, __half); else if (xdt == 1) RS_Y(0, bf16_t); else RS_Y(0, float);
