@@ -1,0 +1,60 @@
+/* Host side (C23) of the MX U-Net forward: the op layer and the graph the reference keeps above its lp_* kernels, restated over
+ * the C ABI of include/mi_lp.h. Names, argument meaning and error behaviour follow the reference's own declarations:
+ *   nn_set_storage / nn_storage / nn_set_prec / nn_conv3d_fwd_gn_stats / nn_conv3d_fwd_x / nn_gn_stats   src/nn.h:100, :194-195, :423-433, :484
+ *   unet_cfg / unet_create / unet_init / unet_forward_x / unet_forward_ct                               src/unet.h:1-30, :141, :186, :428
+ * Tensors are device pointers; an activation is an MX tensor registered with nn_set_storage (dt 8 / 4), as in the reference.
+ */
+#ifndef MI_UNET_H
+#define MI_UNET_H
+#include "mi_lp.h"
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- op layer (src/nn.h) ---- */
+void nn_set_storage(const void *p, size_t bytes, int dt);      /* dt 8 MX-fp8, 4 MX-fp4, 2 fp16 planes, 0 forgets (fp32 planes) */
+int nn_storage(const void *p);                                 /* the dt of the registered range holding p, else 0 */
+void nn_storage_forget(const void *p);
+void nn_set_prec(int p);                                       /* 3: MX-fp4 compute for every conv, else the storage decides (src/nn_bwd.cu:110-112) */
+void nn_set_gn_stored(int on);                                 /* GroupNorm statistics of the decoded stored output (src/nn_core.cu:7; default 0) */
+size_t nn_mx8_bytes(shape5 s);
+size_t nn_mx4_bytes(shape5 s);
+typedef struct { const float *gamma, *beta, *mean, *rstd; int G; } nn_gn_t;          /* src/nn.h:431 */
+/* y = conv3(silu(gn(x))) (G_in 0: x as is) with the GroupNorm statistics of y for G_out groups written to omean / orstd (src/nn.h:423) */
+int nn_conv3d_fwd_gn_stats(const float *x, shape5 xs, int G_in, const float *gamma, const float *beta, const float *mean, const float *rstd,
+                           const float *w, const float *b, int cout, float *y, int G_out, float eps, float *omean, float *orstd);
+/* input-side recompute conv: k 3 stride 1 (split / fused upsample / output statistics), k 3 stride 2, k 1 head (src/nn.h:432) */
+int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn_gn_t *gx2, int c_split, int up, shape5 xs,
+                    const float *w, const float *b, int cout, int k, int stride, float *y, int G_out, float eps, float *omean, float *orstd);
+int nn_gn_stats(const float *x, shape5 s, int G, float eps, float *mean, float *rstd);   /* of a stored MX tensor; -1 when unsupported (src/nn.h:484) */
+const char *nn_check(void);                                    /* src/nn.h:28 */
+
+/* ---- U-Net graph (src/unet.h, src/unet.c:2567-2636, :2867-3121; inference, recompute mode, no residual blocks) ---- */
+#define UNET_MAXLEV 8
+typedef struct {
+    int cin;                   /* input channels (4 for CT windows: z-scored CT, 0, radial dy, dx) */
+    int nlev;                  /* levels */
+    int widths[UNET_MAXLEV];   /* channels per level */
+    int G;                     /* GroupNorm groups (min(G, C) is used, src/unet.c:297) */
+    int head_out;              /* logits */
+    int act_dt;                /* activation storage: 8 MX-fp8, 4 MX-fp4 */
+    int prec;                  /* 3: fp4 compute everywhere (MX-fp4 weights over MX-fp8 storage), else by storage */
+} unet_cfg;
+typedef struct unet unet;
+unet *unet_create(const unet_cfg *cfg, shape5 in);             /* in: the window (n, cin, d, h, w); dims divisible by 2^(nlev-1) */
+void unet_free(unet *u);
+size_t unet_nparams(const unet *u);
+void unet_init(unet *u, uint64_t seed);                        /* Kaiming normal sqrt(2 / (cin 27)), biases 0, head bias -2, gamma 1, beta 0 (src/unet.c:588-607) */
+void unet_get_params(const unet *u, float *host);              /* the flat parameter vector in unet_init's order */
+void unet_set_params(unet *u, const float *host);
+int unet_forward_x(unet *u, const void *x, float *logits);     /* x: device MX tensor (act_dt) of the input; logits: device fp32 [n][head_out][S] */
+/* the input built on the device from a uint8 CT window of one sample (src/unet.c:2858-2865, src/lp_mx_cvt.cu:29-55), then the forward */
+int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, float *logits);
+/* per-layer introspection for parity tests: the k-th conv output tensor (device MX) and its shape, in execution order; NULL past the end */
+const void *unet_layer_out(const unet *u, int k, shape5 *s, const char **name);
+/* the GroupNorm statistics the k-th conv produced (device [n * G] each); returns G, 0 when the layer has none */
+int unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd);
+#ifdef __cplusplus
+}
+#endif
+#endif

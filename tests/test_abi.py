@@ -8,11 +8,11 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def header_functions():
-    text = open(os.path.join(ROOT, "include", "mi_lp.h")).read()
+def header_functions(header="mi_lp.h", prefixes=("lp_", "mi_", "gnp_")):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     names = re.findall(r"\b([a-z][a-z0-9_]*)\s*\([^;{]*\)\s*;", text)
-    return sorted(set(n for n in names if n.startswith(("lp_", "mi_", "gnp_"))))
+    return sorted(set(n for n in names if n.startswith(prefixes)))
 
 
 def test_header_declares_the_forward_subset():
@@ -30,6 +30,16 @@ def test_library_exports_every_declared_symbol():
     for n in header_functions():
         assert hasattr(L, n), "libufsm_lp.so does not export %s" % n
     assert set(header_functions()) == set(lp.EXPORTS)
+
+
+def test_host_library_exports_every_declared_symbol():
+    from ufsm_amd import unet
+    H = unet.load_host()
+    names = header_functions("mi_unet.h", ("nn_", "unet_"))
+    assert "unet_forward_x" in names and "nn_conv3d_fwd_x" in names and "nn_set_storage" in names
+    for n in names:
+        assert hasattr(H, n), "libufsm_host.so does not export %s" % n
+    assert C.sizeof(unet.unet_cfg) == 4 * (2 + unet.UNET_MAXLEV + 4)
 
 
 def test_descriptor_layouts():

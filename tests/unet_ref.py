@@ -1,0 +1,108 @@
+"""The U-Net forward composed from oracle calls (checker of the whole-net parity tests): the same layer order, parameter order and
+GroupNorm hand-offs as src/unet.c:588-607, :2567-2636, :2939-3105, every op evaluated by oracle/ on the host."""
+import numpy as np
+
+import orc
+
+
+def param_layout(cin, widths, head_out):
+    L = len(widths); off = 0; lay = {}
+
+    def conv(name, ci, co, k):
+        nonlocal off
+        lay[name + ".w"] = (off, (co, ci, k ** 3)); off += co * ci * k ** 3
+        lay[name + ".b"] = (off, (co,)); off += co
+
+    def gn(name, c):
+        nonlocal off
+        lay[name + ".gamma"] = (off, (c,)); off += c
+        lay[name + ".beta"] = (off, (c,)); off += c
+
+    for i in range(L):
+        conv("enc%d.c1" % i, widths[i - 1] if i else cin, widths[i], 3); gn("enc%d.n1" % i, widths[i])
+        conv("enc%d.c2" % i, widths[i], widths[i], 3); gn("enc%d.n2" % i, widths[i])
+    for i in range(L - 1):
+        conv("down%d" % i, widths[i], widths[i], 3)
+    for i in range(L - 1):
+        conv("dec%d.c1" % i, widths[i + 1] + widths[i], widths[i], 3); gn("dec%d.n1" % i, widths[i])
+        conv("dec%d.c2" % i, widths[i], widths[i], 3); gn("dec%d.n2" % i, widths[i])
+    conv("head", widths[0], head_out, 1)
+    return lay, off
+
+
+def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0):
+    """xq: MX bytes of the input. Returns (logits fp32 [N][head_out][S], {layer name: MX bytes})."""
+    lay, n = param_layout(cin, widths, head_out)
+    assert params.size == n
+    P = lambda k: np.ascontiguousarray(params[lay[k][0]:lay[k][0] + int(np.prod(lay[k][1]))].reshape(lay[k][1]))
+    L = len(widths); dt = 3 if bits == 8 else 4
+    outs = {}
+    Gof = lambda c: min(G, c)
+    dims = [(D >> i, H >> i, W >> i) for i in range(L)]
+
+    def finalize(sums, c, S):
+        g = Gof(c)
+        mean = np.zeros(N * g, np.float32); rstd = np.zeros(N * g, np.float32)
+        orc.lib().orc_gn_finalize(orc.ptr(sums), N * g, (c // g) * S, 1e-5, orc.ptr(mean), orc.ptr(rstd))
+        return mean, rstd
+
+    def conv(name, x, ci, d, gp=None, x2=None, c_split=0, up=0, gp2=None, stride=1, stats=True):
+        co = lay[name + ".w"][1][0]
+        cb = cbits if (cbits and ci > 8) else (4 if (bits == 4 and ci > 8) else 8)
+        if stride == 2:                       # the reference's stride-2 dispatch: fp4 only for an MX-fp4 32 -> <= 32 channel conv (src/lp_s2.cu:653-671)
+            cb = 4 if (bits == 4 and ci == 32 and co <= 32) else 8
+        y, s = orc.conv3(x, dt, N, ci, d[0], d[1], d[2], P(name + ".w"), P(name + ".b"), co, dt, cbits=cb, stride=stride, x2=x2, c_split=c_split, up=up,
+                         gp=gp, gp2=gp2, Go=Gof(co), want_stats=stats, stored_stats=stored)
+        outs[name] = y
+        return y, s
+
+    cur, blocks = xq, {}
+    for i in range(L):
+        ci = widths[i - 1] if i else cin
+        S = dims[i][0] * dims[i][1] * dims[i][2]
+        a1, s1 = conv("enc%d.c1" % i, cur, ci, dims[i])
+        m1, r1 = finalize(s1, widths[i], S)
+        a2, s2 = conv("enc%d.c2" % i, a1, widths[i], dims[i], gp=orc.gn(P("enc%d.n1.gamma" % i), P("enc%d.n1.beta" % i), m1, r1, Gof(widths[i])))
+        m2, r2 = finalize(s2, widths[i], S)
+        blocks["enc%d" % i] = (a2, orc.gn(P("enc%d.n2.gamma" % i), P("enc%d.n2.beta" % i), m2, r2, Gof(widths[i])), (m2, r2))
+        if i < L - 1:
+            cur, _ = conv("down%d" % i, a2, widths[i], dims[i], gp=blocks["enc%d" % i][1], stride=2, stats=False)
+    for i in range(L - 2, -1, -1):
+        coarse = blocks["enc%d" % (L - 1)] if i == L - 2 else blocks["dec%d" % (i + 1)]
+        skip = blocks["enc%d" % i]
+        S = dims[i][0] * dims[i][1] * dims[i][2]
+        a1, s1 = conv("dec%d.c1" % i, coarse[0], widths[i + 1] + widths[i], dims[i], gp=coarse[1], x2=skip[0], c_split=widths[i + 1], up=1, gp2=skip[1])
+        m1, r1 = finalize(s1, widths[i], S)
+        a2, s2 = conv("dec%d.c2" % i, a1, widths[i], dims[i], gp=orc.gn(P("dec%d.n1.gamma" % i), P("dec%d.n1.beta" % i), m1, r1, Gof(widths[i])))
+        m2, r2 = finalize(s2, widths[i], S)
+        blocks["dec%d" % i] = (a2, orc.gn(P("dec%d.n2.gamma" % i), P("dec%d.n2.beta" % i), m2, r2, Gof(widths[i])), (m2, r2))
+    last = blocks["dec0"] if L > 1 else blocks["enc0"]
+    S = D * H * W
+    logits = np.zeros((N, head_out, S), np.float32)
+    hw = np.ascontiguousarray(P("head.w").reshape(head_out, widths[0])); hb = P("head.b")
+    orc.lib().orc_conv1_mx(bits, orc.ptr(last[0]), N, widths[0], S, orc.ptr(hw), orc.ptr(hb), head_out, last[1], orc.ptr(logits))
+    return logits, outs
+
+
+def layer_inputs(widths):
+    """name -> (x layer, x2 layer, stride, up) of every conv in execution order; 'input' is the network input. The GroupNorm a reader
+    applies is the statistics of the tensor it reads with the parameters of the block norm that follows that tensor."""
+    L = len(widths); g = []
+    for i in range(L):
+        g.append(("enc%d.c1" % i, "input" if i == 0 else "down%d" % (i - 1), None, 1, 0))
+        g.append(("enc%d.c2" % i, "enc%d.c1" % i, None, 1, 0))
+        if i < L - 1:
+            g.append(("down%d" % i, "enc%d.c2" % i, None, 2, 0))
+    for i in range(L - 2, -1, -1):
+        coarse = "enc%d.c2" % (L - 1) if i == L - 2 else "dec%d.c2" % (i + 1)
+        g.append(("dec%d.c1" % i, coarse, "enc%d.c2" % i, 1, 1))
+        g.append(("dec%d.c2" % i, "dec%d.c1" % i, None, 1, 0))
+    return g
+
+
+def norm_of(layer):
+    """the GroupNorm parameters applied to a conv output by its readers: block.c1 -> block.n1, block.c2 -> block.n2; down convs: none."""
+    if layer.startswith("down") or layer == "input":
+        return None
+    blk, c = layer.split(".")
+    return blk + (".n1" if c == "c1" else ".n2")

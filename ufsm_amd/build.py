@@ -40,6 +40,17 @@ def build_hip(verbose=False):
     return LIB
 
 
+HOST_LIB = os.path.join(ROOT, "ufsm_amd", "libufsm_host.so")
+
+
+def build_host():
+    """The C23 host layer (op dispatch + U-Net graph) over the C ABI of libufsm_lp.so."""
+    src = [os.path.join(ROOT, "ufsm_amd", "host", f) for f in ("nn_host.c", "unet.c")]
+    _run(["gcc", "-std=c2x", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "-o", HOST_LIB] + src +
+         ["-L" + os.path.dirname(LIB), "-lufsm_lp", "-Wl,-rpath,$ORIGIN", "-lm"])
+    return HOST_LIB
+
+
 def build_oracle():
     _run(["make", "-B", "liboracle.so"], cwd=ORACLE_DIR)
     return ORACLE_LIB
@@ -48,6 +59,7 @@ def build_oracle():
 def build_all(verbose=False):
     build_oracle()
     build_hip(verbose)
+    build_host()
 
 
 if __name__ == "__main__":

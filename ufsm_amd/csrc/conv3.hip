@@ -22,6 +22,22 @@ __global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int 
     if (threadIdx.x == 0) { gn_acc_add(osum, 2 * (size_t)blockIdx.x, r1[0]); gn_acc_add(osum, 2 * (size_t)blockIdx.x + 1, r2[0]); }
 }
 
+// the same from per-channel records (32 per tile, one channel tile per workgroup)
+__global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, int tiles_per_n, int Co, int Go, double *osum) {
+    const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, cpg = Co / Go;
+    double s = 0.0, ss = 0.0;
+    for (int i = threadIdx.x; i < tiles_per_n * cpg; i += 256) {
+        const int t = i / cpg, ch = gidx * cpg + i % cpg;
+        const float2 p = part[(size_t)(n * tiles_per_n + t) * 32 + ch];
+        s += (double)p.x; ss += (double)p.y;
+    }
+    __shared__ double r1[256], r2[256];
+    r1[threadIdx.x] = s; r2[threadIdx.x] = ss;
+    __syncthreads();
+    for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) { r1[threadIdx.x] += r1[threadIdx.x + st]; r2[threadIdx.x] += r2[threadIdx.x + st]; } __syncthreads(); }
+    if (threadIdx.x == 0) { gn_acc_add(osum, 2 * (size_t)blockIdx.x, r1[0]); gn_acc_add(osum, 2 * (size_t)blockIdx.x + 1, r2[0]); }
+}
+
 // ---- weights: fp32 w[co][ci][27] -> per (chunk, unit pair, 32-row channel tile) fragment-ordered codes + scale bytes ----
 // block = the 32 ci of one (tap, co) (src/lp_f8fwd.cu:54-71, src/lp_f4fwd.cu:53-66); fmaxf amax; padded rows / channels / the odd
 // padding unit are zero codes with scale byte 1
@@ -116,7 +132,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (sp.x2 && xbf < 3) mi_die("%s: split inputs need MX storage", who);
     if (sp.up && (!sp.x2 || xbf < 3 || (xs.d & 1) || (xs.h & 1) || (xs.w & 1) || stride != 1)) mi_die("%s: the fused upsample needs an MX split input and even dims", who);
     if (osum && (Go <= 0 || cout % Go)) mi_die("%s: %d output channels in %d groups", who, cout, Go);
-    if (osum && (cout / Go) % 4) mi_die("%s: fused output statistics need channels per group (%d) to be a multiple of 4", who, cout / Go);
+    if (osum && (cout / Go) % 4 && cout > 32) mi_die("%s: fused output statistics of %d channels need channels per group (%d) to be a multiple of 4", who, cout, cout / Go);
     if (gp.G && ((sp.x2 && sp.gp2.G ? Cx : Ci) % gp.G)) mi_die("%s: GroupNorm groups %d do not divide the channels", who, gp.G);
     if (sp.gp2.G && (!sp.x2 || C2 % sp.gp2.G)) mi_die("%s: second GroupNorm without a matching x2 segment", who);
     const int N = xs.n, D = xs.d, H = xs.h, W = xs.w;
@@ -172,7 +188,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const int nchunks = (a.nbt + cbmax - 1) / cbmax;
     a.CB = (a.nbt + nchunks - 1) / nchunks;
     size_t smem = lds_bytes(a.CB);
-    const size_t red_bytes = (size_t)4 * MT * 8 * 2 * sizeof(float);
+    const size_t red_bytes = (size_t)4 * 32 * 2 * sizeof(float);     // (the larger of the quad and per-channel statistics scratch)
     if (smem < red_bytes) smem = red_bytes;
     smem = (smem + 15) & ~(size_t)15;
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
@@ -203,7 +219,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         MICK();
     }
     a.wq = wq; a.wsc = wsc;
-    if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * MT * 8 * 2 * sizeof(float));
+    a.stat_ch = osum && (cout / Go) % 4 ? 1 : 0;
+    if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * (a.stat_ch ? 32 : MT * 8) * 2 * sizeof(float));
     const bool epi = act != 0;
     const int out = ybf == 3 ? 8 : ybf == 4 ? 4 : 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
@@ -212,7 +229,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     else { if (out == 8) conv3_launch_f4_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f4_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f4_o0(stride, epi, MT, NT, a, smem); }
     if (g_ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
     if (osum) {
-        gn_part_reduce_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum);
+        if (a.stat_ch) gn_part_reduce_ch_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), cout, Go, osum);
+        else gn_part_reduce_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum);
         MICK();
     }
     return 0;

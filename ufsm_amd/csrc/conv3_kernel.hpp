@@ -45,6 +45,7 @@ struct conv_args {
     const float *bias; int Co;
     void *y; int ydt;
     double *osum; float *part; int Go, stored_stats, zs0, zs1;   // part: per tile and channel quad (sum, sum of squares)
+    int stat_ch;                       // 1: per-channel records (channels per group not a multiple of 4; Co <= 32 only)
     const float *ep_a, *ep_b; int act;
     int ntx, nty, ntz, ncs; unsigned ntiles;
 };
@@ -271,6 +272,9 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) { qs[m][q4] = 0.f; qss[m][q4] = 0.f; }
+    float chs[MT == 1 ? 16 : 1], chss[MT == 1 ? 16 : 1];     // per-channel sums (MT 1, stat_ch)
+#pragma unroll
+    for (int i = 0; i < (MT == 1 ? 16 : 1); i++) { chs[i] = 0.f; chss[i] = 0.f; }
     constexpr int YB = OUT == 4 ? 4 : 8;
     const int bwo = mx_bw(a.Co), nbo = mx_nb(a.Co), rbo = mx_rb(bwo, YB);
     uint8_t *yq = (uint8_t *)a.y, *ysc = yq + (size_t)a.N * nbo * So * rbo;
@@ -364,13 +368,35 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
                 }
             }
             if (stats && zst) {
+                if (MT == 1 && a.stat_ch) {
 #pragma unroll
-                for (int i = 0; i < 16; i++) { qs[m][i >> 2] += v[i]; qss[m][i >> 2] += v[i] * v[i]; }
+                    for (int i = 0; i < 16; i++) { chs[i] += v[i]; chss[i] += v[i] * v[i]; }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) { qs[m][i >> 2] += v[i]; qss[m][i >> 2] += v[i] * v[i]; }
+                }
             }
         });
     });
     if (stats) __syncthreads();
-    if (stats) {
+    if (MT == 1 && stats && a.stat_ch) {
+        // any group size (one channel tile): per-channel sums over the 32 voxel lanes, then over the waves; channel of register i of
+        // half h = (i & 3) + 4 h + 8 (i >> 2)
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            float s1 = chs[i], s2 = chss[i];
+#pragma unroll
+            for (int d = 1; d < 32; d <<= 1) { s1 += __shfl_xor(s1, d); s2 += __shfl_xor(s2, d); }
+            const int ch = (i & 3) + 4 * h + 8 * (i >> 2);
+            if (r == 0) { red[(wave * 32 + ch) * 2] = s1; red[(wave * 32 + ch) * 2 + 1] = s2; }
+        }
+        __syncthreads();
+        if (tid < 32) {
+            float s1 = 0.f, s2 = 0.f;
+            for (int w = 0; w < 4; w++) { s1 += red[(w * 32 + tid) * 2]; s2 += red[(w * 32 + tid) * 2 + 1]; }
+            a.part[((size_t)tile * 32 + tid) * 2] = s1; a.part[((size_t)tile * 32 + tid) * 2 + 1] = s2;
+        }
+    } else if (stats) {
         // channels per group a multiple of 4: a quad (m, q4, h) = channels co_base + 32 m + 8 q4 + 4 h .. +3 lies in one group.
         // Sum over the 32 voxel lanes of each half (butterfly, fixed order), then over the 4 waves in wave order, then one
         // exact slot add per quad.

@@ -1,0 +1,96 @@
+/* Op layer of the MX forward path (C23): storage registry, precision policy and the conv entry points that choose the kernel
+   family, own the GroupNorm sum slots and finalize them. Restates what src/nn_bwd.cu:83-155, src/nn_wgrad.cu:103-145,
+   src/nn_fusedgn.cu:22-70 and src/nn_core.cu:376-390 do around the lp_* kernels; no arithmetic happens here. */
+#include "../../include/mi_unet.h"
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#if __STDC_VERSION__ < 202311L      /* (this image's gcc 11 implements C2x without the nullptr constant) */
+#define nullptr ((void *)0)
+#endif
+
+/* ---- storage registry: device ranges holding MX (or fp16) tensors (src/nn_core.cu:376-390) ---- */
+typedef struct { const char *p; size_t bytes; int dt; } reg_t;
+static reg_t *g_reg; static int g_nreg, g_capreg;
+void nn_storage_forget(const void *p) {
+    for (int i = 0; i < g_nreg; i++) if (g_reg[i].p == (const char *)p) { g_reg[i] = g_reg[--g_nreg]; return; }
+}
+void nn_set_storage(const void *p, size_t bytes, int dt) {
+    nn_storage_forget(p);
+    if (!dt || !p) return;
+    if (g_nreg == g_capreg) { g_capreg = g_capreg ? 2 * g_capreg : 64; g_reg = realloc(g_reg, (size_t)g_capreg * sizeof *g_reg); if (!g_reg) { fprintf(stderr, "nn_set_storage: out of memory\n"); abort(); } }
+    g_reg[g_nreg++] = (reg_t){(const char *)p, bytes, dt};
+}
+int nn_storage(const void *p) {
+    for (int i = 0; i < g_nreg; i++) if ((const char *)p >= g_reg[i].p && (const char *)p < g_reg[i].p + g_reg[i].bytes) return g_reg[i].dt;
+    return 0;
+}
+static int g_prec = 0, g_gn_stored = 0;
+void nn_set_prec(int p) { g_prec = p; }
+void nn_set_gn_stored(int on) { g_gn_stored = on; }
+size_t nn_mx8_bytes(shape5 s) { return lp_mx8_bytes(s.n, s.c, (size_t)s.d * s.h * s.w); }
+size_t nn_mx4_bytes(shape5 s) { return lp_mx4_bytes(s.n, s.c, (size_t)s.d * s.h * s.w); }
+const char *nn_check(void) { return lp_check(); }
+
+/* lp dtype code of a tensor (0 fp32, 2 fp16, 3 MX-fp8, 4 MX-fp4) from the registry (ISMX / MXDT, src/nn_common.cuh:118-127) */
+static int lp_dt(const void *p) { const int dt = nn_storage(p); return dt == 8 ? 3 : dt == 4 ? 4 : dt == 2 ? 2 : 0; }
+
+/* the GroupNorm sum slots of the conv in flight (gn_dsums, src/nn_elem.cu:12-17): one grow-only device buffer */
+static double *g_sums; static size_t g_sums_cap;
+static double *gn_dsums(size_t nslots) {
+    if (nslots > g_sums_cap) { if (g_sums) mi_free(g_sums); g_sums = mi_malloc(nslots * MI_GN_SLOT_BYTES); g_sums_cap = nslots; }
+    return g_sums;
+}
+/* statistics of the decoded stored output instead of the pre-quantisation values (gn_fused_stored, src/nn_bwd.cu:67-72) */
+static int gn_fused_stored(int ydt, int cout) { return g_gn_stored && ydt >= 3 && cout >= 16; }
+
+int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn_gn_t *gx2, int c_split, int up, shape5 xs,
+                    const float *w, const float *b, int cout, int k, int stride, float *y, int G_out, float eps, float *omean, float *orstd) {
+    const int xdt = lp_dt(x), ydt = lp_dt(y);
+    if (x2 && lp_dt(x2) != xdt) { fprintf(stderr, "nn_conv3d_fwd_x: x and x2 differ in storage\n"); return -1; }
+    gnp_t gp = gx ? gnp_mk(gx->gamma, gx->beta, gx->mean, gx->rstd, gx->G) : gnp_mk(nullptr, nullptr, nullptr, nullptr, 0);
+    if (k == 1) {                                                   /* the head: MX input, fp32 (or registered fp16) planes out (src/nn_fusedgn.cu:57-62) */
+        if (xdt < 3 || x2 || stride != 1 || G_out) return -1;
+        if (ydt == 2) lp_conv1_fwd_mx_h16(x, xdt, xs, w, b, cout, y, gp); else lp_conv1_fwd_mx(x, xdt, xs, w, b, cout, y, gp);
+        return 0;
+    }
+    if (k != 3) return -1;
+    if (stride == 2) {                                              /* down conv: no split, no output statistics (src/nn_bwd.cu:120-155) */
+        if (x2 || G_out || xdt < 3) return -1;
+        const shape5 ys = {xs.n, cout, (xs.d - 1) / 2 + 1, (xs.h - 1) / 2 + 1, (xs.w - 1) / 2 + 1};
+        lp_conv_fwd_s2_f8(x, xdt, xs, w, b, cout, y, ydt, ys, gp);
+        return 0;
+    }
+    if (stride != 1) return -1;
+    split_t sp; memset(&sp, 0, sizeof sp);
+    if (x2) { sp.x2 = x2; sp.c_split = c_split; sp.up = (int16_t)up; if (gx2) sp.gp2 = gnp_mk(gx2->gamma, gx2->beta, gx2->mean, gx2->rstd, gx2->G); }
+    else if (up) return -1;
+    sp.wkey = (unsigned)((uintptr_t)w >> 4) | 1u;                   /* inference: weights are prepared once per conv (keyed by the weight pointer) */
+    double *sums = nullptr;
+    if (G_out > 0 && omean) {
+        sums = gn_dsums((size_t)2 * xs.n * G_out);
+        mi_gn_sums_zero(sums, 2 * xs.n * G_out);
+        sp.stored_stats = gn_fused_stored(ydt, cout);
+    }
+    /* MX-fp4 storage or precision 3 run the fp4 kernels, everything else fp8; the <= 8 channel network input always runs in fp8
+       (src/nn_bwd.cu:110-112, src/lp_f4fwd.cu:37) */
+    const int f4 = (xdt == 4 || g_prec == 3) && xs.c > 8;
+    (f4 ? lp_conv_fwd_f4 : lp_conv_fwd_f8)(x, xdt, xs, w, b, cout, y, ydt, gp, sums, sums ? G_out : 0, sp);
+    if (sums) mi_gn_finalize(sums, xs.n * G_out, (size_t)(cout / G_out) * xs.d * xs.h * xs.w, eps, omean, orstd);
+    return 0;
+}
+int nn_conv3d_fwd_gn_stats(const float *x, shape5 xs, int G_in, const float *gamma, const float *beta, const float *mean, const float *rstd,
+                           const float *w, const float *b, int cout, float *y, int G_out, float eps, float *omean, float *orstd) {
+    const nn_gn_t g = {gamma, beta, mean, rstd, G_in};
+    return nn_conv3d_fwd_x(x, G_in ? &g : nullptr, nullptr, nullptr, 0, 0, xs, w, b, cout, 3, 1, y, G_out, eps, omean, orstd);
+}
+int nn_gn_stats(const float *x, shape5 s, int G, float eps, float *mean, float *rstd) {
+    const int dt = lp_dt(x);
+    if (dt < 3 || G <= 0 || s.c % G) return -1;
+    const size_t S = (size_t)s.d * s.h * s.w;
+    double *sums = gn_dsums((size_t)2 * s.n * G);
+    mi_gn_sums_zero(sums, 2 * s.n * G);
+    if (lp_gn_sums_mx(x, dt, s.n, s.c, G, S, sums, 0, S)) return -1;
+    mi_gn_finalize(sums, s.n * G, (size_t)(s.c / G) * S, eps, mean, rstd);
+    return 0;
+}

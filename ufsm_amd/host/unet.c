@@ -1,0 +1,180 @@
+/* The U-Net inference graph (C23) over the op layer: two 3x3x3 convs per level with GroupNorm statistics fused into their
+   epilogues and the GroupNorm + SiLU applied by the next reader while it stages its input (recompute mode: no activated tensor is
+   ever stored), 3x3x3 stride-2 down convs, decoder conv1 reading [up2(coarse) | skip] without materialising either, 1x1x1 head.
+   Layer and parameter order follow src/unet.c:588-607 (unet_init) and src/unet.c:2567-2636, :2939-3105 (block_fwd, unet_forward_x). */
+#include "../../include/mi_unet.h"
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#if __STDC_VERSION__ < 202311L      /* (this image's gcc 11 implements C2x without the nullptr constant) */
+#define nullptr ((void *)0)
+#endif
+
+typedef struct { size_t w, b; int cin, cout, k; } convp;           /* offsets into the flat parameter vector */
+typedef struct { size_t gamma, beta; int c; } gnpar;
+typedef struct {
+    convp c1, c2; gnpar n1, n2;
+    shape5 xs, ys;                                                 /* conv1 input shape (all its channels), block output shape */
+    void *a1, *a2;                                                 /* conv outputs (pre-norm, MX) */
+    float *m1, *r1, *m2, *r2;                                      /* their GroupNorm statistics [n * G] */
+} block;
+struct unet {
+    unet_cfg cfg; shape5 in; shape5 ls[UNET_MAXLEV];
+    block enc[UNET_MAXLEV], dec[UNET_MAXLEV];
+    convp down[UNET_MAXLEV], head;
+    void *downo[UNET_MAXLEV];
+    size_t np; float *params;                                      /* device */
+    void *xin;                                                     /* the network input built from a CT window */
+    struct { const void *p; shape5 s; const char *name; const float *mean, *rstd; int G; } outs[64]; int nouts;
+};
+
+static int G_of(const unet *u, int c) { return u->cfg.G < c ? u->cfg.G : c; }      /* src/unet.c:297 */
+static size_t add_conv(convp *c, int cin, int cout, int k, size_t off) { c->cin = cin; c->cout = cout; c->k = k; c->w = off; off += (size_t)cout * cin * k * k * k; c->b = off; return off + cout; }
+static size_t add_gn(gnpar *g, int c, size_t off) { g->c = c; g->gamma = off; g->beta = off + c; return off + 2 * (size_t)c; }
+static size_t act_bytes(const unet *u, shape5 s) { return u->cfg.act_dt == 4 ? nn_mx4_bytes(s) : nn_mx8_bytes(s); }
+static void *act_new(const unet *u, shape5 s) { const size_t b = act_bytes(u, s); void *p = mi_malloc(b); mi_zero(p, b); nn_set_storage(p, b, u->cfg.act_dt); return p; }
+static void act_del(void *p) { if (p) { nn_storage_forget(p); mi_free(p); } }
+static float *f32_new(size_t n) { float *p = mi_malloc(n * 4); mi_zero(p, n * 4); return p; }
+
+unet *unet_create(const unet_cfg *cfg, shape5 in) {
+    const int L = cfg->nlev;
+    if (L < 1 || L > UNET_MAXLEV || in.c != cfg->cin || (cfg->act_dt != 8 && cfg->act_dt != 4)) { fprintf(stderr, "unet_create: bad configuration\n"); return nullptr; }
+    if ((in.d | in.h | in.w) & ((1 << (L - 1)) - 1)) { fprintf(stderr, "unet_create: window %d x %d x %d is not divisible by %d\n", in.d, in.h, in.w, 1 << (L - 1)); return nullptr; }
+    unet *u = calloc(1, sizeof *u);
+    if (!u) return nullptr;
+    u->cfg = *cfg; u->in = in;
+    const int *w = cfg->widths;
+    size_t off = 0;
+    /* parameter order of unet_init: encoder blocks, down convs, decoder blocks, head */
+    for (int i = 0; i < L; i++) {
+        block *b = &u->enc[i];
+        off = add_conv(&b->c1, i ? w[i - 1] : cfg->cin, w[i], 3, off); off = add_gn(&b->n1, w[i], off);
+        off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
+    }
+    for (int i = 0; i < L - 1; i++) off = add_conv(&u->down[i], w[i], w[i], 3, off);         /* the down conv keeps its level's width (src/unet.c:2970) */
+    for (int i = 0; i < L - 1; i++) {
+        block *b = &u->dec[i];
+        off = add_conv(&b->c1, w[i + 1] + w[i], w[i], 3, off); off = add_gn(&b->n1, w[i], off);
+        off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
+    }
+    off = add_conv(&u->head, w[0], cfg->head_out, 1, off);
+    u->np = off;
+    u->params = f32_new(off);
+    for (int i = 0; i < L; i++) u->ls[i] = (shape5){in.n, w[i], in.d >> i, in.h >> i, in.w >> i};
+    for (int i = 0; i < L; i++) {
+        for (int s = 0; s < 2; s++) {
+            block *b = s ? &u->dec[i] : &u->enc[i];
+            if (s && i == L - 1) continue;
+            b->ys = u->ls[i]; b->xs = u->ls[i]; b->xs.c = b->c1.cin;
+            b->a1 = act_new(u, b->ys); b->a2 = act_new(u, b->ys);
+            const size_t ng = (size_t)in.n * G_of(u, w[i]);
+            b->m1 = f32_new(ng); b->r1 = f32_new(ng); b->m2 = f32_new(ng); b->r2 = f32_new(ng);
+        }
+        if (i < L - 1) { shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds); }
+    }
+    u->xin = act_new(u, in);
+    return u;
+}
+void unet_free(unet *u) {
+    if (!u) return;
+    mi_sync();
+    for (int i = 0; i < UNET_MAXLEV; i++) {
+        for (int s = 0; s < 2; s++) { block *b = s ? &u->dec[i] : &u->enc[i]; act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2); }
+        act_del(u->downo[i]);
+    }
+    act_del(u->xin); mi_free(u->params);
+    lp_wmemo_clear();
+    free(u);
+}
+size_t unet_nparams(const unet *u) { return u->np; }
+void unet_get_params(const unet *u, float *host) { mi_sync(); mi_d2h(host, u->params, u->np * 4); }
+void unet_set_params(unet *u, const float *host) { mi_h2d(u->params, host, u->np * 4); lp_wmemo_clear(); }
+
+/* splitmix64 -> uniform -> Box-Muller normal: the distribution of src/unet.c:586-593, not its generator's bits */
+static double unif(uint64_t *s) { uint64_t z = (*s += 0x9e3779b97f4a7c15ull); z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull; z = (z ^ (z >> 27)) * 0x94d049bb133111ebull; z ^= z >> 31; return (double)(z >> 11) * 0x1.0p-53; }
+static double gauss(uint64_t *s) { const double a = unif(s) + 1e-300, b = unif(s); return sqrt(-2 * log(a)) * cos(6.283185307179586 * b); }
+static void init_conv(float *h, const convp *c, uint64_t *seed, double bias) {
+    const size_t nw = (size_t)c->cout * c->cin * c->k * c->k * c->k;
+    const double std = sqrt(2.0 / ((double)c->cin * c->k * c->k * c->k));
+    for (size_t i = 0; i < nw; i++) h[c->w + i] = (float)(std * gauss(seed));
+    for (int i = 0; i < c->cout; i++) h[c->b + i] = (float)bias;
+}
+static void init_gn(float *h, const gnpar *n) { for (int i = 0; i < n->c; i++) { h[n->gamma + i] = 1.f; h[n->beta + i] = 0.f; } }
+void unet_init(unet *u, uint64_t seed) {
+    float *h = calloc(u->np, 4);
+    if (!h) { fprintf(stderr, "unet_init: out of memory\n"); abort(); }
+    const int L = u->cfg.nlev;
+    for (int i = 0; i < L; i++) { init_conv(h, &u->enc[i].c1, &seed, 0); init_gn(h, &u->enc[i].n1); init_conv(h, &u->enc[i].c2, &seed, 0); init_gn(h, &u->enc[i].n2); }
+    for (int i = 0; i < L - 1; i++) init_conv(h, &u->down[i], &seed, 0);
+    for (int i = 0; i < L - 1; i++) { init_conv(h, &u->dec[i].c1, &seed, 0); init_gn(h, &u->dec[i].n1); init_conv(h, &u->dec[i].c2, &seed, 0); init_gn(h, &u->dec[i].n2); }
+    init_conv(h, &u->head, &seed, -2.0);
+    unet_set_params(u, h);
+    free(h);
+}
+
+#define P(u, off) ((u)->params + (off))
+static void note(unet *u, const void *p, shape5 s, const char *name, const float *mean, const float *rstd, int G) {
+    if (u->nouts < 64) { u->outs[u->nouts].p = p; u->outs[u->nouts].s = s; u->outs[u->nouts].name = name; u->outs[u->nouts].mean = mean; u->outs[u->nouts].rstd = rstd; u->outs[u->nouts].G = G; u->nouts++; }
+}
+static nn_gn_t gn_out(const unet *u, const block *b) { return (nn_gn_t){P(u, b->n2.gamma), P(u, b->n2.beta), b->m2, b->r2, G_of(u, b->ys.c)}; }   /* silu(gn(a2)) for the block's readers */
+
+/* conv1 -> a1 (+ its statistics), conv2 reads silu(gn(a1)) while staging -> a2 (+ statistics) (src/unet.c:2567-2636) */
+static int block_fwd(unet *u, block *b, const void *x, const nn_gn_t *gin, const void *xup, const nn_gn_t *gup, int c_split, const char *n1, const char *n2) {
+    const int G = G_of(u, b->c1.cout);
+    int r;
+    if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, b->xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, b->a1, G, 1e-5f, b->m1, b->r1);   /* [up2(coarse) | skip] */
+    else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, b->xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, b->a1, G, 1e-5f, b->m1, b->r1);
+    if (r) return r;
+    note(u, b->a1, b->ys, n1, b->m1, b->r1, G);
+    r = nn_conv3d_fwd_gn_stats(b->a1, b->ys, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, b->a2, G, 1e-5f, b->m2, b->r2);
+    note(u, b->a2, b->ys, n2, b->m2, b->r2, G);
+    return r;
+}
+int unet_forward_x(unet *u, const void *x, float *logits) {
+    static const char *en1[] = {"enc0.c1", "enc1.c1", "enc2.c1", "enc3.c1", "enc4.c1", "enc5.c1", "enc6.c1", "enc7.c1"}, *en2[] = {"enc0.c2", "enc1.c2", "enc2.c2", "enc3.c2", "enc4.c2", "enc5.c2", "enc6.c2", "enc7.c2"};
+    static const char *dn1[] = {"dec0.c1", "dec1.c1", "dec2.c1", "dec3.c1", "dec4.c1", "dec5.c1", "dec6.c1"}, *dn2[] = {"dec0.c2", "dec1.c2", "dec2.c2", "dec3.c2", "dec4.c2", "dec5.c2", "dec6.c2"};
+    static const char *dwn[] = {"down0", "down1", "down2", "down3", "down4", "down5", "down6"};
+    const int L = u->cfg.nlev;
+    const int reg_here = nn_storage(x) != u->cfg.act_dt;           /* the caller's input is looked up by the convs like any activation */
+    if (reg_here) nn_set_storage(x, act_bytes(u, u->in), u->cfg.act_dt);
+    nn_set_prec(u->cfg.prec);
+    u->nouts = 0;
+    const void *cur = x;
+    for (int i = 0; i < L; i++) {
+        if (block_fwd(u, &u->enc[i], cur, nullptr, nullptr, nullptr, 0, en1[i], en2[i])) { if (reg_here) nn_storage_forget(x); return -1; }
+        if (i < L - 1) {                                           /* stride-2 down conv of silu(gn(a2)), width kept (src/unet.c:2970) */
+            const nn_gn_t g = gn_out(u, &u->enc[i]);
+            if (nn_conv3d_fwd_x(u->enc[i].a2, &g, nullptr, nullptr, 0, 0, u->enc[i].ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
+            shape5 ds = u->ls[i + 1]; ds.c = u->cfg.widths[i];
+            note(u, u->downo[i], ds, dwn[i], nullptr, nullptr, 0);
+            cur = u->downo[i];
+        }
+    }
+    for (int i = L - 2; i >= 0; i--) {                             /* decoder: nothing materialised (src/unet.c:3010-3013) */
+        const block *coarse = i == L - 2 ? &u->enc[L - 1] : &u->dec[i + 1];
+        const nn_gn_t gc = gn_out(u, coarse), gs = gn_out(u, &u->enc[i]);
+        if (block_fwd(u, &u->dec[i], u->enc[i].a2, &gs, coarse->a2, &gc, u->cfg.widths[i + 1], dn1[i], dn2[i])) return -1;
+    }
+    const block *last = L > 1 ? &u->dec[0] : &u->enc[0];
+    const nn_gn_t g = gn_out(u, last);
+    nn_set_prec(0);
+    if (reg_here) nn_storage_forget(x);
+    return nn_conv3d_fwd_x(last->a2, &g, nullptr, nullptr, 0, 0, last->ys, P(u, u->head.w), P(u, u->head.b), u->cfg.head_out, 1, 1, logits, 0, 0.f, nullptr, nullptr);
+}
+int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, float *logits) {
+    if (u->in.n != 1 || u->cfg.cin != 4 || u->in.h != u->in.w) { fprintf(stderr, "unet_forward_ct: needs one square window of 4 input channels\n"); return -1; }
+    lp_pred_input_mx(ct, u->in.w, mean, isd, dyo, dxo, axis, 0, u->in.d, u->xin, 2, u->cfg.act_dt == 4 ? 4 : 8);      /* fp16-rounded input values, as predict */
+    return unet_forward_x(u, u->xin, logits);
+}
+int unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd) {
+    if (k < 0 || k >= u->nouts) return 0;
+    *mean = u->outs[k].mean; *rstd = u->outs[k].rstd;
+    return u->outs[k].G;
+}
+const void *unet_layer_out(const unet *u, int k, shape5 *s, const char **name) {
+    if (k < 0 || k >= u->nouts) return nullptr;
+    if (s) *s = u->outs[k].s;
+    if (name) *name = u->outs[k].name;
+    return u->outs[k].p;
+}
