@@ -27,6 +27,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target seconds of CPU work for the cpu_baseline sample")
+    ap.add_argument("--copy-probe", action="store_true", help="run 5 device-to-device copies of 1 GiB and exit: the known-size kernel that scales "
+                    "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards by windows / z-slabs, see DESIGN.md)" % a.gpus, file=sys.stderr)
@@ -36,6 +38,15 @@ def main():
     if lib.mi_init(0) != 0:
         print("bench.py: no gfx950 GPU: the HIP path cannot run (there is no CPU fallback)", file=sys.stderr)
         sys.exit(3)
+    if a.copy_probe:
+        nb = 1 << 30
+        src, dst = DevBuf(nb), DevBuf(nb)
+        lib.mi_zero(src.ptr, nb)
+        for _ in range(5):
+            lib.mi_d2d(dst.ptr, src.ptr, nb)
+        lib.mi_sync(); LP.check()
+        print(json.dumps({"copy_probe_bytes": nb, "copies": 5}))
+        return
     N, Cc, D, L, G = 2, 128, 64, 4, 8
     S = D * D * D
     rng = np.random.default_rng(0)

@@ -445,59 +445,75 @@ void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg
     MICK();
 }
 // decoder up segment (src/lp_common.cuh:618-670): coarse rows -> GN + SiLU -> e4m3 rows with a row scale (amax ignoring NaN) -> 8-term fp32
-// blend (weights .75 / .25, fma order z, y, x, the row scale folded into the weight) -> rows in the compute format at the fine resolution
-template <int BX, int BY>
-__global__ void __launch_bounds__(256) restage_up_k(const uint8_t *x, uint8_t *y, int N, int C, int D, int H, int W, gnp_t gp, int Cg) {
-    // x: C channels at (D/2, H/2, W/2); y: nbo * 32 channels at (D, H, W)
-    const int nbo = (C + 31) / 32, bwx = mx_bw(C), Cy = nbo * 32, Dc = D >> 1, Hc = H >> 1, Wc = W >> 1;
+// blend (weights .75 / .25, fma order z, y, x, the row scale folded into the weight) -> rows in the compute format at the fine resolution.
+// Two passes: the coarse rows are activated and re-quantised once (mi_restage into an MX-fp8 scratch tensor, an eighth of the output),
+// then up_blend_k forms the fine rows. A thread owns the 8 fine voxels whose blend reads one 2x2x2 cell of coarse rows, for 8 of the
+// block's 32 channels: cell (mz, my, mx), each in [-1, dim/2 - 1], covers coarse {m, m + 1} (clamped) and fine {2m + 1, 2m + 2}; the four
+// threads of a cell meet for the row amax through lane exchanges. Each coarse row is decoded once per cell instead of once per fine voxel.
+template <int BY>
+__global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y, int N, int nbo, int D, int H, int W) {
+    const int Dc = D >> 1, Hc = H >> 1, Wc = W >> 1;
     const size_t S = (size_t)D * H * W, Sc = (size_t)Dc * Hc * Wc;
-    const int nbk = blockIdx.y, n = nbk / nbo, blk = nbk % nbo;
-    __shared__ float ca[32], cb[32]; __shared__ int cg[32];
-    if (threadIdx.x < 32) {
-        const int k = threadIdx.x, c = blk * 32 + k;
-        float a = 1.f, b = 0.f; int g = 0;
-        if (gp.G && c < C) { const int ng = n * gp.G + c / (Cg / gp.G); a = gp.rstd[ng] * gp.gamma[c]; b = fmaf(-gp.mean[ng], a, gp.beta[c]); g = 1; }
-        ca[k] = a; cb[k] = b; cg[k] = g;
+    const int nbk = blockIdx.y;                                                   // (n, blk)
+    const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;
+    const int q = (int)(t & 3);
+    const size_t cell = t >> 2, ncx = (size_t)Wc + 1, ncy = (size_t)Hc + 1, ncz = (size_t)Dc + 1;
+    const bool live = cell < ncx * ncy * ncz;
+    const size_t cc = live ? cell : 0;
+    const int mx = (int)(cc % ncx) - 1, my = (int)((cc / ncx) % ncy) - 1, mz = (int)(cc / (ncx * ncy)) - 1;
+    const int cz[2] = {max(mz, 0), min(mz + 1, Dc - 1)}, cy[2] = {max(my, 0), min(my + 1, Hc - 1)}, cx[2] = {max(mx, 0), min(mx + 1, Wc - 1)};
+    const uint8_t *xs = xc + (size_t)N * nbo * Sc * 32;
+    float f[8][8], sc[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const size_t row = (size_t)nbk * Sc + ((size_t)cz[k >> 2] * Hc + cy[(k >> 1) & 1]) * Wc + cx[k & 1];
+        const uint2 w = *(const uint2 *)(xc + row * 32 + q * 8);
+        d_dec4_e4m3(w.x, f[k]); d_dec4_e4m3(w.y, f[k] + 4);
+        sc[k] = d_mx_scale(xs[row]);
     }
-    __syncthreads();
-    const size_t vo = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (vo >= S) return;
-    const int gx = (int)(vo % W), gy = (int)((vo / W) % H), gz = (int)(vo / ((size_t)W * H));
-    const int mz[2] = {gz >> 1, min(max((gz >> 1) + ((gz & 1) ? 1 : -1), 0), Dc - 1)}, my[2] = {gy >> 1, min(max((gy >> 1) + ((gy & 1) ? 1 : -1), 0), Hc - 1)},
-              mx[2] = {gx >> 1, min(max((gx >> 1) + ((gx & 1) ? 1 : -1), 0), Wc - 1)};
-    const uint8_t *sc = mx_scp<BX>(x, N, C, Sc);
-    float acc[32];
+    uint8_t *ys = y + (size_t)N * nbo * S * (BY * 4);
 #pragma unroll
-    for (int k = 0; k < 32; k++) acc[k] = 0.f;
+    for (int p = 0; p < 8; p++) {
+        const int pz = p >> 2, py = (p >> 1) & 1, px = p & 1;                     // fine voxel 2m + 1 + p: p = 0 has its own coarse row at m, p = 1 at m + 1
+        const int gz = 2 * mz + 1 + pz, gy = 2 * my + 1 + py, gx = 2 * mx + 1 + px;
+        float acc[8];
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+        for (int i = 0; i < 8; i++) acc[i] = 0.f;
 #pragma unroll
-        for (int bb = 0; bb < 2; bb++)
+        for (int a = 0; a < 2; a++)
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
-                float r[32];
-                const size_t cv = ((size_t)mz[a] * Hc + my[bb]) * Wc + mx[c];
-                if (bwx == 32) load_row<BX>(x, sc, ((size_t)n * mx_nb(C) + blk) * Sc + cv, 32, r); else load_row<BX>(x, sc, (size_t)n * Sc + cv, bwx, r);
+            for (int b = 0; b < 2; b++)
 #pragma unroll
-                for (int k = 0; k < 32; k++) if (cg[k]) r[k] = d_act_ab(r[k], ca[k], cb[k]);
-                unsigned am = 0u;
+                for (int c = 0; c < 2; c++) {
+                    const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);   // a = 0: the voxel's own coarse row, a = 1: its neighbour
+                    const float w3 = (a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f) * sc[k];
 #pragma unroll
-                for (int k = 0; k < 32; k++) { const unsigned u = __float_as_uint(fabsf(r[k])); am = u <= 0x7f800000u && u > am ? u : am; }
-                const int e = d_mx_exp(__uint_as_float(am), MI_INVQ8);
-                const float m = d_exp2i(-e);
-                const float w3 = (a ? 0.25f : 0.75f) * (bb ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f) * d_mx_scale((unsigned)(e + 127));
+                    for (int i = 0; i < 8; i++) acc[i] = fmaf(w3, f[k][i], acc[i]);
+                }
+        float am = 0.f;
 #pragma unroll
-                for (int k = 0; k < 32; k++) acc[k] = fmaf(w3, d_dec_e4m3(d_enc_e4m3(r[k] * m)), acc[k]);
-            }
-    store_row<BY, false>(y, mx_scp<BY>(y, N, Cy, S), (size_t)nbk * S + vo, 32, acc);
+        for (int i = 0; i < 8; i++) am = fmaxf(am, fabsf(acc[i]));
+        am = fmaxf(am, __shfl_xor(am, 1)); am = fmaxf(am, __shfl_xor(am, 2));
+        const int e = d_mx_exp(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
+        if (!live || gz < 0 || gz >= D || gy < 0 || gy >= H || gx < 0 || gx >= W) continue;
+        const size_t row = (size_t)nbk * S + ((size_t)gz * H + gy) * W + gx;
+        if (BY == 8) {
+            uint2 o; o.x = d_enc4_e4m3(acc[0], acc[1], acc[2], acc[3], e); o.y = d_enc4_e4m3(acc[4], acc[5], acc[6], acc[7], e);
+            *(uint2 *)(y + row * 32 + q * 8) = o;
+        } else *(unsigned *)(y + row * 16 + q * 4) = d_enc8_e2m1(acc, e);
+        if (!q) ys[row] = (uint8_t)(e + 127);
+    }
 }
 void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits) {
     const size_t S = (size_t)D * H * W; if (!S || !N) return;
-    const dim3 grid(nblk_(S, 256), (unsigned)(N * ((C + 31) / 32)));
-    const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
-#define RU(BX, BY) restage_up_k<BX, BY><<<grid, 256>>>(xq, yq, N, C, D, H, W, gp, Cg)
-    if (xdt == 4) { if (ybits == 4) RU(4, 4); else RU(4, 8); } else if (xdt == 3) { if (ybits == 4) RU(8, 4); else RU(8, 8); }
-    else mi_die("fused-upsample input must be an MX tensor (dtype %d)", xdt);
-#undef RU
+    if (xdt != 3 && xdt != 4) mi_die("fused-upsample input must be an MX tensor (dtype %d)", xdt);
+    if ((D | H | W) & 1) mi_die("fused-upsample output dims must be even (%d %d %d)", D, H, W);
+    const int nbo = (C + 31) / 32;
+    const size_t Sc = S / 8;
+    uint8_t *xc = (uint8_t *)mi_ws(MI_WS_UPCOARSE, (size_t)N * nbo * Sc * 33);
+    mi_restage(x, xdt, N, C, Sc, gp, Cg, 0, xc, 8);
+    const size_t cells = (size_t)(D / 2 + 1) * (H / 2 + 1) * (W / 2 + 1);
+    const dim3 grid(nblk_(cells * 4, 256), (unsigned)(N * nbo));
+    if (ybits == 4) up_blend_k<4><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W); else up_blend_k<8><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W);
     MICK();
 }
