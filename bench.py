@@ -17,7 +17,52 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 METRIC = "U-Net infer voxels/s (128^3 patch, MX fp8) + 3x3x3 conv % of MFMA peak"
+TRAFFIC_BYTES_PER_LAUNCH = 187.7e6     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/
 MFMA_PEAK_FP8_TFLOPS = 5033.0          # MI355X dense MXFP8 (2.5 PFLOP/s bf16 x 2)
+
+
+def unet_leg(np, lib, LP, DevBuf, steps, warmup):
+    """configs[3]: the reference-style U-Net forward (cin 4, widths 32/64/128/256, two 3x3x3 convs + GroupNorm + SiLU per level, 3x3x3 stride-2
+    downs, trilinear 2x fused into the decoder convs, skip concat, 1x1x1 head of 8 logits), N 2 x 128^3, MX-fp8 storage and compute, random
+    init, CT-like synthetic input already quantised and resident in HBM."""
+    from ufsm_amd.unet import UNet, make_cfg
+    N, D, widths = 2, 128, [32, 64, 128, 256]
+    S = D ** 3
+    net = UNet(make_cfg(4, widths, G=8, head_out=8, act_dt=8), N, D, D, D, seed=1)
+    rng = np.random.default_rng(3)
+    f = rng.standard_normal((N, D, D, D)).astype(np.float32)
+    for ax in (1, 2, 3):
+        f = (np.roll(f, 1, ax) + f + np.roll(f, -1, ax)) / 3                      # smoothed field -> sheet structure
+    sheet = np.sin(6 * f / f.std() + np.linspace(0, 8, D, dtype=np.float32)[None, None, None, :]) > 0
+    ct = np.clip(np.where(sheet, rng.normal(170, 20, f.shape), rng.normal(60, 20, f.shape)), 0, 255).astype(np.uint8).astype(np.float32)
+    x = np.zeros((N, 4, S), np.float32)
+    x[:, 0] = ((ct - ct.mean()) / ct.std()).reshape(N, S)
+    yy, xx = np.meshgrid(np.arange(D) - 300.0, np.arange(D) + 200.0, indexing="ij")
+    r = np.sqrt(yy * yy + xx * xx) + 1e-6
+    x[:, 2] = np.broadcast_to((yy / r)[None], (D, D, D)).reshape(1, S); x[:, 3] = np.broadcast_to((xx / r)[None], (D, D, D)).reshape(1, S)
+    dx = DevBuf.from_numpy(x)
+    dxq = DevBuf(lib.lp_mx8_bytes(N, 4, S)); lib.lp_f32_to_mx8(dx.ptr, N, 4, S, dxq.ptr)
+    dlog = DevBuf(N * 8 * S * 4)
+    for _ in range(warmup):
+        assert net.forward_x(dxq.ptr, dlog.ptr) == 0
+    lib.mi_sync(); LP.check()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        net.forward_x(dxq.ptr, dlog.ptr)
+    lib.mi_sync(); LP.check()
+    dt = (time.perf_counter() - t0) / steps
+    # conv FLOPs of one forward, logical channels, all taps (tests/bench_lp.c:46)
+    fl, lv = 0.0, [(D >> i) ** 3 for i in range(len(widths))]
+    for i, wd in enumerate(widths):
+        fl += 2 * 27 * ((4 if i == 0 else widths[i - 1]) * wd + wd * wd) * lv[i]      # encoder block
+        if i + 1 < len(widths):
+            fl += 2 * 27 * wd * wd * lv[i + 1]                                    # stride-2 down conv, width kept (src/unet.c:2970)
+            fl += 2 * 27 * ((widths[i + 1] + wd) * wd + wd * wd) * lv[i]          # decoder block on [up | skip]
+    fl += 2 * widths[0] * 8 * lv[0]
+    fl *= N
+    net.close()
+    return {"workload": "configs[3]: U-Net forward, N 2 x 128^3, widths 32/64/128/256, MX-fp8", "value": N * S / dt, "unit": "voxels/s", "ms_per_forward": dt * 1e3,
+            "steps": steps, "gflop_per_forward": fl / 1e9, "tflops": fl / dt / 1e12}
 
 
 def main():
@@ -27,6 +72,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target seconds of CPU work for the cpu_baseline sample")
+    ap.add_argument("--no-unet", action="store_true", help="skip the configs[3] U-Net forward leg")
     ap.add_argument("--copy-probe", action="store_true", help="run 5 device-to-device copies of 1 GiB and exit: the known-size kernel that scales "
                     "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
@@ -103,8 +149,14 @@ def main():
                    "layers": L, "batch": N, "channels": Cc, "dims": [D, D, D]},
         "tflops": L * flops_layer / (ms_step * 1e-3) / 1e12,
         "roofline": {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_FP8_TFLOPS,
-                     "launches": nl.value, "avg_launch_ms": k_ms, "flops_per_launch": flops_layer, "traffic": None},
+                     "launches": nl.value, "avg_launch_ms": k_ms, "flops_per_launch": flops_layer,
+                     # HBM-side bytes per launch: not measurable from inside the process; the figure of the committed counter runs
+                     # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy) for this kernel at this shape
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH, "traffic_source": "profiles/conv3_mx_f8_c128_64cube_hbm_traffic.txt",
+                     "algorithmic_bytes": 2 * N * (Cc // 32) * S * 33 + 28 * Cc * Cc * 33 // 32},
     }
+    if not a.no_unet:
+        out["unet"] = unet_leg(np, lib, LP, DevBuf, max(3, a.steps // 4), max(1, a.warmup))
     if not a.no_cpu_baseline:
         import orc
         # the oracle (a port: the reference has no CPU MX conv) on a bounded z-slab of one layer of the same workload
