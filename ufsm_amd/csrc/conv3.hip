@@ -44,7 +44,7 @@ __global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, i
 __host__ __device__ __forceinline__ int seg_ci(int cp, int Ci, int Cx, int CxP) { if (cp < CxP) return cp < Cx ? cp : -1; const int c = Cx + cp - CxP; return c < Ci ? c : -1; }
 template <int FMT>
 __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uint8_t *__restrict__ wq, unsigned *__restrict__ wsc, int Co, int Ci, int Cx, int CxP,
-                                               int nbt, int CB, int nmt_all, int npairs_all) {
+                                               int nbt, int CB, int nmt_all, int npairs_all, int block_major) {
     constexpr int WTILE = fmt_t<FMT>::WTILE;
     const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     const int Cop = nmt_all * 32;
@@ -59,7 +59,8 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
     for (int side = 0; side < 2; side++) {
         const int u = 2 * q + side;
         float v[32]; float amax = 0.f;
-        const int t = u / nbc, blk = b0 + u % nbc;
+        // K order inside a chunk: tap by tap over its blocks, or (the wide kernel, one chunk) block by block over the taps
+        const int t = block_major ? u % 27 : u / nbc, blk = block_major ? u / 27 : b0 + u % nbc;
 #pragma unroll
         for (int k = 0; k < 32; k++) {
             const int ci = seg_ci(blk * 32 + k, Ci, Cx, CxP);
@@ -164,6 +165,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         if (s == 0) a.nb0p = nbp;
     }
     a.nbt = a.nb0p + (sp.x2 ? (C2 + 31) / 32 : 0);
+    a.wide = a.bws[0] == 32 && (!sp.x2 || a.bws[1] == 32);
     a.N = N; a.D = D; a.H = H; a.W = W; a.Do = Do; a.Ho = Ho; a.Wo = Wo;
     a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
     a.osum = osum; a.Go = Go; a.stored_stats = sp.stored_stats && ybf >= 3; a.zs0 = sp.zlo; a.zs1 = Do - sp.zhi;
@@ -172,33 +174,67 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const int nmt_all = (cout + 31) / 32;
     int MT = nmt_all <= 4 ? nmt_all : nmt_all % 4 == 0 ? 4 : nmt_all % 3 == 0 ? 3 : nmt_all % 2 == 0 ? 2 : 1;
     int NT = (stride == 1 && MT <= 2 && Do >= 4) ? 4 : 2;
+    // 128-channel output slices at stride 1 take the wide kernel (16 accumulators per wavefront, one workgroup per CU)
+    static int big_env = -1;
+    if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel
+    bool big = big_env && stride == 1 && MT == 4 && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
+    if (big) {
+        // The wide kernel streams input block b >= 2 of a tile into LDS while the tile's earlier blocks are multiplied, one copy round per
+        // stage of two pairs, NRND rounds per block, a block starting once block b - 3 has been read for the last time (pair (27 (b - 3) + 26) / 2).
+        // A round issued in stage s is visible two barriers later. Check that every block lands before the step that first fetches from it.
+        const int NRND = ((6 * 10 * 18 + 63) / 64 + 3) / 4, npairs = (27 * a.nbt + 1) >> 1, nfull = npairs >> 1;
+        int fbi = 2, frd = 0;
+        for (int s = 0; s < nfull && big; s++) {
+            if (fbi < a.nbt && (fbi < 3 || ((27 * (fbi - 3) + 26) >> 1) <= 2 * s + 1) && ++frd == NRND) {
+                const int pf = ((27 * fbi) >> 1) - 1;               // the pair during which the block's first fragments are fetched
+                const int need = pf & 1 ? (pf >> 1) - 2 : (pf >> 1) - 3;
+                if (s > need) big = false;
+                frd = 0; fbi++;
+            }
+        }
+        if (fbi < a.nbt) big = false;
+    }
+    if (big) NT = 4;
     const int TZ = NT == 2 ? 2 : 4;
     const int HZ = stride * (TZ - 1) + 3, HY = stride * 7 + 3, HX = stride * 15 + 3, TT = HZ * HY * HX;
     const int RB = fmt == 8 ? 32 : 16, WTILE = fmt == 8 ? 2048 : 1024;
     // LDS of a workgroup holding CB input blocks: weight ring, pair table, halo rows and scale words. Prefer the largest CB that
-    // still lets two workgroups share a CU (160 KB): the second one computes while the first stages its halo or runs its epilogue
+    // still lets two workgroups share a CU (160 KB): the second one computes while the first stages its halo or runs its epilogue.
+    // The wide kernel has a fixed layout: ring of two slots of two pairs, three halo slots of one block, two pair tables.
     auto lds_bytes = [&](int cb) { return (size_t)2 * MT * (WTILE + 256) + (size_t)(((27 * cb + 1) >> 1) + 2) * 32 + (size_t)cb * TT * (RB + 4); };
     int cb2 = 0, cb1 = 0;
-    for (int cb = 1; cb <= a.nbt; cb++) { if (lds_bytes(cb) <= 80 * 1024) cb2 = cb; if (lds_bytes(cb) <= 160 * 1024 - 256) cb1 = cb; }
+    for (int cb = 1; cb <= a.nbt; cb++) { if (lds_bytes(cb) <= 80 * 1024 - 2816) cb2 = cb; if (lds_bytes(cb) <= 160 * 1024 - 3072) cb1 = cb; }   // (room for the epilogue's constants and scratch)
     int cbmax = cb2 ? cb2 : cb1;
     static int cb_env = -1;
     if (cb_env < 0) cb_env = getenv("MI_CONV_CB") ? atoi(getenv("MI_CONV_CB")) : 0;      // tuning knob: blocks per chunk
     if (cb_env > 0 && cb_env <= cb1) cbmax = cb_env;
     if (cbmax < 1) mi_die("%s: tile does not fit LDS", who);
     const int nchunks = (a.nbt + cbmax - 1) / cbmax;
-    a.CB = (a.nbt + nchunks - 1) / nchunks;
-    size_t smem = lds_bytes(a.CB);
-    const size_t red_bytes = (size_t)4 * 32 * 2 * sizeof(float);     // (the larger of the quad and per-channel statistics scratch)
-    if (smem < red_bytes) smem = red_bytes;
+    a.CB = big ? a.nbt : (a.nbt + nchunks - 1) / nchunks; // (the wide kernel has no chunks: its K loop walks block by block)
+    size_t smem = big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     smem = (smem + 15) & ~(size_t)15;
+    a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);      // bias, affine a, b of the workgroup's channels
+    a.red_o = (unsigned)smem; smem += 1024;                                     // statistics scratch
+    if (big) {
+        // rows and scale bytes of positions outside the volume: 64 zero bytes, then 64 bytes of value 1; one page per device, kept for the process
+        static uint8_t *zpage[8];
+        int dv = 0; MIRT(hipGetDevice(&dv)); dv &= 7;
+        if (!zpage[dv]) {
+            uint8_t init[128]; memset(init, 0, 64); memset(init + 64, 1, 64);
+            MIRT(hipMalloc((void **)&zpage[dv], 128));
+            if (!zpage[dv]) mi_die("%s: no device memory for the constant page", who);
+            MIRT(hipMemcpy(zpage[dv], init, 128, hipMemcpyHostToDevice));
+        }
+        a.zpage = zpage[dv];
+    }
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
     a.ntx = (Wo + 15) / 16; a.nty = (Ho + 7) / 8; a.ntz = (Do + TZ - 1) / TZ;
     a.ntiles = (unsigned)((size_t)a.ntx * a.nty * a.ntz * a.ncs * N);
     // ---- weights ----
     int npairs_all = 0;
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) npairs_all += (27 * (a.nbt - b0 < a.CB ? a.nbt - b0 : a.CB) + 1) >> 1;
-    // (four stages of padding: the kernel's weight loads run up to three pairs ahead of the last one)
-    const size_t wq_bytes = (size_t)(npairs_all + 4) * nmt_all * WTILE, wsc_bytes = (size_t)(npairs_all + 4) * nmt_all * 256;
+    // (eight pairs of padding: the kernels' weight loads run up to seven pairs ahead of the last one)
+    const size_t wq_bytes = (size_t)(npairs_all + 8) * nmt_all * WTILE, wsc_bytes = (size_t)(npairs_all + 8) * nmt_all * 256;
     const int CxP = (Cx + 31) / 32 * 32;
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
@@ -214,8 +250,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) {
         const size_t nt = (size_t)npairs_all * nmt_all * 32;
-        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all);
-        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all);
+        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? 1 : 0);
+        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? 1 : 0);
         MICK();
     }
     a.wq = wq; a.wsc = wsc;

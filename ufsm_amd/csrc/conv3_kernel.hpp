@@ -31,15 +31,62 @@
 template <int... Is, typename F> __device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>) { (f(std::integral_constant<int, Is>{}), ...); }
 template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
 
+// ---- lane exchanges without LDS addressing: l ^ 32 by v_permlane32_swap (after swapping x with itself the first result holds the low half
+// twice, the second the high half twice), l ^ 1 and l ^ 2 by DPP quad permutes, l ^ 4 / 8 / 16 by ds_swizzle's bit mode ----
+__device__ __forceinline__ unsigned lane_xor32(unsigned x, int h) {
+    const auto r2 = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+    return h ? r2[0] : r2[1];
+}
+__device__ __forceinline__ float lane_xor32f(float x, int h) { return __uint_as_float(lane_xor32(__float_as_uint(x), h)); }
+template <int MASK> __device__ __forceinline__ float lane_xorf(float x) {
+    static_assert(MASK == 1 || MASK == 2 || MASK == 4 || MASK == 8 || MASK == 16, "lane_xorf mask");
+    const int xi = (int)__float_as_uint(x);
+    int y;
+    if constexpr (MASK == 1) y = __builtin_amdgcn_mov_dpp(xi, 0xB1, 0xF, 0xF, true);          // quad_perm [1, 0, 3, 2]
+    else if constexpr (MASK == 2) y = __builtin_amdgcn_mov_dpp(xi, 0x4E, 0xF, 0xF, true);     // quad_perm [2, 3, 0, 1]
+    else y = __builtin_amdgcn_ds_swizzle(xi, (MASK << 10) | 0x1f);                            // and 0x1f, or 0, xor MASK within 32 lanes
+    return __uint_as_float((unsigned)y);
+}
+// Sums NV (a power of two <= 32) per-lane values over the 32 lanes of each wavefront half in a fixed order. Step k pairs lane r with
+// r ^ 2^k; while more than one value is left the pair splits them (the lane whose bit k is clear keeps the lower half of the indices and
+// receives the partner's lower half), so every step moves half as much as the one before. Returns the index of the value whose total
+// the lane ends with in v[0]: sum over k of bit k of r times NV >> (k + 1); lanes with a set bit at or above log2(NV) hold duplicates.
+template <int NV>
+__device__ __forceinline__ int wave_half_reduce(float (&v)[NV], int r) {
+    int idx = 0;
+    static_for<5>([&](auto K) {
+        constexpr int k = decltype(K)::value, nk = NV >> k;           // values left before this step (0: already one)
+        const bool bit = (r >> k) & 1;
+        if constexpr (nk >= 2) {
+            constexpr int half = nk / 2;
+#pragma unroll
+            for (int i = 0; i < half; i++) {
+                const float send = bit ? v[i] : v[i + half], keep = bit ? v[i + half] : v[i];
+                v[i] = keep + lane_xorf<(1 << k)>(send);
+            }
+            idx += bit ? half : 0;
+        } else v[0] += lane_xorf<(1 << k)>(v[0]);
+    });
+    return idx;
+}
+
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+
+#ifdef DBG_TIMING
+__device__ long long g_dbg[64];
+#define DBG_MARK(i) do { if (blockIdx.x == 8 && threadIdx.x == 0) g_dbg[i] = (long long)__builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define DBG_MARK(i) do { } while (0)
+#endif
 
 struct conv_args {
     const uint8_t *xq[2], *xsc[2];     // input segments (compute-format MX tensors): data, scale plane
     int nbs[2], bws[2];                // blocks per sample and block width of each segment's tensor
     int nb0p;                          // padded blocks of segment 0 (staged blocks [0, nb0p) come from segment 0)
     int nbt, CB;                       // staged 32-channel blocks in total, blocks per LDS chunk
+    int wide;                          // every staged tensor has 32-channel blocks
     int N, D, H, W, Do, Ho, Wo;
     const uint8_t *wq, *wsc; int nmt_all;
     const float *bias; int Co;
@@ -47,6 +94,9 @@ struct conv_args {
     double *osum; float *part; int Go, stored_stats, zs0, zs1;   // part: per tile and channel quad (sum, sum of squares)
     int stat_ch;                       // 1: per-channel records (channels per group not a multiple of 4; Co <= 32 only)
     const float *ep_a, *ep_b; int act;
+    unsigned epi_o;                    // LDS byte offset of the epilogue's per-channel constants: bias, then ep_a, ep_b (MT x 32 floats each)
+    unsigned red_o;                    // LDS byte offset of the statistics scratch (1 KiB)
+    const uint8_t *zpage;              // device memory: 64 zero bytes, then 64 bytes of value 1 (rows and scale bytes of positions outside the volume)
     int ntx, nty, ntz, ncs; unsigned ntiles;
 };
 
@@ -55,6 +105,299 @@ template <> struct fmt_t<8> { static constexpr int RB = 32, NH = 2, WTILE = 2048
 template <> struct fmt_t<4> { static constexpr int RB = 16, NH = 1, WTILE = 1024; };
 
 __device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678f)); }
+
+// geometry of a workgroup's halo: output tile TZ x 8 x 16, input halo HZ x HY x HX positions
+template <int FMT, int STRIDE, int TZ> struct halo_t {
+    static constexpr int HZ = STRIDE * (TZ - 1) + 3, HY = STRIDE * 7 + 3, HX = STRIDE * 15 + 3, TT = HZ * HY * HX, NH = fmt_t<FMT>::NH;
+};
+
+// ---- pair table: per pair and lane half, the byte offsets of the pair's two units (fp8: both; fp4: the half's own) and of
+// the half's scale word. unit u = (tap u / nbc, local block u % nbc); the odd padding unit (zero weights) re-reads unit A ----
+template <int FMT, int STRIDE, int TZ>
+__device__ __forceinline__ void conv_pair_table(unsigned char *lds, unsigned tab_o, int nbc, int tid) {
+    using HL = halo_t<FMT, STRIDE, TZ>;
+    constexpr int HY = HL::HY, HX = HL::HX, TT = HL::TT, NH = HL::NH;
+    const int nunits = 27 * nbc, npairs = (nunits + 1) >> 1;
+    for (int i = tid; i < (npairs + 2) * 2; i += 256) {
+        const int q = min(i >> 1, npairs - 1), hh = i & 1;
+        const int uA = 2 * q, uB = 2 * q + 1 < nunits ? 2 * q + 1 : 2 * q;
+        const int tA = uA / nbc, bA = uA - tA * nbc, tB = uB / nbc, bB = uB - tB * nbc;
+        const int pA = ((tA / 9) * HY + (tA / 3) % 3) * HX + tA % 3, pB = ((tB / 9) * HY + (tB / 3) % 3) * HX + tB % 3;
+        const int dA = (bA * NH * TT + pA) * 16, dB = (bB * NH * TT + pB) * 16, sA = (bA * TT + pA) * 4, sB = (bB * TT + pB) * 4;
+        *(v4i *)(lds + tab_o + i * 16) = (v4i){NH == 2 ? dA : (hh ? dB : dA), dB, hh ? sB : sA, 0};
+    }
+}
+
+// ---- stage the halo of blocks [b0, b0 + nbc): rows copied as stored, zero rows (scale byte 1) outside the tensor.
+// A thread owns up to NE (position, 16-byte half) elements and NS scale positions of the tile, the same for every block, so
+// the index arithmetic is done once and each block costs one address add per element. Loads read a clamped in-tensor
+// address and are zeroed afterwards when the position is outside: no divergent branches. The rows and scale bytes of GB blocks
+// are requested before any of them is written to LDS: one memory round trip per GB blocks. WIDE: all staged tensors have 32-channel
+// blocks (anything but a stored tensor of <= 16 channels read as it is); the narrow-row cases branch per element ----
+template <int FMT, int STRIDE, int TZ, int GB, bool WIDE>
+__device__ __forceinline__ void conv_stage_halo(const conv_args &a, unsigned char *lds, unsigned act_o, unsigned asc_o, int b0, int nbc, int n,
+                                                int iz0, int iy0, int ix0, int tid) {
+    using HL = halo_t<FMT, STRIDE, TZ>;
+    constexpr int HY = HL::HY, HX = HL::HX, TT = HL::TT, NH = HL::NH;
+    constexpr int NE = (TT * NH + 255) / 256, NS = (TT + 255) / 256;
+    const size_t Sin = (size_t)a.D * a.H * a.W;
+    unsigned eoff[NE]; unsigned edst[NE]; bool eok[NE];
+#pragma unroll
+    for (int k = 0; k < NE; k++) {
+        const int i = min(tid + k * 256, TT * NH - 1), pos = i / NH, hf = i - pos * NH;
+        const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
+        const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
+        eok[k] = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
+        const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1);
+        eoff[k] = (unsigned)((cz * a.H + cy) * a.W + cx) * 2u + (unsigned)hf;     // voxel index and half
+        edst[k] = act_o + (hf * TT + pos) * 16;
+    }
+    unsigned soff[NS]; bool sok[NS];
+#pragma unroll
+    for (int k = 0; k < NS; k++) {
+        const int pos = min(tid + k * 256, TT - 1);
+        const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
+        const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
+        sok[k] = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
+        const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1);
+        soff[k] = (unsigned)((cz * a.H + cy) * a.W + cx);
+    }
+    for (int bl0 = 0; bl0 < nbc; bl0 += GB) {
+        v4i val[GB][NE]; bool ok[GB][NE]; unsigned sv[GB][NS]; bool bokg[GB];
+#pragma unroll
+        for (int g = 0; g < GB; g++) {
+            const int bl = min(bl0 + g, nbc - 1);        // (a group's tail re-reads the last block and is not stored)
+            const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
+            const int rb = a.bws[seg] * FMT / 8;         // stored row bytes (16 NH for 32-wide blocks)
+            const bool bok = blk < a.nbs[seg];
+            bokg[g] = bok;
+            const uint8_t *base = a.xq[seg] + ((size_t)n * a.nbs[seg] + min(blk, a.nbs[seg] - 1)) * Sin * rb;
+#pragma unroll
+            for (int k = 0; k < NE; k++) {
+                const unsigned vox = eoff[k] >> 1, hf = NH == 2 ? (eoff[k] & 1u) : 0u;
+                if (WIDE) {                              // every staged tensor has 32-channel blocks: straight-line loads, all in flight together
+                    val[g][k] = *(const v4i *)(base + (size_t)vox * (16 * NH) + hf * 16);
+                    ok[g][k] = eok[k] && bok;
+                } else if (rb >= 16) {
+                    const bool have = rb >= (int)(hf + 1) * 16;
+                    val[g][k] = *(const v4i *)(base + (size_t)vox * rb + (have ? hf * 16 : 0));
+                    ok[g][k] = eok[k] && bok && have;
+                } else {                                 // 8- or 4-byte rows of a <= 8 / <= 16 channel tensor: only half 0 holds data
+                    val[g][k] = (v4i){0, 0, 0, 0};
+                    if (rb == 8) { const int2 t = *(const int2 *)(base + (size_t)vox * 8); val[g][k][0] = t.x; val[g][k][1] = t.y; }
+                    else val[g][k][0] = *(const int *)(base + (size_t)vox * 4);
+                    ok[g][k] = eok[k] && bok && hf == 0;
+                }
+            }
+            const uint8_t *sbase = a.xsc[seg] + ((size_t)n * a.nbs[seg] + min(blk, a.nbs[seg] - 1)) * Sin;
+#pragma unroll
+            for (int k = 0; k < NS; k++) sv[g][k] = sbase[soff[k]];
+        }
+#pragma unroll
+        for (int g = 0; g < GB; g++) {
+            const int bl = bl0 + g;
+            if (bl < nbc) {
+#pragma unroll
+                for (int k = 0; k < NE; k++)
+                    if (tid + k * 256 < TT * NH) *(v4i *)(lds + edst[k] + bl * NH * TT * 16) = ok[g][k] ? val[g][k] : (v4i){0, 0, 0, 0};
+#pragma unroll
+                for (int k = 0; k < NS; k++)
+                    if (tid + k * 256 < TT) *(unsigned *)(lds + asc_o + (bl * TT + tid + k * 256) * 4) = sok[k] && bokg[g] ? sv[g][k] : 1u;
+            }
+        }
+    }
+}
+
+// the epilogue's per-channel constants of the workgroup's MT x 32 channels -> LDS (padding channels: bias 0, affine 1, 0); read after a barrier
+template <int MT, bool EPI>
+__device__ __forceinline__ void conv_epi_consts(const conv_args &a, unsigned char *lds, int cs, int tid) {
+    if (tid < MT * 32) {
+        const int co = cs * MT * 32 + tid;
+        float *p = (float *)(lds + a.epi_o);
+        p[tid] = a.bias && co < a.Co ? a.bias[co] : 0.f;
+        if (EPI) { p[MT * 32 + tid] = a.ep_a && co < a.Co ? a.ep_a[co] : 1.f; p[MT * 64 + tid] = a.ep_a && co < a.Co ? a.ep_b[co] : 0.f; }
+    }
+}
+
+// ---- epilogue (src/lp_common.cuh:1465-1597): bias -> optional affine + activation -> per (voxel, 32-channel block) amax across the
+// lane pair (l, l ^ 32) -> E8M0 exponent -> codes -> row stores; GroupNorm partial sums per tile. acc: the wavefront's MT x NT accumulators;
+// lane (r, h) of tile j holds voxel (oz0 + lz, oy0 + ly0 + 2 j + (r >> 4), ox0 + (r & 15)) ----
+template <int MT, int NT, int OUT, bool EPI, bool PIN = false>
+__device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT][NT], unsigned char *lds, unsigned tile, int n, int cs,
+                                              int oz0, int oy0, int ox0, int lz, int ly0, int tid) {
+    const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    // accumulator layout of the 32x32 MFMA: lane (r = voxel within the tile, h), register i -> channel (i & 3) + 4 h + 8 (i >> 2)
+    const size_t So = (size_t)a.Do * a.Ho * a.Wo;
+    const int co_base = cs * MT * 32;
+    float *red = (float *)(lds + a.red_o);          // stats scratch [4 waves][MT][8 quads][2] floats
+    const bool stats = a.osum != nullptr;
+    float qs[MT][4], qss[MT][4];                    // per lane: sums over its voxels of the 4-channel quads (m, i >> 2)
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) { qs[m][q4] = 0.f; qss[m][q4] = 0.f; }
+    float chs[MT == 1 ? 16 : 1], chss[MT == 1 ? 16 : 1];     // per-channel sums (MT 1, stat_ch)
+#pragma unroll
+    for (int i = 0; i < (MT == 1 ? 16 : 1); i++) { chs[i] = 0.f; chss[i] = 0.f; }
+    constexpr int YB = OUT == 4 ? 4 : 8;
+    const int bwo = mx_bw(a.Co), nbo = mx_nb(a.Co), rbo = mx_rb(bwo, YB);
+    uint8_t *yq = (uint8_t *)a.y, *ysc = yq + (size_t)a.N * nbo * So * rbo;
+    static_for<MT>([&](auto M) {
+        constexpr int m = M;
+        DBG_MARK(16 + m);
+        // the lane's 16 channels of tile m are four runs of 4: (i & 3) + 4 h + 8 (i >> 2)
+        float bias[16], ea[16], eb[16];
+#pragma unroll
+        for (int q4 = 0; q4 < 4; q4++) {
+            const unsigned o = a.epi_o + (m * 32 + 8 * q4 + 4 * h) * 4;
+            const float4 b4 = *(const float4 *)(lds + o);
+            bias[4 * q4] = b4.x; bias[4 * q4 + 1] = b4.y; bias[4 * q4 + 2] = b4.z; bias[4 * q4 + 3] = b4.w;
+            if (EPI) {
+                const float4 a4 = *(const float4 *)(lds + o + MT * 128), e4 = *(const float4 *)(lds + o + MT * 256);
+                ea[4 * q4] = a4.x; ea[4 * q4 + 1] = a4.y; ea[4 * q4 + 2] = a4.z; ea[4 * q4 + 3] = a4.w;
+                eb[4 * q4] = e4.x; eb[4 * q4 + 1] = e4.y; eb[4 * q4 + 2] = e4.z; eb[4 * q4 + 3] = e4.w;
+            }
+        }
+        static_for<NT>([&](auto J) {
+            constexpr int j = J;
+            const int oz = oz0 + lz, oy = oy0 + ly0 + 2 * j + (r >> 4), ox = ox0 + (r & 15);
+            const bool ok = oz < a.Do && oy < a.Ho && ox < a.Wo;
+            const size_t ov = ((size_t)oz * a.Ho + oy) * a.Wo + ox;
+            const bool zst = ok && oz >= a.zs0 && oz < a.zs1;
+            float v[16];
+            float am = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                float av = acc[m][j][i];
+                if (PIN) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(av) : "a"(acc[m][j][i]));   // the accumulators stay in AGPRs until their tile's turn
+                float t = av + bias[i];                       // (padding channels: zero weights and no bias, so they stay 0)
+                if (EPI) {
+                    t = fmaf(t, ea[i], eb[i]);
+                    t = a.act == 1 ? __fdividef(t, 1.f + __expf(-t)) : a.act == 2 ? gelu_erf(t) : a.act == 3 ? fmaxf(t, 0.f) : t;
+                    if (co_base + m * 32 + (i & 3) + 4 * h + 8 * (i >> 2) >= a.Co) t = 0.f;
+                }
+                v[i] = t; am = fmaxf(am, fabsf(t));
+            }
+            if (OUT != 0) {
+                am = fmaxf(am, lane_xor32f(am, h));
+                const int e = d_mx_exp(am, YB == 8 ? MI_INVQ8 : MI_INVQ4);
+                const int blk = (co_base + m * 32) / bwo;                  // bwo < 32 only when Co <= 16: one tile, block 0
+                const size_t row = ((size_t)n * nbo + blk) * So + ov;
+                if (OUT == 8) {
+                    unsigned d[4];
+#pragma unroll
+                    for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc4_e4m3(v[4 * q4], v[4 * q4 + 1], v[4 * q4 + 2], v[4 * q4 + 3], e);
+                    if (a.stored_stats) {
+                        const float sc = d_exp2i(e);
+#pragma unroll
+                        for (int q4 = 0; q4 < 4; q4++) d_dec4_e4m3(d[q4], v + 4 * q4);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) v[i] *= sc;
+                    }
+                    // lane h = 0 holds bytes {0-3, 8-11, 16-19, 24-27}, its partner {4-7, 12-15, 20-23, 28-31}: swap so each stores 16 contiguous bytes
+                    const unsigned s0 = h ? d[0] : d[2], s1 = h ? d[1] : d[3];
+                    const unsigned r0 = lane_xor32(s0, h), r1 = lane_xor32(s1, h);
+                    const uint4 out = h ? make_uint4(r0, d[2], r1, d[3]) : make_uint4(d[0], r0, d[1], r1);
+                    if (ok) {
+                        if (bwo == 32) *(uint4 *)(yq + row * 32 + 16 * h) = out;
+                        else if (bwo == 16) { if (!h) *(uint4 *)(yq + row * 16) = out; }
+                        else if (!h) *(uint2 *)(yq + row * 8) = make_uint2(out.x, out.y);
+                    }
+                } else {
+                    unsigned hw[4];   // 4 channels -> 16 bits each
+                    {
+                        const unsigned w01 = d_enc8_e2m1(v, e), w23 = d_enc8_e2m1(v + 8, e);
+                        hw[0] = w01 & 0xffffu; hw[1] = w01 >> 16; hw[2] = w23 & 0xffffu; hw[3] = w23 >> 16;
+                        if (a.stored_stats) {
+                            const float sc = d_exp2i(e);
+                            d_dec8_e2m1(w01, v); d_dec8_e2m1(w23, v + 8);
+#pragma unroll
+                            for (int i = 0; i < 16; i++) v[i] *= sc;
+                        }
+                    }
+                    // halfword q4 of lane h sits at byte 4 q4 + 2 h of the 16-byte row: lane 0 assembles words 0-1, lane 1 words 2-3
+                    const unsigned mine01 = hw[0] | (hw[1] << 16), mine23 = hw[2] | (hw[3] << 16);
+                    const unsigned send = h ? mine01 : mine23, recv = lane_xor32(send, h);
+                    uint2 out;
+                    if (!h) out = make_uint2((hw[0] & 0xffffu) | ((recv & 0xffffu) << 16), (hw[1] & 0xffffu) | (recv & 0xffff0000u));
+                    else out = make_uint2((recv & 0xffffu) | ((hw[2] & 0xffffu) << 16), (recv >> 16) | ((hw[3] & 0xffffu) << 16));
+                    if (ok) {
+                        if (bwo == 32) *(uint2 *)(yq + row * 16 + 8 * h) = out;
+                        else if (bwo == 16) { if (!h) *(uint2 *)(yq + row * 8) = out; }
+                        else if (!h) *(unsigned *)(yq + row * 4) = out.x;
+                    }
+                }
+                if (ok && !h) ysc[row] = (uint8_t)(e + 127);
+            } else {
+                const size_t o0 = ((size_t)n * a.Co + co_base + m * 32 + 4 * h) * So + ov;
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int cl = (i & 3) + 8 * (i >> 2);            // channel offset from co_base + 32 m + 4 h
+                    const bool cok = ok && co_base + m * 32 + 4 * h + cl < a.Co;
+                    if (a.ydt == 2) {
+                        if (a.Go > 0) v[i] = fabsf(v[i]) > 65504.f ? copysignf(65504.f, v[i]) : v[i];     // src/lp_common.cuh:465, :1567-1569
+                        if (cok) ((__half *)a.y)[o0 + (size_t)cl * So] = __float2half(v[i]);
+                    } else if (cok) ((float *)a.y)[o0 + (size_t)cl * So] = v[i];
+                }
+            }
+            if (stats && zst) {
+                if (MT == 1 && a.stat_ch) {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) { chs[i] += v[i]; chss[i] += v[i] * v[i]; }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 16; i++) { qs[m][i >> 2] += v[i]; qss[m][i >> 2] += v[i] * v[i]; }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);       // one accumulator tile at a time: hoisting the next tiles' reads only costs registers
+        });
+    });
+    DBG_MARK(20);
+    if (stats) __syncthreads();
+    DBG_MARK(21);
+    if (MT == 1 && stats && a.stat_ch) {
+        // any group size (one channel tile): per-channel sums over the 32 voxel lanes, then over the waves; channel of register i of
+        // half h = (i & 3) + 4 h + 8 (i >> 2); value index 2 i + t (t 0 sum, 1 sum of squares)
+        float v[32];
+#pragma unroll
+        for (int i = 0; i < 16; i++) { v[2 * i] = chs[i]; v[2 * i + 1] = chss[i]; }
+        const int idx = wave_half_reduce<32>(v, r), i = idx >> 1;
+        red[(wave * 32 + (i & 3) + 4 * h + 8 * (i >> 2)) * 2 + (idx & 1)] = v[0];
+        __syncthreads();
+        if (tid < 32) {
+            float s1 = 0.f, s2 = 0.f;
+            for (int w = 0; w < 4; w++) { s1 += red[(w * 32 + tid) * 2]; s2 += red[(w * 32 + tid) * 2 + 1]; }
+            a.part[((size_t)tile * 32 + tid) * 2] = s1; a.part[((size_t)tile * 32 + tid) * 2 + 1] = s2;
+        }
+    } else if (stats) {
+        // channels per group a multiple of 4: a quad (m, q4, h) = channels co_base + 32 m + 8 q4 + 4 h .. +3 lies in one group.
+        // Sum over the 32 voxel lanes of each half (fixed order), then over the 4 waves in wave order; value index (4 m + q4) 2 + t
+        constexpr int NV = MT <= 1 ? 8 : MT <= 2 ? 16 : 32;
+        float v[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) v[i] = 0.f;
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) { v[(4 * m + q4) * 2] = qs[m][q4]; v[(4 * m + q4) * 2 + 1] = qss[m][q4]; }
+        const int idx = wave_half_reduce<NV>(v, r);
+        if ((r >> (NV == 8 ? 3 : NV == 16 ? 4 : 5)) == 0 && idx < MT * 8) {
+            const int mq = idx >> 1;                                    // 4 m + q4
+            red[((wave * MT + (mq >> 2)) * 8 + (mq & 3) * 2 + h) * 2 + (idx & 1)] = v[0];
+        }
+        __syncthreads();
+        if (tid < MT * 8) {
+            // per tile and channel quad, the sums over the tile's voxels in wave order; a second kernel adds the tiles of a sample
+            // in a fixed order into the exact sum slots, so the statistics do not depend on the order workgroups finish in
+            const int m = tid >> 3, q8 = tid & 7;                       // q8 = q4 * 2 + h: channels co_base + 32 m + 8 q4 + 4 h .. + 3
+            float s = 0.f, ss = 0.f;
+            for (int w = 0; w < 4; w++) { s += red[((w * MT + m) * 8 + q8) * 2]; ss += red[((w * MT + m) * 8 + q8) * 2 + 1]; }
+            a.part[((size_t)tile * MT * 8 + tid) * 2] = s;
+            a.part[((size_t)tile * MT * 8 + tid) * 2 + 1] = ss;
+        }
+    }
+    DBG_MARK(22);
+}
 
 // FMT: compute format (8 e4m3, 4 e2m1); OUT: 8 / 4 = MX-fp8 / MX-fp4 rows, 0 = fp32 or fp16 planes; EPI: fused affine + activation
 template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI>
@@ -107,88 +450,16 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
 
-    const size_t Sin = (size_t)a.D * a.H * a.W;
     const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 256;
     int pair0 = 0;                                       // global pair index of the chunk's first pair
+    conv_epi_consts<MT, EPI>(a, lds, cs, tid);
 
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) {
         const int nbc = min(a.CB, a.nbt - b0), nunits = 27 * nbc, npairs = (nunits + 1) >> 1;
         __syncthreads();                                 // the previous chunk's readers are done with the halo
-        // ---- pair table: per pair and lane half, the byte offsets of the pair's two units (fp8: both; fp4: the half's own) and of
-        // the half's scale word. unit u = (tap u / nbc, local block u % nbc); the odd padding unit (zero weights) re-reads unit A ----
-        for (int i = tid; i < (npairs + 2) * 2; i += 256) {
-            const int q = min(i >> 1, npairs - 1), hh = i & 1;
-            const int uA = 2 * q, uB = 2 * q + 1 < nunits ? 2 * q + 1 : 2 * q;
-            const int tA = uA / nbc, bA = uA - tA * nbc, tB = uB / nbc, bB = uB - tB * nbc;
-            const int pA = ((tA / 9) * HY + (tA / 3) % 3) * HX + tA % 3, pB = ((tB / 9) * HY + (tB / 3) % 3) * HX + tB % 3;
-            const int dA = (bA * NH * TT + pA) * 16, dB = (bB * NH * TT + pB) * 16, sA = (bA * TT + pA) * 4, sB = (bB * TT + pB) * 4;
-            *(v4i *)(lds + tab_o + i * 16) = (v4i){NH == 2 ? dA : (hh ? dB : dA), dB, hh ? sB : sA, 0};
-        }
-#ifndef DBG_NOSTAGE
-        // ---- stage the halo of blocks [b0, b0 + nbc): rows copied as stored, zero rows (scale byte 1) outside the tensor.
-        // A thread owns up to NE (position, 16-byte half) elements and NS scale positions of the tile, the same for every block, so
-        // the index arithmetic is done once and each block costs one address add per element. Loads read a clamped in-tensor
-        // address and are zeroed afterwards when the position is outside: no divergent branches, all loads of a block in flight ----
-        {
-            constexpr int NE = (TT * NH + 255) / 256, NS = (TT + 255) / 256;
-            unsigned eoff[NE]; unsigned edst[NE]; bool eok[NE];
-#pragma unroll
-            for (int k = 0; k < NE; k++) {
-                const int i = min(tid + k * 256, TT * NH - 1), pos = i / NH, hf = i - pos * NH;
-                const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
-                const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
-                eok[k] = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
-                const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1);
-                eoff[k] = (unsigned)((cz * a.H + cy) * a.W + cx) * 2u + (unsigned)hf;     // voxel index and half
-                edst[k] = act_o + (hf * TT + pos) * 16;
-            }
-            for (int bl = 0; bl < nbc; bl++) {
-                const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
-                const int rb = a.bws[seg] * FMT / 8;         // stored row bytes (16 NH for 32-wide blocks)
-                const bool bok = blk < a.nbs[seg];
-                const uint8_t *base = a.xq[seg] + ((size_t)n * a.nbs[seg] + min(blk, a.nbs[seg] - 1)) * Sin * rb;
-                v4i val[NE]; bool ok[NE];
-#pragma unroll
-                for (int k = 0; k < NE; k++) {
-                    const unsigned vox = eoff[k] >> 1, hf = NH == 2 ? (eoff[k] & 1u) : 0u;
-                    if (rb >= 16) {
-                        const bool have = rb >= (int)(hf + 1) * 16;
-                        val[k] = *(const v4i *)(base + (size_t)vox * rb + (have ? hf * 16 : 0));
-                        ok[k] = eok[k] && bok && have;
-                    } else {                                 // 8- or 4-byte rows of a <= 8 / <= 16 channel tensor: only half 0 holds data
-                        val[k] = (v4i){0, 0, 0, 0};
-                        if (rb == 8) { const int2 t = *(const int2 *)(base + (size_t)vox * 8); val[k][0] = t.x; val[k][1] = t.y; }
-                        else val[k][0] = *(const int *)(base + (size_t)vox * 4);
-                        ok[k] = eok[k] && bok && hf == 0;
-                    }
-                }
-#pragma unroll
-                for (int k = 0; k < NE; k++)
-                    if (tid + k * 256 < TT * NH) *(v4i *)(lds + edst[k] + bl * NH * TT * 16) = ok[k] ? val[k] : (v4i){0, 0, 0, 0};
-            }
-            unsigned soff[NS]; bool sok[NS];
-#pragma unroll
-            for (int k = 0; k < NS; k++) {
-                const int pos = min(tid + k * 256, TT - 1);
-                const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
-                const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
-                sok[k] = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
-                const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1);
-                soff[k] = (unsigned)((cz * a.H + cy) * a.W + cx);
-            }
-            for (int bl = 0; bl < nbc; bl++) {
-                const int sb = b0 + bl, seg = sb >= a.nb0p, blk = seg ? sb - a.nb0p : sb;
-                const bool bok = blk < a.nbs[seg];
-                const uint8_t *base = a.xsc[seg] + ((size_t)n * a.nbs[seg] + min(blk, a.nbs[seg] - 1)) * Sin;
-                unsigned sv[NS];
-#pragma unroll
-                for (int k = 0; k < NS; k++) sv[k] = base[soff[k]];
-#pragma unroll
-                for (int k = 0; k < NS; k++)
-                    if (tid + k * 256 < TT) *(unsigned *)(lds + asc_o + (bl * TT + tid + k * 256) * 4) = sok[k] && bok ? sv[k] : 1u;
-            }
-        }
-#endif
+        conv_pair_table<FMT, STRIDE, TZ>(lds, tab_o, nbc, tid);
+        if (a.wide) conv_stage_halo<FMT, STRIDE, TZ, 1, true>(a, lds, act_o, asc_o, b0, nbc, n, iz0, iy0, ix0, tid);
+        else conv_stage_halo<FMT, STRIDE, TZ, 1, false>(a, lds, act_o, asc_o, b0, nbc, n, iz0, iy0, ix0, tid);
         // ---- weight stages: global -> registers -> ring slot. Every thread moves UPT contiguous 16-byte units and one scale word per
         // stage; offsets wrap instead of being guarded (duplicates store the same value). The prepared-weight buffers carry four
         // stages of padding, so the loads that run ahead of the last pair stay inside them ----
@@ -196,12 +467,10 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
         const uint8_t *wgs = a.wsc + (size_t)pair0 * wsc_ps + (size_t)cs * MT * 256 + (tid * 4) % (MT * 256);
         v4i g[UPT]; unsigned gs = 0;
         auto wload = [&]() {            // the next stage in sequence
-#ifndef DBG_NOWLOAD
 #pragma unroll
             for (int k = 0; k < UPT; k++) g[k] = *(const v4i *)(wgp + k * 16);
             gs = *(const unsigned *)wgs;
             wgp += wq_ps; wgs += wsc_ps;
-#endif
         };
         auto wstore = [&](int slot) {
 #pragma unroll
@@ -240,15 +509,11 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
             T = *(const v4i *)(lds + tabp + 32); tabp += 32;      // the next pair's table entry
         };
         auto mma = [&]() {
-#ifndef DBG_NOMMA
 #pragma unroll
             for (int m = 0; m < MT; m++)
 #pragma unroll
                 for (int j = 0; j < NT; j++)
                     acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[m], fb[j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sa[m], 0, sb[j]);
-#else
-            for (int m = 0; m < MT; m++) for (int j = 0; j < NT; j++) acc[m][j][0] += (float)(fa[m][0] + fb[j][0] + sa[m] + sb[j]);
-#endif
         };
         T = *(const v4i *)(lds + tabp);
         for (int q = 0; q < npairs; q += 2) {
@@ -261,165 +526,8 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
         pair0 += npairs;
     }
 
-    // ================= epilogue =================
-    // accumulator layout of the 32x32 MFMA: lane (r = voxel within the tile, h), register i -> channel (i & 3) + 4 h + 8 (i >> 2)
-    const size_t So = (size_t)a.Do * a.Ho * a.Wo;
-    const int co_base = cs * MT * 32;
-    float *red = (float *)lds;                      // stats scratch [4 waves][MT][8 quads][2] floats (the ring and halo are dead now)
-    const bool stats = a.osum != nullptr;
-    float qs[MT][4], qss[MT][4];                    // per lane: sums over its voxels of the 4-channel quads (m, i >> 2)
-#pragma unroll
-    for (int m = 0; m < MT; m++)
-#pragma unroll
-        for (int q4 = 0; q4 < 4; q4++) { qs[m][q4] = 0.f; qss[m][q4] = 0.f; }
-    float chs[MT == 1 ? 16 : 1], chss[MT == 1 ? 16 : 1];     // per-channel sums (MT 1, stat_ch)
-#pragma unroll
-    for (int i = 0; i < (MT == 1 ? 16 : 1); i++) { chs[i] = 0.f; chss[i] = 0.f; }
-    constexpr int YB = OUT == 4 ? 4 : 8;
-    const int bwo = mx_bw(a.Co), nbo = mx_nb(a.Co), rbo = mx_rb(bwo, YB);
-    uint8_t *yq = (uint8_t *)a.y, *ysc = yq + (size_t)a.N * nbo * So * rbo;
-    static_for<MT>([&](auto M) {
-        constexpr int m = M;
-        float bias[16], ea[16], eb[16];
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const int co = co_base + m * 32 + (i & 3) + 4 * h + 8 * (i >> 2);
-            bias[i] = a.bias && co < a.Co ? a.bias[co] : 0.f;
-            if (EPI) { ea[i] = a.ep_a && co < a.Co ? a.ep_a[co] : 1.f; eb[i] = a.ep_a && co < a.Co ? a.ep_b[co] : 0.f; }
-        }
-        static_for<NT>([&](auto J) {
-            constexpr int j = J;
-            const int oz = oz0 + lz, oy = oy0 + ly0 + 2 * j + (r >> 4), ox = ox0 + (r & 15);
-            const bool ok = oz < a.Do && oy < a.Ho && ox < a.Wo;
-            const size_t ov = ((size_t)oz * a.Ho + oy) * a.Wo + ox;
-            const bool zst = ok && oz >= a.zs0 && oz < a.zs1;
-            float v[16];
-            float am = 0.f;
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                float t = acc[m][j][i] + bias[i];             // (padding channels: zero weights and no bias, so they stay 0)
-                if (EPI) {
-                    t = fmaf(t, ea[i], eb[i]);
-                    t = a.act == 1 ? __fdividef(t, 1.f + __expf(-t)) : a.act == 2 ? gelu_erf(t) : a.act == 3 ? fmaxf(t, 0.f) : t;
-                    if (co_base + m * 32 + (i & 3) + 4 * h + 8 * (i >> 2) >= a.Co) t = 0.f;
-                }
-                v[i] = t; am = fmaxf(am, fabsf(t));
-            }
-            if (OUT != 0) {
-                am = fmaxf(am, __shfl_xor(am, 32));
-                const int e = d_mx_exp(am, YB == 8 ? MI_INVQ8 : MI_INVQ4);
-                const int blk = (co_base + m * 32) / bwo;                  // bwo < 32 only when Co <= 16: one tile, block 0
-                const size_t row = ((size_t)n * nbo + blk) * So + ov;
-                if (OUT == 8) {
-                    unsigned d[4];
-#pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc4_e4m3(v[4 * q4], v[4 * q4 + 1], v[4 * q4 + 2], v[4 * q4 + 3], e);
-                    if (a.stored_stats) {
-                        const float sc = d_exp2i(e);
-#pragma unroll
-                        for (int q4 = 0; q4 < 4; q4++) d_dec4_e4m3(d[q4], v + 4 * q4);
-#pragma unroll
-                        for (int i = 0; i < 16; i++) v[i] *= sc;
-                    }
-                    // lane h = 0 holds bytes {0-3, 8-11, 16-19, 24-27}, its partner {4-7, 12-15, 20-23, 28-31}: swap so each stores 16 contiguous bytes
-                    const unsigned s0 = h ? d[0] : d[2], s1 = h ? d[1] : d[3];
-                    const unsigned r0 = __shfl_xor(s0, 32), r1 = __shfl_xor(s1, 32);
-                    const uint4 out = h ? make_uint4(r0, d[2], r1, d[3]) : make_uint4(d[0], r0, d[1], r1);
-                    if (ok) {
-                        if (bwo == 32) *(uint4 *)(yq + row * 32 + 16 * h) = out;
-                        else if (bwo == 16) { if (!h) *(uint4 *)(yq + row * 16) = out; }
-                        else if (!h) *(uint2 *)(yq + row * 8) = make_uint2(out.x, out.y);
-                    }
-                } else {
-                    unsigned hw[4];   // 4 channels -> 16 bits each
-                    {
-                        const unsigned w01 = d_enc8_e2m1(v, e), w23 = d_enc8_e2m1(v + 8, e);
-                        hw[0] = w01 & 0xffffu; hw[1] = w01 >> 16; hw[2] = w23 & 0xffffu; hw[3] = w23 >> 16;
-                        if (a.stored_stats) {
-                            const float sc = d_exp2i(e);
-                            d_dec8_e2m1(w01, v); d_dec8_e2m1(w23, v + 8);
-#pragma unroll
-                            for (int i = 0; i < 16; i++) v[i] *= sc;
-                        }
-                    }
-                    // halfword q4 of lane h sits at byte 4 q4 + 2 h of the 16-byte row: lane 0 assembles words 0-1, lane 1 words 2-3
-                    const unsigned mine01 = hw[0] | (hw[1] << 16), mine23 = hw[2] | (hw[3] << 16);
-                    const unsigned send = h ? mine01 : mine23, recv = __shfl_xor(send, 32);
-                    uint2 out;
-                    if (!h) out = make_uint2((hw[0] & 0xffffu) | ((recv & 0xffffu) << 16), (hw[1] & 0xffffu) | (recv & 0xffff0000u));
-                    else out = make_uint2((recv & 0xffffu) | ((hw[2] & 0xffffu) << 16), (recv >> 16) | ((hw[3] & 0xffffu) << 16));
-                    if (ok) {
-                        if (bwo == 32) *(uint2 *)(yq + row * 16 + 8 * h) = out;
-                        else if (bwo == 16) { if (!h) *(uint2 *)(yq + row * 8) = out; }
-                        else if (!h) *(unsigned *)(yq + row * 4) = out.x;
-                    }
-                }
-                if (ok && !h) ysc[row] = (uint8_t)(e + 127);
-            } else {
-                const size_t o0 = ((size_t)n * a.Co + co_base + m * 32 + 4 * h) * So + ov;
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const int cl = (i & 3) + 8 * (i >> 2);            // channel offset from co_base + 32 m + 4 h
-                    const bool cok = ok && co_base + m * 32 + 4 * h + cl < a.Co;
-                    if (a.ydt == 2) {
-                        if (a.Go > 0) v[i] = fabsf(v[i]) > 65504.f ? copysignf(65504.f, v[i]) : v[i];     // src/lp_common.cuh:465, :1567-1569
-                        if (cok) ((__half *)a.y)[o0 + (size_t)cl * So] = __float2half(v[i]);
-                    } else if (cok) ((float *)a.y)[o0 + (size_t)cl * So] = v[i];
-                }
-            }
-            if (stats && zst) {
-                if (MT == 1 && a.stat_ch) {
-#pragma unroll
-                    for (int i = 0; i < 16; i++) { chs[i] += v[i]; chss[i] += v[i] * v[i]; }
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 16; i++) { qs[m][i >> 2] += v[i]; qss[m][i >> 2] += v[i] * v[i]; }
-                }
-            }
-        });
-    });
-    if (stats) __syncthreads();
-    if (MT == 1 && stats && a.stat_ch) {
-        // any group size (one channel tile): per-channel sums over the 32 voxel lanes, then over the waves; channel of register i of
-        // half h = (i & 3) + 4 h + 8 (i >> 2)
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            float s1 = chs[i], s2 = chss[i];
-#pragma unroll
-            for (int d = 1; d < 32; d <<= 1) { s1 += __shfl_xor(s1, d); s2 += __shfl_xor(s2, d); }
-            const int ch = (i & 3) + 4 * h + 8 * (i >> 2);
-            if (r == 0) { red[(wave * 32 + ch) * 2] = s1; red[(wave * 32 + ch) * 2 + 1] = s2; }
-        }
-        __syncthreads();
-        if (tid < 32) {
-            float s1 = 0.f, s2 = 0.f;
-            for (int w = 0; w < 4; w++) { s1 += red[(w * 32 + tid) * 2]; s2 += red[(w * 32 + tid) * 2 + 1]; }
-            a.part[((size_t)tile * 32 + tid) * 2] = s1; a.part[((size_t)tile * 32 + tid) * 2 + 1] = s2;
-        }
-    } else if (stats) {
-        // channels per group a multiple of 4: a quad (m, q4, h) = channels co_base + 32 m + 8 q4 + 4 h .. +3 lies in one group.
-        // Sum over the 32 voxel lanes of each half (butterfly, fixed order), then over the 4 waves in wave order, then one
-        // exact slot add per quad.
-#pragma unroll
-        for (int m = 0; m < MT; m++)
-#pragma unroll
-            for (int q4 = 0; q4 < 4; q4++) {
-                float s = qs[m][q4], ss = qss[m][q4];
-#pragma unroll
-                for (int d = 1; d < 32; d <<= 1) { s += __shfl_xor(s, d); ss += __shfl_xor(ss, d); }
-                if (r == 0) { red[((wave * MT + m) * 8 + q4 * 2 + h) * 2] = s; red[((wave * MT + m) * 8 + q4 * 2 + h) * 2 + 1] = ss; }
-            }
-        __syncthreads();
-        if (tid < MT * 8) {
-            // per tile and channel quad, the sums over the tile's voxels in wave order; a second kernel adds the tiles of a sample
-            // in a fixed order into the exact sum slots, so the statistics do not depend on the order workgroups finish in
-            const int m = tid >> 3, q8 = tid & 7;                       // q8 = q4 * 2 + h: channels co_base + 32 m + 8 q4 + 4 h .. + 3
-            float s = 0.f, ss = 0.f;
-            for (int w = 0; w < 4; w++) { s += red[((w * MT + m) * 8 + q8) * 2]; ss += red[((w * MT + m) * 8 + q8) * 2 + 1]; }
-            a.part[((size_t)tile * MT * 8 + tid) * 2] = s;
-            a.part[((size_t)tile * MT * 8 + tid) * 2 + 1] = ss;
-        }
-    }
+    __syncthreads();                                     // the ring and halo are dead: the epilogue reuses LDS for its statistics scratch
+    conv_epilogue<MT, NT, OUT, EPI>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
 }
 
 extern thread_local char g_last_kernel[128];
@@ -433,9 +541,11 @@ static void launch_conv(const conv_args &a, size_t smem) {
     MICK();
     snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_mx_k<fmt %d, stride %d, MT %d, NT %d, out %d, epi %d> CB %d tiles %u", FMT, STRIDE, MT, NT, OUT, (int)EPI, a.CB, a.ntiles);
 }
+#include "conv3_wide.hpp"
 template <int FMT, int STRIDE, int OUT, bool EPI>
 static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     switch (MT * 10 + NT) {
+    case 44: if constexpr (STRIDE == 1) launch_wide<FMT, OUT, EPI>(a, smem); else mi_die("conv3: the wide kernel is stride 1 only"); break;
     case 12: launch_conv<FMT, STRIDE, 1, 2, OUT, EPI>(a, smem); break;
     case 22: launch_conv<FMT, STRIDE, 2, 2, OUT, EPI>(a, smem); break;
     case 32: launch_conv<FMT, STRIDE, 3, 2, OUT, EPI>(a, smem); break;

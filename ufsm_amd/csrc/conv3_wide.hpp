@@ -1,0 +1,277 @@
+// The wide 3x3x3 stride-1 kernel: 128 output channels x 4 x 8 x 16 voxels per tile, one wavefront per SIMD with 16 accumulators (AGPRs).
+//
+// Every weight fragment is reused by 4 voxel tiles and every input fragment by 4 channel tiles, which halves the LDS traffic per MFMA of
+// the 8-accumulator kernel: at full MFMA rate the 4 wavefronts read about 72 B / clk of the CU's 128 B / clk. With a single wavefront per
+// SIMD nothing else hides latency, so the schedule is explicit:
+//   * fragments of pair q + 1 are fetched into a second register set between the MFMAs of pair q (sched_group_barrier pins the
+//     interleave); one workgroup barrier per two pairs;
+//   * all global -> LDS traffic is direct (global_load_lds, no registers): weight stages of two pairs go into a 2-slot ring two stages
+//     ahead; input halo blocks of 32 channels live in 3 LDS slots and the K loop walks the blocks one after the other (taps inside), so
+//     while blocks b, b + 1 are multiplied block b + 2 streams into the third slot; the first blocks of the next tile follow the last one of
+//     this tile and land during the epilogue. Positions outside the volume read a zero row / scale byte 1 from a constant page;
+//   * workgroups are persistent (one per CU) and walk their tiles XCD by XCD.
+// The asynchronous copies are tracked with vmcnt: every copying step issues its weight copies first and then a fixed number of halo
+// copies, all unconditionally (nothing in a step branches, or the MFMA / LDS interleave would fall apart), so "all but the last few"
+// is exactly "the weights have landed".
+#pragma once
+
+__device__ __forceinline__ void dma16(const void *g, unsigned lds_off) {      // lane l: 16 bytes from g (per lane) to LDS lds_off + 16 l
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_off), "v"(g) : "memory");
+}
+__device__ __forceinline__ void dma1(const void *g, unsigned lds_off) {       // lane l: 1 byte from g, zero-extended to the word at LDS lds_off + 4 l
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_ubyte %1, off" ::"s"(lds_off), "v"(g) : "memory");
+}
+// the same with a uniform 64-bit base and a 32-bit per-lane byte offset
+__device__ __forceinline__ void dma16s(unsigned off, const void *base, unsigned lds_off) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_off), "v"(off), "s"(base) : "memory");
+}
+__device__ __forceinline__ void dma1s(unsigned off, const void *base, unsigned lds_off) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_ubyte %1, %2" ::"s"(lds_off), "v"(off), "s"(base) : "memory");
+}
+template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+template <int FMT, int OUT, bool EPI>
+__global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
+    constexpr int MT = 4, NT = 4, TZ = 4;
+    using HL = halo_t<FMT, 1, TZ>;
+    constexpr int TT = HL::TT, HY = HL::HY, HX = HL::HX, NH = HL::NH, WTILE = fmt_t<FMT>::WTILE;
+    constexpr int STG = MT * (WTILE + 256), SLOT = 2 * STG;     // a ring slot holds one stage = two pairs, each MT tiles of codes then MT x 64 scale words
+    constexpr int NG = (TT + 63) / 64, TTP = NG * 64;           // copy groups of 64 halo positions; positions per half padded to whole groups
+    constexpr int HB = NH * TTP * 16 + TTP * 4;                 // a halo slot: rows [half][position][16 B], then one scale word per position
+    constexpr int NRND = (NG + 3) / 4;                          // copy rounds of a block: in a round every wave copies one group (both halves and the scales)
+    constexpr int WCP = MT * WTILE / 1024, WPS = 2 * (WCP + 1); // 1 KiB copies per pair of codes (+ 1 of scales), copies per weight stage
+    extern __shared__ __align__(16) unsigned char lds[];
+    const unsigned lds0 = (unsigned)(size_t)lds;                // LDS byte offset of the dynamic segment (the low word of its flat address)
+    constexpr unsigned halo_o = 2 * SLOT, tab_o = halo_o + 3 * HB;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), r = lane & 31, h = lane >> 5;
+    const int lz = wave, ly0 = 0;
+    unsigned abr[NT], sbr[NT];                                  // the lane's row (its 16-byte half) and scale word of tap (0, 0, 0) inside a halo slot
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        const int p0 = (lz * HY + (2 * j + (r >> 4))) * HX + (r & 15);
+        abr[j] = halo_o + ((NH == 2 ? h * TTP : 0) + p0) * 16;
+        sbr[j] = halo_o + NH * TTP * 16 + p0 * 4;
+    }
+    const unsigned wfa = lane * 16, wfs = MT * WTILE + lane * 4;            // the lane's weight fragment / scale word of pair 0, tile 0 of a slot
+    const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 256;
+    const size_t Sin = (size_t)a.D * a.H * a.W;
+    const int nunits = 27 * a.nbt, npairs = (nunits + 1) >> 1, nfull = npairs >> 1;
+
+    // XCD-aware persistent tile walk: workgroup ids go round robin over the 8 XCDs, each XCD owns a contiguous range of tiles
+    const unsigned per = (a.ntiles + 7u) / 8u, wg_per_xcd = gridDim.x >> 3, xcd = blockIdx.x & 7u, wix = blockIdx.x >> 3;
+    struct tile_t { unsigned tile; int n, cs, oz0, oy0, ox0; bool ok; };
+    auto decode = [&](unsigned it) {
+        tile_t t; const unsigned k = wix + it * wg_per_xcd;
+        t.ok = k < per && xcd * per + k < a.ntiles;
+        t.tile = t.ok ? xcd * per + k : 0u;
+        int tt = (int)t.tile;
+        t.cs = tt % a.ncs; tt /= a.ncs;
+        const int tx = tt % a.ntx; tt /= a.ntx;
+        const int ty = tt % a.nty; tt /= a.nty;
+        const int tz = tt % a.ntz; t.n = tt / a.ntz;
+        t.ox0 = tx * 16; t.oy0 = ty * 8; t.oz0 = tz * TZ;
+        return t;
+    };
+    // One copy round of this wave for block blk of the tile at (n, oz0, oy0, ox0) into the halo slot at byte offset sbase of the halo area:
+    // the two row halves and the scale bytes of 64 halo positions (group 4 rd + wave). It is prepared (addresses: pure arithmetic the
+    // scheduler places anywhere) one step ahead of its issue, and the issue is three copies with every lane active and no branch: positions
+    // outside the volume, past the halo or of blocks past the stored channels read a constant page (zero row, scale byte 1); a round with
+    // nothing to do (go false, or a group past the last) reads the constant page into a junk area. The two halves of a row are requested
+    // back to back, so the second one finds its cache line.
+    const unsigned junk = a.red_o;                              // the statistics scratch (1 KiB) is idle while the K loop runs
+    struct hreq { const uint8_t *row, *sc; unsigned rdst, sdst; };
+    auto prepare = [&](hreq &q, int n, int oz0, int oy0, int ox0, int blk, int rd, unsigned sbase, bool go) {
+        const int g = 4 * rd + wave;
+        const int seg = blk >= a.nb0p, bl = seg ? blk - a.nb0p : blk;
+        const bool real = go && g < NG, bok = real && bl < a.nbs[seg];
+        const size_t plane = (size_t)n * a.nbs[seg] + min(max(bl, 0), a.nbs[seg] - 1);
+        const int pos = g * 64 + lane;
+        const int pz = pos / (HY * HX), rem = pos - pz * (HY * HX), py = rem / HX, px = rem - py * HX;
+        const int gz = oz0 - 1 + pz, gy = oy0 - 1 + py, gx = ox0 - 1 + px;
+        const bool in = bok && pos < TT && gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
+        const size_t vox = (size_t)(unsigned)((gz * a.H + gy) * a.W + gx);
+        q.row = in ? a.xq[seg] + (plane * Sin + vox) * (16 * NH) : a.zpage;
+        q.sc = in ? a.xsc[seg] + plane * Sin + vox : a.zpage + 64;
+        q.rdst = real ? halo_o + sbase + g * 1024 : junk;
+        q.sdst = real ? halo_o + sbase + NH * TTP * 16 + g * 256 : junk;
+    };
+    auto issue = [&](const hreq &q) {
+        dma16(q.row, lds0 + q.rdst);
+        if constexpr (NH == 2) dma16(q.row + 16, lds0 + q.rdst + (q.rdst == junk ? 0u : (unsigned)TTP * 16u));
+        dma1(q.sc, lds0 + q.sdst);
+    };
+    constexpr int NHC = NH + 1;                                 // asynchronous copies of a round
+    // copy k (of NW) of this wave's share of the weight stage of pairs gp0, gp0 + 1 into the ring slot at byte offset so (a wave with fewer
+    // pieces repeats its last one: the count per step stays fixed)
+    constexpr int NW = (WPS + 3) / 4;
+    auto wcopy = [&](int k, int gp0, int cs, unsigned so) {
+        int c = wave + 4 * k;
+        c = c < WPS ? c : c - 4;
+        const int p = c / (WCP + 1), cc = c - p * (WCP + 1);
+        const bool codes = cc < WCP;
+        const uint8_t *src = codes ? a.wq + (size_t)(gp0 + p) * wq_ps + (size_t)cs * MT * WTILE + cc * 1024 : a.wsc + (size_t)(gp0 + p) * wsc_ps + (size_t)cs * MT * 256;
+        dma16s((unsigned)lane * 16u, src, lds0 + so + p * STG + (codes ? cc * 1024 : MT * WTILE));
+    };
+    auto wstage = [&](int gp0, int cs, unsigned so) {
+#pragma unroll
+        for (int k = 0; k < NW; k++) wcopy(k, gp0, cs, so);
+    };
+
+    // K order: unit U = (block U / 27, tap U % 27), pair G = units 2 G, 2 G + 1 (a pair may straddle two blocks; the unit past the end has
+    // zero weights and re-reads the one before). Block b of the workgroup's it-th tile lives in halo slot (it nbt + b) % 3: while blocks
+    // b, b + 1 are multiplied, block b + 2 streams into the slot block b - 1 left; the first two blocks of the next tile follow the last
+    // block of this one.
+    tile_t cur = decode(0);
+    if (!cur.ok) return;
+    const int nnext = min(2, a.nbt);                            // blocks of the next tile requested ahead
+    for (int rd = 0; rd < NRND; rd++) {
+        hreq q;
+        prepare(q, cur.n, cur.oz0, cur.oy0, cur.ox0, 0, rd, 0, true); issue(q);
+        if (nnext > 1) { prepare(q, cur.n, cur.oz0, cur.oy0, cur.ox0, 1, rd, HB, true); issue(q); }
+    }
+    wstage(0, cur.cs, 0); wstage(2, cur.cs, SLOT);
+    unsigned rot = 0;                                           // (it nbt) % 3
+    for (unsigned it = 0;; it++) {
+        const tile_t nxt = decode(it + 1);
+        const int fmax = a.nbt - 1 + (nxt.ok ? nnext : 0);      // blocks to request during this tile: 2 .. nbt - 1 of this tile, then nbt .. of the next
+        wait_vm<0>();                                           // the tile's first blocks and weight stages (and the last tile's stores) are done
+        __syncthreads();
+        DBG_MARK(0);
+        conv_epi_consts<MT, EPI>(a, lds, cur.cs, tid);
+        // pair table of this tile: per pair and lane half {row offset of unit A (fp4: of the half's own unit), of unit B, scale word offset of the half's unit}
+        for (int i = tid; i < (npairs + 2) * 2; i += 256) {
+            const int g = min(i >> 1, npairs - 1), hh = i & 1;
+            const int uA = 2 * g, uB = 2 * g + 1 < nunits ? 2 * g + 1 : 2 * g;
+            const int bA = uA / 27, tA = uA - 27 * bA, bB = uB / 27, tB = uB - 27 * bB;
+            const int oA = (int)((rot + bA) % 3u) * HB + (((tA / 9) * HY + (tA / 3) % 3) * HX + tA % 3) * 16;
+            const int oB = (int)((rot + bB) % 3u) * HB + (((tB / 9) * HY + (tB / 3) % 3) * HX + tB % 3) * 16;
+            const int oH = hh ? oB : oA, sH = (oH / HB) * HB + ((oH % HB) >> 2);
+            *(v4i *)(lds + tab_o + i * 16) = (v4i){NH == 2 ? oA : oH, oB, sH, 0};
+        }
+        v16f acc[MT][NT];
+        {
+            float z;                                            // an opaque zero: the accumulators are cleared here, not hoisted elsewhere
+            asm volatile("v_mov_b32 %0, 0" : "=v"(z));
+#pragma unroll
+            for (int m = 0; m < MT; m++)
+#pragma unroll
+                for (int j = 0; j < NT; j++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) acc[m][j][i] = z;
+        }
+        __syncthreads();
+
+        v8i fb[2][NT], fa[2][MT]; int sb[2][NT], sa[2][MT];
+        v4i T;
+        unsigned tabp = tab_o + h * 16;
+        T = *(const v4i *)(lds + tabp);
+        // one LDS load of the fetch of a pair: index i = 3 f + part over the NT input fragments, then the MT weight fragments; the last
+        // index reads the table entry of the pair after
+        v4i lo[NT + MT], hi[NT + MT];
+        auto ld = [&](auto I, auto NXT, const v4i tt2, unsigned wbase) {
+            constexpr int i = decltype(I)::value, nx = decltype(NXT)::value;
+            constexpr int f = i / 3, part = i % 3;
+            if constexpr (i == 3 * (NT + MT)) { T = *(const v4i *)(lds + tabp + 32); tabp += 32; }
+            else if constexpr (f < NT) {
+                if constexpr (part == 0) lo[f] = *(const v4i *)(lds + abr[f] + tt2[0]);
+                else if constexpr (part == 1) { if constexpr (FMT == 8) hi[f] = *(const v4i *)(lds + abr[f] + tt2[1]); }
+                else sb[nx][f] = *(const int *)(lds + sbr[f] + tt2[2]);
+            } else {
+                constexpr int m = f - NT;
+                if constexpr (part == 0) lo[f] = *(const v4i *)(lds + wfa + wbase + m * WTILE);
+                else if constexpr (part == 1) { if constexpr (FMT == 8) hi[f] = *(const v4i *)(lds + wfa + wbase + m * WTILE + 1024); }
+                else sa[nx][m] = *(const int *)(lds + wfs + wbase + m * 256);
+            }
+        };
+        auto pack = [&](auto NXT) {
+            constexpr int nx = decltype(NXT)::value;
+#pragma unroll
+            for (int f = 0; f < NT; f++) fb[nx][f] = FMT == 8 ? (v8i){lo[f][0], lo[f][1], lo[f][2], lo[f][3], hi[f][0], hi[f][1], hi[f][2], hi[f][3]} : (v8i){lo[f][0], lo[f][1], lo[f][2], lo[f][3], 0, 0, 0, 0};
+#pragma unroll
+            for (int m = 0; m < MT; m++) fa[nx][m] = FMT == 8 ? (v8i){lo[NT + m][0], lo[NT + m][1], lo[NT + m][2], lo[NT + m][3], hi[NT + m][0], hi[NT + m][1], hi[NT + m][2], hi[NT + m][3]} : (v8i){lo[NT + m][0], lo[NT + m][1], lo[NT + m][2], lo[NT + m][3], 0, 0, 0, 0};
+        };
+        constexpr int NL = 3 * (NT + MT) + 1, NM = MT * NT, NSP = NM - 3;      // the fetch is spread over the first NSP MFMAs so it has landed before the barrier
+        {   // pair 0 -> register set 0
+            const v4i tt2 = T;
+            static_for<NL>([&](auto I) { ld(I, std::integral_constant<int, 0>{}, tt2, 0u); });
+            pack(std::integral_constant<int, 0>{});
+        }
+        DBG_MARK(1);
+        // ---- the streaming schedule. fbi: next block to request (>= nbt: of the next tile), frd: its next copy round. A block may be requested
+        // once block fbi - 3, whose slot it takes, has been read for the last time (pair (27 (fbi - 3) + 26) / 2). The host has checked that
+        // with two rounds per stage every block of a tile lands two barriers before its first fetch ----
+        int fbi = 2, frd = 0;
+        auto prep_next = [&](hreq &q, int upto_pair) {          // prepare one copy round; pairs <= upto_pair will have been fetched by every wavefront when it is issued
+            const bool go = fbi <= fmax && (fbi < 3 || ((27 * (fbi - 3) + 26) >> 1) <= upto_pair);
+            const bool own = fbi < a.nbt;
+            prepare(q, own ? cur.n : nxt.n, own ? cur.oz0 : nxt.oz0, own ? cur.oy0 : nxt.oy0, own ? cur.ox0 : nxt.ox0, own ? fbi : fbi - a.nbt, frd,
+                    ((rot + (unsigned)fbi) % 3u) * HB, go);
+            frd += go ? 1 : 0;
+            const bool wrap = frd == NRND;
+            frd = wrap ? 0 : frd; fbi += wrap ? 1 : 0;
+        };
+        hreq rq;
+        // the MFMAs of the pair in register set CUR with the fetch of the next pair (weights at ring offset wbase) between them.
+        // MODE 1: also prepare the copy round the next step will issue. MODE 2: also this step's asynchronous copies, one after every
+        // MFMA from the second on: the weight stage of pairs wgp, wgp + 1 into ring offset wso first, then the prepared round (so that
+        // "all but the last NHC copies" means "the weights")
+        auto step = [&](auto CUR, auto MODE, unsigned wbase, int wgp, unsigned wso, int upto_pair) {
+            constexpr int cu = decltype(CUR)::value, nx = cu ^ 1, mode = decltype(MODE)::value;
+            const v4i tt2 = T;
+            if constexpr (mode == 1) prep_next(rq, upto_pair);
+            static_for<NM>([&](auto K) {
+                constexpr int k = decltype(K)::value, m = k / NT, j = k % NT;
+                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cu][m], fb[cu][j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sa[cu][m], 0, sb[cu][j]);
+                constexpr int l0 = k < NSP ? (k * NL) / NSP : NL, l1 = k < NSP ? ((k + 1) * NL) / NSP : NL;
+                static_for<l1 - l0>([&](auto I) { ld(std::integral_constant<int, l0 + decltype(I)::value>{}, std::integral_constant<int, nx>{}, tt2, wbase); });
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if constexpr (l1 > l0) __builtin_amdgcn_sched_group_barrier(0x100, l1 - l0, 0);
+                if constexpr (mode == 1) __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);     // the preparation's arithmetic, a few instructions per MFMA
+                if constexpr (mode == 2) {                      // (fenced: otherwise the scheduler lifts the copies, and the fetches ordered with them, above the MFMAs)
+                    if constexpr (k >= 1 && k <= NW) { __builtin_amdgcn_sched_barrier(0); wcopy(k - 1, wgp, cur.cs, wso); __builtin_amdgcn_sched_barrier(0); }
+                    if constexpr (k == NW + 2) { __builtin_amdgcn_sched_barrier(0); issue(rq); __builtin_amdgcn_sched_barrier(0); }
+                }
+            });
+            pack(std::integral_constant<int, nx>{});
+        };
+        // stage s = pairs 2 s, 2 s + 1 lives in ring slot s & 1. Step 0 consumes pair 2 s and fetches pair 2 s + 1 from the same slot; after the
+        // barrier every wavefront is done reading that slot, so step 1 requests stage s + 2 into it (to be there one stage later, when
+        // the barrier of stage s + 1 has been passed) and two copy rounds of streaming blocks, while it consumes pair 2 s + 1 and fetches
+        // pair 2 s + 2 from the other slot
+        for (int s = 0; s < nfull; s++) {
+            const unsigned so = (s & 1) * SLOT;
+            step(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, so + STG, 0, 0u, 2 * s + 1);
+            wait_vm<NHC>();                                     // the weight stage requested one stage ago is in LDS: it was issued before that step's NHC halo copies
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            step(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{}, SLOT - so, 2 * (s + 2), so, 0);
+        }
+        if (npairs & 1) step(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, (nfull & 1) * SLOT + STG, 0, 0u, 0);     // the odd last pair (its fetch reads past the end: unused)
+        DBG_MARK(2);
+        wait_vm<0>();
+        __syncthreads();                                        // every wavefront is done with the halo slots and the ring
+        while (fbi <= fmax) { prep_next(rq, npairs); issue(rq); }       // (tiles too short to stream everything)
+        if (nxt.ok) { wstage(0, nxt.cs, 0); wstage(2, nxt.cs, SLOT); }
+        DBG_MARK(3);
+        conv_epilogue<MT, NT, OUT, EPI, true>(a, acc, lds, cur.tile, cur.n, cur.cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+        DBG_MARK(4);
+        if (!nxt.ok) break;
+        cur = nxt; rot = (rot + (unsigned)a.nbt) % 3u;
+    }
+}
+
+template <int FMT, int OUT, bool EPI>
+static void launch_wide(const conv_args &a, size_t smem) {
+    static bool attr[8]; static int ncu[8];
+    int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
+    if (!attr[d]) {
+        MIRT(hipFuncSetAttribute((const void *)conv3_wide_k<FMT, OUT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        hipDeviceProp_t pr; MIRT(hipGetDeviceProperties(&pr, d));
+        ncu[d] = pr.multiProcessorCount > 8 ? pr.multiProcessorCount & ~7 : 8;
+        attr[d] = true;
+    }
+    const unsigned per = (a.ntiles + 7u) / 8u;            // tiles per XCD; one persistent workgroup per CU, a multiple of 8 in all
+    const unsigned nwg = per * 8u < (unsigned)ncu[d] ? per * 8u : (unsigned)ncu[d];
+    conv3_wide_k<FMT, OUT, EPI><<<nwg, 256, smem>>>(a);
+    MICK();
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_wide_k<fmt %d, out %d, epi %d> tiles %u wgs %u", FMT, OUT, (int)EPI, a.ntiles, nwg);
+}

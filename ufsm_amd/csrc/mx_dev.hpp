@@ -99,14 +99,34 @@ __device__ __forceinline__ unsigned d_enc_e2m1x8_hw(const float *v, float pow2e)
     w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, v[6], v[7], pow2e, 3);
     return w;
 }
-// encode with the block exponent e (128: non-finite block, software path with the multiplier 2^-e as the reference forms it)
+// encode with the block exponent e. 128 marks a block holding an infinity or NaN: the reference then multiplies by exp2i(-128), the
+// bits of -inf (src/lp_common.cuh:501), so a finite non-zero value or an infinity saturates with the opposite sign and a zero or a
+// NaN becomes NaN. Those codes have a closed form; they are formed under a wave-uniform branch that finite data never takes.
+__device__ __forceinline__ unsigned d_enc_e4m3_nf(float x) {
+    const unsigned u = __float_as_uint(x), a = u & 0x7fffffffu;
+    return (a == 0u || a > 0x7f800000u) ? 0x7fu : (0x7eu | ((~u >> 24) & 0x80u));
+}
+__device__ __forceinline__ unsigned d_enc_e2m1_nf(float x) {
+    const unsigned u = __float_as_uint(x), a = u & 0x7fffffffu;
+    return (a == 0u || a > 0x7f800000u) ? 7u : (7u | ((~u >> 28) & 8u));
+}
 __device__ __forceinline__ unsigned d_enc4_e4m3(float a, float b, float c, float d, int e) {
-    if (e == 128) { const float m = d_exp2i(-e); return d_enc_e4m3x4(a * m, b * m, c * m, d * m); }
-    return d_enc_e4m3x4_hw(a, b, c, d, d_exp2i(e));
+    unsigned w = d_enc_e4m3x4_hw(a, b, c, d, d_exp2i(e));
+    if (__builtin_amdgcn_ballot_w64(e == 128) != 0ull) {
+        if (e == 128) w = d_enc_e4m3_nf(a) | (d_enc_e4m3_nf(b) << 8) | (d_enc_e4m3_nf(c) << 16) | (d_enc_e4m3_nf(d) << 24);
+    }
+    return w;
 }
 __device__ __forceinline__ unsigned d_enc8_e2m1(const float *v, int e) {
-    if (e == 128) return d_enc_e2m1x8(v, d_exp2i(-e));
-    return d_enc_e2m1x8_hw(v, d_exp2i(e));
+    unsigned w = d_enc_e2m1x8_hw(v, d_exp2i(e));
+    if (__builtin_amdgcn_ballot_w64(e == 128) != 0ull) {
+        if (e == 128) {
+            w = 0u;
+#pragma unroll
+            for (int k = 0; k < 8; k++) w |= d_enc_e2m1_nf(v[k]) << (4 * k);
+        }
+    }
+    return w;
 }
 // decode one word: 4 e4m3 bytes / 8 e2m1 nibbles -> floats (unscaled)
 __device__ __forceinline__ void d_dec4_e4m3(unsigned w, float *v) {
