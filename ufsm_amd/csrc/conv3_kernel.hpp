@@ -222,7 +222,7 @@ __device__ __forceinline__ void conv_epi_consts(const conv_args &a, unsigned cha
 // ---- epilogue (src/lp_common.cuh:1465-1597): bias -> optional affine + activation -> per (voxel, 32-channel block) amax across the
 // lane pair (l, l ^ 32) -> E8M0 exponent -> codes -> row stores; GroupNorm partial sums per tile. acc: the wavefront's MT x NT accumulators;
 // lane (r, h) of tile j holds voxel (oz0 + lz, oy0 + ly0 + 2 j + (r >> 4), ox0 + (r & 15)) ----
-template <int MT, int NT, int OUT, bool EPI, bool PIN = false>
+template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false>
 __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT][NT], unsigned char *lds, unsigned tile, int n, int cs,
                                               int oz0, int oy0, int ox0, int lz, int ly0, int tid) {
     const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
@@ -240,7 +240,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
 #pragma unroll
     for (int i = 0; i < (MT == 1 ? 16 : 1); i++) { chs[i] = 0.f; chss[i] = 0.f; }
     constexpr int YB = OUT == 4 ? 4 : 8;
-    const int bwo = mx_bw(a.Co), nbo = mx_nb(a.Co), rbo = mx_rb(bwo, YB);
+    const int bwo = W32 ? 32 : mx_bw(a.Co), nbo = W32 ? (a.Co + 31) >> 5 : mx_nb(a.Co), rbo = mx_rb(bwo, YB);     // W32: more than 16 output channels, known at compile time
     uint8_t *yq = (uint8_t *)a.y, *ysc = yq + (size_t)a.N * nbo * So * rbo;
     static_for<MT>([&](auto M) {
         constexpr int m = M;
@@ -285,8 +285,15 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                 const size_t row = ((size_t)n * nbo + blk) * So + ov;
                 if (OUT == 8) {
                     unsigned d[4];
+                    const float p2e = d_exp2i(e);
 #pragma unroll
-                    for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc4_e4m3(v[4 * q4], v[4 * q4 + 1], v[4 * q4 + 2], v[4 * q4 + 3], e);
+                    for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc_e4m3x4_hw(v[4 * q4], v[4 * q4 + 1], v[4 * q4 + 2], v[4 * q4 + 3], p2e);
+                    if (__builtin_amdgcn_ballot_w64(e == 128) != 0ull) {      // a block with an infinity or NaN: closed-form codes (never taken by finite data)
+                        if (e == 128) {
+#pragma unroll
+                            for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc4_e4m3_nf(v[4 * q4], v[4 * q4 + 1], v[4 * q4 + 2], v[4 * q4 + 3]);
+                        }
+                    }
                     if (a.stored_stats) {
                         const float sc = d_exp2i(e);
 #pragma unroll
@@ -306,7 +313,11 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                 } else {
                     unsigned hw[4];   // 4 channels -> 16 bits each
                     {
-                        const unsigned w01 = d_enc8_e2m1(v, e), w23 = d_enc8_e2m1(v + 8, e);
+                        const float p2e = d_exp2i(e);
+                        unsigned w01 = d_enc_e2m1x8_hw(v, p2e), w23 = d_enc_e2m1x8_hw(v + 8, p2e);
+                        if (__builtin_amdgcn_ballot_w64(e == 128) != 0ull) {
+                            if (e == 128) { w01 = d_enc8_e2m1_nf(v); w23 = d_enc8_e2m1_nf(v + 8); }
+                        }
                         hw[0] = w01 & 0xffffu; hw[1] = w01 >> 16; hw[2] = w23 & 0xffffu; hw[3] = w23 >> 16;
                         if (a.stored_stats) {
                             const float sc = d_exp2i(e);
@@ -349,7 +360,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                     for (int i = 0; i < 16; i++) { qs[m][i >> 2] += v[i]; qss[m][i >> 2] += v[i] * v[i]; }
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);       // one accumulator tile at a time: hoisting the next tiles' reads only costs registers
+            if (!PIN) __builtin_amdgcn_sched_barrier(0);     // one accumulator tile at a time: hoisting the next tiles' reads only costs registers
         });
     });
     DBG_MARK(20);

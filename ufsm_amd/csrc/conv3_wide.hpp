@@ -252,7 +252,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         while (fbi <= fmax) { prep_next(rq, npairs); issue(rq); }       // (tiles too short to stream everything)
         if (nxt.ok) { wstage(0, nxt.cs, 0); wstage(2, nxt.cs, SLOT); }
         DBG_MARK(3);
-        conv_epilogue<MT, NT, OUT, EPI, true>(a, acc, lds, cur.tile, cur.n, cur.cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+        conv_epilogue<MT, NT, OUT, EPI, true, true>(a, acc, lds, cur.tile, cur.n, cur.cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
         DBG_MARK(4);
         if (!nxt.ok) break;
         cur = nxt; rot = (rot + (unsigned)a.nbt) % 3u;

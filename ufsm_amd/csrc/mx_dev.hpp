@@ -110,21 +110,26 @@ __device__ __forceinline__ unsigned d_enc_e2m1_nf(float x) {
     const unsigned u = __float_as_uint(x), a = u & 0x7fffffffu;
     return (a == 0u || a > 0x7f800000u) ? 7u : (7u | ((~u >> 28) & 8u));
 }
+__device__ __forceinline__ unsigned d_enc4_e4m3_nf(float a, float b, float c, float d) {
+    return d_enc_e4m3_nf(a) | (d_enc_e4m3_nf(b) << 8) | (d_enc_e4m3_nf(c) << 16) | (d_enc_e4m3_nf(d) << 24);
+}
+__device__ __forceinline__ unsigned d_enc8_e2m1_nf(const float *v) {
+    unsigned w = 0u;
+#pragma unroll
+    for (int k = 0; k < 8; k++) w |= d_enc_e2m1_nf(v[k]) << (4 * k);
+    return w;
+}
 __device__ __forceinline__ unsigned d_enc4_e4m3(float a, float b, float c, float d, int e) {
     unsigned w = d_enc_e4m3x4_hw(a, b, c, d, d_exp2i(e));
     if (__builtin_amdgcn_ballot_w64(e == 128) != 0ull) {
-        if (e == 128) w = d_enc_e4m3_nf(a) | (d_enc_e4m3_nf(b) << 8) | (d_enc_e4m3_nf(c) << 16) | (d_enc_e4m3_nf(d) << 24);
+        if (e == 128) w = d_enc4_e4m3_nf(a, b, c, d);
     }
     return w;
 }
 __device__ __forceinline__ unsigned d_enc8_e2m1(const float *v, int e) {
     unsigned w = d_enc_e2m1x8_hw(v, d_exp2i(e));
     if (__builtin_amdgcn_ballot_w64(e == 128) != 0ull) {
-        if (e == 128) {
-            w = 0u;
-#pragma unroll
-            for (int k = 0; k < 8; k++) w |= d_enc_e2m1_nf(v[k]) << (4 * k);
-        }
+        if (e == 128) w = d_enc8_e2m1_nf(v);
     }
     return w;
 }
