@@ -28,6 +28,47 @@ def exact_case(rng, N, Ci, Co, S):
 
 # (bits, N, Ci, Co, D, H, W, stride): ragged W = 20 (tests/test_mx.c:34-45), partial tiles (tests/test_mx4.c:727-760), wide channel
 # counts with odd block counts (tests/test_mx4_wide.c:741-745), stride-2 odd dims (tests/test_mx.c:159-199)
+# the wide kernel (128-channel output slices, stride 1): odd and even block counts, several output slices, ragged tiles, depths that
+# are not a multiple of its 4-deep tile, more tiles than workgroups (persistent walk), fp4
+WIDE_SHAPES = [(8, 1, 96, 128, 5, 9, 18), (8, 1, 32, 128, 3, 8, 16), (8, 2, 128, 256, 6, 10, 33), (8, 1, 384, 128, 4, 8, 16), (8, 3, 64, 128, 9, 17, 40),
+               (4, 1, 160, 128, 7, 8, 16), (4, 2, 64, 256, 4, 16, 16)]
+
+
+@pytest.mark.parametrize("bits,N,Ci,Co,D,H,W", WIDE_SHAPES)
+def test_wide_kernel_exact(gpu, bits, N, Ci, Co, D, H, W):
+    rng = np.random.default_rng(Ci * 17 + Co + D * 3 + bits)
+    S = D * H * W
+    x, w, b = exact_case(rng, N, Ci, Co, S)
+    xdt = 3 if bits == 8 else 4
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    want, wsum = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, acc64=1, Go=8, want_stats=True)
+    got, gsum = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, Go=8, stats=True)
+    assert "conv3_wide_k" in lib.mi_last_kernel().decode()
+    assert np.array_equal(got, want)
+    assert np.allclose(gsum, wsum, rtol=1e-6)
+    wf, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, acc64=1)
+    gf, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits)
+    assert np.array_equal(gf, wf)
+
+
+def test_wide_kernel_decoder_conv(gpu):
+    """[2x upsampled coarse | skip] -> 128 channels with both GroupNorms: the wide kernel on a split, restaged input (12 blocks)."""
+    rng = np.random.default_rng(77)
+    Cu, Cs, Co, (D, H, W) = 256, 128, 128, (4, 8, 16)
+    S, Sc = D * H * W, D * H * W // 8
+    xu = rng.standard_normal((1, Cu, Sc)).astype(np.float32); xs = rng.standard_normal((1, Cs, S)).astype(np.float32)
+    w = (rng.standard_normal((Co, Cu + Cs, 27)) * np.sqrt(2.0 / ((Cu + Cs) * 27))).astype(np.float32)
+    b = (rng.standard_normal(Co) * 0.1).astype(np.float32)
+    qu, qs = orc.f32_to_mx(8, xu, 1, Cu, Sc), orc.f32_to_mx(8, xs, 1, Cs, S)
+    G = 8
+    g1 = [rng.uniform(0.5, 1.5, Cu).astype(np.float32), rng.uniform(-0.3, 0.3, Cu).astype(np.float32), rng.uniform(-0.2, 0.2, G).astype(np.float32), rng.uniform(0.7, 1.4, G).astype(np.float32)]
+    g2 = [rng.uniform(0.5, 1.5, Cs).astype(np.float32), rng.uniform(-0.3, 0.3, Cs).astype(np.float32), rng.uniform(-0.2, 0.2, G).astype(np.float32), rng.uniform(0.7, 1.4, G).astype(np.float32)]
+    want, _ = orc.conv3(qu, 3, 1, Cu + Cs, D, H, W, w, b, Co, 0, x2=qs, c_split=Cu, up=1, gp=orc.gn(*g1, G=G), gp2=orc.gn(*g2, G=G))
+    got, _ = gpu_conv(qu, 3, 1, Cu + Cs, D, H, W, w, b, Co, 0, x2=qs, c_split=Cu, up=1, gp=dev_gn(*g1, G), gp2=dev_gn(*g2, G))
+    assert "conv3_wide_k" in lib.mi_last_kernel().decode()
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-3
+
+
 EXACT_SHAPES = [
     (8, 1, 32, 32, 2, 8, 16, 1), (8, 2, 32, 32, 5, 9, 18, 1), (8, 1, 64, 64, 8, 12, 20, 1), (8, 2, 128, 128, 4, 12, 20, 1), (8, 1, 96, 32, 6, 12, 20, 1),
     (8, 1, 160, 96, 3, 8, 16, 1), (8, 1, 256, 320, 4, 8, 16, 1), (8, 1, 32, 16, 5, 9, 18, 1), (8, 1, 48, 40, 4, 7, 9, 1),
