@@ -17,7 +17,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 METRIC = "U-Net infer voxels/s (128^3 patch, MX fp8) + 3x3x3 conv % of MFMA peak"
-TRAFFIC_BYTES_PER_LAUNCH = 187.7e6     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/
+TRAFFIC_BYTES_PER_LAUNCH = 184.1e6     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/
 MFMA_PEAK_FP8_TFLOPS = 5033.0          # MI355X dense MXFP8 (2.5 PFLOP/s bf16 x 2)
 
 
