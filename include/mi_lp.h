@@ -103,6 +103,12 @@ void mi_event_destroy(void *ev);
    act 0 none, 1 SiLU, 2 GELU (erf), 3 ReLU. bits 8 / 4 selects the compute format. */
 int mi_conv_fwd_fused(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                       const float *ep_a, const float *ep_b, int act, gnp_t gp, double *osum, int Go, split_t sp);
+/* extension with no counterpart in the reference (which zeroes the sum slots, runs the conv and finalizes in three launches,
+   src/nn_bwd.cu:37-56, src/nn_elem.cu:5-17): the stride-1 conv with its output GroupNorm statistics finalized by the conv's own
+   reduction. osum (2 N Go slots) need not be cleared: it is set to this conv's sums; omean / orstd (N Go floats) get
+   mean and 1 / sqrt(var + eps), bit-identical to mi_gn_sums_zero + lp_conv_fwd_f8 / _f4 + mi_gn_finalize. */
+int mi_conv_fwd_gn(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp,
+                   double *osum, int Go, split_t sp, float eps, float *omean, float *orstd);
 /* timing of the 3x3x3 conv kernel launches alone (benchmarks): on != 0 starts recording an event pair around every launch on the
    stream it runs on and clears the totals; read returns the total milliseconds so far and the number of launches (synchronises) */
 void mi_kernel_timing(int on);

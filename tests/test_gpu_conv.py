@@ -285,3 +285,32 @@ def test_full_size_properties(gpu, bits):
         assert np.array_equal(dec[:, :, z0:z1], wdec[:, :, z0:z1])
     # statistics == fp64 sums of the exact pre-quantisation values is checked at small sizes; here: sum of the sums is finite and stable
     assert np.isfinite(gs).all()
+
+
+@pytest.mark.parametrize("bits,Ci,Co,dims", [(8, 128, 128, (4, 8, 16)), (8, 32, 32, (5, 9, 18)), (4, 64, 64, (4, 8, 16)), (8, 32, 16, (4, 8, 16))])
+def test_fused_statistics_finalize(gpu, bits, Ci, Co, dims):
+    """mi_conv_fwd_gn == mi_gn_sums_zero + lp_conv_fwd_* + mi_gn_finalize, bit for bit (mean, rstd, slots), with uncleared slots on entry."""
+    rng = np.random.default_rng(Ci + Co + bits)
+    D, H, W = dims
+    N, S, G = 2, D * H * W, 8
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    dq = to_mx(bits, x)
+    dt = 3 if bits == 8 else 4
+    dw, db = DevBuf.from_numpy(w), DevBuf.from_numpy(b)
+    ybytes = (lib.lp_mx8_bytes if bits == 8 else lib.lp_mx4_bytes)(N, Co, S)
+    xs = shape5(N, Ci, D, H, W)
+    res = []
+    for fused in (False, True):
+        dy = DevBuf(ybytes); dsum = DevBuf.from_numpy(rng.integers(0, 255, N * G * 2 * 24).astype(np.uint8))     # garbage in the slots
+        dm, dr = DevBuf(N * G * 4), DevBuf(N * G * 4)
+        if fused:
+            assert lib.mi_conv_fwd_gn(bits, dq.ptr, dt, xs, dw.ptr, db.ptr, Co, dy.ptr, dt, gnp_t(), dsum.ptr, G, split_t(), 1e-5, dm.ptr, dr.ptr) == 0
+        else:
+            lib.mi_gn_sums_zero(dsum.ptr, N * G * 2)
+            f = lib.lp_conv_fwd_f8 if bits == 8 else lib.lp_conv_fwd_f4
+            assert f(dq.ptr, dt, xs, dw.ptr, db.ptr, Co, dy.ptr, dt, gnp_t(), dsum.ptr, G, split_t()) == 0
+            lib.mi_gn_finalize(dsum.ptr, N * G, (Co // G) * S, 1e-5, dm.ptr, dr.ptr)
+        LP.check()
+        res.append((dy.to_numpy(np.uint8), dsum.to_numpy(np.uint8), dm.to_numpy(np.float32), dr.to_numpy(np.float32)))
+    for u, v in zip(*res):
+        assert np.array_equal(u, v)

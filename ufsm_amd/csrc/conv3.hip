@@ -3,10 +3,32 @@
 // conv3_f*_o*.hip.
 #include "conv3_kernel.hpp"
 
+// what a reduce block does with the (sum, sum of squares) of its (sample, group): add them to the caller's sum slots (the reference's contract,
+// src/lp_common.cuh:1575-1597), or, for a fused call, set the slots and finalize mean / rstd from them right away (src/nn_elem.cu:5-11), which saves
+// the zeroing and finalize launches around the conv
+struct gn_fin_t { float *mean, *rstd; double len; float eps; };
+__device__ __forceinline__ void gn_part_finish(double *osum, double s, double ss, gn_fin_t fin) {
+    const size_t i = 2 * (size_t)blockIdx.x;
+    if (!fin.mean) { gn_acc_add(osum, i, s); gn_acc_add(osum, i + 1, ss); return; }
+    unsigned long long *w = (unsigned long long *)osum + 3 * i;
+    double v[2] = {s, ss}, got[2];
+#pragma unroll
+    for (int k = 0; k < 2; k++) {                       // the slot a single exact add to a cleared slot would leave, and its value read back
+        if (!(fabs(v[k]) < 4.611686018427387904e18)) { w[3 * k] = 0ull; w[3 * k + 1] = 0ull; w[3 * k + 2] = 1ull; got[k] = __longlong_as_double(0x7ff8000000000000ll); continue; }
+        const double f = floor(v[k]);
+        const unsigned long long lo = (unsigned long long)((v[k] - f) * 18446744073709551616.0);
+        w[3 * k] = lo; w[3 * k + 1] = (unsigned long long)(long long)f; w[3 * k + 2] = 0ull;
+        got[k] = (double)(long long)f + (double)lo * 5.42101086242752217e-20;
+    }
+    const double m = got[0] / fin.len, var = got[1] / fin.len - m * m;
+    fin.mean[blockIdx.x] = (float)m;
+    fin.rstd[blockIdx.x] = (float)(1.0 / sqrt((var > 0 ? var : 0) + (double)fin.eps));
+}
+
 // (sum, sum of squares) partials of the tiles -> exact GroupNorm sum slots: one block per (sample, group), double accumulation over
 // the sample's tiles in index order, a fixed tree over the block, one slot add per sum (src/lp_common.cuh:1575-1597 does the same with
 // one fixed-point atomic per block and channel)
-__global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum) {
+__global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum, gn_fin_t fin) {
     // the group's channel quads are consecutive: quad Q = co / 4 lives in channel slice Q / (8 MT), slot Q % (8 MT) of its tile's record
     const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, qpg = Co / Go / 4, nq = MT * 8, nst = tiles_per_n / ncs;
     double s = 0.0, ss = 0.0;
@@ -19,11 +41,11 @@ __global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int 
     r1[threadIdx.x] = s; r2[threadIdx.x] = ss;
     __syncthreads();
     for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) { r1[threadIdx.x] += r1[threadIdx.x + st]; r2[threadIdx.x] += r2[threadIdx.x + st]; } __syncthreads(); }
-    if (threadIdx.x == 0) { gn_acc_add(osum, 2 * (size_t)blockIdx.x, r1[0]); gn_acc_add(osum, 2 * (size_t)blockIdx.x + 1, r2[0]); }
+    if (threadIdx.x == 0) gn_part_finish(osum, r1[0], r2[0], fin);
 }
 
 // the same from per-channel records (32 per tile, one channel tile per workgroup)
-__global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, int tiles_per_n, int Co, int Go, double *osum) {
+__global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, int tiles_per_n, int Co, int Go, double *osum, gn_fin_t fin) {
     const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, cpg = Co / Go;
     double s = 0.0, ss = 0.0;
     for (int i = threadIdx.x; i < tiles_per_n * cpg; i += 256) {
@@ -35,7 +57,7 @@ __global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, i
     r1[threadIdx.x] = s; r2[threadIdx.x] = ss;
     __syncthreads();
     for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) { r1[threadIdx.x] += r1[threadIdx.x + st]; r2[threadIdx.x] += r2[threadIdx.x + st]; } __syncthreads(); }
-    if (threadIdx.x == 0) { gn_acc_add(osum, 2 * (size_t)blockIdx.x, r1[0]); gn_acc_add(osum, 2 * (size_t)blockIdx.x + 1, r2[0]); }
+    if (threadIdx.x == 0) gn_part_finish(osum, r1[0], r2[0], fin);
 }
 
 // ---- weights: fp32 w[co][ci][27] -> per (chunk, unit pair, 32-row channel tile) fragment-ordered codes + scale bytes ----
@@ -121,6 +143,8 @@ extern "C" double mi_kernel_timing_read(long *launches) {       // total millise
 extern "C" const char *mi_last_kernel(void) { return g_last_kernel; }
 
 // the conv of every entry point: fmt 8 / 4 = compute format, stride 1 / 2
+// set by mi_conv_fwd_gn around its conv: finalize the statistics in the reduce kernel
+static thread_local gn_fin_t g_fin = {nullptr, nullptr, 0.0, 0.f};
 static int conv_dispatch(const char *who, int fmt, int stride, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                          gnp_t gp, double *osum, int Go, split_t sp, const float *ep_a, const float *ep_b, int act) {
     if (sp.y2 || sp.o_split || sp.accum || sp.sr || sp.osr || sp.yD || sp.zi0 || sp.Di || sp.o_pad || sp.zw0 || sp.zw1 || sp.yzo)
@@ -265,8 +289,11 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     else { if (out == 8) conv3_launch_f4_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f4_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f4_o0(stride, epi, MT, NT, a, smem); }
     if (g_ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
     if (osum) {
-        if (a.stat_ch) gn_part_reduce_ch_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), cout, Go, osum);
-        else gn_part_reduce_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum);
+        gn_fin_t fin = g_fin;
+        fin.len = (double)(cout / Go) * (double)Do * Ho * Wo;
+        if (fin.mean && (sp.zlo || sp.zhi)) mi_die("%s: fused finalize with a z range", who);
+        if (a.stat_ch) gn_part_reduce_ch_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), cout, Go, osum, fin);
+        else gn_part_reduce_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum, fin);
         MICK();
     }
     return 0;
@@ -286,6 +313,15 @@ extern "C" int lp_conv_fwd_s2_f8(const void *x, int xbf, shape5 xs, const float 
     const bool f4 = xbf == 4 && xs.c == 32 && cout <= 32 && !(xs.d & 1) && !(xs.h & 1) && !(xs.w & 1);
     conv_dispatch("lp_conv_fwd_s2_f8", f4 ? 4 : 8, 2, x, xbf, xs, w, b, cout, y, ybf, gp, nullptr, 0, sp, nullptr, nullptr, 0);
     return f4 ? 3 : 0;
+}
+extern "C" int mi_conv_fwd_gn(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp,
+                              double *osum, int Go, split_t sp, float eps, float *omean, float *orstd) {
+    if (bits != 8 && bits != 4) mi_die("mi_conv_fwd_gn: compute format %d (8 or 4)", bits);
+    if (!osum || !omean || !orstd || Go <= 0) mi_die("mi_conv_fwd_gn: needs sum slots, mean and rstd buffers and groups");
+    g_fin = gn_fin_t{omean, orstd, 0.0, eps};
+    const int rc = conv_dispatch("mi_conv_fwd_gn", bits, 1, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, nullptr, nullptr, 0);
+    g_fin = gn_fin_t{nullptr, nullptr, 0.0, 0.f};
+    return rc;
 }
 extern "C" int mi_conv_fwd_fused(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                                  const float *ep_a, const float *ep_b, int act, gnp_t gp, double *osum, int Go, split_t sp) {

@@ -69,14 +69,15 @@ int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn
     double *sums = nullptr;
     if (G_out > 0 && omean) {
         sums = gn_dsums((size_t)2 * xs.n * G_out);
-        mi_gn_sums_zero(sums, 2 * xs.n * G_out);
         sp.stored_stats = gn_fused_stored(ydt, cout);
     }
     /* MX-fp4 storage or precision 3 run the fp4 kernels, everything else fp8; the <= 8 channel network input always runs in fp8
        (src/nn_bwd.cu:110-112, src/lp_f4fwd.cu:37) */
     const int f4 = (xdt == 4 || g_prec == 3) && xs.c > 8;
-    (f4 ? lp_conv_fwd_f4 : lp_conv_fwd_f8)(x, xdt, xs, w, b, cout, y, ydt, gp, sums, sums ? G_out : 0, sp);
-    if (sums) mi_gn_finalize(sums, xs.n * G_out, (size_t)(cout / G_out) * xs.d * xs.h * xs.w, eps, omean, orstd);
+    /* with output statistics: the conv's reduction sets the slots and finalizes them (the reference's zero / conv / finalize sequence,
+       src/nn_bwd.cu:37-56, in one call) */
+    if (sums) mi_conv_fwd_gn(f4 ? 4 : 8, x, xdt, xs, w, b, cout, y, ydt, gp, sums, G_out, sp, eps, omean, orstd);
+    else (f4 ? lp_conv_fwd_f4 : lp_conv_fwd_f8)(x, xdt, xs, w, b, cout, y, ydt, gp, nullptr, 0, sp);
     return 0;
 }
 int nn_conv3d_fwd_gn_stats(const float *x, shape5 xs, int G_in, const float *gamma, const float *beta, const float *mean, const float *rstd,

@@ -78,6 +78,7 @@ _PROTOS = {
     "mi_event_elapsed_ms": (_F, [_P, _P]),
     "mi_event_destroy": (None, [_P]),
     "mi_conv_fwd_fused": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, _P, _P, _I, gnp_t, _P, _I, split_t]),
+    "mi_conv_fwd_gn": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t, C.c_float, _P, _P]),
     "mi_kernel_timing": (None, [_I]),
     "mi_kernel_timing_read": (C.c_double, [C.POINTER(C.c_long)]),
     "mi_last_kernel": (C.c_char_p, []),
