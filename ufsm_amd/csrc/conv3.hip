@@ -225,7 +225,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // LDS of a workgroup holding CB input blocks: weight ring, pair table, halo rows and scale words. Prefer the largest CB that
     // still lets two workgroups share a CU (160 KB): the second one computes while the first stages its halo or runs its epilogue.
     // The wide kernel has a fixed layout: ring of two slots of two pairs, three halo slots of one block, two pair tables.
-    auto lds_bytes = [&](int cb) { return (size_t)2 * MT * (WTILE + 256) + (size_t)(((27 * cb + 1) >> 1) + 2) * 32 + (size_t)cb * TT * (RB + 4); };
+    const int PPS = MT == 1 ? 7 : MT == 2 ? 2 : 1;        // pairs per ring stage of the general kernel
+    auto lds_bytes = [&](int cb) { return (size_t)2 * PPS * MT * (WTILE + 256) + (size_t)(((27 * cb + 1) >> 1) + 2) * 32 + (size_t)cb * TT * (RB + 4); };
     int cb2 = 0, cb1 = 0;
     for (int cb = 1; cb <= a.nbt; cb++) { if (lds_bytes(cb) <= 80 * 1024 - 2816) cb2 = cb; if (lds_bytes(cb) <= 160 * 1024 - 3072) cb1 = cb; }   // (room for the epilogue's constants and scratch)
     int cbmax = cb2 ? cb2 : cb1;
@@ -257,8 +258,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // ---- weights ----
     int npairs_all = 0;
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) npairs_all += (27 * (a.nbt - b0 < a.CB ? a.nbt - b0 : a.CB) + 1) >> 1;
-    // (eight pairs of padding: the kernels' weight loads run up to seven pairs ahead of the last one)
-    const size_t wq_bytes = (size_t)(npairs_all + 8) * nmt_all * WTILE, wsc_bytes = (size_t)(npairs_all + 8) * nmt_all * 256;
+    // (sixteen pairs of padding: the kernels' weight loads run up to two ring stages ahead of the last pair)
+    const size_t wq_bytes = (size_t)(npairs_all + 16) * nmt_all * WTILE, wsc_bytes = (size_t)(npairs_all + 16) * nmt_all * 256;
     const int CxP = (Cx + 31) / 32 * 32;
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;

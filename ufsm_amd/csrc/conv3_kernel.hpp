@@ -416,12 +416,12 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     constexpr int TZ = NT == 2 ? 2 : 4;
     constexpr int HZ = STRIDE * (TZ - 1) + 3, HY = STRIDE * 7 + 3, HX = STRIDE * 15 + 3, TT = HZ * HY * HX;
     constexpr int NH = fmt_t<FMT>::NH, WTILE = fmt_t<FMT>::WTILE;
-    constexpr int STG = MT * (WTILE + 256);              // one weight stage: MT tiles of codes, then MT x 64 scale words
-    constexpr int UPT = (MT * WTILE / 16 + 255) / 256;   // 16-byte weight units per thread and stage
+    constexpr int STG = MT * (WTILE + 256);              // the weights of one pair: MT tiles of codes, then MT x 64 scale words
+    constexpr int PPS = MT == 1 ? 7 : MT == 2 ? 2 : 1;   // pairs per ring stage
     extern __shared__ __align__(16) unsigned char lds[];
     // LDS: [2 weight stages][pair table (npairs + 2) x 2 x 16 B][halo rows CB * NH * TT * 16 B][halo scales CB * TT words]
     const int tab_bytes = (((27 * a.CB + 1) >> 1) + 2) * 32;
-    const unsigned wring_o = 0, tab_o = 2 * STG, act_o = tab_o + tab_bytes, asc_o = act_o + a.CB * NH * TT * 16;
+    const unsigned wring_o = 0, tab_o = 2 * PPS * STG, act_o = tab_o + tab_bytes, asc_o = act_o + a.CB * NH * TT * 16;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
 
     // XCD-aware tile order: consecutive workgroup ids land on different XCDs (8, round robin), so give each XCD a contiguous
@@ -450,8 +450,7 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
         ab[j] = act_o + ((NH == 2 ? h * TT : 0) + p0) * 16;
         sbse[j] = asc_o + p0 * 4;
     }
-    const unsigned wfa = wring_o + lane * 16, wfs = wring_o + MT * WTILE + lane * 4;    // the lane's weight fragment / scale word in stage slot 0, tile 0
-    const unsigned wcp = wring_o + (tid * UPT * 16) % (MT * WTILE), wcs = wring_o + MT * WTILE + (tid * 4) % (MT * 256);   // the thread's part of a stage copy
+    const unsigned wfa = wring_o + lane * 16, wfs = wring_o + MT * WTILE + lane * 4;    // the lane's weight fragment / scale word of the ring's first pair, tile 0
 
     v16f acc[MT][NT];
 #pragma unroll
@@ -468,36 +467,47 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) {
         const int nbc = min(a.CB, a.nbt - b0), nunits = 27 * nbc, npairs = (nunits + 1) >> 1;
         __syncthreads();                                 // the previous chunk's readers are done with the halo
+        DBG_MARK(0);
         conv_pair_table<FMT, STRIDE, TZ>(lds, tab_o, nbc, tid);
+        DBG_MARK(1);
         if (a.wide) conv_stage_halo<FMT, STRIDE, TZ, 1, true>(a, lds, act_o, asc_o, b0, nbc, n, iz0, iy0, ix0, tid);
         else conv_stage_halo<FMT, STRIDE, TZ, 1, false>(a, lds, act_o, asc_o, b0, nbc, n, iz0, iy0, ix0, tid);
-        // ---- weight stages: global -> registers -> ring slot. Every thread moves UPT contiguous 16-byte units and one scale word per
-        // stage; offsets wrap instead of being guarded (duplicates store the same value). The prepared-weight buffers carry four
-        // stages of padding, so the loads that run ahead of the last pair stay inside them ----
-        const uint8_t *wgp = a.wq + (size_t)pair0 * wq_ps + (size_t)cs * MT * WTILE + (tid * UPT * 16) % (MT * WTILE);
-        const uint8_t *wgs = a.wsc + (size_t)pair0 * wsc_ps + (size_t)cs * MT * 256 + (tid * 4) % (MT * 256);
-        v4i g[UPT]; unsigned gs = 0;
-        auto wload = [&]() {            // the next stage in sequence
+        // ---- weight stages: global -> registers -> ring slot, PPS pairs per stage (more pairs per stage for few channel tiles: with one
+        // tile a pair is only NT MFMAs per wavefront, too little work between two barriers). A thread moves up to UPS 16-byte units per
+        // stage; the prepared-weight buffers carry padding pairs, so the loads that run ahead of the last stage stay inside them ----
+        constexpr int U16 = STG / 16, C16 = MT * WTILE / 16;     // 16-byte units of a pair: codes, then scale words
+        constexpr int UPS = (PPS * U16 + 255) / 256;
+        v4i g[UPS];
+        int wstage = 0;                                      // the next stage to load
+        auto wload = [&]() {
 #pragma unroll
-            for (int k = 0; k < UPT; k++) g[k] = *(const v4i *)(wgp + k * 16);
-            gs = *(const unsigned *)wgs;
-            wgp += wq_ps; wgs += wsc_ps;
+            for (int k = 0; k < UPS; k++) {
+                const int u = min(tid + k * 256, PPS * U16 - 1), p = u / U16, w16 = u - p * U16;
+                const size_t gp = (size_t)(pair0 + wstage * PPS + p);
+                const uint8_t *src = w16 < C16 ? a.wq + gp * wq_ps + (size_t)cs * MT * WTILE + w16 * 16 : a.wsc + gp * wsc_ps + (size_t)cs * MT * 256 + (w16 - C16) * 16;
+                g[k] = *(const v4i *)src;
+            }
+            wstage++;
         };
         auto wstore = [&](int slot) {
 #pragma unroll
-            for (int k = 0; k < UPT; k++) *(v4i *)(lds + wcp + slot * STG + k * 16) = g[k];
-            *(unsigned *)(lds + wcs + slot * STG) = gs;
+            for (int k = 0; k < UPS; k++) {
+                const int u = tid + k * 256;
+                if (u < PPS * U16) *(v4i *)(lds + wring_o + slot * PPS * STG + u * 16) = g[k];
+            }
         };
+        DBG_MARK(2);
         wload(); wstore(0);
         __syncthreads();
+        DBG_MARK(3);
 
-        // ---- K loop over unit pairs, unrolled by 2 so that the ring slot (pair & 1) is static. Step of pair q: start loading stage q + 1 from
-        // L2, fetch the pair's fragments from LDS (halo rows at the table's offsets, weights from ring slot q & 1), run its MFMAs,
-        // move stage q + 1 into the other slot. A second workgroup on the CU covers this one's LDS latency and barriers ----
+        // ---- K loop over stages of PPS unit pairs. Stage st: start loading stage st + 1 from L2; for each of its pairs fetch the fragments
+        // from LDS (halo rows at the table's offsets, weights from ring slot st & 1) and run the MFMAs; move stage st + 1 into the other
+        // slot; one barrier. A second workgroup on the CU covers this one's LDS latency and barriers ----
         v8i fb[NT], fa[MT]; int sb[NT], sa[MT];
         v4i T;
         unsigned tabp = tab_o + (lane >> 5) * 16;          // this half's entry of pair 0
-        auto fetch = [&](int slot) {
+        auto fetch = [&](unsigned wo) {
             const v4i t = T;
 #pragma unroll
             for (int j = 0; j < NT; j++) {
@@ -510,12 +520,12 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
             }
 #pragma unroll
             for (int m = 0; m < MT; m++) {
-                const v4i lo = *(const v4i *)(lds + wfa + slot * STG + m * WTILE);
+                const v4i lo = *(const v4i *)(lds + wfa + wo + m * WTILE);
                 if (FMT == 8) {
-                    const v4i hi = *(const v4i *)(lds + wfa + slot * STG + m * WTILE + 1024);
+                    const v4i hi = *(const v4i *)(lds + wfa + wo + m * WTILE + 1024);
                     fa[m] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 } else fa[m] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                sa[m] = *(const int *)(lds + wfs + slot * STG + m * 256);
+                sa[m] = *(const int *)(lds + wfs + wo + m * 256);
             }
             T = *(const v4i *)(lds + tabp + 32); tabp += 32;      // the next pair's table entry
         };
@@ -527,13 +537,17 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
                     acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[m], fb[j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sa[m], 0, sb[j]);
         };
         T = *(const v4i *)(lds + tabp);
-        for (int q = 0; q < npairs; q += 2) {
-            wload(); fetch(0); mma(); wstore(1);
-            __syncthreads();
-            if (q + 1 >= npairs) break;
-            wload(); fetch(1); mma(); wstore(0);
+        const int nstg = (npairs + PPS - 1) / PPS;
+        for (int st = 0; st < nstg; st++) {
+            const unsigned so = (unsigned)(st & 1) * (PPS * STG);
+            wload();
+#pragma unroll
+            for (int p = 0; p < PPS; p++)
+                if (st * PPS + p < npairs) { fetch(so + p * STG); mma(); }
+            wstore((st & 1) ^ 1);
             __syncthreads();
         }
+        DBG_MARK(4);
         pair0 += npairs;
     }
 
