@@ -552,3 +552,101 @@ void orc_conv1_mx(int xbits, const uint8_t *x, int N, int Ci, size_t S, const fl
         }
     }
 }
+
+/* ---------- MX GEMM (src/lp_mxgemm.cu:1-5, :17-41 staging, :88-113 packing, :266-297 entry) ----------
+   C[M][N] = op(A) op(B) + bias[col] + res[row][col] + beta C; A is [M][K] (ta 0) or [K][M] (ta 1), B is [K][N] (tb 0) or [N][K] (tb 1).
+   Every 32 K-values of an A row / B column get one scale from the fmaxf amax (zero past K), the elements round to e2m1 / e4m3; the
+   products of one 32-K block are summed exactly, the block sums accumulate in fp32 in K order. */
+static void gemm_quant_rows(int bits, const float *X, int tr, int ld, int rows, int K, int nkb, float *Q) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < (int64_t)rows * nkb; i++) {
+        const int r = (int)(i / nkb), kb = (int)(i % nkb);
+        float v[32]; uint8_t codes[32];
+        for (int j = 0; j < 32; j++) { const int k = kb * 32 + j; v[j] = k < K ? (tr ? X[(size_t)k * ld + r] : X[(size_t)r * ld + k]) : 0.f; }
+        const uint8_t sb = orc_store_row(bits, v, 32, codes, 0);
+        orc_load_row(bits, codes, sb, 32, Q + (size_t)i * 32);
+    }
+}
+int orc_mx_gemm(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res) {
+    if (bits != 4 && bits != 8) return -1;
+    if (M <= 0 || N <= 0) return 0;
+    const int nkb = (K + 31) / 32;
+    float *Aq = (float *)malloc((size_t)M * nkb * 32 * sizeof(float) + 4), *Bq = (float *)malloc((size_t)N * nkb * 32 * sizeof(float) + 4);
+    gemm_quant_rows(bits, A, ta, ta ? M : K, M, K, nkb, Aq);
+    gemm_quant_rows(bits, B, !tb, tb ? K : N, N, K, nkb, Bq);    /* B's "rows" are the output columns */
+#pragma omp parallel for schedule(static)
+    for (int64_t ij = 0; ij < (int64_t)M * N; ij++) {
+        const int i = (int)(ij / N), j = (int)(ij % N);
+        const float *a = Aq + (size_t)i * nkb * 32, *b = Bq + (size_t)j * nkb * 32;
+        float acc = 0.f;
+        for (int kb = 0; kb < nkb; kb++) { double s = 0.0; for (int k = 0; k < 32; k++) s += (double)a[kb * 32 + k] * (double)b[kb * 32 + k]; acc += (float)s; }
+        float *p = C + (size_t)i * N + j;
+        *p = acc + (bias ? bias[j] : 0.f) + (res ? res[(size_t)i * N + j] : 0.f) + (beta != 0.f ? beta * *p : 0.f);
+    }
+    free(Aq); free(Bq);
+    return 0;
+}
+
+/* ---------- MX-fp8 attention forward (src/lp_attn8.cu:29-76 conversions, :124-180 forward, :319-328 entry) ----------
+   qkvh: fp16 [3][H][T + 64][48] (T = nseq S; row of token i of sequence s = s S + i). Q and K rows are quantised in two blocks (dims
+   0..31, dims 32..47 zero-padded to 32); V is quantised along the tokens: per (head, dim) one scale per 32 tokens of the sequence
+   (tokens past S are zero). Keys are visited in tiles of 64: logits s = (q . k) log2(e) / sqrt(48), keys past S masked; running maximum
+   m and sum l in base 2; P = 2^(s - m) is quantised per query per 32 keys and multiplied with the quantised V, the accumulator rescaled
+   by 2^(m_old - m_new). o [T][C] = acc / l at column h 48 + d; lse [nseq][H][S] = m + log2(l). */
+void orc_fa8_fwd(const uint16_t *qkvh, float *o, float *lse, int nseq, int S, int H, int C) {
+    enum { HD = 48, FT = 64 };
+    const int64_t T = (int64_t)nseq * S, Tp = T + FT; const int Sp = (S + FT - 1) / FT * FT;
+    const float sl2 = 1.4426950408889634f / sqrtf((float)HD);
+    const uint16_t *Qh = qkvh, *Kh = Qh + (size_t)H * Tp * HD, *Vh = Kh + (size_t)H * Tp * HD;
+    for (int seq = 0; seq < nseq; seq++) for (int h = 0; h < H; h++) {
+        float *qd = (float *)calloc((size_t)Sp * 64, sizeof(float)), *kd = (float *)calloc((size_t)Sp * 64, sizeof(float)), *vd = (float *)calloc((size_t)HD * Sp, sizeof(float));
+        for (int p = 0; p < 2; p++) {
+            const uint16_t *src = (p ? Kh : Qh) + ((size_t)h * Tp + (size_t)seq * S) * HD; float *dst = p ? kd : qd;
+#pragma omp parallel for schedule(static)
+            for (int i = 0; i < S; i++) for (int kb = 0; kb < 2; kb++) {
+                float v[32]; uint8_t codes[32]; const int n = kb ? HD - 32 : 32;
+                for (int j = 0; j < 32; j++) v[j] = j < n ? orc_h16_to_f32(src[(size_t)i * HD + 32 * kb + j]) : 0.f;
+                const uint8_t sb = orc_store_row(8, v, 32, codes, 0);
+                orc_load_row(8, codes, sb, 32, dst + (size_t)i * 64 + 32 * kb);
+            }
+        }
+        const uint16_t *vs = Vh + ((size_t)h * Tp + (size_t)seq * S) * HD;
+#pragma omp parallel for schedule(static)
+        for (int d = 0; d < HD; d++) for (int b = 0; b < Sp / 32; b++) {
+            float v[32]; uint8_t codes[32];
+            for (int r = 0; r < 32; r++) { const int i = b * 32 + r; v[r] = i < S ? orc_h16_to_f32(vs[(size_t)i * HD + d]) : 0.f; }
+            const uint8_t sb = orc_store_row(8, v, 32, codes, 0);
+            orc_load_row(8, codes, sb, 32, vd + (size_t)d * Sp + b * 32);
+        }
+#pragma omp parallel for schedule(dynamic, 16)
+        for (int i = 0; i < S; i++) {
+            float m = -INFINITY, l = 0.f, acc[HD]; for (int d = 0; d < HD; d++) acc[d] = 0.f;
+            const float *q = qd + (size_t)i * 64;
+            for (int kb = 0; kb < S; kb += FT) {
+                float s[FT], mx = -INFINITY;
+                for (int j = 0; j < FT; j++) {
+                    const float *k = kd + (size_t)(kb + j) * 64; float a = 0.f;
+                    for (int b = 0; b < 2; b++) { double t = 0.0; for (int c = 0; c < 32; c++) t += (double)q[32 * b + c] * (double)k[32 * b + c]; a += (float)t; }
+                    s[j] = kb + j < S ? a * sl2 : -INFINITY; mx = fmaxf(mx, s[j]);
+                }
+                const float mn = fmaxf(m, mx), corr = exp2f(m - mn); m = mn; l *= corr;
+                for (int j = 0; j < FT; j++) { s[j] = exp2f(s[j] - m); l += s[j]; }
+                for (int d = 0; d < HD; d++) acc[d] *= corr;
+                for (int b = 0; b < 2; b++) {
+                    uint8_t codes[32]; float pq[32];
+                    const uint8_t sb = orc_store_row(8, s + 32 * b, 32, codes, 0);
+                    orc_load_row(8, codes, sb, 32, pq);
+                    for (int d = 0; d < HD; d++) {
+                        const float *v = vd + (size_t)d * Sp + kb + 32 * b; double t = 0.0;
+                        for (int j = 0; j < 32; j++) t += (double)pq[j] * (double)v[j];
+                        acc[d] += (float)t;
+                    }
+                }
+            }
+            const float il = 1.f / l; float *orow = o + ((size_t)seq * S + i) * C + h * HD;
+            for (int d = 0; d < HD; d++) orow[d] = acc[d] * il;
+            lse[((size_t)seq * H + h) * S + i] = m + log2f(l);
+        }
+        free(qd); free(kd); free(vd);
+    }
+}

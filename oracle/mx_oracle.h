@@ -14,6 +14,12 @@
  *   GroupNorm sums / finalize     pinned: independent fp64 statistics; constant group => rstd = 1/sqrt(eps)
  *   trilinear staging, up2        pinned: closed form 0.75/0.25 separable weights with edge clamp, grid data exact
  *   1x1x1 head                    pinned: plain dot product (GEMM special case)
+ *   orc_mx_gemm                   pinned: == fp64 product of operands quantised by an independent numpy block quantiser
+ *                                 (tests/test_attn.c:375-396), all transpose flags, ragged M / N / K; exact-operand case == integer product
+ *   orc_fa8_fwd                   pinned: closed forms (uniform logits -> mean of the quantised V and lse = log2 S; one dominant key ->
+ *                                 that key's quantised V row, also when the maximum moves between key tiles; keys past S never
+ *                                 contribute) and the reference's own gate, rel. L2 < 0.1 against exact fp64 attention
+ *                                 (tests/test_attn.c:445-446)
  *   SiLU in GN staging            PARITY UNPINNED to the bit: the reference evaluates tanh with NVIDIA's
  *                                 tanh.approx.f32 (src/lp_common.cuh:469-473), not reproducible off that hardware;
  *                                 checked to floor/ceil code neighbours as tests/test_mx4_wide.c:165-175 does
@@ -98,6 +104,10 @@ void orc_up2_mx(int xbits, const uint8_t *x, int N, int C, int D, int H, int W, 
 /* 1x1x1 head (src/lp_mx_conv1.cu:5-21): y[n][co][v] fp32 */
 void orc_conv1_mx(int xbits, const uint8_t *x, int N, int Ci, size_t S, const float *w, const float *b, int Co, orc_gn_t gp, float *y);
 /* GN affine + SiLU of the conv staging (src/lp_common.cuh:474-482): u = fma(v, a, b), u sigmoid(u) correctly rounded */
+/* MX GEMM of row-major fp32 operands quantised along K (src/lp_mxgemm.cu:266-297); 0, or -1 for unsupported bits */
+int orc_mx_gemm(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res);
+/* MX-fp8 attention forward on the fp16 head-major pack (src/lp_attn8.cu:124-180, :319-328); head dim 48 */
+void orc_fa8_fwd(const uint16_t *qkvh, float *o, float *lse, int nseq, int S, int H, int C);
 float orc_act_ab(float v, float a, float b);
 uint16_t orc_f32_to_h16(float f);
 float orc_h16_to_f32(uint16_t h);

@@ -60,6 +60,9 @@ def lib():
         L.orc_f32_to_h16.restype = C.c_uint16; L.orc_f32_to_h16.argtypes = [C.c_float]
         L.orc_h16_to_f32.restype = C.c_float; L.orc_h16_to_f32.argtypes = [C.c_uint16]
         L.orc_threads.restype = C.c_int
+        L.orc_mx_gemm.restype = C.c_int
+        L.orc_mx_gemm.argtypes = [C.c_int] * 6 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p]
+        L.orc_fa8_fwd.restype = None; L.orc_fa8_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
         _lib = L
     return _lib
 
@@ -117,3 +120,21 @@ def conv3(x, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=8, stride=1, x2=None, c_s
     assert rc == 0, rc
     del keep
     return y, sums
+
+
+def mx_gemm(bits, ta, tb, M, N, K, A, B, C0=None, beta=0.0, bias=None, res=None):
+    """C = op(A) op(B) + bias + res + beta C0 with MX-quantised operands; A, B float32 in their stored (possibly transposed) layout."""
+    A = np.ascontiguousarray(A, dtype=np.float32); B = np.ascontiguousarray(B, dtype=np.float32)
+    out = np.zeros((M, N), np.float32) if C0 is None else np.array(C0, dtype=np.float32, copy=True)
+    rc = lib().orc_mx_gemm(bits, ta, tb, M, N, K, ptr(A), ptr(B), ptr(out), beta, ptr(bias), ptr(res))
+    assert rc == 0
+    return out
+
+
+def fa8_fwd(qkvh, nseq, S, H):
+    """qkvh: uint16 (fp16 bits) [3][H][nseq * S + 64][48] -> (o [nseq * S][H * 48], lse [nseq][H][S]) float32."""
+    qkvh = np.ascontiguousarray(qkvh, dtype=np.uint16)
+    assert qkvh.shape == (3, H, nseq * S + 64, 48)
+    o = np.zeros((nseq * S, H * 48), np.float32); lse = np.zeros((nseq, H, S), np.float32)
+    lib().orc_fa8_fwd(ptr(qkvh), ptr(o), ptr(lse), nseq, S, H, H * 48)
+    return o, lse

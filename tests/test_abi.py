@@ -32,6 +32,17 @@ def test_library_exports_every_declared_symbol():
     assert set(header_functions()) == set(lp.EXPORTS)
 
 
+def test_library_exports_the_attention_header():
+    from ufsm_amd import lp
+    L = lp.load()
+    names = header_functions("mi_attn.h", ("lp_", "at_"))
+    assert set(names) == {"lp_mx_gemm", "lp_mx_gemm_ex", "at_fa8_fwd"} == set(lp.ATTN_EXPORTS)
+    for n in names:
+        assert hasattr(L, n), "libufsm_lp.so does not export %s" % n
+    # at_geom as the reference lays it out on LP64 (src/attn.h:81): five ints, padding, seven pointers
+    assert C.sizeof(lp.at_geom) == 24 + 7 * 8 and lp.at_geom.lens.offset == 24 and lp.at_geom.dfr.offset == 72
+
+
 def test_host_library_exports_every_declared_symbol():
     from ufsm_amd import unet
     H = unet.load_host()

@@ -1,0 +1,190 @@
+// MX-fp8 attention forward core: softmax(Q K^T / sqrt(48)) V per sequence and head on block-scaled e4m3 MFMA (32x32x64).
+// Interface and arithmetic: src/lp_attn8.cu:1-13 (definition), :29-76 (conversions), :124-180 (forward), :319-328 (entry) of the reference.
+//
+// The products are formed transposed, S^T = K Q^T and O^T = V^T P^T, so a query is a column of every accumulator: a lane (r, h) holds,
+// for query r of its wavefront, 16 of the 32 keys of each key block and its partner lane (r, h ^ 1) the other 16. All row statistics
+// of the softmax (maximum, sum, the rescale factor, the MX scale of P) are then per lane plus one exchange with the partner.
+// An 8-bit operand fragment of the 32x32x64 MFMA holds, in lane (r, h), bytes 16 h ... 16 h + 15 of both 32-K blocks of row r (and
+// that lane's scale operand is block h's): exactly the 16 + 16 keys whose P the lane has in its accumulators, so P goes from
+// accumulators to the B fragment of the second product in registers with no data exchange at all. The transposed V stores the tokens
+// of a block in the matching order.
+#include <hip/hip_fp16.h>
+#include "mx_dev.hpp"
+#include "../../include/mi_attn.h"
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+#define HD AT_HD
+#define FT 64            // keys per tile; sequences are padded to a multiple of it in the quantised tensors (rows past S are zero)
+
+// Slot k of a 32-token block of the transposed V holds token a8_slot_token(k) of the block: slots 16 h + 4 q + c are lane half h's
+// accumulator elements 4 q + c, which are the block's keys 8 q + 4 h + c.
+__host__ __device__ __forceinline__ int a8_slot_token(int k) { return 8 * ((k >> 2) & 3) + 4 * (k >> 4) + (k & 3); }
+
+// row-quantised q / k: thread per (head, row, 32-dim block); src fp16 [H][Tp][48] (token i of sequence s in row s S + i),
+// dst [H][R][64] e4m3 + scales [H][R][2] (dims 0..31, dims 32..47 zero-padded), R = nseq Sp
+__global__ void __launch_bounds__(256) a8_rq_k(const __half *__restrict__ src, uint8_t *__restrict__ dst, uint8_t *__restrict__ sc, int H, int nseq, int S, int Sp, long long Tp) {
+    const long long R = (long long)nseq * Sp, i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
+    if (i >= (long long)H * R * 2) return;
+    const int kb = (int)(i & 1); const long long hr = i >> 1; const int h = (int)(hr / R); const long long row = hr % R;
+    const int seq = (int)(row / Sp), ii = (int)(row % Sp), n = kb ? HD - 32 : 32;
+    float v[32];
+    const __half *s = src + ((size_t)h * Tp + (size_t)seq * S + min(ii, S - 1)) * HD + 32 * kb;
+#pragma unroll
+    for (int j = 0; j < 32; j++) v[j] = ii < S && j < n ? __half2float(s[j < n ? j : 0]) : 0.f;
+    unsigned codes[8];
+    const unsigned sb = d_quant_row<8, false>(v, 32, codes);
+    uint4 *o = (uint4 *)(dst + ((size_t)h * R + row) * 64 + 32 * kb);
+    o[0] = make_uint4(codes[0], codes[1], codes[2], codes[3]); o[1] = make_uint4(codes[4], codes[5], codes[6], codes[7]);
+    sc[((size_t)h * R + row) * 2 + kb] = (uint8_t)sb;
+}
+// transposed v: workgroup per (head, 32-token block), 64 threads; dst [H][48][R] in slot order + scales [H][48][R / 32]
+__global__ void __launch_bounds__(64) a8_tq_k(const __half *__restrict__ src, uint8_t *__restrict__ dst, uint8_t *__restrict__ sc, int H, int nseq, int S, int Sp, long long Tp) {
+    const long long R = (long long)nseq * Sp; const int nb = (int)(R / 32), h = blockIdx.x / nb, b = blockIdx.x % nb;
+    const long long r0 = (long long)b * 32; const int seq = (int)(r0 / Sp), i0 = (int)(r0 % Sp);
+    __shared__ float t[32][HD + 1];
+    for (int e = threadIdx.x; e < 32 * HD; e += blockDim.x) {
+        const int r = e / HD, d = e % HD, ii = i0 + r;
+        t[r][d] = ii < S ? __half2float(src[((size_t)h * Tp + (size_t)seq * S + ii) * HD + d]) : 0.f;
+    }
+    __syncthreads();
+    const int d = threadIdx.x;
+    if (d >= HD) return;
+    float v[32];
+#pragma unroll
+    for (int k = 0; k < 32; k++) v[k] = t[a8_slot_token(k)][d];
+    unsigned codes[8];
+    const unsigned sb = d_quant_row<8, false>(v, 32, codes);
+    uint4 *o = (uint4 *)(dst + ((size_t)h * HD + d) * R + r0);
+    o[0] = make_uint4(codes[0], codes[1], codes[2], codes[3]); o[1] = make_uint4(codes[4], codes[5], codes[6], codes[7]);
+    sc[((size_t)h * HD + d) * (R / 32) + b] = (uint8_t)sb;
+}
+
+__device__ __forceinline__ float a8_xor32f(float x, int h) {
+    const unsigned u = __float_as_uint(x);
+    const auto r2 = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __uint_as_float(h ? r2[0] : r2[1]);
+}
+// the lane's fragment of a 64-byte row of two 32-K blocks: bytes 16 h ... of each (p already points at byte 16 h)
+__device__ __forceinline__ v8i a8_frag(const uint8_t *p) {
+    const v4i lo = *(const v4i *)p, hi = *(const v4i *)(p + 32);
+    return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+}
+
+// grid (ceil(S / 128), H, nseq), 4 wavefronts of 32 queries each. Fragments are the quantised tensors' rows as they lie in memory
+// (32 contiguous bytes per lane), loaded from global memory directly: a sequence's K and V of one head are 7 KB per 64 keys and stay in
+// L2 / the vector cache across the workgroup's wavefronts.
+__global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, const uint8_t *__restrict__ Q8s, const uint8_t *__restrict__ K8, const uint8_t *__restrict__ K8s,
+                                                const uint8_t *__restrict__ Vt, const uint8_t *__restrict__ Vts, float *__restrict__ o, float *__restrict__ lse,
+                                                int S, int Sp, int H, int C, long long R, float sl2) {
+    const int seq = blockIdx.z, hd = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    const int q0 = blockIdx.x * 128 + wave * 32;
+    if (q0 >= S) return;                                   // (no barriers: a wavefront without queries leaves)
+    const long long rb = (long long)hd * R + (long long)seq * Sp;          // the sequence's first row in the row-quantised tensors
+    const long long c0 = (long long)seq * Sp;                              // its first column in the transposed one
+    const v8i qf = a8_frag(Q8 + (rb + q0 + r) * 64 + 16 * h);
+    const int qs = Q8s[(rb + q0 + r) * 2 + h];
+    const uint8_t *kp = K8 + (rb + r) * 64 + 16 * h, *ksp = K8s + (rb + r) * 2 + h;
+    // V^T rows: dims r and 32 + r (the second tile has 16 real rows; the others multiply zeros)
+    const int d1 = min(32 + r, HD - 1); const bool d1ok = 32 + r < HD;
+    const uint8_t *vp0 = Vt + ((size_t)hd * HD + r) * R + c0 + 16 * h, *vp1 = Vt + ((size_t)hd * HD + d1) * R + c0 + 16 * h;
+    const uint8_t *vs0 = Vts + ((size_t)hd * HD + r) * (R / 32) + c0 / 32 + h, *vs1 = Vts + ((size_t)hd * HD + d1) * (R / 32) + c0 / 32 + h;
+    float m = -INFINITY, l = 0.f;
+    v16f oa[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) oa[t][i] = 0.f;
+    const int nt = (S + FT - 1) / FT;
+    for (int it = 0; it < nt; it++) {
+        const int kb = it * FT;
+        // ---- S^T = K Q^T for the tile's two blocks of 32 keys ----
+        v16f s[2];
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const v8i kf = a8_frag(kp + (size_t)(kb + 32 * b) * 64);
+            const int ks = ksp[(size_t)(kb + 32 * b) * 2];
+            v16f z;
+#pragma unroll
+            for (int i = 0; i < 16; i++) z[i] = 0.f;
+            s[b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf, z, 0, 0, 0, ks, 0, qs);
+        }
+        // next: the V fragments of this tile (independent of the softmax: their latency hides behind it)
+        v8i vf0 = a8_frag(vp0 + kb), vf1 = a8_frag(vp1 + kb);
+        const int e0v = vs0[kb / 32], e1v = vs1[kb / 32];
+        if (!d1ok) vf1 = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
+        // ---- logits in base-2 units, keys past S masked (only the last tile can hold them) ----
+        const bool full = kb + FT <= S;
+        float mx = -INFINITY;
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int key = kb + 32 * b + (i & 3) + 4 * h + 8 * (i >> 2);
+                const float v = full || key < S ? s[b][i] * sl2 : -INFINITY;
+                s[b][i] = v; mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, a8_xor32f(mx, h));
+        const float mn = fmaxf(m, mx), corr = __builtin_amdgcn_exp2f(m - mn);
+        m = mn; l *= corr;
+        float am[2] = {0.f, 0.f};
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) { const float p = __builtin_amdgcn_exp2f(s[b][i] - m); s[b][i] = p; l += p; am[b] = fmaxf(am[b], p); }
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) oa[t][i] *= corr;
+        // ---- P -> e4m3 with one scale per query per 32 keys; the lane's codes are its B fragment, its scale operand is block h's ----
+        unsigned cw[2][4]; int ep[2];
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            am[b] = fmaxf(am[b], a8_xor32f(am[b], h));
+            ep[b] = d_mx_exp(am[b], MI_INVQ8);
+            const float p2e = d_exp2i(ep[b]);
+#pragma unroll
+            for (int q = 0; q < 4; q++) cw[b][q] = d_enc_e4m3x4_hw(s[b][4 * q], s[b][4 * q + 1], s[b][4 * q + 2], s[b][4 * q + 3], p2e);
+        }
+        const v8i pf = {(int)cw[0][0], (int)cw[0][1], (int)cw[0][2], (int)cw[0][3], (int)cw[1][0], (int)cw[1][1], (int)cw[1][2], (int)cw[1][3]};
+        const int ps = (h ? ep[1] : ep[0]) + 127;
+        // ---- O^T += V^T P^T ----
+        oa[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf0, pf, oa[0], 0, 0, 0, e0v, 0, ps);
+        oa[1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf1, pf, oa[1], 0, 0, 0, e1v, 0, ps);
+    }
+    l += a8_xor32f(l, h);
+    const int i = q0 + r;
+    if (i >= S) return;
+    const float il = 1.f / l;
+    float *orow = o + ((size_t)seq * S + i) * C + hd * HD;
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const int d0 = 32 * t + 4 * h + 8 * g;         // accumulator elements 4 g ... 4 g + 3: dims d0 ... d0 + 3
+            if (d0 < HD) *(float4 *)(orow + d0) = make_float4(oa[t][4 * g] * il, oa[t][4 * g + 1] * il, oa[t][4 * g + 2] * il, oa[t][4 * g + 3] * il);
+        }
+    if (!h) lse[((size_t)seq * H + hd) * S + i] = m + __log2f(l);
+}
+
+extern "C" int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom *g, int H, int C) {
+    if (!g || g->nseq <= 0 || g->S <= 0 || H <= 0) return 0;
+    if (C != H * HD) mi_die("at_fa8_fwd: C %d is not %d heads of %d", C, H, HD);
+    if (g->lens || g->rays) mi_die("at_fa8_fwd: per-sequence lengths and ray geometry are not supported");
+    const long long T = (long long)g->nseq * g->S, Tp = T + FT; const int Sp = (g->S + FT - 1) / FT * FT; const long long R = (long long)g->nseq * Sp;
+    const size_t rq = (size_t)H * R * 64, rqs = (size_t)H * R * 2, tq = (size_t)H * HD * R, tqs = (size_t)H * HD * (R / 32);
+    auto al = [](size_t n) { return (n + 255) & ~(size_t)255; };
+    uint8_t *base = (uint8_t *)mi_ws(MI_WS_ATTN, 2 * (al(rq) + al(rqs)) + al(tq) + al(tqs));
+    if (!base) return -1;
+    uint8_t *q8 = base, *k8 = q8 + al(rq), *qs = k8 + al(rq), *ks = qs + al(rqs), *vt = ks + al(rqs), *vts = vt + al(tq);
+    const __half *Qh = (const __half *)qkvh, *Kh = Qh + (size_t)H * Tp * HD, *Vh = Kh + (size_t)H * Tp * HD;
+    const unsigned gq = nblk_((size_t)H * R * 2, 256);
+    a8_rq_k<<<gq, 256>>>(Qh, q8, qs, H, g->nseq, g->S, Sp, Tp);
+    a8_rq_k<<<gq, 256>>>(Kh, k8, ks, H, g->nseq, g->S, Sp, Tp);
+    a8_tq_k<<<(unsigned)(H * (R / 32)), 64>>>(Vh, vt, vts, H, g->nseq, g->S, Sp, Tp);
+    const dim3 grid((unsigned)((g->S + 127) / 128), (unsigned)H, (unsigned)g->nseq);
+    a8_fwd_k<<<grid, 256>>>(q8, qs, k8, ks, vt, vts, o, lse, g->S, Sp, H, C, R, 1.4426950408889634f / sqrtf((float)HD));
+    MICK();
+    return 0;
+}

@@ -228,6 +228,6 @@ void mi_post_error(hipError_t e, const char *file, int line);
 #define MICK() do { hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)
 #define MIRT(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)
 void *mi_ws(int slot, size_t bytes);        // per-device grow-on-demand scratch (the reference's nn_ws, src/nn_core.cu:751)
-enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_UPCOARSE = 5, MI_WS_NSLOTS = 8 };
+enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_UPCOARSE = 5, MI_WS_GEMM = 6, MI_WS_ATTN = 7, MI_WS_NSLOTS = 8 };
 static inline unsigned nblk_(size_t n, unsigned b) { return (unsigned)((n + b - 1) / b); }
 [[noreturn]] void mi_die(const char *fmt, ...);

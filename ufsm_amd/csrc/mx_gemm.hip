@@ -1,0 +1,139 @@
+// MX GEMM of row-major fp32 operands (the attention stage's linear layers): both operands are quantised along K once, into block rows
+// that are MFMA fragments as they lie in memory, then a block-scaled MFMA GEMM runs over the packed bytes.
+// Interface and arithmetic: src/lp_mxgemm.cu:1-5 (definition), :88-113 (packing), :266-297 (entry points) of the reference.
+#include "mx_dev.hpp"
+#include "../../include/mi_attn.h"
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// one thread per (row, 32-K block): X is [rows][K] (TR 0; ld = row stride) or [K][rows] (TR 1). Packed row r = nkb blocks of BPB bytes
+// (K past the operand's K is zero), scales [rows][nkb]. TR: neighbouring threads take neighbouring rows (contiguous reads of each K row).
+template <int BITS, int TR>
+__global__ void __launch_bounds__(256) mx_pack_k(const float *__restrict__ X, int ld, int rows, int K, int nkb, uint8_t *__restrict__ q, uint8_t *__restrict__ sc) {
+    constexpr int BPB = BITS == 8 ? 32 : 16;
+    const long long nblk = (long long)rows * nkb;
+    for (long long b = blockIdx.x * (long long)blockDim.x + threadIdx.x; b < nblk; b += (long long)gridDim.x * blockDim.x) {
+        const int r = TR ? (int)(b % rows) : (int)(b / nkb), kb = TR ? (int)(b / rows) : (int)(b % nkb);
+        float v[32];
+#pragma unroll
+        for (int j = 0; j < 32; j++) { const int k = kb * 32 + j; v[j] = k < K ? (TR ? X[(size_t)k * ld + r] : X[(size_t)r * ld + k]) : 0.f; }
+        unsigned codes[8];
+        const unsigned sb = d_quant_row<BITS, false>(v, 32, codes);
+        uint8_t *o = q + ((size_t)r * nkb + kb) * BPB;
+        *(uint4 *)o = make_uint4(codes[0], codes[1], codes[2], codes[3]);
+        if (BITS == 8) *(uint4 *)(o + 16) = make_uint4(codes[4], codes[5], codes[6], codes[7]);
+        sc[(size_t)r * nkb + kb] = (uint8_t)sb;
+    }
+}
+
+__global__ void gemm_zero_k(float *c, size_t n) {
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) c[i] = 0.f;
+}
+
+// C tile of 128 x 128 per workgroup, 64 x 64 per wavefront = 2 x 2 MFMA tiles of 32 x 32; K in steps of 64 = the two 32-K blocks the
+// scale operands of the lane halves of a 32x32x64 MFMA cover. A lane's fragment is 16 bytes of each of the two blocks (e4m3: bytes
+// 16 h ... of both; e2m1: all 16 bytes of block h), so fragments are loaded from the packed rows in global memory directly: the four
+// wavefronts of a workgroup re-read each other's rows through the vector cache.
+// gridDim.z > 1: split K, each split adds its part into C atomically (C zeroed or kept by the host; no bias / residual then).
+template <int BITS>
+__global__ void __launch_bounds__(256) mx_gemm_k(const uint8_t *__restrict__ Aq, const uint8_t *__restrict__ As, const uint8_t *__restrict__ Bq, const uint8_t *__restrict__ Bs,
+                                                 float *C, int M, int N, int nkb, float beta, const float *__restrict__ bias, const float *res, int sper) {
+    constexpr int BPB = BITS == 8 ? 32 : 16, FM = BITS == 8 ? 0 : 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    const int m0 = blockIdx.y * 128 + (wave >> 1) * 64, n0 = blockIdx.x * 128 + (wave & 1) * 64;
+    if (m0 >= M || n0 >= N) return;                        // (no barriers in this kernel: a wavefront without work leaves)
+    const int nst = nkb >> 1, s0 = (int)blockIdx.z * sper, s1 = min(nst, s0 + sper);
+    const uint8_t *pa[2], *pb[2], *sa[2], *sb[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const size_t ra = (size_t)min(m0 + 32 * i + r, M - 1), rb = (size_t)min(n0 + 32 * i + r, N - 1);       // rows past the edge repeat the last one (never stored)
+        pa[i] = Aq + ra * nkb * BPB + 16 * h; sa[i] = As + ra * nkb + h;         // (e2m1: + 16 h is block h of a step; e4m3: the lane's half of both blocks)
+        pb[i] = Bq + rb * nkb * BPB + 16 * h; sb[i] = Bs + rb * nkb + h;
+    }
+    v16f acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) acc[i][j][q] = 0.f;
+    auto frag = [&](const uint8_t *p) {
+        const v4i lo = *(const v4i *)p;
+        if (BITS == 8) { const v4i hi = *(const v4i *)(p + 32); return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; }
+        return (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+    };
+    for (int s = s0; s < s1; s++) {
+        v8i fa[2], fb[2]; int ea[2], eb[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            fa[i] = frag(pa[i] + (size_t)s * 2 * BPB); ea[i] = sa[i][2 * s];
+            fb[i] = frag(pb[i] + (size_t)s * 2 * BPB); eb[i] = sb[i][2 * s];
+        }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FM, FM, 0, ea[i], 0, eb[j]);
+    }
+    // accumulator element q of lane (r, h): row (q & 3) + 4 h + 8 (q >> 2), column r of its 32 x 32 tile
+    const bool split = gridDim.z > 1;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int col = n0 + 32 * j + r;
+            if (col >= N) continue;
+            const float bv = bias ? bias[col] : 0.f;
+#pragma unroll
+            for (int q = 0; q < 16; q++) {
+                const int row = m0 + 32 * i + (q & 3) + 4 * h + 8 * (q >> 2);
+                if (row >= M) continue;
+                float *p = C + (size_t)row * N + col;
+                if (split) { atomicAdd(p, acc[i][j][q]); continue; }
+                float v = acc[i][j][q] + bv;
+                if (res) v += res[(size_t)row * N + col];
+                if (beta != 0.f) v += beta * *p;
+                *p = v;
+            }
+        }
+}
+
+extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res) {
+    if (bits != 4 && bits != 8) return -1;
+    if (M <= 0 || N <= 0) return 0;
+    if (K < 0) K = 0;
+    const int nkb = (K + 63) / 64 * 2, BPB = bits == 8 ? 32 : 16;         // 32-K blocks of the packed rows (K rounded up to 64)
+    const size_t qa = (size_t)M * nkb * BPB, qb = (size_t)N * nkb * BPB, sa = (size_t)M * nkb, sb = (size_t)N * nkb;
+    auto al = [](size_t n) { return (n + 255) & ~(size_t)255; };
+    uint8_t *base = (uint8_t *)mi_ws(MI_WS_GEMM, al(qa) + al(qb) + al(sa) + al(sb) + 256);
+    if (!base) return -1;
+    uint8_t *Aq = base, *Bq = Aq + al(qa), *As = Bq + al(qb), *Bs = As + al(sa);
+    const int lda = ta ? M : K, ldb = tb ? K : N;
+    if (nkb) {
+        const unsigned ga = nblk_((size_t)M * nkb, 256), gb = nblk_((size_t)N * nkb, 256);
+        if (bits == 8) {
+            if (ta) mx_pack_k<8, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<8, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
+            if (tb) mx_pack_k<8, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<8, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
+        } else {
+            if (ta) mx_pack_k<4, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<4, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
+            if (tb) mx_pack_k<4, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<4, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
+        }
+    }
+    // few output tiles and a long K (the weight-gradient shape, src/lp_mxgemm.cu:259-265): split K so the GPU's 256 CUs have work
+    const int tiles = ((N + 127) / 128) * ((M + 127) / 128), nst = nkb / 2;
+    int ns = !bias && !res && (beta == 0.f || beta == 1.f) && tiles < 128 ? (256 + tiles - 1) / tiles : 1;
+    if (ns > nst / 4) ns = nst / 4 > 1 ? nst / 4 : 1;
+    const int sper = ns > 1 ? (nst + ns - 1) / ns : (nst > 0 ? nst : 1);
+    ns = nst > 0 ? (nst + sper - 1) / sper : 1;
+    if (ns > 1 && beta == 0.f) gemm_zero_k<<<nblk_((size_t)M * N, 256 * 4), 256>>>(C, (size_t)M * N);   // (a kernel, not a memset node: safe under graph capture)
+    const dim3 grid((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128), (unsigned)ns);
+    if (bits == 8) mx_gemm_k<8><<<grid, 256>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
+    else mx_gemm_k<4><<<grid, 256>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
+    MICK();
+    return 0;
+}
+extern "C" int lp_mx_gemm(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta) {
+    return lp_mx_gemm_ex(bits, ta, tb, M, N, K, A, B, C, beta, nullptr, nullptr);
+}

@@ -84,6 +84,20 @@ _PROTOS = {
     "mi_last_kernel": (C.c_char_p, []),
 }
 EXPORTS = tuple(_PROTOS)
+
+
+class at_geom(C.Structure):  # src/attn.h:81
+    _fields_ = [("nseq", C.c_int), ("S", C.c_int), ("D", C.c_int), ("Hh", C.c_int), ("W", C.c_int),
+                ("lens", C.c_void_p), ("pos", C.c_void_p), ("rays", C.c_void_p), ("dfx", C.c_void_p * 3), ("dfr", C.c_void_p)]
+
+
+# include/mi_attn.h
+_ATTN_PROTOS = {
+    "lp_mx_gemm": (_I, [_I, _I, _I, _I, _I, _I, _P, _P, _P, _F]),
+    "lp_mx_gemm_ex": (_I, [_I, _I, _I, _I, _I, _I, _P, _P, _P, _F, _P, _P]),
+    "at_fa8_fwd": (_I, [_P, _P, _P, C.POINTER(at_geom), _I, _I]),
+}
+ATTN_EXPORTS = tuple(_ATTN_PROTOS)
 _lib = None
 
 
@@ -95,7 +109,7 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise RuntimeError("%s is not built: run `python -c 'import __graft_entry__ as g; g.build()'` (hipcc, gfx950)" % LIB_PATH)
     L = C.CDLL(LIB_PATH)
-    for name, (res, args) in _PROTOS.items():
+    for name, (res, args) in list(_PROTOS.items()) + list(_ATTN_PROTOS.items()):
         f = getattr(L, name)  # AttributeError names the missing symbol
         f.restype = res
         f.argtypes = args
