@@ -54,6 +54,18 @@ int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const flo
 const void *unet_layer_out(const unet *u, int k, shape5 *s, const char **name);
 /* the GroupNorm statistics the k-th conv produced (device [n * G] each); returns G, 0 when the layer has none */
 int unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd);
+shape5 unet_in_shape(const unet *u);                          /* the window the graph was created for */
+const unet_cfg *unet_config(const unet *u);
+/* ---- sliding-window prediction of a volume resident in device memory (src/predict.c: the --feather single pass, :282-333, :2538-2545,
+   :3420-3436). vol: uint8 CT [dims0][dims1][dims2]; windows of the graph's size (one cubic sample) with `halo` voxels of context per side
+   tile the volume at stride window - 2 halo in z-y-x order; each runs unet_forward_ct (z-score mean / isd; axis, cy, cx: the scroll axis
+   sign and its centre in volume y / x, axis 0: no direction channels) and places uint8(255 sigmoid(logit 0) + .5) where CT >= the
+   prediction iso over its interior plus `feather` voxels of its upper halo; the window borders are then blended over `feather` voxels
+   (0: none; <= halo) into out: uint8 [dims0][dims1][dims2]. Windows whose CT holds no voxel >= iso are skipped (their interior stays 0
+   and their neighbours' blends renormalise). nwin[0..1] (may be null): windows in all, windows computed. Returns 0, or -1 for a
+   geometry the graph cannot run. Every window's prediction stays in device memory until the blend: nwin (stride + feather)^3 bytes. */
+int unet_predict_volume(unet *u, const uint8_t *vol, const int64_t dims[3], int halo, int feather, float mean, float isd,
+                        int axis, float cy, float cx, uint8_t *out, int64_t nwin[2]);
 #ifdef __cplusplus
 }
 #endif

@@ -650,3 +650,47 @@ void orc_fa8_fwd(const uint16_t *qkvh, float *o, float *lse, int nseq, int S, in
         free(qd); free(kd); free(vd);
     }
 }
+
+/* ---------- sliding-window prediction: placement and feather blend ---------- */
+/* src/nn_elem.cu:1105-1125 (place_isect, pred_place_k): the window voxels inside both the window's interior ([hz, D - hz) x [halo, W - halo)^2)
+   and the target box ([-o, e - o)) become uint8 probabilities at target index ((o_z + z) shard + o_y + y) shard + o_x + x; CT below iso -> 0 */
+void orc_pred_place(const float *lg, const uint8_t *ct, int D, int W, int hz, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, int iso, uint8_t *dsh) {
+    const int z0 = hz > -oz ? hz : -oz, y0 = halo > -oy ? halo : -oy, x0 = halo > -ox ? halo : -ox;
+    const int z1 = D - hz < ez - oz ? D - hz : ez - oz, y1 = W - halo < ey - oy ? W - halo : ey - oy, x1 = W - halo < ex - ox ? W - halo : ex - ox;
+    for (int z = z0; z < z1; z++) for (int y = y0; y < y1; y++) for (int x = x0; x < x1; x++) {
+        const size_t k = ((size_t)z * W + y) * W + x;
+        dsh[((size_t)(oz + z) * shard + (oy + y)) * shard + (ox + x)] = ct[k] >= iso ? (uint8_t)(255.f / (1.f + expf(-lg[k])) + 0.5f) : 0;
+    }
+}
+/* src/predict.c:282-333 (feather_t, fe_val, fe_blend, fe_rows), :334-375 (which earlier windows are held): windows of interior S on a grid
+   nss[3] in z-y-x order, each with its prediction E over [0, S + B)^3 from its interior origin (E: [window][S + B]^3 bytes; present: which
+   windows were computed). The output over a window's interior is its own E except in the lower shell (a coordinate < B), where the
+   windows shifted back by delta in {0,1}^3 that are present are blended with weights prod_d (delta_d ? 1 - u(v_d) : u(v_d)),
+   u(j) = sin^2(pi/2 (j + .5) / B), normalised; bn: the output box, clipped inside the window grid. */
+void orc_feather_blend(const uint8_t *E, const uint8_t *present, int S, int B, const int64_t nss[3], const int64_t bn[3], uint8_t *out) {
+    const int En = S + B; const size_t e3 = (size_t)En * En * En;
+    float u[2][1024];
+    for (int j = 0; j < B; j++) { const double s = sin(M_PI / 2 * (j + 0.5) / B); u[0][j] = (float)(s * s); u[1][j] = (float)(1 - s * s); }
+#pragma omp parallel for schedule(static)
+    for (int64_t gz = 0; gz < bn[0]; gz++) for (int64_t gy = 0; gy < bn[1]; gy++) for (int64_t gx = 0; gx < bn[2]; gx++) {
+        const int64_t a = gz / S, b = gy / S, c = gx / S; const int z = (int)(gz - a * S), y = (int)(gy - b * S), x = (int)(gx - c * S);
+        const int64_t id = (a * nss[1] + b) * nss[2] + c;
+        uint8_t *o = out + ((size_t)gz * bn[1] + gy) * bn[2] + gx;
+        if (!present[id]) { *o = 0; continue; }
+        const uint8_t *e = E + (size_t)id * e3;
+        if (z >= B && y >= B && x >= B) { *o = e[((size_t)z * En + y) * En + x]; continue; }
+        float s = 0, w = 0;
+        for (int d = 0; d < 8; d++) {
+            const int dz = d >> 2 & 1, dy = d >> 1 & 1, dx = d & 1;
+            const int64_t qa = a - dz, qb = b - dy, qc = c - dx;
+            if (qa < 0 || qb < 0 || qc < 0) continue;
+            const int64_t qid = (qa * nss[1] + qb) * nss[2] + qc;
+            if (d && !present[qid]) continue;
+            if ((dz && z >= B) || (dy && y >= B) || (dx && x >= B)) continue;
+            const float wi = (z < B ? u[dz][z] : 1.f) * (y < B ? u[dy][y] : 1.f) * (x < B ? u[dx][x] : 1.f);
+            const uint8_t v = E[(size_t)qid * e3 + ((size_t)(z + dz * S) * En + (y + dy * S)) * En + (x + dx * S)];
+            s += wi * v; w += wi;
+        }
+        *o = w > 0 ? (uint8_t)fminf(255.f, s / w + 0.5f) : 0;
+    }
+}

@@ -20,6 +20,10 @@
  *                                 that key's quantised V row, also when the maximum moves between key tiles; keys past S never
  *                                 contribute) and the reference's own gate, rel. L2 < 0.1 against exact fp64 attention
  *                                 (tests/test_attn.c:445-446)
+ *   orc_pred_place                pinned: box intersection by brute force over all voxels; 255 sigmoid rounded to nearest in fp64
+ *   orc_feather_blend             pinned: the reference's own checks (tests/test_predict_feather.c:95-121): core and first-window voxels
+ *                                 equal the window's own prediction, a z-shell voxel is u(j) own + (1 - u(j)) lower within 1; constant
+ *                                 fields are fixed points; an absent neighbour renormalises
  *   SiLU in GN staging            PARITY UNPINNED to the bit: the reference evaluates tanh with NVIDIA's
  *                                 tanh.approx.f32 (src/lp_common.cuh:469-473), not reproducible off that hardware;
  *                                 checked to floor/ceil code neighbours as tests/test_mx4_wide.c:165-175 does
@@ -108,6 +112,10 @@ void orc_conv1_mx(int xbits, const uint8_t *x, int N, int Ci, size_t S, const fl
 int orc_mx_gemm(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res);
 /* MX-fp8 attention forward on the fp16 head-major pack (src/lp_attn8.cu:124-180, :319-328); head dim 48 */
 void orc_fa8_fwd(const uint16_t *qkvh, float *o, float *lse, int nseq, int S, int H, int C);
+/* sliding-window prediction: sigmoid -> uint8 placement (src/nn_elem.cu:1105-1125) and the one-sided sin^2 feather blend of window borders
+   (src/predict.c:282-333) */
+void orc_pred_place(const float *lg, const uint8_t *ct, int D, int W, int hz, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, int iso, uint8_t *dsh);
+void orc_feather_blend(const uint8_t *E, const uint8_t *present, int S, int B, const int64_t nss[3], const int64_t bn[3], uint8_t *out);
 float orc_act_ab(float v, float a, float b);
 uint16_t orc_f32_to_h16(float f);
 float orc_h16_to_f32(uint16_t h);

@@ -62,6 +62,8 @@ def lib():
         L.orc_threads.restype = C.c_int
         L.orc_mx_gemm.restype = C.c_int
         L.orc_mx_gemm.argtypes = [C.c_int] * 6 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p]
+        L.orc_pred_place.restype = None; L.orc_pred_place.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 12 + [C.c_void_p]
+        L.orc_feather_blend.restype = None; L.orc_feather_blend.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.orc_fa8_fwd.restype = None; L.orc_fa8_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
         _lib = L
     return _lib
@@ -138,3 +140,18 @@ def fa8_fwd(qkvh, nseq, S, H):
     o = np.zeros((nseq * S, H * 48), np.float32); lse = np.zeros((nseq, H, S), np.float32)
     lib().orc_fa8_fwd(ptr(qkvh), ptr(o), ptr(lse), nseq, S, H, H * 48)
     return o, lse
+
+
+def pred_place(lg, ct, D, W, hz, halo, o, e, shard, iso=1, dsh=None):
+    lg = np.ascontiguousarray(lg, np.float32); ct = np.ascontiguousarray(ct, np.uint8)
+    out = np.zeros((shard, shard, shard), np.uint8) if dsh is None else dsh
+    lib().orc_pred_place(ptr(lg), ptr(ct), D, W, hz, halo, o[0], o[1], o[2], e[0], e[1], e[2], shard, iso, ptr(out))
+    return out
+
+
+def feather_blend(E, present, S, B, nss, bn):
+    E = np.ascontiguousarray(E, np.uint8); present = np.ascontiguousarray(present, np.uint8)
+    nss_a = np.asarray(nss, np.int64); bn_a = np.asarray(bn, np.int64)
+    out = np.zeros(tuple(int(v) for v in bn), np.uint8)
+    lib().orc_feather_blend(ptr(E), ptr(present), S, B, ptr(nss_a), ptr(bn_a), ptr(out))
+    return out

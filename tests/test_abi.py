@@ -43,11 +43,20 @@ def test_library_exports_the_attention_header():
     assert C.sizeof(lp.at_geom) == 24 + 7 * 8 and lp.at_geom.lens.offset == 24 and lp.at_geom.dfr.offset == 72
 
 
+def test_library_exports_the_prediction_header():
+    from ufsm_amd import lp
+    L = lp.load()
+    names = header_functions("mi_predict.h", ("nn_", "mi_"))
+    assert set(names) == set(lp.PRED_EXPORTS) and "nn_pred_place" in names and "mi_feather_blend" in names
+    for n in names:
+        assert hasattr(L, n), "libufsm_lp.so does not export %s" % n
+
+
 def test_host_library_exports_every_declared_symbol():
     from ufsm_amd import unet
     H = unet.load_host()
     names = header_functions("mi_unet.h", ("nn_", "unet_"))
-    assert "unet_forward_x" in names and "nn_conv3d_fwd_x" in names and "nn_set_storage" in names
+    assert "unet_forward_x" in names and "nn_conv3d_fwd_x" in names and "nn_set_storage" in names and "unet_predict_volume" in names
     for n in names:
         assert hasattr(H, n), "libufsm_host.so does not export %s" % n
     assert C.sizeof(unet.unet_cfg) == 4 * (2 + unet.UNET_MAXLEV + 4)

@@ -8,7 +8,7 @@ CSRC = os.path.join(ROOT, "ufsm_amd", "csrc")
 LIB = os.path.join(ROOT, "ufsm_amd", "libufsm_lp.so")
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
-HIP_SOURCES = ["rt.hip", "mx_elem.hip", "mx_gemm.hip", "attn8.hip", "conv3.hip"] + ["conv3_f%d_o%d.hip" % (f, o) for f in (8, 4) for o in (8, 4, 0)]
+HIP_SOURCES = ["rt.hip", "mx_elem.hip", "mx_gemm.hip", "attn8.hip", "predict.hip", "conv3.hip"] + ["conv3_f%d_o%d.hip" % (f, o) for f in (8, 4) for o in (8, 4, 0)]
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wno-unused-value",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
@@ -45,7 +45,7 @@ HOST_LIB = os.path.join(ROOT, "ufsm_amd", "libufsm_host.so")
 
 def build_host():
     """The C23 host layer (op dispatch + U-Net graph) over the C ABI of libufsm_lp.so."""
-    src = [os.path.join(ROOT, "ufsm_amd", "host", f) for f in ("nn_host.c", "unet.c")]
+    src = [os.path.join(ROOT, "ufsm_amd", "host", f) for f in ("nn_host.c", "unet.c", "predict.c")]
     _run(["gcc", "-std=c2x", "-O2", "-Wall", "-Wextra", "-fPIC", "-shared", "-o", HOST_LIB] + src +
          ["-L" + os.path.dirname(LIB), "-lufsm_lp", "-Wl,-rpath,$ORIGIN", "-lm"])
     return HOST_LIB

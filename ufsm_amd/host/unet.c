@@ -167,6 +167,8 @@ int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const flo
     lp_pred_input_mx(ct, u->in.w, mean, isd, dyo, dxo, axis, 0, u->in.d, u->xin, 2, u->cfg.act_dt == 4 ? 4 : 8);      /* fp16-rounded input values, as predict */
     return unet_forward_x(u, u->xin, logits);
 }
+shape5 unet_in_shape(const unet *u) { return u->in; }
+const unet_cfg *unet_config(const unet *u) { return &u->cfg; }
 int unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd) {
     if (k < 0 || k >= u->nouts) return 0;
     *mean = u->outs[k].mean; *rstd = u->outs[k].rstd;

@@ -98,6 +98,16 @@ _ATTN_PROTOS = {
     "at_fa8_fwd": (_I, [_P, _P, _P, C.POINTER(at_geom), _I, _I]),
 }
 ATTN_EXPORTS = tuple(_ATTN_PROTOS)
+# include/mi_predict.h
+_PRED_PROTOS = {
+    "nn_set_pred_iso": (None, [_I]),
+    "nn_get_pred_iso": (_I, []),
+    "nn_pred_place_d": (None, [_P, _P] + [_I] * 11 + [_P]),
+    "nn_pred_place": (None, [_P, _P] + [_I] * 9 + [_P]),
+    "mi_ct_window": (None, [_P] + [C.c_int64] * 6 + [_I, _P, _I, _I, _P]),
+    "mi_feather_blend": (_I, [_P, _P, _I, _I, C.POINTER(C.c_int64), C.POINTER(C.c_int64), _P]),
+}
+PRED_EXPORTS = tuple(_PRED_PROTOS)
 _lib = None
 
 
@@ -109,7 +119,7 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise RuntimeError("%s is not built: run `python -c 'import __graft_entry__ as g; g.build()'` (hipcc, gfx950)" % LIB_PATH)
     L = C.CDLL(LIB_PATH)
-    for name, (res, args) in list(_PROTOS.items()) + list(_ATTN_PROTOS.items()):
+    for name, (res, args) in list(_PROTOS.items()) + list(_ATTN_PROTOS.items()) + list(_PRED_PROTOS.items()):
         f = getattr(L, name)  # AttributeError names the missing symbol
         f.restype = res
         f.argtypes = args

@@ -43,6 +43,11 @@ def load_host():
     L.nn_set_prec.restype = None; L.nn_set_prec.argtypes = [C.c_int]
     L.nn_set_gn_stored.restype = None; L.nn_set_gn_stored.argtypes = [C.c_int]
     L.nn_check.restype = C.c_char_p
+    L.unet_in_shape.restype = shape5; L.unet_in_shape.argtypes = [C.c_void_p]
+    L.unet_config.restype = C.POINTER(unet_cfg); L.unet_config.argtypes = [C.c_void_p]
+    L.unet_predict_volume.restype = C.c_int
+    L.unet_predict_volume.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int, C.c_int, C.c_float, C.c_float, C.c_int, C.c_float, C.c_float,
+                                      C.c_void_p, C.POINTER(C.c_int64)]
     _host = L
     return L
 
@@ -79,6 +84,15 @@ class UNet:
 
     def forward_x(self, x_ptr, logits_ptr):
         return self.L.unet_forward_x(self.h, x_ptr, logits_ptr)
+
+    def forward_ct(self, ct_ptr, mean, isd, dyo_ptr, dxo_ptr, axis, logits_ptr):
+        return self.L.unet_forward_ct(self.h, ct_ptr, mean, isd, dyo_ptr, dxo_ptr, axis, logits_ptr)
+
+    def predict_volume(self, vol_ptr, dims, halo, feather, mean, isd, axis, cy, cx, out_ptr):
+        """Sliding-window prediction of a device uint8 volume; returns (rc, windows, windows computed)."""
+        d = (C.c_int64 * 3)(*dims); nw = (C.c_int64 * 2)(0, 0)
+        rc = self.L.unet_predict_volume(self.h, vol_ptr, d, halo, feather, mean, isd, axis, cy, cx, out_ptr, nw)
+        return rc, nw[0], nw[1]
 
     def layer_outs(self):
         out, k = [], 0
