@@ -108,7 +108,7 @@ def main():
                     "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path shards by windows / z-slabs, see DESIGN.md)" % a.gpus, file=sys.stderr)
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path would shard by whole windows, or by z-slabs of one window with a one-plane halo exchange per layer)" % a.gpus, file=sys.stderr)
         sys.exit(2)
     import numpy as np
     from ufsm_amd import lib, LP, shape5, gnp_t, split_t, DevBuf
