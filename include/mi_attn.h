@@ -38,6 +38,49 @@ int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, const float *A,
    softmax denominator plus the maximum logit in base-2 units. C must equal 48 H. Returns 0, or -1 when scratch cannot be allocated. */
 int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom *g, int H, int C);
 
+/* ---- the attention block around those two (forward, self-attention path; src/attn.h:26-81, src/nn_attn.cu) ---- */
+#define AT_DFM_NLV (AT_DFM_MAXL + 1)
+/* channels (H x 48), heads, SwiGLU hidden width, RoPE (0 none, 1 axial on the grid index), register tokens; the deformable fields must be 0
+   (src/attn.h:33) */
+typedef struct { int C, H, F, rope, nreg; float rope_base; int dK, dL, dC[AT_DFM_MAXL]; int dCo, dInit; } at_dims;
+/* one block's parameters: offsets into the flat parameter array, weights [out][in] row major (src/attn.h:39, src/nn_attn.cu:460-480) */
+typedef struct { size_t ln1g, ln1b, wqkv, bqkv, qg, kg, wo, bo, ln2g, ln2b, w1, b1, w2, b2, woa, boa, wvl[AT_DFM_MAXL], bvl[AT_DFM_MAXL]; } at_bp;
+size_t at_block_nparams(const at_dims *d);
+size_t at_block_layout(const at_dims *d, at_bp *bp, size_t off);   /* assigns offsets from off, returns the end */
+/* scratch of one block over T tokens, field for field the reference's (src/attn.h:47-60); this build carves and uses the forward tensors
+   xn, qkv, o, x1, xn2, h, gg, m1, r1, m2, r2, rq, rk, lse, qkvh, amx and leaves the others null */
+typedef struct {
+    float *xn, *qkv, *qkn, *o, *x1, *xn2, *h, *gg, *m1, *r1, *m2, *r2, *rq, *rk, *lse, *dv;
+    float *bA, *bB, *bC, *dx1;
+    float *qkvh, *doh, *amx;
+    float *qkvr, *orr, *dor, *dqr, *dqr2;
+    float *vl[AT_DFM_NLV], *oa, *aw, *dvl[AT_DFM_NLV], *doa;
+    int kept;
+    int vr; float *v1, *own, *dv1; const float *lam; float *glam;
+} at_ws;
+size_t at_ws_bytes(const at_dims *d, long T);                       /* replaces src/nn_attn.cu:529 (forward tensors only here) */
+void at_ws_carve(at_ws *w, const at_dims *d, long T, void *base);   /* replaces src/nn_attn.cu:530 */
+/* the linear layers' precision (src/attn.h:194-195, src/nn_attn.cu:97-135): 4 / 8 = lp_mx_gemm_ex; this build has no fp32 GEMM, 0 is refused */
+void at_set_mx(int bits);
+int at_get_mx(void);
+int at_gemm_ex(int ta, int tb, int M, int N, int K, const float *A, const float *B, float *Cm, float beta, const float *bias, const float *res);
+/* replaces at_ln_fwd (src/attn.h:241, src/nn_attn.cu:150-168): LayerNorm over C per row, eps 1e-5, affine g / b; mean / rstd [T] */
+void at_ln_fwd(const float *x, const float *g, const float *b, float *y, float *mean, float *rstd, long T, int C);
+/* replaces at_glu_fwd (src/attn.h:248, src/nn_attn.cu:438-455): h [T][2F] = [a | b] -> gg [T][F] = silu(a) b */
+void at_glu_fwd(const float *h, float *gg, long T, int F);
+/* replaces at_fa_pack (src/attn.h:203, src/nn_attn_tc.cu:99-136, :371-378): qkv fp32 [T][3C] -> fp16 head-major q, k, v [3][H][T + 64][48];
+   q and k RMS-normalised over the head dims (eps 1e-6) times the gains qg / kg [H][48], then axial rotary pairs on grid tokens (rope 1;
+   g->pos must be null); rq / rk [T][H] the normalisers, amx[1] = max |v| (amx: 4 floats, zeroed here); rows past T zero */
+void at_fa_pack(const float *qkv, const float *qg, const float *kg, void *qkvh, float *rq, float *rk, float *amx, const at_geom *g, int nreg, int C, int rope, float base);
+/* replace at_cs_to_tok / at_tok_to_cs (src/nn_attn.cu:748-759, :802-803): channel-major planes [n][C][Sg] <-> token rows [n][nreg + Sg][C]
+   with the learned register rows reg [nreg][C] prepended (dropped on the way back) */
+void at_cs_to_tok(const float *x, float *t, const float *reg, int n, int C, long Sg, int nreg);
+void at_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg);
+/* replaces at_block_fwd (src/attn.h:..., src/nn_attn.cu:587-633) for self-attention blocks on the MX-fp8 core with MX linears:
+   y = x1 + W2 swiglu(W1 LN2(x1)), x1 = x + Wo attention(pack(Wqkv LN1(x))). P: the parameter array, bp: the block's offsets; x, y fp32
+   [T][C] (T = g->nseq g->S); 0, or -1 for a configuration this build does not run (deformable, rays, value residual, fp32 linears) */
+int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, const float *x, float *y, const at_geom *g, at_ws *w);
+
 #ifdef __cplusplus
 }
 #endif

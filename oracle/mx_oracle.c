@@ -694,3 +694,90 @@ void orc_feather_blend(const uint8_t *E, const uint8_t *present, int S, int B, c
         *o = w > 0 ? (uint8_t)fminf(255.f, s / w + 0.5f) : 0;
     }
 }
+
+/* ---------- attention block around the MX GEMM and the fp8 attention core (src/nn_attn.cu:150-167 LayerNorm, :438-446 SwiGLU, :748-759 token
+   layout, :587-633 block forward; src/nn_attn_tc.cu:99-136 QK-norm + gains + RoPE pack) ---------- */
+void orc_ln_fwd(const float *x, const float *g, const float *b, float *y, float *mean, float *rstd, long T, int C) {
+#pragma omp parallel for schedule(static)
+    for (long r = 0; r < T; r++) {
+        const float *xr = x + (size_t)r * C; double s = 0, q = 0;
+        for (int c = 0; c < C; c++) s += xr[c];
+        const float m = (float)(s / C);
+        for (int c = 0; c < C; c++) { const double d = (double)xr[c] - m; q += d * d; }
+        const float rs = 1.f / sqrtf((float)(q / C) + 1e-5f);
+        for (int c = 0; c < C; c++) y[(size_t)r * C + c] = (xr[c] - m) * rs * g[c] + b[c];
+        if (mean) mean[r] = m;
+        if (rstd) rstd[r] = rs;
+    }
+}
+void orc_glu_fwd(const float *h, float *gg, long T, int F) {
+    for (long t = 0; t < T; t++) for (int f = 0; f < F; f++) { const float a = h[(size_t)t * 2 * F + f], b = h[(size_t)t * 2 * F + F + f]; gg[(size_t)t * F + f] = a / (1.f + expf(-a)) * b; }
+}
+void orc_cs_to_tok(const float *x, float *t, const float *reg, int n, int C, long Sg, int nreg) {
+    const long S = Sg + nreg;
+    for (long r = 0; r < (long)n * S; r++) for (int c = 0; c < C; c++) {
+        const long s = r / S, ts = r % S - nreg;
+        t[(size_t)r * C + c] = ts < 0 ? reg[(size_t)(r % S) * C + c] : x[((size_t)s * C + c) * Sg + ts];
+    }
+}
+void orc_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg) {
+    for (long s = 0; s < n; s++) for (int c = 0; c < C; c++) for (long ts = 0; ts < Sg; ts++) x[((size_t)s * C + c) * Sg + ts] = t[((size_t)s * (Sg + nreg) + nreg + ts) * C + c];
+}
+/* qkv fp32 [T][3C] -> fp16 head-major q, k, v [3][H][T + 64][48]: q and k rows RMS-normalised over the 48 head dims (eps 1e-6) times the gains,
+   then (rope 1, grid tokens only) axial rotary pairs: 16 dims per axis z, y, x, 8 frequencies base^(-f / 8); rq / rk the normalisers,
+   amx[1] = max |v| (amx[0], [2], [3] zero); the 64 rows past T are zero */
+void orc_fa_pack(const float *qkv, const float *qg, const float *kg, uint16_t *qkvh, float *rq, float *rk, float *amx, int nseq, int S, int Hh, int W, int nreg, int C, int rope, float base) {
+    enum { HD = 48, FT = 64 };
+    const int H = C / HD; const long T = (long)nseq * S, Tp = T + FT; const float lbase = log2f(base);
+    float vmax = 0.f;
+    for (int p = 0; p < 3; p++) for (int h = 0; h < H; h++) for (long t = 0; t < Tp; t++) {
+        uint16_t *dst = qkvh + ((size_t)p * H * Tp + (size_t)h * Tp + t) * HD;
+        if (t >= T) { for (int d = 0; d < HD; d++) dst[d] = 0; continue; }
+        float v[HD];
+        for (int d = 0; d < HD; d++) v[d] = qkv[(size_t)t * 3 * C + (size_t)p * C + h * HD + d];
+        if (p < 2) {
+            float s = 0.f; for (int d = 0; d < HD; d++) s += v[d] * v[d];
+            const float r = 1.f / sqrtf(s / HD + 1e-6f); const float *gs = (p ? kg : qg) + h * HD;
+            for (int d = 0; d < HD; d++) v[d] *= r * gs[d];
+            (p ? rk : rq)[t * H + h] = r;
+            const int ts = (int)(t % S) - nreg;
+            if (rope && ts >= 0) {
+                const float pos[3] = {(float)(ts / (Hh * W)), (float)((ts / W) % Hh), (float)(ts % W)};
+                for (int pr = 0; pr < 24; pr++) {
+                    const int ax = pr / 8, fi = pr % 8; const float ang = pos[ax] * exp2f(-lbase * (float)fi / 8.f), sn = sinf(ang), cs = cosf(ang);
+                    const float a = v[ax * 16 + 2 * fi], b = v[ax * 16 + 2 * fi + 1];
+                    v[ax * 16 + 2 * fi] = a * cs - b * sn; v[ax * 16 + 2 * fi + 1] = a * sn + b * cs;
+                }
+            }
+        } else for (int d = 0; d < HD; d++) vmax = fmaxf(vmax, fabsf(v[d]));
+        for (int d = 0; d < HD; d++) dst[d] = orc_f32_to_h16(v[d]);
+    }
+    if (amx) { amx[0] = 0.f; amx[1] = vmax; amx[2] = 0.f; amx[3] = 0.f; }
+}
+/* the self-attention block (pre-LN, MHSA with QK-norm, SwiGLU) with MX linears of `bits` and the fp8 attention core; P: the block's
+   parameters at the offsets of orc_block_layout; x, y fp32 [T][C] */
+size_t orc_block_layout(int C, int F, size_t off, size_t *o) {   /* o[14]: ln1g ln1b wqkv bqkv qg kg wo bo ln2g ln2b w1 b1 w2 b2 (src/nn_attn.cu:460-480) */
+    const size_t c = C, f = F;
+    o[0] = off; off += c; o[1] = off; off += c; o[2] = off; off += 3 * c * c; o[3] = off; off += 3 * c; o[4] = off; off += c; o[5] = off; off += c;
+    o[6] = off; off += c * c; o[7] = off; off += c; o[8] = off; off += c; o[9] = off; off += c; o[10] = off; off += 2 * f * c; o[11] = off; off += 2 * f;
+    o[12] = off; off += c * f; o[13] = off; off += c;
+    return off;
+}
+int orc_block_fwd(int bits, int C, int H, int F, int rope, int nreg, float rope_base, const float *P, const float *x, float *y, int nseq, int S, int Hh, int W) {
+    size_t o[14]; orc_block_layout(C, F, 0, o);
+    const long T = (long)nseq * S;
+    float *xn = malloc((size_t)T * C * 4), *qkv = malloc((size_t)T * 3 * C * 4), *att = malloc((size_t)T * C * 4), *x1 = malloc((size_t)T * C * 4), *hh = malloc((size_t)T * 2 * F * 4), *gg = malloc((size_t)T * F * 4);
+    float *rq = malloc((size_t)T * H * 4), *rk = malloc((size_t)T * H * 4), *lse = malloc((size_t)T * H * 4), amx[4];
+    uint16_t *qh = malloc((size_t)3 * C * (T + 64) * 2);
+    orc_ln_fwd(x, P + o[0], P + o[1], xn, NULL, NULL, T, C);
+    int e = orc_mx_gemm(bits, 0, 1, (int)T, 3 * C, C, xn, P + o[2], qkv, 0.f, P + o[3], NULL);
+    orc_fa_pack(qkv, P + o[4], P + o[5], qh, rq, rk, amx, nseq, S, Hh, W, nreg, C, rope, rope_base);
+    orc_fa8_fwd(qh, att, lse, nseq, S, H, C);
+    e |= orc_mx_gemm(bits, 0, 1, (int)T, C, C, att, P + o[6], x1, 0.f, P + o[7], x);
+    orc_ln_fwd(x1, P + o[8], P + o[9], xn, NULL, NULL, T, C);
+    e |= orc_mx_gemm(bits, 0, 1, (int)T, 2 * F, C, xn, P + o[10], hh, 0.f, P + o[11], NULL);
+    orc_glu_fwd(hh, gg, T, F);
+    e |= orc_mx_gemm(bits, 0, 1, (int)T, C, F, gg, P + o[12], y, 0.f, P + o[13], x1);
+    free(xn); free(qkv); free(att); free(x1); free(hh); free(gg); free(rq); free(rk); free(lse); free(qh);
+    return e;
+}

@@ -20,6 +20,9 @@
  *                                 that key's quantised V row, also when the maximum moves between key tiles; keys past S never
  *                                 contribute) and the reference's own gate, rel. L2 < 0.1 against exact fp64 attention
  *                                 (tests/test_attn.c:445-446)
+ *   orc_ln_fwd, orc_glu_fwd,      pinned: textbook formulas in numpy fp64 (LayerNorm eps 1e-5, SiLU(a) b, RMS-norm eps 1e-6 times gains, rotary
+ *   orc_fa_pack, orc_cs_to_tok    pairs = complex multiplication by exp(i pos base^(-f/8)), norm-preserving), fp16 rounding by numpy
+ *   orc_block_fwd                 pinned: the reference's gate (tests/test_attn.c:398-424): rel. L2 against the exact fp64 block
  *   orc_pred_place                pinned: box intersection by brute force over all voxels; 255 sigmoid rounded to nearest in fp64
  *   orc_feather_blend             pinned: the reference's own checks (tests/test_predict_feather.c:95-121): core and first-window voxels
  *                                 equal the window's own prediction, a z-shell voxel is u(j) own + (1 - u(j)) lower within 1; constant
@@ -112,6 +115,15 @@ void orc_conv1_mx(int xbits, const uint8_t *x, int N, int Ci, size_t S, const fl
 int orc_mx_gemm(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res);
 /* MX-fp8 attention forward on the fp16 head-major pack (src/lp_attn8.cu:124-180, :319-328); head dim 48 */
 void orc_fa8_fwd(const uint16_t *qkvh, float *o, float *lse, int nseq, int S, int H, int C);
+/* the attention block's elementwise pieces and its forward composed from them, orc_mx_gemm and orc_fa8_fwd (src/nn_attn.cu:150-167, :438-446,
+   :460-480, :587-633, :748-759; src/nn_attn_tc.cu:99-136) */
+void orc_ln_fwd(const float *x, const float *g, const float *b, float *y, float *mean, float *rstd, long T, int C);
+void orc_glu_fwd(const float *h, float *gg, long T, int F);
+void orc_cs_to_tok(const float *x, float *t, const float *reg, int n, int C, long Sg, int nreg);
+void orc_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg);
+void orc_fa_pack(const float *qkv, const float *qg, const float *kg, uint16_t *qkvh, float *rq, float *rk, float *amx, int nseq, int S, int Hh, int W, int nreg, int C, int rope, float base);
+size_t orc_block_layout(int C, int F, size_t off, size_t *o);
+int orc_block_fwd(int bits, int C, int H, int F, int rope, int nreg, float rope_base, const float *P, const float *x, float *y, int nseq, int S, int Hh, int W);
 /* sliding-window prediction: sigmoid -> uint8 placement (src/nn_elem.cu:1105-1125) and the one-sided sin^2 feather blend of window borders
    (src/predict.c:282-333) */
 void orc_pred_place(const float *lg, const uint8_t *ct, int D, int W, int hz, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, int iso, uint8_t *dsh);

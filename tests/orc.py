@@ -64,6 +64,13 @@ def lib():
         L.orc_mx_gemm.argtypes = [C.c_int] * 6 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p]
         L.orc_pred_place.restype = None; L.orc_pred_place.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 12 + [C.c_void_p]
         L.orc_feather_blend.restype = None; L.orc_feather_blend.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.orc_ln_fwd.restype = None; L.orc_ln_fwd.argtypes = [C.c_void_p] * 6 + [C.c_long, C.c_int]
+        L.orc_glu_fwd.restype = None; L.orc_glu_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_long, C.c_int]
+        L.orc_cs_to_tok.restype = None; L.orc_cs_to_tok.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_long, C.c_int]
+        L.orc_tok_to_cs.restype = None; L.orc_tok_to_cs.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_long, C.c_int]
+        L.orc_fa_pack.restype = None; L.orc_fa_pack.argtypes = [C.c_void_p] * 7 + [C.c_int] * 7 + [C.c_float]
+        L.orc_block_layout.restype = C.c_size_t; L.orc_block_layout.argtypes = [C.c_int, C.c_int, C.c_size_t, C.c_void_p]
+        L.orc_block_fwd.restype = C.c_int; L.orc_block_fwd.argtypes = [C.c_int] * 6 + [C.c_float, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 4
         L.orc_fa8_fwd.restype = None; L.orc_fa8_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
         _lib = L
     return _lib
@@ -155,3 +162,27 @@ def feather_blend(E, present, S, B, nss, bn):
     out = np.zeros(tuple(int(v) for v in bn), np.uint8)
     lib().orc_feather_blend(ptr(E), ptr(present), S, B, ptr(nss_a), ptr(bn_a), ptr(out))
     return out
+
+
+BLOCK_FIELDS = ("ln1g", "ln1b", "wqkv", "bqkv", "qg", "kg", "wo", "bo", "ln2g", "ln2b", "w1", "b1", "w2", "b2")
+
+
+def block_layout(Cc, F, off=0):
+    o = np.zeros(14, np.uint64)
+    end = lib().orc_block_layout(Cc, F, off, ptr(o))
+    return dict(zip(BLOCK_FIELDS, (int(v) for v in o))), int(end)
+
+
+def fa_pack(qkv, qg, kg, nseq, S, Hh, W, nreg, Cc, rope, base=100.0):
+    H = Cc // 48; T = nseq * S
+    qkv = np.ascontiguousarray(qkv, np.float32); qg = np.ascontiguousarray(qg, np.float32); kg = np.ascontiguousarray(kg, np.float32)
+    qh = np.zeros((3, H, T + 64, 48), np.uint16); rq = np.zeros((T, H), np.float32); rk = np.zeros((T, H), np.float32); amx = np.zeros(4, np.float32)
+    lib().orc_fa_pack(ptr(qkv), ptr(qg), ptr(kg), ptr(qh), ptr(rq), ptr(rk), ptr(amx), nseq, S, Hh, W, nreg, Cc, rope, base)
+    return qh, rq, rk, amx
+
+
+def block_fwd(bits, Cc, H, F, rope, nreg, base, P, x, nseq, S, Hh, W):
+    P = np.ascontiguousarray(P, np.float32); x = np.ascontiguousarray(x, np.float32)
+    y = np.zeros_like(x)
+    assert lib().orc_block_fwd(bits, Cc, H, F, rope, nreg, base, ptr(P), ptr(x), ptr(y), nseq, S, Hh, W) == 0
+    return y

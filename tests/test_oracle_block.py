@@ -1,0 +1,111 @@
+"""Pins of the oracle's attention-block pieces (CPU only): textbook formulas in numpy fp64, and the reference's gate for the whole block
+(tests/test_attn.c:398-424: MX linears and the MX-fp8 core against the exact block, relative L2)."""
+import numpy as np
+import pytest
+
+import orc
+
+
+def ln64(x, g, b, eps=1e-5):
+    m = x.mean(-1, keepdims=True); v = ((x - m) ** 2).mean(-1, keepdims=True)
+    return (x - m) / np.sqrt(v + eps) * g + b
+
+
+def test_layernorm_glu_and_token_layout():
+    rng = np.random.default_rng(0)
+    T, Cc, F = 37, 96, 40
+    x = (2 * rng.standard_normal((T, Cc)) + 1).astype(np.float32); g = rng.uniform(0.5, 1.5, Cc).astype(np.float32); b = rng.standard_normal(Cc).astype(np.float32)
+    y = np.zeros_like(x); m = np.zeros(T, np.float32); r = np.zeros(T, np.float32)
+    orc.lib().orc_ln_fwd(orc.ptr(x), orc.ptr(g), orc.ptr(b), orc.ptr(y), orc.ptr(m), orc.ptr(r), T, Cc)
+    x64 = x.astype(np.float64)
+    assert np.abs(y - ln64(x64, g, b)).max() < 1e-5 and np.abs(m - x64.mean(1)).max() < 1e-6
+    assert np.abs(r - 1 / np.sqrt(x64.var(1) + 1e-5)).max() < 1e-5
+    h = rng.standard_normal((T, 2 * F)).astype(np.float32); gg = np.zeros((T, F), np.float32)
+    orc.lib().orc_glu_fwd(orc.ptr(h), orc.ptr(gg), T, F)
+    a, bb = h[:, :F].astype(np.float64), h[:, F:].astype(np.float64)
+    assert np.abs(gg - a / (1 + np.exp(-a)) * bb).max() < 1e-6
+    n, Sg, nreg = 2, 27, 3
+    xc = rng.standard_normal((n, Cc, Sg)).astype(np.float32); reg = rng.standard_normal((nreg, Cc)).astype(np.float32)
+    tok = np.zeros((n, Sg + nreg, Cc), np.float32)
+    orc.lib().orc_cs_to_tok(orc.ptr(xc), orc.ptr(tok), orc.ptr(reg), n, Cc, Sg, nreg)
+    assert np.array_equal(tok[:, :nreg], np.broadcast_to(reg, (n, nreg, Cc))) and np.array_equal(tok[:, nreg:], xc.transpose(0, 2, 1))
+    back = np.zeros_like(xc)
+    orc.lib().orc_tok_to_cs(orc.ptr(tok), orc.ptr(back), n, Cc, Sg, nreg)
+    assert np.array_equal(back, xc)                                   # registers dropped, the grid tokens back in place
+
+
+@pytest.mark.parametrize("rope", [0, 1])
+def test_pack_is_rms_norm_gains_rotary_and_fp16(rope):
+    rng = np.random.default_rng(1 + rope)
+    nseq, D, nreg, Cc = 2, 3, 2, 96; H = Cc // 48; S = nreg + D ** 3; T = nseq * S
+    qkv = rng.standard_normal((T, 3, H, 48)); qg = 1 + 0.2 * rng.standard_normal((H, 48)); kg = 1 + 0.2 * rng.standard_normal((H, 48))
+    qh, rq, rk, amx = orc.fa_pack(qkv.reshape(T, 3 * Cc), qg, kg, nseq, S, D, D, nreg, Cc, rope, 100.0)
+    x = qkv.astype(np.float32).astype(np.float64)
+    want = np.zeros((3, H, T, 48))
+    for p, gains in ((0, qg), (1, kg)):
+        r = 1 / np.sqrt((x[:, p] ** 2).mean(-1, keepdims=True) + 1e-6)
+        v = x[:, p] * r * gains.astype(np.float32)[None]
+        assert np.abs((rq if p == 0 else rk) - r[..., 0]).max() < 1e-5
+        if rope:
+            ts = np.arange(T) % S - nreg
+            pos = np.stack([ts // (D * D), (ts // D) % D, ts % D], -1).astype(np.float64)           # z, y, x of the grid token
+            for ax in range(3):
+                ang = pos[:, ax, None] * 100.0 ** (-np.arange(8) / 8.0)[None]                      # [T][8]
+                z = (v[..., 16 * ax:16 * ax + 16:2] + 1j * v[..., 16 * ax + 1:16 * ax + 16:2]) * np.exp(1j * ang)[:, None, :]
+                rot = np.stack([z.real, z.imag], -1).reshape(T, H, 16)
+                v[..., 16 * ax:16 * ax + 16] = np.where((ts >= 0)[:, None, None], rot, v[..., 16 * ax:16 * ax + 16])
+        want[p] = v.transpose(1, 0, 2)
+    want[2] = x[:, 2].transpose(1, 0, 2)
+    got = qh.view(np.float16).astype(np.float64)
+    assert (got[:, :, T:] == 0).all()                                  # the 64 padding rows
+    err = np.abs(got[:, :, :T] - want)
+    assert (err <= np.abs(want) * 2.0 ** -10 + 1e-6).all()             # fp16 rounding of the fp32 result (half an ulp of 11 bits, plus fp32 noise)
+    assert abs(amx[1] - np.abs(x[:, 2]).max()) < 1e-6 and amx[0] == 0
+    if rope:                                                           # rotations preserve the norm of every pair; registers are not rotated
+        assert np.abs((got[0, :, :T] ** 2).sum(-1) - (want[0] ** 2).sum(-1)).max() < 0.05
+
+
+def exact_block(P, lay, x, nseq, S, H, Cc, F):
+    P = P.astype(np.float64); x = x.astype(np.float64)
+    g = lambda k, n: P[lay[k]:lay[k] + n]
+    xn = ln64(x, g("ln1g", Cc), g("ln1b", Cc))
+    qkv = xn @ g("wqkv", 3 * Cc * Cc).reshape(3 * Cc, Cc).T + g("bqkv", 3 * Cc)
+    T = nseq * S
+    q, k, v = (qkv[:, i * Cc:(i + 1) * Cc].reshape(T, H, 48) for i in range(3))
+    q = q / np.sqrt((q ** 2).mean(-1, keepdims=True) + 1e-6) * g("qg", Cc).reshape(H, 48)
+    k = k / np.sqrt((k ** 2).mean(-1, keepdims=True) + 1e-6) * g("kg", Cc).reshape(H, 48)
+    o = np.zeros((T, Cc))
+    for s in range(nseq):
+        sl = slice(s * S, (s + 1) * S)
+        for h in range(H):
+            lg = q[sl, h] @ k[sl, h].T / np.sqrt(48.0); e = np.exp(lg - lg.max(1, keepdims=True))
+            o[sl, h * 48:(h + 1) * 48] = (e / e.sum(1, keepdims=True)) @ v[sl, h]
+    x1 = o @ g("wo", Cc * Cc).reshape(Cc, Cc).T + g("bo", Cc) + x
+    xn2 = ln64(x1, g("ln2g", Cc), g("ln2b", Cc))
+    hh = xn2 @ g("w1", 2 * F * Cc).reshape(2 * F, Cc).T + g("b1", 2 * F)
+    gg = hh[:, :F] / (1 + np.exp(-hh[:, :F])) * hh[:, F:]
+    return gg @ g("w2", Cc * F).reshape(Cc, F).T + g("b2", Cc) + x1
+
+
+def make_block(rng, Cc, F):
+    lay, n = orc.block_layout(Cc, F)
+    P = (0.05 * rng.standard_normal(n)).astype(np.float32)                   # as tests/test_attn.c:407-408
+    for k in ("ln1g", "ln2g", "qg", "kg"):
+        P[lay[k]:lay[k] + Cc] = 1
+    return P, lay
+
+
+@pytest.mark.parametrize("bits,tol", [(8, 0.1), (4, 0.35)])
+def test_block_within_reference_gate_of_exact_block(bits, tol):
+    rng = np.random.default_rng(bits)
+    Cc, H, F, nseq, D = 96, 2, 128, 2, 4; S = D ** 3
+    P, lay = make_block(rng, Cc, F)
+    assert orc.block_layout(Cc, F)[1] == 2 * Cc + 3 * Cc * Cc + 3 * Cc + 2 * Cc + Cc * Cc + Cc + 2 * Cc + 2 * F * Cc + 2 * F + Cc * F + Cc      # src/nn_attn.cu:460-480
+    x = rng.standard_normal((nseq * S, Cc)).astype(np.float32)
+    y = orc.block_fwd(bits, Cc, H, F, 0, 0, 100.0, P, x, nseq, S, D, D)
+    ye = exact_block(P, lay, x, nseq, S, H, Cc, F)
+    rel = np.linalg.norm(y - ye) / np.linalg.norm(ye)
+    assert rel < tol, rel
+    # the residual stream dominates y; the gate must also hold on what the block adds
+    rel_d = np.linalg.norm((y - x) - (ye - x)) / np.linalg.norm(ye - x)
+    assert rel_d < 3 * tol, rel_d

@@ -91,8 +91,38 @@ class at_geom(C.Structure):  # src/attn.h:81
                 ("lens", C.c_void_p), ("pos", C.c_void_p), ("rays", C.c_void_p), ("dfx", C.c_void_p * 3), ("dfr", C.c_void_p)]
 
 
+class at_dims(C.Structure):  # src/attn.h:33
+    _fields_ = [("C", C.c_int), ("H", C.c_int), ("F", C.c_int), ("rope", C.c_int), ("nreg", C.c_int), ("rope_base", C.c_float),
+                ("dK", C.c_int), ("dL", C.c_int), ("dC", C.c_int * 3), ("dCo", C.c_int), ("dInit", C.c_int)]
+
+
+class at_bp(C.Structure):  # src/attn.h:39
+    _fields_ = [(n, C.c_size_t) for n in ("ln1g", "ln1b", "wqkv", "bqkv", "qg", "kg", "wo", "bo", "ln2g", "ln2b", "w1", "b1", "w2", "b2", "woa", "boa")] + \
+               [("wvl", C.c_size_t * 3), ("bvl", C.c_size_t * 3)]
+
+
+class at_ws(C.Structure):  # src/attn.h:47-60
+    _fields_ = [(n, C.c_void_p) for n in ("xn", "qkv", "qkn", "o", "x1", "xn2", "h", "gg", "m1", "r1", "m2", "r2", "rq", "rk", "lse", "dv",
+                                          "bA", "bB", "bC", "dx1", "qkvh", "doh", "amx", "qkvr", "orr", "dor", "dqr", "dqr2")] + \
+               [("vl", C.c_void_p * 4), ("oa", C.c_void_p), ("aw", C.c_void_p), ("dvl", C.c_void_p * 4), ("doa", C.c_void_p), ("kept", C.c_int), ("vr", C.c_int),
+                ("v1", C.c_void_p), ("own", C.c_void_p), ("dv1", C.c_void_p), ("lam", C.c_void_p), ("glam", C.c_void_p)]
+
+
 # include/mi_attn.h
 _ATTN_PROTOS = {
+    "at_block_nparams": (_Z, [C.POINTER(at_dims)]),
+    "at_block_layout": (_Z, [C.POINTER(at_dims), C.POINTER(at_bp), _Z]),
+    "at_ws_bytes": (_Z, [C.POINTER(at_dims), C.c_long]),
+    "at_ws_carve": (None, [C.POINTER(at_ws), C.POINTER(at_dims), C.c_long, _P]),
+    "at_set_mx": (None, [_I]),
+    "at_get_mx": (_I, []),
+    "at_gemm_ex": (_I, [_I, _I, _I, _I, _I, _P, _P, _P, _F, _P, _P]),
+    "at_ln_fwd": (None, [_P, _P, _P, _P, _P, _P, C.c_long, _I]),
+    "at_glu_fwd": (None, [_P, _P, C.c_long, _I]),
+    "at_fa_pack": (None, [_P, _P, _P, _P, _P, _P, _P, C.POINTER(at_geom), _I, _I, _I, _F]),
+    "at_cs_to_tok": (None, [_P, _P, _P, _I, _I, C.c_long, _I]),
+    "at_tok_to_cs": (None, [_P, _P, _I, _I, C.c_long, _I]),
+    "at_block_fwd": (_I, [C.POINTER(at_dims), _P, C.POINTER(at_bp), _P, _P, C.POINTER(at_geom), C.POINTER(at_ws)]),
     "lp_mx_gemm": (_I, [_I, _I, _I, _I, _I, _I, _P, _P, _P, _F]),
     "lp_mx_gemm_ex": (_I, [_I, _I, _I, _I, _I, _I, _P, _P, _P, _F, _P, _P]),
     "at_fa8_fwd": (_I, [_P, _P, _P, C.POINTER(at_geom), _I, _I]),
