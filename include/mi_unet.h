@@ -7,6 +7,7 @@
 #ifndef MI_UNET_H
 #define MI_UNET_H
 #include "mi_lp.h"
+#include "mi_attn.h"
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -39,6 +40,13 @@ typedef struct {
     int head_out;              /* logits */
     int act_dt;                /* activation storage: 8 MX-fp8, 4 MX-fp4 */
     int prec;                  /* 3: fp4 compute everywhere (MX-fp4 weights over MX-fp8 storage), else by storage */
+    /* transformer blocks on the bottleneck level's raw output (src/unet.h:72-80; 0 = none): tokens = attn_reg learned register rows + the
+       bottleneck grid, pre-LN blocks (MHSA with QK-norm, heads of 48, SwiGLU) on the MX-fp8 attention core with MX-fp8 linears; the level's
+       output GroupNorm moves after the stage. The bottleneck width must be a multiple of 48 */
+    int attn_blocks;
+    int attn_pe;               /* 1 axial 3-D RoPE, 2 none (0 PEG and 3 scroll RoPE are not provided) */
+    int attn_reg;              /* register tokens per sample */
+    int attn_mlp;              /* SwiGLU hidden width (0: 8/3 of the width rounded up to 32) */
 } unet_cfg;
 typedef struct unet unet;
 unet *unet_create(const unet_cfg *cfg, shape5 in);             /* in: the window (n, cin, d, h, w); dims divisible by 2^(nlev-1) */

@@ -131,3 +131,61 @@ def test_unet_is_deterministic_and_storage_registry(gpu):
     H_.nn_set_storage(dxq.ptr, dxq.nbytes, 4); assert H_.nn_storage(dxq.ptr + 5) == 4
     H_.nn_set_storage(dxq.ptr, 0, 0); assert H_.nn_storage(dxq.ptr) == 0
     net.close()
+
+
+def test_unet_attention_stage(gpu):
+    """The transformer blocks on the bottleneck (src/unet.c:2795-2835): with the initial zero out-projections the stage is an identity on
+    the tokens, so the net must agree with the plain one; with trained-like parameters the stage's output tensor must match the oracle's
+    composition (MX -> fp32 planes -> tokens with registers -> blocks -> planes -> MX) of the device's own bottleneck tensor."""
+    from ufsm_amd.unet import UNet, make_cfg
+    rng = np.random.default_rng(12)
+    N, D = 2, 16; widths = [32, 96]; cin, head_out, nreg, nblk = 4, 2, 3, 2
+    S = D ** 3
+    x = rng.standard_normal((N, cin, S)).astype(np.float32)
+    dxq = to_mx(8, x)
+    plain = UNet(make_cfg(cin, widths, head_out=head_out), N, D, D, D, seed=7)
+    att = UNet(make_cfg(cin, widths, head_out=head_out, attn_blocks=nblk, attn_pe=1, attn_reg=nreg), N, D, D, D, seed=7)
+    pp, pa = plain.params(), att.params()
+    assert np.array_equal(pa[:pp.size], pp)                                  # the attention parameters come last (src/unet.c:490-499)
+    Cb = widths[-1]; F = (8 * Cb // 3 + 31) // 32 * 32
+    lay0, end0 = orc.block_layout(Cb, F, pp.size + nreg * Cb); lay1, end1 = orc.block_layout(Cb, F, end0)
+    assert end1 == pa.size and (pa[lay0["wo"]:lay0["wo"] + Cb * Cb] == 0).all() and (pa[lay0["ln1g"]:lay0["ln1g"] + Cb] == 1).all()
+    assert abs(pa[lay0["wqkv"]:lay0["wqkv"] + 3 * Cb * Cb].std() * np.sqrt(Cb) - 1) < 0.05                  # N(0, 1 / C) (src/unet.c:619)
+    dl0, dl1 = DevBuf(N * head_out * S * 4), DevBuf(N * head_out * S * 4)
+    assert plain.forward_x(dxq.ptr, dl0.ptr) == 0 and att.forward_x(dxq.ptr, dl1.ptr) == 0
+    LP.check()
+    l0, l1 = dl0.to_numpy(np.float32), dl1.to_numpy(np.float32)
+    # identity stage: the decoder reads the re-quantised bottleneck (same decoded values) with statistics of the stored tensor
+    assert np.linalg.norm(l1 - l0) / np.linalg.norm(l0) < 2e-2
+    # ---- non-trivial blocks ----
+    for lay in (lay0, lay1):
+        for k, n in (("wo", Cb * Cb), ("w2", Cb * F), ("bo", Cb), ("b1", 2 * F), ("bqkv", 3 * Cb)):
+            pa[lay[k]:lay[k] + n] = 0.05 * rng.standard_normal(n)
+        for k in ("ln1g", "ln2g", "qg", "kg"):
+            pa[lay[k]:lay[k] + Cb] = rng.uniform(0.8, 1.2, Cb)
+    att.set_params(pa)
+    assert att.forward_x(dxq.ptr, dl1.ptr) == 0
+    LP.check()
+    outs = {name: (ptr, shp) for name, ptr, shp in att.layer_outs()}
+    assert "attn" in outs and outs["attn"][1] == (N, Cb, D // 2, D // 2, D // 2)
+    Sg = (D // 2) ** 3
+
+    def fetch(name):
+        ptr, shp = outs[name]; nb = lib.lp_mx8_bytes(shp[0], shp[1], Sg)
+        buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+        return orc.mx_to_f32(8, buf, N, Cb, Sg)
+
+    xb, got = fetch("enc1.c2"), fetch("attn")
+    tok = np.zeros((N, Sg + nreg, Cb), np.float32)
+    reg = np.ascontiguousarray(pa[pp.size:pp.size + nreg * Cb].reshape(nreg, Cb))
+    orc.lib().orc_cs_to_tok(orc.ptr(xb), orc.ptr(tok), orc.ptr(reg), N, Cb, Sg, nreg)
+    t = tok.reshape(N * (Sg + nreg), Cb)
+    for lay in (lay0, lay1):
+        t = orc.block_fwd(8, Cb, Cb // 48, F, 1, nreg, 100.0, pa[lay["ln1g"]:lay["b2"] + Cb], t, N, Sg + nreg, D // 2, D // 2)
+    want = np.zeros_like(xb)
+    orc.lib().orc_tok_to_cs(orc.ptr(t), orc.ptr(want), N, Cb, Sg, nreg)
+    want = orc.mx_to_f32(8, orc.f32_to_mx(8, want, N, Cb, Sg), N, Cb, Sg)
+    rel = np.linalg.norm(got - want) / np.linalg.norm(want - xb)
+    assert rel < 0.05, rel                                                   # two blocks of MX re-quantisations apart, then one e4m3 rounding
+    assert np.linalg.norm(got - xb) / np.linalg.norm(xb) > 0.05              # and the stage did change the tensor
+    plain.close(); att.close()

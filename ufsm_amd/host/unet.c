@@ -27,6 +27,10 @@ struct unet {
     size_t np; float *params;                                      /* device */
     void *xin;                                                     /* the network input built from a CT window */
     struct { const void *p; shape5 s; const char *name; const float *mean, *rstd; int G; } outs[64]; int nouts;
+    /* the attention stage on the bottleneck (src/unet.c:470-509 set-up, :2795-2835 forward) */
+    int tbn; at_dims tbd; at_bp tbp[16]; size_t reg_off; at_geom tbg; at_ws tbw;
+    block tb;                                                      /* its output: a2 and the statistics m2 / r2 (the level's n2 affine) */
+    float *tb_cs, *tb_tok; void *tb_ws;                            /* fp32 planes [n][C][Sg]; token rows, one buffer per block + 1; block scratch */
 };
 
 static int G_of(const unet *u, int c) { return u->cfg.G < c ? u->cfg.G : c; }      /* src/unet.c:297 */
@@ -59,6 +63,18 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
         off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
     }
     off = add_conv(&u->head, w[0], cfg->head_out, 1, off);
+    if (cfg->attn_blocks > 0) {                                   /* parameters last: registers, then the blocks (src/unet.c:490-499) */
+        const int C = w[L - 1];
+        if (C % AT_HD || cfg->attn_blocks > 16 || (cfg->attn_pe != 1 && cfg->attn_pe != 2) || cfg->attn_reg < 0) {
+            fprintf(stderr, "unet_create: attention blocks need a bottleneck width that is a multiple of %d (got %d), at most 16 blocks, attn_pe 1 (RoPE) or 2 (none)\n", AT_HD, C);
+            free(u); return nullptr;
+        }
+        const int F = cfg->attn_mlp > 0 ? cfg->attn_mlp : (8 * C / 3 + 31) / 32 * 32;
+        u->tbd = (at_dims){C, C / AT_HD, F, cfg->attn_pe == 1 ? 1 : 0, cfg->attn_reg, 100.f};
+        u->reg_off = off; off += (size_t)cfg->attn_reg * C;
+        for (int k = 0; k < cfg->attn_blocks; k++) off = at_block_layout(&u->tbd, &u->tbp[k], off);
+        u->tbn = cfg->attn_blocks;
+    }
     u->np = off;
     u->params = f32_new(off);
     for (int i = 0; i < L; i++) u->ls[i] = (shape5){in.n, w[i], in.d >> i, in.h >> i, in.w >> i};
@@ -74,6 +90,15 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
         if (i < L - 1) { shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds); }
     }
     u->xin = act_new(u, in);
+    if (u->tbn) {
+        const shape5 ys = u->ls[L - 1]; const long Sg = (long)ys.d * ys.h * ys.w, S = Sg + u->tbd.nreg, T = (long)ys.n * S; const int C = u->tbd.C;
+        u->tbg = (at_geom){.nseq = ys.n, .S = (int)S, .D = ys.d, .Hh = ys.h, .W = ys.w};
+        u->tb.ys = ys; u->tb.a2 = act_new(u, ys);
+        const size_t ng = (size_t)in.n * G_of(u, C);
+        u->tb.m2 = f32_new(ng); u->tb.r2 = f32_new(ng);
+        u->tb_cs = f32_new((size_t)ys.n * C * Sg); u->tb_tok = f32_new((size_t)(u->tbn + 1) * T * C);
+        u->tb_ws = mi_malloc(at_ws_bytes(&u->tbd, T)); at_ws_carve(&u->tbw, &u->tbd, T, u->tb_ws);
+    }
     return u;
 }
 void unet_free(unet *u) {
@@ -83,6 +108,7 @@ void unet_free(unet *u) {
         for (int s = 0; s < 2; s++) { block *b = s ? &u->dec[i] : &u->enc[i]; act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2); }
         act_del(u->downo[i]);
     }
+    if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); }
     act_del(u->xin); mi_free(u->params);
     lp_wmemo_clear();
     free(u);
@@ -109,6 +135,16 @@ void unet_init(unet *u, uint64_t seed) {
     for (int i = 0; i < L - 1; i++) init_conv(h, &u->down[i], &seed, 0);
     for (int i = 0; i < L - 1; i++) { init_conv(h, &u->dec[i].c1, &seed, 0); init_gn(h, &u->dec[i].n1); init_conv(h, &u->dec[i].c2, &seed, 0); init_gn(h, &u->dec[i].n2); }
     init_conv(h, &u->head, &seed, -2.0);
+    if (u->tbn) {   /* LayerNorm and QK-norm gains 1, QKV and MLP-in N(0, 1 / C), out projections and biases 0 (identity blocks), registers N(0, 0.02^2) (src/unet.c:612-642) */
+        const int C = u->tbd.C, F = u->tbd.F; const double sd = 1.0 / sqrt((double)C);
+        for (int k = 0; k < u->tbn; k++) {
+            const at_bp *bp = &u->tbp[k];
+            for (int c = 0; c < C; c++) h[bp->ln1g + c] = h[bp->ln2g + c] = h[bp->qg + c] = h[bp->kg + c] = 1.f;
+            for (size_t i = 0; i < (size_t)3 * C * C; i++) h[bp->wqkv + i] = (float)(sd * gauss(&seed));
+            for (size_t i = 0; i < (size_t)2 * F * C; i++) h[bp->w1 + i] = (float)(sd * gauss(&seed));
+        }
+        for (size_t i = 0; i < (size_t)u->tbd.nreg * C; i++) h[u->reg_off + i] = (float)(0.02 * gauss(&seed));
+    }
     unet_set_params(u, h);
     free(h);
 }
@@ -131,6 +167,23 @@ static int block_fwd(unet *u, block *b, const void *x, const nn_gn_t *gin, const
     note(u, b->a2, b->ys, n2, b->m2, b->r2, G);
     return r;
 }
+/* the bottleneck's raw output -> fp32 planes -> token rows with the registers prepended -> blocks -> planes -> a new MX tensor with its
+   GroupNorm statistics: the level's output for the decoder (src/unet.c:2795-2835; no PEG, memory, view or deformable paths) */
+static int tb_fwd(unet *u) {
+    const block *x = &u->enc[u->cfg.nlev - 1]; block *b = &u->tb;
+    const shape5 ys = b->ys; const int C = u->tbd.C, nr = u->tbd.nreg; const size_t Sg = (size_t)ys.d * ys.h * ys.w, TC = (size_t)u->tbg.nseq * u->tbg.S * C;
+    if (u->cfg.act_dt == 4) lp_mx4_to_f32(x->a2, ys.n, C, Sg, u->tb_cs); else lp_mx8_to_f32(x->a2, ys.n, C, Sg, u->tb_cs);
+    at_cs_to_tok(u->tb_cs, u->tb_tok, P(u, u->reg_off), ys.n, C, (long)Sg, nr);
+    at_set_mx(8);
+    for (int k = 0; k < u->tbn; k++)
+        if (at_block_fwd(&u->tbd, u->params, &u->tbp[k], u->tb_tok + (size_t)k * TC, u->tb_tok + (size_t)(k + 1) * TC, &u->tbg, &u->tbw)) { fprintf(stderr, "unet: attention block forward failed\n"); return -1; }
+    at_tok_to_cs(u->tb_tok + (size_t)u->tbn * TC, u->tb_cs, ys.n, C, (long)Sg, nr);
+    if (u->cfg.act_dt == 4) lp_f32_to_mx4(u->tb_cs, ys.n, C, Sg, b->a2); else lp_f32_to_mx8(u->tb_cs, ys.n, C, Sg, b->a2);
+    const int G = G_of(u, C);
+    if (nn_gn_stats(b->a2, ys, G, 1e-5f, b->m2, b->r2)) { fprintf(stderr, "unet: attention stage GroupNorm statistics unsupported for this storage\n"); return -1; }
+    note(u, b->a2, ys, "attn", b->m2, b->r2, G);
+    return 0;
+}
 int unet_forward_x(unet *u, const void *x, float *logits) {
     static const char *en1[] = {"enc0.c1", "enc1.c1", "enc2.c1", "enc3.c1", "enc4.c1", "enc5.c1", "enc6.c1", "enc7.c1"}, *en2[] = {"enc0.c2", "enc1.c2", "enc2.c2", "enc3.c2", "enc4.c2", "enc5.c2", "enc6.c2", "enc7.c2"};
     static const char *dn1[] = {"dec0.c1", "dec1.c1", "dec2.c1", "dec3.c1", "dec4.c1", "dec5.c1", "dec6.c1"}, *dn2[] = {"dec0.c2", "dec1.c2", "dec2.c2", "dec3.c2", "dec4.c2", "dec5.c2", "dec6.c2"};
@@ -151,9 +204,11 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
             cur = u->downo[i];
         }
     }
+    if (u->tbn && tb_fwd(u)) { if (reg_here) nn_storage_forget(x); return -1; }
     for (int i = L - 2; i >= 0; i--) {                             /* decoder: nothing materialised (src/unet.c:3010-3013) */
         const block *coarse = i == L - 2 ? &u->enc[L - 1] : &u->dec[i + 1];
-        const nn_gn_t gc = gn_out(u, coarse), gs = gn_out(u, &u->enc[i]);
+        nn_gn_t gc = gn_out(u, coarse); const nn_gn_t gs = gn_out(u, &u->enc[i]);
+        if (i == L - 2 && u->tbn) { coarse = &u->tb; gc.mean = u->tb.m2; gc.rstd = u->tb.r2; }      /* the stage's output under the level's n2 affine (src/unet.c:508) */
         if (block_fwd(u, &u->dec[i], u->enc[i].a2, &gs, coarse->a2, &gc, u->cfg.widths[i + 1], dn1[i], dn2[i])) return -1;
     }
     const block *last = L > 1 ? &u->dec[0] : &u->enc[0];

@@ -13,7 +13,7 @@ UNET_MAXLEV = 8
 
 class unet_cfg(C.Structure):
     _fields_ = [("cin", C.c_int), ("nlev", C.c_int), ("widths", C.c_int * UNET_MAXLEV), ("G", C.c_int), ("head_out", C.c_int),
-                ("act_dt", C.c_int), ("prec", C.c_int)]
+                ("act_dt", C.c_int), ("prec", C.c_int), ("attn_blocks", C.c_int), ("attn_pe", C.c_int), ("attn_reg", C.c_int), ("attn_mlp", C.c_int)]
 
 
 _host = None
@@ -52,9 +52,10 @@ def load_host():
     return L
 
 
-def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0):
+def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0):
     c = unet_cfg()
     c.cin, c.nlev, c.G, c.head_out, c.act_dt, c.prec = cin, len(widths), G, head_out, act_dt, prec
+    c.attn_blocks, c.attn_pe, c.attn_reg, c.attn_mlp = attn_blocks, attn_pe, attn_reg, attn_mlp
     for i, w in enumerate(widths):
         c.widths[i] = w
     return c
