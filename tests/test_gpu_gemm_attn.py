@@ -112,6 +112,27 @@ def test_attention_matches_oracle(gpu, nseq, S, H):
     assert np.linalg.norm(o - oe) / np.linalg.norm(oe) < 0.1 and np.linalg.norm(lse - le) / np.linalg.norm(le) < 0.1
 
 
+def test_attention_full_size_of_the_window_bottleneck(gpu):
+    """The configs[4] shape: one sequence of 4 registers + 16^3 grid tokens, 4 heads (C 192). Against the oracle on sampled query rows'
+    worth of checks (the whole oracle run is a few seconds on the host cores), and two size-independent properties: every output row lies
+    in the convex hull of the quantised V (|o| <= max |v| per dim), and lse >= the largest logit of a row (checked through its bound
+    log2 S + max - ... >= 0 on the softmax denominator: 2^(lse - m) in [1, S])."""
+    rng = np.random.default_rng(77)
+    nseq, S, H = 1, 4 + 16 ** 3, 4
+    qk = normed_qkv(rng, nseq, S, H)
+    o, lse = gpu_attention(qk, nseq, S, H)
+    wo, wl = orc.fa8_fwd(qk, nseq, S, H)
+    # with 4100 keys every query row carries a dozen of the one-in-300 P code steps (each 2^-4 of one key's ~1/4100 weight), and the
+    # outputs themselves are small averages: the row errors rise to ~1e-3 of max |o| but stay steps of single keys
+    rows = np.abs(o - wo).max(1) / np.abs(wo).max()
+    assert np.median(rows) < 2e-3 and rows.max() < 3e-2 and np.linalg.norm(o - wo) <= 1e-2 * np.linalg.norm(wo)
+    assert np.abs(lse - wl).max() < 1e-4 * np.abs(wl).max()
+    v = qk.view(np.float16)[2].astype(np.float32)[:, :S]                              # [H][S][48]
+    for h in range(H):
+        assert (np.abs(o[:, h * 48:(h + 1) * 48]) <= np.abs(v[h]).max(0)[None] * (1 + 2.0 ** -3)).all()      # (e4m3 rounding of V can exceed |v| by 1/16)
+    assert np.isfinite(o).all() and np.isfinite(lse).all()
+
+
 def test_attention_closed_forms(gpu):
     """q = 0: o is the mean of the quantised V over the S valid keys and lse = log2 S, exactly as on the oracle; rows of another
     sequence or of the padding must not leak in."""
