@@ -139,31 +139,30 @@ __device__ __forceinline__ void conv_stage_halo(const conv_args &a, unsigned cha
                                                 int iz0, int iy0, int ix0, int tid) {
     using HL = halo_t<FMT, STRIDE, TZ>;
     constexpr int HY = HL::HY, HX = HL::HX, TT = HL::TT, NH = HL::NH;
-    constexpr int NE = (TT * NH + 255) / 256, NS = (TT + 255) / 256;
+    // Thread t owns the (position, 16-byte half) elements (t / NH + k PS, t % NH), k < NE, PS = 256 / NH positions apart, and (its half-0
+    // lanes) the scale bytes of the same positions: one set of coordinates serves both. The coordinates of element k + 1 follow from
+    // element k by adding PS = DZ HY HX + DY HX + DX with carries, so only the first needs divisions.
+    constexpr int PS = 256 / NH, NE = (TT + PS - 1) / PS;
+    constexpr int DZ = PS / (HY * HX), DY = (PS - DZ * HY * HX) / HX, DX = PS - DZ * HY * HX - DY * HX;
     const size_t Sin = (size_t)a.D * a.H * a.W;
-    unsigned eoff[NE]; unsigned edst[NE]; bool eok[NE];
+    const int hf = NH == 2 ? tid & 1 : 0, p0 = tid / NH;
+    unsigned evox[NE]; unsigned edst[NE]; bool eok[NE];
+    {
+        int px = p0 % HX, py = (p0 / HX) % HY, pz = p0 / (HX * HY);
 #pragma unroll
-    for (int k = 0; k < NE; k++) {
-        const int i = min(tid + k * 256, TT * NH - 1), pos = i / NH, hf = i - pos * NH;
-        const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
-        const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
-        eok[k] = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
-        const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1);
-        eoff[k] = (unsigned)((cz * a.H + cy) * a.W + cx) * 2u + (unsigned)hf;     // voxel index and half
-        edst[k] = act_o + (hf * TT + pos) * 16;
-    }
-    unsigned soff[NS]; bool sok[NS];
-#pragma unroll
-    for (int k = 0; k < NS; k++) {
-        const int pos = min(tid + k * 256, TT - 1);
-        const int px = pos % HX, py = (pos / HX) % HY, pz = pos / (HX * HY);
-        const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
-        sok[k] = gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
-        const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1);
-        soff[k] = (unsigned)((cz * a.H + cy) * a.W + cx);
+        for (int k = 0; k < NE; k++) {
+            const int gz = iz0 + pz, gy = iy0 + py, gx = ix0 + px;
+            eok[k] = p0 + k * PS < TT && (unsigned)gz < (unsigned)a.D && (unsigned)gy < (unsigned)a.H && (unsigned)gx < (unsigned)a.W;
+            const int cz = min(max(gz, 0), a.D - 1), cy = min(max(gy, 0), a.H - 1), cx = min(max(gx, 0), a.W - 1);      // (a clamped in-tensor address; zeroed after the load)
+            evox[k] = (unsigned)((cz * a.H + cy) * a.W + cx);
+            edst[k] = (unsigned)(hf * TT + min(p0 + k * PS, TT - 1)) * 16u;
+            px += DX; py += DY; pz += DZ;
+            if (px >= HX) { px -= HX; py++; }
+            if (py >= HY) { py -= HY; pz++; }
+        }
     }
     for (int bl0 = 0; bl0 < nbc; bl0 += GB) {
-        v4i val[GB][NE]; bool ok[GB][NE]; unsigned sv[GB][NS]; bool bokg[GB];
+        v4i val[GB][NE]; bool ok[GB][NE]; unsigned sv[GB][NE]; bool bokg[GB];
 #pragma unroll
         for (int g = 0; g < GB; g++) {
             const int bl = min(bl0 + g, nbc - 1);        // (a group's tail re-reads the last block and is not stored)
@@ -174,7 +173,7 @@ __device__ __forceinline__ void conv_stage_halo(const conv_args &a, unsigned cha
             const uint8_t *base = a.xq[seg] + ((size_t)n * a.nbs[seg] + min(blk, a.nbs[seg] - 1)) * Sin * rb;
 #pragma unroll
             for (int k = 0; k < NE; k++) {
-                const unsigned vox = eoff[k] >> 1, hf = NH == 2 ? (eoff[k] & 1u) : 0u;
+                const unsigned vox = evox[k];
                 if (WIDE) {                              // every staged tensor has 32-channel blocks: straight-line loads, all in flight together
                     val[g][k] = *(const v4i *)(base + (size_t)vox * (16 * NH) + hf * 16);
                     ok[g][k] = eok[k] && bok;
@@ -190,8 +189,10 @@ __device__ __forceinline__ void conv_stage_halo(const conv_args &a, unsigned cha
                 }
             }
             const uint8_t *sbase = a.xsc[seg] + ((size_t)n * a.nbs[seg] + min(blk, a.nbs[seg] - 1)) * Sin;
+            if (hf == 0) {
 #pragma unroll
-            for (int k = 0; k < NS; k++) sv[g][k] = sbase[soff[k]];
+                for (int k = 0; k < NE; k++) sv[g][k] = sbase[evox[k]];
+            }
         }
 #pragma unroll
         for (int g = 0; g < GB; g++) {
@@ -199,10 +200,12 @@ __device__ __forceinline__ void conv_stage_halo(const conv_args &a, unsigned cha
             if (bl < nbc) {
 #pragma unroll
                 for (int k = 0; k < NE; k++)
-                    if (tid + k * 256 < TT * NH) *(v4i *)(lds + edst[k] + bl * NH * TT * 16) = ok[g][k] ? val[g][k] : (v4i){0, 0, 0, 0};
+                    if (p0 + k * PS < TT) *(v4i *)(lds + act_o + edst[k] + bl * NH * TT * 16) = ok[g][k] ? val[g][k] : (v4i){0, 0, 0, 0};
+                if (hf == 0) {
 #pragma unroll
-                for (int k = 0; k < NS; k++)
-                    if (tid + k * 256 < TT) *(unsigned *)(lds + asc_o + (bl * TT + tid + k * 256) * 4) = sok[k] && bokg[g] ? sv[g][k] : 1u;
+                    for (int k = 0; k < NE; k++)
+                        if (p0 + k * PS < TT) *(unsigned *)(lds + asc_o + (bl * TT + p0 + k * PS) * 4) = eok[k] && bokg[g] ? sv[g][k] : 1u;
+                }
             }
         }
     }
@@ -443,13 +446,11 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     // the lane's voxel in each of its NT tiles: wave -> (z, y half) for TZ 2, z for TZ 4; tile j -> rows 2j, 2j+1; r -> (row, x)
     int lz, ly0;
     if (NT == 2) { lz = wave >> 1; ly0 = (wave & 1) * 4; } else { lz = wave; ly0 = 0; }
-    unsigned ab[NT], sbse[NT];     // LDS byte addresses of the lane's halo row (its 16-byte half) and scale word for tap (0, 0, 0) of block 0
-#pragma unroll
-    for (int j = 0; j < NT; j++) {
-        const int p0 = ((STRIDE * lz) * HY + STRIDE * (ly0 + 2 * j + (r >> 4))) * HX + STRIDE * (r & 15);
-        ab[j] = act_o + ((NH == 2 ? h * TT : 0) + p0) * 16;
-        sbse[j] = asc_o + p0 * 4;
-    }
+    // LDS byte addresses of the lane's halo row (its 16-byte half) and scale word for tap (0, 0, 0) of block 0, first voxel tile; tile j
+    // lies 2 STRIDE halo rows further: a constant the loads carry in their offset field
+    const int p00 = ((STRIDE * lz) * HY + STRIDE * (ly0 + (r >> 4))) * HX + STRIDE * (r & 15);
+    const unsigned ab0 = act_o + ((NH == 2 ? h * TT : 0) + p00) * 16, sb0 = asc_o + p00 * 4;
+    constexpr unsigned ABJ = 2 * STRIDE * HX * 16, SBJ = 2 * STRIDE * HX * 4;
     const unsigned wfa = wring_o + lane * 16, wfs = wring_o + MT * WTILE + lane * 4;    // the lane's weight fragment / scale word of the ring's first pair, tile 0
 
     v16f acc[MT][NT];
@@ -511,12 +512,12 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
             const v4i t = T;
 #pragma unroll
             for (int j = 0; j < NT; j++) {
-                const v4i lo = *(const v4i *)(lds + ab[j] + t[0]);
+                const v4i lo = *(const v4i *)(lds + (ab0 + t[0]) + j * ABJ);
                 if (FMT == 8) {
-                    const v4i hi = *(const v4i *)(lds + ab[j] + t[1]);
+                    const v4i hi = *(const v4i *)(lds + (ab0 + t[1]) + j * ABJ);
                     fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 } else fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                sb[j] = *(const int *)(lds + sbse[j] + t[2]);
+                sb[j] = *(const int *)(lds + (sb0 + t[2]) + j * SBJ);
             }
 #pragma unroll
             for (int m = 0; m < MT; m++) {
