@@ -47,6 +47,8 @@ typedef struct {
     int attn_pe;               /* 1 axial 3-D RoPE, 2 none (0 PEG and 3 scroll RoPE are not provided) */
     int attn_reg;              /* register tokens per sample */
     int attn_mlp;              /* SwiGLU hidden width (0: 8/3 of the width rounded up to 32) */
+    int down_norm;             /* 1: GroupNorm + SiLU after each stride-2 down conv, applied by the next block's conv1 while it stages its input
+                                  (parameters after the head, src/unet.h:23, src/unet.c:459); 0: the older layout without it */
 } unet_cfg;
 typedef struct unet unet;
 unet *unet_create(const unet_cfg *cfg, shape5 in);             /* in: the window (n, cin, d, h, w); dims divisible by 2^(nlev-1) */
@@ -62,6 +64,16 @@ int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const flo
 const void *unet_layer_out(const unet *u, int k, shape5 *s, const char **name);
 /* the GroupNorm statistics the k-th conv produced (device [n * G] each); returns G, 0 when the layer has none */
 int unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd);
+/* ---- checkpoints in the reference's format (src/unet.c:5534-5650 unet_save, :5650-5700 read_header, :5774-5800 unet_load): one line
+   "UFSM{json}\n", then nparams fp32 weights, the EMA weights and optionally optimizer state. unet_read_header fills cfg (act_dt 8, prec 0)
+   from the header's architecture keys; it returns 0, -1 when the file is unreadable, or -2 naming (stderr) a feature of the checkpoint this
+   build does not run (decoder widths, residual blocks, latent grids, deep supervision, FiLM, fine stems, running-statistics norms, the
+   attention stage's other forms). unet_load / unet_load_ema copy the weights / the EMA weights into a net of the same architecture
+   (checked: nlev, widths, cin, cout, attention blocks, nparams, payload size); unet_save writes weights and EMA (= the weights). ---- */
+int unet_read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step);
+int unet_load(unet *u, const char *path);
+int unet_load_ema(unet *u, const char *path);
+int unet_save(const unet *u, const char *path, int step, const char *extra);   /* extra: a JSON object for the header's "extra" key, or null */
 shape5 unet_in_shape(const unet *u);                          /* the window the graph was created for */
 const unet_cfg *unet_config(const unet *u);
 /* ---- sliding-window prediction of a volume resident in device memory (src/predict.c: the --feather single pass, :282-333, :2538-2545,

@@ -59,7 +59,7 @@ def test_host_library_exports_every_declared_symbol():
     assert "unet_forward_x" in names and "nn_conv3d_fwd_x" in names and "nn_set_storage" in names and "unet_predict_volume" in names
     for n in names:
         assert hasattr(H, n), "libufsm_host.so does not export %s" % n
-    assert C.sizeof(unet.unet_cfg) == 4 * (2 + unet.UNET_MAXLEV + 4 + 4)
+    assert C.sizeof(unet.unet_cfg) == 4 * (2 + unet.UNET_MAXLEV + 4 + 4 + 1)
 
 
 def test_descriptor_layouts():

@@ -1,0 +1,42 @@
+"""The checkpoint header reader on headers as the reference writes them (src/unet.c:5546-5640): host-only, no GPU."""
+import ctypes as C
+
+import pytest
+
+
+def read(tmp_path, header, payload=b""):
+    from ufsm_amd.unet import load_host, unet_cfg
+    H = load_host()
+    p = tmp_path / "h.ckpt"
+    p.write_bytes(header.encode() + payload)
+    cfg = unet_cfg(); n = C.c_size_t(0); step = C.c_int(0)
+    rc = H.unet_read_header(str(p).encode(), C.byref(cfg), C.byref(n), C.byref(step))
+    return rc, cfg, n.value, step.value
+
+
+def test_reads_the_reference_header(tmp_path):
+    # the test net of tests/test_predict_feather.c:73-76 as unet_save writes it (keys in its order, the caller's runtime object as extra)
+    h = ('UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":287937,"step":1,"sparse24":0,"wq":0,"muon_mom":0,'
+         '"extra":{"runtime":{"version":1,"train_window":96,"prec":1,"f16":1,"act_mx4":0,"act_mx8":1,"grad_mx8":1,"input_mx":1,"input_prec":8,"gn_stored":0,"policy":"","optimizer":"muon"}}}\n')
+    rc, cfg, n, step = read(tmp_path, h)
+    assert rc == 0 and (cfg.nlev, cfg.widths[0], cfg.widths[1], cfg.cin, cfg.head_out, cfg.G, cfg.down_norm, cfg.attn_blocks, cfg.act_dt) == (2, 32, 64, 4, 1, 8, 1, 0, 8)
+    assert n == 287937 and step == 1
+
+
+def test_attention_keys_and_extra_shadowing(tmp_path):
+    h = ('UFSM{"nlev":4,"widths":[32,64,128,192],"attn_blocks":2,"attn_pe":1,"attn_reg":4,"attn_mlp":512,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,'
+         '"nparams":5,"step":77,"sparse24":0,"wq":0,"muon_mom":0,"extra":{"nlev":9,"film":3}}\n')
+    rc, cfg, n, step = read(tmp_path, h)                                 # keys inside the caller's extra object do not count
+    assert rc == 0 and (cfg.nlev, cfg.widths[3], cfg.attn_blocks, cfg.attn_pe, cfg.attn_reg, cfg.attn_mlp) == (4, 192, 2, 1, 4, 512) and step == 77
+
+
+@pytest.mark.parametrize("feature", ['"dec_widths":[0,32]', '"half_res":1', '"ds_levels":2', '"film":2', '"fstem":[2,16]', '"gn_ema":1,"ge_n":5', '"attn_vres":1', '"l0_norm":2'])
+def test_refuses_architectures_it_does_not_run(tmp_path, feature):
+    h = 'UFSM{"nlev":2,"widths":[32,64],%s,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":1,"extra":{}}\n' % feature
+    assert read(tmp_path, h)[0] == -2
+
+
+def test_rejects_foreign_files(tmp_path):
+    assert read(tmp_path, "not a checkpoint\n")[0] == -1
+    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"scale_cond":1,"nparams":1}\n')[0] == -2      # voxel-size conditioning
+    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":0,"attn_reg":0,"attn_mlp":256,"cin":4,"cout":1,"nparams":1}\n')[0] == -2   # PEG

@@ -19,16 +19,17 @@ def ct_like(rng, N, D, H, W):
     return np.clip(np.where(sheet, rng.normal(170, 20, f.shape), rng.normal(60, 20, f.shape)), 0, 255).astype(np.uint8)
 
 
-@pytest.mark.parametrize("bits,widths,dims,N", [(8, [32, 64], (8, 16, 16), 2), (8, [32, 64, 128], (16, 16, 32), 1), (4, [32, 64], (8, 16, 16), 1), (8, [16, 32], (8, 8, 16), 1)])
-def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N):
+@pytest.mark.parametrize("bits,widths,dims,N,dn", [(8, [32, 64], (8, 16, 16), 2, 0), (8, [32, 64, 128], (16, 16, 32), 1, 0), (4, [32, 64], (8, 16, 16), 1, 0), (8, [16, 32], (8, 8, 16), 1, 0),
+                                                      (8, [32, 64, 128], (16, 16, 16), 1, 1)])
+def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N, dn):
     from ufsm_amd.unet import UNet, make_cfg
     rng = np.random.default_rng(sum(widths) + bits)
     D, H, W = dims
     S = D * H * W
     cin, head_out, G = 4, 8, 8
-    net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits), N, D, H, W, seed=7)
+    net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits, down_norm=dn), N, D, H, W, seed=7)
     p = net.params()
-    lay, n = unet_ref.param_layout(cin, widths, head_out)
+    lay, n = unet_ref.param_layout(cin, widths, head_out, dn)
     assert n == p.size
     w0 = p[lay["enc0.c1.w"][0]:lay["enc0.c1.w"][0] + 1000]
     assert abs(w0.std() / np.sqrt(2.0 / (cin * 27)) - 1) < 0.1                    # Kaiming normal (src/unet.c:588-593)
@@ -70,7 +71,7 @@ def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N):
     Pm = lambda key: np.ascontiguousarray(p[lay[key][0]:lay[key][0] + int(np.prod(lay[key][1]))].reshape(lay[key][1]))
 
     def gn_of(layer):
-        nm = unet_ref.norm_of(layer)
+        nm = unet_ref.norm_of(layer, dn)
         if nm is None:
             return None
         g, m, r = stat[layer]
@@ -95,6 +96,13 @@ def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N):
             mo = np.zeros(N * g, np.float32); ro = np.zeros(N * g, np.float32)
             orc.lib().orc_gn_finalize(orc.ptr(sums), N * g, (co // g) * d_ * h_ * w_, 1e-5, orc.ptr(mo), orc.ptr(ro))
             assert np.allclose(m, mo, rtol=2e-3, atol=2e-4) and np.allclose(r, ro, rtol=2e-3), name
+        elif dn:                                                   # down_norm: statistics of the device's own stored down-conv output
+            g, m, r = stat[name]
+            sd = np.zeros((N, g, 2), np.float64)
+            orc.lib().orc_gn_sums_mx(bits, orc.ptr(tens[name]), N, co, g, d_ * h_ * w_, orc.ptr(sd), 0, d_ * h_ * w_)
+            mo = np.zeros(N * g, np.float32); ro = np.zeros(N * g, np.float32)
+            orc.lib().orc_gn_finalize(orc.ptr(sd), N * g, (co // g) * d_ * h_ * w_, 1e-5, orc.ptr(mo), orc.ptr(ro))
+            assert np.allclose(m, mo, rtol=1e-4, atol=1e-5) and np.allclose(r, ro, rtol=1e-4), name
     last = "dec0.c2" if len(widths) > 1 else "enc0.c2"
     hw = np.ascontiguousarray(Pm("head.w").reshape(head_out, widths[0])); hb = Pm("head.b")
     want_h = np.zeros((N, head_out, S), np.float32)
@@ -104,7 +112,7 @@ def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N):
     # codes of the next, so two correct evaluations with different fp32 summation orders drift apart to the level of the format's own
     # rounding noise (e4m3: 2^-4 relative per element) and stay there; the reference accepts 0.06-0.08 relative L2 per fp8 op
     # (tests/test_mx.c:32, :44). Bound the drift by that level; exact-operand networks (below) agree bit for bit. ----
-    want, outs = unet_ref.forward(p, cin, widths, G, head_out, bits, xq, N, D, H, W)
+    want, outs = unet_ref.forward(p, cin, widths, G, head_out, bits, xq, N, D, H, W, down_norm=dn)
     rel_l2 = np.linalg.norm(got - want) / np.linalg.norm(want)
     assert rel_l2 < (0.08 if bits == 8 else 0.3), rel_l2
     net.close()
@@ -189,3 +197,41 @@ def test_unet_attention_stage(gpu):
     assert rel < 0.05, rel                                                   # two blocks of MX re-quantisations apart, then one e4m3 rounding
     assert np.linalg.norm(got - xb) / np.linalg.norm(xb) > 0.05              # and the stage did change the tensor
     plain.close(); att.close()
+
+
+def test_checkpoint_round_trip(gpu, tmp_path):
+    """unet_save -> unet_read_header -> unet_create -> unet_load gives the same network: identical parameters and byte-identical logits;
+    a network of another architecture, a truncated payload and a checkpoint of an unsupported feature are refused (src/unet.c:5774-5800)."""
+    import ctypes as C
+    from ufsm_amd.unet import UNet, make_cfg, unet_cfg, load_host
+    H_ = load_host()
+    rng = np.random.default_rng(21)
+    N, D = 1, 16; S = D ** 3
+    cfg = make_cfg(4, [32, 96], head_out=3, attn_blocks=1, attn_pe=1, attn_reg=2, down_norm=1)
+    a = UNet(cfg, N, D, D, D, seed=9)
+    pa = a.params(); pa += (0.01 * rng.standard_normal(pa.size)).astype(np.float32); a.set_params(pa)
+    path = str(tmp_path / "net.ckpt")
+    assert a.save(path, step=123, extra='{"runtime":{"version":1,"note":"nlev\\":99"}}') == 0
+    head = open(path, "rb").readline().decode()
+    assert head.startswith('UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":1,"attn_reg":2,"attn_mlp":256,"cin":4,"cout":3,"G":8,"down_norm":1,"scale_cond":0,"nparams":%d,"step":123,' % pa.size)
+    assert head.rstrip().endswith('}}}')
+    import os
+    assert os.path.getsize(path) == len(head.encode()) + 2 * 4 * pa.size                     # weights + EMA weights
+    c2 = unet_cfg(); npar = C.c_size_t(0); step = C.c_int(0)
+    assert H_.unet_read_header(path.encode(), C.byref(c2), C.byref(npar), C.byref(step)) == 0
+    assert (c2.nlev, list(c2.widths[:2]), c2.cin, c2.head_out, c2.G, c2.down_norm, c2.attn_blocks, c2.attn_pe, c2.attn_reg, c2.attn_mlp) == (2, [32, 96], 4, 3, 8, 1, 1, 1, 2, 256)
+    assert npar.value == pa.size and step.value == 123
+    b = UNet(c2, N, D, D, D, seed=1)
+    assert b.load(path) == 0 and np.array_equal(b.params(), pa) and b.load(path, ema=True) == 0
+    x = rng.standard_normal((N, 4, S)).astype(np.float32); dxq = to_mx(8, x)
+    la, lb = DevBuf(N * 3 * S * 4), DevBuf(N * 3 * S * 4)
+    assert a.forward_x(dxq.ptr, la.ptr) == 0 and b.forward_x(dxq.ptr, lb.ptr) == 0
+    LP.check()
+    assert np.array_equal(la.to_numpy(np.float32), lb.to_numpy(np.float32))
+    other = UNet(make_cfg(4, [32, 96], head_out=3, down_norm=1), N, D, D, D, seed=1)        # no attention blocks: refused
+    assert other.load(path) == -1
+    open(str(tmp_path / "cut.ckpt"), "wb").write(open(path, "rb").read()[:-8])
+    assert b.load(str(tmp_path / "cut.ckpt")) == -1
+    open(str(tmp_path / "film.ckpt"), "wb").write(head.replace(',"cin":', ',"film":2,"cin":').encode() + b"\0" * (8 * pa.size))
+    assert H_.unet_read_header(str(tmp_path / "film.ckpt").encode(), C.byref(c2), None, None) == -2
+    a.close(); b.close(); other.close()

@@ -5,7 +5,7 @@ import numpy as np
 import orc
 
 
-def param_layout(cin, widths, head_out):
+def param_layout(cin, widths, head_out, down_norm=0):
     L = len(widths); off = 0; lay = {}
 
     def conv(name, ci, co, k):
@@ -27,12 +27,15 @@ def param_layout(cin, widths, head_out):
         conv("dec%d.c1" % i, widths[i + 1] + widths[i], widths[i], 3); gn("dec%d.n1" % i, widths[i])
         conv("dec%d.c2" % i, widths[i], widths[i], 3); gn("dec%d.n2" % i, widths[i])
     conv("head", widths[0], head_out, 1)
+    if down_norm:                                    # GroupNorm after each down conv, appended after the head (src/unet.c:459)
+        for i in range(L - 1):
+            gn("dn%d" % i, widths[i])
     return lay, off
 
 
-def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0):
+def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0):
     """xq: MX bytes of the input. Returns (logits fp32 [N][head_out][S], {layer name: MX bytes})."""
-    lay, n = param_layout(cin, widths, head_out)
+    lay, n = param_layout(cin, widths, head_out, down_norm)
     assert params.size == n
     P = lambda k: np.ascontiguousarray(params[lay[k][0]:lay[k][0] + int(np.prod(lay[k][1]))].reshape(lay[k][1]))
     L = len(widths); dt = 3 if bits == 8 else 4
@@ -56,17 +59,23 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
         outs[name] = y
         return y, s
 
-    cur, blocks = xq, {}
+    cur, blocks, gin = xq, {}, None
     for i in range(L):
         ci = widths[i - 1] if i else cin
         S = dims[i][0] * dims[i][1] * dims[i][2]
-        a1, s1 = conv("enc%d.c1" % i, cur, ci, dims[i])
+        a1, s1 = conv("enc%d.c1" % i, cur, ci, dims[i], gp=gin)
         m1, r1 = finalize(s1, widths[i], S)
         a2, s2 = conv("enc%d.c2" % i, a1, widths[i], dims[i], gp=orc.gn(P("enc%d.n1.gamma" % i), P("enc%d.n1.beta" % i), m1, r1, Gof(widths[i])))
         m2, r2 = finalize(s2, widths[i], S)
         blocks["enc%d" % i] = (a2, orc.gn(P("enc%d.n2.gamma" % i), P("enc%d.n2.beta" % i), m2, r2, Gof(widths[i])), (m2, r2))
         if i < L - 1:
             cur, _ = conv("down%d" % i, a2, widths[i], dims[i], gp=blocks["enc%d" % i][1], stride=2, stats=False)
+            if down_norm:                     # statistics of the stored down-conv output, applied by the next conv1 (src/unet.c:2974-2979)
+                Sd = dims[i + 1][0] * dims[i + 1][1] * dims[i + 1][2]; g = Gof(widths[i])
+                sums = np.zeros((N, g, 2), np.float64)
+                orc.lib().orc_gn_sums_mx(bits, orc.ptr(cur), N, widths[i], g, Sd, orc.ptr(sums), 0, Sd)
+                md, rd = finalize(sums, widths[i], Sd)
+                gin = orc.gn(P("dn%d.gamma" % i), P("dn%d.beta" % i), md, rd, g)
     for i in range(L - 2, -1, -1):
         coarse = blocks["enc%d" % (L - 1)] if i == L - 2 else blocks["dec%d" % (i + 1)]
         skip = blocks["enc%d" % i]
@@ -100,9 +109,12 @@ def layer_inputs(widths):
     return g
 
 
-def norm_of(layer):
-    """the GroupNorm parameters applied to a conv output by its readers: block.c1 -> block.n1, block.c2 -> block.n2; down convs: none."""
-    if layer.startswith("down") or layer == "input":
+def norm_of(layer, down_norm=0):
+    """the GroupNorm parameters applied to a conv output by its readers: block.c1 -> block.n1, block.c2 -> block.n2; down convs: none,
+    or dn<i> with down_norm."""
+    if layer.startswith("down"):
+        return "dn" + layer[4:] if down_norm else None
+    if layer == "input":
         return None
     blk, c = layer.split(".")
     return blk + (".n1" if c == "c1" else ".n2")

@@ -24,6 +24,7 @@ struct unet {
     block enc[UNET_MAXLEV], dec[UNET_MAXLEV];
     convp down[UNET_MAXLEV], head;
     void *downo[UNET_MAXLEV];
+    gnpar dn[UNET_MAXLEV]; float *dm[UNET_MAXLEV], *dr[UNET_MAXLEV];   /* down_norm: GroupNorm after down[i], its statistics */
     size_t np; float *params;                                      /* device */
     void *xin;                                                     /* the network input built from a CT window */
     struct { const void *p; shape5 s; const char *name; const float *mean, *rstd; int G; } outs[64]; int nouts;
@@ -63,6 +64,7 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
         off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
     }
     off = add_conv(&u->head, w[0], cfg->head_out, 1, off);
+    if (cfg->down_norm) for (int i = 0; i < L - 1; i++) off = add_gn(&u->dn[i], w[i], off);       /* (appended after the head, src/unet.c:459) */
     if (cfg->attn_blocks > 0) {                                   /* parameters last: registers, then the blocks (src/unet.c:490-499) */
         const int C = w[L - 1];
         if (C % AT_HD || cfg->attn_blocks > 16 || (cfg->attn_pe != 1 && cfg->attn_pe != 2) || cfg->attn_reg < 0) {
@@ -87,7 +89,10 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
             const size_t ng = (size_t)in.n * G_of(u, w[i]);
             b->m1 = f32_new(ng); b->r1 = f32_new(ng); b->m2 = f32_new(ng); b->r2 = f32_new(ng);
         }
-        if (i < L - 1) { shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds); }
+        if (i < L - 1) {
+            shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds);
+            if (cfg->down_norm) { const size_t ng = (size_t)in.n * G_of(u, w[i]); u->dm[i] = f32_new(ng); u->dr[i] = f32_new(ng); }
+        }
     }
     u->xin = act_new(u, in);
     if (u->tbn) {
@@ -106,7 +111,7 @@ void unet_free(unet *u) {
     mi_sync();
     for (int i = 0; i < UNET_MAXLEV; i++) {
         for (int s = 0; s < 2; s++) { block *b = s ? &u->dec[i] : &u->enc[i]; act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2); }
-        act_del(u->downo[i]);
+        act_del(u->downo[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
     }
     if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); }
     act_del(u->xin); mi_free(u->params);
@@ -135,6 +140,7 @@ void unet_init(unet *u, uint64_t seed) {
     for (int i = 0; i < L - 1; i++) init_conv(h, &u->down[i], &seed, 0);
     for (int i = 0; i < L - 1; i++) { init_conv(h, &u->dec[i].c1, &seed, 0); init_gn(h, &u->dec[i].n1); init_conv(h, &u->dec[i].c2, &seed, 0); init_gn(h, &u->dec[i].n2); }
     init_conv(h, &u->head, &seed, -2.0);
+    if (u->cfg.down_norm) for (int i = 0; i < L - 1; i++) init_gn(h, &u->dn[i]);
     if (u->tbn) {   /* LayerNorm and QK-norm gains 1, QKV and MLP-in N(0, 1 / C), out projections and biases 0 (identity blocks), registers N(0, 0.02^2) (src/unet.c:612-642) */
         const int C = u->tbd.C, F = u->tbd.F; const double sd = 1.0 / sqrt((double)C);
         for (int k = 0; k < u->tbn; k++) {
@@ -195,12 +201,17 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
     u->nouts = 0;
     const void *cur = x;
     for (int i = 0; i < L; i++) {
-        if (block_fwd(u, &u->enc[i], cur, nullptr, nullptr, nullptr, 0, en1[i], en2[i])) { if (reg_here) nn_storage_forget(x); return -1; }
+        nn_gn_t gd; const nn_gn_t *gin = nullptr;                  /* down_norm: conv1 reads silu(gn(down conv output)) (src/unet.c:2593) */
+        if (i && u->cfg.down_norm) { gd = (nn_gn_t){P(u, u->dn[i - 1].gamma), P(u, u->dn[i - 1].beta), u->dm[i - 1], u->dr[i - 1], G_of(u, u->cfg.widths[i - 1])}; gin = &gd; }
+        if (block_fwd(u, &u->enc[i], cur, gin, nullptr, nullptr, 0, en1[i], en2[i])) { if (reg_here) nn_storage_forget(x); return -1; }
         if (i < L - 1) {                                           /* stride-2 down conv of silu(gn(a2)), width kept (src/unet.c:2970) */
             const nn_gn_t g = gn_out(u, &u->enc[i]);
             if (nn_conv3d_fwd_x(u->enc[i].a2, &g, nullptr, nullptr, 0, 0, u->enc[i].ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
             shape5 ds = u->ls[i + 1]; ds.c = u->cfg.widths[i];
-            note(u, u->downo[i], ds, dwn[i], nullptr, nullptr, 0);
+            if (u->cfg.down_norm) {                                /* statistics of the stored down-conv output now, the transform in the next conv1's staging (src/unet.c:2974-2979) */
+                if (nn_gn_stats(u->downo[i], ds, G_of(u, ds.c), 1e-5f, u->dm[i], u->dr[i])) { fprintf(stderr, "unet: down_norm GroupNorm statistics unsupported for this storage\n"); return -1; }
+                note(u, u->downo[i], ds, dwn[i], u->dm[i], u->dr[i], G_of(u, ds.c));
+            } else note(u, u->downo[i], ds, dwn[i], nullptr, nullptr, 0);
             cur = u->downo[i];
         }
     }
@@ -234,4 +245,105 @@ const void *unet_layer_out(const unet *u, int k, shape5 *s, const char **name) {
     if (s) *s = u->outs[k].s;
     if (name) *name = u->outs[k].name;
     return u->outs[k].p;
+}
+
+
+/* ---- checkpoints (the reference's file format: src/unet.c:5534-5650, :5650-5700, :5774-5800) ---- */
+static char *header_line(FILE *f) {                                /* the first line without its newline (malloc'ed), the stream left after it */
+    size_t cap = 1 << 16, n = 0; char *s = malloc(cap);
+    for (int c; s && (c = fgetc(f)) != EOF;) {
+        if (c == '\n') { s[n] = 0; return s; }
+        if (n + 2 > cap) { if (cap >= (1u << 22)) break; cap *= 2; char *t = realloc(s, cap); if (!t) break; s = t; }
+        s[n++] = (char)c;
+    }
+    free(s); return nullptr;
+}
+static int key_int(const char *line, const char *key, int dflt) { const char *p = strstr(line, key); return p ? atoi(p + strlen(key)) : dflt; }
+int unet_read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step) {
+    FILE *f = fopen(path, "rb");
+    if (!f) return -1;
+    char *line = header_line(f); fclose(f);
+    if (!line || strncmp(line, "UFSM{", 5)) { free(line); return -1; }
+    char *ex = strstr(line, ",\"extra\":"); if (ex) *ex = 0;       /* (the caller's object may repeat key names) */
+    memset(cfg, 0, sizeof *cfg);
+    cfg->nlev = key_int(line, "\"nlev\":", 0);
+    const char *p = strstr(line, "\"widths\":[");
+    if (cfg->nlev < 1 || cfg->nlev > UNET_MAXLEV || !p) { free(line); return -1; }
+    p += 10;
+    for (int i = 0; i < cfg->nlev; i++) { cfg->widths[i] = atoi(p); p = strchr(p, ','); if (!p) break; p++; }
+    cfg->cin = key_int(line, "\"cin\":", 0); cfg->head_out = key_int(line, "\"cout\":", 0); cfg->G = key_int(line, "\"G\":", 8);
+    cfg->down_norm = key_int(line, "\"down_norm\":", 0);
+    cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
+    cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
+    cfg->act_dt = 8; cfg->prec = 0;
+    if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
+    if (step) *step = key_int(line, "\"step\":", 0);
+    /* architecture features this build's graph does not have */
+    static const char *const no[] = {"\"dec_widths\":", "\"enc_blocks\":", "\"half_res\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"w4_2d\":", "\"ds_levels\":", "\"emb_lev\":",
+                                     "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
+                                     "\"l0_norm\":", "\"scan_norm\":", "\"skip_empty\":", "\"gfilm\":", "\"gn_ema\":", "\"dec_convs\":"};
+    const char *bad = nullptr;
+    for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
+    if (!bad && key_int(line, "\"scale_cond\":", 0)) bad = "\"scale_cond\":";
+    if (!bad && cfg->attn_blocks && cfg->attn_pe != 1 && cfg->attn_pe != 2) bad = "\"attn_pe\": (PEG / scroll RoPE)";
+    if (bad) { fprintf(stderr, "unet_read_header: %s uses %s which this build does not run\n", path, bad); free(line); return -2; }
+    free(line);
+    return cfg->cin > 0 && cfg->head_out > 0 ? 0 : -1;
+}
+static int load_array(unet *u, const char *path, int which) {
+    unet_cfg c; size_t np = 0; int step = 0;
+    const int r = unet_read_header(path, &c, &np, &step);
+    if (r) { if (r == -1) fprintf(stderr, "unet_load: %s: unreadable header\n", path); return -1; }
+    const unet_cfg *m = &u->cfg; const char *bad = nullptr;
+    if (c.nlev != m->nlev) bad = "nlev";
+    for (int i = 0; !bad && i < m->nlev; i++) if (c.widths[i] != m->widths[i]) bad = "widths";
+    if (!bad && c.cin != m->cin) bad = "cin";
+    if (!bad && c.head_out != m->head_out) bad = "cout";
+    if (!bad && c.attn_blocks != m->attn_blocks) bad = "attn_blocks";
+    if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
+    if (!bad && np != u->np) bad = "nparams";
+    if (bad) { fprintf(stderr, "unet_load: %s: \"%s\" differs from this network's\n", path, bad); return -1; }
+    FILE *f = fopen(path, "rb");
+    if (!f) return -1;
+    char *line = header_line(f); free(line);
+    const long off = ftell(f);
+    fseek(f, 0, SEEK_END);
+    const long long have = (long long)ftell(f) - off, a = 4ll * (long long)np;
+    if (have != 2 * a && have != 4 * a && have != 5 * a) {         /* weights + EMA, + AdamW moments, + Muon momentum (src/unet.c:5782-5790) */
+        fprintf(stderr, "unet_load: %s: %lld payload bytes, the header (nparams %zu) needs 2, 4 or 5 arrays of %lld: truncated or not a checkpoint of this format\n", path, have, np, a);
+        fclose(f); return -1;
+    }
+    float *h = malloc((size_t)a);
+    int rc = -1;
+    if (h && !fseek(f, off + (long)(which ? a : 0), SEEK_SET) && fread(h, 4, np, f) == np) {
+        size_t nbad = 0; for (size_t i = 0; i < np; i++) nbad += !isfinite(h[i]);
+        if (nbad) fprintf(stderr, "unet_load: %s: %zu non-finite values\n", path, nbad);
+        else { unet_set_params(u, h); rc = 0; }
+    }
+    free(h); fclose(f);
+    return rc;
+}
+int unet_load(unet *u, const char *path) { return load_array(u, path, 0); }
+int unet_load_ema(unet *u, const char *path) { return load_array(u, path, 1); }
+int unet_save(const unet *u, const char *path, int step, const char *extra) {
+    float *h = malloc(u->np * 4);
+    if (!h) return -1;
+    unet_get_params(u, h);
+    if (nn_check()) { fprintf(stderr, "unet_save: a device error is latched: %s not written\n", path); free(h); return -1; }
+    for (size_t i = 0; i < u->np; i++) if (!isfinite(h[i])) { fprintf(stderr, "unet_save: non-finite weights (first at parameter %zu): %s not written\n", i, path); free(h); return -2; }
+    char tmp[1400]; snprintf(tmp, sizeof tmp, "%s.tmp", path);
+    FILE *f = fopen(tmp, "wb");
+    if (!f) { fprintf(stderr, "unet_save: cannot create %s\n", tmp); free(h); return -1; }
+    fprintf(f, "UFSM{\"nlev\":%d,\"widths\":[", u->cfg.nlev);
+    for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.widths[i]);
+    fputc(']', f);
+    if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
+    fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":0,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.head_out, u->cfg.G,
+            u->cfg.down_norm, u->np, step);
+    fprintf(f, ",\"extra\":%s}\n", extra ? extra : "{}");
+    int ok = fwrite(h, 4, u->np, f) == u->np && fwrite(h, 4, u->np, f) == u->np;      /* weights, EMA weights */
+    ok = !fclose(f) && ok;
+    free(h);
+    if (!ok || rename(tmp, path)) { fprintf(stderr, "unet_save: write error on %s\n", tmp); remove(tmp); return -1; }
+    return 0;
 }

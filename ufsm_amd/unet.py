@@ -13,7 +13,7 @@ UNET_MAXLEV = 8
 
 class unet_cfg(C.Structure):
     _fields_ = [("cin", C.c_int), ("nlev", C.c_int), ("widths", C.c_int * UNET_MAXLEV), ("G", C.c_int), ("head_out", C.c_int),
-                ("act_dt", C.c_int), ("prec", C.c_int), ("attn_blocks", C.c_int), ("attn_pe", C.c_int), ("attn_reg", C.c_int), ("attn_mlp", C.c_int)]
+                ("act_dt", C.c_int), ("prec", C.c_int), ("attn_blocks", C.c_int), ("attn_pe", C.c_int), ("attn_reg", C.c_int), ("attn_mlp", C.c_int), ("down_norm", C.c_int)]
 
 
 _host = None
@@ -45,6 +45,10 @@ def load_host():
     L.nn_check.restype = C.c_char_p
     L.unet_in_shape.restype = shape5; L.unet_in_shape.argtypes = [C.c_void_p]
     L.unet_config.restype = C.POINTER(unet_cfg); L.unet_config.argtypes = [C.c_void_p]
+    L.unet_read_header.restype = C.c_int; L.unet_read_header.argtypes = [C.c_char_p, C.POINTER(unet_cfg), C.POINTER(C.c_size_t), C.POINTER(C.c_int)]
+    L.unet_load.restype = C.c_int; L.unet_load.argtypes = [C.c_void_p, C.c_char_p]
+    L.unet_load_ema.restype = C.c_int; L.unet_load_ema.argtypes = [C.c_void_p, C.c_char_p]
+    L.unet_save.restype = C.c_int; L.unet_save.argtypes = [C.c_void_p, C.c_char_p, C.c_int, C.c_char_p]
     L.unet_predict_volume.restype = C.c_int
     L.unet_predict_volume.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.c_int, C.c_int, C.c_float, C.c_float, C.c_int, C.c_float, C.c_float,
                                       C.c_void_p, C.POINTER(C.c_int64)]
@@ -52,10 +56,10 @@ def load_host():
     return L
 
 
-def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0):
+def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0):
     c = unet_cfg()
     c.cin, c.nlev, c.G, c.head_out, c.act_dt, c.prec = cin, len(widths), G, head_out, act_dt, prec
-    c.attn_blocks, c.attn_pe, c.attn_reg, c.attn_mlp = attn_blocks, attn_pe, attn_reg, attn_mlp
+    c.attn_blocks, c.attn_pe, c.attn_reg, c.attn_mlp, c.down_norm = attn_blocks, attn_pe, attn_reg, attn_mlp, down_norm
     for i, w in enumerate(widths):
         c.widths[i] = w
     return c
@@ -94,6 +98,12 @@ class UNet:
         d = (C.c_int64 * 3)(*dims); nw = (C.c_int64 * 2)(0, 0)
         rc = self.L.unet_predict_volume(self.h, vol_ptr, d, halo, feather, mean, isd, axis, cy, cx, out_ptr, nw)
         return rc, nw[0], nw[1]
+
+    def save(self, path, step=0, extra=None):
+        return self.L.unet_save(self.h, path.encode(), step, extra.encode() if extra else None)
+
+    def load(self, path, ema=False):
+        return (self.L.unet_load_ema if ema else self.L.unet_load)(self.h, path.encode())
 
     def layer_outs(self):
         out, k = [], 0
