@@ -385,10 +385,128 @@ int orc_conv3_staged(const orc_conv_t *c, float *out) {
 static float gelu_f(float x) { return 0.5f * x * (1.f + (float)erf((double)x * 0.70710678118654752440)); }
 static float silu_f(float x) { return (float)((double)x / (1.0 + exp(-(double)x))); }
 
+/* epilogue of one output voxel (src/lp_common.cuh:1492-1535): bias, optional fused activation, store in the output type, statistics */
+static void conv_epilogue(const orc_conv_t *c, int n, size_t ov, size_t So, float *acc, const double *acc64, double *ls) {
+    const int Co = c->Co, cpg = c->Go ? Co / c->Go : 1;
+    const int ybits = c->ydt == 3 ? 8 : 4, ybw = orc_mx_bw(Co), ynb = orc_mx_nb(Co), yrb = rowbytes(ybw, ybits);
+    uint8_t *yq = (uint8_t *)c->y, *ysc = yq + (size_t)c->N * ynb * So * yrb;
+    /* epilogue (src/lp_common.cuh:1492-1535) */
+    for (int co = 0; co < Co; co++) {
+        float v = c->acc64 ? (float)(acc64[co] + (c->b ? (double)c->b[co] : 0.0)) : acc[co] + (c->b ? c->b[co] : 0.f);
+        if (c->fused_act) {
+            if (c->ep_a) v = fmaf(v, c->ep_a[co], c->ep_b[co]);
+            v = c->fused_act == 1 ? silu_f(v) : c->fused_act == 2 ? gelu_f(v) : c->fused_act == 3 ? fmaxf(v, 0.f) : v;
+        }
+        acc[co] = v;
+    }
+    if (c->ydt >= 3) {
+        for (int blk = 0; blk < ynb; blk++) {
+            float r[32]; uint8_t codes[32];
+            for (int k = 0; k < ybw; k++) { const int co = blk * ybw + k; r[k] = co < Co ? acc[co] : 0.f; }
+            const size_t ri = ((size_t)n * ynb + blk) * So + ov;
+            const uint8_t sb = orc_store_row(ybits, r, ybw, codes, 0);
+            memcpy(yq + ri * yrb, codes, (size_t)yrb); ysc[ri] = sb;
+            if (ls && c->stored_stats) { float d[32]; orc_load_row(ybits, codes, sb, ybw, d); for (int k = 0; k < ybw; k++) { const int co = blk * ybw + k; if (co < Co) acc[co] = d[k]; } }
+        }
+    } else if (c->ydt == 2) {
+        for (int co = 0; co < Co; co++) {
+            float v = acc[co];
+            if (c->Go > 0 && fabsf(v) > 65504.f) v = copysignf(65504.f, v);   /* sat_h16 (src/lp_common.cuh:465, :1567-1569) */
+            ((uint16_t *)c->y)[((size_t)n * Co + co) * So + ov] = orc_f32_to_h16(v);
+            acc[co] = v;
+        }
+    } else for (int co = 0; co < Co; co++) ((float *)c->y)[((size_t)n * Co + co) * So + ov] = acc[co];
+    if (ls) for (int co = 0; co < Co; co++) { const double v = acc[co]; ls[2 * (co / cpg)] += v; ls[2 * (co / cpg) + 1] += v * v; }
+}
+
+/* ---------- tap-packed small-channel conv (src/lp_f8fwd.cuh:153-177 weights, :178-400 kernel, :601-609 dispatch) ----------
+   Channels padded to CP in {4, 8, 16}; a K block of 32 = 32 / CP taps x CP channels, so a block mixes positions and the activation
+   operand has ONE scale per staged tile: the 4 x 10 x 18 input positions around a 2 x 8 x 16 output tile (tiles on the output grid from
+   the origin). Values outside the volume and channels >= Ci are zeros and take part in nothing; amax ignores NaN (fmaxf). */
+static int conv3_stem(const orc_conv_t *c) {
+    const int Ci = c->Ci, Co = c->Co, D = c->D, H = c->H, W = c->W;
+    if (c->x2 || c->up || c->stride == 2 || c->cbits != 8 || Ci > 16 || (c->xdt != 0 && Ci > 8)) return -2;
+    const int CP = Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK;
+    const size_t S = (size_t)D * H * W;
+    float *wv = (float *)malloc((size_t)NKB * Co * 32 * sizeof(float)), *wsf = (float *)malloc((size_t)NKB * Co * sizeof(float));
+    for (int kb = 0; kb < NKB; kb++) for (int co = 0; co < Co; co++) {            /* prep_w8s_k */
+        float v[32], amax = 0.f;
+        for (int k = 0; k < 32; k++) { const int tap = kb * TPK + k / CP, ci = k % CP; v[k] = ci < Ci && tap < 27 ? c->w[((size_t)co * Ci + ci) * 27 + tap] : 0.f; amax = fmaxf(amax, fabsf(v[k])); }
+        const int e = orc_mx_exp(amax, INVQ8); const float m = orc_exp2i(-e);
+        for (int k = 0; k < 32; k++) wv[((size_t)kb * Co + co) * 32 + k] = orc_dec_e4m3(orc_enc_e4m3(v[k] * m));
+        wsf[(size_t)kb * Co + co] = orc_mx_scale((unsigned)(e + 127));
+    }
+    const int z0 = c->z1 ? c->z0 : 0, z1 = c->z1 ? c->z1 : D;
+    const int ntz = (D + 1) / 2, nty = (H + 7) / 8, ntx = (W + 15) / 16;
+    float *val = (float *)malloc(S * CP * sizeof(float));
+    chab_t tab[32];
+    for (int n = 0; n < c->N; n++) {
+        /* the conv's input values of this sample: val[voxel][CP] (decoded, after GN + SiLU when the input has one) */
+        chan_table(c, n, Ci, (Ci + 31) / 32 * 32, 32, tab);
+        mxt_t t; if (c->xdt >= 3) t = mxt(c->x, c->xdt == 3 ? 8 : 4, c->N, Ci, S);
+#pragma omp parallel for schedule(static)
+        for (int64_t vi = 0; vi < (int64_t)S; vi++) {
+            float r[32] = {0};
+            if (c->xdt >= 3) mx_row32(&t, n, 0, (size_t)vi, r);
+            else for (int k = 0; k < Ci; k++) { const size_t idx = ((size_t)n * Ci + k) * S + (size_t)vi; r[k] = c->xdt == 2 ? orc_h16_to_f32(((const uint16_t *)c->x)[idx]) : ((const float *)c->x)[idx]; }
+            for (int k = 0; k < CP; k++) val[(size_t)vi * CP + k] = k >= Ci ? 0.f : tab[k].g ? orc_act_ab(r[k], tab[k].a, tab[k].b) : r[k];
+        }
+        double *gs = c->osum ? (double *)calloc((size_t)2 * c->Go, sizeof(double)) : NULL;
+#pragma omp parallel
+        {
+            float *acc = (float *)malloc((size_t)Co * sizeof(float)), *bq = (float *)malloc((size_t)720 * CP * sizeof(float));
+            double *acc64 = (double *)malloc((size_t)Co * sizeof(double));
+            double *ls = gs ? (double *)calloc((size_t)2 * c->Go, sizeof(double)) : NULL;
+#pragma omp for schedule(dynamic, 4)
+            for (int ti = 0; ti < ntz * nty * ntx; ti++) {
+                const int tz = ti / (nty * ntx), ty = ti / ntx % nty, tx = ti % ntx;
+                if (2 * tz + 2 <= z0 || 2 * tz >= z1) continue;
+                /* the tile's 720 staged positions, its amax and scale (src/lp_f8fwd.cuh:340-388) */
+                float amax = 0.f;
+                for (int p = 0; p < 720; p++) {
+                    const int gz = 2 * tz - 1 + p / 180, gy = 8 * ty - 1 + p / 18 % 10, gx = 16 * tx - 1 + p % 18;
+                    const int inb = gz >= 0 && gz < D && gy >= 0 && gy < H && gx >= 0 && gx < W;
+                    for (int k = 0; k < CP; k++) { const float v = inb ? val[(((size_t)gz * H + gy) * W + gx) * CP + k] : 0.f; bq[p * CP + k] = v; amax = fmaxf(amax, fabsf(v)); }
+                }
+                const int e = orc_mx_exp(amax, INVQ8); const float m = orc_exp2i(-e); const double sbf = orc_mx_scale((unsigned)(e + 127));
+                for (int i = 0; i < 720 * CP; i++) bq[i] = orc_dec_e4m3(orc_enc_e4m3(bq[i] * m));
+                for (int l = 0; l < 256; l++) {
+                    const int oz = 2 * tz + l / 128, oy = 8 * ty + l / 16 % 8, ox = 16 * tx + l % 16;
+                    if (oz >= D || oy >= H || ox >= W || oz < z0 || oz >= z1) continue;
+                    const int p0 = ((l / 128) * 10 + l / 16 % 8) * 18 + l % 16;            /* staged position of tap (0, 0, 0) */
+                    for (int co = 0; co < Co; co++) { acc[co] = 0.f; acc64[co] = 0.0; }
+                    for (int kb = 0; kb < NKB; kb++)
+                        for (int co = 0; co < Co; co++) {
+                            const float *wr = wv + ((size_t)kb * Co + co) * 32;
+                            double d = 0.0;
+                            for (int k = 0; k < 32; k++) {
+                                const int tap = kb * TPK + k / CP; if (tap >= 27) break;
+                                d += (double)wr[k] * (double)bq[(p0 + (tap / 9) * 180 + (tap / 3 % 3) * 18 + tap % 3) * CP + k % CP];
+                            }
+                            const double blk = d * (double)wsf[(size_t)kb * Co + co] * sbf;
+                            if (c->acc64) acc64[co] += blk; else acc[co] += (float)blk;
+                        }
+                    conv_epilogue(c, n, ((size_t)oz * H + oy) * W + ox, S, acc, acc64, ls);
+                }
+            }
+            if (ls) {
+#pragma omp critical
+                for (int i = 0; i < 2 * c->Go; i++) gs[i] += ls[i];
+                free(ls);
+            }
+            free(acc); free(acc64); free(bq);
+        }
+        if (gs) { for (int i = 0; i < 2 * c->Go; i++) c->osum[(size_t)n * 2 * c->Go + i] += gs[i]; free(gs); }
+    }
+    free(val); free(wv); free(wsf);
+    return 0;
+}
+
 /* ---------- the convolution (src/lp_f8fwd.cuh:52, :114-148; src/lp_common.cuh:1465-1597) ---------- */
 int orc_conv3(const orc_conv_t *c) {
     staged_t st;
     if (c->cbits != 8 && c->cbits != 4) return -2;
+    if (c->stem_tile) return conv3_stem(c);
     if (build_staged(c, &st)) return -1;
     const int Co = c->Co, nch = st.nch, Cip = st.Cip, s = c->stride == 2 ? 2 : 1;
     const int Do = s == 2 ? (c->D - 1) / 2 + 1 : c->D, Ho = s == 2 ? (c->H - 1) / 2 + 1 : c->H, Wo = s == 2 ? (c->W - 1) / 2 + 1 : c->W;   /* src/nn_bwd.cu:132-135 */
@@ -398,10 +516,7 @@ int orc_conv3(const orc_conv_t *c) {
     orc_prep_w(c->cbits, c->w, Co, c->Ci, c->xdt >= 3 ? st.Cx : c->Ci, c->xdt >= 3 ? st.CxP : (c->Ci + 31) / 32 * 32, Cip, wv, ws, NULL);
     float *wsf = (float *)malloc((size_t)27 * Co * nch * sizeof(float));
     for (size_t i = 0; i < (size_t)27 * Co * nch; i++) wsf[i] = orc_mx_scale(ws[i]);
-    const int ybits = c->ydt == 3 ? 8 : 4, ybw = orc_mx_bw(Co), ynb = orc_mx_nb(Co), yrb = rowbytes(ybw, ybits);
-    uint8_t *yq = (uint8_t *)c->y, *ysc = yq + (size_t)c->N * ynb * So * yrb;
     const int z0 = c->z1 ? c->z0 : 0, z1 = c->z1 ? c->z1 : Do;
-    const int cpg = c->Go ? Co / c->Go : 1;
     for (int n = 0; n < c->N; n++) {
         double *gs = c->osum ? (double *)calloc((size_t)2 * c->Go, sizeof(double)) : NULL;
 #pragma omp parallel
@@ -428,34 +543,7 @@ int orc_conv3(const orc_conv_t *c) {
                             if (c->acc64) acc64[co] += blk; else acc[co] += (float)blk;
                         }
                     }
-                /* epilogue (src/lp_common.cuh:1492-1535) */
-                for (int co = 0; co < Co; co++) {
-                    float v = c->acc64 ? (float)(acc64[co] + (c->b ? (double)c->b[co] : 0.0)) : acc[co] + (c->b ? c->b[co] : 0.f);
-                    if (c->fused_act) {
-                        if (c->ep_a) v = fmaf(v, c->ep_a[co], c->ep_b[co]);
-                        v = c->fused_act == 1 ? silu_f(v) : c->fused_act == 2 ? gelu_f(v) : c->fused_act == 3 ? fmaxf(v, 0.f) : v;
-                    }
-                    acc[co] = v;
-                }
-                const size_t ov = (size_t)vi;
-                if (c->ydt >= 3) {
-                    for (int blk = 0; blk < ynb; blk++) {
-                        float r[32]; uint8_t codes[32];
-                        for (int k = 0; k < ybw; k++) { const int co = blk * ybw + k; r[k] = co < Co ? acc[co] : 0.f; }
-                        const size_t ri = ((size_t)n * ynb + blk) * So + ov;
-                        const uint8_t sb = orc_store_row(ybits, r, ybw, codes, 0);
-                        memcpy(yq + ri * yrb, codes, (size_t)yrb); ysc[ri] = sb;
-                        if (ls && c->stored_stats) { float d[32]; orc_load_row(ybits, codes, sb, ybw, d); for (int k = 0; k < ybw; k++) { const int co = blk * ybw + k; if (co < Co) acc[co] = d[k]; } }
-                    }
-                } else if (c->ydt == 2) {
-                    for (int co = 0; co < Co; co++) {
-                        float v = acc[co];
-                        if (c->Go > 0 && fabsf(v) > 65504.f) v = copysignf(65504.f, v);   /* sat_h16 (src/lp_common.cuh:465, :1567-1569) */
-                        ((uint16_t *)c->y)[((size_t)n * Co + co) * So + ov] = orc_f32_to_h16(v);
-                        acc[co] = v;
-                    }
-                } else for (int co = 0; co < Co; co++) ((float *)c->y)[((size_t)n * Co + co) * So + ov] = acc[co];
-                if (ls) for (int co = 0; co < Co; co++) { const double v = acc[co]; ls[2 * (co / cpg)] += v; ls[2 * (co / cpg) + 1] += v * v; }
+                conv_epilogue(c, n, (size_t)vi, So, acc, acc64, ls);
             }
             if (ls) {
 #pragma omp critical

@@ -106,7 +106,7 @@ def mx_to_f32(bits, q, N, C, S):
 
 
 def conv3(x, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=8, stride=1, x2=None, c_split=0, up=0, gp=None, gp2=None, Go=0, want_stats=False,
-          stored_stats=0, acc64=0, fused_act=0, ep_a=None, ep_b=None, z0=0, z1=0):
+          stored_stats=0, acc64=0, fused_act=0, ep_a=None, ep_b=None, z0=0, z1=0, stem_tile=0):
     """Runs the oracle conv; returns (y, sums or None). y: uint8 MX bytes, float32 or uint16 (fp16 bits) planes [N][Co][So]."""
     c = orc_conv_t()
     keep = [x, x2, w, b, ep_a, ep_b]
@@ -124,7 +124,7 @@ def conv3(x, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=8, stride=1, x2=None, c_s
         y = np.zeros((N, Co, So), dtype=np.float32)
     sums = np.zeros((N, max(Go, 1), 2), dtype=np.float64) if want_stats else None
     c.y, c.ydt, c.osum, c.Go, c.stored_stats = ptr(y), ydt, ptr(sums), Go, stored_stats
-    c.acc64, c.fused_act, c.ep_a, c.ep_b, c.z0, c.z1 = acc64, fused_act, ptr(ep_a), ptr(ep_b), z0, z1
+    c.acc64, c.fused_act, c.ep_a, c.ep_b, c.z0, c.z1, c.stem_tile = acc64, fused_act, ptr(ep_a), ptr(ep_b), z0, z1, stem_tile
     rc = lib().orc_conv3(C.byref(c))
     assert rc == 0, rc
     del keep

@@ -88,7 +88,7 @@ def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N, dn):
             cb = 4 if (bits == 4 and ci == 32 and co <= 32) else 8
         want_l, sums = orc.conv3(tens[xl], dt, N, ci, xs[2], xs[3], xs[4], Pm(name + ".w"), Pm(name + ".b"), co, dt, cbits=cb, stride=stride,
                                  x2=tens[x2l] if x2l else None, c_split=shapes[xl][1] if x2l else 0, up=up, gp=gn_of(xl), gp2=gn_of(x2l) if x2l else None,
-                                 Go=min(G, co), want_stats=stride == 1)
+                                 Go=min(G, co), want_stats=stride == 1, stem_tile=int(ci <= 8 and stride == 1))     # (the tap-packed stem: one scale per tile)
         frac, near = code_mismatch_fraction(bits, tens[name], want_l, N, co, d_ * h_ * w_)
         assert frac < (0.02 if bits == 8 else 0.05) and near, (name, frac, near)
         if stride == 1:                                            # the statistics the device finalised == the oracle's of its own output

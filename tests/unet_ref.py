@@ -55,7 +55,8 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
         if stride == 2:                       # the reference's stride-2 dispatch: fp4 only for an MX-fp4 32 -> <= 32 channel conv (src/lp_s2.cu:653-671)
             cb = 4 if (bits == 4 and ci == 32 and co <= 32) else 8
         y, s = orc.conv3(x, dt, N, ci, d[0], d[1], d[2], P(name + ".w"), P(name + ".b"), co, dt, cbits=cb, stride=stride, x2=x2, c_split=c_split, up=up,
-                         gp=gp, gp2=gp2, Go=Gof(co), want_stats=stats, stored_stats=stored)
+                         gp=gp, gp2=gp2, Go=Gof(co), want_stats=stats, stored_stats=stored,
+                         stem_tile=int(ci <= 8 and stride == 1 and x2 is None))   # the network input: tap-packed kernel, one scale per tile (src/lp_f8fwd.cuh:601-609)
         outs[name] = y
         return y, s
 

@@ -145,6 +145,58 @@ extern "C" const char *mi_last_kernel(void) { return g_last_kernel; }
 // the conv of every entry point: fmt 8 / 4 = compute format, stride 1 / 2
 // set by mi_conv_fwd_gn around its conv: finalize the statistics in the reduce kernel
 static thread_local gn_fin_t g_fin = {nullptr, nullptr, 0.0, 0.f};
+// GroupNorm partial sums of a conv's tiles -> the caller's sum slots (and mean / rstd when mi_conv_fwd_gn asked for them)
+static void conv_stats_reduce(const char *who, const conv_args &a, int MT, split_t sp, double *osum) {
+    gn_fin_t fin = g_fin;
+    fin.len = (double)(a.Co / a.Go) * (double)a.Do * a.Ho * a.Wo;
+    if (fin.mean && (sp.zlo || sp.zhi)) mi_die("%s: fused finalize with a z range", who);
+    if (a.stat_ch) gn_part_reduce_ch_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.Co, a.Go, osum, fin);
+    else gn_part_reduce_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.ncs, MT, a.Co, a.Go, osum, fin);
+    MICK();
+}
+
+// the tap-packed stem (src/lp_f8fwd.cuh:601-609, :421-434): e4m3 compute, one activation scale per staged tile
+static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
+                     gnp_t gp, double *osum, int Go, split_t sp) {
+    const int Ci = xs.c, N = xs.n, D = xs.d, H = xs.h, W = xs.w;
+    const int CP = Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2;
+    conv_args a; memset(&a, 0, sizeof a);
+    a.sx = x; a.sxdt = xbf; a.sCi = Ci;
+    a.sgam = gp.gamma; a.sbet = gp.beta; a.smean = gp.mean; a.srstd = gp.rstd; a.sG = gp.G;
+    a.N = N; a.D = D; a.H = H; a.W = W; a.Do = D; a.Ho = H; a.Wo = W;
+    a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
+    a.osum = osum; a.Go = Go; a.stored_stats = sp.stored_stats && ybf >= 3; a.zs0 = sp.zlo; a.zs1 = D - sp.zhi;
+    const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 ? 2 : 1;
+    size_t smem = ((size_t)720 * CP + 16 + CP * 8 + 15) & ~(size_t)15;     // staged tile, amax word, channel affine
+    a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);
+    a.red_o = (unsigned)smem; smem += 1024;
+    a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
+    a.ntx = (W + 15) / 16; a.nty = (H + 7) / 8; a.ntz = (D + 1) / 2;
+    a.ntiles = (unsigned)((size_t)a.ntx * a.nty * a.ntz * a.ncs * N);
+    const size_t wq_bytes = (size_t)NP * nmt_all * 2048, wsc_bytes = (size_t)NP * nmt_all * 256;
+    int dev = 0; MIRT(hipGetDevice(&dev));
+    uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
+    if (sp.wkey) {                                     // memo entries of this layout: nbt = -CP
+        for (auto &m : g_wmemo)
+            if (m.key == sp.wkey && m.w == w && m.fmt == 8 && m.Co == cout && m.Ci == Ci && m.nbt == -CP && m.nmt_all == nmt_all && m.dev == dev) { wq = m.wq; wsc = m.wsc; have = true; break; }
+        if (!have) {
+            MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes));
+            if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
+            g_wmemo.push_back(wmemo_t{sp.wkey, w, 8, cout, Ci, Ci, -CP, 0, nmt_all, dev, wq, wsc});
+        }
+    } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
+    if (!have) conv3_stem_prep(CP, w, wq, wsc, cout, Ci, nmt_all, NP);
+    a.wq = wq; a.wsc = wsc;
+    a.stat_ch = osum && (cout / Go) % 4 ? 1 : 0;
+    if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * (a.stat_ch ? 32 : MT * 8) * 2 * sizeof(float));
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    if (g_ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
+    conv3_stem_launch(CP, MT, ybf == 3 ? 8 : ybf == 4 ? 4 : 0, a, smem);
+    if (g_ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
+    if (osum) conv_stats_reduce(who, a, MT, sp, osum);
+    return 0;
+}
+
 static int conv_dispatch(const char *who, int fmt, int stride, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                          gnp_t gp, double *osum, int Go, split_t sp, const float *ep_a, const float *ep_b, int act) {
     if (sp.y2 || sp.o_split || sp.accum || sp.sr || sp.osr || sp.yD || sp.zi0 || sp.Di || sp.o_pad || sp.zw0 || sp.zw1 || sp.yzo)
@@ -153,6 +205,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (xbf < 0 || xbf > 4 || !(ybf == 0 || ybf == 2 || ybf == 3 || ybf == 4)) mi_die("%s: unsupported storage types (in %d, out %d)", who, xbf, ybf);
     if (xs.n <= 0 || xs.c <= 0 || xs.d <= 0 || xs.h <= 0 || xs.w <= 0 || cout <= 0) return 0;
     const int Ci = xs.c, Cx = sp.x2 ? sp.c_split : Ci, C2 = Ci - Cx;
+    if (fmt == 4 && Ci <= 8) fmt = 8;                  // the network input computes in e4m3 whatever the activations' format (src/lp_f4fwd.cu:37)
     if (sp.x2 && (Cx <= 0 || C2 <= 0)) mi_die("%s: channel split %d of %d", who, sp.c_split, Ci);
     if (sp.x2 && xbf < 3) mi_die("%s: split inputs need MX storage", who);
     if (sp.up && (!sp.x2 || xbf < 3 || (xs.d & 1) || (xs.h & 1) || (xs.w & 1) || stride != 1)) mi_die("%s: the fused upsample needs an MX split input and even dims", who);
@@ -160,6 +213,12 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (osum && (cout / Go) % 4 && cout > 32) mi_die("%s: fused output statistics of %d channels need channels per group (%d) to be a multiple of 4", who, cout, cout / Go);
     if (gp.G && ((sp.x2 && sp.gp2.G ? Cx : Ci) % gp.G)) mi_die("%s: GroupNorm groups %d do not divide the channels", who, gp.G);
     if (sp.gp2.G && (!sp.x2 || C2 % sp.gp2.G)) mi_die("%s: second GroupNorm without a matching x2 segment", who);
+    // few input channels: the tap-packed kernel with one activation scale per tile (src/lp_f8fwd.cuh:601-609: up to 8 channels of a 16-bit or
+    // MX input, 16 of an fp32 one; same input and output type, or an MX output)
+    static int stem_env = -1;
+    if (stem_env < 0) stem_env = getenv("MI_CONV_STEM") ? atoi(getenv("MI_CONV_STEM")) : 1;     // tuning knob: 0 sends these convs to the general kernel
+    if (stem_env && fmt == 8 && stride == 1 && !sp.x2 && !act && (xbf == 0 || xbf >= 2) && Ci <= (xbf == 0 ? 16 : 8) && (xbf == ybf || ybf >= 3))
+        return conv_stem(who, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp);
     const int N = xs.n, D = xs.d, H = xs.h, W = xs.w;
     const int Do = stride == 2 ? (D - 1) / 2 + 1 : D, Ho = stride == 2 ? (H - 1) / 2 + 1 : H, Wo = stride == 2 ? (W - 1) / 2 + 1 : W;   // src/nn_bwd.cu:132-135
     const size_t S = (size_t)D * H * W;
@@ -289,14 +348,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (fmt == 8) { if (out == 8) conv3_launch_f8_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f8_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f8_o0(stride, epi, MT, NT, a, smem); }
     else { if (out == 8) conv3_launch_f4_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f4_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f4_o0(stride, epi, MT, NT, a, smem); }
     if (g_ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
-    if (osum) {
-        gn_fin_t fin = g_fin;
-        fin.len = (double)(cout / Go) * (double)Do * Ho * Wo;
-        if (fin.mean && (sp.zlo || sp.zhi)) mi_die("%s: fused finalize with a z range", who);
-        if (a.stat_ch) gn_part_reduce_ch_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), cout, Go, osum, fin);
-        else gn_part_reduce_k<<<N * Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / N), a.ncs, MT, cout, Go, osum, fin);
-        MICK();
-    }
+    if (osum) conv_stats_reduce(who, a, MT, sp, osum);
     return 0;
 }
 

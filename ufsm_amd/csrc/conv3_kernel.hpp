@@ -98,6 +98,9 @@ struct conv_args {
     unsigned red_o;                    // LDS byte offset of the statistics scratch (1 KiB)
     const uint8_t *zpage;              // device memory: 64 zero bytes, then 64 bytes of value 1 (rows and scale bytes of positions outside the volume)
     int ntx, nty, ntz, ncs; unsigned ntiles;
+    // tap-packed stem only: the input as stored (0 fp32 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4: one row of 8 channels per voxel) and its GroupNorm
+    const void *sx; int sxdt, sCi;
+    const float *sgam, *sbet, *smean, *srstd; int sG;
 };
 
 template <int FMT> struct fmt_t;
@@ -594,3 +597,6 @@ static void launch_out(int stride, bool epi, int MT, int NT, const conv_args &a,
 #define CONV3_LAUNCH_DECL(FMT, OUT) void conv3_launch_f##FMT##_o##OUT(int stride, bool epi, int MT, int NT, const conv_args &a, size_t smem)
 CONV3_LAUNCH_DECL(8, 8); CONV3_LAUNCH_DECL(8, 4); CONV3_LAUNCH_DECL(8, 0);
 CONV3_LAUNCH_DECL(4, 8); CONV3_LAUNCH_DECL(4, 4); CONV3_LAUNCH_DECL(4, 0);
+// the tap-packed stem (conv3_stem.hip): weight preparation for CP padded channels, kernel launch
+void conv3_stem_prep(int CP, const float *w, uint8_t *wq, uint8_t *wsc, int Co, int Ci, int nmt_all, int np);
+void conv3_stem_launch(int CP, int MT, int out, const conv_args &a, size_t smem);

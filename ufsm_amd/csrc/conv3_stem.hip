@@ -1,0 +1,226 @@
+// Tap-packed small-channel 3x3x3 conv, the network stem (src/lp_f8fwd.cuh:153-177 weights, :178-400 kernel, :601-609 dispatch).
+// Input channels are padded to CP in {4, 8, 16}; a K block of 32 = 32 / CP taps x CP channels, so the 27 taps take ceil(27 CP / 32) blocks
+// instead of 27 nearly empty ones. A block mixes positions, so the activation operand has ONE E8M0 scale per staged tile: the
+// 4 x 10 x 18 input positions around a 2 x 8 x 16 output tile (tiles on the output grid from the origin). The input is read as stored
+// (fp32 / fp16 planes or an MX tensor of one block row per voxel), GroupNorm + SiLU applied when the input carries one, the tile's amax
+// taken over those values (fmaxf: NaN ignored; zeros outside the volume), and the values re-encoded to e4m3 with the tile's scale in LDS.
+//
+// One workgroup per output tile and slice of MT x 32 output channels; four wavefronts, each two 32-voxel MFMA tiles. A 32x32x64 MFMA
+// takes two K blocks: lane (r, h) supplies bytes 16 h .. 16 h + 15 of both, i.e. 16 / CP taps of CP channels per block, read straight
+// from the staged tile [position][CP bytes] at the taps' offsets. The weights' fragments stay in registers. Epilogue: conv_epilogue.
+#include "conv3_kernel.hpp"
+
+template <int CP, int MT, int OUT>
+__global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
+    constexpr int TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2, NT = 2;
+    constexpr int HY = 10, HX = 18, TT = 4 * HY * HX, WTILE = 2048;
+    extern __shared__ __align__(16) unsigned char lds[];
+    // LDS: [staged tile TT x CP bytes][amax word, padded to 16][per channel (a, b) of the GroupNorm affine: CP x float2]
+    constexpr unsigned am_o = TT * CP, ab_o = am_o + 16;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    unsigned tile;
+    {
+        const unsigned per = (a.ntiles + 7u) / 8u;          // consecutive workgroup ids go round the 8 XCDs: a contiguous tile range per XCD
+        tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
+        if (tile >= a.ntiles) return;
+    }
+    int tt = (int)tile;
+    const int cs = tt % a.ncs; tt /= a.ncs;
+    const int tx = tt % a.ntx; tt /= a.ntx;
+    const int ty = tt % a.nty; tt /= a.nty;
+    const int tz = tt % a.ntz; const int n = tt / a.ntz;
+    const int ox0 = tx * 16, oy0 = ty * 8, oz0 = tz * 2;
+    const int Ci = a.sCi;
+    const size_t S = (size_t)a.D * a.H * a.W;
+
+    if (tid == 0) *(unsigned *)(lds + am_o) = 0u;
+    if (tid < CP) {
+        float ga = 1.f, gb = 0.f;
+        if (a.sG && tid < Ci) { const int ng = n * a.sG + tid / (Ci / a.sG); ga = a.srstd[ng] * a.sgam[tid]; gb = fmaf(-a.smean[ng], ga, a.sbet[tid]); }
+        *(float2 *)(lds + ab_o + tid * 8) = make_float2(ga, gb);
+    }
+    conv_epi_consts<MT, false>(a, lds, cs, tid);
+
+    // ---- the weights' fragments and scale words: pair p = K blocks 2 p, 2 p + 1 ----
+    v8i fa[NP][MT]; int sa[NP][MT];
+#pragma unroll
+    for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const size_t t = (size_t)p * a.nmt_all + cs * MT + m;
+            const v4i lo = *(const v4i *)(a.wq + t * WTILE + lane * 16), hi = *(const v4i *)(a.wq + t * WTILE + 1024 + lane * 16);
+            fa[p][m] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            sa[p][m] = *(const int *)(a.wsc + (t * 64 + lane) * 4);
+        }
+
+    // ---- stage: a thread owns positions tid, tid + 256, tid + 512 of the tile ----
+    float v[3][CP];
+    float amax = 0.f;
+    const int xdt = a.sxdt;
+    __syncthreads();                                         // the affine table
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int pos = tid + 256 * j, ix = pos % HX, iy = (pos / HX) % HY, iz = pos / (HY * HX);
+        const int gz = oz0 - 1 + iz, gy = oy0 - 1 + iy, gx = ox0 - 1 + ix;
+        const bool inb = pos < TT && (unsigned)gz < (unsigned)a.D && (unsigned)gy < (unsigned)a.H && (unsigned)gx < (unsigned)a.W;
+        const size_t off = inb ? ((size_t)gz * a.H + gy) * a.W + gx : 0;
+        float x[CP];
+#pragma unroll
+        for (int k = 0; k < CP; k++) x[k] = 0.f;
+        if (xdt == 3) {                                      // one MX-fp8 row of 8 channels per voxel, then the scale plane
+            if constexpr (CP <= 8) {
+                const uint8_t *q = (const uint8_t *)a.sx;
+                const float s = d_mx_scale(q[(size_t)a.N * S * 8 + (size_t)n * S + off]);
+                const uint8_t *row = q + ((size_t)n * S + off) * 8;
+                d_dec4_e4m3(*(const unsigned *)row, x);
+                if constexpr (CP == 8) d_dec4_e4m3(*(const unsigned *)(row + 4), x + 4);
+#pragma unroll
+                for (int k = 0; k < CP; k++) x[k] *= s;
+            }
+        } else if (xdt == 4) {                               // one MX-fp4 row of 8 channels (4 bytes) per voxel
+            if constexpr (CP <= 8) {
+                const uint8_t *q = (const uint8_t *)a.sx;
+                const float s = d_mx_scale(q[(size_t)a.N * S * 4 + (size_t)n * S + off]);
+                float d8[8];
+                d_dec8_e2m1(*(const unsigned *)(q + ((size_t)n * S + off) * 4), d8);
+#pragma unroll
+                for (int k = 0; k < CP; k++) x[k] = d8[k] * s;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < CP; k++)
+                if (k < Ci) {
+                    const size_t idx = ((size_t)n * Ci + k) * S + off;
+                    x[k] = xdt == 2 ? __half2float(((const __half *)a.sx)[idx]) : ((const float *)a.sx)[idx];
+                }
+        }
+#pragma unroll
+        for (int k = 0; k < CP; k++) {
+            float val = x[k];
+            if (a.sG) { const float2 ab = *(const float2 *)(lds + ab_o + k * 8); val = d_act_ab(val, ab.x, ab.y); }
+            val = inb && k < Ci ? val : 0.f;
+            v[j][k] = val; amax = fmaxf(amax, fabsf(val));
+        }
+    }
+    amax = fmaxf(amax, lane_xorf<1>(amax)); amax = fmaxf(amax, lane_xorf<2>(amax)); amax = fmaxf(amax, lane_xorf<4>(amax));
+    amax = fmaxf(amax, lane_xorf<8>(amax)); amax = fmaxf(amax, lane_xorf<16>(amax)); amax = fmaxf(amax, lane_xor32f(amax, h));
+    if (lane == 0) atomicMax((unsigned *)(lds + am_o), __float_as_uint(amax));        // non-negative floats order as their bit patterns
+    __syncthreads();
+    const int e = d_mx_exp(__uint_as_float(*(const unsigned *)(lds + am_o)), MI_INVQ8);
+    const int sb = e + 127;
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int pos = tid + 256 * j;
+        if (pos < TT) {
+#pragma unroll
+            for (int k = 0; k < CP / 4; k++)
+                *(unsigned *)(lds + pos * CP + 4 * k) = d_enc4_e4m3(v[j][4 * k], v[j][4 * k + 1], v[j][4 * k + 2], v[j][4 * k + 3], e);
+        }
+    }
+    __syncthreads();
+
+    // ---- MFMAs: wavefront -> (z, y half), voxel tile j -> rows 2 j, 2 j + 1 of that half, r -> (row, x) ----
+    const int lz = wave >> 1, ly0 = (wave & 1) * 4;
+    const int p00 = (lz * HY + ly0 + (r >> 4)) * HX + (r & 15);
+    v16f acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
+    auto tapoff = [](int tap) { tap = tap > 26 ? 26 : tap; return ((tap / 9) * HY + (tap / 3) % 3) * HX + tap % 3; };     // (taps past 26: zero weights)
+    static_for<NP>([&](auto P) {
+        constexpr int p = P;
+        constexpr int LT = 16 / CP;                          // taps a lane supplies per K block
+        int off[2][LT];
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int i = 0; i < LT; i++) off[s][i] = h ? tapoff((2 * p + s) * TPK + LT + i) : tapoff((2 * p + s) * TPK + i);
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            const int pj = p00 + 2 * j * HX;
+            v8i fb;
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                if constexpr (CP == 4) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) fb[4 * s + i] = *(const int *)(lds + (pj + off[s][i]) * 4);
+                } else if constexpr (CP == 8) {
+#pragma unroll
+                    for (int i = 0; i < 2; i++) { const int2 w2 = *(const int2 *)(lds + (pj + off[s][i]) * 8); fb[4 * s + 2 * i] = w2.x; fb[4 * s + 2 * i + 1] = w2.y; }
+                } else {
+                    const v4i w4 = *(const v4i *)(lds + (pj + off[s][0]) * 16);
+                    fb[4 * s] = w4[0]; fb[4 * s + 1] = w4[1]; fb[4 * s + 2] = w4[2]; fb[4 * s + 3] = w4[3];
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < MT; m++) acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[p][m], fb, acc[m][j], 0, 0, 0, sa[p][m], 0, sb);
+        }
+    });
+    __syncthreads();                                         // the staged tile is dead: the epilogue's scratch may overlay nothing of it, but keep the order
+    conv_epilogue<MT, NT, OUT, false>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
+}
+
+// weights: fp32 w[co][ci][27] -> per (block pair, 32-row channel tile) fragment-ordered e4m3 codes + one scale word per lane
+// (src/lp_f8fwd.cuh:156-177): block kb, k -> tap kb * TPK + k / CP, channel k % CP; zeros past the taps, the channels and the rows
+template <int CP>
+__global__ void __launch_bounds__(128) prep_ws_k(const float *__restrict__ w, uint8_t *__restrict__ wq, unsigned *__restrict__ wsc, int Co, int Ci, int nmt_all, int np) {
+    constexpr int TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x, Cop = nmt_all * 32;
+    if (i >= np * Cop) return;
+    const int cop = i % Cop, p = i / Cop, m = cop >> 5, r = cop & 31;
+    uint8_t *tile = wq + ((size_t)p * nmt_all + m) * 2048;
+    unsigned *tsc = wsc + ((size_t)p * nmt_all + m) * 64;
+#pragma unroll
+    for (int side = 0; side < 2; side++) {
+        const int kb = 2 * p + side;
+        float v[32]; float amax = 0.f;
+#pragma unroll
+        for (int k = 0; k < 32; k++) {
+            const int tap = kb * TPK + k / CP, ci = k % CP;
+            v[k] = (kb < NKB && cop < Co && ci < Ci && tap < 27) ? w[((size_t)cop * Ci + ci) * 27 + tap] : 0.f;
+            amax = fmaxf(amax, fabsf(v[k]));
+        }
+        const int e = d_mx_exp(amax, MI_INVQ8);
+        const float mult = d_exp2i(-e);
+        unsigned c[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) c[j] = d_enc_e4m3x4(v[4 * j] * mult, v[4 * j + 1] * mult, v[4 * j + 2] * mult, v[4 * j + 3] * mult);
+        *(uint4 *)(tile + ((size_t)(side * 64 + r) * 16)) = make_uint4(c[0], c[1], c[2], c[3]);            // lane (r, 0): bytes 0-15 of the block
+        *(uint4 *)(tile + ((size_t)(side * 64 + r + 32) * 16)) = make_uint4(c[4], c[5], c[6], c[7]);       // lane (r, 1): bytes 16-31
+        tsc[r + 32 * side] = (unsigned)(e + 127);
+    }
+}
+
+void conv3_stem_prep(int CP, const float *w, uint8_t *wq, uint8_t *wsc, int Co, int Ci, int nmt_all, int np) {
+    const unsigned nb = nblk_((size_t)np * nmt_all * 32, 128);
+    if (CP == 4) prep_ws_k<4><<<nb, 128>>>(w, wq, (unsigned *)wsc, Co, Ci, nmt_all, np);
+    else if (CP == 8) prep_ws_k<8><<<nb, 128>>>(w, wq, (unsigned *)wsc, Co, Ci, nmt_all, np);
+    else prep_ws_k<16><<<nb, 128>>>(w, wq, (unsigned *)wsc, Co, Ci, nmt_all, np);
+    MICK();
+}
+
+template <int CP, int MT, int OUT>
+static void launch_stem(const conv_args &a, size_t smem) {
+    const unsigned per = (a.ntiles + 7u) / 8u;
+    conv3_stem_k<CP, MT, OUT><<<per * 8u, 256, smem>>>(a);
+    MICK();
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_stem_k<CP %d, MT %d, out %d> tiles %u", CP, MT, OUT, a.ntiles);
+}
+template <int CP, int MT>
+static void launch_stem_out(int out, const conv_args &a, size_t smem) {
+    if (out == 8) launch_stem<CP, MT, 8>(a, smem); else if (out == 4) launch_stem<CP, MT, 4>(a, smem); else launch_stem<CP, MT, 0>(a, smem);
+}
+void conv3_stem_launch(int CP, int MT, int out, const conv_args &a, size_t smem) {
+    switch (CP * 10 + MT) {
+    case 41: launch_stem_out<4, 1>(out, a, smem); break;
+    case 42: launch_stem_out<4, 2>(out, a, smem); break;
+    case 81: launch_stem_out<8, 1>(out, a, smem); break;
+    case 82: launch_stem_out<8, 2>(out, a, smem); break;
+    case 161: launch_stem_out<16, 1>(out, a, smem); break;
+    case 162: launch_stem_out<16, 2>(out, a, smem); break;
+    default: mi_die("conv3 stem: no kernel for CP %d MT %d", CP, MT);
+    }
+}
