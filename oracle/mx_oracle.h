@@ -30,8 +30,10 @@
  *   SiLU in GN staging            PARITY UNPINNED to the bit: the reference evaluates tanh with NVIDIA's
  *                                 tanh.approx.f32 (src/lp_common.cuh:469-473), not reproducible off that hardware;
  *                                 checked to floor/ceil code neighbours as tests/test_mx4_wide.c:165-175 does
- *   stem tile scale (Ci <= 8)     PARITY UNPINNED to the bit: one scale per staged tile depends on the reference's tile
- *                                 geometry (src/lp_f8fwd.cuh:374-380); restated with that geometry, tolerance only
+ *   orc_conv3 with stem_tile      the tap-packed small-channel conv (src/lp_f8fwd.cuh:153-400): exact operands equal the fp64
+ *                                 convolution for the three channel paddings and all input types; one large value coarsens exactly the
+ *                                 output voxels of the 2 x 8 x 16 tiles whose 4 x 10 x 18 halo holds it; a one-tile volume returns the
+ *                                 tensor under one scale (tests/test_oracle_stem.py)
  */
 #ifndef MX_ORACLE_H
 #define MX_ORACLE_H

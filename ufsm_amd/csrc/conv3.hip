@@ -166,7 +166,7 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     a.N = N; a.D = D; a.H = H; a.W = W; a.Do = D; a.Ho = H; a.Wo = W;
     a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
     a.osum = osum; a.Go = Go; a.stored_stats = sp.stored_stats && ybf >= 3; a.zs0 = sp.zlo; a.zs1 = D - sp.zhi;
-    const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 ? 2 : 1;
+    const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 && CP < 16 ? 2 : 1;     // (16 padded channels: 7 weight fragment pairs per channel tile, one tile fits the registers)
     size_t smem = ((size_t)720 * CP + 16 + CP * 8 + 15) & ~(size_t)15;     // staged tile, amax word, channel affine
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);
     a.red_o = (unsigned)smem; smem += 1024;

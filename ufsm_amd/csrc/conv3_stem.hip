@@ -220,7 +220,6 @@ void conv3_stem_launch(int CP, int MT, int out, const conv_args &a, size_t smem)
     case 81: launch_stem_out<8, 1>(out, a, smem); break;
     case 82: launch_stem_out<8, 2>(out, a, smem); break;
     case 161: launch_stem_out<16, 1>(out, a, smem); break;
-    case 162: launch_stem_out<16, 2>(out, a, smem); break;
     default: mi_die("conv3 stem: no kernel for CP %d MT %d", CP, MT);
     }
 }
