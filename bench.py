@@ -65,6 +65,58 @@ def unet_leg(np, lib, LP, DevBuf, steps, warmup):
             "steps": steps, "gflop_per_forward": fl / 1e9, "tflops": fl / dt / 1e12}
 
 
+def hbm_leg(np, lib, LP, DevBuf):
+    """The HBM-bound kernels of the path at the level-0 shapes of configs[3] (N 2, 32 channels, 128^3; the upsample from 64 channels at 64^3;
+    the stem 4 -> 32): algorithmic bytes (each tensor read or written once: 33 / 32 B per MX-fp8 element) over the time of one call, averaged
+    over 10 back-to-back calls between two device synchronisations, against the 8 TB/s HBM peak."""
+    from ufsm_amd import shape5, gnp_t, split_t
+    N, C, D = 2, 32, 128
+    S = D ** 3
+    rng = np.random.default_rng(5)
+    mx = lambda c, s: N * ((c + 31) // 32) * s * 33 if c > 8 else N * s * 9
+    x = rng.standard_normal((N, C, S)).astype(np.float32)
+    dx = DevBuf.from_numpy(x); del x
+    q = DevBuf(lib.lp_mx8_bytes(N, C, S)); q2 = DevBuf(lib.lp_mx8_bytes(N, C, S))
+    lib.lp_f32_to_mx8(dx.ptr, N, C, S, q.ptr)
+    G = 8
+    gam = DevBuf.from_numpy(rng.uniform(0.5, 1.5, C).astype(np.float32)); bet = DevBuf.from_numpy(rng.uniform(-.5, .5, C).astype(np.float32))
+    mean = DevBuf.from_numpy(rng.uniform(-.2, .2, N * G).astype(np.float32)); rstd = DevBuf.from_numpy(rng.uniform(.8, 1.2, N * G).astype(np.float32))
+    gp = gnp_t(gam.ptr, bet.ptr, mean.ptr, rstd.ptr, G)
+    s5 = shape5(N, C, D, D, D)
+    sums = DevBuf(N * G * 2 * 24)
+    w1 = DevBuf.from_numpy((rng.standard_normal((8, C)) * 0.1).astype(np.float32)); b1 = DevBuf.from_numpy(np.zeros(8, np.float32))
+    logits = DevBuf(N * 8 * S * 4)
+    Cc, Sc = 64, (D // 2) ** 3
+    xc = DevBuf.from_numpy(rng.standard_normal((N, Cc, Sc)).astype(np.float32)); qc = DevBuf(lib.lp_mx8_bytes(N, Cc, Sc)); lib.lp_f32_to_mx8(xc.ptr, N, Cc, Sc, qc.ptr)
+    qu = DevBuf(lib.lp_mx8_bytes(N, Cc, S))
+    x4 = DevBuf.from_numpy(rng.standard_normal((N, 4, S)).astype(np.float32)); q4 = DevBuf(lib.lp_mx8_bytes(N, 4, S)); lib.lp_f32_to_mx8(x4.ptr, N, 4, S, q4.ptr)
+    ws = DevBuf.from_numpy((rng.standard_normal((C, 4, 27)) * 0.1).astype(np.float32)); bs = DevBuf.from_numpy(np.zeros(C, np.float32))
+    sp = split_t(); sp.wkey = 901
+    cases = [
+        ("f32_to_mx_k (lp_f32_to_mx8, 32 ch)", N * C * S * 4 + mx(C, S), lambda: lib.lp_f32_to_mx8(dx.ptr, N, C, S, q2.ptr)),
+        ("mx_to_f32_k (lp_mx8_to_f32, 32 ch)", N * C * S * 4 + mx(C, S), lambda: lib.lp_mx8_to_f32(q.ptr, N, C, S, dx.ptr)),
+        ("gn_silu_apply_mx_k (GN + SiLU + requant, 32 ch; the conv pre-pass restage32_k is the same arithmetic)", 2 * mx(C, S), lambda: lib.lp_gn_silu_apply_mx(q.ptr, 3, s5, G, gam.ptr, bet.ptr, mean.ptr, rstd.ptr, q2.ptr, 3)),
+        ("gn_sums_mx_k (lp_gn_sums_mx, 32 ch)", mx(C, S), lambda: lib.lp_gn_sums_mx(q.ptr, 3, N, C, G, S, sums.ptr, 0, S)),
+        ("add_mx_k (lp_add_mx, 32 ch)", 3 * mx(C, S), lambda: lib.lp_add_mx(q2.ptr, q.ptr, s5, 3, 0)),
+        ("conv1_mx_k (1x1x1 head 32 -> 8 with GN + SiLU, fp32 logits)", mx(C, S) + N * 8 * S * 4, lambda: lib.lp_conv1_fwd_mx(q.ptr, 3, s5, w1.ptr, b1.ptr, 8, logits.ptr, gp)),
+        ("up2_mx_k (trilinear 2x, 64 ch, 64^3 -> 128^3)", mx(Cc, Sc) + mx(Cc, S), lambda: lib.lp_up2_fwd_mx(qc.ptr, 3, shape5(N, Cc, D // 2, D // 2, D // 2), qu.ptr, 3, gnp_t())),
+        ("conv3_stem_k (3x3x3 stem 4 -> 32, MX-fp8 in / out)", mx(4, S) + mx(C, S), lambda: lib.lp_conv_fwd_f8(q4.ptr, 3, shape5(N, 4, D, D, D), ws.ptr, bs.ptr, C, q2.ptr, 3, gnp_t(), None, 0, sp)),
+    ]
+    rows = []
+    for name, nbytes, call in cases:
+        for _ in range(3):
+            call()
+        lib.mi_sync(); LP.check()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            call()
+        lib.mi_sync(); LP.check()
+        dt = (time.perf_counter() - t0) / 10
+        rows.append({"kernel": name, "bytes": nbytes, "us": dt * 1e6, "GBps": nbytes / dt / 1e9, "frac_of_hbm_peak": nbytes / dt / 8e12})
+    lib.lp_wmemo_clear()
+    return rows
+
+
 def sliding_leg(np, lib, LP, DevBuf):
     """configs[4]: a 512 x 1024 x 1024 uint8 volume resident in HBM, 128^3 windows with 16 voxels of halo (stride 96), per window a U-Net of
     widths 32/64/128/192 with MX-fp4 weights over MX-fp8 activations (prec 3) and two transformer blocks (MX-fp8 attention core, MX-fp8
@@ -105,6 +157,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target seconds of CPU work for the cpu_baseline sample")
     ap.add_argument("--no-unet", action="store_true", help="skip the configs[3] U-Net forward leg")
     ap.add_argument("--no-sliding", action="store_true", help="skip the configs[4]-geometry sliding-window leg")
+    ap.add_argument("--no-hbm", action="store_true", help="skip the HBM-bound kernels leg")
     ap.add_argument("--copy-probe", action="store_true", help="run 5 device-to-device copies of 1 GiB and exit: the known-size kernel that scales "
                     "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     a = ap.parse_args()
@@ -191,6 +244,8 @@ def main():
         out["unet"] = unet_leg(np, lib, LP, DevBuf, max(3, a.steps // 4), max(1, a.warmup))
     if not a.no_sliding:
         out["sliding_window"] = sliding_leg(np, lib, LP, DevBuf)
+    if not a.no_hbm:
+        out["hbm_kernels"] = hbm_leg(np, lib, LP, DevBuf)
     if not a.no_cpu_baseline:
         import orc
         # the oracle (a port: the reference has no CPU MX conv) on a bounded z-slab of one layer of the same workload

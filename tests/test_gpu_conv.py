@@ -314,3 +314,70 @@ def test_fused_statistics_finalize(gpu, bits, Ci, Co, dims):
         res.append((dy.to_numpy(np.uint8), dsum.to_numpy(np.uint8), dm.to_numpy(np.float32), dr.to_numpy(np.float32)))
     for u, v in zip(*res):
         assert np.array_equal(u, v)
+
+
+@pytest.mark.parametrize("case", ["general32", "wide128", "stem4", "decoder_up", "fp4_64", "gn_input"])
+def test_z_range_slabs_equal_whole(gpu, case):
+    """split_t's z-range (zi0 / Di: output plane z reads input plane z + zi0 of a depth-Di input) with direct slab outputs (yzo / yD), the
+    reference's in-place slab inference (src/nn_lp.h:36-40, src/nn_bwd.cu:33-46): the conv computed slab by slab into the full-depth output,
+    statistics accumulating over the calls, is byte-identical to one call over the whole tensor (tests/test_infer_mem.c's contract)."""
+    rng = np.random.default_rng(hash(case) % 1000)
+    bits, xdt, up, gn = 8, 3, 0, False
+    Cu = 0
+    if case == "general32": N, Ci, Co, D, H, W, slabs = 2, 32, 32, 12, 16, 32, (4, 8)
+    elif case == "wide128": N, Ci, Co, D, H, W, slabs = 1, 64, 128, 16, 8, 32, (8, 4, 4)
+    elif case == "stem4": N, Ci, Co, D, H, W, slabs = 2, 4, 32, 10, 16, 16, (4, 6)
+    elif case == "decoder_up": N, Ci, Co, D, H, W, slabs, up, gn, Cu = 1, 96, 32, 16, 16, 16, (4, 4, 8), 1, True, 64
+    elif case == "fp4_64": N, Ci, Co, D, H, W, slabs, bits, xdt = 1, 64, 64, 12, 8, 16, (8, 4), 4, 4
+    else: N, Ci, Co, D, H, W, slabs, gn = 2, 64, 64, 8, 16, 16, (4, 4), True
+    S = D * H * W
+    G = 8
+    w = (rng.standard_normal((Co, Ci, 27)) * np.sqrt(2.0 / (Ci * 27))).astype(np.float32)
+    b = (rng.standard_normal(Co) * 0.1).astype(np.float32)
+    dw, db = DevBuf.from_numpy(w), DevBuf.from_numpy(b)
+    sp = split_t(); keep = []
+    if up:
+        Cs = Ci - Cu
+        xu = rng.standard_normal((N, Cu, S // 8)).astype(np.float32); xs_ = rng.standard_normal((N, Cs, S)).astype(np.float32)
+        dx, dx2 = DevBuf.from_numpy(orc.f32_to_mx(bits, xu, N, Cu, S // 8)), DevBuf.from_numpy(orc.f32_to_mx(bits, xs_, N, Cs, S))
+        sp.x2, sp.c_split, sp.up = dx2.ptr, Cu, 1
+        g1 = dev_gn(rng.uniform(.5, 1.5, Cu).astype(np.float32), rng.uniform(-.3, .3, Cu).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.7, 1.4, N * G).astype(np.float32), G)
+        g2 = dev_gn(rng.uniform(.5, 1.5, Cs).astype(np.float32), rng.uniform(-.3, .3, Cs).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.7, 1.4, N * G).astype(np.float32), G)
+        sp.gp2 = g2                                     # (a copy of the struct: g2 itself keeps the device buffers alive)
+        keep += [dx2, g2]
+    else:
+        x = rng.standard_normal((N, Ci, S)).astype(np.float32)
+        dx = DevBuf.from_numpy(orc.f32_to_mx(bits, x, N, Ci, S))
+        g1 = dev_gn(rng.uniform(.5, 1.5, Ci).astype(np.float32), rng.uniform(-.3, .3, Ci).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.7, 1.4, N * G).astype(np.float32), G) if gn else gnp_t()
+    f = lib.lp_conv_fwd_f8 if bits == 8 else lib.lp_conv_fwd_f4
+    ybytes = orc.mx_bytes(bits, N, Co, S)
+    ywhole, yslab = DevBuf(ybytes), DevBuf(ybytes)
+    sw, ss = DevBuf(N * G * 2 * 24), DevBuf(N * G * 2 * 24)
+    lib.mi_gn_sums_zero(sw.ptr, 2 * N * G); lib.mi_gn_sums_zero(ss.ptr, 2 * N * G)
+    sp.stored_stats = 1
+    assert f(dx.ptr, xdt, shape5(N, Ci, D, H, W), dw.ptr, db.ptr, Co, ywhole.ptr, xdt, g1, sw.ptr, G, sp) == 0
+    kernel = lib.mi_last_kernel().decode()
+    z0 = 0
+    for sk in slabs:
+        sp.zi0, sp.Di, sp.yzo, sp.yD = z0, D, z0, D
+        assert f(dx.ptr, xdt, shape5(N, Ci, sk, H, W), dw.ptr, db.ptr, Co, yslab.ptr, xdt, g1, ss.ptr, G, sp) == 0
+        z0 += sk
+    assert z0 == D
+    LP.check()
+    assert np.array_equal(ywhole.to_numpy(np.uint8), yslab.to_numpy(np.uint8)), kernel
+    a, c = np.zeros((N, G, 2), np.float64), np.zeros((N, G, 2), np.float64)
+    da, dc = DevBuf(a.nbytes), DevBuf(c.nbytes)
+    lib.mi_gn_sums_get(sw.ptr, 2 * N * G, da.ptr); lib.mi_gn_sums_get(ss.ptr, 2 * N * G, dc.ptr)
+    a, c = da.to_numpy(np.float64), dc.to_numpy(np.float64)
+    assert np.allclose(a, c, rtol=1e-12, atol=1e-9), kernel
+    # a slab into its own depth-sk output (the temp of the reference's in-place form): the same planes
+    sk = slabs[0]
+    sp.zi0, sp.Di, sp.yzo, sp.yD = slabs[0] if len(slabs) > 1 else 0, D, 0, 0
+    sk2 = slabs[1] if len(slabs) > 1 else sk
+    ytmp = DevBuf(orc.mx_bytes(bits, N, Co, sk2 * H * W))
+    assert f(dx.ptr, xdt, shape5(N, Ci, sk2, H, W), dw.ptr, db.ptr, Co, ytmp.ptr, xdt, g1, None, 0, sp) == 0
+    LP.check()
+    full = orc.mx_to_f32(bits, ywhole.to_numpy(np.uint8), N, Co, S).reshape(N, Co, D, H * W)
+    part = orc.mx_to_f32(bits, ytmp.to_numpy(np.uint8), N, Co, sk2 * H * W).reshape(N, Co, sk2, H * W)
+    zz = slabs[0] if len(slabs) > 1 else 0
+    assert np.array_equal(part, full[:, :, zz:zz + sk2])

@@ -158,20 +158,21 @@ static void conv_stats_reduce(const char *who, const conv_args &a, int MT, split
 // the tap-packed stem (src/lp_f8fwd.cuh:601-609, :421-434): e4m3 compute, one activation scale per staged tile
 static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                      gnp_t gp, double *osum, int Go, split_t sp) {
-    const int Ci = xs.c, N = xs.n, D = xs.d, H = xs.h, W = xs.w;
+    const int Ci = xs.c, N = xs.n, D = sp.Di ? sp.Di : xs.d, Do = xs.d, H = xs.h, W = xs.w;      // D: the input's depth (z-range), Do: output planes
     const int CP = Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2;
     conv_args a; memset(&a, 0, sizeof a);
     a.sx = x; a.sxdt = xbf; a.sCi = Ci;
     a.sgam = gp.gamma; a.sbet = gp.beta; a.smean = gp.mean; a.srstd = gp.rstd; a.sG = gp.G;
-    a.N = N; a.D = D; a.H = H; a.W = W; a.Do = D; a.Ho = H; a.Wo = W;
+    a.N = N; a.D = D; a.H = H; a.W = W; a.Do = Do; a.Ho = H; a.Wo = W;
+    a.zi0 = sp.Di ? sp.zi0 : 0; a.yD = sp.yD; a.yzo = sp.yD ? sp.yzo : 0;
     a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
-    a.osum = osum; a.Go = Go; a.stored_stats = sp.stored_stats && ybf >= 3; a.zs0 = sp.zlo; a.zs1 = D - sp.zhi;
+    a.osum = osum; a.Go = Go; a.stored_stats = sp.stored_stats && ybf >= 3; a.zs0 = sp.zlo; a.zs1 = Do - sp.zhi;
     const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 && CP < 16 ? 2 : 1;     // (16 padded channels: 7 weight fragment pairs per channel tile, one tile fits the registers)
     size_t smem = ((size_t)720 * CP + 16 + CP * 8 + 15) & ~(size_t)15;     // staged tile, amax word, channel affine
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);
     a.red_o = (unsigned)smem; smem += 1024;
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
-    a.ntx = (W + 15) / 16; a.nty = (H + 7) / 8; a.ntz = (D + 1) / 2;
+    a.ntx = (W + 15) / 16; a.nty = (H + 7) / 8; a.ntz = (Do + 1) / 2;
     a.ntiles = (unsigned)((size_t)a.ntx * a.nty * a.ntz * a.ncs * N);
     const size_t wq_bytes = (size_t)NP * nmt_all * 2048, wsc_bytes = (size_t)NP * nmt_all * 256;
     int dev = 0; MIRT(hipGetDevice(&dev));
@@ -199,8 +200,12 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
 
 static int conv_dispatch(const char *who, int fmt, int stride, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                          gnp_t gp, double *osum, int Go, split_t sp, const float *ep_a, const float *ep_b, int act) {
-    if (sp.y2 || sp.o_split || sp.accum || sp.sr || sp.osr || sp.yD || sp.zi0 || sp.Di || sp.o_pad || sp.zw0 || sp.zw1 || sp.yzo)
-        mi_die("%s: split outputs, accumulate, stochastic rounding and z-slab / z-window fields of split_t are not built here (inference forward only)", who);
+    if (sp.y2 || sp.o_split || sp.accum || sp.sr || sp.osr || sp.o_pad || sp.zw0 || sp.zw1)
+        mi_die("%s: split outputs, accumulate, stochastic rounding and the z-window fields of split_t are not built here (inference forward only)", who);
+    // z-range (src/nn_lp.h:36-40, src/nn_bwd.cu:33-36): the xs.d output planes read input plane z + zi0 of depth-Di inputs; direct slab output:
+    // the MX output is planes [yzo, yzo + xs.d) of a depth-yD tensor
+    if ((sp.Di || sp.zi0) && (stride != 1 || sp.zi0 < 0 || sp.zi0 + xs.d > sp.Di)) mi_die("%s: z-range %d + %d of depth %d (stride %d)", who, sp.zi0, xs.d, sp.Di, stride);
+    if ((sp.yD || sp.yzo) && (stride != 1 || sp.yzo < 0 || sp.yzo + xs.d > sp.yD)) mi_die("%s: slab output %d + %d of depth %d (stride %d)", who, sp.yzo, xs.d, sp.yD, stride);
     if (gp.ns || sp.gp2.ns) mi_die("%s: slab-local GroupNorm statistics are not supported", who);
     if (xbf < 0 || xbf > 4 || !(ybf == 0 || ybf == 2 || ybf == 3 || ybf == 4)) mi_die("%s: unsupported storage types (in %d, out %d)", who, xbf, ybf);
     if (xs.n <= 0 || xs.c <= 0 || xs.d <= 0 || xs.h <= 0 || xs.w <= 0 || cout <= 0) return 0;
@@ -208,7 +213,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (fmt == 4 && Ci <= 8) fmt = 8;                  // the network input computes in e4m3 whatever the activations' format (src/lp_f4fwd.cu:37)
     if (sp.x2 && (Cx <= 0 || C2 <= 0)) mi_die("%s: channel split %d of %d", who, sp.c_split, Ci);
     if (sp.x2 && xbf < 3) mi_die("%s: split inputs need MX storage", who);
-    if (sp.up && (!sp.x2 || xbf < 3 || (xs.d & 1) || (xs.h & 1) || (xs.w & 1) || stride != 1)) mi_die("%s: the fused upsample needs an MX split input and even dims", who);
+    if (sp.up && (!sp.x2 || xbf < 3 || ((sp.Di ? sp.Di : xs.d) & 1) || (xs.h & 1) || (xs.w & 1) || stride != 1)) mi_die("%s: the fused upsample needs an MX split input and even dims", who);
     if (osum && (Go <= 0 || cout % Go)) mi_die("%s: %d output channels in %d groups", who, cout, Go);
     if (osum && (cout / Go) % 4 && cout > 32) mi_die("%s: fused output statistics of %d channels need channels per group (%d) to be a multiple of 4", who, cout, cout / Go);
     if (gp.G && ((sp.x2 && sp.gp2.G ? Cx : Ci) % gp.G)) mi_die("%s: GroupNorm groups %d do not divide the channels", who, gp.G);
@@ -219,9 +224,10 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (stem_env < 0) stem_env = getenv("MI_CONV_STEM") ? atoi(getenv("MI_CONV_STEM")) : 1;     // tuning knob: 0 sends these convs to the general kernel
     if (stem_env && fmt == 8 && stride == 1 && !sp.x2 && !act && (xbf == 0 || xbf >= 2) && Ci <= (xbf == 0 ? 16 : 8) && (xbf == ybf || ybf >= 3))
         return conv_stem(who, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp);
-    const int N = xs.n, D = xs.d, H = xs.h, W = xs.w;
-    const int Do = stride == 2 ? (D - 1) / 2 + 1 : D, Ho = stride == 2 ? (H - 1) / 2 + 1 : H, Wo = stride == 2 ? (W - 1) / 2 + 1 : W;   // src/nn_bwd.cu:132-135
+    const int N = xs.n, D = sp.Di ? sp.Di : xs.d, H = xs.h, W = xs.w;           // D: the inputs' depth
+    const int Do = stride == 2 ? (D - 1) / 2 + 1 : xs.d, Ho = stride == 2 ? (H - 1) / 2 + 1 : H, Wo = stride == 2 ? (W - 1) / 2 + 1 : W;   // src/nn_bwd.cu:132-135
     const size_t S = (size_t)D * H * W;
+    const int zlo = sp.Di ? (sp.zi0 > 0 ? sp.zi0 - 1 : 0) : 0, zhi = sp.Di ? (sp.zi0 + xs.d + 1 < D ? sp.zi0 + xs.d + 1 : D) : D;      // input planes this launch reads
     const int fdt = fmt == 8 ? 3 : 4;
     conv_args a; memset(&a, 0, sizeof a);
     // ---- operands: a segment is read as stored when it already is the compute format with nothing to apply, else re-staged once ----
@@ -240,8 +246,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         } else {
             const size_t bytes = (size_t)N * nbp * S * (mx_rb(32, fmt) + 1);
             uint8_t *st = (uint8_t *)mi_ws(s ? MI_WS_X2STAGE : MI_WS_XSTAGE, bytes);
-            if (upseg) mi_restage_up(segx[s], xbf, N, segC[s], D, H, W, g, Cg, st, fmt);
-            else mi_restage(segx[s], xbf, N, segC[s], S, g, Cg, cg0, st, fmt);
+            if (upseg) mi_restage_up_sub(segx[s], xbf, N, segC[s], D, H, W, g, Cg, st, fmt, zlo, zhi);
+            else mi_restage_sub(segx[s], xbf, N, segC[s], (size_t)(zhi - zlo) * H * W, g, Cg, cg0, st, fmt, S, (size_t)zlo * H * W);
             a.xq[s] = st; a.xsc[s] = st + (size_t)N * nbp * S * mx_rb(32, fmt);
             a.nbs[s] = nbp; a.bws[s] = 32;
         }
@@ -250,6 +256,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     a.nbt = a.nb0p + (sp.x2 ? (C2 + 31) / 32 : 0);
     a.wide = a.bws[0] == 32 && (!sp.x2 || a.bws[1] == 32);
     a.N = N; a.D = D; a.H = H; a.W = W; a.Do = Do; a.Ho = Ho; a.Wo = Wo;
+    a.zi0 = sp.Di ? sp.zi0 : 0; a.yD = sp.yD; a.yzo = sp.yD ? sp.yzo : 0;
     a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
     a.osum = osum; a.Go = Go; a.stored_stats = sp.stored_stats && ybf >= 3; a.zs0 = sp.zlo; a.zs1 = Do - sp.zhi;
     a.ep_a = ep_a; a.ep_b = ep_b; a.act = act;

@@ -87,7 +87,9 @@ struct conv_args {
     int nb0p;                          // padded blocks of segment 0 (staged blocks [0, nb0p) come from segment 0)
     int nbt, CB;                       // staged 32-channel blocks in total, blocks per LDS chunk
     int wide;                          // every staged tensor has 32-channel blocks
-    int N, D, H, W, Do, Ho, Wo;
+    int N, D, H, W, Do, Ho, Wo;       // D x H x W: the staged input tensors; Do x Ho x Wo: the output planes this launch computes
+    int zi0;                           // z-range: output plane z reads input plane z + zi0 (stride 1)
+    int yD, yzo;                       // direct slab output: the MX output is planes [yzo, yzo + Do) of a depth-yD tensor (yD 0: a depth-Do tensor)
     const uint8_t *wq, *wsc; int nmt_all;
     const float *bias; int Co;
     void *y; int ydt;
@@ -233,7 +235,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                                               int oz0, int oy0, int ox0, int lz, int ly0, int tid) {
     const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
     // accumulator layout of the 32x32 MFMA: lane (r = voxel within the tile, h), register i -> channel (i & 3) + 4 h + 8 (i >> 2)
-    const size_t So = (size_t)a.Do * a.Ho * a.Wo;
+    const size_t So = (size_t)(a.yD ? a.yD : a.Do) * a.Ho * a.Wo;      // voxels per channel plane of the output tensor
     const int co_base = cs * MT * 32;
     float *red = (float *)(lds + a.red_o);          // stats scratch [4 waves][MT][8 quads][2] floats
     const bool stats = a.osum != nullptr;
@@ -268,7 +270,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
             constexpr int j = J;
             const int oz = oz0 + lz, oy = oy0 + ly0 + 2 * j + (r >> 4), ox = ox0 + (r & 15);
             const bool ok = oz < a.Do && oy < a.Ho && ox < a.Wo;
-            const size_t ov = ((size_t)oz * a.Ho + oy) * a.Wo + ox;
+            const size_t ov = ((size_t)(oz + a.yzo) * a.Ho + oy) * a.Wo + ox;
             const bool zst = ok && oz >= a.zs0 && oz < a.zs1;
             float v[16];
             float am = 0.f;
@@ -444,7 +446,7 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     const int ty = tt % a.nty; tt /= a.nty;
     const int tz = tt % a.ntz; const int n = tt / a.ntz;
     const int ox0 = tx * 16, oy0 = ty * 8, oz0 = tz * TZ;
-    const int ix0 = STRIDE * ox0 - 1, iy0 = STRIDE * oy0 - 1, iz0 = STRIDE * oz0 - 1;
+    const int ix0 = STRIDE * ox0 - 1, iy0 = STRIDE * oy0 - 1, iz0 = STRIDE * oz0 - 1 + a.zi0;
 
     // the lane's voxel in each of its NT tiles: wave -> (z, y half) for TZ 2, z for TZ 4; tile j -> rows 2j, 2j+1; r -> (row, x)
     int lz, ly0;

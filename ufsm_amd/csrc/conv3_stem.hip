@@ -61,7 +61,7 @@ __global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
 #pragma unroll
     for (int j = 0; j < 3; j++) {
         const int pos = tid + 256 * j, ix = pos % HX, iy = (pos / HX) % HY, iz = pos / (HY * HX);
-        const int gz = oz0 - 1 + iz, gy = oy0 - 1 + iy, gx = ox0 - 1 + ix;
+        const int gz = oz0 - 1 + iz + a.zi0, gy = oy0 - 1 + iy, gx = ox0 - 1 + ix;
         const bool inb = pos < TT && (unsigned)gz < (unsigned)a.D && (unsigned)gy < (unsigned)a.H && (unsigned)gx < (unsigned)a.W;
         const size_t off = inb ? ((size_t)gz * a.H + gy) * a.W + gx : 0;
         float x[CP];

@@ -87,7 +87,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         const size_t plane = (size_t)n * a.nbs[seg] + min(max(bl, 0), a.nbs[seg] - 1);
         const int pos = g * 64 + lane;
         const int pz = pos / (HY * HX), rem = pos - pz * (HY * HX), py = rem / HX, px = rem - py * HX;
-        const int gz = oz0 - 1 + pz, gy = oy0 - 1 + py, gx = ox0 - 1 + px;
+        const int gz = oz0 - 1 + pz + a.zi0, gy = oy0 - 1 + py, gx = ox0 - 1 + px;
         const bool in = bok && pos < TT && gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
         const size_t vox = (size_t)(unsigned)((gz * a.H + gy) * a.W + gx);
         q.row = in ? a.xq[seg] + (plane * Sin + vox) * (16 * NH) : a.zpage;

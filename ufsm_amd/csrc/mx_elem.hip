@@ -138,11 +138,64 @@ __global__ void __launch_bounds__(256) gn_silu_apply_mx_k(const void *xv, uint8_
     }
     store_row<BY, true>(y, mx_scp<BY>(y, N, C, S), i, bw, r);
 }
+// the same for an MX source of 32-channel blocks, two lanes per row (each lane one contiguous 16-channel half in and out, the per-channel
+// mean / rstd / gamma / beta of the block in LDS): a wavefront reads and writes contiguous memory
+template <int BX, int BY>
+__global__ void __launch_bounds__(256) gn_silu_apply32_k(const uint8_t *x, uint8_t *y, int N, int C, int G, size_t S, const float *gamma, const float *beta, const float *mean, const float *rstd) {
+    const int nb = C / 32, blk = blockIdx.y, n = blockIdx.z;
+    __shared__ float4 co[32];                                      // (mean, rstd, gamma, beta) of the block's channels
+    if (threadIdx.x < 32) { const int c = blk * 32 + threadIdx.x, ng = n * G + c / (C / G); co[threadIdx.x] = make_float4(mean[ng], rstd[ng], gamma[c], beta[c]); }
+    __syncthreads();
+    const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;
+    const size_t v = t >> 1; const int hf = (int)(t & 1);
+    if (v >= S) return;
+    constexpr int IB = BX * 2, OB = BY * 2;                        // bytes of a 16-channel half row
+    const size_t row = ((size_t)n * nb + blk) * S + v;
+    const uint8_t *xs = x + (size_t)N * nb * S * (IB * 2);
+    uint8_t *ys = y + (size_t)N * nb * S * (OB * 2);
+    unsigned w[4] = {0u, 0u, 0u, 0u};
+    if (BX == 8) { const uint4 q = *(const uint4 *)(x + row * 32 + hf * 16); w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w; }
+    else { const uint2 q = *(const uint2 *)(x + row * 16 + hf * 8); w[0] = q.x; w[1] = q.y; }
+    const float sc = d_mx_scale(xs[row]);
+    float r[16];
+    if (BX == 8) { d_dec4_e4m3(w[0], r); d_dec4_e4m3(w[1], r + 4); d_dec4_e4m3(w[2], r + 8); d_dec4_e4m3(w[3], r + 12); }
+    else { d_dec8_e2m1(w[0], r); d_dec8_e2m1(w[1], r + 8); }
+    unsigned am = 0u;
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        const float4 q = co[hf * 16 + k];
+        const float u = fmaf((r[k] * sc - q.x) * q.y, q.z, q.w);
+        r[k] = __fdividef(u, 1.f + __expf(-u));
+        am = d_amax_u(am, r[k]);
+    }
+    const unsigned ao = (unsigned)__shfl_xor((int)am, 1);
+    am = ao > am ? ao : am;
+    const int e = d_mx_exp(__uint_as_float(am), BY == 8 ? MI_INVQ8 : MI_INVQ4);
+    if (BY == 8) {
+        uint4 o;
+        o.x = d_enc4_e4m3(r[0], r[1], r[2], r[3], e); o.y = d_enc4_e4m3(r[4], r[5], r[6], r[7], e);
+        o.z = d_enc4_e4m3(r[8], r[9], r[10], r[11], e); o.w = d_enc4_e4m3(r[12], r[13], r[14], r[15], e);
+        *(uint4 *)(y + row * 32 + hf * 16) = o;
+    } else {
+        uint2 o; o.x = d_enc8_e2m1(r, e); o.y = d_enc8_e2m1(r + 8, e);
+        *(uint2 *)(y + row * 16 + hf * 8) = o;
+    }
+    if (!hf) ys[row] = (uint8_t)(e + 127);
+}
 extern "C" void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, const float *gamma, const float *beta, const float *mean, const float *rstd, void *y, int ydt) {
     const size_t S = (size_t)s.d * s.h * s.w, n = (size_t)s.n * mx_nb(s.c) * S;
     if (ydt != 3 && ydt != 4) mi_die("lp_gn_silu_apply_mx: output dtype %d is not MX", ydt);
     if (G <= 0 || s.c % G) mi_die("lp_gn_silu_apply_mx: %d channels in %d groups", s.c, G);
     if (!n) return;
+    if (xdt >= 3 && s.c % 32 == 0) {
+        const dim3 grid(nblk_(2 * S, 256), (unsigned)(s.c / 32), (unsigned)s.n);
+        const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
+#define GS32(BX, BY) gn_silu_apply32_k<BX, BY><<<grid, 256>>>(xq, yq, s.n, s.c, G, S, gamma, beta, mean, rstd)
+        if (xdt == 3) { if (ydt == 3) GS32(8, 8); else GS32(8, 4); } else { if (ydt == 3) GS32(4, 8); else GS32(4, 4); }
+#undef GS32
+        MICK();
+        return;
+    }
 #define GSA(BX, BY, TI) gn_silu_apply_mx_k<BX, BY, TI><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, s.n, s.c, G, S, gamma, beta, mean, rstd)
 #define GSA_Y(BX, TI) do { if (ydt == 4) GSA(BX, 4, TI); else GSA(BX, 8, TI); } while (0)
     if (xdt == 4) GSA_Y(4, float); else if (xdt == 3) GSA_Y(8, float); else if (xdt == 2) GSA_Y(0, __half); else if (xdt == 1) GSA_Y(0, bf16_t); else GSA_Y(0, float);
@@ -233,8 +286,26 @@ extern "C" void lp_add_mx(void *y, const void *x, shape5 s, int dt, unsigned sr)
 }
 
 // ---- GroupNorm (sum, sum of squares) of a stored MX tensor into fixed-point slots (src/lp_mx_gnsums.cu:8-101) ----
-// A block reduces a slab of voxels of one (n, channel block): per-thread fp64 partials per channel, a tree over the block in LDS
-// (fixed order: deterministic), one slot add per channel group touched.
+// Sums 32 per-lane fp64 values over the 32 lanes of each wavefront half in a fixed order: step k pairs lane r with r ^ 2^k and the pair
+// splits the values left (the lane whose bit k is clear keeps the lower half of the indices and receives the partner's). Returns the index
+// of the value whose total the lane holds in v[0] afterwards: sum over k of bit k of r times 16 >> k.
+__device__ __forceinline__ int wave_half_reduce_f64(double (&v)[32], int r) {
+    int idx = 0;
+#pragma unroll
+    for (int k = 0; k < 5; k++) {
+        const int half = 16 >> k;
+        const bool bit = (r >> k) & 1;
+#pragma unroll
+        for (int i = 0; i < half; i++) {
+            const double send = bit ? v[i] : v[i + half], keep = bit ? v[i + half] : v[i];
+            v[i] = keep + __shfl_xor(send, 1 << k);
+        }
+        idx += bit ? half : 0;
+    }
+    return idx;
+}
+// A block reduces a slab of voxels of one (n, channel block): per-thread fp64 partials per channel, then a fixed-order (deterministic)
+// reduction over the block.
 template <int B>
 __global__ void __launch_bounds__(256) gn_sums_mx_k(const uint8_t *x, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1, int n0) {
     const int bw = mx_bw(C), nb = mx_nb(C), cpg = C / G, blk = blockIdx.y, n = n0 + (int)blockIdx.z, nsl = gridDim.x;
@@ -249,22 +320,29 @@ __global__ void __launch_bounds__(256) gn_sums_mx_k(const uint8_t *x, int N, int
 #pragma unroll
         for (int k = 0; k < 32; k++) { const double d = (double)r[k]; s1[k] += d; s2[k] += d * d; }
     }
-    __shared__ double red[256];
-    for (int k = 0; k < bw; k++) {
-        const int c = blk * bw + k; if (c >= C) break;
-        for (int pass = 0; pass < 2; pass++) {
-            red[threadIdx.x] = pass ? s2[k] : s1[k];
-            __syncthreads();
-            for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) red[threadIdx.x] += red[threadIdx.x + st]; __syncthreads(); }
-            if (threadIdx.x == 0) gn_acc_add(sums, 2 * ((size_t)n * G + c / cpg) + pass, red[0]);
-            __syncthreads();
+    // each channel's partials: a fixed-order exchange tree over the 32 lanes of a wavefront half (every step halves the values a lane
+    // carries), the other half by one more exchange, the four wavefronts through LDS; then one slot add per channel and moment
+    const int lane = threadIdx.x & 63, r = lane & 31;
+    const int i1 = wave_half_reduce_f64(s1, r), i2 = wave_half_reduce_f64(s2, r);
+    const double t1 = s1[0] + __shfl_xor(s1[0], 32), t2 = s2[0] + __shfl_xor(s2[0], 32);
+    __shared__ double red[4][64], tot[64];
+    if (lane < 32) { red[threadIdx.x >> 6][i1] = t1; red[threadIdx.x >> 6][32 + i2] = t2; }
+    __syncthreads();
+    if (threadIdx.x < 64) tot[threadIdx.x] = ((red[0][threadIdx.x] + red[1][threadIdx.x]) + red[2][threadIdx.x]) + red[3][threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x < 64) {                                  // the first channel of every group inside the block adds the group's channels in order
+        const int k = threadIdx.x & 31, pass = threadIdx.x >> 5, c = blk * bw + k, g = c / cpg;
+        if (k < bw && c < C && (k == 0 || (c - 1) / cpg != g)) {
+            double acc = 0.0;
+            for (int kk = k; kk < bw && blk * bw + kk < C && (blk * bw + kk) / cpg == g; kk++) acc += tot[pass * 32 + kk];
+            gn_acc_add(sums, 2 * ((size_t)n * G + g) + pass, acc);
         }
     }
 }
 extern "C" int lp_gn_sums_mx_n(const void *x, int xdt, int N, int C, int G, size_t S, double *sums, size_t v0, size_t v1, int n0, int cnt) {
     if ((xdt != 3 && xdt != 4) || G <= 0 || C % G) return -1;
     if (v1 <= v0 || cnt <= 0) return 0;
-    size_t nsl = (v1 - v0 + 4095) / 4096; if (nsl > 1024) nsl = 1024;
+    size_t nsl = (v1 - v0 + 8191) / 8192; if (nsl > 512) nsl = 512;      // (few, large slabs: every block ends in atomic adds to the same few slots)
     const dim3 grid((unsigned)nsl, (unsigned)mx_nb(C), (unsigned)cnt);
     if (xdt == 4) gn_sums_mx_k<4><<<grid, 256>>>((const uint8_t *)x, N, C, G, S, sums, v0, v1, n0);
     else gn_sums_mx_k<8><<<grid, 256>>>((const uint8_t *)x, N, C, G, S, sums, v0, v1, n0);
@@ -353,20 +431,20 @@ extern "C" int lp_conv1_fwd_mx_r(const void *x, int xdt, shape5 xs, const float 
 // ---- operand re-staging for the conv dispatch (the arithmetic of src/lp_f8fwd.cuh:88-113 applied once per tensor instead of once per
 // staged halo position): any source (planes or MX) -> optional GN + SiLU (staging form) -> rows in the compute format, blocks of 32 ----
 template <int BX, int BY, typename TI>
-__global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0) {
-    // y: an MX tensor of nbo * 32 channels (bw 32). gp over Cg channels of which this tensor holds [cg0, cg0 + C) (whole-input GroupNorm of a split input)
+__global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, size_t Ss, size_t v0) {
+    // voxels [v0, v0 + S) of tensors holding Ss voxels per (sample, channel / block), source and result alike; y: an MX tensor of nbo * 32 channels (bw 32). gp over Cg channels of which this tensor holds [cg0, cg0 + C) (whole-input GroupNorm of a split input)
     const int nbo = (C + 31) / 32, bwx = mx_bw(C), Cy = nbo * 32;
     const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     if (i >= (size_t)N * nbo * S) return;
     const size_t v = i % S; const int blk = (int)((i / S) % nbo), n = (int)(i / (S * nbo));
     float r[32];
     if (BX != 0) {
-        const uint8_t *x = (const uint8_t *)xv; const uint8_t *sc = mx_scp<BX ? BX : 8>(x, N, C, S);
-        if (bwx == 32) load_row<BX ? BX : 8>(x, sc, ((size_t)n * mx_nb(C) + blk) * S + v, 32, r);
-        else load_row<BX ? BX : 8>(x, sc, (size_t)n * S + v, bwx, r);           // C <= 16: one narrow block, zero-extended
+        const uint8_t *x = (const uint8_t *)xv; const uint8_t *sc = mx_scp<BX ? BX : 8>(x, N, C, Ss);
+        if (bwx == 32) load_row<BX ? BX : 8>(x, sc, ((size_t)n * mx_nb(C) + blk) * Ss + v0 + v, 32, r);
+        else load_row<BX ? BX : 8>(x, sc, (size_t)n * Ss + v0 + v, bwx, r);     // C <= 16: one narrow block, zero-extended
     } else {
 #pragma unroll
-        for (int k = 0; k < 32; k++) { const int c = blk * 32 + k; r[k] = c < C ? ldx((const TI *)xv, ((size_t)n * C + c) * S + v) : 0.f; }
+        for (int k = 0; k < 32; k++) { const int c = blk * 32 + k; r[k] = c < C ? ldx((const TI *)xv, ((size_t)n * C + c) * Ss + v0 + v) : 0.f; }
     }
     if (gp.G) {
         const int cpg = Cg / gp.G;
@@ -377,13 +455,13 @@ __global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int
             else r[k] = 0.f;
         }
     }
-    store_row<BY, false>(y, mx_scp<BY>(y, N, Cy, S), i, 32, r);
+    store_row<BY, false>(y, mx_scp<BY>(y, N, Cy, Ss), ((size_t)n * nbo + blk) * Ss + v0 + v, 32, r);
 }
 // the same for an MX source with 32-wide blocks, two lanes per row: each lane moves one 16-channel half (16 or 8 contiguous bytes in,
 // 16 or 8 out), so a wavefront reads and writes contiguous memory; the halves' amaxes meet through one lane exchange. The (a, b)
 // coefficients of the block's 32 channels are formed once per workgroup in LDS. HBM-bound: (bits_in + bits_out) / 8 + 2/32 bytes per element.
 template <int BX, int BY>
-__global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0) {
+__global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, size_t Ss, size_t v0) {
     const int nb = C / 32, blk = blockIdx.y, n = blockIdx.z;
     __shared__ float sa[32], sb[32];
     if (threadIdx.x < 32) {
@@ -396,9 +474,9 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
     const size_t v = t >> 1; const int hf = (int)(t & 1);
     if (v >= S) return;                                            // (S even or odd: the pair of lanes of a row leaves together)
     constexpr int IB = BX * 2, OB = BY * 2;                        // bytes of a 16-channel half row
-    const size_t row = ((size_t)n * nb + blk) * S + v;
-    const uint8_t *xs = x + (size_t)N * nb * S * (IB * 2);
-    uint8_t *ys = y + (size_t)N * nb * S * (OB * 2);
+    const size_t row = ((size_t)n * nb + blk) * Ss + v0 + v;
+    const uint8_t *xs = x + (size_t)N * nb * Ss * (IB * 2);
+    uint8_t *ys = y + (size_t)N * nb * Ss * (OB * 2);
     unsigned w[4] = {0u, 0u, 0u, 0u};
     if (BX == 8) { const uint4 q = *(const uint4 *)(x + row * 32 + hf * 16); w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w; }
     else { const uint2 q = *(const uint2 *)(x + row * 16 + hf * 8); w[0] = q.x; w[1] = q.y; }
@@ -427,23 +505,25 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
     }
     if (!hf) ys[row] = (uint8_t)(e + 127);
 }
-void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits) {
+// voxels [v0, v0 + S) of tensors holding Ss voxels per (sample, channel / block): the result has the source's geometry, only that range is written
+void mi_restage_sub(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits, size_t Ss, size_t v0) {
     const size_t n = (size_t)N * ((C + 31) / 32) * S; if (!n) return;
     if (xdt >= 3 && C % 32 == 0) {
         const dim3 grid(nblk_(2 * S, 256), (unsigned)(C / 32), (unsigned)N);
         const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
-        if (xdt == 3) { if (ybits == 8) restage32_k<8, 8><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0); else restage32_k<8, 4><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0); }
-        else { if (ybits == 8) restage32_k<4, 8><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0); else restage32_k<4, 4><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0); }
+        if (xdt == 3) { if (ybits == 8) restage32_k<8, 8><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0, Ss, v0); else restage32_k<8, 4><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0, Ss, v0); }
+        else { if (ybits == 8) restage32_k<4, 8><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0, Ss, v0); else restage32_k<4, 4><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0, Ss, v0); }
         MICK();
         return;
     }
-#define RS(BX, BY, TI) restage_k<BX, BY, TI><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, N, C, S, gp, Cg, cg0)
+#define RS(BX, BY, TI) restage_k<BX, BY, TI><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, N, C, S, gp, Cg, cg0, Ss, v0)
 #define RS_Y(BX, TI) do { if (ybits == 4) RS(BX, 4, TI); else RS(BX, 8, TI); } while (0)
     if (xdt == 4) RS_Y(4, float); else if (xdt == 3) RS_Y(8, float); else if (xdt == 2) RS_Y(0, __half); else if (xdt == 1) RS_Y(0, bf16_t); else RS_Y(0, float);
 #undef RS_Y
 #undef RS
     MICK();
 }
+void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits) { mi_restage_sub(x, xdt, N, C, S, gp, Cg, cg0, y, ybits, S, 0); }
 // decoder up segment (src/lp_common.cuh:618-670): coarse rows -> GN + SiLU -> e4m3 rows with a row scale (amax ignoring NaN) -> 8-term fp32
 // blend (weights .75 / .25, fma order z, y, x, the row scale folded into the weight) -> rows in the compute format at the fine resolution.
 // Two passes: the coarse rows are activated and re-quantised once (mi_restage into an MX-fp8 scratch tensor, an eighth of the output),
@@ -451,22 +531,24 @@ void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg
 // block's 32 channels: cell (mz, my, mx), each in [-1, dim/2 - 1], covers coarse {m, m + 1} (clamped) and fine {2m + 1, 2m + 2}; the four
 // threads of a cell meet for the row amax through lane exchanges. Each coarse row is decoded once per cell instead of once per fine voxel.
 template <int BY>
-__global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y, int N, int nbo, int D, int H, int W) {
+__global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y, int N, int nbo, int D, int H, int W, int zlo, int zhi, int clo, int Dcs, int mz0, int ncz_) {
+    // fine planes [zlo, zhi) of the depth-D result, written at their place in the depth-D tensor y; xc holds the coarse planes [clo, clo + Dcs)
+    // compactly; cells mz0 .. mz0 + ncz_ - 1 along z (the whole tensor: zlo 0, zhi D, clo 0, Dcs D / 2, mz0 -1, ncz_ D / 2 + 1)
     const int Dc = D >> 1, Hc = H >> 1, Wc = W >> 1;
-    const size_t S = (size_t)D * H * W, Sc = (size_t)Dc * Hc * Wc;
+    const size_t S = (size_t)D * H * W, Sc = (size_t)Dcs * Hc * Wc;
     const int nbk = blockIdx.y;                                                   // (n, blk)
     const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;
     const int q = (int)(t & 3);
-    const size_t cell = t >> 2, ncx = (size_t)Wc + 1, ncy = (size_t)Hc + 1, ncz = (size_t)Dc + 1;
+    const size_t cell = t >> 2, ncx = (size_t)Wc + 1, ncy = (size_t)Hc + 1, ncz = (size_t)ncz_;
     const bool live = cell < ncx * ncy * ncz;
     const size_t cc = live ? cell : 0;
-    const int mx = (int)(cc % ncx) - 1, my = (int)((cc / ncx) % ncy) - 1, mz = (int)(cc / (ncx * ncy)) - 1;
+    const int mx = (int)(cc % ncx) - 1, my = (int)((cc / ncx) % ncy) - 1, mz = (int)(cc / (ncx * ncy)) + mz0;
     const int cz[2] = {max(mz, 0), min(mz + 1, Dc - 1)}, cy[2] = {max(my, 0), min(my + 1, Hc - 1)}, cx[2] = {max(mx, 0), min(mx + 1, Wc - 1)};
     const uint8_t *xs = xc + (size_t)N * nbo * Sc * 32;
     float f[8][8], sc[8];
 #pragma unroll
     for (int k = 0; k < 8; k++) {
-        const size_t row = (size_t)nbk * Sc + ((size_t)cz[k >> 2] * Hc + cy[(k >> 1) & 1]) * Wc + cx[k & 1];
+        const size_t row = (size_t)nbk * Sc + ((size_t)(cz[k >> 2] - clo) * Hc + cy[(k >> 1) & 1]) * Wc + cx[k & 1];
         const uint2 w = *(const uint2 *)(xc + row * 32 + q * 8);
         d_dec4_e4m3(w.x, f[k]); d_dec4_e4m3(w.y, f[k] + 4);
         sc[k] = d_mx_scale(xs[row]);
@@ -495,7 +577,7 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
         for (int i = 0; i < 8; i++) am = fmaxf(am, fabsf(acc[i]));
         am = fmaxf(am, __shfl_xor(am, 1)); am = fmaxf(am, __shfl_xor(am, 2));
         const int e = d_mx_exp(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
-        if (!live || gz < 0 || gz >= D || gy < 0 || gy >= H || gx < 0 || gx >= W) continue;
+        if (!live || gz < zlo || gz >= zhi || gy < 0 || gy >= H || gx < 0 || gx >= W) continue;
         const size_t row = (size_t)nbk * S + ((size_t)gz * H + gy) * W + gx;
         if (BY == 8) {
             uint2 o; o.x = d_enc4_e4m3(acc[0], acc[1], acc[2], acc[3], e); o.y = d_enc4_e4m3(acc[4], acc[5], acc[6], acc[7], e);
@@ -504,16 +586,22 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
         if (!q) ys[row] = (uint8_t)(e + 127);
     }
 }
-void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits) {
-    const size_t S = (size_t)D * H * W; if (!S || !N) return;
+// fine planes [zlo, zhi) of the upsampled depth-D tensor, written at their place in the depth-D MX tensor y
+void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int zlo, int zhi) {
+    if (!N || zhi <= zlo || !H || !W) return;
     if (xdt != 3 && xdt != 4) mi_die("fused-upsample input must be an MX tensor (dtype %d)", xdt);
     if ((D | H | W) & 1) mi_die("fused-upsample output dims must be even (%d %d %d)", D, H, W);
-    const int nbo = (C + 31) / 32;
-    const size_t Sc = S / 8;
-    uint8_t *xc = (uint8_t *)mi_ws(MI_WS_UPCOARSE, (size_t)N * nbo * Sc * 33);
-    mi_restage(x, xdt, N, C, Sc, gp, Cg, 0, xc, 8);
-    const size_t cells = (size_t)(D / 2 + 1) * (H / 2 + 1) * (W / 2 + 1);
+    const int nbo = (C + 31) / 32, Dc = D / 2;
+    // cells mz cover fine planes 2 mz + 1, 2 mz + 2 and read coarse planes mz, mz + 1 (clamped)
+    const int mz0 = (zlo - 2) >> 1 < -1 ? -1 : (zlo - 2) >> 1, mz1 = (zhi - 2) >> 1, ncz = mz1 - mz0 + 1;
+    const int clo = mz0 < 0 ? 0 : mz0, chi = (mz1 + 1 > Dc - 1 ? Dc - 1 : mz1 + 1) + 1, Dcs = chi - clo;
+    const size_t Scp = (size_t)(H / 2) * (W / 2);
+    uint8_t *xc = (uint8_t *)mi_ws(MI_WS_UPCOARSE, (size_t)N * nbo * Dc * Scp * 33);          // the coarse tensor's geometry; planes [clo, clo + Dcs) are filled
+    mi_restage_sub(x, xdt, N, C, (size_t)Dcs * Scp, gp, Cg, 0, xc, 8, (size_t)Dc * Scp, (size_t)clo * Scp);
+    const size_t cells = (size_t)ncz * (H / 2 + 1) * (W / 2 + 1);
     const dim3 grid(nblk_(cells * 4, 256), (unsigned)(N * nbo));
-    if (ybits == 4) up_blend_k<4><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W); else up_blend_k<8><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W);
+    if (ybits == 4) up_blend_k<4><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W, zlo, zhi, 0, Dc, mz0, ncz);
+    else up_blend_k<8><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W, zlo, zhi, 0, Dc, mz0, ncz);
     MICK();
 }
+void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits) { mi_restage_up_sub(x, xdt, N, C, D, H, W, gp, Cg, y, ybits, 0, D); }
