@@ -27,6 +27,10 @@ int nn_conv3d_fwd_gn_stats(const float *x, shape5 xs, int G_in, const float *gam
 /* input-side recompute conv: k 3 stride 1 (split / fused upsample / output statistics), k 3 stride 2, k 1 head (src/nn.h:432) */
 int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn_gn_t *gx2, int c_split, int up, shape5 xs,
                     const float *w, const float *b, int cout, int k, int stride, float *y, int G_out, float eps, float *omean, float *orstd);
+void nn_set_zrange(int zi0, int Di, int first, int last, int Do, int zo);   /* the next stride-1 MX convs compute output planes [zo, zo + xs.d) of a depth-Do tensor, plane z reading
+                                                                               input plane z + zi0 of a depth-Di input; sums zeroed by the first, finalised by the last call; Di 0 = off
+                                                                               (src/nn_bwd.cu:33-36) */
+void nn_set_zrange_out(int on);                                /* ... straight into their planes of the depth-Do MX output (src/nn_bwd.cu:41-42) */
 int nn_gn_stats(const float *x, shape5 s, int G, float eps, float *mean, float *rstd);   /* of a stored MX tensor; -1 when unsupported (src/nn.h:484) */
 const char *nn_check(void);                                    /* src/nn.h:28 */
 
@@ -74,6 +78,9 @@ int unet_read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step
 int unet_load(unet *u, const char *path);
 int unet_load_ema(unet *u, const char *path);
 int unet_save(const unet *u, const char *path, int step, const char *extra);   /* extra: a JSON object for the header's "extra" key, or null */
+void unet_set_infer_slab(int planes);                         /* inference: the level-0 convs in z-slabs of this many planes (rounded up to a multiple of 4), each slab written
+                                                                 straight into the full-depth tensors; byte-identical logits; 0 = off (src/unet.h:422-424, direct slab outputs) */
+int unet_get_infer_slab(void);
 shape5 unet_in_shape(const unet *u);                          /* the window the graph was created for */
 const unet_cfg *unet_config(const unet *u);
 /* ---- sliding-window prediction of a volume resident in device memory (src/predict.c: the --feather single pass, :282-333, :2538-2545,

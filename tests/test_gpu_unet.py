@@ -235,3 +235,48 @@ def test_checkpoint_round_trip(gpu, tmp_path):
     open(str(tmp_path / "film.ckpt"), "wb").write(head.replace(',"cin":', ',"film":2,"cin":').encode() + b"\0" * (8 * pa.size))
     assert H_.unet_read_header(str(tmp_path / "film.ckpt").encode(), C.byref(c2), None, None) == -2
     a.close(); b.close(); other.close()
+
+
+@pytest.mark.parametrize("bits,dims,slab,attn", [(8, (32, 32, 32), 8, 0), (8, (24, 16, 32), 16, 0), (4, (16, 32, 32), 4, 0), (8, (32, 32, 32), 16, 1)])
+def test_slab_inference_is_byte_identical(gpu, bits, dims, slab, attn):
+    """unet_set_infer_slab: the level-0 convs (stem, encoder conv2, decoder conv1 over [up | skip], decoder conv2) run in z-slabs through the
+    z-range with direct slab outputs; logits, every stored tensor and every GroupNorm statistic equal the whole-tensor forward's
+    (tests/test_infer_mem.c: byte-identical logits)."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    H_ = load_host()
+    rng = np.random.default_rng(slab + bits)
+    D, H, W = dims
+    N, S = 2, D * H * W
+    widths = [32, 96] if attn else [32, 64]
+    net = UNet(make_cfg(4, widths, G=8, head_out=3, act_dt=bits, attn_blocks=attn, attn_pe=1, down_norm=1), N, D, H, W, seed=5)
+    x = rng.standard_normal((N, 4, S)).astype(np.float32); dxq = to_mx(bits, x)
+    la, lb = DevBuf(N * 3 * S * 4), DevBuf(N * 3 * S * 4)
+    assert H_.unet_get_infer_slab() == 0
+    assert net.forward_x(dxq.ptr, la.ptr) == 0
+    LP.check()
+    def fetch():
+        out = {}
+        for k, (name, ptr, shp) in enumerate(net.layer_outs()):
+            nb = (lib.lp_mx8_bytes if bits == 8 else lib.lp_mx4_bytes)(shp[0], shp[1], shp[2] * shp[3] * shp[4])
+            buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+            g, mp, rp = net.layer_stats(k)
+            m = np.empty(N * g, np.float32); r = np.empty(N * g, np.float32)
+            if g:
+                lib.mi_d2h(m.ctypes.data, mp, m.nbytes); lib.mi_d2h(r.ctypes.data, rp, r.nbytes)
+            out[name] = (buf, m, r)
+        return out
+    whole = fetch()
+    assert {"enc0.c1", "enc0.c2", "dec0.c1", "dec0.c2"} <= set(whole)
+    H_.unet_set_infer_slab(slab - 1)                       # rounded up to a multiple of 4
+    try:
+        assert H_.unet_get_infer_slab() == slab
+        assert net.forward_x(dxq.ptr, lb.ptr) == 0
+        LP.check()
+    finally:
+        H_.unet_set_infer_slab(0)
+    assert np.array_equal(la.to_numpy(np.float32), lb.to_numpy(np.float32))
+    slabbed = fetch()
+    for name, (t, m, r) in whole.items():
+        t2, m2, r2 = slabbed[name]
+        assert np.array_equal(t2, t) and np.array_equal(m2, m) and np.array_equal(r2, r), name
+    net.close()

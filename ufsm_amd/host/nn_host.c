@@ -44,6 +44,14 @@ static double *gn_dsums(size_t nslots) {
 /* statistics of the decoded stored output instead of the pre-quantisation values (gn_fused_stored, src/nn_bwd.cu:67-72) */
 static int gn_fused_stored(int ydt, int cout) { return g_gn_stored && ydt >= 3 && cout >= 16; }
 
+/* z-range (src/nn_bwd.cu:33-46): the next 3^3 stride-1 MX convs compute output planes [zo, zo + xs.d) of a depth-Do tensor, output plane z
+   reading input plane z + zi0 of a depth-Di input; their output GroupNorm sums are zeroed only by the first slab's call and finalised
+   (over all Do planes) only by the last's. Di 0 = off. With nn_set_zrange_out the MX outputs go straight to their planes of the depth-Do
+   output tensor instead of a depth-xs.d one. Per host thread. */
+static _Thread_local int g_zr_z0, g_zr_Di, g_zr_first, g_zr_last, g_zr_Do, g_zr_zo, g_zr_out;
+void nn_set_zrange(int zi0, int Di, int first, int last, int Do, int zo) { g_zr_z0 = zi0; g_zr_Di = Di; g_zr_first = first; g_zr_last = last; g_zr_Do = Do; g_zr_zo = zo; }
+void nn_set_zrange_out(int on) { g_zr_out = on; }
+
 int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn_gn_t *gx2, int c_split, int up, shape5 xs,
                     const float *w, const float *b, int cout, int k, int stride, float *y, int G_out, float eps, float *omean, float *orstd) {
     const int xdt = lp_dt(x), ydt = lp_dt(y);
@@ -74,6 +82,15 @@ int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn
     /* MX-fp4 storage or precision 3 run the fp4 kernels, everything else fp8; the <= 8 channel network input always runs in fp8
        (src/nn_bwd.cu:110-112, src/lp_f4fwd.cu:37) */
     const int f4 = (xdt == 4 || g_prec == 3) && xs.c > 8;
+    if (g_zr_Di) {                                                  /* a slab of the conv: zero / accumulate / finalize spread over the calls */
+        if (xdt < 3 || ydt < 3) { fprintf(stderr, "nn_conv3d_fwd_x: the z-range needs MX storage\n"); return -1; }
+        sp.zi0 = (int16_t)g_zr_z0; sp.Di = (int16_t)g_zr_Di;
+        if (g_zr_out) { sp.yzo = (int16_t)g_zr_zo; sp.yD = (int16_t)g_zr_Do; }
+        if (sums && g_zr_first) mi_gn_sums_zero(sums, 2 * xs.n * G_out);
+        (f4 ? lp_conv_fwd_f4 : lp_conv_fwd_f8)(x, xdt, xs, w, b, cout, y, ydt, gp, sums, sums ? G_out : 0, sp);
+        if (sums && g_zr_last) mi_gn_finalize(sums, xs.n * G_out, (size_t)(cout / G_out) * g_zr_Do * xs.h * xs.w, eps, omean, orstd);
+        return 0;
+    }
     /* with output statistics: the conv's reduction sets the slots and finalizes them (the reference's zero / conv / finalize sequence,
        src/nn_bwd.cu:37-56, in one call) */
     if (sums) mi_conv_fwd_gn(f4 ? 4 : 8, x, xdt, xs, w, b, cout, y, ydt, gp, sums, G_out, sp, eps, omean, orstd);

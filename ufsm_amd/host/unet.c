@@ -161,16 +161,28 @@ static void note(unet *u, const void *p, shape5 s, const char *name, const float
 }
 static nn_gn_t gn_out(const unet *u, const block *b) { return (nn_gn_t){P(u, b->n2.gamma), P(u, b->n2.beta), b->m2, b->r2, G_of(u, b->ys.c)}; }   /* silu(gn(a2)) for the block's readers */
 
+/* inference in z-slabs (src/unet.h:422-424, src/unet.c:2499-2550 with direct slab outputs): the level-0 convs run slab by slab through the
+   z-range, each slab's planes written straight into the full-depth output; results are those of the whole-tensor convs */
+static int g_infer_slab;
+void unet_set_infer_slab(int planes) { g_infer_slab = planes > 0 ? (planes + 3) / 4 * 4 : 0; }
+int unet_get_infer_slab(void) { return g_infer_slab; }
+
 /* conv1 -> a1 (+ its statistics), conv2 reads silu(gn(a1)) while staging -> a2 (+ statistics) (src/unet.c:2567-2636) */
-static int block_fwd(unet *u, block *b, const void *x, const nn_gn_t *gin, const void *xup, const nn_gn_t *gup, int c_split, const char *n1, const char *n2) {
-    const int G = G_of(u, b->c1.cout);
-    int r;
-    if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, b->xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, b->a1, G, 1e-5f, b->m1, b->r1);   /* [up2(coarse) | skip] */
-    else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, b->xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, b->a1, G, 1e-5f, b->m1, b->r1);
-    if (r) return r;
-    note(u, b->a1, b->ys, n1, b->m1, b->r1, G);
-    r = nn_conv3d_fwd_gn_stats(b->a1, b->ys, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, b->a2, G, 1e-5f, b->m2, b->r2);
-    note(u, b->a2, b->ys, n2, b->m2, b->r2, G);
+static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t *gin, const void *xup, const nn_gn_t *gup, int c_split, const char *n1, const char *n2) {
+    const int G = G_of(u, b->c1.cout), D = b->ys.d, s = level == 0 && g_infer_slab && g_infer_slab < D ? g_infer_slab : 0;
+    int r = 0;
+    for (int conv = 1; conv <= 2 && !r; conv++) {
+        for (int z0 = 0, sk; z0 < D && !r; z0 += sk) {
+            sk = s && D - z0 > s ? s : D - z0;
+            shape5 xs = conv == 1 ? b->xs : b->ys;
+            if (s) { nn_set_zrange(z0, D, z0 == 0, z0 + sk >= D, D, z0); nn_set_zrange_out(1); xs.d = sk; }
+            if (conv == 2) r = nn_conv3d_fwd_gn_stats(b->a1, xs, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, b->a2, G, 1e-5f, b->m2, b->r2);
+            else if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, b->a1, G, 1e-5f, b->m1, b->r1);   /* [up2(coarse) | skip] */
+            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, b->a1, G, 1e-5f, b->m1, b->r1);
+            if (s) { nn_set_zrange(0, 0, 0, 0, 0, 0); nn_set_zrange_out(0); }
+        }
+        if (!r) { if (conv == 1) note(u, b->a1, b->ys, n1, b->m1, b->r1, G); else note(u, b->a2, b->ys, n2, b->m2, b->r2, G); }
+    }
     return r;
 }
 /* the bottleneck's raw output -> fp32 planes -> token rows with the registers prepended -> blocks -> planes -> a new MX tensor with its
@@ -203,7 +215,7 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
     for (int i = 0; i < L; i++) {
         nn_gn_t gd; const nn_gn_t *gin = nullptr;                  /* down_norm: conv1 reads silu(gn(down conv output)) (src/unet.c:2593) */
         if (i && u->cfg.down_norm) { gd = (nn_gn_t){P(u, u->dn[i - 1].gamma), P(u, u->dn[i - 1].beta), u->dm[i - 1], u->dr[i - 1], G_of(u, u->cfg.widths[i - 1])}; gin = &gd; }
-        if (block_fwd(u, &u->enc[i], cur, gin, nullptr, nullptr, 0, en1[i], en2[i])) { if (reg_here) nn_storage_forget(x); return -1; }
+        if (block_fwd(u, &u->enc[i], i, cur, gin, nullptr, nullptr, 0, en1[i], en2[i])) { if (reg_here) nn_storage_forget(x); return -1; }
         if (i < L - 1) {                                           /* stride-2 down conv of silu(gn(a2)), width kept (src/unet.c:2970) */
             const nn_gn_t g = gn_out(u, &u->enc[i]);
             if (nn_conv3d_fwd_x(u->enc[i].a2, &g, nullptr, nullptr, 0, 0, u->enc[i].ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
@@ -220,7 +232,7 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
         const block *coarse = i == L - 2 ? &u->enc[L - 1] : &u->dec[i + 1];
         nn_gn_t gc = gn_out(u, coarse); const nn_gn_t gs = gn_out(u, &u->enc[i]);
         if (i == L - 2 && u->tbn) { coarse = &u->tb; gc.mean = u->tb.m2; gc.rstd = u->tb.r2; }      /* the stage's output under the level's n2 affine (src/unet.c:508) */
-        if (block_fwd(u, &u->dec[i], u->enc[i].a2, &gs, coarse->a2, &gc, u->cfg.widths[i + 1], dn1[i], dn2[i])) return -1;
+        if (block_fwd(u, &u->dec[i], i, u->enc[i].a2, &gs, coarse->a2, &gc, u->cfg.widths[i + 1], dn1[i], dn2[i])) return -1;
     }
     const block *last = L > 1 ? &u->dec[0] : &u->enc[0];
     const nn_gn_t g = gn_out(u, last);

@@ -44,6 +44,10 @@ def load_host():
     L.nn_set_gn_stored.restype = None; L.nn_set_gn_stored.argtypes = [C.c_int]
     L.nn_check.restype = C.c_char_p
     L.unet_in_shape.restype = shape5; L.unet_in_shape.argtypes = [C.c_void_p]
+    L.unet_set_infer_slab.restype = None; L.unet_set_infer_slab.argtypes = [C.c_int]
+    L.unet_get_infer_slab.restype = C.c_int; L.unet_get_infer_slab.argtypes = []
+    L.nn_set_zrange.restype = None; L.nn_set_zrange.argtypes = [C.c_int] * 6
+    L.nn_set_zrange_out.restype = None; L.nn_set_zrange_out.argtypes = [C.c_int]
     L.unet_config.restype = C.POINTER(unet_cfg); L.unet_config.argtypes = [C.c_void_p]
     L.unet_read_header.restype = C.c_int; L.unet_read_header.argtypes = [C.c_char_p, C.POINTER(unet_cfg), C.POINTER(C.c_size_t), C.POINTER(C.c_int)]
     L.unet_load.restype = C.c_int; L.unet_load.argtypes = [C.c_void_p, C.c_char_p]
