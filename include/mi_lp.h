@@ -25,9 +25,11 @@ typedef struct {                                                                
     const void *x2; int c_split; void *y2; int o_split; int accum; gnp_t gp2; int16_t up, yD; unsigned sr; unsigned wkey;
     int zlo, zhi; int stored_stats; unsigned osr; int16_t zi0, Di, o_pad, zw0, zw1, yzo;
 } split_t;
-/* Fields honoured by this build: x2, c_split, gp2, up, wkey, stored_stats, zlo, zhi. Training / slab fields (y2, o_split, accum,
-   sr, osr, yD, zi0, Di, o_pad, zw0, zw1, yzo) must be zero: a call that sets one prints a message and aborts, as the reference
-   does for combinations it does not support (src/lp_f8fwd.cu:28). Slab-local GroupNorm (gnp_t.ns > 0) likewise. */
+/* Fields honoured by this build: x2, c_split, gp2, up, wkey, stored_stats, zlo, zhi, and the z-range of the reference's slab inference:
+   zi0 / Di (output plane z of the xs.d planes computed reads input plane z + zi0 of depth-Di inputs; Di 0 = off) and yzo / yD (the MX
+   output is planes [yzo, yzo + xs.d) of a depth-yD tensor; yD 0 = a depth-xs.d tensor), stride 1 (src/nn_lp.h:36-40). Training and
+   z-window fields (y2, o_split, accum, sr, osr, o_pad, zw0, zw1) must be zero: a call that sets one prints a message and aborts, as the
+   reference does for unsupported combinations (src/lp_f8fwd.cu:28). Slab-local GroupNorm (gnp_t.ns > 0) likewise. */
 
 /* GroupNorm sum slots (src/gnacc.cuh:8-9): `osum` / `sums` buffers are arrays of 3 x uint64 fixed-point slots (24 bytes each:
    fraction in units of 2^-64, signed integer part, count of non-finite contributions), two per (sample, group): sum, sum of squares */
