@@ -45,13 +45,11 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     constexpr unsigned halo_o = 2 * SLOT, tab_o = halo_o + 3 * HB;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), r = lane & 31, h = lane >> 5;
     const int lz = wave, ly0 = 0;
-    unsigned abr[NT], sbr[NT];                                  // the lane's row (its 16-byte half) and scale word of tap (0, 0, 0) inside a halo slot
-#pragma unroll
-    for (int j = 0; j < NT; j++) {
-        const int p0 = (lz * HY + (2 * j + (r >> 4))) * HX + (r & 15);
-        abr[j] = halo_o + ((NH == 2 ? h * TTP : 0) + p0) * 16;
-        sbr[j] = halo_o + NH * TTP * 16 + p0 * 4;
-    }
+    // the lane's row (its 16-byte half) and scale word of tap (0, 0, 0) inside a halo slot for its first voxel tile; tile j lies two halo rows
+    // further: a constant the loads carry in their offset field
+    const int p00 = (lz * HY + (r >> 4)) * HX + (r & 15);
+    const unsigned abr0 = halo_o + ((NH == 2 ? h * TTP : 0) + p00) * 16, sbr0 = halo_o + NH * TTP * 16 + p00 * 4;
+    constexpr unsigned ABJ = 2 * HX * 16, SBJ = 2 * HX * 4;
     const unsigned wfa = lane * 16, wfs = MT * WTILE + lane * 4;            // the lane's weight fragment / scale word of pair 0, tile 0 of a slot
     const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 256;
     const size_t Sin = (size_t)a.D * a.H * a.W;
@@ -72,26 +70,73 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         t.ox0 = tx * 16; t.oy0 = ty * 8; t.oz0 = tz * TZ;
         return t;
     };
-    // One copy round of this wave for block blk of the tile at (n, oz0, oy0, ox0) into the halo slot at byte offset sbase of the halo area:
-    // the two row halves and the scale bytes of 64 halo positions (group 4 rd + wave). It is prepared (addresses: pure arithmetic the
-    // scheduler places anywhere) one step ahead of its issue, and the issue is three copies with every lane active and no branch: positions
-    // outside the volume, past the halo or of blocks past the stored channels read a constant page (zero row, scale byte 1); a round with
-    // nothing to do (go false, or a group past the last) reads the constant page into a junk area. The two halves of a row are requested
-    // back to back, so the second one finds its cache line.
+    // One copy round of this wave = the two row halves and the scale bytes of 64 halo positions (group 4 rd + wave of the NG groups a block's
+    // halo has) for one block of a tile. The issue is three copies with every lane active and no branch: positions outside the volume, past
+    // the halo or of blocks past the stored channels read a constant page (zero row, scale byte 1); a round with nothing to do (go false, or a
+    // group past the last) reads the constant page into a junk area. The two halves of a row are requested back to back, so the second one
+    // finds its cache line. The request's addresses are prepared one step ahead of its issue from data that is formed once per kernel or
+    // once per tile, so that a round costs a handful of instructions the scheduler places between the MFMAs:
+    //   * per lane and round rd, the position's offset inside a tile's halo as a voxel offset of the volume, (pz H + py) W + px, and its
+    //     packed coordinates (kernel constants). The offsets sit in a ring of five registers that turns by one whenever a round is consumed:
+    //     its head is the round to request next (rounds cycle 0 .. NRND - 1 block after block);
+    //   * per lane and tile (this one, the next one), a bit per round: the position is inside the halo and the volume;
+    //   * per tile, the voxel offset of the halo's first position (may be negative), and in lane i of a register group the base addresses of
+    //     the rows and scale bytes of request block i: blocks 0 .. nbt - 1 of this tile, then the first blocks of the next one.
     const unsigned junk = a.red_o;                              // the statistics scratch (1 KiB) is idle while the K loop runs
     struct hreq { const uint8_t *row, *sc; unsigned rdst, sdst; };
-    auto prepare = [&](hreq &q, int n, int oz0, int oy0, int ox0, int blk, int rd, unsigned sbase, bool go) {
-        const int g = 4 * rd + wave;
+    static_assert(NRND == 5, "the round ring below has five entries");
+    unsigned pc[NRND];                                          // px | py << 8 | pz << 16 | (position inside the halo) << 24
+    unsigned ring0, ring1, ring2, ring3, ring4;
+    {
+        unsigned dl[NRND];
+#pragma unroll
+        for (int rd = 0; rd < NRND; rd++) {
+            const int g = 4 * rd + wave, pos = g * 64 + lane;
+            const int pz = pos / (HY * HX), rem = pos - pz * (HY * HX), py = rem / HX, px = rem - py * HX;
+            pc[rd] = (unsigned)px | ((unsigned)py << 8) | ((unsigned)pz << 16) | ((g < NG && pos < TT ? 1u : 0u) << 24);
+            dl[rd] = (unsigned)((pz * a.H + py) * a.W + px);
+        }
+        ring0 = dl[0]; ring1 = dl[1]; ring2 = dl[2]; ring3 = dl[3]; ring4 = dl[4];
+    }
+    struct treq { unsigned mask; int base; };                   // a tile's validity bits (per lane) and first-position voxel offset (uniform)
+    auto tile_req = [&](const tile_t &t) {
+        treq q; q.mask = 0u;
+        const int z0 = t.oz0 - 1 + a.zi0, y0 = t.oy0 - 1, x0 = t.ox0 - 1;
+#pragma unroll
+        for (int rd = 0; rd < NRND; rd++) {
+            const int gz = z0 + (int)((pc[rd] >> 16) & 255u), gy = y0 + (int)((pc[rd] >> 8) & 255u), gx = x0 + (int)(pc[rd] & 255u);
+            const bool in = (pc[rd] >> 24) && (unsigned)gz < (unsigned)a.D && (unsigned)gy < (unsigned)a.H && (unsigned)gx < (unsigned)a.W;
+            q.mask |= in ? 1u << rd : 0u;
+        }
+        q.base = (z0 * a.H + y0) * a.W + x0;
+        return q;
+    };
+    // lane i: request block i (i < nbt: block i of tile c; else block i - nbt of tile x): row base, scale base, block holds stored channels
+    unsigned long long tb_row = 0, tb_sc = 0; int tb_ok = 0;
+    auto block_table = [&](const tile_t &c, const tile_t &x) {
+        const int i = lane, own = i < a.nbt, blk = own ? i : i - a.nbt, n = own ? c.n : x.n;
         const int seg = blk >= a.nb0p, bl = seg ? blk - a.nb0p : blk;
-        const bool real = go && g < NG, bok = real && bl < a.nbs[seg];
-        const size_t plane = (size_t)n * a.nbs[seg] + min(max(bl, 0), a.nbs[seg] - 1);
-        const int pos = g * 64 + lane;
-        const int pz = pos / (HY * HX), rem = pos - pz * (HY * HX), py = rem / HX, px = rem - py * HX;
-        const int gz = oz0 - 1 + pz + a.zi0, gy = oy0 - 1 + py, gx = ox0 - 1 + px;
-        const bool in = bok && pos < TT && gz >= 0 && gz < a.D && gy >= 0 && gy < a.H && gx >= 0 && gx < a.W;
-        const size_t vox = (size_t)(unsigned)((gz * a.H + gy) * a.W + gx);
-        q.row = in ? a.xq[seg] + (plane * Sin + vox) * (16 * NH) : a.zpage;
-        q.sc = in ? a.xsc[seg] + plane * Sin + vox : a.zpage + 64;
+        const int nbs = seg ? a.nbs[1] : a.nbs[0];
+        const uint8_t *xq = seg ? a.xq[1] : a.xq[0], *xsc = seg ? a.xsc[1] : a.xsc[0];
+        const size_t plane = ((size_t)n * nbs + min(max(bl, 0), max(nbs - 1, 0))) * Sin;
+        tb_row = (unsigned long long)(size_t)(xq + plane * (16 * NH)); tb_sc = (unsigned long long)(size_t)(xsc + plane);
+        tb_ok = blk < a.nbt && bl < nbs;
+    };
+    treq rq_cur, rq_nxt;
+    auto lane64 = [&](unsigned long long v, int i) {
+        const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)v, i), hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(v >> 32), i);
+        return (unsigned long long)lo | ((unsigned long long)hi << 32);
+    };
+    // the round rd (uniform) of request block ti of the tile whose data is (mask, base), into the halo slot at byte offset sbase; go false: a
+    // round into the junk area. d: the lane's offset for that round (the ring's head, or a compile-time pick)
+    auto prepare = [&](hreq &q, unsigned mask, int base, int ti, int rd, unsigned d, unsigned sbase, bool go) {
+        const int g = 4 * rd + wave;
+        const bool real = go & (g < NG);
+        const bool in = real & (__builtin_amdgcn_readlane(tb_ok, ti) != 0) & (((mask >> rd) & 1u) != 0u);
+        const unsigned vox = (unsigned)base + d;
+        const uint8_t *rb = (const uint8_t *)(size_t)lane64(tb_row, ti), *sb = (const uint8_t *)(size_t)lane64(tb_sc, ti);
+        q.row = in ? rb + (size_t)vox * (16 * NH) : a.zpage;
+        q.sc = in ? sb + vox : a.zpage + 64;
         q.rdst = real ? halo_o + sbase + g * 1024 : junk;
         q.sdst = real ? halo_o + sbase + NH * TTP * 16 + g * 256 : junk;
     };
@@ -124,15 +169,23 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     tile_t cur = decode(0);
     if (!cur.ok) return;
     const int nnext = min(2, a.nbt);                            // blocks of the next tile requested ahead
-    for (int rd = 0; rd < NRND; rd++) {
-        hreq q;
-        prepare(q, cur.n, cur.oz0, cur.oy0, cur.ox0, 0, rd, 0, true); issue(q);
-        if (nnext > 1) { prepare(q, cur.n, cur.oz0, cur.oy0, cur.ox0, 1, rd, HB, true); issue(q); }
+    rq_nxt = tile_req(cur);
+    block_table(cur, cur);
+    {
+        const unsigned d5[NRND] = {ring0, ring1, ring2, ring3, ring4};
+#pragma unroll
+        for (int rd = 0; rd < NRND; rd++) {
+            hreq q;
+            prepare(q, rq_nxt.mask, rq_nxt.base, 0, rd, d5[rd], 0, true); issue(q);
+            if (nnext > 1) { prepare(q, rq_nxt.mask, rq_nxt.base, 1, rd, d5[rd], HB, true); issue(q); }
+        }
     }
     wstage(0, cur.cs, 0); wstage(2, cur.cs, SLOT);
     unsigned rot = 0;                                           // (it nbt) % 3
     for (unsigned it = 0;; it++) {
         const tile_t nxt = decode(it + 1);
+        rq_cur = rq_nxt; rq_nxt = tile_req(nxt);
+        block_table(cur, nxt);
         const int fmax = a.nbt - 1 + (nxt.ok ? nnext : 0);      // blocks to request during this tile: 2 .. nbt - 1 of this tile, then nbt .. of the next
         wait_vm<0>();                                           // the tile's first blocks and weight stages (and the last tile's stores) are done
         __syncthreads();
@@ -173,9 +226,9 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
             constexpr int f = i / 3, part = i % 3;
             if constexpr (i == 3 * (NT + MT)) { T = *(const v4i *)(lds + tabp + 32); tabp += 32; }
             else if constexpr (f < NT) {
-                if constexpr (part == 0) lo[f] = *(const v4i *)(lds + abr[f] + tt2[0]);
-                else if constexpr (part == 1) { if constexpr (FMT == 8) hi[f] = *(const v4i *)(lds + abr[f] + tt2[1]); }
-                else sb[nx][f] = *(const int *)(lds + sbr[f] + tt2[2]);
+                if constexpr (part == 0) lo[f] = *(const v4i *)(lds + (abr0 + tt2[0]) + f * ABJ);
+                else if constexpr (part == 1) { if constexpr (FMT == 8) hi[f] = *(const v4i *)(lds + (abr0 + tt2[1]) + f * ABJ); }
+                else sb[nx][f] = *(const int *)(lds + (sbr0 + tt2[2]) + f * SBJ);
             } else {
                 constexpr int m = f - NT;
                 if constexpr (part == 0) lo[f] = *(const v4i *)(lds + wfa + wbase + m * WTILE);
@@ -202,10 +255,11 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         // with two rounds per stage every block of a tile lands two barriers before its first fetch ----
         int fbi = 2, frd = 0;
         auto prep_next = [&](hreq &q, int upto_pair) {          // prepare one copy round; pairs <= upto_pair will have been fetched by every wavefront when it is issued
-            const bool go = fbi <= fmax && (fbi < 3 || ((27 * (fbi - 3) + 26) >> 1) <= upto_pair);
+            const bool go = (fbi <= fmax) & ((fbi < 3) | (((27 * (fbi - 3) + 26) >> 1) <= upto_pair));       // (bitwise: no branches in a step)
             const bool own = fbi < a.nbt;
-            prepare(q, own ? cur.n : nxt.n, own ? cur.oz0 : nxt.oz0, own ? cur.oy0 : nxt.oy0, own ? cur.ox0 : nxt.ox0, own ? fbi : fbi - a.nbt, frd,
-                    ((rot + (unsigned)fbi) % 3u) * HB, go);
+            prepare(q, own ? rq_cur.mask : rq_nxt.mask, own ? rq_cur.base : rq_nxt.base, fbi, frd, ring0, ((rot + (unsigned)fbi) % 3u) * HB, go);
+            const unsigned t0 = ring0;                          // a consumed round turns the ring
+            ring0 = go ? ring1 : ring0; ring1 = go ? ring2 : ring1; ring2 = go ? ring3 : ring2; ring3 = go ? ring4 : ring3; ring4 = go ? t0 : ring4;
             frd += go ? 1 : 0;
             const bool wrap = frd == NRND;
             frd = wrap ? 0 : frd; fbi += wrap ? 1 : 0;
