@@ -77,6 +77,13 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
     const int q = gp - pb, m = cop >> 5, r = cop & 31;
     uint8_t *tile = wq + ((size_t)gp * nmt_all + m) * WTILE;
     unsigned *tsc = wsc + ((size_t)gp * nmt_all + m) * 64;      // one word per lane: the byte the MFMA reads is the low one
+    int tss = 1;                                                // words between two lanes' scale words
+    if (block_major) {
+        // the wide kernel's layout: per 128-channel slice, pair after pair the image of its LDS stage: four tiles of codes, then per lane the
+        // four tiles' scale words
+        uint8_t *img = wq + ((size_t)(m >> 2) * (npairs_all + 16) + gp) * (size_t)(4 * (WTILE + 256));
+        tile = img + (m & 3) * WTILE; tsc = (unsigned *)(img + 4 * WTILE) + (m & 3); tss = 4;
+    }
 #pragma unroll
     for (int side = 0; side < 2; side++) {
         const int u = 2 * q + side;
@@ -103,7 +110,7 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
             for (int j = 0; j < 4; j++) c[j] = d_enc_e2m1x8(v + 8 * j, mult);
             *(uint4 *)(tile + ((size_t)(r + 32 * side) * 16)) = make_uint4(c[0], c[1], c[2], c[3]);            // lane (r, side): the unit's 32 nibbles
         }
-        tsc[r + 32 * side] = (unsigned)(e + 127);
+        tsc[(r + 32 * side) * tss] = (unsigned)(e + 127);
     }
 }
 
@@ -325,18 +332,21 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     int npairs_all = 0;
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) npairs_all += (27 * (a.nbt - b0 < a.CB ? a.nbt - b0 : a.CB) + 1) >> 1;
     // (sixteen pairs of padding: the kernels' weight loads run up to two ring stages ahead of the last pair)
-    const size_t wq_bytes = (size_t)(npairs_all + 16) * nmt_all * WTILE, wsc_bytes = (size_t)(npairs_all + 16) * nmt_all * 256;
+    // (the wide kernel's weights are one buffer: codes and scale words interleaved pair by pair; its scale buffer is a stub)
+    const size_t wq_bytes = (size_t)(npairs_all + 16) * nmt_all * (big ? WTILE + 256 : WTILE), wsc_bytes = big ? 256 : (size_t)(npairs_all + 16) * nmt_all * 256;
+    a.wstride = (unsigned)((size_t)(npairs_all + 16) * 4 * (WTILE + 256));
+    const int memoCB = big ? -a.CB : a.CB;
     const int CxP = (Cx + 31) / 32 * 32;
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
     if (sp.wkey) {
         for (auto &m : g_wmemo)
-            if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == a.CB && m.nmt_all == nmt_all && m.dev == dev) { wq = m.wq; wsc = m.wsc; have = true; break; }
+            if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == memoCB && m.nmt_all == nmt_all && m.dev == dev) { wq = m.wq; wsc = m.wsc; have = true; break; }
         if (!have) {
             MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes));
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
             MIRT(hipMemsetAsync(wq, 0, wq_bytes, 0)); MIRT(hipMemsetAsync(wsc, 0, wsc_bytes, 0));
-            g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, a.CB, nmt_all, dev, wq, wsc});
+            g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, memoCB, nmt_all, dev, wq, wsc});
         }
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) {

@@ -91,6 +91,7 @@ struct conv_args {
     int zi0;                           // z-range: output plane z reads input plane z + zi0 (stride 1)
     int yD, yzo;                       // direct slab output: the MX output is planes [yzo, yzo + Do) of a depth-yD tensor (yD 0: a depth-Do tensor)
     const uint8_t *wq, *wsc; int nmt_all;
+    unsigned wstride;                  // wide kernel: bytes between the weight images of two 128-channel slices
     const float *bias; int Co;
     void *y; int ydt;
     double *osum; float *part; int Go, stored_stats, zs0, zs1;   // part: per tile and channel quad (sum, sum of squares)

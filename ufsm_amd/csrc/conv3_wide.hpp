@@ -28,6 +28,10 @@ __device__ __forceinline__ void dma16s(unsigned off, const void *base, unsigned 
 __device__ __forceinline__ void dma1s(unsigned off, const void *base, unsigned lds_off) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_ubyte %1, %2" ::"s"(lds_off), "v"(off), "s"(base) : "memory");
 }
+// the same with the LDS offset formed in the instruction: m0 = ldsb + IMM
+template <int IMM> __device__ __forceinline__ void dma16si(unsigned off, const void *base, unsigned ldsb) {
+    asm volatile("s_add_u32 m0, %0, %3\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(ldsb), "v"(off), "s"(base), "n"(IMM) : "memory", "scc");
+}
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
 template <int FMT, int OUT, bool EPI>
@@ -39,7 +43,8 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     constexpr int NG = (TT + 63) / 64, TTP = NG * 64;           // copy groups of 64 halo positions; positions per half padded to whole groups
     constexpr int HB = NH * TTP * 16 + TTP * 4;                 // a halo slot: rows [half][position][16 B], then one scale word per position
     constexpr int NRND = (NG + 3) / 4;                          // copy rounds of a block: in a round every wave copies one group (both halves and the scales)
-    constexpr int WCP = MT * WTILE / 1024, WPS = 2 * (WCP + 1); // 1 KiB copies per pair of codes (+ 1 of scales), copies per weight stage
+    constexpr int NCH = SLOT / 1024;                            // 1 KiB copies per weight stage: the prepared weights hold the ring slot's image, stage after stage
+    static_assert(SLOT % 1024 == 0, "a weight stage is a whole number of 1 KiB copies");
     extern __shared__ __align__(16) unsigned char lds[];
     const unsigned lds0 = (unsigned)(size_t)lds;                // LDS byte offset of the dynamic segment (the low word of its flat address)
     constexpr unsigned halo_o = 2 * SLOT, tab_o = halo_o + 3 * HB;
@@ -50,8 +55,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     const int p00 = (lz * HY + (r >> 4)) * HX + (r & 15);
     const unsigned abr0 = halo_o + ((NH == 2 ? h * TTP : 0) + p00) * 16, sbr0 = halo_o + NH * TTP * 16 + p00 * 4;
     constexpr unsigned ABJ = 2 * HX * 16, SBJ = 2 * HX * 4;
-    const unsigned wfa = lane * 16, wfs = MT * WTILE + lane * 4;            // the lane's weight fragment / scale word of pair 0, tile 0 of a slot
-    const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 256;
+    const unsigned wfa = lane * 16, wfs = MT * WTILE + lane * 16;           // the lane's weight fragment of tile 0 / its MT scale words of pair 0 of a slot
     const size_t Sin = (size_t)a.D * a.H * a.W;
     const int nunits = 27 * a.nbt, npairs = (nunits + 1) >> 1, nfull = npairs >> 1;
 
@@ -146,20 +150,23 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         dma1(q.sc, lds0 + q.sdst);
     };
     constexpr int NHC = NH + 1;                                 // asynchronous copies of a round
-    // copy k (of NW) of this wave's share of the weight stage of pairs gp0, gp0 + 1 into the ring slot at byte offset so (a wave with fewer
-    // pieces repeats its last one: the count per step stays fixed)
-    constexpr int NW = (WPS + 3) / 4;
-    auto wcopy = [&](int k, int gp0, int cs, unsigned so) {
-        int c = wave + 4 * k;
-        c = c < WPS ? c : c - 4;
-        const int p = c / (WCP + 1), cc = c - p * (WCP + 1);
-        const bool codes = cc < WCP;
-        const uint8_t *src = codes ? a.wq + (size_t)(gp0 + p) * wq_ps + (size_t)cs * MT * WTILE + cc * 1024 : a.wsc + (size_t)(gp0 + p) * wsc_ps + (size_t)cs * MT * 256;
-        dma16s((unsigned)lane * 16u, src, lds0 + so + p * STG + (codes ? cc * 1024 : MT * WTILE));
-    };
-    auto wstage = [&](int gp0, int cs, unsigned so) {
+    // The weight stage of pairs 2 s, 2 s + 1 of channel slice cs is SLOT contiguous bytes at wq + cs wstride + s SLOT, the image of a ring
+    // slot: per pair the MT tiles of codes, then per lane its MT scale words. Wave w copies the 1 KiB pieces w, w + 4, ... (NW of them; a wave
+    // with fewer repeats its last one: the count per step stays fixed). A copy is one instruction pair: m0 = slot + piece, load.
+    constexpr int NW = (NCH + 3) / 4;
+    unsigned wvo[NW];                                           // the lane's byte offset inside a stage for copy k
 #pragma unroll
-        for (int k = 0; k < NW; k++) wcopy(k, gp0, cs, so);
+    for (int k = 0; k < NW; k++) { int c = wave + 4 * k; c = c < NCH ? c : c - 4; wvo[k] = (unsigned)c * 1024u + (unsigned)lane * 16u; }
+    const unsigned wd0 = lds0 + (unsigned)wave * 1024u;         // LDS address of the wave's first piece in slot 0
+    const unsigned wdl = (wave + 4 * (NW - 1) < NCH) ? (unsigned)(NW - 1) * 4096u : (unsigned)(NW - 2) * 4096u;   // its last piece
+    auto wcopy = [&](auto K, const uint8_t *src, unsigned so) {
+        constexpr int k = decltype(K)::value;
+        if constexpr (k < NW - 1) dma16si<k * 4096>(wvo[k], src, wd0 + so);
+        else dma16s(wvo[k], src, wd0 + so + wdl);
+    };
+    auto wstage = [&](int st, int cs, unsigned so) {            // stage st of slice cs into the ring slot at byte offset so
+        const uint8_t *src = a.wq + (size_t)cs * a.wstride + (size_t)st * SLOT;
+        static_for<NW>([&](auto K) { wcopy(K, src, so); });
     };
 
     // K order: unit U = (block U / 27, tap U % 27), pair G = units 2 G, 2 G + 1 (a pair may straddle two blocks; the unit past the end has
@@ -180,7 +187,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
             if (nnext > 1) { prepare(q, rq_nxt.mask, rq_nxt.base, 1, rd, d5[rd], HB, true); issue(q); }
         }
     }
-    wstage(0, cur.cs, 0); wstage(2, cur.cs, SLOT);
+    wstage(0, cur.cs, 0); wstage(1, cur.cs, SLOT);
     unsigned rot = 0;                                           // (it nbt) % 3
     for (unsigned it = 0;; it++) {
         const tile_t nxt = decode(it + 1);
@@ -214,7 +221,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         }
         __syncthreads();
 
-        v8i fb[2][NT], fa[2][MT]; int sb[2][NT], sa[2][MT];
+        v8i fb[2][NT], fa[2][MT]; int sb[2][NT]; v4i sav[2];
         v4i T;
         unsigned tabp = tab_o + h * 16;
         T = *(const v4i *)(lds + tabp);
@@ -233,7 +240,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
                 constexpr int m = f - NT;
                 if constexpr (part == 0) lo[f] = *(const v4i *)(lds + wfa + wbase + m * WTILE);
                 else if constexpr (part == 1) { if constexpr (FMT == 8) hi[f] = *(const v4i *)(lds + wfa + wbase + m * WTILE + 1024); }
-                else sa[nx][m] = *(const int *)(lds + wfs + wbase + m * 256);
+                else if constexpr (m == 0) sav[nx] = *(const v4i *)(lds + wfs + wbase);      // the MT scale words of the pair at once
             }
         };
         auto pack = [&](auto NXT) {
@@ -269,20 +276,20 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         // MODE 1: also prepare the copy round the next step will issue. MODE 2: also this step's asynchronous copies, one after every
         // MFMA from the second on: the weight stage of pairs wgp, wgp + 1 into ring offset wso first, then the prepared round (so that
         // "all but the last NHC copies" means "the weights")
-        auto step = [&](auto CUR, auto MODE, unsigned wbase, int wgp, unsigned wso, int upto_pair) {
+        auto step = [&](auto CUR, auto MODE, unsigned wbase, const uint8_t *wsrc, unsigned wso, int upto_pair) {
             constexpr int cu = decltype(CUR)::value, nx = cu ^ 1, mode = decltype(MODE)::value;
             const v4i tt2 = T;
             if constexpr (mode == 1) prep_next(rq, upto_pair);
             static_for<NM>([&](auto K) {
                 constexpr int k = decltype(K)::value, m = k / NT, j = k % NT;
-                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cu][m], fb[cu][j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sa[cu][m], 0, sb[cu][j]);
+                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cu][m], fb[cu][j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sav[cu][m], 0, sb[cu][j]);
                 constexpr int l0 = k < NSP ? (k * NL) / NSP : NL, l1 = k < NSP ? ((k + 1) * NL) / NSP : NL;
                 static_for<l1 - l0>([&](auto I) { ld(std::integral_constant<int, l0 + decltype(I)::value>{}, std::integral_constant<int, nx>{}, tt2, wbase); });
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                 if constexpr (l1 > l0) __builtin_amdgcn_sched_group_barrier(0x100, l1 - l0, 0);
                 if constexpr (mode == 1) __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);     // the preparation's arithmetic, a few instructions per MFMA
                 if constexpr (mode == 2) {                      // (fenced: otherwise the scheduler lifts the copies, and the fetches ordered with them, above the MFMAs)
-                    if constexpr (k >= 1 && k <= NW) { __builtin_amdgcn_sched_barrier(0); wcopy(k - 1, wgp, cur.cs, wso); __builtin_amdgcn_sched_barrier(0); }
+                    if constexpr (k >= 1 && k <= NW) { __builtin_amdgcn_sched_barrier(0); wcopy(std::integral_constant<int, k - 1>{}, wsrc, wso); __builtin_amdgcn_sched_barrier(0); }
                     if constexpr (k == NW + 2) { __builtin_amdgcn_sched_barrier(0); issue(rq); __builtin_amdgcn_sched_barrier(0); }
                 }
             });
@@ -292,19 +299,20 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         // barrier every wavefront is done reading that slot, so step 1 requests stage s + 2 into it (to be there one stage later, when
         // the barrier of stage s + 1 has been passed) and two copy rounds of streaming blocks, while it consumes pair 2 s + 1 and fetches
         // pair 2 s + 2 from the other slot
-        for (int s = 0; s < nfull; s++) {
+        const uint8_t *wsrc = a.wq + (size_t)cur.cs * a.wstride + (size_t)2 * SLOT;      // stage s + 2 is requested during stage s
+        for (int s = 0; s < nfull; s++, wsrc += SLOT) {
             const unsigned so = (s & 1) * SLOT;
-            step(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, so + STG, 0, 0u, 2 * s + 1);
+            step(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, so + STG, nullptr, 0u, 2 * s + 1);
             wait_vm<NHC>();                                     // the weight stage requested one stage ago is in LDS: it was issued before that step's NHC halo copies
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            step(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{}, SLOT - so, 2 * (s + 2), so, 0);
+            step(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{}, SLOT - so, wsrc, so, 0);
         }
-        if (npairs & 1) step(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, (nfull & 1) * SLOT + STG, 0, 0u, 0);     // the odd last pair (its fetch reads past the end: unused)
+        if (npairs & 1) step(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, (nfull & 1) * SLOT + STG, nullptr, 0u, 0);     // the odd last pair (its fetch reads past the end: unused)
         DBG_MARK(2);
         wait_vm<0>();
         __syncthreads();                                        // every wavefront is done with the halo slots and the ring
         while (fbi <= fmax) { prep_next(rq, npairs); issue(rq); }       // (tiles too short to stream everything)
-        if (nxt.ok) { wstage(0, nxt.cs, 0); wstage(2, nxt.cs, SLOT); }
+        if (nxt.ok) { wstage(0, nxt.cs, 0); wstage(1, nxt.cs, SLOT); }
         DBG_MARK(3);
         conv_epilogue<MT, NT, OUT, EPI, true, true>(a, acc, lds, cur.tile, cur.n, cur.cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
         DBG_MARK(4);
