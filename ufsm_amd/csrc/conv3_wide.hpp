@@ -117,7 +117,9 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     };
     // lane i: request block i (i < nbt: block i of tile c; else block i - nbt of tile x): row base, scale base, block holds stored channels
     unsigned long long tb_row = 0, tb_sc = 0; int tb_ok = 0;
-    auto block_table = [&](const tile_t &c, const tile_t &x) {
+    int tb_gate = 0, tb_base = 0, tb_slot = 0, tb_msh = 0;      // also per request block: first pair after which it may be requested, its tile's first-position
+                                                                // voxel offset, its halo slot's byte offset, the shift of its tile's validity bits
+    auto block_table = [&](const tile_t &c, const tile_t &x, int fmax, unsigned rot, int bcur, int bnxt) {
         const int i = lane, own = i < a.nbt, blk = own ? i : i - a.nbt, n = own ? c.n : x.n;
         const int seg = blk >= a.nb0p, bl = seg ? blk - a.nb0p : blk;
         const int nbs = seg ? a.nbs[1] : a.nbs[0];
@@ -125,6 +127,10 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         const size_t plane = ((size_t)n * nbs + min(max(bl, 0), max(nbs - 1, 0))) * Sin;
         tb_row = (unsigned long long)(size_t)(xq + plane * (16 * NH)); tb_sc = (unsigned long long)(size_t)(xsc + plane);
         tb_ok = blk < a.nbt && bl < nbs;
+        tb_gate = i > fmax ? 0x7fffffff : i < 3 ? -1 : (27 * (i - 3) + 26) >> 1;       // block i takes the slot block i - 3 is read from until that pair
+        tb_base = own ? bcur : bnxt;
+        tb_slot = (int)((rot + (unsigned)i) % 3u) * HB;
+        tb_msh = own ? 0 : 8;
     };
     treq rq_cur, rq_nxt;
     auto lane64 = [&](unsigned long long v, int i) {
@@ -177,7 +183,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     if (!cur.ok) return;
     const int nnext = min(2, a.nbt);                            // blocks of the next tile requested ahead
     rq_nxt = tile_req(cur);
-    block_table(cur, cur);
+    block_table(cur, cur, 1, 0u, rq_nxt.base, rq_nxt.base);
     {
         const unsigned d5[NRND] = {ring0, ring1, ring2, ring3, ring4};
 #pragma unroll
@@ -192,8 +198,9 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     for (unsigned it = 0;; it++) {
         const tile_t nxt = decode(it + 1);
         rq_cur = rq_nxt; rq_nxt = tile_req(nxt);
-        block_table(cur, nxt);
         const int fmax = a.nbt - 1 + (nxt.ok ? nnext : 0);      // blocks to request during this tile: 2 .. nbt - 1 of this tile, then nbt .. of the next
+        block_table(cur, nxt, fmax, rot, rq_cur.base, rq_nxt.base);
+        const unsigned mask2 = rq_cur.mask | (rq_nxt.mask << 8);            // validity bits of both tiles
         wait_vm<0>();                                           // the tile's first blocks and weight stages (and the last tile's stores) are done
         __syncthreads();
         DBG_MARK(0);
@@ -235,7 +242,10 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
             else if constexpr (f < NT) {
                 if constexpr (part == 0) lo[f] = *(const v4i *)(lds + (abr0 + tt2[0]) + f * ABJ);
                 else if constexpr (part == 1) { if constexpr (FMT == 8) hi[f] = *(const v4i *)(lds + (abr0 + tt2[1]) + f * ABJ); }
-                else sb[nx][f] = *(const int *)(lds + (sbr0 + tt2[2]) + f * SBJ);
+                else if constexpr (f % 2 == 0) {                // two tiles' scale words back to back: one two-address LDS read
+                    sb[nx][f] = *(const int *)(lds + (sbr0 + tt2[2]) + f * SBJ);
+                    sb[nx][f + 1] = *(const int *)(lds + (sbr0 + tt2[2]) + (f + 1) * SBJ);
+                }
             } else {
                 constexpr int m = f - NT;
                 if constexpr (part == 0) lo[f] = *(const v4i *)(lds + wfa + wbase + m * WTILE);
@@ -262,9 +272,8 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         // with two rounds per stage every block of a tile lands two barriers before its first fetch ----
         int fbi = 2, frd = 0;
         auto prep_next = [&](hreq &q, int upto_pair) {          // prepare one copy round; pairs <= upto_pair will have been fetched by every wavefront when it is issued
-            const bool go = (fbi <= fmax) & ((fbi < 3) | (((27 * (fbi - 3) + 26) >> 1) <= upto_pair));       // (bitwise: no branches in a step)
-            const bool own = fbi < a.nbt;
-            prepare(q, own ? rq_cur.mask : rq_nxt.mask, own ? rq_cur.base : rq_nxt.base, fbi, frd, ring0, ((rot + (unsigned)fbi) % 3u) * HB, go);
+            const bool go = __builtin_amdgcn_readlane(tb_gate, fbi) <= upto_pair;
+            prepare(q, mask2 >> __builtin_amdgcn_readlane(tb_msh, fbi), __builtin_amdgcn_readlane(tb_base, fbi), fbi, frd, ring0, (unsigned)__builtin_amdgcn_readlane(tb_slot, fbi), go);
             const unsigned t0 = ring0;                          // a consumed round turns the ring
             ring0 = go ? ring1 : ring0; ring1 = go ? ring2 : ring1; ring2 = go ? ring3 : ring2; ring3 = go ? ring4 : ring3; ring4 = go ? t0 : ring4;
             frd += go ? 1 : 0;
