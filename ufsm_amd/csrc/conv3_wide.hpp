@@ -215,17 +215,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
             const int oH = hh ? oB : oA, sH = (oH / HB) * HB + ((oH % HB) >> 2);
             *(v4i *)(lds + tab_o + i * 16) = (v4i){NH == 2 ? oA : oH, oB, sH, 0};
         }
-        v16f acc[MT][NT];
-        {
-            float z;                                            // an opaque zero: the accumulators are cleared here, not hoisted elsewhere
-            asm volatile("v_mov_b32 %0, 0" : "=v"(z));
-#pragma unroll
-            for (int m = 0; m < MT; m++)
-#pragma unroll
-                for (int j = 0; j < NT; j++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) acc[m][j][i] = z;
-        }
+        v16f acc[MT][NT];                                       // (not cleared: the tile's first pair multiplies onto a zero operand)
         __syncthreads();
 
         v8i fb[2][NT], fa[2][MT]; int sb[2][NT]; v4i sav[2];
@@ -285,13 +275,15 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         // MODE 1: also prepare the copy round the next step will issue. MODE 2: also this step's asynchronous copies, one after every
         // MFMA from the second on: the weight stage of pairs wgp, wgp + 1 into ring offset wso first, then the prepared round (so that
         // "all but the last NHC copies" means "the weights")
-        auto step = [&](auto CUR, auto MODE, unsigned wbase, const uint8_t *wsrc, unsigned wso, int upto_pair) {
+        auto step = [&](auto CUR, auto MODE, auto FIRST, unsigned wbase, const uint8_t *wsrc, unsigned wso, int upto_pair) {
             constexpr int cu = decltype(CUR)::value, nx = cu ^ 1, mode = decltype(MODE)::value;
+            constexpr bool first = decltype(FIRST)::value;      // the tile's first pair: the accumulators start from its products
             const v4i tt2 = T;
             if constexpr (mode == 1) prep_next(rq, upto_pair);
             static_for<NM>([&](auto K) {
                 constexpr int k = decltype(K)::value, m = k / NT, j = k % NT;
-                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cu][m], fb[cu][j], acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sav[cu][m], 0, sb[cu][j]);
+                const v16f c0 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[cu][m], fb[cu][j], first ? c0 : acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sav[cu][m], 0, sb[cu][j]);
                 constexpr int l0 = k < NSP ? (k * NL) / NSP : NL, l1 = k < NSP ? ((k + 1) * NL) / NSP : NL;
                 static_for<l1 - l0>([&](auto I) { ld(std::integral_constant<int, l0 + decltype(I)::value>{}, std::integral_constant<int, nx>{}, tt2, wbase); });
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
@@ -309,14 +301,22 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         // the barrier of stage s + 1 has been passed) and two copy rounds of streaming blocks, while it consumes pair 2 s + 1 and fetches
         // pair 2 s + 2 from the other slot
         const uint8_t *wsrc = a.wq + (size_t)cur.cs * a.wstride + (size_t)2 * SLOT;      // stage s + 2 is requested during stage s
-        for (int s = 0; s < nfull; s++, wsrc += SLOT) {
+        constexpr std::integral_constant<bool, false> NOTFIRST{};
+        {   // stage 0, peeled: its first step starts the accumulators
+            step(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, std::integral_constant<bool, true>{}, STG, nullptr, 0u, 1);
+            wait_vm<NHC>();
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            step(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{}, NOTFIRST, SLOT, wsrc, 0u, 0);
+            wsrc += SLOT;
+        }
+        for (int s = 1; s < nfull; s++, wsrc += SLOT) {
             const unsigned so = (s & 1) * SLOT;
-            step(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, so + STG, nullptr, 0u, 2 * s + 1);
+            step(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{}, NOTFIRST, so + STG, nullptr, 0u, 2 * s + 1);
             wait_vm<NHC>();                                     // the weight stage requested one stage ago is in LDS: it was issued before that step's NHC halo copies
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            step(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{}, SLOT - so, wsrc, so, 0);
+            step(std::integral_constant<int, 1>{}, std::integral_constant<int, 2>{}, NOTFIRST, SLOT - so, wsrc, so, 0);
         }
-        if (npairs & 1) step(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, (nfull & 1) * SLOT + STG, nullptr, 0u, 0);     // the odd last pair (its fetch reads past the end: unused)
+        if (npairs & 1) step(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, NOTFIRST, (nfull & 1) * SLOT + STG, nullptr, 0u, 0);     // the odd last pair (its fetch reads past the end: unused)
         DBG_MARK(2);
         wait_vm<0>();
         __syncthreads();                                        // every wavefront is done with the halo slots and the ring
