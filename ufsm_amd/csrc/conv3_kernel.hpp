@@ -231,7 +231,9 @@ __device__ __forceinline__ void conv_epi_consts(const conv_args &a, unsigned cha
 // ---- epilogue (src/lp_common.cuh:1465-1597): bias -> optional affine + activation -> per (voxel, 32-channel block) amax across the
 // lane pair (l, l ^ 32) -> E8M0 exponent -> codes -> row stores; GroupNorm partial sums per tile. acc: the wavefront's MT x NT accumulators;
 // lane (r, h) of tile j holds voxel (oz0 + lz, oy0 + ly0 + 2 j + (r >> 4), ox0 + (r & 15)) ----
-template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false>
+// FULL: the tile lies inside the output and the statistics cover all of its planes (uniform, checked by the caller): no per-lane predicates,
+// so the whole epilogue is straight-line code the scheduler can interleave across the accumulator tiles
+template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false>
 __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT][NT], unsigned char *lds, unsigned tile, int n, int cs,
                                               int oz0, int oy0, int ox0, int lz, int ly0, int tid) {
     const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
@@ -270,9 +272,9 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
         static_for<NT>([&](auto J) {
             constexpr int j = J;
             const int oz = oz0 + lz, oy = oy0 + ly0 + 2 * j + (r >> 4), ox = ox0 + (r & 15);
-            const bool ok = oz < a.Do && oy < a.Ho && ox < a.Wo;
+            const bool ok = FULL || (oz < a.Do && oy < a.Ho && ox < a.Wo);
             const size_t ov = ((size_t)(oz + a.yzo) * a.Ho + oy) * a.Wo + ox;
-            const bool zst = ok && oz >= a.zs0 && oz < a.zs1;
+            const bool zst = FULL || (ok && oz >= a.zs0 && oz < a.zs1);
             float v[16];
             float am = 0.f;
 #pragma unroll

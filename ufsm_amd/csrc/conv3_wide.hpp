@@ -323,7 +323,9 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         while (fbi <= fmax) { prep_next(rq, npairs); issue(rq); }       // (tiles too short to stream everything)
         if (nxt.ok) { wstage(0, nxt.cs, 0); wstage(1, nxt.cs, SLOT); }
         DBG_MARK(3);
-        conv_epilogue<MT, NT, OUT, EPI, true, true>(a, acc, lds, cur.tile, cur.n, cur.cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+        if (cur.oz0 + TZ <= a.Do && cur.oy0 + 8 <= a.Ho && cur.ox0 + 16 <= a.Wo && a.zs0 <= cur.oz0 && a.zs1 >= cur.oz0 + TZ)      // (uniform)
+            conv_epilogue<MT, NT, OUT, EPI, true, true, true>(a, acc, lds, cur.tile, cur.n, cur.cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+        else conv_epilogue<MT, NT, OUT, EPI, true, true>(a, acc, lds, cur.tile, cur.n, cur.cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
         DBG_MARK(4);
         if (!nxt.ok) break;
         cur = nxt; rot = (rot + (unsigned)a.nbt) % 3u;
