@@ -17,7 +17,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 METRIC = "U-Net infer voxels/s (128^3 patch, MX fp8) + 3x3x3 conv % of MFMA peak"
-TRAFFIC_BYTES_PER_LAUNCH = 184.1e6     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/
+TRAFFIC_BYTES_PER_LAUNCH = 183.9e6     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/
 MFMA_PEAK_FP8_TFLOPS = 5033.0          # MI355X dense MXFP8 (2.5 PFLOP/s bf16 x 2)
 
 
@@ -151,8 +151,8 @@ def sliding_leg(np, lib, LP, DevBuf):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target seconds of CPU work for the cpu_baseline sample")
     ap.add_argument("--no-unet", action="store_true", help="skip the configs[3] U-Net forward leg")
