@@ -201,9 +201,8 @@ def main():
             dst = act[l & 1]
             gp = gnp_t() if l == 0 else LP.gn(gam[l - 1], bet[l - 1], mean[l - 1], rstd[l - 1], G)
             sp = split_t(); sp.wkey = 100 + l            # weights are constant across steps: prepared once (inference)
-            lib.mi_gn_sums_zero(sums[l].ptr, N * G * 2)
-            lib.lp_conv_fwd_f8(src.ptr, 3, xs, ws[l].ptr, bs[l].ptr, Cc, dst.ptr, 3, gp, sums[l].ptr, G, sp)
-            lib.mi_gn_finalize(sums[l].ptr, N * G, (Cc // G) * S, 1e-5, mean[l].ptr, rstd[l].ptr)
+            # the op layer's call (host/nn_host.c): conv with fused statistics whose reduction sets the sum slots and finalises mean / rstd
+            lib.mi_conv_fwd_gn(8, src.ptr, 3, xs, ws[l].ptr, bs[l].ptr, Cc, dst.ptr, 3, gp, sums[l].ptr, G, sp, 1e-5, mean[l].ptr, rstd[l].ptr)
             src = dst
 
     for _ in range(a.warmup):
