@@ -25,6 +25,9 @@ typedef struct { int nseq, S, D, Hh, W; const int *lens; const float *pos; const
    one E8M0 scale per 32 K from the fmaxf maximum, round to nearest; block-scaled MFMA products, fp32 accumulation. Returns 0, or -1 for
    another bit width. */
 int lp_mx_gemm(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *Cm, float beta);
+/* no counterpart in the reference: keep operand B's packed MX form across this thread's calls, keyed by pointer and shape (inference: B is a
+   constant weight matrix); dropped by lp_wmemo_clear(). Off by default. */
+void lp_mx_gemm_bmemo(int on);
 /* replaces lp_mx_gemm_ex (src/attn.h:189; src/lp_mxgemm.cu:281-294): the same with an epilogue, C = op(A) op(B) + bias[col] (null: none)
    + res[row][col] (null: none; row stride N; may alias C only with beta 0) + beta C. With few output tiles and a long K (no bias,
    no residual, beta 0 or 1) the K range is split over workgroups that add into C with floating-point atomics, as the reference does:

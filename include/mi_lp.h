@@ -45,6 +45,9 @@ int lp_conv_fwd_s2_f8(const void *x, int xbf, shape5 xs, const float *w, const f
 /* prepared-weight memo (src/nn_lp.h:56-57): a conv called with sp.wkey != 0 reuses its quantised weights until the next step / clear */
 void lp_wmemo_step(unsigned step);
 void lp_wmemo_clear(void);
+/* no counterpart in the reference (its stride-2 entry carries no split_t and prepares the weights per call): memo id of the calling thread's
+   next lp_conv_fwd_s2_f8, as split_t.wkey for the stride-1 entries; consumed by that call. For inference loops with constant weights. */
+void mi_conv_s2_wkey(unsigned wkey);
 gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean, const float *rstd, int G);   /* src/nn_lp.h:19 */
 int lp_gn_slab_any(void);                                                                         /* src/nn_lp.h:20: always 0 here */
 

@@ -72,14 +72,14 @@ __device__ __forceinline__ v8i a8_frag(const uint8_t *p) {
     return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
 }
 
-// grid (ceil(S / 128), H, nseq), 4 wavefronts of 32 queries each. Fragments are the quantised tensors' rows as they lie in memory
+// grid (ceil(S / (32 nw)), H, nseq), nw = 4 or 1 wavefronts of 32 queries each. Fragments are the quantised tensors' rows as they lie in memory
 // (32 contiguous bytes per lane), loaded from global memory directly: a sequence's K and V of one head are 7 KB per 64 keys and stay in
 // L2 / the vector cache across the workgroup's wavefronts.
 __global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, const uint8_t *__restrict__ Q8s, const uint8_t *__restrict__ K8, const uint8_t *__restrict__ K8s,
                                                 const uint8_t *__restrict__ Vt, const uint8_t *__restrict__ Vts, float *__restrict__ o, float *__restrict__ lse,
                                                 int S, int Sp, int H, int C, long long R, float sl2) {
     const int seq = blockIdx.z, hd = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
-    const int q0 = blockIdx.x * 128 + wave * 32;
+    const int q0 = (blockIdx.x * (blockDim.x >> 6) + wave) * 32;      // wavefronts are independent: any number per workgroup
     if (q0 >= S) return;                                   // (no barriers: a wavefront without queries leaves)
     const long long rb = (long long)hd * R + (long long)seq * Sp;          // the sequence's first row in the row-quantised tensors
     const long long c0 = (long long)seq * Sp;                              // its first column in the transposed one
@@ -183,8 +183,10 @@ extern "C" int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom 
     a8_rq_k<<<gq, 256>>>(Qh, q8, qs, H, g->nseq, g->S, Sp, Tp);
     a8_rq_k<<<gq, 256>>>(Kh, k8, ks, H, g->nseq, g->S, Sp, Tp);
     a8_tq_k<<<(unsigned)(H * (R / 32)), 64>>>(Vh, vt, vts, H, g->nseq, g->S, Sp, Tp);
-    const dim3 grid((unsigned)((g->S + 127) / 128), (unsigned)H, (unsigned)g->nseq);
-    a8_fwd_k<<<grid, 256>>>(q8, qs, k8, ks, vt, vts, o, lse, g->S, Sp, H, C, R, 1.4426950408889634f / sqrtf((float)HD));
+    // few query tiles (a 16^3 bottleneck: 129 per head): one wavefront per workgroup, so that every CU gets some
+    const int nw = (size_t)((g->S + 127) / 128) * H * g->nseq >= 512 ? 4 : 1;
+    const dim3 grid((unsigned)((g->S + 32 * nw - 1) / (32 * nw)), (unsigned)H, (unsigned)g->nseq);
+    a8_fwd_k<<<grid, 64 * nw>>>(q8, qs, k8, ks, vt, vts, o, lse, g->S, Sp, H, C, R, 1.4426950408889634f / sqrtf((float)HD));
     MICK();
     return 0;
 }

@@ -118,9 +118,11 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
 struct wmemo_t { unsigned key; const float *w; int fmt, Co, Ci, Cx, nbt, CB, nmt_all, dev; uint8_t *wq, *wsc; };
 static std::vector<wmemo_t> g_wmemo;
 static unsigned g_wstep = 0;
+void mx_gemm_memo_clear(void);
 extern "C" void lp_wmemo_clear(void) {
-    if (g_wmemo.empty()) return;
     MIRT(hipDeviceSynchronize());
+    mx_gemm_memo_clear();
+    if (g_wmemo.empty()) return;
     for (auto &m : g_wmemo) { MIRT(hipFree(m.wq)); MIRT(hipFree(m.wsc)); }
     g_wmemo.clear();
 }
@@ -375,10 +377,14 @@ extern "C" int lp_conv_fwd_f8(const void *x, int xbf, shape5 xs, const float *w,
 extern "C" int lp_conv_fwd_f4(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp) {
     return conv_dispatch("lp_conv_fwd_f4", 4, 1, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, nullptr, nullptr, 0);
 }
+// prepared-weight memo id of the calling thread's next stride-2 conv (its signature carries no split_t): 0 = prepare per call
+static thread_local unsigned g_s2_wkey = 0;
+extern "C" void mi_conv_s2_wkey(unsigned wkey) { g_s2_wkey = wkey; }
 extern "C" int lp_conv_fwd_s2_f8(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, shape5 ys, gnp_t gp) {
     const int Do = (xs.d - 1) / 2 + 1, Ho = (xs.h - 1) / 2 + 1, Wo = (xs.w - 1) / 2 + 1;
     if (ys.d != Do || ys.h != Ho || ys.w != Wo || ys.c != cout || ys.n != xs.n) mi_die("lp_conv_fwd_s2_f8: output shape %d x %d x %d x %d x %d does not match a stride-2 conv of the input", ys.n, ys.c, ys.d, ys.h, ys.w);
     split_t sp; memset(&sp, 0, sizeof sp);
+    sp.wkey = g_s2_wkey; g_s2_wkey = 0;
     // compute format as the reference's dispatch (src/lp_s2.cu:647-754): fp4 only for an MX-fp4 32 -> <= 32 channel conv on even dims, else fp8
     const bool f4 = xbf == 4 && xs.c == 32 && cout <= 32 && !(xs.d & 1) && !(xs.h & 1) && !(xs.w & 1);
     conv_dispatch("lp_conv_fwd_s2_f8", f4 ? 4 : 8, 2, x, xbf, xs, w, b, cout, y, ybf, gp, nullptr, 0, sp, nullptr, nullptr, 0);

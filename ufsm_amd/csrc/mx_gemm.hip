@@ -1,6 +1,7 @@
 // MX GEMM of row-major fp32 operands (the attention stage's linear layers): both operands are quantised along K once, into block rows
 // that are MFMA fragments as they lie in memory, then a block-scaled MFMA GEMM runs over the packed bytes.
 // Interface and arithmetic: src/lp_mxgemm.cu:1-5 (definition), :88-113 (packing), :266-297 (entry points) of the reference.
+#include <vector>
 #include "mx_dev.hpp"
 #include "../../include/mi_attn.h"
 
@@ -100,6 +101,17 @@ __global__ void __launch_bounds__(256) mx_gemm_k(const uint8_t *__restrict__ Aq,
         }
 }
 
+// Packed form of operand B kept across calls (inference: B is a weight matrix that does not change): keyed by pointer and shape, on by
+// lp_mx_gemm_bmemo(1) for the calling thread, dropped by lp_wmemo_clear() like the convs' prepared weights.
+struct bmemo_t { const float *B; int bits, tb, N, K, dev; uint8_t *q, *s; };
+static std::vector<bmemo_t> g_bmemo;
+static thread_local int g_bmemo_on = 0;
+extern "C" void lp_mx_gemm_bmemo(int on) { g_bmemo_on = on != 0; }
+void mx_gemm_memo_clear(void) {
+    for (auto &m : g_bmemo) { MIRT(hipFree(m.q)); MIRT(hipFree(m.s)); }
+    g_bmemo.clear();
+}
+
 extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res) {
     if (bits != 4 && bits != 8) return -1;
     if (M <= 0 || N <= 0) return 0;
@@ -111,14 +123,24 @@ extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, cons
     if (!base) return -1;
     uint8_t *Aq = base, *Bq = Aq + al(qa), *As = Bq + al(qb), *Bs = As + al(sa);
     const int lda = ta ? M : K, ldb = tb ? K : N;
+    bool bhave = false;
+    if (g_bmemo_on && nkb) {
+        int dev = 0; MIRT(hipGetDevice(&dev));
+        for (auto &m : g_bmemo) if (m.B == B && m.bits == bits && m.tb == tb && m.N == N && m.K == K && m.dev == dev) { Bq = m.q; Bs = m.s; bhave = true; break; }
+        if (!bhave) {
+            uint8_t *q = nullptr, *sc = nullptr;
+            MIRT(hipMalloc((void **)&q, al(qb))); MIRT(hipMalloc((void **)&sc, al(sb)));
+            if (q && sc) { g_bmemo.push_back(bmemo_t{B, bits, tb, N, K, dev, q, sc}); Bq = q; Bs = sc; }     // (packed below, found by the next call)
+        }
+    }
     if (nkb) {
         const unsigned ga = nblk_((size_t)M * nkb, 256), gb = nblk_((size_t)N * nkb, 256);
         if (bits == 8) {
             if (ta) mx_pack_k<8, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<8, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
-            if (tb) mx_pack_k<8, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<8, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
+            if (bhave) {} else if (tb) mx_pack_k<8, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<8, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
         } else {
             if (ta) mx_pack_k<4, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<4, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
-            if (tb) mx_pack_k<4, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<4, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
+            if (bhave) {} else if (tb) mx_pack_k<4, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<4, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
         }
     }
     // few output tiles and a long K (the weight-gradient shape, src/lp_mxgemm.cu:259-265): split K so the GPU's 256 CUs have work

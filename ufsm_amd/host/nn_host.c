@@ -66,6 +66,7 @@ int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn
     if (stride == 2) {                                              /* down conv: no split, no output statistics (src/nn_bwd.cu:120-155) */
         if (x2 || G_out || xdt < 3) return -1;
         const shape5 ys = {xs.n, cout, (xs.d - 1) / 2 + 1, (xs.h - 1) / 2 + 1, (xs.w - 1) / 2 + 1};
+        mi_conv_s2_wkey((unsigned)((uintptr_t)w >> 4) | 1u);        /* inference: prepared once per conv, as the stride-1 convs below */
         lp_conv_fwd_s2_f8(x, xdt, xs, w, b, cout, y, ydt, ys, gp);
         return 0;
     }

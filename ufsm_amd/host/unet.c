@@ -193,8 +193,10 @@ static int tb_fwd(unet *u) {
     if (u->cfg.act_dt == 4) lp_mx4_to_f32(x->a2, ys.n, C, Sg, u->tb_cs); else lp_mx8_to_f32(x->a2, ys.n, C, Sg, u->tb_cs);
     at_cs_to_tok(u->tb_cs, u->tb_tok, P(u, u->reg_off), ys.n, C, (long)Sg, nr);
     at_set_mx(8);
+    lp_mx_gemm_bmemo(1);                                           /* inference: the linears' weights are packed once (dropped by unet_set_params) */
     for (int k = 0; k < u->tbn; k++)
-        if (at_block_fwd(&u->tbd, u->params, &u->tbp[k], u->tb_tok + (size_t)k * TC, u->tb_tok + (size_t)(k + 1) * TC, &u->tbg, &u->tbw)) { fprintf(stderr, "unet: attention block forward failed\n"); return -1; }
+        if (at_block_fwd(&u->tbd, u->params, &u->tbp[k], u->tb_tok + (size_t)k * TC, u->tb_tok + (size_t)(k + 1) * TC, &u->tbg, &u->tbw)) { lp_mx_gemm_bmemo(0); fprintf(stderr, "unet: attention block forward failed\n"); return -1; }
+    lp_mx_gemm_bmemo(0);
     at_tok_to_cs(u->tb_tok + (size_t)u->tbn * TC, u->tb_cs, ys.n, C, (long)Sg, nr);
     if (u->cfg.act_dt == 4) lp_f32_to_mx4(u->tb_cs, ys.n, C, Sg, b->a2); else lp_f32_to_mx8(u->tb_cs, ys.n, C, Sg, b->a2);
     const int G = G_of(u, C);

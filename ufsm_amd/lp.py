@@ -37,6 +37,7 @@ _PROTOS = {
     "lp_conv_fwd_s2_f8": (_I, [_P, _I, shape5, _P, _P, _I, _P, _I, shape5, gnp_t]),
     "lp_wmemo_step": (None, [C.c_uint]),
     "lp_wmemo_clear": (None, []),
+    "mi_conv_s2_wkey": (None, [C.c_uint]),
     "gnp_mk": (gnp_t, [_P, _P, _P, _P, _I]),
     "lp_gn_slab_any": (_I, []),
     "lp_mx8_bytes": (_Z, [_I, _I, _Z]),
@@ -124,6 +125,7 @@ _ATTN_PROTOS = {
     "at_tok_to_cs": (None, [_P, _P, _I, _I, C.c_long, _I]),
     "at_block_fwd": (_I, [C.POINTER(at_dims), _P, C.POINTER(at_bp), _P, _P, C.POINTER(at_geom), C.POINTER(at_ws)]),
     "lp_mx_gemm": (_I, [_I, _I, _I, _I, _I, _I, _P, _P, _P, _F]),
+    "lp_mx_gemm_bmemo": (None, [_I]),
     "lp_mx_gemm_ex": (_I, [_I, _I, _I, _I, _I, _I, _P, _P, _P, _F, _P, _P]),
     "at_fa8_fwd": (_I, [_P, _P, _P, C.POINTER(at_geom), _I, _I]),
 }
