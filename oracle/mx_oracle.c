@@ -419,19 +419,25 @@ static void conv_epilogue(const orc_conv_t *c, int n, size_t ov, size_t So, floa
     if (ls) for (int co = 0; co < Co; co++) { const double v = acc[co]; ls[2 * (co / cpg)] += v; ls[2 * (co / cpg) + 1] += v * v; }
 }
 
-/* ---------- tap-packed small-channel conv (src/lp_f8fwd.cuh:153-177 weights, :178-400 kernel, :601-609 dispatch) ----------
-   Channels padded to CP in {4, 8, 16}; a K block of 32 = 32 / CP taps x CP channels, so a block mixes positions and the activation
-   operand has ONE scale per staged tile: the 4 x 10 x 18 input positions around a 2 x 8 x 16 output tile (tiles on the output grid from
-   the origin). Values outside the volume and channels >= Ci are zeros and take part in nothing; amax ignores NaN (fmaxf). */
+/* ---------- tap-packed small-channel convs ----------
+   stem_tile 1 (src/lp_f8fwd.cuh:153-177 weights, :178-400 kernel, :601-609 dispatch): channels padded to CP in {4, 8, 16}; a K block of 32 =
+   32 / CP taps x CP channels, so a block mixes positions and the activation operand has ONE scale per staged tile: the 4 x 10 x 18 input
+   positions around a 2 x 8 x 16 output tile (tiles on the output grid from the origin).
+   stem_tile 2 (src/lp_f8fwd.cu:72-92 weights, src/lp_f8fwd.cuh:447-563 kernel, :626 dispatch): 9 .. 16 channels in slots of 16, two K blocks
+   per tap row (kz, ky): [kx0 | kx1] and [kx2 | 0], so a block spans two positions of one staged row and the activation operand has one
+   scale per staged ROW: the 18 positions x - 1 .. x + 16 of a (z, y) line inside a 16-wide x tile.
+   Values outside the volume and channels >= Ci are zeros; amax ignores NaN (fmaxf). */
 static int conv3_stem(const orc_conv_t *c) {
-    const int Ci = c->Ci, Co = c->Co, D = c->D, H = c->H, W = c->W;
-    if (c->x2 || c->up || c->stride == 2 || c->cbits != 8 || Ci > 16 || (c->xdt != 0 && Ci > 8)) return -2;
-    const int CP = Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK;
+    const int Ci = c->Ci, Co = c->Co, D = c->D, H = c->H, W = c->W, rowmode = c->stem_tile == 2;
+    if (c->x2 || c->up || c->stride == 2 || c->cbits != 8 || Ci > 16 || (!rowmode && c->xdt != 0 && Ci > 8)) return -2;
+    const int CP = rowmode ? 16 : Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = 32 / CP, NKB = rowmode ? 18 : (27 + TPK - 1) / TPK;
     const size_t S = (size_t)D * H * W;
+    /* K block kb, element k -> (tap, channel), tap 27 = none */
+#define STEM_TAP(kb, k) (rowmode ? (2 * ((kb) & 1) + ((k) >> 4) < 3 ? ((kb) >> 1) * 3 + 2 * ((kb) & 1) + ((k) >> 4) : 27) : ((kb) * TPK + (k) / CP < 27 ? (kb) * TPK + (k) / CP : 27))
     float *wv = (float *)malloc((size_t)NKB * Co * 32 * sizeof(float)), *wsf = (float *)malloc((size_t)NKB * Co * sizeof(float));
-    for (int kb = 0; kb < NKB; kb++) for (int co = 0; co < Co; co++) {            /* prep_w8s_k */
+    for (int kb = 0; kb < NKB; kb++) for (int co = 0; co < Co; co++) {            /* prep_w8s_k / prep_w8p_k */
         float v[32], amax = 0.f;
-        for (int k = 0; k < 32; k++) { const int tap = kb * TPK + k / CP, ci = k % CP; v[k] = ci < Ci && tap < 27 ? c->w[((size_t)co * Ci + ci) * 27 + tap] : 0.f; amax = fmaxf(amax, fabsf(v[k])); }
+        for (int k = 0; k < 32; k++) { const int tap = STEM_TAP(kb, k), ci = k % CP; v[k] = ci < Ci && tap < 27 ? c->w[((size_t)co * Ci + ci) * 27 + tap] : 0.f; amax = fmaxf(amax, fabsf(v[k])); }
         const int e = orc_mx_exp(amax, INVQ8); const float m = orc_exp2i(-e);
         for (int k = 0; k < 32; k++) wv[((size_t)kb * Co + co) * 32 + k] = orc_dec_e4m3(orc_enc_e4m3(v[k] * m));
         wsf[(size_t)kb * Co + co] = orc_mx_scale((unsigned)(e + 127));
@@ -457,19 +463,24 @@ static int conv3_stem(const orc_conv_t *c) {
             float *acc = (float *)malloc((size_t)Co * sizeof(float)), *bq = (float *)malloc((size_t)720 * CP * sizeof(float));
             double *acc64 = (double *)malloc((size_t)Co * sizeof(double));
             double *ls = gs ? (double *)calloc((size_t)2 * c->Go, sizeof(double)) : NULL;
+            double rsf[40];                                   /* scale of each staged row (rowmode) or of the tile (all equal) */
 #pragma omp for schedule(dynamic, 4)
             for (int ti = 0; ti < ntz * nty * ntx; ti++) {
                 const int tz = ti / (nty * ntx), ty = ti / ntx % nty, tx = ti % ntx;
                 if (2 * tz + 2 <= z0 || 2 * tz >= z1) continue;
-                /* the tile's 720 staged positions, its amax and scale (src/lp_f8fwd.cuh:340-388) */
-                float amax = 0.f;
+                /* the tile's 720 staged positions = 40 rows of 18, their amax and scales (src/lp_f8fwd.cuh:340-388, :480-520) */
+                float amax[40]; for (int r = 0; r < 40; r++) amax[r] = 0.f;
                 for (int p = 0; p < 720; p++) {
                     const int gz = 2 * tz - 1 + p / 180, gy = 8 * ty - 1 + p / 18 % 10, gx = 16 * tx - 1 + p % 18;
                     const int inb = gz >= 0 && gz < D && gy >= 0 && gy < H && gx >= 0 && gx < W;
-                    for (int k = 0; k < CP; k++) { const float v = inb ? val[(((size_t)gz * H + gy) * W + gx) * CP + k] : 0.f; bq[p * CP + k] = v; amax = fmaxf(amax, fabsf(v)); }
+                    for (int k = 0; k < CP; k++) { const float v = inb ? val[(((size_t)gz * H + gy) * W + gx) * CP + k] : 0.f; bq[p * CP + k] = v; amax[p / 18] = fmaxf(amax[p / 18], fabsf(v)); }
                 }
-                const int e = orc_mx_exp(amax, INVQ8); const float m = orc_exp2i(-e); const double sbf = orc_mx_scale((unsigned)(e + 127));
-                for (int i = 0; i < 720 * CP; i++) bq[i] = orc_dec_e4m3(orc_enc_e4m3(bq[i] * m));
+                if (!rowmode) { float am = 0.f; for (int r = 0; r < 40; r++) am = fmaxf(am, amax[r]); for (int r = 0; r < 40; r++) amax[r] = am; }
+                for (int r = 0; r < 40; r++) {
+                    const int e = orc_mx_exp(amax[r], INVQ8); const float m = orc_exp2i(-e);
+                    rsf[r] = orc_mx_scale((unsigned)(e + 127));
+                    for (int i = r * 18 * CP; i < (r + 1) * 18 * CP; i++) bq[i] = orc_dec_e4m3(orc_enc_e4m3(bq[i] * m));
+                }
                 for (int l = 0; l < 256; l++) {
                     const int oz = 2 * tz + l / 128, oy = 8 * ty + l / 16 % 8, ox = 16 * tx + l % 16;
                     if (oz >= D || oy >= H || ox >= W || oz < z0 || oz >= z1) continue;
@@ -478,12 +489,13 @@ static int conv3_stem(const orc_conv_t *c) {
                     for (int kb = 0; kb < NKB; kb++)
                         for (int co = 0; co < Co; co++) {
                             const float *wr = wv + ((size_t)kb * Co + co) * 32;
-                            double d = 0.0;
+                            double d = 0.0; int row = 0;
                             for (int k = 0; k < 32; k++) {
-                                const int tap = kb * TPK + k / CP; if (tap >= 27) break;
-                                d += (double)wr[k] * (double)bq[(p0 + (tap / 9) * 180 + (tap / 3 % 3) * 18 + tap % 3) * CP + k % CP];
+                                const int tap = STEM_TAP(kb, k); if (tap >= 27) continue;
+                                const int p = p0 + (tap / 9) * 180 + (tap / 3 % 3) * 18 + tap % 3;
+                                d += (double)wr[k] * (double)bq[p * CP + k % CP]; row = p / 18;
                             }
-                            const double blk = d * (double)wsf[(size_t)kb * Co + co] * sbf;
+                            const double blk = d * (double)wsf[(size_t)kb * Co + co] * rsf[row];     /* (a block's positions share the row, or the tile, scale) */
                             if (c->acc64) acc64[co] += blk; else acc[co] += (float)blk;
                         }
                     conv_epilogue(c, n, ((size_t)oz * H + oy) * W + ox, S, acc, acc64, ls);
@@ -498,6 +510,7 @@ static int conv3_stem(const orc_conv_t *c) {
         }
         if (gs) { for (int i = 0; i < 2 * c->Go; i++) c->osum[(size_t)n * 2 * c->Go + i] += gs[i]; free(gs); }
     }
+#undef STEM_TAP
     free(val); free(wv); free(wsf);
     return 0;
 }

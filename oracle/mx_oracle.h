@@ -34,6 +34,8 @@
  *                                 convolution for the three channel paddings and all input types; one large value coarsens exactly the
  *                                 output voxels of the 2 x 8 x 16 tiles whose 4 x 10 x 18 halo holds it; a one-tile volume returns the
  *                                 tensor under one scale (tests/test_oracle_stem.py)
+ *   ... with stem_tile 2          the 9 .. 16 channel form with one scale per staged row (src/lp_f8fwd.cuh:447-563): exact operands equal the
+ *                                 fp64 convolution; one large value coarsens exactly the outputs of its x tile that read its (z, y) line
  */
 #ifndef MX_ORACLE_H
 #define MX_ORACLE_H
@@ -95,7 +97,8 @@ typedef struct {
     int acc64;                         /* 1: accumulate in fp64 (exact-operand checks) */
     int fused_act; const float *ep_a, *ep_b;   /* extension: epilogue affine + activation (1 SiLU, 2 GELU, 3 ReLU) before requant */
     int z0, z1;                        /* output z planes [z0, z1) only (z1 0: all): the bounded CPU-baseline slab */
-    int stem_tile;                     /* 1: one activation scale per staged 4x10x18 tile (Ci <= 8 tap-packed stem) */
+    int stem_tile;                     /* 1: one activation scale per staged 4x10x18 tile (Ci <= 8 tap-packed stem); 2: 9 .. 16 channels, two taps per K
+                                          block, one activation scale per staged row of 18 positions */
 } orc_conv_t;
 /* 3x3x3 forward conv with MX operands (src/lp_f8fwd.cuh:19-151, src/lp_common.cuh:1465-1597, src/lp_s2.cu:4-9) */
 int orc_conv3(const orc_conv_t *c);

@@ -116,3 +116,47 @@ def test_stem_nonfinite_and_weight_memo(gpu):
     assert bad[:2, :8, :16].all() and bad.sum() == 2 * 8 * 16                                      # voxel 5 = (0, 0, 5): only the first tile's halo holds it
     clean, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, None, Co, 3)
     assert np.array_equal(orc.mx_to_f32(8, clean, N, Co, S)[fin], dg[fin])
+
+
+# ---- 9 .. 16 channels of an MX or fp16 input: two taps per K block, one activation scale per staged row (src/lp_f8fwd.cuh:447-563) ----
+@pytest.mark.parametrize("xdt,Ci,Co,dims", [(3, 16, 32, (4, 8, 16)), (3, 9, 16, (3, 9, 17)), (3, 12, 48, (5, 11, 21)), (4, 16, 32, (3, 8, 33)), (2, 10, 64, (2, 8, 16)), (3, 16, 96, (4, 16, 32))])
+def test_row_scale_conv_exact_operands(gpu, xdt, Ci, Co, dims):
+    rng = np.random.default_rng(xdt * 100 + Ci * 7 + Co)
+    D, H, W = dims
+    N, S = 2, D * H * W
+    x = refnp.gen_exact(rng, (N, Ci, S), force6=False)
+    w = refnp.gen_exact(rng, (Co, Ci, 27), force6=False)
+    b = (GRID[rng.integers(0, 8, Co)] * 0.25).astype(np.float32)
+    xin = stored(x, xdt, N, Ci, S)
+    G = 8 if Co % 8 == 0 else 1
+    for ydt in (3, 4):
+        want, ws = orc.conv3(xin, xdt, N, Ci, D, H, W, w, b, Co, ydt, stem_tile=2, acc64=1, Go=G, want_stats=True)
+        got, gs = gpu_conv(xin, xdt, N, Ci, D, H, W, w, b, Co, ydt, Go=G, stats=(Co // G) % 4 == 0 or Co <= 32)
+        assert "conv3_p16_k" in lib.mi_last_kernel().decode()
+        assert np.array_equal(got, want), ydt
+        if gs is not None:
+            assert np.abs(gs - ws).max() / np.abs(ws).max() < 1e-5
+
+
+@pytest.mark.parametrize("xdt,Ci,Co,dims,gn", [(3, 16, 32, (6, 20, 40), False), (3, 11, 64, (5, 9, 35), False), (2, 16, 32, (4, 8, 24), False), (3, 16, 32, (4, 12, 20), True)])
+def test_row_scale_conv_random_data(gpu, xdt, Ci, Co, dims, gn):
+    rng = np.random.default_rng(xdt + Ci + Co)
+    D, H, W = dims
+    N, S = 2, D * H * W
+    x = rng.standard_normal((N, Ci, S)).astype(np.float32)
+    x[:, :, S // 3] *= 40.0                                                   # rows of very different scales
+    w = (rng.standard_normal((Co, Ci, 27)) * np.sqrt(2.0 / (Ci * 27))).astype(np.float32)
+    b = (rng.standard_normal(Co) * 0.1).astype(np.float32)
+    xin = stored(x, xdt, N, Ci, S)
+    og = dg = None
+    if gn:
+        G = 4
+        p = [rng.uniform(0.5, 1.5, Ci).astype(np.float32), rng.uniform(-.5, .5, Ci).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+        og, dg = orc.gn(*p, G), dev_gn(*p, G)
+    wq, ws = orc.conv3(xin, xdt, N, Ci, D, H, W, w, b, Co, 3, stem_tile=2, Go=8, want_stats=True, stored_stats=1, gp=og)
+    gq, gs = gpu_conv(xin, xdt, N, Ci, D, H, W, w, b, Co, 3, Go=8, stats=True, stored_stats=1, gp=dg)
+    assert "conv3_p16_k" in lib.mi_last_kernel().decode()
+    frac, near = code_mismatch_fraction(8, gq, wq, N, Co, S)
+    assert frac < (2e-2 if gn else 5e-3) and near
+    dec = orc.mx_to_f32(8, gq, N, Co, S).astype(np.float64).reshape(N, 8, -1)
+    assert np.allclose(gs[:, :, 0], dec.sum(-1), rtol=1e-5, atol=1e-3) and np.allclose(gs[:, :, 1], (dec * dec).sum(-1), rtol=1e-5)

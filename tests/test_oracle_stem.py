@@ -78,3 +78,46 @@ def test_single_tile_uses_one_scale_for_the_whole_operand():
     e = refnp.scale_exp(np.abs(x).max(), 448.0)
     q = np.array([orc.lib().orc_dec_e4m3(orc.lib().orc_enc_e4m3(float(v))) for v in (x * np.float32(2.0 ** -e)).ravel()], np.float32).reshape(x.shape) * np.float32(2.0 ** e)
     assert np.array_equal(y, q)
+
+
+# ---- the 9 .. 16 channel packed conv: two taps per K block, one activation scale per staged row (src/lp_f8fwd.cuh:447-563) ----
+@pytest.mark.parametrize("xdt,Ci,Co,dims", [(3, 16, 32, (4, 8, 16)), (3, 9, 16, (3, 9, 17)), (3, 12, 48, (5, 11, 21)), (4, 16, 32, (3, 8, 33)), (2, 10, 64, (2, 8, 16))])
+def test_row_scale_conv_exact_operands_equal_fp64_conv(xdt, Ci, Co, dims):
+    rng = np.random.default_rng(xdt * 100 + Ci * 7 + Co)
+    D, H, W = dims
+    N, S = 2, D * H * W
+    x = refnp.gen_exact(rng, (N, Ci, S), force6=False)
+    w = refnp.gen_exact(rng, (Co, Ci, 27), force6=False)
+    b = (GRID[rng.integers(0, 8, Co)] * 0.25).astype(np.float32)
+    want = refnp.conv3d_f64(x.reshape(N, Ci, D, H, W), w, b, 1)
+    assert np.array_equal(want.astype(np.float32).astype(np.float64), want)
+    xin = stored(x, xdt, N, Ci, S)
+    y32, _ = orc.conv3(xin, xdt, N, Ci, D, H, W, w, b, Co, 0, stem_tile=2)
+    assert np.array_equal(y32.reshape(want.shape), want.astype(np.float32))
+    yq, _ = orc.conv3(xin, xdt, N, Ci, D, H, W, w, b, Co, 3, stem_tile=2)
+    assert np.array_equal(orc.mx_to_f32(8, yq, N, Co, S), refnp.mx_quant_tensor(want.astype(np.float32).reshape(N, Co, S), 8))
+
+
+def test_row_scale_conv_one_large_value_coarsens_exactly_its_row():
+    rng = np.random.default_rng(6)
+    N, Ci, Co, D, H, W = 1, 12, 8, 5, 12, 40
+    S = D * H * W
+    x = (rng.integers(-3, 4, (N, Ci, D, H, W)) * 2.0 ** -10).astype(np.float32)
+    zs, ys, xs = 2, 5, 8                                             # inside the first 16-wide x tile only (its rows span x = -1 .. 16)
+    x[0, 3, zs, ys, xs] = 384.0
+    w = refnp.gen_exact(rng, (Co, Ci, 27), force6=False)
+    y, _ = orc.conv3(orc.f32_to_mx(8, x.reshape(N, Ci, S), N, Ci, S), 3, N, Ci, D, H, W, w, None, Co, 0, stem_tile=2)
+    xs_in = orc.mx_to_f32(8, orc.f32_to_mx(8, x.reshape(N, Ci, S), N, Ci, S), N, Ci, S).reshape(N, Ci, D, H, W)   # the stored operand (the spike's own
+    exact = refnp.conv3d_f64(xs_in.astype(np.float64), w, None, 1).astype(np.float32).reshape(N, Co, D, H, W)   # voxel row is coarse already)
+    xc = xs_in.copy()
+    steps = np.arange(-8, 9, dtype=np.float32)
+    seg = xc[0, :, zs, ys, 0:17]; small = np.abs(seg) < 1.0          # the staged row of tile 0: x = -1 .. 16, under the spike's scale 2^0
+    seg[small] = steps[refnp.round_to_grid(seg[small] * 512.0, steps)] / 512.0
+    xc[0, :, zs, ys, 0:17] = seg
+    coarse = refnp.conv3d_f64(xc.astype(np.float64), w, None, 1).astype(np.float32).reshape(N, Co, D, H, W)
+    y = y.reshape(N, Co, D, H, W)
+    assert np.array_equal(y[..., :16], coarse[..., :16])             # outputs of the x tile whose row holds the value
+    assert np.array_equal(y[..., 16:], exact[..., 16:])              # the next tile quantises x = 15, 16 of that line with its own row scale
+    assert not np.array_equal(coarse[..., :16], exact[..., :16])
+    far = np.ones((D, H), bool); far[zs - 1:zs + 2, ys - 1:ys + 2] = False
+    assert np.array_equal(y[:, :, far], exact[:, :, far])            # only outputs whose taps read that (z, y) line

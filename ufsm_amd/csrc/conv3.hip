@@ -165,10 +165,11 @@ static void conv_stats_reduce(const char *who, const conv_args &a, int MT, split
 }
 
 // the tap-packed stem (src/lp_f8fwd.cuh:601-609, :421-434): e4m3 compute, one activation scale per staged tile
+// rows: the 9 .. 16 channel form, two taps per K block and one activation scale per staged row (src/lp_f8fwd.cuh:447-563, :626)
 static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
-                     gnp_t gp, double *osum, int Go, split_t sp) {
+                     gnp_t gp, double *osum, int Go, split_t sp, bool rows) {
     const int Ci = xs.c, N = xs.n, D = sp.Di ? sp.Di : xs.d, Do = xs.d, H = xs.h, W = xs.w;      // D: the input's depth (z-range), Do: output planes
-    const int CP = Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2;
+    const int CP = rows ? 0 : Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = rows ? 2 : 32 / CP, NKB = rows ? 18 : (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2;
     conv_args a; memset(&a, 0, sizeof a);
     a.sx = x; a.sxdt = xbf; a.sCi = Ci;
     a.sgam = gp.gamma; a.sbet = gp.beta; a.smean = gp.mean; a.srstd = gp.rstd; a.sG = gp.G;
@@ -176,8 +177,8 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     a.zi0 = sp.Di ? sp.zi0 : 0; a.yD = sp.yD; a.yzo = sp.yD ? sp.yzo : 0;
     a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
     a.osum = osum; a.Go = Go; a.stored_stats = sp.stored_stats && ybf >= 3; a.zs0 = sp.zlo; a.zs1 = Do - sp.zhi;
-    const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 && CP < 16 ? 2 : 1;     // (16 padded channels: 7 weight fragment pairs per channel tile, one tile fits the registers)
-    size_t smem = ((size_t)720 * CP + 16 + CP * 8 + 15) & ~(size_t)15;     // staged tile, amax word, channel affine
+    const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 && CP && CP < 16 ? 2 : 1;     // (16 channels per slot: 7 or 9 weight fragment pairs per channel tile, one tile fits the registers)
+    size_t smem = rows ? (size_t)720 * 16 + 16 + 40 * 4 + 16 * 8 : ((size_t)720 * CP + 16 + CP * 8 + 15) & ~(size_t)15;     // staged tile, (zero row, row words | amax word), channel affine
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);
     a.red_o = (unsigned)smem; smem += 1024;
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
@@ -188,11 +189,11 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
     if (sp.wkey) {                                     // memo entries of this layout: nbt = -CP
         for (auto &m : g_wmemo)
-            if (m.key == sp.wkey && m.w == w && m.fmt == 8 && m.Co == cout && m.Ci == Ci && m.nbt == -CP && m.nmt_all == nmt_all && m.dev == dev) { wq = m.wq; wsc = m.wsc; have = true; break; }
+            if (m.key == sp.wkey && m.w == w && m.fmt == 8 && m.Co == cout && m.Ci == Ci && m.nbt == -CP - 1 && m.nmt_all == nmt_all && m.dev == dev) { wq = m.wq; wsc = m.wsc; have = true; break; }
         if (!have) {
             MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes));
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
-            g_wmemo.push_back(wmemo_t{sp.wkey, w, 8, cout, Ci, Ci, -CP, 0, nmt_all, dev, wq, wsc});
+            g_wmemo.push_back(wmemo_t{sp.wkey, w, 8, cout, Ci, Ci, -CP - 1, 0, nmt_all, dev, wq, wsc});
         }
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) conv3_stem_prep(CP, w, wq, wsc, cout, Ci, nmt_all, NP);
@@ -232,7 +233,10 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     static int stem_env = -1;
     if (stem_env < 0) stem_env = getenv("MI_CONV_STEM") ? atoi(getenv("MI_CONV_STEM")) : 1;     // tuning knob: 0 sends these convs to the general kernel
     if (stem_env && fmt == 8 && stride == 1 && !sp.x2 && !act && (xbf == 0 || xbf >= 2) && Ci <= (xbf == 0 ? 16 : 8) && (xbf == ybf || ybf >= 3))
-        return conv_stem(who, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp);
+        return conv_stem(who, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, false);
+    // 9 .. 16 channels of an MX or fp16 input: two taps per K block, one activation scale per staged row (src/lp_f8fwd.cuh:626)
+    if (stem_env && fmt == 8 && stride == 1 && !sp.x2 && !act && xbf >= 2 && Ci <= 16 && (xbf == ybf || ybf >= 3))
+        return conv_stem(who, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, true);
     const int N = xs.n, D = sp.Di ? sp.Di : xs.d, H = xs.h, W = xs.w;           // D: the inputs' depth
     const int Do = stride == 2 ? (D - 1) / 2 + 1 : xs.d, Ho = stride == 2 ? (H - 1) / 2 + 1 : H, Wo = stride == 2 ? (W - 1) / 2 + 1 : W;   // src/nn_bwd.cu:132-135
     const size_t S = (size_t)D * H * W;

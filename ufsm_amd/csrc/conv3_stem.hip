@@ -163,6 +163,163 @@ __global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
     conv_epilogue<MT, NT, OUT, false>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
 }
 
+// ---- 9 .. 16 input channels (src/lp_f8fwd.cuh:447-563, weights src/lp_f8fwd.cu:72-92): the channels sit in slots of 16 and a tap row
+// (kz, ky) is two K blocks, [kx0 | kx1] and [kx2 | 0], so a conv is 9 MFMAs per tile pair instead of 27 half-empty ones. A block spans two
+// positions of one staged row, so the activation operand has one E8M0 scale per staged ROW: the 18 positions x - 1 .. x + 16 of a (z, y)
+// line of the tile (amax by LDS atomicMax over the row; fmaxf semantics). Same tile, wavefront layout and epilogue as the stem kernel.
+// Lane (r, h) of an MFMA supplies bytes 16 h .. 16 h + 15 of both blocks: h = 0 the rows of positions p (kx0) and p + 2 (kx2), h = 1 the row of
+// p + 1 (kx1) and a zero row; its scale operand is the staged row's.
+template <int MT, int OUT>
+__global__ void __launch_bounds__(256, 2) conv3_p16_k(const conv_args a) {
+    constexpr int NT = 2, HY = 10, HX = 18, NROW = 4 * HY, TT = NROW * HX, WTILE = 2048;
+    extern __shared__ __align__(16) unsigned char lds[];
+    // LDS: [staged tile TT x 16 bytes][zero row 16][row amax / scale words NROW][per channel (a, b): 16 x float2]
+    constexpr unsigned z_o = TT * 16, ra_o = z_o + 16, ab_o = ra_o + NROW * 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    unsigned tile;
+    {
+        const unsigned per = (a.ntiles + 7u) / 8u;
+        tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
+        if (tile >= a.ntiles) return;
+    }
+    int tt = (int)tile;
+    const int cs = tt % a.ncs; tt /= a.ncs;
+    const int tx = tt % a.ntx; tt /= a.ntx;
+    const int ty = tt % a.nty; tt /= a.nty;
+    const int tz = tt % a.ntz; const int n = tt / a.ntz;
+    const int ox0 = tx * 16, oy0 = ty * 8, oz0 = tz * 2;
+    const int Ci = a.sCi;
+    const size_t S = (size_t)a.D * a.H * a.W;
+    if (tid < 4) *(unsigned *)(lds + z_o + tid * 4) = 0u;
+    if (tid < NROW) *(unsigned *)(lds + ra_o + tid * 4) = 0u;
+    if (tid < 16) {
+        float ga = 1.f, gb = 0.f;
+        if (a.sG && tid < Ci) { const int ng = n * a.sG + tid / (Ci / a.sG); ga = a.srstd[ng] * a.sgam[tid]; gb = fmaf(-a.smean[ng], ga, a.sbet[tid]); }
+        *(float2 *)(lds + ab_o + tid * 8) = make_float2(ga, gb);
+    }
+    conv_epi_consts<MT, false>(a, lds, cs, tid);
+    v8i fa[9][MT]; int sa[9][MT];
+#pragma unroll
+    for (int p = 0; p < 9; p++)
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const size_t t = (size_t)p * a.nmt_all + cs * MT + m;
+            const v4i lo = *(const v4i *)(a.wq + t * WTILE + lane * 16), hi = *(const v4i *)(a.wq + t * WTILE + 1024 + lane * 16);
+            fa[p][m] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            sa[p][m] = *(const int *)(a.wsc + (t * 64 + lane) * 4);
+        }
+    __syncthreads();
+    // ---- stage: a thread owns positions tid, tid + 256, tid + 512; values stay in registers until the row's amax is known ----
+    float v[3][16];
+    const int xdt = a.sxdt;
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int pos = tid + 256 * j, row = pos / HX, ix = pos - row * HX;
+        const int gz = oz0 - 1 + row / HY + a.zi0, gy = oy0 - 1 + row % HY, gx = ox0 - 1 + ix;
+        const bool inb = pos < TT && (unsigned)gz < (unsigned)a.D && (unsigned)gy < (unsigned)a.H && (unsigned)gx < (unsigned)a.W;
+        const size_t off = inb ? ((size_t)gz * a.H + gy) * a.W + gx : 0;
+        float x[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) x[k] = 0.f;
+        if (xdt == 3) {                                      // one MX-fp8 row of 16 channels per voxel, then the scale plane
+            const uint8_t *q = (const uint8_t *)a.sx;
+            const float s = d_mx_scale(q[(size_t)a.N * S * 16 + (size_t)n * S + off]);
+            const uint4 w4 = *(const uint4 *)(q + ((size_t)n * S + off) * 16);
+            d_dec4_e4m3(w4.x, x); d_dec4_e4m3(w4.y, x + 4); d_dec4_e4m3(w4.z, x + 8); d_dec4_e4m3(w4.w, x + 12);
+#pragma unroll
+            for (int k = 0; k < 16; k++) x[k] *= s;
+        } else if (xdt == 4) {                               // one MX-fp4 row of 16 channels (8 bytes) per voxel
+            const uint8_t *q = (const uint8_t *)a.sx;
+            const float s = d_mx_scale(q[(size_t)a.N * S * 8 + (size_t)n * S + off]);
+            const uint2 w2 = *(const uint2 *)(q + ((size_t)n * S + off) * 8);
+            d_dec8_e2m1(w2.x, x); d_dec8_e2m1(w2.y, x + 8);
+#pragma unroll
+            for (int k = 0; k < 16; k++) x[k] *= s;
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; k++)
+                if (k < Ci) {
+                    const size_t idx = ((size_t)n * Ci + k) * S + off;
+                    x[k] = xdt == 2 ? __half2float(((const __half *)a.sx)[idx]) : ((const float *)a.sx)[idx];
+                }
+        }
+        float am = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            float val = x[k];
+            if (a.sG) { const float2 ab = *(const float2 *)(lds + ab_o + k * 8); val = d_act_ab(val, ab.x, ab.y); }
+            val = inb && k < Ci ? val : 0.f;
+            v[j][k] = val; am = fmaxf(am, fabsf(val));
+        }
+        if (pos < TT && am != 0.f) atomicMax((unsigned *)(lds + ra_o + row * 4), __float_as_uint(am));
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 3; j++) {
+        const int pos = tid + 256 * j, row = pos / HX;
+        if (pos < TT) {
+            const int e = d_mx_exp(__uint_as_float(*(const unsigned *)(lds + ra_o + row * 4)), MI_INVQ8);
+            uint4 o;
+            o.x = d_enc4_e4m3(v[j][0], v[j][1], v[j][2], v[j][3], e); o.y = d_enc4_e4m3(v[j][4], v[j][5], v[j][6], v[j][7], e);
+            o.z = d_enc4_e4m3(v[j][8], v[j][9], v[j][10], v[j][11], e); o.w = d_enc4_e4m3(v[j][12], v[j][13], v[j][14], v[j][15], e);
+            *(uint4 *)(lds + pos * 16) = o;
+        }
+    }
+    __syncthreads();                                         // every position is encoded with its row's amax ...
+    if (tid < NROW) { unsigned *p = (unsigned *)(lds + ra_o + tid * 4); *p = (unsigned)(d_mx_exp(__uint_as_float(*p), MI_INVQ8) + 127); }
+    __syncthreads();                                         // ... which then becomes the row's scale word
+    const int lz = wave >> 1, ly0 = (wave & 1) * 4;
+    const int row00 = lz * HY + ly0 + (r >> 4), p00 = row00 * HX + (r & 15);
+    v16f acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
+    static_for<9>([&](auto R) {
+        constexpr int tr = R, kz = tr / 3, ky = tr % 3;
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            const int row = row00 + 2 * j + kz * HY + ky, p = p00 + (2 * j + kz * HY + ky) * HX;
+            const v4i lo = *(const v4i *)(lds + (p + h) * 16);
+            const v4i hi = *(const v4i *)(lds + (h ? z_o : (unsigned)(p + 2) * 16u));
+            const v8i fb = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            const int sb = *(const int *)(lds + ra_o + row * 4);
+#pragma unroll
+            for (int m = 0; m < MT; m++) acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[tr][m], fb, acc[m][j], 0, 0, 0, sa[tr][m], 0, sb);
+        }
+    });
+    __syncthreads();
+    conv_epilogue<MT, NT, OUT, false>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
+}
+// its weights: tap row r = (kz, ky), block 2 r = [kx0 | kx1], block 2 r + 1 = [kx2 | 0], 16 channels per slot (src/lp_f8fwd.cu:72-92)
+__global__ void __launch_bounds__(128) prep_wp16_k(const float *__restrict__ w, uint8_t *__restrict__ wq, unsigned *__restrict__ wsc, int Co, int Ci, int nmt_all) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x, Cop = nmt_all * 32;
+    if (i >= 9 * Cop) return;
+    const int cop = i % Cop, p = i / Cop, m = cop >> 5, r = cop & 31;
+    uint8_t *tile = wq + ((size_t)p * nmt_all + m) * 2048;
+    unsigned *tsc = wsc + ((size_t)p * nmt_all + m) * 64;
+#pragma unroll
+    for (int side = 0; side < 2; side++) {
+        float v[32]; float amax = 0.f;
+#pragma unroll
+        for (int k = 0; k < 32; k++) {
+            const int kx = 2 * side + (k >> 4), ci = k & 15;
+            v[k] = (kx < 3 && cop < Co && ci < Ci) ? w[((size_t)cop * Ci + ci) * 27 + p * 3 + kx] : 0.f;
+            amax = fmaxf(amax, fabsf(v[k]));
+        }
+        const int e = d_mx_exp(amax, MI_INVQ8);
+        const float mult = d_exp2i(-e);
+        unsigned c[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) c[j] = d_enc_e4m3x4(v[4 * j] * mult, v[4 * j + 1] * mult, v[4 * j + 2] * mult, v[4 * j + 3] * mult);
+        *(uint4 *)(tile + ((size_t)(side * 64 + r) * 16)) = make_uint4(c[0], c[1], c[2], c[3]);
+        *(uint4 *)(tile + ((size_t)(side * 64 + r + 32) * 16)) = make_uint4(c[4], c[5], c[6], c[7]);
+        tsc[r + 32 * side] = (unsigned)(e + 127);
+    }
+}
+
 // weights: fp32 w[co][ci][27] -> per (block pair, 32-row channel tile) fragment-ordered e4m3 codes + one scale word per lane
 // (src/lp_f8fwd.cuh:156-177): block kb, k -> tap kb * TPK + k / CP, channel k % CP; zeros past the taps, the channels and the rows
 template <int CP>
@@ -196,6 +353,7 @@ __global__ void __launch_bounds__(128) prep_ws_k(const float *__restrict__ w, ui
 
 void conv3_stem_prep(int CP, const float *w, uint8_t *wq, uint8_t *wsc, int Co, int Ci, int nmt_all, int np) {
     const unsigned nb = nblk_((size_t)np * nmt_all * 32, 128);
+    if (CP == 0) { prep_wp16_k<<<nb, 128>>>(w, wq, (unsigned *)wsc, Co, Ci, nmt_all); MICK(); return; }       // (CP 0: the two-taps-per-block layout)
     if (CP == 4) prep_ws_k<4><<<nb, 128>>>(w, wq, (unsigned *)wsc, Co, Ci, nmt_all, np);
     else if (CP == 8) prep_ws_k<8><<<nb, 128>>>(w, wq, (unsigned *)wsc, Co, Ci, nmt_all, np);
     else prep_ws_k<16><<<nb, 128>>>(w, wq, (unsigned *)wsc, Co, Ci, nmt_all, np);
@@ -213,7 +371,19 @@ template <int CP, int MT>
 static void launch_stem_out(int out, const conv_args &a, size_t smem) {
     if (out == 8) launch_stem<CP, MT, 8>(a, smem); else if (out == 4) launch_stem<CP, MT, 4>(a, smem); else launch_stem<CP, MT, 0>(a, smem);
 }
+template <int MT, int OUT>
+static void launch_p16(const conv_args &a, size_t smem) {
+    const unsigned per = (a.ntiles + 7u) / 8u;
+    conv3_p16_k<MT, OUT><<<per * 8u, 256, smem>>>(a);
+    MICK();
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_p16_k<MT %d, out %d> tiles %u", MT, OUT, a.ntiles);
+}
 void conv3_stem_launch(int CP, int MT, int out, const conv_args &a, size_t smem) {
+    if (CP == 0) {
+        if (MT == 1) { if (out == 8) launch_p16<1, 8>(a, smem); else if (out == 4) launch_p16<1, 4>(a, smem); else launch_p16<1, 0>(a, smem); }
+        else mi_die("conv3 p16: no kernel for MT %d", MT);
+        return;
+    }
     switch (CP * 10 + MT) {
     case 41: launch_stem_out<4, 1>(out, a, smem); break;
     case 42: launch_stem_out<4, 2>(out, a, smem); break;
