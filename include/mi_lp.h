@@ -48,6 +48,10 @@ void lp_wmemo_clear(void);
 /* no counterpart in the reference (its stride-2 entry carries no split_t and prepares the weights per call): memo id of the calling thread's
    next lp_conv_fwd_s2_f8, as split_t.wkey for the stride-1 entries; consumed by that call. For inference loops with constant weights. */
 void mi_conv_s2_wkey(unsigned wkey);
+/* no counterpart in the reference (its convs transform their input while staging, every time): GroupNorm + SiLU of x and re-quantisation to
+   MX-fp8 / MX-fp4 (ybits 8 / 4) once, for a tensor several convs read; they then take y with no GroupNorm. s.c a multiple of 32. In a split
+   input, gp2.G = -1 says "x2 carries no GroupNorm, gp is x's own" (gp2.G = 0 keeps the reference's meaning: gp spans both segments). */
+int mi_conv_prestage(const void *x, int xdt, shape5 s, gnp_t gp, void *y, int ybits);
 gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean, const float *rstd, int G);   /* src/nn_lp.h:19 */
 int lp_gn_slab_any(void);                                                                         /* src/nn_lp.h:20: always 0 here */
 

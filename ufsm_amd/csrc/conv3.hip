@@ -226,8 +226,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (sp.up && (!sp.x2 || xbf < 3 || ((sp.Di ? sp.Di : xs.d) & 1) || (xs.h & 1) || (xs.w & 1) || stride != 1)) mi_die("%s: the fused upsample needs an MX split input and even dims", who);
     if (osum && (Go <= 0 || cout % Go)) mi_die("%s: %d output channels in %d groups", who, cout, Go);
     if (osum && (cout / Go) % 4 && cout > 32) mi_die("%s: fused output statistics of %d channels need channels per group (%d) to be a multiple of 4", who, cout, cout / Go);
-    if (gp.G && ((sp.x2 && sp.gp2.G ? Cx : Ci) % gp.G)) mi_die("%s: GroupNorm groups %d do not divide the channels", who, gp.G);
-    if (sp.gp2.G && (!sp.x2 || C2 % sp.gp2.G)) mi_die("%s: second GroupNorm without a matching x2 segment", who);
+    if (gp.G > 0 && ((sp.x2 && sp.gp2.G ? Cx : Ci) % gp.G)) mi_die("%s: GroupNorm groups %d do not divide the channels", who, gp.G);
+    if (sp.gp2.G > 0 && (!sp.x2 || C2 % sp.gp2.G)) mi_die("%s: second GroupNorm without a matching x2 segment", who);
     // few input channels: the tap-packed kernel with one activation scale per tile (src/lp_f8fwd.cuh:601-609: up to 8 channels of a 16-bit or
     // MX input, 16 of an fp32 one; same input and output type, or an MX output)
     static int stem_env = -1;
@@ -244,10 +244,12 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const int fdt = fmt == 8 ? 3 : 4;
     conv_args a; memset(&a, 0, sizeof a);
     // ---- operands: a segment is read as stored when it already is the compute format with nothing to apply, else re-staged once ----
+    // (gp2.G < 0, an extension: x2 carries no GroupNorm and gp is x's own; the reference's gp2.G == 0 means gp spans both segments)
     const bool s2g = sp.x2 && sp.gp2.G;
+    if (sp.gp2.G < 0) sp.gp2 = gnp_mk(nullptr, nullptr, nullptr, nullptr, 0);
     const void *segx[2] = {x, sp.x2}; const int segC[2] = {Cx, C2};
     for (int s = 0; s < (sp.x2 ? 2 : 1); s++) {
-        gnp_t g = s2g ? (s ? sp.gp2 : gp) : gp;
+        const gnp_t g = s2g ? (s ? sp.gp2 : gp) : gp;
         const int Cg = s2g ? segC[s] : Ci, cg0 = s2g ? 0 : (s ? Cx : 0);
         const bool upseg = s == 0 && sp.up;
         const bool direct = xbf == fdt && !g.G && !upseg;
@@ -375,6 +377,14 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     return 0;
 }
 
+// the consumer-side transform of a conv input (GroupNorm + SiLU while staging, re-quantisation to the compute format) done once into an MX
+// tensor of the same channels, for a tensor several convs read: they then take y as a plain input and stage it as stored. Channels a
+// multiple of 32. The bits of the convs' results do not change (the same pre-pass runs inside a conv otherwise).
+extern "C" int mi_conv_prestage(const void *x, int xdt, shape5 s, gnp_t gp, void *y, int ybits) {
+    if ((ybits != 8 && ybits != 4) || s.c % 32 || xdt < 0 || xdt > 4 || (gp.G > 0 && s.c % gp.G) || gp.ns) return -1;
+    mi_restage(x, xdt, s.n, s.c, (size_t)s.d * s.h * s.w, gp, s.c, 0, y, ybits);
+    return 0;
+}
 extern "C" int lp_conv_fwd_f8(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp) {
     return conv_dispatch("lp_conv_fwd_f8", 8, 1, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, nullptr, nullptr, 0);
 }

@@ -72,7 +72,7 @@ int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn
     }
     if (stride != 1) return -1;
     split_t sp; memset(&sp, 0, sizeof sp);
-    if (x2) { sp.x2 = x2; sp.c_split = c_split; sp.up = (int16_t)up; if (gx2) sp.gp2 = gnp_mk(gx2->gamma, gx2->beta, gx2->mean, gx2->rstd, gx2->G); }
+    if (x2) { sp.x2 = x2; sp.c_split = c_split; sp.up = (int16_t)up; if (gx2) sp.gp2 = gnp_mk(gx2->gamma, gx2->beta, gx2->mean, gx2->rstd, gx2->G); }   /* (gx2->G -1: x2 without GroupNorm) */
     else if (up) return -1;
     sp.wkey = (unsigned)((uintptr_t)w >> 4) | 1u;                   /* inference: weights are prepared once per conv (keyed by the weight pointer) */
     double *sums = nullptr;

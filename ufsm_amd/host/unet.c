@@ -24,6 +24,7 @@ struct unet {
     block enc[UNET_MAXLEV], dec[UNET_MAXLEV];
     convp down[UNET_MAXLEV], head;
     void *downo[UNET_MAXLEV];
+    void *skipst[UNET_MAXLEV];         /* silu(gn(enc[i].a2)) in the compute format, formed once for its two readers (down conv, decoder conv1); null: each reader transforms it */
     gnpar dn[UNET_MAXLEV]; float *dm[UNET_MAXLEV], *dr[UNET_MAXLEV];   /* down_norm: GroupNorm after down[i], its statistics */
     size_t np; float *params;                                      /* device */
     void *xin;                                                     /* the network input built from a CT window */
@@ -91,6 +92,8 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
         }
         if (i < L - 1) {
             shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds);
+            /* both readers of the skip compute in e4m3 from MX-fp8 storage: one shared pre-stage (any other combination: the readers' formats differ) */
+            if (cfg->act_dt == 8 && cfg->prec != 3 && w[i] % 32 == 0) u->skipst[i] = act_new(u, u->enc[i].ys);
             if (cfg->down_norm) { const size_t ng = (size_t)in.n * G_of(u, w[i]); u->dm[i] = f32_new(ng); u->dr[i] = f32_new(ng); }
         }
     }
@@ -111,7 +114,7 @@ void unet_free(unet *u) {
     mi_sync();
     for (int i = 0; i < UNET_MAXLEV; i++) {
         for (int s = 0; s < 2; s++) { block *b = s ? &u->dec[i] : &u->enc[i]; act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2); }
-        act_del(u->downo[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
+        act_del(u->downo[i]); act_del(u->skipst[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
     }
     if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); }
     act_del(u->xin); mi_free(u->params);
@@ -220,7 +223,9 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
         if (block_fwd(u, &u->enc[i], i, cur, gin, nullptr, nullptr, 0, en1[i], en2[i])) { if (reg_here) nn_storage_forget(x); return -1; }
         if (i < L - 1) {                                           /* stride-2 down conv of silu(gn(a2)), width kept (src/unet.c:2970) */
             const nn_gn_t g = gn_out(u, &u->enc[i]);
-            if (nn_conv3d_fwd_x(u->enc[i].a2, &g, nullptr, nullptr, 0, 0, u->enc[i].ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
+            const int pre = u->skipst[i] != nullptr;
+            if (pre && mi_conv_prestage(u->enc[i].a2, 3, u->enc[i].ys, gnp_mk(g.gamma, g.beta, g.mean, g.rstd, g.G), u->skipst[i], 8)) return -1;
+            if (nn_conv3d_fwd_x(pre ? u->skipst[i] : u->enc[i].a2, pre ? nullptr : &g, nullptr, nullptr, 0, 0, u->enc[i].ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
             shape5 ds = u->ls[i + 1]; ds.c = u->cfg.widths[i];
             if (u->cfg.down_norm) {                                /* statistics of the stored down-conv output now, the transform in the next conv1's staging (src/unet.c:2974-2979) */
                 if (nn_gn_stats(u->downo[i], ds, G_of(u, ds.c), 1e-5f, u->dm[i], u->dr[i])) { fprintf(stderr, "unet: down_norm GroupNorm statistics unsupported for this storage\n"); return -1; }
@@ -234,7 +239,8 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
         const block *coarse = i == L - 2 ? &u->enc[L - 1] : &u->dec[i + 1];
         nn_gn_t gc = gn_out(u, coarse); const nn_gn_t gs = gn_out(u, &u->enc[i]);
         if (i == L - 2 && u->tbn) { coarse = &u->tb; gc.mean = u->tb.m2; gc.rstd = u->tb.r2; }      /* the stage's output under the level's n2 affine (src/unet.c:508) */
-        if (block_fwd(u, &u->dec[i], i, u->enc[i].a2, &gs, coarse->a2, &gc, u->cfg.widths[i + 1], dn1[i], dn2[i])) return -1;
+        static const nn_gn_t none = {nullptr, nullptr, nullptr, nullptr, -1};          /* the pre-staged skip: no GroupNorm left to apply */
+        if (block_fwd(u, &u->dec[i], i, u->skipst[i] ? u->skipst[i] : u->enc[i].a2, u->skipst[i] ? &none : &gs, coarse->a2, &gc, u->cfg.widths[i + 1], dn1[i], dn2[i])) return -1;
     }
     const block *last = L > 1 ? &u->dec[0] : &u->enc[0];
     const nn_gn_t g = gn_out(u, last);
