@@ -279,6 +279,10 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const int nmt_all = (cout + 31) / 32;
     int MT = nmt_all <= 4 ? nmt_all : nmt_all % 4 == 0 ? 4 : nmt_all % 3 == 0 ? 3 : nmt_all % 2 == 0 ? 2 : 1;
     int NT = (stride == 1 && MT <= 2 && Do >= 4) ? 4 : 2;
+    // stride 2 with few tiles (the coarse levels): one-plane tiles double the workgroups; with enough tiles the two-plane tile is faster
+    // (measured: 128 -> 128 at 32^3 -> 16^3, N 2: 32 tiles 0.072 ms, 64 tiles 0.042 ms; 32 -> 32 at 128^3: 0.090 vs 0.120 ms)
+    if (stride == 2 && (MT == 1 || MT == 2 || MT == 4) &&
+        (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 1) / 2) * (nmt_all / MT) * N < 256) NT = 1;
     // 128-channel output slices at stride 1 take the wide kernel (16 accumulators per wavefront, one workgroup per CU)
     static int big_env = -1;
     if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel
@@ -300,7 +304,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         if (fbi < a.nbt) big = false;
     }
     if (big) NT = 4;
-    const int TZ = NT == 2 ? 2 : 4;
+    const int TZ = NT == 1 ? 1 : NT == 2 ? 2 : 4;
     const int HZ = stride * (TZ - 1) + 3, HY = stride * 7 + 3, HX = stride * 15 + 3, TT = HZ * HY * HX;
     const int RB = fmt == 8 ? 32 : 16, WTILE = fmt == 8 ? 2048 : 1024;
     // LDS of a workgroup holding CB input blocks: weight ring, pair table, halo rows and scale words. Prefer the largest CB that

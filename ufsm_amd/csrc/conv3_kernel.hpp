@@ -424,7 +424,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
 // FMT: compute format (8 e4m3, 4 e2m1); OUT: 8 / 4 = MX-fp8 / MX-fp4 rows, 0 = fp32 or fp16 planes; EPI: fused affine + activation
 template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI>
 __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
-    constexpr int TZ = NT == 2 ? 2 : 4;
+    constexpr int TZ = NT == 1 ? 1 : NT == 2 ? 2 : 4;       // output planes of a workgroup's tile (x 8 x 16)
     constexpr int HZ = STRIDE * (TZ - 1) + 3, HY = STRIDE * 7 + 3, HX = STRIDE * 15 + 3, TT = HZ * HY * HX;
     constexpr int NH = fmt_t<FMT>::NH, WTILE = fmt_t<FMT>::WTILE;
     constexpr int STG = MT * (WTILE + 256);              // the weights of one pair: MT tiles of codes, then MT x 64 scale words
@@ -451,9 +451,9 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     const int ox0 = tx * 16, oy0 = ty * 8, oz0 = tz * TZ;
     const int ix0 = STRIDE * ox0 - 1, iy0 = STRIDE * oy0 - 1, iz0 = STRIDE * oz0 - 1 + a.zi0;
 
-    // the lane's voxel in each of its NT tiles: wave -> (z, y half) for TZ 2, z for TZ 4; tile j -> rows 2j, 2j+1; r -> (row, x)
+    // the lane's voxel in each of its NT tiles: wave -> y row pair for TZ 1, (z, y half) for TZ 2, z for TZ 4; tile j -> rows 2j, 2j+1; r -> (row, x)
     int lz, ly0;
-    if (NT == 2) { lz = wave >> 1; ly0 = (wave & 1) * 4; } else { lz = wave; ly0 = 0; }
+    if (NT == 1) { lz = 0; ly0 = wave * 2; } else if (NT == 2) { lz = wave >> 1; ly0 = (wave & 1) * 4; } else { lz = wave; ly0 = 0; }
     // LDS byte addresses of the lane's halo row (its 16-byte half) and scale word for tap (0, 0, 0) of block 0, first voxel tile; tile j
     // lies 2 STRIDE halo rows further: a constant the loads carry in their offset field
     const int p00 = ((STRIDE * lz) * HY + STRIDE * (ly0 + (r >> 4))) * HX + STRIDE * (r & 15);
@@ -580,6 +580,10 @@ template <int FMT, int STRIDE, int OUT, bool EPI>
 static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     switch (MT * 10 + NT) {
     case 44: if constexpr (STRIDE == 1) launch_wide<FMT, OUT, EPI>(a, smem); else mi_die("conv3: the wide kernel is stride 1 only"); break;
+    // (one-plane tiles, stride 2 only: its halo is 8 input positions per output, and a 3 x 17 x 33 halo lets two workgroups share a CU)
+    case 11: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 1, 1, OUT, EPI>(a, smem); break; }
+    case 21: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 2, 1, OUT, EPI>(a, smem); break; }
+    case 41: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 4, 1, OUT, EPI>(a, smem); break; }
     case 12: launch_conv<FMT, STRIDE, 1, 2, OUT, EPI>(a, smem); break;
     case 22: launch_conv<FMT, STRIDE, 2, 2, OUT, EPI>(a, smem); break;
     case 32: launch_conv<FMT, STRIDE, 3, 2, OUT, EPI>(a, smem); break;
