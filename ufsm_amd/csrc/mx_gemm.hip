@@ -43,7 +43,9 @@ __global__ void __launch_bounds__(256) mx_gemm_k(const uint8_t *__restrict__ Aq,
                                                  float *C, int M, int N, int nkb, float beta, const float *__restrict__ bias, const float *res, int sper) {
     constexpr int BPB = BITS == 8 ? 32 : 16, FM = BITS == 8 ? 0 : 4;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
-    const int m0 = blockIdx.y * 128 + (wave >> 1) * 64, n0 = blockIdx.x * 128 + (wave & 1) * 64;
+    // a wavefront owns a 64 x 64 tile; a workgroup is 2 x 2 of them, or a single one (few tiles: more workgroups than CUs that way)
+    const int wt = blockDim.x == 256 ? 2 : 1;
+    const int m0 = (blockIdx.y * wt + (wave >> 1)) * 64, n0 = (blockIdx.x * wt + (wave & 1)) * 64;
     if (m0 >= M || n0 >= N) return;                        // (no barriers in this kernel: a wavefront without work leaves)
     const int nst = nkb >> 1, s0 = (int)blockIdx.z * sper, s1 = min(nst, s0 + sper);
     const uint8_t *pa[2], *pb[2], *sa[2], *sb[2];
@@ -65,18 +67,24 @@ __global__ void __launch_bounds__(256) mx_gemm_k(const uint8_t *__restrict__ Aq,
         if (BITS == 8) { const v4i hi = *(const v4i *)(p + 32); return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; }
         return (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
     };
-    for (int s = s0; s < s1; s++) {
-        v8i fa[2], fb[2]; int ea[2], eb[2];
+    // the fragments of step s + 1 are requested before the MFMAs of step s (rows are read straight from global memory / L2)
+    v8i fa[2], fb[2]; int ea[2], eb[2];
+    auto load = [&](int s) {
 #pragma unroll
         for (int i = 0; i < 2; i++) {
             fa[i] = frag(pa[i] + (size_t)s * 2 * BPB); ea[i] = sa[i][2 * s];
             fb[i] = frag(pb[i] + (size_t)s * 2 * BPB); eb[i] = sb[i][2 * s];
         }
+    };
+    if (s0 < s1) load(s0);
+    for (int s = s0; s < s1; s++) {
+        v8i ca[2] = {fa[0], fa[1]}, cb[2] = {fb[0], fb[1]}; const int xa[2] = {ea[0], ea[1]}, xb[2] = {eb[0], eb[1]};
+        if (s + 1 < s1) load(s + 1);
 #pragma unroll
         for (int i = 0; i < 2; i++)
 #pragma unroll
             for (int j = 0; j < 2; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], FM, FM, 0, ea[i], 0, eb[j]);
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ca[i], cb[j], acc[i][j], FM, FM, 0, xa[i], 0, xb[j]);
     }
     // accumulator element q of lane (r, h): row (q & 3) + 4 h + 8 (q >> 2), column r of its 32 x 32 tile
     const bool split = gridDim.z > 1;
@@ -150,9 +158,10 @@ extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, cons
     const int sper = ns > 1 ? (nst + ns - 1) / ns : (nst > 0 ? nst : 1);
     ns = nst > 0 ? (nst + sper - 1) / sper : 1;
     if (ns > 1 && beta == 0.f) gemm_zero_k<<<nblk_((size_t)M * N, 256 * 4), 256>>>(C, (size_t)M * N);   // (a kernel, not a memset node: safe under graph capture)
-    const dim3 grid((unsigned)((N + 127) / 128), (unsigned)((M + 127) / 128), (unsigned)ns);
-    if (bits == 8) mx_gemm_k<8><<<grid, 256>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
-    else mx_gemm_k<4><<<grid, 256>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
+    const int wt = (size_t)tiles * ns >= 512 ? 2 : 1;              // (few tiles: one wavefront per workgroup)
+    const dim3 grid((unsigned)((N + 64 * wt - 1) / (64 * wt)), (unsigned)((M + 64 * wt - 1) / (64 * wt)), (unsigned)ns);
+    if (bits == 8) mx_gemm_k<8><<<grid, 64 * wt * wt>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
+    else mx_gemm_k<4><<<grid, 64 * wt * wt>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
     MICK();
     return 0;
 }
