@@ -97,22 +97,32 @@ __global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, 
 #pragma unroll
         for (int i = 0; i < 16; i++) oa[t][i] = 0.f;
     const int nt = (S + FT - 1) / FT;
+    // The K and V fragments of tile it + 1 are requested before tile it is worked on: with one or a few wavefronts per SIMD nothing else hides
+    // the L2 latency of a tile's loads. (The last iteration re-requests its own tile.)
+    v8i kfn[2], vfn[2]; int ksn[2], evn[2];
+    auto request = [&](int it) {
+        const int kb = it * FT;
+#pragma unroll
+        for (int b = 0; b < 2; b++) { kfn[b] = a8_frag(kp + (size_t)(kb + 32 * b) * 64); ksn[b] = ksp[(size_t)(kb + 32 * b) * 2]; }
+        vfn[0] = a8_frag(vp0 + kb); vfn[1] = a8_frag(vp1 + kb);
+        evn[0] = vs0[kb / 32]; evn[1] = vs1[kb / 32];
+    };
+    request(0);
     for (int it = 0; it < nt; it++) {
         const int kb = it * FT;
+        const v8i kf[2] = {kfn[0], kfn[1]}; const int ks[2] = {ksn[0], ksn[1]};
+        v8i vf0 = vfn[0], vf1 = vfn[1];
+        const int e0v = evn[0], e1v = evn[1];
+        request(min(it + 1, nt - 1));
         // ---- S^T = K Q^T for the tile's two blocks of 32 keys ----
         v16f s[2];
 #pragma unroll
         for (int b = 0; b < 2; b++) {
-            const v8i kf = a8_frag(kp + (size_t)(kb + 32 * b) * 64);
-            const int ks = ksp[(size_t)(kb + 32 * b) * 2];
             v16f z;
 #pragma unroll
             for (int i = 0; i < 16; i++) z[i] = 0.f;
-            s[b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf, qf, z, 0, 0, 0, ks, 0, qs);
+            s[b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[b], qf, z, 0, 0, 0, ks[b], 0, qs);
         }
-        // next: the V fragments of this tile (independent of the softmax: their latency hides behind it)
-        v8i vf0 = a8_frag(vp0 + kb), vf1 = a8_frag(vp1 + kb);
-        const int e0v = vs0[kb / 32], e1v = vs1[kb / 32];
         if (!d1ok) vf1 = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
         // ---- logits in base-2 units, keys past S masked (only the last tile can hold them) ----
         const bool full = kb + FT <= S;
