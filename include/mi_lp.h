@@ -48,6 +48,11 @@ void lp_wmemo_clear(void);
 /* no counterpart in the reference (its stride-2 entry carries no split_t and prepares the weights per call): memo id of the calling thread's
    next lp_conv_fwd_s2_f8, as split_t.wkey for the stride-1 entries; consumed by that call. For inference loops with constant weights. */
 void mi_conv_s2_wkey(unsigned wkey);
+/* Tuning knob of the tap-packed kernel for <= 4 input channels: consecutive z tiles a workgroup walks (weights and constants set up once,
+ * the next tile's input in flight during this tile's MFMAs). 0 (default) = chosen from the launch size. Results do not depend on it.
+ * Calling thread only. The reference's kernel walks up to 32 (8 for wider rows),
+ * overridden by UFSM_F8S_ZC (src/lp_f8fwd.cuh:412-416). */
+void mi_conv_stem_zc(int zc);
 /* no counterpart in the reference (its convs transform their input while staging, every time): GroupNorm + SiLU of x and re-quantisation to
    MX-fp8 / MX-fp4 (ybits 8 / 4) once, for a tensor several convs read; they then take y with no GroupNorm. s.c a multiple of 32. In a split
    input, gp2.G = -1 says "x2 carries no GroupNorm, gp is x's own" (gp2.G = 0 keeps the reference's meaning: gp spans both segments). */

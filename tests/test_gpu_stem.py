@@ -18,6 +18,15 @@ def stored(x, xdt, N, Ci, S):
     return np.ascontiguousarray(x.astype(np.float16).view(np.uint16)) if xdt == 2 else x
 
 
+@pytest.fixture(params=[0, 2], ids=["zc_auto", "zc2"], autouse=True)
+def stem_zc(request):
+    """Every case runs with the launch's own choice of z tiles per workgroup (1 at these sizes) and with 2 forced (several tiles per
+    workgroup, a ragged last group): the results may not depend on it."""
+    lib.mi_conv_stem_zc(request.param)
+    yield
+    lib.mi_conv_stem_zc(0)
+
+
 # (input type, Ci, Co, dims): the three channel paddings (4, 8, 16), one and several channel tiles and slices, ragged tiles, odd depths
 SHAPES = [(3, 4, 32, (4, 8, 16)), (3, 4, 32, (5, 11, 21)), (3, 3, 16, (3, 9, 17)), (3, 8, 48, (4, 9, 18)), (3, 6, 64, (2, 8, 33)), (3, 4, 160, (3, 8, 16)),
           (4, 4, 32, (3, 8, 16)), (4, 8, 64, (4, 12, 20)), (2, 8, 32, (4, 8, 16)), (0, 16, 32, (3, 10, 17)), (0, 11, 24, (2, 8, 16)), (0, 2, 8, (3, 5, 7))]

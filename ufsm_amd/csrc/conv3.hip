@@ -166,6 +166,7 @@ static void conv_stats_reduce(const char *who, const conv_args &a, int MT, split
 
 // the tap-packed stem (src/lp_f8fwd.cuh:601-609, :421-434): e4m3 compute, one activation scale per staged tile
 // rows: the 9 .. 16 channel form, two taps per K block and one activation scale per staged row (src/lp_f8fwd.cuh:447-563, :626)
+static thread_local int g_stem_zc = 0;      // tuning knob (mi_conv_stem_zc): z tiles per workgroup of the tap-packed kernel, 0 = chosen from the launch size
 static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                      gnp_t gp, double *osum, int Go, split_t sp, bool rows) {
     const int Ci = xs.c, N = xs.n, D = sp.Di ? sp.Di : xs.d, Do = xs.d, H = xs.h, W = xs.w;      // D: the input's depth (z-range), Do: output planes
@@ -184,6 +185,11 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
     a.ntx = (W + 15) / 16; a.nty = (H + 7) / 8; a.ntz = (Do + 1) / 2;
     a.ntiles = (unsigned)((size_t)a.ntx * a.nty * a.ntz * a.ncs * N);
+    // z tiles per workgroup (tap-packed kernel: the set-up is amortised, the next tile's loads overlap): up to 4 while >= 8 workgroups per CU remain
+    a.zc = 1;
+    if (!rows && CP <= 4 && g_stem_zc > 0) a.zc = g_stem_zc < a.ntz ? g_stem_zc : a.ntz;
+    else if (!rows && CP <= 4) { a.zc = 4; while (a.zc > 1 && (size_t)a.ntx * a.nty * ((a.ntz + a.zc - 1) / a.zc) * a.ncs * N < 2048) a.zc--; }
+    a.ngrp = (unsigned)((size_t)a.ntx * a.nty * ((a.ntz + a.zc - 1) / a.zc) * a.ncs * N);
     const size_t wq_bytes = (size_t)NP * nmt_all * 2048, wsc_bytes = (size_t)NP * nmt_all * 256;
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
@@ -398,6 +404,7 @@ extern "C" int lp_conv_fwd_f4(const void *x, int xbf, shape5 xs, const float *w,
 // prepared-weight memo id of the calling thread's next stride-2 conv (its signature carries no split_t): 0 = prepare per call
 static thread_local unsigned g_s2_wkey = 0;
 extern "C" void mi_conv_s2_wkey(unsigned wkey) { g_s2_wkey = wkey; }
+extern "C" void mi_conv_stem_zc(int zc) { g_stem_zc = zc; }
 extern "C" int lp_conv_fwd_s2_f8(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, shape5 ys, gnp_t gp) {
     const int Do = (xs.d - 1) / 2 + 1, Ho = (xs.h - 1) / 2 + 1, Wo = (xs.w - 1) / 2 + 1;
     if (ys.d != Do || ys.h != Ho || ys.w != Wo || ys.c != cout || ys.n != xs.n) mi_die("lp_conv_fwd_s2_f8: output shape %d x %d x %d x %d x %d does not match a stride-2 conv of the input", ys.n, ys.c, ys.d, ys.h, ys.w);

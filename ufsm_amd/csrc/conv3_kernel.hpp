@@ -104,6 +104,7 @@ struct conv_args {
     // tap-packed stem only: the input as stored (0 fp32 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4: one row of 8 channels per voxel) and its GroupNorm
     const void *sx; int sxdt, sCi;
     const float *sgam, *sbet, *smean, *srstd; int sG;
+    int zc; unsigned ngrp;             // consecutive z tiles a workgroup walks, workgroups with work
 };
 
 template <int FMT> struct fmt_t;

@@ -18,18 +18,23 @@ __global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
     // LDS: [staged tile TT x CP bytes][amax word, padded to 16][per channel (a, b) of the GroupNorm affine: CP x float2]
     constexpr unsigned am_o = TT * CP, ab_o = am_o + 16;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
-    unsigned tile;
+    // a workgroup walks a.zc consecutive z tiles of one (x, y) column: weights, constants and the channel table are set up once, and the next
+    // tile's input rows are in flight while this tile is multiplied and stored
+    constexpr bool ZL = CP <= 4;                             // (wider rows: the weights' fragments fill the registers, one tile per workgroup)
+    const int zc = ZL ? a.zc : 1, nzg = (a.ntz + zc - 1) / zc;
+    unsigned grp;
     {
-        const unsigned per = (a.ntiles + 7u) / 8u;          // consecutive workgroup ids go round the 8 XCDs: a contiguous tile range per XCD
-        tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
-        if (tile >= a.ntiles) return;
+        const unsigned per = (a.ngrp + 7u) / 8u;            // consecutive workgroup ids go round the 8 XCDs: a contiguous range per XCD
+        grp = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
+        if (grp >= a.ngrp) return;
     }
-    int tt = (int)tile;
+    int tt = (int)grp;
     const int cs = tt % a.ncs; tt /= a.ncs;
     const int tx = tt % a.ntx; tt /= a.ntx;
     const int ty = tt % a.nty; tt /= a.nty;
-    const int tz = tt % a.ntz; const int n = tt / a.ntz;
-    const int ox0 = tx * 16, oy0 = ty * 8, oz0 = tz * 2;
+    const int zg = tt % nzg; const int n = tt / nzg;
+    const int ox0 = tx * 16, oy0 = ty * 8;
+    const int tz0 = zg * zc, tz1 = ZL ? min(a.ntz, tz0 + zc) : tz0 + 1;
     const int Ci = a.sCi;
     const size_t S = (size_t)a.D * a.H * a.W;
 
@@ -53,114 +58,160 @@ __global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
             sa[p][m] = *(const int *)(a.wsc + (t * 64 + lane) * 4);
         }
 
-    // ---- stage: a thread owns positions tid, tid + 256, tid + 512 of the tile ----
-    float v[3][CP];
-    float amax = 0.f;
+    // ---- a thread owns positions tid, tid + 256, tid + 512 of a tile; their (y, x) part is the same for every z tile ----
     const int xdt = a.sxdt;
-    __syncthreads();                                         // the affine table
+    int piz[3]; size_t pyx[3]; bool pin[3];
 #pragma unroll
     for (int j = 0; j < 3; j++) {
-        const int pos = tid + 256 * j, ix = pos % HX, iy = (pos / HX) % HY, iz = pos / (HY * HX);
-        const int gz = oz0 - 1 + iz + a.zi0, gy = oy0 - 1 + iy, gx = ox0 - 1 + ix;
-        const bool inb = pos < TT && (unsigned)gz < (unsigned)a.D && (unsigned)gy < (unsigned)a.H && (unsigned)gx < (unsigned)a.W;
-        const size_t off = inb ? ((size_t)gz * a.H + gy) * a.W + gx : 0;
-        float x[CP];
+        const int pos = tid + 256 * j, ix = pos % HX, iy = (pos / HX) % HY;
+        const int gy = oy0 - 1 + iy, gx = ox0 - 1 + ix;
+        piz[j] = pos / (HY * HX);
+        pin[j] = pos < TT && (unsigned)gy < (unsigned)a.H && (unsigned)gx < (unsigned)a.W;
+        pyx[j] = pin[j] ? (size_t)gy * a.W + gx : 0;
+    }
+    unsigned raw0[3], raw1[3]; unsigned rsc[3]; bool rin[3];
+    auto request = [&](int tz) __attribute__((always_inline)) {                             // the raw input of tile tz -> registers
 #pragma unroll
-        for (int k = 0; k < CP; k++) x[k] = 0.f;
-        if (xdt == 3) {                                      // one MX-fp8 row of 8 channels per voxel, then the scale plane
-            if constexpr (CP <= 8) {
+        for (int j = 0; j < 3; j++) {
+            const int gz = 2 * tz - 1 + piz[j] + a.zi0;
+            rin[j] = pin[j] && (unsigned)gz < (unsigned)a.D;
+            const size_t off = rin[j] ? (size_t)gz * a.H * a.W + pyx[j] : 0;
+            if constexpr (CP <= 8) {                         // one MX row of 8 channels per voxel (fp8: 8 bytes, fp4: 4), then the scale plane
                 const uint8_t *q = (const uint8_t *)a.sx;
-                const float s = d_mx_scale(q[(size_t)a.N * S * 8 + (size_t)n * S + off]);
-                const uint8_t *row = q + ((size_t)n * S + off) * 8;
-                d_dec4_e4m3(*(const unsigned *)row, x);
-                if constexpr (CP == 8) d_dec4_e4m3(*(const unsigned *)(row + 4), x + 4);
-#pragma unroll
-                for (int k = 0; k < CP; k++) x[k] *= s;
+                const size_t rb = xdt == 3 ? 8 : 4;
+                const uint8_t *row = q + ((size_t)n * S + off) * rb;
+                rsc[j] = q[(size_t)a.N * S * rb + (size_t)n * S + off];
+                raw0[j] = *(const unsigned *)row;
+                if constexpr (CP == 8) raw1[j] = *(const unsigned *)(row + 4);     // (fp4: the next voxel's row or the scale plane's start, unused)
             }
-        } else if (xdt == 4) {                               // one MX-fp4 row of 8 channels (4 bytes) per voxel
-            if constexpr (CP <= 8) {
-                const uint8_t *q = (const uint8_t *)a.sx;
-                const float s = d_mx_scale(q[(size_t)a.N * S * 4 + (size_t)n * S + off]);
-                float d8[8];
-                d_dec8_e2m1(*(const unsigned *)(q + ((size_t)n * S + off) * 4), d8);
-#pragma unroll
-                for (int k = 0; k < CP; k++) x[k] = d8[k] * s;
-            }
-        } else {
-#pragma unroll
-            for (int k = 0; k < CP; k++)
-                if (k < Ci) {
-                    const size_t idx = ((size_t)n * Ci + k) * S + off;
-                    x[k] = xdt == 2 ? __half2float(((const __half *)a.sx)[idx]) : ((const float *)a.sx)[idx];
-                }
         }
+    };
+    const bool planes = xdt < 3;
+    constexpr bool PFP = CP <= 4;                            // plane inputs are requested a tile ahead only where the registers allow it
+    float pv[3][PFP ? CP : 1];                               // plane inputs (fp32, or fp16 widened): the values themselves
+    auto plane_vals = [&](int tz, int j, float *dst) __attribute__((always_inline)) {       // position j's CP plane values of tile tz
+        const int gz = 2 * tz - 1 + piz[j] + a.zi0;
+        rin[j] = pin[j] && (unsigned)gz < (unsigned)a.D;
+        const size_t off = rin[j] ? (size_t)gz * a.H * a.W + pyx[j] : 0;
 #pragma unroll
         for (int k = 0; k < CP; k++) {
-            float val = x[k];
-            if (a.sG) { const float2 ab = *(const float2 *)(lds + ab_o + k * 8); val = d_act_ab(val, ab.x, ab.y); }
-            val = inb && k < Ci ? val : 0.f;
-            v[j][k] = val; amax = fmaxf(amax, fabsf(val));
+            float f = 0.f;
+            if (k < Ci) { const size_t idx = ((size_t)n * Ci + k) * S + off; f = xdt == 2 ? __half2float(((const __half *)a.sx)[idx]) : ((const float *)a.sx)[idx]; }
+            dst[k] = f;
         }
-    }
-    amax = fmaxf(amax, lane_xorf<1>(amax)); amax = fmaxf(amax, lane_xorf<2>(amax)); amax = fmaxf(amax, lane_xorf<4>(amax));
-    amax = fmaxf(amax, lane_xorf<8>(amax)); amax = fmaxf(amax, lane_xorf<16>(amax)); amax = fmaxf(amax, lane_xor32f(amax, h));
-    if (lane == 0) atomicMax((unsigned *)(lds + am_o), __float_as_uint(amax));        // non-negative floats order as their bit patterns
-    __syncthreads();
-    const int e = d_mx_exp(__uint_as_float(*(const unsigned *)(lds + am_o)), MI_INVQ8);
-    const int sb = e + 127;
+    };
+    auto request_any = [&](int tz) __attribute__((always_inline)) {
+        if (planes) {
+            if constexpr (PFP) {
 #pragma unroll
-    for (int j = 0; j < 3; j++) {
-        const int pos = tid + 256 * j;
-        if (pos < TT) {
-#pragma unroll
-            for (int k = 0; k < CP / 4; k++)
-                *(unsigned *)(lds + pos * CP + 4 * k) = d_enc4_e4m3(v[j][4 * k], v[j][4 * k + 1], v[j][4 * k + 2], v[j][4 * k + 3], e);
-        }
-    }
-    __syncthreads();
-
-    // ---- MFMAs: wavefront -> (z, y half), voxel tile j -> rows 2 j, 2 j + 1 of that half, r -> (row, x) ----
+                for (int j = 0; j < 3; j++) plane_vals(tz, j, pv[j]);
+            }
+        } else request(tz);
+    };
+    request_any(tz0);
     const int lz = wave >> 1, ly0 = (wave & 1) * 4;
     const int p00 = (lz * HY + ly0 + (r >> 4)) * HX + (r & 15);
-    v16f acc[MT][NT];
+    __syncthreads();                                         // the affine table, the cleared amax word
+
+    for (int tz = tz0; tz < tz1; tz++) {
+        // ---- values of this tile: decode, GroupNorm + SiLU, amax ----
+        float v[3][CP];
+        float amax = 0.f;
 #pragma unroll
-    for (int m = 0; m < MT; m++)
+        for (int j = 0; j < 3; j++) {
+            float x[CP];
 #pragma unroll
-        for (int j = 0; j < NT; j++)
+            for (int k = 0; k < CP; k++) x[k] = 0.f;
+            if (planes) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
-    auto tapoff = [](int tap) { tap = tap > 26 ? 26 : tap; return ((tap / 9) * HY + (tap / 3) % 3) * HX + tap % 3; };     // (taps past 26: zero weights)
-    static_for<NP>([&](auto P) {
-        constexpr int p = P;
-        constexpr int LT = 16 / CP;                          // taps a lane supplies per K block
-        int off[2][LT];
+                for (int k = 0; k < CP; k++) { if constexpr (PFP) x[k] = pv[j][k]; }
+                if constexpr (!PFP) plane_vals(tz, j, x);
+            } else if (xdt == 3) {
+                if constexpr (CP <= 8) {
+                    const float sc = d_mx_scale(rsc[j]);
+                    d_dec4_e4m3(raw0[j], x);
+                    if constexpr (CP == 8) d_dec4_e4m3(raw1[j], x + 4);
 #pragma unroll
-        for (int s = 0; s < 2; s++)
+                    for (int k = 0; k < CP; k++) x[k] *= sc;
+                }
+            } else {
+                if constexpr (CP <= 8) {
+                    const float sc = d_mx_scale(rsc[j]);
+                    float d8[8];
+                    d_dec8_e2m1(raw0[j], d8);
 #pragma unroll
-            for (int i = 0; i < LT; i++) off[s][i] = h ? tapoff((2 * p + s) * TPK + LT + i) : tapoff((2 * p + s) * TPK + i);
-#pragma unroll
-        for (int j = 0; j < NT; j++) {
-            const int pj = p00 + 2 * j * HX;
-            v8i fb;
-#pragma unroll
-            for (int s = 0; s < 2; s++) {
-                if constexpr (CP == 4) {
-#pragma unroll
-                    for (int i = 0; i < 4; i++) fb[4 * s + i] = *(const int *)(lds + (pj + off[s][i]) * 4);
-                } else if constexpr (CP == 8) {
-#pragma unroll
-                    for (int i = 0; i < 2; i++) { const int2 w2 = *(const int2 *)(lds + (pj + off[s][i]) * 8); fb[4 * s + 2 * i] = w2.x; fb[4 * s + 2 * i + 1] = w2.y; }
-                } else {
-                    const v4i w4 = *(const v4i *)(lds + (pj + off[s][0]) * 16);
-                    fb[4 * s] = w4[0]; fb[4 * s + 1] = w4[1]; fb[4 * s + 2] = w4[2]; fb[4 * s + 3] = w4[3];
+                    for (int k = 0; k < CP; k++) x[k] = d8[k] * sc;
                 }
             }
 #pragma unroll
-            for (int m = 0; m < MT; m++) acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[p][m], fb, acc[m][j], 0, 0, 0, sa[p][m], 0, sb);
+            for (int k = 0; k < CP; k++) {
+                float val = x[k];
+                if (a.sG) { const float2 ab = *(const float2 *)(lds + ab_o + k * 8); val = d_act_ab(val, ab.x, ab.y); }
+                val = rin[j] && k < Ci ? val : 0.f;
+                v[j][k] = val; amax = fmaxf(amax, fabsf(val));
+            }
         }
-    });
-    __syncthreads();                                         // the staged tile is dead: the epilogue's scratch may overlay nothing of it, but keep the order
-    conv_epilogue<MT, NT, OUT, false>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
+        amax = fmaxf(amax, lane_xorf<1>(amax)); amax = fmaxf(amax, lane_xorf<2>(amax)); amax = fmaxf(amax, lane_xorf<4>(amax));
+        amax = fmaxf(amax, lane_xorf<8>(amax)); amax = fmaxf(amax, lane_xorf<16>(amax)); amax = fmaxf(amax, lane_xor32f(amax, h));
+        if (lane == 0) atomicMax((unsigned *)(lds + am_o), __float_as_uint(amax));        // non-negative floats order as their bit patterns
+        __syncthreads();
+        const int e = d_mx_exp(__uint_as_float(*(const unsigned *)(lds + am_o)), MI_INVQ8);
+        const int sb = e + 127;
+#pragma unroll
+        for (int j = 0; j < 3; j++) {
+            const int pos = tid + 256 * j;
+            if (pos < TT) {
+#pragma unroll
+                for (int k = 0; k < CP / 4; k++)
+                    *(unsigned *)(lds + pos * CP + 4 * k) = d_enc4_e4m3(v[j][4 * k], v[j][4 * k + 1], v[j][4 * k + 2], v[j][4 * k + 3], e);
+            }
+        }
+        __syncthreads();
+        if (tid == 0) *(unsigned *)(lds + am_o) = 0u;        // (everyone has read it; the next tile's maxima come after this tile's last barrier)
+        if (tz + 1 < tz1) request_any(tz + 1);       // the next tile's rows travel during this tile's MFMAs and epilogue
+
+        // ---- MFMAs: wavefront -> (z, y half), voxel tile j -> rows 2 j, 2 j + 1 of that half, r -> (row, x) ----
+        v16f acc[MT][NT];
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
+        auto tapoff = [](int tap) { tap = tap > 26 ? 26 : tap; return ((tap / 9) * HY + (tap / 3) % 3) * HX + tap % 3; };     // (taps past 26: zero weights)
+        static_for<NP>([&](auto P) {
+            constexpr int p = P;
+            constexpr int LT = 16 / CP;                      // taps a lane supplies per K block
+            int off[2][LT];
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int i = 0; i < LT; i++) off[s][i] = h ? tapoff((2 * p + s) * TPK + LT + i) : tapoff((2 * p + s) * TPK + i);
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                const int pj = p00 + 2 * j * HX;
+                v8i fb;
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+                    if constexpr (CP == 4) {
+#pragma unroll
+                        for (int i = 0; i < 4; i++) fb[4 * s + i] = *(const int *)(lds + (pj + off[s][i]) * 4);
+                    } else if constexpr (CP == 8) {
+#pragma unroll
+                        for (int i = 0; i < 2; i++) { const int2 w2 = *(const int2 *)(lds + (pj + off[s][i]) * 8); fb[4 * s + 2 * i] = w2.x; fb[4 * s + 2 * i + 1] = w2.y; }
+                    } else {
+                        const v4i w4 = *(const v4i *)(lds + (pj + off[s][0]) * 16);
+                        fb[4 * s] = w4[0]; fb[4 * s + 1] = w4[1]; fb[4 * s + 2] = w4[2]; fb[4 * s + 3] = w4[3];
+                    }
+                }
+#pragma unroll
+                for (int m = 0; m < MT; m++) acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[p][m], fb, acc[m][j], 0, 0, 0, sa[p][m], 0, sb);
+            }
+        });
+        __syncthreads();                                     // the staged tile has been read: the next tile may overwrite it, the epilogue use its scratch
+        const unsigned tile = (unsigned)(((((size_t)n * a.ntz + tz) * a.nty + ty) * a.ntx + tx) * a.ncs + cs);       // the tile's place among the statistics partials
+        conv_epilogue<MT, NT, OUT, false>(a, acc, lds, tile, n, cs, 2 * tz, oy0, ox0, lz, ly0, tid);       // (its statistics scratch is next written two barriers on)
+    }
 }
 
 // ---- 9 .. 16 input channels (src/lp_f8fwd.cuh:447-563, weights src/lp_f8fwd.cu:72-92): the channels sit in slots of 16 and a tap row
@@ -362,7 +413,7 @@ void conv3_stem_prep(int CP, const float *w, uint8_t *wq, uint8_t *wsc, int Co, 
 
 template <int CP, int MT, int OUT>
 static void launch_stem(const conv_args &a, size_t smem) {
-    const unsigned per = (a.ntiles + 7u) / 8u;
+    const unsigned per = (a.ngrp + 7u) / 8u;
     conv3_stem_k<CP, MT, OUT><<<per * 8u, 256, smem>>>(a);
     MICK();
     snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_stem_k<CP %d, MT %d, out %d> tiles %u", CP, MT, OUT, a.ntiles);
