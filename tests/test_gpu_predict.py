@@ -91,7 +91,7 @@ def test_predict_volume_equals_windows_run_one_by_one(gpu):
     vol = np.clip(60 + 0.8 * z + 0.5 * y + 40 * np.sin(0.3 * x + 0.2 * y) * np.cos(0.15 * z) + rng.integers(0, 16, dims), 0, 255).astype(np.uint8)
     vol[:S, :S, S:] = 0                                                     # window (0, 0, 1) is air: skipped
     net = UNet(make_cfg(4, [16, 32], G=8, head_out=1, act_dt=8), 1, W, W, W, seed=5)
-    p = net.params(); p[-1] = 0.0; net.set_params(p)                      # head bias 0: probabilities spread around 1/2
+    p = net.params(); p[-1] = 0.0; net.set_params(p)                      # head bias 0: probabilities centred on 0.5
     dv = DevBuf.from_numpy(vol); dout = DevBuf(vol.size); dplain = DevBuf(vol.size)
     mean, isd, axis, cy, cx = 100.0, 1 / 50.0, 1, 40.0, -20.0
     rc, nw, ndone = net.predict_volume(dv.ptr, dims, halo, B, mean, isd, axis, cy, cx, dout.ptr)

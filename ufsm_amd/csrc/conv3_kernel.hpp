@@ -105,6 +105,7 @@ struct conv_args {
     const void *sx; int sxdt, sCi;
     const float *sgam, *sbet, *smean, *srstd; int sG;
     int zc; unsigned ngrp;             // consecutive z tiles a workgroup walks, workgroups with work
+    bool areg;                         // general kernel: the weights' fragments stay in registers (one channel tile, one input block)
 };
 
 template <int FMT> struct fmt_t;
@@ -423,7 +424,9 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
 }
 
 // FMT: compute format (8 e4m3, 4 e2m1); OUT: 8 / 4 = MX-fp8 / MX-fp4 rows, 0 = fp32 or fp16 planes; EPI: fused affine + activation
-template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI>
+// AREG (one channel tile, one input block: <= 32 channels in and out): the 14 pairs of weight fragments live in registers, the K loop has no
+// weight ring, no pair table and no barriers, and the halo offsets of the taps are instruction immediates
+template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI, bool AREG = false>
 __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     constexpr int TZ = NT == 1 ? 1 : NT == 2 ? 2 : 4;       // output planes of a workgroup's tile (x 8 x 16)
     constexpr int HZ = STRIDE * (TZ - 1) + 3, HY = STRIDE * 7 + 3, HX = STRIDE * 15 + 3, TT = HZ * HY * HX;
@@ -432,8 +435,8 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     constexpr int PPS = MT == 1 ? 7 : MT == 2 ? 2 : 1;   // pairs per ring stage
     extern __shared__ __align__(16) unsigned char lds[];
     // LDS: [2 weight stages][pair table (npairs + 2) x 2 x 16 B][halo rows CB * NH * TT * 16 B][halo scales CB * TT words]
-    const int tab_bytes = (((27 * a.CB + 1) >> 1) + 2) * 32;
-    const unsigned wring_o = 0, tab_o = 2 * PPS * STG, act_o = tab_o + tab_bytes, asc_o = act_o + a.CB * NH * TT * 16;
+    const int tab_bytes = AREG ? 0 : (((27 * a.CB + 1) >> 1) + 2) * 32;
+    const unsigned wring_o = 0, tab_o = AREG ? 0 : 2 * PPS * STG, act_o = tab_o + tab_bytes, asc_o = act_o + a.CB * NH * TT * 16;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
 
     // XCD-aware tile order: consecutive workgroup ids land on different XCDs (8, round robin), so give each XCD a contiguous
@@ -474,6 +477,41 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     int pair0 = 0;                                       // global pair index of the chunk's first pair
     conv_epi_consts<MT, EPI>(a, lds, cs, tid);
 
+    if constexpr (AREG) {
+        static_assert(MT == 1, "one channel tile");
+        constexpr int NP = 14;                               // 27 taps of one block, two per MFMA; the 28th unit has zero weights
+        v8i far[NP]; int sar[NP];
+#pragma unroll
+        for (int p = 0; p < NP; p++) {                       // requested before the halo is staged: their latency hides behind it
+            const uint8_t *wp = a.wq + (size_t)p * wq_ps + (size_t)cs * WTILE + lane * 16;
+            const v4i lo = *(const v4i *)wp;
+            if (FMT == 8) { const v4i hi = *(const v4i *)(wp + 1024); far[p] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; }
+            else far[p] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+            sar[p] = *(const int *)(a.wsc + (size_t)p * wsc_ps + (size_t)cs * 256 + lane * 4);
+        }
+        if (a.wide) conv_stage_halo<FMT, STRIDE, TZ, 1, true>(a, lds, act_o, asc_o, 0, 1, n, iz0, iy0, ix0, tid);
+        else conv_stage_halo<FMT, STRIDE, TZ, 1, false>(a, lds, act_o, asc_o, 0, 1, n, iz0, iy0, ix0, tid);
+        __syncthreads();
+        static_for<NP>([&](auto P) {
+            constexpr int p = P, tA = 2 * p, tB = 2 * p + 1 < 27 ? 2 * p + 1 : 2 * p;
+            constexpr int pA = ((tA / 9) * HY + (tA / 3) % 3) * HX + tA % 3, pB = ((tB / 9) * HY + (tB / 3) % 3) * HX + tB % 3;
+            // fp8: both units' rows (the lane's half plane); fp4: the half's own unit. The scale word is the half's own unit's
+            const unsigned ao = ab0 + (NH == 2 ? pA : (h ? pB : pA)) * 16, so = sb0 + (h ? pB : pA) * 4;
+            v8i fb[NT]; int sb[NT];
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                const v4i lo = *(const v4i *)(lds + ao + j * ABJ);
+                if (FMT == 8) {
+                    const v4i hi = *(const v4i *)(lds + ab0 + pB * 16 + j * ABJ);
+                    fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                } else fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+                sb[j] = *(const int *)(lds + so + j * SBJ);
+            }
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+                acc[0][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(far[p], fb[j], acc[0][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sar[p], 0, sb[j]);
+        });
+    } else
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) {
         const int nbc = min(a.CB, a.nbt - b0), nunits = 27 * nbc, npairs = (nunits + 1) >> 1;
         __syncthreads();                                 // the previous chunk's readers are done with the halo
@@ -566,15 +604,15 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
 }
 
 extern thread_local char g_last_kernel[128];
-template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI>
+template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI, bool AREG = false>
 static void launch_conv(const conv_args &a, size_t smem) {
     static bool attr[8];
     int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
-    if (!attr[d]) { MIRT(hipFuncSetAttribute((const void *)conv3_mx_k<FMT, STRIDE, MT, NT, OUT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); attr[d] = true; }
+    if (!attr[d]) { MIRT(hipFuncSetAttribute((const void *)conv3_mx_k<FMT, STRIDE, MT, NT, OUT, EPI, AREG>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); attr[d] = true; }
     const unsigned per = (a.ntiles + 7u) / 8u;
-    conv3_mx_k<FMT, STRIDE, MT, NT, OUT, EPI><<<per * 8u, 256, smem>>>(a);
+    conv3_mx_k<FMT, STRIDE, MT, NT, OUT, EPI, AREG><<<per * 8u, 256, smem>>>(a);
     MICK();
-    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_mx_k<fmt %d, stride %d, MT %d, NT %d, out %d, epi %d> CB %d tiles %u", FMT, STRIDE, MT, NT, OUT, (int)EPI, a.CB, a.ntiles);
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_mx_k<fmt %d, stride %d, MT %d, NT %d, out %d, epi %d%s> CB %d tiles %u", FMT, STRIDE, MT, NT, OUT, (int)EPI, AREG ? ", weights in registers" : "", a.CB, a.ntiles);
 }
 #include "conv3_wide.hpp"
 template <int FMT, int STRIDE, int OUT, bool EPI>
@@ -585,11 +623,12 @@ static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     case 11: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 1, 1, OUT, EPI>(a, smem); break; }
     case 21: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 2, 1, OUT, EPI>(a, smem); break; }
     case 41: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 4, 1, OUT, EPI>(a, smem); break; }
-    case 12: launch_conv<FMT, STRIDE, 1, 2, OUT, EPI>(a, smem); break;
+    case 12: if constexpr (STRIDE == 1) { if (a.areg) { launch_conv<FMT, 1, 1, 2, OUT, EPI, true>(a, smem); break; } }
+             launch_conv<FMT, STRIDE, 1, 2, OUT, EPI>(a, smem); break;
     case 22: launch_conv<FMT, STRIDE, 2, 2, OUT, EPI>(a, smem); break;
     case 32: launch_conv<FMT, STRIDE, 3, 2, OUT, EPI>(a, smem); break;
     case 42: launch_conv<FMT, STRIDE, 4, 2, OUT, EPI>(a, smem); break;
-    case 14: if constexpr (STRIDE == 1) { launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
+    case 14: if constexpr (STRIDE == 1) { if (a.areg) launch_conv<FMT, 1, 1, 4, OUT, EPI, true>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
     case 24: if constexpr (STRIDE == 1) { launch_conv<FMT, 1, 2, 4, OUT, EPI>(a, smem); break; }
     default: mi_die("conv3: no kernel for MT %d NT %d stride %d", MT, NT, STRIDE);
     }
