@@ -328,13 +328,13 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const int nchunks = (a.nbt + cbmax - 1) / cbmax;
     a.CB = big ? a.nbt : (a.nbt + nchunks - 1) / nchunks; // (the wide kernel has no chunks: its K loop walks block by block)
     static int areg_env = -1;
-    if (areg_env < 0) areg_env = getenv("MI_CONV_AREG") ? atoi(getenv("MI_CONV_AREG")) : 1;      // tuning knob: 0 keeps the weight ring for every shape
-    a.areg = areg_env && !big && stride == 1 && MT == 1 && a.nbt == 1 && (NT == 2 || NT == 4);
-    size_t smem = a.areg ? (size_t)TT * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
+    if (areg_env < 0) areg_env = getenv("MI_CONV_AREG") ? atoi(getenv("MI_CONV_AREG")) : 1;      // tuning knob: 0 keeps the general kernel for every shape
+    a.areg = areg_env && !big && !(osum && (cout / Go) % 4) && stride == 1 && MT == 1 && a.nbt == 1 && a.wide && (NT == 2 || NT == 4);
+    size_t smem = a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     smem = (smem + 15) & ~(size_t)15;
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);      // bias, affine a, b of the workgroup's channels
     a.red_o = (unsigned)smem; smem += 1024;                                     // statistics scratch
-    if (big) {
+    if (big || a.areg) {
         // rows and scale bytes of positions outside the volume: 64 zero bytes, then 64 bytes of value 1; one page per device, kept for the process
         static uint8_t *zpage[8];
         int dv = 0; MIRT(hipGetDevice(&dv)); dv &= 7;

@@ -105,7 +105,7 @@ struct conv_args {
     const void *sx; int sxdt, sCi;
     const float *sgam, *sbet, *smean, *srstd; int sG;
     int zc; unsigned ngrp;             // consecutive z tiles a workgroup walks, workgroups with work
-    bool areg;                         // general kernel: the weights' fragments stay in registers (one channel tile, one input block)
+    bool areg;                         // the persistent small-channel kernel (one channel tile, one input block, weights in registers) takes the launch
 };
 
 template <int FMT> struct fmt_t;
@@ -235,7 +235,8 @@ __device__ __forceinline__ void conv_epi_consts(const conv_args &a, unsigned cha
 // lane (r, h) of tile j holds voxel (oz0 + lz, oy0 + ly0 + 2 j + (r >> 4), ox0 + (r & 15)) ----
 // FULL: the tile lies inside the output and the statistics cover all of its planes (uniform, checked by the caller): no per-lane predicates,
 // so the whole epilogue is straight-line code the scheduler can interleave across the accumulator tiles
-template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false>
+// NOCH: the caller never takes per-channel statistics records (stat_ch): their 32 sums are not kept
+template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false, bool NOCH = false>
 __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT][NT], unsigned char *lds, unsigned tile, int n, int cs,
                                               int oz0, int oy0, int ox0, int lz, int ly0, int tid) {
     const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
@@ -249,9 +250,10 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
     for (int m = 0; m < MT; m++)
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) { qs[m][q4] = 0.f; qss[m][q4] = 0.f; }
-    float chs[MT == 1 ? 16 : 1], chss[MT == 1 ? 16 : 1];     // per-channel sums (MT 1, stat_ch)
+    constexpr bool CH = MT == 1 && !NOCH;
+    float chs[CH ? 16 : 1], chss[CH ? 16 : 1];               // per-channel sums (MT 1, stat_ch)
 #pragma unroll
-    for (int i = 0; i < (MT == 1 ? 16 : 1); i++) { chs[i] = 0.f; chss[i] = 0.f; }
+    for (int i = 0; i < (CH ? 16 : 1); i++) { chs[i] = 0.f; chss[i] = 0.f; }
     constexpr int YB = OUT == 4 ? 4 : 8;
     const int bwo = W32 ? 32 : mx_bw(a.Co), nbo = W32 ? (a.Co + 31) >> 5 : mx_nb(a.Co), rbo = mx_rb(bwo, YB);     // W32: more than 16 output channels, known at compile time
     uint8_t *yq = (uint8_t *)a.y, *ysc = yq + (size_t)a.N * nbo * So * rbo;
@@ -286,7 +288,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                 float t = av + bias[i];                       // (padding channels: zero weights and no bias, so they stay 0)
                 if (EPI) {
                     t = fmaf(t, ea[i], eb[i]);
-                    t = a.act == 1 ? __fdividef(t, 1.f + __expf(-t)) : a.act == 2 ? gelu_erf(t) : a.act == 3 ? fmaxf(t, 0.f) : t;
+                    t = a.act == 1 ? d_silu(t) : a.act == 2 ? gelu_erf(t) : a.act == 3 ? fmaxf(t, 0.f) : t;
                     if (co_base + m * 32 + (i & 3) + 4 * h + 8 * (i >> 2) >= a.Co) t = 0.f;
                 }
                 v[i] = t; am = fmaxf(am, fabsf(t));
@@ -365,9 +367,9 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                 }
             }
             if (stats && zst) {
-                if (MT == 1 && a.stat_ch) {
+                if (CH && a.stat_ch) {
 #pragma unroll
-                    for (int i = 0; i < 16; i++) { chs[i] += v[i]; chss[i] += v[i] * v[i]; }
+                    for (int i = 0; i < (CH ? 16 : 1); i++) { chs[i] += v[i]; chss[i] += v[i] * v[i]; }
                 } else {
 #pragma unroll
                     for (int i = 0; i < 16; i++) { qs[m][i >> 2] += v[i]; qss[m][i >> 2] += v[i] * v[i]; }
@@ -379,12 +381,12 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
     DBG_MARK(20);
     if (stats) __syncthreads();
     DBG_MARK(21);
-    if (MT == 1 && stats && a.stat_ch) {
+    if (CH && stats && a.stat_ch) {
         // any group size (one channel tile): per-channel sums over the 32 voxel lanes, then over the waves; channel of register i of
         // half h = (i & 3) + 4 h + 8 (i >> 2); value index 2 i + t (t 0 sum, 1 sum of squares)
         float v[32];
 #pragma unroll
-        for (int i = 0; i < 16; i++) { v[2 * i] = chs[i]; v[2 * i + 1] = chss[i]; }
+        for (int i = 0; i < (CH ? 16 : 1); i++) { v[2 * i] = chs[i]; v[2 * i + 1] = chss[i]; }
         const int idx = wave_half_reduce<32>(v, r), i = idx >> 1;
         red[(wave * 32 + (i & 3) + 4 * h + 8 * (i >> 2)) * 2 + (idx & 1)] = v[0];
         __syncthreads();
@@ -424,9 +426,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
 }
 
 // FMT: compute format (8 e4m3, 4 e2m1); OUT: 8 / 4 = MX-fp8 / MX-fp4 rows, 0 = fp32 or fp16 planes; EPI: fused affine + activation
-// AREG (one channel tile, one input block: <= 32 channels in and out): the 14 pairs of weight fragments live in registers, the K loop has no
-// weight ring, no pair table and no barriers, and the halo offsets of the taps are instruction immediates
-template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI, bool AREG = false>
+template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI>
 __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     constexpr int TZ = NT == 1 ? 1 : NT == 2 ? 2 : 4;       // output planes of a workgroup's tile (x 8 x 16)
     constexpr int HZ = STRIDE * (TZ - 1) + 3, HY = STRIDE * 7 + 3, HX = STRIDE * 15 + 3, TT = HZ * HY * HX;
@@ -435,8 +435,8 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     constexpr int PPS = MT == 1 ? 7 : MT == 2 ? 2 : 1;   // pairs per ring stage
     extern __shared__ __align__(16) unsigned char lds[];
     // LDS: [2 weight stages][pair table (npairs + 2) x 2 x 16 B][halo rows CB * NH * TT * 16 B][halo scales CB * TT words]
-    const int tab_bytes = AREG ? 0 : (((27 * a.CB + 1) >> 1) + 2) * 32;
-    const unsigned wring_o = 0, tab_o = AREG ? 0 : 2 * PPS * STG, act_o = tab_o + tab_bytes, asc_o = act_o + a.CB * NH * TT * 16;
+    const int tab_bytes = (((27 * a.CB + 1) >> 1) + 2) * 32;
+    const unsigned wring_o = 0, tab_o = 2 * PPS * STG, act_o = tab_o + tab_bytes, asc_o = act_o + a.CB * NH * TT * 16;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
 
     // XCD-aware tile order: consecutive workgroup ids land on different XCDs (8, round robin), so give each XCD a contiguous
@@ -477,41 +477,6 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     int pair0 = 0;                                       // global pair index of the chunk's first pair
     conv_epi_consts<MT, EPI>(a, lds, cs, tid);
 
-    if constexpr (AREG) {
-        static_assert(MT == 1, "one channel tile");
-        constexpr int NP = 14;                               // 27 taps of one block, two per MFMA; the 28th unit has zero weights
-        v8i far[NP]; int sar[NP];
-#pragma unroll
-        for (int p = 0; p < NP; p++) {                       // requested before the halo is staged: their latency hides behind it
-            const uint8_t *wp = a.wq + (size_t)p * wq_ps + (size_t)cs * WTILE + lane * 16;
-            const v4i lo = *(const v4i *)wp;
-            if (FMT == 8) { const v4i hi = *(const v4i *)(wp + 1024); far[p] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; }
-            else far[p] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-            sar[p] = *(const int *)(a.wsc + (size_t)p * wsc_ps + (size_t)cs * 256 + lane * 4);
-        }
-        if (a.wide) conv_stage_halo<FMT, STRIDE, TZ, 1, true>(a, lds, act_o, asc_o, 0, 1, n, iz0, iy0, ix0, tid);
-        else conv_stage_halo<FMT, STRIDE, TZ, 1, false>(a, lds, act_o, asc_o, 0, 1, n, iz0, iy0, ix0, tid);
-        __syncthreads();
-        static_for<NP>([&](auto P) {
-            constexpr int p = P, tA = 2 * p, tB = 2 * p + 1 < 27 ? 2 * p + 1 : 2 * p;
-            constexpr int pA = ((tA / 9) * HY + (tA / 3) % 3) * HX + tA % 3, pB = ((tB / 9) * HY + (tB / 3) % 3) * HX + tB % 3;
-            // fp8: both units' rows (the lane's half plane); fp4: the half's own unit. The scale word is the half's own unit's
-            const unsigned ao = ab0 + (NH == 2 ? pA : (h ? pB : pA)) * 16, so = sb0 + (h ? pB : pA) * 4;
-            v8i fb[NT]; int sb[NT];
-#pragma unroll
-            for (int j = 0; j < NT; j++) {
-                const v4i lo = *(const v4i *)(lds + ao + j * ABJ);
-                if (FMT == 8) {
-                    const v4i hi = *(const v4i *)(lds + ab0 + pB * 16 + j * ABJ);
-                    fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                } else fb[j] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
-                sb[j] = *(const int *)(lds + so + j * SBJ);
-            }
-#pragma unroll
-            for (int j = 0; j < NT; j++)
-                acc[0][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(far[p], fb[j], acc[0][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, sar[p], 0, sb[j]);
-        });
-    } else
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) {
         const int nbc = min(a.CB, a.nbt - b0), nunits = 27 * nbc, npairs = (nunits + 1) >> 1;
         __syncthreads();                                 // the previous chunk's readers are done with the halo
@@ -604,17 +569,18 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
 }
 
 extern thread_local char g_last_kernel[128];
-template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI, bool AREG = false>
+template <int FMT, int STRIDE, int MT, int NT, int OUT, bool EPI>
 static void launch_conv(const conv_args &a, size_t smem) {
     static bool attr[8];
     int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
-    if (!attr[d]) { MIRT(hipFuncSetAttribute((const void *)conv3_mx_k<FMT, STRIDE, MT, NT, OUT, EPI, AREG>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); attr[d] = true; }
+    if (!attr[d]) { MIRT(hipFuncSetAttribute((const void *)conv3_mx_k<FMT, STRIDE, MT, NT, OUT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024)); attr[d] = true; }
     const unsigned per = (a.ntiles + 7u) / 8u;
-    conv3_mx_k<FMT, STRIDE, MT, NT, OUT, EPI, AREG><<<per * 8u, 256, smem>>>(a);
+    conv3_mx_k<FMT, STRIDE, MT, NT, OUT, EPI><<<per * 8u, 256, smem>>>(a);
     MICK();
-    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_mx_k<fmt %d, stride %d, MT %d, NT %d, out %d, epi %d%s> CB %d tiles %u", FMT, STRIDE, MT, NT, OUT, (int)EPI, AREG ? ", weights in registers" : "", a.CB, a.ntiles);
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_mx_k<fmt %d, stride %d, MT %d, NT %d, out %d, epi %d> CB %d tiles %u", FMT, STRIDE, MT, NT, OUT, (int)EPI, a.CB, a.ntiles);
 }
 #include "conv3_wide.hpp"
+#include "conv3_small.hpp"
 template <int FMT, int STRIDE, int OUT, bool EPI>
 static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     switch (MT * 10 + NT) {
@@ -623,12 +589,12 @@ static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     case 11: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 1, 1, OUT, EPI>(a, smem); break; }
     case 21: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 2, 1, OUT, EPI>(a, smem); break; }
     case 41: if constexpr (STRIDE == 2) { launch_conv<FMT, 2, 4, 1, OUT, EPI>(a, smem); break; }
-    case 12: if constexpr (STRIDE == 1) { if (a.areg) { launch_conv<FMT, 1, 1, 2, OUT, EPI, true>(a, smem); break; } }
+    case 12: if constexpr (STRIDE == 1) { if (a.areg) { launch_small<FMT, 2, OUT, EPI>(a, smem); break; } }
              launch_conv<FMT, STRIDE, 1, 2, OUT, EPI>(a, smem); break;
     case 22: launch_conv<FMT, STRIDE, 2, 2, OUT, EPI>(a, smem); break;
     case 32: launch_conv<FMT, STRIDE, 3, 2, OUT, EPI>(a, smem); break;
     case 42: launch_conv<FMT, STRIDE, 4, 2, OUT, EPI>(a, smem); break;
-    case 14: if constexpr (STRIDE == 1) { if (a.areg) launch_conv<FMT, 1, 1, 4, OUT, EPI, true>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
+    case 14: if constexpr (STRIDE == 1) { if (a.areg) launch_small<FMT, 4, OUT, EPI>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
     case 24: if constexpr (STRIDE == 1) { launch_conv<FMT, 1, 2, 4, OUT, EPI>(a, smem); break; }
     default: mi_die("conv3: no kernel for MT %d NT %d stride %d", MT, NT, STRIDE);
     }

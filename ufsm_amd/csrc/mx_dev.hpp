@@ -204,9 +204,13 @@ __device__ __forceinline__ void d_store_row_words(uint8_t *p, int bw, const unsi
     else *(unsigned *)p = w[0];
 }
 // GN + SiLU of the conv staging (src/lp_common.cuh:474-482): u = fma(x, a, b), then u * sigmoid(u) (= h + h tanh(h), h = u / 2)
+// silu(u) = u / (1 + exp(-u)) by the hardware exponential and reciprocal (v_exp_f32, v_rcp_f32: about 2 ulp in all; a true division
+// would be eleven more instructions per element, and every kernel that applies it is bound by its instruction count). u -> -inf: the
+// exponential overflows to inf, its reciprocal is 0 and the product -0
+__device__ __forceinline__ float d_silu(float u) { return u * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(u * -1.44269504f)); }
 __device__ __forceinline__ float d_act_ab(float v, float a, float b) {
     const float u = fmaf(v, a, b);
-    return __fdividef(u, 1.f + __expf(-u));     // u -> -inf: exp overflows to inf and the quotient is -0
+    return d_silu(u);
 }
 
 // exact fixed-point GroupNorm sum slot add (src/gnacc.cuh:12-20): slot = [fraction, 2^-64 units][integer part][non-finite count];

@@ -133,7 +133,7 @@ __global__ void __launch_bounds__(256) gn_silu_apply_mx_k(const void *xv, uint8_
 #pragma unroll
     for (int k = 0; k < 32; k++) {
         const int c = blk * bw + k;
-        if (k < bw && c < C) { const int ng = n * G + c / cpg; const float u = fmaf((r[k] - mean[ng]) * rstd[ng], gamma[c], beta[c]); r[k] = __fdividef(u, 1.f + __expf(-u)); }
+        if (k < bw && c < C) { const int ng = n * G + c / cpg; const float u = fmaf((r[k] - mean[ng]) * rstd[ng], gamma[c], beta[c]); r[k] = d_silu(u); }
         else r[k] = 0.f;
     }
     store_row<BY, true>(y, mx_scp<BY>(y, N, C, S), i, bw, r);
@@ -165,7 +165,7 @@ __global__ void __launch_bounds__(256) gn_silu_apply32_k(const uint8_t *x, uint8
     for (int k = 0; k < 16; k++) {
         const float4 q = co[hf * 16 + k];
         const float u = fmaf((r[k] * sc - q.x) * q.y, q.z, q.w);
-        r[k] = __fdividef(u, 1.f + __expf(-u));
+        r[k] = d_silu(u);
         am = d_amax_u(am, r[k]);
     }
     const unsigned ao = (unsigned)__shfl_xor((int)am, 1);
@@ -460,6 +460,7 @@ __global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int
 // the same for an MX source with 32-wide blocks, two lanes per row: each lane moves one 16-channel half (16 or 8 contiguous bytes in,
 // 16 or 8 out), so a wavefront reads and writes contiguous memory; the halves' amaxes meet through one lane exchange. The (a, b)
 // coefficients of the block's 32 channels are formed once per workgroup in LDS. HBM-bound: (bits_in + bits_out) / 8 + 2/32 bytes per element.
+constexpr int RS32_R = 4;                                          // rows per thread of restage32_k
 template <int BX, int BY>
 __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, size_t Ss, size_t v0) {
     const int nb = C / 32, blk = blockIdx.y, n = blockIdx.z;
@@ -470,46 +471,60 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
         sa[threadIdx.x] = a; sb[threadIdx.x] = b;
     }
     __syncthreads();
-    const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;       // (voxel, half)
-    const size_t v = t >> 1; const int hf = (int)(t & 1);
-    if (v >= S) return;                                            // (S even or odd: the pair of lanes of a row leaves together)
+    // A workgroup moves RS32_R x 128 consecutive voxels of the block, a thread one 16-channel half of RS32_R rows 128 voxels apart: the rows are
+    // requested together (one memory round trip per thread instead of one per row) and the coefficients' set-up is paid once per RS32_R rows
     constexpr int IB = BX * 2, OB = BY * 2;                        // bytes of a 16-channel half row
-    const size_t row = ((size_t)n * nb + blk) * Ss + v0 + v;
+    const int hf = threadIdx.x & 1;
+    const size_t vb = blockIdx.x * (size_t)(128 * RS32_R) + (threadIdx.x >> 1);
+    const size_t row0 = ((size_t)n * nb + blk) * Ss + v0;
     const uint8_t *xs = x + (size_t)N * nb * Ss * (IB * 2);
     uint8_t *ys = y + (size_t)N * nb * Ss * (OB * 2);
-    unsigned w[4] = {0u, 0u, 0u, 0u};
-    if (BX == 8) { const uint4 q = *(const uint4 *)(x + row * 32 + hf * 16); w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w; }
-    else { const uint2 q = *(const uint2 *)(x + row * 16 + hf * 8); w[0] = q.x; w[1] = q.y; }
-    const float sc = d_mx_scale(xs[row]);
-    float r[16];
-    if (BX == 8) { d_dec4_e4m3(w[0], r); d_dec4_e4m3(w[1], r + 4); d_dec4_e4m3(w[2], r + 8); d_dec4_e4m3(w[3], r + 12); }
-    else { d_dec8_e2m1(w[0], r); d_dec8_e2m1(w[1], r + 8); }
+    unsigned w[RS32_R][4]; unsigned sby[RS32_R];
 #pragma unroll
-    for (int k = 0; k < 16; k++) {
-        const float xv = r[k] * sc;
-        r[k] = gp.G ? d_act_ab(xv, sa[hf * 16 + k], sb[hf * 16 + k]) : xv;
+    for (int i = 0; i < RS32_R; i++) {
+        const size_t v = vb + (size_t)i * 128, row = row0 + (v < S ? v : S - 1);      // (rows past the end re-read the last one and are not stored)
+        w[i][2] = 0u; w[i][3] = 0u;
+        if (BX == 8) { const uint4 q = *(const uint4 *)(x + row * 32 + hf * 16); w[i][0] = q.x; w[i][1] = q.y; w[i][2] = q.z; w[i][3] = q.w; }
+        else { const uint2 q = *(const uint2 *)(x + row * 16 + hf * 8); w[i][0] = q.x; w[i][1] = q.y; }
+        sby[i] = xs[row];
     }
-    float am = 0.f;
+    float ca[16], cb[16];
 #pragma unroll
-    for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(r[k]));
-    am = fmaxf(am, __shfl_xor(am, 1));
-    const int e = d_mx_exp(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
-    if (BY == 8) {
-        uint4 o;
-        o.x = d_enc4_e4m3(r[0], r[1], r[2], r[3], e); o.y = d_enc4_e4m3(r[4], r[5], r[6], r[7], e);
-        o.z = d_enc4_e4m3(r[8], r[9], r[10], r[11], e); o.w = d_enc4_e4m3(r[12], r[13], r[14], r[15], e);
-        *(uint4 *)(y + row * 32 + hf * 16) = o;
-    } else {
-        uint2 o; o.x = d_enc8_e2m1(r, e); o.y = d_enc8_e2m1(r + 8, e);
-        *(uint2 *)(y + row * 16 + hf * 8) = o;
+    for (int k = 0; k < 16; k++) { ca[k] = sa[hf * 16 + k]; cb[k] = sb[hf * 16 + k]; }
+#pragma unroll
+    for (int i = 0; i < RS32_R; i++) {
+        const size_t v = vb + (size_t)i * 128, row = row0 + v;
+        const float sc = d_mx_scale(sby[i]);
+        float r[16];
+        if (BX == 8) { d_dec4_e4m3(w[i][0], r); d_dec4_e4m3(w[i][1], r + 4); d_dec4_e4m3(w[i][2], r + 8); d_dec4_e4m3(w[i][3], r + 12); }
+        else { d_dec8_e2m1(w[i][0], r); d_dec8_e2m1(w[i][1], r + 8); }
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const float xv = r[k] * sc;
+            r[k] = gp.G ? d_act_ab(xv, ca[k], cb[k]) : xv;
+        }
+        float am = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(r[k]));
+        am = fmaxf(am, __shfl_xor(am, 1));
+        const int e = d_mx_exp(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
+        if (BY == 8) {
+            uint4 o;
+            o.x = d_enc4_e4m3(r[0], r[1], r[2], r[3], e); o.y = d_enc4_e4m3(r[4], r[5], r[6], r[7], e);
+            o.z = d_enc4_e4m3(r[8], r[9], r[10], r[11], e); o.w = d_enc4_e4m3(r[12], r[13], r[14], r[15], e);
+            if (v < S) *(uint4 *)(y + row * 32 + hf * 16) = o;
+        } else {
+            uint2 o; o.x = d_enc8_e2m1(r, e); o.y = d_enc8_e2m1(r + 8, e);
+            if (v < S) *(uint2 *)(y + row * 16 + hf * 8) = o;
+        }
+        if (!hf && v < S) ys[row] = (uint8_t)(e + 127);
     }
-    if (!hf) ys[row] = (uint8_t)(e + 127);
 }
 // voxels [v0, v0 + S) of tensors holding Ss voxels per (sample, channel / block): the result has the source's geometry, only that range is written
 void mi_restage_sub(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits, size_t Ss, size_t v0) {
     const size_t n = (size_t)N * ((C + 31) / 32) * S; if (!n) return;
     if (xdt >= 3 && C % 32 == 0) {
-        const dim3 grid(nblk_(2 * S, 256), (unsigned)(C / 32), (unsigned)N);
+        const dim3 grid(nblk_(S, 128 * RS32_R), (unsigned)(C / 32), (unsigned)N);
         const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
         if (xdt == 3) { if (ybits == 8) restage32_k<8, 8><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0, Ss, v0); else restage32_k<8, 4><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0, Ss, v0); }
         else { if (ybits == 8) restage32_k<4, 8><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0, Ss, v0); else restage32_k<4, 4><<<grid, 256>>>(xq, yq, N, C, S, gp, Cg, cg0, Ss, v0); }
