@@ -34,13 +34,19 @@ template <int B, bool NANPROP> __device__ __forceinline__ void store_row(uint8_t
     sc[i] = (uint8_t)sb;
 }
 
+// launch shape of the row kernels: 256 voxels per workgroup along x, (sample, block) along y
+static dim3 rows_grid(int N, int nb, size_t S) {
+    if ((size_t)N * nb > 65535) mi_die("MX row kernel: %d samples x %d blocks exceed the launch grid", N, nb);
+    return dim3(nblk_(S, 256), (unsigned)(N * nb));
+}
 // ---- fp32 / 16-bit planes [n][C][S] -> MX (src/lp_mx_cvt.cu:9-19) ----
 template <int B, typename TI>
 __global__ void __launch_bounds__(256) f32_to_mx_k(const TI *x, uint8_t *y, int N, int C, size_t S) {
     const int bw = mx_bw(C), nb = mx_nb(C);
-    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (i >= (size_t)N * nb * S) return;
-    const size_t v = i % S; const int blk = (int)((i / S) % nb), n = (int)(i / (S * nb));
+    const size_t v = blockIdx.x * (size_t)blockDim.x + threadIdx.x;       // grid: x over the voxels, y = n nb + blk (uniform: no per-thread divisions)
+    if (v >= S) return;
+    const int blk = (int)(blockIdx.y % (unsigned)nb), n = (int)(blockIdx.y / (unsigned)nb);
+    const size_t i = (size_t)blockIdx.y * S + v;
     float r[32];
 #pragma unroll
     for (int k = 0; k < 32; k++) { const int c = blk * bw + k; r[k] = k < bw && c < C ? ldx(x, ((size_t)n * C + c) * S + v) : 0.f; }
@@ -49,15 +55,15 @@ __global__ void __launch_bounds__(256) f32_to_mx_k(const TI *x, uint8_t *y, int 
 template <int B> static void f32_to_mx(const float *x, int N, int C, size_t S, void *y) {
     const size_t n = (size_t)N * mx_nb(C) * S;
     if (!n) return;
-    f32_to_mx_k<B, float><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, N, C, S); MICK();
+    f32_to_mx_k<B, float><<<rows_grid(N, mx_nb(C), S), 256>>>(x, (uint8_t *)y, N, C, S); MICK();
 }
 extern "C" void lp_f32_to_mx8(const float *x, int N, int C, size_t S, void *y) { f32_to_mx<8>(x, N, C, S, y); }
 extern "C" void lp_f32_to_mx4(const float *x, int N, int C, size_t S, void *y) { f32_to_mx<4>(x, N, C, S, y); }
 template <int B> static void h16_to_mx(const void *x, int dt, int N, int C, size_t S, void *y) {
     const size_t n = (size_t)N * mx_nb(C) * S;
     if (!n) return;
-    if (dt == 2) f32_to_mx_k<B, __half><<<nblk_(n, 256), 256>>>((const __half *)x, (uint8_t *)y, N, C, S);
-    else if (dt == 1) f32_to_mx_k<B, bf16_t><<<nblk_(n, 256), 256>>>((const bf16_t *)x, (uint8_t *)y, N, C, S);
+    if (dt == 2) f32_to_mx_k<B, __half><<<rows_grid(N, mx_nb(C), S), 256>>>((const __half *)x, (uint8_t *)y, N, C, S);
+    else if (dt == 1) f32_to_mx_k<B, bf16_t><<<rows_grid(N, mx_nb(C), S), 256>>>((const bf16_t *)x, (uint8_t *)y, N, C, S);
     else mi_die("lp_h16_to_mx%d: dtype %d is not 16-bit (1 bf16, 2 fp16)", B, dt);
     MICK();
 }
@@ -68,9 +74,10 @@ extern "C" void lp_h16_to_mx4(const void *x, int dt, int N, int C, size_t S, voi
 template <int B>
 __global__ void __launch_bounds__(256) mx_to_f32_k(const uint8_t *x, float *y, int N, int C, size_t S) {
     const int bw = mx_bw(C), nb = mx_nb(C);
-    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (i >= (size_t)N * nb * S) return;
-    const size_t v = i % S; const int blk = (int)((i / S) % nb), n = (int)(i / (S * nb));
+    const size_t v = blockIdx.x * (size_t)blockDim.x + threadIdx.x;       // grid: x over the voxels, y = n nb + blk (uniform: no per-thread divisions)
+    if (v >= S) return;
+    const int blk = (int)(blockIdx.y % (unsigned)nb), n = (int)(blockIdx.y / (unsigned)nb);
+    const size_t i = (size_t)blockIdx.y * S + v;
     float r[32];
     load_row<B>(x, mx_scp<B>(x, N, C, S), i, bw, r);
 #pragma unroll
@@ -78,11 +85,11 @@ __global__ void __launch_bounds__(256) mx_to_f32_k(const uint8_t *x, float *y, i
 }
 extern "C" void lp_mx8_to_f32(const void *x, int N, int C, size_t S, float *y) {
     const size_t n = (size_t)N * mx_nb(C) * S; if (!n) return;
-    mx_to_f32_k<8><<<nblk_(n, 256), 256>>>((const uint8_t *)x, y, N, C, S); MICK();
+    mx_to_f32_k<8><<<rows_grid(N, mx_nb(C), S), 256>>>((const uint8_t *)x, y, N, C, S); MICK();
 }
 extern "C" void lp_mx4_to_f32(const void *x, int N, int C, size_t S, float *y) {
     const size_t n = (size_t)N * mx_nb(C) * S; if (!n) return;
-    mx_to_f32_k<4><<<nblk_(n, 256), 256>>>((const uint8_t *)x, y, N, C, S); MICK();
+    mx_to_f32_k<4><<<rows_grid(N, mx_nb(C), S), 256>>>((const uint8_t *)x, y, N, C, S); MICK();
 }
 
 // ---- network input rows (src/lp_mx_cvt.cu:29-55): z-scored CT, 0, unit direction away from the axis -> one 8-wide row per voxel ----
@@ -121,9 +128,10 @@ extern "C" void lp_pred_input_mx8(const uint8_t *ct, int W, float mean, float is
 template <int BX, int BY, typename TI>
 __global__ void __launch_bounds__(256) gn_silu_apply_mx_k(const void *xv, uint8_t *y, int N, int C, int G, size_t S, const float *gamma, const float *beta, const float *mean, const float *rstd) {
     const int bw = mx_bw(C), nb = mx_nb(C), cpg = C / G;
-    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (i >= (size_t)N * nb * S) return;
-    const size_t v = i % S; const int blk = (int)((i / S) % nb), n = (int)(i / (S * nb));
+    const size_t v = blockIdx.x * (size_t)blockDim.x + threadIdx.x;       // grid: x over the voxels, y = n nb + blk (uniform: no per-thread divisions)
+    if (v >= S) return;
+    const int blk = (int)(blockIdx.y % (unsigned)nb), n = (int)(blockIdx.y / (unsigned)nb);
+    const size_t i = (size_t)blockIdx.y * S + v;
     float r[32];
     if (BX != 0) { const uint8_t *x = (const uint8_t *)xv; load_row<BX ? BX : 8>(x, mx_scp<BX ? BX : 8>(x, N, C, S), i, bw, r); }
     else {
@@ -196,7 +204,7 @@ extern "C" void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, con
         MICK();
         return;
     }
-#define GSA(BX, BY, TI) gn_silu_apply_mx_k<BX, BY, TI><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, s.n, s.c, G, S, gamma, beta, mean, rstd)
+#define GSA(BX, BY, TI) gn_silu_apply_mx_k<BX, BY, TI><<<rows_grid(s.n, mx_nb(s.c), S), 256>>>(x, (uint8_t *)y, s.n, s.c, G, S, gamma, beta, mean, rstd)
 #define GSA_Y(BX, TI) do { if (ydt == 4) GSA(BX, 4, TI); else GSA(BX, 8, TI); } while (0)
     if (xdt == 4) GSA_Y(4, float); else if (xdt == 3) GSA_Y(8, float); else if (xdt == 2) GSA_Y(0, __half); else if (xdt == 1) GSA_Y(0, bf16_t); else GSA_Y(0, float);
 #undef GSA_Y
@@ -434,9 +442,9 @@ template <int BX, int BY, typename TI>
 __global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, size_t Ss, size_t v0) {
     // voxels [v0, v0 + S) of tensors holding Ss voxels per (sample, channel / block), source and result alike; y: an MX tensor of nbo * 32 channels (bw 32). gp over Cg channels of which this tensor holds [cg0, cg0 + C) (whole-input GroupNorm of a split input)
     const int nbo = (C + 31) / 32, bwx = mx_bw(C), Cy = nbo * 32;
-    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (i >= (size_t)N * nbo * S) return;
-    const size_t v = i % S; const int blk = (int)((i / S) % nbo), n = (int)(i / (S * nbo));
+    const size_t v = blockIdx.x * (size_t)blockDim.x + threadIdx.x;       // grid: x over the voxels, y = n nbo + blk (uniform: no per-thread divisions)
+    if (v >= S) return;
+    const int blk = (int)(blockIdx.y % (unsigned)nbo), n = (int)(blockIdx.y / (unsigned)nbo);
     float r[32];
     if (BX != 0) {
         const uint8_t *x = (const uint8_t *)xv; const uint8_t *sc = mx_scp<BX ? BX : 8>(x, N, C, Ss);
@@ -531,7 +539,7 @@ void mi_restage_sub(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, in
         MICK();
         return;
     }
-#define RS(BX, BY, TI) restage_k<BX, BY, TI><<<nblk_(n, 256), 256>>>(x, (uint8_t *)y, N, C, S, gp, Cg, cg0, Ss, v0)
+#define RS(BX, BY, TI) restage_k<BX, BY, TI><<<rows_grid(N, (C + 31) / 32, S), 256>>>(x, (uint8_t *)y, N, C, S, gp, Cg, cg0, Ss, v0)
 #define RS_Y(BX, TI) do { if (ybits == 4) RS(BX, 4, TI); else RS(BX, 8, TI); } while (0)
     if (xdt == 4) RS_Y(4, float); else if (xdt == 3) RS_Y(8, float); else if (xdt == 2) RS_Y(0, __half); else if (xdt == 1) RS_Y(0, bf16_t); else RS_Y(0, float);
 #undef RS_Y
@@ -552,12 +560,13 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
     const int Dc = D >> 1, Hc = H >> 1, Wc = W >> 1;
     const size_t S = (size_t)D * H * W, Sc = (size_t)Dcs * Hc * Wc;
     const int nbk = blockIdx.y;                                                   // (n, blk)
-    const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;
-    const int q = (int)(t & 3);
-    const size_t cell = t >> 2, ncx = (size_t)Wc + 1, ncy = (size_t)Hc + 1, ncz = (size_t)ncz_;
-    const bool live = cell < ncx * ncy * ncz;
-    const size_t cc = live ? cell : 0;
-    const int mx = (int)(cc % ncx) - 1, my = (int)((cc / ncx) % ncy) - 1, mz = (int)(cc / (ncx * ncy)) + mz0;
+    // grid: x over the (my, mx) cells of one z layer of cells (four threads each), y = (n, blk), z = the layer: one 32-bit division per thread
+    const unsigned t = blockIdx.x * 256u + threadIdx.x;
+    const int q = (int)(t & 3u);
+    const unsigned cell = t >> 2, ncx = (unsigned)Wc + 1u, ncy = (unsigned)Hc + 1u;
+    const bool live = cell < ncx * ncy;
+    const unsigned cc = live ? cell : 0u, cyi = cc / ncx;
+    const int mx = (int)(cc - cyi * ncx) - 1, my = (int)cyi - 1, mz = (int)blockIdx.z + mz0;
     const int cz[2] = {max(mz, 0), min(mz + 1, Dc - 1)}, cy[2] = {max(my, 0), min(my + 1, Hc - 1)}, cx[2] = {max(mx, 0), min(mx + 1, Wc - 1)};
     const uint8_t *xs = xc + (size_t)N * nbo * Sc * 32;
     float f[8][8], sc[8];
@@ -613,8 +622,9 @@ void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W
     const size_t Scp = (size_t)(H / 2) * (W / 2);
     uint8_t *xc = (uint8_t *)mi_ws(MI_WS_UPCOARSE, (size_t)N * nbo * Dc * Scp * 33);          // the coarse tensor's geometry; planes [clo, clo + Dcs) are filled
     mi_restage_sub(x, xdt, N, C, (size_t)Dcs * Scp, gp, Cg, 0, xc, 8, (size_t)Dc * Scp, (size_t)clo * Scp);
-    const size_t cells = (size_t)ncz * (H / 2 + 1) * (W / 2 + 1);
-    const dim3 grid(nblk_(cells * 4, 256), (unsigned)(N * nbo));
+    const size_t cells = (size_t)(H / 2 + 1) * (W / 2 + 1);                                   // per z layer of cells
+    if ((size_t)N * nbo > 65535 || ncz > 65535) mi_die("fused upsample: launch grid (%d x %d blocks, %d cell layers)", N, nbo, ncz);
+    const dim3 grid(nblk_(cells * 4, 256), (unsigned)(N * nbo), (unsigned)ncz);
     if (ybits == 4) up_blend_k<4><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W, zlo, zhi, 0, Dc, mz0, ncz);
     else up_blend_k<8><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W, zlo, zhi, 0, Dc, mz0, ncz);
     MICK();
