@@ -160,6 +160,8 @@ def main():
     ap.add_argument("--no-hbm", action="store_true", help="skip the HBM-bound kernels leg")
     ap.add_argument("--copy-probe", action="store_true", help="run 5 device-to-device copies of 1 GiB and exit: the known-size kernel that scales "
                     "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--conv-probe", default="", metavar="Ci,Co,N,D,bits", help="time one 3x3x3 conv shape (MX in / out of the compute format, fused statistics) "
+                    "over --steps launches after --warmup, print one JSON line and exit: the command rocprofv3 counter runs of the other conv kernels use")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (the path would shard by whole windows, or by z-slabs of one window with a one-plane halo exchange per layer)" % a.gpus, file=sys.stderr)
@@ -177,6 +179,32 @@ def main():
             lib.mi_d2d(dst.ptr, src.ptr, nb)
         lib.mi_sync(); LP.check()
         print(json.dumps({"copy_probe_bytes": nb, "copies": 5}))
+        return
+    if a.conv_probe:
+        import ctypes as C
+        Ci, Co, N, D, bits = [int(v) for v in a.conv_probe.split(",")]
+        S = D * D * D
+        rng = np.random.default_rng(0)
+        dx = DevBuf.from_numpy(rng.standard_normal((N, Ci, S)).astype(np.float32))
+        mxb, cvt, conv, dt = (lib.lp_mx8_bytes, lib.lp_f32_to_mx8, lib.lp_conv_fwd_f8, 3) if bits == 8 else (lib.lp_mx4_bytes, lib.lp_f32_to_mx4, lib.lp_conv_fwd_f4, 4)
+        dxq = DevBuf(mxb(N, Ci, S)); cvt(dx.ptr, N, Ci, S, dxq.ptr)
+        dw = DevBuf.from_numpy((rng.standard_normal((Co, Ci, 27)) * np.sqrt(2.0 / (Ci * 27))).astype(np.float32))
+        db = DevBuf.from_numpy((rng.standard_normal(Co) * 0.1).astype(np.float32))
+        dy = DevBuf(mxb(N, Co, S)); dsum = DevBuf(N * 8 * 2 * 24)
+        sp = split_t(); sp.wkey = 7; xs = shape5(N, Ci, D, D, D)
+        for _ in range(a.warmup):
+            conv(dxq.ptr, dt, xs, dw.ptr, db.ptr, Co, dy.ptr, dt, gnp_t(), dsum.ptr, 8, sp)
+        lib.mi_kernel_timing(1)
+        for _ in range(a.steps):
+            conv(dxq.ptr, dt, xs, dw.ptr, db.ptr, Co, dy.ptr, dt, gnp_t(), dsum.ptr, 8, sp)
+        nl = C.c_long(0)
+        ms = lib.mi_kernel_timing_read(C.byref(nl)) / max(nl.value, 1)
+        lib.mi_kernel_timing(0); LP.check()
+        fl = 2.0 * 27 * Ci * Co * N * S
+        peak = 5033.0 if bits == 8 else 10066.0
+        print(json.dumps({"conv_probe": a.conv_probe, "kernel": lib.mi_last_kernel().decode(), "launches": int(nl.value), "avg_launch_ms": ms,
+                          "tflops": fl / ms / 1e9, "frac_of_mfma_peak": fl / ms / 1e9 / peak,
+                          "algorithmic_bytes": int(mxb(N, Ci, S) + mxb(N, Co, S)), "GBps": (mxb(N, Ci, S) + mxb(N, Co, S)) / ms / 1e6}))
         return
     N, Cc, D, L, G = 2, 128, 64, 4, 8
     S = D * D * D

@@ -7,9 +7,11 @@
 //   * the halo of the next tile is copied global -> LDS directly (global_load_lds, no registers) into a second buffer before the current
 //     tile's MFMAs start and has landed when they are done: a tile is MFMAs, epilogue and one barrier. Positions outside the volume read
 //     a zero row / scale byte 1 from a constant page;
-// Measured at 32 -> 32 channels, 2 x 128^3, MX-fp8 (8192 tiles): 0.151 ms; the K loop alone 0.093 ms with one or with two wavefronts per SIMD
-// (the LDS pipe: two 16-byte reads and a scale word per lane and MFMA, about 100 clocks per MFMA of 64), the epilogue alone 0.051 ms, the
-// copies 0.01 - 0.03 ms. The two workgroups of a CU drift into the same phase, so the parts add up instead of hiding each other.
+// Measured at 32 -> 32 channels, 2 x 128^3, MX-fp8 (8192 tiles): 0.151 ms; the K loop alone 0.087 - 0.093 ms with one or with two wavefronts per
+// SIMD (72 % of the matrix pipe's cycles at the 1.82 GHz the part settles at under it; 0.077 ms at 1.71 GHz with half the LDS reads), the
+// epilogue alone 0.051 ms, the copies 0.01 - 0.03 ms. The parts add up whatever the arrangement: a start offset between the CU's two
+// workgroups changes nothing, and one workgroup of two groups of four wavefronts that alternate MFMA and epilogue phases behind barriers
+// (one wavefront of a SIMD in its K loop while the other runs its epilogue) took 0.169 ms. What remains is doing less per tile.
 #pragma once
 
 template <int FMT, int NT, int OUT, bool EPI>
