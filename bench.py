@@ -181,7 +181,6 @@ def main():
         print(json.dumps({"copy_probe_bytes": nb, "copies": 5}))
         return
     if a.conv_probe:
-        import ctypes as C
         Ci, Co, N, D, bits = [int(v) for v in a.conv_probe.split(",")]
         S = D * D * D
         rng = np.random.default_rng(0)
