@@ -329,7 +329,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     a.CB = big ? a.nbt : (a.nbt + nchunks - 1) / nchunks; // (the wide kernel has no chunks: its K loop walks block by block)
     static int areg_env = -1;
     if (areg_env < 0) areg_env = getenv("MI_CONV_AREG") ? atoi(getenv("MI_CONV_AREG")) : 1;      // tuning knob: 0 keeps the general kernel for every shape
-    a.areg = areg_env && !big && !(osum && (cout / Go) % 4) && stride == 1 && MT == 1 && a.nbt == 1 && a.wide && (NT == 2 || NT == 4);
+    a.areg = areg_env && !big && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && a.nbt == 1 && a.wide && (NT == 2 || NT == 4);
     size_t smem = a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     smem = (smem + 15) & ~(size_t)15;
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);      // bias, affine a, b of the workgroup's channels

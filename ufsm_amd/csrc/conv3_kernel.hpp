@@ -309,12 +309,13 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                             for (int q4 = 0; q4 < 4; q4++) d[q4] = d_enc4_e4m3_nf(v[4 * q4], v[4 * q4 + 1], v[4 * q4 + 2], v[4 * q4 + 3]);
                         }
                     }
-                    if (a.stored_stats) {
+                    if (a.stored_stats) {                // the statistics are those of the stored values: decode the codes at the block's scale
                         const float sc = d_exp2i(e);
 #pragma unroll
-                        for (int q4 = 0; q4 < 4; q4++) d_dec4_e4m3(d[q4], v + 4 * q4);
-#pragma unroll
-                        for (int i = 0; i < 16; i++) v[i] *= sc;
+                        for (int q4 = 0; q4 < 4; q4++) {
+                            const mi_v2f lo = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(d[q4], sc, false), hi = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(d[q4], sc, true);
+                            v[4 * q4] = lo[0]; v[4 * q4 + 1] = lo[1]; v[4 * q4 + 2] = hi[0]; v[4 * q4 + 3] = hi[1];
+                        }
                     }
                     // lane h = 0 holds bytes {0-3, 8-11, 16-19, 24-27}, its partner {4-7, 12-15, 20-23, 28-31}: swap so each stores 16 contiguous bytes
                     const unsigned s0 = h ? d[0] : d[2], s1 = h ? d[1] : d[3];
@@ -565,7 +566,13 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     }
 
     __syncthreads();                                     // the ring and halo are dead: the epilogue reuses LDS for its statistics scratch
-    conv_epilogue<MT, NT, OUT, EPI>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
+    // (uniform) the tile lies inside the output and the statistics cover its planes: the epilogue without per-lane predicates; more than 16
+    // output channels (always with two or more channel tiles): 32-wide output rows known at compile time
+    const bool full = oz0 + TZ <= a.Do && oy0 + 8 <= a.Ho && ox0 + 16 <= a.Wo && a.zs0 <= oz0 && a.zs1 >= oz0 + TZ;
+    if (MT > 1 || a.Co > 16) {
+        if (full) conv_epilogue<MT, NT, OUT, EPI, false, true, true>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
+        else conv_epilogue<MT, NT, OUT, EPI, false, true, false>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
+    } else conv_epilogue<MT, NT, OUT, EPI>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
 }
 
 extern thread_local char g_last_kernel[128];

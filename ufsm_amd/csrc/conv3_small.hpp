@@ -138,8 +138,8 @@ __global__ void __launch_bounds__(256, 2) conv3_small_k(const conv_args a) {
         });
         wait_vm<0>();                                           // this wavefront's copies of the next halo have landed (before the epilogue's stores are counted)
         if (cur.oz0 + TZ <= a.Do && cur.oy0 + 8 <= a.Ho && cur.ox0 + 16 <= a.Wo && a.zs0 <= cur.oz0 && a.zs1 >= cur.oz0 + TZ)      // (uniform)
-            conv_epilogue<1, NT, OUT, EPI, false, false, true, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
-        else conv_epilogue<1, NT, OUT, EPI, false, false, false, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+            conv_epilogue<1, NT, OUT, EPI, false, true, true, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+        else conv_epilogue<1, NT, OUT, EPI, false, true, false, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
         if (!nxt.ok) break;
         __syncthreads();                                        // every wavefront's copies have landed and everyone is done reading this tile's buffer
         cur = nxt;
