@@ -566,13 +566,7 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     }
 
     __syncthreads();                                     // the ring and halo are dead: the epilogue reuses LDS for its statistics scratch
-    // (uniform) the tile lies inside the output and the statistics cover its planes: the epilogue without per-lane predicates; more than 16
-    // output channels (always with two or more channel tiles): 32-wide output rows known at compile time
-    const bool full = oz0 + TZ <= a.Do && oy0 + 8 <= a.Ho && ox0 + 16 <= a.Wo && a.zs0 <= oz0 && a.zs1 >= oz0 + TZ;
-    if (MT > 1 || a.Co > 16) {
-        if (full) conv_epilogue<MT, NT, OUT, EPI, false, true, true>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
-        else conv_epilogue<MT, NT, OUT, EPI, false, true, false>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
-    } else conv_epilogue<MT, NT, OUT, EPI>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
+    conv_epilogue<MT, NT, OUT, EPI>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
 }
 
 extern thread_local char g_last_kernel[128];

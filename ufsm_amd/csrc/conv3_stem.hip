@@ -210,7 +210,11 @@ __global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
         });
         __syncthreads();                                     // the staged tile has been read: the next tile may overwrite it, the epilogue use its scratch
         const unsigned tile = (unsigned)(((((size_t)n * a.ntz + tz) * a.nty + ty) * a.ntx + tx) * a.ncs + cs);       // the tile's place among the statistics partials
-        conv_epilogue<MT, NT, OUT, false>(a, acc, lds, tile, n, cs, 2 * tz, oy0, ox0, lz, ly0, tid);       // (its statistics scratch is next written two barriers on)
+        // (uniform) more than 16 output channels: 32-wide output rows known at compile time; the tile inside the output and the statistics' planes:
+        // no per-lane predicates. (The statistics scratch is next written two barriers on)
+        if (a.Co > 16 && 2 * tz + 2 <= a.Do && oy0 + 8 <= a.Ho && ox0 + 16 <= a.Wo && a.zs0 <= 2 * tz && a.zs1 >= 2 * tz + 2)
+            conv_epilogue<MT, NT, OUT, false, false, true, true>(a, acc, lds, tile, n, cs, 2 * tz, oy0, ox0, lz, ly0, tid);
+        else conv_epilogue<MT, NT, OUT, false>(a, acc, lds, tile, n, cs, 2 * tz, oy0, ox0, lz, ly0, tid);
     }
 }
 
