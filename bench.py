@@ -117,7 +117,7 @@ def hbm_leg(np, lib, LP, DevBuf):
     return rows
 
 
-def sliding_leg(np, lib, LP, DevBuf):
+def sliding_leg(np, lib, LP, DevBuf, nbatch=8):
     """configs[4]: a 512 x 1024 x 1024 uint8 volume resident in HBM, 128^3 windows with 16 voxels of halo (stride 96), per window a U-Net of
     widths 32/64/128/192 with MX-fp4 weights over MX-fp8 activations (prec 3) and two transformer blocks (MX-fp8 attention core, MX-fp8
     linears, 4 heads of 48, axial RoPE, 4 register tokens) on the 16^3 = 4096 bottleneck tokens, one head channel, sigmoid -> uint8
@@ -130,7 +130,7 @@ def sliding_leg(np, lib, LP, DevBuf):
     vol = (115 + 55 * np.sin(r * 0.35 + 0.02 * z)).astype(np.float32)
     vol += rng.integers(-20, 21, (1, dims[1], dims[2])).astype(np.float32) + rng.integers(-10, 11, (dims[0], 1, 1)).astype(np.float32)
     vol = np.clip(vol, 1, 255).astype(np.uint8)
-    net = UNet(make_cfg(4, [32, 64, 128, 192], G=8, head_out=1, act_dt=8, prec=3, attn_blocks=2, attn_pe=1, attn_reg=4), 1, W, W, W, seed=1)
+    net = UNet(make_cfg(4, [32, 64, 128, 192], G=8, head_out=1, act_dt=8, prec=3, attn_blocks=2, attn_pe=1, attn_reg=4), nbatch, W, W, W, seed=1)  # nbatch windows per forward
     dv = DevBuf.from_numpy(vol); dout = DevBuf(vol.size, zero=False)
     small = (W, W, W)                                                                 # warm-up: one window (weights prepared, scratch grown)
     rc, _, _ = net.predict_volume(dv.ptr, small, halo, B, 115.0, 1 / 40.0, 1, 400.0, -300.0, dout.ptr)
@@ -144,7 +144,7 @@ def sliding_leg(np, lib, LP, DevBuf):
     head = dout.to_numpy(np.uint8)[:1 << 20]
     net.close()
     nvox = float(dims[0]) * dims[1] * dims[2]
-    return {"workload": "configs[4]: 512x1024x1024 uint8 in HBM, 128^3 windows, halo 16, feather 16, U-Net 32/64/128/192, MX-fp4 weights over MX-fp8 activations, 2 attention blocks on 16^3 tokens (MX-fp8 core)",
+    return {"workload": "configs[4]: 512x1024x1024 uint8 in HBM, 128^3 windows, halo 16, feather 16, U-Net 32/64/128/192, MX-fp4 weights over MX-fp8 activations, 2 attention blocks on 16^3 tokens (MX-fp8 core), %d windows per forward" % nbatch,
             "value": nvox / dt, "unit": "voxels/s", "seconds": dt, "windows": int(nw), "windows_computed": int(ndone), "output_mean_first_mib": float(head.mean())}
 
 
@@ -158,6 +158,7 @@ def main():
     ap.add_argument("--no-unet", action="store_true", help="skip the configs[3] U-Net forward leg")
     ap.add_argument("--no-sliding", action="store_true", help="skip the configs[4]-geometry sliding-window leg")
     ap.add_argument("--no-hbm", action="store_true", help="skip the HBM-bound kernels leg")
+    ap.add_argument("--windows-per-forward", type=int, default=8, help="sliding-window leg: windows batched into one forward")
     ap.add_argument("--copy-probe", action="store_true", help="run 5 device-to-device copies of 1 GiB and exit: the known-size kernel that scales "
                     "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--conv-probe", default="", metavar="Ci,Co,N,D,bits", help="time one 3x3x3 conv shape (MX in / out of the compute format, fused statistics) "
@@ -269,7 +270,7 @@ def main():
     if not a.no_unet:
         out["unet"] = unet_leg(np, lib, LP, DevBuf, max(3, a.steps // 4), max(1, a.warmup))
     if not a.no_sliding:
-        out["sliding_window"] = sliding_leg(np, lib, LP, DevBuf)
+        out["sliding_window"] = sliding_leg(np, lib, LP, DevBuf, a.windows_per_forward)
     if not a.no_hbm:
         out["hbm_kernels"] = hbm_leg(np, lib, LP, DevBuf)
     if not a.no_cpu_baseline:

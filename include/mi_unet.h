@@ -64,6 +64,8 @@ void unet_set_params(unet *u, const float *host);
 int unet_forward_x(unet *u, const void *x, float *logits);     /* x: device MX tensor (act_dt) of the input; logits: device fp32 [n][head_out][S] */
 /* the input built on the device from a uint8 CT window of one sample (src/unet.c:2858-2865, src/lp_mx_cvt.cu:29-55), then the forward */
 int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, float *logits);
+/* the same over the network's in.n windows in one forward (window n -> sample n; per-sample results equal the one-window forward's) */
+int unet_forward_ct_n(unet *u, const uint8_t *const *ct, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, float *logits);
 /* per-layer introspection for parity tests: the k-th conv output tensor (device MX) and its shape, in execution order; NULL past the end */
 const void *unet_layer_out(const unet *u, int k, shape5 *s, const char **name);
 /* the GroupNorm statistics the k-th conv produced (device [n * G] each); returns G, 0 when the layer has none */
@@ -84,8 +86,8 @@ int unet_get_infer_slab(void);
 shape5 unet_in_shape(const unet *u);                          /* the window the graph was created for */
 const unet_cfg *unet_config(const unet *u);
 /* ---- sliding-window prediction of a volume resident in device memory (src/predict.c: the --feather single pass, :282-333, :2538-2545,
-   :3420-3436). vol: uint8 CT [dims0][dims1][dims2]; windows of the graph's size (one cubic sample) with `halo` voxels of context per side
-   tile the volume at stride window - 2 halo in z-y-x order; each runs unet_forward_ct (z-score mean / isd; axis, cy, cx: the scroll axis
+   :3420-3436). vol: uint8 CT [dims0][dims1][dims2]; windows of the graph's size (cubic; the graph's in.n samples are that many windows per forward) with
+   `halo` voxels of context per side tile the volume at stride window - 2 halo in z-y-x order; each runs as a sample of unet_forward_ct_n (z-score mean / isd; axis, cy, cx: the scroll axis
    sign and its centre in volume y / x, axis 0: no direction channels) and places uint8(255 sigmoid(logit 0) + .5) where CT >= the
    prediction iso over its interior plus `feather` voxels of its upper halo; the window borders are then blended over `feather` voxels
    (0: none; <= halo) into out: uint8 [dims0][dims1][dims2]. Windows whose CT holds no voxel >= iso are skipped (their interior stays 0

@@ -125,3 +125,31 @@ def test_predict_volume_equals_windows_run_one_by_one(gpu):
     assert (got[shell] != plain[shell]).mean() > 0.25                        # the blended shells moved (windows disagree: per-window GroupNorm)
     assert (got[:S, :S, S:] == 0).all() and got.std() > 5                    # the air window stays empty; the output is not constant
     net.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("attn", [0, 1])
+def test_predict_volume_batched_windows_equal_single(gpu, attn):
+    """A graph created for two (three) samples runs that many windows per forward: samples are independent, so the prediction is the
+    one-window graph's byte for byte, with an odd number of windows (11: the last batch is incomplete) and with an attention stage."""
+    from ufsm_amd.unet import UNet, make_cfg
+    rng = np.random.default_rng(9)
+    W, halo, B = 32, 8, 8; S = W - 2 * halo
+    dims = (40, 32, 24)
+    z, y, x = np.meshgrid(np.arange(dims[0]), np.arange(dims[1]), np.arange(dims[2]), indexing="ij")
+    vol = np.clip(70 + 0.6 * z + 0.7 * y + 35 * np.sin(0.25 * x + 0.3 * y) * np.cos(0.2 * z) + rng.integers(0, 16, dims), 0, 255).astype(np.uint8)
+    vol[:S, :S, S:] = 0                                                     # one air window: 11 of 12 computed
+    dv = DevBuf.from_numpy(vol)
+    kw = dict(attn_blocks=1, attn_pe=1, attn_reg=2) if attn else {}
+    widths = [16, 192] if attn else [16, 32]
+    outs = []
+    for nb in (1, 2, 3):
+        net = UNet(make_cfg(4, widths, G=8, head_out=1, act_dt=8, **kw), nb, W, W, W, seed=5)
+        p = net.params(); p[-1] = 0.0; net.set_params(p)
+        dout = DevBuf(vol.size)
+        rc, nw, ndone = net.predict_volume(dv.ptr, dims, halo, B, 100.0, 1 / 50.0, 1, 40.0, -20.0, dout.ptr)
+        assert rc == 0 and nw == 12 and ndone == 11
+        outs.append(dout.to_numpy(np.uint8, dims))
+        net.close()
+    assert outs[0].max() > 0 and outs[0].std() > 0
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])

@@ -99,7 +99,7 @@ template <int HD> __device__ __forceinline__ float in_round(float v) {
     return v;
 }
 template <int B, int HD>
-__global__ void __launch_bounds__(256) pred_in_mx_k(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, uint8_t *y) {
+__global__ void __launch_bounds__(256) pred_in_mx_k(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, uint8_t *y, int N, int n) {
     const size_t S = (size_t)nz * W * W, i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     if (i >= S) return;
     const int xx = (int)(i % W), yy = (int)((i / W) % W), z = z0 + (int)(i / ((size_t)W * W));
@@ -109,16 +109,21 @@ __global__ void __launch_bounds__(256) pred_in_mx_k(const uint8_t *ct, int W, fl
     for (int k = 0; k < 32; k++) r[k] = 0.f;
     r[0] = in_round<HD>(((float)ct[(size_t)z * W * W + (size_t)yy * W + xx] - mean) * isd); r[1] = in_round<HD>(0.f);
     r[2] = in_round<HD>(__fmul_rn(dy, inv)); r[3] = in_round<HD>(__fmul_rn(dx, inv));     // (axis 0: the products are signed zeros, kept as such)
-    store_row<B, true>(y, mx_scp<B>(y, 1, 4, S), i, 8, r);
+    store_row<B, true>(y, mx_scp<B>(y, N, 4, S), (size_t)n * S + i, 8, r);       // sample n of an N-sample tensor: its rows, then the tensor's scale plane
 }
-extern "C" void lp_pred_input_mx(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits) {
+// sample n of an N-sample input tensor (the reference's entry is one window: N 1, n 0)
+extern "C" void mi_pred_input_mx_n(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits, int N, int n) {
     const size_t S = (size_t)nz * W * W; if (!S) return;
+    if (N < 1 || n < 0 || n >= N) mi_die("mi_pred_input_mx_n: sample %d of %d", n, N);
     uint8_t *yy = (uint8_t *)y;
-#define PIN(B, HD) pred_in_mx_k<B, HD><<<nblk_(S, 256), 256>>>(ct, W, mean, isd, dyo, dxo, axis, z0, nz, yy)
+#define PIN(B, HD) pred_in_mx_k<B, HD><<<nblk_(S, 256), 256>>>(ct, W, mean, isd, dyo, dxo, axis, z0, nz, yy, N, n)
     if (bits == 4) { if (hd == 2) PIN(4, 2); else if (hd == 1) PIN(4, 1); else PIN(4, 0); }
     else { if (hd == 2) PIN(8, 2); else if (hd == 1) PIN(8, 1); else PIN(8, 0); }
 #undef PIN
     MICK();
+}
+extern "C" void lp_pred_input_mx(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits) {
+    mi_pred_input_mx_n(ct, W, mean, isd, dyo, dxo, axis, z0, nz, y, hd, bits, 1, 0);
 }
 extern "C" void lp_pred_input_mx8(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd) {
     lp_pred_input_mx(ct, W, mean, isd, dyo, dxo, axis, z0, nz, y, hd, 8);

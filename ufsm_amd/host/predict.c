@@ -9,35 +9,59 @@ int unet_predict_volume(unet *u, const uint8_t *vol, const int64_t dims[3], int 
                         int axis, float cy, float cx, uint8_t *out, int64_t nwin[2]) {
     const shape5 in = unet_in_shape(u);
     const int W = in.w, S = W - 2 * halo, B = feather, En = S + B;
-    if (in.n != 1 || in.d != W || in.h != W || halo < 0 || S <= 0 || B < 0 || B > halo || B > S || B > 1024) {
-        fprintf(stderr, "unet_predict_volume: needs one cubic window, 0 <= feather <= halo, window - 2 halo > 0 and feather <= it (window %d x %d x %d, halo %d, feather %d)\n",
+    if (in.n < 1 || in.n > 16 || in.d != W || in.h != W || halo < 0 || S <= 0 || B < 0 || B > halo || B > S || B > 1024) {
+        fprintf(stderr, "unet_predict_volume: needs cubic windows (1 .. 16 per forward), 0 <= feather <= halo, window - 2 halo > 0 and feather <= it (window %d x %d x %d, halo %d, feather %d)\n",
                 in.d, in.h, in.w, halo, feather);
         return -1;
     }
     int64_t nss[3], total = 1;
     for (int d = 0; d < 3; d++) { if (dims[d] <= 0) return -1; nss[d] = (dims[d] + S - 1) / S; total *= nss[d]; }
     const size_t w3 = (size_t)W * W * W, e3 = (size_t)En * En * En;
-    uint8_t *E = mi_malloc((size_t)total * e3), *ctw = mi_malloc(w3), *dpres = mi_malloc((size_t)total);
-    float *lg = mi_malloc((size_t)unet_config(u)->head_out * w3 * sizeof(float)), *doff = mi_malloc(2 * (size_t)W * sizeof(float));
-    unsigned *dany = mi_malloc(sizeof(unsigned));
+    uint8_t *E = mi_malloc((size_t)total * e3), *ctw = mi_malloc((size_t)in.n * w3), *dpres = mi_malloc((size_t)total);
+    const size_t lgn = (size_t)unet_config(u)->head_out * w3;      /* logits of one window */
+    float *lg = mi_malloc((size_t)in.n * lgn * sizeof(float)), *doff = mi_malloc((size_t)total * 2 * W * sizeof(float));
+    unsigned *dany = mi_malloc((size_t)total * sizeof(unsigned));
     uint8_t *present = calloc((size_t)total, 1);
-    float *hoff = malloc(2 * (size_t)W * sizeof(float));
-    int rc = present && hoff ? 0 : -1;
+    unsigned *hany = malloc((size_t)total * sizeof(unsigned));
+    float *hoff = malloc((size_t)total * 2 * W * sizeof(float));
+    int rc = present && hoff && hany ? 0 : -1;
     int64_t done = 0;
     const int iso = nn_get_pred_iso();
-    for (int64_t a = 0; a < nss[0] && !rc; a++) for (int64_t b = 0; b < nss[1] && !rc; b++) for (int64_t c = 0; c < nss[2] && !rc; c++) {
-        const int64_t id = (a * nss[1] + b) * nss[2] + c, oz = a * S - halo, oy = b * S - halo, ox = c * S - halo;
-        mi_zero(dany, sizeof(unsigned));
-        mi_ct_window(vol, dims[0], dims[1], dims[2], oz, oy, ox, W, ctw, iso, halo, dany);
-        unsigned any = 0; mi_d2h(&any, dany, sizeof any);
-        if (!any) continue;                                 /* air: not computed; its neighbours renormalise */
-        for (int z = 0; z < W; z++) { hoff[z] = (float)oy - cy; hoff[W + z] = (float)ox - cx; }      /* the window rows' / columns' offsets from the scroll axis, per plane */
-        mi_h2d(doff, hoff, 2 * (size_t)W * sizeof(float));
-        if (unet_forward_ct(u, ctw, mean, isd, doff, doff + W, axis, lg)) { rc = -1; break; }
-        /* E: the interior and B voxels of the upper halo, window coordinates [halo, halo + S + B) -> [0, S + B) (src/predict.c:3426-3427) */
-        nn_pred_place(lg, ctw, W, halo - B, -halo, -halo, -halo, En, En, En, En, E + (size_t)id * e3);
-        present[id] = 1; done++;
+    /* Pass 1, no host round trip per window: every window's "holds a voxel >= iso in its interior" flag (air windows are not computed; their
+     * neighbours renormalise) and the table of the window rows' / columns' offsets from the scroll axis, then one copy each way. The forwards
+     * of pass 2 are then enqueued back to back and the GPU never waits for the host. */
+    if (!rc) {
+        mi_zero(dany, (size_t)total * sizeof(unsigned));
+        for (int64_t a = 0; a < nss[0]; a++) for (int64_t b = 0; b < nss[1]; b++) for (int64_t c = 0; c < nss[2]; c++) {
+            const int64_t id = (a * nss[1] + b) * nss[2] + c, oz = a * S - halo, oy = b * S - halo, ox = c * S - halo;
+            mi_ct_window(vol, dims[0], dims[1], dims[2], oz, oy, ox, W, ctw, iso, halo, dany + id);
+            float *ho = hoff + (size_t)id * 2 * W;
+            for (int z = 0; z < W; z++) { ho[z] = (float)oy - cy; ho[W + z] = (float)ox - cx; }
+        }
+        mi_d2h(hany, dany, (size_t)total * sizeof(unsigned));
+        mi_h2d(doff, hoff, (size_t)total * 2 * W * sizeof(float));
     }
+    /* Pass 2: the windows that hold material, in z-y-x order, in.n per forward (window j of a batch -> sample j; samples are independent, so a
+     * window's prediction does not depend on its batch; a last, incomplete batch repeats its last window and places it once) */
+    int64_t *list = malloc((size_t)(total ? total : 1) * sizeof(int64_t)), np = 0;
+    if (!list) rc = -1;
+    for (int64_t id = 0; id < total && !rc; id++) if (hany[id]) list[np++] = id;
+    for (int64_t k = 0; k < np && !rc; k += in.n) {
+        const uint8_t *cts[16]; const float *dyos[16], *dxos[16]; int64_t ids[16];
+        for (int j = 0; j < in.n; j++) {
+            const int64_t id = list[k + j < np ? k + j : np - 1], a = id / (nss[1] * nss[2]), b = (id / nss[2]) % nss[1], c = id % nss[2];
+            ids[j] = id;
+            mi_ct_window(vol, dims[0], dims[1], dims[2], a * S - halo, b * S - halo, c * S - halo, W, ctw + (size_t)j * w3, iso, halo, NULL);
+            cts[j] = ctw + (size_t)j * w3; dyos[j] = doff + (size_t)id * 2 * W; dxos[j] = dyos[j] + W;
+        }
+        if (unet_forward_ct_n(u, cts, mean, isd, dyos, dxos, axis, lg)) { rc = -1; break; }
+        for (int j = 0; j < in.n && k + j < np; j++) {
+            /* E: the interior and B voxels of the upper halo, window coordinates [halo, halo + S + B) -> [0, S + B) (src/predict.c:3426-3427) */
+            nn_pred_place(lg + (size_t)j * lgn, cts[j], W, halo - B, -halo, -halo, -halo, En, En, En, En, E + (size_t)ids[j] * e3);
+            present[ids[j]] = 1; done++;
+        }
+    }
+    free(list);
     if (!rc) {
         mi_h2d(dpres, present, (size_t)total);
         rc = mi_feather_blend(E, dpres, S, B, nss, dims, out);
@@ -47,6 +71,6 @@ int unet_predict_volume(unet *u, const uint8_t *vol, const int64_t dims[3], int 
     if (nwin) { nwin[0] = total; nwin[1] = done; }
     mi_sync();
     mi_free(E); mi_free(ctw); mi_free(dpres); mi_free(lg); mi_free(doff); mi_free(dany);
-    free(present); free(hoff);
+    free(present); free(hoff); free(hany);
     return rc;
 }

@@ -249,8 +249,14 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
     return nn_conv3d_fwd_x(last->a2, &g, nullptr, nullptr, 0, 0, last->ys, P(u, u->head.w), P(u, u->head.b), u->cfg.head_out, 1, 1, logits, 0, 0.f, nullptr, nullptr);
 }
 int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, float *logits) {
-    if (u->in.n != 1 || u->cfg.cin != 4 || u->in.h != u->in.w) { fprintf(stderr, "unet_forward_ct: needs one square window of 4 input channels\n"); return -1; }
-    lp_pred_input_mx(ct, u->in.w, mean, isd, dyo, dxo, axis, 0, u->in.d, u->xin, 2, u->cfg.act_dt == 4 ? 4 : 8);      /* fp16-rounded input values, as predict */
+    if (u->in.n != 1) { fprintf(stderr, "unet_forward_ct: needs one square window of 4 input channels\n"); return -1; }
+    return unet_forward_ct_n(u, &ct, mean, isd, &dyo, &dxo, axis, logits);
+}
+/* one forward over in.n windows: window n's input rows go to sample n (fp16-rounded input values, as predict); logits [n][head_out][voxels] */
+int unet_forward_ct_n(unet *u, const uint8_t *const *ct, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, float *logits) {
+    if (u->cfg.cin != 4 || u->in.h != u->in.w) { fprintf(stderr, "unet_forward_ct: needs square windows of 4 input channels\n"); return -1; }
+    for (int n = 0; n < u->in.n; n++)
+        mi_pred_input_mx_n(ct[n], u->in.w, mean, isd, dyo[n], dxo[n], axis, 0, u->in.d, u->xin, 2, u->cfg.act_dt == 4 ? 4 : 8, u->in.n, n);
     return unet_forward_x(u, u->xin, logits);
 }
 shape5 unet_in_shape(const unet *u) { return u->in; }

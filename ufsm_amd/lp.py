@@ -52,6 +52,7 @@ _PROTOS = {
     "lp_mx4_to_f32": (None, [_P, _I, _I, _Z, _P]),
     "lp_pred_input_mx": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I, _I]),
     "lp_pred_input_mx8": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I]),
+    "mi_pred_input_mx_n": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I]),
     "lp_gn_silu_apply_mx": (None, [_P, _I, shape5, _I, _P, _P, _P, _P, _P, _I]),
     "lp_add_mx": (None, [_P, _P, shape5, _I, C.c_uint]),
     "lp_up2_fwd_mx": (None, [_P, _I, shape5, _P, _I, gnp_t]),
