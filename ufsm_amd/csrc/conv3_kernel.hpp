@@ -566,7 +566,9 @@ __global__ void __launch_bounds__(256, 2) conv3_mx_k(const conv_args a) {
     }
 
     __syncthreads();                                     // the ring and halo are dead: the epilogue reuses LDS for its statistics scratch
-    conv_epilogue<MT, NT, OUT, EPI, false, (MT > 1)>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);      // (two or more channel tiles: more than 32 output channels, 32-wide output rows)
+    // (uniform) more than 16 output channels, always so with two or more channel tiles: 32-wide output rows known at compile time
+    if (MT > 1 || a.Co > 16) conv_epilogue<MT, NT, OUT, EPI, false, true>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
+    else conv_epilogue<MT, NT, OUT, EPI>(a, acc, lds, tile, n, cs, oz0, oy0, ox0, lz, ly0, tid);
 }
 
 extern thread_local char g_last_kernel[128];
