@@ -1,13 +1,14 @@
 // The small-channel 3x3x3 stride-1 kernel: one channel tile and one input block (<= 32 channels in and out), TZ x 8 x 16 voxels per tile.
 //
-// With 32 output channels every input fragment feeds a single MFMA, so the K loop is bound by LDS reads and everything around it has to
-// get out of its way:
+// With 32 output channels every input fragment feeds a single MFMA (two 16-byte LDS reads and a scale word per lane and MFMA), and the
+// epilogue is as long as half the MFMAs, so everything else has to get out of the way:
 //   * workgroups are persistent (two per CU) and walk their tiles XCD by XCD; the 14 pairs of weight fragments are loaded into registers
 //     once per workgroup, so the K loop has no weight ring, no pair table and no barriers, and the taps' halo offsets are instruction immediates;
 //   * the halo of the next tile is copied global -> LDS directly (global_load_lds, no registers) into a second buffer before the current
 //     tile's MFMAs start and has landed when they are done: a tile is MFMAs, epilogue and one barrier. Positions outside the volume read
 //     a zero row / scale byte 1 from a constant page;
-// Measured at 32 -> 32 channels, 2 x 128^3, MX-fp8 (8192 tiles): 0.151 ms; the K loop alone 0.087 - 0.093 ms with one or with two wavefronts per
+//   * the epilogue's output rows are 32 wide at compile time (more than 16 output channels; fewer go to the general kernel).
+// Measured at 32 -> 32 channels, 2 x 128^3, MX-fp8 (8192 tiles): 0.133 ms; before the epilogue's last diet 0.151 ms, of which the K loop alone 0.087 - 0.093 ms with one or with two wavefronts per
 // SIMD (72 % of the matrix pipe's cycles at the 1.82 GHz the part settles at under it; 0.077 ms at 1.71 GHz with half the LDS reads), the
 // epilogue alone 0.051 ms, the copies 0.01 - 0.03 ms. The parts add up whatever the arrangement: a start offset between the CU's two
 // workgroups changes nothing, and one workgroup of two groups of four wavefronts that alternate MFMA and epilogue phases behind barriers
