@@ -32,7 +32,8 @@ __global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int 
     // the group's channel quads are consecutive: quad Q = co / 4 lives in channel slice Q / (8 MT), slot Q % (8 MT) of its tile's record
     const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, qpg = Co / Go / 4, nq = MT * 8, nst = tiles_per_n / ncs;
     double s = 0.0, ss = 0.0;
-    for (int i = threadIdx.x; i < nst * qpg; i += 256) {
+#pragma unroll 8
+    for (int i = threadIdx.x; i < nst * qpg; i += 256) {                   // (unrolled: the records' loads of several rounds are in flight together)
         const int st = i / qpg, Q = gidx * qpg + i % qpg, cs = Q / nq, qd = Q - cs * nq;
         const float2 p = part[(size_t)(n * tiles_per_n + st * ncs + cs) * nq + qd];
         s += (double)p.x; ss += (double)p.y;
