@@ -80,10 +80,11 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
     unsigned *tsc = wsc + ((size_t)gp * nmt_all + m) * 64;      // one word per lane: the byte the MFMA reads is the low one
     int tss = 1;                                                // words between two lanes' scale words
     if (block_major) {
-        // the wide kernel's layout: per 128-channel slice, pair after pair the image of its LDS stage: four tiles of codes, then per lane the
-        // four tiles' scale words
-        uint8_t *img = wq + ((size_t)(m >> 2) * (npairs_all + 16) + gp) * (size_t)(4 * (WTILE + 256));
-        tile = img + (m & 3) * WTILE; tsc = (unsigned *)(img + 4 * WTILE) + (m & 3); tss = 4;
+        // the wide kernel's layout (block_major = its channel tiles per workgroup, 4 or 2): per slice of that many tiles, pair after pair the
+        // image of its LDS stage: the tiles' codes, then per lane the tiles' scale words
+        const int MW = block_major, sl = m / MW, mi = m - sl * MW;
+        uint8_t *img = wq + ((size_t)sl * (npairs_all + 16) + gp) * (size_t)(MW * (WTILE + 256));
+        tile = img + mi * WTILE; tsc = (unsigned *)(img + MW * WTILE) + mi; tss = MW;
     }
 #pragma unroll
     for (int side = 0; side < 2; side++) {
@@ -292,8 +293,10 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 1) / 2) * (nmt_all / MT) * N < 256) NT = 1;
     // 128-channel output slices at stride 1 take the wide kernel (16 accumulators per wavefront, one workgroup per CU)
     static int big_env = -1;
-    if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel
-    bool big = big_env && stride == 1 && MT == 4 && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
+    if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel, 2 sends every 64-channel layer to the wide kernel too
+    // (64 output channels: two channel tiles per workgroup; it pays from four input blocks on: 192 -> 64 at 2 x 64^3 0.190 -> 0.178 ms, 64 -> 64 the same
+    // as the general kernel. MI_CONV_WIDE=2 sends every such layer there)
+    bool big = big_env && stride == 1 && (MT == 4 || (MT == 2 && (big_env > 1 || a.nbt >= 4))) && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
     if (big) {
         // The wide kernel streams input block b >= 2 of a tile into LDS while the tile's earlier blocks are multiplied, one copy round per
         // stage of two pairs, NRND rounds per block, a block starting once block b - 3 has been read for the last time (pair (27 (b - 3) + 26) / 2).
@@ -356,8 +359,9 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // (sixteen pairs of padding: the kernels' weight loads run up to two ring stages ahead of the last pair)
     // (the wide kernel's weights are one buffer: codes and scale words interleaved pair by pair; its scale buffer is a stub)
     const size_t wq_bytes = (size_t)(npairs_all + 16) * nmt_all * (big ? WTILE + 256 : WTILE), wsc_bytes = big ? 256 : (size_t)(npairs_all + 16) * nmt_all * 256;
-    a.wstride = (unsigned)((size_t)(npairs_all + 16) * 4 * (WTILE + 256));
+    a.wstride = (unsigned)((size_t)(npairs_all + 16) * MT * (WTILE + 256));
     const int memoCB = big ? -a.CB : a.CB;
+    a.big = big;
     const int CxP = (Cx + 31) / 32 * 32;
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
@@ -373,8 +377,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) {
         const size_t nt = (size_t)npairs_all * nmt_all * 32;
-        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? 1 : 0);
-        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? 1 : 0);
+        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : 0);
+        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : 0);
         MICK();
     }
     a.wq = wq; a.wsc = wsc;

@@ -105,6 +105,7 @@ struct conv_args {
     const void *sx; int sxdt, sCi;
     const float *sgam, *sbet, *smean, *srstd; int sG;
     int zc; unsigned ngrp;             // consecutive z tiles a workgroup walks, workgroups with work
+    bool big;                          // the wide kernel takes the launch (MT 4, or MT 2 with NT 4)
     bool areg;                         // the persistent small-channel kernel (one channel tile, one input block, weights in registers) takes the launch
 };
 
@@ -598,7 +599,7 @@ static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     case 32: launch_conv<FMT, STRIDE, 3, 2, OUT, EPI>(a, smem); break;
     case 42: launch_conv<FMT, STRIDE, 4, 2, OUT, EPI>(a, smem); break;
     case 14: if constexpr (STRIDE == 1) { if (a.areg) launch_small<FMT, 4, OUT, EPI>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
-    case 24: if constexpr (STRIDE == 1) { launch_conv<FMT, 1, 2, 4, OUT, EPI>(a, smem); break; }
+    case 24: if constexpr (STRIDE == 1) { if (a.big) launch_wide<FMT, OUT, EPI, 2>(a, smem); else launch_conv<FMT, 1, 2, 4, OUT, EPI>(a, smem); break; }
     default: mi_die("conv3: no kernel for MT %d NT %d stride %d", MT, NT, STRIDE);
     }
 }

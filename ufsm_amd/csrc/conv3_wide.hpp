@@ -34,9 +34,11 @@ template <int IMM> __device__ __forceinline__ void dma16si(unsigned off, const v
 }
 template <int N> __device__ __forceinline__ void wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-template <int FMT, int OUT, bool EPI>
+// MT: channel tiles of 32 per workgroup: 4 (slices of 128 output channels) or 2 (64-channel layers: 8 accumulators per wavefront)
+template <int FMT, int OUT, bool EPI, int MT = 4>
 __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
-    constexpr int MT = 4, NT = 4, TZ = 4;
+    constexpr int NT = 4, TZ = 4;
+    static_assert(MT == 4 || MT == 2, "channel tiles per workgroup");
     using HL = halo_t<FMT, 1, TZ>;
     constexpr int TT = HL::TT, HY = HL::HY, HX = HL::HX, NH = HL::NH, WTILE = fmt_t<FMT>::WTILE;
     constexpr int STG = MT * (WTILE + 256), SLOT = 2 * STG;     // a ring slot holds one stage = two pairs, each MT tiles of codes then MT x 64 scale words
@@ -55,7 +57,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     const int p00 = (lz * HY + (r >> 4)) * HX + (r & 15);
     const unsigned abr0 = halo_o + ((NH == 2 ? h * TTP : 0) + p00) * 16, sbr0 = halo_o + NH * TTP * 16 + p00 * 4;
     constexpr unsigned ABJ = 2 * HX * 16, SBJ = 2 * HX * 4;
-    const unsigned wfa = lane * 16, wfs = MT * WTILE + lane * 16;           // the lane's weight fragment of tile 0 / its MT scale words of pair 0 of a slot
+    const unsigned wfa = lane * 16, wfs = MT * WTILE + lane * (MT * 4);     // the lane's weight fragment of tile 0 / its MT scale words of pair 0 of a slot
     const size_t Sin = (size_t)a.D * a.H * a.W;
     const int nunits = 27 * a.nbt, npairs = (nunits + 1) >> 1, nfull = npairs >> 1;
 
@@ -218,7 +220,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         v16f acc[MT][NT];                                       // (not cleared: the tile's first pair multiplies onto a zero operand)
         __syncthreads();
 
-        v8i fb[2][NT], fa[2][MT]; int sb[2][NT]; v4i sav[2];
+        v8i fb[2][NT], fa[2][MT]; int sb[2][NT]; int sav[2][MT];
         v4i T;
         unsigned tabp = tab_o + h * 16;
         T = *(const v4i *)(lds + tabp);
@@ -240,7 +242,10 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
                 constexpr int m = f - NT;
                 if constexpr (part == 0) lo[f] = *(const v4i *)(lds + wfa + wbase + m * WTILE);
                 else if constexpr (part == 1) { if constexpr (FMT == 8) hi[f] = *(const v4i *)(lds + wfa + wbase + m * WTILE + 1024); }
-                else if constexpr (m == 0) sav[nx] = *(const v4i *)(lds + wfs + wbase);      // the MT scale words of the pair at once
+                else if constexpr (m == 0) {                    // the MT scale words of the pair at once
+                    if constexpr (MT == 4) { const v4i t4 = *(const v4i *)(lds + wfs + wbase); sav[nx][0] = t4[0]; sav[nx][1] = t4[1]; sav[nx][2] = t4[2]; sav[nx][3] = t4[3]; }
+                    else { const int2 t2 = *(const int2 *)(lds + wfs + wbase); sav[nx][0] = t2.x; sav[nx][1] = t2.y; }
+                }
             }
         };
         auto pack = [&](auto NXT) {
@@ -332,19 +337,19 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
     }
 }
 
-template <int FMT, int OUT, bool EPI>
+template <int FMT, int OUT, bool EPI, int MT = 4>
 static void launch_wide(const conv_args &a, size_t smem) {
     static bool attr[8]; static int ncu[8];
     int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
     if (!attr[d]) {
-        MIRT(hipFuncSetAttribute((const void *)conv3_wide_k<FMT, OUT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        MIRT(hipFuncSetAttribute((const void *)conv3_wide_k<FMT, OUT, EPI, MT>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         hipDeviceProp_t pr; MIRT(hipGetDeviceProperties(&pr, d));
         ncu[d] = pr.multiProcessorCount > 8 ? pr.multiProcessorCount & ~7 : 8;
         attr[d] = true;
     }
     const unsigned per = (a.ntiles + 7u) / 8u;            // tiles per XCD; one persistent workgroup per CU, a multiple of 8 in all
     const unsigned nwg = per * 8u < (unsigned)ncu[d] ? per * 8u : (unsigned)ncu[d];
-    conv3_wide_k<FMT, OUT, EPI><<<nwg, 256, smem>>>(a);
+    conv3_wide_k<FMT, OUT, EPI, MT><<<nwg, 256, smem>>>(a);
     MICK();
-    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_wide_k<fmt %d, out %d, epi %d> tiles %u wgs %u", FMT, OUT, (int)EPI, a.ntiles, nwg);
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_wide_k<fmt %d, out %d, epi %d%s> tiles %u wgs %u", FMT, OUT, (int)EPI, MT == 2 ? ", MT 2" : "", a.ntiles, nwg);
 }
