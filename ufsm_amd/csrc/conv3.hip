@@ -286,6 +286,13 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // ---- tile shape: MT channel tiles of 32 per workgroup, NT voxel tiles of 32 per wavefront, MT * NT <= 8 accumulators ----
     const int nmt_all = (cout + 31) / 32;
     int MT = nmt_all <= 4 ? nmt_all : nmt_all % 4 == 0 ? 4 : nmt_all % 3 == 0 ? 3 : nmt_all % 2 == 0 ? 2 : 1;
+    bool halved = false;
+    {   // few tiles of 128 channels (the coarse levels): slices of 64 channels double the workgroups of the wide kernel
+        static int split_env = -1;
+        if (split_env < 0) split_env = getenv("MI_CONV_SPLIT") ? atoi(getenv("MI_CONV_SPLIT")) : 192;    // tuning knob: tile count below which the slices are halved (0: never)
+        if (stride == 1 && MT == 4 && nmt_all % 4 == 0 && Do >= 3 &&
+            (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 3) / 4) * (nmt_all / 4) * N < (size_t)split_env) { MT = 2; halved = true; }
+    }
     int NT = (stride == 1 && MT <= 2 && Do >= 4) ? 4 : 2;
     // stride 2 with few tiles (the coarse levels): one-plane tiles double the workgroups; with enough tiles the two-plane tile is faster
     // (measured: 128 -> 128 at 32^3 -> 16^3, N 2: 32 tiles 0.072 ms, 64 tiles 0.042 ms; 32 -> 32 at 128^3: 0.090 vs 0.120 ms)
@@ -296,7 +303,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel, 2 sends every 64-channel layer to the wide kernel too
     // (64 output channels: two channel tiles per workgroup; it pays from four input blocks on: 192 -> 64 at 2 x 64^3 0.190 -> 0.178 ms, 64 -> 64 the same
     // as the general kernel. MI_CONV_WIDE=2 sends every such layer there)
-    bool big = big_env && stride == 1 && (MT == 4 || (MT == 2 && (big_env > 1 || a.nbt >= 4))) && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
+    bool big = big_env && stride == 1 && (MT == 4 || (MT == 2 && (big_env > 1 || a.nbt >= 4 || halved))) && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
     if (big) {
         // The wide kernel streams input block b >= 2 of a tile into LDS while the tile's earlier blocks are multiplied, one copy round per
         // stage of two pairs, NRND rounds per block, a block starting once block b - 3 has been read for the last time (pair (27 (b - 3) + 26) / 2).
