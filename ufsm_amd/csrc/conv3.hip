@@ -216,6 +216,7 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     return 0;
 }
 
+static int split_s2_env() { static int v = -1; if (v < 0) v = getenv("MI_CONV_SPLIT_S2") ? atoi(getenv("MI_CONV_SPLIT_S2")) : 1; return v; }      // tuning knob: 0 keeps four channel tiles
 static int conv_dispatch(const char *who, int fmt, int stride, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                          gnp_t gp, double *osum, int Go, split_t sp, const float *ep_a, const float *ep_b, int act) {
     if (sp.y2 || sp.o_split || sp.accum || sp.sr || sp.osr || sp.o_pad || sp.zw0 || sp.zw1)
@@ -298,6 +299,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // (measured: 128 -> 128 at 32^3 -> 16^3, N 2: 32 tiles 0.072 ms, 64 tiles 0.042 ms; 32 -> 32 at 128^3: 0.090 vs 0.120 ms)
     if (stride == 2 && (MT == 1 || MT == 2 || MT == 4) &&
         (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 1) / 2) * (nmt_all / MT) * N < 256) NT = 1;
+    // ... and still fewer one-plane tiles than half the CUs: two channel tiles per workgroup instead of four
+    if (stride == 2 && MT == 4 && NT == 1 && split_s2_env() && (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * Do * (nmt_all / 4) * N < 128) MT = 2;
     // 128-channel output slices at stride 1 take the wide kernel (16 accumulators per wavefront, one workgroup per CU)
     static int big_env = -1;
     if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel, 2 sends every 64-channel layer to the wide kernel too
