@@ -53,6 +53,9 @@ void mi_conv_s2_wkey(unsigned wkey);
  * Calling thread only. The reference's kernel walks up to 32 (8 for wider rows),
  * overridden by UFSM_F8S_ZC (src/lp_f8fwd.cuh:412-416). */
 void mi_conv_stem_zc(int zc);
+/* tuning knob of the calling thread (no counterpart in the reference): stride-1 launches with fewer tiles of 128 output channels than this run as
+   slices of 64 channels, twice the workgroups; 0: never, -1: the default (192, or MI_CONV_SPLIT). The results do not depend on it. */
+void mi_conv_split(int tiles);
 /* no counterpart in the reference (its convs transform their input while staging, every time): GroupNorm + SiLU of x and re-quantisation to
    MX-fp8 / MX-fp4 (ybits 8 / 4) once, for a tensor several convs read; they then take y with no GroupNorm. s.c a multiple of 32. In a split
    input, gp2.G = -1 says "x2 carries no GroupNorm, gp is x's own" (gp2.G = 0 keeps the reference's meaning: gp spans both segments). */

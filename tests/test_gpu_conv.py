@@ -34,8 +34,17 @@ WIDE_SHAPES = [(8, 1, 96, 128, 5, 9, 18), (8, 1, 32, 128, 3, 8, 16), (8, 2, 128,
                (4, 1, 160, 128, 7, 8, 16), (4, 2, 64, 256, 4, 16, 16)]
 
 
+@pytest.fixture(params=[0, -1], ids=["slices128", "slices64"])
+def slice_split(request):
+    """These launches have few tiles, which by default run as slices of 64 channels (two channel tiles per workgroup); 0 keeps the slices of 128
+    (four channel tiles, the form the large layers run in): both forms of the wide kernel see every shape."""
+    lib.mi_conv_split(request.param)
+    yield request.param
+    lib.mi_conv_split(-1)
+
+
 @pytest.mark.parametrize("bits,N,Ci,Co,D,H,W", WIDE_SHAPES)
-def test_wide_kernel_exact(gpu, bits, N, Ci, Co, D, H, W):
+def test_wide_kernel_exact(gpu, slice_split, bits, N, Ci, Co, D, H, W):
     rng = np.random.default_rng(Ci * 17 + Co + D * 3 + bits)
     S = D * H * W
     x, w, b = exact_case(rng, N, Ci, Co, S)
@@ -43,7 +52,8 @@ def test_wide_kernel_exact(gpu, bits, N, Ci, Co, D, H, W):
     xq = orc.f32_to_mx(bits, x, N, Ci, S)
     want, wsum = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, acc64=1, Go=8, want_stats=True)
     got, gsum = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, Go=8, stats=True)
-    assert "conv3_wide_k" in lib.mi_last_kernel().decode()
+    name = lib.mi_last_kernel().decode()
+    assert "conv3_wide_k" in name and ("MT 2" in name) == (slice_split != 0)
     assert np.array_equal(got, want)
     assert np.allclose(gsum, wsum, rtol=1e-6)
     wf, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, acc64=1)

@@ -216,6 +216,8 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     return 0;
 }
 
+static thread_local int g_split = -1;       // mi_conv_split: the calling thread's tile count below which 128-channel slices are halved (-1: the default)
+extern "C" void mi_conv_split(int tiles) { g_split = tiles; }
 static int split_s2_env() { static int v = -1; if (v < 0) v = getenv("MI_CONV_SPLIT_S2") ? atoi(getenv("MI_CONV_SPLIT_S2")) : 1; return v; }      // tuning knob: 0 keeps four channel tiles
 static int conv_dispatch(const char *who, int fmt, int stride, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                          gnp_t gp, double *osum, int Go, split_t sp, const float *ep_a, const float *ep_b, int act) {
@@ -291,8 +293,9 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     {   // few tiles of 128 channels (the coarse levels): slices of 64 channels double the workgroups of the wide kernel
         static int split_env = -1;
         if (split_env < 0) split_env = getenv("MI_CONV_SPLIT") ? atoi(getenv("MI_CONV_SPLIT")) : 192;    // tuning knob: tile count below which the slices are halved (0: never)
+        const int split = g_split >= 0 ? g_split : split_env;
         if (stride == 1 && MT == 4 && nmt_all % 4 == 0 && Do >= 3 &&
-            (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 3) / 4) * (nmt_all / 4) * N < (size_t)split_env) { MT = 2; halved = true; }
+            (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 3) / 4) * (nmt_all / 4) * N < (size_t)split) { MT = 2; halved = true; }
     }
     int NT = (stride == 1 && MT <= 2 && Do >= 4) ? 4 : 2;
     // stride 2 with few tiles (the coarse levels): one-plane tiles double the workgroups; with enough tiles the two-plane tile is faster
