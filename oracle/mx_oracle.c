@@ -218,6 +218,7 @@ void orc_pred_input_mx(int bits, const uint8_t *ct, int W, float mean, float isd
         float r[8] = {0};
         r[0] = ((float)ct[(size_t)z * W * W + (size_t)yy * W + xx] - mean) * isd; r[2] = dy * inv; r[3] = dx * inv;
         if (hd == 2) for (int k = 0; k < 4; k++) r[k] = orc_h16_to_f32(orc_f32_to_h16(r[k]));
+        else if (hd == 1) for (int k = 0; k < 4; k++) { uint32_t u = f2u(r[k]); if ((u & 0x7fffffffu) <= 0x7f800000u) { u += 0x7fffu + ((u >> 16) & 1u); r[k] = u2f(u & 0xffff0000u); } }   /* bf16, round to nearest even */
         sc[i] = orc_store_row(bits, r, 8, y + (size_t)i * rb, 1);
     }
 }

@@ -259,6 +259,38 @@ def test_weight_memo(gpu):
     lib.lp_wmemo_clear()
 
 
+def test_weight_memo_keeps_layouts_apart(gpu):
+    """One memoised 128 -> 128 conv (same weights, same wkey) at tile counts on either side of the slice-split threshold, and with the
+    per-thread split knob toggled between calls: the wide kernel's weight image differs between its two forms (four or two channel tiles
+    per workgroup), so each form must find its own prepared weights. Exact operands: every result equals the oracle."""
+    rng = np.random.default_rng(71)
+    Ci = Co = 128
+    D, H, W = 16, 32, 64
+    S = D * H * W
+    w = refnp.gen_exact(rng, (Co, Ci, 27)); b = (GRID[rng.integers(0, 8, Co)] * 0.25).astype(np.float32)
+    dw, db = DevBuf.from_numpy(w), DevBuf.from_numpy(b)
+    sp = split_t(); sp.wkey = 4321
+    lib.lp_wmemo_clear()
+
+    def run(N, xq):
+        dxq = DevBuf.from_numpy(xq); dy = DevBuf(lib.lp_mx8_bytes(N, Co, S))
+        assert lib.lp_conv_fwd_f8(dxq.ptr, 3, shape5(N, Ci, D, H, W), dw.ptr, db.ptr, Co, dy.ptr, 3, gnp_t(), None, 0, sp) == 0
+        LP.check()
+        return dy.to_numpy(np.uint8), lib.mi_last_kernel().decode()
+
+    xq = {N: orc.f32_to_mx(8, refnp.gen_exact(rng, (N, Ci, S)), N, Ci, S) for N in (2, 3)}
+    want = {N: orc.conv3(xq[N], 3, N, Ci, D, H, W, w, b, Co, 3, acc64=1)[0] for N in (2, 3)}
+    seen = set()
+    for N, split in [(2, -1), (3, -1), (2, -1), (2, 0), (3, 1 << 20), (2, -1), (3, -1)]:      # 128 tiles: halved by default; 192: not
+        lib.mi_conv_split(split)
+        got, name = run(N, xq[N])
+        seen.add("MT 2" in name)
+        assert "conv3_wide_k" in name and np.array_equal(got, want[N]), (N, split, name)
+    lib.mi_conv_split(-1)
+    assert seen == {True, False}
+    lib.lp_wmemo_clear()
+
+
 def test_nonfinite_input_propagates(gpu):
     """A NaN block (scale byte 0xFF) reaches every output voxel whose taps touch it and nothing else (tests/test_mx4.c:139-168)."""
     rng = np.random.default_rng(80)

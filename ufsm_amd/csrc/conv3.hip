@@ -2,6 +2,7 @@
 // GroupNorm partial-sum reduction. The kernel itself is conv3_kernel.hpp, instantiated per (compute format, output kind) in
 // conv3_f*_o*.hip.
 #include "conv3_kernel.hpp"
+#include <mutex>
 
 // what a reduce block does with the (sum, sum of squares) of its (sample, group): add them to the caller's sum slots (the reference's contract,
 // src/lp_common.cuh:1575-1597), or, for a fused call, set the slots and finalize mean / rstd from them right away (src/nn_elem.cu:5-11), which saves
@@ -117,13 +118,16 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
 }
 
 // ---- prepared-weight memo (src/lp_f4fwd.cuh:748-770): keyed by the conv id sp.wkey and the layout ----
-struct wmemo_t { unsigned key; const float *w; int fmt, Co, Ci, Cx, nbt, CB, nmt_all, dev; uint8_t *wq, *wsc; };
+// (lay: what else fixes the image's layout: the wide kernel's channel tiles per workgroup, which follow the launch's tile count and mi_conv_split; 0 otherwise)
+struct wmemo_t { unsigned key; const float *w; int fmt, Co, Ci, Cx, nbt, CB, nmt_all, dev, lay; uint8_t *wq, *wsc; };
 static std::vector<wmemo_t> g_wmemo;
+static std::mutex g_wmemo_mu;      // host threads driving different devices share the list (one thread per device: the per-device scratch is not guarded)
 static unsigned g_wstep = 0;
 void mx_gemm_memo_clear(void);
 extern "C" void lp_wmemo_clear(void) {
     MIRT(hipDeviceSynchronize());
     mx_gemm_memo_clear();
+    std::lock_guard<std::mutex> lk(g_wmemo_mu);
     if (g_wmemo.empty()) return;
     for (auto &m : g_wmemo) { MIRT(hipFree(m.wq)); MIRT(hipFree(m.wsc)); }
     g_wmemo.clear();
@@ -196,12 +200,13 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
     if (sp.wkey) {                                     // memo entries of this layout: nbt = -CP
+        std::lock_guard<std::mutex> lk(g_wmemo_mu);
         for (auto &m : g_wmemo)
             if (m.key == sp.wkey && m.w == w && m.fmt == 8 && m.Co == cout && m.Ci == Ci && m.nbt == -CP - 1 && m.nmt_all == nmt_all && m.dev == dev) { wq = m.wq; wsc = m.wsc; have = true; break; }
         if (!have) {
             MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes));
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
-            g_wmemo.push_back(wmemo_t{sp.wkey, w, 8, cout, Ci, Ci, -CP - 1, 0, nmt_all, dev, wq, wsc});
+            g_wmemo.push_back(wmemo_t{sp.wkey, w, 8, cout, Ci, Ci, -CP - 1, 0, nmt_all, dev, 0, wq, wsc});
         }
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) conv3_stem_prep(CP, w, wq, wsc, cout, Ci, nmt_all, NP);
@@ -379,13 +384,14 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
     if (sp.wkey) {
+        std::lock_guard<std::mutex> lk(g_wmemo_mu);
         for (auto &m : g_wmemo)
-            if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == memoCB && m.nmt_all == nmt_all && m.dev == dev) { wq = m.wq; wsc = m.wsc; have = true; break; }
+            if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == memoCB && m.nmt_all == nmt_all && m.dev == dev && m.lay == (big ? MT : 0)) { wq = m.wq; wsc = m.wsc; have = true; break; }
         if (!have) {
             MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes));
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
             MIRT(hipMemsetAsync(wq, 0, wq_bytes, 0)); MIRT(hipMemsetAsync(wsc, 0, wsc_bytes, 0));
-            g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, memoCB, nmt_all, dev, wq, wsc});
+            g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, memoCB, nmt_all, dev, big ? MT : 0, wq, wsc});
         }
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) {

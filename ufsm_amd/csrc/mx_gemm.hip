@@ -2,6 +2,7 @@
 // that are MFMA fragments as they lie in memory, then a block-scaled MFMA GEMM runs over the packed bytes.
 // Interface and arithmetic: src/lp_mxgemm.cu:1-5 (definition), :88-113 (packing), :266-297 (entry points) of the reference.
 #include <vector>
+#include <mutex>
 #include "mx_dev.hpp"
 #include "../../include/mi_attn.h"
 
@@ -113,9 +114,11 @@ __global__ void __launch_bounds__(256) mx_gemm_k(const uint8_t *__restrict__ Aq,
 // lp_mx_gemm_bmemo(1) for the calling thread, dropped by lp_wmemo_clear() like the convs' prepared weights.
 struct bmemo_t { const float *B; int bits, tb, N, K, dev; uint8_t *q, *s; };
 static std::vector<bmemo_t> g_bmemo;
+static std::mutex g_bmemo_mu;
 static thread_local int g_bmemo_on = 0;
 extern "C" void lp_mx_gemm_bmemo(int on) { g_bmemo_on = on != 0; }
 void mx_gemm_memo_clear(void) {
+    std::lock_guard<std::mutex> lk(g_bmemo_mu);
     for (auto &m : g_bmemo) { MIRT(hipFree(m.q)); MIRT(hipFree(m.s)); }
     g_bmemo.clear();
 }
@@ -134,6 +137,7 @@ extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, cons
     bool bhave = false;
     if (g_bmemo_on && nkb) {
         int dev = 0; MIRT(hipGetDevice(&dev));
+        std::lock_guard<std::mutex> lk(g_bmemo_mu);
         for (auto &m : g_bmemo) if (m.B == B && m.bits == bits && m.tb == tb && m.N == N && m.K == K && m.dev == dev) { Bq = m.q; Bs = m.s; bhave = true; break; }
         if (!bhave) {
             uint8_t *q = nullptr, *sc = nullptr;
