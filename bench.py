@@ -42,13 +42,12 @@ def unet_leg(np, lib, LP, DevBuf, steps, warmup):
     x[:, 2] = np.broadcast_to((yy / r)[None], (D, D, D)).reshape(1, S); x[:, 3] = np.broadcast_to((xx / r)[None], (D, D, D)).reshape(1, S)
     dx = DevBuf.from_numpy(x)
     dxq = DevBuf(lib.lp_mx8_bytes(N, 4, S)); lib.lp_f32_to_mx8(dx.ptr, N, 4, S, dxq.ptr)
-    dlog = DevBuf(N * 8 * S * 4)
     for _ in range(warmup):
-        assert net.forward_x(dxq.ptr, dlog.ptr) == 0
+        assert net.forward_mx(dxq.ptr)
     lib.mi_sync(); LP.check()
     t0 = time.perf_counter()
     for _ in range(steps):
-        net.forward_x(dxq.ptr, dlog.ptr)
+        net.forward_mx(dxq.ptr)                                                     # (the logits stay in the net's own device buffer)
     lib.mi_sync(); LP.check()
     dt = (time.perf_counter() - t0) / steps
     # conv FLOPs of one forward, logical channels, all taps (tests/bench_lp.c:46)

@@ -31,6 +31,17 @@ typedef struct {                                                                
    z-window fields (y2, o_split, accum, sr, osr, o_pad, zw0, zw1) must be zero: a call that sets one prints a message and aborts, as the
    reference does for unsupported combinations (src/lp_f8fwd.cu:28). Slab-local GroupNorm (gnp_t.ns > 0) likewise. */
 
+/* tile masks of a masked ("skip-empty") conv (src/nn_lp.h:44): m the output tiles to compute, nullptr: dense */
+typedef struct { const uint8_t *m, *mi; int my, mx, zoff; } skipm_t;
+/* What the reference's kernel units ask its op layer before a conv (src/nn_lp.h:45-48, src/lp_common.cuh:42; defined there in
+   src/nn_skip.cu:130-157 and src/nn_bwd.cu:57). This library asks the same questions before every conv launch and refuses (message +
+   abort) a masked conv or an active z-window, which it does not build. Its own definitions are weak and answer "dense" / "no window":
+   linked into the reference, the reference's definitions take over. */
+skipm_t lp_skip_get(shape5 xs, split_t sp, int fwd);
+int nn_skip_fwd_level(shape5 xs, split_t sp);
+int nn_skip_masks(shape5 xs, split_t sp);
+int zw_win(int D, int *z0, int *z1);
+
 /* GroupNorm sum slots (src/gnacc.cuh:8-9): `osum` / `sums` buffers are arrays of 3 x uint64 fixed-point slots (24 bytes each:
    fraction in units of 2^-64, signed integer part, count of non-finite contributions), two per (sample, group): sum, sum of squares */
 #define MI_GN_SLOT_BYTES 24

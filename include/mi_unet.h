@@ -1,7 +1,7 @@
 /* Host side (C23) of the MX U-Net forward: the op layer and the graph the reference keeps above its lp_* kernels, restated over
  * the C ABI of include/mi_lp.h. Names, argument meaning and error behaviour follow the reference's own declarations:
  *   nn_set_storage / nn_storage / nn_set_prec / nn_conv3d_fwd_gn_stats / nn_conv3d_fwd_x / nn_gn_stats   src/nn.h:100, :194-195, :423-433, :484
- *   unet_cfg / unet_create / unet_init / unet_forward_x / unet_forward_ct                               src/unet.h:1-30, :141, :186, :428
+ *   unet_cfg / unet_create / unet_init / unet_forward_x / unet_forward_ct                               src/unet.h:18-128, :141, :176, :186, :428
  * Tensors are device pointers; an activation is an MX tensor registered with nn_set_storage (dt 8 / 4), as in the reference.
  */
 #ifndef MI_UNET_H
@@ -16,7 +16,8 @@ extern "C" {
 void nn_set_storage(const void *p, size_t bytes, int dt);      /* dt 8 MX-fp8, 4 MX-fp4, 2 fp16 planes, 0 forgets (fp32 planes) */
 int nn_storage(const void *p);                                 /* the dt of the registered range holding p, else 0 */
 void nn_storage_forget(const void *p);
-void nn_set_prec(int p);                                       /* 3: MX-fp4 compute for every conv, else the storage decides (src/nn_bwd.cu:110-112) */
+void nn_set_prec(int p);                                       /* 3: MX-fp4 compute for every conv, else the storage decides (src/nn.h:100, src/nn_bwd.cu:110-112) */
+int nn_get_prec(void);                                         /* src/nn.h:115 */
 void nn_set_gn_stored(int on);                                 /* GroupNorm statistics of the decoded stored output (src/nn_core.cu:7; default 0) */
 size_t nn_mx8_bytes(shape5 s);
 size_t nn_mx4_bytes(shape5 s);
@@ -34,67 +35,114 @@ void nn_set_zrange_out(int on);                                /* ... straight i
 int nn_gn_stats(const float *x, shape5 s, int G, float eps, float *mean, float *rstd);   /* of a stored MX tensor; -1 when unsupported (src/nn.h:484) */
 const char *nn_check(void);                                    /* src/nn.h:28 */
 
-/* ---- U-Net graph (src/unet.h, src/unet.c:2567-2636, :2867-3121; inference, recompute mode, no residual blocks) ---- */
+/* ---- U-Net graph (src/unet.h, src/unet.c:2567-2636, :2867-3121; inference, recompute mode) ----
+   The entry points below carry the reference's names AND signatures (src/unet.h:18-128 unet_cfg, :141 unet_create, :157 unet_free, :159-160,
+   :176, :185-187 forward, :258 unet_use_ema, :344-347 checkpoints, :357 unet_peek, :369-370 storage, :422 slabs, :428 unet_forward_ct), so a
+   caller written against src/unet.h (predict.c) links against this library unchanged. Everything this build adds is named mi_unet_*. */
 #define UNET_MAXLEV 8
+/* The reference's configuration record, field for field (src/unet.h:18-128): the layout is part of the boundary. This build runs the plain
+   U-Net (+ down_norm, + self-attention blocks with RoPE / no positional encoding and register tokens). Fields it honours: nlev, widths, cin,
+   cout, G, down_norm, attn_blocks, attn_pe (1 or 2), attn_reg, attn_mlp; dec_widths / dec_convs may repeat the defaults (widths[i] / 2);
+   half_res and scan_norm concern the caller only. Any other field must be 0: unet_create prints which one is not and returns NULL. */
 typedef struct {
-    int cin;                   /* input channels (4 for CT windows: z-scored CT, 0, radial dy, dx) */
-    int nlev;                  /* levels */
-    int widths[UNET_MAXLEV];   /* channels per level */
-    int G;                     /* GroupNorm groups (min(G, C) is used, src/unet.c:297) */
-    int head_out;              /* logits */
-    int act_dt;                /* activation storage: 8 MX-fp8, 4 MX-fp4 */
-    int prec;                  /* 3: fp4 compute everywhere (MX-fp4 weights over MX-fp8 storage), else by storage */
-    /* transformer blocks on the bottleneck level's raw output (src/unet.h:72-80; 0 = none): tokens = attn_reg learned register rows + the
-       bottleneck grid, pre-LN blocks (MHSA with QK-norm, heads of 48, SwiGLU) on the MX-fp8 attention core with MX-fp8 linears; the level's
-       output GroupNorm moves after the stage. The bottleneck width must be a multiple of 48 */
+    int nlev;
+    int widths[UNET_MAXLEV];
+    int cin, cout;
+    int G;
+    int down_norm;
+    int scale_cond;
+    int dec_widths[UNET_MAXLEV];
+    int enc_blocks[UNET_MAXLEV];
+    int dec_convs[UNET_MAXLEV];
+    int ds_levels;
+    int lat_guide;
+    int lat_nsub;
+    int8_t lat_sub[16];
+    int half_res;
+    int w4_2d;
+    int l0_norm;
+    int l0_slab;
+    int gfilm;
+    int scan_norm;
+    int gn_ema;
     int attn_blocks;
-    int attn_pe;               /* 1 axial 3-D RoPE, 2 none (0 PEG and 3 scroll RoPE are not provided) */
-    int attn_reg;              /* register tokens per sample */
-    int attn_mlp;              /* SwiGLU hidden width (0: 8/3 of the width rounded up to 32) */
-    int down_norm;             /* 1: GroupNorm + SiLU after each stride-2 down conv, applied by the next block's conv1 while it stages its input
-                                  (parameters after the head, src/unet.h:23, src/unet.c:459); 0: the older layout without it */
+    int attn_pe;
+    int attn_reg;
+    int attn_mlp;
+    int attn_vres;
+    int attn_axis;
+    int attn_repeat;
+    int attn_mem;
+    int view_P, view_patch;
+    int attn_deform, attn_dlev;
+    int attn_dco;
+    int attn_dinit;
+    int emb_lev, emb_ch;
+    int film;
+    int skip_thr, skip_margin, skip_nl;
+    int fstem, fstem_out;
+    int lat_dec, lat_dec_raw, lat_dec_ng, lat_dec_wq;
 } unet_cfg;
 typedef struct unet unet;
-unet *unet_create(const unet_cfg *cfg, shape5 in);             /* in: the window (n, cin, d, h, w); dims divisible by 2^(nlev-1) */
+unet *unet_create(const unet_cfg *cfg);                        /* src/unet.h:141; parameters allocated, activations when the first forward names a shape */
 void unet_free(unet *u);
+const unet_cfg *unet_cfg_of(const unet *u);                    /* src/unet.h:159 */
 size_t unet_nparams(const unet *u);
-void unet_init(unet *u, uint64_t seed);                        /* Kaiming normal sqrt(2 / (cin 27)), biases 0, head bias -2, gamma 1, beta 0 (src/unet.c:588-607) */
-void unet_get_params(const unet *u, float *host);              /* the flat parameter vector in unet_init's order */
-void unet_set_params(unet *u, const float *host);
-int unet_forward_x(unet *u, const void *x, float *logits);     /* x: device MX tensor (act_dt) of the input; logits: device fp32 [n][head_out][S] */
-/* the input built on the device from a uint8 CT window of one sample (src/unet.c:2858-2865, src/lp_mx_cvt.cu:29-55), then the forward */
-int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, float *logits);
-/* the same over the network's in.n windows in one forward (window n -> sample n; per-sample results equal the one-window forward's) */
-int unet_forward_ct_n(unet *u, const uint8_t *const *ct, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, float *logits);
-/* per-layer introspection for parity tests: the k-th conv output tensor (device MX) and its shape, in execution order; NULL past the end */
-const void *unet_layer_out(const unet *u, int k, shape5 *s, const char **name);
-/* the GroupNorm statistics the k-th conv produced (device [n * G] each); returns G, 0 when the layer has none */
-int unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd);
-/* ---- checkpoints in the reference's format (src/unet.c:5534-5650 unet_save, :5650-5700 read_header, :5774-5800 unet_load): one line
-   "UFSM{json}\n", then nparams fp32 weights, the EMA weights and optionally optimizer state. unet_read_header fills cfg (act_dt 8, prec 0)
-   from the header's architecture keys; it returns 0, -1 when the file is unreadable, or -2 naming (stderr) a feature of the checkpoint this
-   build does not run (decoder widths, residual blocks, latent grids, deep supervision, FiLM, fine stems, running-statistics norms, the
-   attention stage's other forms). unet_load / unet_load_ema copy the weights / the EMA weights into a net of the same architecture
-   (checked: nlev, widths, cin, cout, attention blocks, nparams, payload size); unet_save writes weights and EMA (= the weights). ---- */
-int unet_read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step);
-int unet_load(unet *u, const char *path);
-int unet_load_ema(unet *u, const char *path);
-int unet_save(const unet *u, const char *path, int step, const char *extra);   /* extra: a JSON object for the header's "extra" key, or null */
+void unet_init(unet *u, uint64_t seed);                        /* Kaiming normal sqrt(2 / (cin 27)), biases 0, head bias -2, gamma 1, beta 0 (src/unet.c:588-607); the EMA copy = the weights */
+float *unet_param_ptr(unet *u);                                /* device pointers of the flat fp32 weights and of their EMA copy (src/unet.h:203-204), unet_init's order */
+float *unet_ema_ptr(unet *u);
+void unet_use_ema(unet *u, int on);                            /* forward with the EMA weights (1) or the live ones (0) (src/unet.h:258) */
+/* activation storage of the networks built from now on (src/unet.h:369-370): MX-fp8 (the default here; this build has no 16-bit storage, so
+   unet_set_act_mx8(0) without mx4 is refused at the next forward) or packed MX-fp4, which takes precedence. The compute precision follows the
+   op layer's policy (nn_set_prec(3): MX-fp4 weights over either storage). A change rebuilds the activations at the next forward. */
+void unet_set_act_mx8(int on);
+void unet_set_act_mx4(int on);
+int unet_act_mx(void);                                         /* src/unet.h:430 */
+/* Forward for one input shape xs = (n, cin, d, h, w), dims divisible by 2^(nlev-1); activation buffers are (re)allocated when the shape or
+   the storage mode changes. train must be 0 (inference build: 1 aborts with a message). Returns the logits, fp32 [n][cout][d][h][w] on the
+   device, owned by the net and valid until its next forward (src/unet.h:183-187). x: fp32 planes [n][cin][d][h][w]; unet_forward_x with
+   x_h16: fp16 planes, read in place. Either is converted to the MX input tensor first (lp_f32_to_mx* / lp_h16_to_mx*, src/unet.c:2909-2919). */
+const float *unet_forward(unet *u, const float *x, shape5 xs, int train);
+const float *unet_forward_x(unet *u, const void *x, shape5 xs, int train, int x_h16);
+shape5 unet_out_shape(const unet *u, shape5 xs);
+/* the input built on the device from the uint8 CT window(s) (src/unet.h:428, src/unet.c:2858-2865, src/lp_mx_cvt.cu:29-55), then the forward.
+   ct: xs.n windows of d x h x w voxels back to back (the reference's predict passes one); dyo / dxo: per window plane the row / column offset
+   from the scroll axis, xs.d floats per window back to back; h16: the 16-bit type the input values are rounded to (2 fp16, 1 bf16, 0 none).
+   xs.c must be 4 and xs.h == xs.w. */
+const float *unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, shape5 xs, int h16);
 void unet_set_infer_slab(int planes);                         /* inference: the level-0 convs in z-slabs of this many planes (rounded up to a multiple of 4), each slab written
                                                                  straight into the full-depth tensors; byte-identical logits; 0 = off (src/unet.h:422-424, direct slab outputs) */
-int unet_get_infer_slab(void);
-shape5 unet_in_shape(const unet *u);                          /* the window the graph was created for */
-const unet_cfg *unet_config(const unet *u);
+/* ---- checkpoints in the reference's format (src/unet.h:342-357; src/unet.c:5534-5650 unet_save, :5650-5755 header, :5774-5800 unet_load): one
+   line "UFSM{json}\n", then nparams fp32 weights, the EMA weights and optionally optimizer state (skipped here). unet_peek fills cfg and step
+   from the header: 0, -1 when the file is unreadable, -2 naming (stderr) a feature of the checkpoint this build does not run. unet_load copies
+   weights and EMA weights into a net of the same architecture (checked: nlev, widths, cin, cout, attention blocks, down_norm, nparams,
+   payload size) and returns the saved step, or -1. unet_save writes weights and EMA. ---- */
+int unet_peek(const char *path, unet_cfg *cfg, int *step);
+int unet_load(unet *u, const char *path);
+int unet_save(const unet *u, const char *path, int step, const char *extra_json);
+/* ---- additions of this build (no counterpart in src/unet.h) ---- */
+void mi_unet_get_params(const unet *u, float *host);           /* the live weights, flat, unet_init's order */
+void mi_unet_set_params(unet *u, const float *host);           /* ... and the EMA copy with them; drops the prepared-weight memos */
+/* the forward on an input that already is the net's MX tensor (lp_f32_to_mx* output or lp_pred_input_mx rows), device pointer */
+const float *mi_unet_forward_mx(unet *u, const void *xmx, shape5 xs);
+/* unet_forward_ct with the windows and their offset rows given one pointer each (window n -> sample n; windows of a batch need not be contiguous) */
+const float *mi_unet_forward_ct_n(unet *u, const uint8_t *const *ct, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, shape5 xs, int h16);
+/* per-layer introspection for parity tests: the k-th conv output tensor of the last forward (device MX) and its shape, in execution order; NULL past the end */
+const void *mi_unet_layer_out(const unet *u, int k, shape5 *s, const char **name);
+/* the GroupNorm statistics the k-th conv produced (device [n * G] each); returns G, 0 when the layer has none */
+int mi_unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd);
+int mi_unet_infer_slab(void);                                  /* unet_set_infer_slab's current value */
+size_t mi_unet_peek_nparams(const char *path);                 /* the header's "nparams" (0: unreadable) */
 /* ---- sliding-window prediction of a volume resident in device memory (src/predict.c: the --feather single pass, :282-333, :2538-2545,
-   :3420-3436). vol: uint8 CT [dims0][dims1][dims2]; windows of the graph's size (cubic; the graph's in.n samples are that many windows per forward) with
-   `halo` voxels of context per side tile the volume at stride window - 2 halo in z-y-x order; each runs as a sample of unet_forward_ct_n (z-score mean / isd; axis, cy, cx: the scroll axis
+   :3420-3436). vol: uint8 CT [dims0][dims1][dims2]; cubic windows of `window` voxels, `nbatch` (1 .. 16) per forward, with
+   `halo` voxels of context per side tile the volume at stride window - 2 halo in z-y-x order; each runs as a sample of unet_forward_ct (z-score mean / isd; axis, cy, cx: the scroll axis
    sign and its centre in volume y / x, axis 0: no direction channels) and places uint8(255 sigmoid(logit 0) + .5) where CT >= the
    prediction iso over its interior plus `feather` voxels of its upper halo; the window borders are then blended over `feather` voxels
    (0: none; <= halo) into out: uint8 [dims0][dims1][dims2]. Windows whose CT holds no voxel >= iso are skipped (their interior stays 0
    and their neighbours' blends renormalise). nwin[0..1] (may be null): windows in all, windows computed. Returns 0, or -1 for a
    geometry the graph cannot run. Every window's prediction stays in device memory until the blend: nwin (stride + feather)^3 bytes. */
-int unet_predict_volume(unet *u, const uint8_t *vol, const int64_t dims[3], int halo, int feather, float mean, float isd,
-                        int axis, float cy, float cx, uint8_t *out, int64_t nwin[2]);
+int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, const int64_t dims[3], int halo, int feather, float mean, float isd,
+                           int axis, float cy, float cx, uint8_t *out, int64_t nwin[2]);
 #ifdef __cplusplus
 }
 #endif

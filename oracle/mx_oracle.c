@@ -241,11 +241,24 @@ void orc_prep_w(int bits, const float *w, int Co, int Ci, int Cx, int CxP, int C
     }
 }
 
+/* a third summation order for drift studies (acc64 == 2): fp32 accumulation whose every add is rounded toward zero, as a datapath that
+   aligns and truncates its addends does. A legitimate fp32-accumulated result, within one ulp per add of the other two. */
+static float add_chop(float acc, double blk) {
+    const double t = (double)acc + blk; float f = (float)t;
+    if (isfinite(f) && fabs((double)f) > fabs(t)) f = nextafterf(f, 0.f);
+    return f;
+}
+/* 0 (default): the exact u sigmoid(u), correctly rounded; 1: the same function evaluated in fp32 by a fast path (product with the fp32
+   reciprocal of 1 + expf(-u): a few ulp off), the kind of evaluation a GPU makes. For drift studies only. */
+static int g_act_mode = 0, g_align_bits = 24;
+void orc_set_act_mode(int m) { g_act_mode = m; }
+void orc_set_align_bits(int b) { g_align_bits = b; }   /* width of the acc64 == 3 adder below its largest addend's leading bit */
 /* ---------- GN + SiLU of the conv staging (src/lp_common.cuh:258, :474-482): u = fma(x, a, b), h = u / 2, h + h tanh(h) ---------- */
 float orc_act_ab(float v, float a, float b) {
     /* the reference's h + h tanh(h), h = u / 2, is u sigmoid(u); its tanh is NVIDIA's tanh.approx (about 2^-11), so the oracle takes
        the exact value of the same function, correctly rounded: any faithful evaluation is inside the reference's own error */
     const float u = fmaf(v, a, b);
+    if (g_act_mode == 1) { const float d = 1.f + expf(-u), r = 1.f / d; return u * r; }
     return (float)((double)u / (1.0 + exp(-(double)u)));
 }
 static void gn_ab(const orc_gn_t *g, int n, int cc, int Cg, float *a, float *b) {
@@ -393,7 +406,7 @@ static void conv_epilogue(const orc_conv_t *c, int n, size_t ov, size_t So, floa
     uint8_t *yq = (uint8_t *)c->y, *ysc = yq + (size_t)c->N * ynb * So * yrb;
     /* epilogue (src/lp_common.cuh:1492-1535) */
     for (int co = 0; co < Co; co++) {
-        float v = c->acc64 ? (float)(acc64[co] + (c->b ? (double)c->b[co] : 0.0)) : acc[co] + (c->b ? c->b[co] : 0.f);
+        float v = c->acc64 == 1 ? (float)(acc64[co] + (c->b ? (double)c->b[co] : 0.0)) : acc[co] + (c->b ? c->b[co] : 0.f);
         if (c->fused_act) {
             if (c->ep_a) v = fmaf(v, c->ep_a[co], c->ep_b[co]);
             v = c->fused_act == 1 ? silu_f(v) : c->fused_act == 2 ? gelu_f(v) : c->fused_act == 3 ? fmaxf(v, 0.f) : v;
@@ -497,7 +510,7 @@ static int conv3_stem(const orc_conv_t *c) {
                                 d += (double)wr[k] * (double)bq[p * CP + k % CP]; row = p / 18;
                             }
                             const double blk = d * (double)wsf[(size_t)kb * Co + co] * rsf[row];     /* (a block's positions share the row, or the tile, scale) */
-                            if (c->acc64) acc64[co] += blk; else acc[co] += (float)blk;
+                            if (c->acc64 == 1) acc64[co] += blk; else if (c->acc64 == 2) acc[co] = add_chop(acc[co], blk); else acc[co] += (float)blk;
                         }
                     conv_epilogue(c, n, ((size_t)oz * H + oy) * W + ox, S, acc, acc64, ls);
                 }
@@ -554,7 +567,20 @@ int orc_conv3(const orc_conv_t *c) {
                             double d = 0.0;                              /* exact: products of code values, 32 terms */
                             for (int k = 0; k < 32; k++) d += (double)wr[k] * (double)xv[k];
                             const double blk = d * (double)wsf[((size_t)t * Co + co) * nch + ch] * (double)xs;
-                            if (c->acc64) acc64[co] += blk; else acc[co] += (float)blk;
+                            if (c->acc64 == 3) {                        /* drift studies: an adder that aligns the block's products and the running sum to the
+                                                                           largest exponent among them and drops what falls below g_align_bits bits of it */
+                                const double sc = (double)wsf[((size_t)t * Co + co) * nch + ch] * (double)xs;
+                                double mx = fabs((double)acc[co]);
+                                for (int k = 0; k < 32; k++) { const double pk = fabs((double)wr[k] * (double)xv[k] * sc); if (pk > mx) mx = pk; }
+                                if (mx > 0 && isfinite(mx)) {
+                                    int ex; (void)frexp(mx, &ex);
+                                    const double q = ldexp(1.0, ex - g_align_bits);
+                                    double tsum = trunc((double)acc[co] / q);
+                                    for (int k = 0; k < 32; k++) tsum += trunc((double)wr[k] * (double)xv[k] * sc / q);
+                                    acc[co] = add_chop(0.f, tsum * q);
+                                } else acc[co] += (float)blk;
+                            } else
+                            if (c->acc64 == 1) acc64[co] += blk; else if (c->acc64 == 2) acc[co] = add_chop(acc[co], blk); else acc[co] += (float)blk;
                         }
                     }
                 conv_epilogue(c, n, (size_t)vi, So, acc, acc64, ls);

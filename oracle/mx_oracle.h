@@ -94,7 +94,7 @@ typedef struct {
     /* output */
     void *y; int ydt;                  /* 0 fp32 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4 */
     double *osum; int Go; int stored_stats;   /* plain doubles [N][Go][2] (sum, sum of squares), accumulated */
-    int acc64;                         /* 1: accumulate in fp64 (exact-operand checks) */
+    int acc64;                         /* 1: accumulate in fp64 (exact-operand checks); 2: fp32 with every add rounded toward zero, 3: an aligning, truncating block adder (drift studies) */
     int fused_act; const float *ep_a, *ep_b;   /* extension: epilogue affine + activation (1 SiLU, 2 GELU, 3 ReLU) before requant */
     int z0, z1;                        /* output z planes [z0, z1) only (z1 0: all): the bounded CPU-baseline slab */
     int stem_tile;                     /* 1: one activation scale per staged 4x10x18 tile (Ci <= 8 tap-packed stem); 2: 9 .. 16 channels, two taps per K
@@ -134,6 +134,8 @@ int orc_block_fwd(int bits, int C, int H, int F, int rope, int nreg, float rope_
 void orc_pred_place(const float *lg, const uint8_t *ct, int D, int W, int hz, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, int iso, uint8_t *dsh);
 void orc_feather_blend(const uint8_t *E, const uint8_t *present, int S, int B, const int64_t nss[3], const int64_t bn[3], uint8_t *out);
 float orc_act_ab(float v, float a, float b);
+void orc_set_align_bits(int b);         /* drift studies: width of the acc64 == 3 adder (default 24) */
+void orc_set_act_mode(int m);          /* drift studies: 1 evaluates the activation by a fast fp32 path (a few ulp off), 0 (default) exactly */
 uint16_t orc_f32_to_h16(float f);
 float orc_h16_to_f32(uint16_t h);
 int orc_threads(void);

@@ -60,6 +60,8 @@ def lib():
         L.orc_f32_to_h16.restype = C.c_uint16; L.orc_f32_to_h16.argtypes = [C.c_float]
         L.orc_h16_to_f32.restype = C.c_float; L.orc_h16_to_f32.argtypes = [C.c_uint16]
         L.orc_threads.restype = C.c_int
+        L.orc_set_align_bits.restype = None; L.orc_set_align_bits.argtypes = [C.c_int]
+        L.orc_set_act_mode.restype = None; L.orc_set_act_mode.argtypes = [C.c_int]
         L.orc_mx_gemm.restype = C.c_int
         L.orc_mx_gemm.argtypes = [C.c_int] * 6 + [C.c_void_p, C.c_void_p, C.c_void_p, C.c_float, C.c_void_p, C.c_void_p]
         L.orc_pred_place.restype = None; L.orc_pred_place.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 12 + [C.c_void_p]

@@ -9,9 +9,9 @@ def read(tmp_path, header, payload=b""):
     H = load_host()
     p = tmp_path / "h.ckpt"
     p.write_bytes(header.encode() + payload)
-    cfg = unet_cfg(); n = C.c_size_t(0); step = C.c_int(0)
-    rc = H.unet_read_header(str(p).encode(), C.byref(cfg), C.byref(n), C.byref(step))
-    return rc, cfg, n.value, step.value
+    cfg = unet_cfg(); step = C.c_int(0)
+    rc = H.unet_peek(str(p).encode(), C.byref(cfg), C.byref(step))
+    return rc, cfg, H.mi_unet_peek_nparams(str(p).encode()), step.value
 
 
 def test_reads_the_reference_header(tmp_path):
@@ -19,7 +19,7 @@ def test_reads_the_reference_header(tmp_path):
     h = ('UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":287937,"step":1,"sparse24":0,"wq":0,"muon_mom":0,'
          '"extra":{"runtime":{"version":1,"train_window":96,"prec":1,"f16":1,"act_mx4":0,"act_mx8":1,"grad_mx8":1,"input_mx":1,"input_prec":8,"gn_stored":0,"policy":"","optimizer":"muon"}}}\n')
     rc, cfg, n, step = read(tmp_path, h)
-    assert rc == 0 and (cfg.nlev, cfg.widths[0], cfg.widths[1], cfg.cin, cfg.head_out, cfg.G, cfg.down_norm, cfg.attn_blocks, cfg.act_dt) == (2, 32, 64, 4, 1, 8, 1, 0, 8)
+    assert rc == 0 and (cfg.nlev, cfg.widths[0], cfg.widths[1], cfg.cin, cfg.cout, cfg.G, cfg.down_norm, cfg.attn_blocks, cfg.half_res) == (2, 32, 64, 4, 1, 8, 1, 0, 0)
     assert n == 287937 and step == 1
 
 
@@ -30,7 +30,14 @@ def test_attention_keys_and_extra_shadowing(tmp_path):
     assert rc == 0 and (cfg.nlev, cfg.widths[3], cfg.attn_blocks, cfg.attn_pe, cfg.attn_reg, cfg.attn_mlp) == (4, 192, 2, 1, 4, 512) and step == 77
 
 
-@pytest.mark.parametrize("feature", ['"dec_widths":[0,32]', '"half_res":1', '"ds_levels":2', '"film":2', '"fstem":[2,16]', '"gn_ema":1,"ge_n":5', '"attn_vres":1', '"l0_norm":2'])
+def test_caller_side_keys_pass_through(tmp_path):
+    # half-resolution windows and per-scan normalisation are transforms the caller applies around the forward (src/unet.h:52-56, :88-89): no refusal
+    h = 'UFSM{"nlev":2,"widths":[32,64],"half_res":1,"scan_norm":1,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":1,"extra":{}}\n'
+    rc, cfg, n, step = read(tmp_path, h)
+    assert rc == 0 and cfg.half_res == 1 and cfg.scan_norm == 1
+
+
+@pytest.mark.parametrize("feature", ['"dec_widths":[0,32]', '"enc_blocks":[0,1]', '"ds_levels":2', '"film":2', '"fstem":[2,16]', '"gn_ema":1,"ge_n":5', '"attn_vres":1', '"l0_norm":2'])
 def test_refuses_architectures_it_does_not_run(tmp_path, feature):
     h = 'UFSM{"nlev":2,"widths":[32,64],%s,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":1,"extra":{}}\n' % feature
     assert read(tmp_path, h)[0] == -2

@@ -200,7 +200,7 @@ def test_unet_attention_stage(gpu):
 
 
 def test_checkpoint_round_trip(gpu, tmp_path):
-    """unet_save -> unet_read_header -> unet_create -> unet_load gives the same network: identical parameters and byte-identical logits;
+    """unet_save -> unet_peek -> unet_create -> unet_load gives the same network: identical parameters and byte-identical logits;
     a network of another architecture, a truncated payload and a checkpoint of an unsupported feature are refused (src/unet.c:5774-5800)."""
     import ctypes as C
     from ufsm_amd.unet import UNet, make_cfg, unet_cfg, load_host
@@ -217,12 +217,12 @@ def test_checkpoint_round_trip(gpu, tmp_path):
     assert head.rstrip().endswith('}}}')
     import os
     assert os.path.getsize(path) == len(head.encode()) + 2 * 4 * pa.size                     # weights + EMA weights
-    c2 = unet_cfg(); npar = C.c_size_t(0); step = C.c_int(0)
-    assert H_.unet_read_header(path.encode(), C.byref(c2), C.byref(npar), C.byref(step)) == 0
-    assert (c2.nlev, list(c2.widths[:2]), c2.cin, c2.head_out, c2.G, c2.down_norm, c2.attn_blocks, c2.attn_pe, c2.attn_reg, c2.attn_mlp) == (2, [32, 96], 4, 3, 8, 1, 1, 1, 2, 256)
-    assert npar.value == pa.size and step.value == 123
+    c2 = unet_cfg(); step = C.c_int(0)
+    assert H_.unet_peek(path.encode(), C.byref(c2), C.byref(step)) == 0
+    assert (c2.nlev, list(c2.widths[:2]), c2.cin, c2.cout, c2.G, c2.down_norm, c2.attn_blocks, c2.attn_pe, c2.attn_reg, c2.attn_mlp) == (2, [32, 96], 4, 3, 8, 1, 1, 1, 2, 256)
+    assert H_.mi_unet_peek_nparams(path.encode()) == pa.size and step.value == 123
     b = UNet(c2, N, D, D, D, seed=1)
-    assert b.load(path) == 0 and np.array_equal(b.params(), pa) and b.load(path, ema=True) == 0
+    assert b.load(path) == 123 and np.array_equal(b.params(), pa)                          # the saved step (src/unet.h:345-347)
     x = rng.standard_normal((N, 4, S)).astype(np.float32); dxq = to_mx(8, x)
     la, lb = DevBuf(N * 3 * S * 4), DevBuf(N * 3 * S * 4)
     assert a.forward_x(dxq.ptr, la.ptr) == 0 and b.forward_x(dxq.ptr, lb.ptr) == 0
@@ -233,8 +233,67 @@ def test_checkpoint_round_trip(gpu, tmp_path):
     open(str(tmp_path / "cut.ckpt"), "wb").write(open(path, "rb").read()[:-8])
     assert b.load(str(tmp_path / "cut.ckpt")) == -1
     open(str(tmp_path / "film.ckpt"), "wb").write(head.replace(',"cin":', ',"film":2,"cin":').encode() + b"\0" * (8 * pa.size))
-    assert H_.unet_read_header(str(tmp_path / "film.ckpt").encode(), C.byref(c2), None, None) == -2
+    assert H_.unet_peek(str(tmp_path / "film.ckpt").encode(), C.byref(c2), None) == -2
+    # the EMA copy (src/unet.h:258): a file whose second array differs loads into the EMA weights, which unet_use_ema switches the forward to
+    raw = open(path, "rb").read(); hl = len(head.encode())
+    ema = (pa * np.float32(0.5)).astype(np.float32)
+    open(str(tmp_path / "ema.ckpt"), "wb").write(raw[:hl + 4 * pa.size] + ema.tobytes())
+    assert b.load(str(tmp_path / "ema.ckpt")) == 123 and np.array_equal(b.params(), pa)
+    he = np.empty(pa.size, np.float32); lib.mi_d2h(he.ctypes.data, H_.unet_ema_ptr(b.h), he.nbytes)
+    assert np.array_equal(he, ema)
+    b.use_ema(True)
+    assert b.forward_x(dxq.ptr, lb.ptr) == 0
+    assert not np.array_equal(la.to_numpy(np.float32), lb.to_numpy(np.float32))
+    b.use_ema(False)
+    assert b.forward_x(dxq.ptr, lb.ptr) == 0 and np.array_equal(la.to_numpy(np.float32), lb.to_numpy(np.float32))
     a.close(); b.close(); other.close()
+
+
+def test_reference_signature_forwards(gpu):
+    """unet_forward / unet_forward_x / unet_forward_ct as src/unet.h:176, :186, :428 declare them: fp32 or fp16 planes (or the CT window) in, the
+    net's own logits out, activations built lazily for the shape named by the call and rebuilt when it changes; each equals the forward on
+    the MX tensor the matching converter makes of the same input."""
+    import ctypes as C
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    H_ = load_host()
+    rng = np.random.default_rng(33)
+    net = UNet(make_cfg(4, [32, 64], head_out=3), 1, 8, 16, 16, seed=4)
+    for (N, D, H, W) in [(1, 8, 16, 16), (2, 4, 8, 8)]:                      # the second call changes the shape: rebuilt, no stale buffers
+        S = D * H * W
+        xs = shape5(N, 4, D, H, W)
+        x = rng.standard_normal((N, 4, S)).astype(np.float32)
+        dx = DevBuf.from_numpy(x); dxh = DevBuf.from_numpy(x.astype(np.float16))
+        o = H_.unet_out_shape(net.h, xs)
+        assert (o.n, o.c, o.d, o.h, o.w) == (N, 3, D, H, W)
+        nbytes = N * 3 * S * 4
+        def fetch(p):
+            assert p
+            out = np.empty(N * 3 * S, np.float32); lib.mi_sync(); lib.mi_d2h(out.ctypes.data, p, nbytes); return out
+        l32 = fetch(H_.unet_forward(net.h, dx.ptr, xs, 0))
+        l32x = fetch(H_.unet_forward_x(net.h, dx.ptr, xs, 0, 0))
+        l16 = fetch(H_.unet_forward_x(net.h, dxh.ptr, xs, 0, 1))
+        want32 = fetch(H_.mi_unet_forward_mx(net.h, to_mx(8, x).ptr, xs))
+        want16 = fetch(H_.mi_unet_forward_mx(net.h, to_mx(8, x.astype(np.float16).astype(np.float32)).ptr, xs))
+        LP.check()
+        assert np.array_equal(l32, want32) and np.array_equal(l32x, want32) and np.array_equal(l16, want16)
+    # the CT window form, two windows in one call: rows of window n from ct + n W^3 and offsets dyo + n D
+    Wd = 16; xs = shape5(2, 4, Wd, Wd, Wd); S = Wd ** 3
+    ct = rng.integers(0, 255, (2, Wd, Wd, Wd)).astype(np.uint8)
+    dyo = rng.uniform(-40, -20, (2, Wd)).astype(np.float32); dxo = rng.uniform(20, 40, (2, Wd)).astype(np.float32)
+    dct, ddy, ddx = DevBuf.from_numpy(ct), DevBuf.from_numpy(dyo), DevBuf.from_numpy(dxo)
+    p = H_.unet_forward_ct(net.h, dct.ptr, 120.0, 1 / 50.0, ddy.ptr, ddx.ptr, 1, xs, 2)
+    assert p
+    got = np.empty(2 * 3 * S, np.float32); lib.mi_sync(); lib.mi_d2h(got.ctypes.data, p, got.nbytes)
+    xin = DevBuf(lib.lp_mx8_bytes(2, 4, S))
+    for n in range(2):
+        lib.mi_pred_input_mx_n(dct.ptr + n * S, Wd, 120.0, 1 / 50.0, ddy.ptr + 4 * Wd * n, ddx.ptr + 4 * Wd * n, 1, 0, Wd, xin.ptr, 2, 8, 2, n)
+    want = np.empty_like(got); q = H_.mi_unet_forward_mx(net.h, xin.ptr, xs); lib.mi_sync(); lib.mi_d2h(want.ctypes.data, q, want.nbytes)
+    LP.check()
+    assert np.array_equal(got, want)
+    # a configuration field this build does not run is refused by name, not ignored
+    bad = make_cfg(4, [32, 64]); bad.film = 2
+    assert not H_.unet_create(C.byref(bad))
+    net.close()
 
 
 @pytest.mark.parametrize("bits,dims,slab,attn", [(8, (32, 32, 32), 8, 0), (8, (24, 16, 32), 16, 0), (4, (16, 32, 32), 4, 0), (8, (32, 32, 32), 16, 1)])
@@ -251,7 +310,7 @@ def test_slab_inference_is_byte_identical(gpu, bits, dims, slab, attn):
     net = UNet(make_cfg(4, widths, G=8, head_out=3, act_dt=bits, attn_blocks=attn, attn_pe=1, down_norm=1), N, D, H, W, seed=5)
     x = rng.standard_normal((N, 4, S)).astype(np.float32); dxq = to_mx(bits, x)
     la, lb = DevBuf(N * 3 * S * 4), DevBuf(N * 3 * S * 4)
-    assert H_.unet_get_infer_slab() == 0
+    assert H_.mi_unet_infer_slab() == 0
     assert net.forward_x(dxq.ptr, la.ptr) == 0
     LP.check()
     def fetch():
@@ -269,7 +328,7 @@ def test_slab_inference_is_byte_identical(gpu, bits, dims, slab, attn):
     assert {"enc0.c1", "enc0.c2", "dec0.c1", "dec0.c2"} <= set(whole)
     H_.unet_set_infer_slab(slab - 1)                       # rounded up to a multiple of 4
     try:
-        assert H_.unet_get_infer_slab() == slab
+        assert H_.mi_unet_infer_slab() == slab
         assert net.forward_x(dxq.ptr, lb.ptr) == 0
         LP.check()
     finally:

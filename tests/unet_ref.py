@@ -33,8 +33,9 @@ def param_layout(cin, widths, head_out, down_norm=0):
     return lay, off
 
 
-def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0):
-    """xq: MX bytes of the input. Returns (logits fp32 [N][head_out][S], {layer name: MX bytes})."""
+def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0, acc64=0):
+    """xq: MX bytes of the input. Returns (logits fp32 [N][head_out][S], {layer name: MX bytes}). acc64: the convs' contraction summed in
+    double and rounded once (else in fp32, block by block): two correct summation orders of the same graph."""
     lay, n = param_layout(cin, widths, head_out, down_norm)
     assert params.size == n
     P = lambda k: np.ascontiguousarray(params[lay[k][0]:lay[k][0] + int(np.prod(lay[k][1]))].reshape(lay[k][1]))
@@ -55,7 +56,7 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
         if stride == 2:                       # the reference's stride-2 dispatch: fp4 only for an MX-fp4 32 -> <= 32 channel conv (src/lp_s2.cu:653-671)
             cb = 4 if (bits == 4 and ci == 32 and co <= 32) else 8
         y, s = orc.conv3(x, dt, N, ci, d[0], d[1], d[2], P(name + ".w"), P(name + ".b"), co, dt, cbits=cb, stride=stride, x2=x2, c_split=c_split, up=up,
-                         gp=gp, gp2=gp2, Go=Gof(co), want_stats=stats, stored_stats=stored,
+                         gp=gp, gp2=gp2, Go=Gof(co), want_stats=stats, stored_stats=stored, acc64=acc64,
                          stem_tile=int(ci <= 8 and stride == 1 and x2 is None))   # the network input: tap-packed kernel, one scale per tile (src/lp_f8fwd.cuh:601-609)
         outs[name] = y
         return y, s

@@ -46,13 +46,14 @@ __global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int 
     if (threadIdx.x == 0) gn_part_finish(osum, r1[0], r2[0], fin);
 }
 
-// the same from per-channel records (32 per tile, one channel tile per workgroup)
-__global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, int tiles_per_n, int Co, int Go, double *osum, gn_fin_t fin) {
-    const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, cpg = Co / Go;
+// the same from per-channel records (32 per tile: launches whose channels per group are not a multiple of 4 run one channel tile per workgroup,
+// ncs channel slices of 32 per spatial tile)
+__global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, int tiles_per_n, int ncs, int Co, int Go, double *osum, gn_fin_t fin) {
+    const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, cpg = Co / Go, nst = tiles_per_n / ncs;
     double s = 0.0, ss = 0.0;
-    for (int i = threadIdx.x; i < tiles_per_n * cpg; i += 256) {
-        const int t = i / cpg, ch = gidx * cpg + i % cpg;
-        const float2 p = part[(size_t)(n * tiles_per_n + t) * 32 + ch];
+    for (int i = threadIdx.x; i < nst * cpg; i += 256) {
+        const int st = i / cpg, ch = gidx * cpg + i % cpg;
+        const float2 p = part[((size_t)n * tiles_per_n + (size_t)st * ncs + (ch >> 5)) * 32 + (ch & 31)];
         s += (double)p.x; ss += (double)p.y;
     }
     __shared__ double r1[256], r2[256];
@@ -165,7 +166,7 @@ static void conv_stats_reduce(const char *who, const conv_args &a, int MT, split
     gn_fin_t fin = g_fin;
     fin.len = (double)(a.Co / a.Go) * (double)a.Do * a.Ho * a.Wo;
     if (fin.mean && (sp.zlo || sp.zhi)) mi_die("%s: fused finalize with a z range", who);
-    if (a.stat_ch) gn_part_reduce_ch_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.Co, a.Go, osum, fin);
+    if (a.stat_ch) gn_part_reduce_ch_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.ncs, a.Co, a.Go, osum, fin);
     else gn_part_reduce_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.ncs, MT, a.Co, a.Go, osum, fin);
     MICK();
 }
@@ -184,7 +185,8 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     a.zi0 = sp.Di ? sp.zi0 : 0; a.yD = sp.yD; a.yzo = sp.yD ? sp.yzo : 0;
     a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
     a.osum = osum; a.Go = Go; a.stored_stats = sp.stored_stats && ybf >= 3; a.zs0 = sp.zlo; a.zs1 = Do - sp.zhi;
-    const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 && CP && CP < 16 ? 2 : 1;     // (16 channels per slot: 7 or 9 weight fragment pairs per channel tile, one tile fits the registers)
+    // (16 channels per slot: 7 or 9 weight fragment pairs per channel tile, one tile fits the registers; per-channel statistics records: one tile per workgroup)
+    const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 && CP && CP < 16 && !(osum && (cout / Go) % 4) ? 2 : 1;
     size_t smem = rows ? (size_t)720 * 16 + 16 + 40 * 4 + 16 * 8 : ((size_t)720 * CP + 16 + CP * 8 + 15) & ~(size_t)15;     // staged tile, (zero row, row words | amax word), channel affine
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);
     a.red_o = (unsigned)smem; smem += 1024;
@@ -233,6 +235,9 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if ((sp.Di || sp.zi0) && (stride != 1 || sp.zi0 < 0 || sp.zi0 + xs.d > sp.Di)) mi_die("%s: z-range %d + %d of depth %d (stride %d)", who, sp.zi0, xs.d, sp.Di, stride);
     if ((sp.yD || sp.yzo) && (stride != 1 || sp.yzo < 0 || sp.yzo + xs.d > sp.yD)) mi_die("%s: slab output %d + %d of depth %d (stride %d)", who, sp.yzo, xs.d, sp.yD, stride);
     if (gp.ns || sp.gp2.ns) mi_die("%s: slab-local GroupNorm statistics are not supported", who);
+    // the op layer's masks and z-window (the reference's kernels ask the same before a launch: src/lp_f4fwd.cuh:1134-1223, src/nn_bwd.cu:89)
+    { int za = 0, zb = 0; if (zw_win(xs.d, &za, &zb)) mi_die("%s: a z-window [%d, %d) is set; windows are not built here (inference forward only)", who, za, zb); }
+    if (lp_skip_get(xs, sp, 1).m || nn_skip_masks(xs, sp)) mi_die("%s: the op layer asks for a masked (skip-empty) conv, which is not built here", who);
     if (xbf < 0 || xbf > 4 || !(ybf == 0 || ybf == 2 || ybf == 3 || ybf == 4)) mi_die("%s: unsupported storage types (in %d, out %d)", who, xbf, ybf);
     if (xs.n <= 0 || xs.c <= 0 || xs.d <= 0 || xs.h <= 0 || xs.w <= 0 || cout <= 0) return 0;
     const int Ci = xs.c, Cx = sp.x2 ? sp.c_split : Ci, C2 = Ci - Cx;
@@ -241,7 +246,6 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (sp.x2 && xbf < 3) mi_die("%s: split inputs need MX storage", who);
     if (sp.up && (!sp.x2 || xbf < 3 || ((sp.Di ? sp.Di : xs.d) & 1) || (xs.h & 1) || (xs.w & 1) || stride != 1)) mi_die("%s: the fused upsample needs an MX split input and even dims", who);
     if (osum && (Go <= 0 || cout % Go)) mi_die("%s: %d output channels in %d groups", who, cout, Go);
-    if (osum && (cout / Go) % 4 && cout > 32) mi_die("%s: fused output statistics of %d channels need channels per group (%d) to be a multiple of 4", who, cout, cout / Go);
     if (gp.G > 0 && ((sp.x2 && sp.gp2.G ? Cx : Ci) % gp.G)) mi_die("%s: GroupNorm groups %d do not divide the channels", who, gp.G);
     if (sp.gp2.G > 0 && (!sp.x2 || C2 % sp.gp2.G)) mi_die("%s: second GroupNorm without a matching x2 segment", who);
     // few input channels: the tap-packed kernel with one activation scale per tile (src/lp_f8fwd.cuh:601-609: up to 8 channels of a 16-bit or
@@ -294,6 +298,8 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // ---- tile shape: MT channel tiles of 32 per workgroup, NT voxel tiles of 32 per wavefront, MT * NT <= 8 accumulators ----
     const int nmt_all = (cout + 31) / 32;
     int MT = nmt_all <= 4 ? nmt_all : nmt_all % 4 == 0 ? 4 : nmt_all % 3 == 0 ? 3 : nmt_all % 2 == 0 ? 2 : 1;
+    // channels per group not a multiple of 4 (80 channels in 8 groups): the statistics are per-channel records of one channel tile per workgroup
+    if (osum && (cout / Go) % 4) MT = 1;
     bool halved = false;
     {   // few tiles of 128 channels (the coarse levels): slices of 64 channels double the workgroups of the wide kernel
         static int split_env = -1;

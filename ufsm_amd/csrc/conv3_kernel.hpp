@@ -95,7 +95,7 @@ struct conv_args {
     const float *bias; int Co;
     void *y; int ydt;
     double *osum; float *part; int Go, stored_stats, zs0, zs1;   // part: per tile and channel quad (sum, sum of squares)
-    int stat_ch;                       // 1: per-channel records (channels per group not a multiple of 4; Co <= 32 only)
+    int stat_ch;                       // 1: per-channel records, 32 per tile (channels per group not a multiple of 4; one channel tile per workgroup)
     const float *ep_a, *ep_b; int act;
     unsigned epi_o;                    // LDS byte offset of the epilogue's per-channel constants: bias, then ep_a, ep_b (MT x 32 floats each)
     unsigned red_o;                    // LDS byte offset of the statistics scratch (1 KiB)

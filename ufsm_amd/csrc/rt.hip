@@ -99,3 +99,10 @@ extern "C" gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean
     gnp_t g; memset(&g, 0, sizeof g); g.gamma = gamma; g.beta = beta; g.mean = mean; g.rstd = rstd; g.G = G; return g;
 }
 extern "C" int lp_gn_slab_any(void) { return 0; }
+
+// ---- the op layer's answers about masked convs and the z-window (src/nn_skip.cu:130-157, src/nn_bwd.cu:57): weak, so the reference's own
+// definitions replace them when this library is linked into it; standing alone every conv is dense and no window is set ----
+extern "C" __attribute__((weak)) skipm_t lp_skip_get(shape5, split_t, int) { skipm_t s; memset(&s, 0, sizeof s); return s; }
+extern "C" __attribute__((weak)) int nn_skip_fwd_level(shape5, split_t) { return 0; }
+extern "C" __attribute__((weak)) int nn_skip_masks(shape5, split_t) { return 0; }
+extern "C" __attribute__((weak)) int zw_win(int, int *, int *) { return 0; }

@@ -27,6 +27,7 @@ int nn_storage(const void *p) {
 }
 static int g_prec = 0, g_gn_stored = 0;
 void nn_set_prec(int p) { g_prec = p; }
+int nn_get_prec(void) { return g_prec; }
 void nn_set_gn_stored(int on) { g_gn_stored = on; }
 size_t nn_mx8_bytes(shape5 s) { return lp_mx8_bytes(s.n, s.c, (size_t)s.d * s.h * s.w); }
 size_t nn_mx4_bytes(shape5 s) { return lp_mx4_bytes(s.n, s.c, (size_t)s.d * s.h * s.w); }

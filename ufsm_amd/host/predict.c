@@ -5,12 +5,12 @@
 #include "../../include/mi_unet.h"
 #include "../../include/mi_predict.h"
 
-int unet_predict_volume(unet *u, const uint8_t *vol, const int64_t dims[3], int halo, int feather, float mean, float isd,
-                        int axis, float cy, float cx, uint8_t *out, int64_t nwin[2]) {
-    const shape5 in = unet_in_shape(u);
+int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, const int64_t dims[3], int halo, int feather, float mean, float isd,
+                           int axis, float cy, float cx, uint8_t *out, int64_t nwin[2]) {
+    const shape5 in = {nbatch, 4, window, window, window};
     const int W = in.w, S = W - 2 * halo, B = feather, En = S + B;
     if (in.n < 1 || in.n > 16 || in.d != W || in.h != W || halo < 0 || S <= 0 || B < 0 || B > halo || B > S || B > 1024) {
-        fprintf(stderr, "unet_predict_volume: needs cubic windows (1 .. 16 per forward), 0 <= feather <= halo, window - 2 halo > 0 and feather <= it (window %d x %d x %d, halo %d, feather %d)\n",
+        fprintf(stderr, "mi_unet_predict_volume: needs cubic windows (1 .. 16 per forward), 0 <= feather <= halo, window - 2 halo > 0 and feather <= it (window %d x %d x %d, halo %d, feather %d)\n",
                 in.d, in.h, in.w, halo, feather);
         return -1;
     }
@@ -18,8 +18,8 @@ int unet_predict_volume(unet *u, const uint8_t *vol, const int64_t dims[3], int 
     for (int d = 0; d < 3; d++) { if (dims[d] <= 0) return -1; nss[d] = (dims[d] + S - 1) / S; total *= nss[d]; }
     const size_t w3 = (size_t)W * W * W, e3 = (size_t)En * En * En;
     uint8_t *E = mi_malloc((size_t)total * e3), *ctw = mi_malloc((size_t)in.n * w3), *dpres = mi_malloc((size_t)total);
-    const size_t lgn = (size_t)unet_config(u)->head_out * w3;      /* logits of one window */
-    float *lg = mi_malloc((size_t)in.n * lgn * sizeof(float)), *doff = mi_malloc((size_t)total * 2 * W * sizeof(float));
+    const size_t lgn = (size_t)unet_cfg_of(u)->cout * w3;      /* logits of one window */
+    float *doff = mi_malloc((size_t)total * 2 * W * sizeof(float));
     unsigned *dany = mi_malloc((size_t)total * sizeof(unsigned));
     uint8_t *present = calloc((size_t)total, 1);
     unsigned *hany = malloc((size_t)total * sizeof(unsigned));
@@ -54,7 +54,8 @@ int unet_predict_volume(unet *u, const uint8_t *vol, const int64_t dims[3], int 
             mi_ct_window(vol, dims[0], dims[1], dims[2], a * S - halo, b * S - halo, c * S - halo, W, ctw + (size_t)j * w3, iso, halo, NULL);
             cts[j] = ctw + (size_t)j * w3; dyos[j] = doff + (size_t)id * 2 * W; dxos[j] = dyos[j] + W;
         }
-        if (unet_forward_ct_n(u, cts, mean, isd, dyos, dxos, axis, lg)) { rc = -1; break; }
+        const float *lg = mi_unet_forward_ct_n(u, cts, mean, isd, dyos, dxos, axis, in, 2);      /* (fp16-rounded input values, as predict) */
+        if (!lg) { rc = -1; break; }
         for (int j = 0; j < in.n && k + j < np; j++) {
             /* E: the interior and B voxels of the upper halo, window coordinates [halo, halo + S + B) -> [0, S + B) (src/predict.c:3426-3427) */
             nn_pred_place(lg + (size_t)j * lgn, cts[j], W, halo - B, -halo, -halo, -halo, En, En, En, En, E + (size_t)ids[j] * e3);
@@ -70,7 +71,7 @@ int unet_predict_volume(unet *u, const uint8_t *vol, const int64_t dims[3], int 
     }
     if (nwin) { nwin[0] = total; nwin[1] = done; }
     mi_sync();
-    mi_free(E); mi_free(ctw); mi_free(dpres); mi_free(lg); mi_free(doff); mi_free(dany);
+    mi_free(E); mi_free(ctw); mi_free(dpres); mi_free(doff); mi_free(dany);
     free(present); free(hoff); free(hany);
     return rc;
 }

@@ -20,14 +20,17 @@ typedef struct {
     float *m1, *r1, *m2, *r2;                                      /* their GroupNorm statistics [n * G] */
 } block;
 struct unet {
-    unet_cfg cfg; shape5 in; shape5 ls[UNET_MAXLEV];
+    unet_cfg cfg;
+    /* the activations, built for one input shape and storage mode (rebuilt when either changes: src/unet.c:2876) */
+    int built, act_dt, prec; shape5 in; shape5 ls[UNET_MAXLEV];
     block enc[UNET_MAXLEV], dec[UNET_MAXLEV];
     convp down[UNET_MAXLEV], head;
     void *downo[UNET_MAXLEV];
     void *skipst[UNET_MAXLEV];         /* silu(gn(enc[i].a2)) in the compute format, formed once for its two readers (down conv, decoder conv1); null: each reader transforms it */
     gnpar dn[UNET_MAXLEV]; float *dm[UNET_MAXLEV], *dr[UNET_MAXLEV];   /* down_norm: GroupNorm after down[i], its statistics */
-    size_t np; float *params;                                      /* device */
-    void *xin;                                                     /* the network input built from a CT window */
+    size_t np; float *p, *ema, *params;                            /* device: live weights, EMA copy, the one the forward reads */
+    void *xin;                                                     /* the network input as an MX tensor */
+    float *logits;                                                 /* [n][cout][S], owned by the net */
     struct { const void *p; shape5 s; const char *name; const float *mean, *rstd; int G; } outs[64]; int nouts;
     /* the attention stage on the bottleneck (src/unet.c:470-509 set-up, :2795-2835 forward) */
     int tbn; at_dims tbd; at_bp tbp[16]; size_t reg_off; at_geom tbg; at_ws tbw;
@@ -35,21 +38,58 @@ struct unet {
     float *tb_cs, *tb_tok; void *tb_ws;                            /* fp32 planes [n][C][Sg]; token rows, one buffer per block + 1; block scratch */
 };
 
+/* activation storage of the nets built from now on (src/unet.c:700-706): MX-fp8 unless MX-fp4 is asked for */
+static int g_act_mx8 = 1, g_act_mx4 = 0;
+void unet_set_act_mx8(int on) { g_act_mx8 = on != 0; }
+void unet_set_act_mx4(int on) { g_act_mx4 = on != 0; }
+int unet_act_mx(void) { return g_act_mx8 || g_act_mx4; }
+static int act_dt_now(void) { return g_act_mx4 ? 4 : 8; }
+
 static int G_of(const unet *u, int c) { return u->cfg.G < c ? u->cfg.G : c; }      /* src/unet.c:297 */
 static size_t add_conv(convp *c, int cin, int cout, int k, size_t off) { c->cin = cin; c->cout = cout; c->k = k; c->w = off; off += (size_t)cout * cin * k * k * k; c->b = off; return off + cout; }
 static size_t add_gn(gnpar *g, int c, size_t off) { g->c = c; g->gamma = off; g->beta = off + c; return off + 2 * (size_t)c; }
-static size_t act_bytes(const unet *u, shape5 s) { return u->cfg.act_dt == 4 ? nn_mx4_bytes(s) : nn_mx8_bytes(s); }
-static void *act_new(const unet *u, shape5 s) { const size_t b = act_bytes(u, s); void *p = mi_malloc(b); mi_zero(p, b); nn_set_storage(p, b, u->cfg.act_dt); return p; }
+static size_t act_bytes(const unet *u, shape5 s) { return u->act_dt == 4 ? nn_mx4_bytes(s) : nn_mx8_bytes(s); }
+static void *act_new(const unet *u, shape5 s) { const size_t b = act_bytes(u, s); void *p = mi_malloc(b); mi_zero(p, b); nn_set_storage(p, b, u->act_dt); return p; }
 static void act_del(void *p) { if (p) { nn_storage_forget(p); mi_free(p); } }
 static float *f32_new(size_t n) { float *p = mi_malloc(n * 4); mi_zero(p, n * 4); return p; }
 
-unet *unet_create(const unet_cfg *cfg, shape5 in) {
+/* a field of the reference's configuration this build's graph does not run: named, so the caller knows which */
+static const char *cfg_unsupported(const unet_cfg *c) {
+    if (c->scale_cond) return "scale_cond";
+    for (int i = 0; i < UNET_MAXLEV; i++) {
+        if (c->dec_widths[i] && (i >= c->nlev || c->dec_widths[i] != c->widths[i])) return "dec_widths";
+        if (c->enc_blocks[i]) return "enc_blocks";
+        if (c->dec_convs[i] && c->dec_convs[i] != 2) return "dec_convs";
+    }
+    if (c->ds_levels) return "ds_levels";
+    if (c->lat_guide || c->lat_nsub) return "lat_guide";
+    if (c->w4_2d) return "w4_2d";
+    if (c->l0_norm || c->l0_slab) return "l0_norm";
+    if (c->gfilm) return "gfilm";
+    if (c->gn_ema) return "gn_ema";
+    if (c->attn_vres) return "attn_vres";
+    if (c->attn_axis) return "attn_axis";
+    if (c->attn_repeat > 1) return "attn_repeat";
+    if (c->attn_mem) return "attn_mem";
+    if (c->view_P || c->view_patch) return "view_P";
+    if (c->attn_deform || c->attn_dlev || c->attn_dco || c->attn_dinit) return "attn_deform";
+    if (c->emb_lev || c->emb_ch) return "emb_lev";
+    if (c->film) return "film";
+    if (c->skip_thr || c->skip_margin || c->skip_nl) return "skip_empty";
+    if (c->fstem || c->fstem_out) return "fstem";
+    if (c->lat_dec || c->lat_dec_raw || c->lat_dec_ng || c->lat_dec_wq) return "lat_dec";
+    return nullptr;
+}
+
+unet *unet_create(const unet_cfg *cfg) {
     const int L = cfg->nlev;
-    if (L < 1 || L > UNET_MAXLEV || in.c != cfg->cin || (cfg->act_dt != 8 && cfg->act_dt != 4)) { fprintf(stderr, "unet_create: bad configuration\n"); return nullptr; }
-    if ((in.d | in.h | in.w) & ((1 << (L - 1)) - 1)) { fprintf(stderr, "unet_create: window %d x %d x %d is not divisible by %d\n", in.d, in.h, in.w, 1 << (L - 1)); return nullptr; }
+    if (L < 1 || L > UNET_MAXLEV || cfg->cin < 1 || cfg->cout < 1 || cfg->G < 1) { fprintf(stderr, "unet_create: bad configuration (nlev %d, cin %d, cout %d, G %d)\n", L, cfg->cin, cfg->cout, cfg->G); return nullptr; }
+    for (int i = 0; i < L; i++) if (cfg->widths[i] < 1) { fprintf(stderr, "unet_create: width %d of level %d\n", cfg->widths[i], i); return nullptr; }
+    const char *bad = cfg_unsupported(cfg);
+    if (bad) { fprintf(stderr, "unet_create: the configuration sets \"%s\", which this build's graph does not run\n", bad); return nullptr; }
     unet *u = calloc(1, sizeof *u);
     if (!u) return nullptr;
-    u->cfg = *cfg; u->in = in;
+    u->cfg = *cfg;
     const int *w = cfg->widths;
     size_t off = 0;
     /* parameter order of unet_init: encoder blocks, down convs, decoder blocks, head */
@@ -64,7 +104,7 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
         off = add_conv(&b->c1, w[i + 1] + w[i], w[i], 3, off); off = add_gn(&b->n1, w[i], off);
         off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
     }
-    off = add_conv(&u->head, w[0], cfg->head_out, 1, off);
+    off = add_conv(&u->head, w[0], cfg->cout, 1, off);
     if (cfg->down_norm) for (int i = 0; i < L - 1; i++) off = add_gn(&u->dn[i], w[i], off);       /* (appended after the head, src/unet.c:459) */
     if (cfg->attn_blocks > 0) {                                   /* parameters last: registers, then the blocks (src/unet.c:490-499) */
         const int C = w[L - 1];
@@ -73,13 +113,41 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
             free(u); return nullptr;
         }
         const int F = cfg->attn_mlp > 0 ? cfg->attn_mlp : (8 * C / 3 + 31) / 32 * 32;
-        u->tbd = (at_dims){C, C / AT_HD, F, cfg->attn_pe == 1 ? 1 : 0, cfg->attn_reg, 100.f};
+        u->tbd = (at_dims){.C = C, .H = C / AT_HD, .F = F, .rope = cfg->attn_pe == 1 ? 1 : 0, .nreg = cfg->attn_reg, .rope_base = 100.f};
         u->reg_off = off; off += (size_t)cfg->attn_reg * C;
         for (int k = 0; k < cfg->attn_blocks; k++) off = at_block_layout(&u->tbd, &u->tbp[k], off);
         u->tbn = cfg->attn_blocks;
     }
     u->np = off;
-    u->params = f32_new(off);
+    u->p = f32_new(off); u->ema = f32_new(off); u->params = u->p;
+    return u;
+}
+/* the activation buffers of the current build */
+static void free_acts(unet *u) {
+    if (!u->built) return;
+    mi_sync();
+    for (int i = 0; i < UNET_MAXLEV; i++) {
+        for (int s = 0; s < 2; s++) {
+            block *b = s ? &u->dec[i] : &u->enc[i];
+            act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2);
+            b->a1 = b->a2 = nullptr; b->m1 = b->r1 = b->m2 = b->r2 = nullptr;
+        }
+        act_del(u->downo[i]); act_del(u->skipst[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
+        u->downo[i] = u->skipst[i] = nullptr; u->dm[i] = u->dr[i] = nullptr;
+    }
+    if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); u->tb.a2 = nullptr; u->tb.m2 = u->tb.r2 = nullptr; u->tb_cs = u->tb_tok = nullptr; u->tb_ws = nullptr; }
+    act_del(u->xin); u->xin = nullptr;
+    mi_free(u->logits); u->logits = nullptr;
+    u->built = 0; u->nouts = 0;
+}
+/* (re)build for input shape `in` under the storage mode and precision policy in force (build_acts, src/unet.c:2876) */
+static int build_acts(unet *u, shape5 in) {
+    const unet_cfg *cfg = &u->cfg; const int L = cfg->nlev; const int *w = cfg->widths;
+    if (in.n < 1 || in.c != cfg->cin || in.d < 1 || in.h < 1 || in.w < 1) { fprintf(stderr, "unet: input shape %d x %d x %d x %d x %d does not fit a net of %d input channels\n", in.n, in.c, in.d, in.h, in.w, cfg->cin); return -1; }
+    if ((in.d | in.h | in.w) & ((1 << (L - 1)) - 1)) { fprintf(stderr, "unet: spatial size %dx%dx%d must be divisible by %d\n", in.d, in.h, in.w, 1 << (L - 1)); abort(); }   /* (src/unet.c:2875) */
+    if (!unet_act_mx()) { fprintf(stderr, "unet: this build stores activations as MX-fp8 or MX-fp4 only (unet_set_act_mx8 / unet_set_act_mx4)\n"); return -1; }
+    free_acts(u);
+    u->in = in; u->act_dt = act_dt_now(); u->prec = nn_get_prec();
     for (int i = 0; i < L; i++) u->ls[i] = (shape5){in.n, w[i], in.d >> i, in.h >> i, in.w >> i};
     for (int i = 0; i < L; i++) {
         for (int s = 0; s < 2; s++) {
@@ -93,11 +161,12 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
         if (i < L - 1) {
             shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds);
             /* both readers of the skip compute in e4m3 from MX-fp8 storage: one shared pre-stage (any other combination: the readers' formats differ) */
-            if (cfg->act_dt == 8 && cfg->prec != 3 && w[i] % 32 == 0) u->skipst[i] = act_new(u, u->enc[i].ys);
+            if (u->act_dt == 8 && u->prec != 3 && w[i] % 32 == 0) u->skipst[i] = act_new(u, u->enc[i].ys);
             if (cfg->down_norm) { const size_t ng = (size_t)in.n * G_of(u, w[i]); u->dm[i] = f32_new(ng); u->dr[i] = f32_new(ng); }
         }
     }
     u->xin = act_new(u, in);
+    u->logits = f32_new((size_t)in.n * cfg->cout * in.d * in.h * in.w);
     if (u->tbn) {
         const shape5 ys = u->ls[L - 1]; const long Sg = (long)ys.d * ys.h * ys.w, S = Sg + u->tbd.nreg, T = (long)ys.n * S; const int C = u->tbd.C;
         u->tbg = (at_geom){.nseq = ys.n, .S = (int)S, .D = ys.d, .Hh = ys.h, .W = ys.w};
@@ -107,23 +176,29 @@ unet *unet_create(const unet_cfg *cfg, shape5 in) {
         u->tb_cs = f32_new((size_t)ys.n * C * Sg); u->tb_tok = f32_new((size_t)(u->tbn + 1) * T * C);
         u->tb_ws = mi_malloc(at_ws_bytes(&u->tbd, T)); at_ws_carve(&u->tbw, &u->tbd, T, u->tb_ws);
     }
-    return u;
+    u->built = 1;
+    return 0;
+}
+static int ensure_built(unet *u, shape5 xs) {
+    if (u->built && !memcmp(&u->in, &xs, sizeof xs) && u->act_dt == act_dt_now() && u->prec == nn_get_prec()) return 0;
+    return build_acts(u, xs);
 }
 void unet_free(unet *u) {
     if (!u) return;
     mi_sync();
-    for (int i = 0; i < UNET_MAXLEV; i++) {
-        for (int s = 0; s < 2; s++) { block *b = s ? &u->dec[i] : &u->enc[i]; act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2); }
-        act_del(u->downo[i]); act_del(u->skipst[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
-    }
-    if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); }
-    act_del(u->xin); mi_free(u->params);
+    free_acts(u);
+    mi_free(u->p); mi_free(u->ema);
     lp_wmemo_clear();
     free(u);
 }
 size_t unet_nparams(const unet *u) { return u->np; }
-void unet_get_params(const unet *u, float *host) { mi_sync(); mi_d2h(host, u->params, u->np * 4); }
-void unet_set_params(unet *u, const float *host) { mi_h2d(u->params, host, u->np * 4); lp_wmemo_clear(); }
+const unet_cfg *unet_cfg_of(const unet *u) { return &u->cfg; }
+float *unet_param_ptr(unet *u) { return u->p; }
+float *unet_ema_ptr(unet *u) { return u->ema; }
+void unet_use_ema(unet *u, int on) { float *w = on ? u->ema : u->p; if (w != u->params) { u->params = w; lp_wmemo_clear(); } }      /* (the prepared weights are keyed by pointer; dropped all the same) */
+void mi_unet_get_params(const unet *u, float *host) { mi_sync(); mi_d2h(host, u->p, u->np * 4); }
+void mi_unet_set_params(unet *u, const float *host) { mi_h2d(u->p, host, u->np * 4); mi_h2d(u->ema, host, u->np * 4); lp_wmemo_clear(); }
+shape5 unet_out_shape(const unet *u, shape5 xs) { return (shape5){xs.n, u->cfg.cout, xs.d, xs.h, xs.w}; }
 
 /* splitmix64 -> uniform -> Box-Muller normal: the distribution of src/unet.c:586-593, not its generator's bits */
 static double unif(uint64_t *s) { uint64_t z = (*s += 0x9e3779b97f4a7c15ull); z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull; z = (z ^ (z >> 27)) * 0x94d049bb133111ebull; z ^= z >> 31; return (double)(z >> 11) * 0x1.0p-53; }
@@ -154,7 +229,7 @@ void unet_init(unet *u, uint64_t seed) {
         }
         for (size_t i = 0; i < (size_t)u->tbd.nreg * C; i++) h[u->reg_off + i] = (float)(0.02 * gauss(&seed));
     }
-    unet_set_params(u, h);
+    mi_unet_set_params(u, h);
     free(h);
 }
 
@@ -168,7 +243,7 @@ static nn_gn_t gn_out(const unet *u, const block *b) { return (nn_gn_t){P(u, b->
    z-range, each slab's planes written straight into the full-depth output; results are those of the whole-tensor convs */
 static int g_infer_slab;
 void unet_set_infer_slab(int planes) { g_infer_slab = planes > 0 ? (planes + 3) / 4 * 4 : 0; }
-int unet_get_infer_slab(void) { return g_infer_slab; }
+int mi_unet_infer_slab(void) { return g_infer_slab; }
 
 /* conv1 -> a1 (+ its statistics), conv2 reads silu(gn(a1)) while staging -> a2 (+ statistics) (src/unet.c:2567-2636) */
 static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t *gin, const void *xup, const nn_gn_t *gup, int c_split, const char *n1, const char *n2) {
@@ -193,34 +268,32 @@ static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t 
 static int tb_fwd(unet *u) {
     const block *x = &u->enc[u->cfg.nlev - 1]; block *b = &u->tb;
     const shape5 ys = b->ys; const int C = u->tbd.C, nr = u->tbd.nreg; const size_t Sg = (size_t)ys.d * ys.h * ys.w, TC = (size_t)u->tbg.nseq * u->tbg.S * C;
-    if (u->cfg.act_dt == 4) lp_mx4_to_f32(x->a2, ys.n, C, Sg, u->tb_cs); else lp_mx8_to_f32(x->a2, ys.n, C, Sg, u->tb_cs);
+    if (u->act_dt == 4) lp_mx4_to_f32(x->a2, ys.n, C, Sg, u->tb_cs); else lp_mx8_to_f32(x->a2, ys.n, C, Sg, u->tb_cs);
     at_cs_to_tok(u->tb_cs, u->tb_tok, P(u, u->reg_off), ys.n, C, (long)Sg, nr);
     at_set_mx(8);
-    lp_mx_gemm_bmemo(1);                                           /* inference: the linears' weights are packed once (dropped by unet_set_params) */
+    lp_mx_gemm_bmemo(1);                                           /* inference: the linears' weights are packed once (dropped when the weights change) */
     for (int k = 0; k < u->tbn; k++)
         if (at_block_fwd(&u->tbd, u->params, &u->tbp[k], u->tb_tok + (size_t)k * TC, u->tb_tok + (size_t)(k + 1) * TC, &u->tbg, &u->tbw)) { lp_mx_gemm_bmemo(0); fprintf(stderr, "unet: attention block forward failed\n"); return -1; }
     lp_mx_gemm_bmemo(0);
     at_tok_to_cs(u->tb_tok + (size_t)u->tbn * TC, u->tb_cs, ys.n, C, (long)Sg, nr);
-    if (u->cfg.act_dt == 4) lp_f32_to_mx4(u->tb_cs, ys.n, C, Sg, b->a2); else lp_f32_to_mx8(u->tb_cs, ys.n, C, Sg, b->a2);
+    if (u->act_dt == 4) lp_f32_to_mx4(u->tb_cs, ys.n, C, Sg, b->a2); else lp_f32_to_mx8(u->tb_cs, ys.n, C, Sg, b->a2);
     const int G = G_of(u, C);
     if (nn_gn_stats(b->a2, ys, G, 1e-5f, b->m2, b->r2)) { fprintf(stderr, "unet: attention stage GroupNorm statistics unsupported for this storage\n"); return -1; }
     note(u, b->a2, ys, "attn", b->m2, b->r2, G);
     return 0;
 }
-int unet_forward_x(unet *u, const void *x, float *logits) {
+/* the graph on the MX input tensor x (src/unet.c:2939-3105) */
+static int graph_fwd(unet *u, const void *x) {
     static const char *en1[] = {"enc0.c1", "enc1.c1", "enc2.c1", "enc3.c1", "enc4.c1", "enc5.c1", "enc6.c1", "enc7.c1"}, *en2[] = {"enc0.c2", "enc1.c2", "enc2.c2", "enc3.c2", "enc4.c2", "enc5.c2", "enc6.c2", "enc7.c2"};
     static const char *dn1[] = {"dec0.c1", "dec1.c1", "dec2.c1", "dec3.c1", "dec4.c1", "dec5.c1", "dec6.c1"}, *dn2[] = {"dec0.c2", "dec1.c2", "dec2.c2", "dec3.c2", "dec4.c2", "dec5.c2", "dec6.c2"};
     static const char *dwn[] = {"down0", "down1", "down2", "down3", "down4", "down5", "down6"};
     const int L = u->cfg.nlev;
-    const int reg_here = nn_storage(x) != u->cfg.act_dt;           /* the caller's input is looked up by the convs like any activation */
-    if (reg_here) nn_set_storage(x, act_bytes(u, u->in), u->cfg.act_dt);
-    nn_set_prec(u->cfg.prec);
     u->nouts = 0;
     const void *cur = x;
     for (int i = 0; i < L; i++) {
         nn_gn_t gd; const nn_gn_t *gin = nullptr;                  /* down_norm: conv1 reads silu(gn(down conv output)) (src/unet.c:2593) */
         if (i && u->cfg.down_norm) { gd = (nn_gn_t){P(u, u->dn[i - 1].gamma), P(u, u->dn[i - 1].beta), u->dm[i - 1], u->dr[i - 1], G_of(u, u->cfg.widths[i - 1])}; gin = &gd; }
-        if (block_fwd(u, &u->enc[i], i, cur, gin, nullptr, nullptr, 0, en1[i], en2[i])) { if (reg_here) nn_storage_forget(x); return -1; }
+        if (block_fwd(u, &u->enc[i], i, cur, gin, nullptr, nullptr, 0, en1[i], en2[i])) return -1;
         if (i < L - 1) {                                           /* stride-2 down conv of silu(gn(a2)), width kept (src/unet.c:2970) */
             const nn_gn_t g = gn_out(u, &u->enc[i]);
             const int pre = u->skipst[i] != nullptr;
@@ -234,7 +307,7 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
             cur = u->downo[i];
         }
     }
-    if (u->tbn && tb_fwd(u)) { if (reg_here) nn_storage_forget(x); return -1; }
+    if (u->tbn && tb_fwd(u)) return -1;
     for (int i = L - 2; i >= 0; i--) {                             /* decoder: nothing materialised (src/unet.c:3010-3013) */
         const block *coarse = i == L - 2 ? &u->enc[L - 1] : &u->dec[i + 1];
         nn_gn_t gc = gn_out(u, coarse); const nn_gn_t gs = gn_out(u, &u->enc[i]);
@@ -244,29 +317,49 @@ int unet_forward_x(unet *u, const void *x, float *logits) {
     }
     const block *last = L > 1 ? &u->dec[0] : &u->enc[0];
     const nn_gn_t g = gn_out(u, last);
-    nn_set_prec(0);
-    if (reg_here) nn_storage_forget(x);
-    return nn_conv3d_fwd_x(last->a2, &g, nullptr, nullptr, 0, 0, last->ys, P(u, u->head.w), P(u, u->head.b), u->cfg.head_out, 1, 1, logits, 0, 0.f, nullptr, nullptr);
+    return nn_conv3d_fwd_x(last->a2, &g, nullptr, nullptr, 0, 0, last->ys, P(u, u->head.w), P(u, u->head.b), u->cfg.cout, 1, 1, u->logits, 0, 0.f, nullptr, nullptr);
 }
-int unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, float *logits) {
-    if (u->in.n != 1) { fprintf(stderr, "unet_forward_ct: needs one square window of 4 input channels\n"); return -1; }
-    return unet_forward_ct_n(u, &ct, mean, isd, &dyo, &dxo, axis, logits);
+/* every exit of a forward passes here: the caller's tensor leaves the storage registry again (a stale range would make a later allocation
+   inside it look like MX storage) */
+const float *mi_unet_forward_mx(unet *u, const void *xmx, shape5 xs) {
+    if (ensure_built(u, xs)) return nullptr;
+    const int reg_here = xmx != u->xin && nn_storage(xmx) != u->act_dt;     /* the input is looked up by the convs like any activation */
+    if (reg_here) nn_set_storage(xmx, act_bytes(u, u->in), u->act_dt);
+    const int rc = graph_fwd(u, xmx);
+    if (reg_here) nn_storage_forget(xmx);
+    return rc ? nullptr : u->logits;
 }
-/* one forward over in.n windows: window n's input rows go to sample n (fp16-rounded input values, as predict); logits [n][head_out][voxels] */
-int unet_forward_ct_n(unet *u, const uint8_t *const *ct, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, float *logits) {
-    if (u->cfg.cin != 4 || u->in.h != u->in.w) { fprintf(stderr, "unet_forward_ct: needs square windows of 4 input channels\n"); return -1; }
-    for (int n = 0; n < u->in.n; n++)
-        mi_pred_input_mx_n(ct[n], u->in.w, mean, isd, dyo[n], dxo[n], axis, 0, u->in.d, u->xin, 2, u->cfg.act_dt == 4 ? 4 : 8, u->in.n, n);
-    return unet_forward_x(u, u->xin, logits);
+const float *unet_forward_x(unet *u, const void *x, shape5 xs, int train, int x_h16) {
+    if (train) { fprintf(stderr, "unet_forward_x: this is an inference build (train must be 0)\n"); abort(); }
+    if (ensure_built(u, xs)) return nullptr;
+    const size_t S = (size_t)xs.d * xs.h * xs.w;
+    /* the input conversion of src/unet.c:2909-2919: fp32 planes, or the 16-bit storage type read in place (fp16 here) -> the MX input tensor */
+    if (x_h16) { if (u->act_dt == 4) lp_h16_to_mx4(x, 2, xs.n, xs.c, S, u->xin); else lp_h16_to_mx8(x, 2, xs.n, xs.c, S, u->xin); }
+    else if (u->act_dt == 4) lp_f32_to_mx4(x, xs.n, xs.c, S, u->xin); else lp_f32_to_mx8(x, xs.n, xs.c, S, u->xin);
+    return mi_unet_forward_mx(u, u->xin, xs);
 }
-shape5 unet_in_shape(const unet *u) { return u->in; }
-const unet_cfg *unet_config(const unet *u) { return &u->cfg; }
-int unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd) {
+const float *unet_forward(unet *u, const float *x, shape5 xs, int train) { return unet_forward_x(u, x, xs, train, 0); }
+/* one forward over xs.n windows: window n's input rows go to sample n; logits [n][cout][voxels] */
+const float *mi_unet_forward_ct_n(unet *u, const uint8_t *const *ct, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, shape5 xs, int h16) {
+    if (xs.c != 4 || u->cfg.cin != 4 || xs.h != xs.w) { fprintf(stderr, "unet_forward_ct: needs square windows of 4 input channels\n"); return nullptr; }
+    if (ensure_built(u, xs)) return nullptr;
+    for (int n = 0; n < xs.n; n++)
+        mi_pred_input_mx_n(ct[n], xs.w, mean, isd, dyo[n], dxo[n], axis, 0, xs.d, u->xin, h16, u->act_dt == 4 ? 4 : 8, xs.n, n);
+    return mi_unet_forward_mx(u, u->xin, xs);
+}
+const float *unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, shape5 xs, int h16) {
+    if (xs.n < 1 || xs.n > 64) { fprintf(stderr, "unet_forward_ct: %d windows per forward (1 .. 64)\n", xs.n); return nullptr; }
+    const uint8_t *cts[64]; const float *dys[64], *dxs[64];
+    const size_t w3 = (size_t)xs.d * xs.h * xs.w;
+    for (int n = 0; n < xs.n; n++) { cts[n] = ct + (size_t)n * w3; dys[n] = dyo + (size_t)n * xs.d; dxs[n] = dxo + (size_t)n * xs.d; }
+    return mi_unet_forward_ct_n(u, cts, mean, isd, dys, dxs, axis, xs, h16);
+}
+int mi_unet_layer_stats(const unet *u, int k, const float **mean, const float **rstd) {
     if (k < 0 || k >= u->nouts) return 0;
     *mean = u->outs[k].mean; *rstd = u->outs[k].rstd;
     return u->outs[k].G;
 }
-const void *unet_layer_out(const unet *u, int k, shape5 *s, const char **name) {
+const void *mi_unet_layer_out(const unet *u, int k, shape5 *s, const char **name) {
     if (k < 0 || k >= u->nouts) return nullptr;
     if (s) *s = u->outs[k].s;
     if (name) *name = u->outs[k].name;
@@ -285,7 +378,7 @@ static char *header_line(FILE *f) {                                /* the first 
     free(s); return nullptr;
 }
 static int key_int(const char *line, const char *key, int dflt) { const char *p = strstr(line, key); return p ? atoi(p + strlen(key)) : dflt; }
-int unet_read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step) {
+static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step) {
     FILE *f = fopen(path, "rb");
     if (!f) return -1;
     char *line = header_line(f); fclose(f);
@@ -297,34 +390,37 @@ int unet_read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step
     if (cfg->nlev < 1 || cfg->nlev > UNET_MAXLEV || !p) { free(line); return -1; }
     p += 10;
     for (int i = 0; i < cfg->nlev; i++) { cfg->widths[i] = atoi(p); p = strchr(p, ','); if (!p) break; p++; }
-    cfg->cin = key_int(line, "\"cin\":", 0); cfg->head_out = key_int(line, "\"cout\":", 0); cfg->G = key_int(line, "\"G\":", 8);
+    cfg->cin = key_int(line, "\"cin\":", 0); cfg->cout = key_int(line, "\"cout\":", 0); cfg->G = key_int(line, "\"G\":", 8);
     cfg->down_norm = key_int(line, "\"down_norm\":", 0);
     cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
     cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
-    cfg->act_dt = 8; cfg->prec = 0;
+    cfg->half_res = key_int(line, "\"half_res\":", 0); cfg->scan_norm = key_int(line, "\"scan_norm\":", 0);      /* (the caller's business: the graph does not use them) */
     if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
-    static const char *const no[] = {"\"dec_widths\":", "\"enc_blocks\":", "\"half_res\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"w4_2d\":", "\"ds_levels\":", "\"emb_lev\":",
+    static const char *const no[] = {"\"dec_widths\":", "\"enc_blocks\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"w4_2d\":", "\"ds_levels\":", "\"emb_lev\":",
                                      "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
-                                     "\"l0_norm\":", "\"scan_norm\":", "\"skip_empty\":", "\"gfilm\":", "\"gn_ema\":", "\"dec_convs\":"};
+                                     "\"l0_norm\":", "\"skip_empty\":", "\"gfilm\":", "\"gn_ema\":", "\"dec_convs\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
     if (!bad && key_int(line, "\"scale_cond\":", 0)) bad = "\"scale_cond\":";
     if (!bad && cfg->attn_blocks && cfg->attn_pe != 1 && cfg->attn_pe != 2) bad = "\"attn_pe\": (PEG / scroll RoPE)";
-    if (bad) { fprintf(stderr, "unet_read_header: %s uses %s which this build does not run\n", path, bad); free(line); return -2; }
+    if (bad) { fprintf(stderr, "unet_peek: %s uses %s which this build does not run\n", path, bad); free(line); return -2; }
     free(line);
-    return cfg->cin > 0 && cfg->head_out > 0 ? 0 : -1;
+    return cfg->cin > 0 && cfg->cout > 0 ? 0 : -1;
 }
-static int load_array(unet *u, const char *path, int which) {
+int unet_peek(const char *path, unet_cfg *cfg, int *step) { return read_header(path, cfg, nullptr, step); }      /* src/unet.c:5756 */
+size_t mi_unet_peek_nparams(const char *path) { unet_cfg c; size_t np = 0; return read_header(path, &c, &np, nullptr) == -1 ? 0 : np; }
+/* weights and EMA weights into a net of the same architecture; the saved step, or -1 (src/unet.c:5774-5800) */
+int unet_load(unet *u, const char *path) {
     unet_cfg c; size_t np = 0; int step = 0;
-    const int r = unet_read_header(path, &c, &np, &step);
+    const int r = read_header(path, &c, &np, &step);
     if (r) { if (r == -1) fprintf(stderr, "unet_load: %s: unreadable header\n", path); return -1; }
     const unet_cfg *m = &u->cfg; const char *bad = nullptr;
     if (c.nlev != m->nlev) bad = "nlev";
     for (int i = 0; !bad && i < m->nlev; i++) if (c.widths[i] != m->widths[i]) bad = "widths";
     if (!bad && c.cin != m->cin) bad = "cin";
-    if (!bad && c.head_out != m->head_out) bad = "cout";
+    if (!bad && c.cout != m->cout) bad = "cout";
     if (!bad && c.attn_blocks != m->attn_blocks) bad = "attn_blocks";
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && np != u->np) bad = "nparams";
@@ -341,35 +437,38 @@ static int load_array(unet *u, const char *path, int which) {
     }
     float *h = malloc((size_t)a);
     int rc = -1;
-    if (h && !fseek(f, off + (long)(which ? a : 0), SEEK_SET) && fread(h, 4, np, f) == np) {
-        size_t nbad = 0; for (size_t i = 0; i < np; i++) nbad += !isfinite(h[i]);
-        if (nbad) fprintf(stderr, "unet_load: %s: %zu non-finite values\n", path, nbad);
-        else { unet_set_params(u, h); rc = 0; }
+    if (h && !fseek(f, off, SEEK_SET)) {
+        rc = step;
+        for (int which = 0; which < 2 && rc >= 0; which++) {       /* the weights, then their EMA copy */
+            if (fread(h, 4, np, f) != np) { rc = -1; break; }
+            size_t nbad = 0; for (size_t i = 0; i < np; i++) nbad += !isfinite(h[i]);
+            if (nbad) { fprintf(stderr, "unet_load: %s: %zu non-finite values\n", path, nbad); rc = -1; break; }
+            mi_h2d(which ? u->ema : u->p, h, (size_t)a);
+        }
+        lp_wmemo_clear();
     }
     free(h); fclose(f);
     return rc;
 }
-int unet_load(unet *u, const char *path) { return load_array(u, path, 0); }
-int unet_load_ema(unet *u, const char *path) { return load_array(u, path, 1); }
 int unet_save(const unet *u, const char *path, int step, const char *extra) {
-    float *h = malloc(u->np * 4);
-    if (!h) return -1;
-    unet_get_params(u, h);
-    if (nn_check()) { fprintf(stderr, "unet_save: a device error is latched: %s not written\n", path); free(h); return -1; }
-    for (size_t i = 0; i < u->np; i++) if (!isfinite(h[i])) { fprintf(stderr, "unet_save: non-finite weights (first at parameter %zu): %s not written\n", i, path); free(h); return -2; }
+    float *h = malloc(u->np * 4), *he = malloc(u->np * 4);
+    if (!h || !he) { free(h); free(he); return -1; }
+    mi_sync(); mi_d2h(h, u->p, u->np * 4); mi_d2h(he, u->ema, u->np * 4);
+    if (nn_check()) { fprintf(stderr, "unet_save: a device error is latched: %s not written\n", path); free(h); free(he); return -1; }
+    for (size_t i = 0; i < u->np; i++) if (!isfinite(h[i]) || !isfinite(he[i])) { fprintf(stderr, "unet_save: non-finite weights (first at parameter %zu): %s not written\n", i, path); free(h); free(he); return -2; }
     char tmp[1400]; snprintf(tmp, sizeof tmp, "%s.tmp", path);
     FILE *f = fopen(tmp, "wb");
-    if (!f) { fprintf(stderr, "unet_save: cannot create %s\n", tmp); free(h); return -1; }
+    if (!f) { fprintf(stderr, "unet_save: cannot create %s\n", tmp); free(h); free(he); return -1; }
     fprintf(f, "UFSM{\"nlev\":%d,\"widths\":[", u->cfg.nlev);
     for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.widths[i]);
     fputc(']', f);
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
-    fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":0,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.head_out, u->cfg.G,
+    fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":0,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.cout, u->cfg.G,
             u->cfg.down_norm, u->np, step);
     fprintf(f, ",\"extra\":%s}\n", extra ? extra : "{}");
-    int ok = fwrite(h, 4, u->np, f) == u->np && fwrite(h, 4, u->np, f) == u->np;      /* weights, EMA weights */
+    int ok = fwrite(h, 4, u->np, f) == u->np && fwrite(he, 4, u->np, f) == u->np;      /* weights, EMA weights */
     ok = !fclose(f) && ok;
-    free(h);
+    free(h); free(he);
     if (!ok || rename(tmp, path)) { fprintf(stderr, "unet_save: write error on %s\n", tmp); remove(tmp); return -1; }
     return 0;
 }

@@ -30,6 +30,11 @@ class split_t(C.Structure):  # src/nn_lp.h:32
 
 assert C.sizeof(split_t) <= 128  # src/nn_lp.h:41
 
+
+class skipm_t(C.Structure):  # src/nn_lp.h:44
+    _fields_ = [("m", C.c_void_p), ("mi", C.c_void_p), ("my", C.c_int), ("mx", C.c_int), ("zoff", C.c_int)]
+
+
 _P, _I, _Z, _F = C.c_void_p, C.c_int, C.c_size_t, C.c_float
 _PROTOS = {
     "lp_conv_fwd_f8": (_I, [_P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t]),
@@ -43,6 +48,10 @@ _PROTOS = {
     "mi_conv_prestage": (_I, [_P, _I, shape5, gnp_t, _P, _I]),
     "gnp_mk": (gnp_t, [_P, _P, _P, _P, _I]),
     "lp_gn_slab_any": (_I, []),
+    "lp_skip_get": (skipm_t, [shape5, split_t, _I]),
+    "nn_skip_fwd_level": (_I, [shape5, split_t]),
+    "nn_skip_masks": (_I, [shape5, split_t]),
+    "zw_win": (_I, [_I, _P, _P]),
     "lp_mx8_bytes": (_Z, [_I, _I, _Z]),
     "lp_mx4_bytes": (_Z, [_I, _I, _Z]),
     "lp_f32_to_mx8": (None, [_P, _I, _I, _Z, _P]),
