@@ -425,3 +425,151 @@ def test_z_range_slabs_equal_whole(gpu, case):
     part = orc.mx_to_f32(bits, ytmp.to_numpy(np.uint8), N, Co, sk2 * H * W).reshape(N, Co, sk2, H * W)
     zz = slabs[0] if len(slabs) > 1 else 0
     assert np.array_equal(part, full[:, :, zz:zz + sk2])
+
+
+# ---- the fp4-storage shapes of the BASELINE's third configuration and the fp4 entry's small-channel rows ----
+@pytest.mark.parametrize("Ci,Co,dims,gn", [(128, 128, (16, 16, 16), False), (128, 256, (12, 10, 14), False), (128, 256, (16, 16, 32), True), (96, 96, (13, 10, 17), True)])
+def test_stride2_wide_mx4_input_computes_in_e4m3(gpu, Ci, Co, dims, gn):
+    """A wide MX-fp4 tensor through the stride-2 entry: the reference keeps fp4 compute for exactly 32 -> <= 32 channels and runs every other
+    MX-fp4 input on the e4m3 kernel, the stored rows decoded, (GroupNorm + SiLU,) re-quantised to e4m3 per (voxel, 32 channels), the weights
+    e4m3 blocks (src/lp_s2.cu:653-671, :729-749); the call returns 0, not 3. Exact operands equal the oracle byte for byte."""
+    rng = np.random.default_rng(Ci + Co + dims[0])
+    D, H, W = dims
+    N, S, G = 2, D * H * W, 8
+    if gn:
+        x, w, b = rand_case(rng, N, Ci, Co, S)
+        p = [rng.uniform(0.5, 1.5, Ci).astype(np.float32), rng.uniform(-.5, .5, Ci).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    else:
+        x, w, b = exact_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(4, x, N, Ci, S)
+    dxq, dw, db = DevBuf.from_numpy(xq), DevBuf.from_numpy(w), DevBuf.from_numpy(b)
+    Do, Ho, Wo = out_dims(D, H, W, 2)
+    So = Do * Ho * Wo
+    dy = DevBuf(lib.lp_mx4_bytes(N, Co, So))
+    g = dev_gn(*p, G) if gn else gnp_t()
+    rc = lib.lp_conv_fwd_s2_f8(dxq.ptr, 4, shape5(N, Ci, D, H, W), dw.ptr, db.ptr, Co, dy.ptr, 4, shape5(N, Co, Do, Ho, Wo), g)
+    LP.check()
+    assert rc == 0 and "fmt 8, stride 2" in lib.mi_last_kernel().decode()
+    got = dy.to_numpy(np.uint8)
+    want, _ = orc.conv3(xq, 4, N, Ci, D, H, W, w, b, Co, 4, cbits=8, stride=2, gp=orc.gn(*p, G) if gn else None, acc64=0 if gn else 1)
+    if gn:
+        frac, near = code_mismatch_fraction(4, got, want, N, Co, So)
+        assert frac < 5e-3 and near
+    else:
+        assert np.array_equal(got, want)
+    # ... while 32 -> 32 on even dims of an MX-fp4 tensor does compute in e2m1 and says so
+    x2, w2, b2 = exact_case(rng, 1, 32, 32, 16 * 16 * 16)
+    q2 = orc.f32_to_mx(4, x2, 1, 32, 4096)
+    d2, dw2, db2, dy2 = DevBuf.from_numpy(q2), DevBuf.from_numpy(w2), DevBuf.from_numpy(b2), DevBuf(lib.lp_mx4_bytes(1, 32, 512))
+    assert lib.lp_conv_fwd_s2_f8(d2.ptr, 4, shape5(1, 32, 16, 16, 16), dw2.ptr, db2.ptr, 32, dy2.ptr, 4, shape5(1, 32, 8, 8, 8), gnp_t()) == 3
+    LP.check()
+    assert np.array_equal(dy2.to_numpy(np.uint8), orc.conv3(q2, 4, 1, 32, 16, 16, 16, w2, b2, 32, 4, cbits=4, stride=2, acc64=1)[0])
+
+
+@pytest.mark.parametrize("Cu,Cs,Co,dims,gn", [(256, 128, 128, (4, 8, 16), False), (256, 128, 128, (8, 8, 16), True), (320, 256, 256, (4, 8, 16), False), (64, 32, 32, (8, 16, 16), True)])
+def test_fp4_decoder_conv_fused_upsample(gpu, Cu, Cs, Co, dims, gn):
+    """The MX-fp4 decoder conv1 over [2x trilinear up(coarse) | skip] (256 + 128 -> 128: the BASELINE's fp4 up path; 320 + 256 -> 256:
+    tests/test_mx4_wide.c:749-751). Grid-valued coarse data with a +6 in every block blend exactly in any arithmetic (tests/test_mx4_wide.c:18-19):
+    the fp32 output equals the oracle; with GroupNorm + SiLU on both segments the e2m1 operands agree up to neighbouring codes of the staged rows."""
+    rng = np.random.default_rng(60 + Cu + Cs)
+    D, H, W = dims
+    N, S, Sc, G = 1, D * H * W, (D // 2) * (H // 2) * (W // 2), 8
+    if gn:
+        xa = rng.standard_normal((N, Cu, Sc)).astype(np.float32); xb = rng.standard_normal((N, Cs, S)).astype(np.float32)
+        w = (rng.standard_normal((Co, Cu + Cs, 27)) * np.sqrt(2.0 / ((Cu + Cs) * 27))).astype(np.float32)
+    else:
+        xa = refnp.gen_exact(rng, (N, Cu, Sc)); xa[np.abs(xa) == 6] = 6.0      # (+6, not -6: the blend of equal-sign maxima stays the block maximum)
+        xb = refnp.gen_exact(rng, (N, Cs, S)); w = refnp.gen_exact(rng, (Co, Cu + Cs, 27))
+    qa, qb = orc.f32_to_mx(4, xa, N, Cu, Sc), orc.f32_to_mx(4, xb, N, Cs, S)
+    p = [rng.uniform(0.5, 1.5, Cu).astype(np.float32), rng.uniform(-.5, .5, Cu).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    p2 = [rng.uniform(0.5, 1.5, Cs).astype(np.float32), rng.uniform(-.5, .5, Cs).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    want, _ = orc.conv3(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=4, x2=qb, c_split=Cu, up=1, gp=orc.gn(*p, G) if gn else None, gp2=orc.gn(*p2, G) if gn else None)
+    got, _ = gpu_conv(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=4, x2=qb, c_split=Cu, up=1, gp=dev_gn(*p, G) if gn else None, gp2=dev_gn(*p2, G) if gn else None)
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err < (3e-2 if gn else 1e-5), err
+    if not gn:                                                     # the blend of grid values is a multiple of 1/64 of at most 6: re-quantised to e2m1 it is not exact,
+        wq, _ = orc.conv3(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 4, cbits=4, x2=qb, c_split=Cu, up=1)   # but both sides round the same values: identical output codes
+        gq, _ = gpu_conv(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 4, cbits=4, x2=qb, c_split=Cu, up=1)
+        assert np.array_equal(gq, wq)
+
+
+@pytest.mark.parametrize("Ci,Co,dims", [(16, 16, (12, 12, 16)), (12, 32, (6, 12, 20)), (9, 16, (5, 9, 18)), (16, 64, (4, 8, 16))])
+def test_fp4_entry_9_to_16_channels(gpu, Ci, Co, dims):
+    """lp_conv_fwd_f4 on 9 - 16 input channels (one 16-wide stored block). The reference's packed kernel scales each 16-channel group of a position
+    and each (tap, output channel) group of 16 weights on its own (src/lp_f4fwd.cuh:786-800, src/lp_f4fwd.cu:85-100): the operands of a
+    32-block holding the 16 channels and 16 zeros. Exact operands: every output type equals the oracle."""
+    rng = np.random.default_rng(Ci * 3 + Co)
+    D, H, W = dims
+    N, S = 2, D * H * W
+    x = refnp.gen_exact(rng, (N, Ci, S), block=16); w = refnp.gen_exact(rng, (Co, Ci, 27), block=16)
+    b = (GRID[rng.integers(0, 8, Co)] * 0.25).astype(np.float32)
+    xq = orc.f32_to_mx(4, x, N, Ci, S)
+    for ydt in (0, 4, 3):
+        want, ws = orc.conv3(xq, 4, N, Ci, D, H, W, w, b, Co, ydt, cbits=4, acc64=1, Go=min(8, Co), want_stats=True)
+        got, gs = gpu_conv(xq, 4, N, Ci, D, H, W, w, b, Co, ydt, cbits=4, Go=min(8, Co), stats=True)
+        assert np.array_equal(got, want), (ydt, lib.mi_last_kernel().decode())
+        assert np.allclose(gs, ws, rtol=1e-6)
+    xr, wr, br = rand_case(rng, N, Ci, Co, S)                      # random data with GroupNorm on the input (tests/test_mx4.c:224-270: 16 -> 32 with GN)
+    G = 1 if Ci % 4 else 4
+    p = [rng.uniform(0.5, 1.5, Ci).astype(np.float32), rng.uniform(-.5, .5, Ci).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    xrq = orc.f32_to_mx(4, xr, N, Ci, S)
+    want, _ = orc.conv3(xrq, 4, N, Ci, D, H, W, wr, br, Co, 0, cbits=4, gp=orc.gn(*p, G))
+    got, _ = gpu_conv(xrq, 4, N, Ci, D, H, W, wr, br, Co, 0, cbits=4, gp=dev_gn(*p, G))
+    assert np.abs(got - want).max() / np.abs(want).max() < 3e-2
+
+
+@pytest.mark.parametrize("Cu,Cs,Co,dims", [(16, 16, 16, (12, 12, 16)), (12, 16, 16, (4, 8, 16)), (16, 8, 8, (8, 8, 16))])
+def test_fp4_fused_upsample_small_channels(gpu, Cu, Cs, Co, dims):
+    """The level-0 decoder conv of a narrow net: <= 16 coarse + <= 16 skip channels -> <= 16, MX-fp4, the coarse segment read through the fused
+    trilinear 2x (src/lp_f4up.cu:141-291). Grid data with a +6 per block: the blend is exact, outputs equal the oracle; random data with both
+    GroupNorms within the e2m1 staging tolerance."""
+    rng = np.random.default_rng(Cu + Cs * 5 + Co)
+    D, H, W = dims
+    N, S, Sc, G = 2, D * H * W, (D // 2) * (H // 2) * (W // 2), 4
+    xa = refnp.gen_exact(rng, (N, Cu, Sc), block=16); xa[np.abs(xa) == 6] = 6.0
+    xb = refnp.gen_exact(rng, (N, Cs, S), block=16 if Cs > 8 else 8); w = refnp.gen_exact(rng, (Co, Cu + Cs, 27), block=16)
+    qa, qb = orc.f32_to_mx(4, xa, N, Cu, Sc), orc.f32_to_mx(4, xb, N, Cs, S)
+    want, _ = orc.conv3(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=4, x2=qb, c_split=Cu, up=1)
+    got, _ = gpu_conv(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=4, x2=qb, c_split=Cu, up=1)
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-5
+    wq, _ = orc.conv3(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 4, cbits=4, x2=qb, c_split=Cu, up=1)
+    gq, _ = gpu_conv(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 4, cbits=4, x2=qb, c_split=Cu, up=1)
+    assert np.array_equal(gq, wq)
+    xa = rng.standard_normal((N, Cu, Sc)).astype(np.float32); xb = rng.standard_normal((N, Cs, S)).astype(np.float32)
+    w = (rng.standard_normal((Co, Cu + Cs, 27)) * np.sqrt(2.0 / ((Cu + Cs) * 27))).astype(np.float32)
+    qa, qb = orc.f32_to_mx(4, xa, N, Cu, Sc), orc.f32_to_mx(4, xb, N, Cs, S)
+    p = [rng.uniform(0.5, 1.5, Cu).astype(np.float32), rng.uniform(-.5, .5, Cu).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    p2 = [rng.uniform(0.5, 1.5, Cs).astype(np.float32), rng.uniform(-.5, .5, Cs).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    want, _ = orc.conv3(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=4, x2=qb, c_split=Cu, up=1, gp=orc.gn(*p, G), gp2=orc.gn(*p2, G))
+    got, _ = gpu_conv(qa, 4, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=4, x2=qb, c_split=Cu, up=1, gp=dev_gn(*p, G), gp2=dev_gn(*p2, G))
+    assert np.abs(got - want).max() / np.abs(want).max() < 3e-2
+
+
+def test_config2_full_size_down_and_decoder(gpu):
+    """The BASELINE's fp4 configuration at its stated sizes, exact operands, compared on sampled output planes with the oracle restricted to
+    them: the stride-2 down conv 128 -> 256 from 64^3, N 2 (MX-fp4 storage, e4m3 compute), and the decoder conv over [up(256 @ 32^3) | skip
+    (128 @ 64^3)] -> 128 (e2m1 compute); reruns byte-identical."""
+    rng = np.random.default_rng(222)
+    N, D = 2, 64
+    S, Sc = D ** 3, (D // 2) ** 3
+    x, w, b = exact_case(rng, N, 128, 256, S)
+    xq = orc.f32_to_mx(4, x, N, 128, S)
+    got, _ = gpu_conv(xq, 4, N, 128, D, D, D, w, b, 256, 4, stride=2)
+    got2, _ = gpu_conv(xq, 4, N, 128, D, D, D, w, b, 256, 4, stride=2)
+    assert np.array_equal(got, got2)
+    dec = orc.mx_to_f32(4, got, N, 256, Sc).reshape(N, 256, D // 2, D // 2, D // 2)
+    for z in (0, D // 4, D // 2 - 1):
+        want, _ = orc.conv3(xq, 4, N, 128, D, D, D, w, b, 256, 4, cbits=8, stride=2, z0=z, z1=z + 1, acc64=1)
+        wd = orc.mx_to_f32(4, want, N, 256, Sc).reshape(N, 256, D // 2, D // 2, D // 2)
+        assert np.array_equal(dec[:, :, z], wd[:, :, z]), z
+    del x, xq, got, got2, dec
+    xa = refnp.gen_exact(rng, (N, 256, Sc)); xa[np.abs(xa) == 6] = 6.0
+    xb = refnp.gen_exact(rng, (N, 128, S)); w = refnp.gen_exact(rng, (128, 384, 27))
+    qa, qb = orc.f32_to_mx(4, xa, N, 256, Sc), orc.f32_to_mx(4, xb, N, 128, S)
+    got, _ = gpu_conv(qa, 4, N, 384, D, D, D, w, None, 128, 4, cbits=4, x2=qb, c_split=256, up=1)
+    assert "conv3_wide_k" in lib.mi_last_kernel().decode()
+    dec = orc.mx_to_f32(4, got, N, 128, S).reshape(N, 128, D, D, D)
+    for z in (0, 31, D - 1):
+        want, _ = orc.conv3(qa, 4, N, 384, D, D, D, w, None, 128, 4, cbits=4, x2=qb, c_split=256, up=1, z0=z, z1=z + 1)
+        wd = orc.mx_to_f32(4, want, N, 128, S).reshape(N, 128, D, D, D)
+        assert np.array_equal(dec[:, :, z], wd[:, :, z]), z

@@ -5,7 +5,7 @@ import pytest
 
 import orc
 import unet_ref
-from gpuutil import DevBuf, LP, lib, to_mx, code_mismatch_fraction
+from gpuutil import DevBuf, LP, lib, to_mx, code_mismatch_fraction, shape5
 
 pytestmark = pytest.mark.gpu
 
@@ -20,7 +20,9 @@ def ct_like(rng, N, D, H, W):
 
 
 @pytest.mark.parametrize("bits,widths,dims,N,dn", [(8, [32, 64], (8, 16, 16), 2, 0), (8, [32, 64, 128], (16, 16, 32), 1, 0), (4, [32, 64], (8, 16, 16), 1, 0), (8, [16, 32], (8, 8, 16), 1, 0),
-                                                      (8, [32, 64, 128], (16, 16, 16), 1, 1)])
+                                                      (8, [32, 64, 128], (16, 16, 16), 1, 1),
+                                                      # the four levels of the BASELINE's U-Net: the 256-wide level, dec2.c1 at 384 -> 128 and the halved slices of the wide kernel inside the graph
+                                                      (8, [32, 64, 128, 256], (32, 32, 32), 1, 0), (4, [32, 64, 128, 256], (16, 32, 32), 1, 0)])
 def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N, dn):
     from ufsm_amd.unet import UNet, make_cfg
     rng = np.random.default_rng(sum(widths) + bits)
@@ -114,7 +116,14 @@ def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N, dn):
     # (tests/test_mx.c:32, :44). Bound the drift by that level; exact-operand networks (below) agree bit for bit. ----
     want, outs = unet_ref.forward(p, cin, widths, G, head_out, bits, xq, N, D, H, W, down_norm=dn)
     rel_l2 = np.linalg.norm(got - want) / np.linalg.norm(want)
-    assert rel_l2 < (0.08 if bits == 8 else 0.3), rel_l2
+    if bits == 8:
+        # twice the level two oracle evaluations settle at when their accumulators differ the way the MFMA's differs from fp32
+        # (0.04 - 0.046: tests/test_oracle_unet_drift.py; measured here 0.033 - 0.044)
+        assert rel_l2 < 0.08, rel_l2
+    else:
+        # e2m1 products are short enough for the matrix unit to sum exactly and the SiLU pre-pass rounds like the oracle's: the MX-fp4 net
+        # meets the whole-net bar free-running (measured 1e-7; a single flipped code would show as percents, see the drift study)
+        assert np.abs(got - want).max() / np.abs(want).max() < 1e-2, (rel_l2, np.abs(got - want).max() / np.abs(want).max())
     net.close()
 
 
@@ -338,4 +347,87 @@ def test_slab_inference_is_byte_identical(gpu, bits, dims, slab, attn):
     for name, (t, m, r) in whole.items():
         t2, m2, r2 = slabbed[name]
         assert np.array_equal(t2, t) and np.array_equal(m2, m) and np.array_equal(r2, r), name
+    net.close()
+
+
+
+def test_config3_full_size_forward_properties(gpu):
+    """The BASELINE's U-Net at its stated size (N 2 x 128^3, widths 32/64/128/256, MX-fp8): too large for a whole-graph oracle run, so
+    size-independent properties: byte-identical logits run to run, finite logits, every stored tensor's GroupNorm statistics equal the fp64
+    statistics of the values the conv produced within the fp32 partial sums' tolerance (checked against the decoded stored tensor: the
+    quantisation moves a mean by far less than 1e-2 of the standard deviation), and the two level-0 layers that dominate the forward - the
+    decoder conv over [up(64) | skip(32)] -> 32 and the head - compared with the oracle on three z planes, the oracle fed the device's own
+    input tensors and statistics."""
+    from ufsm_amd.unet import UNet, make_cfg
+    rng = np.random.default_rng(11)
+    N, D, widths, cin, head_out, G = 2, 128, [32, 64, 128, 256], 4, 8, 8
+    S = D ** 3
+    net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=8), N, D, D, D, seed=2)
+    p = net.params()
+    lay, n = unet_ref.param_layout(cin, widths, head_out)
+    for k, (off, shp) in lay.items():
+        if k.endswith(".gamma"):
+            p[off:off + shp[0]] = rng.uniform(0.7, 1.3, shp[0])
+        if k.endswith(".beta") or (k.endswith(".b") and k != "head.b"):
+            p[off:off + shp[0]] = rng.uniform(-0.2, 0.2, shp[0])
+    net.set_params(p)
+    ct = ct_like(rng, N, D, D, D).astype(np.float32)
+    x = np.zeros((N, cin, S), np.float32)
+    x[:, 0] = ((ct - ct.mean()) / ct.std()).reshape(N, S)
+    yy, xx = np.meshgrid(np.arange(D) - 300.0, np.arange(D) + 200.0, indexing="ij")
+    r = np.sqrt(yy * yy + xx * xx) + 1e-6
+    x[:, 2] = np.broadcast_to((yy / r)[None], (D, D, D)).reshape(1, S); x[:, 3] = np.broadcast_to((xx / r)[None], (D, D, D)).reshape(1, S)
+    dxq = to_mx(8, x); del x, ct
+    dlog = DevBuf(N * head_out * S * 4)
+    assert net.forward_x(dxq.ptr, dlog.ptr) == 0
+    LP.check()
+    got = dlog.to_numpy(np.float32, (N, head_out, S))
+    assert np.isfinite(got).all()
+    assert net.forward_x(dxq.ptr, dlog.ptr) == 0
+    assert np.array_equal(got, dlog.to_numpy(np.float32, (N, head_out, S)))
+    outs = {name: (k, ptr, shp) for k, (name, ptr, shp) in enumerate(net.layer_outs())}
+    assert set(outs) == {"%s%d.c%d" % (b, i, c) for b in ("enc",) for i in range(4) for c in (1, 2)} | {"dec%d.c%d" % (i, c) for i in range(3) for c in (1, 2)} | {"down%d" % i for i in range(3)}
+
+    def fetch(name):
+        k, ptr, shp = outs[name]
+        nb = lib.lp_mx8_bytes(shp[0], shp[1], shp[2] * shp[3] * shp[4])
+        buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+        g, mp, rp = net.layer_stats(k)
+        m = np.empty(N * g, np.float32); rr = np.empty(N * g, np.float32)
+        if g:
+            lib.mi_d2h(m.ctypes.data, mp, m.nbytes); lib.mi_d2h(rr.ctypes.data, rp, rr.nbytes)
+        return buf, shp, g, m, rr
+
+    Pm = lambda key: np.ascontiguousarray(p[lay[key][0]:lay[key][0] + int(np.prod(lay[key][1]))].reshape(lay[key][1]))
+    for name in outs:                                              # statistics of every conv output against its decoded stored tensor
+        if name.startswith("down"):
+            continue
+        buf, shp, g, m, rr = fetch(name)
+        Sl = shp[2] * shp[3] * shp[4]
+        sums = np.zeros((N, g, 2), np.float64)
+        orc.lib().orc_gn_sums_mx(8, orc.ptr(buf), N, shp[1], g, Sl, orc.ptr(sums), 0, Sl)
+        mo = np.zeros(N * g, np.float32); ro = np.zeros(N * g, np.float32)
+        orc.lib().orc_gn_finalize(orc.ptr(sums), N * g, (shp[1] // g) * Sl, 1e-5, orc.ptr(mo), orc.ptr(ro))
+        assert np.all(np.abs(m - mo) * ro < 1e-2) and np.allclose(rr, ro, rtol=1e-2), name
+    # dec0.c1 on three planes: inputs dec1.c2 (coarse, 64 channels at 64^3) and enc0.c2 (skip), each under its block's second norm
+    cu, cs, c1 = fetch("dec1.c2"), fetch("enc0.c2"), fetch("dec0.c1")
+    gu = orc.gn(Pm("dec1.n2.gamma"), Pm("dec1.n2.beta"), cu[3], cu[4], cu[2]); gs = orc.gn(Pm("enc0.n2.gamma"), Pm("enc0.n2.beta"), cs[3], cs[4], cs[2])
+    dec = orc.mx_to_f32(8, c1[0], N, 32, S).reshape(N, 32, D, D * D)
+    for z in (0, 77, D - 1):
+        want, _ = orc.conv3(cu[0], 3, N, 96, D, D, D, Pm("dec0.c1.w"), Pm("dec0.c1.b"), 32, 3, x2=cs[0], c_split=64, up=1, gp=gu, gp2=gs, z0=z, z1=z + 1)
+        wd = orc.mx_to_f32(8, want, N, 32, S).reshape(N, 32, D, D * D)[:, :, z]
+        diff = dec[:, :, z] != wd
+        assert diff.mean() < 0.02 and np.all(np.abs(dec[:, :, z] - wd)[diff] <= 0.26 * np.maximum(np.abs(wd), np.abs(dec[:, :, z]))[diff] + 2.0 ** -7 * np.abs(wd).max()), (z, diff.mean())
+    # the head on three planes of the device's own dec0.c2
+    c2 = fetch("dec0.c2")
+    g2 = orc.gn(Pm("dec0.n2.gamma"), Pm("dec0.n2.beta"), c2[3], c2[4], c2[2])
+    hw = np.ascontiguousarray(Pm("head.w").reshape(head_out, 32)); hb = Pm("head.b")
+    rows = orc.mx_to_f32(8, c2[0], N, 32, S).reshape(N, 32, D, D * D)
+    for z in (0, 64, D - 1):
+        sl = np.ascontiguousarray(rows[:, :, z])                   # [N][32][D*D] planes of one z -> a small MX tensor (lossless: already on the grid)
+        q = orc.f32_to_mx(8, sl, N, 32, D * D)
+        want = np.zeros((N, head_out, D * D), np.float32)
+        orc.lib().orc_conv1_mx(8, orc.ptr(q), N, 32, D * D, orc.ptr(hw), orc.ptr(hb), head_out, g2, orc.ptr(want))
+        gz = got.reshape(N, head_out, D, D * D)[:, :, z]
+        assert np.abs(gz - want).max() / np.abs(want).max() < 1e-4, z
     net.close()
