@@ -143,6 +143,17 @@ int mi_conv_fwd_gn(int bits, const void *x, int xbf, shape5 xs, const float *w, 
    stream it runs on and clears the totals; read returns the total milliseconds so far and the number of launches (synchronises) */
 void mi_kernel_timing(int on);
 double mi_kernel_timing_read(long *launches);
+/* No counterpart in the reference. lp_conv_fwd_f8 / lp_conv_fwd_f4 (bits 8 / 4) for callers that cannot allocate device memory: code under
+   HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. Same arguments, same kernels and bit-identical results, but every
+   byte of scratch (prepared weights, re-staged operands, statistics partials, the constant page) comes from one fixed device array of
+   mi_conv_static_scratch_bytes() = 64 MiB that each GPU the library runs on holds until the process ends; the call makes no hipMalloc /
+   hipFree (split_t.wkey is ignored: weights are prepared per call). A call whose scratch could exceed the array prints what it needs and
+   returns -1 with nothing launched (an input already in the compute format without GroupNorm needs only its weights: any size fits;
+   with GroupNorm or another storage format the re-staged operand must fit: e.g. 128 channels at 2 x 32^3). Calls on one GPU share the
+   array: calls that overlap on a GPU (two host threads, two streams) race; nothing in it needs clearing between calls. */
+int mi_conv_fwd_static(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp);
+size_t mi_conv_static_scratch_bytes(void);
+long mi_alloc_count(void);                     /* device allocations made by this library so far (scratch growth, memo entries, mi_malloc): diagnostics */
 /* name of the conv kernel variant the last conv call on this thread launched (diagnostics / tests), "" if none */
 const char *mi_last_kernel(void);
 #ifdef __cplusplus

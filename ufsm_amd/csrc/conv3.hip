@@ -201,12 +201,12 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     const size_t wq_bytes = (size_t)NP * nmt_all * 2048, wsc_bytes = (size_t)NP * nmt_all * 256;
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
-    if (sp.wkey) {                                     // memo entries of this layout: nbt = -CP
+    if (sp.wkey && !mi_ws_arena_on()) {                // memo entries of this layout: nbt = -CP (the entry point that must not allocate prepares per call)
         std::lock_guard<std::mutex> lk(g_wmemo_mu);
         for (auto &m : g_wmemo)
             if (m.key == sp.wkey && m.w == w && m.fmt == 8 && m.Co == cout && m.Ci == Ci && m.nbt == -CP - 1 && m.nmt_all == nmt_all && m.dev == dev) { wq = m.wq; wsc = m.wsc; have = true; break; }
         if (!have) {
-            MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes));
+            MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes)); mi_count_alloc(); mi_count_alloc();
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
             g_wmemo.push_back(wmemo_t{sp.wkey, w, 8, cout, Ci, Ci, -CP - 1, 0, nmt_all, dev, 0, wq, wsc});
         }
@@ -216,13 +216,15 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     a.stat_ch = osum && (cout / Go) % 4 ? 1 : 0;
     if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * (a.stat_ch ? 32 : MT * 8) * 2 * sizeof(float));
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    if (g_ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
+    const bool ktime = g_ktime && !mi_ws_arena_on();
+    if (ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
     conv3_stem_launch(CP, MT, ybf == 3 ? 8 : ybf == 4 ? 4 : 0, a, smem);
-    if (g_ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
+    if (ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
     if (osum) conv_stats_reduce(who, a, MT, sp, osum);
     return 0;
 }
 
+static thread_local const uint8_t *g_static_zpage = nullptr;     // the constant page of the calling thread's conv when it runs on the fixed scratch
 static thread_local int g_split = -1;       // mi_conv_split: the calling thread's tile count below which 128-channel slices are halved (-1: the default)
 extern "C" void mi_conv_split(int tiles) { g_split = tiles; }
 static int split_s2_env() { static int v = -1; if (v < 0) v = getenv("MI_CONV_SPLIT_S2") ? atoi(getenv("MI_CONV_SPLIT_S2")) : 1; return v; }      // tuning knob: 0 keeps four channel tiles
@@ -364,15 +366,19 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     a.red_o = (unsigned)smem; smem += 1024;                                     // statistics scratch
     if (big || a.areg) {
         // rows and scale bytes of positions outside the volume: 64 zero bytes, then 64 bytes of value 1; one page per device, kept for the process
+        // (the entry point that must not allocate keeps its own at the head of its fixed scratch)
         static uint8_t *zpage[8];
         int dv = 0; MIRT(hipGetDevice(&dv)); dv &= 7;
-        if (!zpage[dv]) {
-            uint8_t init[128]; memset(init, 0, 64); memset(init + 64, 1, 64);
-            MIRT(hipMalloc((void **)&zpage[dv], 128));
-            if (!zpage[dv]) mi_die("%s: no device memory for the constant page", who);
-            MIRT(hipMemcpy(zpage[dv], init, 128, hipMemcpyHostToDevice));
+        if (mi_ws_arena_on()) a.zpage = g_static_zpage;
+        else {
+            if (!zpage[dv]) {
+                uint8_t init[128]; memset(init, 0, 64); memset(init + 64, 1, 64);
+                MIRT(hipMalloc((void **)&zpage[dv], 128)); mi_count_alloc();
+                if (!zpage[dv]) mi_die("%s: no device memory for the constant page", who);
+                MIRT(hipMemcpy(zpage[dv], init, 128, hipMemcpyHostToDevice));
+            }
+            a.zpage = zpage[dv];
         }
-        a.zpage = zpage[dv];
     }
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
     a.ntx = (Wo + 15) / 16; a.nty = (Ho + 7) / 8; a.ntz = (Do + TZ - 1) / TZ;
@@ -389,12 +395,12 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const int CxP = (Cx + 31) / 32 * 32;
     int dev = 0; MIRT(hipGetDevice(&dev));
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
-    if (sp.wkey) {
+    if (sp.wkey && !mi_ws_arena_on()) {
         std::lock_guard<std::mutex> lk(g_wmemo_mu);
         for (auto &m : g_wmemo)
             if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == memoCB && m.nmt_all == nmt_all && m.dev == dev && m.lay == (big ? MT : 0)) { wq = m.wq; wsc = m.wsc; have = true; break; }
         if (!have) {
-            MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes));
+            MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes)); mi_count_alloc(); mi_count_alloc();
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
             MIRT(hipMemsetAsync(wq, 0, wq_bytes, 0)); MIRT(hipMemsetAsync(wsc, 0, wsc_bytes, 0));
             g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, memoCB, nmt_all, dev, big ? MT : 0, wq, wsc});
@@ -412,10 +418,11 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const bool epi = act != 0;
     const int out = ybf == 3 ? 8 : ybf == 4 ? 4 : 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
-    if (g_ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
+    const bool ktime = g_ktime && !mi_ws_arena_on();
+    if (ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
     if (fmt == 8) { if (out == 8) conv3_launch_f8_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f8_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f8_o0(stride, epi, MT, NT, a, smem); }
     else { if (out == 8) conv3_launch_f4_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f4_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f4_o0(stride, epi, MT, NT, a, smem); }
-    if (g_ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
+    if (ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
     if (osum) conv_stats_reduce(who, a, MT, sp, osum);
     return 0;
 }
@@ -462,4 +469,69 @@ extern "C" int mi_conv_fwd_fused(int bits, const void *x, int xbf, shape5 xs, co
     if (bits != 8 && bits != 4) mi_die("mi_conv_fwd_fused: compute format %d (8 or 4)", bits);
     if (act < 0 || act > 3 || (!act && ep_a) || (!ep_a != !ep_b)) mi_die("mi_conv_fwd_fused: activation %d / affine arguments", act);
     return conv_dispatch("mi_conv_fwd_fused", bits, 1, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, ep_a, ep_b, act);
+}
+
+// ---- the stride-1 convs for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc) ----
+// Every byte of device memory the conv needs beyond its inputs and outputs - prepared weights, re-staged operands, the coarse rows of a fused
+// upsample, per-tile statistics partials, the constant page of out-of-volume rows - is carved from one file-scope device array. The array is a
+// host-side stand-in by name: its device address is taken once per device and only that address is used from then on.
+#define MI_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+static __device__ __align__(256) unsigned char scratch[MI_STATIC_SCRATCH_BYTES];
+static unsigned char *g_scratch_ptr[8];        // per device: the address of that device's copy of the array
+static std::mutex g_scratch_mu;
+extern "C" size_t mi_conv_static_scratch_bytes(void) { return MI_STATIC_SCRATCH_BYTES; }
+// an upper bound of what conv_dispatch will request from mi_ws for this call, following its choices (every request rounded up to 256 bytes)
+static size_t conv_scratch_bound(int fmt, const void *x2, int xbf, shape5 xs, int cout, gnp_t gp, const double *osum, split_t sp) {
+    auto al = [](size_t n) { return ((n + 255) & ~(size_t)255) + 256; };
+    const int Ci = xs.c, Cx = x2 ? sp.c_split : Ci, C2 = Ci - Cx, N = xs.n, D = sp.Di ? sp.Di : xs.d;
+    if (fmt == 4 && Ci <= 8) fmt = 8;
+    const size_t S = (size_t)D * xs.h * xs.w, So = (size_t)xs.d * xs.h * xs.w;
+    const int nmt_all = (cout + 31) / 32, fdt = fmt == 8 ? 3 : 4;
+    const size_t tiles = (size_t)((xs.w + 15) / 16) * ((xs.h + 7) / 8) * xs.d * nmt_all * N;           // one-plane tiles of one channel tile: no launch has more
+    size_t need = 256;                                              // the constant page
+    if (Ci <= 16 && !x2 && fmt == 8) need += al((size_t)9 * nmt_all * 2048) + al((size_t)9 * nmt_all * 256);      // the tap-packed kernels' weights
+    const int nbt = (Cx + 31) / 32 + (x2 ? (C2 + 31) / 32 : 0);
+    need += al(((size_t)(27 * nbt + 1) / 2 + nbt + 16) * nmt_all * 2304) + al(((size_t)(27 * nbt + 1) / 2 + nbt + 16) * nmt_all * 256);
+    const bool s2g = x2 && sp.gp2.G;
+    for (int s = 0; s < (x2 ? 2 : 1); s++) {
+        const gnp_t g = s2g ? (s ? sp.gp2 : gp) : gp;
+        const bool upseg = s == 0 && sp.up, direct = xbf == fdt && !(g.G > 0) && !upseg;
+        const int C = s ? C2 : Cx;
+        if (!direct) need += al((size_t)N * ((C + 31) / 32) * S * 33);
+        if (upseg) need += al((size_t)N * ((C + 31) / 32) * (S / 8) * 33);
+    }
+    if (osum) need += al(tiles * 32 * 2 * sizeof(float));
+    (void)So;
+    return need;
+}
+static int conv_fwd_static(const char *who, int fmt, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp) {
+    int dv = 0; MIRT(hipGetDevice(&dv)); dv &= 7;
+    {   // set-up, once per device with that device current: the array's address on this device, and the constant page at its head
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        if (!g_scratch_ptr[dv]) {
+            unsigned char *ptr = nullptr;
+            const hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !ptr) { fprintf(stderr, "%s: the fixed scratch has no address on device %d: %s\n", who, dv, hipGetErrorString(e)); return -2; }
+            uint8_t init[128]; memset(init, 0, 64); memset(init + 64, 1, 64);
+            if (hipMemcpy(ptr, init, 128, hipMemcpyHostToDevice) != hipSuccess) { fprintf(stderr, "%s: cannot initialise the fixed scratch on device %d\n", who, dv); return -2; }
+            g_scratch_ptr[dv] = ptr;
+        }
+    }
+    const size_t need = conv_scratch_bound(fmt, sp.x2, xbf, xs, cout, gp, osum, sp);
+    if (need > MI_STATIC_SCRATCH_BYTES) {
+        fprintf(stderr, "%s: this call needs up to %zu bytes of scratch (prepared weights, re-staged operands, statistics partials); the fixed scratch holds %zu. "
+                        "Use lp_conv_fwd_f8 / lp_conv_fwd_f4, which allocate, or pass an input that is already in the compute format without GroupNorm\n", who, need, (size_t)MI_STATIC_SCRATCH_BYTES);
+        return -1;
+    }
+    unsigned char *ptr = g_scratch_ptr[dv];
+    g_static_zpage = ptr;                                          // bytes [0, 128): zero rows, then scale bytes of value 1
+    mi_ws_arena(ptr + 256, MI_STATIC_SCRATCH_BYTES - 256);         // everything else is carved per call, and fully written before it is read
+    const int rc = conv_dispatch(who, fmt, 1, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, nullptr, nullptr, 0);
+    mi_ws_arena(nullptr, 0);
+    g_static_zpage = nullptr;
+    return rc;
+}
+extern "C" int mi_conv_fwd_static(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp) {
+    if (bits != 8 && bits != 4) { fprintf(stderr, "mi_conv_fwd_static: compute format %d (8 or 4)\n", bits); return -1; }
+    return conv_fwd_static("mi_conv_fwd_static", bits, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp);
 }

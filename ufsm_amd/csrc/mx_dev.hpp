@@ -234,6 +234,9 @@ void mi_post_error(hipError_t e, const char *file, int line);
 #define MICK() do { hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)
 #define MIRT(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)
 void *mi_ws(int slot, size_t bytes);        // per-device grow-on-demand scratch (the reference's nn_ws, src/nn_core.cu:751)
+void mi_ws_arena(void *base, size_t cap);   // the calling thread's scratch requests come from this fixed region until mi_ws_arena(nullptr, 0)
+bool mi_ws_arena_on(void);
+void mi_count_alloc(void);                  // bookkeeping: one more device allocation made by the library
 enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_UPCOARSE = 5, MI_WS_GEMM = 6, MI_WS_ATTN = 7, MI_WS_NSLOTS = 8 };
 static inline unsigned nblk_(size_t n, unsigned b) { return (unsigned)((n + b - 1) / b); }
 [[noreturn]] void mi_die(const char *fmt, ...);

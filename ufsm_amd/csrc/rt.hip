@@ -35,7 +35,7 @@ extern "C" int mi_init(int device) {
 }
 extern "C" void *mi_malloc(size_t bytes) {
     void *p = nullptr;
-    hipError_t e = hipMalloc(&p, bytes ? bytes : 1);
+    hipError_t e = hipMalloc(&p, bytes ? bytes : 1); mi_count_alloc();
     if (e != hipSuccess) mi_die("mi_malloc: %zu bytes: %s", bytes, hipGetErrorString(e));
     return p;
 }
@@ -49,12 +49,27 @@ extern "C" void mi_sync(void) { MIRT(hipDeviceSynchronize()); }
 
 // per-device scratch: grow on demand, contents valid until the next request of the same slot on the same device
 static void *g_ws[8][MI_WS_NSLOTS]; static size_t g_wscap[8][MI_WS_NSLOTS];
+// device allocations this library has made so far (scratch growth, memo entries, mi_malloc): lets a caller check that a code path made none
+static long g_nalloc = 0;
+void mi_count_alloc(void) { __atomic_add_fetch(&g_nalloc, 1, __ATOMIC_RELAXED); }
+extern "C" long mi_alloc_count(void) { return __atomic_load_n(&g_nalloc, __ATOMIC_RELAXED); }
+// a fixed region the calling thread's scratch requests are carved from instead (the entry point that must not allocate): requests are
+// handed out back to back, 256-byte aligned; one that does not fit ends the process with a message (the entry point checks its bound first)
+static thread_local unsigned char *g_arena = nullptr; static thread_local size_t g_arena_off = 0, g_arena_cap = 0;
+void mi_ws_arena(void *base, size_t cap) { g_arena = (unsigned char *)base; g_arena_off = 0; g_arena_cap = base ? cap : 0; }
+bool mi_ws_arena_on(void) { return g_arena != nullptr; }
 void *mi_ws(int slot, size_t bytes) {
+    if (g_arena) {
+        const size_t need = (bytes + 255) & ~(size_t)255;
+        if (g_arena_off + need > g_arena_cap) mi_die("mi_ws: slot %d needs %zu bytes, %zu of the fixed scratch's %zu are taken", slot, need, g_arena_off, g_arena_cap);
+        void *p = g_arena + g_arena_off; g_arena_off += need;
+        return p;
+    }
     int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
     if (bytes > g_wscap[d][slot]) {
         if (g_ws[d][slot]) { MIRT(hipDeviceSynchronize()); MIRT(hipFree(g_ws[d][slot])); }
         const size_t cap = bytes + bytes / 8 + 4096;
-        hipError_t e = hipMalloc(&g_ws[d][slot], cap);
+        hipError_t e = hipMalloc(&g_ws[d][slot], cap); mi_count_alloc();
         if (e != hipSuccess) mi_die("mi_ws: slot %d, %zu bytes: %s", slot, cap, hipGetErrorString(e));
         g_wscap[d][slot] = cap;
     }

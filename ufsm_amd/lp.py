@@ -93,6 +93,9 @@ _PROTOS = {
     "mi_event_destroy": (None, [_P]),
     "mi_conv_fwd_fused": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, _P, _P, _I, gnp_t, _P, _I, split_t]),
     "mi_conv_fwd_gn": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t, C.c_float, _P, _P]),
+    "mi_conv_fwd_static": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t]),
+    "mi_conv_static_scratch_bytes": (_Z, []),
+    "mi_alloc_count": (C.c_long, []),
     "mi_kernel_timing": (None, [_I]),
     "mi_kernel_timing_read": (C.c_double, [C.POINTER(C.c_long)]),
     "mi_last_kernel": (C.c_char_p, []),
