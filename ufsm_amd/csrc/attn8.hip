@@ -22,43 +22,53 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // accumulator elements 4 q + c, which are the block's keys 8 q + 4 h + c.
 __host__ __device__ __forceinline__ int a8_slot_token(int k) { return 8 * ((k >> 2) & 3) + 4 * (k >> 4) + (k & 3); }
 
-// row-quantised q / k: thread per (head, row, 32-dim block); src fp16 [H][Tp][48] (token i of sequence s in row s S + i),
-// dst [H][R][64] e4m3 + scales [H][R][2] (dims 0..31, dims 32..47 zero-padded), R = nseq Sp
-__global__ void __launch_bounds__(256) a8_rq_k(const __half *__restrict__ src, uint8_t *__restrict__ dst, uint8_t *__restrict__ sc, int H, int nseq, int S, int Sp, long long Tp) {
-    const long long R = (long long)nseq * Sp, i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
-    if (i >= (long long)H * R * 2) return;
-    const int kb = (int)(i & 1); const long long hr = i >> 1; const int h = (int)(hr / R); const long long row = hr % R;
-    const int seq = (int)(row / Sp), ii = (int)(row % Sp), n = kb ? HD - 32 : 32;
-    float v[32];
-    const __half *s = src + ((size_t)h * Tp + (size_t)seq * S + min(ii, S - 1)) * HD + 32 * kb;
+// ---- operand quantisation (src/lp_attn8.cu:29-76): the fp16 head-major pack [3][H][Tp][48] -> e4m3 blocks of 32 with one E8M0 scale each ----
+// q and k rows: dst [H][R][64] e4m3 + scales [H][R][2], R = nseq Sp rows (token i of sequence s in row s Sp + i, rows past S zero). A row's 64
+// output bytes are four 16-byte quarters: dims 0-15 and 16-31 (block 0), 32-47 and sixteen zeros (block 1). Four neighbouring lanes own a row,
+// each one quarter: 32 bytes of halves in (two 16-byte loads), 16 bytes of codes out, the block's amax through one exchange with the
+// partner quarter. blockIdx.y: 0 the queries, 1 the keys.
+__global__ void __launch_bounds__(256) a8_rows_k(const __half *__restrict__ src_q, uint8_t *__restrict__ dst_q, uint8_t *__restrict__ sc_q, int H, int nseq, int S, int Sp, long long Tp, size_t part_src, size_t part_dst, size_t part_sc) {
+    const long long R = (long long)nseq * Sp, i = blockIdx.x * 256ll + threadIdx.x, hr = i >> 2;
+    if (hr >= (long long)H * R) return;
+    const int qt = (int)(i & 3), h = (int)(hr / R); const long long row = hr - (long long)h * R;
+    const int seq = (int)(row / Sp), ii = (int)(row - (long long)seq * Sp);
+    const __half *src = src_q + blockIdx.y * part_src; uint8_t *dst = dst_q + blockIdx.y * part_dst, *sc = sc_q + blockIdx.y * part_sc;
+    float v[16];
 #pragma unroll
-    for (int j = 0; j < 32; j++) v[j] = ii < S && j < n ? __half2float(s[j < n ? j : 0]) : 0.f;
-    unsigned codes[8];
-    const unsigned sb = d_quant_row<8, false>(v, 32, codes);
-    uint4 *o = (uint4 *)(dst + ((size_t)h * R + row) * 64 + 32 * kb);
-    o[0] = make_uint4(codes[0], codes[1], codes[2], codes[3]); o[1] = make_uint4(codes[4], codes[5], codes[6], codes[7]);
-    sc[((size_t)h * R + row) * 2 + kb] = (uint8_t)sb;
-}
-// transposed v: workgroup per (head, 32-token block), 64 threads; dst [H][48][R] in slot order + scales [H][48][R / 32]
-__global__ void __launch_bounds__(64) a8_tq_k(const __half *__restrict__ src, uint8_t *__restrict__ dst, uint8_t *__restrict__ sc, int H, int nseq, int S, int Sp, long long Tp) {
-    const long long R = (long long)nseq * Sp; const int nb = (int)(R / 32), h = blockIdx.x / nb, b = blockIdx.x % nb;
-    const long long r0 = (long long)b * 32; const int seq = (int)(r0 / Sp), i0 = (int)(r0 % Sp);
-    __shared__ float t[32][HD + 1];
-    for (int e = threadIdx.x; e < 32 * HD; e += blockDim.x) {
-        const int r = e / HD, d = e % HD, ii = i0 + r;
-        t[r][d] = ii < S ? __half2float(src[((size_t)h * Tp + (size_t)seq * S + ii) * HD + d]) : 0.f;
+    for (int k = 0; k < 16; k++) v[k] = 0.f;
+    if (ii < S && qt < 3) {
+        const uint4 *p = (const uint4 *)(src + ((size_t)h * Tp + (size_t)seq * S + ii) * HD + 16 * qt);
+        const uint4 a = p[0], b = p[1];
+        const unsigned w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) { const __half2 hh = *(const __half2 *)&w[k]; v[2 * k] = __low2float(hh); v[2 * k + 1] = __high2float(hh); }
     }
-    __syncthreads();
-    const int d = threadIdx.x;
-    if (d >= HD) return;
+    float am = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(v[k]));
+    am = fmaxf(am, __shfl_xor(am, 1));                             // quarters (0, 1) and (2, 3) are the two blocks
+    const int e = d_mx_exp(am, MI_INVQ8);
+    *(uint4 *)(dst + (size_t)hr * 64 + 16 * qt) = make_uint4(d_enc4_e4m3(v[0], v[1], v[2], v[3], e), d_enc4_e4m3(v[4], v[5], v[6], v[7], e), d_enc4_e4m3(v[8], v[9], v[10], v[11], e), d_enc4_e4m3(v[12], v[13], v[14], v[15], e));
+    if (!(qt & 1)) sc[(size_t)hr * 2 + (qt >> 1)] = (uint8_t)(e + 127);
+}
+// transposed v: dst [H][48][R] with the 32 tokens of a block in slot order + scales [H][48][R / 32]. One wavefront per (head, 32-token block),
+// lane d < 48 owns dim d: it gathers the block's 32 values of its dim (each gather reads one token's 96 contiguous bytes across the lanes),
+// quantises them as one block and writes 32 contiguous bytes.
+__global__ void __launch_bounds__(256) a8_vt_k(const __half *__restrict__ src, uint8_t *__restrict__ dst, uint8_t *__restrict__ sc, int H, int nseq, int S, int Sp, long long Tp) {
+    const long long R = (long long)nseq * Sp, nb = R / 32, wb = blockIdx.x * 4ll + (threadIdx.x >> 6);
+    const int d = threadIdx.x & 63;
+    if (wb >= (long long)H * nb || d >= HD) return;
+    const int h = (int)(wb / nb); const long long b = wb - (long long)h * nb, r0 = b * 32;
+    const int seq = (int)(r0 / Sp), i0 = (int)(r0 - (long long)seq * Sp);       // (Sp is a multiple of 64: a block never straddles two sequences)
+    const __half *base = src + ((size_t)h * Tp + (size_t)seq * S) * HD + d;
     float v[32];
 #pragma unroll
-    for (int k = 0; k < 32; k++) v[k] = t[a8_slot_token(k)][d];
+    for (int k = 0; k < 32; k++) { const int ii = i0 + a8_slot_token(k); v[k] = ii < S ? __half2float(base[(size_t)ii * HD]) : 0.f; }
     unsigned codes[8];
     const unsigned sb = d_quant_row<8, false>(v, 32, codes);
     uint4 *o = (uint4 *)(dst + ((size_t)h * HD + d) * R + r0);
     o[0] = make_uint4(codes[0], codes[1], codes[2], codes[3]); o[1] = make_uint4(codes[4], codes[5], codes[6], codes[7]);
-    sc[((size_t)h * HD + d) * (R / 32) + b] = (uint8_t)sb;
+    sc[((size_t)h * HD + d) * nb + b] = (uint8_t)sb;
 }
 
 __device__ __forceinline__ float a8_xor32f(float x, int h) {
@@ -189,10 +199,9 @@ extern "C" int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom 
     if (!base) return -1;
     uint8_t *q8 = base, *k8 = q8 + al(rq), *qs = k8 + al(rq), *ks = qs + al(rqs), *vt = ks + al(rqs), *vts = vt + al(tq);
     const __half *Qh = (const __half *)qkvh, *Kh = Qh + (size_t)H * Tp * HD, *Vh = Kh + (size_t)H * Tp * HD;
-    const unsigned gq = nblk_((size_t)H * R * 2, 256);
-    a8_rq_k<<<gq, 256>>>(Qh, q8, qs, H, g->nseq, g->S, Sp, Tp);
-    a8_rq_k<<<gq, 256>>>(Kh, k8, ks, H, g->nseq, g->S, Sp, Tp);
-    a8_tq_k<<<(unsigned)(H * (R / 32)), 64>>>(Vh, vt, vts, H, g->nseq, g->S, Sp, Tp);
+    // (queries and keys in one launch: their sources, code planes and scale planes each lie one fixed stride apart)
+    a8_rows_k<<<dim3(nblk_((size_t)H * R * 4, 256), 2), 256>>>(Qh, q8, qs, H, g->nseq, g->S, Sp, Tp, (size_t)(Kh - Qh), (size_t)(k8 - q8), (size_t)(ks - qs));
+    a8_vt_k<<<nblk_((size_t)H * (R / 32), 4), 256>>>(Vh, vt, vts, H, g->nseq, g->S, Sp, Tp);
     // few query tiles (a 16^3 bottleneck: 129 per head): one wavefront per workgroup, so that every CU gets some
     const int nw = (size_t)((g->S + 127) / 128) * H * g->nseq >= 512 ? 4 : 1;
     const dim3 grid((unsigned)((g->S + 32 * nw - 1) / (32 * nw)), (unsigned)H, (unsigned)g->nseq);

@@ -8,107 +8,193 @@
 #define HD AT_HD
 #define FT 64
 
-// LayerNorm: one wavefront per row; two passes over the row (mean, then centred squares), as the reference
-__global__ void __launch_bounds__(256) at_ln_k(const float *__restrict__ x, const float *__restrict__ g, const float *__restrict__ b, float *__restrict__ y,
-                                               float *__restrict__ mean, float *__restrict__ rstd, long long T, int C) {
-    const long long row = (blockIdx.x * (long long)blockDim.x + threadIdx.x) >> 6; const int lane = threadIdx.x & 63;
+// ---- LayerNorm (src/nn_attn.cu:150-168): y = (x - mean) rstd g + b, mean and biased variance of the row, eps 1e-5 ----
+// One wavefront per token row, the row resident in registers: lane l holds the float4 chunks l, l + 64, ... (NV of them), so the row is read
+// from HBM once (16-byte accesses, a wavefront 1 KiB contiguous), the mean and the centred sum of squares are two butterfly reductions over
+// register values, and the result leaves as 16-byte stores.
+template <int NV>
+__global__ void __launch_bounds__(256) ln_row_k(const float4 *__restrict__ x, const float *__restrict__ g, const float *__restrict__ b, float4 *__restrict__ y,
+                                                float *__restrict__ mean, float *__restrict__ rstd, long long T, int C4) {
+    const long long row = blockIdx.x * 4ll + (threadIdx.x >> 6); const int lane = threadIdx.x & 63;
     if (row >= T) return;
-    const float *xr = x + row * C;
+    const float4 *xr = x + row * C4;
+    float4 v[NV];
     float s = 0.f;
-    for (int c = lane; c < C; c += 64) s += xr[c];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = lane + 64 * i;
+        v[i] = c < C4 ? xr[c] : make_float4(0.f, 0.f, 0.f, 0.f);
+        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+#pragma unroll
     for (int o = 32; o; o >>= 1) s += __shfl_xor(s, o);
-    const float m = s / C; float q = 0.f;
-    for (int c = lane; c < C; c += 64) { const float d = xr[c] - m; q += d * d; }
+    const float C = (float)(4 * C4), m = s / C;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        if (lane + 64 * i < C4) {
+            v[i].x -= m; v[i].y -= m; v[i].z -= m; v[i].w -= m;
+            q += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+        }
+    }
+#pragma unroll
     for (int o = 32; o; o >>= 1) q += __shfl_xor(q, o);
     const float r = 1.f / sqrtf(q / C + 1e-5f);
-    for (int c = lane; c < C; c += 64) y[row * C + c] = (xr[c] - m) * r * g[c] + b[c];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        const int c = lane + 64 * i;
+        if (c < C4) {
+            // (gains and shifts sit at arbitrary offsets of the flat parameter vector: dword loads)
+            const float4 gg = make_float4(g[4 * c], g[4 * c + 1], g[4 * c + 2], g[4 * c + 3]), bb = make_float4(b[4 * c], b[4 * c + 1], b[4 * c + 2], b[4 * c + 3]);
+            y[row * C4 + c] = make_float4(fmaf(v[i].x * r, gg.x, bb.x), fmaf(v[i].y * r, gg.y, bb.y), fmaf(v[i].z * r, gg.z, bb.z), fmaf(v[i].w * r, gg.w, bb.w));
+        }
+    }
     if (!lane) { if (mean) mean[row] = m; if (rstd) rstd[row] = r; }
 }
 extern "C" void at_ln_fwd(const float *x, const float *g, const float *b, float *y, float *mean, float *rstd, long T, int C) {
     if (T <= 0) return;
-    at_ln_k<<<nblk_((size_t)T * 64, 256), 256>>>(x, g, b, y, mean, rstd, T, C);
+    if (C <= 0 || (C & 3) || C > 2048 || (((uintptr_t)x | (uintptr_t)y) & 15)) mi_die("at_ln_fwd: rows of %d channels (a multiple of 4, at most 2048, rows 16-byte aligned)", C);
+    const int C4 = C / 4, nv = (C4 + 63) / 64;
+    const unsigned grid = nblk_((size_t)T, 4);
+#define LN(NV) ln_row_k<NV><<<grid, 256>>>((const float4 *)x, g, b, (float4 *)y, mean, rstd, T, C4)
+    if (nv <= 1) LN(1); else if (nv <= 2) LN(2); else if (nv <= 4) LN(4); else LN(8);
+#undef LN
     MICK();
 }
-__global__ void __launch_bounds__(256) at_glu_k(const float *__restrict__ h, float *__restrict__ gg, long long T, int F) {
-    const long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
-    if (i >= T * F) return;
-    const long long t = i / F; const int f = (int)(i % F);
-    const float a = h[t * 2 * F + f], b = h[t * 2 * F + F + f];
-    gg[i] = a / (1.f + expf(-a)) * b;
+// ---- SwiGLU (src/nn_attn.cu:438-455): gg[t][f] = silu(h[t][f]) h[t][F + f]; four features per thread, 16-byte accesses ----
+__global__ void __launch_bounds__(256) glu_rows_k(const float4 *__restrict__ h, float4 *__restrict__ gg, int F4) {
+    const int f = blockIdx.x * 256 + threadIdx.x;                  // grid: x over the row's float4 chunks, y over the tokens
+    if (f >= F4) return;
+    const size_t t = blockIdx.y + (size_t)blockIdx.z * 65535u;
+    const float4 a = h[t * 2 * F4 + f], b = h[t * 2 * F4 + F4 + f];
+    gg[t * F4 + f] = make_float4(a.x / (1.f + expf(-a.x)) * b.x, a.y / (1.f + expf(-a.y)) * b.y, a.z / (1.f + expf(-a.z)) * b.z, a.w / (1.f + expf(-a.w)) * b.w);
+}
+__global__ void __launch_bounds__(256) glu_any_k(const float *__restrict__ h, float *__restrict__ gg, size_t n, int F) {       // widths that are not a multiple of 4
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (i >= n) return;
+    const size_t t = i / (unsigned)F; const int f = (int)(i - t * F);
+    const float a = h[t * 2 * F + f];
+    gg[i] = a / (1.f + expf(-a)) * h[t * 2 * F + F + f];
 }
 extern "C" void at_glu_fwd(const float *h, float *gg, long T, int F) {
     if (T <= 0 || F <= 0) return;
-    at_glu_k<<<nblk_((size_t)T * F, 256), 256>>>(h, gg, T, F);
+    if ((F & 3) == 0 && !(((uintptr_t)h | (uintptr_t)gg) & 15)) {
+        const unsigned ty = (unsigned)(T < 65535 ? T : 65535), tz = (unsigned)((T + 65534) / 65535);
+        if ((long)ty * tz != T) { glu_any_k<<<nblk_((size_t)T * F, 256), 256>>>(h, gg, (size_t)T * F, F); MICK(); return; }      // (a token count the 2-D grid does not tile)
+        glu_rows_k<<<dim3(nblk_((size_t)F / 4, 256), ty, tz), 256>>>((const float4 *)h, (float4 *)gg, F / 4);
+    } else glu_any_k<<<nblk_((size_t)T * F, 256), 256>>>(h, gg, (size_t)T * F, F);
     MICK();
 }
-__global__ void __launch_bounds__(256) at_cs_to_tok_k(const float *__restrict__ x, float *__restrict__ t, const float *__restrict__ reg, int n, int C, long long Sg, int nreg) {
-    const long long S = Sg + nreg, i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
-    if (i >= (long long)n * S * C) return;
-    const int c = (int)(i % C); const long long r = i / C; const int s = (int)(r / S); const long long ts = r % S - nreg;
-    t[i] = ts < 0 ? reg[(r % S) * C + c] : x[((long long)s * C + c) * Sg + ts];
+// ---- channel planes [n][C][Sg] <-> token rows [n][nreg + Sg][C] (src/nn_attn.cu:748-759): a transpose, done through 32 x 32 LDS tiles so that
+// both the plane side (contiguous in the token index) and the row side (contiguous in the channel) move whole 128-byte lines; the learned
+// register rows are copied in front of each sample's tokens ----
+template <bool TO_TOK>
+__global__ void __launch_bounds__(256) tok_transpose_k(const float *__restrict__ src, float *__restrict__ dst, int C, long long Sg, int nreg) {
+    __shared__ float tile[32][33];
+    const int n = blockIdx.z, c0 = blockIdx.y * 32, tx = threadIdx.x & 31, ty = threadIdx.x >> 5;      // ty 0 .. 7
+    const long long s0 = blockIdx.x * 32ll, S = Sg + nreg;
+    const float *planes = TO_TOK ? src : nullptr; float *planes_o = TO_TOK ? nullptr : dst;
+    if (TO_TOK) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) { const int c = c0 + ty + 8 * k; const long long sp = s0 + tx; tile[ty + 8 * k][tx] = c < C && sp < Sg ? planes[((long long)n * C + c) * Sg + sp] : 0.f; }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 4; k++) { const long long sp = s0 + ty + 8 * k; const int c = c0 + tx; if (sp < Sg && c < C) dst[((long long)n * S + nreg + sp) * C + c] = tile[tx][ty + 8 * k]; }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 4; k++) { const long long sp = s0 + ty + 8 * k; const int c = c0 + tx; tile[ty + 8 * k][tx] = sp < Sg && c < C ? src[((long long)n * S + nreg + sp) * C + c] : 0.f; }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 4; k++) { const int c = c0 + ty + 8 * k; const long long sp = s0 + tx; if (c < C && sp < Sg) planes_o[((long long)n * C + c) * Sg + sp] = tile[tx][ty + 8 * k]; }
+    }
 }
-__global__ void __launch_bounds__(256) at_tok_to_cs_k(const float *__restrict__ t, float *__restrict__ x, int n, int C, long long Sg, int nreg) {
-    const long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
-    if (i >= (long long)n * C * Sg) return;
-    const long long ts = i % Sg; const int c = (int)((i / Sg) % C), s = (int)(i / (Sg * C));
-    x[i] = t[((long long)s * (Sg + nreg) + nreg + ts) * C + c];
+__global__ void __launch_bounds__(256) reg_rows_k(const float *__restrict__ reg, float *__restrict__ t, int n, int C, long long S, int nreg) {
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x, per = (size_t)nreg * C;
+    if (i >= per * n) return;
+    const size_t s = i / per, k = i - s * per;
+    t[s * (size_t)S * C + k] = reg[k];
 }
 extern "C" void at_cs_to_tok(const float *x, float *t, const float *reg, int n, int C, long Sg, int nreg) {
-    const size_t m = (size_t)n * (Sg + nreg) * C; if (!m) return;
-    at_cs_to_tok_k<<<nblk_(m, 256), 256>>>(x, t, reg, n, C, Sg, nreg); MICK();
+    if (n <= 0 || C <= 0) return;
+    if (n > 65535 || (C + 31) / 32 > 65535) mi_die("at_cs_to_tok: %d samples x %d channels exceed the launch grid", n, C);
+    if (Sg > 0) tok_transpose_k<true><<<dim3(nblk_((size_t)Sg, 32), (unsigned)((C + 31) / 32), (unsigned)n), 256>>>(x, t, C, Sg, nreg);
+    if (nreg > 0) reg_rows_k<<<nblk_((size_t)n * nreg * C, 256), 256>>>(reg, t, n, C, Sg + nreg, nreg);
+    MICK();
 }
 extern "C" void at_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg) {
-    const size_t m = (size_t)n * C * Sg; if (!m) return;
-    at_tok_to_cs_k<<<nblk_(m, 256), 256>>>(t, x, n, C, Sg, nreg); MICK();
+    if (n <= 0 || C <= 0 || Sg <= 0) return;
+    if (n > 65535 || (C + 31) / 32 > 65535) mi_die("at_tok_to_cs: %d samples x %d channels exceed the launch grid", n, C);
+    tok_transpose_k<false><<<dim3(nblk_((size_t)Sg, 32), (unsigned)((C + 31) / 32), (unsigned)n), 256>>>(t, x, C, Sg, nreg);
+    MICK();
 }
 
-// one thread per (token row incl. the 64 padding rows, head, q / k / v): 48 values in registers
-__global__ void __launch_bounds__(128) at_pack_k(const float *__restrict__ qkv, const float *__restrict__ qg, const float *__restrict__ kg, __half *Qh, __half *Kh, __half *Vh,
-                                                 float *rq, float *rk, float *amx, long long T, int C, int S, int Hh, int W, int nreg, int rope, float lbase) {
-    const int H = C / HD; const long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
-    if (i >= (T + FT) * H * 3) return;
-    const int p = (int)(i % 3); const long long th = i / 3; const int h = (int)(th % H); const long long t = th / H;
-    __half *dst = (p == 0 ? Qh : p == 1 ? Kh : Vh) + ((size_t)h * (T + FT) + t) * HD;
-    if (t >= T) { for (int d = 0; d < HD; d += 8) *(uint4 *)(dst + d) = make_uint4(0, 0, 0, 0); return; }
-    const float *xs = qkv + t * 3 * C + p * C + h * HD;
-    float v[HD];
+// ---- QKV pack (src/nn_attn_tc.cu:99-136): per (token, head) the 48 q and k dims are RMS-normalised (eps 1e-6) and scaled by their learned
+// gains, grid tokens rotated by the axial 3-D rotary embedding (16 dims per axis: pair f of axis a turns by pos_a base^(-f / 8)), v passes
+// through; all three go to the fp16 head-major layout [3][H][T + 64][48] the attention core reads (64 zero rows of padding).
+// A unit = one (token, part, head) = 48 values = six 8-dim slices; eight neighbouring lanes own a unit (two idle), each slice is two 16-byte
+// loads and one 16-byte store of eight halves. The sum of squares meets over the unit's lanes; a rotary pair never leaves its lane
+// (slice j covers pairs 4 (j & 1) .. + 3 of axis j / 2). ----
+__global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv, const float *__restrict__ qg, const float *__restrict__ kg, __half *__restrict__ out,
+                                                  float *__restrict__ rq, float *__restrict__ rk, float *__restrict__ amx, long long T, int H, int S, int Hh, int W, int nreg, int rope, float lbase) {
+    const long long unit = (blockIdx.x * 256ll + threadIdx.x) >> 3; const int j = threadIdx.x & 7;
+    const long long Tp = T + FT, nunits = Tp * H * 3;
+    if (unit >= nunits) return;
+    const int h = (int)(unit % H); const long long tp = unit / H; const int p = (int)(tp % 3); const long long t = tp / 3;      // units of a token are neighbours: its 3 H x 192 bytes are read together
+    const int C = H * HD;
+    __half *dst = out + (((size_t)p * H + h) * Tp + t) * HD + 8 * j;
+    if (t >= T) { if (j < 6) *(uint4 *)dst = make_uint4(0u, 0u, 0u, 0u); return; }
+    float v[8];
+    if (j < 6) {
+        const float4 *xs = (const float4 *)(qkv + t * 3 * C + p * C + h * HD + 8 * j);
+        const float4 a = xs[0], b = xs[1];
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
 #pragma unroll
-    for (int d = 0; d < HD; d += 4) { const float4 f = *(const float4 *)(xs + d); v[d] = f.x; v[d + 1] = f.y; v[d + 2] = f.z; v[d + 3] = f.w; }
+        for (int i = 0; i < 8; i++) v[i] = 0.f;
+    }
     if (p < 2) {
-        float s = 0.f;
+        float ss = 0.f;
 #pragma unroll
-        for (int d = 0; d < HD; d++) s += v[d] * v[d];
-        const float r = 1.f / sqrtf(s / HD + 1e-6f); const float *gs = (p ? kg : qg) + h * HD;
+        for (int i = 0; i < 8; i++) ss = fmaf(v[i], v[i], ss);
+        ss += __shfl_xor(ss, 1); ss += __shfl_xor(ss, 2); ss += __shfl_xor(ss, 4);
+        const float r = 1.f / sqrtf(ss / HD + 1e-6f);
+        if (j == 0) (p ? rk : rq)[t * H + h] = r;
+        if (j < 6) {
+            const float *gs = (p ? kg : qg) + h * HD + 8 * j;      // (the gains sit at an arbitrary offset of the flat parameter vector: dword loads)
 #pragma unroll
-        for (int d = 0; d < HD; d++) v[d] *= r * gs[d];
-        (p ? rk : rq)[t * H + h] = r;
-        const int ts = (int)(t % S) - nreg;
-        if (rope && ts >= 0) {
-            const float pos[3] = {(float)(ts / (Hh * W)), (float)((ts / W) % Hh), (float)(ts % W)};
+            for (int i = 0; i < 8; i++) v[i] *= r * gs[i];
+            const int ts = (int)(t % S) - nreg;
+            if (rope && ts >= 0) {
+                const int ax = j >> 1;
+                const float pos = ax == 0 ? (float)(ts / (Hh * W)) : ax == 1 ? (float)((ts / W) % Hh) : (float)(ts % W);
 #pragma unroll
-            for (int pr = 0; pr < 24; pr++) {
-                const int ax = pr / 8, fi = pr % 8; float sn, cs; sincosf(pos[ax] * exp2f(-lbase * (float)fi / 8.f), &sn, &cs);
-                const float a = v[ax * 16 + 2 * fi], b = v[ax * 16 + 2 * fi + 1];
-                v[ax * 16 + 2 * fi] = a * cs - b * sn; v[ax * 16 + 2 * fi + 1] = a * sn + b * cs;
+                for (int i = 0; i < 4; i++) {
+                    const int fi = 4 * (j & 1) + i;
+                    float sn, cs; sincosf(pos * exp2f(-lbase * (float)fi / 8.f), &sn, &cs);
+                    const float a = v[2 * i], b = v[2 * i + 1];
+                    v[2 * i] = a * cs - b * sn; v[2 * i + 1] = a * sn + b * cs;
+                }
             }
         }
     } else {
         float m = 0.f;
 #pragma unroll
-        for (int d = 0; d < HD; d++) m = fmaxf(m, fabsf(v[d]));
-        atomicMax((unsigned *)amx + 1, __float_as_uint(m));     // (non-negative floats order as their bit patterns)
+        for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
+        m = fmaxf(m, __shfl_xor(m, 1)); m = fmaxf(m, __shfl_xor(m, 2)); m = fmaxf(m, __shfl_xor(m, 4));
+        if (j == 0) atomicMax((unsigned *)amx + 1, __float_as_uint(m));     // (non-negative floats order as their bit patterns)
     }
-#pragma unroll
-    for (int d = 0; d < HD; d += 2) *(__half2 *)(dst + d) = __floats2half2_rn(v[d], v[d + 1]);
+    if (j < 6) {
+        const __half2 h0 = __floats2half2_rn(v[0], v[1]), h1 = __floats2half2_rn(v[2], v[3]), h2 = __floats2half2_rn(v[4], v[5]), h3 = __floats2half2_rn(v[6], v[7]);
+        *(uint4 *)dst = make_uint4(*(const unsigned *)&h0, *(const unsigned *)&h1, *(const unsigned *)&h2, *(const unsigned *)&h3);
+    }
 }
 __global__ void at_zero4_k(float *p) { if (threadIdx.x < 4) p[threadIdx.x] = 0.f; }
 extern "C" void at_fa_pack(const float *qkv, const float *qg, const float *kg, void *qkvh, float *rq, float *rk, float *amx, const at_geom *g, int nreg, int C, int rope, float base) {
     if (g->pos) mi_die("at_fa_pack: per-token rotary positions are not supported");
     if (C % HD || (C & 3)) mi_die("at_fa_pack: C %d is not a whole number of heads of %d", C, HD);
     const long long T = (long long)g->nseq * g->S, Tp = T + FT; const int H = C / HD;
-    __half *Qh = (__half *)qkvh, *Kh = Qh + (size_t)H * Tp * HD, *Vh = Kh + (size_t)H * Tp * HD;
     at_zero4_k<<<1, 64>>>(amx);
-    at_pack_k<<<nblk_((size_t)Tp * H * 3, 128), 128>>>(qkv, qg, kg, Qh, Kh, Vh, rq, rk, amx, T, C, g->S, g->Hh, g->W, nreg, rope, log2f(base));
+    qkv_pack_k<<<nblk_((size_t)Tp * H * 3 * 8, 256), 256>>>(qkv, qg, kg, (__half *)qkvh, rq, rk, amx, T, H, g->S, g->Hh, g->W, nreg, rope, log2f(base));
     MICK();
 }
 
@@ -146,18 +232,27 @@ extern "C" int at_gemm_ex(int ta, int tb, int M, int N, int K, const float *A, c
     return lp_mx_gemm_ex(g_at_mx, ta, tb, M, N, K, A, B, Cm, beta, bias, res);
 }
 
+// The pre-LN block (src/nn_attn.cu:587-633): x1 = x + Wo attn(pack(Wqkv LN1(x))), y = x1 + W2 swiglu(W1 LN2(x1)). Each of the four linears
+// is one MX GEMM with its bias and, for the two that close a residual branch, the residual folded into the GEMM's epilogue.
+namespace {
+struct linear_t { const float *w, *b; int out, in; };
+inline int linear(const linear_t &l, long T, const float *in, float *out, const float *residual) {
+    return at_gemm_ex(0, 1, (int)T, l.out, l.in, in, l.w, out, 0.f, l.b, residual);
+}
+}
 extern "C" int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, const float *x, float *y, const at_geom *g, at_ws *w) {
     if (d->dK > 0 || g->rays || g->lens || g->pos || w->vr || d->rope > 1 || d->C != d->H * HD) return -1;
     const long T = (long)g->nseq * g->S; const int C = d->C, F = d->F;
-    int e = 0;
+    const linear_t qkv = {P + bp->wqkv, P + bp->bqkv, 3 * C, C}, proj = {P + bp->wo, P + bp->bo, C, C}, up = {P + bp->w1, P + bp->b1, 2 * F, C}, down = {P + bp->w2, P + bp->b2, C, F};
+    // attention branch
     at_ln_fwd(x, P + bp->ln1g, P + bp->ln1b, w->xn, w->m1, w->r1, T, C);
-    e |= at_gemm_ex(0, 1, (int)T, 3 * C, C, w->xn, P + bp->wqkv, w->qkv, 0.f, P + bp->bqkv, nullptr); if (e) return e;
+    if (int e = linear(qkv, T, w->xn, w->qkv, nullptr)) return e;
     at_fa_pack(w->qkv, P + bp->qg, P + bp->kg, w->qkvh, w->rq, w->rk, w->amx, g, d->nreg, C, d->rope, d->rope_base);
-    e |= at_fa8_fwd(w->qkvh, w->o, w->lse, g, d->H, C); if (e) return e;
-    e |= at_gemm_ex(0, 1, (int)T, C, C, w->o, P + bp->wo, w->x1, 0.f, P + bp->bo, x); if (e) return e;
+    if (int e = at_fa8_fwd(w->qkvh, w->o, w->lse, g, d->H, C)) return e;
+    if (int e = linear(proj, T, w->o, w->x1, x)) return e;
+    // MLP branch
     at_ln_fwd(w->x1, P + bp->ln2g, P + bp->ln2b, w->xn2, w->m2, w->r2, T, C);
-    e |= at_gemm_ex(0, 1, (int)T, 2 * F, C, w->xn2, P + bp->w1, w->h, 0.f, P + bp->b1, nullptr); if (e) return e;
+    if (int e = linear(up, T, w->xn2, w->h, nullptr)) return e;
     at_glu_fwd(w->h, w->gg, T, F);
-    e |= at_gemm_ex(0, 1, (int)T, C, F, w->gg, P + bp->w2, y, 0.f, P + bp->b2, w->x1);
-    return e;
+    return linear(down, T, w->gg, y, w->x1);
 }

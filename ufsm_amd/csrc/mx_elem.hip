@@ -93,30 +93,63 @@ extern "C" void lp_mx4_to_f32(const void *x, int N, int C, size_t S, float *y) {
 }
 
 // ---- network input rows (src/lp_mx_cvt.cu:29-55): z-scored CT, 0, unit direction away from the axis -> one 8-wide row per voxel ----
-template <int HD> __device__ __forceinline__ float in_round(float v) {
+// Only channels 0, 2 and 3 of a row are ever non-zero, so a row is formed in registers from three values: amax over the three (integer,
+// NaN-propagating), one exponent, one packed encode. A thread owns VPT = 4 neighbouring voxels of a row of the window when W % 4 == 0
+// (one 4-byte CT load, 32 or 16 contiguous bytes of rows and one word of scale bytes out), else one voxel.
+template <int HD> __device__ __forceinline__ float in_round(float v) {                         // the 16-bit type the reference's input passes through
     if (HD == 2) return __half2float(__float2half(v));
     if (HD == 1) { unsigned u = __float_as_uint(v); if ((u & 0x7fffffffu) > 0x7f800000u) return v; u += 0x7fffu + ((u >> 16) & 1u); return __uint_as_float(u & 0xffff0000u); }
     return v;
 }
-template <int B, int HD>
-__global__ void __launch_bounds__(256) pred_in_mx_k(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, uint8_t *y, int N, int n) {
-    const size_t S = (size_t)nz * W * W, i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (i >= S) return;
-    const int xx = (int)(i % W), yy = (int)((i / W) % W), z = z0 + (int)(i / ((size_t)W * W));
-    const float dy = dyo[z] + (float)yy, dx = dxo[z] + (float)xx, inv = axis ? (float)axis / (sqrtf(fmaf(dy, dy, dx * dx)) + 1e-6f) : 0.f;
-    float r[32];
+template <int B, int HD, int VPT>
+__global__ void __launch_bounds__(256) pred_rows_k(const uint8_t *__restrict__ ct, int W, float mean, float isd, const float *__restrict__ dyo, const float *__restrict__ dxo, int axis, int z0, size_t S,
+                                                   uint8_t *__restrict__ yrows, uint8_t *__restrict__ ysc) {
+    const size_t v0 = (blockIdx.x * (size_t)256 + threadIdx.x) * VPT;         // first voxel of the thread, relative to plane z0
+    if (v0 >= S) return;
+    const unsigned row = (unsigned)(v0 / (unsigned)W), xx0 = (unsigned)(v0 - (size_t)row * W), yy = row % (unsigned)W, z = (unsigned)z0 + row / (unsigned)W;
+    const uint8_t *src = ct + ((size_t)z * W + yy) * W + xx0;
+    unsigned cw;
+    if (VPT == 4) cw = *(const unsigned *)src; else cw = *src;
+    const float dy = dyo[z] + (float)yy, dx0 = dxo[z] + (float)xx0;
+    unsigned codes[VPT * (B == 8 ? 2 : 1)], sb = 0u;
 #pragma unroll
-    for (int k = 0; k < 32; k++) r[k] = 0.f;
-    r[0] = in_round<HD>(((float)ct[(size_t)z * W * W + (size_t)yy * W + xx] - mean) * isd); r[1] = in_round<HD>(0.f);
-    r[2] = in_round<HD>(__fmul_rn(dy, inv)); r[3] = in_round<HD>(__fmul_rn(dx, inv));     // (axis 0: the products are signed zeros, kept as such)
-    store_row<B, true>(y, mx_scp<B>(y, N, 4, S), (size_t)n * S + i, 8, r);       // sample n of an N-sample tensor: its rows, then the tensor's scale plane
+    for (int i = 0; i < VPT; i++) {
+        const float dx = i ? dxo[z] + (float)(xx0 + i) : dx0;
+        float r0 = ((float)((cw >> (8 * i)) & 255u) - mean) * isd, r2, r3;
+        if (axis) {
+            const float inv = (float)axis / (sqrtf(fmaf(dy, dy, dx * dx)) + 1e-6f);
+            r2 = __fmul_rn(dy, inv); r3 = __fmul_rn(dx, inv);
+        } else { r2 = copysignf(0.f, dy); r3 = copysignf(0.f, dx); }       // d * 0: a zero with d's sign, which the 16-bit rounding and the encoders keep
+        r0 = in_round<HD>(r0); r2 = in_round<HD>(r2); r3 = in_round<HD>(r3);
+        unsigned am = d_amax_u(d_amax_u(d_amax_u(0u, r0), r2), r3);
+        const int e = d_mx_exp(__uint_as_float(am), B == 8 ? MI_INVQ8 : MI_INVQ4);
+        if (B == 8) {
+            codes[2 * i] = d_enc4_e4m3(r0, 0.f, r2, r3, e);
+            codes[2 * i + 1] = e == 128 ? 0x7f7f7f7fu : 0u;                   // (a non-finite row: its zeros encode as NaN too, src/lp_common.cuh:501)
+        } else {
+            const float r[8] = {r0, 0.f, r2, r3, 0.f, 0.f, 0.f, 0.f};
+            codes[i] = d_enc8_e2m1(r, e);
+        }
+        sb |= (unsigned)(e + 127) << (8 * i);
+    }
+    if (VPT == 4) {
+        if (B == 8) { *(uint4 *)(yrows + v0 * 8) = make_uint4(codes[0], codes[1], codes[2], codes[3]); *(uint4 *)(yrows + v0 * 8 + 16) = make_uint4(codes[4], codes[5], codes[6], codes[7]); }
+        else *(uint4 *)(yrows + v0 * 4) = make_uint4(codes[0], codes[1], codes[2], codes[3]);
+        *(unsigned *)(ysc + v0) = sb;
+    } else {
+        if (B == 8) *(uint2 *)(yrows + v0 * 8) = make_uint2(codes[0], codes[1]); else *(unsigned *)(yrows + v0 * 4) = codes[0];
+        ysc[v0] = (uint8_t)sb;
+    }
 }
 // sample n of an N-sample input tensor (the reference's entry is one window: N 1, n 0)
 extern "C" void mi_pred_input_mx_n(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits, int N, int n) {
     const size_t S = (size_t)nz * W * W; if (!S) return;
     if (N < 1 || n < 0 || n >= N) mi_die("mi_pred_input_mx_n: sample %d of %d", n, N);
-    uint8_t *yy = (uint8_t *)y;
-#define PIN(B, HD) pred_in_mx_k<B, HD><<<nblk_(S, 256), 256>>>(ct, W, mean, isd, dyo, dxo, axis, z0, nz, yy, N, n)
+    const int rb = bits == 4 ? 4 : 8;                                           // bytes of an 8-channel row
+    uint8_t *yrows = (uint8_t *)y + (size_t)n * S * rb, *ysc = (uint8_t *)y + (size_t)N * S * rb + (size_t)n * S;      // sample n's rows; the tensor's scale plane follows all rows
+    const bool v4 = W % 4 == 0 && ((uintptr_t)ct & 3) == 0 && ((uintptr_t)ysc & 3) == 0 && ((uintptr_t)yrows & 15) == 0;
+#define PIN(B, HD) do { if (v4) pred_rows_k<B, HD, 4><<<nblk_(S / 4, 256), 256>>>(ct, W, mean, isd, dyo, dxo, axis, z0, S, yrows, ysc); \
+                        else pred_rows_k<B, HD, 1><<<nblk_(S, 256), 256>>>(ct, W, mean, isd, dyo, dxo, axis, z0, S, yrows, ysc); } while (0)
     if (bits == 4) { if (hd == 2) PIN(4, 2); else if (hd == 1) PIN(4, 1); else PIN(4, 0); }
     else { if (hd == 2) PIN(8, 2); else if (hd == 1) PIN(8, 1); else PIN(8, 0); }
 #undef PIN
@@ -130,26 +163,42 @@ extern "C" void lp_pred_input_mx8(const uint8_t *ct, int W, float mean, float is
 }
 
 // ---- y = MX(silu(gn(x))) (src/lp_mx_gn.cu:5-31): v = (x - mean) rstd gamma + beta, v / (1 + exp(-v)) ----
+// Any source (MX rows of 8 / 16 / 32 channels, fp32 / fp16 / bf16 planes) and channel count: a thread owns one (sample, block, voxel) row; the
+// block's per-channel (mean, rstd, gamma, beta) are formed once per workgroup in LDS; the row is transformed in place eight channels at a time
 template <int BX, int BY, typename TI>
-__global__ void __launch_bounds__(256) gn_silu_apply_mx_k(const void *xv, uint8_t *y, int N, int C, int G, size_t S, const float *gamma, const float *beta, const float *mean, const float *rstd) {
-    const int bw = mx_bw(C), nb = mx_nb(C), cpg = C / G;
-    const size_t v = blockIdx.x * (size_t)blockDim.x + threadIdx.x;       // grid: x over the voxels, y = n nb + blk (uniform: no per-thread divisions)
+__global__ void __launch_bounds__(256) gn_silu_rows_k(const void *__restrict__ xv, uint8_t *__restrict__ y, int N, int C, int G, size_t S,
+                                                      const float *__restrict__ gamma, const float *__restrict__ beta, const float *__restrict__ mean, const float *__restrict__ rstd) {
+    const int bw = mx_bw(C), nb = mx_nb(C);
+    const int blk = (int)(blockIdx.y % (unsigned)nb), n = (int)(blockIdx.y / (unsigned)nb), c0 = blk * bw, live = min(bw, C - c0);
+    __shared__ float4 co[32];
+    if (threadIdx.x < 32) {
+        const int c = c0 + (int)threadIdx.x;
+        float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
+        if ((int)threadIdx.x < live) { const int ng = n * G + c / (C / G); q = make_float4(mean[ng], rstd[ng], gamma[c], beta[c]); }
+        co[threadIdx.x] = q;
+    }
+    __syncthreads();
+    const size_t v = blockIdx.x * (size_t)256 + threadIdx.x;
     if (v >= S) return;
-    const int blk = (int)(blockIdx.y % (unsigned)nb), n = (int)(blockIdx.y / (unsigned)nb);
-    const size_t i = (size_t)blockIdx.y * S + v;
+    const size_t row = (size_t)blockIdx.y * S + v;
     float r[32];
-    if (BX != 0) { const uint8_t *x = (const uint8_t *)xv; load_row<BX ? BX : 8>(x, mx_scp<BX ? BX : 8>(x, N, C, S), i, bw, r); }
+    if (BX != 0) { const uint8_t *x = (const uint8_t *)xv; load_row<BX ? BX : 8>(x, mx_scp<BX ? BX : 8>(x, N, C, S), row, bw, r); }
     else {
+        const TI *xp = (const TI *)xv + ((size_t)n * C + c0) * S + v;
 #pragma unroll
-        for (int k = 0; k < 32; k++) { const int c = blk * bw + k; r[k] = k < bw && c < C ? ldx((const TI *)xv, ((size_t)n * C + c) * S + v) : 0.f; }
+        for (int k = 0; k < 32; k++) r[k] = k < live ? ldx(xp, (size_t)k * S) : 0.f;
     }
 #pragma unroll
-    for (int k = 0; k < 32; k++) {
-        const int c = blk * bw + k;
-        if (k < bw && c < C) { const int ng = n * G + c / cpg; const float u = fmaf((r[k] - mean[ng]) * rstd[ng], gamma[c], beta[c]); r[k] = d_silu(u); }
-        else r[k] = 0.f;
+    for (int g8 = 0; g8 < 4; g8++) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int k = 8 * g8 + i;
+            const float4 q = co[k];
+            const float u = fmaf((r[k] - q.x) * q.y, q.z, q.w);
+            r[k] = k < live ? d_silu(u) : 0.f;
+        }
     }
-    store_row<BY, true>(y, mx_scp<BY>(y, N, C, S), i, bw, r);
+    store_row<BY, true>(y, mx_scp<BY>(y, N, C, S), row, bw, r);
 }
 // the same for an MX source of 32-channel blocks, two lanes per row (each lane one contiguous 16-channel half in and out, the per-channel
 // mean / rstd / gamma / beta of the block in LDS): a wavefront reads and writes contiguous memory
@@ -209,7 +258,7 @@ extern "C" void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, con
         MICK();
         return;
     }
-#define GSA(BX, BY, TI) gn_silu_apply_mx_k<BX, BY, TI><<<rows_grid(s.n, mx_nb(s.c), S), 256>>>(x, (uint8_t *)y, s.n, s.c, G, S, gamma, beta, mean, rstd)
+#define GSA(BX, BY, TI) gn_silu_rows_k<BX, BY, TI><<<rows_grid(s.n, mx_nb(s.c), S), 256>>>(x, (uint8_t *)y, s.n, s.c, G, S, gamma, beta, mean, rstd)
 #define GSA_Y(BX, TI) do { if (ydt == 4) GSA(BX, 4, TI); else GSA(BX, 8, TI); } while (0)
     if (xdt == 4) GSA_Y(4, float); else if (xdt == 3) GSA_Y(8, float); else if (xdt == 2) GSA_Y(0, __half); else if (xdt == 1) GSA_Y(0, bf16_t); else GSA_Y(0, float);
 #undef GSA_Y
@@ -218,58 +267,92 @@ extern "C" void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, con
 }
 
 // ---- trilinear 2x upsample (src/lp_mx_gn.cu:34-73, :151-186): out[o] = .75 in[o/2] + .25 in[o/2 -+ 1] per axis, edge clamp ----
-template <int BX, int BY>
-__global__ void __launch_bounds__(256) up2_mx_k(const uint8_t *x, uint8_t *y, int N, int Cx, int b0, int Cy, int D, int H, int W, gnp_t gp) {
-    // x: Cx channels, blocks b0.. feed y's blocks 0..; y: Cy channels
-    const int bwx = mx_bw(Cx), nbx = mx_nb(Cx), bwy = mx_bw(Cy), nby = mx_nb(Cy), Do = 2 * D, Ho = 2 * H, Wo = 2 * W;
+// Cell form: the 8 fine voxels 2m + 1 + {0, 1}^3 read exactly the 8 coarse rows m + {0, 1}^3 (clamped), so a thread owns one cell (mz, my, mx),
+// each in [-1, dim - 1], for one 8-channel granule of the block: every coarse row is decoded (and, with GroupNorm, activated) once per cell
+// instead of once per fine voxel, and the eight blends are register arithmetic. BW / 8 neighbouring threads share a cell and meet for the row's
+// amax through lane exchanges. The 8-term sum keeps the reference's order: own row first, then the x, y, z neighbours (a, b, c loops, c fastest).
+template <int BX, int BY, int BW>
+__global__ void __launch_bounds__(256) up2_cell_k(const uint8_t *__restrict__ x, uint8_t *__restrict__ y, int N, int Cx, int b0, int Cy, int D, int H, int W, gnp_t gp) {
+    constexpr int QP = BW / 8, IB = BX, OB = BY;                   // threads per cell; bytes of an 8-channel granule in and out
+    const int nbx = mx_nb(Cx), nby = mx_nb(Cy), Do = 2 * D, Ho = 2 * H, Wo = 2 * W;
     const size_t S = (size_t)D * H * W, So = (size_t)Do * Ho * Wo;
-    const int nbk = blockIdx.y, n = nbk / nby, blk = nbk % nby;
+    const int nbk = blockIdx.y, n = nbk / nby, blk = nbk % nby, live = min(BW, Cy - blk * BW);
     __shared__ float ca[32], cb[32];
     if (threadIdx.x < 32) {
-        const int k = threadIdx.x, ci = blk * bwy + k;
+        const int k = threadIdx.x, ci = blk * BW + k;
         float a = 1.f, b = 0.f;
-        if (gp.G && k < bwy && ci < Cy) { const int ng = n * gp.G + ci / (Cy / gp.G); a = gp.rstd[ng] * gp.gamma[ci]; b = fmaf(-gp.mean[ng], a, gp.beta[ci]); }
+        if (gp.G && k < live) { const int ng = n * gp.G + ci / (Cy / gp.G); a = gp.rstd[ng] * gp.gamma[ci]; b = fmaf(-gp.mean[ng], a, gp.beta[ci]); }
         ca[k] = a; cb[k] = b;
     }
     __syncthreads();
-    const size_t vo = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (vo >= So) return;
-    const int ox = (int)(vo % Wo), oy = (int)((vo / Wo) % Ho), oz = (int)(vo / ((size_t)Wo * Ho));
-    const int mz[2] = {oz >> 1, min(max((oz >> 1) + ((oz & 1) ? 1 : -1), 0), D - 1)}, my[2] = {oy >> 1, min(max((oy >> 1) + ((oy & 1) ? 1 : -1), 0), H - 1)},
-              mx[2] = {ox >> 1, min(max((ox >> 1) + ((ox & 1) ? 1 : -1), 0), W - 1)};
-    const uint8_t *sc = mx_scp<BX>(x, N, Cx, S);
-    const int kmax = min(bwy, Cy - blk * bwy);
-    float acc[32];
+    const unsigned t = blockIdx.x * 256u + threadIdx.x, q = t % QP, cell = t / QP, ncx = (unsigned)W + 1u, ncy = (unsigned)H + 1u;
+    const bool have = cell < ncx * ncy;
+    const unsigned cc = have ? cell : 0u, cyi = cc / ncx;
+    const int mx = (int)(cc - cyi * ncx) - 1, my = (int)cyi - 1, mz = (int)blockIdx.z - 1;
+    const int cz[2] = {max(mz, 0), min(mz + 1, D - 1)}, cy[2] = {max(my, 0), min(my + 1, H - 1)}, cx[2] = {max(mx, 0), min(mx + 1, W - 1)};
+    const uint8_t *xs = mx_scp<BX>(x, N, Cx, S);
+    const size_t xrow0 = ((size_t)n * nbx + b0 + blk) * S;
+    float f[8][8];
 #pragma unroll
-    for (int k = 0; k < 32; k++) acc[k] = 0.f;
+    for (int k = 0; k < 8; k++) {
+        const size_t row = xrow0 + ((size_t)cz[k >> 2] * H + cy[(k >> 1) & 1]) * W + cx[k & 1];
+        const uint8_t *p = x + row * (BW * BX / 8) + q * IB;
+        if (BX == 8) { const uint2 w = *(const uint2 *)p; d_dec4_e4m3(w.x, f[k]); d_dec4_e4m3(w.y, f[k] + 4); }
+        else d_dec8_e2m1(*(const unsigned *)p, f[k]);
+        const float sc = d_mx_scale(xs[row]);
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+        for (int i = 0; i < 8; i++) {
+            const int ch = (int)q * 8 + i;
+            const float v = f[k][i] * sc;
+            f[k][i] = gp.G && ch < live ? d_act_ab(v, ca[ch], cb[ch]) : v;
+        }
+    }
+    uint8_t *ysc = mx_scp<BY>(y, N, Cy, So);
 #pragma unroll
-        for (int bb = 0; bb < 2; bb++)
+    for (int p = 0; p < 8; p++) {
+        const int pz = p >> 2, py = (p >> 1) & 1, px = p & 1;                 // fine voxel 2m + 1 + p: for p = 0 its own coarse row is m, for p = 1 it is m + 1
+        const int gz = 2 * mz + 1 + pz, gy = 2 * my + 1 + py, gx = 2 * mx + 1 + px;
+        float acc[8];
 #pragma unroll
-            for (int c = 0; c < 2; c++) {
-                float r[32];
-                const float w3 = (a ? 0.25f : 0.75f) * (bb ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f);
-                load_row<BX>(x, sc, ((size_t)n * nbx + b0 + blk) * S + ((size_t)mz[a] * H + my[bb]) * W + mx[c], bwx, r);
-                if (gp.G) {
+        for (int i = 0; i < 8; i++) acc[i] = 0.f;
 #pragma unroll
-                    for (int k = 0; k < 32; k++) if (k < kmax) r[k] = d_act_ab(r[k], ca[k], cb[k]);
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int c = 0; c < 2; c++) {
+                    const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);
+                    const float w3 = (a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f);
+#pragma unroll
+                    for (int i = 0; i < 8; i++) acc[i] = fmaf(w3, f[k][i], acc[i]);
                 }
+        unsigned am = 0u;                                                      // NaN-propagating amax (src/lp_mxops.cpp row store), over the cell's QP lanes
 #pragma unroll
-                for (int k = 0; k < 32; k++) acc[k] = fmaf(w3, r[k], acc[k]);
-            }
-    store_row<BY, true>(y, mx_scp<BY>(y, N, Cy, So), (size_t)nbk * So + vo, bwy, acc);
+        for (int i = 0; i < 8; i++) am = d_amax_u(am, acc[i]);
+        if (QP >= 2) { const unsigned o = (unsigned)__shfl_xor((int)am, 1); am = o > am ? o : am; }
+        if (QP >= 4) { const unsigned o = (unsigned)__shfl_xor((int)am, 2); am = o > am ? o : am; }
+        const int e = d_mx_exp(__uint_as_float(am), BY == 8 ? MI_INVQ8 : MI_INVQ4);
+        if (!have || gz < 0 || gz >= Do || gy < 0 || gy >= Ho || gx < 0 || gx >= Wo) continue;
+        const size_t row = (size_t)nbk * So + ((size_t)gz * Ho + gy) * Wo + gx;
+        uint8_t *dst = y + row * (BW * BY / 8) + q * OB;
+        if (BY == 8) *(uint2 *)dst = make_uint2(d_enc4_e4m3(acc[0], acc[1], acc[2], acc[3], e), d_enc4_e4m3(acc[4], acc[5], acc[6], acc[7], e));
+        else *(unsigned *)dst = d_enc8_e2m1(acc, e);
+        if (!q) ysc[row] = (uint8_t)(e + 127);
+    }
 }
 static void up2_launch(const void *x, int xdt, shape5 xs, int b0, int Cy, void *y, int ydt, gnp_t gp, const char *who) {
     if ((xdt != 3 && xdt != 4) || (ydt != 3 && ydt != 4)) mi_die("%s: dtypes %d -> %d are not MX", who, xdt, ydt);
     if (gp.G && (gp.ns || xs.c % gp.G)) mi_die("%s: GroupNorm of %d channels in %d groups (slab-local statistics are not supported)", who, xs.c, gp.G);
-    const size_t So = 8 * (size_t)xs.d * xs.h * xs.w;
-    if (!So || !xs.n) return;
-    const dim3 grid(nblk_(So, 256), (unsigned)(xs.n * mx_nb(Cy)));
+    if (!xs.d || !xs.h || !xs.w || !xs.n) return;
+    const int bw = mx_bw(Cy), qp = bw / 8;
+    if ((size_t)xs.n * mx_nb(Cy) > 65535 || xs.d + 1 > 65535) mi_die("%s: launch grid (%d samples x %d blocks, %d cell layers)", who, xs.n, mx_nb(Cy), xs.d + 1);
+    const dim3 grid(nblk_((size_t)(xs.h + 1) * (xs.w + 1) * qp, 256), (unsigned)(xs.n * mx_nb(Cy)), (unsigned)(xs.d + 1));
     const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
-#define U2(BX, BY) up2_mx_k<BX, BY><<<grid, 256>>>(xq, yq, xs.n, xs.c, b0, Cy, xs.d, xs.h, xs.w, gp)
+#define U2W(BX, BY, BW) up2_cell_k<BX, BY, BW><<<grid, 256>>>(xq, yq, xs.n, xs.c, b0, Cy, xs.d, xs.h, xs.w, gp)
+#define U2(BX, BY) do { if (bw == 32) U2W(BX, BY, 32); else if (bw == 16) U2W(BX, BY, 16); else U2W(BX, BY, 8); } while (0)
     if (xdt == 4) { if (ydt == 4) U2(4, 4); else U2(4, 8); } else { if (ydt == 4) U2(8, 4); else U2(8, 8); }
 #undef U2
+#undef U2W
     MICK();
 }
 extern "C" void lp_up2_fwd_mx(const void *x, int xdt, shape5 xs, void *y, int ydt, gnp_t gp) { up2_launch(x, xdt, xs, 0, xs.c, y, ydt, gp, "lp_up2_fwd_mx"); }
@@ -279,22 +362,63 @@ extern "C" void lp_up2_fwd_mx_blocks(const void *x, int xdt, shape5 xs, int b0, 
     up2_launch(x, xdt, xs, b0, 32 * nbk, y, ydt, g0, "lp_up2_fwd_mx_blocks");
 }
 
-// ---- y += x (src/lp_mx_gn.cu:134-150) ----
-template <int B> __global__ void __launch_bounds__(256) add_mx_k(uint8_t *y, const uint8_t *x, int N, int C, size_t S) {
-    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (i >= (size_t)N * mx_nb(C) * S) return;
-    const int bw = mx_bw(C);
-    float a[32], b[32];
-    load_row<B>(y, mx_scp<B>(y, N, C, S), i, bw, a); load_row<B>(x, mx_scp<B>(x, N, C, S), i, bw, b);
+// ---- y += x (src/lp_mx_gn.cu:134-150): both rows decoded, summed in fp32, the sum re-quantised with its own scale ----
+// 32-channel blocks: two lanes per row, a lane one contiguous 16-channel half of both operands and of the result (a wavefront reads and
+// writes contiguous memory), ROWS rows per thread requested together; the halves' amaxes meet through one lane exchange
+constexpr int ADD_ROWS = 4;
+template <int B>
+__global__ void __launch_bounds__(256) add32_k(uint8_t *__restrict__ y, const uint8_t *__restrict__ x, size_t rows) {
+    constexpr int HB = B * 2;                                      // bytes of a 16-channel half row
+    const int hf = threadIdx.x & 1;
+    const size_t r0 = blockIdx.x * (size_t)(128 * ADD_ROWS) + (threadIdx.x >> 1);
+    uint8_t *ys = y + rows * (2 * HB); const uint8_t *xs = x + rows * (2 * HB);
+    unsigned wa[ADD_ROWS][4], wb[ADD_ROWS][4], sa[ADD_ROWS], sb[ADD_ROWS];
 #pragma unroll
-    for (int k = 0; k < 32; k++) a[k] += b[k];
-    store_row<B, true>(y, mx_scp<B>(y, N, C, S), i, bw, a);
+    for (int i = 0; i < ADD_ROWS; i++) {
+        const size_t r = r0 + (size_t)i * 128, rr = r < rows ? r : rows - 1;
+        if (B == 8) { const uint4 p = *(const uint4 *)(y + rr * 32 + hf * 16), q = *(const uint4 *)(x + rr * 32 + hf * 16); wa[i][0] = p.x; wa[i][1] = p.y; wa[i][2] = p.z; wa[i][3] = p.w; wb[i][0] = q.x; wb[i][1] = q.y; wb[i][2] = q.z; wb[i][3] = q.w; }
+        else { const uint2 p = *(const uint2 *)(y + rr * 16 + hf * 8), q = *(const uint2 *)(x + rr * 16 + hf * 8); wa[i][0] = p.x; wa[i][1] = p.y; wb[i][0] = q.x; wb[i][1] = q.y; wa[i][2] = wa[i][3] = wb[i][2] = wb[i][3] = 0u; }
+        sa[i] = ys[rr]; sb[i] = xs[rr];
+    }
+#pragma unroll
+    for (int i = 0; i < ADD_ROWS; i++) {
+        const size_t r = r0 + (size_t)i * 128;
+        float a[16], b[16];
+        if (B == 8) { for (int j = 0; j < 4; j++) { d_dec4_e4m3(wa[i][j], a + 4 * j); d_dec4_e4m3(wb[i][j], b + 4 * j); } }
+        else { for (int j = 0; j < 2; j++) { d_dec8_e2m1(wa[i][j], a + 8 * j); d_dec8_e2m1(wb[i][j], b + 8 * j); } }
+        const float fa = d_mx_scale(sa[i]), fb = d_mx_scale(sb[i]);
+        unsigned am = 0u;
+#pragma unroll
+        for (int k = 0; k < 16; k++) { a[k] = __fadd_rn(a[k] * fa, b[k] * fb); am = d_amax_u(am, a[k]); }     // (two rounded products, one rounded sum: no contraction)
+        const unsigned ao = (unsigned)__shfl_xor((int)am, 1);
+        am = ao > am ? ao : am;
+        const int e = d_mx_exp(__uint_as_float(am), B == 8 ? MI_INVQ8 : MI_INVQ4);
+        if (r >= rows) continue;
+        if (B == 8) *(uint4 *)(y + r * 32 + hf * 16) = make_uint4(d_enc4_e4m3(a[0], a[1], a[2], a[3], e), d_enc4_e4m3(a[4], a[5], a[6], a[7], e), d_enc4_e4m3(a[8], a[9], a[10], a[11], e), d_enc4_e4m3(a[12], a[13], a[14], a[15], e));
+        else *(uint2 *)(y + r * 16 + hf * 8) = make_uint2(d_enc8_e2m1(a, e), d_enc8_e2m1(a + 8, e));
+        if (!hf) ys[r] = (uint8_t)(e + 127);
+    }
+}
+// narrow rows (<= 16 channels): one thread per row
+template <int B> __global__ void __launch_bounds__(256) add_rows_k(uint8_t *__restrict__ y, const uint8_t *__restrict__ x, size_t rows, int bw) {
+    const size_t r = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (r >= rows) return;
+    uint8_t *ys = y + rows * mx_rb(bw, B); const uint8_t *xs = x + rows * mx_rb(bw, B);
+    float a[32], b[32];
+    load_row<B>(y, ys, r, bw, a); load_row<B>(x, xs, r, bw, b);
+#pragma unroll
+    for (int k = 0; k < 32; k++) a[k] = __fadd_rn(a[k], b[k]);
+    store_row<B, true>(y, ys, r, bw, a);
 }
 extern "C" void lp_add_mx(void *y, const void *x, shape5 s, int dt, unsigned sr) {
     if (sr) mi_die("lp_add_mx: stochastic rounding (sr %u) belongs to training and is not built here", sr);
     const size_t rows = (size_t)s.n * mx_nb(s.c) * s.d * s.h * s.w; if (!rows) return;
-    if (dt == 4) add_mx_k<4><<<nblk_(rows, 256), 256>>>((uint8_t *)y, (const uint8_t *)x, s.n, s.c, (size_t)s.d * s.h * s.w);
-    else add_mx_k<8><<<nblk_(rows, 256), 256>>>((uint8_t *)y, (const uint8_t *)x, s.n, s.c, (size_t)s.d * s.h * s.w);
+    const int bw = mx_bw(s.c);
+    if (bw == 32) {
+        if (dt == 4) add32_k<4><<<nblk_(rows, 128 * ADD_ROWS), 256>>>((uint8_t *)y, (const uint8_t *)x, rows);
+        else add32_k<8><<<nblk_(rows, 128 * ADD_ROWS), 256>>>((uint8_t *)y, (const uint8_t *)x, rows);
+    } else if (dt == 4) add_rows_k<4><<<nblk_(rows, 256), 256>>>((uint8_t *)y, (const uint8_t *)x, rows, bw);
+    else add_rows_k<8><<<nblk_(rows, 256), 256>>>((uint8_t *)y, (const uint8_t *)x, rows, bw);
     MICK();
 }
 

@@ -8,24 +8,33 @@ static int g_pred_iso = 1;
 extern "C" void nn_set_pred_iso(int t) { g_pred_iso = t < 1 ? 1 : t; }
 extern "C" int nn_get_pred_iso(void) { return g_pred_iso; }
 
-struct place_box { int z0, y0, x0, nz, ny, nx; };
-// one thread per voxel of the intersection of the window's interior and the target box (src/nn_elem.cu:1108-1121)
-__global__ void __launch_bounds__(256) pred_place_k(const float *__restrict__ lg, const uint8_t *__restrict__ ct, place_box B, int W, int oz, int oy, int ox, int shard,
+// ---- placement (src/nn_elem.cu:1103-1130): out = CT >= iso ? uint8(255 sigmoid(logit) + .5) : 0 over the window's interior clipped to the
+// target box. The clipped region is rows of nx voxels; a thread owns a run of PLACE_RUN voxels of one row (its logits and CT bytes are two
+// contiguous reads, its bytes one contiguous write), the runs of a row are neighbouring threads ----
+constexpr int PLACE_RUN = 8;
+struct place_rows_t { int z0, y0, x0, ny, nx, nrun; };
+__global__ void __launch_bounds__(256) place_rows_k(const float *__restrict__ lg, const uint8_t *__restrict__ ct, place_rows_t P, size_t nthreads, int W, int oz, int oy, int ox, int shard,
                                                     uint8_t *__restrict__ dsh, int iso) {
-    const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
-    if (i >= (size_t)B.nz * B.ny * B.nx) return;
-    const int x = B.x0 + (int)(i % B.nx), y = B.y0 + (int)((i / B.nx) % B.ny), z = B.z0 + (int)(i / ((size_t)B.ny * B.nx));
-    const size_t k = ((size_t)z * W + y) * W + x;
-    dsh[((size_t)(oz + z) * shard + (oy + y)) * shard + (ox + x)] = ct[k] >= iso ? (uint8_t)(255.f / (1.f + expf(-lg[k])) + 0.5f) : 0;
+    const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (t >= nthreads) return;
+    const size_t row = t / (unsigned)P.nrun;
+    const int run = (int)(t - row * P.nrun), y = P.y0 + (int)(row % (unsigned)P.ny), z = P.z0 + (int)(row / (unsigned)P.ny), x = P.x0 + run * PLACE_RUN;
+    const int n = min(PLACE_RUN, P.x0 + P.nx - x);
+    const float *l = lg + ((size_t)z * W + y) * W + x; const uint8_t *c = ct + ((size_t)z * W + y) * W + x;
+    uint8_t *o = dsh + ((size_t)(oz + z) * shard + (oy + y)) * shard + (ox + x);
+    float v[PLACE_RUN]; uint8_t m[PLACE_RUN];
+#pragma unroll
+    for (int i = 0; i < PLACE_RUN; i++) { const int k = i < n ? i : 0; v[i] = l[k]; m[i] = c[k]; }
+#pragma unroll
+    for (int i = 0; i < PLACE_RUN; i++) if (i < n) o[i] = m[i] >= iso ? (uint8_t)(255.f / (1.f + expf(-v[i])) + 0.5f) : (uint8_t)0;
 }
 extern "C" void nn_pred_place_d(const float *lg, const uint8_t *ct, int D, int W, int hz, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, uint8_t *dsh) {
-    place_box b;
-    const int z1 = min(D - hz, ez - oz), y1 = min(W - halo, ey - oy), x1 = min(W - halo, ex - ox);
-    b.z0 = max(hz, -oz); b.y0 = max(halo, -oy); b.x0 = max(halo, -ox);
-    b.nz = max(z1 - b.z0, 0); b.ny = max(y1 - b.y0, 0); b.nx = max(x1 - b.x0, 0);
-    const size_t n = (size_t)b.nz * b.ny * b.nx;
-    if (!n) return;
-    pred_place_k<<<nblk_(n, 256), 256>>>(lg, ct, b, W, oz, oy, ox, shard, dsh, g_pred_iso);
+    // window voxel v lands at o + v of the target; kept: v inside the interior [h, dim - h) of its axis and o + v inside [0, e)
+    const int lo[3] = {max(hz, -oz), max(halo, -oy), max(halo, -ox)}, hi[3] = {min(D - hz, ez - oz), min(W - halo, ey - oy), min(W - halo, ex - ox)};
+    if (hi[0] <= lo[0] || hi[1] <= lo[1] || hi[2] <= lo[2]) return;
+    place_rows_t P = {lo[0], lo[1], lo[2], hi[1] - lo[1], hi[2] - lo[2], (hi[2] - lo[2] + PLACE_RUN - 1) / PLACE_RUN};
+    const size_t nthreads = (size_t)(hi[0] - lo[0]) * P.ny * P.nrun;
+    place_rows_k<<<nblk_(nthreads, 256), 256>>>(lg, ct, P, nthreads, W, oz, oy, ox, shard, dsh, g_pred_iso);
     MICK();
 }
 extern "C" void nn_pred_place(const float *lg, const uint8_t *ct, int W, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, uint8_t *dsh) {
