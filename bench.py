@@ -1,10 +1,14 @@
 #!/usr/bin/env python3
-"""Benchmark of the MX conv hot path on one MI355X.
+"""Benchmark of the MX U-Net forward path on one MI355X. Prints one JSON line.
 
-Workload (BASELINE.json configs[1]): a stack of four 3x3x3 convolutions, Cin = Cout = 128, batch 2, 64^3 voxels, MX-fp8 (e4m3 + E8M0
-per 32 channels) activations and weights, bias, GroupNorm(8) statistics fused into each conv's epilogue, the previous layer's
-GroupNorm affine + SiLU applied to the conv's input, MX-fp8 re-quantised output: the reference's block structure (src/unet.c:2567-2636).
-A step = one pass of the stack over one batch resident in HBM. Prints one JSON line."""
+value / ms_per_step (BASELINE.json configs[3], the metric's "U-Net infer voxels/s (128^3 patch, MX fp8)"): one forward of the reference-style
+U-Net (cin 4, widths 32/64/128/256, two 3x3x3 convs + GroupNorm + SiLU per level, 3x3x3 stride-2 downs, trilinear 2x fused into the decoder
+convs, skip concat, 1x1x1 head of 8 logits) over N 2 x 128^3 voxels, MX-fp8 storage and compute, the quantised input resident in HBM. A step =
+one forward; the prepared (quantised, re-laid-out) weights are memoised across forwards as an inference loop keeps them - the reference's
+fp8 path re-quantises them per call (src/lp_f8fwd.cu:54-71; about 15 us per layer here). `roofline`: the forward's dominant kernel (most
+total time among its conv launches, HIP events around every launch on its stream).
+conv_stack (configs[1], the metric's "3x3x3 conv % of MFMA peak"): four 3x3x3 convs 128 -> 128, N 2, 64^3, MX-fp8, bias + GroupNorm(8)
+statistics fused, the previous layer's GroupNorm + SiLU on the input; its own `roofline` is the conv kernel alone."""
 import argparse
 import ctypes as C
 import json
@@ -18,13 +22,16 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 METRIC = "U-Net infer voxels/s (128^3 patch, MX fp8) + 3x3x3 conv % of MFMA peak"
 TRAFFIC_BYTES_PER_LAUNCH = 183.9e6     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/
+# HBM bytes per launch of the U-Net's dominant conv from committed counter runs: layer -> (bytes, source); absent: not measured
+KERNEL_TRAFFIC = {}
 MFMA_PEAK_FP8_TFLOPS = 5033.0          # MI355X dense MXFP8 (2.5 PFLOP/s bf16 x 2)
 
 
 def unet_leg(np, lib, LP, DevBuf, steps, warmup):
     """configs[3]: the reference-style U-Net forward (cin 4, widths 32/64/128/256, two 3x3x3 convs + GroupNorm + SiLU per level, 3x3x3 stride-2
     downs, trilinear 2x fused into the decoder convs, skip concat, 1x1x1 head of 8 logits), N 2 x 128^3, MX-fp8 storage and compute, random
-    init, CT-like synthetic input already quantised and resident in HBM."""
+    init, CT-like synthetic input already quantised and resident in HBM. Two timed passes: the forwards alone (wall clock: `value`), then the
+    same number of forwards with an event pair around every conv launch (per-kernel times for the roofline; the events cost a little)."""
     from ufsm_amd.unet import UNet, make_cfg
     N, D, widths = 2, 128, [32, 64, 128, 256]
     S = D ** 3
@@ -50,6 +57,28 @@ def unet_leg(np, lib, LP, DevBuf, steps, warmup):
         net.forward_mx(dxq.ptr)                                                     # (the logits stay in the net's own device buffer)
     lib.mi_sync(); LP.check()
     dt = (time.perf_counter() - t0) / steps
+    # per-kernel: every conv launch of `steps` more forwards, grouped by kernel variant and layer position within the forward
+    lib.mi_kernel_timing(1)
+    for _ in range(steps):
+        net.forward_mx(dxq.ptr)
+    lib.mi_sync()
+    nlog = lib.mi_kernel_timing_launch(-1, None, None, None, 0)
+    per_fwd = nlog // steps
+    layers = {}
+    name = C.create_string_buffer(128); ms = C.c_float(0); fl = C.c_double(0)
+    for i in range(nlog):
+        lib.mi_kernel_timing_launch(i, C.byref(ms), C.byref(fl), name, 128)
+        k = i % per_fwd
+        e = layers.setdefault(k, {"kernel": name.value.decode(), "flops": fl.value, "ms": 0.0, "n": 0})
+        e["ms"] += ms.value; e["n"] += 1
+    lib.mi_kernel_timing(0); LP.check()
+    order = ["enc0.c1", "enc0.c2", "down0", "enc1.c1", "enc1.c2", "down1", "enc2.c1", "enc2.c2", "down2", "enc3.c1", "enc3.c2",
+             "dec2.c1", "dec2.c2", "dec1.c1", "dec1.c2", "dec0.c1", "dec0.c2"]
+    convs = []
+    for k in sorted(layers):
+        e = layers[k]; avg = e["ms"] / e["n"]
+        convs.append({"layer": order[k] if per_fwd == len(order) else "conv%d" % k, "kernel": e["kernel"], "avg_launch_ms": avg, "tflops": e["flops"] / avg / 1e9,
+                      "frac_of_mxfp8_peak": e["flops"] / avg / 1e9 / MFMA_PEAK_FP8_TFLOPS, "flops_per_launch": e["flops"]})
     # conv FLOPs of one forward, logical channels, all taps (tests/bench_lp.c:46)
     fl, lv = 0.0, [(D >> i) ** 3 for i in range(len(widths))]
     for i, wd in enumerate(widths):
@@ -60,8 +89,10 @@ def unet_leg(np, lib, LP, DevBuf, steps, warmup):
     fl += 2 * widths[0] * 8 * lv[0]
     fl *= N
     net.close()
+    dom = max(convs, key=lambda c: c["avg_launch_ms"])
     return {"workload": "configs[3]: U-Net forward, N 2 x 128^3, widths 32/64/128/256, MX-fp8", "value": N * S / dt, "unit": "voxels/s", "ms_per_forward": dt * 1e3,
-            "steps": steps, "gflop_per_forward": fl / 1e9, "tflops": fl / dt / 1e12}
+            "steps": steps, "gflop_per_forward": fl / 1e9, "tflops": fl / dt / 1e12, "conv_launches": convs,
+            "conv_ms_per_forward": sum(c["avg_launch_ms"] for c in convs)}, dom
 
 
 def hbm_leg(np, lib, LP, DevBuf):
@@ -150,11 +181,11 @@ def sliding_leg(np, lib, LP, DevBuf, nbatch=8):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=40)
+    ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="target seconds of CPU work for the cpu_baseline sample")
-    ap.add_argument("--no-unet", action="store_true", help="skip the configs[3] U-Net forward leg")
+    ap.add_argument("--no-stack", action="store_true", help="skip the configs[1] conv-stack leg")
     ap.add_argument("--no-sliding", action="store_true", help="skip the configs[4]-geometry sliding-window leg")
     ap.add_argument("--no-hbm", action="store_true", help="skip the HBM-bound kernels leg")
     ap.add_argument("--windows-per-forward", type=int, default=8, help="sliding-window leg: windows batched into one forward")
@@ -205,6 +236,49 @@ def main():
                           "tflops": fl / ms / 1e9, "frac_of_mfma_peak": fl / ms / 1e9 / peak,
                           "algorithmic_bytes": int(mxb(N, Ci, S) + mxb(N, Co, S)), "GBps": (mxb(N, Ci, S) + mxb(N, Co, S)) / ms / 1e6}))
         return
+    out = {"metric": METRIC, "unit": "voxels/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+           "dtype": "mxfp8 (e4m3 x e4m3 block-scaled, fp32 accumulate)", "data": "synthetic",
+           "weights": "prepared (quantised, re-laid-out) once and memoised across the timed forwards, as an inference loop keeps them"}
+    u, dom = unet_leg(np, lib, LP, DevBuf, a.steps, a.warmup)
+    out["value"] = u["value"]; out["ms_per_step"] = u["ms_per_forward"]; out["tflops"] = u["tflops"]
+    out["config"] = {"workload": u["workload"], "batch": 2, "dims": [128, 128, 128], "widths": [32, 64, 128, 256], "cin": 4, "head_out": 8, "gflop_per_forward": u["gflop_per_forward"]}
+    prof = KERNEL_TRAFFIC.get(dom["layer"])
+    out["roofline"] = {"bound": "mfma", "kernel": "%s (%s)" % (dom["kernel"], dom["layer"]), "achieved": dom["tflops"], "peak": MFMA_PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+                       "frac": dom["frac_of_mxfp8_peak"], "avg_launch_ms": dom["avg_launch_ms"], "launches": a.steps, "flops_per_launch": dom["flops_per_launch"],
+                       "traffic": prof[0] if prof else None, "traffic_source": prof[1] if prof else None}
+    out["unet"] = u
+    stack = None
+    if not a.no_stack:
+        stack, xq0, w_host_l0 = stack_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, max(a.steps, 20), max(a.warmup, 5))
+        out["conv_stack"] = stack
+    if not a.no_sliding:
+        out["sliding_window"] = sliding_leg(np, lib, LP, DevBuf, a.windows_per_forward)
+    if not a.no_hbm:
+        out["hbm_kernels"] = hbm_leg(np, lib, LP, DevBuf)
+    if not a.no_cpu_baseline:
+        import orc
+        # the oracle (a port: the reference has no CPU MX conv) on a bounded z-slab of the forward's heaviest layer shape class: one 128 -> 128 conv
+        # at N 2 x 64^3, scaled by the forward's FLOPs to voxels/s of the whole U-Net
+        N, Cc, D = 2, 128, 64
+        S = D ** 3
+        rng = np.random.default_rng(0)
+        if stack is None:
+            xq0 = orc.f32_to_mx(8, rng.standard_normal((N, Cc, S)).astype(np.float32), N, Cc, S)
+            w_host_l0 = (rng.standard_normal((Cc, Cc, 27)) * np.sqrt(2.0 / (Cc * 27))).astype(np.float32)
+        nthreads = orc.lib().orc_threads()
+        t = time.perf_counter(); orc.conv3(xq0, 3, N, Cc, D, D, D, w_host_l0, None, Cc, 3, z0=0, z1=1); dt1 = time.perf_counter() - t
+        nz = int(max(1, min(D, a.cpu_seconds / max(dt1, 1e-3))))
+        t = time.perf_counter(); orc.conv3(xq0, 3, N, Cc, D, D, D, w_host_l0, None, Cc, 3, z0=D // 2 - nz // 2, z1=D // 2 - nz // 2 + nz); dt = time.perf_counter() - t
+        gflops = 2.0 * 27 * Cc * Cc * N * S * nz / D / dt / 1e9
+        out["cpu_baseline"] = {"value": 2 * 128 ** 3 / (u["gflop_per_forward"] / gflops), "unit": "voxels/s", "cores": nthreads, "kind": "port",
+                               "sample": "oracle orc_conv3 (the reference has no CPU MX conv) on %d of %d output z planes of a 128 -> 128 conv at N 2 x 64^3: %.1f GFLOP/s, "
+                                         "scaled by the forward's %.0f GFLOP to U-Net voxels/s" % (nz, D, gflops, u["gflop_per_forward"]),
+                               "gflops": gflops}
+    print(json.dumps(out))
+
+
+def stack_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, steps, warmup):
+    """configs[1]: 4 x (3x3x3 conv 128 -> 128, N 2, 64^3, MX-fp8 in / out, bias + GroupNorm(8) statistics, GN + SiLU on the input)."""
     N, Cc, D, L, G = 2, 128, 64, 4, 8
     S = D * D * D
     rng = np.random.default_rng(0)
@@ -219,7 +293,6 @@ def main():
         ws.append(DevBuf.from_numpy(w)); bs.append(DevBuf.from_numpy((rng.standard_normal(Cc) * 0.1).astype(np.float32)))
         gam.append(DevBuf.from_numpy(np.ones(Cc, np.float32))); bet.append(DevBuf.from_numpy(np.zeros(Cc, np.float32)))
         mean.append(DevBuf(N * G * 4)); rstd.append(DevBuf(N * G * 4)); sums.append(DevBuf(N * G * 2 * 24))
-    w_host_l0 = w
     xs = shape5(N, Cc, D, D, D)
 
     def step():
@@ -232,13 +305,13 @@ def main():
             lib.mi_conv_fwd_gn(8, src.ptr, 3, xs, ws[l].ptr, bs[l].ptr, Cc, dst.ptr, 3, gp, sums[l].ptr, G, sp, 1e-5, mean[l].ptr, rstd[l].ptr)
             src = dst
 
-    for _ in range(a.warmup):
+    for _ in range(warmup):
         step()
     LP.check()
     lib.mi_kernel_timing(1)
     lib.mi_sync()
     t0 = time.perf_counter()
-    for _ in range(a.steps):
+    for _ in range(steps):
         step()
     lib.mi_sync()
     t1 = time.perf_counter()
@@ -247,44 +320,19 @@ def main():
     kms = lib.mi_kernel_timing_read(C.byref(nl))
     lib.mi_kernel_timing(0)
     kernel = lib.mi_last_kernel().decode()
-    ms_step = (t1 - t0) * 1e3 / a.steps
-    vox_per_step = N * S
+    ms_step = (t1 - t0) * 1e3 / steps
     flops_layer = 2.0 * 27 * Cc * Cc * N * S               # logical channels, all 27 taps (tests/bench_lp.c:46)
     k_ms = kms / max(nl.value, 1)
     achieved = flops_layer / (k_ms * 1e-3) / 1e12
-    out = {
-        "metric": METRIC, "value": vox_per_step / (ms_step * 1e-3), "unit": "voxels/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "mxfp8 (e4m3 x e4m3, fp32 accumulate)",
-        "data": "synthetic",
-        "config": {"workload": "configs[1]: 4 x (3x3x3 conv 128->128, N 2, 64^3, MX-fp8 in/out, bias + GroupNorm(8) stats, GN+SiLU on the input)",
-                   "layers": L, "batch": N, "channels": Cc, "dims": [D, D, D]},
-        "tflops": L * flops_layer / (ms_step * 1e-3) / 1e12,
-        "roofline": {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_FP8_TFLOPS,
-                     "launches": nl.value, "avg_launch_ms": k_ms, "flops_per_launch": flops_layer,
-                     # HBM-side bytes per launch: not measurable from inside the process; the figure of the committed counter runs
-                     # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy) for this kernel at this shape
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH, "traffic_source": "profiles/conv3_mx_f8_c128_64cube_hbm_traffic.txt",
-                     "algorithmic_bytes": 2 * N * (Cc // 32) * S * 33 + 28 * Cc * Cc * 33 // 32},
-    }
-    if not a.no_unet:
-        out["unet"] = unet_leg(np, lib, LP, DevBuf, max(3, a.steps // 4), max(1, a.warmup))
-    if not a.no_sliding:
-        out["sliding_window"] = sliding_leg(np, lib, LP, DevBuf, a.windows_per_forward)
-    if not a.no_hbm:
-        out["hbm_kernels"] = hbm_leg(np, lib, LP, DevBuf)
-    if not a.no_cpu_baseline:
-        import orc
-        # the oracle (a port: the reference has no CPU MX conv) on a bounded z-slab of one layer of the same workload
-        xq = x0.to_numpy(np.uint8)
-        nthreads = orc.lib().orc_threads()
-        t = time.perf_counter(); orc.conv3(xq, 3, N, Cc, D, D, D, w_host_l0, None, Cc, 3, z0=0, z1=1); dt1 = time.perf_counter() - t
-        nz = int(max(1, min(D, a.cpu_seconds / max(dt1, 1e-3))))
-        t = time.perf_counter(); orc.conv3(xq, 3, N, Cc, D, D, D, w_host_l0, None, Cc, 3, z0=D // 2 - nz // 2, z1=D // 2 - nz // 2 + nz); dt = time.perf_counter() - t
-        layer_s = dt * D / nz                                   # a whole layer, extrapolated from the slab
-        out["cpu_baseline"] = {"value": vox_per_step / (L * layer_s), "unit": "voxels/s", "cores": nthreads, "kind": "port",
-                               "sample": "oracle orc_conv3 on %d of %d output z planes (both samples) of layer 0, scaled to the 4-layer stack" % (nz, D),
-                               "gflops": flops_layer * nz / D / dt / 1e9}
-    print(json.dumps(out))
+    rec = {"workload": "configs[1]: 4 x (3x3x3 conv 128->128, N 2, 64^3, MX-fp8 in/out, bias + GroupNorm(8) stats, GN+SiLU on the input)",
+           "value": N * S / (ms_step * 1e-3), "unit": "voxels/s", "ms_per_step": ms_step, "steps": steps, "warmup": warmup, "tflops": L * flops_layer / (ms_step * 1e-3) / 1e12,
+           "roofline": {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_FP8_TFLOPS,
+                        "launches": nl.value, "avg_launch_ms": k_ms, "flops_per_launch": flops_layer,
+                        # HBM-side bytes per launch: not measurable from inside the process; the figure of the committed counter runs
+                        # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy) for this kernel at this shape
+                        "traffic": TRAFFIC_BYTES_PER_LAUNCH, "traffic_source": "profiles/conv3_mx_f8_c128_64cube_hbm_traffic.txt",
+                        "algorithmic_bytes": 2 * N * (Cc // 32) * S * 33 + 28 * Cc * Cc * 33 // 32}}
+    return rec, x0.to_numpy(np.uint8), w
 
 
 if __name__ == "__main__":

@@ -143,6 +143,9 @@ int mi_conv_fwd_gn(int bits, const void *x, int xbf, shape5 xs, const float *w, 
    stream it runs on and clears the totals; read returns the total milliseconds so far and the number of launches (synchronises) */
 void mi_kernel_timing(int on);
 double mi_kernel_timing_read(long *launches);
+/* launch i of the log kept since mi_kernel_timing(1), in launch order: its milliseconds, its algorithmic FLOPs (2 x 27 x Cin x Cout x output
+   voxels, logical channels) and its kernel variant's name; returns the number of launches logged (synchronises) */
+long mi_kernel_timing_launch(long i, float *ms, double *flops, char *name, size_t name_bytes);
 /* No counterpart in the reference. lp_conv_fwd_f8 / lp_conv_fwd_f4 (bits 8 / 4) for callers that cannot allocate device memory: code under
    HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. Same arguments, same kernels and bit-identical results, but every
    byte of scratch (prepared weights, re-staged operands, statistics partials, the constant page) comes from one fixed device array of

@@ -76,12 +76,12 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
     if (i >= (size_t)npairs_all * Cop) return;
     const int cop = (int)(i % Cop), gp = (int)(i / Cop);
     int b0 = 0, pb = 0, nbc = 0;
-    for (;; b0 += CB) { nbc = min(CB, nbt - b0); const int np = (27 * nbc + 1) >> 1; if (gp < pb + np) break; pb += np; }
+    if (block_major >= 0) for (;; b0 += CB) { nbc = min(CB, nbt - b0); const int np = (27 * nbc + 1) >> 1; if (gp < pb + np) break; pb += np; }
     const int q = gp - pb, m = cop >> 5, r = cop & 31;
     uint8_t *tile = wq + ((size_t)gp * nmt_all + m) * WTILE;
     unsigned *tsc = wsc + ((size_t)gp * nmt_all + m) * 64;      // one word per lane: the byte the MFMA reads is the low one
     int tss = 1;                                                // words between two lanes' scale words
-    if (block_major) {
+    if (block_major > 0) {
         // the wide kernel's layout (block_major = its channel tiles per workgroup, 4 or 2): per slice of that many tiles, pair after pair the
         // image of its LDS stage: the tiles' codes, then per lane the tiles' scale words
         const int MW = block_major, sl = m / MW, mi = m - sl * MW;
@@ -92,12 +92,21 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
     for (int side = 0; side < 2; side++) {
         const int u = 2 * q + side;
         float v[32]; float amax = 0.f;
-        // K order inside a chunk: tap by tap over its blocks, or (the wide kernel, one chunk) block by block over the taps
-        const int t = block_major ? u % 27 : u / nbc, blk = block_major ? u / 27 : b0 + u % nbc;
+        // K order inside a chunk: tap by tap over its blocks, or (the wide kernel, one chunk) block by block over the taps; the row kernel
+        // (block_major < 0): per block 15 pairs (class c, ky), class c < 3 = taps (c, ky, 0 | 1), class 3 = (0 | 1, ky, 2), class 4 = (2, ky, 2 | none)
+        int t = block_major ? u % 27 : u / nbc, blk = block_major ? u / 27 : b0 + u % nbc;
+        bool unit_ok = u < 27 * nbc;
+        if (block_major < 0) {
+            const int qq = gp % 15, c = qq / 3, ky = qq % 3;
+            blk = gp / 15;
+            const int kz = c < 3 ? c : c == 3 ? side : 2, kx = c < 3 ? side : 2;
+            t = kz * 9 + ky * 3 + kx;
+            unit_ok = !(c == 4 && side == 1);
+        }
 #pragma unroll
         for (int k = 0; k < 32; k++) {
             const int ci = seg_ci(blk * 32 + k, Ci, Cx, CxP);
-            v[k] = (u < 27 * nbc && cop < Co && ci >= 0) ? w[((size_t)cop * Ci + ci) * 27 + t] : 0.f;
+            v[k] = (unit_ok && cop < Co && ci >= 0) ? w[((size_t)cop * Ci + ci) * 27 + t] : 0.f;
             amax = fmaxf(amax, fabsf(v[k]));
         }
         const int e = d_mx_exp(amax, FMT == 8 ? MI_INVQ8 : MI_INVQ4);
@@ -139,22 +148,43 @@ thread_local char g_last_kernel[128] = "";
 
 // optional timing of the conv kernel launches alone (benchmarks): event pairs on the stream the kernel runs on
 static bool g_ktime = false;
-static std::vector<std::pair<hipEvent_t, hipEvent_t>> g_kev;
+struct kev_t { hipEvent_t e0, e1; double flops; char name[96]; };
+static std::vector<kev_t> g_kev;
 static double g_kms = 0.0; static long g_kn = 0;
+struct klaunch_t { float ms; double flops; char name[96]; };
+static std::vector<klaunch_t> g_klog;             // every timed launch since mi_kernel_timing(1), in launch order
 extern "C" void mi_kernel_timing(int on) {
-    for (auto &e : g_kev) { MIRT(hipEventDestroy(e.first)); MIRT(hipEventDestroy(e.second)); }
-    g_kev.clear(); g_kms = 0.0; g_kn = 0; g_ktime = on != 0;
+    for (auto &e : g_kev) { MIRT(hipEventDestroy(e.e0)); MIRT(hipEventDestroy(e.e1)); }
+    g_kev.clear(); g_klog.clear(); g_kms = 0.0; g_kn = 0; g_ktime = on != 0;
 }
-extern "C" double mi_kernel_timing_read(long *launches) {       // total milliseconds of the timed launches so far (synchronises)
+static void ktime_collect() {
     for (auto &e : g_kev) {
         float ms = 0.f;
-        MIRT(hipEventSynchronize(e.second)); MIRT(hipEventElapsedTime(&ms, e.first, e.second));
+        MIRT(hipEventSynchronize(e.e1)); MIRT(hipEventElapsedTime(&ms, e.e0, e.e1));
         g_kms += ms; g_kn++;
-        MIRT(hipEventDestroy(e.first)); MIRT(hipEventDestroy(e.second));
+        klaunch_t l; l.ms = ms; l.flops = e.flops; memcpy(l.name, e.name, sizeof l.name); g_klog.push_back(l);
+        MIRT(hipEventDestroy(e.e0)); MIRT(hipEventDestroy(e.e1));
     }
     g_kev.clear();
+}
+extern "C" double mi_kernel_timing_read(long *launches) {       // total milliseconds of the timed launches so far (synchronises)
+    ktime_collect();
     if (launches) *launches = g_kn;
     return g_kms;
+}
+extern "C" long mi_kernel_timing_launch(long i, float *ms, double *flops, char *name, size_t name_bytes) {     // launch i of the log; returns the log's length (synchronises)
+    ktime_collect();
+    if (i >= 0 && i < (long)g_klog.size()) {
+        if (ms) *ms = g_klog[i].ms;
+        if (flops) *flops = g_klog[i].flops;
+        if (name && name_bytes) { strncpy(name, g_klog[i].name, name_bytes - 1); name[name_bytes - 1] = 0; }
+    }
+    return (long)g_klog.size();
+}
+static void ktime_push(hipEvent_t ev0, hipEvent_t ev1, double flops) {
+    kev_t k; k.e0 = ev0; k.e1 = ev1; k.flops = flops;
+    strncpy(k.name, g_last_kernel, sizeof k.name - 1); k.name[sizeof k.name - 1] = 0;
+    g_kev.push_back(k);
 }
 extern "C" const char *mi_last_kernel(void) { return g_last_kernel; }
 
@@ -219,7 +249,7 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     const bool ktime = g_ktime && !mi_ws_arena_on();
     if (ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
     conv3_stem_launch(CP, MT, ybf == 3 ? 8 : ybf == 4 ? 4 : 0, a, smem);
-    if (ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
+    if (ktime) { MIRT(hipEventRecord(ev1, 0)); ktime_push(ev0, ev1, 2.0 * 27 * Ci * (double)cout * N * Do * H * W); }
     if (osum) conv_stats_reduce(who, a, MT, sp, osum);
     return 0;
 }
@@ -360,11 +390,18 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     static int areg_env = -1;
     if (areg_env < 0) areg_env = getenv("MI_CONV_AREG") ? atoi(getenv("MI_CONV_AREG")) : 1;      // tuning knob: 0 keeps the general kernel for every shape
     a.areg = areg_env && !big && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && a.nbt == 1 && a.wide && (NT == 2 || NT == 4);
-    size_t smem = a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
+    // one channel tile of 17 .. 32 output channels from two or more input blocks on a volume wider than one 16-voxel tile: the row kernel (runs
+    // of 32 voxels along x, input fragments shared by the three ky taps). One input block stays with the kernel that keeps its weights in
+    // registers, which measures a few percent faster there (both are bound by the halo's cache misses in flight, and it loads no weights)
+    static int row_env = -1;
+    if (row_env < 0) row_env = getenv("MI_CONV_ROW") ? atoi(getenv("MI_CONV_ROW")) : 1;      // tuning knob: 0 keeps the other kernels for these shapes, 2 also takes one input block
+    a.row = row_env && !big && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 ? 1 : 2) && a.nbt <= 64;
+    if (a.row) { a.areg = false; a.CB = a.nbt; }
+    size_t smem = a.row ? (size_t)2 * 2048 * (RB + 4) : a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     smem = (smem + 15) & ~(size_t)15;
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);      // bias, affine a, b of the workgroup's channels
     a.red_o = (unsigned)smem; smem += 1024;                                     // statistics scratch
-    if (big || a.areg) {
+    if (big || a.areg || a.row) {
         // rows and scale bytes of positions outside the volume: 64 zero bytes, then 64 bytes of value 1; one page per device, kept for the process
         // (the entry point that must not allocate keeps its own at the head of its fixed scratch)
         static uint8_t *zpage[8];
@@ -381,11 +418,12 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         }
     }
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
-    a.ntx = (Wo + 15) / 16; a.nty = (Ho + 7) / 8; a.ntz = (Do + TZ - 1) / TZ;
+    a.ntx = a.row ? (Wo + 31) / 32 : (Wo + 15) / 16; a.nty = (Ho + 7) / 8; a.ntz = (Do + TZ - 1) / TZ;      // (the row kernel: 4 x 8 x 32 voxels per tile)
     a.ntiles = (unsigned)((size_t)a.ntx * a.nty * a.ntz * a.ncs * N);
     // ---- weights ----
     int npairs_all = 0;
     for (int b0 = 0; b0 < a.nbt; b0 += a.CB) npairs_all += (27 * (a.nbt - b0 < a.CB ? a.nbt - b0 : a.CB) + 1) >> 1;
+    if (a.row) npairs_all = 15 * a.nbt;              // (15 pairs per input block: its tap classes)
     // (sixteen pairs of padding: the kernels' weight loads run up to two ring stages ahead of the last pair)
     // (the wide kernel's weights are one buffer: codes and scale words interleaved pair by pair; its scale buffer is a stub)
     const size_t wq_bytes = (size_t)(npairs_all + 16) * nmt_all * (big ? WTILE + 256 : WTILE), wsc_bytes = big ? 256 : (size_t)(npairs_all + 16) * nmt_all * 256;
@@ -398,18 +436,18 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (sp.wkey && !mi_ws_arena_on()) {
         std::lock_guard<std::mutex> lk(g_wmemo_mu);
         for (auto &m : g_wmemo)
-            if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == memoCB && m.nmt_all == nmt_all && m.dev == dev && m.lay == (big ? MT : 0)) { wq = m.wq; wsc = m.wsc; have = true; break; }
+            if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == memoCB && m.nmt_all == nmt_all && m.dev == dev && m.lay == (big ? MT : a.row ? 100 : 0)) { wq = m.wq; wsc = m.wsc; have = true; break; }
         if (!have) {
             MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes)); mi_count_alloc(); mi_count_alloc();
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
             MIRT(hipMemsetAsync(wq, 0, wq_bytes, 0)); MIRT(hipMemsetAsync(wsc, 0, wsc_bytes, 0));
-            g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, memoCB, nmt_all, dev, big ? MT : 0, wq, wsc});
+            g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, memoCB, nmt_all, dev, big ? MT : a.row ? 100 : 0, wq, wsc});
         }
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) {
         const size_t nt = (size_t)npairs_all * nmt_all * 32;
-        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : 0);
-        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : 0);
+        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : 0);
+        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : 0);
         MICK();
     }
     a.wq = wq; a.wsc = wsc;
@@ -422,7 +460,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
     if (fmt == 8) { if (out == 8) conv3_launch_f8_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f8_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f8_o0(stride, epi, MT, NT, a, smem); }
     else { if (out == 8) conv3_launch_f4_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f4_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f4_o0(stride, epi, MT, NT, a, smem); }
-    if (ktime) { MIRT(hipEventRecord(ev1, 0)); g_kev.push_back({ev0, ev1}); }
+    if (ktime) { MIRT(hipEventRecord(ev1, 0)); ktime_push(ev0, ev1, 2.0 * 27 * Ci * (double)cout * N * Do * Ho * Wo); }
     if (osum) conv_stats_reduce(who, a, MT, sp, osum);
     return 0;
 }
@@ -491,7 +529,7 @@ static size_t conv_scratch_bound(int fmt, const void *x2, int xbf, shape5 xs, in
     size_t need = 256;                                              // the constant page
     if (Ci <= 16 && !x2 && fmt == 8) need += al((size_t)9 * nmt_all * 2048) + al((size_t)9 * nmt_all * 256);      // the tap-packed kernels' weights
     const int nbt = (Cx + 31) / 32 + (x2 ? (C2 + 31) / 32 : 0);
-    need += al(((size_t)(27 * nbt + 1) / 2 + nbt + 16) * nmt_all * 2304) + al(((size_t)(27 * nbt + 1) / 2 + nbt + 16) * nmt_all * 256);
+    need += al(((size_t)(27 * nbt + 1) / 2 + 2 * nbt + 16) * nmt_all * 2304) + al(((size_t)(27 * nbt + 1) / 2 + 2 * nbt + 16) * nmt_all * 256);      // (at most 15 pairs per block)
     const bool s2g = x2 && sp.gp2.G;
     for (int s = 0; s < (x2 ? 2 : 1); s++) {
         const gnp_t g = s2g ? (s ? sp.gp2 : gp) : gp;

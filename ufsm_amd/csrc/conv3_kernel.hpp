@@ -107,6 +107,7 @@ struct conv_args {
     int zc; unsigned ngrp;             // consecutive z tiles a workgroup walks, workgroups with work
     bool big;                          // the wide kernel takes the launch (MT 4, or MT 2 with NT 4)
     bool areg;                         // the persistent small-channel kernel (one channel tile, one input block, weights in registers) takes the launch
+    bool row;                          // the row kernel (one channel tile, any number of input blocks, 4 x 8 x 32 voxel tiles) takes the launch
 };
 
 template <int FMT> struct fmt_t;
@@ -237,7 +238,9 @@ __device__ __forceinline__ void conv_epi_consts(const conv_args &a, unsigned cha
 // FULL: the tile lies inside the output and the statistics cover all of its planes (uniform, checked by the caller): no per-lane predicates,
 // so the whole epilogue is straight-line code the scheduler can interleave across the accumulator tiles
 // NOCH: the caller never takes per-channel statistics records (stat_ch): their 32 sums are not kept
-template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false, bool NOCH = false>
+// NW: wavefronts of the workgroup (their partial statistics are summed in wave order); ROW: the row kernel's voxel mapping, lane r of tile j
+// holds voxel (oz0 + lz, oy0 + ly0 + j, ox0 + r) of a 32-voxel run along x
+template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false, bool NOCH = false, int NW = 4, bool ROW = false>
 __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT][NT], unsigned char *lds, unsigned tile, int n, int cs,
                                               int oz0, int oy0, int ox0, int lz, int ly0, int tid) {
     const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
@@ -252,6 +255,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) { qs[m][q4] = 0.f; qss[m][q4] = 0.f; }
     constexpr bool CH = MT == 1 && !NOCH;
+    static_assert(!CH || NW == 4, "per-channel statistics records: four wavefronts");
     float chs[CH ? 16 : 1], chss[CH ? 16 : 1];               // per-channel sums (MT 1, stat_ch)
 #pragma unroll
     for (int i = 0; i < (CH ? 16 : 1); i++) { chs[i] = 0.f; chss[i] = 0.f; }
@@ -276,7 +280,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
         }
         static_for<NT>([&](auto J) {
             constexpr int j = J;
-            const int oz = oz0 + lz, oy = oy0 + ly0 + 2 * j + (r >> 4), ox = ox0 + (r & 15);
+            const int oz = oz0 + lz, oy = ROW ? oy0 + ly0 + j : oy0 + ly0 + 2 * j + (r >> 4), ox = ROW ? ox0 + r : ox0 + (r & 15);
             const bool ok = FULL || (oz < a.Do && oy < a.Ho && ox < a.Wo);
             const size_t ov = ((size_t)(oz + a.yzo) * a.Ho + oy) * a.Wo + ox;
             const bool zst = FULL || (ok && oz >= a.zs0 && oz < a.zs1);
@@ -394,7 +398,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
         __syncthreads();
         if (tid < 32) {
             float s1 = 0.f, s2 = 0.f;
-            for (int w = 0; w < 4; w++) { s1 += red[(w * 32 + tid) * 2]; s2 += red[(w * 32 + tid) * 2 + 1]; }
+            for (int w = 0; w < NW; w++) { s1 += red[(w * 32 + tid) * 2]; s2 += red[(w * 32 + tid) * 2 + 1]; }
             a.part[((size_t)tile * 32 + tid) * 2] = s1; a.part[((size_t)tile * 32 + tid) * 2 + 1] = s2;
         }
     } else if (stats) {
@@ -419,7 +423,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
             // in a fixed order into the exact sum slots, so the statistics do not depend on the order workgroups finish in
             const int m = tid >> 3, q8 = tid & 7;                       // q8 = q4 * 2 + h: channels co_base + 32 m + 8 q4 + 4 h .. + 3
             float s = 0.f, ss = 0.f;
-            for (int w = 0; w < 4; w++) { s += red[((w * MT + m) * 8 + q8) * 2]; ss += red[((w * MT + m) * 8 + q8) * 2 + 1]; }
+            for (int w = 0; w < NW; w++) { s += red[((w * MT + m) * 8 + q8) * 2]; ss += red[((w * MT + m) * 8 + q8) * 2 + 1]; }
             a.part[((size_t)tile * MT * 8 + tid) * 2] = s;
             a.part[((size_t)tile * MT * 8 + tid) * 2 + 1] = ss;
         }
@@ -585,6 +589,7 @@ static void launch_conv(const conv_args &a, size_t smem) {
 }
 #include "conv3_wide.hpp"
 #include "conv3_small.hpp"
+#include "conv3_row.hpp"
 template <int FMT, int STRIDE, int OUT, bool EPI>
 static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     switch (MT * 10 + NT) {
@@ -598,7 +603,7 @@ static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     case 22: launch_conv<FMT, STRIDE, 2, 2, OUT, EPI>(a, smem); break;
     case 32: launch_conv<FMT, STRIDE, 3, 2, OUT, EPI>(a, smem); break;
     case 42: launch_conv<FMT, STRIDE, 4, 2, OUT, EPI>(a, smem); break;
-    case 14: if constexpr (STRIDE == 1) { if (a.areg) launch_small<FMT, 4, OUT, EPI>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
+    case 14: if constexpr (STRIDE == 1) { if (a.row) launch_row<FMT, OUT, EPI>(a, smem); else if (a.areg) launch_small<FMT, 4, OUT, EPI>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
     case 24: if constexpr (STRIDE == 1) { if (a.big) launch_wide<FMT, OUT, EPI, 2>(a, smem); else launch_conv<FMT, 1, 2, 4, OUT, EPI>(a, smem); break; }
     default: mi_die("conv3: no kernel for MT %d NT %d stride %d", MT, NT, STRIDE);
     }

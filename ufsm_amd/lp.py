@@ -98,6 +98,7 @@ _PROTOS = {
     "mi_alloc_count": (C.c_long, []),
     "mi_kernel_timing": (None, [_I]),
     "mi_kernel_timing_read": (C.c_double, [C.POINTER(C.c_long)]),
+    "mi_kernel_timing_launch": (C.c_long, [C.c_long, C.POINTER(C.c_float), C.POINTER(C.c_double), C.c_char_p, _Z]),
     "mi_last_kernel": (C.c_char_p, []),
 }
 EXPORTS = tuple(_PROTOS)
