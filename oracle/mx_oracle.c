@@ -140,6 +140,33 @@ float orc_h16_to_f32(uint16_t h) {
     return u2f(s | ((e + 112u) << 23) | (m << 13));
 }
 
+/* a double -> binary16, round to nearest even (the double is the exact value to round) */
+static uint16_t f64_to_h16(double x) {
+    const uint16_t s = signbit(x) ? 0x8000u : 0u;
+    double a = fabs(x);
+    if (a != a) return (uint16_t)(s | 0x7e00u);
+    if (a >= 65520.0) return (uint16_t)(s | 0x7c00u);
+    if (a == 0.0) return s;
+    int ex; frexp(a, &ex);                                  /* a = f 2^ex, f in [.5, 1): leading bit at 2^(ex - 1) */
+    const int q = ex - 1 < -14 ? -24 : ex - 1 - 10;          /* the quantum's exponent: 11 significant bits, or the subnormal step */
+    const double k = rint(ldexp(a, -q));                    /* exact scaling, rint ties to even in the default rounding mode */
+    const double r = ldexp(k, q);
+    if (r >= 65536.0) return (uint16_t)(s | 0x7c00u);
+    return (uint16_t)(s | orc_f32_to_h16((float)r));        /* r is a binary16 value: the conversion is exact */
+}
+/* binary16 fused multiply-add of binary16 operands, one rounding (HFMA2, src/lp_common.cuh:703). The product of two 11-bit significands
+   is exact in a double; the sum with c is formed with its rounding error (two-sum), and where the double sum sits exactly on a binary16
+   tie while the error is not zero it is moved off the tie in the error's direction before the one rounding to binary16 */
+static uint16_t h16_fma(uint16_t a, uint16_t b, uint16_t c) {
+    const double p = (double)orc_h16_to_f32(a) * (double)orc_h16_to_f32(b), cd = (double)orc_h16_to_f32(c);
+    if (p != p || cd != cd || isinf(p) || isinf(cd)) return f64_to_h16(p + cd);
+    double sum = p + cd;
+    const double bb = sum - p, err = (p - (sum - bb)) + (cd - bb);
+    if (err != 0.0) sum = nextafter(sum, err > 0.0 ? INFINITY : -INFINITY);   /* (only matters on a tie; elsewhere one double ulp changes nothing) */
+    return f64_to_h16(sum);
+}
+uint16_t orc_h16_fma(uint16_t a, uint16_t b, uint16_t c) { return h16_fma(a, b, c); }
+
 /* ---------- one block row (src/lp_mxops.cuh:45-65 for the NaN-propagating amax; src/lp_f8fwd.cuh:90-103 for fmaxf) ---------- */
 static void enc_codes(int bits, const float *v, int bw, float m, uint8_t *codes) {
     if (bits == 8) for (int k = 0; k < bw; k++) codes[k] = (uint8_t)orc_enc_e4m3(v[k] * m);
@@ -294,7 +321,7 @@ static void quant_row(int cbits, const float *v, float *sv, float *sf) {
     for (int k = 0; k < 32; k++) sv[k] = cbits == 8 ? orc_dec_e4m3(codes[k]) : orc_dec_e2m1((codes[k >> 1] >> (4 * (k & 1))) & 15u);
 }
 /* decoder up segment (src/lp_common.cuh:618-670): coarse rows -> GN + SiLU -> e4m3 rows with a row scale (amax ignoring NaN) */
-static void coarse_rows(const orc_conv_t *c, int n, int blk, int Cx, const chab_t *tab, int Dc, int Hc, int Wc, float *cv /* [Sc][32 codes + scale] */) {
+static void coarse_rows(const orc_conv_t *c, int n, int blk, int Cx, const chab_t *tab, int Dc, int Hc, int Wc, float *cv /* [Sc][32 codes + scale] */, uint8_t *cvsb /* [Sc] scale bytes */) {
     const size_t Sc = (size_t)Dc * Hc * Wc;
     const mxt_t t = mxt(c->x, c->xdt == 3 ? 8 : 4, c->N, Cx, Sc);
     for (size_t v = 0; v < Sc; v++) {
@@ -306,6 +333,7 @@ static void coarse_rows(const orc_conv_t *c, int n, int blk, int Cx, const chab_
         /* stored as code and scale; the blend multiplies the weight by the scale first (stage_up_smem) */
         for (int k = 0; k < 32; k++) cv[v * 33 + k] = orc_dec_e4m3(orc_enc_e4m3(r[k] * m));
         cv[v * 33 + 32] = s;
+        cvsb[v] = (uint8_t)(e + 127);
     }
 }
 static int build_staged(const orc_conv_t *c, staged_t *st) {
@@ -318,6 +346,8 @@ static int build_staged(const orc_conv_t *c, staged_t *st) {
     st->sf = (float *)malloc((size_t)c->N * st->nch * S * sizeof(float));
     if (!st->sv || !st->sf) return -1;
     const int G = c->gp.G || c->gp2.G;
+    /* the fp4 entry blends the fused upsample in binary16 (src/lp_f4fwd.cuh:1135-1136, UFSM_UP_H2 default), the fp8 entry in fp32; up 2 / 3 force one */
+    const int uph2 = c->up == 2 || (c->up == 1 && c->cbits == 4);
     const int Dc = c->D >> 1, Hc = c->H >> 1, Wc = c->W >> 1;
     for (int n = 0; n < c->N; n++) {
         chab_t *tab = (chab_t *)malloc((size_t)Cip * sizeof(chab_t));
@@ -325,8 +355,8 @@ static int build_staged(const orc_conv_t *c, staged_t *st) {
         for (int ch = 0; ch < st->nch; ch++) {
             const int upc = mxin && c->up && ch * 32 < CxP;
             const int sec = mxin && ch * 32 >= CxP;       /* chunk of the x2 segment */
-            float *cv = NULL;
-            if (upc) { cv = (float *)malloc((size_t)Dc * Hc * Wc * 33 * sizeof(float)); coarse_rows(c, n, ch, Cx, tab, Dc, Hc, Wc, cv); }
+            float *cv = NULL; uint8_t *cvsb = NULL;
+            if (upc) { cv = (float *)malloc((size_t)Dc * Hc * Wc * 33 * sizeof(float)); cvsb = (uint8_t *)malloc((size_t)Dc * Hc * Wc); coarse_rows(c, n, ch, Cx, tab, Dc, Hc, Wc, cv, cvsb); }
             mxt_t t;
             if (mxin) t = sec ? mxt(c->x2, xbits, c->N, c->Ci - Cx, S) : mxt(c->x, xbits, c->N, Cx, S);
             const int blk = sec ? ch - CxP / 32 : ch;
@@ -342,6 +372,21 @@ static int build_staged(const orc_conv_t *c, staged_t *st) {
                     my[0] = gy >> 1; my[1] = my[0] + ((gy & 1) ? 1 : -1); if (my[1] < 0) my[1] = 0; if (my[1] > Hc - 1) my[1] = Hc - 1;
                     mx[0] = gx >> 1; mx[1] = mx[0] + ((gx & 1) ? 1 : -1); if (mx[1] < 0) mx[1] = 0; if (mx[1] > Wc - 1) mx[1] = Wc - 1;
                     for (int k = 0; k < 32; k++) r[k] = 0.f;
+                    if (uph2) {   /* binary16 blend (stage_up_smem_h2, src/lp_common.cuh:674-712): weights relative to the largest of the 8 rows' scales */
+                        unsigned em = 0;
+                        for (int t8 = 0; t8 < 8; t8++) { const unsigned sb = cvsb[((size_t)mz[t8 >> 2] * Hc + my[(t8 >> 1) & 1]) * Wc + mx[t8 & 1]]; if (sb > em) em = sb; }
+                        uint16_t acc[32];
+                        for (int k = 0; k < 32; k++) acc[k] = 0;
+                        for (int a = 0; a < 2; a++) for (int b = 0; b < 2; b++) for (int cc = 0; cc < 2; cc++) {
+                            const size_t ri = ((size_t)mz[a] * Hc + my[b]) * Wc + mx[cc];
+                            const float *row = cv + ri * 33;
+                            const int de = (int)cvsb[ri] - (int)em;
+                            const uint16_t w3 = orc_f32_to_h16((a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (cc ? 0.25f : 0.75f) * (de >= -126 ? u2f((uint32_t)(127 + de) << 23) : 0.f));
+                            for (int k = 0; k < 32; k++) acc[k] = h16_fma(w3, orc_f32_to_h16(row[k]), acc[k]);      /* (an e4m3 value is a binary16 value) */
+                        }
+                        const float sm = orc_mx_scale(em);
+                        for (int k = 0; k < 32; k++) r[k] = orc_h16_to_f32(acc[k]) * sm;
+                    } else
                     for (int a = 0; a < 2; a++) for (int b = 0; b < 2; b++) for (int cc = 0; cc < 2; cc++) {
                         const float *row = cv + (((size_t)mz[a] * Hc + my[b]) * Wc + mx[cc]) * 33;
                         const float w3 = (a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (cc ? 0.25f : 0.75f) * row[32];
@@ -379,7 +424,7 @@ static int build_staged(const orc_conv_t *c, staged_t *st) {
                     quant_row(c->cbits, r, sv, sf);
                 }
             }
-            free(cv);
+            free(cv); free(cvsb);
         }
         free(tab);
     }

@@ -86,7 +86,8 @@ typedef struct {
     const void *x; int xdt;            /* 0 fp32 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4 */
     int N, Ci, D, H, W;                /* output-resolution input dims for stride 1; the input's dims for stride 2 */
     const void *x2; int c_split;       /* channels >= c_split come from x2 (same dtype) */
-    int up;                            /* the x segment is stored at D/2 x H/2 x W/2 and read trilinearly upsampled */
+    int up;                            /* the x segment is stored at D/2 x H/2 x W/2 and read trilinearly upsampled: 1 the entry's own blend (fp32 chain
+                                          for e4m3 compute, binary16 for e2m1 compute), 2 binary16, 3 fp32 */
     orc_gn_t gp, gp2;                  /* GN + SiLU of x (or of all channels when gp2.G == 0) and of x2 */
     /* weights */
     const float *w, *b; int Co; int stride;   /* 3x3x3, pad 1, stride 1 or 2 */
@@ -138,6 +139,7 @@ void orc_set_align_bits(int b);         /* drift studies: width of the acc64 == 
 void orc_set_act_mode(int m);          /* drift studies: 1 evaluates the activation by a fast fp32 path (a few ulp off), 0 (default) exactly */
 uint16_t orc_f32_to_h16(float f);
 float orc_h16_to_f32(uint16_t h);
+uint16_t orc_h16_fma(uint16_t a, uint16_t b, uint16_t c);   /* binary16 fused multiply-add, one rounding */
 int orc_threads(void);
 #ifdef __cplusplus
 }

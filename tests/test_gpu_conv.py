@@ -573,3 +573,26 @@ def test_config2_full_size_down_and_decoder(gpu):
         want, _ = orc.conv3(qa, 4, N, 384, D, D, D, w, None, 128, 4, cbits=4, x2=qb, c_split=256, up=1, z0=z, z1=z + 1)
         wd = orc.mx_to_f32(4, want, N, 128, S).reshape(N, 128, D, D, D)
         assert np.array_equal(dec[:, :, z], wd[:, :, z]), z
+
+
+@pytest.mark.parametrize("cbits,up", [(4, 1), (4, 2), (4, 3), (8, 1), (8, 2)])
+def test_fused_upsample_blend_modes(gpu, cbits, up):
+    """The fused-upsample staging's two blends on non-grid data with row scales spread over 2^12: the fp4 entry's default (up 1) is the binary16
+    blend (src/lp_common.cuh:674-712, chosen at src/lp_f4fwd.cuh:1135-1136), the fp8 entry's the fp32 chain; up 2 / 3 force one. The e2m1 products
+    of the matrix cores are summed exactly, so under e2m1 compute the fp32 output agrees with the oracle's fp64 accumulation to 1e-5 only if
+    every staged code is the same: one differing code of a row shows as ~1e-2."""
+    rng = np.random.default_rng(300 + 10 * cbits + up)
+    N, Cu, Cs, Co, D, H, W = 1, 64, 32, 32, 8, 8, 16
+    S, Sc = D * H * W, (D // 2) * (H // 2) * (W // 2)
+    xa = (rng.standard_normal((N, Cu, Sc)) * np.exp(rng.uniform(-4, 4, (N, 1, Sc)))).astype(np.float32)
+    xb = rng.standard_normal((N, Cs, S)).astype(np.float32)
+    w = (rng.standard_normal((Co, Cu + Cs, 27)) * np.sqrt(2.0 / ((Cu + Cs) * 27))).astype(np.float32)
+    qa, qb = orc.f32_to_mx(8, xa, N, Cu, Sc), orc.f32_to_mx(8, xb, N, Cs, S)
+    want, _ = orc.conv3(qa, 3, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=cbits, x2=qb, c_split=Cu, up=up, acc64=1)
+    got, _ = gpu_conv(qa, 3, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=cbits, x2=qb, c_split=Cu, up=up)
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err < (1e-5 if cbits == 4 else 2e-3), err
+    if cbits == 4 and up != 1:                                      # the entry's default is the binary16 blend, and the two blends are different operands
+        other, _ = orc.conv3(qa, 3, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=4, x2=qb, c_split=Cu, up=5 - up, acc64=1)
+        d = np.abs(got - other).max() / np.abs(want).max()
+        assert d > 1e-4, d

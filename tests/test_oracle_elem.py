@@ -163,3 +163,124 @@ def test_gn_silu_apply_closed_forms():
     orc.lib().orc_gn_silu_apply_mx(orc.ptr(big), 0, 1, 32, 8, orc.gn(one, zero, np.zeros(1, np.float32), np.ones(1, np.float32), 1), orc.ptr(got3), 8)
     d3 = decoded(8, got3, 1, 32, 8)
     assert np.all(d3[0, :16] == 40.0) and np.all(d3[0, 16:] == 0.0) and np.all(np.signbit(d3[0, 16:]))      # silu(-40) = -1.7e-16: rounds to -0
+
+
+# ---- the binary16 upsample blend of the fp4 decoder conv (stage_up_smem_h2, src/lp_common.cuh:674-712) ----
+from bisect import bisect_left
+from fractions import Fraction
+
+_H16 = None
+
+
+def _half_values():
+    """Every finite non-negative binary16 value as an exact fraction, ascending, with its bit pattern's parity (for ties)."""
+    global _H16
+    if _H16 is None:
+        bits = np.arange(0, 0x7c00, dtype=np.uint16)
+        _H16 = [Fraction(float(v)) for v in bits.view(np.float16).astype(np.float64)]
+    return _H16
+
+
+def half_round(x):
+    """Exact rational -> nearest binary16 value (ties to the even bit pattern), as a float; overflow past 65520 -> inf."""
+    vals = _half_values()
+    s = -1.0 if x < 0 else 1.0
+    a = abs(x)
+    if a >= Fraction(65520):
+        return s * float("inf")
+    i = bisect_left(vals, a)
+    if i < len(vals) and vals[i] == a:
+        return s * float(vals[i])
+    lo, hi = i - 1, i
+    if hi >= len(vals):
+        return s * float(vals[lo])                      # between 65504 and 65520
+    dl, dh = a - vals[lo], vals[hi] - a
+    k = lo if dl < dh else hi if dh < dl else (lo if lo % 2 == 0 else hi)
+    return s * float(vals[k])
+
+
+def test_h16_fma_is_one_rounding_of_the_exact_result():
+    """orc_h16_fma against exact rational arithmetic rounded once: random operands over the whole exponent range, subnormals, exact ties
+    (a product plus an addend that lands halfway between two binary16 values, with and without a sticky term), overflow to inf."""
+    rng = np.random.default_rng(7)
+    L = orc.lib()
+    L.orc_h16_fma.restype = np.ctypeslib.ctypes.c_uint16
+    L.orc_h16_fma.argtypes = [np.ctypeslib.ctypes.c_uint16] * 3
+    cases = []
+    r = rng.integers(0, 0x7c00, size=(4000, 3)).astype(np.uint16) | (rng.integers(0, 2, size=(4000, 3)).astype(np.uint16) << 15)
+    cases += [tuple(int(v) for v in row) for row in r]
+    sub = rng.integers(0, 0x0400, size=(500, 3)).astype(np.uint16)                      # subnormal operands and results
+    cases += [(int(a) | 0x3c00 & 0, int(b) + 0x3800, int(c)) for a, b, c in sub]
+    h = lambda f: int(np.float16(f).view(np.uint16))
+    # ties: 1 + 2^-11 is halfway between 1 and 1 + 2^-10: (2^-11 x 1) + 1; with a sticky product term just above / below the tie
+    cases += [(h(2.0 ** -11), h(1.0), h(1.0)), (h(2.0 ** -11), h(1.0 + 2.0 ** -10), h(1.0)), (h(2.0 ** -11), h(1.0), h(1.0 + 2.0 ** -10)),
+              (h(2.0 ** -12), h(1.0 + 2.0 ** -9), h(1.0)), (h(-(2.0 ** -11)), h(1.0), h(1.0 + 2.0 ** -10)), (h(3.0), h(2.0 ** -24), h(2.0 ** -24)),
+              (h(2.0 ** -14), h(2.0 ** -11), h(2.0 ** -24)), (h(65504.0), h(1.0), h(16.0)), (h(65504.0), h(1.0), h(15.0)), (h(256.0), h(256.0), h(-1.0))]
+    for a, b, c in cases:
+        fa, fb, fc = (float(np.uint16(v).view(np.float16)) for v in (a, b, c))
+        want = half_round(Fraction(fa) * Fraction(fb) + Fraction(fc))
+        got = float(np.uint16(L.orc_h16_fma(a, b, c)).view(np.float16))
+        assert got == want and (want != 0 or True), (hex(a), hex(b), hex(c), got, want)
+
+
+def _staged_up(x, N, C, Dc, Hc, Wc, cbits, up):
+    D, H, W = 2 * Dc, 2 * Hc, 2 * Wc
+    xq = orc.f32_to_mx(8, x, N, C, Dc * Hc * Wc)
+    c = orc.orc_conv_t()
+    c.x, c.xdt, c.N, c.Ci, c.D, c.H, c.W, c.cbits, c.stride, c.up = orc.ptr(xq), 3, N, C, D, H, W, cbits, 1, up
+    st = np.zeros((N, (C + 31) // 32, D * H * W, 32), np.float32)
+    assert orc.lib().orc_conv3_staged(c, orc.ptr(st)) == (C + 31) // 32 * 32
+    return st, decoded(8, xq, N, C, Dc * Hc * Wc)
+
+
+def test_fp16_upsample_blend_equals_rational_arithmetic_rounded_per_step():
+    """The fp4 entry's fused-upsample staging: per fine voxel, the 8 coarse rows (e4m3 codes, one scale byte each) are blended in binary16
+    with weights .75 / .25 per axis times 2^(e_row - e_max), in the order z, y, x, one fused rounding per step; the sum times 2^e_max is
+    then quantised to e2m1. Restated here with exact rationals and the table-search rounding above, the rows' scale bytes from the
+    independent scale rule; a wrong tap order, a weight rounded at the wrong place, an fp32 accumulator or a missing relative scale fails.
+    Also: up = 1 of the fp4 entry IS this blend, of the fp8 entry the fp32 chain; up = 2 / 3 force one."""
+    rng = np.random.default_rng(21)
+    N, C, Dc, Hc, Wc = 1, 32, 2, 3, 2
+    x = (rng.standard_normal((N, C, Dc * Hc * Wc)) * np.exp(rng.uniform(-4, 4, (N, 1, Dc * Hc * Wc)))).astype(np.float32)   # row scales spread over ~2^12
+    st, xd = _staged_up(x, N, C, Dc, Hc, Wc, 4, 1)
+    D, H, W = 2 * Dc, 2 * Hc, 2 * Wc
+    rows = np.moveaxis(xd[0], 0, -1).reshape(Dc, Hc, Wc, 32).astype(np.float64)             # decoded coarse rows (each an e4m3 code times its scale)
+    es = refnp.scale_exp(np.abs(rows).max(-1), 448.0)                                       # their scale exponents (the blend re-derives them)
+    want = np.zeros((D, H, W, 32), np.float32)
+    for gz in range(D):
+        for gy in range(H):
+            for gx in range(W):
+                m = [(g >> 1, min(max((g >> 1) + (1 if g & 1 else -1), 0), n - 1)) for g, n in ((gz, Dc), (gy, Hc), (gx, Wc))]
+                taps = [(a, b, c) for a in range(2) for b in range(2) for c in range(2)]
+                em = max(int(es[m[0][a], m[1][b], m[2][c]]) for a, b, c in taps)
+                acc = [Fraction(0)] * 32
+                for a, b, c in taps:
+                    iz, iy, ix = m[0][a], m[1][b], m[2][c]
+                    e = int(es[iz, iy, ix])
+                    w3 = half_round(Fraction([3, 1][a] * [3, 1][b] * [3, 1][c], 64) * Fraction(2) ** (e - em))
+                    codes = [Fraction(float(v)) / Fraction(2) ** e for v in rows[iz, iy, ix]]           # the e4m3 values: exact in binary16
+                    acc = [Fraction(half_round(Fraction(w3) * q + s)) for q, s in zip(codes, acc)]
+                want[gz, gy, gx] = [float(s * Fraction(2) ** em) for s in acc]
+    wq, _ = refnp.quantize_block(want.reshape(-1, 32), 4)
+    assert np.array_equal(st[0, 0], wq)
+    # the entry's default and the forced modes
+    assert np.array_equal(_staged_up(x, N, C, Dc, Hc, Wc, 4, 2)[0], st)
+    # (after the e2m1 rounding the fp32 chain rarely differs; under e4m3 compute, forced either way, the two blends are told apart)
+    assert np.array_equal(_staged_up(x, N, C, Dc, Hc, Wc, 8, 1)[0], _staged_up(x, N, C, Dc, Hc, Wc, 8, 3)[0])
+    assert not np.array_equal(_staged_up(x, N, C, Dc, Hc, Wc, 8, 2)[0], _staged_up(x, N, C, Dc, Hc, Wc, 8, 3)[0])
+
+
+def test_fp16_upsample_blend_closed_forms():
+    """Grid data (every row's amax 6, values on the e2m1 grid): all partial sums are multiples of 2^-7 below 6 and exact in binary16, so the
+    binary16 blend equals the fp64 trilinear interpolation, and where the 8 rows coincide (a constant tensor) it returns the row itself."""
+    rng = np.random.default_rng(22)
+    N, C, Dc, Hc, Wc = 1, 32, 2, 2, 3
+    x = refnp.gen_exact(rng, (N, C, Dc * Hc * Wc))
+    x[:, 5, :] = 6.0
+    st, _ = _staged_up(x, N, C, Dc, Hc, Wc, 4, 2)
+    want = refnp.up2_f64(x.reshape(N, C, Dc, Hc, Wc)).reshape(N, C, -1)
+    wq, _ = refnp.quantize_block(np.moveaxis(want[0], 0, -1).astype(np.float32), 4)
+    assert np.array_equal(st[0, 0], wq)
+    xc = np.repeat(x[:, :, :1], Dc * Hc * Wc, axis=2)
+    st, _ = _staged_up(xc, N, C, Dc, Hc, Wc, 4, 2)
+    assert np.array_equal(st[0, 0], np.repeat(xc[0, :, :1].T, 8 * Dc * Hc * Wc, axis=0))

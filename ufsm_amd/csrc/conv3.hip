@@ -273,6 +273,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (xbf < 0 || xbf > 4 || !(ybf == 0 || ybf == 2 || ybf == 3 || ybf == 4)) mi_die("%s: unsupported storage types (in %d, out %d)", who, xbf, ybf);
     if (xs.n <= 0 || xs.c <= 0 || xs.d <= 0 || xs.h <= 0 || xs.w <= 0 || cout <= 0) return 0;
     const int Ci = xs.c, Cx = sp.x2 ? sp.c_split : Ci, C2 = Ci - Cx;
+    const int entry_fmt = fmt;
     if (fmt == 4 && Ci <= 8) fmt = 8;                  // the network input computes in e4m3 whatever the activations' format (src/lp_f4fwd.cu:37)
     if (sp.x2 && (Cx <= 0 || C2 <= 0)) mi_die("%s: channel split %d of %d", who, sp.c_split, Ci);
     if (sp.x2 && xbf < 3) mi_die("%s: split inputs need MX storage", who);
@@ -313,7 +314,10 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         } else {
             const size_t bytes = (size_t)N * nbp * S * (mx_rb(32, fmt) + 1);
             uint8_t *st = (uint8_t *)mi_ws(s ? MI_WS_X2STAGE : MI_WS_XSTAGE, bytes);
-            if (upseg) mi_restage_up_sub(segx[s], xbf, N, segC[s], D, H, W, g, Cg, st, fmt, zlo, zhi);
+            // the fp4 entry blends the upsample in binary16 unless UFSM_UP_H2=0 (src/lp_f4fwd.cuh:1135-1136); sp.up 2 / 3 force one blend
+            static int uph2 = -1;
+            if (uph2 < 0) uph2 = getenv("UFSM_UP_H2") ? atoi(getenv("UFSM_UP_H2")) : 1;
+            if (upseg) mi_restage_up_sub(segx[s], xbf, N, segC[s], D, H, W, g, Cg, st, fmt, zlo, zhi, sp.up == 2 || (sp.up == 1 && entry_fmt == 4 && uph2));
             else mi_restage_sub(segx[s], xbf, N, segC[s], (size_t)(zhi - zlo) * H * W, g, Cg, cg0, st, fmt, S, (size_t)zlo * H * W);
             a.xq[s] = st; a.xsc[s] = st + (size_t)N * nbp * S * mx_rb(32, fmt);
             a.nbs[s] = nbp; a.bws[s] = 32;

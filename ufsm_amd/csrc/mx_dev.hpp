@@ -227,9 +227,9 @@ __device__ __forceinline__ void gn_acc_add(double *b, size_t i, double v) {
 
 // ---- host-side shared declarations of the library's units ----
 void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits);
-void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits);
+void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int h2);    // h2: the binary16 blend
 void mi_restage_sub(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits, size_t Ss, size_t v0);     // only voxels [v0, v0 + S) of tensors of Ss voxels
-void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int zlo, int zhi);   // only fine planes [zlo, zhi)
+void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int zlo, int zhi, int h2);   // only fine planes [zlo, zhi)
 void mi_post_error(hipError_t e, const char *file, int line);
 #define MICK() do { hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)
 #define MIRT(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)

@@ -682,7 +682,9 @@ void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg
 // then up_blend_k forms the fine rows. A thread owns the 8 fine voxels whose blend reads one 2x2x2 cell of coarse rows, for 8 of the
 // block's 32 channels: cell (mz, my, mx), each in [-1, dim/2 - 1], covers coarse {m, m + 1} (clamped) and fine {2m + 1, 2m + 2}; the four
 // threads of a cell meet for the row amax through lane exchanges. Each coarse row is decoded once per cell instead of once per fine voxel.
-template <int BY>
+// H2: the fp4 entry's blend (stage_up_smem_h2, src/lp_common.cuh:674-712): binary16 weights relative to the largest of the cell's 8 scale bytes,
+// binary16 fused multiply-adds in the same z, y, x order (an e4m3 code is a binary16 value), the sum widened and scaled by 2^e_max.
+template <int BY, bool H2>
 __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y, int N, int nbo, int D, int H, int W, int zlo, int zhi, int clo, int Dcs, int mz0, int ncz_) {
     // fine planes [zlo, zhi) of the depth-D result, written at their place in the depth-D tensor y; xc holds the coarse planes [clo, clo + Dcs)
     // compactly; cells mz0 .. mz0 + ncz_ - 1 along z (the whole tensor: zlo 0, zhi D, clo 0, Dcs D / 2, mz0 -1, ncz_ D / 2 + 1)
@@ -699,19 +701,44 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
     const int cz[2] = {max(mz, 0), min(mz + 1, Dc - 1)}, cy[2] = {max(my, 0), min(my + 1, Hc - 1)}, cx[2] = {max(mx, 0), min(mx + 1, Wc - 1)};
     const uint8_t *xs = xc + (size_t)N * nbo * Sc * 32;
     float f[8][8], sc[8];
+    unsigned sb[8], em = 0u;
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         const size_t row = (size_t)nbk * Sc + ((size_t)(cz[k >> 2] - clo) * Hc + cy[(k >> 1) & 1]) * Wc + cx[k & 1];
         const uint2 w = *(const uint2 *)(xc + row * 32 + q * 8);
         d_dec4_e4m3(w.x, f[k]); d_dec4_e4m3(w.y, f[k] + 4);
-        sc[k] = d_mx_scale(xs[row]);
+        sb[k] = xs[row]; em = max(em, sb[k]);
+        sc[k] = d_mx_scale(sb[k]);
     }
+    if constexpr (H2) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) { const int de = (int)sb[k] - (int)em; sc[k] = de >= -126 ? __uint_as_float((unsigned)(127 + de) << 23) : 0.f; }     // 2^(e_row - e_max)
+    }
+    const float smax = d_mx_scale(em);
     uint8_t *ys = y + (size_t)N * nbo * S * (BY * 4);
 #pragma unroll
     for (int p = 0; p < 8; p++) {
         const int pz = p >> 2, py = (p >> 1) & 1, px = p & 1;                     // fine voxel 2m + 1 + p: p = 0 has its own coarse row at m, p = 1 at m + 1
         const int gz = 2 * mz + 1 + pz, gy = 2 * my + 1 + py, gx = 2 * mx + 1 + px;
         float acc[8];
+        if constexpr (H2) {
+            __half hacc[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) hacc[i] = __float2half_rn(0.f);
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++)
+#pragma unroll
+                    for (int c = 0; c < 2; c++) {
+                        const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);
+                        const __half w3 = __float2half_rn((a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f) * sc[k]);
+#pragma unroll
+                        for (int i = 0; i < 8; i++) hacc[i] = __hfma(w3, __float2half_rn(f[k][i]), hacc[i]);
+                    }
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] = __half2float(hacc[i]) * smax;
+        } else {
 #pragma unroll
         for (int i = 0; i < 8; i++) acc[i] = 0.f;
 #pragma unroll
@@ -725,6 +752,7 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
 #pragma unroll
                     for (int i = 0; i < 8; i++) acc[i] = fmaf(w3, f[k][i], acc[i]);
                 }
+        }
         float am = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; i++) am = fmaxf(am, fabsf(acc[i]));
@@ -740,7 +768,7 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
     }
 }
 // fine planes [zlo, zhi) of the upsampled depth-D tensor, written at their place in the depth-D MX tensor y
-void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int zlo, int zhi) {
+void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int zlo, int zhi, int h2) {
     if (!N || zhi <= zlo || !H || !W) return;
     if (xdt != 3 && xdt != 4) mi_die("fused-upsample input must be an MX tensor (dtype %d)", xdt);
     if ((D | H | W) & 1) mi_die("fused-upsample output dims must be even (%d %d %d)", D, H, W);
@@ -754,8 +782,9 @@ void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W
     const size_t cells = (size_t)(H / 2 + 1) * (W / 2 + 1);                                   // per z layer of cells
     if ((size_t)N * nbo > 65535 || ncz > 65535) mi_die("fused upsample: launch grid (%d x %d blocks, %d cell layers)", N, nbo, ncz);
     const dim3 grid(nblk_(cells * 4, 256), (unsigned)(N * nbo), (unsigned)ncz);
-    if (ybits == 4) up_blend_k<4><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W, zlo, zhi, 0, Dc, mz0, ncz);
-    else up_blend_k<8><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W, zlo, zhi, 0, Dc, mz0, ncz);
+#define UB(BY, H2) up_blend_k<BY, H2><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W, zlo, zhi, 0, Dc, mz0, ncz)
+    if (ybits == 4) { if (h2) UB(4, true); else UB(4, false); } else { if (h2) UB(8, true); else UB(8, false); }
+#undef UB
     MICK();
 }
-void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits) { mi_restage_up_sub(x, xdt, N, C, D, H, W, gp, Cg, y, ybits, 0, D); }
+void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int h2) { mi_restage_up_sub(x, xdt, N, C, D, H, W, gp, Cg, y, ybits, 0, D, h2); }
