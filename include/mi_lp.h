@@ -133,6 +133,14 @@ void mi_event_destroy(void *ev);
    act 0 none, 1 SiLU, 2 GELU (erf), 3 ReLU. bits 8 / 4 selects the compute format. */
 int mi_conv_fwd_fused(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                       const float *ep_a, const float *ep_b, int act, gnp_t gp, double *osum, int Go, split_t sp);
+/* extensions with no counterpart in the reference (whose down conv is 3x3x3 stride 2, src/lp_s2.cu:4-9, and whose upsample is trilinear,
+   src/lp_mx_gn.cu:32-33): the 2x2x2 stride-2 conv (w [cout][cin][2][2][2], output dims halved: the input's must be even) and the 2x2x2 stride-2
+   transposed conv (w [cin][cout][2][2][2], output dims doubled) with the operand rules of the 3x3x3 entries: x an MX tensor (xbf 3 / 4) with an
+   optional GroupNorm + SiLU (gp), rows re-quantised to the compute format (bits 8 / 4) per voxel and 32 channels unless they are stored in it,
+   weights scaled per (tap, output channel, 32 input channels), fp32 accumulation, bias, y an MX tensor (ybf 3 / 4) or fp32 / fp16 planes (0 / 2).
+   No output statistics. 0 on success, -1 for arguments they do not take. */
+int mi_conv_down2_fwd(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp);
+int mi_convt_up2_fwd(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp);
 /* extension with no counterpart in the reference (which zeroes the sum slots, runs the conv and finalizes in three launches,
    src/nn_bwd.cu:37-56, src/nn_elem.cu:5-17): the stride-1 conv with its output GroupNorm statistics finalized by the conv's own
    reduction. osum (2 N Go slots) need not be cleared: it is set to this conv's sums; omean / orstd (N Go floats) get

@@ -643,6 +643,66 @@ int orc_conv3(const orc_conv_t *c) {
     return 0;
 }
 
+/* ---------- 2x2x2 stride-2 convolutions (no counterpart in the reference, whose down conv is 3x3x3 stride 2 and whose upsample is trilinear:
+   src/lp_s2.cu:4-9, src/lp_mx_gn.cu:32-33): the same operand rules as orc_conv3 applied to the two other stride-2 layers a U-Net can have.
+   Activations: the staged rows of build_staged (stored MX block as is, or GN + SiLU and re-quantisation per voxel and 32 channels); weights:
+   one E8M0 scale per (tap, output channel, 32 input channels) as orc_prep_w; block products summed in fp32 (acc64: fp64) tap-major then
+   block; the epilogue of orc_conv3.
+   down: y[co][oz][oy][ox] = b[co] + sum_{ci, dz, dy, dx} w[co][ci][dz][dy][dx] x[ci][2 oz + dz][2 oy + dy][2 ox + dx]          (w as torch Conv3d)
+   up:   y[co][2 iz + dz][2 iy + dy][2 ix + dx] = b[co] + sum_ci w[ci][co][dz][dy][dx] x[ci][iz][iy][ix]                        (w as torch ConvTranspose3d)
+   Pins: tests/test_oracle_conv2.py (fp64 closed forms on exact operands; down = orc_conv3 at stride 2 with the taps embedded in a 3x3x3 kernel) */
+int orc_conv2(const orc_conv_t *c, int up) {
+    staged_t st;
+    if ((c->cbits != 8 && c->cbits != 4) || c->x2 || c->up || c->xdt < 3) return -2;
+    if (!up && ((c->D | c->H | c->W) & 1)) return -2;
+    orc_conv_t cs = *c; cs.stride = 1;
+    if (build_staged(&cs, &st)) return -1;
+    const int Co = c->Co, Ci = c->Ci, nch = st.nch, Cip = st.Cip;
+    const int Do = up ? 2 * c->D : c->D / 2, Ho = up ? 2 * c->H : c->H / 2, Wo = up ? 2 * c->W : c->W / 2;
+    const size_t So = (size_t)Do * Ho * Wo;
+    float *wv = (float *)malloc((size_t)8 * Co * Cip * sizeof(float)), *wsf = (float *)malloc((size_t)8 * Co * nch * sizeof(float));
+    for (int i = 0; i < 8 * Co * nch; i++) {
+        const int ch = i % nch, co = (i / nch) % Co, t = i / (nch * Co);
+        float v[32]; uint8_t codes[32];
+        for (int k = 0; k < 32; k++) { const int ci = ch * 32 + k; v[k] = ci < Ci ? (up ? c->w[((size_t)ci * Co + co) * 8 + t] : c->w[((size_t)co * Ci + ci) * 8 + t]) : 0.f; }
+        wsf[i] = orc_mx_scale(orc_store_row(c->cbits, v, 32, codes, 0));
+        for (int k = 0; k < 32; k++) wv[(size_t)i * 32 + k] = c->cbits == 8 ? orc_dec_e4m3(codes[k]) : orc_dec_e2m1((codes[k >> 1] >> (4 * (k & 1))) & 15u);
+    }
+    orc_conv_t ce = *c; ce.osum = NULL; ce.Go = 0;
+    for (int n = 0; n < c->N; n++) {
+#pragma omp parallel
+        {
+            float *acc = (float *)malloc((size_t)Co * sizeof(float));
+            double *acc64 = (double *)malloc((size_t)Co * sizeof(double));
+#pragma omp for schedule(dynamic, 64)
+            for (int64_t vi = 0; vi < (int64_t)So; vi++) {
+                const int oz = (int)(vi / ((int64_t)Ho * Wo)), oy = (int)(vi / Wo % Ho), ox = (int)(vi % Wo);
+                for (int co = 0; co < Co; co++) { acc[co] = 0.f; acc64[co] = 0.0; }
+                for (int t = 0; t < 8; t++) {
+                    if (up && t != ((oz & 1) << 2 | (oy & 1) << 1 | (ox & 1))) continue;          /* an output voxel of the transposed conv has one tap */
+                    const int iz = up ? oz >> 1 : 2 * oz + (t >> 2), iy = up ? oy >> 1 : 2 * oy + ((t >> 1) & 1), ix = up ? ox >> 1 : 2 * ox + (t & 1);
+                    const size_t iv = ((size_t)iz * c->H + iy) * c->W + ix;
+                    for (int ch = 0; ch < nch; ch++) {
+                        const float *xv = st.sv + (((size_t)n * nch + ch) * st.S + iv) * 32;
+                        const float xs = st.sf[((size_t)n * nch + ch) * st.S + iv];
+                        for (int co = 0; co < Co; co++) {
+                            const float *wr = wv + (((size_t)t * Co + co) * nch + ch) * 32;
+                            double d = 0.0;
+                            for (int k = 0; k < 32; k++) d += (double)wr[k] * (double)xv[k];
+                            const double blk = d * (double)wsf[((size_t)t * Co + co) * nch + ch] * (double)xs;
+                            if (c->acc64 == 1) acc64[co] += blk; else acc[co] += (float)blk;
+                        }
+                    }
+                }
+                conv_epilogue(&ce, n, (size_t)vi, So, acc, acc64, NULL);
+            }
+            free(acc); free(acc64);
+        }
+    }
+    free(wv); free(wsf); free(st.sv); free(st.sf);
+    return 0;
+}
+
 /* ---------- GroupNorm ---------- */
 void orc_gn_finalize(const double *sums, int NG, size_t len, float eps, float *mean, float *rstd) {   /* src/nn_elem.cu:5-11 */
     for (int i = 0; i < NG; i++) {

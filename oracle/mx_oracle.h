@@ -103,6 +103,9 @@ typedef struct {
 } orc_conv_t;
 /* 3x3x3 forward conv with MX operands (src/lp_f8fwd.cuh:19-151, src/lp_common.cuh:1465-1597, src/lp_s2.cu:4-9) */
 int orc_conv3(const orc_conv_t *c);
+/* 2x2x2 stride-2 conv (up 0: w [Co][Ci][2][2][2], output dims halved) or transposed conv (up 1: w [Ci][Co][2][2][2], output dims doubled) with
+   MX operands: c->x an MX tensor of c->D x c->H x c->W, optional c->gp; stride, x2, up, osum, z0 / z1 and stem_tile of c are not used */
+int orc_conv2(const orc_conv_t *c, int up);
 /* staged (quantised) operand of a conv's input only: values = decoded code * scale per (n, padded channel, voxel) */
 int orc_conv3_staged(const orc_conv_t *c, float *staged);
 

@@ -51,6 +51,7 @@ def lib():
         L.orc_prep_w.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.orc_conv3.restype = C.c_int; L.orc_conv3.argtypes = [C.POINTER(orc_conv_t)]
         L.orc_conv3_staged.restype = C.c_int; L.orc_conv3_staged.argtypes = [C.POINTER(orc_conv_t), C.c_void_p]
+        L.orc_conv2.restype = C.c_int; L.orc_conv2.argtypes = [C.POINTER(orc_conv_t), C.c_int]
         L.orc_gn_finalize.restype = None; L.orc_gn_finalize.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_void_p, C.c_void_p]
         L.orc_gn_sums_mx.restype = None; L.orc_gn_sums_mx.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t]
         L.orc_gn_silu_apply_mx.restype = None; L.orc_gn_silu_apply_mx.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_size_t, orc_gn_t, C.c_void_p, C.c_int]
@@ -131,6 +132,20 @@ def conv3(x, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=8, stride=1, x2=None, c_s
     assert rc == 0, rc
     del keep
     return y, sums
+
+
+def conv2(x, xdt, N, Ci, D, H, W, w, b, Co, ydt, up, cbits=8, gp=None, acc64=0):
+    """The oracle's 2x2x2 stride-2 conv (up 0, w [Co][Ci][8]) or transposed conv (up 1, w [Ci][Co][8]) of an MX tensor; y as conv3."""
+    c = orc_conv_t()
+    c.x, c.xdt, c.N, c.Ci, c.D, c.H, c.W = ptr(x), xdt, N, Ci, D, H, W
+    c.gp = gp if gp is not None else orc_gn_t(); c.gp2 = orc_gn_t()
+    c.w, c.b, c.Co, c.stride, c.cbits, c.acc64 = ptr(w), ptr(b), Co, 1, cbits, acc64
+    So = (8 * D * H * W) if up else (D // 2) * (H // 2) * (W // 2)
+    y = np.zeros(mx_bytes(8 if ydt == 3 else 4, N, Co, So), dtype=np.uint8) if ydt >= 3 else np.zeros((N, Co, So), dtype=np.uint16 if ydt == 2 else np.float32)
+    c.y, c.ydt = ptr(y), ydt
+    rc = lib().orc_conv2(C.byref(c), up)
+    assert rc == 0, rc
+    return y
 
 
 def mx_gemm(bits, ta, tb, M, N, K, A, B, C0=None, beta=0.0, bias=None, res=None):

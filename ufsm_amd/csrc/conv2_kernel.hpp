@@ -1,0 +1,135 @@
+// 2x2x2 stride-2 convolution and transposed convolution with MX operands: the two other stride-2 layers a U-Net can have (the reference has a 3x3x3
+// stride-2 down conv and a trilinear upsample, src/lp_s2.cu:4-9, src/lp_mx_gn.cu:32-33; these follow the same operand rules: rows of 32 channels per
+// voxel with their E8M0 scale, weights scaled per (tap, output channel, 32 input channels), fp32 accumulation, the convs' own epilogue).
+//
+// Neither op has a halo: an input row feeds exactly one output voxel (down) or the eight voxels above it, one per tap (up). So both are GEMMs
+// whose activation operand is read straight from the stored tensor into MFMA fragments, with no LDS and no re-layout: a voxel's row of block b is
+// 32 (e4m3) or 16 (e2m1) contiguous bytes, lanes of a voxel tile read neighbouring rows, and lane (r, h) of a 32x32x64 MFMA takes bytes 16 h .. of
+// both rows of a K pair (e4m3) or the whole row of unit h (e2m1), with unit h's scale byte.
+//   down: column = output voxel, K = (tap, block) tap-major: pair units 2 p, 2 p + 1; the row of unit (t, b) is voxel (2 oz + dz, 2 oy + dy, 2 ox + dx)
+//   up:   column = input voxel; the eight taps are eight GEMMs over K = blocks on the same rows, each followed by an epilogue whose output
+//         voxel is (2 iz + dz, 2 iy + dy, 2 ix + dx)
+// A wavefront owns NT = 2 tiles of 32 consecutive columns (linear voxel index) and MT channel tiles of 32; the weights' fragments come from
+// global memory in the prepared lane order (a few KiB per K pair, shared by every wavefront: cache hits).
+#pragma once
+#include "conv3_kernel.hpp"
+
+template <int FMT, int OUT, bool UP, int MT>
+__global__ void __launch_bounds__(256, 2) conv2_mx_k(const conv_args a) {
+    constexpr int NT = 2, RB = fmt_t<FMT>::RB, WTILE = fmt_t<FMT>::WTILE;
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    const int n = blockIdx.z, cs = blockIdx.y, nb = a.nbs[0];
+    const size_t Sin = (size_t)a.D * a.H * a.W;
+    const long long Scol = UP ? (long long)Sin : (long long)a.Do * a.Ho * a.Wo;
+    conv_epi_consts<MT, false>(a, lds, cs, tid);
+    __syncthreads();
+    const long long ct0 = ((long long)blockIdx.x * 4 + wave) * NT;
+    if (ct0 * 32 >= Scol) return;                            // (no barrier follows)
+    // the lane's column of each tile: its input voxel (down: the voxel of tap (0, 0, 0)) and, for the epilogue, the coordinates
+    size_t iv0[NT]; int c0[NT], c1[NT], c2[NT]; bool cok[NT];
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        const long long col = (ct0 + j) * 32 + r;
+        cok[j] = col < Scol;
+        const long long cc = cok[j] ? col : 0;
+        const int Wc = UP ? a.W : a.Wo, Hc = UP ? a.H : a.Ho;
+        c2[j] = (int)(cc % Wc); c1[j] = (int)(cc / Wc % Hc); c0[j] = (int)(cc / ((long long)Wc * Hc));
+        iv0[j] = UP ? (size_t)cc : ((size_t)(2 * c0[j]) * a.H + 2 * c1[j]) * a.W + 2 * c2[j];
+    }
+    const uint8_t *xq = a.xq[0] + (size_t)n * nb * Sin * RB, *xsc = a.xsc[0] + (size_t)n * nb * Sin;
+    // the activation fragment of tile j for the K pair (block b0 at voxel offset o0 | block b1 at o1; ok1: the second unit exists)
+    struct bfrag { v8i f; int sb; };
+    auto fetch = [&](int j, int b0, size_t o0, int b1, size_t o1, bool ok1) {
+        bfrag q;
+        const size_t v0 = (size_t)b0 * Sin + iv0[j] + o0, v1 = (size_t)b1 * Sin + iv0[j] + o1;
+        if constexpr (FMT == 8) {
+            const v4i lo = *(const v4i *)(xq + v0 * RB + 16 * h);
+            v4i hi = {0, 0, 0, 0};
+            if (ok1) hi = *(const v4i *)(xq + v1 * RB + 16 * h);
+            q.f = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        } else {
+            v4i lo = {0, 0, 0, 0};
+            if (!h || ok1) lo = *(const v4i *)(xq + (h ? v1 : v0) * RB);
+            q.f = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+        }
+        q.sb = h ? (ok1 ? (int)xsc[v1] : 127) : (int)xsc[v0];
+        return q;
+    };
+    struct afrag { v8i f; int s; };
+    auto wfetch = [&](int gp, int m) {
+        afrag q;
+        const size_t t = (size_t)gp * a.nmt_all + cs * MT + m;
+        const v4i lo = *(const v4i *)(a.wq + t * WTILE + lane * 16);
+        if constexpr (FMT == 8) { const v4i hi = *(const v4i *)(a.wq + t * WTILE + 1024 + lane * 16); q.f = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; }
+        else q.f = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+        q.s = *(const int *)(a.wsc + (t * 64 + lane) * 4);
+        return q;
+    };
+    v16f acc[MT][NT];
+    auto clear = [&]() {
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
+    };
+    auto step = [&](int gp, const bfrag (&fb)[NT]) {
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+            const afrag fa = wfetch(gp, m);
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa.f, fb[j].f, acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, fa.s, 0, fb[j].sb);
+        }
+    };
+    long long ovx[NT];
+    if constexpr (!UP) {
+        clear();
+        const int np = 4 * nb;                               // 8 taps x nb blocks, in pairs
+        for (int p = 0; p < np; p++) {
+            const int u0 = 2 * p, u1 = u0 + 1, t0 = u0 / nb, b0 = u0 - t0 * nb, t1 = u1 / nb, b1 = u1 - t1 * nb;
+            const size_t o0 = ((size_t)(t0 >> 2) * a.H + ((t0 >> 1) & 1)) * a.W + (t0 & 1), o1 = ((size_t)(t1 >> 2) * a.H + ((t1 >> 1) & 1)) * a.W + (t1 & 1);
+            bfrag fb[NT];
+#pragma unroll
+            for (int j = 0; j < NT; j++) fb[j] = fetch(j, b0, o0, b1, o1, true);
+            step(p, fb);
+        }
+#pragma unroll
+        for (int j = 0; j < NT; j++) ovx[j] = cok[j] ? (ct0 + j) * 32 + r : -1;
+        conv_epilogue<MT, NT, OUT, false, false, false, false, true, 4, true>(a, acc, lds, 0u, n, cs, 0, 0, 0, 0, 0, tid, ovx);
+    } else {
+        const int npt = (nb + 1) >> 1;
+        for (int t = 0; t < 8; t++) {
+            clear();
+            for (int pp = 0; pp < npt; pp++) {
+                bfrag fb[NT];
+#pragma unroll
+                for (int j = 0; j < NT; j++) fb[j] = fetch(j, 2 * pp, 0, 2 * pp + 1 < nb ? 2 * pp + 1 : 2 * pp, 0, 2 * pp + 1 < nb);
+                step(t * npt + pp, fb);
+            }
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+                ovx[j] = cok[j] ? ((long long)(2 * c0[j] + (t >> 2)) * a.Ho + 2 * c1[j] + ((t >> 1) & 1)) * a.Wo + 2 * c2[j] + (t & 1) : -1;
+            conv_epilogue<MT, NT, OUT, false, false, false, false, true, 4, true>(a, acc, lds, 0u, n, cs, 0, 0, 0, 0, 0, tid, ovx);
+        }
+    }
+}
+
+template <int FMT, int OUT, bool UP, int MT>
+static void launch_conv2_mt(const conv_args &a, dim3 grid, size_t smem) {
+    conv2_mx_k<FMT, OUT, UP, MT><<<grid, 256, smem>>>(a);
+    MICK();
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv2_mx_k<fmt %d, out %d, up %d, MT %d> blocks %d grid %u x %u x %u", FMT, OUT, (int)UP, MT, a.nbs[0], grid.x, grid.y, grid.z);
+}
+template <int FMT>
+static void launch_conv2(int out, int up, int MT, const conv_args &a, dim3 grid, size_t smem) {
+#define C2_MT(OUT, UP) do { if (MT == 4) launch_conv2_mt<FMT, OUT, UP, 4>(a, grid, smem); else if (MT == 2) launch_conv2_mt<FMT, OUT, UP, 2>(a, grid, smem); else launch_conv2_mt<FMT, OUT, UP, 1>(a, grid, smem); } while (0)
+#define C2_UP(OUT) do { if (up) C2_MT(OUT, true); else C2_MT(OUT, false); } while (0)
+    if (out == 8) C2_UP(8); else if (out == 4) C2_UP(4); else C2_UP(0);
+#undef C2_UP
+#undef C2_MT
+}
+void conv2_launch_f8(int out, int up, int MT, const conv_args &a, dim3 grid, size_t smem);
+void conv2_launch_f4(int out, int up, int MT, const conv_args &a, dim3 grid, size_t smem);

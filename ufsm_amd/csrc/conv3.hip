@@ -91,7 +91,7 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
 #pragma unroll
     for (int side = 0; side < 2; side++) {
         const int u = 2 * q + side;
-        float v[32]; float amax = 0.f;
+        float v[32];
         // K order inside a chunk: tap by tap over its blocks, or (the wide kernel, one chunk) block by block over the taps; the row kernel
         // (block_major < 0): per block 15 pairs (class c, ky), class c < 3 = taps (c, ky, 0 | 1), class 3 = (0 | 1, ky, 2), class 4 = (2, ky, 2 | none)
         int t = block_major ? u % 27 : u / nbc, blk = block_major ? u / 27 : b0 + u % nbc;
@@ -107,23 +107,8 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
         for (int k = 0; k < 32; k++) {
             const int ci = seg_ci(blk * 32 + k, Ci, Cx, CxP);
             v[k] = (unit_ok && cop < Co && ci >= 0) ? w[((size_t)cop * Ci + ci) * 27 + t] : 0.f;
-            amax = fmaxf(amax, fabsf(v[k]));
         }
-        const int e = d_mx_exp(amax, FMT == 8 ? MI_INVQ8 : MI_INVQ4);
-        const float mult = d_exp2i(-e);
-        if (FMT == 8) {
-            unsigned c[8];
-#pragma unroll
-            for (int j = 0; j < 8; j++) c[j] = d_enc_e4m3x4(v[4 * j] * mult, v[4 * j + 1] * mult, v[4 * j + 2] * mult, v[4 * j + 3] * mult);
-            *(uint4 *)(tile + ((size_t)(side * 64 + r) * 16)) = make_uint4(c[0], c[1], c[2], c[3]);            // lane (r, 0): bytes 0-15
-            *(uint4 *)(tile + ((size_t)(side * 64 + r + 32) * 16)) = make_uint4(c[4], c[5], c[6], c[7]);       // lane (r, 1): bytes 16-31
-        } else {
-            unsigned c[4];
-#pragma unroll
-            for (int j = 0; j < 4; j++) c[j] = d_enc_e2m1x8(v + 8 * j, mult);
-            *(uint4 *)(tile + ((size_t)(r + 32 * side) * 16)) = make_uint4(c[0], c[1], c[2], c[3]);            // lane (r, side): the unit's 32 nibbles
-        }
-        tsc[(r + 32 * side) * tss] = (unsigned)(e + 127);
+        prep_store_unit<FMT>(tile, tsc, tss, side, r, v);
     }
 }
 

@@ -242,7 +242,7 @@ __device__ __forceinline__ void conv_epi_consts(const conv_args &a, unsigned cha
 // holds voxel (oz0 + lz, oy0 + ly0 + j, ox0 + r) of a 32-voxel run along x
 template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false, bool NOCH = false, int NW = 4, bool ROW = false>
 __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT][NT], unsigned char *lds, unsigned tile, int n, int cs,
-                                              int oz0, int oy0, int ox0, int lz, int ly0, int tid) {
+                                              int oz0, int oy0, int ox0, int lz, int ly0, int tid, const long long *ovx = nullptr) {
     const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
     // accumulator layout of the 32x32 MFMA: lane (r = voxel within the tile, h), register i -> channel (i & 3) + 4 h + 8 (i >> 2)
     const size_t So = (size_t)(a.yD ? a.yD : a.Do) * a.Ho * a.Wo;      // voxels per channel plane of the output tensor
@@ -281,9 +281,10 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
         static_for<NT>([&](auto J) {
             constexpr int j = J;
             const int oz = oz0 + lz, oy = ROW ? oy0 + ly0 + j : oy0 + ly0 + 2 * j + (r >> 4), ox = ROW ? ox0 + r : ox0 + (r & 15);
-            const bool ok = FULL || (oz < a.Do && oy < a.Ho && ox < a.Wo);
-            const size_t ov = ((size_t)(oz + a.yzo) * a.Ho + oy) * a.Wo + ox;
-            const bool zst = FULL || (ok && oz >= a.zs0 && oz < a.zs1);
+            // ovx: the caller's own voxel mapping (the 2x2x2 stride-2 kernels): the lane's output voxel of tile j, negative = none
+            const bool ok = ovx ? ovx[j] >= 0 : (FULL || (oz < a.Do && oy < a.Ho && ox < a.Wo));
+            const size_t ov = ovx ? (size_t)ovx[j] : ((size_t)(oz + a.yzo) * a.Ho + oy) * a.Wo + ox;
+            const bool zst = ovx ? ok : (FULL || (ok && oz >= a.zs0 && oz < a.zs1));
             float v[16];
             float am = 0.f;
 #pragma unroll
@@ -429,6 +430,30 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
         }
     }
     DBG_MARK(22);
+}
+
+// one unit (32 input channels of one tap and output channel) of a prepared weight tile: E8M0 scale from the amax, codes, the lane order the MFMA
+// reads (e4m3: lane (r, h) holds bytes 16 h .. of both units of the pair; e2m1: lane (r, side) holds unit side), scale word per lane
+template <int FMT>
+__device__ __forceinline__ void prep_store_unit(uint8_t *tile, unsigned *tsc, int tss, int side, int r, const float *v) {
+    float amax = 0.f;
+#pragma unroll
+    for (int k = 0; k < 32; k++) amax = fmaxf(amax, fabsf(v[k]));
+    const int e = d_mx_exp(amax, FMT == 8 ? MI_INVQ8 : MI_INVQ4);
+    const float mult = d_exp2i(-e);
+    if (FMT == 8) {
+        unsigned c[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) c[j] = d_enc_e4m3x4(v[4 * j] * mult, v[4 * j + 1] * mult, v[4 * j + 2] * mult, v[4 * j + 3] * mult);
+        *(uint4 *)(tile + ((size_t)(side * 64 + r) * 16)) = make_uint4(c[0], c[1], c[2], c[3]);            // lane (r, 0): bytes 0-15
+        *(uint4 *)(tile + ((size_t)(side * 64 + r + 32) * 16)) = make_uint4(c[4], c[5], c[6], c[7]);       // lane (r, 1): bytes 16-31
+    } else {
+        unsigned c[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) c[j] = d_enc_e2m1x8(v + 8 * j, mult);
+        *(uint4 *)(tile + ((size_t)(r + 32 * side) * 16)) = make_uint4(c[0], c[1], c[2], c[3]);            // lane (r, side): the unit's 32 nibbles
+    }
+    tsc[(r + 32 * side) * tss] = (unsigned)(e + 127);
 }
 
 // FMT: compute format (8 e4m3, 4 e2m1); OUT: 8 / 4 = MX-fp8 / MX-fp4 rows, 0 = fp32 or fp16 planes; EPI: fused affine + activation

@@ -92,6 +92,8 @@ _PROTOS = {
     "mi_event_elapsed_ms": (_F, [_P, _P]),
     "mi_event_destroy": (None, [_P]),
     "mi_conv_fwd_fused": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, _P, _P, _I, gnp_t, _P, _I, split_t]),
+    "mi_conv_down2_fwd": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t]),
+    "mi_convt_up2_fwd": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t]),
     "mi_conv_fwd_gn": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t, C.c_float, _P, _P]),
     "mi_conv_fwd_static": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t]),
     "mi_conv_static_scratch_bytes": (_Z, []),
