@@ -56,6 +56,13 @@ int lp_conv_fwd_s2_f8(const void *x, int xbf, shape5 xs, const float *w, const f
 /* prepared-weight memo (src/nn_lp.h:56-57): a conv called with sp.wkey != 0 reuses its quantised weights until the next step / clear */
 void lp_wmemo_step(unsigned step);
 void lp_wmemo_clear(void);
+/* 2-D fp4 weight scales (src/nn_lp.h:58, src/lp_f4fwd.cu:67-83): the stride-1 e2m1 weight preps of more than 16 input channels take one E8M0
+   scale per tap and 32 x 32 (output x input channel) tile; a change drops the prepared weights. Default from UFSM_W4_2D (0). */
+void lp_set_w4_2d(int on);
+/* w [Co][Ci][T] rounded in place to MX-fp4 values, one scale per Bo x Bi block and tap (src/nn_lp.h:124, src/lp_mx_cvt.cu:369-395);
+   nn_fakeq_w4_2d (src/nn.h:774): B x B blocks */
+void lp_fakeq_w4(float *w, int Co, int Ci, int T, int Bo, int Bi);
+void nn_fakeq_w4_2d(float *w, int Co, int Ci, int T, int B);
 /* no counterpart in the reference (its stride-2 entry carries no split_t and prepares the weights per call): memo id of the calling thread's
    next lp_conv_fwd_s2_f8, as split_t.wkey for the stride-1 entries; consumed by that call. For inference loops with constant weights. */
 void mi_conv_s2_wkey(unsigned wkey);

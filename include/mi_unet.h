@@ -92,6 +92,10 @@ void unet_init(unet *u, uint64_t seed);                        /* Kaiming normal
 float *unet_param_ptr(unet *u);                                /* device pointers of the flat fp32 weights and of their EMA copy (src/unet.h:203-204), unet_init's order */
 float *unet_ema_ptr(unet *u);
 void unet_use_ema(unet *u, int on);                            /* forward with the EMA weights (1) or the live ones (0) (src/unet.h:258) */
+/* no counterpart in the reference, which re-forms the forward copy of a cfg.w4_2d net's weights before every forward (src/unet.c:5310-5326): here
+   the copy (fp4 convs' weights rounded per 32 x 32 block and tap) is re-formed after unet_load / mi_unet_set_params / unet_use_ema; a caller that
+   writes the weights through unet_param_ptr / unet_ema_ptr says so with this call (it also drops the prepared-weight memo) */
+void mi_unet_weights_changed(unet *u);
 /* activation storage of the networks built from now on (src/unet.h:369-370): MX-fp8 (the default here; this build has no 16-bit storage, so
    unet_set_act_mx8(0) without mx4 is refused at the next forward) or packed MX-fp4, which takes precedence. The compute precision follows the
    op layer's policy (nn_set_prec(3): MX-fp4 weights over either storage). A change rebuilds the activations at the next forward. */

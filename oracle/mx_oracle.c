@@ -253,21 +253,44 @@ void orc_pred_input_mx(int bits, const uint8_t *ct, int W, float mean, float isd
 /* ---------- weights (src/lp_f8fwd.cu:54-71; src/lp_f4fwd.cu:53-66): one block = the 32 ci of one (tap, co) ----------
    padded input channel cp -> real channel (src/lp_common.cuh:235): MX inputs pad each of the two segments to 32 */
 static int seg_ci(int cp, int Ci, int Cx, int CxP) { if (cp < CxP) return cp < Cx ? cp : -1; const int c = Cx + cp - CxP; return c < Ci ? c : -1; }
-void orc_prep_w(int bits, const float *w, int Co, int Ci, int Cx, int CxP, int Cip, float *wv, uint8_t *ws, uint8_t *wcodes) {
+/* 2-D fp4 weight scales (src/lp_f4fwd.cu:67-83, lp_set_w4_2d): the e2m1 prep takes the amax, and so the scale, over the 32 x 32 tile of 32
+   output channels (co / 32; rows past Co are zeros) and the 32 input channels of the block, instead of per output channel */
+static int g_w4_2d = 0;
+void orc_set_w4_2d(int on) { g_w4_2d = on; }
+static uint8_t store_row_amax(int bits, const float *v, float amax, uint8_t *codes) {
+    const int e = orc_mx_exp(amax, bits == 8 ? INVQ8 : INVQ4);
+    enc_codes(bits, v, 32, orc_exp2i(-e), codes);
+    return (uint8_t)(e + 127);
+}
+static void prep_w(int bits, const float *w, int Co, int Ci, int Cx, int CxP, int Cip, float *wv, uint8_t *ws, uint8_t *wcodes, int w2d_on) {
     const int nch = Cip / 32;
+    const int w2d = w2d_on && bits == 4 && Ci > 16;
 #pragma omp parallel for schedule(static)
     for (int i = 0; i < 27 * Co * nch; i++) {
         const int ch = i % nch, co = (i / nch) % Co, t = i / (nch * Co);
         float v[32]; uint8_t codes[32];
         for (int k = 0; k < 32; k++) { const int ci = seg_ci(ch * 32 + k, Ci, Cx, CxP); v[k] = ci >= 0 ? w[((size_t)co * Ci + ci) * 27 + t] : 0.f; }
-        const uint8_t sb = orc_store_row(bits, v, 32, codes, 0);
+        float am2 = 0.f;
+        if (w2d) for (int c2 = co / 32 * 32; c2 < co / 32 * 32 + 32 && c2 < Co; c2++) for (int k = 0; k < 32; k++) { const int ci = seg_ci(ch * 32 + k, Ci, Cx, CxP); if (ci >= 0) am2 = fmaxf(am2, fabsf(w[((size_t)c2 * Ci + ci) * 27 + t])); }
+        const uint8_t sb = w2d ? store_row_amax(bits, v, am2, codes) : orc_store_row(bits, v, 32, codes, 0);
         ws[i] = sb;
         if (wcodes) memcpy(wcodes + (size_t)i * rowbytes(32, bits), codes, rowbytes(32, bits));
         float *dst = wv + ((size_t)t * Co + co) * Cip + ch * 32;
         for (int k = 0; k < 32; k++) dst[k] = bits == 8 ? orc_dec_e4m3(codes[k]) : orc_dec_e2m1((codes[k >> 1] >> (4 * (k & 1))) & 15u);
     }
 }
+void orc_prep_w(int bits, const float *w, int Co, int Ci, int Cx, int CxP, int Cip, float *wv, uint8_t *ws, uint8_t *wcodes) { prep_w(bits, w, Co, Ci, Cx, CxP, Cip, wv, ws, wcodes, g_w4_2d); }
 
+/* w [Co][Ci][T] rounded in place to MX-fp4 values with one scale per Bo x Bi block and tap (src/lp_mx_cvt.cu:369-395) */
+void orc_fakeq_w4(float *w, int Co, int Ci, int T, int Bo, int Bi) {
+    for (int o0 = 0; o0 < Co; o0 += Bo) for (int i0 = 0; i0 < Ci; i0 += Bi) for (int t = 0; t < T; t++) {
+        const int no = Co - o0 < Bo ? Co - o0 : Bo, ni = Ci - i0 < Bi ? Ci - i0 : Bi;
+        float amax = 0.f;
+        for (int o = 0; o < no; o++) for (int i = 0; i < ni; i++) amax = fmaxf(amax, fabsf(w[((size_t)(o0 + o) * Ci + i0 + i) * T + t]));
+        const int e = orc_mx_exp(amax, INVQ4); const float m = orc_exp2i(-e), sc = orc_exp2i(e);
+        for (int o = 0; o < no; o++) for (int i = 0; i < ni; i++) { float *p = w + ((size_t)(o0 + o) * Ci + i0 + i) * T + t; *p = orc_dec_e2m1(orc_enc_e2m1(*p * m)) * sc; }
+    }
+}
 /* a third summation order for drift studies (acc64 == 2): fp32 accumulation whose every add is rounded toward zero, as a datapath that
    aligns and truncates its addends does. A legitimate fp32-accumulated result, within one ulp per add of the other two. */
 static float add_chop(float acc, double blk) {
@@ -585,7 +608,7 @@ int orc_conv3(const orc_conv_t *c) {
     const size_t So = (size_t)Do * Ho * Wo;
     float *wv = (float *)malloc((size_t)27 * Co * Cip * sizeof(float));
     uint8_t *ws = (uint8_t *)malloc((size_t)27 * Co * nch);
-    orc_prep_w(c->cbits, c->w, Co, c->Ci, c->xdt >= 3 ? st.Cx : c->Ci, c->xdt >= 3 ? st.CxP : (c->Ci + 31) / 32 * 32, Cip, wv, ws, NULL);
+    prep_w(c->cbits, c->w, Co, c->Ci, c->xdt >= 3 ? st.Cx : c->Ci, c->xdt >= 3 ? st.CxP : (c->Ci + 31) / 32 * 32, Cip, wv, ws, NULL, g_w4_2d && s == 1);   /* (2-D scales: the stride-1 preps only, src/lp_f4fwd.cuh:1163) */
     float *wsf = (float *)malloc((size_t)27 * Co * nch * sizeof(float));
     for (size_t i = 0; i < (size_t)27 * Co * nch; i++) wsf[i] = orc_mx_scale(ws[i]);
     const int z0 = c->z1 ? c->z0 : 0, z1 = c->z1 ? c->z1 : Do;

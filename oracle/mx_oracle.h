@@ -106,6 +106,9 @@ int orc_conv3(const orc_conv_t *c);
 /* 2x2x2 stride-2 conv (up 0: w [Co][Ci][2][2][2], output dims halved) or transposed conv (up 1: w [Ci][Co][2][2][2], output dims doubled) with
    MX operands: c->x an MX tensor of c->D x c->H x c->W, optional c->gp; stride, x2, up, osum, z0 / z1 and stem_tile of c are not used */
 int orc_conv2(const orc_conv_t *c, int up);
+/* 2-D fp4 weight scales of the stride-1 e2m1 preps (lp_set_w4_2d, src/lp_f4fwd.cu:67-83) and the in-place fake quantisation (src/lp_mx_cvt.cu:369-395) */
+void orc_set_w4_2d(int on);
+void orc_fakeq_w4(float *w, int Co, int Ci, int T, int Bo, int Bi);
 /* staged (quantised) operand of a conv's input only: values = decoded code * scale per (n, padded channel, voxel) */
 int orc_conv3_staged(const orc_conv_t *c, float *staged);
 

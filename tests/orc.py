@@ -51,6 +51,8 @@ def lib():
         L.orc_prep_w.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.orc_conv3.restype = C.c_int; L.orc_conv3.argtypes = [C.POINTER(orc_conv_t)]
         L.orc_conv3_staged.restype = C.c_int; L.orc_conv3_staged.argtypes = [C.POINTER(orc_conv_t), C.c_void_p]
+        L.orc_set_w4_2d.restype = None; L.orc_set_w4_2d.argtypes = [C.c_int]
+        L.orc_fakeq_w4.restype = None; L.orc_fakeq_w4.argtypes = [C.c_void_p] + [C.c_int] * 5
         L.orc_conv2.restype = C.c_int; L.orc_conv2.argtypes = [C.POINTER(orc_conv_t), C.c_int]
         L.orc_gn_finalize.restype = None; L.orc_gn_finalize.argtypes = [C.c_void_p, C.c_int, C.c_size_t, C.c_float, C.c_void_p, C.c_void_p]
         L.orc_gn_sums_mx.restype = None; L.orc_gn_sums_mx.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t]

@@ -43,6 +43,12 @@ def test_refuses_architectures_it_does_not_run(tmp_path, feature):
     assert read(tmp_path, h)[0] == -2
 
 
+def test_reads_the_2d_weight_scale_key(tmp_path):
+    h = 'UFSM{"nlev":2,"widths":[32,64],"w4_2d":1,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":3,"extra":{}}\n'
+    rc, cfg, n, step = read(tmp_path, h)
+    assert rc == 0 and cfg.w4_2d == 1 and step == 3
+
+
 def test_rejects_foreign_files(tmp_path):
     assert read(tmp_path, "not a checkpoint\n")[0] == -1
     assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"scale_cond":1,"nparams":1}\n')[0] == -2      # voxel-size conditioning

@@ -69,7 +69,7 @@ __global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, i
 __host__ __device__ __forceinline__ int seg_ci(int cp, int Ci, int Cx, int CxP) { if (cp < CxP) return cp < Cx ? cp : -1; const int c = Cx + cp - CxP; return c < Ci ? c : -1; }
 template <int FMT>
 __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uint8_t *__restrict__ wq, unsigned *__restrict__ wsc, int Co, int Ci, int Cx, int CxP,
-                                               int nbt, int CB, int nmt_all, int npairs_all, int block_major) {
+                                               int nbt, int CB, int nmt_all, int npairs_all, int block_major, int w2d) {
     constexpr int WTILE = fmt_t<FMT>::WTILE;
     const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     const int Cop = nmt_all * 32;
@@ -108,7 +108,7 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
             const int ci = seg_ci(blk * 32 + k, Ci, Cx, CxP);
             v[k] = (unit_ok && cop < Co && ci >= 0) ? w[((size_t)cop * Ci + ci) * 27 + t] : 0.f;
         }
-        prep_store_unit<FMT>(tile, tsc, tss, side, r, v);
+        prep_store_unit<FMT>(tile, tsc, tss, side, r, v, w2d != 0);      // (32 consecutive threads hold a channel tile's rows of this pair)
     }
 }
 
@@ -127,6 +127,11 @@ extern "C" void lp_wmemo_clear(void) {
     for (auto &m : g_wmemo) { MIRT(hipFree(m.wq)); MIRT(hipFree(m.wsc)); }
     g_wmemo.clear();
 }
+// 2-D fp4 weight scales (src/lp_f4fwd.cu:4, :67-83): one E8M0 scale per tap and 32 x 32 (output x input channel) tile instead of per output
+// channel; a setting change drops the prepared weights. Default from UFSM_W4_2D, as the reference
+static int g_w2d = -1;
+static int g_w2d_on(void) { if (g_w2d < 0) g_w2d = getenv("UFSM_W4_2D") ? atoi(getenv("UFSM_W4_2D")) : 0; return g_w2d; }
+extern "C" void lp_set_w4_2d(int on) { g_w2d = on ? 1 : 0; lp_wmemo_clear(); }
 extern "C" void lp_wmemo_step(unsigned step) { if (step != g_wstep) { g_wstep = step; lp_wmemo_clear(); } }
 
 thread_local char g_last_kernel[128] = "";
@@ -435,8 +440,10 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) {
         const size_t nt = (size_t)npairs_all * nmt_all * 32;
-        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : 0);
-        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : 0);
+        // 2-D fp4 weight scales (lp_set_w4_2d): the stride-1 e2m1 preps of more than 16 input channels, as src/lp_f4fwd.cuh:1163
+        const int w2d = g_w2d_on() && fmt == 4 && stride == 1 && Ci > 16;
+        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : 0, 0);
+        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : 0, w2d);
         MICK();
     }
     a.wq = wq; a.wsc = wsc;

@@ -434,11 +434,16 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
 
 // one unit (32 input channels of one tap and output channel) of a prepared weight tile: E8M0 scale from the amax, codes, the lane order the MFMA
 // reads (e4m3: lane (r, h) holds bytes 16 h .. of both units of the pair; e2m1: lane (r, side) holds unit side), scale word per lane
+// tile2d: one scale for the 32 x 32 (output x input channel) tile, the maximum over the 32 lanes that hold the tile's rows (2-D weight scales)
 template <int FMT>
-__device__ __forceinline__ void prep_store_unit(uint8_t *tile, unsigned *tsc, int tss, int side, int r, const float *v) {
+__device__ __forceinline__ void prep_store_unit(uint8_t *tile, unsigned *tsc, int tss, int side, int r, const float *v, bool tile2d = false) {
     float amax = 0.f;
 #pragma unroll
     for (int k = 0; k < 32; k++) amax = fmaxf(amax, fabsf(v[k]));
+    if (tile2d) {
+#pragma unroll
+        for (int o = 16; o; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    }
     const int e = d_mx_exp(amax, FMT == 8 ? MI_INVQ8 : MI_INVQ4);
     const float mult = d_exp2i(-e);
     if (FMT == 8) {

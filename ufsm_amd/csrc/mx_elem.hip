@@ -788,3 +788,30 @@ void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W
     MICK();
 }
 void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int h2) { mi_restage_up_sub(x, xdt, N, C, D, H, W, gp, Cg, y, ybits, 0, D, h2); }
+
+// weights w [Co][Ci][T] rounded in place to MX-fp4 values with one E8M0 scale per Bo x Bi (output x input channel) block and tap (src/lp_mx_cvt.cu:369-395):
+// the forward's per-output-channel blocks of 32 inputs inside a 32 x 32 block then re-quantise these values exactly. One wavefront per (tap, block).
+__global__ void __launch_bounds__(256) fakeq_w4_k(float *w, int Co, int Ci, int T, int Bo, int Bi) {
+    const int nbo = (Co + Bo - 1) / Bo, nbi = (Ci + Bi - 1) / Bi, lane = threadIdx.x & 63;
+    const size_t wid = (blockIdx.x * (size_t)blockDim.x + threadIdx.x) >> 6;
+    if (wid >= (size_t)T * nbo * nbi) return;                 // (uniform per wavefront)
+    const int t = (int)(wid % T), bi = (int)((wid / T) % nbi), bo = (int)(wid / ((size_t)T * nbi));
+    const int o0 = bo * Bo, i0 = bi * Bi, no = min(Bo, Co - o0), ni = min(Bi, Ci - i0);
+    float amax = 0.f;
+    for (int e = lane; e < no * ni; e += 64) amax = fmaxf(amax, fabsf(w[((size_t)(o0 + e / ni) * Ci + i0 + e % ni) * T + t]));
+#pragma unroll
+    for (int o = 32; o; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+    const int ex = d_mx_exp(amax, MI_INVQ4);
+    const float m = d_exp2i(-ex), sc = d_exp2i(ex);
+    for (int e = lane; e < no * ni; e += 64) {
+        float *p = w + ((size_t)(o0 + e / ni) * Ci + i0 + e % ni) * T + t;
+        *p = d_dec_e2m1(d_enc_e2m1(*p * m)) * sc;
+    }
+}
+extern "C" void lp_fakeq_w4(float *w, int Co, int Ci, int T, int Bo, int Bi) {
+    if (Co <= 0 || Ci <= 0 || T <= 0 || Bo <= 0 || Bi <= 0) return;
+    const size_t nw = (size_t)T * ((Co + Bo - 1) / Bo) * ((Ci + Bi - 1) / Bi);
+    fakeq_w4_k<<<nblk_(nw * 64, 256), 256>>>(w, Co, Ci, T, Bo, Bi);
+    MICK();
+}
+extern "C" void nn_fakeq_w4_2d(float *w, int Co, int Ci, int T, int B) { lp_fakeq_w4(w, Co, Ci, T, B, B); }      // src/nn_elem.cu:192

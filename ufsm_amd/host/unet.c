@@ -29,6 +29,7 @@ struct unet {
     void *skipst[UNET_MAXLEV];         /* silu(gn(enc[i].a2)) in the compute format, formed once for its two readers (down conv, decoder conv1); null: each reader transforms it */
     gnpar dn[UNET_MAXLEV]; float *dm[UNET_MAXLEV], *dr[UNET_MAXLEV];   /* down_norm: GroupNorm after down[i], its statistics */
     size_t np; float *p, *ema, *params;                            /* device: live weights, EMA copy, the one the forward reads */
+    float *src, *wm; int wm_ok;                                    /* cfg.w4_2d: the selected weights (p or ema), their forward copy with the fp4 convs' weights rounded per 32 x 32 block, whether it is current */
     void *xin;                                                     /* the network input as an MX tensor */
     float *logits;                                                 /* [n][cout][S], owned by the net */
     struct { const void *p; shape5 s; const char *name; const float *mean, *rstd; int G; } outs[64]; int nouts;
@@ -63,7 +64,6 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     }
     if (c->ds_levels) return "ds_levels";
     if (c->lat_guide || c->lat_nsub) return "lat_guide";
-    if (c->w4_2d) return "w4_2d";
     if (c->l0_norm || c->l0_slab) return "l0_norm";
     if (c->gfilm) return "gfilm";
     if (c->gn_ema) return "gn_ema";
@@ -119,7 +119,8 @@ unet *unet_create(const unet_cfg *cfg) {
         u->tbn = cfg->attn_blocks;
     }
     u->np = off;
-    u->p = f32_new(off); u->ema = f32_new(off); u->params = u->p;
+    u->p = f32_new(off); u->ema = f32_new(off); u->params = u->src = u->p;
+    if (cfg->w4_2d) { u->wm = f32_new(off); u->params = u->wm; }
     return u;
 }
 /* the activation buffers of the current build */
@@ -187,7 +188,7 @@ void unet_free(unet *u) {
     if (!u) return;
     mi_sync();
     free_acts(u);
-    mi_free(u->p); mi_free(u->ema);
+    mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm);
     lp_wmemo_clear();
     free(u);
 }
@@ -195,9 +196,31 @@ size_t unet_nparams(const unet *u) { return u->np; }
 const unet_cfg *unet_cfg_of(const unet *u) { return &u->cfg; }
 float *unet_param_ptr(unet *u) { return u->p; }
 float *unet_ema_ptr(unet *u) { return u->ema; }
-void unet_use_ema(unet *u, int on) { float *w = on ? u->ema : u->p; if (w != u->params) { u->params = w; lp_wmemo_clear(); } }      /* (the prepared weights are keyed by pointer; dropped all the same) */
+void unet_use_ema(unet *u, int on) {      /* (the prepared weights are keyed by pointer; dropped all the same) */
+    float *w = on ? u->ema : u->p;
+    if (w == u->src) return;
+    u->src = w;
+    if (u->wm) u->wm_ok = 0; else u->params = w;
+    lp_wmemo_clear();
+}
+/* cfg.w4_2d (src/unet.h:47-51, src/unet.c:5292-5326): the forward reads a copy of the selected weights in which the stride-1 3^3 convs' weights
+   (not the network input conv, not the down convs) are rounded to MX-fp4 values with one scale per 32 x 32 (output x input channel) block and tap.
+   The reference forms the copy before every forward; here it is formed when the weights were replaced through this interface (set / load /
+   EMA switch). A caller that writes through unet_param_ptr calls mi_unet_weights_changed. */
+void mi_unet_weights_changed(unet *u) { u->wm_ok = 0; lp_wmemo_clear(); }
+static void fw_refresh(unet *u) {
+    if (!u->wm || u->wm_ok) return;
+    mi_d2d(u->wm, u->src, u->np * 4);
+    const int L = u->cfg.nlev;
+    const convp *cs[4 * UNET_MAXLEV]; int n = 0;
+    for (int i = 0; i < L; i++) { if (i) cs[n++] = &u->enc[i].c1; cs[n++] = &u->enc[i].c2; }
+    for (int i = 0; i < L - 1; i++) { cs[n++] = &u->dec[i].c1; cs[n++] = &u->dec[i].c2; }
+    for (int i = 0; i < n; i++) nn_fakeq_w4_2d(u->wm + cs[i]->w, cs[i]->cout, cs[i]->cin, 27, 32);
+    lp_wmemo_clear();
+    u->wm_ok = 1;
+}
 void mi_unet_get_params(const unet *u, float *host) { mi_sync(); mi_d2h(host, u->p, u->np * 4); }
-void mi_unet_set_params(unet *u, const float *host) { mi_h2d(u->p, host, u->np * 4); mi_h2d(u->ema, host, u->np * 4); lp_wmemo_clear(); }
+void mi_unet_set_params(unet *u, const float *host) { mi_h2d(u->p, host, u->np * 4); mi_h2d(u->ema, host, u->np * 4); u->wm_ok = 0; lp_wmemo_clear(); }
 shape5 unet_out_shape(const unet *u, shape5 xs) { return (shape5){xs.n, u->cfg.cout, xs.d, xs.h, xs.w}; }
 
 /* splitmix64 -> uniform -> Box-Muller normal: the distribution of src/unet.c:586-593, not its generator's bits */
@@ -323,6 +346,7 @@ static int graph_fwd(unet *u, const void *x) {
    inside it look like MX storage) */
 const float *mi_unet_forward_mx(unet *u, const void *xmx, shape5 xs) {
     if (ensure_built(u, xs)) return nullptr;
+    fw_refresh(u);
     const int reg_here = xmx != u->xin && nn_storage(xmx) != u->act_dt;     /* the input is looked up by the convs like any activation */
     if (reg_here) nn_set_storage(xmx, act_bytes(u, u->in), u->act_dt);
     const int rc = graph_fwd(u, xmx);
@@ -391,14 +415,14 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     p += 10;
     for (int i = 0; i < cfg->nlev; i++) { cfg->widths[i] = atoi(p); p = strchr(p, ','); if (!p) break; p++; }
     cfg->cin = key_int(line, "\"cin\":", 0); cfg->cout = key_int(line, "\"cout\":", 0); cfg->G = key_int(line, "\"G\":", 8);
-    cfg->down_norm = key_int(line, "\"down_norm\":", 0);
+    cfg->down_norm = key_int(line, "\"down_norm\":", 0); cfg->w4_2d = key_int(line, "\"w4_2d\":", 0);
     cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
     cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
     cfg->half_res = key_int(line, "\"half_res\":", 0); cfg->scan_norm = key_int(line, "\"scan_norm\":", 0);      /* (the caller's business: the graph does not use them) */
     if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
-    static const char *const no[] = {"\"dec_widths\":", "\"enc_blocks\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"w4_2d\":", "\"ds_levels\":", "\"emb_lev\":",
+    static const char *const no[] = {"\"dec_widths\":", "\"enc_blocks\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"ds_levels\":", "\"emb_lev\":",
                                      "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
                                      "\"l0_norm\":", "\"skip_empty\":", "\"gfilm\":", "\"gn_ema\":", "\"dec_convs\":"};
     const char *bad = nullptr;
@@ -423,6 +447,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.cout != m->cout) bad = "cout";
     if (!bad && c.attn_blocks != m->attn_blocks) bad = "attn_blocks";
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
+    if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
     if (!bad && np != u->np) bad = "nparams";
     if (bad) { fprintf(stderr, "unet_load: %s: \"%s\" differs from this network's\n", path, bad); return -1; }
     FILE *f = fopen(path, "rb");
@@ -443,7 +468,7 @@ int unet_load(unet *u, const char *path) {
             if (fread(h, 4, np, f) != np) { rc = -1; break; }
             size_t nbad = 0; for (size_t i = 0; i < np; i++) nbad += !isfinite(h[i]);
             if (nbad) { fprintf(stderr, "unet_load: %s: %zu non-finite values\n", path, nbad); rc = -1; break; }
-            mi_h2d(which ? u->ema : u->p, h, (size_t)a);
+            mi_h2d(which ? u->ema : u->p, h, (size_t)a); u->wm_ok = 0;
         }
         lp_wmemo_clear();
     }
@@ -463,6 +488,7 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.widths[i]);
     fputc(']', f);
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
+    if (u->cfg.w4_2d) fprintf(f, ",\"w4_2d\":%d", u->cfg.w4_2d);                                  /* (where src/unet.c:5561 writes it: before cin) */
     fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":0,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.cout, u->cfg.G,
             u->cfg.down_norm, u->np, step);
     fprintf(f, ",\"extra\":%s}\n", extra ? extra : "{}");

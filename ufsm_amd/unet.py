@@ -42,6 +42,7 @@ def load_host():
     L.unet_param_ptr.restype = P; L.unet_param_ptr.argtypes = [P]
     L.unet_ema_ptr.restype = P; L.unet_ema_ptr.argtypes = [P]
     L.unet_use_ema.restype = None; L.unet_use_ema.argtypes = [P, _I]
+    L.mi_unet_weights_changed.restype = None; L.mi_unet_weights_changed.argtypes = [P]
     L.unet_set_act_mx8.restype = None; L.unet_set_act_mx8.argtypes = [_I]
     L.unet_set_act_mx4.restype = None; L.unet_set_act_mx4.argtypes = [_I]
     L.unet_act_mx.restype = _I; L.unet_act_mx.argtypes = []
@@ -76,12 +77,12 @@ def load_host():
     return L
 
 
-def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0):
+def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0, w4_2d=0):
     """The reference's configuration record plus, as Python attributes, what the reference keeps in process-wide switches: the activation
     storage (unet_set_act_mx4) and the compute precision policy (nn_set_prec), which UNet applies around its calls."""
     c = unet_cfg()
     c.cin, c.nlev, c.G, c.cout = cin, len(widths), G, head_out
-    c.attn_blocks, c.attn_pe, c.attn_reg, c.attn_mlp, c.down_norm = attn_blocks, attn_pe if attn_blocks else 0, attn_reg, attn_mlp, down_norm
+    c.attn_blocks, c.attn_pe, c.attn_reg, c.attn_mlp, c.down_norm, c.w4_2d = attn_blocks, attn_pe if attn_blocks else 0, attn_reg, attn_mlp, down_norm, w4_2d
     for i, w in enumerate(widths):
         c.widths[i] = w
     c.act_dt, c.prec = act_dt, prec
