@@ -23,7 +23,7 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 METRIC = "U-Net infer voxels/s (128^3 patch, MX fp8) + 3x3x3 conv % of MFMA peak"
 TRAFFIC_BYTES_PER_LAUNCH = 183.9e6     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/
 # HBM bytes per launch of the U-Net's dominant conv from committed counter runs: layer -> (bytes, source); absent: not measured
-KERNEL_TRAFFIC = {}
+KERNEL_TRAFFIC = {"dec0.c1": (809.1e6, "profiles/conv3_row_f8_c96to32_128cube_counters.txt (the same kernel and tensor sizes on a one-segment 96-channel input)")}
 MFMA_PEAK_FP8_TFLOPS = 5033.0          # MI355X dense MXFP8 (2.5 PFLOP/s bf16 x 2)
 
 
