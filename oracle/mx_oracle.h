@@ -36,6 +36,19 @@
  *                                 tensor under one scale (tests/test_oracle_stem.py)
  *   ... with stem_tile 2          the 9 .. 16 channel form with one scale per staged row (src/lp_f8fwd.cuh:447-563): exact operands equal the
  *                                 fp64 convolution; one large value coarsens exactly the outputs of its x tile that read its (z, y) line
+ *   orc_h16_to_mx                 pinned: numpy float16 values through the independent block quantiser (tests/test_oracle_elem.py)
+ *   orc_pred_input_mx             pinned: a numpy statement of src/lp_mx_cvt.cu:24-41 through the independent block quantiser, all axes, the
+ *                                 16-bit roundings, signed zeros (tests/test_oracle_elem.py). PARITY UNPINNED against the reference binary for
+ *                                 channels 2 and 3: it is built with -use_fast_math, whose approximate division and square root are not
+ *                                 defined to the bit; this restatement and the device use IEEE operations
+ *   orc_gn_silu_apply_mx          pinned: fp64 SiLU of the fp32 affine through the independent quantiser with the reference's neighbour-code
+ *                                 acceptance, and closed forms (tests/test_oracle_elem.py); its SiLU bits as above
+ *   binary16 upsample blend       pinned: orc_h16_fma == one rounding of the exact rational result; the staged operand == src/lp_common.cuh:674-712
+ *                                 restated in exact rationals rounded per step; grid data == the fp64 interpolation (tests/test_oracle_elem.py)
+ *   orc_conv2                     pinned: fp64 closed forms on exact operands, orc_conv3 at stride 2 with the taps embedded in a 3x3x3 kernel,
+ *                                 adjointness of the two ops (tests/test_oracle_conv2.py). No counterpart in the reference.
+ *   2-D fp4 weight scales,        pinned: the numpy block quantiser on whole tiles; the reference's invariant that per-channel blocks re-quantise
+ *   orc_fakeq_w4                  the fake-quantised values exactly (tests/test_oracle_w4_2d.py)
  */
 #ifndef MX_ORACLE_H
 #define MX_ORACLE_H

@@ -64,8 +64,8 @@ static int conv2_dispatch(const char *who, int up, int bits, const void *x, int 
     const size_t smem = a.red_o + 1024;
     const long long Scol = up ? (long long)S : (long long)a.Do * a.Ho * a.Wo;
     const long long gx = ((Scol + 31) / 32 + 7) / 8;         // 4 wavefronts x 2 tiles of 32 columns per workgroup
-    if (gx > 0x7fffffffLL || a.ncs > 65535) mi_die("%s: launch grid", who);
-    const dim3 grid((unsigned)gx, (unsigned)a.ncs, (unsigned)N);
+    if (gx > 0x7fffffffLL || a.ncs > 8191) mi_die("%s: launch grid", who);
+    const dim3 grid((unsigned)gx, (unsigned)(up ? 8 * a.ncs : a.ncs), (unsigned)N);      // (up: one tap per workgroup)
     const int out = ybf == 3 ? 8 : ybf == 4 ? 4 : 0;
     if (fmt == 8) conv2_launch_f8(out, up, MT, a, grid, smem); else conv2_launch_f4(out, up, MT, a, grid, smem);
     return 0;

@@ -7,8 +7,8 @@
 // 32 (e4m3) or 16 (e2m1) contiguous bytes, lanes of a voxel tile read neighbouring rows, and lane (r, h) of a 32x32x64 MFMA takes bytes 16 h .. of
 // both rows of a K pair (e4m3) or the whole row of unit h (e2m1), with unit h's scale byte.
 //   down: column = output voxel, K = (tap, block) tap-major: pair units 2 p, 2 p + 1; the row of unit (t, b) is voxel (2 oz + dz, 2 oy + dy, 2 ox + dx)
-//   up:   column = input voxel; the eight taps are eight GEMMs over K = blocks on the same rows, each followed by an epilogue whose output
-//         voxel is (2 iz + dz, 2 iy + dy, 2 ix + dx)
+//   up:   column = input voxel; the eight taps are eight GEMMs over K = blocks on the same rows (one tap per workgroup), each followed by an
+//         epilogue whose output voxel is (2 iz + dz, 2 iy + dy, 2 ix + dx)
 // A wavefront owns NT = 2 tiles of 32 consecutive columns (linear voxel index) and MT channel tiles of 32; the weights' fragments come from
 // global memory in the prepared lane order (a few KiB per K pair, shared by every wavefront: cache hits).
 #pragma once
@@ -19,7 +19,7 @@ __global__ void __launch_bounds__(256, 2) conv2_mx_k(const conv_args a) {
     constexpr int NT = 2, RB = fmt_t<FMT>::RB, WTILE = fmt_t<FMT>::WTILE;
     extern __shared__ __align__(16) unsigned char lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
-    const int n = blockIdx.z, cs = blockIdx.y, nb = a.nbs[0];
+    const int n = blockIdx.z, cs = UP ? (int)(blockIdx.y % (unsigned)a.ncs) : (int)blockIdx.y, nb = a.nbs[0];      // (up: blockIdx.y = tap x channel slices)
     const size_t Sin = (size_t)a.D * a.H * a.W;
     const long long Scol = UP ? (long long)Sin : (long long)a.Do * a.Ho * a.Wo;
     conv_epi_consts<MT, false>(a, lds, cs, tid);
@@ -101,7 +101,8 @@ __global__ void __launch_bounds__(256, 2) conv2_mx_k(const conv_args a) {
         conv_epilogue<MT, NT, OUT, false, false, false, false, true, 4, true>(a, acc, lds, 0u, n, cs, 0, 0, 0, 0, 0, tid, ovx);
     } else {
         const int npt = (nb + 1) >> 1;
-        for (int t = 0; t < 8; t++) {
+        {
+            const int t = (int)(blockIdx.y / (unsigned)a.ncs);   // one tap per workgroup: eight times the workgroups, the rows re-read through the L2
             clear();
             for (int pp = 0; pp < npt; pp++) {
                 bfrag fb[NT];
