@@ -188,3 +188,26 @@ def test_conv2_past_4gib(gpu):
         want = orc.conv2(q1, 3, 1, Ci, D, D, D, w, None, Co, 3, up, cbits=8, acc64=1)
         for n in (0, N - 1):
             assert np.array_equal(fetch_mx(y, 8, N, Co, So, n), want), (up, n)
+
+
+def test_empty_tensors_are_no_ops(gpu):
+    """Zero samples or zero voxels: every entry point returns without a launch error and writes nothing."""
+    d = DevBuf(4096); w = DevBuf(1 << 20); y = DevBuf(4096)
+    lib.mi_zero(y.ptr, 4096)
+    g, sp = gnp_t(), split_t()
+    gg = dev_gn(np.ones(32, np.float32), np.zeros(32, np.float32), np.zeros(8, np.float32), np.ones(8, np.float32), 8)
+    for N, D in ((0, 8), (1, 0)):
+        S = D ** 3
+        xs = shape5(N, 32, D, D, D)
+        lib.lp_f32_to_mx8(d.ptr, N, 32, S, y.ptr); lib.lp_f32_to_mx4(d.ptr, N, 32, S, y.ptr)
+        lib.lp_mx8_to_f32(d.ptr, N, 32, S, y.ptr); lib.lp_mx4_to_f32(d.ptr, N, 32, S, y.ptr)
+        assert lib.lp_conv_fwd_f8(d.ptr, 3, xs, w.ptr, None, 32, y.ptr, 3, g, None, 0, sp) == 0
+        assert lib.lp_conv_fwd_f4(d.ptr, 4, xs, w.ptr, None, 64, y.ptr, 4, g, None, 0, sp) == 0
+        Do = (D - 1) // 2 + 1 if D else 1                                   # (the entry's C formula: (0 - 1) / 2 + 1 = 1)
+        lib.lp_conv_fwd_s2_f8(d.ptr, 3, xs, w.ptr, None, 32, y.ptr, 3, shape5(N, 32, Do, Do, Do), g)
+        lib.lp_conv1_fwd_mx(d.ptr, 3, xs, w.ptr, None, 8, y.ptr, g)
+        lib.lp_up2_fwd_mx(d.ptr, 3, xs, y.ptr, 3, g)
+        lib.lp_add_mx(y.ptr, d.ptr, xs, 3, 0)
+        lib.lp_gn_silu_apply_mx(d.ptr, 3, xs, 8, gg.gamma, gg.beta, gg.mean, gg.rstd, y.ptr, 3)
+        LP.check()
+    assert not y.to_numpy(np.uint8).any()
