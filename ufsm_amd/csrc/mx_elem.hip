@@ -426,19 +426,21 @@ extern "C" void lp_add_mx(void *y, const void *x, shape5 s, int dt, unsigned sr)
 // Sums 32 per-lane fp64 values over the 32 lanes of each wavefront half in a fixed order: step k pairs lane r with r ^ 2^k and the pair
 // splits the values left (the lane whose bit k is clear keeps the lower half of the indices and receives the partner's). Returns the index
 // of the value whose total the lane holds in v[0] afterwards: sum over k of bit k of r times 16 >> k.
+template <int K>
+__device__ __forceinline__ void wave_half_reduce_f64_step(double (&v)[32], int r, int &idx) {      // (a template per step: every index is a constant, the values stay in registers)
+    constexpr int half = 16 >> K;
+    const bool bit = (r >> K) & 1;
+#pragma unroll
+    for (int i = 0; i < half; i++) {
+        const double send = bit ? v[i] : v[i + half], keep = bit ? v[i + half] : v[i];
+        v[i] = keep + __shfl_xor(send, 1 << K);
+    }
+    idx += bit ? half : 0;
+}
 __device__ __forceinline__ int wave_half_reduce_f64(double (&v)[32], int r) {
     int idx = 0;
-#pragma unroll
-    for (int k = 0; k < 5; k++) {
-        const int half = 16 >> k;
-        const bool bit = (r >> k) & 1;
-#pragma unroll
-        for (int i = 0; i < half; i++) {
-            const double send = bit ? v[i] : v[i + half], keep = bit ? v[i + half] : v[i];
-            v[i] = keep + __shfl_xor(send, 1 << k);
-        }
-        idx += bit ? half : 0;
-    }
+    wave_half_reduce_f64_step<0>(v, r, idx); wave_half_reduce_f64_step<1>(v, r, idx); wave_half_reduce_f64_step<2>(v, r, idx);
+    wave_half_reduce_f64_step<3>(v, r, idx); wave_half_reduce_f64_step<4>(v, r, idx);
     return idx;
 }
 // A block reduces a slab of voxels of one (n, channel block): per-thread fp64 partials per channel, then a fixed-order (deterministic)
