@@ -495,12 +495,13 @@ extern "C" int lp_gn_sums_mx(const void *x, int xdt, int N, int C, int G, size_t
 // ---- 1x1x1 head (src/lp_mx_conv1.cu:5-21): y[n][co][v] = b[co] + sum_ci w[co][ci] act(x[ci][v]), fp32 FMA in ci order ----
 // Thread per voxel; weights, bias and the GN coefficients of the sample staged in LDS once per block; CO outputs per pass in registers.
 template <int B, int CO, typename YT>
-__global__ void __launch_bounds__(256) conv1_mx_k(const uint8_t *x, const float *w, const float *b, YT *y, int N, int Ci, size_t S, gnp_t gp, int Co, int co0,
+__global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const float *w, const float *b, YT *y, int N, int Ci, size_t S, gnp_t gp, int Co, int co0,
                                                   size_t vb, size_t nv, size_t ly) {
-    extern __shared__ float c1s[];          // [CO][Ci] weights, [CO] bias, [Ci] a, [Ci] b
-    float *sw = c1s, *sb = sw + CO * Ci, *sa = sb + CO, *sbb = sa + Ci;
+    extern __shared__ __align__(16) float c1s[];          // [Ci][CO] weights (input-channel major: a channel's CO weights are one or two 16-byte reads at an
+                                                          // immediate offset from the block's base), [CO] bias, [Ci] a, [Ci] b
+    float *sw = c1s, *sb = sw + CO * Ci, *sa = sb + 8, *sbb = sa + ((Ci + 3) & ~3);      // (every array starts on 16 bytes when Ci is a multiple of 4; the fast path needs Ci % 32 == 0)
     const int n = blockIdx.y, bw = mx_bw(Ci), nb = mx_nb(Ci);
-    for (int i = threadIdx.x; i < CO * Ci; i += 256) { const int co = co0 + i / Ci; sw[i] = co < Co ? w[(size_t)co * Ci + i % Ci] : 0.f; }
+    for (int i = threadIdx.x; i < CO * Ci; i += 256) { const int co = co0 + i % CO, ci = i / CO; sw[i] = co < Co ? w[(size_t)co * Ci + ci] : 0.f; }
     for (int i = threadIdx.x; i < CO; i += 256) sb[i] = b && co0 + i < Co ? b[co0 + i] : 0.f;
     for (int i = threadIdx.x; i < Ci; i += 256) {
         float a = 1.f, bb = 0.f;
@@ -518,13 +519,47 @@ __global__ void __launch_bounds__(256) conv1_mx_k(const uint8_t *x, const float 
     for (int blk = 0; blk < nb; blk++) {
         float r[32];
         load_row<B>(x, sc, ((size_t)n * nb + blk) * S + v, bw, r);
+        if (bw == 32 && (blk + 1) * 32 <= Ci) {                  // (uniform) a whole 32-channel block: straight-line code, every LDS operand at an immediate offset
+            const float *swb = sw + (size_t)blk * 32 * CO, *sab = sa + blk * 32, *sbb2 = sbb + blk * 32;
+            if (gp.G) {
+#pragma unroll
+                for (int k4 = 0; k4 < 8; k4++) {
+                    const float4 ta = *(const float4 *)(sab + 4 * k4), tb = *(const float4 *)(sbb2 + 4 * k4);
+                    r[4 * k4] = d_act_ab(r[4 * k4], ta.x, tb.x); r[4 * k4 + 1] = d_act_ab(r[4 * k4 + 1], ta.y, tb.y);
+                    r[4 * k4 + 2] = d_act_ab(r[4 * k4 + 2], ta.z, tb.z); r[4 * k4 + 3] = d_act_ab(r[4 * k4 + 3], ta.w, tb.w);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 32; k++) {
+                float wv[CO];
+                if constexpr (CO >= 4) {
+#pragma unroll
+                    for (int q = 0; q < CO / 4; q++) { const float4 w4 = *(const float4 *)(swb + k * CO + 4 * q); wv[4 * q] = w4.x; wv[4 * q + 1] = w4.y; wv[4 * q + 2] = w4.z; wv[4 * q + 3] = w4.w; }
+                } else {
+#pragma unroll
+                    for (int co = 0; co < CO; co++) wv[co] = swb[k * CO + co];
+                }
+#pragma unroll
+                for (int co = 0; co < CO; co++) acc[co] = fmaf(wv[co], r[k], acc[co]);
+                if (k % 4 == 3) __builtin_amdgcn_sched_barrier(0);     // (a thread uses each weight once: reading them all ahead only costs registers)
+            }
+            continue;
+        }
 #pragma unroll
         for (int k = 0; k < 32; k++) {
             const int ci = blk * bw + k;
             if (k < bw && ci < Ci) {
                 const float xv = gp.G ? d_act_ab(r[k], sa[ci], sbb[ci]) : r[k];
+                float wv[CO];
+                if constexpr (CO >= 4) {
 #pragma unroll
-                for (int co = 0; co < CO; co++) acc[co] = fmaf(sw[co * Ci + ci], xv, acc[co]);
+                    for (int q = 0; q < CO / 4; q++) { const float4 w4 = *(const float4 *)(sw + (size_t)ci * CO + 4 * q); wv[4 * q] = w4.x; wv[4 * q + 1] = w4.y; wv[4 * q + 2] = w4.z; wv[4 * q + 3] = w4.w; }
+                } else {
+#pragma unroll
+                    for (int co = 0; co < CO; co++) wv[co] = sw[ci * CO + co];
+                }
+#pragma unroll
+                for (int co = 0; co < CO; co++) acc[co] = fmaf(wv[co], xv, acc[co]);
             }
         }
     }
@@ -545,7 +580,7 @@ static void conv1_launch(const void *x, int xdt, shape5 xs, const float *w, cons
     const uint8_t *xq = (const uint8_t *)x;
     for (int co0 = 0; co0 < cout; co0 += 8) {
         const int rem = cout - co0;
-        const size_t sm = ((size_t)8 * xs.c + 8 + 2 * (size_t)xs.c) * sizeof(float);
+        const size_t sm = ((size_t)8 * xs.c + 8 + 2 * (size_t)((xs.c + 3) & ~3)) * sizeof(float);
 #define C1(B, CO) conv1_mx_k<B, CO, YT><<<grid, 256, sm>>>(xq, w, b, y, xs.n, xs.c, S, gp, cout, co0, vb, nv, ly)
         if (xdt == 4) { if (rem >= 8) C1(4, 8); else if (rem >= 4) { C1(4, 4); co0 -= 4; } else if (rem >= 2) { C1(4, 2); co0 -= 6; } else { C1(4, 1); co0 -= 7; } }
         else { if (rem >= 8) C1(8, 8); else if (rem >= 4) { C1(8, 4); co0 -= 4; } else if (rem >= 2) { C1(8, 2); co0 -= 6; } else { C1(8, 1); co0 -= 7; } }
