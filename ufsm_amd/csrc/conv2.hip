@@ -10,7 +10,7 @@ __global__ void __launch_bounds__(128) prep_w2_k(const float *__restrict__ w, ui
     const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     const int Cop = nmt_all * 32;
     if (i >= (size_t)npairs * Cop) return;
-    const int cop = (int)(i % Cop), gp = (int)(i / Cop), m = cop >> 5, r = cop & 31, npt = (nb + 1) >> 1;
+    const int cop = (int)(i % Cop), gp = (int)(i / Cop), m = cop >> 5, r = cop & 31, npt = (nb + 1) >> 1, cw = (cop & ~31) + mi_row_chan(r);     // row r carries output channel cw
     uint8_t *tile = wq + ((size_t)gp * nmt_all + m) * WTILE;
     unsigned *tsc = wsc + ((size_t)gp * nmt_all + m) * 64;
 #pragma unroll
@@ -21,7 +21,7 @@ __global__ void __launch_bounds__(128) prep_w2_k(const float *__restrict__ w, ui
 #pragma unroll
         for (int k = 0; k < 32; k++) {
             const int ci = blk * 32 + k;
-            v[k] = (blk < nb && cop < Co && ci < Ci) ? (up ? w[((size_t)ci * Co + cop) * 8 + t] : w[((size_t)cop * Ci + ci) * 8 + t]) : 0.f;
+            v[k] = (blk < nb && cw < Co && ci < Ci) ? (up ? w[((size_t)ci * Co + cw) * 8 + t] : w[((size_t)cw * Ci + ci) * 8 + t]) : 0.f;
         }
         prep_store_unit<FMT>(tile, tsc, 1, side, r, v);
     }

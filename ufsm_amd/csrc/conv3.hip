@@ -77,7 +77,7 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
     const int cop = (int)(i % Cop), gp = (int)(i / Cop);
     int b0 = 0, pb = 0, nbc = 0;
     if (block_major >= 0) for (;; b0 += CB) { nbc = min(CB, nbt - b0); const int np = (27 * nbc + 1) >> 1; if (gp < pb + np) break; pb += np; }
-    const int q = gp - pb, m = cop >> 5, r = cop & 31;
+    const int q = gp - pb, m = cop >> 5, r = cop & 31, cw = (cop & ~31) + mi_row_chan(r);       // row r of the tile carries output channel cw
     uint8_t *tile = wq + ((size_t)gp * nmt_all + m) * WTILE;
     unsigned *tsc = wsc + ((size_t)gp * nmt_all + m) * 64;      // one word per lane: the byte the MFMA reads is the low one
     int tss = 1;                                                // words between two lanes' scale words
@@ -106,7 +106,7 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
 #pragma unroll
         for (int k = 0; k < 32; k++) {
             const int ci = seg_ci(blk * 32 + k, Ci, Cx, CxP);
-            v[k] = (unit_ok && cop < Co && ci >= 0) ? w[((size_t)cop * Ci + ci) * 27 + t] : 0.f;
+            v[k] = (unit_ok && cw < Co && ci >= 0) ? w[((size_t)cw * Ci + ci) * 27 + t] : 0.f;
         }
         prep_store_unit<FMT>(tile, tsc, tss, side, r, v, w2d != 0);      // (32 consecutive threads hold a channel tile's rows of this pair)
     }
@@ -213,10 +213,10 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
     a.ntx = (W + 15) / 16; a.nty = (H + 7) / 8; a.ntz = (Do + 1) / 2;
     a.ntiles = (unsigned)((size_t)a.ntx * a.nty * a.ntz * a.ncs * N);
-    // z tiles per workgroup (tap-packed kernel: the set-up is amortised, the next tile's loads overlap): up to 4 while >= 8 workgroups per CU remain
+    // z tiles per workgroup (tap-packed kernel: the set-up is amortised, the next tile's loads overlap): up to 8 while >= 8 workgroups per CU remain
     a.zc = 1;
     if (!rows && CP <= 4 && g_stem_zc > 0) a.zc = g_stem_zc < a.ntz ? g_stem_zc : a.ntz;
-    else if (!rows && CP <= 4) { a.zc = 4; while (a.zc > 1 && (size_t)a.ntx * a.nty * ((a.ntz + a.zc - 1) / a.zc) * a.ncs * N < 2048) a.zc--; }
+    else if (!rows && CP <= 4) { a.zc = 8; while (a.zc > 1 && (size_t)a.ntx * a.nty * ((a.ntz + a.zc - 1) / a.zc) * a.ncs * N < 2048) a.zc--; }
     a.ngrp = (unsigned)((size_t)a.ntx * a.nty * ((a.ntz + a.zc - 1) / a.zc) * a.ncs * N);
     const size_t wq_bytes = (size_t)NP * nmt_all * 2048, wsc_bytes = (size_t)NP * nmt_all * 256;
     int dev = 0; MIRT(hipGetDevice(&dev));

@@ -38,6 +38,15 @@ __device__ __forceinline__ unsigned lane_xor32(unsigned x, int h) {
     return h ? r2[0] : r2[1];
 }
 __device__ __forceinline__ float lane_xor32f(float x, int h) { return __uint_as_float(lane_xor32(__float_as_uint(x), h)); }
+// the maximum of a lane's value and its partner's (l ^ 32): the swap leaves the low halves' values in one result and the high halves' in the other
+__device__ __forceinline__ float lane_pair_max(float x) {
+    const auto r2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r2[0]), __uint_as_float(r2[1]));
+}
+// Output channel (within its tile of 32) of row r of a prepared weight tile. The 32x32 MFMA leaves row (i & 3) + 4 h + 8 (i >> 2) in register i
+// of lane half h; the weights' rows are laid out so that this is channel 16 h + i: a lane holds 16 consecutive channels, i.e. its half of a
+// stored 32-channel row, and nothing is exchanged between the halves
+__host__ __device__ constexpr int mi_row_chan(int r) { return 16 * ((r >> 2) & 1) + (r & 3) + 4 * (r >> 3); }
 template <int MASK> __device__ __forceinline__ float lane_xorf(float x) {
     static_assert(MASK == 1 || MASK == 2 || MASK == 4 || MASK == 8 || MASK == 16, "lane_xorf mask");
     const int xi = (int)__float_as_uint(x);
@@ -234,17 +243,17 @@ __device__ __forceinline__ void conv_epi_consts(const conv_args &a, unsigned cha
 
 // ---- epilogue (src/lp_common.cuh:1465-1597): bias -> optional affine + activation -> per (voxel, 32-channel block) amax across the
 // lane pair (l, l ^ 32) -> E8M0 exponent -> codes -> row stores; GroupNorm partial sums per tile. acc: the wavefront's MT x NT accumulators;
-// lane (r, h) of tile j holds voxel (oz0 + lz, oy0 + ly0 + 2 j + (r >> 4), ox0 + (r & 15)) ----
+// register i of lane (r, h) is channel 16 h + i of the tile (mi_row_chan: the prepared weights' row order); lane (r, h) of tile j holds voxel (oz0 + lz, oy0 + ly0 + 2 j + (r >> 4), ox0 + (r & 15)) ----
 // FULL: the tile lies inside the output and the statistics cover all of its planes (uniform, checked by the caller): no per-lane predicates,
 // so the whole epilogue is straight-line code the scheduler can interleave across the accumulator tiles
-// NOCH: the caller never takes per-channel statistics records (stat_ch): their 32 sums are not kept
+// NOCH: this call takes no per-channel statistics records (the caller has checked stat_ch, or never sets it): their 32 sums are not kept
 // NW: wavefronts of the workgroup (their partial statistics are summed in wave order); ROW: the row kernel's voxel mapping, lane r of tile j
 // holds voxel (oz0 + lz, oy0 + ly0 + j, ox0 + r) of a 32-voxel run along x
 template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false, bool NOCH = false, int NW = 4, bool ROW = false>
 __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT][NT], unsigned char *lds, unsigned tile, int n, int cs,
                                               int oz0, int oy0, int ox0, int lz, int ly0, int tid, const long long *ovx = nullptr) {
     const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
-    // accumulator layout of the 32x32 MFMA: lane (r = voxel within the tile, h), register i -> channel (i & 3) + 4 h + 8 (i >> 2)
+    // accumulator layout of the 32x32 MFMA: lane (r = voxel within the tile, h), register i -> row (i & 3) + 4 h + 8 (i >> 2) = channel 16 h + i
     const size_t So = (size_t)(a.yD ? a.yD : a.Do) * a.Ho * a.Wo;      // voxels per channel plane of the output tensor
     const int co_base = cs * MT * 32;
     float *red = (float *)(lds + a.red_o);          // stats scratch [4 waves][MT][8 quads][2] floats
@@ -265,11 +274,11 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
     static_for<MT>([&](auto M) {
         constexpr int m = M;
         DBG_MARK(16 + m);
-        // the lane's 16 channels of tile m are four runs of 4: (i & 3) + 4 h + 8 (i >> 2)
+        // the lane's 16 channels of tile m: 16 h + i
         float bias[16], ea[16], eb[16];
 #pragma unroll
         for (int q4 = 0; q4 < 4; q4++) {
-            const unsigned o = a.epi_o + (m * 32 + 8 * q4 + 4 * h) * 4;
+            const unsigned o = a.epi_o + (m * 32 + 16 * h + 4 * q4) * 4;
             const float4 b4 = *(const float4 *)(lds + o);
             bias[4 * q4] = b4.x; bias[4 * q4 + 1] = b4.y; bias[4 * q4 + 2] = b4.z; bias[4 * q4 + 3] = b4.w;
             if (EPI) {
@@ -295,12 +304,12 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                 if (EPI) {
                     t = fmaf(t, ea[i], eb[i]);
                     t = a.act == 1 ? d_silu(t) : a.act == 2 ? gelu_erf(t) : a.act == 3 ? fmaxf(t, 0.f) : t;
-                    if (co_base + m * 32 + (i & 3) + 4 * h + 8 * (i >> 2) >= a.Co) t = 0.f;
+                    if (co_base + m * 32 + 16 * h + i >= a.Co) t = 0.f;
                 }
                 v[i] = t; am = fmaxf(am, fabsf(t));
             }
             if (OUT != 0) {
-                am = fmaxf(am, lane_xor32f(am, h));
+                am = lane_pair_max(am);
                 const int e = d_mx_exp(am, YB == 8 ? MI_INVQ8 : MI_INVQ4);
                 const int blk = (co_base + m * 32) / bwo;                  // bwo < 32 only when Co <= 16: one tile, block 0
                 const size_t row = ((size_t)n * nbo + blk) * So + ov;
@@ -323,37 +332,25 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                             v[4 * q4] = lo[0]; v[4 * q4 + 1] = lo[1]; v[4 * q4 + 2] = hi[0]; v[4 * q4 + 3] = hi[1];
                         }
                     }
-                    // lane h = 0 holds bytes {0-3, 8-11, 16-19, 24-27}, its partner {4-7, 12-15, 20-23, 28-31}: swap so each stores 16 contiguous bytes
-                    const unsigned s0 = h ? d[0] : d[2], s1 = h ? d[1] : d[3];
-                    const unsigned r0 = lane_xor32(s0, h), r1 = lane_xor32(s1, h);
-                    const uint4 out = h ? make_uint4(r0, d[2], r1, d[3]) : make_uint4(d[0], r0, d[1], r1);
+                    const uint4 out = make_uint4(d[0], d[1], d[2], d[3]);      // bytes 16 h .. 16 h + 15 of the row
                     if (ok) {
                         if (bwo == 32) *(uint4 *)(yq + row * 32 + 16 * h) = out;
                         else if (bwo == 16) { if (!h) *(uint4 *)(yq + row * 16) = out; }
                         else if (!h) *(uint2 *)(yq + row * 8) = make_uint2(out.x, out.y);
                     }
                 } else {
-                    unsigned hw[4];   // 4 channels -> 16 bits each
-                    {
-                        const float p2e = d_exp2i(e);
-                        unsigned w01 = d_enc_e2m1x8_hw(v, p2e), w23 = d_enc_e2m1x8_hw(v + 8, p2e);
-                        if (__builtin_amdgcn_ballot_w64(e == 128) != 0ull) {
-                            if (e == 128) { w01 = d_enc8_e2m1_nf(v); w23 = d_enc8_e2m1_nf(v + 8); }
-                        }
-                        hw[0] = w01 & 0xffffu; hw[1] = w01 >> 16; hw[2] = w23 & 0xffffu; hw[3] = w23 >> 16;
-                        if (a.stored_stats) {
-                            const float sc = d_exp2i(e);
-                            d_dec8_e2m1(w01, v); d_dec8_e2m1(w23, v + 8);
-#pragma unroll
-                            for (int i = 0; i < 16; i++) v[i] *= sc;
-                        }
+                    const float p2e = d_exp2i(e);
+                    unsigned w01 = d_enc_e2m1x8_hw(v, p2e), w23 = d_enc_e2m1x8_hw(v + 8, p2e);
+                    if (__builtin_amdgcn_ballot_w64(e == 128) != 0ull) {
+                        if (e == 128) { w01 = d_enc8_e2m1_nf(v); w23 = d_enc8_e2m1_nf(v + 8); }
                     }
-                    // halfword q4 of lane h sits at byte 4 q4 + 2 h of the 16-byte row: lane 0 assembles words 0-1, lane 1 words 2-3
-                    const unsigned mine01 = hw[0] | (hw[1] << 16), mine23 = hw[2] | (hw[3] << 16);
-                    const unsigned send = h ? mine01 : mine23, recv = lane_xor32(send, h);
-                    uint2 out;
-                    if (!h) out = make_uint2((hw[0] & 0xffffu) | ((recv & 0xffffu) << 16), (hw[1] & 0xffffu) | (recv & 0xffff0000u));
-                    else out = make_uint2((recv & 0xffffu) | ((hw[2] & 0xffffu) << 16), (recv >> 16) | ((hw[3] & 0xffffu) << 16));
+                    if (a.stored_stats) {
+                        const float sc = d_exp2i(e);
+                        d_dec8_e2m1(w01, v); d_dec8_e2m1(w23, v + 8);
+#pragma unroll
+                        for (int i = 0; i < 16; i++) v[i] *= sc;
+                    }
+                    const uint2 out = make_uint2(w01, w23);           // bytes 8 h .. 8 h + 7 of the row
                     if (ok) {
                         if (bwo == 32) *(uint2 *)(yq + row * 16 + 8 * h) = out;
                         else if (bwo == 16) { if (!h) *(uint2 *)(yq + row * 8) = out; }
@@ -362,11 +359,11 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
                 }
                 if (ok && !h) ysc[row] = (uint8_t)(e + 127);
             } else {
-                const size_t o0 = ((size_t)n * a.Co + co_base + m * 32 + 4 * h) * So + ov;
+                const size_t o0 = ((size_t)n * a.Co + co_base + m * 32 + 16 * h) * So + ov;
 #pragma unroll
                 for (int i = 0; i < 16; i++) {
-                    const int cl = (i & 3) + 8 * (i >> 2);            // channel offset from co_base + 32 m + 4 h
-                    const bool cok = ok && co_base + m * 32 + 4 * h + cl < a.Co;
+                    const int cl = i;                                 // channel offset from co_base + 32 m + 16 h
+                    const bool cok = ok && co_base + m * 32 + 16 * h + cl < a.Co;
                     if (a.ydt == 2) {
                         if (a.Go > 0) v[i] = fabsf(v[i]) > 65504.f ? copysignf(65504.f, v[i]) : v[i];     // src/lp_common.cuh:465, :1567-1569
                         if (cok) ((__half *)a.y)[o0 + (size_t)cl * So] = __float2half(v[i]);
@@ -390,12 +387,12 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
     DBG_MARK(21);
     if (CH && stats && a.stat_ch) {
         // any group size (one channel tile): per-channel sums over the 32 voxel lanes, then over the waves; channel of register i of
-        // half h = (i & 3) + 4 h + 8 (i >> 2); value index 2 i + t (t 0 sum, 1 sum of squares)
+        // half h = 16 h + i; value index 2 i + t (t 0 sum, 1 sum of squares)
         float v[32];
 #pragma unroll
         for (int i = 0; i < (CH ? 16 : 1); i++) { v[2 * i] = chs[i]; v[2 * i + 1] = chss[i]; }
         const int idx = wave_half_reduce<32>(v, r), i = idx >> 1;
-        red[(wave * 32 + (i & 3) + 4 * h + 8 * (i >> 2)) * 2 + (idx & 1)] = v[0];
+        red[(wave * 32 + 16 * h + i) * 2 + (idx & 1)] = v[0];
         __syncthreads();
         if (tid < 32) {
             float s1 = 0.f, s2 = 0.f;
@@ -403,7 +400,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
             a.part[((size_t)tile * 32 + tid) * 2] = s1; a.part[((size_t)tile * 32 + tid) * 2 + 1] = s2;
         }
     } else if (stats) {
-        // channels per group a multiple of 4: a quad (m, q4, h) = channels co_base + 32 m + 8 q4 + 4 h .. +3 lies in one group.
+        // channels per group a multiple of 4: a quad (m, q4, h) = channels co_base + 32 m + 16 h + 4 q4 .. +3 lies in one group.
         // Sum over the 32 voxel lanes of each half (fixed order), then over the 4 waves in wave order; value index (4 m + q4) 2 + t
         constexpr int NV = MT <= 1 ? 8 : MT <= 2 ? 16 : 32;
         float v[NV];
@@ -416,13 +413,13 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
         const int idx = wave_half_reduce<NV>(v, r);
         if ((r >> (NV == 8 ? 3 : NV == 16 ? 4 : 5)) == 0 && idx < MT * 8) {
             const int mq = idx >> 1;                                    // 4 m + q4
-            red[((wave * MT + (mq >> 2)) * 8 + (mq & 3) * 2 + h) * 2 + (idx & 1)] = v[0];
+            red[((wave * MT + (mq >> 2)) * 8 + 4 * h + (mq & 3)) * 2 + (idx & 1)] = v[0];
         }
         __syncthreads();
         if (tid < MT * 8) {
             // per tile and channel quad, the sums over the tile's voxels in wave order; a second kernel adds the tiles of a sample
             // in a fixed order into the exact sum slots, so the statistics do not depend on the order workgroups finish in
-            const int m = tid >> 3, q8 = tid & 7;                       // q8 = q4 * 2 + h: channels co_base + 32 m + 8 q4 + 4 h .. + 3
+            const int m = tid >> 3, q8 = tid & 7;                       // q8 = 4 h + q4: channels co_base + 32 m + 4 q8 .. + 3
             float s = 0.f, ss = 0.f;
             for (int w = 0; w < NW; w++) { s += red[((w * MT + m) * 8 + q8) * 2]; ss += red[((w * MT + m) * 8 + q8) * 2 + 1]; }
             a.part[((size_t)tile * MT * 8 + tid) * 2] = s;

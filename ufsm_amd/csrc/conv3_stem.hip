@@ -11,7 +11,7 @@
 #include "conv3_kernel.hpp"
 
 template <int CP, int MT, int OUT>
-__global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
+__global__ void __launch_bounds__(256, MT == 1 ? 3 : 2) conv3_stem_k(const conv_args a) {
     constexpr int TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2, NT = 2;
     constexpr int HY = 10, HX = 18, TT = 4 * HY * HX, WTILE = 2048;
     extern __shared__ __align__(16) unsigned char lds[];
@@ -179,6 +179,8 @@ __global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
         auto tapoff = [](int tap) { tap = tap > 26 ? 26 : tap; return ((tap / 9) * HY + (tap / 3) % 3) * HX + tap % 3; };     // (taps past 26: zero weights)
+        int p00v = p00, hv = h;                              // (opaque per tile: the fragment addresses are formed here, not kept in registers across the z tiles)
+        asm volatile("" : "+v"(p00v), "+v"(hv));
         static_for<NP>([&](auto P) {
             constexpr int p = P;
             constexpr int LT = 16 / CP;                      // taps a lane supplies per K block
@@ -186,10 +188,10 @@ __global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
 #pragma unroll
             for (int s = 0; s < 2; s++)
 #pragma unroll
-                for (int i = 0; i < LT; i++) off[s][i] = h ? tapoff((2 * p + s) * TPK + LT + i) : tapoff((2 * p + s) * TPK + i);
+                for (int i = 0; i < LT; i++) off[s][i] = hv ? tapoff((2 * p + s) * TPK + LT + i) : tapoff((2 * p + s) * TPK + i);
 #pragma unroll
             for (int j = 0; j < NT; j++) {
-                const int pj = p00 + 2 * j * HX;
+                const int pj = p00v + 2 * j * HX;
                 v8i fb;
 #pragma unroll
                 for (int s = 0; s < 2; s++) {
@@ -212,8 +214,9 @@ __global__ void __launch_bounds__(256, 2) conv3_stem_k(const conv_args a) {
         const unsigned tile = (unsigned)(((((size_t)n * a.ntz + tz) * a.nty + ty) * a.ntx + tx) * a.ncs + cs);       // the tile's place among the statistics partials
         // (uniform) more than 16 output channels: 32-wide output rows known at compile time; the tile inside the output and the statistics' planes:
         // no per-lane predicates. (The statistics scratch is next written two barriers on)
-        if (a.Co > 16 && 2 * tz + 2 <= a.Do && oy0 + 8 <= a.Ho && ox0 + 16 <= a.Wo && a.zs0 <= 2 * tz && a.zs1 >= 2 * tz + 2)
-            conv_epilogue<MT, NT, OUT, false, false, true, true>(a, acc, lds, tile, n, cs, 2 * tz, oy0, ox0, lz, ly0, tid);
+        // and no per-channel statistics records (their 32 sums per lane would cost the third workgroup per CU)
+        if (a.Co > 16 && !a.stat_ch && 2 * tz + 2 <= a.Do && oy0 + 8 <= a.Ho && ox0 + 16 <= a.Wo && a.zs0 <= 2 * tz && a.zs1 >= 2 * tz + 2)
+            conv_epilogue<MT, NT, OUT, false, false, true, true, true>(a, acc, lds, tile, n, cs, 2 * tz, oy0, ox0, lz, ly0, tid);
         else conv_epilogue<MT, NT, OUT, false>(a, acc, lds, tile, n, cs, 2 * tz, oy0, ox0, lz, ly0, tid);
     }
 }
@@ -352,7 +355,7 @@ __global__ void __launch_bounds__(256, 2) conv3_p16_k(const conv_args a) {
 __global__ void __launch_bounds__(128) prep_wp16_k(const float *__restrict__ w, uint8_t *__restrict__ wq, unsigned *__restrict__ wsc, int Co, int Ci, int nmt_all) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x, Cop = nmt_all * 32;
     if (i >= 9 * Cop) return;
-    const int cop = i % Cop, p = i / Cop, m = cop >> 5, r = cop & 31;
+    const int cop = i % Cop, p = i / Cop, m = cop >> 5, r = cop & 31, cw = (cop & ~31) + mi_row_chan(r);      // row r of the tile carries output channel cw
     uint8_t *tile = wq + ((size_t)p * nmt_all + m) * 2048;
     unsigned *tsc = wsc + ((size_t)p * nmt_all + m) * 64;
 #pragma unroll
@@ -361,7 +364,7 @@ __global__ void __launch_bounds__(128) prep_wp16_k(const float *__restrict__ w, 
 #pragma unroll
         for (int k = 0; k < 32; k++) {
             const int kx = 2 * side + (k >> 4), ci = k & 15;
-            v[k] = (kx < 3 && cop < Co && ci < Ci) ? w[((size_t)cop * Ci + ci) * 27 + p * 3 + kx] : 0.f;
+            v[k] = (kx < 3 && cw < Co && ci < Ci) ? w[((size_t)cw * Ci + ci) * 27 + p * 3 + kx] : 0.f;
             amax = fmaxf(amax, fabsf(v[k]));
         }
         const int e = d_mx_exp(amax, MI_INVQ8);
@@ -382,7 +385,7 @@ __global__ void __launch_bounds__(128) prep_ws_k(const float *__restrict__ w, ui
     constexpr int TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK;
     const int i = blockIdx.x * blockDim.x + threadIdx.x, Cop = nmt_all * 32;
     if (i >= np * Cop) return;
-    const int cop = i % Cop, p = i / Cop, m = cop >> 5, r = cop & 31;
+    const int cop = i % Cop, p = i / Cop, m = cop >> 5, r = cop & 31, cw = (cop & ~31) + mi_row_chan(r);      // row r of the tile carries output channel cw
     uint8_t *tile = wq + ((size_t)p * nmt_all + m) * 2048;
     unsigned *tsc = wsc + ((size_t)p * nmt_all + m) * 64;
 #pragma unroll
@@ -392,7 +395,7 @@ __global__ void __launch_bounds__(128) prep_ws_k(const float *__restrict__ w, ui
 #pragma unroll
         for (int k = 0; k < 32; k++) {
             const int tap = kb * TPK + k / CP, ci = k % CP;
-            v[k] = (kb < NKB && cop < Co && ci < Ci && tap < 27) ? w[((size_t)cop * Ci + ci) * 27 + tap] : 0.f;
+            v[k] = (kb < NKB && cw < Co && ci < Ci && tap < 27) ? w[((size_t)cw * Ci + ci) * 27 + tap] : 0.f;
             amax = fmaxf(amax, fabsf(v[k]));
         }
         const int e = d_mx_exp(amax, MI_INVQ8);
