@@ -38,10 +38,11 @@ __device__ __forceinline__ unsigned lane_xor32(unsigned x, int h) {
     return h ? r2[0] : r2[1];
 }
 __device__ __forceinline__ float lane_xor32f(float x, int h) { return __uint_as_float(lane_xor32(__float_as_uint(x), h)); }
-// the maximum of a lane's value and its partner's (l ^ 32): the swap leaves the low halves' values in one result and the high halves' in the other
+// the maximum of a lane's value and its partner's (l ^ 32) for values that are not negative and not NaN (an amax): such floats order as their
+// bit patterns; the swap leaves the low halves' values in one result and the high halves' in the other
 __device__ __forceinline__ float lane_pair_max(float x) {
     const auto r2 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-    return fmaxf(__uint_as_float(r2[0]), __uint_as_float(r2[1]));
+    return __uint_as_float(r2[0] > r2[1] ? r2[0] : r2[1]);
 }
 // Output channel (within its tile of 32) of row r of a prepared weight tile. The 32x32 MFMA leaves row (i & 3) + 4 h + 8 (i >> 2) in register i
 // of lane half h; the weights' rows are laid out so that this is channel 16 h + i: a lane holds 16 consecutive channels, i.e. its half of a
@@ -271,6 +272,12 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
     constexpr int YB = OUT == 4 ? 4 : 8;
     const int bwo = W32 ? 32 : mx_bw(a.Co), nbo = W32 ? (a.Co + 31) >> 5 : mx_nb(a.Co), rbo = mx_rb(bwo, YB);     // W32: more than 16 output channels, known at compile time
     uint8_t *yq = (uint8_t *)a.y, *ysc = yq + (size_t)a.N * nbo * So * rbo;
+    // the lane's output voxel: tile j lies JS rows of the volume below tile 0, so one offset per lane and epilogue and a uniform step per tile;
+    // the row index of (tile m, tile j) = rowb + m * mstep + j * jstep (bwo < 32 only when Co <= 16: one channel tile, block 0)
+    constexpr int JS = ROW ? 1 : 2;
+    const int oz = oz0 + lz, oyb = ROW ? oy0 + ly0 : oy0 + ly0 + (r >> 4), ox = ROW ? ox0 + r : ox0 + (r & 15);
+    const size_t ovb = ovx ? 0 : ((size_t)(oz + a.yzo) * a.Ho + oyb) * a.Wo + ox;
+    const size_t rowb = ((size_t)n * nbo + co_base / bwo) * So + ovb, mstep = bwo == 32 ? So : 0, jstep = ovx ? 0 : (size_t)JS * a.Wo;
     static_for<MT>([&](auto M) {
         constexpr int m = M;
         DBG_MARK(16 + m);
@@ -289,10 +296,10 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
         }
         static_for<NT>([&](auto J) {
             constexpr int j = J;
-            const int oz = oz0 + lz, oy = ROW ? oy0 + ly0 + j : oy0 + ly0 + 2 * j + (r >> 4), ox = ROW ? ox0 + r : ox0 + (r & 15);
+            const int oy = oyb + JS * j;
             // ovx: the caller's own voxel mapping (the 2x2x2 stride-2 kernels): the lane's output voxel of tile j, negative = none
             const bool ok = ovx ? ovx[j] >= 0 : (FULL || (oz < a.Do && oy < a.Ho && ox < a.Wo));
-            const size_t ov = ovx ? (size_t)ovx[j] : ((size_t)(oz + a.yzo) * a.Ho + oy) * a.Wo + ox;
+            const size_t ov = ovx ? (size_t)ovx[j] : ovb + j * jstep;
             const bool zst = ovx ? ok : (FULL || (ok && oz >= a.zs0 && oz < a.zs1));
             float v[16];
             float am = 0.f;
@@ -311,8 +318,7 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
             if (OUT != 0) {
                 am = lane_pair_max(am);
                 const int e = d_mx_exp(am, YB == 8 ? MI_INVQ8 : MI_INVQ4);
-                const int blk = (co_base + m * 32) / bwo;                  // bwo < 32 only when Co <= 16: one tile, block 0
-                const size_t row = ((size_t)n * nbo + blk) * So + ov;
+                const size_t row = rowb + m * mstep + (ovx ? (size_t)ovx[j] : j * jstep);
                 if (OUT == 8) {
                     unsigned d[4];
                     const float p2e = d_exp2i(e);

@@ -152,7 +152,7 @@ __global__ void __launch_bounds__(256, MT == 1 ? 3 : 2) conv3_stem_k(const conv_
             }
         }
         amax = fmaxf(amax, lane_xorf<1>(amax)); amax = fmaxf(amax, lane_xorf<2>(amax)); amax = fmaxf(amax, lane_xorf<4>(amax));
-        amax = fmaxf(amax, lane_xorf<8>(amax)); amax = fmaxf(amax, lane_xorf<16>(amax)); amax = fmaxf(amax, lane_xor32f(amax, h));
+        amax = fmaxf(amax, lane_xorf<8>(amax)); amax = fmaxf(amax, lane_xorf<16>(amax)); amax = lane_pair_max(amax);
         if (lane == 0) atomicMax((unsigned *)(lds + am_o), __float_as_uint(amax));        // non-negative floats order as their bit patterns
         __syncthreads();
         const int e = d_mx_exp(__uint_as_float(*(const unsigned *)(lds + am_o)), MI_INVQ8);

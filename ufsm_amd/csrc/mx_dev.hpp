@@ -86,7 +86,7 @@ __device__ __forceinline__ float d_dec_e2m1(unsigned n) {
 typedef short mi_v2s __attribute__((ext_vector_type(2)));
 typedef float mi_v2f __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ unsigned d_enc_e4m3x4_hw(float a, float b, float c, float d, float pow2e) {
-    mi_v2s o = {0, 0};
+    mi_v2s o = __builtin_bit_cast(mi_v2s, a);                  // (any bits: each conversion writes one half of the word, the two write both)
     o = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, a, b, pow2e, false);
     o = __builtin_amdgcn_cvt_scalef32_pk_fp8_f32(o, c, d, pow2e, true);
     return __builtin_bit_cast(unsigned, o);
