@@ -61,6 +61,28 @@ def test_wide_kernel_exact(gpu, slice_split, bits, N, Ci, Co, D, H, W):
     assert np.array_equal(gf, wf)
 
 
+@pytest.mark.parametrize("Ci,Co,split", [(32, 128, 0), (64, 128, 0), (32, 128, 1 << 30)])
+def test_wide_kernel_persistent_walk_few_blocks(gpu, Ci, Co, split):
+    """More tiles than workgroups (every workgroup walks two or four tiles) on inputs of one and two blocks, slices of 128 and of 64 channels:
+    the blocks of a workgroup's next tile are requested while the current one is multiplied, whatever the block count (a one-block input
+    has only the next tile's block to request)."""
+    rng = np.random.default_rng(Ci + Co)
+    N, D, H, W = 2, 32, 64, 64
+    S = D * H * W
+    x, w, b = exact_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(8, x, N, Ci, S)
+    lib.mi_conv_split(split)
+    try:
+        got, gsum = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 3, cbits=8, Go=8, stats=True)
+    finally:
+        lib.mi_conv_split(-1)
+    name = lib.mi_last_kernel().decode()
+    assert "conv3_wide_k" in name and ("tiles 1024 wgs 256" if split else "tiles 512 wgs 256") in name and ("MT 2" in name) == (split != 0)
+    want, wsum = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 3, cbits=8, acc64=1, Go=8, want_stats=True)
+    assert np.array_equal(got, want)
+    assert np.allclose(gsum, wsum, rtol=1e-6)
+
+
 def test_wide_kernel_decoder_conv(gpu):
     """[2x upsampled coarse | skip] -> 128 channels with both GroupNorms: the wide kernel on a split, restaged input (12 blocks)."""
     rng = np.random.default_rng(77)

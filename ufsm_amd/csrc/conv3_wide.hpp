@@ -265,7 +265,7 @@ __global__ void __launch_bounds__(256, 1) conv3_wide_k(const conv_args a) {
         // ---- the streaming schedule. fbi: next block to request (>= nbt: of the next tile), frd: its next copy round. A block may be requested
         // once block fbi - 3, whose slot it takes, has been read for the last time (pair (27 (fbi - 3) + 26) / 2). The host has checked that
         // with two rounds per stage every block of a tile lands two barriers before its first fetch ----
-        int fbi = 2, frd = 0;
+        int fbi = nnext, frd = 0;                             // (blocks 0 .. nnext - 1 of this tile were requested during the tile before, or ahead of the first)
         auto prep_next = [&](hreq &q, int upto_pair) {          // prepare one copy round; pairs <= upto_pair will have been fetched by every wavefront when it is issued
             const bool go = __builtin_amdgcn_readlane(tb_gate, fbi) <= upto_pair;
             prepare(q, mask2 >> __builtin_amdgcn_readlane(tb_msh, fbi), __builtin_amdgcn_readlane(tb_base, fbi), fbi, frd, ring0, (unsigned)__builtin_amdgcn_readlane(tb_slot, fbi), go);
