@@ -74,6 +74,10 @@ void mi_conv_stem_zc(int zc);
 /* tuning knob of the calling thread (no counterpart in the reference): stride-1 launches with fewer tiles of 128 output channels than this run as
    slices of 64 channels, twice the workgroups; 0: never, -1: the default (192, or MI_CONV_SPLIT). The results do not depend on it. */
 void mi_conv_split(int tiles);
+/* Extension: which kernel takes the calling thread's 3x3x3 stride-2 convs on 32-channel rows. -1 (default): the kernel that reads the taps' rows
+   straight from the stored tensor when the launch has enough output voxels to fill the device, else the general kernel (staged halo);
+   0: always the general kernel; 1: the direct kernel whenever its operands allow it. The results are the same conv either way. */
+void mi_conv_s2_direct(int mode);
 /* no counterpart in the reference (its convs transform their input while staging, every time): GroupNorm + SiLU of x and re-quantisation to
    MX-fp8 / MX-fp4 (ybits 8 / 4) once, for a tensor several convs read; they then take y with no GroupNorm. s.c a multiple of 32. In a split
    input, gp2.G = -1 says "x2 carries no GroupNorm, gp is x's own" (gp2.G = 0 keeps the reference's meaning: gp spans both segments). */

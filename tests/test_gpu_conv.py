@@ -109,6 +109,51 @@ EXACT_SHAPES = [
 ]
 
 
+# the stride-2 kernel that reads the taps' rows from the stored tensor (large launches take it by default): odd and even dims, one to five
+# input blocks, 32 / 64 / 128 / 96 output channels, both formats (fp4 compute only for 32 -> <= 32 on even dims, src/lp_s2.cu:647-754)
+S2_DIRECT_SHAPES = [(8, 1, 32, 32, 16, 16, 16), (8, 1, 64, 64, 13, 10, 17), (8, 2, 128, 128, 8, 16, 32), (4, 1, 32, 32, 16, 16, 16), (8, 1, 96, 96, 12, 10, 14),
+                    (8, 2, 160, 64, 5, 7, 33), (4, 1, 64, 128, 6, 12, 20), (8, 1, 32, 40, 3, 5, 7)]
+
+
+@pytest.mark.parametrize("mode", [0, 1], ids=["general", "direct"])
+@pytest.mark.parametrize("bits,N,Ci,Co,D,H,W", S2_DIRECT_SHAPES)
+def test_stride2_kernels_exact(gpu, mode, bits, N, Ci, Co, D, H, W):
+    rng = np.random.default_rng(Ci * 31 + Co * 5 + D)
+    S = D * H * W
+    x, w, b = exact_case(rng, N, Ci, Co, S)
+    xdt = 3 if bits == 8 else 4
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    cb = 4 if bits == 4 and Ci == 32 and Co <= 32 and not (D | H | W) & 1 else 8      # the compute format the entry point picks
+    lib.mi_conv_s2_direct(mode)
+    try:
+        for ydt in (0, 2, xdt):                                   # fp32 / fp16 planes == the exact host conv; the MX output byte-identical
+            want, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=cb, stride=2, acc64=1)
+            got, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=cb, stride=2)
+            assert ("conv3s2_mx_k" in lib.mi_last_kernel().decode()) == (mode == 1), lib.mi_last_kernel().decode()
+            assert np.array_equal(got, want), ydt
+    finally:
+        lib.mi_conv_s2_direct(-1)
+
+
+def test_stride2_direct_kernel_groupnorm_input(gpu):
+    """The direct kernel behind lp_conv_fwd_s2_f8 with a GroupNorm + SiLU input (re-staged once); random data against the oracle's fp32 result."""
+    rng = np.random.default_rng(91)
+    N, Ci, Co, D, H, W, G = 2, 64, 64, 32, 32, 64, 8
+    S = D * H * W
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(8, x, N, Ci, S)
+    p = [rng.uniform(.5, 1.5, Ci).astype(np.float32), rng.uniform(-.3, .3, Ci).astype(np.float32)]
+    mean, rstd = rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.7, 1.4, N * G).astype(np.float32)
+    want, _ = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 0, cbits=8, stride=2, gp=orc.gn(p[0], p[1], mean, rstd, G), acc64=0)
+    lib.mi_conv_s2_direct(1)
+    try:
+        got, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 0, cbits=8, stride=2, gp=dev_gn(p[0], p[1], mean, rstd, G))
+    finally:
+        lib.mi_conv_s2_direct(-1)
+    assert "conv3s2_mx_k" in lib.mi_last_kernel().decode()
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-2
+
+
 @pytest.mark.parametrize("bits,N,Ci,Co,D,H,W,stride", EXACT_SHAPES)
 def test_exact_operand_conv(gpu, bits, N, Ci, Co, D, H, W, stride):
     rng = np.random.default_rng(Ci * 131 + Co * 7 + D + stride)

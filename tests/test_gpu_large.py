@@ -55,6 +55,7 @@ CONVS = [  # name, Ci, Co, dims, N, stride, bits, gn, kernel name part
     ("row", 96, 32, (8, 32, 32), 5400, 1, 8, False, "conv3_row_k"),
     ("small", 32, 32, (16, 32, 32), 8000, 1, 8, False, "conv3_small_k"),
     ("general fp4 stride 2", 64, 64, (16, 32, 32), 7800, 2, 4, False, "stride 2"),
+    ("direct fp4 stride 2", 64, 64, (16, 32, 32), 7800, 2, 4, False, "conv3s2_mx_k"),
     ("restaged GroupNorm input", 64, 64, (16, 16, 32), 8000, 1, 8, True, "conv3_"),
 ]
 
@@ -81,7 +82,11 @@ def test_conv_past_4gib(gpu, name, Ci, Co, dims, N, stride, bits, gn, kpart):
     lib.mi_gn_sums_zero(sums.ptr, 2 * N * G)
     xs = shape5(N, Ci, D, H, W)
     if stride == 2:
-        rc = lib.lp_conv_fwd_s2_f8(xin.ptr, xdt, xs, dw.ptr, db.ptr, Co, y.ptr, xdt, shape5(N, Co, Do, Ho, Wo), g)
+        lib.mi_conv_s2_direct(1 if name.startswith("direct") else 0)     # both stride-2 kernels at this size (by default the launch size picks one)
+        try:
+            rc = lib.lp_conv_fwd_s2_f8(xin.ptr, xdt, xs, dw.ptr, db.ptr, Co, y.ptr, xdt, shape5(N, Co, Do, Ho, Wo), g)
+        finally:
+            lib.mi_conv_s2_direct(-1)
         assert rc in (0, 3)
     else:
         rc = (lib.lp_conv_fwd_f8 if bits == 8 else lib.lp_conv_fwd_f4)(xin.ptr, xdt, xs, dw.ptr, db.ptr, Co, y.ptr, xdt, g, sums.ptr, G, split_t())

@@ -118,6 +118,147 @@ __global__ void __launch_bounds__(256, 2) conv2_mx_k(const conv_args a) {
     }
 }
 
+// ---- the 3x3x3 stride-2 conv (src/lp_s2.cu:4-9) read the same way: no LDS staging, every tap's rows straight from the stored tensor ----
+// A staged halo serves a stride-2 tile badly (5 x 17 x 33 positions through registers and LDS for 2 x 8 x 16 outputs), and the rows a tap needs lie
+// 64 bytes apart: the three kx taps of a wavefront's 64 consecutive output voxels together read one contiguous run of input rows, which the vector
+// cache serves line by line. Column = output voxel, K in the pair order of mi_s2_unit (the weights are prepared in the same order); unit (t, b) of a column is the row of block b at voxel (2 oz + kz - 1, 2 oy + ky - 1, 2 ox + kx - 1), zeros outside the volume.
+// The next pair's rows and weights are requested before the current pair is multiplied.
+template <int FMT, int OUT, int MT>
+__global__ void __launch_bounds__(256, MT <= 2 ? 4 : 2) conv3s2_mx_k(const conv_args a) {
+    constexpr int NT = 2, RB = fmt_t<FMT>::RB, WTILE = fmt_t<FMT>::WTILE;
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    const int n = blockIdx.z, cs = (int)blockIdx.y, nb = a.nbt;
+    const size_t Sin = (size_t)a.D * a.H * a.W;
+    const long long Scol = (long long)a.Do * a.Ho * a.Wo;
+    conv_epi_consts<MT, false>(a, lds, cs, tid);
+    // the K order as a table (after the statistics scratch): per pair and side, tap | block << 5, bit 31 set for a padding unit
+    const int np = (27 * nb + 1) >> 1;
+    int *utab = (int *)(lds + a.red_o + 1024);
+    for (int i = tid; i < 2 * np + 8; i += 256) {
+        int t = 13, b = 0;
+        const bool ok = (i >> 1) < np && mi_s2_unit(i >> 1, i & 1, nb, &t, &b);
+        utab[i] = ok ? t | (b << 5) : (int)0x80000000u | 13;
+    }
+    __syncthreads();
+    const long long ct0 = ((long long)blockIdx.x * 4 + wave) * NT;
+    if (ct0 * 32 >= Scol) return;                            // (no barrier follows)
+    // the lane's column of each tile: the input voxel of the centre tap and, per dimension, which of the offsets -1, 0, +1 stay inside the volume
+    long long ivc[NT]; unsigned vm[NT]; bool cok[NT];
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        const long long col = (ct0 + j) * 32 + r;
+        cok[j] = col < Scol;
+        const long long cc = cok[j] ? col : 0;
+        const int ox = (int)(cc % a.Wo), oy = (int)(cc / a.Wo % a.Ho), oz = (int)(cc / ((long long)a.Wo * a.Ho));
+        ivc[j] = ((long long)(2 * oz) * a.H + 2 * oy) * a.W + 2 * ox;
+        unsigned m = 0;
+#pragma unroll
+        for (int d = 0; d < 3; d++) {
+            m |= ((unsigned)(2 * oz + d - 1) < (unsigned)a.D ? 1u : 0u) << d;
+            m |= ((unsigned)(2 * oy + d - 1) < (unsigned)a.H ? 1u : 0u) << (3 + d);
+            m |= ((unsigned)(2 * ox + d - 1) < (unsigned)a.W ? 1u : 0u) << (6 + d);
+        }
+        vm[j] = cok[j] ? m : 0u;
+    }
+    const uint8_t *xq[2] = {a.xq[0], a.xq[1]}, *xsc[2] = {a.xsc[0], a.xsc[1]};
+    struct bfrag { v4i lo, hi; int sb; };
+    struct unit_t { const uint8_t *q, *sc; long long off; unsigned bit; };      // (uniform) rows and scale bytes of the unit's block, voxel offset from the centre tap, validity bits
+    auto unit = [&](int p, int side) {
+        unit_t q;
+        const int e = __builtin_amdgcn_readfirstlane(utab[2 * p + side]);      // (p <= np + 3: the entries past the last pair are padding units)
+        const bool ok = e >= 0;
+        const int t = e & 31, b = (e & 0x7fffffff) >> 5;
+        const int kz = t / 9, ky = (t / 3) % 3, kx = t % 3;
+        const int seg = b >= a.nb0p, bl = seg ? b - a.nb0p : b;
+        const size_t plane = ((size_t)n * (seg ? a.nbs[1] : a.nbs[0]) + bl) * Sin;
+        q.q = (seg ? xq[1] : xq[0]) + plane * RB; q.sc = (seg ? xsc[1] : xsc[0]) + plane;
+        q.off = ((long long)(kz - 1) * a.H + (ky - 1)) * a.W + (kx - 1);
+        q.bit = ok ? (1u << kz) | (8u << ky) | (64u << kx) : 0x80000000u;      // (a padding unit, the pair past the end: never valid)
+        return q;
+    };
+    auto fetch = [&](int j, const unit_t &u0, const unit_t &u1) {
+        bfrag q;
+        const bool v0 = (vm[j] & u0.bit) == u0.bit, v1 = (vm[j] & u1.bit) == u1.bit;
+        const long long p0 = v0 ? ivc[j] + u0.off : 0, p1 = v1 ? ivc[j] + u1.off : 0;
+        const v4i z4 = {0, 0, 0, 0};
+        if constexpr (FMT == 8) {
+            q.lo = *(const v4i *)(u0.q + p0 * RB + 16 * h); q.hi = *(const v4i *)(u1.q + p1 * RB + 16 * h);
+            q.lo = v0 ? q.lo : z4; q.hi = v1 ? q.hi : z4;
+        } else {
+            q.lo = *(const v4i *)((h ? u1.q : u0.q) + (h ? p1 : p0) * RB);
+            q.lo = (h ? v1 : v0) ? q.lo : z4; q.hi = z4;
+        }
+        q.sb = h ? (v1 ? (int)u1.sc[p1] : 127) : (v0 ? (int)u0.sc[p0] : 127);      // (a row outside the volume: zero codes, scale 1)
+        return q;
+    };
+    struct afrag { v4i lo, hi; int s; };
+    auto wfetch = [&](int gp, int m) {
+        afrag q;
+        const size_t t = (size_t)gp * a.nmt_all + cs * MT + m;
+        q.lo = *(const v4i *)(a.wq + t * WTILE + lane * 16);
+        if constexpr (FMT == 8) q.hi = *(const v4i *)(a.wq + t * WTILE + 1024 + lane * 16); else q.hi = (v4i){0, 0, 0, 0};
+        q.s = *(const int *)(a.wsc + (t * 64 + lane) * 4);
+        return q;
+    };
+    v16f acc[MT][NT];
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
+    // a ring of RING register sets: the rows and weights of pairs p + 1 .. p + RING - 1 are in flight while pair p is multiplied (a wavefront has
+    // little else to hide the loads' latency behind: two MFMAs per channel tile and pair)
+    constexpr int RING = 2;                                  // (measured, 32 -> 32 from 2 x 128^3: two sets at four wavefronts per SIMD 0.071 ms, four sets at three 0.075 ms)
+    bfrag fb[RING][NT]; afrag fa[RING][MT];
+    auto request = [&](int p, auto SET) {
+        constexpr int set = decltype(SET)::value;
+        const unit_t u0 = unit(p, 0), u1 = unit(p, 1);
+#pragma unroll
+        for (int j = 0; j < NT; j++) fb[set][j] = fetch(j, u0, u1);
+#pragma unroll
+        for (int m = 0; m < MT; m++) fa[set][m] = wfetch(p, m);
+    };
+    auto multiply = [&](auto SET) {
+        constexpr int set = decltype(SET)::value;
+#pragma unroll
+        for (int m = 0; m < MT; m++)
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                const v8i A = {fa[set][m].lo[0], fa[set][m].lo[1], fa[set][m].lo[2], fa[set][m].lo[3], fa[set][m].hi[0], fa[set][m].hi[1], fa[set][m].hi[2], fa[set][m].hi[3]};
+                const v8i B = {fb[set][j].lo[0], fb[set][j].lo[1], fb[set][j].lo[2], fb[set][j].lo[3], fb[set][j].hi[0], fb[set][j].hi[1], fb[set][j].hi[2], fb[set][j].hi[3]};
+                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A, B, acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, fa[set][m].s, 0, fb[set][j].sb);
+            }
+    };
+    static_for<RING - 1>([&](auto I) { request(decltype(I)::value, I); });
+    for (int p = 0; p < np; p += RING) {                     // (pairs past the last one are padding units with zero weights; their products are never formed)
+        static_for<RING>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            if (p + i < np) {                                // (uniform)
+                request(p + i + RING - 1, std::integral_constant<int, (i + RING - 1) % RING>{});
+                multiply(I);
+            }
+        });
+    }
+    long long ovx[NT];
+#pragma unroll
+    for (int j = 0; j < NT; j++) ovx[j] = cok[j] ? (ct0 + j) * 32 + r : -1;
+    conv_epilogue<MT, NT, OUT, false, false, false, false, true, 4, true>(a, acc, lds, 0u, n, cs, 0, 0, 0, 0, 0, tid, ovx);
+}
+
+template <int FMT, int OUT, int MT>
+static void launch_conv3s2_mt(const conv_args &a, dim3 grid, size_t smem) {
+    conv3s2_mx_k<FMT, OUT, MT><<<grid, 256, smem>>>(a);
+    MICK();
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3s2_mx_k<fmt %d, out %d, MT %d> blocks %d grid %u x %u x %u", FMT, OUT, MT, a.nbt, grid.x, grid.y, grid.z);
+}
+template <int FMT>
+static void launch_conv3s2(int out, int MT, const conv_args &a, dim3 grid, size_t smem) {
+#define C3S2_MT(OUT) do { if (MT == 4) launch_conv3s2_mt<FMT, OUT, 4>(a, grid, smem); else if (MT == 2) launch_conv3s2_mt<FMT, OUT, 2>(a, grid, smem); else launch_conv3s2_mt<FMT, OUT, 1>(a, grid, smem); } while (0)
+    if (out == 8) C3S2_MT(8); else if (out == 4) C3S2_MT(4); else C3S2_MT(0);
+#undef C3S2_MT
+}
 template <int FMT, int OUT, bool UP, int MT>
 static void launch_conv2_mt(const conv_args &a, dim3 grid, size_t smem) {
     conv2_mx_k<FMT, OUT, UP, MT><<<grid, 256, smem>>>(a);

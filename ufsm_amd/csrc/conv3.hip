@@ -93,10 +93,12 @@ __global__ void __launch_bounds__(128) prep_w_k(const float *__restrict__ w, uin
         const int u = 2 * q + side;
         float v[32];
         // K order inside a chunk: tap by tap over its blocks, or (the wide kernel, one chunk) block by block over the taps; the row kernel
-        // (block_major < 0): per block 15 pairs (class c, ky), class c < 3 = taps (c, ky, 0 | 1), class 3 = (0 | 1, ky, 2), class 4 = (2, ky, 2 | none)
+        // (block_major -1): per block 15 pairs (class c, ky), class c < 3 = taps (c, ky, 0 | 1), class 3 = (0 | 1, ky, 2), class 4 = (2, ky, 2 | none);
+        // the direct stride-2 kernel (block_major -2): mi_s2_unit
         int t = block_major ? u % 27 : u / nbc, blk = block_major ? u / 27 : b0 + u % nbc;
         bool unit_ok = u < 27 * nbc;
-        if (block_major < 0) {
+        if (block_major == -2) unit_ok = mi_s2_unit(gp, side, nbt, &t, &blk);
+        else if (block_major < 0) {
             const int qq = gp % 15, c = qq / 3, ky = qq % 3;
             blk = gp / 15;
             const int kz = c < 3 ? c : c == 3 ? side : 2, kx = c < 3 ? side : 2;
@@ -247,6 +249,8 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
 static thread_local const uint8_t *g_static_zpage = nullptr;     // the constant page of the calling thread's conv when it runs on the fixed scratch
 static thread_local int g_split = -1;       // mi_conv_split: the calling thread's tile count below which 128-channel slices are halved (-1: the default)
 extern "C" void mi_conv_split(int tiles) { g_split = tiles; }
+static thread_local int g_s2d = -1;         // mi_conv_s2_direct: the calling thread's choice of stride-2 kernel (-1: by launch size)
+extern "C" void mi_conv_s2_direct(int mode) { g_s2d = mode; }
 static int split_s2_env() { static int v = -1; if (v < 0) v = getenv("MI_CONV_SPLIT_S2") ? atoi(getenv("MI_CONV_SPLIT_S2")) : 1; return v; }      // tuning knob: 0 keeps four channel tiles
 static int conv_dispatch(const char *who, int fmt, int stride, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                          gnp_t gp, double *osum, int Go, split_t sp, const float *ep_a, const float *ep_b, int act) {
@@ -341,6 +345,19 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 1) / 2) * (nmt_all / MT) * N < 256) NT = 1;
     // ... and still fewer one-plane tiles than half the CUs: two channel tiles per workgroup instead of four
     if (stride == 2 && MT == 4 && NT == 1 && split_s2_env() && (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * Do * (nmt_all / 4) * N < 128) MT = 2;
+    // stride 2 on 32-channel rows with enough output voxels (four workgroups per CU or more): the kernel that reads every tap's rows straight from
+    // the stored tensor (no staged halo). Measured in the 32/64/128/256 forward at 2 x 128^3: 32 -> 32 from 128^3 0.093 -> 0.071 ms; 64 -> 64 from
+    // 64^3 is slower there, 0.030 -> 0.037 ms, and stays with the general kernel. Runs of 64 output voxels per wavefront; channel tiles per
+    // workgroup halved while fewer than two workgroups per CU would run
+    static int s2d_env = -1;
+    if (s2d_env < 0) s2d_env = getenv("MI_CONV_S2D") ? atoi(getenv("MI_CONV_S2D")) : 1;       // tuning knob: 0 keeps the general kernel for stride 2
+    const size_t s2runs = ((size_t)Do * Ho * Wo + 63) / 64;
+    const bool s2d = s2d_env && g_s2d != 0 && stride == 2 && a.wide && !act && N <= 65535 && (g_s2d > 0 || (s2runs + 3) / 4 * N >= (size_t)s2d_env * 1024);
+    if (s2d) {
+        MT = nmt_all % 4 == 0 ? 4 : nmt_all % 2 == 0 ? 2 : 1;
+        while (MT > 1 && (s2runs + 3) / 4 * (size_t)(nmt_all / MT) * N < 512) MT >>= 1;
+        NT = 2;
+    }
     // 128-channel output slices at stride 1 take the wide kernel (16 accumulators per wavefront, one workgroup per CU)
     static int big_env = -1;
     if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel, 2 sends every 64-channel layer to the wide kernel too
@@ -380,21 +397,23 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (cb_env > 0 && cb_env <= cb1) cbmax = cb_env;
     if (cbmax < 1) mi_die("%s: tile does not fit LDS", who);
     const int nchunks = (a.nbt + cbmax - 1) / cbmax;
-    a.CB = big ? a.nbt : (a.nbt + nchunks - 1) / nchunks; // (the wide kernel has no chunks: its K loop walks block by block)
+    a.CB = big || s2d ? a.nbt : (a.nbt + nchunks - 1) / nchunks; // (the wide kernel has no chunks: its K loop walks block by block; the direct stride-2 kernel: one chunk, tap-major)
     static int areg_env = -1;
     if (areg_env < 0) areg_env = getenv("MI_CONV_AREG") ? atoi(getenv("MI_CONV_AREG")) : 1;      // tuning knob: 0 keeps the general kernel for every shape
-    a.areg = areg_env && !big && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && a.nbt == 1 && a.wide && (NT == 2 || NT == 4);
+    a.areg = areg_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && a.nbt == 1 && a.wide && (NT == 2 || NT == 4);
     // one channel tile of 17 .. 32 output channels from two or more input blocks on a volume wider than one 16-voxel tile: the row kernel (runs
     // of 32 voxels along x, input fragments shared by the three ky taps). One input block stays with the kernel that keeps its weights in
     // registers, which measures a few percent faster there (both are bound by the halo's cache misses in flight, and it loads no weights)
     static int row_env = -1;
     if (row_env < 0) row_env = getenv("MI_CONV_ROW") ? atoi(getenv("MI_CONV_ROW")) : 1;      // tuning knob: 0 keeps the other kernels for these shapes, 2 also takes one input block
-    a.row = row_env && !big && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 ? 1 : 2) && a.nbt <= 64;
+    a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 ? 1 : 2) && a.nbt <= 64;
     if (a.row) { a.areg = false; a.CB = a.nbt; }
     size_t smem = a.row ? (size_t)2 * 2048 * (RB + 4) : a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
+    if (s2d) smem = 0;
     smem = (smem + 15) & ~(size_t)15;
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);      // bias, affine a, b of the workgroup's channels
     a.red_o = (unsigned)smem; smem += 1024;                                     // statistics scratch
+    if (s2d) smem += (size_t)(27 * a.nbt + 1 + 8) * sizeof(int);                // the direct stride-2 kernel's K-order table
     if (big || a.areg || a.row) {
         // rows and scale bytes of positions outside the volume: 64 zero bytes, then 64 bytes of value 1; one page per device, kept for the process
         // (the entry point that must not allocate keeps its own at the head of its fixed scratch)
@@ -430,20 +449,20 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (sp.wkey && !mi_ws_arena_on()) {
         std::lock_guard<std::mutex> lk(g_wmemo_mu);
         for (auto &m : g_wmemo)
-            if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == memoCB && m.nmt_all == nmt_all && m.dev == dev && m.lay == (big ? MT : a.row ? 100 : 0)) { wq = m.wq; wsc = m.wsc; have = true; break; }
+            if (m.key == sp.wkey && m.w == w && m.fmt == fmt && m.Co == cout && m.Ci == Ci && m.Cx == Cx && m.nbt == a.nbt && m.CB == memoCB && m.nmt_all == nmt_all && m.dev == dev && m.lay == (big ? MT : a.row ? 100 : s2d ? 200 : 0)) { wq = m.wq; wsc = m.wsc; have = true; break; }
         if (!have) {
             MIRT(hipMalloc((void **)&wq, wq_bytes)); MIRT(hipMalloc((void **)&wsc, wsc_bytes)); mi_count_alloc(); mi_count_alloc();
             if (!wq || !wsc) mi_die("%s: no device memory for the prepared weights", who);
             MIRT(hipMemsetAsync(wq, 0, wq_bytes, 0)); MIRT(hipMemsetAsync(wsc, 0, wsc_bytes, 0));
-            g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, memoCB, nmt_all, dev, big ? MT : a.row ? 100 : 0, wq, wsc});
+            g_wmemo.push_back(wmemo_t{sp.wkey, w, fmt, cout, Ci, Cx, a.nbt, memoCB, nmt_all, dev, big ? MT : a.row ? 100 : s2d ? 200 : 0, wq, wsc});
         }
     } else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
     if (!have) {
         const size_t nt = (size_t)npairs_all * nmt_all * 32;
         // 2-D fp4 weight scales (lp_set_w4_2d): the stride-1 e2m1 preps of more than 16 input channels, as src/lp_f4fwd.cuh:1163
         const int w2d = g_w2d_on() && fmt == 4 && stride == 1 && Ci > 16;
-        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : 0, 0);
-        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : 0, w2d);
+        if (fmt == 8) prep_w_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : s2d ? -2 : 0, 0);
+        else prep_w_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, Cx, CxP, a.nbt, a.CB, nmt_all, npairs_all, big ? MT : a.row ? -1 : s2d ? -2 : 0, w2d);
         MICK();
     }
     a.wq = wq; a.wsc = wsc;
@@ -454,7 +473,10 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     const bool ktime = g_ktime && !mi_ws_arena_on();
     if (ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
-    if (fmt == 8) { if (out == 8) conv3_launch_f8_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f8_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f8_o0(stride, epi, MT, NT, a, smem); }
+    if (s2d) {
+        const dim3 grid((unsigned)((s2runs + 3) / 4), (unsigned)a.ncs, (unsigned)N);
+        if (fmt == 8) conv3s2_launch_f8(out, MT, a, grid, smem); else conv3s2_launch_f4(out, MT, a, grid, smem);
+    } else if (fmt == 8) { if (out == 8) conv3_launch_f8_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f8_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f8_o0(stride, epi, MT, NT, a, smem); }
     else { if (out == 8) conv3_launch_f4_o8(stride, epi, MT, NT, a, smem); else if (out == 4) conv3_launch_f4_o4(stride, epi, MT, NT, a, smem); else conv3_launch_f4_o0(stride, epi, MT, NT, a, smem); }
     if (ktime) { MIRT(hipEventRecord(ev1, 0)); ktime_push(ev0, ev1, 2.0 * 27 * Ci * (double)cout * N * Do * Ho * Wo); }
     if (osum) conv_stats_reduce(who, a, MT, sp, osum);

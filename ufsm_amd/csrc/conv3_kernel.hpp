@@ -651,6 +651,20 @@ static void launch_out(int stride, bool epi, int MT, int NT, const conv_args &a,
 
 
 // one translation unit per (compute format, output kind) instantiates its kernels behind this entry
+// K order of the direct stride-2 kernel. The rows of taps kx = 0 and kx = 1 of a column are neighbours in memory (voxels 2 ox - 1, 2 ox), so they
+// form a pair: its two loads read whole cache lines. Rows (kz, ky) are taken two at a time: per row and block the pair (kx 0 | kx 1), then the
+// kx = 2 units of both rows, block after block, in pairs of their own (their lines were fetched by the pairs just before). nb blocks:
+// 3 nb pairs per two rows, the ninth row nb + ceil(nb / 2); ceil(27 nb / 2) pairs in all. Returns whether the unit exists (else: padding).
+__host__ __device__ __forceinline__ bool mi_s2_unit(int gp, int side, int nb, int *tap, int *blk) {
+    const int G = gp < 12 * nb ? gp / (3 * nb) : 4, q = gp - G * 3 * nb, nrow = G < 4 ? 2 : 1;
+    int row, b, kx; bool ok = true;
+    if (q < nrow * nb) { row = 2 * G + q / nb; b = q % nb; kx = side; }
+    else { const int idx = 2 * (q - nrow * nb) + side; ok = idx < nrow * nb; const int id = ok ? idx : 0; row = 2 * G + id / nb; b = id % nb; kx = 2; }
+    *tap = row * 3 + kx; *blk = b;
+    return ok;
+}
+void conv3s2_launch_f8(int out, int MT, const conv_args &a, dim3 grid, size_t smem);      // (the direct stride-2 kernel: conv2_kernel.hpp)
+void conv3s2_launch_f4(int out, int MT, const conv_args &a, dim3 grid, size_t smem);
 #define CONV3_LAUNCH_DECL(FMT, OUT) void conv3_launch_f##FMT##_o##OUT(int stride, bool epi, int MT, int NT, const conv_args &a, size_t smem)
 CONV3_LAUNCH_DECL(8, 8); CONV3_LAUNCH_DECL(8, 4); CONV3_LAUNCH_DECL(8, 0);
 CONV3_LAUNCH_DECL(4, 8); CONV3_LAUNCH_DECL(4, 4); CONV3_LAUNCH_DECL(4, 0);
