@@ -10,8 +10,9 @@
 // from the staged tile [position][CP bytes] at the taps' offsets. The weights' fragments stay in registers. Epilogue: conv_epilogue.
 #include "conv3_kernel.hpp"
 
-template <int CP, int MT, int OUT>
-__global__ void __launch_bounds__(256, MT == 1 ? 3 : 2) conv3_stem_k(const conv_args a) {
+// PL: the input is fp32 / fp16 planes (else an MX tensor): a template parameter so that the path not taken holds no registers
+template <int CP, int MT, int OUT, bool PL>
+__global__ void __launch_bounds__(256, MT == 1 ? (CP == 8 ? 4 : 3) : (CP == 8 ? 3 : 2)) conv3_stem_k(const conv_args a) {
     constexpr int TPK = 32 / CP, NKB = (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2, NT = 2;
     constexpr int HY = 10, HX = 18, TT = 4 * HY * HX, WTILE = 2048;
     extern __shared__ __align__(16) unsigned char lds[];
@@ -86,7 +87,7 @@ __global__ void __launch_bounds__(256, MT == 1 ? 3 : 2) conv3_stem_k(const conv_
             }
         }
     };
-    const bool planes = xdt < 3;
+    constexpr bool planes = PL;
     constexpr bool PFP = CP <= 4;                            // plane inputs are requested a tile ahead only where the registers allow it
     float pv[3][PFP ? CP : 1];                               // plane inputs (fp32, or fp16 widened): the values themselves
     auto plane_vals = [&](int tz, int j, float *dst) __attribute__((always_inline)) {       // position j's CP plane values of tile tz
@@ -421,7 +422,9 @@ void conv3_stem_prep(int CP, const float *w, uint8_t *wq, uint8_t *wsc, int Co, 
 template <int CP, int MT, int OUT>
 static void launch_stem(const conv_args &a, size_t smem) {
     const unsigned per = (a.ngrp + 7u) / 8u;
-    conv3_stem_k<CP, MT, OUT><<<per * 8u, 256, smem>>>(a);
+    if (a.sxdt < 3) conv3_stem_k<CP, MT, OUT, true><<<per * 8u, 256, smem>>>(a);
+    else if constexpr (CP <= 8) conv3_stem_k<CP, MT, OUT, false><<<per * 8u, 256, smem>>>(a);
+    else mi_die("conv3 stem: 16-channel rows are fp32 planes");
     MICK();
     snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_stem_k<CP %d, MT %d, out %d> tiles %u", CP, MT, OUT, a.ntiles);
 }
