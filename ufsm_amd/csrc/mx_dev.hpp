@@ -170,9 +170,33 @@ __device__ __forceinline__ unsigned d_quant_row(const float *v, int bw, unsigned
     return (unsigned)(e + 127);
 }
 // decode a row held in words (8 words fp8 / 4 words fp4) times the scale
+// The converting instructions take the scale as an operand: checked on the device over every code and scale byte, their result equals
+// decode x d_mx_scale(sbyte) bit for bit for the scale bytes 1 .. 254 (subnormal and overflowing products included) and differs for 0 (the
+// reference's scale is 0.0 there, the instruction's 2^-127) and 255 (inf against NaN). Wavefronts that hold neither byte take the one-instruction
+// form; the others decode and multiply.
+__device__ __forceinline__ bool d_scale_plain(unsigned sbyte) { return __builtin_amdgcn_ballot_w64(((sbyte + 1u) & 255u) < 2u) == 0ull; }
+__device__ __forceinline__ void d_dec4_e4m3_scaled(unsigned w, float s, float *v) {
+    const mi_v2f lo = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(w, s, false), hi = __builtin_amdgcn_cvt_scalef32_pk_f32_fp8(w, s, true);
+    v[0] = lo[0]; v[1] = lo[1]; v[2] = hi[0]; v[3] = hi[1];
+}
+__device__ __forceinline__ void d_dec8_e2m1_scaled(unsigned w, float s, float *v) {
+    const mi_v2f a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, s, 0), b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, s, 1);
+    const mi_v2f c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, s, 2), d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, s, 3);
+    v[0] = a[0]; v[1] = a[1]; v[2] = b[0]; v[3] = b[1]; v[4] = c[0]; v[5] = c[1]; v[6] = d[0]; v[7] = d[1];
+}
 template <int BITS>
 __device__ __forceinline__ void d_dequant_row(const unsigned *codes, unsigned sbyte, float *v) {
     const float s = d_mx_scale(sbyte);
+    if (d_scale_plain(sbyte)) {
+        if (BITS == 8) {
+#pragma unroll
+            for (int j = 0; j < 8; j++) d_dec4_e4m3_scaled(codes[j], s, v + 4 * j);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; j++) d_dec8_e2m1_scaled(codes[j], s, v + 8 * j);
+        }
+        return;
+    }
     if (BITS == 8) {
 #pragma unroll
         for (int j = 0; j < 8; j++) d_dec4_e4m3(codes[j], v + 4 * j);

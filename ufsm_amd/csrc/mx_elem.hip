@@ -218,15 +218,23 @@ __global__ void __launch_bounds__(256) gn_silu_apply32_k(const uint8_t *x, uint8
     unsigned w[4] = {0u, 0u, 0u, 0u};
     if (BX == 8) { const uint4 q = *(const uint4 *)(x + row * 32 + hf * 16); w[0] = q.x; w[1] = q.y; w[2] = q.z; w[3] = q.w; }
     else { const uint2 q = *(const uint2 *)(x + row * 16 + hf * 8); w[0] = q.x; w[1] = q.y; }
-    const float sc = d_mx_scale(xs[row]);
+    const unsigned sby = xs[row];
+    const float sc = d_mx_scale(sby);
     float r[16];
-    if (BX == 8) { d_dec4_e4m3(w[0], r); d_dec4_e4m3(w[1], r + 4); d_dec4_e4m3(w[2], r + 8); d_dec4_e4m3(w[3], r + 12); }
-    else { d_dec8_e2m1(w[0], r); d_dec8_e2m1(w[1], r + 8); }
+    if (d_scale_plain(sby)) {                                 // (uniform) the conversions apply the scale
+        if (BX == 8) { d_dec4_e4m3_scaled(w[0], sc, r); d_dec4_e4m3_scaled(w[1], sc, r + 4); d_dec4_e4m3_scaled(w[2], sc, r + 8); d_dec4_e4m3_scaled(w[3], sc, r + 12); }
+        else { d_dec8_e2m1_scaled(w[0], sc, r); d_dec8_e2m1_scaled(w[1], sc, r + 8); }
+    } else {
+        if (BX == 8) { d_dec4_e4m3(w[0], r); d_dec4_e4m3(w[1], r + 4); d_dec4_e4m3(w[2], r + 8); d_dec4_e4m3(w[3], r + 12); }
+        else { d_dec8_e2m1(w[0], r); d_dec8_e2m1(w[1], r + 8); }
+#pragma unroll
+        for (int k = 0; k < 16; k++) r[k] *= sc;
+    }
     unsigned am = 0u;
 #pragma unroll
     for (int k = 0; k < 16; k++) {
         const float4 q = co[hf * 16 + k];
-        const float u = fmaf((r[k] * sc - q.x) * q.y, q.z, q.w);
+        const float u = fmaf((r[k] - q.x) * q.y, q.z, q.w);
         r[k] = d_silu(u);
         am = d_amax_u(am, r[k]);
     }
@@ -670,13 +678,17 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
         const size_t v = vb + (size_t)i * 128, row = row0 + v;
         const float sc = d_mx_scale(sby[i]);
         float r[16];
-        if (BX == 8) { d_dec4_e4m3(w[i][0], r); d_dec4_e4m3(w[i][1], r + 4); d_dec4_e4m3(w[i][2], r + 8); d_dec4_e4m3(w[i][3], r + 12); }
-        else { d_dec8_e2m1(w[i][0], r); d_dec8_e2m1(w[i][1], r + 8); }
+        if (d_scale_plain(sby[i])) {                          // (uniform) the conversions apply the scale
+            if (BX == 8) { d_dec4_e4m3_scaled(w[i][0], sc, r); d_dec4_e4m3_scaled(w[i][1], sc, r + 4); d_dec4_e4m3_scaled(w[i][2], sc, r + 8); d_dec4_e4m3_scaled(w[i][3], sc, r + 12); }
+            else { d_dec8_e2m1_scaled(w[i][0], sc, r); d_dec8_e2m1_scaled(w[i][1], sc, r + 8); }
+        } else {
+            if (BX == 8) { d_dec4_e4m3(w[i][0], r); d_dec4_e4m3(w[i][1], r + 4); d_dec4_e4m3(w[i][2], r + 8); d_dec4_e4m3(w[i][3], r + 12); }
+            else { d_dec8_e2m1(w[i][0], r); d_dec8_e2m1(w[i][1], r + 8); }
 #pragma unroll
-        for (int k = 0; k < 16; k++) {
-            const float xv = r[k] * sc;
-            r[k] = gp.G ? d_act_ab(xv, ca[k], cb[k]) : xv;
+            for (int k = 0; k < 16; k++) r[k] *= sc;
         }
+#pragma unroll
+        for (int k = 0; k < 16; k++) r[k] = gp.G ? d_act_ab(r[k], ca[k], cb[k]) : r[k];
         float am = 0.f;
 #pragma unroll
         for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(r[k]));
