@@ -137,6 +137,45 @@ def test_gn_silu_apply(gpu, xdt, yb, Cc):
     assert (np.abs(gd - wd) <= np.maximum(np.abs(wd), np.abs(gd)) * (0.26 if yb == 8 else 0.67) + 1e-30).all()
 
 
+@pytest.mark.parametrize("xb", [8, 4])
+def test_row_decode_at_the_extreme_scale_bytes(gpu, xb):
+    """Stored rows whose scale byte is 0, 1, 254 or 255 next to ordinary ones: the device decodes a row by the converting instruction with the
+    scale as its operand unless a wavefront holds byte 0 (the format's scale there is 0.0, the instruction's 2^-127) or 255 (inf against NaN),
+    which take decode x scale. MX -> fp32 planes (bit for bit, NaN for NaN) and the GroupNorm + SiLU apply of the same tensor (statistics that
+    keep the transformed values in range) against the oracle."""
+    rng = np.random.default_rng(40 + xb)
+    N, C, S = 1, 32, 4096
+    rb = 32 if xb == 8 else 16
+    codes = rng.integers(0, 256, (N, 1, S, rb), dtype=np.uint8)
+    if xb == 8:
+        codes[(codes & 0x7f) == 0x7f] = 0x3c                            # (no NaN codes: the rows' values are then finite wherever the scale is)
+    sc = rng.integers(110, 140, (N, 1, S), dtype=np.uint8)
+    sc[0, 0, 5::64] = 0; sc[0, 0, 70::64] = 1; sc[0, 0, 135::64] = 254   # each extreme byte in wavefronts of its own and ordinary wavefronts between
+    sc[0, 0, 200::128] = 255
+    xin = np.concatenate([codes.reshape(-1), sc.reshape(-1)])
+    assert xin.size == orc.mx_bytes(xb, N, C, S)
+    dq = DevBuf.from_numpy(xin)
+    df = DevBuf(N * C * S * 4)
+    (lib.lp_mx8_to_f32 if xb == 8 else lib.lp_mx4_to_f32)(dq.ptr, N, C, S, df.ptr); LP.check()
+    got, want = df.to_numpy(np.float32).reshape(N, C, S), orc.mx_to_f32(xb, xin, N, C, S)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(got[~np.isnan(got)].view(np.uint32), want[~np.isnan(want)].view(np.uint32))
+    assert np.isnan(want).any() and (want[0, :, 5] == 0).all() and np.isinf(want).any()
+    G = 8
+    gam = rng.uniform(0.5, 1.5, C).astype(np.float32); bet = rng.uniform(-.5, .5, C).astype(np.float32)
+    mean = rng.uniform(-.2, .2, N * G).astype(np.float32); rstd = rng.uniform(.8, 1.2, N * G).astype(np.float32) * 1e-3
+    g = dev_gn(gam, bet, mean, rstd, G)
+    dy = DevBuf(mx_bytes(8, N, C, S))
+    lib.lp_gn_silu_apply_mx(dq.ptr, 3 if xb == 8 else 4, shape5(N, C, S, 1, 1), G, g.gamma, g.beta, g.mean, g.rstd, dy.ptr, 3); LP.check()
+    wy = np.zeros(orc.mx_bytes(8, N, C, S), np.uint8)
+    orc.lib().orc_gn_silu_apply_mx(orc.ptr(xin), 3 if xb == 8 else 4, N, C, S, orc.gn(gam, bet, mean, rstd, G), orc.ptr(wy), 8)
+    gd, wd = orc.mx_to_f32(8, dy.to_numpy(np.uint8), N, C, S), orc.mx_to_f32(8, wy, N, C, S)
+    fin = np.isfinite(wd) & np.isfinite(gd)
+    assert np.array_equal(np.isfinite(gd).all(axis=1), np.isfinite(wd).all(axis=1))          # the same rows are non-finite
+    assert (gd[fin] != wd[fin]).mean() < 1e-3
+    assert (np.abs(gd[fin] - wd[fin]) <= np.maximum(np.abs(wd[fin]), np.abs(gd[fin])) * 0.26 + 1e-30).all()
+
+
 @pytest.mark.parametrize("xb,yb,gn,Cc,dims", [(8, 8, False, 32, (6, 6, 6)), (4, 4, False, 32, (6, 6, 6)), (8, 8, True, 32, (6, 6, 6)), (4, 8, True, 32, (6, 6, 6)),
                                               (8, 8, False, 64, (5, 7, 9)), (8, 4, False, 48, (3, 4, 11)), (8, 8, False, 16, (4, 5, 6)), (4, 4, False, 12, (3, 5, 4)), (8, 8, False, 8, (2, 3, 5)),
                                               (8, 8, True, 16, (4, 4, 6)), (4, 4, True, 8, (3, 3, 3)), (8, 8, False, 32, (1, 1, 1)), (8, 8, True, 80, (4, 6, 5))])
