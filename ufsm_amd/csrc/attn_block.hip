@@ -136,6 +136,16 @@ extern "C" void at_tok_to_cs(const float *t, float *x, int n, int C, long Sg, in
 // (slice j covers pairs 4 (j & 1) .. + 3 of axis j / 2). ----
 __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv, const float *__restrict__ qg, const float *__restrict__ kg, __half *__restrict__ out,
                                                   float *__restrict__ rq, float *__restrict__ rk, float *__restrict__ amx, long long T, int H, int S, int Hh, int W, int nreg, int rope, float lbase) {
+    // the rotary angles take few values - position along an axis x frequency - and a sine / cosine pair costs far more than the rest of a unit:
+    // a block forms the table once (the same expression the per-value form evaluates, so the same bits), positions up to RP per axis
+    constexpr int RP = 64;
+    __shared__ float2 rtab[RP * 8];
+    const int pmax = max(max(S / (Hh * W), Hh), W);         // positions along an axis: < pmax (registers included in S: an upper bound)
+    const bool tab = rope && pmax <= RP;
+    if (tab) {
+        for (int i = threadIdx.x; i < pmax * 8; i += 256) { float sn, cs; sincosf((float)(i >> 3) * exp2f(-lbase * (float)(i & 7) / 8.f), &sn, &cs); rtab[i] = make_float2(sn, cs); }
+        __syncthreads();
+    }
     const long long unit = (blockIdx.x * 256ll + threadIdx.x) >> 3; const int j = threadIdx.x & 7;
     const long long Tp = T + FT, nunits = Tp * H * 3;
     if (unit >= nunits) return;
@@ -170,7 +180,9 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
                     const int fi = 4 * (j & 1) + i;
-                    float sn, cs; sincosf(pos * exp2f(-lbase * (float)fi / 8.f), &sn, &cs);
+                    float sn, cs;
+                    if (tab) { const float2 sc2 = rtab[(int)pos * 8 + fi]; sn = sc2.x; cs = sc2.y; }
+                    else sincosf(pos * exp2f(-lbase * (float)fi / 8.f), &sn, &cs);
                     const float a = v[2 * i], b = v[2 * i + 1];
                     v[2 * i] = a * cs - b * sn; v[2 * i + 1] = a * sn + b * cs;
                 }

@@ -765,15 +765,22 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
     }
     const float smax = d_mx_scale(em);
     uint8_t *ys = y + (size_t)N * nbo * S * (BY * 4);
+    __half2 hf[H2 ? 8 : 1][4];                                // H2: the rows' values as binary16 pairs (an e4m3 value is one exactly), formed once per cell
+    if constexpr (H2) {
+#pragma unroll
+        for (int k = 0; k < 8; k++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) hf[k][i] = __floats2half2_rn(f[k][2 * i], f[k][2 * i + 1]);
+    }
 #pragma unroll
     for (int p = 0; p < 8; p++) {
         const int pz = p >> 2, py = (p >> 1) & 1, px = p & 1;                     // fine voxel 2m + 1 + p: p = 0 has its own coarse row at m, p = 1 at m + 1
         const int gz = 2 * mz + 1 + pz, gy = 2 * my + 1 + py, gx = 2 * mx + 1 + px;
         float acc[8];
         if constexpr (H2) {
-            __half hacc[8];
+            __half2 hacc[4];                                  // two channels per packed fused multiply-add: each half rounds once, as the scalar form
 #pragma unroll
-            for (int i = 0; i < 8; i++) hacc[i] = __float2half_rn(0.f);
+            for (int i = 0; i < 4; i++) hacc[i] = __floats2half2_rn(0.f, 0.f);
 #pragma unroll
             for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -781,12 +788,12 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
 #pragma unroll
                     for (int c = 0; c < 2; c++) {
                         const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);
-                        const __half w3 = __float2half_rn((a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f) * sc[k]);
+                        const __half2 w3 = __half2half2(__float2half_rn((a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f) * sc[k]));
 #pragma unroll
-                        for (int i = 0; i < 8; i++) hacc[i] = __hfma(w3, __float2half_rn(f[k][i]), hacc[i]);
+                        for (int i = 0; i < 4; i++) hacc[i] = __hfma2(w3, hf[k][i], hacc[i]);
                     }
 #pragma unroll
-            for (int i = 0; i < 8; i++) acc[i] = __half2float(hacc[i]) * smax;
+            for (int i = 0; i < 4; i++) { acc[2 * i] = __low2float(hacc[i]) * smax; acc[2 * i + 1] = __high2float(hacc[i]) * smax; }
         } else {
 #pragma unroll
         for (int i = 0; i < 8; i++) acc[i] = 0.f;
