@@ -148,57 +148,69 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
     }
     const long long unit = (blockIdx.x * 256ll + threadIdx.x) >> 3; const int j = threadIdx.x & 7;
     const long long Tp = T + FT, nunits = Tp * H * 3;
-    if (unit >= nunits) return;
-    const int h = (int)(unit % H); const long long tp = unit / H; const int p = (int)(tp % 3); const long long t = tp / 3;      // units of a token are neighbours: its 3 H x 192 bytes are read together
-    const int C = H * HD;
-    __half *dst = out + (((size_t)p * H + h) * Tp + t) * HD + 8 * j;
-    if (t >= T) { if (j < 6) *(uint4 *)dst = make_uint4(0u, 0u, 0u, 0u); return; }
-    float v[8];
-    if (j < 6) {
-        const float4 *xs = (const float4 *)(qkv + t * 3 * C + p * C + h * HD + 8 * j);
-        const float4 a = xs[0], b = xs[1];
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    } else {
+    // the largest |v| of the call: per unit over its lanes, per block through one LDS word, one global atomic per block (one per unit made
+    // 10^5 atomics on one address the kernel's whole run time)
+    __shared__ unsigned bmax;
+    if (threadIdx.x == 0) bmax = 0u;
+    __syncthreads();
+    if (unit < nunits) {
+        const int h = (int)(unit % H); const long long tp = unit / H; const int p = (int)(tp % 3); const long long t = tp / 3;      // units of a token are neighbours: its 3 H x 192 bytes are read together
+        const int C = H * HD;
+        __half *dst = out + (((size_t)p * H + h) * Tp + t) * HD + 8 * j;
+        if (t >= T) { if (j < 6) *(uint4 *)dst = make_uint4(0u, 0u, 0u, 0u); }
+        else {
+            float v[8];
+            if (j < 6) {
+                const float4 *xs = (const float4 *)(qkv + t * 3 * C + p * C + h * HD + 8 * j);
+                const float4 a = xs[0], b = xs[1];
+                v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+            } else {
 #pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = 0.f;
-    }
-    if (p < 2) {
-        float ss = 0.f;
+                for (int i = 0; i < 8; i++) v[i] = 0.f;
+            }
+            if (p < 2) {
+                float ss = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; i++) ss = fmaf(v[i], v[i], ss);
-        ss += __shfl_xor(ss, 1); ss += __shfl_xor(ss, 2); ss += __shfl_xor(ss, 4);
-        const float r = 1.f / sqrtf(ss / HD + 1e-6f);
-        if (j == 0) (p ? rk : rq)[t * H + h] = r;
-        if (j < 6) {
-            const float *gs = (p ? kg : qg) + h * HD + 8 * j;      // (the gains sit at an arbitrary offset of the flat parameter vector: dword loads)
+                for (int i = 0; i < 8; i++) ss = fmaf(v[i], v[i], ss);
+                ss += __shfl_xor(ss, 1); ss += __shfl_xor(ss, 2); ss += __shfl_xor(ss, 4);
+                const float r = 1.f / sqrtf(ss / HD + 1e-6f);
+                if (j == 0) (p ? rk : rq)[t * H + h] = r;
+                if (j < 6) {
+                    const float *gs = (p ? kg : qg) + h * HD + 8 * j;      // (the gains sit at an arbitrary offset of the flat parameter vector: dword loads)
 #pragma unroll
-            for (int i = 0; i < 8; i++) v[i] *= r * gs[i];
-            const int ts = (int)(t % S) - nreg;
-            if (rope && ts >= 0) {
-                const int ax = j >> 1;
-                const float pos = ax == 0 ? (float)(ts / (Hh * W)) : ax == 1 ? (float)((ts / W) % Hh) : (float)(ts % W);
+                    for (int i = 0; i < 8; i++) v[i] *= r * gs[i];
+                    const int ts = (int)(t % S) - nreg;
+                    if (rope && ts >= 0) {
+                        const int ax = j >> 1;
+                        const float pos = ax == 0 ? (float)(ts / (Hh * W)) : ax == 1 ? (float)((ts / W) % Hh) : (float)(ts % W);
 #pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int fi = 4 * (j & 1) + i;
-                    float sn, cs;
-                    if (tab) { const float2 sc2 = rtab[(int)pos * 8 + fi]; sn = sc2.x; cs = sc2.y; }
-                    else sincosf(pos * exp2f(-lbase * (float)fi / 8.f), &sn, &cs);
-                    const float a = v[2 * i], b = v[2 * i + 1];
-                    v[2 * i] = a * cs - b * sn; v[2 * i + 1] = a * sn + b * cs;
+                        for (int i = 0; i < 4; i++) {
+                            const int fi = 4 * (j & 1) + i;
+                            float sn, cs;
+                            if (tab) { const float2 sc2 = rtab[(int)pos * 8 + fi]; sn = sc2.x; cs = sc2.y; }
+                            else sincosf(pos * exp2f(-lbase * (float)fi / 8.f), &sn, &cs);
+                            const float a = v[2 * i], b = v[2 * i + 1];
+                            v[2 * i] = a * cs - b * sn; v[2 * i + 1] = a * sn + b * cs;
+                        }
+                    }
                 }
+            } else {
+                float m = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
+                m = fmaxf(m, __shfl_xor(m, 1)); m = fmaxf(m, __shfl_xor(m, 2)); m = fmaxf(m, __shfl_xor(m, 4));
+                if (j == 0) atomicMax(&bmax, __float_as_uint(m));               // (non-negative floats order as their bit patterns)
+            }
+            if (j < 6) {
+                const __half2 h0 = __floats2half2_rn(v[0], v[1]), h1 = __floats2half2_rn(v[2], v[3]), h2 = __floats2half2_rn(v[4], v[5]), h3 = __floats2half2_rn(v[6], v[7]);
+                *(uint4 *)dst = make_uint4(*(const unsigned *)&h0, *(const unsigned *)&h1, *(const unsigned *)&h2, *(const unsigned *)&h3);
             }
         }
-    } else {
-        float m = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
-        m = fmaxf(m, __shfl_xor(m, 1)); m = fmaxf(m, __shfl_xor(m, 2)); m = fmaxf(m, __shfl_xor(m, 4));
-        if (j == 0) atomicMax((unsigned *)amx + 1, __float_as_uint(m));     // (non-negative floats order as their bit patterns)
     }
-    if (j < 6) {
-        const __half2 h0 = __floats2half2_rn(v[0], v[1]), h1 = __floats2half2_rn(v[2], v[3]), h2 = __floats2half2_rn(v[4], v[5]), h3 = __floats2half2_rn(v[6], v[7]);
-        *(uint4 *)dst = make_uint4(*(const unsigned *)&h0, *(const unsigned *)&h1, *(const unsigned *)&h2, *(const unsigned *)&h3);
-    }
+    __syncthreads();
+    // (the running maximum only grows: a block whose own maximum does not exceed the value it reads has nothing to add, which spares the
+    // single address all but a few of the 10^4 blocks' atomics)
+    if (threadIdx.x == 0 && bmax > *(volatile unsigned *)((unsigned *)amx + 1)) atomicMax((unsigned *)amx + 1, bmax);
 }
 __global__ void at_zero4_k(float *p) { if (threadIdx.x < 4) p[threadIdx.x] = 0.f; }
 extern "C" void at_fa_pack(const float *qkv, const float *qg, const float *kg, void *qkvh, float *rq, float *rk, float *amx, const at_geom *g, int nreg, int C, int rope, float base) {
