@@ -53,14 +53,23 @@ __global__ void __launch_bounds__(256) ct_window_k(const uint8_t *__restrict__ v
     const uint8_t *src = vol + ((size_t)(rowin ? gz : 0) * Y + (rowin ? gy : 0)) * X;
     unsigned found = 0u;
     uint8_t *dst = win + ((size_t)z * W + y) * W + xc * 16;
-    for (int k = 0; k < 16 && xc * 16 + k < W; k++) {
-        const long long gx = ox + xc * 16 + k;
-        const uint8_t v = rowin && gx >= 0 && gx < X ? src[gx] : (uint8_t)0;
-        dst[k] = v;
+    const bool core_zy = z >= halo && z < W - halo && y >= halo && y < W - halo;
+    unsigned wd[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
         const int xw = xc * 16 + k;
-        found |= v >= iso && z >= halo && z < W - halo && y >= halo && y < W - halo && xw >= halo && xw < W - halo;
+        const long long gx = ox + xw;
+        const unsigned v = rowin && xw < W && gx >= 0 && gx < X ? (unsigned)src[gx] : 0u;
+        wd[k >> 2] |= v << (8 * (k & 3));
+        found |= (int)v >= iso && core_zy && xw >= halo && xw < W - halo;
     }
-    if (any && found) atomicOr(any, 1u);
+    if (xc * 16 + 16 <= W && (W & 15) == 0) *(uint4 *)dst = make_uint4(wd[0], wd[1], wd[2], wd[3]);      // (rows of a multiple of 16 voxels: 16-byte aligned)
+    else for (int k = 0; k < 16 && xc * 16 + k < W; k++) dst[k] = (uint8_t)(wd[k >> 2] >> (8 * (k & 3)));
+    // the flag only ever becomes 1: one atomic per wavefront that found material, and none once the flag reads set (a window of material made
+    // every thread's atomic queue on the one address)
+    if (any && __builtin_amdgcn_ballot_w64(found != 0u) != 0ull) {
+        if ((threadIdx.x & 63) == __builtin_ctzll(__builtin_amdgcn_ballot_w64(true)) && *(volatile unsigned *)any == 0u) atomicOr(any, 1u);
+    }
 }
 extern "C" void mi_ct_window(const uint8_t *vol, int64_t Z, int64_t Y, int64_t X, int64_t oz, int64_t oy, int64_t ox, int W, uint8_t *win, int iso, int halo, unsigned *any) {
     if (W <= 0) return;
