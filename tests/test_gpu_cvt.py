@@ -261,7 +261,10 @@ def test_gn_sums_and_finalize(gpu, bits, Cc, G):
     assert (dd.to_numpy(np.float64) == 0).all()
 
 
-@pytest.mark.parametrize("bits,Ci,Co,gn,h16", [(8, 16, 1, False, False), (8, 32, 8, True, False), (4, 32, 11, True, False), (8, 64, 8, False, True), (8, 32, 20, True, False)])
+# (34 and 70 input channels: a whole 32-channel block, which takes the kernel's straight-line form, followed by a ragged one, with channel counts that
+# are not multiples of 4 and output groups of 2 and 1 channels)
+@pytest.mark.parametrize("bits,Ci,Co,gn,h16", [(8, 16, 1, False, False), (8, 32, 8, True, False), (4, 32, 11, True, False), (8, 64, 8, False, True), (8, 32, 20, True, False),
+                                              (8, 34, 3, False, False), (4, 70, 5, False, False)])
 def test_head(gpu, bits, Ci, Co, gn, h16):
     rng = np.random.default_rng(9)
     N, D, H, W, G = 2, 5, 6, 7, 8

@@ -507,7 +507,7 @@ __global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const flo
                                                   size_t vb, size_t nv, size_t ly) {
     extern __shared__ __align__(16) float c1s[];          // [Ci][CO] weights (input-channel major: a channel's CO weights are one or two 16-byte reads at an
                                                           // immediate offset from the block's base), [CO] bias, [Ci] a, [Ci] b
-    float *sw = c1s, *sb = sw + CO * Ci, *sa = sb + 8, *sbb = sa + ((Ci + 3) & ~3);      // (every array starts on 16 bytes when Ci is a multiple of 4; the fast path needs Ci % 32 == 0)
+    float *sw = c1s, *sb = sw + ((CO * Ci + 3) & ~3), *sa = sb + 8, *sbb = sa + ((Ci + 3) & ~3);      // (every array starts on 16 bytes: the fast path reads 16-byte vectors of sw, sa and sbb)
     const int n = blockIdx.y, bw = mx_bw(Ci), nb = mx_nb(Ci);
     for (int i = threadIdx.x; i < CO * Ci; i += 256) { const int co = co0 + i % CO, ci = i / CO; sw[i] = co < Co ? w[(size_t)co * Ci + ci] : 0.f; }
     for (int i = threadIdx.x; i < CO; i += 256) sb[i] = b && co0 + i < Co ? b[co0 + i] : 0.f;
