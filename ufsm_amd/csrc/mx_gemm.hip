@@ -16,11 +16,18 @@ template <int BITS, int TR>
 __global__ void __launch_bounds__(256) mx_pack_k(const float *__restrict__ X, int ld, int rows, int K, int nkb, uint8_t *__restrict__ q, uint8_t *__restrict__ sc) {
     constexpr int BPB = BITS == 8 ? 32 : 16;
     const long long nblk = (long long)rows * nkb;
+    const bool v4 = (ld & 3) == 0 && ((size_t)X & 15) == 0;     // rows start on 16 bytes
     for (long long b = blockIdx.x * (long long)blockDim.x + threadIdx.x; b < nblk; b += (long long)gridDim.x * blockDim.x) {
         const int r = TR ? (int)(b % rows) : (int)(b / nkb), kb = TR ? (int)(b / rows) : (int)(b % nkb);
         float v[32];
+        if (!TR && v4 && kb * 32 + 32 <= K) {                // a whole block of a row-major operand: eight 16-byte loads (a lane's 128 bytes are contiguous)
+            const float4 *p4 = (const float4 *)(X + (size_t)r * ld + kb * 32);
 #pragma unroll
-        for (int j = 0; j < 32; j++) { const int k = kb * 32 + j; v[j] = k < K ? (TR ? X[(size_t)k * ld + r] : X[(size_t)r * ld + k]) : 0.f; }
+            for (int j = 0; j < 8; j++) { const float4 t = p4[j]; v[4 * j] = t.x; v[4 * j + 1] = t.y; v[4 * j + 2] = t.z; v[4 * j + 3] = t.w; }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 32; j++) { const int k = kb * 32 + j; v[j] = k < K ? (TR ? X[(size_t)k * ld + r] : X[(size_t)r * ld + k]) : 0.f; }
+        }
         unsigned codes[8];
         const unsigned sb = d_quant_row<BITS, false>(v, 32, codes);
         uint8_t *o = q + ((size_t)r * nkb + kb) * BPB;
