@@ -41,19 +41,20 @@ __global__ void gemm_zero_k(float *c, size_t n) {
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) c[i] = 0.f;
 }
 
-// C tile of 128 x 128 per workgroup, 64 x 64 per wavefront = 2 x 2 MFMA tiles of 32 x 32; K in steps of 64 = the two 32-K blocks the
+// C tile of 64 x 256 per workgroup (four wavefronts side by side along N), 64 x 64 per wavefront = 2 x 2 MFMA tiles of 32 x 32; K in steps of 64 = the two 32-K blocks the
 // scale operands of the lane halves of a 32x32x64 MFMA cover. A lane's fragment is 16 bytes of each of the two blocks (e4m3: bytes
 // 16 h ... of both; e2m1: all 16 bytes of block h), so fragments are loaded from the packed rows in global memory directly: the four
-// wavefronts of a workgroup re-read each other's rows through the vector cache.
+// wavefronts of a workgroup read the same A rows through the vector cache.
 // gridDim.z > 1: split K, each split adds its part into C atomically (C zeroed or kept by the host; no bias / residual then).
 template <int BITS>
 __global__ void __launch_bounds__(256) mx_gemm_k(const uint8_t *__restrict__ Aq, const uint8_t *__restrict__ As, const uint8_t *__restrict__ Bq, const uint8_t *__restrict__ Bs,
                                                  float *C, int M, int N, int nkb, float beta, const float *__restrict__ bias, const float *res, int sper) {
     constexpr int BPB = BITS == 8 ? 32 : 16, FM = BITS == 8 ? 0 : 4;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
-    // a wavefront owns a 64 x 64 tile; a workgroup is 2 x 2 of them, or a single one (few tiles: more workgroups than CUs that way)
-    const int wt = blockDim.x == 256 ? 2 : 1;
-    const int m0 = (blockIdx.y * wt + (wave >> 1)) * 64, n0 = (blockIdx.x * wt + (wave & 1)) * 64;
+    // a wavefront owns a 64 x 64 tile; a workgroup is four of them in a row, or a single one (few tiles: more workgroups than CUs that way)
+    // (four wavefronts: side by side along N, so the workgroup writes runs of 1 KiB of a C row and shares its A rows)
+    const int wn = blockDim.x >> 6;
+    const int m0 = blockIdx.y * 64, n0 = (blockIdx.x * wn + wave) * 64;
     if (m0 >= M || n0 >= N) return;                        // (no barriers in this kernel: a wavefront without work leaves)
     const int nst = nkb >> 1, s0 = (int)blockIdx.z * sper, s1 = min(nst, s0 + sper);
     const uint8_t *pa[2], *pb[2], *sa[2], *sb[2];
@@ -170,9 +171,10 @@ extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, cons
     ns = nst > 0 ? (nst + sper - 1) / sper : 1;
     if (ns > 1 && beta == 0.f) gemm_zero_k<<<nblk_((size_t)M * N, 256 * 4), 256>>>(C, (size_t)M * N);   // (a kernel, not a memset node: safe under graph capture)
     const int wt = (size_t)tiles * ns >= 512 ? 2 : 1;              // (few tiles: one wavefront per workgroup)
-    const dim3 grid((unsigned)((N + 64 * wt - 1) / (64 * wt)), (unsigned)((M + 64 * wt - 1) / (64 * wt)), (unsigned)ns);
-    if (bits == 8) mx_gemm_k<8><<<grid, 64 * wt * wt>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
-    else mx_gemm_k<4><<<grid, 64 * wt * wt>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
+    const int wn = wt == 2 ? 4 : 1;                                // wavefronts per workgroup, side by side along N
+    const dim3 grid((unsigned)((N + 64 * wn - 1) / (64 * wn)), (unsigned)((M + 63) / 64), (unsigned)ns);
+    if (bits == 8) mx_gemm_k<8><<<grid, 64 * wn>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
+    else mx_gemm_k<4><<<grid, 64 * wn>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
     MICK();
     return 0;
 }
