@@ -60,9 +60,10 @@ def test_feather_blend_is_bit_exact(gpu, S, B, nss, bn, absent):
     assert lib.mi_feather_blend(dE.ptr, dp.ptr, S, S + 1, nss_a, bn_a, do.ptr) == -1     # B > S: refused
 
 
-def test_ct_window_gather(gpu):
+@pytest.mark.parametrize("W", [24, 32])          # rows of 24 voxels are stored byte by byte, rows of a multiple of 16 as 16-byte vectors
+def test_ct_window_gather(gpu, W):
     rng = np.random.default_rng(9)
-    Z, Y, X, W = 20, 33, 47, 24
+    Z, Y, X = 20, 33, 47
     vol = rng.integers(0, 256, (Z, Y, X)).astype(np.uint8)
     dv = DevBuf.from_numpy(vol)
     for (oz, oy, ox) in [(-5, -5, -5), (3, 12, 30), (10, 20, 40)]:
