@@ -128,6 +128,7 @@ void mi_zero(void *p, size_t bytes);
 void mi_h2d(void *dst, const void *src, size_t bytes);
 void mi_d2h(void *dst, const void *src, size_t bytes);
 void mi_d2d(void *dst, const void *src, size_t bytes);
+void mi_d2d_rows(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows);   /* rows runs of width bytes at the two pitches, in stream order */
 void mi_sync(void);
 void mi_ws_release(void);                      /* frees the per-device scratch (prepared weights, staged operands) */
 /* GroupNorm finalize from sum slots: mean, rstd of NG = N * G groups of `len` elements each (src/nn_elem.cu:5-11) */

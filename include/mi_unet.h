@@ -114,8 +114,13 @@ shape5 unet_out_shape(const unet *u, shape5 xs);
    from the scroll axis, xs.d floats per window back to back; h16: the 16-bit type the input values are rounded to (2 fp16, 1 bf16, 0 none).
    xs.c must be 4 and xs.h == xs.w. */
 const float *unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, shape5 xs, int h16);
-void unet_set_infer_slab(int planes);                         /* inference: the level-0 convs in z-slabs of this many planes (rounded up to a multiple of 4), each slab written
-                                                                 straight into the full-depth tensors; byte-identical logits; 0 = off (src/unet.h:422-424, direct slab outputs) */
+void unet_set_infer_slab(int planes);                         /* inference: the convs of level 0 (and of level 1 when the net has three or more levels; UFSM_INFER_SLAB_L1=0:
+                                                                 level 0 only) in z-slabs of this many planes (rounded up to a multiple of 4); byte-identical logits; 0 = off
+                                                                 (src/unet.h:422) */
+void unet_set_slab_direct(int on);                            /* on (the default): each slab is written straight into the full-depth tensors. Off: the in-place form, one buffer per
+                                                                 slab level for all its tensors, a slab temp and a carry plane, plane copies after each slab (src/unet.h:424,
+                                                                 src/unet.c:2435-2440, :2540-2542); the same bytes, about four tensors of each such level less memory. The reference
+                                                                 picks the form from the card's free memory (src/unet.c:1168-1173); here the caller does. */
 /* ---- checkpoints in the reference's format (src/unet.h:342-357; src/unet.c:5534-5650 unet_save, :5650-5755 header, :5774-5800 unet_load): one
    line "UFSM{json}\n", then nparams fp32 weights, the EMA weights and optionally optimizer state (skipped here). unet_peek fills cfg and step
    from the header: 0, -1 when the file is unreadable, -2 naming (stderr) a feature of the checkpoint this build does not run. unet_load copies

@@ -305,17 +305,21 @@ def test_reference_signature_forwards(gpu):
     net.close()
 
 
-@pytest.mark.parametrize("bits,dims,slab,attn", [(8, (32, 32, 32), 8, 0), (8, (24, 16, 32), 16, 0), (4, (16, 32, 32), 4, 0), (8, (32, 32, 32), 16, 1)])
-def test_slab_inference_is_byte_identical(gpu, bits, dims, slab, attn):
-    """unet_set_infer_slab: the level-0 convs (stem, encoder conv2, decoder conv1 over [up | skip], decoder conv2) run in z-slabs through the
-    z-range with direct slab outputs; logits, every stored tensor and every GroupNorm statistic equal the whole-tensor forward's
-    (tests/test_infer_mem.c: byte-identical logits)."""
+@pytest.mark.parametrize("direct", [1, 0])
+@pytest.mark.parametrize("bits,dims,slab,attn,widths", [(8, (32, 32, 32), 8, 0, [32, 64]), (8, (24, 16, 32), 16, 0, [32, 64]), (4, (16, 32, 32), 4, 0, [32, 64]),
+                                                        (8, (32, 32, 32), 16, 1, [32, 96]), (8, (32, 32, 32), 8, 0, [32, 64, 128]), (8, (40, 16, 32), 16, 0, [32, 32, 64]),
+                                                        (4, (32, 16, 32), 8, 0, [32, 64, 64]), (8, (32, 16, 16), 16, 0, [32, 64, 64])])
+def test_slab_inference_is_byte_identical(gpu, bits, dims, slab, attn, widths, direct):
+    """unet_set_infer_slab: the convs of level 0 (stem, encoder conv2, decoder conv1 over [up | skip], decoder conv2) and, in nets of three
+    levels, of level 1 run in z-slabs through the z-range; logits, every stored tensor and every GroupNorm statistic equal the whole-tensor
+    forward's (tests/test_infer_mem.c: byte-identical logits). direct 1: slabs written straight into the full-depth tensors; 0: the in-place
+    form (unet_set_slab_direct(0)), where a slab level's tensors share one buffer, slabs go through a temp and a carry plane, and of that
+    level's tensors only the last written (the decoder's conv2 output) can still be read back afterwards."""
     from ufsm_amd.unet import UNet, make_cfg, load_host
     H_ = load_host()
     rng = np.random.default_rng(slab + bits)
     D, H, W = dims
     N, S = 2, D * H * W
-    widths = [32, 96] if attn else [32, 64]
     net = UNet(make_cfg(4, widths, G=8, head_out=3, act_dt=bits, attn_blocks=attn, attn_pe=1, down_norm=1), N, D, H, W, seed=5)
     x = rng.standard_normal((N, 4, S)).astype(np.float32); dxq = to_mx(bits, x)
     la, lb = DevBuf(N * 3 * S * 4), DevBuf(N * 3 * S * 4)
@@ -336,17 +340,28 @@ def test_slab_inference_is_byte_identical(gpu, bits, dims, slab, attn):
     whole = fetch()
     assert {"enc0.c1", "enc0.c2", "dec0.c1", "dec0.c2"} <= set(whole)
     H_.unet_set_infer_slab(slab - 1)                       # rounded up to a multiple of 4
+    H_.unet_set_slab_direct(direct)
     try:
         assert H_.mi_unet_infer_slab() == slab
         assert net.forward_x(dxq.ptr, lb.ptr) == 0
         LP.check()
+        slabbed = fetch()
+        where = {name: ptr for name, ptr, _ in net.layer_outs()}
+        for i in range(2 if len(widths) > 2 else 1):       # one buffer per slab level in the in-place form, four otherwise
+            assert len({where[f"{e}{i}.{c}"] for e in ("enc", "dec") for c in ("c1", "c2")}) == (4 if direct else 1)
     finally:
-        H_.unet_set_infer_slab(0)
+        H_.unet_set_infer_slab(0); H_.unet_set_slab_direct(1)
     assert np.array_equal(la.to_numpy(np.float32), lb.to_numpy(np.float32))
-    slabbed = fetch()
+    gone = set() if direct else {f"{e}{i}.{c}" for i in range(2 if len(widths) > 2 else 1) for e, c in (("enc", "c1"), ("enc", "c2"), ("dec", "c1"))}
+    assert set(slabbed) == set(whole)
     for name, (t, m, r) in whole.items():
         t2, m2, r2 = slabbed[name]
-        assert np.array_equal(t2, t) and np.array_equal(m2, m) and np.array_equal(r2, r), name
+        assert np.array_equal(m2, m) and np.array_equal(r2, r), name
+        assert name in gone or np.array_equal(t2, t), name
+    # the same net, back in the whole-tensor form (its buffers are rebuilt): still the same logits
+    assert net.forward_x(dxq.ptr, lb.ptr) == 0
+    LP.check()
+    assert np.array_equal(la.to_numpy(np.float32), lb.to_numpy(np.float32))
     net.close()
 
 

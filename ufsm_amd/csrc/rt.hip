@@ -45,6 +45,10 @@ extern "C" void mi_zero(void *p, size_t bytes) { MIRT(hipMemsetAsync(p, 0, bytes
 extern "C" void mi_h2d(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice)); }
 extern "C" void mi_d2h(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost)); }
 extern "C" void mi_d2d(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, 0)); }
+// `rows` runs of `width` bytes, run r at dst + r * dpitch from src + r * spitch (a range of planes of every channel block of an MX tensor)
+extern "C" void mi_d2d_rows(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows) {
+    if (width && rows) MIRT(hipMemcpy2DAsync(dst, dpitch, src, spitch, width, rows, hipMemcpyDeviceToDevice, 0));
+}
 extern "C" void mi_sync(void) { MIRT(hipDeviceSynchronize()); }
 
 // per-device scratch: grow on demand, contents valid until the next request of the same slot on the same device

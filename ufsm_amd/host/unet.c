@@ -23,6 +23,8 @@ struct unet {
     unet_cfg cfg;
     /* the activations, built for one input shape and storage mode (rebuilt when either changes: src/unet.c:2876) */
     int built, act_dt, prec; shape5 in; shape5 ls[UNET_MAXLEV];
+    int slab_ip, slab_nl, slab_s;      /* the build's in-place slab plan: on, and over how many levels (a level's tensors all live in enc[i].a2's buffer) */
+    void *slab_tmp[2], *slab_carry[2]; /* per such level: one slab of output planes, and the plane that waits for the next slab */
     block enc[UNET_MAXLEV], dec[UNET_MAXLEV];
     convp down[UNET_MAXLEV], head;
     void *downo[UNET_MAXLEV];
@@ -123,6 +125,24 @@ unet *unet_create(const unet_cfg *cfg) {
     if (cfg->w4_2d) { u->wm = f32_new(off); u->params = u->wm; }
     return u;
 }
+/* inference in z-slabs (src/unet.h:422-424, src/unet.c:2499-2550): the convs of level 0 (and of level 1 in nets of three or more levels,
+   src/unet.c:1165) run slab by slab through the z-range; results are those of the whole-tensor convs.
+   Direct form (the default, src/unet.c:216, :1167): each slab's planes go straight into the full-depth output tensor.
+   In-place form (unet_set_slab_direct(0); src/unet.c:2435-2440): every tensor of such a level lives in one buffer X; a conv whose input is X
+   writes its slab into a temp, whose planes but the last then go into X (the next slab still reads the old last plane); that last plane
+   waits in a carry plane until the next slab is computed. One slab temp, one plane and X replace a1, a2, the decoder's a1 and a2 and the
+   pre-staged skip of the level. */
+static int g_infer_slab, g_slab_direct = 1;
+void unet_set_infer_slab(int planes) { g_infer_slab = planes > 0 ? (planes + 3) / 4 * 4 : 0; }
+void unet_set_slab_direct(int on) { g_slab_direct = on != 0; }
+int mi_unet_infer_slab(void) { return g_infer_slab; }
+static int slab_levels(const unet *u) {      /* how many of the finest levels run in slabs (UFSM_INFER_SLAB_L1=0: level 0 only) */
+    if (!g_infer_slab) return 0;
+    const char *e = getenv("UFSM_INFER_SLAB_L1");
+    return u->cfg.nlev > 2 && !(e && atoi(e) == 0) ? 2 : 1;
+}
+static int slab_inplace_now(const unet *u) { return g_infer_slab && !g_slab_direct && u->cfg.nlev > 1; }
+
 /* the activation buffers of the current build */
 static void free_acts(unet *u) {
     if (!u->built) return;
@@ -130,6 +150,7 @@ static void free_acts(unet *u) {
     for (int i = 0; i < UNET_MAXLEV; i++) {
         for (int s = 0; s < 2; s++) {
             block *b = s ? &u->dec[i] : &u->enc[i];
+            if (u->slab_ip && i < u->slab_nl) { if (s) b->a2 = nullptr; b->a1 = nullptr; }       /* (aliases of enc[i].a2) */
             act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2);
             b->a1 = b->a2 = nullptr; b->m1 = b->r1 = b->m2 = b->r2 = nullptr;
         }
@@ -137,9 +158,10 @@ static void free_acts(unet *u) {
         u->downo[i] = u->skipst[i] = nullptr; u->dm[i] = u->dr[i] = nullptr;
     }
     if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); u->tb.a2 = nullptr; u->tb.m2 = u->tb.r2 = nullptr; u->tb_cs = u->tb_tok = nullptr; u->tb_ws = nullptr; }
+    for (int i = 0; i < 2; i++) { act_del(u->slab_tmp[i]); act_del(u->slab_carry[i]); u->slab_tmp[i] = u->slab_carry[i] = nullptr; }
     act_del(u->xin); u->xin = nullptr;
     mi_free(u->logits); u->logits = nullptr;
-    u->built = 0; u->nouts = 0;
+    u->built = 0; u->nouts = 0; u->slab_ip = u->slab_nl = u->slab_s = 0;
 }
 /* (re)build for input shape `in` under the storage mode and precision policy in force (build_acts, src/unet.c:2876) */
 static int build_acts(unet *u, shape5 in) {
@@ -149,22 +171,28 @@ static int build_acts(unet *u, shape5 in) {
     if (!unet_act_mx()) { fprintf(stderr, "unet: this build stores activations as MX-fp8 or MX-fp4 only (unet_set_act_mx8 / unet_set_act_mx4)\n"); return -1; }
     free_acts(u);
     u->in = in; u->act_dt = act_dt_now(); u->prec = nn_get_prec();
+    u->slab_ip = slab_inplace_now(u); u->slab_nl = u->slab_ip ? slab_levels(u) : 0; u->slab_s = u->slab_ip ? g_infer_slab : 0;
     for (int i = 0; i < L; i++) u->ls[i] = (shape5){in.n, w[i], in.d >> i, in.h >> i, in.w >> i};
     for (int i = 0; i < L; i++) {
         for (int s = 0; s < 2; s++) {
             block *b = s ? &u->dec[i] : &u->enc[i];
             if (s && i == L - 1) continue;
             b->ys = u->ls[i]; b->xs = u->ls[i]; b->xs.c = b->c1.cin;
-            b->a1 = act_new(u, b->ys); b->a2 = act_new(u, b->ys);
+            if (i < u->slab_nl) { b->a2 = s ? u->enc[i].a2 : act_new(u, b->ys); b->a1 = b->a2; }
+            else { b->a1 = act_new(u, b->ys); b->a2 = act_new(u, b->ys); }
             const size_t ng = (size_t)in.n * G_of(u, w[i]);
             b->m1 = f32_new(ng); b->r1 = f32_new(ng); b->m2 = f32_new(ng); b->r2 = f32_new(ng);
         }
         if (i < L - 1) {
             shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds);
             /* both readers of the skip compute in e4m3 from MX-fp8 storage: one shared pre-stage (any other combination: the readers' formats differ) */
-            if (u->act_dt == 8 && u->prec != 3 && w[i] % 32 == 0) u->skipst[i] = act_new(u, u->enc[i].ys);
+            if (u->act_dt == 8 && u->prec != 3 && w[i] % 32 == 0 && i >= u->slab_nl) u->skipst[i] = act_new(u, u->enc[i].ys);
             if (cfg->down_norm) { const size_t ng = (size_t)in.n * G_of(u, w[i]); u->dm[i] = f32_new(ng); u->dr[i] = f32_new(ng); }
         }
+    }
+    for (int i = 0; i < u->slab_nl; i++) {
+        shape5 t = u->ls[i]; if (u->slab_s < t.d) t.d = u->slab_s;
+        u->slab_tmp[i] = act_new(u, t); t.d = 1; u->slab_carry[i] = act_new(u, t);
     }
     u->xin = act_new(u, in);
     u->logits = f32_new((size_t)in.n * cfg->cout * in.d * in.h * in.w);
@@ -181,7 +209,8 @@ static int build_acts(unet *u, shape5 in) {
     return 0;
 }
 static int ensure_built(unet *u, shape5 xs) {
-    if (u->built && !memcmp(&u->in, &xs, sizeof xs) && u->act_dt == act_dt_now() && u->prec == nn_get_prec()) return 0;
+    const int ip = slab_inplace_now(u);
+    if (u->built && !memcmp(&u->in, &xs, sizeof xs) && u->act_dt == act_dt_now() && u->prec == nn_get_prec() && u->slab_ip == ip && (!ip || (u->slab_nl == slab_levels(u) && u->slab_s == g_infer_slab))) return 0;
     return build_acts(u, xs);
 }
 void unet_free(unet *u) {
@@ -262,25 +291,40 @@ static void note(unet *u, const void *p, shape5 s, const char *name, const float
 }
 static nn_gn_t gn_out(const unet *u, const block *b) { return (nn_gn_t){P(u, b->n2.gamma), P(u, b->n2.beta), b->m2, b->r2, G_of(u, b->ys.c)}; }   /* silu(gn(a2)) for the block's readers */
 
-/* inference in z-slabs (src/unet.h:422-424, src/unet.c:2499-2550 with direct slab outputs): the level-0 convs run slab by slab through the
-   z-range, each slab's planes written straight into the full-depth output; results are those of the whole-tensor convs */
-static int g_infer_slab;
-void unet_set_infer_slab(int planes) { g_infer_slab = planes > 0 ? (planes + 3) / 4 * 4 : 0; }
-int mi_unet_infer_slab(void) { return g_infer_slab; }
-
-/* conv1 -> a1 (+ its statistics), conv2 reads silu(gn(a1)) while staging -> a2 (+ statistics) (src/unet.c:2567-2636) */
+/* planes [s0, s0 + n) of the MX tensor src (depth Ds) -> planes [d0, d0 + n) of dst (depth Dd), every sample and channel block: a block's
+   element rows and its scales are each contiguous over a range of planes (mx_copy_planes, src/unet.c:2410-2422) */
+static void copy_planes(const unet *u, void *dst, int Dd, int d0, const void *src, int Ds, int s0, int n, shape5 s) {
+    if (n <= 0) return;
+    const int bw = s.c <= 8 ? 8 : s.c <= 16 ? 16 : 32, nb = (s.c + bw - 1) / bw, rb = u->act_dt == 4 ? bw / 2 : bw;
+    const size_t hw = (size_t)s.h * s.w, Sd = (size_t)Dd * hw, Ss = (size_t)Ds * hw, rows = (size_t)s.n * nb;
+    mi_d2d_rows((char *)dst + (size_t)d0 * hw * rb, Sd * rb, (const char *)src + (size_t)s0 * hw * rb, Ss * rb, (size_t)n * hw * rb, rows);
+    mi_d2d_rows((char *)dst + rows * Sd * rb + (size_t)d0 * hw, Sd, (const char *)src + rows * Ss * rb + (size_t)s0 * hw, Ss, (size_t)n * hw, rows);
+}
+/* conv1 -> a1 (+ its statistics), conv2 reads silu(gn(a1)) while staging -> a2 (+ statistics) (src/unet.c:2567-2636); in z-slabs when asked for
+   (slab_run, src/unet.c:2499-2545) */
 static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t *gin, const void *xup, const nn_gn_t *gup, int c_split, const char *n1, const char *n2) {
-    const int G = G_of(u, b->c1.cout), D = b->ys.d, s = level == 0 && g_infer_slab && g_infer_slab < D ? g_infer_slab : 0;
+    const int G = G_of(u, b->c1.cout), D = b->ys.d, ip = u->slab_ip && level < u->slab_nl;
+    const int s = level >= slab_levels(u) ? 0 : g_infer_slab < D ? g_infer_slab : ip ? D : 0;      /* (in place: a level of fewer planes is one slab) */
+    void *tmp = ip ? u->slab_tmp[level] : nullptr, *carry = ip ? u->slab_carry[level] : nullptr;
     int r = 0;
     for (int conv = 1; conv <= 2 && !r; conv++) {
-        for (int z0 = 0, sk; z0 < D && !r; z0 += sk) {
+        void *y = conv == 1 ? b->a1 : b->a2;
+        const int over = ip && (conv == 2 || x == y);              /* the conv reads the buffer it writes: through the temp */
+        for (int z0 = 0, k = 0, sk; z0 < D && !r; z0 += sk, k++) {
             sk = s && D - z0 > s ? s : D - z0;
+            const int last = z0 + sk >= D;
             shape5 xs = conv == 1 ? b->xs : b->ys;
-            if (s) { nn_set_zrange(z0, D, z0 == 0, z0 + sk >= D, D, z0); nn_set_zrange_out(1); xs.d = sk; }
-            if (conv == 2) r = nn_conv3d_fwd_gn_stats(b->a1, xs, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, b->a2, G, 1e-5f, b->m2, b->r2);
-            else if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, b->a1, G, 1e-5f, b->m1, b->r1);   /* [up2(coarse) | skip] */
-            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, b->a1, G, 1e-5f, b->m1, b->r1);
+            if (s) { nn_set_zrange(z0, D, z0 == 0, last, D, z0); nn_set_zrange_out(!over); xs.d = sk; }
+            void *o = over ? tmp : y;
+            if (conv == 2) r = nn_conv3d_fwd_gn_stats(b->a1, xs, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, o, G, 1e-5f, b->m2, b->r2);
+            else if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, G, 1e-5f, b->m1, b->r1);   /* [up2(coarse) | skip] */
+            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, G, 1e-5f, b->m1, b->r1);
             if (s) { nn_set_zrange(0, 0, 0, 0, 0, 0); nn_set_zrange_out(0); }
+            if (over && !r) {                                      /* planes below the next slab's first input plane are dead: the last one waits */
+                if (k) copy_planes(u, y, D, z0 - 1, carry, 1, 0, 1, b->ys);
+                copy_planes(u, y, D, z0, tmp, sk, 0, last ? sk : sk - 1, b->ys);
+                if (!last) copy_planes(u, carry, 1, 0, tmp, sk, sk - 1, 1, b->ys);
+            }
         }
         if (!r) { if (conv == 1) note(u, b->a1, b->ys, n1, b->m1, b->r1, G); else note(u, b->a2, b->ys, n2, b->m2, b->r2, G); }
     }

@@ -83,6 +83,7 @@ _PROTOS = {
     "mi_h2d": (None, [_P, _P, _Z]),
     "mi_d2h": (None, [_P, _P, _Z]),
     "mi_d2d": (None, [_P, _P, _Z]),
+    "mi_d2d_rows": (None, [_P, _Z, _P, _Z, _Z, _Z]),
     "mi_sync": (None, []),
     "mi_ws_release": (None, []),
     "mi_gn_finalize": (None, [_P, _I, _Z, _F, _P, _P]),
