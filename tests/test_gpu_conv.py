@@ -34,10 +34,10 @@ WIDE_SHAPES = [(8, 1, 96, 128, 5, 9, 18), (8, 1, 32, 128, 3, 8, 16), (8, 2, 128,
                (4, 1, 160, 128, 7, 8, 16), (4, 2, 64, 256, 4, 16, 16)]
 
 
-@pytest.fixture(params=[0, -1], ids=["slices128", "slices64"])
+@pytest.fixture(params=[0, 1 << 30], ids=["slices128", "slices64"])
 def slice_split(request):
-    """These launches have few tiles, which by default run as slices of 64 channels (two channel tiles per workgroup); 0 keeps the slices of 128
-    (four channel tiles, the form the large layers run in): both forms of the wide kernel see every shape."""
+    """Launches of few tiles run as slices of 64 channels (two channel tiles per workgroup) when the tile count is under the split; 0 keeps the
+    slices of 128 (four channel tiles, the form the large layers run in): both forms of the wide kernel see every shape."""
     lib.mi_conv_split(request.param)
     yield request.param
     lib.mi_conv_split(-1)
@@ -59,6 +59,23 @@ def test_wide_kernel_exact(gpu, slice_split, bits, N, Ci, Co, D, H, W):
     wf, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, acc64=1)
     gf, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits)
     assert np.array_equal(gf, wf)
+
+
+@pytest.mark.parametrize("bits,N,Ci,Co,D,H,W", WIDE_SHAPES[:3] + WIDE_SHAPES[5:])
+def test_few_tiles_default_dispatch(gpu, bits, N, Ci, Co, D, H, W):
+    """The default rule for launches of very few tiles (the coarsest levels): one channel tile and two planes per workgroup on the general
+    kernel instead of the wide kernel's slices."""
+    rng = np.random.default_rng(Ci * 19 + Co + D * 5 + bits)
+    S = D * H * W
+    x, w, b = exact_case(rng, N, Ci, Co, S)
+    xdt = 3 if bits == 8 else 4
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    want, wsum = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, acc64=1, Go=8, want_stats=True)
+    got, gsum = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, Go=8, stats=True)
+    name = lib.mi_last_kernel().decode()
+    assert "conv3_mx_k" in name and "MT 1, NT 2" in name, name
+    assert np.array_equal(got, want)
+    assert np.allclose(gsum, wsum, rtol=1e-6)
 
 
 @pytest.mark.parametrize("Ci,Co,split", [(32, 128, 0), (64, 128, 0), (32, 128, 1 << 30)])
@@ -96,9 +113,14 @@ def test_wide_kernel_decoder_conv(gpu):
     g1 = [rng.uniform(0.5, 1.5, Cu).astype(np.float32), rng.uniform(-0.3, 0.3, Cu).astype(np.float32), rng.uniform(-0.2, 0.2, G).astype(np.float32), rng.uniform(0.7, 1.4, G).astype(np.float32)]
     g2 = [rng.uniform(0.5, 1.5, Cs).astype(np.float32), rng.uniform(-0.3, 0.3, Cs).astype(np.float32), rng.uniform(-0.2, 0.2, G).astype(np.float32), rng.uniform(0.7, 1.4, G).astype(np.float32)]
     want, _ = orc.conv3(qu, 3, 1, Cu + Cs, D, H, W, w, b, Co, 0, x2=qs, c_split=Cu, up=1, gp=orc.gn(*g1, G=G), gp2=orc.gn(*g2, G=G))
-    got, _ = gpu_conv(qu, 3, 1, Cu + Cs, D, H, W, w, b, Co, 0, x2=qs, c_split=Cu, up=1, gp=dev_gn(*g1, G), gp2=dev_gn(*g2, G))
-    assert "conv3_wide_k" in lib.mi_last_kernel().decode()
-    assert np.abs(got - want).max() / np.abs(want).max() < 1e-3
+    for split, kern in ((1 << 30, "conv3_wide_k"), (-1, "conv3_mx_k")):       # forced slices of 64 on the wide kernel; the default for so few tiles
+        lib.mi_conv_split(split)
+        try:
+            got, _ = gpu_conv(qu, 3, 1, Cu + Cs, D, H, W, w, b, Co, 0, x2=qs, c_split=Cu, up=1, gp=dev_gn(*g1, G), gp2=dev_gn(*g2, G))
+        finally:
+            lib.mi_conv_split(-1)
+        assert kern in lib.mi_last_kernel().decode()
+        assert np.abs(got - want).max() / np.abs(want).max() < 1e-3
 
 
 EXACT_SHAPES = [

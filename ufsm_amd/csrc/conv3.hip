@@ -339,6 +339,15 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
             (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 3) / 4) * (nmt_all / 4) * N < (size_t)split) { MT = 2; halved = true; }
     }
     int NT = (stride == 1 && MT <= 2 && Do >= 4) ? 4 : 2;
+    // ... and when even the slices of 64 give fewer than 128 workgroups (256 -> 256 at 2 x 16^3: 64): one channel tile and two planes per workgroup
+    // on the general kernel, four times the workgroups (measured in the 32/64/128/256 forward: 128 -> 256 0.032 -> 0.026 ms, 256 -> 256
+    // 0.050 -> 0.038 ms; from 256 slices of 64 on, the wide kernel is the faster one: 128 -> 128 at 2 x 32^3 0.034 against 0.052 ms)
+    bool coarse = false;
+    {
+        static int ce = -1;
+        if (ce < 0) ce = getenv("MI_CONV_COARSE") ? atoi(getenv("MI_CONV_COARSE")) : 1;      // tuning knob: 0 keeps the wide kernel's slices of 64 there (as does a split forced through mi_conv_split)
+        if (ce && halved && g_split < 0 && (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 3) / 4) * (nmt_all / 2) * N < 128) { coarse = true; NT = 2; MT = 1; halved = false; }
+    }
     // stride 2 with few tiles (the coarse levels): one-plane tiles double the workgroups; with enough tiles the two-plane tile is faster
     // (measured: 128 -> 128 at 32^3 -> 16^3, N 2: 32 tiles 0.072 ms, 64 tiles 0.042 ms; 32 -> 32 at 128^3: 0.090 vs 0.120 ms)
     if (stride == 2 && (MT == 1 || MT == 2 || MT == 4) &&
@@ -366,7 +375,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel, 2 sends every 64-channel layer to the wide kernel too
     // (64 output channels: two channel tiles per workgroup; it pays from four input blocks on: 192 -> 64 at 2 x 64^3 0.190 -> 0.178 ms, 64 -> 64 the same
     // as the general kernel. MI_CONV_WIDE=2 sends every such layer there)
-    bool big = big_env && stride == 1 && (MT == 4 || (MT == 2 && (big_env > 1 || a.nbt >= 4 || halved))) && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
+    bool big = !coarse && big_env && stride == 1 && (MT == 4 || (MT == 2 && (big_env > 1 || a.nbt >= 4 || halved))) && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
     if (big) {
         // The wide kernel streams input block b >= 2 of a tile into LDS while the tile's earlier blocks are multiplied, one copy round per
         // stage of two pairs, NRND rounds per block, a block starting once block b - 3 has been read for the last time (pair (27 (b - 3) + 26) / 2).
@@ -403,13 +412,13 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     a.CB = big || s2d ? a.nbt : (a.nbt + nchunks - 1) / nchunks; // (the wide kernel has no chunks: its K loop walks block by block; the direct stride-2 kernel: one chunk, tap-major)
     static int areg_env = -1;
     if (areg_env < 0) areg_env = getenv("MI_CONV_AREG") ? atoi(getenv("MI_CONV_AREG")) : 1;      // tuning knob: 0 keeps the general kernel for every shape
-    a.areg = areg_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && a.nbt == 1 && a.wide && (NT == 2 || NT == 4);
+    a.areg = areg_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && nmt_all == 1 && stride == 1 && a.nbt == 1 && a.wide && (NT == 2 || NT == 4);      // (one channel tile in all: these kernels have no channel slices)
     // one channel tile of 17 .. 32 output channels from two or more input blocks on a volume wider than one 16-voxel tile: the row kernel (runs
     // of 32 voxels along x, input fragments shared by the three ky taps). One input block stays with the kernel that keeps its weights in
     // registers, which measures a few percent faster there (both are bound by the halo's cache misses in flight, and it loads no weights)
     static int row_env = -1;
     if (row_env < 0) row_env = getenv("MI_CONV_ROW") ? atoi(getenv("MI_CONV_ROW")) : 1;      // tuning knob: 0 keeps the other kernels for these shapes, 2 also takes one input block
-    a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && stride == 1 && MT == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 ? 1 : 2) && a.nbt <= 64;
+    a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && nmt_all == 1 && stride == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 ? 1 : 2) && a.nbt <= 64;
     if (a.row) { a.areg = false; a.CB = a.nbt; }
     size_t smem = a.row ? (size_t)2 * 2048 * (RB + 4) : a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     if (s2d) smem = 0;
