@@ -354,6 +354,9 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
         (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * ((Do + 1) / 2) * (nmt_all / MT) * N < 256) NT = 1;
     // ... and still fewer one-plane tiles than half the CUs: two channel tiles per workgroup instead of four
     if (stride == 2 && MT == 4 && NT == 1 && split_s2_env() && (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * Do * (nmt_all / 4) * N < 128) MT = 2;
+    // ... and one while two would still leave CUs idle (128 -> 128 from 2 x 32^3: 128 workgroups 0.035 ms, 256 workgroups 0.024 ms; the two-plane
+    // tiles of 64 -> 64 from 2 x 64^3, 256 workgroups, are the fastest form there: 0.030 ms against 0.039 with 512 one-plane tiles)
+    if (stride == 2 && MT == 2 && NT == 1 && split_s2_env() && (size_t)((Wo + 15) / 16) * ((Ho + 7) / 8) * Do * (nmt_all / 2) * N < 256) MT = 1;
     // stride 2 on 32-channel rows with enough output voxels (four workgroups per CU or more): the kernel that reads every tap's rows straight from
     // the stored tensor (no staged halo). Measured in the 32/64/128/256 forward at 2 x 128^3: 32 -> 32 from 128^3 0.093 -> 0.071 ms; 64 -> 64 from
     // 64^3 is slower there, 0.030 -> 0.037 ms, and stays with the general kernel. Runs of 64 output voxels per wavefront; channel tiles per
