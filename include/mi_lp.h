@@ -29,7 +29,10 @@ typedef struct {                                                                
    zi0 / Di (output plane z of the xs.d planes computed reads input plane z + zi0 of depth-Di inputs; Di 0 = off) and yzo / yD (the MX
    output is planes [yzo, yzo + xs.d) of a depth-yD tensor; yD 0 = a depth-xs.d tensor), stride 1 (src/nn_lp.h:36-40). Training and
    z-window fields (y2, o_split, accum, sr, osr, o_pad, zw0, zw1) must be zero: a call that sets one prints a message and aborts, as the
-   reference does for unsupported combinations (src/lp_f8fwd.cu:28). Slab-local GroupNorm (gnp_t.ns > 0) likewise. */
+   reference does for unsupported combinations (src/lp_f8fwd.cu:28).
+   Slab-local GroupNorm statistics (gnp_t.ns > 0, src/nn_lp.h:15-18: mean / rstd hold one row per (sample, z-slab), [n][ns][G]; plane z reads
+   row n * ns + clamp((z + zo) / zs, 0, ns - 1); zhw = voxels per plane) are honoured by every reader of an MX tensor: the conv entries (both
+   segments' of a split input; not the upsampled segment's), the stride-2 entry, the 1x1x1 head, lp_gn_silu_apply_mx and mi_conv_prestage. */
 
 /* tile masks of a masked ("skip-empty") conv (src/nn_lp.h:44): m the output tiles to compute, nullptr: dense */
 typedef struct { const uint8_t *m, *mi; int my, mx, zoff; } skipm_t;
@@ -83,7 +86,10 @@ void mi_conv_s2_direct(int mode);
    input, gp2.G = -1 says "x2 carries no GroupNorm, gp is x's own" (gp2.G = 0 keeps the reference's meaning: gp spans both segments). */
 int mi_conv_prestage(const void *x, int xdt, shape5 s, gnp_t gp, void *y, int ybits);
 gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean, const float *rstd, int G);   /* src/nn_lp.h:19 */
-int lp_gn_slab_any(void);                                                                         /* src/nn_lp.h:20: always 0 here */
+int lp_gn_slab_any(void);                                                                         /* src/nn_lp.h:20: any statistics array registered */
+/* the statistics array `mean` holds one row per (sample, z-slab) with this geometry: every gnp_t gnp_mk builds from it (and lp_gn_silu_apply_mx,
+   which takes the pointers) carries it. ns <= 0 removes the entry, a null mean clears the registry (src/nn.h:471, src/nn_fwd.cu:12-22) */
+void lp_gn_slab_reg(const float *mean, int zs, int zo, int ns, int zhw);
 
 /* ---- MX tensor conversions (src/nn_lp.h:111-118, :126; src/lp_mx_cvt.cu:6-79, :429-447) ---- */
 size_t lp_mx8_bytes(int N, int C, size_t S);

@@ -311,14 +311,23 @@ float orc_act_ab(float v, float a, float b) {
     if (g_act_mode == 1) { const float d = 1.f + expf(-u), r = 1.f / d; return u * r; }
     return (float)((double)u / (1.0 + exp(-(double)u)));
 }
-static void gn_ab(const orc_gn_t *g, int n, int cc, int Cg, float *a, float *b) {
-    const int ng = n * g->G + cc / (Cg / g->G);
+/* src/lp_slab.cuh:7-12: per-sample statistics read row n; slab-local ones the row of the plane's slab, the first and last slab taking
+   whatever lies before and after them */
+int orc_gn_row(const orc_gn_t *g, int n, int z) {
+    if (!g->ns) return n;
+    int s = (z + g->zo) / g->zs;
+    s = s < 0 ? 0 : s >= g->ns ? g->ns - 1 : s;
+    return n * g->ns + s;
+}
+/* (nr: the statistics row) */
+static void gn_ab(const orc_gn_t *g, int nr, int cc, int Cg, float *a, float *b) {
+    const int ng = nr * g->G + cc / (Cg / g->G);
     *a = g->rstd[ng] * g->gamma[cc];
     *b = fmaf(-g->mean[ng], *a, g->beta[cc]);               /* tests/test_mx4_wide.c:119 */
 }
-/* per padded-channel (a, b, has_gn) table of sample n */
+/* per padded-channel (a, b, has_gn) table of sample n at input plane z (the plane only matters to slab-local statistics) */
 typedef struct { float a, b; int g, ci; } chab_t;
-static void chan_table(const orc_conv_t *c, int n, int Cx, int CxP, int Cip, chab_t *tab) {
+static void chan_table(const orc_conv_t *c, int n, int z, int Cx, int CxP, int Cip, chab_t *tab) {
     const int s2g = c->x2 && c->gp2.G;
     for (int cp = 0; cp < Cip; cp++) {
         const int mxin = c->xdt >= 3;
@@ -327,7 +336,7 @@ static void chan_table(const orc_conv_t *c, int n, int Cx, int CxP, int Cip, cha
         if (ci >= 0) {
             const orc_gn_t *q = s2g && ci >= Cx ? &c->gp2 : &c->gp;
             const int cc = s2g && ci >= Cx ? ci - Cx : ci, Cg = s2g ? (ci >= Cx ? c->Ci - Cx : Cx) : c->Ci;
-            if (q->G) { gn_ab(q, n, cc, Cg, &t.a, &t.b); t.g = 1; }
+            if (q->G) { gn_ab(q, orc_gn_row(q, n, z), cc, Cg, &t.a, &t.b); t.g = 1; }
         }
         tab[cp] = t;
     }
@@ -372,9 +381,13 @@ static int build_staged(const orc_conv_t *c, staged_t *st) {
     /* the fp4 entry blends the fused upsample in binary16 (src/lp_f4fwd.cuh:1135-1136, UFSM_UP_H2 default), the fp8 entry in fp32; up 2 / 3 force one */
     const int uph2 = c->up == 2 || (c->up == 1 && c->cbits == 4);
     const int Dc = c->D >> 1, Hc = c->H >> 1, Wc = c->W >> 1;
+    if (c->up && c->gp.G && c->gp.ns) return -1;           /* (slab-local statistics of the upsampled segment: no reader of the reference takes them) */
+    const int slabs = (c->gp.G && c->gp.ns) || (c->gp2.G && c->gp2.ns);
+    const size_t HW = (size_t)c->H * c->W;
     for (int n = 0; n < c->N; n++) {
-        chab_t *tab = (chab_t *)malloc((size_t)Cip * sizeof(chab_t));
-        chan_table(c, n, Cx, CxP, Cip, tab);
+        /* the table of plane 0, and with slab-local statistics one per input plane behind it */
+        chab_t *tab = (chab_t *)malloc((size_t)Cip * (slabs ? c->D : 1) * sizeof(chab_t));
+        for (int z = 0; z < (slabs ? c->D : 1); z++) chan_table(c, n, z, Cx, CxP, Cip, tab + (size_t)z * Cip);
         for (int ch = 0; ch < st->nch; ch++) {
             const int upc = mxin && c->up && ch * 32 < CxP;
             const int sec = mxin && ch * 32 >= CxP;       /* chunk of the x2 segment */
@@ -428,12 +441,14 @@ static int build_staged(const orc_conv_t *c, staged_t *st) {
                         }
                     } else {
                         mx_row32(&t, n, blk, v, r);
-                        for (int k = 0; k < 32; k++) { const chab_t *q = &tab[ch * 32 + k]; r[k] = q->ci < 0 ? 0.f : q->g ? orc_act_ab(r[k], q->a, q->b) : r[k]; }
+                        const chab_t *tz = tab + (slabs ? (v / HW) * (size_t)Cip : 0);
+                        for (int k = 0; k < 32; k++) { const chab_t *q = &tz[ch * 32 + k]; r[k] = q->ci < 0 ? 0.f : q->g ? orc_act_ab(r[k], q->a, q->b) : r[k]; }
                         quant_row(c->cbits, r, sv, sf);
                     }
                 } else {     /* plane-major fp32 / fp16 input, quantised per (voxel, 32 channels) */
+                    const chab_t *tz = tab + (slabs ? (v / HW) * (size_t)Cip : 0);
                     for (int k = 0; k < 32; k++) {
-                        const chab_t *q = &tab[ch * 32 + k];
+                        const chab_t *q = &tz[ch * 32 + k];
                         float xv = 0.f;
                         if (q->ci >= 0) {
                             const int sec2 = c->x2 && q->ci >= Cx;
@@ -512,6 +527,7 @@ static void conv_epilogue(const orc_conv_t *c, int n, size_t ov, size_t So, floa
 static int conv3_stem(const orc_conv_t *c) {
     const int Ci = c->Ci, Co = c->Co, D = c->D, H = c->H, W = c->W, rowmode = c->stem_tile == 2;
     if (c->x2 || c->up || c->stride == 2 || c->cbits != 8 || Ci > 16 || (!rowmode && c->xdt != 0 && Ci > 8)) return -2;
+    if (c->gp.G && c->gp.ns) return -3;     /* (slab-local statistics on the few-channel forms: not restated) */
     const int CP = rowmode ? 16 : Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = 32 / CP, NKB = rowmode ? 18 : (27 + TPK - 1) / TPK;
     const size_t S = (size_t)D * H * W;
     /* K block kb, element k -> (tap, channel), tap 27 = none */
@@ -530,7 +546,7 @@ static int conv3_stem(const orc_conv_t *c) {
     chab_t tab[32];
     for (int n = 0; n < c->N; n++) {
         /* the conv's input values of this sample: val[voxel][CP] (decoded, after GN + SiLU when the input has one) */
-        chan_table(c, n, Ci, (Ci + 31) / 32 * 32, 32, tab);
+        chan_table(c, n, 0, Ci, (Ci + 31) / 32 * 32, 32, tab);
         mxt_t t; if (c->xdt >= 3) t = mxt(c->x, c->xdt == 3 ? 8 : 4, c->N, Ci, S);
 #pragma omp parallel for schedule(static)
         for (int64_t vi = 0; vi < (int64_t)S; vi++) {
@@ -758,7 +774,7 @@ void orc_gn_silu_apply_mx(const void *x, int xdt, int N, int C, size_t S, orc_gn
         else for (int k = 0; k < bw; k++) { const int c = blk * bw + k; if (c < C) r[k] = ((const float *)x)[((size_t)n * C + c) * S + v]; }
         for (int k = 0; k < bw; k++) {
             const int c = blk * bw + k; if (c >= C) { r[k] = 0.f; continue; }
-            const int ng = n * gp.G + c / cpg;
+            const int ng = orc_gn_row(&gp, n, gp.ns ? (int)(v / (size_t)gp.zhw) : 0) * gp.G + c / cpg;
             r[k] = apply_silu(r[k], gp.mean[ng], gp.rstd[ng], gp.gamma[c], gp.beta[c]);
         }
         ysc[i] = orc_store_row(ybits, r, bw, y + (size_t)i * yrb, 1);
@@ -800,7 +816,7 @@ void orc_conv1_mx(int xbits, const uint8_t *x, int N, int Ci, size_t S, const fl
         const size_t v = (size_t)i % S; const int n = (int)((size_t)i / S);
         float xin[1024];
         for (int blk = 0; blk < t.nb; blk++) mx_row32(&t, n, blk, v, xin + blk * t.bw);
-        if (gp.G) for (int ci = 0; ci < Ci; ci++) { const int ng = n * gp.G + ci / cpg; const float a = gp.rstd[ng] * gp.gamma[ci], bb = fmaf(-gp.mean[ng], a, gp.beta[ci]); xin[ci] = orc_act_ab(xin[ci], a, bb); }
+        if (gp.G) for (int ci = 0; ci < Ci; ci++) { const int ng = orc_gn_row(&gp, n, gp.ns ? (int)(v / (size_t)gp.zhw) : 0) * gp.G + ci / cpg; const float a = gp.rstd[ng] * gp.gamma[ci], bb = fmaf(-gp.mean[ng], a, gp.beta[ci]); xin[ci] = orc_act_ab(xin[ci], a, bb); }
         for (int co = 0; co < Co; co++) {
             float acc = b ? b[co] : 0.f;
             for (int ci = 0; ci < Ci; ci++) acc = fmaf(w[(size_t)co * Ci + ci], xin[ci], acc);

@@ -36,6 +36,10 @@
  *                                 tensor under one scale (tests/test_oracle_stem.py)
  *   ... with stem_tile 2          the 9 .. 16 channel form with one scale per staged row (src/lp_f8fwd.cuh:447-563): exact operands equal the
  *                                 fp64 convolution; one large value coarsens exactly the outputs of its x tile that read its (z, y) line
+ *   slab-local statistics         pinned (orc_gn_row and its use in orc_conv3, orc_gn_silu_apply_mx, orc_conv1_mx; src/lp_slab.cuh:7-12): rows
+ *                                 against slab ranges written from the definition; a slab's planes cut out of the tensor and run through
+ *                                 the per-sample function with that slab's rows give the same bytes; conv output planes away from a slab
+ *                                 boundary equal the per-sample conv's, those at it equal neither (tests/test_oracle_slab_gn.py)
  *   orc_h16_to_mx                 pinned: numpy float16 values through the independent block quantiser (tests/test_oracle_elem.py)
  *   orc_pred_input_mx             pinned: a numpy statement of src/lp_mx_cvt.cu:24-41 through the independent block quantiser, all axes, the
  *                                 16-bit roundings, signed zeros (tests/test_oracle_elem.py). PARITY UNPINNED against the reference binary for
@@ -91,8 +95,10 @@ void orc_pred_input_mx(int bits, const uint8_t *ct, int W, float mean, float isd
    values, not yet scaled) and scale bytes ws[t][co][Cip/32]; Cip = padded input channels of the (split) input ---- */
 void orc_prep_w(int bits, const float *w, int Co, int Ci, int Cx, int CxP, int Cip, float *wv, uint8_t *ws, uint8_t *wcodes);
 
-/* ---- GroupNorm descriptor of an input segment (src/nn_lp.h:15) ---- */
-typedef struct { const float *gamma, *beta, *mean, *rstd; int G; } orc_gn_t;
+/* ---- GroupNorm descriptor of an input segment (src/nn_lp.h:15-18). ns > 0, slab-local statistics: mean / rstd hold one row per (sample,
+   z-slab), [n][ns][G]; plane z reads row n * ns + clamp((z + zo) / zs, 0, ns - 1) (src/lp_slab.cuh:7-12); zhw = voxels per plane ---- */
+typedef struct { const float *gamma, *beta, *mean, *rstd; int G; int zs, zo, ns, zhw; } orc_gn_t;
+int orc_gn_row(const orc_gn_t *g, int n, int z);      /* the statistics row of sample n at plane z */
 
 typedef struct {
     /* input */

@@ -9,7 +9,8 @@ LIB_PATH = os.path.join(ROOT, "oracle", "liboracle.so")
 
 
 class orc_gn_t(C.Structure):
-    _fields_ = [("gamma", C.c_void_p), ("beta", C.c_void_p), ("mean", C.c_void_p), ("rstd", C.c_void_p), ("G", C.c_int)]
+    _fields_ = [("gamma", C.c_void_p), ("beta", C.c_void_p), ("mean", C.c_void_p), ("rstd", C.c_void_p), ("G", C.c_int),
+                ("zs", C.c_int), ("zo", C.c_int), ("ns", C.c_int), ("zhw", C.c_int)]
 
 
 class orc_conv_t(C.Structure):
@@ -51,6 +52,7 @@ def lib():
         L.orc_prep_w.argtypes = [C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.orc_conv3.restype = C.c_int; L.orc_conv3.argtypes = [C.POINTER(orc_conv_t)]
         L.orc_conv3_staged.restype = C.c_int; L.orc_conv3_staged.argtypes = [C.POINTER(orc_conv_t), C.c_void_p]
+        L.orc_gn_row.restype = C.c_int; L.orc_gn_row.argtypes = [C.POINTER(orc_gn_t), C.c_int, C.c_int]
         L.orc_set_w4_2d.restype = None; L.orc_set_w4_2d.argtypes = [C.c_int]
         L.orc_fakeq_w4.restype = None; L.orc_fakeq_w4.argtypes = [C.c_void_p] + [C.c_int] * 5
         L.orc_conv2.restype = C.c_int; L.orc_conv2.argtypes = [C.POINTER(orc_conv_t), C.c_int]
@@ -85,10 +87,13 @@ def ptr(a):
     return a.ctypes.data if a is not None else None
 
 
-def gn(gamma=None, beta=None, mean=None, rstd=None, G=0):
+def gn(gamma=None, beta=None, mean=None, rstd=None, G=0, slab=None):
+    """slab = (zs, zo, ns, zhw): mean / rstd hold one row per (sample, z-slab), [n][ns][G] (src/nn_lp.h:15-18)."""
     g = orc_gn_t()
     if G:
         g.gamma, g.beta, g.mean, g.rstd, g.G = ptr(gamma), ptr(beta), ptr(mean), ptr(rstd), G
+        if slab:
+            g.zs, g.zo, g.ns, g.zhw = slab
     return g
 
 

@@ -20,7 +20,7 @@ def test_header_declares_the_forward_subset():
     for must in ["lp_conv_fwd_f8", "lp_conv_fwd_f4", "lp_conv_fwd_s2_f8", "lp_f32_to_mx8", "lp_f32_to_mx4", "lp_h16_to_mx8", "lp_mx8_to_f32", "lp_mx4_to_f32",
                  "lp_mx8_bytes", "lp_mx4_bytes", "lp_pred_input_mx", "lp_pred_input_mx8", "lp_gn_silu_apply_mx", "lp_add_mx", "lp_up2_fwd_mx", "lp_up2_fwd_mx_blocks",
                  "lp_conv1_fwd_mx", "lp_conv1_fwd_mx_h16", "lp_conv1_fwd_mx_h16_r", "lp_conv1_fwd_mx_r", "lp_gn_sums_mx", "lp_gn_sums_mx_n", "lp_check", "gnp_mk",
-                 "lp_gn_slab_any", "lp_wmemo_step", "lp_wmemo_clear", "lp_skip_get", "nn_skip_masks", "zw_win"]:
+                 "lp_gn_slab_any", "lp_gn_slab_reg", "lp_wmemo_step", "lp_wmemo_clear", "lp_skip_get", "nn_skip_masks", "zw_win"]:
         assert must in names, must
 
 
@@ -99,6 +99,20 @@ def test_size_helpers_and_no_device_behaviour():
     assert lib.lp_mx4_bytes(2, 128, 1000) == 2 * 4 * 1000 * 17
     assert lib.lp_mx8_bytes(1, 4, 10) == 10 * 9 and lib.lp_mx8_bytes(1, 12, 10) == 10 * 17 and lib.lp_mx4_bytes(1, 12, 10) == 10 * 9
     assert lib.lp_gn_slab_any() == 0
+    # the slab statistics registry is host state: gnp_mk copies a registered mean array's geometry, and only that array's (src/nn_fwd.cu:12-35)
+    lib.lp_gn_slab_reg(0x1000, 64, 3, 2, 4096)
+    try:
+        g = lib.gnp_mk(0x10, 0x20, 0x1000, 0x2000, 8)
+        assert lib.lp_gn_slab_any() == 1 and (g.G, g.zs, g.zo, g.ns, g.zhw) == (8, 64, 3, 2, 4096)
+        g = lib.gnp_mk(0x10, 0x20, 0x3000, 0x2000, 8)
+        assert (g.G, g.zs, g.zo, g.ns, g.zhw) == (8, 0, 0, 0, 0)
+        lib.lp_gn_slab_reg(0x1000, 32, 0, 4, 100)          # a second registration of the same array replaces the first
+        g = lib.gnp_mk(0x10, 0x20, 0x1000, 0x2000, 8)
+        assert (g.zs, g.zo, g.ns, g.zhw) == (32, 0, 4, 100)
+        lib.lp_gn_slab_reg(0x1000, 0, 0, 0, 0)              # ns <= 0 removes it
+        assert lib.lp_gn_slab_any() == 0 and lib.gnp_mk(0x10, 0x20, 0x1000, 0x2000, 8).ns == 0
+    finally:
+        lib.lp_gn_slab_reg(None, 0, 0, 0, 0)
     # standing alone the library answers the op-layer questions itself: every conv dense, no z-window (src/nn_lp.h:44-49, src/lp_common.cuh:42)
     from ufsm_amd import shape5, split_t
     sk = lib.lp_skip_get(shape5(1, 32, 8, 8, 16), split_t(), 1)

@@ -49,6 +49,15 @@ def test_reads_the_2d_weight_scale_key(tmp_path):
     assert rc == 0 and cfg.w4_2d == 1 and step == 3
 
 
+def test_reads_the_slab_statistics_keys(tmp_path):
+    # cfg.l0_norm 4 as unet_save writes it (src/unet.c:5577-5578, read at :5726); the other level-0 modes (1 none, 2 ema, 3 ws) stay refused
+    h = 'UFSM{"nlev":2,"widths":[32,64],"l0_norm":4,"l0_slab":16,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":3,"extra":{"l0_norm":2}}\n'
+    rc, cfg, n, step = read(tmp_path, h)
+    assert rc == 0 and (cfg.l0_norm, cfg.l0_slab) == (4, 16)
+    for mode in (1, 2, 3):
+        assert read(tmp_path, h.replace('"l0_norm":4,"l0_slab":16', '"l0_norm":%d' % mode))[0] == -2
+
+
 def test_rejects_foreign_files(tmp_path):
     assert read(tmp_path, "not a checkpoint\n")[0] == -1
     assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"scale_cond":1,"nparams":1}\n')[0] == -2      # voxel-size conditioning

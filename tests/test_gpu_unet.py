@@ -1,5 +1,7 @@
 """Whole-net parity: the C23 host graph (libufsm_host.so) over the HIP kernels against the same graph composed from oracle calls.
 Bar (north star): logits within 1e-2 of the oracle's (max-abs-rel); per-layer MX outputs differ only by neighbouring codes."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -445,4 +447,113 @@ def test_config3_full_size_forward_properties(gpu):
         orc.lib().orc_conv1_mx(8, orc.ptr(q), N, 32, D * D, orc.ptr(hw), orc.ptr(hb), head_out, g2, orc.ptr(want))
         gz = got.reshape(N, head_out, D, D * D)[:, :, z]
         assert np.abs(gz - want).max() / np.abs(want).max() < 1e-4, z
+    net.close()
+
+
+@pytest.mark.parametrize("bits,widths,dims,N,slab,infer", [(8, [32, 64], (16, 16, 16), 2, 8, 0), (8, [32, 64, 128], (16, 16, 32), 1, 4, 0), (4, [32, 64], (16, 16, 16), 1, 8, 0),
+                                                            (8, [24, 32], (16, 8, 16), 1, 8, 0), (8, [32, 64], (16, 16, 16), 1, 8, 8)])
+def test_unet_l0_norm_slab(gpu, tmp_path, bits, widths, dims, N, slab, infer):
+    """cfg.l0_norm 4 (src/unet.h:52-59, the kernel path of src/unet.c:992-1003): the four GroupNorms of level 0 and the head's input one take
+    their statistics per z-slab of l0_slab planes; every reader applies each plane's slab. The device statistics equal those of its own stored
+    tensors slab by slab, every layer equals the oracle conv on the inputs and statistics the device layer read, and the logits the oracle
+    head's. infer: also with the level-0 convs run in z-slabs of that many planes (unet_set_infer_slab): the same logits, byte for byte."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    rng = np.random.default_rng(sum(widths) + bits + slab)
+    D, H, W = dims
+    S, HW, ns = D * H * W, H * W, D // slab
+    cin, head_out, G = 4, 3, 8
+    net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits, l0_norm=4, l0_slab=slab), N, D, H, W, seed=11)
+    H0 = load_host()
+    for bad in (make_cfg(cin, [16, 32], l0_norm=4, l0_slab=slab), make_cfg(cin, [64, 64], l0_norm=4, l0_slab=slab), make_cfg(cin, widths, l0_norm=2)):
+        assert not H0.unet_create(C.byref(bad))                   # refused by name at creation, not in the forward
+    p = net.params()
+    lay, n = unet_ref.param_layout(cin, widths, head_out, 0)
+    assert n == p.size                                             # (the mode adds no parameters)
+    for k, (off, shp) in lay.items():
+        if k.endswith(".gamma"):
+            p[off:off + shp[0]] = rng.uniform(0.7, 1.3, shp[0])
+        if k.endswith(".beta") or (k.endswith(".b") and k != "head.b"):
+            p[off:off + shp[0]] = rng.uniform(-0.2, 0.2, shp[0])
+    net.set_params(p)
+    x = rng.standard_normal((N, cin, S)).astype(np.float32)
+    x[:, 0] *= np.repeat(np.linspace(0.5, 2.0, D), HW)[None]      # a drift along z: the slabs' statistics differ
+    dxq = to_mx(bits, x); xq = dxq.to_numpy(np.uint8)
+    dlog = DevBuf(N * head_out * S * 4)
+    assert net.forward_x(dxq.ptr, dlog.ptr) == 0
+    LP.check()
+    got = dlog.to_numpy(np.float32, (N, head_out, S))
+    dt = 3 if bits == 8 else 4
+    tens, stat, shapes = {"input": xq}, {}, {"input": (N, cin, D, H, W)}
+    for k, (name, ptr, shp) in enumerate(net.layer_outs()):
+        nb = (lib.lp_mx8_bytes if bits == 8 else lib.lp_mx4_bytes)(shp[0], shp[1], shp[2] * shp[3] * shp[4])
+        buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+        tens[name], shapes[name] = buf, shp
+        g, mp, rp = net.layer_stats(k)
+        if g:
+            rows = N * (ns if name in ("enc0.c1", "enc0.c2", "dec0.c1", "dec0.c2") else 1)
+            m = np.empty(rows * g, np.float32); r = np.empty(rows * g, np.float32)
+            lib.mi_d2h(m.ctypes.data, mp, m.nbytes); lib.mi_d2h(r.ctypes.data, rp, r.nbytes)
+            stat[name] = (g, m, r)
+    LP.check()
+    Pm = lambda key: np.ascontiguousarray(p[lay[key][0]:lay[key][0] + int(np.prod(lay[key][1]))].reshape(lay[key][1]))
+    l0 = ("enc0.c1", "enc0.c2", "dec0.c1", "dec0.c2")
+    for name in l0:                                                # statistics of the device's own stored tensor, slab by slab
+        g, m, r = stat[name]
+        mo, ro = unet_ref.slab_stats(bits, tens[name], N, widths[0], g, D, HW, slab)
+        assert np.allclose(m, mo, rtol=1e-5, atol=1e-6) and np.allclose(r, ro, rtol=1e-5), name
+        assert np.abs(m.reshape(N, ns, g)[:, 0] - m.reshape(N, ns, g)[:, -1]).max() > 1e-3 or name != "enc0.c1"
+
+    def gn_of(layer):
+        nm = unet_ref.norm_of(layer, 0)
+        if nm is None:
+            return None
+        g, m, r = stat[layer]
+        return orc.gn(Pm(nm + ".gamma"), Pm(nm + ".beta"), m, r, g, slab=(slab, 0, ns, HW) if layer in l0 else None)
+
+    for name, xl, x2l, stride, up in unet_ref.layer_inputs(widths):
+        n_, co, d_, h_, w_ = shapes[name]
+        xs = shapes[x2l] if up else shapes[xl]
+        ci = shapes[xl][1] + (shapes[x2l][1] if x2l else 0)
+        cb = 8 if (bits == 8 or ci <= 8) else 4
+        if stride == 2:
+            cb = 4 if (bits == 4 and ci == 32 and co <= 32) else 8
+        want_l, _ = orc.conv3(tens[xl], dt, N, ci, xs[2], xs[3], xs[4], Pm(name + ".w"), Pm(name + ".b"), co, dt, cbits=cb, stride=stride,
+                              x2=tens[x2l] if x2l else None, c_split=shapes[xl][1] if x2l else 0, up=up, gp=gn_of(xl), gp2=gn_of(x2l) if x2l else None,
+                              stem_tile=int(ci <= 8 and stride == 1))
+        frac, near = code_mismatch_fraction(bits, tens[name], want_l, N, co, d_ * h_ * w_)
+        assert frac < (0.02 if bits == 8 else 0.05) and near, (name, frac, near)
+    last = "dec0.c2"
+    want = np.zeros((N, head_out, S), np.float32)
+    hw_ = np.ascontiguousarray(Pm("head.w").reshape(head_out, widths[0]))
+    orc.lib().orc_conv1_mx(bits, orc.ptr(tens[last]), N, widths[0], S, orc.ptr(hw_), orc.ptr(Pm("head.b")), head_out, gn_of(last), orc.ptr(want))
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-5
+    if infer:
+        H_ = load_host()
+        for direct in (1, 0):
+            H_.unet_set_infer_slab(infer); H_.unet_set_slab_direct(direct)
+            try:
+                d2 = DevBuf(N * head_out * S * 4)
+                assert net.forward_x(dxq.ptr, d2.ptr) == 0
+                LP.check()
+            finally:
+                H_.unet_set_infer_slab(0); H_.unet_set_slab_direct(1)
+            assert np.array_equal(d2.to_numpy(np.float32, (N, head_out, S)), got), direct
+    # the mode travels with the checkpoint (src/unet.c:5577-5578, :5726): save -> peek -> create -> load gives the same logits
+    from ufsm_amd.unet import unet_cfg
+    path = str(tmp_path / "l0.ckpt")
+    assert net.save(path, step=5, extra="{}") == 0
+    head = open(path, "rb").readline().decode()
+    assert ',"l0_norm":4,"l0_slab":%d,"cin":' % slab in head
+    c2 = unet_cfg()
+    assert H0.unet_peek(path.encode(), C.byref(c2), None) == 0 and (c2.l0_norm, c2.l0_slab) == (4, slab)
+    c2.act_dt, c2.prec = bits, 0
+    twin = UNet(c2, N, D, H, W, seed=1)
+    assert twin.load(path) == 5
+    d3 = DevBuf(N * head_out * S * 4)
+    assert twin.forward_x(dxq.ptr, d3.ptr) == 0
+    LP.check()
+    assert np.array_equal(d3.to_numpy(np.float32, (N, head_out, S)), got)
+    plain = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits), N, D, H, W, seed=1)      # per-sample GroupNorm at level 0: another architecture
+    assert plain.load(path) == -1
+    plain.close(); twin.close()
     net.close()

@@ -33,9 +33,22 @@ def param_layout(cin, widths, head_out, down_norm=0):
     return lay, off
 
 
-def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0, acc64=0):
+def slab_stats(bits, y, N, c, g, D, HW, zs):
+    """cfg.l0_norm 4 (src/unet.c:992-1003): statistics [n][slab][G] of a stored level-0 tensor of at most 32 channels, slabs of zs planes: a pass
+    over the tensor seen as n * slabs samples of zs planes (one channel block: a slab is a sample of the same layout)."""
+    assert c <= 32 and D % zs == 0
+    ns = D // zs
+    sums = np.zeros((N * ns, g, 2), np.float64)
+    orc.lib().orc_gn_sums_mx(bits, orc.ptr(y), N * ns, c, g, zs * HW, orc.ptr(sums), 0, zs * HW)
+    mean = np.zeros(N * ns * g, np.float32); rstd = np.zeros(N * ns * g, np.float32)
+    orc.lib().orc_gn_finalize(orc.ptr(sums), N * ns * g, (c // g) * zs * HW, 1e-5, orc.ptr(mean), orc.ptr(rstd))
+    return mean, rstd
+
+
+def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0, acc64=0, l0_slab=0):
     """xq: MX bytes of the input. Returns (logits fp32 [N][head_out][S], {layer name: MX bytes}). acc64: the convs' contraction summed in
-    double and rounded once (else in fp32, block by block): two correct summation orders of the same graph."""
+    double and rounded once (else in fp32, block by block): two correct summation orders of the same graph. l0_slab > 0: cfg.l0_norm 4, the
+    level-0 GroupNorms on statistics per z-slab of that many planes."""
     lay, n = param_layout(cin, widths, head_out, down_norm)
     assert params.size == n
     P = lambda k: np.ascontiguousarray(params[lay[k][0]:lay[k][0] + int(np.prod(lay[k][1]))].reshape(lay[k][1]))
@@ -43,6 +56,17 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
     outs = {}
     Gof = lambda c: min(G, c)
     dims = [(D >> i, H >> i, W >> i) for i in range(L)]
+
+    live = []
+
+    def l0gn(i, norm, y, ms):
+        """the GroupNorm a reader of level i's tensor y applies: per-sample statistics ms, or, at level 0 under l0_slab, the tensor's per-slab ones"""
+        c, g = widths[i], Gof(widths[i])
+        if i == 0 and l0_slab:
+            m, r = slab_stats(bits, y, N, c, g, D, H * W, l0_slab)
+            live.append((m, r))                  # (the descriptor holds plain addresses)
+            return orc.gn(P(norm + ".gamma"), P(norm + ".beta"), m, r, g, slab=(l0_slab, 0, D // l0_slab, H * W)), (m, r)
+        return orc.gn(P(norm + ".gamma"), P(norm + ".beta"), ms[0], ms[1], g), ms
 
     def finalize(sums, c, S):
         g = Gof(c)
@@ -67,9 +91,10 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
         S = dims[i][0] * dims[i][1] * dims[i][2]
         a1, s1 = conv("enc%d.c1" % i, cur, ci, dims[i], gp=gin)
         m1, r1 = finalize(s1, widths[i], S)
-        a2, s2 = conv("enc%d.c2" % i, a1, widths[i], dims[i], gp=orc.gn(P("enc%d.n1.gamma" % i), P("enc%d.n1.beta" % i), m1, r1, Gof(widths[i])))
+        a2, s2 = conv("enc%d.c2" % i, a1, widths[i], dims[i], gp=l0gn(i, "enc%d.n1" % i, a1, (m1, r1))[0])
         m2, r2 = finalize(s2, widths[i], S)
-        blocks["enc%d" % i] = (a2, orc.gn(P("enc%d.n2.gamma" % i), P("enc%d.n2.beta" % i), m2, r2, Gof(widths[i])), (m2, r2))
+        g2, (m2, r2) = l0gn(i, "enc%d.n2" % i, a2, (m2, r2))
+        blocks["enc%d" % i] = (a2, g2, (m2, r2))
         if i < L - 1:
             cur, _ = conv("down%d" % i, a2, widths[i], dims[i], gp=blocks["enc%d" % i][1], stride=2, stats=False)
             if down_norm:                     # statistics of the stored down-conv output, applied by the next conv1 (src/unet.c:2974-2979)
@@ -84,9 +109,10 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
         S = dims[i][0] * dims[i][1] * dims[i][2]
         a1, s1 = conv("dec%d.c1" % i, coarse[0], widths[i + 1] + widths[i], dims[i], gp=coarse[1], x2=skip[0], c_split=widths[i + 1], up=1, gp2=skip[1])
         m1, r1 = finalize(s1, widths[i], S)
-        a2, s2 = conv("dec%d.c2" % i, a1, widths[i], dims[i], gp=orc.gn(P("dec%d.n1.gamma" % i), P("dec%d.n1.beta" % i), m1, r1, Gof(widths[i])))
+        a2, s2 = conv("dec%d.c2" % i, a1, widths[i], dims[i], gp=l0gn(i, "dec%d.n1" % i, a1, (m1, r1))[0])
         m2, r2 = finalize(s2, widths[i], S)
-        blocks["dec%d" % i] = (a2, orc.gn(P("dec%d.n2.gamma" % i), P("dec%d.n2.beta" % i), m2, r2, Gof(widths[i])), (m2, r2))
+        g2, (m2, r2) = l0gn(i, "dec%d.n2" % i, a2, (m2, r2))
+        blocks["dec%d" % i] = (a2, g2, (m2, r2))
     last = blocks["dec0"] if L > 1 else blocks["enc0"]
     S = D * H * W
     logits = np.zeros((N, head_out, S), np.float32)

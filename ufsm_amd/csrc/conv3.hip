@@ -199,6 +199,7 @@ static thread_local int g_stem_zc = 0;      // tuning knob (mi_conv_stem_zc): z 
 static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                      gnp_t gp, double *osum, int Go, split_t sp, bool rows) {
     const int Ci = xs.c, N = xs.n, D = sp.Di ? sp.Di : xs.d, Do = xs.d, H = xs.h, W = xs.w;      // D: the input's depth (z-range), Do: output planes
+    if (gp.G && gp.ns) mi_die("%s: slab-local GroupNorm statistics on an input of %d channels (the few-channel kernels form their coefficients per sample)", who, Ci);
     const int CP = rows ? 0 : Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = rows ? 2 : 32 / CP, NKB = rows ? 18 : (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2;
     conv_args a; memset(&a, 0, sizeof a);
     a.sx = x; a.sxdt = xbf; a.sCi = Ci;
@@ -260,7 +261,9 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // the MX output is planes [yzo, yzo + xs.d) of a depth-yD tensor
     if ((sp.Di || sp.zi0) && (stride != 1 || sp.zi0 < 0 || sp.zi0 + xs.d > sp.Di)) mi_die("%s: z-range %d + %d of depth %d (stride %d)", who, sp.zi0, xs.d, sp.Di, stride);
     if ((sp.yD || sp.yzo) && (stride != 1 || sp.yzo < 0 || sp.yzo + xs.d > sp.yD)) mi_die("%s: slab output %d + %d of depth %d (stride %d)", who, sp.yzo, xs.d, sp.yD, stride);
-    if (gp.ns || sp.gp2.ns) mi_die("%s: slab-local GroupNorm statistics are not supported", who);
+    // slab-local GroupNorm statistics (gnp_t.ns > 0, src/nn_lp.h:15-18): every GroupNorm + SiLU of a conv input is applied by the re-staging pass
+    // below, which runs once per slab the launch's input planes meet; the kernels never see statistics
+    if (gp.ns && sp.up) mi_die("%s: slab-local GroupNorm statistics on the upsampled segment are not supported (the skip segment's are)", who);
     // the op layer's masks and z-window (the reference's kernels ask the same before a launch: src/lp_f4fwd.cuh:1134-1223, src/nn_bwd.cu:89)
     { int za = 0, zb = 0; if (zw_win(xs.d, &za, &zb)) mi_die("%s: a z-window [%d, %d) is set; windows are not built here (inference forward only)", who, za, zb); }
     if (lp_skip_get(xs, sp, 1).m || nn_skip_masks(xs, sp)) mi_die("%s: the op layer asks for a masked (skip-empty) conv, which is not built here", who);
@@ -312,7 +315,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
             static int uph2 = -1;
             if (uph2 < 0) uph2 = getenv("UFSM_UP_H2") ? atoi(getenv("UFSM_UP_H2")) : 1;
             if (upseg) mi_restage_up_sub(segx[s], xbf, N, segC[s], D, H, W, g, Cg, st, fmt, zlo, zhi, sp.up == 2 || (sp.up == 1 && entry_fmt == 4 && uph2));
-            else mi_restage_sub(segx[s], xbf, N, segC[s], (size_t)(zhi - zlo) * H * W, g, Cg, cg0, st, fmt, S, (size_t)zlo * H * W);
+            else gn_for_slabs(who, g, H * W, zlo, zhi, [&](int z0, int z1, gnp_t gs) { mi_restage_sub(segx[s], xbf, N, segC[s], (size_t)(z1 - z0) * H * W, gs, Cg, cg0, st, fmt, S, (size_t)z0 * H * W); });
             a.xq[s] = st; a.xsc[s] = st + (size_t)N * nbp * S * mx_rb(32, fmt);
             a.nbs[s] = nbp; a.bws[s] = 32;
         }
@@ -502,8 +505,9 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
 // tensor of the same channels, for a tensor several convs read: they then take y as a plain input and stage it as stored. Channels a
 // multiple of 32. The bits of the convs' results do not change (the same pre-pass runs inside a conv otherwise).
 extern "C" int mi_conv_prestage(const void *x, int xdt, shape5 s, gnp_t gp, void *y, int ybits) {
-    if ((ybits != 8 && ybits != 4) || s.c % 32 || xdt < 0 || xdt > 4 || (gp.G > 0 && s.c % gp.G) || gp.ns) return -1;
-    mi_restage(x, xdt, s.n, s.c, (size_t)s.d * s.h * s.w, gp, s.c, 0, y, ybits);
+    if ((ybits != 8 && ybits != 4) || s.c % 32 || xdt < 0 || xdt > 4 || (gp.G > 0 && s.c % gp.G)) return -1;
+    const size_t hw = (size_t)s.h * s.w;
+    gn_for_slabs("mi_conv_prestage", gp, s.h * s.w, 0, s.d, [&](int z0, int z1, gnp_t gs) { mi_restage_sub(x, xdt, s.n, s.c, (size_t)(z1 - z0) * hw, gs, s.c, 0, y, ybits, (size_t)s.d * hw, (size_t)z0 * hw); });
     return 0;
 }
 extern "C" int lp_conv_fwd_f8(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp) {

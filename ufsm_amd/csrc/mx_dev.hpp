@@ -264,3 +264,20 @@ void mi_count_alloc(void);                  // bookkeeping: one more device allo
 enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_UPCOARSE = 5, MI_WS_GEMM = 6, MI_WS_ATTN = 7, MI_WS_NSLOTS = 8 };
 static inline unsigned nblk_(size_t n, unsigned b) { return (unsigned)((n + b - 1) / b); }
 [[noreturn]] void mi_die(const char *fmt, ...);
+// ---- slab-local GroupNorm statistics (gnp_t.ns > 0: src/nn_lp.h:15-18, src/lp_slab.cuh:7-12): the statistics hold one row per (sample,
+// z-slab), [n][ns][G]; plane z of the tensor reads row n * ns + clamp((z + zo) / zs, 0, ns - 1). The kernels here read ONE row per sample and
+// launch: the host walks the slabs that meet the planes a launch covers and hands each launch a gnp_t resolved to its slab (zs = 0, zo = the
+// slab's index), which d_gn_row turns into the row. ns == 0: the per-sample statistics, row n. ----
+__device__ __forceinline__ int d_gn_row(const gnp_t &g, int n) { return g.ns ? n * g.ns + g.zo : n; }
+// f(z0, z1, g) for the planes [z0, z1) of each slab that meets [zlo, zhi) (once, with g itself, for per-sample statistics); hw: the tensor's
+// voxels per plane, which the geometry must agree with
+template <class F> static void gn_for_slabs(const char *who, gnp_t g, int hw, int zlo, int zhi, F f) {
+    if (!g.G || !g.ns) { f(zlo, zhi, g); return; }
+    if (g.zs <= 0 || g.zo < 0 || g.zo >= g.zs || g.zhw != hw) mi_die("%s: slab-local GroupNorm geometry (zs %d, zo %d, ns %d, zhw %d) does not fit planes of %d voxels", who, g.zs, g.zo, g.ns, g.zhw, hw);
+    for (int s = 0; s < g.ns; s++) {
+        const long long a = s == 0 ? zlo : (long long)s * g.zs - g.zo, b = s == g.ns - 1 ? zhi : (long long)(s + 1) * g.zs - g.zo;
+        const int z0 = (int)(a > zlo ? a : zlo), z1 = (int)(b < zhi ? b : zhi);
+        if (z0 < z1) { gnp_t r = g; r.zs = 0; r.zo = s; f(z0, z1, r); }
+    }
+}
+

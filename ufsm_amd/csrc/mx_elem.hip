@@ -167,19 +167,21 @@ extern "C" void lp_pred_input_mx8(const uint8_t *ct, int W, float mean, float is
 // block's per-channel (mean, rstd, gamma, beta) are formed once per workgroup in LDS; the row is transformed in place eight channels at a time
 template <int BX, int BY, typename TI>
 __global__ void __launch_bounds__(256) gn_silu_rows_k(const void *__restrict__ xv, uint8_t *__restrict__ y, int N, int C, int G, size_t S,
-                                                      const float *__restrict__ gamma, const float *__restrict__ beta, const float *__restrict__ mean, const float *__restrict__ rstd) {
+                                                      const float *__restrict__ gamma, const float *__restrict__ beta, const float *__restrict__ mean, const float *__restrict__ rstd,
+                                                      size_t v0, size_t nv, int rs, int r0) {       // voxels [v0, v0 + nv) of each sample; statistics row n * rs + r0
     const int bw = mx_bw(C), nb = mx_nb(C);
     const int blk = (int)(blockIdx.y % (unsigned)nb), n = (int)(blockIdx.y / (unsigned)nb), c0 = blk * bw, live = min(bw, C - c0);
     __shared__ float4 co[32];
     if (threadIdx.x < 32) {
         const int c = c0 + (int)threadIdx.x;
         float4 q = make_float4(0.f, 0.f, 0.f, 0.f);
-        if ((int)threadIdx.x < live) { const int ng = n * G + c / (C / G); q = make_float4(mean[ng], rstd[ng], gamma[c], beta[c]); }
+        if ((int)threadIdx.x < live) { const int ng = (n * rs + r0) * G + c / (C / G); q = make_float4(mean[ng], rstd[ng], gamma[c], beta[c]); }
         co[threadIdx.x] = q;
     }
     __syncthreads();
-    const size_t v = blockIdx.x * (size_t)256 + threadIdx.x;
-    if (v >= S) return;
+    const size_t vi = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (vi >= nv) return;
+    const size_t v = v0 + vi;
     const size_t row = (size_t)blockIdx.y * S + v;
     float r[32];
     if (BX != 0) { const uint8_t *x = (const uint8_t *)xv; load_row<BX ? BX : 8>(x, mx_scp<BX ? BX : 8>(x, N, C, S), row, bw, r); }
@@ -203,14 +205,16 @@ __global__ void __launch_bounds__(256) gn_silu_rows_k(const void *__restrict__ x
 // the same for an MX source of 32-channel blocks, two lanes per row (each lane one contiguous 16-channel half in and out, the per-channel
 // mean / rstd / gamma / beta of the block in LDS): a wavefront reads and writes contiguous memory
 template <int BX, int BY>
-__global__ void __launch_bounds__(256) gn_silu_apply32_k(const uint8_t *x, uint8_t *y, int N, int C, int G, size_t S, const float *gamma, const float *beta, const float *mean, const float *rstd) {
+__global__ void __launch_bounds__(256) gn_silu_apply32_k(const uint8_t *x, uint8_t *y, int N, int C, int G, size_t S, const float *gamma, const float *beta, const float *mean, const float *rstd,
+                                                         size_t v0, size_t nv, int rs, int r0) {    // voxels [v0, v0 + nv) of each sample; statistics row n * rs + r0
     const int nb = C / 32, blk = blockIdx.y, n = blockIdx.z;
     __shared__ float4 co[32];                                      // (mean, rstd, gamma, beta) of the block's channels
-    if (threadIdx.x < 32) { const int c = blk * 32 + threadIdx.x, ng = n * G + c / (C / G); co[threadIdx.x] = make_float4(mean[ng], rstd[ng], gamma[c], beta[c]); }
+    if (threadIdx.x < 32) { const int c = blk * 32 + threadIdx.x, ng = (n * rs + r0) * G + c / (C / G); co[threadIdx.x] = make_float4(mean[ng], rstd[ng], gamma[c], beta[c]); }
     __syncthreads();
     const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;
-    const size_t v = t >> 1; const int hf = (int)(t & 1);
-    if (v >= S) return;
+    const int hf = (int)(t & 1);
+    if ((t >> 1) >= nv) return;
+    const size_t v = v0 + (t >> 1);
     constexpr int IB = BX * 2, OB = BY * 2;                        // bytes of a 16-channel half row
     const size_t row = ((size_t)n * nb + blk) * S + v;
     const uint8_t *xs = x + (size_t)N * nb * S * (IB * 2);
@@ -252,26 +256,37 @@ __global__ void __launch_bounds__(256) gn_silu_apply32_k(const uint8_t *x, uint8
     }
     if (!hf) ys[row] = (uint8_t)(e + 127);
 }
-extern "C" void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, const float *gamma, const float *beta, const float *mean, const float *rstd, void *y, int ydt) {
-    const size_t S = (size_t)s.d * s.h * s.w, n = (size_t)s.n * mx_nb(s.c) * S;
-    if (ydt != 3 && ydt != 4) mi_die("lp_gn_silu_apply_mx: output dtype %d is not MX", ydt);
-    if (G <= 0 || s.c % G) mi_die("lp_gn_silu_apply_mx: %d channels in %d groups", s.c, G);
-    if (!n) return;
+// voxels [v0, v0 + nv) of each sample, statistics row n * rs + r0
+static void gn_silu_apply_range(const void *x, int xdt, shape5 s, int G, const float *gamma, const float *beta, const float *mean, const float *rstd, void *y, int ydt,
+                                size_t v0, size_t nv, int rs, int r0) {
+    const size_t S = (size_t)s.d * s.h * s.w;
+    if (!nv) return;
     if (xdt >= 3 && s.c % 32 == 0) {
-        const dim3 grid(nblk_(2 * S, 256), (unsigned)(s.c / 32), (unsigned)s.n);
+        const dim3 grid(nblk_(2 * nv, 256), (unsigned)(s.c / 32), (unsigned)s.n);
         const uint8_t *xq = (const uint8_t *)x; uint8_t *yq = (uint8_t *)y;
-#define GS32(BX, BY) gn_silu_apply32_k<BX, BY><<<grid, 256>>>(xq, yq, s.n, s.c, G, S, gamma, beta, mean, rstd)
+#define GS32(BX, BY) gn_silu_apply32_k<BX, BY><<<grid, 256>>>(xq, yq, s.n, s.c, G, S, gamma, beta, mean, rstd, v0, nv, rs, r0)
         if (xdt == 3) { if (ydt == 3) GS32(8, 8); else GS32(8, 4); } else { if (ydt == 3) GS32(4, 8); else GS32(4, 4); }
 #undef GS32
         MICK();
         return;
     }
-#define GSA(BX, BY, TI) gn_silu_rows_k<BX, BY, TI><<<rows_grid(s.n, mx_nb(s.c), S), 256>>>(x, (uint8_t *)y, s.n, s.c, G, S, gamma, beta, mean, rstd)
+#define GSA(BX, BY, TI) gn_silu_rows_k<BX, BY, TI><<<rows_grid(s.n, mx_nb(s.c), nv), 256>>>(x, (uint8_t *)y, s.n, s.c, G, S, gamma, beta, mean, rstd, v0, nv, rs, r0)
 #define GSA_Y(BX, TI) do { if (ydt == 4) GSA(BX, 4, TI); else GSA(BX, 8, TI); } while (0)
     if (xdt == 4) GSA_Y(4, float); else if (xdt == 3) GSA_Y(8, float); else if (xdt == 2) GSA_Y(0, __half); else if (xdt == 1) GSA_Y(0, bf16_t); else GSA_Y(0, float);
 #undef GSA_Y
 #undef GSA
     MICK();
+}
+// a mean array registered with lp_gn_slab_reg holds one row per (sample, z-slab): each slab's planes with their row (the registry lookup of
+// the reference's to_gnp, src/nn_lp.h:18)
+extern "C" void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, const float *gamma, const float *beta, const float *mean, const float *rstd, void *y, int ydt) {
+    const size_t hw = (size_t)s.h * s.w, S = (size_t)s.d * hw, n = (size_t)s.n * mx_nb(s.c) * S;
+    if (ydt != 3 && ydt != 4) mi_die("lp_gn_silu_apply_mx: output dtype %d is not MX", ydt);
+    if (G <= 0 || s.c % G) mi_die("lp_gn_silu_apply_mx: %d channels in %d groups", s.c, G);
+    if (!n) return;
+    gn_for_slabs("lp_gn_silu_apply_mx", gnp_mk(gamma, beta, mean, rstd, G), s.h * s.w, 0, s.d, [&](int z0, int z1, gnp_t gs) {
+        gn_silu_apply_range(x, xdt, s, G, gamma, beta, mean, rstd, y, ydt, (size_t)z0 * hw, (size_t)(z1 - z0) * hw, gs.ns ? gs.ns : 1, gs.ns ? gs.zo : 0);
+    });
 }
 
 // ---- trilinear 2x upsample (src/lp_mx_gn.cu:34-73, :151-186): out[o] = .75 in[o/2] + .25 in[o/2 -+ 1] per axis, edge clamp ----
@@ -513,7 +528,7 @@ __global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const flo
     for (int i = threadIdx.x; i < CO; i += 256) sb[i] = b && co0 + i < Co ? b[co0 + i] : 0.f;
     for (int i = threadIdx.x; i < Ci; i += 256) {
         float a = 1.f, bb = 0.f;
-        if (gp.G) { const int ng = n * gp.G + i / (Ci / gp.G); a = gp.rstd[ng] * gp.gamma[i]; bb = fmaf(-gp.mean[ng], a, gp.beta[i]); }
+        if (gp.G) { const int ng = d_gn_row(gp, n) * gp.G + i / (Ci / gp.G); a = gp.rstd[ng] * gp.gamma[i]; bb = fmaf(-gp.mean[ng], a, gp.beta[i]); }
         sa[i] = a; sbb[i] = bb;
     }
     __syncthreads();
@@ -578,9 +593,21 @@ __global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const flo
     }
 }
 template <typename YT>
+static void conv1_launch_row(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, YT *y, gnp_t gp, size_t vb, size_t nv, size_t ly, const char *who);
+// voxels [vb, vb + nv) of every sample; with slab-local GroupNorm statistics one launch per slab the range meets (its voxels, its statistics row)
+template <typename YT>
 static void conv1_launch(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, YT *y, gnp_t gp, size_t vb, size_t nv, size_t ly, const char *who) {
+    if (!gp.G || !gp.ns || !nv) { conv1_launch_row<YT>(x, xdt, xs, w, b, cout, y, gp, vb, nv, ly, who); return; }
+    const size_t hw = (size_t)xs.h * xs.w;
+    gn_for_slabs(who, gp, xs.h * xs.w, (int)(vb / hw), (int)((vb + nv + hw - 1) / hw), [&](int z0, int z1, gnp_t gs) {
+        const size_t a = (size_t)z0 * hw > vb ? (size_t)z0 * hw : vb, e = (size_t)z1 * hw < vb + nv ? (size_t)z1 * hw : vb + nv;
+        if (a < e) conv1_launch_row<YT>(x, xdt, xs, w, b, cout, y + (a - vb), gs, a, e - a, ly, who);
+    });
+}
+template <typename YT>
+static void conv1_launch_row(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, YT *y, gnp_t gp, size_t vb, size_t nv, size_t ly, const char *who) {
     if (xdt != 3 && xdt != 4) mi_die("%s: input dtype %d is not MX", who, xdt);
-    if (gp.G && (gp.ns || xs.c % gp.G)) mi_die("%s: GroupNorm of %d channels in %d groups (slab-local statistics are not supported)", who, xs.c, gp.G);
+    if (gp.G && xs.c % gp.G) mi_die("%s: GroupNorm of %d channels in %d groups", who, xs.c, gp.G);
     if (xs.c > 1024) mi_die("%s: %d input channels (at most 1024)", who, xs.c);
     const size_t S = (size_t)xs.d * xs.h * xs.w;
     if (!nv || !xs.n) return;
@@ -633,7 +660,7 @@ __global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int
 #pragma unroll
         for (int k = 0; k < 32; k++) {
             const int c = blk * 32 + k;
-            if (c < C) { const int ng = n * gp.G + (cg0 + c) / cpg; const float a = gp.rstd[ng] * gp.gamma[cg0 + c], b = fmaf(-gp.mean[ng], a, gp.beta[cg0 + c]); r[k] = d_act_ab(r[k], a, b); }
+            if (c < C) { const int ng = d_gn_row(gp, n) * gp.G + (cg0 + c) / cpg; const float a = gp.rstd[ng] * gp.gamma[cg0 + c], b = fmaf(-gp.mean[ng], a, gp.beta[cg0 + c]); r[k] = d_act_ab(r[k], a, b); }
             else r[k] = 0.f;
         }
     }
@@ -649,7 +676,7 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
     __shared__ float sa[32], sb[32];
     if (threadIdx.x < 32) {
         float a = 1.f, b = 0.f;
-        if (gp.G) { const int c = cg0 + blk * 32 + threadIdx.x, ng = n * gp.G + c / (Cg / gp.G); a = gp.rstd[ng] * gp.gamma[c]; b = fmaf(-gp.mean[ng], a, gp.beta[c]); }
+        if (gp.G) { const int c = cg0 + blk * 32 + threadIdx.x, ng = d_gn_row(gp, n) * gp.G + c / (Cg / gp.G); a = gp.rstd[ng] * gp.gamma[c]; b = fmaf(-gp.mean[ng], a, gp.beta[c]); }
         sa[threadIdx.x] = a; sb[threadIdx.x] = b;
     }
     __syncthreads();

@@ -5,6 +5,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <mutex>
 
 static thread_local hipError_t g_err = hipSuccess;      // first error since the last lp_check (src/lp_common.cuh:35-38)
 static thread_local char g_errmsg[256];
@@ -114,10 +115,31 @@ extern "C" void mi_gn_sums_zero(double *sums, int nslots) {
     const size_t n = (size_t)nslots * 6;   // 24 bytes = 6 words
     fill_u32_k<<<nblk_(n, 256), 256>>>((unsigned *)sums, n, 0u); MICK();
 }
-extern "C" gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean, const float *rstd, int G) {   // src/nn_lp.h:19
-    gnp_t g; memset(&g, 0, sizeof g); g.gamma = gamma; g.beta = beta; g.mean = mean; g.rstd = rstd; g.G = G; return g;
+// ---- slab-local GroupNorm statistics (src/nn_lp.h:15-20, src/nn_fwd.cu:5-35): statistics arrays that hold one row per (sample, z-slab),
+// [n][ns][G], and their geometry; every gnp_t made by gnp_mk from a registered mean array carries it. ns <= 0 removes mean's entry, a null
+// mean clears the registry ----
+static struct { const float *mean; int zs, zo, ns, zhw; } g_slab[32];
+static int g_nslab = 0;
+static std::mutex g_slab_mu;
+extern "C" void lp_gn_slab_reg(const float *mean, int zs, int zo, int ns, int zhw) {
+    std::lock_guard<std::mutex> lk(g_slab_mu);
+    if (!mean) { g_nslab = 0; return; }
+    int i = 0;
+    while (i < g_nslab && g_slab[i].mean != mean) i++;
+    if (ns <= 0) { if (i < g_nslab) g_slab[i] = g_slab[--g_nslab]; return; }
+    if (zs <= 0 || zo < 0 || zo >= zs || zhw <= 0) mi_die("lp_gn_slab_reg: %d planes per slab, offset %d, %d voxels per plane", zs, zo, zhw);
+    if (i == g_nslab) { if (g_nslab == 32) mi_die("lp_gn_slab_reg: more than 32 slab statistics arrays"); g_nslab++; }
+    g_slab[i].mean = mean; g_slab[i].zs = zs; g_slab[i].zo = zo; g_slab[i].ns = ns; g_slab[i].zhw = zhw;
 }
-extern "C" int lp_gn_slab_any(void) { return 0; }
+extern "C" int lp_gn_slab_any(void) { std::lock_guard<std::mutex> lk(g_slab_mu); return g_nslab > 0; }
+extern "C" gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean, const float *rstd, int G) {   // src/nn_lp.h:19
+    gnp_t g; memset(&g, 0, sizeof g); g.gamma = gamma; g.beta = beta; g.mean = mean; g.rstd = rstd; g.G = G;
+    if (G > 0 && mean) {
+        std::lock_guard<std::mutex> lk(g_slab_mu);
+        for (int i = 0; i < g_nslab; i++) if (g_slab[i].mean == mean) { g.zs = g_slab[i].zs; g.zo = g_slab[i].zo; g.ns = g_slab[i].ns; g.zhw = g_slab[i].zhw; break; }
+    }
+    return g;
+}
 
 // ---- the op layer's answers about masked convs and the z-window (src/nn_skip.cu:130-157, src/nn_bwd.cu:57): weak, so the reference's own
 // definitions replace them when this library is linked into it; standing alone every conv is dense and no window is set ----

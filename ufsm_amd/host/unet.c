@@ -23,6 +23,7 @@ struct unet {
     unet_cfg cfg;
     /* the activations, built for one input shape and storage mode (rebuilt when either changes: src/unet.c:2876) */
     int built, act_dt, prec; shape5 in; shape5 ls[UNET_MAXLEV];
+    int l0s_zs, l0s_ns;                /* cfg.l0_norm 4: planes per statistics slab and slabs of the current build (0: per-sample statistics) */
     int slab_ip, slab_nl, slab_s;      /* the build's in-place slab plan: on, and over how many levels (a level's tensors all live in enc[i].a2's buffer) */
     void *slab_tmp[2], *slab_carry[2]; /* per such level: one slab of output planes, and the plane that waits for the next slab */
     block enc[UNET_MAXLEV], dec[UNET_MAXLEV];
@@ -66,7 +67,10 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     }
     if (c->ds_levels) return "ds_levels";
     if (c->lat_guide || c->lat_nsub) return "lat_guide";
-    if (c->l0_norm || c->l0_slab) return "l0_norm";
+    if (c->l0_norm && c->l0_norm != 4) return "l0_norm (only 0, GroupNorm, and 4, per z-slab statistics)";
+    if (c->l0_norm == 4 && c->widths[0] > 32) return "l0_norm 4 with more than 32 level-0 channels";   /* (one MX channel block: a slab is a sample of the same layout) */
+    if (c->l0_norm == 4 && c->widths[0] <= 16) return "l0_norm 4 with 16 or fewer level-0 channels";   /* (the few-channel conv kernels read per-sample statistics only) */
+    if (c->l0_slab && c->l0_norm != 4) return "l0_slab without l0_norm 4";
     if (c->gfilm) return "gfilm";
     if (c->gn_ema) return "gn_ema";
     if (c->attn_vres) return "attn_vres";
@@ -151,6 +155,7 @@ static void free_acts(unet *u) {
         for (int s = 0; s < 2; s++) {
             block *b = s ? &u->dec[i] : &u->enc[i];
             if (u->slab_ip && i < u->slab_nl) { if (s) b->a2 = nullptr; b->a1 = nullptr; }       /* (aliases of enc[i].a2) */
+            if (i == 0 && u->l0s_ns) { if (b->m1) lp_gn_slab_reg(b->m1, 0, 0, 0, 0); if (b->m2) lp_gn_slab_reg(b->m2, 0, 0, 0, 0); }
             act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2);
             b->a1 = b->a2 = nullptr; b->m1 = b->r1 = b->m2 = b->r2 = nullptr;
         }
@@ -161,7 +166,7 @@ static void free_acts(unet *u) {
     for (int i = 0; i < 2; i++) { act_del(u->slab_tmp[i]); act_del(u->slab_carry[i]); u->slab_tmp[i] = u->slab_carry[i] = nullptr; }
     act_del(u->xin); u->xin = nullptr;
     mi_free(u->logits); u->logits = nullptr;
-    u->built = 0; u->nouts = 0; u->slab_ip = u->slab_nl = u->slab_s = 0;
+    u->built = 0; u->nouts = 0; u->slab_ip = u->slab_nl = u->slab_s = 0; u->l0s_zs = u->l0s_ns = 0;
 }
 /* (re)build for input shape `in` under the storage mode and precision policy in force (build_acts, src/unet.c:2876) */
 static int build_acts(unet *u, shape5 in) {
@@ -169,8 +174,12 @@ static int build_acts(unet *u, shape5 in) {
     if (in.n < 1 || in.c != cfg->cin || in.d < 1 || in.h < 1 || in.w < 1) { fprintf(stderr, "unet: input shape %d x %d x %d x %d x %d does not fit a net of %d input channels\n", in.n, in.c, in.d, in.h, in.w, cfg->cin); return -1; }
     if ((in.d | in.h | in.w) & ((1 << (L - 1)) - 1)) { fprintf(stderr, "unet: spatial size %dx%dx%d must be divisible by %d\n", in.d, in.h, in.w, 1 << (L - 1)); abort(); }   /* (src/unet.c:2875) */
     if (!unet_act_mx()) { fprintf(stderr, "unet: this build stores activations as MX-fp8 or MX-fp4 only (unet_set_act_mx8 / unet_set_act_mx4)\n"); return -1; }
+    if (cfg->l0_norm == 4 && in.d % (cfg->l0_slab > 0 ? cfg->l0_slab : 64)) { fprintf(stderr, "unet: l0_norm 4 needs a depth (%d) that is a multiple of the %d planes of a statistics slab\n", in.d, cfg->l0_slab > 0 ? cfg->l0_slab : 64); return -1; }
     free_acts(u);
     u->in = in; u->act_dt = act_dt_now(); u->prec = nn_get_prec();
+    /* cfg.l0_norm 4 (src/unet.h:52-59; the kernel path of src/unet.c:992-1003): the four GroupNorms of level 0 take their statistics per z-slab of
+       l0_slab planes (0: 64). The statistics arrays hold [n][slab][G] and are registered with their geometry, which every reader's gnp_t then carries */
+    u->l0s_zs = cfg->l0_norm == 4 ? (cfg->l0_slab > 0 ? cfg->l0_slab : 64) : 0; u->l0s_ns = u->l0s_zs ? in.d / u->l0s_zs : 0;
     u->slab_ip = slab_inplace_now(u); u->slab_nl = u->slab_ip ? slab_levels(u) : 0; u->slab_s = u->slab_ip ? g_infer_slab : 0;
     for (int i = 0; i < L; i++) u->ls[i] = (shape5){in.n, w[i], in.d >> i, in.h >> i, in.w >> i};
     for (int i = 0; i < L; i++) {
@@ -180,8 +189,9 @@ static int build_acts(unet *u, shape5 in) {
             b->ys = u->ls[i]; b->xs = u->ls[i]; b->xs.c = b->c1.cin;
             if (i < u->slab_nl) { b->a2 = s ? u->enc[i].a2 : act_new(u, b->ys); b->a1 = b->a2; }
             else { b->a1 = act_new(u, b->ys); b->a2 = act_new(u, b->ys); }
-            const size_t ng = (size_t)in.n * G_of(u, w[i]);
+            const size_t ng = (size_t)in.n * G_of(u, w[i]) * (i == 0 && u->l0s_ns ? u->l0s_ns : 1);
             b->m1 = f32_new(ng); b->r1 = f32_new(ng); b->m2 = f32_new(ng); b->r2 = f32_new(ng);
+            if (i == 0 && u->l0s_ns) { lp_gn_slab_reg(b->m1, u->l0s_zs, 0, u->l0s_ns, in.h * in.w); lp_gn_slab_reg(b->m2, u->l0s_zs, 0, u->l0s_ns, in.h * in.w); }
         }
         if (i < L - 1) {
             shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds);
@@ -304,6 +314,9 @@ static void copy_planes(const unet *u, void *dst, int Dd, int d0, const void *sr
    (slab_run, src/unet.c:2499-2545) */
 static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t *gin, const void *xup, const nn_gn_t *gup, int c_split, const char *n1, const char *n2) {
     const int G = G_of(u, b->c1.cout), D = b->ys.d, ip = u->slab_ip && level < u->slab_nl;
+    /* per-slab statistics (level 0 under cfg.l0_norm 4): the convs reduce nothing; a pass over the stored output, seen as n * slabs samples of
+       l0_slab planes (one channel block: a slab is a sample of the same layout), fills the [n][slab][G] rows (src/unet.c:996-998) */
+    const int l0s = level == 0 && u->l0s_ns, Gc = l0s ? 0 : G;
     const int s = level >= slab_levels(u) ? 0 : g_infer_slab < D ? g_infer_slab : ip ? D : 0;      /* (in place: a level of fewer planes is one slab) */
     void *tmp = ip ? u->slab_tmp[level] : nullptr, *carry = ip ? u->slab_carry[level] : nullptr;
     int r = 0;
@@ -316,15 +329,19 @@ static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t 
             shape5 xs = conv == 1 ? b->xs : b->ys;
             if (s) { nn_set_zrange(z0, D, z0 == 0, last, D, z0); nn_set_zrange_out(!over); xs.d = sk; }
             void *o = over ? tmp : y;
-            if (conv == 2) r = nn_conv3d_fwd_gn_stats(b->a1, xs, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, o, G, 1e-5f, b->m2, b->r2);
-            else if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, G, 1e-5f, b->m1, b->r1);   /* [up2(coarse) | skip] */
-            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, G, 1e-5f, b->m1, b->r1);
+            if (conv == 2) r = nn_conv3d_fwd_gn_stats(b->a1, xs, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, o, Gc, 1e-5f, b->m2, b->r2);
+            else if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, b->m1, b->r1);   /* [up2(coarse) | skip] */
+            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, b->m1, b->r1);
             if (s) { nn_set_zrange(0, 0, 0, 0, 0, 0); nn_set_zrange_out(0); }
             if (over && !r) {                                      /* planes below the next slab's first input plane are dead: the last one waits */
                 if (k) copy_planes(u, y, D, z0 - 1, carry, 1, 0, 1, b->ys);
                 copy_planes(u, y, D, z0, tmp, sk, 0, last ? sk : sk - 1, b->ys);
                 if (!last) copy_planes(u, carry, 1, 0, tmp, sk, sk - 1, 1, b->ys);
             }
+        }
+        if (!r && l0s) {
+            shape5 ps = b->ys; ps.n *= u->l0s_ns; ps.d = u->l0s_zs;
+            if (nn_gn_stats(y, ps, G, 1e-5f, conv == 1 ? b->m1 : b->m2, conv == 1 ? b->r1 : b->r2)) { fprintf(stderr, "unet: per-slab GroupNorm statistics unsupported for this storage\n"); r = -1; }
         }
         if (!r) { if (conv == 1) note(u, b->a1, b->ys, n1, b->m1, b->r1, G); else note(u, b->a2, b->ys, n2, b->m2, b->r2, G); }
     }
@@ -460,6 +477,7 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     for (int i = 0; i < cfg->nlev; i++) { cfg->widths[i] = atoi(p); p = strchr(p, ','); if (!p) break; p++; }
     cfg->cin = key_int(line, "\"cin\":", 0); cfg->cout = key_int(line, "\"cout\":", 0); cfg->G = key_int(line, "\"G\":", 8);
     cfg->down_norm = key_int(line, "\"down_norm\":", 0); cfg->w4_2d = key_int(line, "\"w4_2d\":", 0);
+    cfg->l0_norm = key_int(line, "\"l0_norm\":", 0); cfg->l0_slab = key_int(line, "\"l0_slab\":", 0);      /* (src/unet.c:5726) */
     cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
     cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
     cfg->half_res = key_int(line, "\"half_res\":", 0); cfg->scan_norm = key_int(line, "\"scan_norm\":", 0);      /* (the caller's business: the graph does not use them) */
@@ -468,10 +486,11 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     /* architecture features this build's graph does not have */
     static const char *const no[] = {"\"dec_widths\":", "\"enc_blocks\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"ds_levels\":", "\"emb_lev\":",
                                      "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
-                                     "\"l0_norm\":", "\"skip_empty\":", "\"gfilm\":", "\"gn_ema\":", "\"dec_convs\":"};
+                                     "\"skip_empty\":", "\"gfilm\":", "\"gn_ema\":", "\"dec_convs\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
     if (!bad && key_int(line, "\"scale_cond\":", 0)) bad = "\"scale_cond\":";
+    if (!bad && cfg->l0_norm && cfg->l0_norm != 4) bad = "\"l0_norm\": (none / ema / ws)";
     if (!bad && cfg->attn_blocks && cfg->attn_pe != 1 && cfg->attn_pe != 2) bad = "\"attn_pe\": (PEG / scroll RoPE)";
     if (bad) { fprintf(stderr, "unet_peek: %s uses %s which this build does not run\n", path, bad); free(line); return -2; }
     free(line);
@@ -492,6 +511,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.attn_blocks != m->attn_blocks) bad = "attn_blocks";
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
+    if (!bad && (c.l0_norm != m->l0_norm || (c.l0_norm == 4 && (c.l0_slab > 0 ? c.l0_slab : 64) != (m->l0_slab > 0 ? m->l0_slab : 64)))) bad = "l0_norm / l0_slab";
     if (!bad && np != u->np) bad = "nparams";
     if (bad) { fprintf(stderr, "unet_load: %s: \"%s\" differs from this network's\n", path, bad); return -1; }
     FILE *f = fopen(path, "rb");
@@ -531,8 +551,11 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     fprintf(f, "UFSM{\"nlev\":%d,\"widths\":[", u->cfg.nlev);
     for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.widths[i]);
     fputc(']', f);
+    /* (the reference's key order, src/unet.c:5561-5578: w4_2d, the attention keys, l0_norm / l0_slab, then cin) */
+    if (u->cfg.w4_2d) fprintf(f, ",\"w4_2d\":%d", u->cfg.w4_2d);
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
-    if (u->cfg.w4_2d) fprintf(f, ",\"w4_2d\":%d", u->cfg.w4_2d);                                  /* (where src/unet.c:5561 writes it: before cin) */
+    if (u->cfg.l0_norm) fprintf(f, ",\"l0_norm\":%d", u->cfg.l0_norm);
+    if (u->cfg.l0_norm == 4) fprintf(f, ",\"l0_slab\":%d", u->cfg.l0_slab);
     fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":0,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.cout, u->cfg.G,
             u->cfg.down_norm, u->np, step);
     fprintf(f, ",\"extra\":%s}\n", extra ? extra : "{}");

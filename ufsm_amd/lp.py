@@ -49,6 +49,7 @@ _PROTOS = {
     "mi_conv_prestage": (_I, [_P, _I, shape5, gnp_t, _P, _I]),
     "gnp_mk": (gnp_t, [_P, _P, _P, _P, _I]),
     "lp_gn_slab_any": (_I, []),
+    "lp_gn_slab_reg": (None, [_P, _I, _I, _I, _I]),
     "lp_skip_get": (skipm_t, [shape5, split_t, _I]),
     "nn_skip_fwd_level": (_I, [shape5, split_t]),
     "nn_skip_masks": (_I, [shape5, split_t]),

@@ -78,7 +78,7 @@ def load_host():
     return L
 
 
-def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0, w4_2d=0):
+def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0):
     """The reference's configuration record plus, as Python attributes, what the reference keeps in process-wide switches: the activation
     storage (unet_set_act_mx4) and the compute precision policy (nn_set_prec), which UNet applies around its calls."""
     c = unet_cfg()
@@ -86,6 +86,7 @@ def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn
     c.attn_blocks, c.attn_pe, c.attn_reg, c.attn_mlp, c.down_norm, c.w4_2d = attn_blocks, attn_pe if attn_blocks else 0, attn_reg, attn_mlp, down_norm, w4_2d
     for i, w in enumerate(widths):
         c.widths[i] = w
+    c.l0_norm, c.l0_slab = l0_norm, l0_slab
     c.act_dt, c.prec = act_dt, prec
     return c
 
