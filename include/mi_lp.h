@@ -66,6 +66,11 @@ void lp_set_w4_2d(int on);
    nn_fakeq_w4_2d (src/nn.h:774): B x B blocks */
 void lp_fakeq_w4(float *w, int Co, int Ci, int T, int Bo, int Bi);
 void nn_fakeq_w4_2d(float *w, int Co, int Ci, int T, int B);
+/* the level-0 normalisation alternatives' device helpers (src/nn.h:465-477, src/nn_l0norm.cu): constant GroupNorm statistics for N samples (run
+   null: mean 0, rstd 1; else run = [mean G | var G] and rstd = 1 / sqrt(var + eps)); scaled weight standardisation per output channel over its
+   fan-in of n contiguous weights, wh = gain (w - mean) / (std sqrt(n) + eps) (wh may be w) */
+void nn_gn_const_fill(float *mean, float *rstd, const float *run, int N, int G, float eps);
+void nn_ws_fwd(float *wh, const float *w, int cout, int n, float gain, float eps);
 /* no counterpart in the reference (its stride-2 entry carries no split_t and prepares the weights per call): memo id of the calling thread's
    next lp_conv_fwd_s2_f8, as split_t.wkey for the stride-1 entries; consumed by that call. For inference loops with constant weights. */
 void mi_conv_s2_wkey(unsigned wkey);

@@ -37,7 +37,7 @@ def test_caller_side_keys_pass_through(tmp_path):
     assert rc == 0 and cfg.half_res == 1 and cfg.scan_norm == 1
 
 
-@pytest.mark.parametrize("feature", ['"dec_widths":[0,32]', '"enc_blocks":[0,1]', '"ds_levels":2', '"film":2', '"fstem":[2,16]', '"gn_ema":1,"ge_n":5', '"attn_vres":1', '"l0_norm":2'])
+@pytest.mark.parametrize("feature", ['"dec_widths":[0,32]', '"enc_blocks":[0,1]', '"ds_levels":2', '"film":2', '"fstem":[2,16]', '"gn_ema":1,"ge_n":5', '"attn_vres":1', '"l0_norm":7'])
 def test_refuses_architectures_it_does_not_run(tmp_path, feature):
     h = 'UFSM{"nlev":2,"widths":[32,64],%s,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":1,"extra":{}}\n' % feature
     assert read(tmp_path, h)[0] == -2
@@ -50,12 +50,15 @@ def test_reads_the_2d_weight_scale_key(tmp_path):
 
 
 def test_reads_the_slab_statistics_keys(tmp_path):
-    # cfg.l0_norm 4 as unet_save writes it (src/unet.c:5577-5578, read at :5726); the other level-0 modes (1 none, 2 ema, 3 ws) stay refused
+    # cfg.l0_norm as unet_save writes it (src/unet.c:5577-5584, read at :5726-5739): 4 with its slab depth, 1 (none) / 3 (ws) bare, 2 (ema) with the running statistics
     h = 'UFSM{"nlev":2,"widths":[32,64],"l0_norm":4,"l0_slab":16,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":3,"extra":{"l0_norm":2}}\n'
     rc, cfg, n, step = read(tmp_path, h)
     assert rc == 0 and (cfg.l0_norm, cfg.l0_slab) == (4, 16)
-    for mode in (1, 2, 3):
-        assert read(tmp_path, h.replace('"l0_norm":4,"l0_slab":16', '"l0_norm":%d' % mode))[0] == -2
+    for mode in (1, 3):
+        rc, cfg, n, step = read(tmp_path, h.replace('"l0_norm":4,"l0_slab":16', '"l0_norm":%d' % mode))
+        assert rc == 0 and (cfg.l0_norm, cfg.l0_slab) == (mode, 0)
+    rc, cfg, n, step = read(tmp_path, h.replace('"l0_norm":4,"l0_slab":16', '"l0_norm":2,"l0_n":40,"l0_warm":100,"l0_mom":0.01,"l0_run":[0.5,1,2]'))
+    assert rc == 0 and cfg.l0_norm == 2
 
 
 def test_rejects_foreign_files(tmp_path):

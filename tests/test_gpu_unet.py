@@ -464,7 +464,7 @@ def test_unet_l0_norm_slab(gpu, tmp_path, bits, widths, dims, N, slab, infer):
     cin, head_out, G = 4, 3, 8
     net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits, l0_norm=4, l0_slab=slab), N, D, H, W, seed=11)
     H0 = load_host()
-    for bad in (make_cfg(cin, [16, 32], l0_norm=4, l0_slab=slab), make_cfg(cin, [64, 64], l0_norm=4, l0_slab=slab), make_cfg(cin, widths, l0_norm=2)):
+    for bad in (make_cfg(cin, [16, 32], l0_norm=4, l0_slab=slab), make_cfg(cin, [64, 64], l0_norm=4, l0_slab=slab), make_cfg(cin, widths, l0_norm=7), make_cfg(cin, widths, l0_norm=0, l0_slab=8)):
         assert not H0.unet_create(C.byref(bad))                   # refused by name at creation, not in the forward
     p = net.params()
     lay, n = unet_ref.param_layout(cin, widths, head_out, 0)
@@ -556,4 +556,152 @@ def test_unet_l0_norm_slab(gpu, tmp_path, bits, widths, dims, N, slab, infer):
     plain = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits), N, D, H, W, seed=1)      # per-sample GroupNorm at level 0: another architecture
     assert plain.load(path) == -1
     plain.close(); twin.close()
+    net.close()
+
+
+def ws_f64(w, gain, eps=1e-5):
+    """scaled weight standardisation per output channel over its fan-in (src/nn_l0norm.cu:45-63), numpy fp64"""
+    w2 = w.reshape(w.shape[0], -1).astype(np.float64)
+    mu = w2.mean(1, keepdims=True); sd = np.sqrt(((w2 - mu) ** 2).mean(1, keepdims=True))
+    return ((w2 - mu) * (gain / (sd * np.sqrt(w2.shape[1]) + eps))).astype(np.float32).reshape(w.shape)
+
+
+def test_level0_norm_device_helpers(gpu):
+    """nn_gn_const_fill (src/nn_l0norm.cu:10-20) and nn_ws_fwd (:45-63) against their definitions and what the definitions imply: a standardised
+    fan-in has mean 0 and norm gain (up to eps), and is unchanged by a positive rescaling or a shift of the weights."""
+    rng = np.random.default_rng(3)
+    N, G = 3, 8
+    run = np.concatenate([rng.standard_normal(G), rng.uniform(0.1, 4, G)]).astype(np.float32)
+    dm, dr, drun = DevBuf(N * G * 4), DevBuf(N * G * 4), DevBuf.from_numpy(run)
+    lib.nn_gn_const_fill(dm.ptr, dr.ptr, None, N, G, 1e-5); LP.check()
+    assert (dm.to_numpy(np.float32) == 0).all() and (dr.to_numpy(np.float32) == 1).all()
+    lib.nn_gn_const_fill(dm.ptr, dr.ptr, drun.ptr, N, G, 1e-5); LP.check()
+    assert np.array_equal(dm.to_numpy(np.float32, (N, G)), np.broadcast_to(run[:G], (N, G)))
+    assert np.allclose(dr.to_numpy(np.float32, (N, G)), np.broadcast_to(1 / np.sqrt(run[G:].astype(np.float64) + 1e-5), (N, G)), rtol=3e-7)
+    for cout, n, gain in ((32, 4 * 27, 1.0), (32, 32 * 27, 1.7), (5, 96 * 27, 0.5), (7, 50, 2.0)):
+        w = (rng.standard_normal((cout, n)) * rng.uniform(0.01, 3, (cout, 1)) + rng.uniform(-1, 1, (cout, 1))).astype(np.float32)
+        dw, dh = DevBuf.from_numpy(w), DevBuf(w.nbytes)
+        lib.nn_ws_fwd(dh.ptr, dw.ptr, cout, n, gain, 1e-5); LP.check()
+        h = dh.to_numpy(np.float32, (cout, n))
+        assert np.abs(h - ws_f64(w, gain)).max() <= 2e-7 * np.abs(h).max()
+        assert np.abs(h.astype(np.float64).mean(1)).max() < 1e-7 and np.allclose(np.linalg.norm(h.astype(np.float64), axis=1), gain, rtol=1e-3)
+        w2 = (w.astype(np.float64) * 4 + 0.5).astype(np.float32)          # (exact: a power-of-two scale and a shift within the mantissa)
+        d2 = DevBuf.from_numpy(w2)
+        lib.nn_ws_fwd(d2.ptr, d2.ptr, cout, n, gain, 1e-5); LP.check()   # in place
+        assert np.abs(d2.to_numpy(np.float32, (cout, n)) - h).max() <= 1e-4 * np.abs(h).max()
+
+
+@pytest.mark.parametrize("mode,bits,widths", [(1, 8, [32, 64]), (3, 8, [32, 64]), (2, 8, [32, 64]), (3, 4, [32, 64, 128]), (2, 8, [16, 32])])
+def test_unet_l0_norm_constant_modes(gpu, tmp_path, mode, bits, widths):
+    """cfg.l0_norm 1 (none), 2 (ema) and 3 (ws) (src/unet.h:52-58): the four level-0 GroupNorms and the head's input one read constant statistics
+    (mean 0 / rstd 1, or the checkpoint's running statistics once their warm-up is over); ws also standardises the four level-0 convs' weights.
+    Every layer equals the oracle conv on the device layer's inputs with those statistics and weights; the logits equal the oracle head's."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    H0 = load_host()
+    rng = np.random.default_rng(mode * 7 + bits)
+    N, (D, H, W) = 2, (8, 16, 16)
+    S = D * H * W
+    cin, head_out, G = 4, 3, 8
+    net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits, l0_norm=mode), N, D, H, W, seed=13)
+    p = net.params()
+    lay, n = unet_ref.param_layout(cin, widths, head_out, 0)
+    assert n == p.size
+    for k, (off, shp) in lay.items():
+        if k.endswith(".gamma"):
+            p[off:off + shp[0]] = rng.uniform(0.7, 1.3, shp[0])
+        if k.endswith(".beta") or (k.endswith(".b") and k != "head.b"):
+            p[off:off + shp[0]] = rng.uniform(-0.2, 0.2, shp[0])
+    net.set_params(p)
+    x = rng.standard_normal((N, cin, S)).astype(np.float32)
+    dxq = to_mx(bits, x); xq = dxq.to_numpy(np.uint8)
+    l0 = ("enc0.c1", "enc0.c2", "dec0.c1", "dec0.c2")
+    g0 = min(G, widths[0])
+    run = None
+    if mode == 2:
+        # a fresh net is in its warm-up (no updates yet): live GroupNorm statistics, the logits of the same weights under cfg.l0_norm 0
+        assert H0.unet_l0_updates(net.h) == 0
+        plain = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits), N, D, H, W, seed=1); plain.set_params(p)
+        da, db = DevBuf(N * head_out * S * 4), DevBuf(N * head_out * S * 4)
+        assert net.forward_x(dxq.ptr, da.ptr) == 0 and plain.forward_x(dxq.ptr, db.ptr) == 0
+        LP.check()
+        assert np.array_equal(da.to_numpy(np.float32), db.to_numpy(np.float32))
+        plain.close()
+        # a checkpoint past its warm-up: the header carries [live: 4 sites x (mean G | var G)][EMA weights: the same] (src/unet.c:5579-5584)
+        path = str(tmp_path / "ema.ckpt")
+        assert net.save(path, step=9, extra="{}") == 0
+        raw = open(path, "rb").read(); head = raw[:raw.index(b"\n") + 1].decode()
+        assert ',"l0_norm":2,"l0_n":0,"l0_warm":100,"l0_mom":0.00999999978,"l0_run":[0,' in head
+        run = np.concatenate([np.concatenate([rng.uniform(-0.3, 0.3, g0), rng.uniform(0.3, 2.0, g0)]) for _ in range(8)]).astype(np.float32)
+        i0, i1 = head.index(',"l0_n":'), head.index(']', head.index('"l0_run":[')) + 1
+        new = head[:i0] + ',"l0_n":250,"l0_warm":200,"l0_mom":0.01,"l0_run":[' + ",".join("%.9g" % v for v in run) + "]" + head[i1:]
+        open(path, "wb").write(new.encode() + raw[len(head.encode()):])
+        assert net.load(path) == 9 and H0.unet_l0_updates(net.h) == 250
+    dlog = DevBuf(N * head_out * S * 4)
+    assert net.forward_x(dxq.ptr, dlog.ptr) == 0
+    LP.check()
+    got = dlog.to_numpy(np.float32, (N, head_out, S))
+    dt = 3 if bits == 8 else 4
+    tens, stat, shapes = {"input": xq}, {}, {"input": (N, cin, D, H, W)}
+    for k, (name, ptr, shp) in enumerate(net.layer_outs()):
+        nb = (lib.lp_mx8_bytes if bits == 8 else lib.lp_mx4_bytes)(shp[0], shp[1], shp[2] * shp[3] * shp[4])
+        buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+        tens[name], shapes[name] = buf, shp
+        g, mp, rp = net.layer_stats(k)
+        if g:
+            m = np.empty(N * g, np.float32); r = np.empty(N * g, np.float32)
+            lib.mi_d2h(m.ctypes.data, mp, m.nbytes); lib.mi_d2h(r.ctypes.data, rp, r.nbytes)
+            stat[name] = (g, m, r)
+    LP.check()
+    for site, name in enumerate(l0):                               # the constants every level-0 reader saw
+        g, m, r = stat[name]
+        if mode == 2:
+            rs = run[site * 2 * g0:(site + 1) * 2 * g0]
+            assert np.array_equal(m.reshape(N, g), np.broadcast_to(rs[:g0], (N, g)))
+            assert np.allclose(r.reshape(N, g), np.broadcast_to(1 / np.sqrt(rs[g0:].astype(np.float64) + 1e-5), (N, g)), rtol=3e-7)
+        else:
+            assert (m == 0).all() and (r == 1).all(), name
+    Pm = lambda key: np.ascontiguousarray(p[lay[key][0]:lay[key][0] + int(np.prod(lay[key][1]))].reshape(lay[key][1]))
+    # 1 / std(silu(z)), z ~ N(0, 1), by the quadrature of src/unet.c:543-547
+    zz = np.arange(-24000, 24001) * 5e-4; pz = np.exp(-0.5 * zz * zz) * 5e-4 / np.sqrt(2 * np.pi); yz = zz / (1 + np.exp(-zz))
+    gain = 1.0 / np.sqrt((pz * yz * yz).sum() - (pz * yz).sum() ** 2)
+    zs_ = np.random.default_rng(0).standard_normal(2_000_000); ys_ = zs_ / (1 + np.exp(-zs_))
+    assert abs(gain - 1.0 / ys_.std()) < 5e-3                      # (the same moment by sampling)
+
+    def Wt(name):
+        w = Pm(name + ".w")
+        return ws_f64(w, 1.0 if name == "enc0.c1" else gain) if (mode == 3 and name in l0) else w
+
+    def gn_of(layer):
+        nm = unet_ref.norm_of(layer, 0)
+        if nm is None:
+            return None
+        g, m, r = stat[layer]
+        return orc.gn(Pm(nm + ".gamma"), Pm(nm + ".beta"), m, r, g)
+
+    for name, xl, x2l, stride, up in unet_ref.layer_inputs(widths):
+        n_, co, d_, h_, w_ = shapes[name]
+        xs = shapes[x2l] if up else shapes[xl]
+        ci = shapes[xl][1] + (shapes[x2l][1] if x2l else 0)
+        cb = 8 if (bits == 8 or ci <= 8) else 4
+        if stride == 2:
+            cb = 4 if (bits == 4 and ci == 32 and co <= 32) else 8
+        want_l, _ = orc.conv3(tens[xl], dt, N, ci, xs[2], xs[3], xs[4], Wt(name), Pm(name + ".b"), co, dt, cbits=cb, stride=stride,
+                              x2=tens[x2l] if x2l else None, c_split=shapes[xl][1] if x2l else 0, up=up, gp=gn_of(xl), gp2=gn_of(x2l) if x2l else None,
+                              stem_tile=int(ci <= 8 and stride == 1))
+        frac, near = code_mismatch_fraction(bits, tens[name], want_l, N, co, d_ * h_ * w_)
+        assert frac < (0.02 if bits == 8 else 0.05) and near, (name, frac, near)
+    want = np.zeros((N, head_out, S), np.float32)
+    hw_ = np.ascontiguousarray(Pm("head.w").reshape(head_out, widths[0]))
+    orc.lib().orc_conv1_mx(bits, orc.ptr(tens["dec0.c2"]), N, widths[0], S, orc.ptr(hw_), orc.ptr(Pm("head.b")), head_out, gn_of("dec0.c2"), orc.ptr(want))
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-5
+    if mode == 3:                                                  # the standardisation follows the weights: the EMA copy's own, and a parameter update
+        path = str(tmp_path / "ws.ckpt")
+        assert net.save(path, step=1, extra="{}") == 0 and ',"l0_norm":3,"cin":' in open(path, "rb").readline().decode()
+        twin = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits, l0_norm=3), N, D, H, W, seed=2)
+        assert twin.load(path) == 1
+        d2 = DevBuf(N * head_out * S * 4)
+        assert twin.forward_x(dxq.ptr, d2.ptr) == 0
+        LP.check()
+        assert np.array_equal(d2.to_numpy(np.float32, (N, head_out, S)), got)
+        twin.close()
     net.close()

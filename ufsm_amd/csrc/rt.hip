@@ -115,6 +115,41 @@ extern "C" void mi_gn_sums_zero(double *sums, int nslots) {
     const size_t n = (size_t)nslots * 6;   // 24 bytes = 6 words
     fill_u32_k<<<nblk_(n, 256), 256>>>((unsigned *)sums, n, 0u); MICK();
 }
+// ---- constant GroupNorm statistics for N samples (src/nn.h:465-473, src/nn_l0norm.cu:10-20): run null: mean 0, rstd 1; else run = [mean G | var G] ----
+__global__ void gn_const_k(float *mean, float *rstd, const float *run, int NG, int G, float eps) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= NG) return;
+    const int g = i % G;
+    mean[i] = run ? run[g] : 0.f;
+    rstd[i] = run ? 1.f / sqrtf(run[G + g] + eps) : 1.f;
+}
+extern "C" void nn_gn_const_fill(float *mean, float *rstd, const float *run, int N, int G, float eps) {
+    if (N * G > 0) { gn_const_k<<<nblk_((size_t)N * G, 64), 64>>>(mean, rstd, run, N * G, G, eps); MICK(); }
+}
+// ---- scaled weight standardisation (src/nn.h:477, src/nn_l0norm.cu:45-63): per output channel over its fan-in of n contiguous weights,
+// wh = gain (w - mean) / (std sqrt(n) + eps), mean and population std in double. One wavefront per output channel (a fan-in is 108 .. a few
+// thousand weights): a lane sums every 64th weight, the moments meet through lane exchanges ----
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__global__ void __launch_bounds__(256) ws_fwd_k(float *wh, const float *w, int cout, int n, float gain, float eps) {
+    const int o = blockIdx.x * 4 + (int)(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (o >= cout) return;
+    const float *wo = w + (size_t)o * n; float *ho = wh + (size_t)o * n;
+    double s = 0.0;
+    for (int i = lane; i < n; i += 64) s += (double)wo[i];
+    const double mu = wave_sum_f64(s) / n;
+    double v = 0.0;
+    for (int i = lane; i < n; i += 64) { const double d = (double)wo[i] - mu; v += d * d; }
+    const double sd = sqrt(wave_sum_f64(v) / n), sc = (double)gain / (sd * sqrt((double)n) + (double)eps);
+    for (int i = lane; i < n; i += 64) ho[i] = (float)(((double)wo[i] - mu) * sc);
+}
+extern "C" void nn_ws_fwd(float *wh, const float *w, int cout, int n, float gain, float eps) {
+    if (cout > 0 && n > 0) { ws_fwd_k<<<nblk_((size_t)cout, 4), 256>>>(wh, w, cout, n, gain, eps); MICK(); }
+}
+
 // ---- slab-local GroupNorm statistics (src/nn_lp.h:15-20, src/nn_fwd.cu:5-35): statistics arrays that hold one row per (sample, z-slab),
 // [n][ns][G], and their geometry; every gnp_t made by gnp_mk from a registered mean array carries it. ns <= 0 removes mean's entry, a null
 // mean clears the registry ----

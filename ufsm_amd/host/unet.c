@@ -23,6 +23,9 @@ struct unet {
     unet_cfg cfg;
     /* the activations, built for one input shape and storage mode (rebuilt when either changes: src/unet.c:2876) */
     int built, act_dt, prec; shape5 in; shape5 ls[UNET_MAXLEV];
+    /* cfg.l0_norm 1 .. 3 (src/unet.h:52-58): the level-0 GroupNorms on constant statistics: mean 0 / rstd 1 (none, ws) or the checkpoint's running
+       statistics once its warm-up is over (ema: l0run = [live weights: 4 sites x (mean G | var G)][EMA weights: the same], device; l0_n updates so far) */
+    float *l0run; long l0_n; int l0_warm; float l0_mom; float ws_gain;
     int l0s_zs, l0s_ns;                /* cfg.l0_norm 4: planes per statistics slab and slabs of the current build (0: per-sample statistics) */
     int slab_ip, slab_nl, slab_s;      /* the build's in-place slab plan: on, and over how many levels (a level's tensors all live in enc[i].a2's buffer) */
     void *slab_tmp[2], *slab_carry[2]; /* per such level: one slab of output planes, and the plane that waits for the next slab */
@@ -67,7 +70,8 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     }
     if (c->ds_levels) return "ds_levels";
     if (c->lat_guide || c->lat_nsub) return "lat_guide";
-    if (c->l0_norm && c->l0_norm != 4) return "l0_norm (only 0, GroupNorm, and 4, per z-slab statistics)";
+    if (c->l0_norm < 0 || c->l0_norm > 4) return "l0_norm (0 GroupNorm, 1 none, 2 ema, 3 ws, 4 slab)";
+    if (c->l0_norm == 2 && (c->G < c->widths[0] ? c->G : c->widths[0]) > 64) return "l0_norm 2 with more than 64 groups";
     if (c->l0_norm == 4 && c->widths[0] > 32) return "l0_norm 4 with more than 32 level-0 channels";   /* (one MX channel block: a slab is a sample of the same layout) */
     if (c->l0_norm == 4 && c->widths[0] <= 16) return "l0_norm 4 with 16 or fewer level-0 channels";   /* (the few-channel conv kernels read per-sample statistics only) */
     if (c->l0_slab && c->l0_norm != 4) return "l0_slab without l0_norm 4";
@@ -126,7 +130,14 @@ unet *unet_create(const unet_cfg *cfg) {
     }
     u->np = off;
     u->p = f32_new(off); u->ema = f32_new(off); u->params = u->src = u->p;
-    if (cfg->w4_2d) { u->wm = f32_new(off); u->params = u->wm; }
+    if (cfg->w4_2d || cfg->l0_norm == 3) { u->wm = f32_new(off); u->params = u->wm; }
+    if (cfg->l0_norm == 3) {           /* 1 / std(silu(z)), z ~ N(0, 1): the gain of the convs that read a SiLU output (the quadrature of src/unet.c:543-547) */
+        double s1 = 0, s2 = 0;
+        for (int i = -24000; i <= 24000; i++) { const double z = i * 5e-4, p = exp(-0.5 * z * z) * 5e-4 / sqrt(2 * 3.14159265358979323846), y = z / (1 + exp(-z)); s1 += p * y; s2 += p * y * y; }
+        u->ws_gain = (float)(1.0 / sqrt(s2 - s1 * s1));
+    }
+    u->l0_mom = 0.01f; u->l0_warm = 100;                          /* (src/unet.c:549) */
+    if (cfg->l0_norm == 2) u->l0run = f32_new((size_t)16 * G_of(u, w[0]));
     return u;
 }
 /* inference in z-slabs (src/unet.h:422-424, src/unet.c:2499-2550): the convs of level 0 (and of level 1 in nets of three or more levels,
@@ -227,7 +238,7 @@ void unet_free(unet *u) {
     if (!u) return;
     mi_sync();
     free_acts(u);
-    mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm);
+    mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm); if (u->l0run) mi_free(u->l0run);
     lp_wmemo_clear();
     free(u);
 }
@@ -251,10 +262,16 @@ static void fw_refresh(unet *u) {
     if (!u->wm || u->wm_ok) return;
     mi_d2d(u->wm, u->src, u->np * 4);
     const int L = u->cfg.nlev;
-    const convp *cs[4 * UNET_MAXLEV]; int n = 0;
-    for (int i = 0; i < L; i++) { if (i) cs[n++] = &u->enc[i].c1; cs[n++] = &u->enc[i].c2; }
-    for (int i = 0; i < L - 1; i++) { cs[n++] = &u->dec[i].c1; cs[n++] = &u->dec[i].c2; }
-    for (int i = 0; i < n; i++) nn_fakeq_w4_2d(u->wm + cs[i]->w, cs[i]->cout, cs[i]->cin, 27, 32);
+    if (u->cfg.l0_norm == 3) {         /* ws: the four level-0 3^3 convs standardised per output channel over its fan-in; the network input conv without the SiLU gain (src/unet.c:5298-5304, :5311-5318) */
+        const convp *wc[4] = {&u->enc[0].c1, &u->enc[0].c2, &u->dec[0].c1, &u->dec[0].c2};
+        for (int i = 0; i < (L > 1 ? 4 : 2); i++) nn_ws_fwd(u->wm + wc[i]->w, u->src + wc[i]->w, wc[i]->cout, wc[i]->cin * 27, i ? u->ws_gain : 1.f, 1e-5f);
+    }
+    if (u->cfg.w4_2d) {
+        const convp *cs[4 * UNET_MAXLEV]; int n = 0;
+        for (int i = 0; i < L; i++) { if (i) cs[n++] = &u->enc[i].c1; cs[n++] = &u->enc[i].c2; }
+        for (int i = 0; i < L - 1; i++) { cs[n++] = &u->dec[i].c1; cs[n++] = &u->dec[i].c2; }
+        for (int i = 0; i < n; i++) nn_fakeq_w4_2d(u->wm + cs[i]->w, cs[i]->cout, cs[i]->cin, 27, 32);
+    }
     lp_wmemo_clear();
     u->wm_ok = 1;
 }
@@ -310,13 +327,24 @@ static void copy_planes(const unet *u, void *dst, int Dd, int d0, const void *sr
     mi_d2d_rows((char *)dst + (size_t)d0 * hw * rb, Sd * rb, (const char *)src + (size_t)s0 * hw * rb, Ss * rb, (size_t)n * hw * rb, rows);
     mi_d2d_rows((char *)dst + rows * Sd * rb + (size_t)d0 * hw, Sd, (const char *)src + rows * Ss * rb + (size_t)s0 * hw, Ss, (size_t)n * hw, rows);
 }
+/* cfg.l0_norm 1 / 3 always, 2 once the running statistics' warm-up is over (src/unet.c:2315): the level-0 GroupNorms read constant statistics,
+   written at the start of every forward (src/unet.c:2318-2323) */
+static int l0_const(const unet *u) { const int md = u->cfg.l0_norm; return md == 1 || md == 3 || (md == 2 && u->l0_n > 0 && u->l0_n >= u->l0_warm); }
+static void l0_const_fill(unet *u) {
+    const int G = G_of(u, u->cfg.widths[0]), N = u->in.n;
+    for (int i = 0; i < (u->cfg.nlev > 1 ? 2 : 1); i++) for (int k = 1; k <= 2; k++) {
+        block *b = i ? &u->dec[0] : &u->enc[0];
+        const float *run = u->cfg.l0_norm == 2 ? u->l0run + (u->src == u->ema ? (size_t)8 * G : 0) + (size_t)(2 * i + k - 1) * 2 * G : nullptr;      /* (the EMA weights have their own) */
+        nn_gn_const_fill(k == 1 ? b->m1 : b->m2, k == 1 ? b->r1 : b->r2, run, N, G, 1e-5f);
+    }
+}
 /* conv1 -> a1 (+ its statistics), conv2 reads silu(gn(a1)) while staging -> a2 (+ statistics) (src/unet.c:2567-2636); in z-slabs when asked for
    (slab_run, src/unet.c:2499-2545) */
 static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t *gin, const void *xup, const nn_gn_t *gup, int c_split, const char *n1, const char *n2) {
     const int G = G_of(u, b->c1.cout), D = b->ys.d, ip = u->slab_ip && level < u->slab_nl;
     /* per-slab statistics (level 0 under cfg.l0_norm 4): the convs reduce nothing; a pass over the stored output, seen as n * slabs samples of
        l0_slab planes (one channel block: a slab is a sample of the same layout), fills the [n][slab][G] rows (src/unet.c:996-998) */
-    const int l0s = level == 0 && u->l0s_ns, Gc = l0s ? 0 : G;
+    const int l0s = level == 0 && u->l0s_ns, Gc = l0s || (level == 0 && l0_const(u)) ? 0 : G;       /* (constant statistics: nothing to reduce either) */
     const int s = level >= slab_levels(u) ? 0 : g_infer_slab < D ? g_infer_slab : ip ? D : 0;      /* (in place: a level of fewer planes is one slab) */
     void *tmp = ip ? u->slab_tmp[level] : nullptr, *carry = ip ? u->slab_carry[level] : nullptr;
     int r = 0;
@@ -373,6 +401,7 @@ static int graph_fwd(unet *u, const void *x) {
     static const char *dwn[] = {"down0", "down1", "down2", "down3", "down4", "down5", "down6"};
     const int L = u->cfg.nlev;
     u->nouts = 0;
+    if (l0_const(u)) l0_const_fill(u);
     const void *cur = x;
     for (int i = 0; i < L; i++) {
         nn_gn_t gd; const nn_gn_t *gin = nullptr;                  /* down_norm: conv1 reads silu(gn(down conv output)) (src/unet.c:2593) */
@@ -463,7 +492,9 @@ static char *header_line(FILE *f) {                                /* the first 
     free(s); return nullptr;
 }
 static int key_int(const char *line, const char *key, int dflt) { const char *p = strstr(line, key); return p ? atoi(p + strlen(key)) : dflt; }
-static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step) {
+/* the running level-0 statistics a checkpoint of cfg.l0_norm 2 carries (src/unet.c:5579-5584, :5737-5739): their state and 16 G values */
+typedef struct { long n; int warm; float mom; int cnt; float run[1024]; } l0_hdr;
+static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step, l0_hdr *l0) {
     FILE *f = fopen(path, "rb");
     if (!f) return -1;
     char *line = header_line(f); fclose(f);
@@ -490,18 +521,25 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
     if (!bad && key_int(line, "\"scale_cond\":", 0)) bad = "\"scale_cond\":";
-    if (!bad && cfg->l0_norm && cfg->l0_norm != 4) bad = "\"l0_norm\": (none / ema / ws)";
+    if (!bad && (cfg->l0_norm < 0 || cfg->l0_norm > 4)) bad = "\"l0_norm\":";
+    if (l0) {
+        memset(l0, 0, sizeof *l0);
+        l0->n = key_int(line, "\"l0_n\":", 0); l0->warm = key_int(line, "\"l0_warm\":", 100);
+        const char *q = strstr(line, "\"l0_mom\":"); l0->mom = q ? strtof(q + 9, nullptr) : 0.01f;
+        if ((q = strstr(line, "\"l0_run\":["))) { q += 10; while (l0->cnt < 1024 && *q && *q != ']') { char *e; l0->run[l0->cnt] = strtof(q, &e); if (e == q) break; l0->cnt++; q = e; if (*q == ',') q++; } }
+    }
     if (!bad && cfg->attn_blocks && cfg->attn_pe != 1 && cfg->attn_pe != 2) bad = "\"attn_pe\": (PEG / scroll RoPE)";
     if (bad) { fprintf(stderr, "unet_peek: %s uses %s which this build does not run\n", path, bad); free(line); return -2; }
     free(line);
     return cfg->cin > 0 && cfg->cout > 0 ? 0 : -1;
 }
-int unet_peek(const char *path, unet_cfg *cfg, int *step) { return read_header(path, cfg, nullptr, step); }      /* src/unet.c:5756 */
-size_t mi_unet_peek_nparams(const char *path) { unet_cfg c; size_t np = 0; return read_header(path, &c, &np, nullptr) == -1 ? 0 : np; }
+int unet_peek(const char *path, unet_cfg *cfg, int *step) { return read_header(path, cfg, nullptr, step, nullptr); }      /* src/unet.c:5756 */
+size_t mi_unet_peek_nparams(const char *path) { unet_cfg c; size_t np = 0; return read_header(path, &c, &np, nullptr, nullptr) == -1 ? 0 : np; }
 /* weights and EMA weights into a net of the same architecture; the saved step, or -1 (src/unet.c:5774-5800) */
 int unet_load(unet *u, const char *path) {
     unet_cfg c; size_t np = 0; int step = 0;
-    const int r = read_header(path, &c, &np, &step);
+    static _Thread_local l0_hdr l0;
+    const int r = read_header(path, &c, &np, &step, &l0);
     if (r) { if (r == -1) fprintf(stderr, "unet_load: %s: unreadable header\n", path); return -1; }
     const unet_cfg *m = &u->cfg; const char *bad = nullptr;
     if (c.nlev != m->nlev) bad = "nlev";
@@ -537,8 +575,14 @@ int unet_load(unet *u, const char *path) {
         lp_wmemo_clear();
     }
     free(h); fclose(f);
+    if (rc >= 0 && u->cfg.l0_norm == 2) {                          /* the running statistics; a checkpoint without them: a fresh warm-up on live statistics (src/unet.c:5841-5845) */
+        const int n = 16 * G_of(u, u->cfg.widths[0]);
+        if (l0.cnt == n) { mi_h2d(u->l0run, l0.run, (size_t)n * 4); u->l0_n = l0.n; u->l0_warm = l0.warm; u->l0_mom = l0.mom; }
+        else { mi_zero(u->l0run, (size_t)n * 4); u->l0_n = 0; }
+    }
     return rc;
 }
+long unet_l0_updates(const unet *u) { return u->l0_n; }           /* src/unet.h:314 */
 int unet_save(const unet *u, const char *path, int step, const char *extra) {
     float *h = malloc(u->np * 4), *he = malloc(u->np * 4);
     if (!h || !he) { free(h); free(he); return -1; }
@@ -556,6 +600,13 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
     if (u->cfg.l0_norm) fprintf(f, ",\"l0_norm\":%d", u->cfg.l0_norm);
     if (u->cfg.l0_norm == 4) fprintf(f, ",\"l0_slab\":%d", u->cfg.l0_slab);
+    if (u->cfg.l0_norm == 2) {                                     /* the running statistics and their state (src/unet.c:5579-5584) */
+        const int n = 16 * G_of(u, u->cfg.widths[0]); float r[1024];
+        mi_d2h(r, u->l0run, (size_t)n * 4);
+        fprintf(f, ",\"l0_n\":%ld,\"l0_warm\":%d,\"l0_mom\":%.9g,\"l0_run\":[", u->l0_n, u->l0_warm, (double)u->l0_mom);
+        for (int i = 0; i < n; i++) fprintf(f, "%s%.9g", i ? "," : "", (double)r[i]);
+        fputc(']', f);
+    }
     fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":0,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.cout, u->cfg.G,
             u->cfg.down_norm, u->np, step);
     fprintf(f, ",\"extra\":%s}\n", extra ? extra : "{}");

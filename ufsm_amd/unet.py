@@ -65,6 +65,7 @@ def load_host():
     L.nn_check.restype = C.c_char_p
     L.unet_set_infer_slab.restype = None; L.unet_set_infer_slab.argtypes = [_I]
     L.unet_set_slab_direct.restype = None; L.unet_set_slab_direct.argtypes = [_I]
+    L.unet_l0_updates.restype = C.c_long; L.unet_l0_updates.argtypes = [C.c_void_p]
     L.mi_unet_infer_slab.restype = _I; L.mi_unet_infer_slab.argtypes = []
     L.nn_set_zrange.restype = None; L.nn_set_zrange.argtypes = [_I] * 6
     L.nn_set_zrange_out.restype = None; L.nn_set_zrange_out.argtypes = [_I]
