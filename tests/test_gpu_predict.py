@@ -154,3 +154,62 @@ def test_predict_volume_batched_windows_equal_single(gpu, attn):
         net.close()
     assert outs[0].max() > 0 and outs[0].std() > 0
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+@pytest.mark.gpu
+def test_config4_full_volume_prediction_properties(gpu):
+    """The whole 512 x 1024 x 1024 volume of the sliding-window configuration (128^3 windows, halo 16, feather 16: 6 x 11 x 11 = 726 windows,
+    eight per forward; widths 32/64/128/192, MX-fp4 weights over MX-fp8 activations, two attention blocks) through the driver, checked by what
+    does not depend on the size (tests/test_predict_feather.c:108-121): core voxels and the first window equal the unfeathered prediction byte
+    for byte, blended shells differ; windows at the far corner and in the middle, gathered, run alone on a one-window graph and placed through
+    the C ABI, equal the unfeathered prediction of their region (offsets past 2^29 voxels, the incomplete last batch); a second run is identical."""
+    from ufsm_amd.unet import UNet, make_cfg
+    dims, W, halo, B = (512, 1024, 1024), 128, 16, 16
+    S = W - 2 * halo
+    rng = np.random.default_rng(7)
+    z = np.arange(dims[0], dtype=np.float32)[:, None, None]; y = np.arange(dims[1], dtype=np.float32)[None, :, None]; x = np.arange(dims[2], dtype=np.float32)[None, None, :]
+    r = np.sqrt((y - 400.0) ** 2 + (x + 300.0) ** 2)
+    vol = (115 + 55 * np.sin(r * 0.35 + 0.02 * z)).astype(np.float32)
+    vol += rng.integers(-20, 21, (1, dims[1], dims[2])).astype(np.float32) + rng.integers(-10, 11, (dims[0], 1, 1)).astype(np.float32)
+    vol = np.clip(vol, 1, 255).astype(np.uint8)
+    del r
+    cfgk = dict(G=8, head_out=1, act_dt=8, prec=3, attn_blocks=2, attn_pe=1, attn_reg=4)
+    net = UNet(make_cfg(4, [32, 64, 128, 192], **cfgk), 8, W, W, W, seed=1)
+    p = net.params()
+    dv = DevBuf.from_numpy(vol); dout = DevBuf(vol.size); dplain = DevBuf(vol.size)
+    args = (115.0, 1 / 40.0, 1, 400.0, -300.0)
+    rc, nw, ndone = net.predict_volume(dv.ptr, dims, halo, B, *args, dout.ptr)
+    LP.check()
+    assert rc == 0 and nw == 6 * 11 * 11 and ndone == nw
+    got = dout.to_numpy(np.uint8, dims)
+    rc, _, _ = net.predict_volume(dv.ptr, dims, halo, B, *args, dout.ptr)
+    LP.check()
+    assert rc == 0 and np.array_equal(dout.to_numpy(np.uint8, dims), got)   # deterministic
+    rc, _, _ = net.predict_volume(dv.ptr, dims, halo, 0, *args, dplain.ptr)
+    LP.check()
+    assert rc == 0
+    plain = dplain.to_numpy(np.uint8, dims)
+    assert got.std() > 5 and got.max() > 128                               # not constant, both sides of one half
+    sh = [(np.arange(d) % S) < B for d in dims]
+    insh = sh[0][:, None, None] | sh[1][None, :, None] | sh[2][None, None, :]
+    assert np.array_equal(got[~insh], plain[~insh])                          # core voxels: the plain prediction
+    assert np.array_equal(got[:S, :S, :S], plain[:S, :S, :S])                # first window: nothing to blend with
+    first = (np.arange(dims[0]) < S)[:, None, None] & (np.arange(dims[1]) < S)[None, :, None] & (np.arange(dims[2]) < S)[None, None, :]
+    shell = insh & ~first & (plain > 0)
+    assert (got[shell] != plain[shell]).mean() > 0.25                        # the blended shells moved
+    del insh, shell, first
+    # ---- sampled windows run alone on a one-window graph: the plain prediction of their S^3 region ----
+    one = UNet(make_cfg(4, [32, 64, 128, 192], **cfgk), 1, W, W, W, seed=2); one.set_params(p)
+    dlg = DevBuf(W ** 3 * 4); dw = DevBuf(W ** 3); dE = DevBuf(S ** 3)
+    for a, b, c in ((0, 0, 0), (3, 5, 6), (5, 10, 10), (5, 0, 10)):          # (the last ones: ragged ends 512 - 480 = 32 planes, 1024 - 960 = 64 rows)
+        o = (a * S - halo, b * S - halo, c * S - halo)
+        lib.mi_ct_window(dv.ptr, dims[0], dims[1], dims[2], o[0], o[1], o[2], W, dw.ptr, 1, halo, None)
+        off = DevBuf.from_numpy(np.concatenate([np.full(W, o[1] - args[3], np.float32), np.full(W, o[2] - args[4], np.float32)]))
+        assert one.forward_ct(dw.ptr, args[0], args[1], off.ptr, off.ptr + 4 * W, args[2], dlg.ptr) == 0
+        lib.mi_zero(dE.ptr, S ** 3)
+        lib.nn_pred_place(dlg.ptr, dw.ptr, W, halo, -halo, -halo, -halo, S, S, S, S, dE.ptr)
+        LP.check()
+        E = dE.to_numpy(np.uint8, (S, S, S))
+        reg = plain[a * S:(a + 1) * S, b * S:(b + 1) * S, c * S:(c + 1) * S]
+        assert np.array_equal(E[:reg.shape[0], :reg.shape[1], :reg.shape[2]], reg), (a, b, c)
+    one.close(); net.close()
