@@ -527,7 +527,6 @@ static void conv_epilogue(const orc_conv_t *c, int n, size_t ov, size_t So, floa
 static int conv3_stem(const orc_conv_t *c) {
     const int Ci = c->Ci, Co = c->Co, D = c->D, H = c->H, W = c->W, rowmode = c->stem_tile == 2;
     if (c->x2 || c->up || c->stride == 2 || c->cbits != 8 || Ci > 16 || (!rowmode && c->xdt != 0 && Ci > 8)) return -2;
-    if (c->gp.G && c->gp.ns) return -3;     /* (slab-local statistics on the few-channel forms: not restated) */
     const int CP = rowmode ? 16 : Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = 32 / CP, NKB = rowmode ? 18 : (27 + TPK - 1) / TPK;
     const size_t S = (size_t)D * H * W;
     /* K block kb, element k -> (tap, channel), tap 27 = none */
@@ -543,17 +542,20 @@ static int conv3_stem(const orc_conv_t *c) {
     const int z0 = c->z1 ? c->z0 : 0, z1 = c->z1 ? c->z1 : D;
     const int ntz = (D + 1) / 2, nty = (H + 7) / 8, ntx = (W + 15) / 16;
     float *val = (float *)malloc(S * CP * sizeof(float));
-    chab_t tab[32];
+    const int slabs = c->gp.G && c->gp.ns;
+    chab_t *tab = (chab_t *)malloc((size_t)32 * (slabs ? D : 1) * sizeof(chab_t));
     for (int n = 0; n < c->N; n++) {
-        /* the conv's input values of this sample: val[voxel][CP] (decoded, after GN + SiLU when the input has one) */
-        chan_table(c, n, 0, Ci, (Ci + 31) / 32 * 32, 32, tab);
+        /* the conv's input values of this sample: val[voxel][CP] (decoded, after GN + SiLU when the input has one; slab-local statistics: each
+           plane's own coefficients, src/lp_f8fwd.cuh:497) */
+        for (int z = 0; z < (slabs ? D : 1); z++) chan_table(c, n, z, Ci, (Ci + 31) / 32 * 32, 32, tab + (size_t)z * 32);
         mxt_t t; if (c->xdt >= 3) t = mxt(c->x, c->xdt == 3 ? 8 : 4, c->N, Ci, S);
 #pragma omp parallel for schedule(static)
         for (int64_t vi = 0; vi < (int64_t)S; vi++) {
             float r[32] = {0};
             if (c->xdt >= 3) mx_row32(&t, n, 0, (size_t)vi, r);
             else for (int k = 0; k < Ci; k++) { const size_t idx = ((size_t)n * Ci + k) * S + (size_t)vi; r[k] = c->xdt == 2 ? orc_h16_to_f32(((const uint16_t *)c->x)[idx]) : ((const float *)c->x)[idx]; }
-            for (int k = 0; k < CP; k++) val[(size_t)vi * CP + k] = k >= Ci ? 0.f : tab[k].g ? orc_act_ab(r[k], tab[k].a, tab[k].b) : r[k];
+            const chab_t *tz = tab + (slabs ? (size_t)(vi / ((int64_t)H * W)) * 32 : 0);
+            for (int k = 0; k < CP; k++) val[(size_t)vi * CP + k] = k >= Ci ? 0.f : tz[k].g ? orc_act_ab(r[k], tz[k].a, tz[k].b) : r[k];
         }
         double *gs = c->osum ? (double *)calloc((size_t)2 * c->Go, sizeof(double)) : NULL;
 #pragma omp parallel
@@ -609,7 +611,7 @@ static int conv3_stem(const orc_conv_t *c) {
         if (gs) { for (int i = 0; i < 2 * c->Go; i++) c->osum[(size_t)n * 2 * c->Go + i] += gs[i]; free(gs); }
     }
 #undef STEM_TAP
-    free(val); free(wv); free(wsf);
+    free(val); free(wv); free(wsf); free(tab);
     return 0;
 }
 

@@ -194,3 +194,38 @@ def test_prestage_slab_statistics(gpu):
     LP.check()
     staged, _ = gpu_conv(dst.to_numpy(np.uint8), 3, N, Ci, D, H, W, w, b, Co, 3)
     assert np.array_equal(staged, direct)
+
+
+@pytest.mark.parametrize("Ci,tile,zs,zo,ns,kern", [(8, 1, 6, 0, 2, "conv3_stem_k"), (4, 1, 4, 1, 3, "conv3_stem_k"), (16, 2, 6, 0, 2, "conv3_p16_k"), (12, 2, 5, 2, 3, "conv3_p16_k")])
+def test_few_channel_convs_slab_statistics(gpu, Ci, tile, zs, zo, ns, kern):
+    """The tap-packed and the row-scale kernels (inputs of at most 16 channels) form one coefficient table per slab and take each staged
+    position's plane (src/lp_f8fwd.cuh:497): against the oracle to the per-sample tests' bar, with output statistics, also through the z-range."""
+    from ufsm_amd import split_t
+    rng = np.random.default_rng(Ci + zs)
+    N, Co, (D, H, W), G = 2, 32, (12, 12, 20), 4
+    S = D * H * W
+    xq = orc.f32_to_mx(8, rng.standard_normal((N, Ci, S)).astype(np.float32), N, Ci, S)
+    w = (rng.standard_normal((Co, Ci, 27)) * np.sqrt(2.0 / (Ci * 27))).astype(np.float32); b = (rng.standard_normal(Co) * 0.1).astype(np.float32)
+    gam = rng.uniform(0.5, 1.5, Ci).astype(np.float32); bet = rng.uniform(-.5, .5, Ci).astype(np.float32)
+    mean, rstd = stats(rng, N, ns, G)
+    slab = (zs, zo, ns, H * W)
+    want, wsum = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 3, stem_tile=tile, Go=8, want_stats=True, stored_stats=1, gp=orc.gn(gam, bet, mean, rstd, G, slab=slab))
+    got, gsum = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 3, Go=8, stats=True, stored_stats=1, gp=dev_gn_slab(gam, bet, mean, rstd, G, slab))
+    assert kern in lib.mi_last_kernel().decode()
+    from gpuutil import code_mismatch_fraction
+    frac, near = code_mismatch_fraction(8, got, want, N, Co, S)
+    assert frac < 2e-2 and near
+    dec = orc.mx_to_f32(8, got, N, Co, S).astype(np.float64).reshape(N, 8, -1)
+    assert np.allclose(gsum[:, :, 0], dec.sum(-1), rtol=1e-5, atol=1e-3) and np.allclose(gsum[:, :, 1], (dec * dec).sum(-1), rtol=1e-5)
+    # the slabs' rows matter (another tensor with the first slab's rows everywhere) ...
+    flat, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 3, gp=dev_gn(gam, bet, row(mean, 0), row(rstd, 0), G))
+    assert not np.array_equal(flat, got)
+    # ... and z-range slabs of 4 output planes into the full-depth tensor give the whole conv's bytes
+    dq, dw, db = DevBuf.from_numpy(xq), DevBuf.from_numpy(w), DevBuf.from_numpy(b)
+    dy = DevBuf(mx_bytes(8, N, Co, S))
+    g = dev_gn_slab(gam, bet, mean, rstd, G, slab)
+    for z0 in range(0, D, 4):
+        sp = split_t(); sp.zi0, sp.Di, sp.yzo, sp.yD = z0, D, z0, D
+        assert lib.lp_conv_fwd_f8(dq.ptr, 3, shape5(N, Ci, 4, H, W), dw.ptr, db.ptr, Co, dy.ptr, 3, g, None, 0, sp) == 0
+    LP.check()
+    assert np.array_equal(dy.to_numpy(np.uint8), got)

@@ -161,3 +161,31 @@ def test_conv_output_planes_around_a_slab_boundary(stride):
             assert np.array_equal(y[:, :, z], per[1][:, :, z]), z
         else:
             assert not np.array_equal(y[:, :, z], per[0][:, :, z]) and not np.array_equal(y[:, :, z], per[1][:, :, z]), z
+
+
+@pytest.mark.parametrize("Ci,tile", [(8, 1), (4, 1), (16, 2), (12, 2)])
+def test_few_channel_conv_output_planes_around_a_slab_boundary(Ci, tile):
+    """The few-channel forms (one activation scale per staged tile, or per staged row; src/lp_f8fwd.cuh:497 takes the slab row per staged
+    plane): output planes whose staged input planes lie in one slab equal the conv with that slab's rows as per-sample statistics. The
+    tap-packed form's tile scale couples the planes of a two-plane tile, so whole tiles are compared there."""
+    rng = np.random.default_rng(Ci + tile)
+    N, Co, D, H, W, G = 1, 32, 12, 8, 16, 4
+    zs, zo, ns = 6, 0, 2                                   # boundary between input planes 5 and 6
+    S = D * H * W
+    xq = orc.f32_to_mx(8, rng.standard_normal((N, Ci, S)).astype(np.float32), N, Ci, S)
+    w = (rng.standard_normal((Co, Ci, 27)) * 0.1).astype(np.float32); b = rng.standard_normal(Co).astype(np.float32)
+    gam = rng.uniform(0.5, 1.5, Ci).astype(np.float32); bet = rng.uniform(-0.5, 0.5, Ci).astype(np.float32)
+    mean, rstd = stats(rng, N, ns, G)
+    y, _ = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 0, stem_tile=tile, gp=orc.gn(gam, bet, mean, rstd, G, slab=(zs, zo, ns, H * W)))
+    per = [orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 0, stem_tile=tile, gp=orc.gn(gam, bet, np.ascontiguousarray(mean[:, s]), np.ascontiguousarray(rstd[:, s]), G))[0] for s in range(ns)]
+    y = y.reshape(N, Co, D, -1); per = [p.reshape(N, Co, D, -1) for p in per]
+    for z in range(D):
+        t0 = z & ~1                                        # the staged planes of the output plane's tile (tap-packed) or of the plane itself
+        lo, hi = (t0 - 1, t0 + 2) if tile == 1 else (z - 1, z + 1)
+        lo, hi = max(lo, 0), min(hi, D - 1)
+        if hi < zs:
+            assert np.array_equal(y[:, :, z], per[0][:, :, z]), z
+        elif lo >= zs:
+            assert np.array_equal(y[:, :, z], per[1][:, :, z]), z
+        elif max(z - 1, 0) < zs <= min(z + 1, D - 1):      # the plane's own taps straddle the boundary (a straddling tile's other plane may
+            assert not np.array_equal(y[:, :, z], per[0][:, :, z]) and not np.array_equal(y[:, :, z], per[1][:, :, z]), z      # share its scale with a per-sample run)

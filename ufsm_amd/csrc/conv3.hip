@@ -199,11 +199,13 @@ static thread_local int g_stem_zc = 0;      // tuning knob (mi_conv_stem_zc): z 
 static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf,
                      gnp_t gp, double *osum, int Go, split_t sp, bool rows) {
     const int Ci = xs.c, N = xs.n, D = sp.Di ? sp.Di : xs.d, Do = xs.d, H = xs.h, W = xs.w;      // D: the input's depth (z-range), Do: output planes
-    if (gp.G && gp.ns) mi_die("%s: slab-local GroupNorm statistics on an input of %d channels (the few-channel kernels form their coefficients per sample)", who, Ci);
+    if (gp.G && gp.ns && (gp.zs <= 0 || gp.zo < 0 || gp.zo >= gp.zs || gp.zhw != H * W || gp.ns > 256))
+        mi_die("%s: slab-local GroupNorm geometry (zs %d, zo %d, ns %d, zhw %d) does not fit planes of %d voxels (at most 256 slabs)", who, gp.zs, gp.zo, gp.ns, gp.zhw, H * W);
     const int CP = rows ? 0 : Ci <= 4 ? 4 : Ci <= 8 ? 8 : 16, TPK = rows ? 2 : 32 / CP, NKB = rows ? 18 : (27 + TPK - 1) / TPK, NP = (NKB + 1) / 2;
     conv_args a; memset(&a, 0, sizeof a);
     a.sx = x; a.sxdt = xbf; a.sCi = Ci;
     a.sgam = gp.gamma; a.sbet = gp.beta; a.smean = gp.mean; a.srstd = gp.rstd; a.sG = gp.G;
+    if (gp.G && gp.ns) { a.szs = gp.zs; a.szo = gp.zo; a.sns = gp.ns; }      // (each slab's coefficient table in LDS: the staged positions take their plane's)
     a.N = N; a.D = D; a.H = H; a.W = W; a.Do = Do; a.Ho = H; a.Wo = W;
     a.zi0 = sp.Di ? sp.zi0 : 0; a.yD = sp.yD; a.yzo = sp.yD ? sp.yzo : 0;
     a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
@@ -211,6 +213,7 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     // (16 channels per slot: 7 or 9 weight fragment pairs per channel tile, one tile fits the registers; per-channel statistics records: one tile per workgroup)
     const int nmt_all = (cout + 31) / 32, MT = nmt_all % 2 == 0 && CP && CP < 16 && !(osum && (cout / Go) % 4) ? 2 : 1;
     size_t smem = rows ? (size_t)720 * 16 + 16 + 40 * 4 + 16 * 8 : ((size_t)720 * CP + 16 + CP * 8 + 15) & ~(size_t)15;     // staged tile, (zero row, row words | amax word), channel affine
+    if (a.sns > 1) smem += (size_t)(a.sns - 1) * (rows ? 16 : CP) * 8;      // (one affine table per slab)
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);
     a.red_o = (unsigned)smem; smem += 1024;
     a.nmt_all = nmt_all; a.ncs = nmt_all / MT;

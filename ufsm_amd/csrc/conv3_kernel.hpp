@@ -114,6 +114,7 @@ struct conv_args {
     // tap-packed stem only: the input as stored (0 fp32 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4: one row of 8 channels per voxel) and its GroupNorm
     const void *sx; int sxdt, sCi;
     const float *sgam, *sbet, *smean, *srstd; int sG;
+    int szs, szo, sns;            // slab-local statistics of the few-channel kernels' input (gnp_t zs / zo / ns; sns 0: per sample): plane z reads row n sns + clamp((z + szo) / szs)
     int zc; unsigned ngrp;             // consecutive z tiles a workgroup walks, workgroups with work
     bool big;                          // the wide kernel takes the launch (MT 4, or MT 2 with NT 4)
     bool areg;                         // the persistent small-channel kernel (one channel tile, one input block, weights in registers) takes the launch

@@ -40,10 +40,11 @@ __global__ void __launch_bounds__(256, MT == 1 ? (CP == 8 ? 4 : 3) : (CP == 8 ? 
     const size_t S = (size_t)a.D * a.H * a.W;
 
     if (tid == 0) *(unsigned *)(lds + am_o) = 0u;
-    if (tid < CP) {
+    for (int i = tid; i < CP * (a.sns ? a.sns : 1); i += 256) {          // (slab-local statistics: one table per slab, back to back)
+        const int k = i % CP, row = a.sns ? n * a.sns + i / CP : n;
         float ga = 1.f, gb = 0.f;
-        if (a.sG && tid < Ci) { const int ng = n * a.sG + tid / (Ci / a.sG); ga = a.srstd[ng] * a.sgam[tid]; gb = fmaf(-a.smean[ng], ga, a.sbet[tid]); }
-        *(float2 *)(lds + ab_o + tid * 8) = make_float2(ga, gb);
+        if (a.sG && k < Ci) { const int ng = row * a.sG + k / (Ci / a.sG); ga = a.srstd[ng] * a.sgam[k]; gb = fmaf(-a.smean[ng], ga, a.sbet[k]); }
+        *(float2 *)(lds + ab_o + i * 8) = make_float2(ga, gb);
     }
     conv_epi_consts<MT, false>(a, lds, cs, tid);
 
@@ -144,10 +145,12 @@ __global__ void __launch_bounds__(256, MT == 1 ? (CP == 8 ? 4 : 3) : (CP == 8 ? 
                     for (int k = 0; k < CP; k++) x[k] = d8[k] * sc;
                 }
             }
+            unsigned abj = ab_o;
+            if (a.sns) { int s = (2 * tz - 1 + piz[j] + a.zi0 + a.szo) / a.szs; s = s < 0 ? 0 : s >= a.sns ? a.sns - 1 : s; abj += (unsigned)s * CP * 8; }     // the table of the position's plane
 #pragma unroll
             for (int k = 0; k < CP; k++) {
                 float val = x[k];
-                if (a.sG) { const float2 ab = *(const float2 *)(lds + ab_o + k * 8); val = d_act_ab(val, ab.x, ab.y); }
+                if (a.sG) { const float2 ab = *(const float2 *)(lds + abj + k * 8); val = d_act_ab(val, ab.x, ab.y); }
                 val = rin[j] && k < Ci ? val : 0.f;
                 v[j][k] = val; amax = fmaxf(amax, fabsf(val));
             }
@@ -251,10 +254,11 @@ __global__ void __launch_bounds__(256, 2) conv3_p16_k(const conv_args a) {
     const size_t S = (size_t)a.D * a.H * a.W;
     if (tid < 4) *(unsigned *)(lds + z_o + tid * 4) = 0u;
     if (tid < NROW) *(unsigned *)(lds + ra_o + tid * 4) = 0u;
-    if (tid < 16) {
+    for (int i = tid; i < 16 * (a.sns ? a.sns : 1); i += 256) {          // (slab-local statistics: one table per slab, back to back)
+        const int k = i & 15, row = a.sns ? n * a.sns + (i >> 4) : n;
         float ga = 1.f, gb = 0.f;
-        if (a.sG && tid < Ci) { const int ng = n * a.sG + tid / (Ci / a.sG); ga = a.srstd[ng] * a.sgam[tid]; gb = fmaf(-a.smean[ng], ga, a.sbet[tid]); }
-        *(float2 *)(lds + ab_o + tid * 8) = make_float2(ga, gb);
+        if (a.sG && k < Ci) { const int ng = row * a.sG + k / (Ci / a.sG); ga = a.srstd[ng] * a.sgam[k]; gb = fmaf(-a.smean[ng], ga, a.sbet[k]); }
+        *(float2 *)(lds + ab_o + i * 8) = make_float2(ga, gb);
     }
     conv_epi_consts<MT, false>(a, lds, cs, tid);
     v8i fa[9][MT]; int sa[9][MT];
@@ -303,10 +307,12 @@ __global__ void __launch_bounds__(256, 2) conv3_p16_k(const conv_args a) {
                 }
         }
         float am = 0.f;
+        unsigned abj = ab_o;
+        if (a.sns) { int s = (gz + a.szo) / a.szs; s = s < 0 ? 0 : s >= a.sns ? a.sns - 1 : s; abj += (unsigned)s * 128; }     // the table of the position's plane
 #pragma unroll
         for (int k = 0; k < 16; k++) {
             float val = x[k];
-            if (a.sG) { const float2 ab = *(const float2 *)(lds + ab_o + k * 8); val = d_act_ab(val, ab.x, ab.y); }
+            if (a.sG) { const float2 ab = *(const float2 *)(lds + abj + k * 8); val = d_act_ab(val, ab.x, ab.y); }
             val = inb && k < Ci ? val : 0.f;
             v[j][k] = val; am = fmaxf(am, fabsf(val));
         }

@@ -73,7 +73,6 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->l0_norm < 0 || c->l0_norm > 4) return "l0_norm (0 GroupNorm, 1 none, 2 ema, 3 ws, 4 slab)";
     if (c->l0_norm == 2 && (c->G < c->widths[0] ? c->G : c->widths[0]) > 64) return "l0_norm 2 with more than 64 groups";
     if (c->l0_norm == 4 && c->widths[0] > 32) return "l0_norm 4 with more than 32 level-0 channels";   /* (one MX channel block: a slab is a sample of the same layout) */
-    if (c->l0_norm == 4 && c->widths[0] <= 16) return "l0_norm 4 with 16 or fewer level-0 channels";   /* (the few-channel conv kernels read per-sample statistics only) */
     if (c->l0_slab && c->l0_norm != 4) return "l0_slab without l0_norm 4";
     if (c->gfilm) return "gfilm";
     if (c->gn_ema) return "gn_ema";
