@@ -127,6 +127,8 @@ void unet_set_slab_direct(int on);                            /* on (the default
    weights and EMA weights into a net of the same architecture (checked: nlev, widths, cin, cout, attention blocks, down_norm, nparams,
    payload size) and returns the saved step, or -1. unet_save writes weights and EMA. ---- */
 int unet_peek(const char *path, unet_cfg *cfg, int *step);
+void unet_gn_ema_live(unet *u, int on);                        /* cfg.gn_ema: 1 = forwards normalise with the window's own statistics instead of the running ones (src/unet.h:172) */
+long unet_gn_ema_updates(const unet *u);                       /* cfg.gn_ema: updates the loaded running statistics have seen (src/unet.h:288); 0: live statistics */
 long unet_l0_updates(const unet *u);                           /* cfg.l0_norm 2: updates the loaded running statistics have seen (src/unet.h:275-299); the forward uses them
                                                                   once that count has reached the checkpoint's warm-up, live GroupNorm statistics before */
 int unet_load(unet *u, const char *path);

@@ -705,3 +705,87 @@ def test_unet_l0_norm_constant_modes(gpu, tmp_path, mode, bits, widths):
         assert np.array_equal(d2.to_numpy(np.float32, (N, head_out, S)), got)
         twin.close()
     net.close()
+
+
+@pytest.mark.parametrize("widths,dn,attn", [([32, 64, 128], 1, 0), ([32, 96], 0, 1)])
+def test_unet_gn_ema(gpu, tmp_path, widths, dn, attn):
+    """cfg.gn_ema (src/unet.h:67-71): every GroupNorm site (block norms of all levels, down norms, the attention stage's output) reads the
+    checkpoint's running statistics once they have seen an update, in the order of gn_sites (src/unet.c:5125-5135), [mean G | var G] per
+    site, the EMA weights their own copy; before that, and under unet_gn_ema_live, the window's own statistics."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    H0 = load_host()
+    rng = np.random.default_rng(len(widths) + dn)
+    N, (D, H, W), bits = 2, (16, 16, 16), 8
+    S = D * H * W
+    cin, head_out, G = 4, 3, 8
+    kw = dict(G=G, head_out=head_out, act_dt=bits, down_norm=dn, attn_blocks=attn, attn_pe=1, attn_reg=2)
+    net = UNet(make_cfg(cin, widths, gn_ema=1, **kw), N, D, H, W, seed=17)
+    plain = UNet(make_cfg(cin, widths, **kw), N, D, H, W, seed=1)
+    p = net.params(); plain.set_params(p)
+    x = rng.standard_normal((N, cin, S)).astype(np.float32); dxq = to_mx(bits, x)
+    def run(n):
+        d = DevBuf(N * head_out * S * 4)
+        assert n.forward_x(dxq.ptr, d.ptr) == 0
+        LP.check()
+        return d.to_numpy(np.float32, (N, head_out, S))
+    ref = run(plain)
+    assert H0.unet_gn_ema_updates(net.h) == 0 and np.array_equal(run(net), ref)      # no running statistics yet: the window's own
+    # a checkpoint whose statistics have seen updates
+    L = len(widths)
+    sites = [("enc%d.c%d" % (i, k), min(G, widths[i])) for i in range(L) for k in (1, 2)]
+    sites += [("down%d" % i, min(G, widths[i])) for i in range(L - 1)] if dn else []
+    sites += [("dec%d.c%d" % (i, k), min(G, widths[i])) for i in range(L - 2, -1, -1) for k in (1, 2)]
+    sites += [("attn", min(G, widths[-1]))] if attn else []
+    ns = 2 * sum(g for _, g in sites)
+    runs = [np.concatenate([np.concatenate([rng.uniform(-0.3, 0.3, g), rng.uniform(0.3, 2.0, g)]) for _, g in sites]).astype(np.float32) for _ in range(2)]
+    path = str(tmp_path / "ge.ckpt")
+    assert net.save(path, step=4, extra="{}") == 0
+    raw = open(path, "rb").read(); head = raw[:raw.index(b"\n") + 1].decode()
+    assert ',"gn_ema":1,"ge_n":0,"ge_warm":500,' in head and head.count(",", head.index('"ge_run":['), head.index("]", head.index('"ge_run":['))) == 2 * ns - 1
+    i0, i1 = head.index(',"ge_n":'), head.index(']', head.index('"ge_run":[')) + 1
+    new = head[:i0] + ',"ge_n":7,"ge_warm":500,"ge_mom":0.01,"ge_run":[' + ",".join("%.9g" % v for v in np.concatenate(runs)) + "]" + head[i1:]
+    open(path, "wb").write(new.encode() + raw[len(head.encode()):])
+    assert plain.load(path) == -1                                   # another architecture
+    assert net.load(path) == 4 and H0.unet_gn_ema_updates(net.h) == 7
+    for which in (0, 1):                                            # the live weights' statistics, then the EMA weights' own
+        H0.unet_use_ema(net.h, which)
+        got = run(net)
+        assert not np.array_equal(got, ref)
+        stat, tens, shapes = {}, {}, {}
+        for k, (name, ptr, shp) in enumerate(net.layer_outs()):
+            nb = lib.lp_mx8_bytes(shp[0], shp[1], shp[2] * shp[3] * shp[4])
+            buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+            tens[name], shapes[name] = buf, shp
+            g, mp, rp = net.layer_stats(k)
+            if g:
+                m = np.empty(N * g, np.float32); r = np.empty(N * g, np.float32)
+                lib.mi_d2h(m.ctypes.data, mp, m.nbytes); lib.mi_d2h(r.ctypes.data, rp, r.nbytes)
+                stat[name] = (g, m, r)
+        o = 0
+        for name, g in sites:
+            gg, m, r = stat[name]
+            assert gg == g
+            assert np.array_equal(m.reshape(N, g), np.broadcast_to(runs[which][o:o + g], (N, g))), name
+            assert np.allclose(r.reshape(N, g), np.broadcast_to(1 / np.sqrt(runs[which][o + g:o + 2 * g].astype(np.float64) + 1e-5), (N, g)), rtol=3e-7), name
+            o += 2 * g
+        # the last conv and the head under those statistics (the other layers' readers are covered by the per-layer tests of the plain graph)
+        lay, _ = unet_ref.param_layout(cin, widths, head_out, dn) if not attn else (None, None)
+        if lay is not None:
+            Pm = lambda key: np.ascontiguousarray(p[lay[key][0]:lay[key][0] + int(np.prod(lay[key][1]))].reshape(lay[key][1]))
+            g1, m1, r1 = stat["dec0.c1"]; g2, m2, r2 = stat["dec0.c2"]
+            want_l, _ = orc.conv3(tens["dec0.c1"], 3, N, widths[0], D, H, W, Pm("dec0.c2.w"), Pm("dec0.c2.b"), widths[0], 3, gp=orc.gn(Pm("dec0.n1.gamma"), Pm("dec0.n1.beta"), m1, r1, g1))
+            frac, near = code_mismatch_fraction(bits, tens["dec0.c2"], want_l, N, widths[0], S)
+            assert frac < 0.02 and near
+            want = np.zeros((N, head_out, S), np.float32)
+            hw_ = np.ascontiguousarray(Pm("head.w").reshape(head_out, widths[0]))
+            orc.lib().orc_conv1_mx(bits, orc.ptr(tens["dec0.c2"]), N, widths[0], S, orc.ptr(hw_), orc.ptr(Pm("head.b")), head_out, orc.gn(Pm("dec0.n2.gamma"), Pm("dec0.n2.beta"), m2, r2, g2), orc.ptr(want))
+            assert np.abs(got - want).max() / np.abs(want).max() < 2e-5
+    H0.unet_use_ema(net.h, 0)
+    H0.unet_gn_ema_live(net.h, 1)
+    assert np.array_equal(run(net), ref)                            # the window's own statistics again
+    H0.unet_gn_ema_live(net.h, 0)
+    # a second save carries the loaded statistics
+    assert net.save(path, step=5, extra="{}") == 0
+    head2 = open(path, "rb").readline().decode()
+    assert ',"ge_n":7,"ge_warm":500,' in head2 and ("%.9g" % runs[1][-1]) in head2
+    plain.close(); net.close()

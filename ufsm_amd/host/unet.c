@@ -26,6 +26,9 @@ struct unet {
     /* cfg.l0_norm 1 .. 3 (src/unet.h:52-58): the level-0 GroupNorms on constant statistics: mean 0 / rstd 1 (none, ws) or the checkpoint's running
        statistics once its warm-up is over (ema: l0run = [live weights: 4 sites x (mean G | var G)][EMA weights: the same], device; l0_n updates so far) */
     float *l0run; long l0_n; int l0_warm; float l0_mom; float ws_gain;
+    /* cfg.gn_ema (src/unet.h:67-71): every GroupNorm (all levels, down norms, the attention stage's) on the checkpoint's running statistics:
+       ge_run = [live weights: ge_ns values][EMA weights: the same], per site pair [mean G | var G] in the order of gn_sites (src/unet.c:5125-5135) */
+    float *ge_run; size_t ge_ns; long ge_n; int ge_warm, ge_live; float ge_mom;
     int l0s_zs, l0s_ns;                /* cfg.l0_norm 4: planes per statistics slab and slabs of the current build (0: per-sample statistics) */
     int slab_ip, slab_nl, slab_s;      /* the build's in-place slab plan: on, and over how many levels (a level's tensors all live in enc[i].a2's buffer) */
     void *slab_tmp[2], *slab_carry[2]; /* per such level: one slab of output planes, and the plane that waits for the next slab */
@@ -75,7 +78,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->l0_norm == 4 && c->widths[0] > 32) return "l0_norm 4 with more than 32 level-0 channels";   /* (one MX channel block: a slab is a sample of the same layout) */
     if (c->l0_slab && c->l0_norm != 4) return "l0_slab without l0_norm 4";
     if (c->gfilm) return "gfilm";
-    if (c->gn_ema) return "gn_ema";
+    if (c->gn_ema && c->l0_norm) return "gn_ema with l0_norm (src/unet.c:551)";
     if (c->attn_vres) return "attn_vres";
     if (c->attn_axis) return "attn_axis";
     if (c->attn_repeat > 1) return "attn_repeat";
@@ -90,6 +93,20 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     return nullptr;
 }
 
+/* the GroupNorm statistics sites in the reference's order (gn_sites, src/unet.c:5125-5135): encoder blocks (conv1's, conv2's), down norms,
+   decoder blocks from the coarsest, the attention stage's output; a site is a (mean, rstd) pair of g groups, its running statistics
+   [mean g | var g] at offset off. Fills up to 192 entries when the arrays are given; returns the number of values. */
+static size_t ge_sites(unet *u, float **mean, float **rstd, int *g, size_t *off) {
+    size_t o = 0; int k = 0; const int L = u->cfg.nlev;
+#define GE_SITE(m, r, gg) do { if (mean && k < 192) { mean[k] = (m); rstd[k] = (r); g[k] = (gg); off[k] = o; } k++; o += 2 * (size_t)(gg); } while (0)
+    for (int i = 0; i < L; i++) { block *b = &u->enc[i]; GE_SITE(b->m1, b->r1, G_of(u, b->c1.cout)); GE_SITE(b->m2, b->r2, G_of(u, b->c2.cout)); }
+    if (u->cfg.down_norm) for (int i = 0; i < L - 1; i++) GE_SITE(u->dm[i], u->dr[i], G_of(u, u->cfg.widths[i]));
+    for (int i = L - 2; i >= 0; i--) { block *b = &u->dec[i]; GE_SITE(b->m1, b->r1, G_of(u, b->c1.cout)); GE_SITE(b->m2, b->r2, G_of(u, b->c2.cout)); }
+    if (u->tbn) GE_SITE(u->tb.m2, u->tb.r2, G_of(u, u->tbd.C));
+#undef GE_SITE
+    if (mean && k > 192) { fprintf(stderr, "unet: gn_ema: %d GroupNorm sites (at most 192)\n", k); abort(); }
+    return o;
+}
 unet *unet_create(const unet_cfg *cfg) {
     const int L = cfg->nlev;
     if (L < 1 || L > UNET_MAXLEV || cfg->cin < 1 || cfg->cout < 1 || cfg->G < 1) { fprintf(stderr, "unet_create: bad configuration (nlev %d, cin %d, cout %d, G %d)\n", L, cfg->cin, cfg->cout, cfg->G); return nullptr; }
@@ -137,6 +154,11 @@ unet *unet_create(const unet_cfg *cfg) {
     }
     u->l0_mom = 0.01f; u->l0_warm = 100;                          /* (src/unet.c:549) */
     if (cfg->l0_norm == 2) u->l0run = f32_new((size_t)16 * G_of(u, w[0]));
+    if (cfg->gn_ema) {
+        u->ge_ns = ge_sites(u, nullptr, nullptr, nullptr, nullptr);
+        if (u->ge_ns > 4096) { fprintf(stderr, "unet_create: gn_ema: %zu statistics (at most 4096)\n", u->ge_ns); mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm); free(u); return nullptr; }
+        u->ge_run = f32_new(2 * u->ge_ns); u->ge_mom = 0.01f; u->ge_warm = 500;      /* (src/unet.c:550) */
+    }
     return u;
 }
 /* inference in z-slabs (src/unet.h:422-424, src/unet.c:2499-2550): the convs of level 0 (and of level 1 in nets of three or more levels,
@@ -237,7 +259,7 @@ void unet_free(unet *u) {
     if (!u) return;
     mi_sync();
     free_acts(u);
-    mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm); if (u->l0run) mi_free(u->l0run);
+    mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm); if (u->l0run) mi_free(u->l0run); if (u->ge_run) mi_free(u->ge_run);
     lp_wmemo_clear();
     free(u);
 }
@@ -329,6 +351,18 @@ static void copy_planes(const unet *u, void *dst, int Dd, int d0, const void *sr
 /* cfg.l0_norm 1 / 3 always, 2 once the running statistics' warm-up is over (src/unet.c:2315): the level-0 GroupNorms read constant statistics,
    written at the start of every forward (src/unet.c:2318-2323) */
 static int l0_const(const unet *u) { const int md = u->cfg.l0_norm; return md == 1 || md == 3 || (md == 2 && u->l0_n > 0 && u->l0_n >= u->l0_warm); }
+/* cfg.gn_ema at inference (ge_begin, src/unet.c:2229-2250): once the running statistics have seen an update, every site reads them (unless
+   unet_gn_ema_live asks for the window's own); no conv or statistics pass reduces anything */
+static int ge_const(const unet *u) { return u->cfg.gn_ema && u->ge_n > 0 && !u->ge_live; }
+void unet_gn_ema_live(unet *u, int on) { u->ge_live = on != 0; }
+static void ge_const_fill(unet *u) {
+    float *m[192], *r[192]; int g[192]; size_t off[192];
+    ge_sites(u, m, r, g, off);
+    size_t o = 0; int n = 0;
+    while (o < u->ge_ns) { o = off[n] + 2 * (size_t)g[n]; n++; }
+    const float *run = u->ge_run + (u->src == u->ema ? u->ge_ns : 0);                       /* (the EMA weights have their own) */
+    for (int k = 0; k < n; k++) nn_gn_const_fill(m[k], r[k], run + off[k], u->in.n, g[k], 1e-5f);
+}
 static void l0_const_fill(unet *u) {
     const int G = G_of(u, u->cfg.widths[0]), N = u->in.n;
     for (int i = 0; i < (u->cfg.nlev > 1 ? 2 : 1); i++) for (int k = 1; k <= 2; k++) {
@@ -343,7 +377,7 @@ static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t 
     const int G = G_of(u, b->c1.cout), D = b->ys.d, ip = u->slab_ip && level < u->slab_nl;
     /* per-slab statistics (level 0 under cfg.l0_norm 4): the convs reduce nothing; a pass over the stored output, seen as n * slabs samples of
        l0_slab planes (one channel block: a slab is a sample of the same layout), fills the [n][slab][G] rows (src/unet.c:996-998) */
-    const int l0s = level == 0 && u->l0s_ns, Gc = l0s || (level == 0 && l0_const(u)) ? 0 : G;       /* (constant statistics: nothing to reduce either) */
+    const int l0s = level == 0 && u->l0s_ns, Gc = l0s || (level == 0 && l0_const(u)) || ge_const(u) ? 0 : G;       /* (constant statistics: nothing to reduce either) */
     const int s = level >= slab_levels(u) ? 0 : g_infer_slab < D ? g_infer_slab : ip ? D : 0;      /* (in place: a level of fewer planes is one slab) */
     void *tmp = ip ? u->slab_tmp[level] : nullptr, *carry = ip ? u->slab_carry[level] : nullptr;
     int r = 0;
@@ -389,7 +423,7 @@ static int tb_fwd(unet *u) {
     at_tok_to_cs(u->tb_tok + (size_t)u->tbn * TC, u->tb_cs, ys.n, C, (long)Sg, nr);
     if (u->act_dt == 4) lp_f32_to_mx4(u->tb_cs, ys.n, C, Sg, b->a2); else lp_f32_to_mx8(u->tb_cs, ys.n, C, Sg, b->a2);
     const int G = G_of(u, C);
-    if (nn_gn_stats(b->a2, ys, G, 1e-5f, b->m2, b->r2)) { fprintf(stderr, "unet: attention stage GroupNorm statistics unsupported for this storage\n"); return -1; }
+    if (!ge_const(u) && nn_gn_stats(b->a2, ys, G, 1e-5f, b->m2, b->r2)) { fprintf(stderr, "unet: attention stage GroupNorm statistics unsupported for this storage\n"); return -1; }
     note(u, b->a2, ys, "attn", b->m2, b->r2, G);
     return 0;
 }
@@ -401,6 +435,7 @@ static int graph_fwd(unet *u, const void *x) {
     const int L = u->cfg.nlev;
     u->nouts = 0;
     if (l0_const(u)) l0_const_fill(u);
+    if (ge_const(u)) ge_const_fill(u);
     const void *cur = x;
     for (int i = 0; i < L; i++) {
         nn_gn_t gd; const nn_gn_t *gin = nullptr;                  /* down_norm: conv1 reads silu(gn(down conv output)) (src/unet.c:2593) */
@@ -413,7 +448,7 @@ static int graph_fwd(unet *u, const void *x) {
             if (nn_conv3d_fwd_x(pre ? u->skipst[i] : u->enc[i].a2, pre ? nullptr : &g, nullptr, nullptr, 0, 0, u->enc[i].ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
             shape5 ds = u->ls[i + 1]; ds.c = u->cfg.widths[i];
             if (u->cfg.down_norm) {                                /* statistics of the stored down-conv output now, the transform in the next conv1's staging (src/unet.c:2974-2979) */
-                if (nn_gn_stats(u->downo[i], ds, G_of(u, ds.c), 1e-5f, u->dm[i], u->dr[i])) { fprintf(stderr, "unet: down_norm GroupNorm statistics unsupported for this storage\n"); return -1; }
+                if (!ge_const(u) && nn_gn_stats(u->downo[i], ds, G_of(u, ds.c), 1e-5f, u->dm[i], u->dr[i])) { fprintf(stderr, "unet: down_norm GroupNorm statistics unsupported for this storage\n"); return -1; }
                 note(u, u->downo[i], ds, dwn[i], u->dm[i], u->dr[i], G_of(u, ds.c));
             } else note(u, u->downo[i], ds, dwn[i], nullptr, nullptr, 0);
             cur = u->downo[i];
@@ -492,7 +527,7 @@ static char *header_line(FILE *f) {                                /* the first 
 }
 static int key_int(const char *line, const char *key, int dflt) { const char *p = strstr(line, key); return p ? atoi(p + strlen(key)) : dflt; }
 /* the running level-0 statistics a checkpoint of cfg.l0_norm 2 carries (src/unet.c:5579-5584, :5737-5739): their state and 16 G values */
-typedef struct { long n; int warm; float mom; int cnt; float run[1024]; } l0_hdr;
+typedef struct { long n; int warm; float mom; int cnt; float run[1024]; long gn; int gwarm; float gmom; int gcnt; float grun[8192]; } l0_hdr;      /* (and cfg.gn_ema's: src/unet.c:5744-5751) */
 static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *step, l0_hdr *l0) {
     FILE *f = fopen(path, "rb");
     if (!f) return -1;
@@ -508,6 +543,7 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     cfg->cin = key_int(line, "\"cin\":", 0); cfg->cout = key_int(line, "\"cout\":", 0); cfg->G = key_int(line, "\"G\":", 8);
     cfg->down_norm = key_int(line, "\"down_norm\":", 0); cfg->w4_2d = key_int(line, "\"w4_2d\":", 0);
     cfg->l0_norm = key_int(line, "\"l0_norm\":", 0); cfg->l0_slab = key_int(line, "\"l0_slab\":", 0);      /* (src/unet.c:5726) */
+    cfg->gn_ema = key_int(line, "\"gn_ema\":", 0);
     cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
     cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
     cfg->half_res = key_int(line, "\"half_res\":", 0); cfg->scan_norm = key_int(line, "\"scan_norm\":", 0);      /* (the caller's business: the graph does not use them) */
@@ -516,7 +552,7 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     /* architecture features this build's graph does not have */
     static const char *const no[] = {"\"dec_widths\":", "\"enc_blocks\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"ds_levels\":", "\"emb_lev\":",
                                      "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
-                                     "\"skip_empty\":", "\"gfilm\":", "\"gn_ema\":", "\"dec_convs\":"};
+                                     "\"skip_empty\":", "\"gfilm\":", "\"dec_convs\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
     if (!bad && key_int(line, "\"scale_cond\":", 0)) bad = "\"scale_cond\":";
@@ -525,6 +561,9 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
         memset(l0, 0, sizeof *l0);
         l0->n = key_int(line, "\"l0_n\":", 0); l0->warm = key_int(line, "\"l0_warm\":", 100);
         const char *q = strstr(line, "\"l0_mom\":"); l0->mom = q ? strtof(q + 9, nullptr) : 0.01f;
+        l0->gn = key_int(line, "\"ge_n\":", 0); l0->gwarm = key_int(line, "\"ge_warm\":", 500);
+        q = strstr(line, "\"ge_mom\":"); l0->gmom = q ? strtof(q + 9, nullptr) : 0.01f;
+        if ((q = strstr(line, "\"ge_run\":["))) { q += 10; while (l0->gcnt < 8192 && *q && *q != ']') { char *e; l0->grun[l0->gcnt] = strtof(q, &e); if (e == q) break; l0->gcnt++; q = e; if (*q == ',') q++; } }
         if ((q = strstr(line, "\"l0_run\":["))) { q += 10; while (l0->cnt < 1024 && *q && *q != ']') { char *e; l0->run[l0->cnt] = strtof(q, &e); if (e == q) break; l0->cnt++; q = e; if (*q == ',') q++; } }
     }
     if (!bad && cfg->attn_blocks && cfg->attn_pe != 1 && cfg->attn_pe != 2) bad = "\"attn_pe\": (PEG / scroll RoPE)";
@@ -548,6 +587,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.attn_blocks != m->attn_blocks) bad = "attn_blocks";
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
+    if (!bad && c.gn_ema != m->gn_ema) bad = "gn_ema";
     if (!bad && (c.l0_norm != m->l0_norm || (c.l0_norm == 4 && (c.l0_slab > 0 ? c.l0_slab : 64) != (m->l0_slab > 0 ? m->l0_slab : 64)))) bad = "l0_norm / l0_slab";
     if (!bad && np != u->np) bad = "nparams";
     if (bad) { fprintf(stderr, "unet_load: %s: \"%s\" differs from this network's\n", path, bad); return -1; }
@@ -579,8 +619,15 @@ int unet_load(unet *u, const char *path) {
         if (l0.cnt == n) { mi_h2d(u->l0run, l0.run, (size_t)n * 4); u->l0_n = l0.n; u->l0_warm = l0.warm; u->l0_mom = l0.mom; }
         else { mi_zero(u->l0run, (size_t)n * 4); u->l0_n = 0; }
     }
+    if (rc >= 0 && u->cfg.gn_ema) {                                /* a checkpoint without the statistics, or with non-finite ones: live statistics until a trainer has made some (src/unet.c:5846-5860) */
+        int ok = l0.gcnt == (int)(2 * u->ge_ns);
+        for (int i = 0; ok && i < l0.gcnt; i++) ok = isfinite(l0.grun[i]);
+        if (ok) { mi_h2d(u->ge_run, l0.grun, (size_t)l0.gcnt * 4); u->ge_n = l0.gn; u->ge_warm = l0.gwarm; u->ge_mom = l0.gmom; }
+        else { mi_zero(u->ge_run, 2 * u->ge_ns * 4); u->ge_n = 0; }
+    }
     return rc;
 }
+long unet_gn_ema_updates(const unet *u) { return u->ge_n; }       /* src/unet.h:280 */
 long unet_l0_updates(const unet *u) { return u->l0_n; }           /* src/unet.h:314 */
 int unet_save(const unet *u, const char *path, int step, const char *extra) {
     float *h = malloc(u->np * 4), *he = malloc(u->np * 4);
@@ -599,6 +646,15 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
     if (u->cfg.l0_norm) fprintf(f, ",\"l0_norm\":%d", u->cfg.l0_norm);
     if (u->cfg.l0_norm == 4) fprintf(f, ",\"l0_slab\":%d", u->cfg.l0_slab);
+    if (u->cfg.gn_ema) {                                           /* every site's running statistics and their state (src/unet.c:5587-5592; written after l0_norm's keys there too) */
+        float *r = malloc(2 * u->ge_ns * 4);
+        if (r) {
+            mi_d2h(r, u->ge_run, 2 * u->ge_ns * 4);
+            fprintf(f, ",\"gn_ema\":1,\"ge_n\":%ld,\"ge_warm\":%d,\"ge_mom\":%.9g,\"ge_run\":[", u->ge_n, u->ge_warm, (double)u->ge_mom);
+            for (size_t i = 0; i < 2 * u->ge_ns; i++) fprintf(f, "%s%.9g", i ? "," : "", (double)r[i]);
+            fputc(']', f); free(r);
+        }
+    }
     if (u->cfg.l0_norm == 2) {                                     /* the running statistics and their state (src/unet.c:5579-5584) */
         const int n = 16 * G_of(u, u->cfg.widths[0]); float r[1024];
         mi_d2h(r, u->l0run, (size_t)n * 4);

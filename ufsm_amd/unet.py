@@ -66,6 +66,8 @@ def load_host():
     L.unet_set_infer_slab.restype = None; L.unet_set_infer_slab.argtypes = [_I]
     L.unet_set_slab_direct.restype = None; L.unet_set_slab_direct.argtypes = [_I]
     L.unet_l0_updates.restype = C.c_long; L.unet_l0_updates.argtypes = [C.c_void_p]
+    L.unet_gn_ema_updates.restype = C.c_long; L.unet_gn_ema_updates.argtypes = [C.c_void_p]
+    L.unet_gn_ema_live.restype = None; L.unet_gn_ema_live.argtypes = [C.c_void_p, _I]
     L.mi_unet_infer_slab.restype = _I; L.mi_unet_infer_slab.argtypes = []
     L.nn_set_zrange.restype = None; L.nn_set_zrange.argtypes = [_I] * 6
     L.nn_set_zrange_out.restype = None; L.nn_set_zrange_out.argtypes = [_I]
@@ -79,7 +81,7 @@ def load_host():
     return L
 
 
-def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0):
+def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0, gn_ema=0):
     """The reference's configuration record plus, as Python attributes, what the reference keeps in process-wide switches: the activation
     storage (unet_set_act_mx4) and the compute precision policy (nn_set_prec), which UNet applies around its calls."""
     c = unet_cfg()
@@ -87,7 +89,7 @@ def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn
     c.attn_blocks, c.attn_pe, c.attn_reg, c.attn_mlp, c.down_norm, c.w4_2d = attn_blocks, attn_pe if attn_blocks else 0, attn_reg, attn_mlp, down_norm, w4_2d
     for i, w in enumerate(widths):
         c.widths[i] = w
-    c.l0_norm, c.l0_slab = l0_norm, l0_slab
+    c.l0_norm, c.l0_slab, c.gn_ema = l0_norm, l0_slab, gn_ema
     c.act_dt, c.prec = act_dt, prec
     return c
 
