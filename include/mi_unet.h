@@ -89,7 +89,7 @@ void unet_free(unet *u);
 const unet_cfg *unet_cfg_of(const unet *u);                    /* src/unet.h:159 */
 size_t unet_nparams(const unet *u);
 void unet_init(unet *u, uint64_t seed);                        /* Kaiming normal sqrt(2 / (cin 27)), biases 0, head bias -2, gamma 1, beta 0 (src/unet.c:588-607); the EMA copy = the weights */
-float *unet_param_ptr(unet *u);                                /* device pointers of the flat fp32 weights and of their EMA copy (src/unet.h:203-204), unet_init's order */
+float *unet_param_ptr(unet *u);                                /* device pointers of the flat fp32 weights and of their EMA copy (src/unet.h:203-204), in unet_create's layout (src/unet.c:451-459: encoder blocks, downs, decoder blocks from the coarsest, head, down norms, attention stage) */
 float *unet_ema_ptr(unet *u);
 void unet_use_ema(unet *u, int on);                            /* forward with the EMA weights (1) or the live ones (0) (src/unet.h:258) */
 /* no counterpart in the reference, which re-forms the forward copy of a cfg.w4_2d net's weights before every forward (src/unet.c:5310-5326): here
@@ -134,7 +134,7 @@ long unet_l0_updates(const unet *u);                           /* cfg.l0_norm 2:
 int unet_load(unet *u, const char *path);
 int unet_save(const unet *u, const char *path, int step, const char *extra_json);
 /* ---- additions of this build (no counterpart in src/unet.h) ---- */
-void mi_unet_get_params(const unet *u, float *host);           /* the live weights, flat, unet_init's order */
+void mi_unet_get_params(const unet *u, float *host);           /* the live weights, flat, in that layout */
 void mi_unet_set_params(unet *u, const float *host);           /* ... and the EMA copy with them; drops the prepared-weight memos */
 /* the forward on an input that already is the net's MX tensor (lp_f32_to_mx* output or lp_pred_input_mx rows), device pointer */
 const float *mi_unet_forward_mx(unet *u, const void *xmx, shape5 xs);

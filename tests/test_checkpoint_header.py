@@ -16,11 +16,33 @@ def read(tmp_path, header, payload=b""):
 
 def test_reads_the_reference_header(tmp_path):
     # the test net of tests/test_predict_feather.c:73-76 as unet_save writes it (keys in its order, the caller's runtime object as extra)
-    h = ('UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":287937,"step":1,"sparse24":0,"wq":0,"muon_mom":0,'
+    h = ('UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":336129,"step":1,"sparse24":0,"wq":0,"muon_mom":0,'
          '"extra":{"runtime":{"version":1,"train_window":96,"prec":1,"f16":1,"act_mx4":0,"act_mx8":1,"grad_mx8":1,"input_mx":1,"input_prec":8,"gn_stored":0,"policy":"","optimizer":"muon"}}}\n')
     rc, cfg, n, step = read(tmp_path, h)
     assert rc == 0 and (cfg.nlev, cfg.widths[0], cfg.widths[1], cfg.cin, cfg.cout, cfg.G, cfg.down_norm, cfg.attn_blocks, cfg.half_res) == (2, 32, 64, 4, 1, 8, 1, 0, 0)
-    assert n == 287937 and step == 1
+    assert n == 336129 and step == 1
+
+
+def test_parameter_layout_follows_unet_create():
+    """The flat layout the tests' graph (tests/unet_ref.py) and the host library share, against the reference's unet_create (src/unet.c:451-459):
+    encoder blocks, down convs, the decoder blocks from the coarsest level to level 0, the head, the down norms; a block is c1.w, c1.b, n1.gamma,
+    n1.beta, c2.w, c2.b, n2.gamma, n2.beta. The count of the two-level test net above, term by term."""
+    import unet_ref
+    lay, n = unet_ref.param_layout(4, [32, 64], 1, 1)
+    enc0 = 32 * 4 * 27 + 32 + 64 + 32 * 32 * 27 + 32 + 64
+    enc1 = 64 * 32 * 27 + 64 + 128 + 64 * 64 * 27 + 64 + 128
+    down0 = 32 * 32 * 27 + 32
+    dec0 = 32 * 96 * 27 + 32 + 64 + 32 * 32 * 27 + 32 + 64
+    assert n == enc0 + enc1 + down0 + dec0 + (32 + 1) + 64 == 336129
+    lay, n = unet_ref.param_layout(4, [8, 16, 32, 64], 2, 1)
+    order = [k[:-2] for k in lay if k.endswith(".w")] + [k[:-6] for k in lay if k.startswith("dn") and k.endswith(".gamma")]
+    assert order == ["enc0.c1", "enc0.c2", "enc1.c1", "enc1.c2", "enc2.c1", "enc2.c2", "enc3.c1", "enc3.c2", "down0", "down1", "down2",
+                     "dec2.c1", "dec2.c2", "dec1.c1", "dec1.c2", "dec0.c1", "dec0.c2", "head", "dn0", "dn1", "dn2"]
+    offs = [lay[k][0] for k in lay]
+    assert offs == sorted(offs) and lay["dec2.c1.w"][1] == (32, 64 + 32, 27) and lay["dec0.c1.w"][1] == (8, 16 + 8, 27)      # [up(coarse) | skip] input channels
+    keys = list(lay)
+    i = keys.index("dec1.c1.w")
+    assert keys[i:i + 8] == ["dec1.c1.w", "dec1.c1.b", "dec1.n1.gamma", "dec1.n1.beta", "dec1.c2.w", "dec1.c2.b", "dec1.n2.gamma", "dec1.n2.beta"]
 
 
 def test_attention_keys_and_extra_shadowing(tmp_path):

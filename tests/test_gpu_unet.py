@@ -39,7 +39,8 @@ def test_unet_forward_matches_oracle_graph(gpu, bits, widths, dims, N, dn):
     assert abs(w0.std() / np.sqrt(2.0 / (cin * 27)) - 1) < 0.1                    # Kaiming normal (src/unet.c:588-593)
     assert (p[lay["head.b"][0]:lay["head.b"][0] + head_out] == -2).all()            # head bias -2 (src/unet.c:607)
     # make the GroupNorm affine non-trivial so a wrong parameter hand-off cannot hide behind gamma 1 / beta 0
-    for k, (off, shp) in lay.items():
+    for k in unet_ref.draw_order(lay):
+        off, shp = lay[k]
         if k.endswith(".gamma"):
             p[off:off + shp[0]] = rng.uniform(0.7, 1.3, shp[0])
         if k.endswith(".beta") or (k.endswith(".b") and k != "head.b"):
@@ -382,7 +383,8 @@ def test_config3_full_size_forward_properties(gpu):
     net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=8), N, D, D, D, seed=2)
     p = net.params()
     lay, n = unet_ref.param_layout(cin, widths, head_out)
-    for k, (off, shp) in lay.items():
+    for k in unet_ref.draw_order(lay):
+        off, shp = lay[k]
         if k.endswith(".gamma"):
             p[off:off + shp[0]] = rng.uniform(0.7, 1.3, shp[0])
         if k.endswith(".beta") or (k.endswith(".b") and k != "head.b"):
@@ -469,7 +471,8 @@ def test_unet_l0_norm_slab(gpu, tmp_path, bits, widths, dims, N, slab, infer):
     p = net.params()
     lay, n = unet_ref.param_layout(cin, widths, head_out, 0)
     assert n == p.size                                             # (the mode adds no parameters)
-    for k, (off, shp) in lay.items():
+    for k in unet_ref.draw_order(lay):
+        off, shp = lay[k]
         if k.endswith(".gamma"):
             p[off:off + shp[0]] = rng.uniform(0.7, 1.3, shp[0])
         if k.endswith(".beta") or (k.endswith(".b") and k != "head.b"):
@@ -606,7 +609,8 @@ def test_unet_l0_norm_constant_modes(gpu, tmp_path, mode, bits, widths):
     p = net.params()
     lay, n = unet_ref.param_layout(cin, widths, head_out, 0)
     assert n == p.size
-    for k, (off, shp) in lay.items():
+    for k in unet_ref.draw_order(lay):
+        off, shp = lay[k]
         if k.endswith(".gamma"):
             p[off:off + shp[0]] = rng.uniform(0.7, 1.3, shp[0])
         if k.endswith(".beta") or (k.endswith(".b") and k != "head.b"):

@@ -14,7 +14,9 @@ import unet_ref
 def make_net(rng, cin, widths, head_out):
     lay, n = unet_ref.param_layout(cin, widths, head_out)
     p = np.zeros(n, np.float32)
-    for k, (off, shp) in lay.items():
+    keys = unet_ref.draw_order(lay)       # (the seeds below were chosen for the nets this order gives)
+    for k in keys:
+        off, shp = lay[k]
         sz = int(np.prod(shp))
         if k.endswith(".w"):
             p[off:off + sz] = rng.standard_normal(sz) * np.sqrt(2.0 / (shp[1] * shp[2]))

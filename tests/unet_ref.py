@@ -23,7 +23,7 @@ def param_layout(cin, widths, head_out, down_norm=0):
         conv("enc%d.c2" % i, widths[i], widths[i], 3); gn("enc%d.n2" % i, widths[i])
     for i in range(L - 1):
         conv("down%d" % i, widths[i], widths[i], 3)
-    for i in range(L - 1):
+    for i in range(L - 2, -1, -1):                   # the decoder blocks from the coarsest (src/unet.c:456)
         conv("dec%d.c1" % i, widths[i + 1] + widths[i], widths[i], 3); gn("dec%d.n1" % i, widths[i])
         conv("dec%d.c2" % i, widths[i], widths[i], 3); gn("dec%d.n2" % i, widths[i])
     conv("head", widths[0], head_out, 1)
@@ -31,6 +31,17 @@ def param_layout(cin, widths, head_out, down_norm=0):
         for i in range(L - 1):
             gn("dn%d" % i, widths[i])
     return lay, off
+
+
+def draw_order(lay):
+    """The layout's keys with the decoder blocks from level 0 up (the encoder's order), wherever they sit in the flat vector: tests that draw
+    random parameters key by key use it, so a seed names the same net whatever the flat layout is."""
+    keys = list(lay)
+    dec = [k for k in keys if k.startswith("dec")]
+    if dec:
+        first = keys.index(dec[0])
+        keys[first:first + len(dec)] = sorted(dec, key=lambda k: (int(k[3:k.index(".")]), dec.index(k)))
+    return keys
 
 
 def slab_stats(bits, y, N, c, g, D, HW, zs):

@@ -1,7 +1,7 @@
 /* The U-Net inference graph (C23) over the op layer: two 3x3x3 convs per level with GroupNorm statistics fused into their
    epilogues and the GroupNorm + SiLU applied by the next reader while it stages its input (recompute mode: no activated tensor is
    ever stored), 3x3x3 stride-2 down convs, decoder conv1 reading [up2(coarse) | skip] without materialising either, 1x1x1 head.
-   Layer and parameter order follow src/unet.c:588-607 (unet_init) and src/unet.c:2567-2636, :2939-3105 (block_fwd, unet_forward_x). */
+   Parameter layout: src/unet.c:451-459 (unet_create); initialisation: src/unet.c:588-607 (unet_init); layer order: src/unet.c:2567-2636, :2939-3105 (block_fwd, unet_forward_x). */
 #include "../../include/mi_unet.h"
 #include <math.h>
 #include <stdio.h>
@@ -118,14 +118,14 @@ unet *unet_create(const unet_cfg *cfg) {
     u->cfg = *cfg;
     const int *w = cfg->widths;
     size_t off = 0;
-    /* parameter order of unet_init: encoder blocks, down convs, decoder blocks, head */
+    /* the layout of the reference's unet_create (src/unet.c:451-459): encoder blocks, down convs, decoder blocks from the coarsest, head, down norms, attention stage */
     for (int i = 0; i < L; i++) {
         block *b = &u->enc[i];
         off = add_conv(&b->c1, i ? w[i - 1] : cfg->cin, w[i], 3, off); off = add_gn(&b->n1, w[i], off);
         off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
     }
     for (int i = 0; i < L - 1; i++) off = add_conv(&u->down[i], w[i], w[i], 3, off);         /* the down conv keeps its level's width (src/unet.c:2970) */
-    for (int i = 0; i < L - 1; i++) {
+    for (int i = L - 2; i >= 0; i--) {                             /* the decoder blocks from the coarsest (src/unet.c:456) */
         block *b = &u->dec[i];
         off = add_conv(&b->c1, w[i + 1] + w[i], w[i], 3, off); off = add_gn(&b->n1, w[i], off);
         off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
