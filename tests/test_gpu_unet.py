@@ -793,3 +793,111 @@ def test_unet_gn_ema(gpu, tmp_path, widths, dn, attn):
     head2 = open(path, "rb").readline().decode()
     assert ',"ge_n":7,"ge_warm":500,' in head2 and ("%.9g" % runs[1][-1]) in head2
     plain.close(); net.close()
+
+
+@pytest.mark.parametrize("bits,widths,dec_widths,dec_convs", [(8, [32, 64, 128], [0, 32], None), (8, [32, 64, 128], None, [2, 1]), (8, [32, 64, 96, 128], [0, 32, 64], [1, 2, 1]),
+                                                               (4, [32, 64, 128], [32, 32], [1, 1])])
+def test_unet_decoder_variants(gpu, tmp_path, bits, widths, dec_widths, dec_convs):
+    """cfg.dec_widths (a decoder block narrower than its level's encoder, src/unet.c:298-300, :452-456) and cfg.dec_convs 1 (one-conv decoder
+    blocks whose output goes by n1, src/unet.c:357-362, :2581-2582): layout size, every layer against the oracle conv on the device layer's
+    inputs, the logits against the oracle head, the checkpoint round trip, slab inference (a level whose decoder differs from its encoder
+    cannot share one buffer: the in-place request runs the direct form there)."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host, unet_cfg
+    H0 = load_host()
+    rng = np.random.default_rng(sum(widths) + bits)
+    N, (D, H, W) = 1, (16, 16, 16)
+    S = D * H * W
+    cin, head_out, G = 4, 3, 8
+    net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits, dec_widths=dec_widths, dec_convs=dec_convs), N, D, H, W, seed=19)
+    p = net.params()
+    lay, n = unet_ref.param_layout(cin, widths, head_out, 0, dec_widths, dec_convs)
+    assert n == p.size
+    for k in unet_ref.draw_order(lay):
+        off, shp = lay[k]
+        if k.endswith(".gamma"):
+            p[off:off + shp[0]] = rng.uniform(0.7, 1.3, shp[0])
+        if k.endswith(".beta") or (k.endswith(".b") and k != "head.b"):
+            p[off:off + shp[0]] = rng.uniform(-0.2, 0.2, shp[0])
+    net.set_params(p)
+    x = rng.standard_normal((N, cin, S)).astype(np.float32)
+    dxq = to_mx(bits, x); xq = dxq.to_numpy(np.uint8)
+    dlog = DevBuf(N * head_out * S * 4)
+    assert net.forward_x(dxq.ptr, dlog.ptr) == 0
+    LP.check()
+    got = dlog.to_numpy(np.float32, (N, head_out, S))
+    dt = 3 if bits == 8 else 4
+    tens, stat, shapes = {"input": xq}, {}, {"input": (N, cin, D, H, W)}
+    for k, (name, ptr, shp) in enumerate(net.layer_outs()):
+        nb = (lib.lp_mx8_bytes if bits == 8 else lib.lp_mx4_bytes)(shp[0], shp[1], shp[2] * shp[3] * shp[4])
+        buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+        tens[name], shapes[name] = buf, shp
+        g, mp, rp = net.layer_stats(k)
+        if g:
+            m = np.empty(N * g, np.float32); r = np.empty(N * g, np.float32)
+            lib.mi_d2h(m.ctypes.data, mp, m.nbytes); lib.mi_d2h(r.ctypes.data, rp, r.nbytes)
+            stat[name] = (g, m, r)
+    graph = unet_ref.layer_inputs(widths, dec_convs)
+    assert [nm for nm, *_ in graph] == [nm for nm in tens if nm != "input"]
+    for i in range(len(widths) - 1):
+        assert shapes["dec%d.c1" % i][1] == unet_ref.dec_width(widths, dec_widths, i)
+    Pm = lambda key: np.ascontiguousarray(p[lay[key][0]:lay[key][0] + int(np.prod(lay[key][1]))].reshape(lay[key][1]))
+
+    def gn_of(layer):
+        nm = unet_ref.norm_of(layer, 0)
+        if nm is None:
+            return None
+        g, m, r = stat[layer]
+        return orc.gn(Pm(nm + ".gamma"), Pm(nm + ".beta"), m, r, g)
+
+    for name, xl, x2l, stride, up in graph:
+        n_, co, d_, h_, w_ = shapes[name]
+        xs = shapes[x2l] if up else shapes[xl]
+        ci = shapes[xl][1] + (shapes[x2l][1] if x2l else 0)
+        cb = 8 if (bits == 8 or ci <= 8) else 4
+        if stride == 2:
+            cb = 4 if (bits == 4 and ci == 32 and co <= 32) else 8
+        want_l, sums = orc.conv3(tens[xl], dt, N, ci, xs[2], xs[3], xs[4], Pm(name + ".w"), Pm(name + ".b"), co, dt, cbits=cb, stride=stride,
+                                 x2=tens[x2l] if x2l else None, c_split=shapes[xl][1] if x2l else 0, up=up, gp=gn_of(xl), gp2=gn_of(x2l) if x2l else None,
+                                 Go=min(G, co), want_stats=stride == 1, stem_tile=int(ci <= 8 and stride == 1))
+        frac, near = code_mismatch_fraction(bits, tens[name], want_l, N, co, d_ * h_ * w_)
+        assert frac < (0.02 if bits == 8 else 0.05) and near, (name, frac, near)
+        if stride == 1:
+            g, m, r = stat[name]
+            mo = np.zeros(N * g, np.float32); ro = np.zeros(N * g, np.float32)
+            orc.lib().orc_gn_finalize(orc.ptr(sums), N * g, (co // g) * d_ * h_ * w_, 1e-5, orc.ptr(mo), orc.ptr(ro))
+            assert np.allclose(m, mo, rtol=2e-3, atol=2e-4) and np.allclose(r, ro, rtol=2e-3), name
+    last = "dec0.c1" if unet_ref.is_single(dec_convs, 0) else "dec0.c2"
+    want = np.zeros((N, head_out, S), np.float32)
+    hw_ = np.ascontiguousarray(Pm("head.w").reshape(head_out, widths[0]))
+    orc.lib().orc_conv1_mx(bits, orc.ptr(tens[last]), N, widths[0], S, orc.ptr(hw_), orc.ptr(Pm("head.b")), head_out, gn_of(last), orc.ptr(want))
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-5
+    # slab inference in both forms: the same logits
+    for direct in (1, 0):
+        H0.unet_set_infer_slab(8); H0.unet_set_slab_direct(direct)
+        try:
+            d2 = DevBuf(N * head_out * S * 4)
+            assert net.forward_x(dxq.ptr, d2.ptr) == 0
+            LP.check()
+        finally:
+            H0.unet_set_infer_slab(0); H0.unet_set_slab_direct(1)
+        assert np.array_equal(d2.to_numpy(np.float32, (N, head_out, S)), got), direct
+    # the checkpoint carries the variant
+    path = str(tmp_path / "dv.ckpt")
+    assert net.save(path, step=2, extra="{}") == 0
+    head = open(path, "rb").readline().decode()
+    if dec_widths and any(dec_widths):
+        assert ',"dec_widths":[%s]' % ",".join(str((dec_widths + [0] * 8)[i]) for i in range(len(widths))) in head
+    if dec_convs and 1 in dec_convs:
+        assert ',"dec_convs":[%s]' % ",".join(str((dec_convs + [0] * 8)[i]) for i in range(len(widths))) in head
+    c2 = unet_cfg()
+    assert H0.unet_peek(path.encode(), C.byref(c2), None) == 0
+    c2.act_dt, c2.prec = bits, 0
+    twin = UNet(c2, N, D, H, W, seed=3)
+    assert twin.load(path) == 2 and np.array_equal(twin.params(), p)
+    d3 = DevBuf(N * head_out * S * 4)
+    assert twin.forward_x(dxq.ptr, d3.ptr) == 0
+    LP.check()
+    assert np.array_equal(d3.to_numpy(np.float32, (N, head_out, S)), got)
+    plain = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits), N, D, H, W, seed=1)
+    assert plain.load(path) == -1
+    plain.close(); twin.close(); net.close()

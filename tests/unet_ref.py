@@ -5,7 +5,17 @@ import numpy as np
 import orc
 
 
-def param_layout(cin, widths, head_out, down_norm=0):
+def dec_width(widths, dec_widths, i):
+    """output channels of the block the decoder upsamples into level i - 1 (dw_of, src/unet.c:298-300): 0 or the bottom level: the encoder's"""
+    return widths[i] if (i >= len(widths) - 1 or not dec_widths or i >= len(dec_widths) or not dec_widths[i]) else dec_widths[i]
+
+
+def is_single(dec_convs, i):
+    return bool(dec_convs) and i < len(dec_convs) and dec_convs[i] == 1
+
+
+def param_layout(cin, widths, head_out, down_norm=0, dec_widths=None, dec_convs=None):
+    """dec_widths / dec_convs: cfg.dec_widths (a decoder block's width, 0 = the encoder's) and cfg.dec_convs (1: one conv, src/unet.c:357-362)"""
     L = len(widths); off = 0; lay = {}
 
     def conv(name, ci, co, k):
@@ -24,8 +34,10 @@ def param_layout(cin, widths, head_out, down_norm=0):
     for i in range(L - 1):
         conv("down%d" % i, widths[i], widths[i], 3)
     for i in range(L - 2, -1, -1):                   # the decoder blocks from the coarsest (src/unet.c:456)
-        conv("dec%d.c1" % i, widths[i + 1] + widths[i], widths[i], 3); gn("dec%d.n1" % i, widths[i])
-        conv("dec%d.c2" % i, widths[i], widths[i], 3); gn("dec%d.n2" % i, widths[i])
+        d = dec_width(widths, dec_widths, i)
+        conv("dec%d.c1" % i, dec_width(widths, dec_widths, i + 1) + widths[i], d, 3); gn("dec%d.n1" % i, d)
+        if not is_single(dec_convs, i):
+            conv("dec%d.c2" % i, d, d, 3); gn("dec%d.n2" % i, d)
     conv("head", widths[0], head_out, 1)
     if down_norm:                                    # GroupNorm after each down conv, appended after the head (src/unet.c:459)
         for i in range(L - 1):
@@ -56,11 +68,11 @@ def slab_stats(bits, y, N, c, g, D, HW, zs):
     return mean, rstd
 
 
-def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0, acc64=0, l0_slab=0):
+def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0, acc64=0, l0_slab=0, dec_widths=None, dec_convs=None):
     """xq: MX bytes of the input. Returns (logits fp32 [N][head_out][S], {layer name: MX bytes}). acc64: the convs' contraction summed in
     double and rounded once (else in fp32, block by block): two correct summation orders of the same graph. l0_slab > 0: cfg.l0_norm 4, the
     level-0 GroupNorms on statistics per z-slab of that many planes."""
-    lay, n = param_layout(cin, widths, head_out, down_norm)
+    lay, n = param_layout(cin, widths, head_out, down_norm, dec_widths, dec_convs)
     assert params.size == n
     P = lambda k: np.ascontiguousarray(params[lay[k][0]:lay[k][0] + int(np.prod(lay[k][1]))].reshape(lay[k][1]))
     L = len(widths); dt = 3 if bits == 8 else 4
@@ -70,9 +82,9 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
 
     live = []
 
-    def l0gn(i, norm, y, ms):
-        """the GroupNorm a reader of level i's tensor y applies: per-sample statistics ms, or, at level 0 under l0_slab, the tensor's per-slab ones"""
-        c, g = widths[i], Gof(widths[i])
+    def l0gn(i, norm, y, ms, c=None):
+        """the GroupNorm a reader of level i's tensor y (c channels) applies: per-sample statistics ms, or, at level 0 under l0_slab, the tensor's per-slab ones"""
+        c = c or widths[i]; g = Gof(c)
         if i == 0 and l0_slab:
             m, r = slab_stats(bits, y, N, c, g, D, H * W, l0_slab)
             live.append((m, r))                  # (the descriptor holds plain addresses)
@@ -118,11 +130,16 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
         coarse = blocks["enc%d" % (L - 1)] if i == L - 2 else blocks["dec%d" % (i + 1)]
         skip = blocks["enc%d" % i]
         S = dims[i][0] * dims[i][1] * dims[i][2]
-        a1, s1 = conv("dec%d.c1" % i, coarse[0], widths[i + 1] + widths[i], dims[i], gp=coarse[1], x2=skip[0], c_split=widths[i + 1], up=1, gp2=skip[1])
-        m1, r1 = finalize(s1, widths[i], S)
-        a2, s2 = conv("dec%d.c2" % i, a1, widths[i], dims[i], gp=l0gn(i, "dec%d.n1" % i, a1, (m1, r1))[0])
-        m2, r2 = finalize(s2, widths[i], S)
-        g2, (m2, r2) = l0gn(i, "dec%d.n2" % i, a2, (m2, r2))
+        dw, dc = dec_width(widths, dec_widths, i), dec_width(widths, dec_widths, i + 1)
+        a1, s1 = conv("dec%d.c1" % i, coarse[0], dc + widths[i], dims[i], gp=coarse[1], x2=skip[0], c_split=dc, up=1, gp2=skip[1])
+        m1, r1 = finalize(s1, dw, S)
+        if is_single(dec_convs, i):                   # one conv: its output is the block's, under n1 (src/unet.c:2581-2582)
+            g1, (m1, r1) = l0gn(i, "dec%d.n1" % i, a1, (m1, r1), dw)
+            blocks["dec%d" % i] = (a1, g1, (m1, r1))
+            continue
+        a2, s2 = conv("dec%d.c2" % i, a1, dw, dims[i], gp=l0gn(i, "dec%d.n1" % i, a1, (m1, r1), dw)[0])
+        m2, r2 = finalize(s2, dw, S)
+        g2, (m2, r2) = l0gn(i, "dec%d.n2" % i, a2, (m2, r2), dw)
         blocks["dec%d" % i] = (a2, g2, (m2, r2))
     last = blocks["dec0"] if L > 1 else blocks["enc0"]
     S = D * H * W
@@ -132,19 +149,21 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
     return logits, outs
 
 
-def layer_inputs(widths):
+def layer_inputs(widths, dec_convs=None):
     """name -> (x layer, x2 layer, stride, up) of every conv in execution order; 'input' is the network input. The GroupNorm a reader
     applies is the statistics of the tensor it reads with the parameters of the block norm that follows that tensor."""
     L = len(widths); g = []
+    dout = lambda i: "dec%d.c%d" % (i, 1 if is_single(dec_convs, i) else 2)
     for i in range(L):
         g.append(("enc%d.c1" % i, "input" if i == 0 else "down%d" % (i - 1), None, 1, 0))
         g.append(("enc%d.c2" % i, "enc%d.c1" % i, None, 1, 0))
         if i < L - 1:
             g.append(("down%d" % i, "enc%d.c2" % i, None, 2, 0))
     for i in range(L - 2, -1, -1):
-        coarse = "enc%d.c2" % (L - 1) if i == L - 2 else "dec%d.c2" % (i + 1)
+        coarse = "enc%d.c2" % (L - 1) if i == L - 2 else dout(i + 1)
         g.append(("dec%d.c1" % i, coarse, "enc%d.c2" % i, 1, 1))
-        g.append(("dec%d.c2" % i, "dec%d.c1" % i, None, 1, 0))
+        if not is_single(dec_convs, i):
+            g.append(("dec%d.c2" % i, "dec%d.c1" % i, None, 1, 0))
     return g
 
 

@@ -17,6 +17,7 @@ typedef struct {
     convp c1, c2; gnpar n1, n2;
     shape5 xs, ys;                                                 /* conv1 input shape (all its channels), block output shape */
     void *a1, *a2;                                                 /* conv outputs (pre-norm, MX) */
+    int single;                                                    /* cfg.dec_convs 1: one conv, its output is a2 with the statistics m2 / r2 and the norm n2 = n1; no c2, a1 unused (src/unet.c:69, :357-362) */
     float *m1, *r1, *m2, *r2;                                      /* their GroupNorm statistics [n * G] */
 } block;
 struct unet {
@@ -57,6 +58,8 @@ static int act_dt_now(void) { return g_act_mx4 ? 4 : 8; }
 
 static int G_of(const unet *u, int c) { return u->cfg.G < c ? u->cfg.G : c; }      /* src/unet.c:297 */
 static size_t add_conv(convp *c, int cin, int cout, int k, size_t off) { c->cin = cin; c->cout = cout; c->k = k; c->w = off; off += (size_t)cout * cin * k * k * k; c->b = off; return off + cout; }
+/* output channels of the block the decoder upsamples into level i - 1: cfg.dec_widths[i], 0 or the bottom level: the encoder's (src/unet.c:298-300) */
+static int dw_of(const unet_cfg *c, int i) { return i >= c->nlev - 1 || !c->dec_widths[i] ? c->widths[i] : c->dec_widths[i]; }
 static size_t add_gn(gnpar *g, int c, size_t off) { g->c = c; g->gamma = off; g->beta = off + c; return off + 2 * (size_t)c; }
 static size_t act_bytes(const unet *u, shape5 s) { return u->act_dt == 4 ? nn_mx4_bytes(s) : nn_mx8_bytes(s); }
 static void *act_new(const unet *u, shape5 s) { const size_t b = act_bytes(u, s); void *p = mi_malloc(b); mi_zero(p, b); nn_set_storage(p, b, u->act_dt); return p; }
@@ -67,9 +70,10 @@ static float *f32_new(size_t n) { float *p = mi_malloc(n * 4); mi_zero(p, n * 4)
 static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->scale_cond) return "scale_cond";
     for (int i = 0; i < UNET_MAXLEV; i++) {
-        if (c->dec_widths[i] && (i >= c->nlev || c->dec_widths[i] != c->widths[i])) return "dec_widths";
+        /* decoder widths: at most the level's encoder width, and that width at level 0 (the head's input); the bottom level has no decoder (src/unet.c:452-455) */
+        if (c->dec_widths[i] && (i >= c->nlev - 1 || c->dec_widths[i] > c->widths[i] || c->dec_widths[i] < 0 || (i == 0 && c->dec_widths[0] != c->widths[0]))) return "dec_widths";
         if (c->enc_blocks[i]) return "enc_blocks";
-        if (c->dec_convs[i] && c->dec_convs[i] != 2) return "dec_convs";
+        if (c->dec_convs[i] && c->dec_convs[i] != 2 && c->dec_convs[i] != 1) return "dec_convs";
     }
     if (c->ds_levels) return "ds_levels";
     if (c->lat_guide || c->lat_nsub) return "lat_guide";
@@ -125,10 +129,12 @@ unet *unet_create(const unet_cfg *cfg) {
         off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
     }
     for (int i = 0; i < L - 1; i++) off = add_conv(&u->down[i], w[i], w[i], 3, off);         /* the down conv keeps its level's width (src/unet.c:2970) */
-    for (int i = L - 2; i >= 0; i--) {                             /* the decoder blocks from the coarsest (src/unet.c:456) */
+    for (int i = L - 2; i >= 0; i--) {                             /* the decoder blocks from the coarsest (src/unet.c:456); conv1 reads [up2(coarse: dw(i + 1)) | skip: w[i]] */
         block *b = &u->dec[i];
-        off = add_conv(&b->c1, w[i + 1] + w[i], w[i], 3, off); off = add_gn(&b->n1, w[i], off);
-        off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
+        const int d = dw_of(cfg, i);
+        off = add_conv(&b->c1, dw_of(cfg, i + 1) + w[i], d, 3, off); off = add_gn(&b->n1, d, off);
+        if (cfg->dec_convs[i] == 1) { b->c2 = b->c1; b->c2.cin = d; b->n2 = b->n1; b->single = 1; }      /* one conv: c2 / n2 alias c1 / n1 */
+        else { off = add_conv(&b->c2, d, d, 3, off); off = add_gn(&b->n2, d, off); }
     }
     off = add_conv(&u->head, w[0], cfg->cout, 1, off);
     if (cfg->down_norm) for (int i = 0; i < L - 1; i++) off = add_gn(&u->dn[i], w[i], off);       /* (appended after the head, src/unet.c:459) */
@@ -213,15 +219,18 @@ static int build_acts(unet *u, shape5 in) {
        l0_slab planes (0: 64). The statistics arrays hold [n][slab][G] and are registered with their geometry, which every reader's gnp_t then carries */
     u->l0s_zs = cfg->l0_norm == 4 ? (cfg->l0_slab > 0 ? cfg->l0_slab : 64) : 0; u->l0s_ns = u->l0s_zs ? in.d / u->l0s_zs : 0;
     u->slab_ip = slab_inplace_now(u); u->slab_nl = u->slab_ip ? slab_levels(u) : 0; u->slab_s = u->slab_ip ? g_infer_slab : 0;
+    /* (a level shares one buffer only if its decoder block has the encoder's width and two convs: the reference's slab_w_ok / any_single
+       conditions, src/unet.c:1163; the levels that do not qualify run the direct form) */
+    for (int i = 0; i < u->slab_nl; i++) if (u->dec[i].c1.cout != w[i] || u->dec[i].single) u->slab_nl = i;
     for (int i = 0; i < L; i++) u->ls[i] = (shape5){in.n, w[i], in.d >> i, in.h >> i, in.w >> i};
     for (int i = 0; i < L; i++) {
         for (int s = 0; s < 2; s++) {
             block *b = s ? &u->dec[i] : &u->enc[i];
             if (s && i == L - 1) continue;
-            b->ys = u->ls[i]; b->xs = u->ls[i]; b->xs.c = b->c1.cin;
+            b->ys = u->ls[i]; b->ys.c = b->c1.cout; b->xs = u->ls[i]; b->xs.c = b->c1.cin;
             if (i < u->slab_nl) { b->a2 = s ? u->enc[i].a2 : act_new(u, b->ys); b->a1 = b->a2; }
-            else { b->a1 = act_new(u, b->ys); b->a2 = act_new(u, b->ys); }
-            const size_t ng = (size_t)in.n * G_of(u, w[i]) * (i == 0 && u->l0s_ns ? u->l0s_ns : 1);
+            else { b->a1 = b->single ? nullptr : act_new(u, b->ys); b->a2 = act_new(u, b->ys); }
+            const size_t ng = (size_t)in.n * G_of(u, b->ys.c) * (i == 0 && u->l0s_ns ? u->l0s_ns : 1);
             b->m1 = f32_new(ng); b->r1 = f32_new(ng); b->m2 = f32_new(ng); b->r2 = f32_new(ng);
             if (i == 0 && u->l0s_ns) { lp_gn_slab_reg(b->m1, u->l0s_zs, 0, u->l0s_ns, in.h * in.w); lp_gn_slab_reg(b->m2, u->l0s_zs, 0, u->l0s_ns, in.h * in.w); }
         }
@@ -252,7 +261,7 @@ static int build_acts(unet *u, shape5 in) {
 }
 static int ensure_built(unet *u, shape5 xs) {
     const int ip = slab_inplace_now(u);
-    if (u->built && !memcmp(&u->in, &xs, sizeof xs) && u->act_dt == act_dt_now() && u->prec == nn_get_prec() && u->slab_ip == ip && (!ip || (u->slab_nl == slab_levels(u) && u->slab_s == g_infer_slab))) return 0;
+    if (u->built && !memcmp(&u->in, &xs, sizeof xs) && u->act_dt == act_dt_now() && u->prec == nn_get_prec() && u->slab_ip == ip && (!ip || u->slab_s == g_infer_slab)) return 0;
     return build_acts(u, xs);
 }
 void unet_free(unet *u) {
@@ -285,12 +294,12 @@ static void fw_refresh(unet *u) {
     const int L = u->cfg.nlev;
     if (u->cfg.l0_norm == 3) {         /* ws: the four level-0 3^3 convs standardised per output channel over its fan-in; the network input conv without the SiLU gain (src/unet.c:5298-5304, :5311-5318) */
         const convp *wc[4] = {&u->enc[0].c1, &u->enc[0].c2, &u->dec[0].c1, &u->dec[0].c2};
-        for (int i = 0; i < (L > 1 ? 4 : 2); i++) nn_ws_fwd(u->wm + wc[i]->w, u->src + wc[i]->w, wc[i]->cout, wc[i]->cin * 27, i ? u->ws_gain : 1.f, 1e-5f);
+        for (int i = 0; i < (L > 1 ? (u->dec[0].single ? 3 : 4) : 2); i++) nn_ws_fwd(u->wm + wc[i]->w, u->src + wc[i]->w, wc[i]->cout, wc[i]->cin * 27, i ? u->ws_gain : 1.f, 1e-5f);
     }
     if (u->cfg.w4_2d) {
         const convp *cs[4 * UNET_MAXLEV]; int n = 0;
         for (int i = 0; i < L; i++) { if (i) cs[n++] = &u->enc[i].c1; cs[n++] = &u->enc[i].c2; }
-        for (int i = 0; i < L - 1; i++) { cs[n++] = &u->dec[i].c1; cs[n++] = &u->dec[i].c2; }
+        for (int i = 0; i < L - 1; i++) { cs[n++] = &u->dec[i].c1; if (!u->dec[i].single) cs[n++] = &u->dec[i].c2; }
         for (int i = 0; i < n; i++) nn_fakeq_w4_2d(u->wm + cs[i]->w, cs[i]->cout, cs[i]->cin, 27, 32);
     }
     lp_wmemo_clear();
@@ -316,7 +325,7 @@ void unet_init(unet *u, uint64_t seed) {
     const int L = u->cfg.nlev;
     for (int i = 0; i < L; i++) { init_conv(h, &u->enc[i].c1, &seed, 0); init_gn(h, &u->enc[i].n1); init_conv(h, &u->enc[i].c2, &seed, 0); init_gn(h, &u->enc[i].n2); }
     for (int i = 0; i < L - 1; i++) init_conv(h, &u->down[i], &seed, 0);
-    for (int i = 0; i < L - 1; i++) { init_conv(h, &u->dec[i].c1, &seed, 0); init_gn(h, &u->dec[i].n1); init_conv(h, &u->dec[i].c2, &seed, 0); init_gn(h, &u->dec[i].n2); }
+    for (int i = 0; i < L - 1; i++) { init_conv(h, &u->dec[i].c1, &seed, 0); init_gn(h, &u->dec[i].n1); if (!u->dec[i].single) { init_conv(h, &u->dec[i].c2, &seed, 0); init_gn(h, &u->dec[i].n2); } }
     init_conv(h, &u->head, &seed, -2.0);
     if (u->cfg.down_norm) for (int i = 0; i < L - 1; i++) init_gn(h, &u->dn[i]);
     if (u->tbn) {   /* LayerNorm and QK-norm gains 1, QKV and MLP-in N(0, 1 / C), out projections and biases 0 (identity blocks), registers N(0, 0.02^2) (src/unet.c:612-642) */
@@ -367,6 +376,7 @@ static void l0_const_fill(unet *u) {
     const int G = G_of(u, u->cfg.widths[0]), N = u->in.n;
     for (int i = 0; i < (u->cfg.nlev > 1 ? 2 : 1); i++) for (int k = 1; k <= 2; k++) {
         block *b = i ? &u->dec[0] : &u->enc[0];
+        if (k == 1 && b->single) continue;                         /* (src/unet.c:2320) */
         const float *run = u->cfg.l0_norm == 2 ? u->l0run + (u->src == u->ema ? (size_t)8 * G : 0) + (size_t)(2 * i + k - 1) * 2 * G : nullptr;      /* (the EMA weights have their own) */
         nn_gn_const_fill(k == 1 ? b->m1 : b->m2, k == 1 ? b->r1 : b->r2, run, N, G, 1e-5f);
     }
@@ -381,18 +391,20 @@ static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t 
     const int s = level >= slab_levels(u) ? 0 : g_infer_slab < D ? g_infer_slab : ip ? D : 0;      /* (in place: a level of fewer planes is one slab) */
     void *tmp = ip ? u->slab_tmp[level] : nullptr, *carry = ip ? u->slab_carry[level] : nullptr;
     int r = 0;
-    for (int conv = 1; conv <= 2 && !r; conv++) {
+    for (int conv = b->single ? 2 : 1; conv <= 2 && !r; conv++) {  /* (one-conv decoder block: its conv, with c1's weights, writes a2 and the statistics m2 / r2, src/unet.c:2581-2582) */
         void *y = conv == 1 ? b->a1 : b->a2;
-        const int over = ip && (conv == 2 || x == y);              /* the conv reads the buffer it writes: through the temp */
+        const int first = conv == 1 || b->single;                  /* this conv reads the block's input */
+        const int over = ip && (!first || x == y);                 /* the conv reads the buffer it writes: through the temp */
+        float *om = conv == 1 ? b->m1 : b->m2, *orr = conv == 1 ? b->r1 : b->r2;
         for (int z0 = 0, k = 0, sk; z0 < D && !r; z0 += sk, k++) {
             sk = s && D - z0 > s ? s : D - z0;
             const int last = z0 + sk >= D;
-            shape5 xs = conv == 1 ? b->xs : b->ys;
+            shape5 xs = first ? b->xs : b->ys;
             if (s) { nn_set_zrange(z0, D, z0 == 0, last, D, z0); nn_set_zrange_out(!over); xs.d = sk; }
             void *o = over ? tmp : y;
-            if (conv == 2) r = nn_conv3d_fwd_gn_stats(b->a1, xs, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, o, Gc, 1e-5f, b->m2, b->r2);
-            else if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, b->m1, b->r1);   /* [up2(coarse) | skip] */
-            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, b->m1, b->r1);
+            if (!first) r = nn_conv3d_fwd_gn_stats(b->a1, xs, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, o, Gc, 1e-5f, om, orr);
+            else if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, om, orr);   /* [up2(coarse) | skip] */
+            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, om, orr);
             if (s) { nn_set_zrange(0, 0, 0, 0, 0, 0); nn_set_zrange_out(0); }
             if (over && !r) {                                      /* planes below the next slab's first input plane are dead: the last one waits */
                 if (k) copy_planes(u, y, D, z0 - 1, carry, 1, 0, 1, b->ys);
@@ -402,9 +414,9 @@ static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t 
         }
         if (!r && l0s) {
             shape5 ps = b->ys; ps.n *= u->l0s_ns; ps.d = u->l0s_zs;
-            if (nn_gn_stats(y, ps, G, 1e-5f, conv == 1 ? b->m1 : b->m2, conv == 1 ? b->r1 : b->r2)) { fprintf(stderr, "unet: per-slab GroupNorm statistics unsupported for this storage\n"); r = -1; }
+            if (nn_gn_stats(y, ps, G, 1e-5f, om, orr)) { fprintf(stderr, "unet: per-slab GroupNorm statistics unsupported for this storage\n"); r = -1; }
         }
-        if (!r) { if (conv == 1) note(u, b->a1, b->ys, n1, b->m1, b->r1, G); else note(u, b->a2, b->ys, n2, b->m2, b->r2, G); }
+        if (!r) note(u, y, b->ys, first ? n1 : n2, om, orr, G);    /* (a one-conv block's output goes by its conv's name) */
     }
     return r;
 }
@@ -460,7 +472,7 @@ static int graph_fwd(unet *u, const void *x) {
         nn_gn_t gc = gn_out(u, coarse); const nn_gn_t gs = gn_out(u, &u->enc[i]);
         if (i == L - 2 && u->tbn) { coarse = &u->tb; gc.mean = u->tb.m2; gc.rstd = u->tb.r2; }      /* the stage's output under the level's n2 affine (src/unet.c:508) */
         static const nn_gn_t none = {nullptr, nullptr, nullptr, nullptr, -1};          /* the pre-staged skip: no GroupNorm left to apply */
-        if (block_fwd(u, &u->dec[i], i, u->skipst[i] ? u->skipst[i] : u->enc[i].a2, u->skipst[i] ? &none : &gs, coarse->a2, &gc, u->cfg.widths[i + 1], dn1[i], dn2[i])) return -1;
+        if (block_fwd(u, &u->dec[i], i, u->skipst[i] ? u->skipst[i] : u->enc[i].a2, u->skipst[i] ? &none : &gs, coarse->a2, &gc, coarse->ys.c, dn1[i], dn2[i])) return -1;
     }
     const block *last = L > 1 ? &u->dec[0] : &u->enc[0];
     const nn_gn_t g = gn_out(u, last);
@@ -541,6 +553,8 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     p += 10;
     for (int i = 0; i < cfg->nlev; i++) { cfg->widths[i] = atoi(p); p = strchr(p, ','); if (!p) break; p++; }
     cfg->cin = key_int(line, "\"cin\":", 0); cfg->cout = key_int(line, "\"cout\":", 0); cfg->G = key_int(line, "\"G\":", 8);
+    if ((p = strstr(line, "\"dec_widths\":["))) { p += 14; for (int i = 0; i < UNET_MAXLEV && *p && *p != ']'; i++) { char *e; cfg->dec_widths[i] = (int)strtol(p, &e, 10); p = e; if (*p == ',') p++; } }      /* (src/unet.c:5674) */
+    if ((p = strstr(line, "\"dec_convs\":["))) { p += 13; for (int i = 0; i < UNET_MAXLEV && *p && *p != ']'; i++) { char *e; cfg->dec_convs[i] = (int)strtol(p, &e, 10); p = e; if (*p == ',') p++; } }        /* (src/unet.c:5700) */
     cfg->down_norm = key_int(line, "\"down_norm\":", 0); cfg->w4_2d = key_int(line, "\"w4_2d\":", 0);
     cfg->l0_norm = key_int(line, "\"l0_norm\":", 0); cfg->l0_slab = key_int(line, "\"l0_slab\":", 0);      /* (src/unet.c:5726) */
     cfg->gn_ema = key_int(line, "\"gn_ema\":", 0);
@@ -550,9 +564,9 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
-    static const char *const no[] = {"\"dec_widths\":", "\"enc_blocks\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"ds_levels\":", "\"emb_lev\":",
+    static const char *const no[] = {"\"enc_blocks\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"ds_levels\":", "\"emb_lev\":",
                                      "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
-                                     "\"skip_empty\":", "\"gfilm\":", "\"dec_convs\":"};
+                                     "\"skip_empty\":", "\"gfilm\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
     if (!bad && key_int(line, "\"scale_cond\":", 0)) bad = "\"scale_cond\":";
@@ -588,6 +602,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
     if (!bad && c.gn_ema != m->gn_ema) bad = "gn_ema";
+    for (int i = 0; !bad && i < m->nlev - 1; i++) { if (dw_of(&c, i) != dw_of(m, i)) bad = "dec_widths"; if ((c.dec_convs[i] == 1) != (m->dec_convs[i] == 1)) bad = "dec_convs"; }
     if (!bad && (c.l0_norm != m->l0_norm || (c.l0_norm == 4 && (c.l0_slab > 0 ? c.l0_slab : 64) != (m->l0_slab > 0 ? m->l0_slab : 64)))) bad = "l0_norm / l0_slab";
     if (!bad && np != u->np) bad = "nparams";
     if (bad) { fprintf(stderr, "unet_load: %s: \"%s\" differs from this network's\n", path, bad); return -1; }
@@ -641,6 +656,8 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     fprintf(f, "UFSM{\"nlev\":%d,\"widths\":[", u->cfg.nlev);
     for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.widths[i]);
     fputc(']', f);
+    { int any = 0; for (int i = 0; i < u->cfg.nlev; i++) any |= u->cfg.dec_widths[i] != 0;       /* (only when set, src/unet.c:5549-5550) */
+      if (any) { fputs(",\"dec_widths\":[", f); for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.dec_widths[i]); fputc(']', f); } }
     /* (the reference's key order, src/unet.c:5561-5578: w4_2d, the attention keys, l0_norm / l0_slab, then cin) */
     if (u->cfg.w4_2d) fprintf(f, ",\"w4_2d\":%d", u->cfg.w4_2d);
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
@@ -662,6 +679,8 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
         for (int i = 0; i < n; i++) fprintf(f, "%s%.9g", i ? "," : "", (double)r[i]);
         fputc(']', f);
     }
+    { int any = 0; for (int i = 0; i < u->cfg.nlev; i++) any |= u->cfg.dec_convs[i] == 1;        /* (src/unet.c:5595-5596) */
+      if (any) { fputs(",\"dec_convs\":[", f); for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.dec_convs[i]); fputc(']', f); } }
     fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":0,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.cout, u->cfg.G,
             u->cfg.down_norm, u->np, step);
     fprintf(f, ",\"extra\":%s}\n", extra ? extra : "{}");
