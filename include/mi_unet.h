@@ -43,7 +43,7 @@ const char *nn_check(void);                                    /* src/nn.h:28 */
 /* The reference's configuration record, field for field (src/unet.h:18-128): the layout is part of the boundary. This build runs the plain
    U-Net (+ down_norm, + self-attention blocks with RoPE / no positional encoding and register tokens). Fields it honours: nlev, widths, cin,
    cout, G, down_norm, attn_blocks, attn_pe (1 or 2), attn_reg, attn_mlp, dec_widths (0: the encoder's width), dec_convs (1: one-conv decoder block),
-   w4_2d, l0_norm (0 .. 4) with l0_slab, gn_ema; half_res and scan_norm concern the caller only. Any other field must be 0: unet_create prints which one is not and returns NULL. */
+   enc_blocks (residual blocks after encoder levels >= 1), w4_2d, l0_norm (0 .. 4) with l0_slab, gn_ema; half_res and scan_norm concern the caller only. Any other field must be 0: unet_create prints which one is not and returns NULL. */
 typedef struct {
     int nlev;
     int widths[UNET_MAXLEV];

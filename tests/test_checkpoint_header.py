@@ -59,7 +59,7 @@ def test_caller_side_keys_pass_through(tmp_path):
     assert rc == 0 and cfg.half_res == 1 and cfg.scan_norm == 1
 
 
-@pytest.mark.parametrize("feature", ['"lat_guide":1', '"enc_blocks":[0,1]', '"ds_levels":2', '"film":2', '"fstem":[2,16]', '"gfilm":1', '"attn_vres":1', '"l0_norm":7'])
+@pytest.mark.parametrize("feature", ['"lat_guide":1', '"emb_lev":1,"emb_ch":8', '"ds_levels":2', '"film":2', '"fstem":[2,16]', '"gfilm":1', '"attn_vres":1', '"l0_norm":7'])
 def test_refuses_architectures_it_does_not_run(tmp_path, feature):
     h = 'UFSM{"nlev":2,"widths":[32,64],%s,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":1,"extra":{}}\n' % feature
     assert read(tmp_path, h)[0] == -2
@@ -85,9 +85,9 @@ def test_reads_the_slab_statistics_keys(tmp_path):
 
 def test_reads_the_decoder_variants(tmp_path):
     # cfg.dec_widths / cfg.dec_convs as unet_save writes them (src/unet.c:5549-5550, :5595-5596; read at :5674, :5700)
-    h = 'UFSM{"nlev":3,"widths":[32,64,128],"dec_widths":[0,32,0],"dec_convs":[2,1,0],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":3,"extra":{}}\n'
+    h = 'UFSM{"nlev":3,"widths":[32,64,128],"dec_widths":[0,32,0],"enc_blocks":[0,2,1],"dec_convs":[2,1,0],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":3,"extra":{}}\n'
     rc, cfg, n, step = read(tmp_path, h)
-    assert rc == 0 and list(cfg.dec_widths[:3]) == [0, 32, 0] and list(cfg.dec_convs[:3]) == [2, 1, 0] and list(cfg.widths[:3]) == [32, 64, 128]
+    assert rc == 0 and list(cfg.dec_widths[:3]) == [0, 32, 0] and list(cfg.dec_convs[:3]) == [2, 1, 0] and list(cfg.widths[:3]) == [32, 64, 128] and list(cfg.enc_blocks[:3]) == [0, 2, 1]
 
 
 def test_reads_the_running_statistics_key(tmp_path):

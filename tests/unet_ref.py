@@ -14,8 +14,9 @@ def is_single(dec_convs, i):
     return bool(dec_convs) and i < len(dec_convs) and dec_convs[i] == 1
 
 
-def param_layout(cin, widths, head_out, down_norm=0, dec_widths=None, dec_convs=None):
-    """dec_widths / dec_convs: cfg.dec_widths (a decoder block's width, 0 = the encoder's) and cfg.dec_convs (1: one conv, src/unet.c:357-362)"""
+def param_layout(cin, widths, head_out, down_norm=0, dec_widths=None, dec_convs=None, enc_blocks=None):
+    """dec_widths / dec_convs: cfg.dec_widths (a decoder block's width, 0 = the encoder's) and cfg.dec_convs (1: one conv, src/unet.c:357-362);
+    enc_blocks: cfg.enc_blocks, residual blocks after encoder level i, their parameters after everything older (src/unet.c:461-465)"""
     L = len(widths); off = 0; lay = {}
 
     def conv(name, ci, co, k):
@@ -42,7 +43,24 @@ def param_layout(cin, widths, head_out, down_norm=0, dec_widths=None, dec_convs=
     if down_norm:                                    # GroupNorm after each down conv, appended after the head (src/unet.c:459)
         for i in range(L - 1):
             gn("dn%d" % i, widths[i])
+    for i, nb in enumerate(enc_blocks or []):
+        for k in range(nb):
+            conv("rb%d.%d.c1" % (i, k), widths[i], widths[i], 3); gn("rb%d.%d.n1" % (i, k), widths[i])
+            conv("rb%d.%d.c2" % (i, k), widths[i], widths[i], 3); gn("rb%d.%d.n2" % (i, k), widths[i])
     return lay, off
+
+
+def add_mx(bits, a, b, N, C, S):
+    """y = a + b on MX tensors: decode, add in fp32, re-quantise (lp_add_mx, src/lp_mx_gn.cu:134-143)"""
+    return orc.f32_to_mx(bits, orc.mx_to_f32(bits, a, N, C, S) + orc.mx_to_f32(bits, b, N, C, S), N, C, S)
+
+
+def stored_stats(bits, y, N, c, g, S):
+    sums = np.zeros((N, g, 2), np.float64)
+    orc.lib().orc_gn_sums_mx(bits, orc.ptr(y), N, c, g, S, orc.ptr(sums), 0, S)
+    mean = np.zeros(N * g, np.float32); rstd = np.zeros(N * g, np.float32)
+    orc.lib().orc_gn_finalize(orc.ptr(sums), N * g, (c // g) * S, 1e-5, orc.ptr(mean), orc.ptr(rstd))
+    return mean, rstd
 
 
 def draw_order(lay):
@@ -68,11 +86,11 @@ def slab_stats(bits, y, N, c, g, D, HW, zs):
     return mean, rstd
 
 
-def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0, acc64=0, l0_slab=0, dec_widths=None, dec_convs=None):
+def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, stored=0, down_norm=0, acc64=0, l0_slab=0, dec_widths=None, dec_convs=None, enc_blocks=None):
     """xq: MX bytes of the input. Returns (logits fp32 [N][head_out][S], {layer name: MX bytes}). acc64: the convs' contraction summed in
     double and rounded once (else in fp32, block by block): two correct summation orders of the same graph. l0_slab > 0: cfg.l0_norm 4, the
     level-0 GroupNorms on statistics per z-slab of that many planes."""
-    lay, n = param_layout(cin, widths, head_out, down_norm, dec_widths, dec_convs)
+    lay, n = param_layout(cin, widths, head_out, down_norm, dec_widths, dec_convs, enc_blocks)
     assert params.size == n
     P = lambda k: np.ascontiguousarray(params[lay[k][0]:lay[k][0] + int(np.prod(lay[k][1]))].reshape(lay[k][1]))
     L = len(widths); dt = 3 if bits == 8 else 4
@@ -118,6 +136,16 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
         m2, r2 = finalize(s2, widths[i], S)
         g2, (m2, r2) = l0gn(i, "enc%d.n2" % i, a2, (m2, r2))
         blocks["enc%d" % i] = (a2, g2, (m2, r2))
+        for k in range((enc_blocks or [0] * L)[i]):      # residual blocks (rblock_fwd, src/unet.c:2656-2671): the stage output replaces enc<i>'s
+            nm = "rb%d.%d" % (i, k); prev = blocks["enc%d" % i]
+            b1, t1 = conv(nm + ".c1", prev[0], widths[i], dims[i], gp=prev[1])
+            bm1, br1 = finalize(t1, widths[i], S)
+            b2, _ = conv(nm + ".c2", b1, widths[i], dims[i], gp=orc.gn(P(nm + ".n1.gamma"), P(nm + ".n1.beta"), bm1, br1, Gof(widths[i])), stats=False)
+            b2 = add_mx(bits, b2, prev[0], N, widths[i], S); outs[nm + ".c2"] = b2
+            bm2, br2 = stored_stats(bits, b2, N, widths[i], Gof(widths[i]), S)
+            live.append((bm1, br1, bm2, br2))
+            blocks["enc%d" % i] = (b2, orc.gn(P(nm + ".n2.gamma"), P(nm + ".n2.beta"), bm2, br2, Gof(widths[i])), (bm2, br2))
+            a2 = b2
         if i < L - 1:
             cur, _ = conv("down%d" % i, a2, widths[i], dims[i], gp=blocks["enc%d" % i][1], stride=2, stats=False)
             if down_norm:                     # statistics of the stored down-conv output, applied by the next conv1 (src/unet.c:2974-2979)
@@ -149,19 +177,24 @@ def forward(params, cin, widths, G, head_out, bits, xq, N, D, H, W, cbits=None, 
     return logits, outs
 
 
-def layer_inputs(widths, dec_convs=None):
+def layer_inputs(widths, dec_convs=None, enc_blocks=None):
     """name -> (x layer, x2 layer, stride, up) of every conv in execution order; 'input' is the network input. The GroupNorm a reader
     applies is the statistics of the tensor it reads with the parameters of the block norm that follows that tensor."""
     L = len(widths); g = []
     dout = lambda i: "dec%d.c%d" % (i, 1 if is_single(dec_convs, i) else 2)
+    nrb = lambda i: (enc_blocks or [0] * L)[i] if i < len(enc_blocks or [0] * L) else 0
+    eout = lambda i: "rb%d.%d.c2" % (i, nrb(i) - 1) if nrb(i) else "enc%d.c2" % i      # the stage output: the last residual block's (a rb c2 tensor is its conv + the previous output)
     for i in range(L):
         g.append(("enc%d.c1" % i, "input" if i == 0 else "down%d" % (i - 1), None, 1, 0))
         g.append(("enc%d.c2" % i, "enc%d.c1" % i, None, 1, 0))
+        for k in range(nrb(i)):
+            g.append(("rb%d.%d.c1" % (i, k), "rb%d.%d.c2" % (i, k - 1) if k else "enc%d.c2" % i, None, 1, 0))
+            g.append(("rb%d.%d.c2" % (i, k), "rb%d.%d.c1" % (i, k), None, 1, 0))
         if i < L - 1:
-            g.append(("down%d" % i, "enc%d.c2" % i, None, 2, 0))
+            g.append(("down%d" % i, eout(i), None, 2, 0))
     for i in range(L - 2, -1, -1):
-        coarse = "enc%d.c2" % (L - 1) if i == L - 2 else dout(i + 1)
-        g.append(("dec%d.c1" % i, coarse, "enc%d.c2" % i, 1, 1))
+        coarse = eout(L - 1) if i == L - 2 else dout(i + 1)
+        g.append(("dec%d.c1" % i, coarse, eout(i), 1, 1))
         if not is_single(dec_convs, i):
             g.append(("dec%d.c2" % i, "dec%d.c1" % i, None, 1, 0))
     return g
@@ -174,5 +207,5 @@ def norm_of(layer, down_norm=0):
         return "dn" + layer[4:] if down_norm else None
     if layer == "input":
         return None
-    blk, c = layer.split(".")
+    blk, c = layer.rsplit(".", 1)
     return blk + (".n1" if c == "c1" else ".n2")

@@ -34,6 +34,7 @@ struct unet {
     int slab_ip, slab_nl, slab_s;      /* the build's in-place slab plan: on, and over how many levels (a level's tensors all live in enc[i].a2's buffer) */
     void *slab_tmp[2], *slab_carry[2]; /* per such level: one slab of output planes, and the plane that waits for the next slab */
     block enc[UNET_MAXLEV], dec[UNET_MAXLEV];
+    block *rb[UNET_MAXLEV]; char (*rbn[UNET_MAXLEV])[2][16];      /* cfg.enc_blocks: residual blocks after encoder level i (src/unet.c:96, :461-465), the names of their convs */
     convp down[UNET_MAXLEV], head;
     void *downo[UNET_MAXLEV];
     void *skipst[UNET_MAXLEV];         /* silu(gn(enc[i].a2)) in the compute format, formed once for its two readers (down conv, decoder conv1); null: each reader transforms it */
@@ -72,7 +73,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     for (int i = 0; i < UNET_MAXLEV; i++) {
         /* decoder widths: at most the level's encoder width, and that width at level 0 (the head's input); the bottom level has no decoder (src/unet.c:452-455) */
         if (c->dec_widths[i] && (i >= c->nlev - 1 || c->dec_widths[i] > c->widths[i] || c->dec_widths[i] < 0 || (i == 0 && c->dec_widths[0] != c->widths[0]))) return "dec_widths";
-        if (c->enc_blocks[i]) return "enc_blocks";
+        if (c->enc_blocks[i] < 0 || c->enc_blocks[i] > 64 || (c->enc_blocks[i] && (i == 0 || i >= c->nlev))) return "enc_blocks (levels 1 and deeper)";      /* (src/unet.c:462) */
         if (c->dec_convs[i] && c->dec_convs[i] != 2 && c->dec_convs[i] != 1) return "dec_convs";
     }
     if (c->ds_levels) return "ds_levels";
@@ -106,6 +107,7 @@ static size_t ge_sites(unet *u, float **mean, float **rstd, int *g, size_t *off)
     for (int i = 0; i < L; i++) { block *b = &u->enc[i]; GE_SITE(b->m1, b->r1, G_of(u, b->c1.cout)); GE_SITE(b->m2, b->r2, G_of(u, b->c2.cout)); }
     if (u->cfg.down_norm) for (int i = 0; i < L - 1; i++) GE_SITE(u->dm[i], u->dr[i], G_of(u, u->cfg.widths[i]));
     for (int i = L - 2; i >= 0; i--) { block *b = &u->dec[i]; GE_SITE(b->m1, b->r1, G_of(u, b->c1.cout)); GE_SITE(b->m2, b->r2, G_of(u, b->c2.cout)); }
+    for (int i = 0; i < L; i++) for (int j = 0; j < u->cfg.enc_blocks[i]; j++) { block *b = &u->rb[i][j]; GE_SITE(b->m1, b->r1, G_of(u, b->c1.cout)); GE_SITE(b->m2, b->r2, G_of(u, b->c2.cout)); }
     if (u->tbn) GE_SITE(u->tb.m2, u->tb.r2, G_of(u, u->tbd.C));
 #undef GE_SITE
     if (mean && k > 192) { fprintf(stderr, "unet: gn_ema: %d GroupNorm sites (at most 192)\n", k); abort(); }
@@ -138,6 +140,15 @@ unet *unet_create(const unet_cfg *cfg) {
     }
     off = add_conv(&u->head, w[0], cfg->cout, 1, off);
     if (cfg->down_norm) for (int i = 0; i < L - 1; i++) off = add_gn(&u->dn[i], w[i], off);       /* (appended after the head, src/unet.c:459) */
+    for (int i = 0; i < L; i++) if (cfg->enc_blocks[i] > 0) {      /* residual blocks after encoder level i: parameters after everything older (src/unet.c:461-465) */
+        u->rb[i] = calloc((size_t)cfg->enc_blocks[i], sizeof(block)); u->rbn[i] = calloc((size_t)cfg->enc_blocks[i], sizeof *u->rbn[i]);
+        for (int k = 0; k < cfg->enc_blocks[i]; k++) {
+            block *b = &u->rb[i][k];
+            off = add_conv(&b->c1, w[i], w[i], 3, off); off = add_gn(&b->n1, w[i], off);
+            off = add_conv(&b->c2, w[i], w[i], 3, off); off = add_gn(&b->n2, w[i], off);
+            snprintf(u->rbn[i][k][0], 16, "rb%d.%d.c1", i, k); snprintf(u->rbn[i][k][1], 16, "rb%d.%d.c2", i, k);
+        }
+    }
     if (cfg->attn_blocks > 0) {                                   /* parameters last: registers, then the blocks (src/unet.c:490-499) */
         const int C = w[L - 1];
         if (C % AT_HD || cfg->attn_blocks > 16 || (cfg->attn_pe != 1 && cfg->attn_pe != 2) || cfg->attn_reg < 0) {
@@ -197,6 +208,11 @@ static void free_acts(unet *u) {
             act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2);
             b->a1 = b->a2 = nullptr; b->m1 = b->r1 = b->m2 = b->r2 = nullptr;
         }
+        for (int k = 0; k < u->cfg.enc_blocks[i]; k++) {
+            block *b = &u->rb[i][k];
+            act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2);
+            b->a1 = b->a2 = nullptr; b->m1 = b->r1 = b->m2 = b->r2 = nullptr;
+        }
         act_del(u->downo[i]); act_del(u->skipst[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
         u->downo[i] = u->skipst[i] = nullptr; u->dm[i] = u->dr[i] = nullptr;
     }
@@ -221,7 +237,7 @@ static int build_acts(unet *u, shape5 in) {
     u->slab_ip = slab_inplace_now(u); u->slab_nl = u->slab_ip ? slab_levels(u) : 0; u->slab_s = u->slab_ip ? g_infer_slab : 0;
     /* (a level shares one buffer only if its decoder block has the encoder's width and two convs: the reference's slab_w_ok / any_single
        conditions, src/unet.c:1163; the levels that do not qualify run the direct form) */
-    for (int i = 0; i < u->slab_nl; i++) if (u->dec[i].c1.cout != w[i] || u->dec[i].single) u->slab_nl = i;
+    for (int i = 0; i < u->slab_nl; i++) if (u->dec[i].c1.cout != w[i] || u->dec[i].single || cfg->enc_blocks[i]) u->slab_nl = i;
     for (int i = 0; i < L; i++) u->ls[i] = (shape5){in.n, w[i], in.d >> i, in.h >> i, in.w >> i};
     for (int i = 0; i < L; i++) {
         for (int s = 0; s < 2; s++) {
@@ -233,6 +249,13 @@ static int build_acts(unet *u, shape5 in) {
             const size_t ng = (size_t)in.n * G_of(u, b->ys.c) * (i == 0 && u->l0s_ns ? u->l0s_ns : 1);
             b->m1 = f32_new(ng); b->r1 = f32_new(ng); b->m2 = f32_new(ng); b->r2 = f32_new(ng);
             if (i == 0 && u->l0s_ns) { lp_gn_slab_reg(b->m1, u->l0s_zs, 0, u->l0s_ns, in.h * in.w); lp_gn_slab_reg(b->m2, u->l0s_zs, 0, u->l0s_ns, in.h * in.w); }
+        }
+        for (int k = 0; k < cfg->enc_blocks[i]; k++) {
+            block *b = &u->rb[i][k];
+            b->ys = b->xs = u->ls[i];
+            b->a1 = act_new(u, b->ys); b->a2 = act_new(u, b->ys);
+            const size_t ng = (size_t)in.n * G_of(u, w[i]);
+            b->m1 = f32_new(ng); b->r1 = f32_new(ng); b->m2 = f32_new(ng); b->r2 = f32_new(ng);
         }
         if (i < L - 1) {
             shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds);
@@ -269,6 +292,7 @@ void unet_free(unet *u) {
     mi_sync();
     free_acts(u);
     mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm); if (u->l0run) mi_free(u->l0run); if (u->ge_run) mi_free(u->ge_run);
+    for (int i = 0; i < UNET_MAXLEV; i++) { free(u->rb[i]); free(u->rbn[i]); }
     lp_wmemo_clear();
     free(u);
 }
@@ -301,6 +325,9 @@ static void fw_refresh(unet *u) {
         for (int i = 0; i < L; i++) { if (i) cs[n++] = &u->enc[i].c1; cs[n++] = &u->enc[i].c2; }
         for (int i = 0; i < L - 1; i++) { cs[n++] = &u->dec[i].c1; if (!u->dec[i].single) cs[n++] = &u->dec[i].c2; }
         for (int i = 0; i < n; i++) nn_fakeq_w4_2d(u->wm + cs[i]->w, cs[i]->cout, cs[i]->cin, 27, 32);
+        n = 0;
+        for (int i = 0; i < L; i++) for (int k = 0; k < u->cfg.enc_blocks[i]; k++) { if (n + 2 > 4 * UNET_MAXLEV) { for (int j = 0; j < n; j++) nn_fakeq_w4_2d(u->wm + cs[j]->w, cs[j]->cout, cs[j]->cin, 27, 32); n = 0; } cs[n++] = &u->rb[i][k].c1; cs[n++] = &u->rb[i][k].c2; }      /* (src/unet.c:5338) */
+        for (int i = 0; i < n; i++) nn_fakeq_w4_2d(u->wm + cs[i]->w, cs[i]->cout, cs[i]->cin, 27, 32);
     }
     lp_wmemo_clear();
     u->wm_ok = 1;
@@ -327,6 +354,12 @@ void unet_init(unet *u, uint64_t seed) {
     for (int i = 0; i < L - 1; i++) init_conv(h, &u->down[i], &seed, 0);
     for (int i = 0; i < L - 1; i++) { init_conv(h, &u->dec[i].c1, &seed, 0); init_gn(h, &u->dec[i].n1); if (!u->dec[i].single) { init_conv(h, &u->dec[i].c2, &seed, 0); init_gn(h, &u->dec[i].n2); } }
     init_conv(h, &u->head, &seed, -2.0);
+    for (int i = 0; i < L; i++) for (int k = 0; k < u->cfg.enc_blocks[i]; k++) {      /* residual blocks start as the identity: conv2's weights zero (src/unet.c:606-610) */
+        block *b = &u->rb[i][k];
+        init_conv(h, &b->c1, &seed, 0); init_gn(h, &b->n1); init_conv(h, &b->c2, &seed, 0); init_gn(h, &b->n2);
+        const char *nz = getenv("UFSM_RB_NONZERO");
+        if (!(nz && atoi(nz))) memset(h + b->c2.w, 0, (size_t)b->c2.cout * b->c2.cin * 27 * 4);
+    }
     if (u->cfg.down_norm) for (int i = 0; i < L - 1; i++) init_gn(h, &u->dn[i]);
     if (u->tbn) {   /* LayerNorm and QK-norm gains 1, QKV and MLP-in N(0, 1 / C), out projections and biases 0 (identity blocks), registers N(0, 0.02^2) (src/unet.c:612-642) */
         const int C = u->tbd.C, F = u->tbd.F; const double sd = 1.0 / sqrt((double)C);
@@ -346,6 +379,8 @@ void unet_init(unet *u, uint64_t seed) {
 static void note(unet *u, const void *p, shape5 s, const char *name, const float *mean, const float *rstd, int G) {
     if (u->nouts < 64) { u->outs[u->nouts].p = p; u->outs[u->nouts].s = s; u->outs[u->nouts].name = name; u->outs[u->nouts].mean = mean; u->outs[u->nouts].rstd = rstd; u->outs[u->nouts].G = G; u->nouts++; }
 }
+/* the block whose output is level i's encoder output (skip, down-conv input, bottom): the last residual block, else enc[i] (src/unet.c:302-303) */
+static block *stage_out(unet *u, int i) { return u->cfg.enc_blocks[i] > 0 ? &u->rb[i][u->cfg.enc_blocks[i] - 1] : &u->enc[i]; }
 static nn_gn_t gn_out(const unet *u, const block *b) { return (nn_gn_t){P(u, b->n2.gamma), P(u, b->n2.beta), b->m2, b->r2, G_of(u, b->ys.c)}; }   /* silu(gn(a2)) for the block's readers */
 
 /* planes [s0, s0 + n) of the MX tensor src (depth Ds) -> planes [d0, d0 + n) of dst (depth Dd), every sample and channel block: a block's
@@ -423,7 +458,7 @@ static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t 
 /* the bottleneck's raw output -> fp32 planes -> token rows with the registers prepended -> blocks -> planes -> a new MX tensor with its
    GroupNorm statistics: the level's output for the decoder (src/unet.c:2795-2835; no PEG, memory, view or deformable paths) */
 static int tb_fwd(unet *u) {
-    const block *x = &u->enc[u->cfg.nlev - 1]; block *b = &u->tb;
+    const block *x = stage_out(u, u->cfg.nlev - 1); block *b = &u->tb;
     const shape5 ys = b->ys; const int C = u->tbd.C, nr = u->tbd.nreg; const size_t Sg = (size_t)ys.d * ys.h * ys.w, TC = (size_t)u->tbg.nseq * u->tbg.S * C;
     if (u->act_dt == 4) lp_mx4_to_f32(x->a2, ys.n, C, Sg, u->tb_cs); else lp_mx8_to_f32(x->a2, ys.n, C, Sg, u->tb_cs);
     at_cs_to_tok(u->tb_cs, u->tb_tok, P(u, u->reg_off), ys.n, C, (long)Sg, nr);
@@ -437,6 +472,19 @@ static int tb_fwd(unet *u) {
     const int G = G_of(u, C);
     if (!ge_const(u) && nn_gn_stats(b->a2, ys, G, 1e-5f, b->m2, b->r2)) { fprintf(stderr, "unet: attention stage GroupNorm statistics unsupported for this storage\n"); return -1; }
     note(u, b->a2, ys, "attn", b->m2, b->r2, G);
+    return 0;
+}
+/* a residual block (rblock_fwd, src/unet.c:2656-2671): conv1 of silu(gn(prev's output)) with statistics, conv2 of silu(gn(a1)) without, the
+   previous output added into it (MX: decode, add, re-quantise), then the statistics of the stored sum */
+static int rblock_fwd(unet *u, block *b, block *prev, const char (*nm)[16]) {
+    const int G = G_of(u, b->c1.cout), Gc = ge_const(u) ? 0 : G;
+    const nn_gn_t gi = gn_out(u, prev);
+    if (nn_conv3d_fwd_gn_stats(prev->a2, b->xs, gi.G, gi.gamma, gi.beta, gi.mean, gi.rstd, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, b->a1, Gc, 1e-5f, b->m1, b->r1)) return -1;
+    note(u, b->a1, b->ys, nm[0], b->m1, b->r1, G);
+    if (nn_conv3d_fwd_gn_stats(b->a1, b->ys, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, b->a2, 0, 1e-5f, nullptr, nullptr)) return -1;
+    lp_add_mx(b->a2, prev->a2, b->ys, u->act_dt, 0u);
+    if (!ge_const(u) && nn_gn_stats(b->a2, b->ys, G, 1e-5f, b->m2, b->r2)) { fprintf(stderr, "unet: residual block GroupNorm statistics unsupported for this storage\n"); return -1; }
+    note(u, b->a2, b->ys, nm[1], b->m2, b->r2, G);
     return 0;
 }
 /* the graph on the MX input tensor x (src/unet.c:2939-3105) */
@@ -453,11 +501,13 @@ static int graph_fwd(unet *u, const void *x) {
         nn_gn_t gd; const nn_gn_t *gin = nullptr;                  /* down_norm: conv1 reads silu(gn(down conv output)) (src/unet.c:2593) */
         if (i && u->cfg.down_norm) { gd = (nn_gn_t){P(u, u->dn[i - 1].gamma), P(u, u->dn[i - 1].beta), u->dm[i - 1], u->dr[i - 1], G_of(u, u->cfg.widths[i - 1])}; gin = &gd; }
         if (block_fwd(u, &u->enc[i], i, cur, gin, nullptr, nullptr, 0, en1[i], en2[i])) return -1;
+        for (int k = 0; k < u->cfg.enc_blocks[i]; k++) if (rblock_fwd(u, &u->rb[i][k], k ? &u->rb[i][k - 1] : &u->enc[i], u->rbn[i][k])) return -1;      /* (src/unet.c:2963) */
         if (i < L - 1) {                                           /* stride-2 down conv of silu(gn(a2)), width kept (src/unet.c:2970) */
-            const nn_gn_t g = gn_out(u, &u->enc[i]);
+            const block *so = stage_out(u, i);
+            const nn_gn_t g = gn_out(u, so);
             const int pre = u->skipst[i] != nullptr;
-            if (pre && mi_conv_prestage(u->enc[i].a2, 3, u->enc[i].ys, gnp_mk(g.gamma, g.beta, g.mean, g.rstd, g.G), u->skipst[i], 8)) return -1;
-            if (nn_conv3d_fwd_x(pre ? u->skipst[i] : u->enc[i].a2, pre ? nullptr : &g, nullptr, nullptr, 0, 0, u->enc[i].ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
+            if (pre && mi_conv_prestage(so->a2, 3, so->ys, gnp_mk(g.gamma, g.beta, g.mean, g.rstd, g.G), u->skipst[i], 8)) return -1;
+            if (nn_conv3d_fwd_x(pre ? u->skipst[i] : so->a2, pre ? nullptr : &g, nullptr, nullptr, 0, 0, so->ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
             shape5 ds = u->ls[i + 1]; ds.c = u->cfg.widths[i];
             if (u->cfg.down_norm) {                                /* statistics of the stored down-conv output now, the transform in the next conv1's staging (src/unet.c:2974-2979) */
                 if (!ge_const(u) && nn_gn_stats(u->downo[i], ds, G_of(u, ds.c), 1e-5f, u->dm[i], u->dr[i])) { fprintf(stderr, "unet: down_norm GroupNorm statistics unsupported for this storage\n"); return -1; }
@@ -468,11 +518,11 @@ static int graph_fwd(unet *u, const void *x) {
     }
     if (u->tbn && tb_fwd(u)) return -1;
     for (int i = L - 2; i >= 0; i--) {                             /* decoder: nothing materialised (src/unet.c:3010-3013) */
-        const block *coarse = i == L - 2 ? &u->enc[L - 1] : &u->dec[i + 1];
-        nn_gn_t gc = gn_out(u, coarse); const nn_gn_t gs = gn_out(u, &u->enc[i]);
+        const block *coarse = i == L - 2 ? stage_out(u, L - 1) : &u->dec[i + 1], *skip = stage_out(u, i);
+        nn_gn_t gc = gn_out(u, coarse); const nn_gn_t gs = gn_out(u, skip);
         if (i == L - 2 && u->tbn) { coarse = &u->tb; gc.mean = u->tb.m2; gc.rstd = u->tb.r2; }      /* the stage's output under the level's n2 affine (src/unet.c:508) */
         static const nn_gn_t none = {nullptr, nullptr, nullptr, nullptr, -1};          /* the pre-staged skip: no GroupNorm left to apply */
-        if (block_fwd(u, &u->dec[i], i, u->skipst[i] ? u->skipst[i] : u->enc[i].a2, u->skipst[i] ? &none : &gs, coarse->a2, &gc, coarse->ys.c, dn1[i], dn2[i])) return -1;
+        if (block_fwd(u, &u->dec[i], i, u->skipst[i] ? u->skipst[i] : skip->a2, u->skipst[i] ? &none : &gs, coarse->a2, &gc, coarse->ys.c, dn1[i], dn2[i])) return -1;
     }
     const block *last = L > 1 ? &u->dec[0] : &u->enc[0];
     const nn_gn_t g = gn_out(u, last);
@@ -554,6 +604,7 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     for (int i = 0; i < cfg->nlev; i++) { cfg->widths[i] = atoi(p); p = strchr(p, ','); if (!p) break; p++; }
     cfg->cin = key_int(line, "\"cin\":", 0); cfg->cout = key_int(line, "\"cout\":", 0); cfg->G = key_int(line, "\"G\":", 8);
     if ((p = strstr(line, "\"dec_widths\":["))) { p += 14; for (int i = 0; i < UNET_MAXLEV && *p && *p != ']'; i++) { char *e; cfg->dec_widths[i] = (int)strtol(p, &e, 10); p = e; if (*p == ',') p++; } }      /* (src/unet.c:5674) */
+    if ((p = strstr(line, "\"enc_blocks\":["))) { p += 14; for (int i = 0; i < UNET_MAXLEV && *p && *p != ']'; i++) { char *e; cfg->enc_blocks[i] = (int)strtol(p, &e, 10); p = e; if (*p == ',') p++; } }      /* (src/unet.c:5675) */
     if ((p = strstr(line, "\"dec_convs\":["))) { p += 13; for (int i = 0; i < UNET_MAXLEV && *p && *p != ']'; i++) { char *e; cfg->dec_convs[i] = (int)strtol(p, &e, 10); p = e; if (*p == ',') p++; } }        /* (src/unet.c:5700) */
     cfg->down_norm = key_int(line, "\"down_norm\":", 0); cfg->w4_2d = key_int(line, "\"w4_2d\":", 0);
     cfg->l0_norm = key_int(line, "\"l0_norm\":", 0); cfg->l0_slab = key_int(line, "\"l0_slab\":", 0);      /* (src/unet.c:5726) */
@@ -564,7 +615,7 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
-    static const char *const no[] = {"\"enc_blocks\":", "\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"ds_levels\":", "\"emb_lev\":",
+    static const char *const no[] = {"\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"ds_levels\":", "\"emb_lev\":",
                                      "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
                                      "\"skip_empty\":", "\"gfilm\":"};
     const char *bad = nullptr;
@@ -602,6 +653,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
     if (!bad && c.gn_ema != m->gn_ema) bad = "gn_ema";
+    for (int i = 0; !bad && i < m->nlev; i++) if (c.enc_blocks[i] != m->enc_blocks[i]) bad = "enc_blocks";
     for (int i = 0; !bad && i < m->nlev - 1; i++) { if (dw_of(&c, i) != dw_of(m, i)) bad = "dec_widths"; if ((c.dec_convs[i] == 1) != (m->dec_convs[i] == 1)) bad = "dec_convs"; }
     if (!bad && (c.l0_norm != m->l0_norm || (c.l0_norm == 4 && (c.l0_slab > 0 ? c.l0_slab : 64) != (m->l0_slab > 0 ? m->l0_slab : 64)))) bad = "l0_norm / l0_slab";
     if (!bad && np != u->np) bad = "nparams";
@@ -658,6 +710,8 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     fputc(']', f);
     { int any = 0; for (int i = 0; i < u->cfg.nlev; i++) any |= u->cfg.dec_widths[i] != 0;       /* (only when set, src/unet.c:5549-5550) */
       if (any) { fputs(",\"dec_widths\":[", f); for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.dec_widths[i]); fputc(']', f); } }
+    { int any = 0; for (int i = 0; i < u->cfg.nlev; i++) any |= u->cfg.enc_blocks[i] != 0;       /* (src/unet.c:5551-5552) */
+      if (any) { fputs(",\"enc_blocks\":[", f); for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.enc_blocks[i]); fputc(']', f); } }
     /* (the reference's key order, src/unet.c:5561-5578: w4_2d, the attention keys, l0_norm / l0_slab, then cin) */
     if (u->cfg.w4_2d) fprintf(f, ",\"w4_2d\":%d", u->cfg.w4_2d);
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);

@@ -81,7 +81,7 @@ def load_host():
     return L
 
 
-def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0, gn_ema=0, dec_widths=None, dec_convs=None):
+def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0, gn_ema=0, dec_widths=None, dec_convs=None, enc_blocks=None):
     """The reference's configuration record plus, as Python attributes, what the reference keeps in process-wide switches: the activation
     storage (unet_set_act_mx4) and the compute precision policy (nn_set_prec), which UNet applies around its calls."""
     c = unet_cfg()
@@ -94,6 +94,8 @@ def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn
         c.dec_widths[i] = d
     for i, d in enumerate(dec_convs or []):
         c.dec_convs[i] = d
+    for i, d in enumerate(enc_blocks or []):
+        c.enc_blocks[i] = d
     c.act_dt, c.prec = act_dt, prec
     return c
 
