@@ -925,3 +925,37 @@ def test_unet_decoder_variants(gpu, tmp_path, bits, widths, dec_widths, dec_conv
     plain = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits), N, D, H, W, seed=1)
     assert plain.load(path) == -1
     plain.close(); twin.close(); net.close()
+
+
+def test_training_only_heads_keep_their_place(gpu, tmp_path):
+    """cfg.ds_levels (deep-supervision heads of decoder levels 1 .. ds_levels) and cfg.emb_lev / emb_ch (the distillation head) are outputs of
+    training; their weights sit in the parameter vector (after the down norms / residual blocks and after the attention stage, src/unet.c:467,
+    :511), so a checkpoint of such a net loads and predicts what the same weights predict without them."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host, unet_cfg
+    H0 = load_host()
+    rng = np.random.default_rng(23)
+    N, (D, H, W), widths, cin, head_out = 1, (16, 16, 16), [32, 64, 128], 4, 3
+    S = D * H * W
+    plain = UNet(make_cfg(cin, widths, head_out=head_out, down_norm=1), N, D, H, W, seed=5)
+    aux = UNet(make_cfg(cin, widths, head_out=head_out, down_norm=1, ds_levels=1, emb_lev=1, emb_ch=8), N, D, H, W, seed=6)
+    pp = plain.params(); pa = aux.params()
+    nds, nemb = 64 * head_out + head_out, 64 * 8 + 8              # 1x1x1 heads on decoder level 1 (64 channels)
+    assert pa.size == pp.size + nds + nemb
+    assert (pa[pp.size + 64 * head_out:pp.size + nds] == -2).all()           # a deep-supervision head starts as the main head does (bias -2)
+    pa[:pp.size] = pp; aux.set_params(pa)
+    x = rng.standard_normal((N, cin, S)).astype(np.float32); dxq = to_mx(8, x)
+    la, lb = DevBuf(N * head_out * S * 4), DevBuf(N * head_out * S * 4)
+    assert plain.forward_x(dxq.ptr, la.ptr) == 0 and aux.forward_x(dxq.ptr, lb.ptr) == 0
+    LP.check()
+    assert np.array_equal(la.to_numpy(np.float32), lb.to_numpy(np.float32))
+    path = str(tmp_path / "aux.ckpt")
+    assert aux.save(path, step=8, extra="{}") == 0
+    head = open(path, "rb").readline().decode()
+    assert ',"ds_levels":1,"emb_lev":1,"emb_ch":8,' in head
+    c2 = unet_cfg()
+    assert H0.unet_peek(path.encode(), C.byref(c2), None) == 0 and (c2.ds_levels, c2.emb_lev, c2.emb_ch) == (1, 1, 8)
+    assert plain.load(path) == -1
+    c2.act_dt, c2.prec = 8, 0
+    twin = UNet(c2, N, D, H, W, seed=9)
+    assert twin.load(path) == 8 and np.array_equal(twin.params(), pa)
+    twin.close(); plain.close(); aux.close()

@@ -36,6 +36,7 @@ struct unet {
     block enc[UNET_MAXLEV], dec[UNET_MAXLEV];
     block *rb[UNET_MAXLEV]; char (*rbn[UNET_MAXLEV])[2][16];      /* cfg.enc_blocks: residual blocks after encoder level i (src/unet.c:96, :461-465), the names of their convs */
     convp down[UNET_MAXLEV], head;
+    convp ds[UNET_MAXLEV], eh;         /* cfg.ds_levels / cfg.emb_lev: the deep-supervision heads of decoder levels 1 .. ds_levels and the distillation head: training-time outputs, here only their place in the parameter vector (src/unet.c:467, :511) */
     void *downo[UNET_MAXLEV];
     void *skipst[UNET_MAXLEV];         /* silu(gn(enc[i].a2)) in the compute format, formed once for its two readers (down conv, decoder conv1); null: each reader transforms it */
     gnpar dn[UNET_MAXLEV]; float *dm[UNET_MAXLEV], *dr[UNET_MAXLEV];   /* down_norm: GroupNorm after down[i], its statistics */
@@ -76,7 +77,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
         if (c->enc_blocks[i] < 0 || c->enc_blocks[i] > 64 || (c->enc_blocks[i] && (i == 0 || i >= c->nlev))) return "enc_blocks (levels 1 and deeper)";      /* (src/unet.c:462) */
         if (c->dec_convs[i] && c->dec_convs[i] != 2 && c->dec_convs[i] != 1) return "dec_convs";
     }
-    if (c->ds_levels) return "ds_levels";
+    if (c->ds_levels < 0 || (c->ds_levels > 0 && c->ds_levels > c->nlev - 2)) return "ds_levels (decoder levels 1 .. nlev - 2)";      /* (src/unet.c:466) */
     if (c->lat_guide || c->lat_nsub) return "lat_guide";
     if (c->l0_norm < 0 || c->l0_norm > 4) return "l0_norm (0 GroupNorm, 1 none, 2 ema, 3 ws, 4 slab)";
     if (c->l0_norm == 2 && (c->G < c->widths[0] ? c->G : c->widths[0]) > 64) return "l0_norm 2 with more than 64 groups";
@@ -90,7 +91,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->attn_mem) return "attn_mem";
     if (c->view_P || c->view_patch) return "view_P";
     if (c->attn_deform || c->attn_dlev || c->attn_dco || c->attn_dinit) return "attn_deform";
-    if (c->emb_lev || c->emb_ch) return "emb_lev";
+    if (c->emb_lev < 0 || (c->emb_lev > 0 && (c->emb_lev > c->nlev - 2 || c->emb_ch <= 0)) || (!c->emb_lev && c->emb_ch)) return "emb_lev (decoder levels 1 .. nlev - 2, at least one channel)";      /* (src/unet.c:510) */
     if (c->film) return "film";
     if (c->skip_thr || c->skip_margin || c->skip_nl) return "skip_empty";
     if (c->fstem || c->fstem_out) return "fstem";
@@ -149,6 +150,7 @@ unet *unet_create(const unet_cfg *cfg) {
             snprintf(u->rbn[i][k][0], 16, "rb%d.%d.c1", i, k); snprintf(u->rbn[i][k][1], 16, "rb%d.%d.c2", i, k);
         }
     }
+    for (int j = 1; j <= cfg->ds_levels; j++) off = add_conv(&u->ds[j], dw_of(cfg, j), cfg->cout, 1, off);
     if (cfg->attn_blocks > 0) {                                   /* parameters last: registers, then the blocks (src/unet.c:490-499) */
         const int C = w[L - 1];
         if (C % AT_HD || cfg->attn_blocks > 16 || (cfg->attn_pe != 1 && cfg->attn_pe != 2) || cfg->attn_reg < 0) {
@@ -161,6 +163,7 @@ unet *unet_create(const unet_cfg *cfg) {
         for (int k = 0; k < cfg->attn_blocks; k++) off = at_block_layout(&u->tbd, &u->tbp[k], off);
         u->tbn = cfg->attn_blocks;
     }
+    if (cfg->emb_lev) off = add_conv(&u->eh, dw_of(cfg, cfg->emb_lev), cfg->emb_ch, 1, off);        /* (after the attention stage, src/unet.c:511) */
     u->np = off;
     u->p = f32_new(off); u->ema = f32_new(off); u->params = u->src = u->p;
     if (cfg->w4_2d || cfg->l0_norm == 3) { u->wm = f32_new(off); u->params = u->wm; }
@@ -360,6 +363,8 @@ void unet_init(unet *u, uint64_t seed) {
         const char *nz = getenv("UFSM_RB_NONZERO");
         if (!(nz && atoi(nz))) memset(h + b->c2.w, 0, (size_t)b->c2.cout * b->c2.cin * 27 * 4);
     }
+    for (int j = 1; j <= u->cfg.ds_levels; j++) init_conv(h, &u->ds[j], &seed, -2.0);                /* as the main head (src/unet.c:611-612) */
+    if (u->cfg.emb_lev) init_conv(h, &u->eh, &seed, 0.0);
     if (u->cfg.down_norm) for (int i = 0; i < L - 1; i++) init_gn(h, &u->dn[i]);
     if (u->tbn) {   /* LayerNorm and QK-norm gains 1, QKV and MLP-in N(0, 1 / C), out projections and biases 0 (identity blocks), registers N(0, 0.02^2) (src/unet.c:612-642) */
         const int C = u->tbd.C, F = u->tbd.F; const double sd = 1.0 / sqrt((double)C);
@@ -609,13 +614,14 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     cfg->down_norm = key_int(line, "\"down_norm\":", 0); cfg->w4_2d = key_int(line, "\"w4_2d\":", 0);
     cfg->l0_norm = key_int(line, "\"l0_norm\":", 0); cfg->l0_slab = key_int(line, "\"l0_slab\":", 0);      /* (src/unet.c:5726) */
     cfg->gn_ema = key_int(line, "\"gn_ema\":", 0);
+    cfg->ds_levels = key_int(line, "\"ds_levels\":", 0); cfg->emb_lev = key_int(line, "\"emb_lev\":", 0); cfg->emb_ch = key_int(line, "\"emb_ch\":", 0);      /* (src/unet.c:5562-5563) */
     cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
     cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
     cfg->half_res = key_int(line, "\"half_res\":", 0); cfg->scan_norm = key_int(line, "\"scan_norm\":", 0);      /* (the caller's business: the graph does not use them) */
     if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
-    static const char *const no[] = {"\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":", "\"ds_levels\":", "\"emb_lev\":",
+    static const char *const no[] = {"\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":",
                                      "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
                                      "\"skip_empty\":", "\"gfilm\":"};
     const char *bad = nullptr;
@@ -653,6 +659,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
     if (!bad && c.gn_ema != m->gn_ema) bad = "gn_ema";
+    if (!bad && (c.ds_levels != m->ds_levels || c.emb_lev != m->emb_lev || c.emb_ch != m->emb_ch)) bad = "ds_levels / emb_lev";
     for (int i = 0; !bad && i < m->nlev; i++) if (c.enc_blocks[i] != m->enc_blocks[i]) bad = "enc_blocks";
     for (int i = 0; !bad && i < m->nlev - 1; i++) { if (dw_of(&c, i) != dw_of(m, i)) bad = "dec_widths"; if ((c.dec_convs[i] == 1) != (m->dec_convs[i] == 1)) bad = "dec_convs"; }
     if (!bad && (c.l0_norm != m->l0_norm || (c.l0_norm == 4 && (c.l0_slab > 0 ? c.l0_slab : 64) != (m->l0_slab > 0 ? m->l0_slab : 64)))) bad = "l0_norm / l0_slab";
@@ -714,6 +721,8 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
       if (any) { fputs(",\"enc_blocks\":[", f); for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.enc_blocks[i]); fputc(']', f); } }
     /* (the reference's key order, src/unet.c:5561-5578: w4_2d, the attention keys, l0_norm / l0_slab, then cin) */
     if (u->cfg.w4_2d) fprintf(f, ",\"w4_2d\":%d", u->cfg.w4_2d);
+    if (u->cfg.ds_levels) fprintf(f, ",\"ds_levels\":%d", u->cfg.ds_levels);
+    if (u->cfg.emb_lev) fprintf(f, ",\"emb_lev\":%d,\"emb_ch\":%d", u->cfg.emb_lev, u->cfg.emb_ch);
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
     if (u->cfg.l0_norm) fprintf(f, ",\"l0_norm\":%d", u->cfg.l0_norm);
     if (u->cfg.l0_norm == 4) fprintf(f, ",\"l0_slab\":%d", u->cfg.l0_slab);
