@@ -153,10 +153,12 @@ def test_unet_is_deterministic_and_storage_registry(gpu):
     net.close()
 
 
-def test_unet_attention_stage(gpu):
+@pytest.mark.parametrize("rep", [1, 2])
+def test_unet_attention_stage(gpu, rep):
     """The transformer blocks on the bottleneck (src/unet.c:2795-2835): with the initial zero out-projections the stage is an identity on
     the tokens, so the net must agree with the plain one; with trained-like parameters the stage's output tensor must match the oracle's
-    composition (MX -> fp32 planes -> tokens with registers -> blocks -> planes -> MX) of the device's own bottleneck tensor."""
+    composition (MX -> fp32 planes -> tokens with registers -> blocks -> planes -> MX) of the device's own bottleneck tensor. rep 2:
+    cfg.attn_repeat, the block stack applied twice with the same weights (application k runs block k % attn_blocks, src/unet.c:2816)."""
     from ufsm_amd.unet import UNet, make_cfg
     rng = np.random.default_rng(12)
     N, D = 2, 16; widths = [32, 96]; cin, head_out, nreg, nblk = 4, 2, 3, 2
@@ -164,7 +166,7 @@ def test_unet_attention_stage(gpu):
     x = rng.standard_normal((N, cin, S)).astype(np.float32)
     dxq = to_mx(8, x)
     plain = UNet(make_cfg(cin, widths, head_out=head_out), N, D, D, D, seed=7)
-    att = UNet(make_cfg(cin, widths, head_out=head_out, attn_blocks=nblk, attn_pe=1, attn_reg=nreg), N, D, D, D, seed=7)
+    att = UNet(make_cfg(cin, widths, head_out=head_out, attn_blocks=nblk, attn_pe=1, attn_reg=nreg, attn_repeat=rep), N, D, D, D, seed=7)
     pp, pa = plain.params(), att.params()
     assert np.array_equal(pa[:pp.size], pp)                                  # the attention parameters come last (src/unet.c:490-499)
     Cb = widths[-1]; F = (8 * Cb // 3 + 31) // 32 * 32
@@ -200,13 +202,13 @@ def test_unet_attention_stage(gpu):
     reg = np.ascontiguousarray(pa[pp.size:pp.size + nreg * Cb].reshape(nreg, Cb))
     orc.lib().orc_cs_to_tok(orc.ptr(xb), orc.ptr(tok), orc.ptr(reg), N, Cb, Sg, nreg)
     t = tok.reshape(N * (Sg + nreg), Cb)
-    for lay in (lay0, lay1):
+    for lay in (lay0, lay1) * rep:
         t = orc.block_fwd(8, Cb, Cb // 48, F, 1, nreg, 100.0, pa[lay["ln1g"]:lay["b2"] + Cb], t, N, Sg + nreg, D // 2, D // 2)
     want = np.zeros_like(xb)
     orc.lib().orc_tok_to_cs(orc.ptr(t), orc.ptr(want), N, Cb, Sg, nreg)
     want = orc.mx_to_f32(8, orc.f32_to_mx(8, want, N, Cb, Sg), N, Cb, Sg)
     rel = np.linalg.norm(got - want) / np.linalg.norm(want - xb)
-    assert rel < 0.05, rel                                                   # two blocks of MX re-quantisations apart, then one e4m3 rounding
+    assert rel < 0.05 * rep, rel                                             # two (four) blocks of MX re-quantisations apart, then one e4m3 rounding
     assert np.linalg.norm(got - xb) / np.linalg.norm(xb) > 0.05              # and the stage did change the tensor
     plain.close(); att.close()
 

@@ -87,7 +87,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->gn_ema && c->l0_norm) return "gn_ema with l0_norm (src/unet.c:551)";
     if (c->attn_vres) return "attn_vres";
     if (c->attn_axis) return "attn_axis";
-    if (c->attn_repeat > 1) return "attn_repeat";
+    if (c->attn_repeat < 0 || (c->attn_repeat > 1 && (!c->attn_blocks || c->attn_blocks * c->attn_repeat > 64))) return "attn_repeat";
     if (c->attn_mem) return "attn_mem";
     if (c->view_P || c->view_patch) return "view_P";
     if (c->attn_deform || c->attn_dlev || c->attn_dco || c->attn_dinit) return "attn_deform";
@@ -279,7 +279,7 @@ static int build_acts(unet *u, shape5 in) {
         u->tb.ys = ys; u->tb.a2 = act_new(u, ys);
         const size_t ng = (size_t)in.n * G_of(u, C);
         u->tb.m2 = f32_new(ng); u->tb.r2 = f32_new(ng);
-        u->tb_cs = f32_new((size_t)ys.n * C * Sg); u->tb_tok = f32_new((size_t)(u->tbn + 1) * T * C);
+        u->tb_cs = f32_new((size_t)ys.n * C * Sg); u->tb_tok = f32_new((size_t)3 * T * C);     /* the stage's input rows and two buffers the applications alternate between */
         u->tb_ws = mi_malloc(at_ws_bytes(&u->tbd, T)); at_ws_carve(&u->tbw, &u->tbd, T, u->tb_ws);
     }
     u->built = 1;
@@ -469,10 +469,15 @@ static int tb_fwd(unet *u) {
     at_cs_to_tok(u->tb_cs, u->tb_tok, P(u, u->reg_off), ys.n, C, (long)Sg, nr);
     at_set_mx(8);
     lp_mx_gemm_bmemo(1);                                           /* inference: the linears' weights are packed once (dropped when the weights change) */
-    for (int k = 0; k < u->tbn; k++)
-        if (at_block_fwd(&u->tbd, u->params, &u->tbp[k], u->tb_tok + (size_t)k * TC, u->tb_tok + (size_t)(k + 1) * TC, &u->tbg, &u->tbw)) { lp_mx_gemm_bmemo(0); fprintf(stderr, "unet: attention block forward failed\n"); return -1; }
+    const int tba = u->tbn * (u->cfg.attn_repeat > 1 ? u->cfg.attn_repeat : 1);      /* application k runs block k % tbn (cfg.attn_repeat, src/unet.c:2816) */
+    float *tin = u->tb_tok;
+    for (int k = 0; k < tba; k++) {
+        float *tout = u->tb_tok + (size_t)(1 + (k & 1)) * TC;
+        if (at_block_fwd(&u->tbd, u->params, &u->tbp[k % u->tbn], tin, tout, &u->tbg, &u->tbw)) { lp_mx_gemm_bmemo(0); fprintf(stderr, "unet: attention block forward failed\n"); return -1; }
+        tin = tout;
+    }
     lp_mx_gemm_bmemo(0);
-    at_tok_to_cs(u->tb_tok + (size_t)u->tbn * TC, u->tb_cs, ys.n, C, (long)Sg, nr);
+    at_tok_to_cs(tin, u->tb_cs, ys.n, C, (long)Sg, nr);
     if (u->act_dt == 4) lp_f32_to_mx4(u->tb_cs, ys.n, C, Sg, b->a2); else lp_f32_to_mx8(u->tb_cs, ys.n, C, Sg, b->a2);
     const int G = G_of(u, C);
     if (!ge_const(u) && nn_gn_stats(b->a2, ys, G, 1e-5f, b->m2, b->r2)) { fprintf(stderr, "unet: attention stage GroupNorm statistics unsupported for this storage\n"); return -1; }
@@ -617,12 +622,13 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     cfg->ds_levels = key_int(line, "\"ds_levels\":", 0); cfg->emb_lev = key_int(line, "\"emb_lev\":", 0); cfg->emb_ch = key_int(line, "\"emb_ch\":", 0);      /* (src/unet.c:5562-5563) */
     cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
     cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
+    cfg->attn_repeat = key_int(line, "\"attn_repeat\":", 0);
     cfg->half_res = key_int(line, "\"half_res\":", 0); cfg->scan_norm = key_int(line, "\"scan_norm\":", 0);      /* (the caller's business: the graph does not use them) */
     if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
     static const char *const no[] = {"\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":",
-                                     "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_repeat\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
+                                     "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
                                      "\"skip_empty\":", "\"gfilm\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
@@ -656,6 +662,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.cin != m->cin) bad = "cin";
     if (!bad && c.cout != m->cout) bad = "cout";
     if (!bad && c.attn_blocks != m->attn_blocks) bad = "attn_blocks";
+    if (!bad && (c.attn_repeat > 1 ? c.attn_repeat : 1) != (m->attn_repeat > 1 ? m->attn_repeat : 1)) bad = "attn_repeat";
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
     if (!bad && c.gn_ema != m->gn_ema) bad = "gn_ema";
@@ -724,6 +731,7 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     if (u->cfg.ds_levels) fprintf(f, ",\"ds_levels\":%d", u->cfg.ds_levels);
     if (u->cfg.emb_lev) fprintf(f, ",\"emb_lev\":%d,\"emb_ch\":%d", u->cfg.emb_lev, u->cfg.emb_ch);
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
+    if (u->cfg.attn_blocks && u->cfg.attn_repeat > 1) fprintf(f, ",\"attn_repeat\":%d", u->cfg.attn_repeat);      /* (src/unet.c:5571) */
     if (u->cfg.l0_norm) fprintf(f, ",\"l0_norm\":%d", u->cfg.l0_norm);
     if (u->cfg.l0_norm == 4) fprintf(f, ",\"l0_slab\":%d", u->cfg.l0_slab);
     if (u->cfg.gn_ema) {                                           /* every site's running statistics and their state (src/unet.c:5587-5592; written after l0_norm's keys there too) */
