@@ -799,7 +799,9 @@ def test_unet_gn_ema(gpu, tmp_path, widths, dn, attn):
 
 @pytest.mark.parametrize("bits,widths,dec_widths,dec_convs,enc_blocks", [(8, [32, 64, 128], [0, 32], None, None), (8, [32, 64, 128], None, [2, 1], None),
                                                                           (8, [32, 64, 96, 128], [0, 32, 64], [1, 2, 1], None), (4, [32, 64, 128], [32, 32], [1, 1], None),
-                                                                          (8, [32, 64, 128], None, None, [0, 1, 2]), (4, [32, 64, 96], [0, 32], [2, 1], [0, 2, 1])])
+                                                                          (8, [32, 64, 128], None, None, [0, 1, 2]), (4, [32, 64, 96], [0, 32], [2, 1], [0, 2, 1]),
+                                                                          # the widths and decoder of the reference's production net (six levels 32 .. 192, level-1 decoder 32 wide)
+                                                                          (8, [32, 64, 96, 128, 160, 192], [0, 32], None, None)])
 def test_unet_decoder_variants(gpu, tmp_path, bits, widths, dec_widths, dec_convs, enc_blocks):
     """cfg.dec_widths (a decoder block narrower than its level's encoder, src/unet.c:298-300, :452-456) and cfg.dec_convs 1 (one-conv decoder
     blocks whose output goes by n1, src/unet.c:357-362, :2581-2582): layout size, every layer against the oracle conv on the device layer's
@@ -810,7 +812,7 @@ def test_unet_decoder_variants(gpu, tmp_path, bits, widths, dec_widths, dec_conv
     from ufsm_amd.unet import UNet, make_cfg, load_host, unet_cfg
     H0 = load_host()
     rng = np.random.default_rng(sum(widths) + bits)
-    N, (D, H, W) = 1, (16, 16, 16)
+    N, (D, H, W) = 1, ((16, 16, 16) if len(widths) < 6 else (32, 32, 64))
     S = D * H * W
     cin, head_out, G = 4, 3, 8
     net = UNet(make_cfg(cin, widths, G=G, head_out=head_out, act_dt=bits, dec_widths=dec_widths, dec_convs=dec_convs, enc_blocks=enc_blocks), N, D, H, W, seed=19)
