@@ -70,6 +70,7 @@ void nn_fakeq_w4_2d(float *w, int Co, int Ci, int T, int B);
    null: mean 0, rstd 1; else run = [mean G | var G] and rstd = 1 / sqrt(var + eps)); scaled weight standardisation per output channel over its
    fan-in of n contiguous weights, wh = gain (w - mean) / (std sqrt(n) + eps) (wh may be w) */
 void nn_gn_const_fill(float *mean, float *rstd, const float *run, int N, int G, float eps);
+void nn_axpy(float *y, float a, const float *x, size_t n);      /* y += a x (src/nn.h) */
 void nn_ws_fwd(float *wh, const float *w, int cout, int n, float gain, float eps);
 /* no counterpart in the reference (its stride-2 entry carries no split_t and prepares the weights per call): memo id of the calling thread's
    next lp_conv_fwd_s2_f8, as split_t.wkey for the stride-1 entries; consumed by that call. For inference loops with constant weights. */

@@ -127,6 +127,8 @@ void unet_set_slab_direct(int on);                            /* on (the default
    weights and EMA weights into a net of the same architecture (checked: nlev, widths, cin, cout, attention blocks, down_norm, nparams,
    payload size) and returns the saved step, or -1. unet_save writes weights and EMA. ---- */
 int unet_peek(const char *path, unet_cfg *cfg, int *step);
+void unet_set_scale(unet *u, double um);                       /* cfg.scale_cond nets: the input voxel size of the following forwards; the stem bias is b + c v with c = log2(um / 4.8) (src/unet.h:24, :141-144) */
+void unet_set_cond(unet *u, float c);                          /* ... or the code c itself (src/unet.h:146-147) */
 void unet_gn_ema_live(unet *u, int on);                        /* cfg.gn_ema: 1 = forwards normalise with the window's own statistics instead of the running ones (src/unet.h:172) */
 long unet_gn_ema_updates(const unet *u);                       /* cfg.gn_ema: updates the loaded running statistics have seen (src/unet.h:288); 0: live statistics */
 long unet_l0_updates(const unet *u);                           /* cfg.l0_norm 2: updates the loaded running statistics have seen (src/unet.h:275-299); the forward uses them

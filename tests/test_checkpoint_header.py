@@ -94,10 +94,12 @@ def test_reads_the_running_statistics_key(tmp_path):
     # cfg.gn_ema with its statistics (src/unet.c:5587-5592, read at :5744-5751)
     h = 'UFSM{"nlev":2,"widths":[32,64],"gn_ema":1,"ge_n":5,"ge_warm":500,"ge_mom":0.01,"ge_run":[0,1,0,1],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":3,"extra":{}}\n'
     rc, cfg, n, step = read(tmp_path, h)
-    assert rc == 0 and cfg.gn_ema == 1 and cfg.l0_norm == 0
+    assert rc == 0 and cfg.gn_ema == 1 and cfg.l0_norm == 0 and cfg.scale_cond == 0
+    rc, cfg, n, step = read(tmp_path, 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":1,"nparams":10,"step":3,"extra":{}}\n')
+    assert rc == 0 and cfg.scale_cond == 1                          # voxel-size conditioning (src/unet.c:5672)
 
 
 def test_rejects_foreign_files(tmp_path):
     assert read(tmp_path, "not a checkpoint\n")[0] == -1
-    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"scale_cond":1,"nparams":1}\n')[0] == -2      # voxel-size conditioning
+    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"film":1,"nparams":1}\n')[0] == -2            # conditioning by scalar codes
     assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":0,"attn_reg":0,"attn_mlp":256,"cin":4,"cout":1,"nparams":1}\n')[0] == -2   # PEG

@@ -713,6 +713,64 @@ def test_unet_l0_norm_constant_modes(gpu, tmp_path, mode, bits, widths):
     net.close()
 
 
+@pytest.mark.parametrize("widths,cin,eb", [([32, 64], 4, None), ([16, 32, 64], 1, [0, 1, 0])])
+def test_unet_scale_cond(gpu, tmp_path, widths, cin, eb):
+    """cfg.scale_cond (src/unet.h:24, :141-147): the stem conv's bias of a forward is b + c v, v a learned vector of widths[0] floats after the
+    down norms' parameters (src/unet.c:460) and c = log2(um / 4.8) for an input voxel size of um micrometres (src/unet.c:1943, :2880-2885).
+    The same net without the vector and with that bias written into its stem gives the same bytes; c and the vector's place survive a checkpoint."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    H0 = load_host()
+    rng = np.random.default_rng(cin)
+    N, (D, H, W), bits, head_out = 1, (16, 16, 16), 8, 2
+    S = D * H * W
+    kw = dict(G=8, head_out=head_out, act_dt=bits, down_norm=1, enc_blocks=eb)
+    net = UNet(make_cfg(cin, widths, scale_cond=1, **kw), N, D, H, W, seed=3)
+    plain = UNet(make_cfg(cin, widths, **kw), N, D, H, W, seed=4)
+    lay_c, n_c = unet_ref.param_layout(cin, widths, head_out, 1, enc_blocks=eb, scale_cond=1)
+    lay_p, n_p = unet_ref.param_layout(cin, widths, head_out, 1, enc_blocks=eb)
+    p = net.params()
+    assert p.size == n_c == n_p + widths[0]
+    o, shp = lay_c["scale_cond"]
+    assert shp == (widths[0],) and o == lay_c["dn%d.beta" % (len(widths) - 2)][0] + widths[-2]
+    v = rng.uniform(-0.5, 0.5, widths[0]).astype(np.float32); p[o:o + widths[0]] = v; net.set_params(p)
+    x = rng.standard_normal((N, cin, S)).astype(np.float32); dxq = to_mx(bits, x)
+
+    def run(n):
+        d = DevBuf(N * head_out * S * 4)
+        assert n.forward_x(dxq.ptr, d.ptr) == 0
+        LP.check()
+        return d.to_numpy(np.float32, (N, head_out, S))
+
+    def with_bias(c):                                               # the plain net: every tensor by name, the stem bias b + c v in fp32 fused multiply-add
+        q = np.zeros(n_p, np.float32)
+        for k, (po, ps) in lay_p.items():
+            m = int(np.prod(ps)); q[po:po + m] = p[lay_c[k][0]:lay_c[k][0] + m]
+        bo = lay_p["enc0.c1.b"][0]
+        q[bo:bo + widths[0]] = (np.float64(np.float32(c)) * v.astype(np.float64) + q[bo:bo + widths[0]].astype(np.float64)).astype(np.float32)
+        plain.set_params(q)
+        return run(plain)
+
+    base = with_bias(0.0)
+    assert np.array_equal(run(net), base)                           # no scale set: c = 0
+    outs = []
+    for um in (2.4, 7.91, 4.8):
+        H0.unet_set_scale(net.h, um)
+        got = run(net); outs.append(got)
+        assert np.array_equal(got, with_bias(np.log2(um / 4.8)))
+    assert not np.array_equal(outs[0], base) and not np.array_equal(outs[0], outs[1]) and np.array_equal(outs[2], base)
+    H0.unet_set_cond(net.h, -0.75)
+    assert np.array_equal(run(net), with_bias(-0.75))
+    assert np.array_equal(net.params(), p)                          # the stored bias is untouched: the sum lives in a buffer of the forward
+    path = str(tmp_path / "sc.ckpt")
+    assert net.save(path, step=9, extra="{}") == 0
+    assert b',"down_norm":1,"scale_cond":1,"nparams":%d,' % n_c in open(path, "rb").readline()
+    assert plain.load(path) == -1                                   # another architecture
+    other = UNet(make_cfg(cin, widths, scale_cond=1, **kw), N, D, H, W, seed=5)
+    assert other.load(path) == 9 and np.array_equal(other.params(), p)
+    H0.unet_set_cond(other.h, -0.75)
+    assert np.array_equal(run(other), with_bias(-0.75))
+
+
 @pytest.mark.parametrize("widths,dn,attn", [([32, 64, 128], 1, 0), ([32, 96], 0, 1)])
 def test_unet_gn_ema(gpu, tmp_path, widths, dn, attn):
     """cfg.gn_ema (src/unet.h:67-71): every GroupNorm site (block norms of all levels, down norms, the attention stage's output) reads the

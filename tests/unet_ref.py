@@ -14,7 +14,7 @@ def is_single(dec_convs, i):
     return bool(dec_convs) and i < len(dec_convs) and dec_convs[i] == 1
 
 
-def param_layout(cin, widths, head_out, down_norm=0, dec_widths=None, dec_convs=None, enc_blocks=None):
+def param_layout(cin, widths, head_out, down_norm=0, dec_widths=None, dec_convs=None, enc_blocks=None, scale_cond=0):
     """dec_widths / dec_convs: cfg.dec_widths (a decoder block's width, 0 = the encoder's) and cfg.dec_convs (1: one conv, src/unet.c:357-362);
     enc_blocks: cfg.enc_blocks, residual blocks after encoder level i, their parameters after everything older (src/unet.c:461-465)"""
     L = len(widths); off = 0; lay = {}
@@ -43,6 +43,8 @@ def param_layout(cin, widths, head_out, down_norm=0, dec_widths=None, dec_convs=
     if down_norm:                                    # GroupNorm after each down conv, appended after the head (src/unet.c:459)
         for i in range(L - 1):
             gn("dn%d" % i, widths[i])
+    if scale_cond:                                   # the voxel-size conditioning vector: widths[0] floats, before the residual blocks (src/unet.c:460)
+        lay["scale_cond"] = (off, (widths[0],)); off += widths[0]
     for i, nb in enumerate(enc_blocks or []):
         for k in range(nb):
             conv("rb%d.%d.c1" % (i, k), widths[i], widths[i], 3); gn("rb%d.%d.n1" % (i, k), widths[i])

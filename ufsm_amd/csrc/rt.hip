@@ -115,6 +115,14 @@ extern "C" void mi_gn_sums_zero(double *sums, int nslots) {
     const size_t n = (size_t)nslots * 6;   // 24 bytes = 6 words
     fill_u32_k<<<nblk_(n, 256), 256>>>((unsigned *)sums, n, 0u); MICK();
 }
+// ---- y += a x over n floats (nn_axpy, src/nn.h): the stem bias of a scale-conditioned net ----
+// (a few dozen values in practice: one wavefront strides over them, one fused multiply-add each, as the reference's contracted a * x + y)
+__global__ void __launch_bounds__(64) scaled_add_k(float *__restrict__ y, float a, const float *__restrict__ x, size_t n) {
+    for (size_t i = blockIdx.x * 64 + threadIdx.x; i < n; i += (size_t)gridDim.x * 64) y[i] = fmaf(a, x[i], y[i]);
+}
+extern "C" void nn_axpy(float *y, float a, const float *x, size_t n) {
+    if (n) { scaled_add_k<<<(unsigned)(n < 65536 ? (n + 63) / 64 : 1024), 64>>>(y, a, x, n); MICK(); }
+}
 // ---- constant GroupNorm statistics for N samples (src/nn.h:465-473, src/nn_l0norm.cu:10-20): run null: mean 0, rstd 1; else run = [mean G | var G] ----
 __global__ void gn_const_k(float *mean, float *rstd, const float *run, int NG, int G, float eps) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;

@@ -27,6 +27,7 @@ struct unet {
     /* cfg.l0_norm 1 .. 3 (src/unet.h:52-58): the level-0 GroupNorms on constant statistics: mean 0 / rstd 1 (none, ws) or the checkpoint's running
        statistics once its warm-up is over (ema: l0run = [live weights: 4 sites x (mean G | var G)][EMA weights: the same], device; l0_n updates so far) */
     float *l0run; long l0_n; int l0_warm; float l0_mom; float ws_gain;
+    size_t sc_w; float sc_c; float *stem_b;                        /* cfg.scale_cond (src/unet.h:24, src/unet.c:129): the conditioning vector's offset, the current code, the stem bias b + c v of a forward */
     /* cfg.gn_ema (src/unet.h:67-71): every GroupNorm (all levels, down norms, the attention stage's) on the checkpoint's running statistics:
        ge_run = [live weights: ge_ns values][EMA weights: the same], per site pair [mean G | var G] in the order of gn_sites (src/unet.c:5125-5135) */
     float *ge_run; size_t ge_ns; long ge_n; int ge_warm, ge_live; float ge_mom;
@@ -70,7 +71,6 @@ static float *f32_new(size_t n) { float *p = mi_malloc(n * 4); mi_zero(p, n * 4)
 
 /* a field of the reference's configuration this build's graph does not run: named, so the caller knows which */
 static const char *cfg_unsupported(const unet_cfg *c) {
-    if (c->scale_cond) return "scale_cond";
     for (int i = 0; i < UNET_MAXLEV; i++) {
         /* decoder widths: at most the level's encoder width, and that width at level 0 (the head's input); the bottom level has no decoder (src/unet.c:452-455) */
         if (c->dec_widths[i] && (i >= c->nlev - 1 || c->dec_widths[i] > c->widths[i] || c->dec_widths[i] < 0 || (i == 0 && c->dec_widths[0] != c->widths[0]))) return "dec_widths";
@@ -141,6 +141,7 @@ unet *unet_create(const unet_cfg *cfg) {
     }
     off = add_conv(&u->head, w[0], cfg->cout, 1, off);
     if (cfg->down_norm) for (int i = 0; i < L - 1; i++) off = add_gn(&u->dn[i], w[i], off);       /* (appended after the head, src/unet.c:459) */
+    if (cfg->scale_cond) { u->sc_w = off; off += (size_t)w[0]; }  /* (src/unet.c:460) */
     for (int i = 0; i < L; i++) if (cfg->enc_blocks[i] > 0) {      /* residual blocks after encoder level i: parameters after everything older (src/unet.c:461-465) */
         u->rb[i] = calloc((size_t)cfg->enc_blocks[i], sizeof(block)); u->rbn[i] = calloc((size_t)cfg->enc_blocks[i], sizeof *u->rbn[i]);
         for (int k = 0; k < cfg->enc_blocks[i]; k++) {
@@ -296,6 +297,7 @@ void unet_free(unet *u) {
     free_acts(u);
     mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm); if (u->l0run) mi_free(u->l0run); if (u->ge_run) mi_free(u->ge_run);
     for (int i = 0; i < UNET_MAXLEV; i++) { free(u->rb[i]); free(u->rbn[i]); }
+    if (u->stem_b) mi_free(u->stem_b);
     lp_wmemo_clear();
     free(u);
 }
@@ -444,7 +446,7 @@ static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t 
             void *o = over ? tmp : y;
             if (!first) r = nn_conv3d_fwd_gn_stats(b->a1, xs, G, P(u, b->n1.gamma), P(u, b->n1.beta), b->m1, b->r1, P(u, b->c2.w), P(u, b->c2.b), b->c2.cout, o, Gc, 1e-5f, om, orr);
             else if (xup) r = nn_conv3d_fwd_x(xup, gup, x, gin, c_split, 1, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, om, orr);   /* [up2(coarse) | skip] */
-            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, om, orr);
+            else r = nn_conv3d_fwd_x(x, gin, nullptr, nullptr, 0, 0, xs, P(u, b->c1.w), b == &u->enc[0] && u->cfg.scale_cond ? u->stem_b : P(u, b->c1.b), b->c1.cout, 3, 1, o, Gc, 1e-5f, om, orr);
             if (s) { nn_set_zrange(0, 0, 0, 0, 0, 0); nn_set_zrange_out(0); }
             if (over && !r) {                                      /* planes below the next slab's first input plane are dead: the last one waits */
                 if (k) copy_planes(u, y, D, z0 - 1, carry, 1, 0, 1, b->ys);
@@ -506,6 +508,12 @@ static int graph_fwd(unet *u, const void *x) {
     u->nouts = 0;
     if (l0_const(u)) l0_const_fill(u);
     if (ge_const(u)) ge_const_fill(u);
+    if (u->cfg.scale_cond) {                                       /* the stem bias of this forward: b + c v (src/unet.c:2880-2885) */
+        const int c0 = u->enc[0].c1.cout;
+        if (!u->stem_b) u->stem_b = f32_new((size_t)c0);
+        mi_d2d(u->stem_b, P(u, u->enc[0].c1.b), (size_t)c0 * 4);
+        nn_axpy(u->stem_b, u->sc_c, P(u, u->sc_w), (size_t)c0);
+    }
     const void *cur = x;
     for (int i = 0; i < L; i++) {
         nn_gn_t gd; const nn_gn_t *gin = nullptr;                  /* down_norm: conv1 reads silu(gn(down conv output)) (src/unet.c:2593) */
@@ -632,7 +640,7 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
                                      "\"skip_empty\":", "\"gfilm\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
-    if (!bad && key_int(line, "\"scale_cond\":", 0)) bad = "\"scale_cond\":";
+    cfg->scale_cond = key_int(line, "\"scale_cond\":", 0);
     if (!bad && (cfg->l0_norm < 0 || cfg->l0_norm > 4)) bad = "\"l0_norm\":";
     if (l0) {
         memset(l0, 0, sizeof *l0);
@@ -666,6 +674,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
     if (!bad && c.gn_ema != m->gn_ema) bad = "gn_ema";
+    if (!bad && (c.scale_cond != 0) != (m->scale_cond != 0)) bad = "scale_cond";
     if (!bad && (c.ds_levels != m->ds_levels || c.emb_lev != m->emb_lev || c.emb_ch != m->emb_ch)) bad = "ds_levels / emb_lev";
     for (int i = 0; !bad && i < m->nlev; i++) if (c.enc_blocks[i] != m->enc_blocks[i]) bad = "enc_blocks";
     for (int i = 0; !bad && i < m->nlev - 1; i++) { if (dw_of(&c, i) != dw_of(m, i)) bad = "dec_widths"; if ((c.dec_convs[i] == 1) != (m->dec_convs[i] == 1)) bad = "dec_convs"; }
@@ -708,6 +717,8 @@ int unet_load(unet *u, const char *path) {
     }
     return rc;
 }
+void unet_set_scale(unet *u, double um) { u->sc_c = um > 0 ? (float)log2(um / 4.8) : 0.f; }      /* the code of an input voxel size: log2(um / 4.8) (src/unet.h:141-144, src/unet.c:1943) */
+void unet_set_cond(unet *u, float c) { u->sc_c = c; }             /* the code itself (src/unet.h:146-147) */
 long unet_gn_ema_updates(const unet *u) { return u->ge_n; }       /* src/unet.h:280 */
 long unet_l0_updates(const unet *u) { return u->l0_n; }           /* src/unet.h:314 */
 int unet_save(const unet *u, const char *path, int step, const char *extra) {
@@ -752,8 +763,8 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     }
     { int any = 0; for (int i = 0; i < u->cfg.nlev; i++) any |= u->cfg.dec_convs[i] == 1;        /* (src/unet.c:5595-5596) */
       if (any) { fputs(",\"dec_convs\":[", f); for (int i = 0; i < u->cfg.nlev; i++) fprintf(f, "%s%d", i ? "," : "", u->cfg.dec_convs[i]); fputc(']', f); } }
-    fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":0,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.cout, u->cfg.G,
-            u->cfg.down_norm, u->np, step);
+    fprintf(f, ",\"cin\":%d,\"cout\":%d,\"G\":%d,\"down_norm\":%d,\"scale_cond\":%d,\"nparams\":%zu,\"step\":%d,\"sparse24\":0,\"wq\":0,\"muon_mom\":0", u->cfg.cin, u->cfg.cout, u->cfg.G,
+            u->cfg.down_norm, u->cfg.scale_cond, u->np, step);
     fprintf(f, ",\"extra\":%s}\n", extra ? extra : "{}");
     int ok = fwrite(h, 4, u->np, f) == u->np && fwrite(he, 4, u->np, f) == u->np;      /* weights, EMA weights */
     ok = !fclose(f) && ok;
