@@ -71,6 +71,12 @@ void nn_fakeq_w4_2d(float *w, int Co, int Ci, int T, int B);
    fan-in of n contiguous weights, wh = gain (w - mean) / (std sqrt(n) + eps) (wh may be w) */
 void nn_gn_const_fill(float *mean, float *rstd, const float *run, int N, int G, float eps);
 void nn_axpy(float *y, float a, const float *x, size_t n);      /* y += a x (src/nn.h) */
+/* FiLM on a GroupNorm's affine (src/nn.h:494-504): the norm's C channels at offsets gam / bet of the parameter vector p, its K x C pairs at fo
+   (scales first); the effective pair goes into the forward weights fw. nn_film_fwd: K <= 4 host codes, from p's affine. nn_gfilm_fwd: K device
+   codes gv, from the affine fw holds (kept in g1). nn_gfilm_pool: g[c] = mean over S of x[c S + s] */
+void nn_film_fwd(const float *p, float *fw, size_t gam, size_t bet, size_t fo, int C, int K, const float *codes);
+void nn_gfilm_pool(const float *x, int C, long S, float *g);
+void nn_gfilm_fwd(const float *p, float *fw, size_t gam, size_t bet, size_t fo, int C, int K, const float *gv, float *g1);
 void nn_ws_fwd(float *wh, const float *w, int cout, int n, float gain, float eps);
 /* no counterpart in the reference (its stride-2 entry carries no split_t and prepares the weights per call): memo id of the calling thread's
    next lp_conv_fwd_s2_f8, as split_t.wkey for the stride-1 entries; consumed by that call. For inference loops with constant weights. */

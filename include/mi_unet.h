@@ -128,6 +128,10 @@ void unet_set_slab_direct(int on);                            /* on (the default
    payload size) and returns the saved step, or -1. unet_save writes weights and EMA. ---- */
 int unet_peek(const char *path, unet_cfg *cfg, int *step);
 void unet_set_scale(unet *u, double um);                       /* cfg.scale_cond nets: the input voxel size of the following forwards; the stem bias is b + c v with c = log2(um / 4.8) (src/unet.h:24, :141-144) */
+void unet_set_film(unet *u, const float *codes, int k);        /* cfg.film nets: the k <= 4 codes of the following forwards (src/unet.h:148-149); the block norms' effective affines are remade when they change */
+size_t unet_gfilm_off(const unet *u);                          /* cfg.gfilm: the offset of its first scale / shift pair in the parameter vector (src/unet.h:160) */
+const float *mi_unet_gfilm_codes(const unet *u);               /* cfg.gfilm: the pooled codes of the last forward, widths[nlev-1] device floats (no counterpart in the reference's interface: its tests freeze them through the environment) */
+size_t mi_unet_film_off(const unet *u);                        /* cfg.film: the same for its pairs (no counterpart in the reference's interface: its tests print the offset) */
 void unet_set_cond(unet *u, float c);                          /* ... or the code c itself (src/unet.h:146-147) */
 void unet_gn_ema_live(unet *u, int on);                        /* cfg.gn_ema: 1 = forwards normalise with the window's own statistics instead of the running ones (src/unet.h:172) */
 long unet_gn_ema_updates(const unet *u);                       /* cfg.gn_ema: updates the loaded running statistics have seen (src/unet.h:288); 0: live statistics */

@@ -78,7 +78,7 @@ def test_unet_header_matches_the_cited_reference_signatures():
                  "const float *unet_forward_x(unet *u, const void *x, shape5 xs, int train, int x_h16);", "shape5 unet_out_shape(const unet *u, shape5 xs);",
                  "const float *unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, shape5 xs, int h16);",
                  "void unet_use_ema(unet *u, int on);", "int unet_save(const unet *u, const char *path, int step, const char *extra_json);", "int unet_load(unet *u, const char *path);",
-                 "int unet_peek(const char *path, unet_cfg *cfg, int *step);", "void unet_set_act_mx8(int on);", "void unet_set_act_mx4(int on);", "void unet_set_infer_slab(int planes);", "void unet_set_slab_direct(int on);", "void unet_set_scale(unet *u, double um);", "void unet_set_cond(unet *u, float c);",
+                 "int unet_peek(const char *path, unet_cfg *cfg, int *step);", "void unet_set_act_mx8(int on);", "void unet_set_act_mx4(int on);", "void unet_set_infer_slab(int planes);", "void unet_set_slab_direct(int on);", "void unet_set_scale(unet *u, double um);", "void unet_set_cond(unet *u, float c);", "void unet_set_film(unet *u, const float *codes, int k);", "size_t unet_gfilm_off(const unet *u);",
                  "const unet_cfg *unet_cfg_of(const unet *u);", "float *unet_param_ptr(unet *u);", "void unet_init(unet *u, uint64_t seed);"]:
         assert decl in flat, decl
 

@@ -771,6 +771,164 @@ def test_unet_scale_cond(gpu, tmp_path, widths, cin, eb):
     assert np.array_equal(run(other), with_bias(-0.75))
 
 
+def fma32(a, b, c):
+    """fp32 fused multiply-add of arrays through float64: the product is exact there, the sum rounds to 53 bits before the 24."""
+    return (np.asarray(a, np.float32).astype(np.float64) * np.asarray(b, np.float32).astype(np.float64) + np.asarray(c, np.float32).astype(np.float64)).astype(np.float32)
+
+
+def film_affine(gamma, beta, A, Dm, codes):
+    """The effective affine of a FiLM'd norm (src/nn.h:494-504): gamma (1 + sum_k c_k A_k), beta + sum_k c_k D_k, the sums as chains of
+    fused multiply-adds from k = 0; A, Dm [K][C]."""
+    s, t = np.zeros_like(gamma), np.zeros_like(beta)
+    for k, ck in enumerate(codes):
+        s, t = fma32(np.float32(ck), A[k], s), fma32(np.float32(ck), Dm[k], t)
+    return gamma * (np.float32(1) + s), beta + t
+
+
+def test_film_device_helpers(gpu):
+    """nn_film_fwd, nn_gfilm_pool, nn_gfilm_fwd (src/nn.h:494-504) against their definitions on random vectors; everything else of the forward
+    weights stays as it was."""
+    rng = np.random.default_rng(8)
+    for C_, K in ((96, 3), (32, 1), (200, 4), (64, 0)):
+        gam, bet = 7, 7 + C_ + 3
+        fo = bet + C_ + 5; n = fo + 2 * K * C_ + 9
+        p = rng.standard_normal(n).astype(np.float32); fw0 = rng.standard_normal(n).astype(np.float32)
+        codes = rng.uniform(-2, 2, 4).astype(np.float32)
+        dp, dfw = DevBuf.from_numpy(p), DevBuf.from_numpy(fw0)
+        lib.nn_film_fwd(dp.ptr, dfw.ptr, gam, bet, fo, C_, K, codes.ctypes.data); LP.check()
+        fw = dfw.to_numpy(np.float32)
+        A, Dm = p[fo:fo + K * C_].reshape(K, C_), p[fo + K * C_:fo + 2 * K * C_].reshape(K, C_)
+        wg, wb = film_affine(p[gam:gam + C_], p[bet:bet + C_], A, Dm, codes[:K])
+        assert np.array_equal(fw[gam:gam + C_], wg) and np.array_equal(fw[bet:bet + C_], wb)
+        keep = np.ones(n, bool); keep[gam:gam + C_] = keep[bet:bet + C_] = False
+        assert np.array_equal(fw[keep], fw0[keep]) and np.array_equal(dp.to_numpy(np.float32), p)
+        if K == 0:
+            assert np.array_equal(wg, p[gam:gam + C_]) and np.array_equal(wb, p[bet:bet + C_])
+    for C_, S_ in ((40, 1000), (96, 512), (3, 7), (192, 64)):
+        x = (rng.standard_normal((C_, S_)) * rng.uniform(0.1, 5, (C_, 1)) + rng.uniform(-2, 2, (C_, 1))).astype(np.float32)
+        dx, dg = DevBuf.from_numpy(x), DevBuf(C_ * 4)
+        lib.nn_gfilm_pool(dx.ptr, C_, S_, dg.ptr); LP.check()
+        assert np.array_equal(dg.to_numpy(np.float32), x.astype(np.float64).mean(1).astype(np.float32))
+    for C_, K in ((96, 64), (32, 192), (70, 5)):
+        gam, bet = 3, 3 + C_
+        fo = bet + C_ + 1; n = fo + 2 * K * C_
+        p = (0.2 * rng.standard_normal(n)).astype(np.float32); fw0 = rng.standard_normal(n).astype(np.float32)
+        gv = rng.standard_normal(K).astype(np.float32)
+        dp, dfw, dgv, dg1 = DevBuf.from_numpy(p), DevBuf.from_numpy(fw0), DevBuf.from_numpy(gv), DevBuf(C_ * 4)
+        lib.nn_gfilm_fwd(dp.ptr, dfw.ptr, gam, bet, fo, C_, K, dgv.ptr, dg1.ptr); LP.check()
+        fw = dfw.to_numpy(np.float32)
+        A, B = p[fo:fo + K * C_].reshape(K, C_), p[fo + K * C_:].reshape(K, C_)
+        wg, wb = film_affine(fw0[gam:gam + C_], fw0[bet:bet + C_], A, B, gv)      # from the affine the forward weights held
+        assert np.array_equal(fw[gam:gam + C_], wg) and np.array_equal(fw[bet:bet + C_], wb) and np.array_equal(dg1.to_numpy(np.float32), fw0[gam:gam + C_])
+        keep = np.ones(n, bool); keep[gam:gam + 2 * C_] = False
+        assert np.array_equal(fw[keep], fw0[keep])
+
+
+@pytest.mark.parametrize("widths,film,gfilm,attn,dc", [([32, 64, 128], 2, 0, 0, None), ([32, 96], 1, 1, 1, None), ([32, 64, 96], 0, 1, 2, [1, 2, 0]), ([32], 4, 0, 0, None)])
+def test_unet_film(gpu, tmp_path, widths, film, gfilm, attn, dc):
+    """cfg.film (src/unet.h:108-111): K codes per forward scale and shift the output norms of the encoder blocks, then of the decoder blocks from
+    the coarsest, through K x C pairs appended to the parameter vector (src/unet.c:372-380, :513). cfg.gfilm (src/unet.h:60-64): the decoder
+    blocks' output norms once more, the codes being the attention stage's output averaged over the window's tokens (src/unet.c:386-398, :516-520).
+    The same net without the pairs and with the effective affines written into its norms gives the same bytes; zero pairs are the donor's
+    function; the keys and the pairs survive a checkpoint."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    H0 = load_host()
+    rng = np.random.default_rng(film * 8 + gfilm)
+    L = len(widths)
+    N, (D, H, W), bits, head_out, cin = 1, (16, 16, 16), 8, 2, 4
+    S = D * H * W
+    kw = dict(G=8, head_out=head_out, act_dt=bits, down_norm=1, attn_blocks=attn, attn_pe=1, attn_reg=2, dec_convs=dc)
+    net = UNet(make_cfg(cin, widths, film=film, gfilm=gfilm, **kw), N, D, H, W, seed=3)
+    plain = UNet(make_cfg(cin, widths, **kw), N, D, H, W, seed=3)
+    p, q0 = net.params(), plain.params()
+    lay, _ = unet_ref.param_layout(cin, widths, head_out, 1, dec_convs=dc)
+    norms = ["enc%d.n2" % j for j in range(L)] + ["dec%d.%s" % (i, "n1" if unet_ref.is_single(dc, i) else "n2") for i in range(L - 2, -1, -1)]
+    nf = sum(2 * film * widths[int(k[3])] for k in norms)
+    ng = sum(2 * widths[-1] * widths[int(k[3])] for k in norms[L:]) if gfilm else 0
+    assert p.size == q0.size + nf + ng and np.array_equal(p[:q0.size], q0) and not p[q0.size:].any()      # appended last, zero: the donor's function
+    if film: assert H0.mi_unet_film_off(net.h) == q0.size
+    if gfilm: assert H0.unet_gfilm_off(net.h) == q0.size + nf
+    x = rng.standard_normal((N, cin, S)).astype(np.float32); dxq = to_mx(bits, x)
+
+    def run(n):
+        d = DevBuf(N * head_out * S * 4)
+        assert n.forward_x(dxq.ptr, d.ptr) == 0
+        LP.check()
+        return d.to_numpy(np.float32, (N, head_out, S))
+
+    def codes(c):
+        a = np.asarray(c, np.float32)
+        H0.unet_set_film(net.h, a.ctypes.data_as(C.POINTER(C.c_float)), a.size)
+
+    base = run(plain)
+    codes([1.5, -0.5, 0.25, 2.0][:film])
+    assert np.array_equal(run(net), base)
+    if attn:                                                        # trained-like attention blocks: the pooled codes are not the stage's input
+        Cb = widths[-1]; F = (8 * Cb // 3 + 31) // 32 * 32
+        o = q0.size - sum(orc.block_layout(Cb, F, 0)[1] for _ in range(attn))
+        for _ in range(attn):
+            bl, o = orc.block_layout(Cb, F, o)
+            for k, n in (("wo", Cb * Cb), ("w2", Cb * F), ("bo", Cb)):
+                p[bl[k]:bl[k] + n] = 0.05 * rng.standard_normal(n)
+        assert o == q0.size
+    p[q0.size:] = rng.uniform(-0.3, 0.3, nf + ng)
+    net.set_params(p)
+
+    def want(cs, gv):                                               # the plain net under the effective affines
+        q = p[:q0.size].copy()
+        fo, go = q0.size, q0.size + nf
+        for j, k in enumerate(norms):
+            c = widths[int(k[3])]; og, ob = lay[k + ".gamma"][0], lay[k + ".beta"][0]
+            g, b = q[og:og + c], q[ob:ob + c]
+            if film:
+                g, b = film_affine(g, b, p[fo:fo + film * c].reshape(film, c), p[fo + film * c:fo + 2 * film * c].reshape(film, c), cs)
+                fo += 2 * film * c
+            if gfilm and j >= L:
+                K = widths[-1]
+                g, b = film_affine(g, b, p[go:go + K * c].reshape(K, c), p[go + K * c:go + 2 * K * c].reshape(K, c), gv)
+                go += 2 * K * c
+            q[og:og + c], q[ob:ob + c] = g, b
+        plain.set_params(q)
+        return run(plain)
+
+    def pooled():
+        g = np.empty(widths[-1], np.float32)
+        lib.mi_sync(); lib.mi_d2h(g.ctypes.data, H0.mi_unet_gfilm_codes(net.h), g.nbytes)
+        return g
+
+    outs = []
+    for cs in ([0.0] * film, [1.5, -0.5, 0.25, 2.0][:film], [-1.0, 0.75, 0.5, -0.125][:film]) if film else ([],):
+        codes(cs)
+        got = run(net); outs.append(got)
+        gv = pooled() if gfilm else None
+        assert np.array_equal(got, want(np.asarray(cs, np.float32), gv)), cs
+        assert np.array_equal(run(net), got)                        # again: the affines are remade from the stored ones, not compounded
+    if film and not attn:
+        assert np.array_equal(outs[0], base)                        # zero codes: the donor's function whatever the pairs
+    if film:
+        assert not np.array_equal(outs[1], outs[0]) and not np.array_equal(outs[2], outs[1])
+    if gfilm:                                                       # the codes are the stage's output tokens' mean: of the stored tensor's values up to its e4m3 rounding
+        ptr, shp = {name: (ptr, shp) for name, ptr, shp in net.layer_outs()}["attn"]
+        Sg = shp[2] * shp[3] * shp[4]; nb = lib.lp_mx8_bytes(shp[0], shp[1], Sg)
+        buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+        st = orc.mx_to_f32(8, buf, 1, widths[-1], Sg).reshape(widths[-1], Sg).astype(np.float64)
+        gv = pooled()
+        assert np.abs(gv - st.mean(1)).max() < 0.05 * np.abs(st).mean() and np.abs(gv).max() > 0
+    assert np.array_equal(net.params(), p)
+    path = str(tmp_path / "film.ckpt")
+    assert net.save(path, step=2, extra="{}") == 0
+    head = open(path, "rb").readline()
+    assert (b',"film":%d,' % film in head) == bool(film) and (b',"gfilm":1,' in head) == bool(gfilm) and b'"nparams":%d,' % p.size in head
+    assert plain.load(path) == -1
+    other = UNet(make_cfg(cin, widths, film=film, gfilm=gfilm, **kw), N, D, H, W, seed=9)
+    assert other.load(path) == 2 and np.array_equal(other.params(), p)
+    if film:
+        a = np.asarray([-1.0, 0.75, 0.5, -0.125][:film], np.float32)
+        H0.unet_set_film(other.h, a.ctypes.data_as(C.POINTER(C.c_float)), a.size)
+    assert np.array_equal(run(other), outs[-1])
+    net.close(); plain.close(); other.close()
+
+
 @pytest.mark.parametrize("widths,dn,attn", [([32, 64, 128], 1, 0), ([32, 96], 0, 1)])
 def test_unet_gn_ema(gpu, tmp_path, widths, dn, attn):
     """cfg.gn_ema (src/unet.h:67-71): every GroupNorm site (block norms of all levels, down norms, the attention stage's output) reads the

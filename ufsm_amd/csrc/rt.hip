@@ -115,6 +115,54 @@ extern "C" void mi_gn_sums_zero(double *sums, int nslots) {
     const size_t n = (size_t)nslots * 6;   // 24 bytes = 6 words
     fill_u32_k<<<nblk_(n, 256), 256>>>((unsigned *)sums, n, 0u); MICK();
 }
+// ---- FiLM on GroupNorm affines (src/nn.h:494-504): a norm of C channels at offsets gam / bet of the parameter vector p, its K x C pairs A
+// (scale) and D (shift) at fo, A first. cfg.film: K host codes c, fw gamma = gamma (1 + sum_k c_k A_kc), fw beta = beta + sum_k c_k D_kc.
+// cfg.gfilm: the codes are a device vector (the attention stage's output averaged over the window's tokens) and the affine before is the one
+// fw already holds (kept in g1). The sums are fused multiply-add chains from k = 0, as the reference's contracted loop ----
+struct film_codes_t { float c[4]; };
+__global__ void __launch_bounds__(64) film_affine_k(const float *__restrict__ p, float *__restrict__ fw, size_t gam, size_t bet, size_t fo, int C, int K, film_codes_t cc) {
+    const int c = blockIdx.x * 64 + threadIdx.x;
+    if (c >= C) return;
+    const float *A = p + fo + c, *D = A + (size_t)K * C;
+    float s = 0.f, t = 0.f;
+    for (int k = 0; k < K; k++) { s = fmaf(cc.c[k], A[(size_t)k * C], s); t = fmaf(cc.c[k], D[(size_t)k * C], t); }
+    const float one_s = 1.f + s;
+    fw[gam + c] = p[gam + c] * one_s;
+    fw[bet + c] = p[bet + c] + t;
+}
+extern "C" void nn_film_fwd(const float *p, float *fw, size_t gam, size_t bet, size_t fo, int C, int K, const float *codes) {
+    if (C <= 0) return;
+    if (K < 0 || K > 4) mi_die("nn_film_fwd: 0 .. 4 codes, not %d", K);
+    film_codes_t cc = {{0.f, 0.f, 0.f, 0.f}};
+    for (int k = 0; k < K; k++) cc.c[k] = codes[k];
+    film_affine_k<<<(C + 63) / 64, 64>>>(p, fw, gam, bet, fo, C, K, cc); MICK();
+}
+// g[c] = mean over S of x[c S + s]: one workgroup of 256 per channel, fp64 partial sums of the strided elements, a halving tree over the 256
+__global__ void __launch_bounds__(256) chan_mean_k(const float *__restrict__ x, long S, float *__restrict__ g) {
+    __shared__ double part[256];
+    const float *row = x + (size_t)blockIdx.x * S;
+    double a = 0;
+    for (long s = threadIdx.x; s < S; s += 256) a += (double)row[s];
+    part[threadIdx.x] = a;
+    __syncthreads();
+    for (int h = 128; h; h >>= 1) { if ((int)threadIdx.x < h) part[threadIdx.x] += part[threadIdx.x + h]; __syncthreads(); }
+    if (!threadIdx.x) g[blockIdx.x] = (float)(part[0] / (double)S);
+}
+extern "C" void nn_gfilm_pool(const float *x, int C, long S, float *g) { if (C > 0 && S > 0) { chan_mean_k<<<C, 256>>>(x, S, g); MICK(); } }
+__global__ void __launch_bounds__(64) gfilm_affine_k(const float *__restrict__ p, float *__restrict__ fw, size_t gam, size_t bet, size_t fo, int C, int K, const float *__restrict__ gv, float *__restrict__ g1) {
+    const int c = blockIdx.x * 64 + threadIdx.x;
+    if (c >= C) return;
+    const float *A = p + fo + c, *B = A + (size_t)K * C;
+    float s = 0.f, t = 0.f;
+    for (int k = 0; k < K; k++) { const float gk = gv[k]; s = fmaf(gk, A[(size_t)k * C], s); t = fmaf(gk, B[(size_t)k * C], t); }
+    const float before = fw[gam + c], one_s = 1.f + s;
+    g1[c] = before;
+    fw[gam + c] = before * one_s;
+    fw[bet + c] = fw[bet + c] + t;
+}
+extern "C" void nn_gfilm_fwd(const float *p, float *fw, size_t gam, size_t bet, size_t fo, int C, int K, const float *gv, float *g1) {
+    if (C > 0) { gfilm_affine_k<<<(C + 63) / 64, 64>>>(p, fw, gam, bet, fo, C, K, gv, g1); MICK(); }
+}
 // ---- y += a x over n floats (nn_axpy, src/nn.h): the stem bias of a scale-conditioned net ----
 // (a few dozen values in practice: one wavefront strides over them, one fused multiply-add each, as the reference's contracted a * x + y)
 __global__ void __launch_bounds__(64) scaled_add_k(float *__restrict__ y, float a, const float *__restrict__ x, size_t n) {

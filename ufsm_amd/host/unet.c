@@ -27,6 +27,11 @@ struct unet {
     /* cfg.l0_norm 1 .. 3 (src/unet.h:52-58): the level-0 GroupNorms on constant statistics: mean 0 / rstd 1 (none, ws) or the checkpoint's running
        statistics once its warm-up is over (ema: l0run = [live weights: 4 sites x (mean G | var G)][EMA weights: the same], device; l0_n updates so far) */
     float *l0run; long l0_n; int l0_warm; float l0_mom; float ws_gain;
+    /* cfg.film (src/unet.h:108-111): K codes per forward scale and shift the output norms of the encoder blocks (level 0 up) and then of the decoder
+       blocks (coarsest first): film_off = the first norm's K x C scale / shift pair, the pairs in that order; the effective affines live in the
+       forward weight copy. cfg.gfilm (src/unet.h:60-64): the decoder blocks' output norms once more, by the attention stage's output averaged over
+       the window's tokens (gf_K = widths[L-1] device codes gf_g); gf_g1 keeps the affines before */
+    size_t film_off, gf_off; float film_c[4]; int film_ok, gf_K; float *gf_g, *gf_g1;
     size_t sc_w; float sc_c; float *stem_b;                        /* cfg.scale_cond (src/unet.h:24, src/unet.c:129): the conditioning vector's offset, the current code, the stem bias b + c v of a forward */
     /* cfg.gn_ema (src/unet.h:67-71): every GroupNorm (all levels, down norms, the attention stage's) on the checkpoint's running statistics:
        ge_run = [live weights: ge_ns values][EMA weights: the same], per site pair [mean G | var G] in the order of gn_sites (src/unet.c:5125-5135) */
@@ -83,7 +88,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->l0_norm == 2 && (c->G < c->widths[0] ? c->G : c->widths[0]) > 64) return "l0_norm 2 with more than 64 groups";
     if (c->l0_norm == 4 && c->widths[0] > 32) return "l0_norm 4 with more than 32 level-0 channels";   /* (one MX channel block: a slab is a sample of the same layout) */
     if (c->l0_slab && c->l0_norm != 4) return "l0_slab without l0_norm 4";
-    if (c->gfilm) return "gfilm";
+    if (c->gfilm && (!c->attn_blocks || c->nlev < 2)) return "gfilm without the attention stage (src/unet.c:517)";
     if (c->gn_ema && c->l0_norm) return "gn_ema with l0_norm (src/unet.c:551)";
     if (c->attn_vres) return "attn_vres";
     if (c->attn_axis) return "attn_axis";
@@ -92,7 +97,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->view_P || c->view_patch) return "view_P";
     if (c->attn_deform || c->attn_dlev || c->attn_dco || c->attn_dinit) return "attn_deform";
     if (c->emb_lev < 0 || (c->emb_lev > 0 && (c->emb_lev > c->nlev - 2 || c->emb_ch <= 0)) || (!c->emb_lev && c->emb_ch)) return "emb_lev (decoder levels 1 .. nlev - 2, at least one channel)";      /* (src/unet.c:510) */
-    if (c->film) return "film";
+    if (c->film < 0 || c->film > 4) return "film (0 .. 4 codes, src/unet.c:512)";
     if (c->skip_thr || c->skip_margin || c->skip_nl) return "skip_empty";
     if (c->fstem || c->fstem_out) return "fstem";
     if (c->lat_dec || c->lat_dec_raw || c->lat_dec_ng || c->lat_dec_wq) return "lat_dec";
@@ -114,6 +119,8 @@ static size_t ge_sites(unet *u, float **mean, float **rstd, int *g, size_t *off)
     if (mean && k > 192) { fprintf(stderr, "unet: gn_ema: %d GroupNorm sites (at most 192)\n", k); abort(); }
     return o;
 }
+/* cfg.film's norms, j < 2 L - 1: the encoder blocks' output norms from level 0, then the decoder blocks' from the coarsest (src/unet.c:372-373) */
+static const gnpar *film_norm(const unet *u, int j) { const int L = u->cfg.nlev; return j < L ? &u->enc[j].n2 : &u->dec[L - 2 - (j - L)].n2; }
 unet *unet_create(const unet_cfg *cfg) {
     const int L = cfg->nlev;
     if (L < 1 || L > UNET_MAXLEV || cfg->cin < 1 || cfg->cout < 1 || cfg->G < 1) { fprintf(stderr, "unet_create: bad configuration (nlev %d, cin %d, cout %d, G %d)\n", L, cfg->cin, cfg->cout, cfg->G); return nullptr; }
@@ -165,9 +172,16 @@ unet *unet_create(const unet_cfg *cfg) {
         u->tbn = cfg->attn_blocks;
     }
     if (cfg->emb_lev) off = add_conv(&u->eh, dw_of(cfg, cfg->emb_lev), cfg->emb_ch, 1, off);        /* (after the attention stage, src/unet.c:511) */
+    if (cfg->film) { u->film_off = off; for (int j = 0; j < 2 * L - 1; j++) off += (size_t)2 * cfg->film * film_norm(u, j)->c; }      /* (src/unet.c:513) */
+    if (cfg->gfilm) {                                              /* one pair per decoder block's output norm, the coarsest first (src/unet.c:516-520) */
+        u->gf_K = w[L - 1]; u->gf_off = off;
+        int cs = 0;
+        for (int i = L - 2; i >= 0; i--) { off += (size_t)2 * u->gf_K * u->dec[i].n2.c; cs += u->dec[i].n2.c; }
+        u->gf_g = f32_new((size_t)u->gf_K); u->gf_g1 = f32_new((size_t)cs);
+    }
     u->np = off;
     u->p = f32_new(off); u->ema = f32_new(off); u->params = u->src = u->p;
-    if (cfg->w4_2d || cfg->l0_norm == 3) { u->wm = f32_new(off); u->params = u->wm; }
+    if (cfg->w4_2d || cfg->l0_norm == 3 || cfg->film || cfg->gfilm) { u->wm = f32_new(off); u->params = u->wm; }
     if (cfg->l0_norm == 3) {           /* 1 / std(silu(z)), z ~ N(0, 1): the gain of the convs that read a SiLU output (the quadrature of src/unet.c:543-547) */
         double s1 = 0, s2 = 0;
         for (int i = -24000; i <= 24000; i++) { const double z = i * 5e-4, p = exp(-0.5 * z * z) * 5e-4 / sqrt(2 * 3.14159265358979323846), y = z / (1 + exp(-z)); s1 += p * y; s2 += p * y * y; }
@@ -298,6 +312,7 @@ void unet_free(unet *u) {
     mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm); if (u->l0run) mi_free(u->l0run); if (u->ge_run) mi_free(u->ge_run);
     for (int i = 0; i < UNET_MAXLEV; i++) { free(u->rb[i]); free(u->rbn[i]); }
     if (u->stem_b) mi_free(u->stem_b);
+    if (u->gf_g) { mi_free(u->gf_g); mi_free(u->gf_g1); }
     lp_wmemo_clear();
     free(u);
 }
@@ -317,8 +332,18 @@ void unet_use_ema(unet *u, int on) {      /* (the prepared weights are keyed by 
    The reference forms the copy before every forward; here it is formed when the weights were replaced through this interface (set / load /
    EMA switch). A caller that writes through unet_param_ptr calls mi_unet_weights_changed. */
 void mi_unet_weights_changed(unet *u) { u->wm_ok = 0; lp_wmemo_clear(); }
+static void film_one(unet *u, int j) {                             /* norm j's effective affine of the current codes, from the selected weights into the copy */
+    size_t fo = u->film_off;
+    for (int k = 0; k < j; k++) fo += (size_t)2 * u->cfg.film * film_norm(u, k)->c;
+    const gnpar *n = film_norm(u, j);
+    nn_film_fwd(u->src, u->wm, n->gamma, n->beta, fo, n->c, u->cfg.film, u->film_c);
+}
 static void fw_refresh(unet *u) {
-    if (!u->wm || u->wm_ok) return;
+    if (!u->wm) return;
+    if (u->wm_ok) {                                                /* the copy is current but for the codes' affines (src/unet.c:374-380) */
+        if (u->cfg.film && !u->film_ok) { for (int j = 0; j < 2 * u->cfg.nlev - 1; j++) film_one(u, j); u->film_ok = 1; }
+        return;
+    }
     mi_d2d(u->wm, u->src, u->np * 4);
     const int L = u->cfg.nlev;
     if (u->cfg.l0_norm == 3) {         /* ws: the four level-0 3^3 convs standardised per output channel over its fan-in; the network input conv without the SiLU gain (src/unet.c:5298-5304, :5311-5318) */
@@ -334,8 +359,25 @@ static void fw_refresh(unet *u) {
         for (int i = 0; i < L; i++) for (int k = 0; k < u->cfg.enc_blocks[i]; k++) { if (n + 2 > 4 * UNET_MAXLEV) { for (int j = 0; j < n; j++) nn_fakeq_w4_2d(u->wm + cs[j]->w, cs[j]->cout, cs[j]->cin, 27, 32); n = 0; } cs[n++] = &u->rb[i][k].c1; cs[n++] = &u->rb[i][k].c2; }      /* (src/unet.c:5338) */
         for (int i = 0; i < n; i++) nn_fakeq_w4_2d(u->wm + cs[i]->w, cs[i]->cout, cs[i]->cin, 27, 32);
     }
+    if (u->cfg.film) { for (int j = 0; j < 2 * L - 1; j++) film_one(u, j); u->film_ok = 1; }
     lp_wmemo_clear();
     u->wm_ok = 1;
+}
+/* cfg.gfilm, after the attention stage (its output in tb_cs, fp32 [C][S], one window): the pooled tokens are the codes of the decoder blocks'
+   output norms, applied to the affines the copy would hold without them: the selected weights' or cfg.film's (src/unet.c:386-398) */
+static int gfilm_fwd(unet *u, long S) {
+    if (u->tb.ys.n != 1) { fprintf(stderr, "unet: gfilm takes one window per forward (src/unet.c:390)\n"); return -1; }
+    const int L = u->cfg.nlev, K = u->gf_K;
+    nn_gfilm_pool(u->tb_cs, K, S, u->gf_g);
+    size_t fo = u->gf_off; int co = 0;
+    for (int i = L - 2; i >= 0; i--) {
+        const gnpar *n = &u->dec[i].n2;
+        if (u->cfg.film) film_one(u, L + (L - 2 - i));
+        else { mi_d2d(u->wm + n->gamma, u->src + n->gamma, (size_t)n->c * 4); mi_d2d(u->wm + n->beta, u->src + n->beta, (size_t)n->c * 4); }
+        nn_gfilm_fwd(u->src, u->wm, n->gamma, n->beta, fo, n->c, K, u->gf_g, u->gf_g1 + co);
+        fo += (size_t)2 * K * n->c; co += n->c;
+    }
+    return 0;
 }
 void mi_unet_get_params(const unet *u, float *host) { mi_sync(); mi_d2h(host, u->p, u->np * 4); }
 void mi_unet_set_params(unet *u, const float *host) { mi_h2d(u->p, host, u->np * 4); mi_h2d(u->ema, host, u->np * 4); u->wm_ok = 0; lp_wmemo_clear(); }
@@ -480,6 +522,7 @@ static int tb_fwd(unet *u) {
     }
     lp_mx_gemm_bmemo(0);
     at_tok_to_cs(tin, u->tb_cs, ys.n, C, (long)Sg, nr);
+    if (u->cfg.gfilm && gfilm_fwd(u, (long)Sg)) return -1;        /* (src/unet.c:2827) */
     if (u->act_dt == 4) lp_f32_to_mx4(u->tb_cs, ys.n, C, Sg, b->a2); else lp_f32_to_mx8(u->tb_cs, ys.n, C, Sg, b->a2);
     const int G = G_of(u, C);
     if (!ge_const(u) && nn_gn_stats(b->a2, ys, G, 1e-5f, b->m2, b->r2)) { fprintf(stderr, "unet: attention stage GroupNorm statistics unsupported for this storage\n"); return -1; }
@@ -636,11 +679,13 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
     static const char *const no[] = {"\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":",
-                                     "\"film\":", "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
-                                     "\"skip_empty\":", "\"gfilm\":"};
+                                     "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
+                                     "\"skip_empty\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
     cfg->scale_cond = key_int(line, "\"scale_cond\":", 0);
+    cfg->film = key_int(line, "\"film\":", 0); cfg->gfilm = key_int(line, "\"gfilm\":", 0);      /* (src/unet.c:5683, :5742) */
+    if (!bad && (cfg->film < 0 || cfg->film > 4)) bad = "\"film\":";
     if (!bad && (cfg->l0_norm < 0 || cfg->l0_norm > 4)) bad = "\"l0_norm\":";
     if (l0) {
         memset(l0, 0, sizeof *l0);
@@ -675,6 +720,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
     if (!bad && c.gn_ema != m->gn_ema) bad = "gn_ema";
     if (!bad && (c.scale_cond != 0) != (m->scale_cond != 0)) bad = "scale_cond";
+    if (!bad && (c.film != m->film || (c.gfilm != 0) != (m->gfilm != 0))) bad = "film / gfilm";
     if (!bad && (c.ds_levels != m->ds_levels || c.emb_lev != m->emb_lev || c.emb_ch != m->emb_ch)) bad = "ds_levels / emb_lev";
     for (int i = 0; !bad && i < m->nlev; i++) if (c.enc_blocks[i] != m->enc_blocks[i]) bad = "enc_blocks";
     for (int i = 0; !bad && i < m->nlev - 1; i++) { if (dw_of(&c, i) != dw_of(m, i)) bad = "dec_widths"; if ((c.dec_convs[i] == 1) != (m->dec_convs[i] == 1)) bad = "dec_convs"; }
@@ -718,6 +764,14 @@ int unet_load(unet *u, const char *path) {
     return rc;
 }
 void unet_set_scale(unet *u, double um) { u->sc_c = um > 0 ? (float)log2(um / 4.8) : 0.f; }      /* the code of an input voxel size: log2(um / 4.8) (src/unet.h:141-144, src/unet.c:1943) */
+void unet_set_film(unet *u, const float *codes, int k) {         /* cfg.film nets: the K codes of the following forwards (src/unet.h:148-149, src/unet.c:443) */
+    float c[4];
+    for (int i = 0; i < 4; i++) c[i] = i < k && codes ? codes[i] : 0.f;
+    if (memcmp(c, u->film_c, sizeof c)) { memcpy(u->film_c, c, sizeof c); u->film_ok = 0; }
+}
+size_t unet_gfilm_off(const unet *u) { return u->gf_off; }      /* (src/unet.h:160) */
+size_t mi_unet_film_off(const unet *u) { return u->film_off; }
+const float *mi_unet_gfilm_codes(const unet *u) { return u->gf_g; }      /* cfg.gfilm: the last forward's pooled codes (device, widths[L-1] floats) */
 void unet_set_cond(unet *u, float c) { u->sc_c = c; }             /* the code itself (src/unet.h:146-147) */
 long unet_gn_ema_updates(const unet *u) { return u->ge_n; }       /* src/unet.h:280 */
 long unet_l0_updates(const unet *u) { return u->l0_n; }           /* src/unet.h:314 */
@@ -741,10 +795,12 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     if (u->cfg.w4_2d) fprintf(f, ",\"w4_2d\":%d", u->cfg.w4_2d);
     if (u->cfg.ds_levels) fprintf(f, ",\"ds_levels\":%d", u->cfg.ds_levels);
     if (u->cfg.emb_lev) fprintf(f, ",\"emb_lev\":%d,\"emb_ch\":%d", u->cfg.emb_lev, u->cfg.emb_ch);
+    if (u->cfg.film) fprintf(f, ",\"film\":%d", u->cfg.film);     /* (src/unet.c:5564) */
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
     if (u->cfg.attn_blocks && u->cfg.attn_repeat > 1) fprintf(f, ",\"attn_repeat\":%d", u->cfg.attn_repeat);      /* (src/unet.c:5571) */
     if (u->cfg.l0_norm) fprintf(f, ",\"l0_norm\":%d", u->cfg.l0_norm);
     if (u->cfg.l0_norm == 4) fprintf(f, ",\"l0_slab\":%d", u->cfg.l0_slab);
+    if (u->cfg.gfilm) fputs(",\"gfilm\":1", f);                    /* (src/unet.c:5588) */
     if (u->cfg.gn_ema) {                                           /* every site's running statistics and their state (src/unet.c:5587-5592; written after l0_norm's keys there too) */
         float *r = malloc(2 * u->ge_ns * 4);
         if (r) {

@@ -101,6 +101,9 @@ _PROTOS = {
     "nn_gn_const_fill": (None, [_P, _P, _P, _I, _I, _F]),
     "nn_ws_fwd": (None, [_P, _P, _I, _I, _F, _F]),
     "nn_axpy": (None, [_P, _F, _P, _Z]),
+    "nn_film_fwd": (None, [_P, _P, _Z, _Z, _Z, _I, _I, _P]),
+    "nn_gfilm_pool": (None, [_P, _I, C.c_long, _P]),
+    "nn_gfilm_fwd": (None, [_P, _P, _Z, _Z, _Z, _I, _I, _P, _P]),
     "mi_conv_down2_fwd": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t]),
     "mi_convt_up2_fwd": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t]),
     "mi_conv_fwd_gn": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t, C.c_float, _P, _P]),
