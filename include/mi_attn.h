@@ -81,7 +81,8 @@ void at_cs_to_tok(const float *x, float *t, const float *reg, int n, int C, long
 void at_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg);
 /* replaces at_block_fwd (src/attn.h:..., src/nn_attn.cu:587-633) for self-attention blocks on the MX-fp8 core with MX linears:
    y = x1 + W2 swiglu(W1 LN2(x1)), x1 = x + Wo attention(pack(Wqkv LN1(x))). P: the parameter array, bp: the block's offsets; x, y fp32
-   [T][C] (T = g->nseq g->S); 0, or -1 for a configuration this build does not run (deformable, rays, value residual, fp32 linears) */
+   [T][C] (T = g->nseq g->S); 0, or -1 for a configuration this build does not run (deformable, rays, fp32 linears). w->vr 1 keeps the block's V rows in w->v1; 2 replaces V by
+   v + w->lam[head] (w->v1 - v) and keeps the own rows in w->own when given (the value residual, src/nn_attn.cu:535-542, :609-610) */
 int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, const float *x, float *y, const at_geom *g, at_ws *w);
 
 #ifdef __cplusplus

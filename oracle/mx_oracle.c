@@ -1038,6 +1038,12 @@ size_t orc_block_layout(int C, int F, size_t off, size_t *o) {   /* o[14]: ln1g 
     return off;
 }
 int orc_block_fwd(int bits, int C, int H, int F, int rope, int nreg, float rope_base, const float *P, const float *x, float *y, int nseq, int S, int Hh, int W) {
+    return orc_block_fwd_vr(bits, C, H, F, rope, nreg, rope_base, P, x, y, nseq, S, Hh, W, 0, NULL, NULL);
+}
+/* the same with the value residual (src/nn_attn.cu:535-542, :609-610): vr 1 copies the block's V rows [T][C] into v1; vr 2 replaces V by
+   v + lam[head] (v1 - v), one fused multiply-add, before the pack. Pinned by its special cases (lam 0: the plain block; lam 1: the
+   first block's V) and by the exact block in fp64 (tests/test_oracle_block.py) */
+int orc_block_fwd_vr(int bits, int C, int H, int F, int rope, int nreg, float rope_base, const float *P, const float *x, float *y, int nseq, int S, int Hh, int W, int vr, float *v1, const float *lam) {
     size_t o[14]; orc_block_layout(C, F, 0, o);
     const long T = (long)nseq * S;
     float *xn = malloc((size_t)T * C * 4), *qkv = malloc((size_t)T * 3 * C * 4), *att = malloc((size_t)T * C * 4), *x1 = malloc((size_t)T * C * 4), *hh = malloc((size_t)T * 2 * F * 4), *gg = malloc((size_t)T * F * 4);
@@ -1045,6 +1051,10 @@ int orc_block_fwd(int bits, int C, int H, int F, int rope, int nreg, float rope_
     uint16_t *qh = malloc((size_t)3 * C * (T + 64) * 2);
     orc_ln_fwd(x, P + o[0], P + o[1], xn, NULL, NULL, T, C);
     int e = orc_mx_gemm(bits, 0, 1, (int)T, 3 * C, C, xn, P + o[2], qkv, 0.f, P + o[3], NULL);
+    for (long t = 0; vr && t < T; t++) for (int c = 0; c < C; c++) {
+        float *v = qkv + (size_t)t * 3 * C + 2 * C + c;
+        if (vr == 1) v1[(size_t)t * C + c] = *v; else *v = fmaf(lam[c / (C / H)], v1[(size_t)t * C + c] - *v, *v);
+    }
     orc_fa_pack(qkv, P + o[4], P + o[5], qh, rq, rk, amx, nseq, S, Hh, W, nreg, C, rope, rope_base);
     orc_fa8_fwd(qh, att, lse, nseq, S, H, C);
     e |= orc_mx_gemm(bits, 0, 1, (int)T, C, C, att, P + o[6], x1, 0.f, P + o[7], x);

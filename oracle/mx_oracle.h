@@ -23,6 +23,9 @@
  *   orc_ln_fwd, orc_glu_fwd,      pinned: textbook formulas in numpy fp64 (LayerNorm eps 1e-5, SiLU(a) b, RMS-norm eps 1e-6 times gains, rotary
  *   orc_fa_pack, orc_cs_to_tok    pairs = complex multiplication by exp(i pos base^(-f/8)), norm-preserving), fp16 rounding by numpy
  *   orc_block_fwd                 pinned: the reference's gate (tests/test_attn.c:398-424): rel. L2 against the exact fp64 block
+ *   orc_block_fwd_vr              the value residual (src/nn_attn.cu:535-542, :609-610): pinned by the exact fp64 block with V mixed from the
+ *                                 definition, within the same gate, and by the special cases lam 0 (the plain block, bit for bit) and
+ *                                 lam 1 on one head (that head's V rows replaced by another projection's, the other heads untouched)
  *   orc_pred_place                pinned: box intersection by brute force over all voxels; 255 sigmoid rounded to nearest in fp64
  *   orc_feather_blend             pinned: the reference's own checks (tests/test_predict_feather.c:95-121): core and first-window voxels
  *                                 equal the window's own prediction, a z-shell voxel is u(j) own + (1 - u(j)) lower within 1; constant
@@ -155,6 +158,7 @@ void orc_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg);
 void orc_fa_pack(const float *qkv, const float *qg, const float *kg, uint16_t *qkvh, float *rq, float *rk, float *amx, int nseq, int S, int Hh, int W, int nreg, int C, int rope, float base);
 size_t orc_block_layout(int C, int F, size_t off, size_t *o);
 int orc_block_fwd(int bits, int C, int H, int F, int rope, int nreg, float rope_base, const float *P, const float *x, float *y, int nseq, int S, int Hh, int W);
+int orc_block_fwd_vr(int bits, int C, int H, int F, int rope, int nreg, float rope_base, const float *P, const float *x, float *y, int nseq, int S, int Hh, int W, int vr, float *v1, const float *lam);
 /* sliding-window prediction: sigmoid -> uint8 placement (src/nn_elem.cu:1105-1125) and the one-sided sin^2 feather blend of window borders
    (src/predict.c:282-333) */
 void orc_pred_place(const float *lg, const uint8_t *ct, int D, int W, int hz, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, int iso, uint8_t *dsh);

@@ -78,6 +78,7 @@ def lib():
         L.orc_fa_pack.restype = None; L.orc_fa_pack.argtypes = [C.c_void_p] * 7 + [C.c_int] * 7 + [C.c_float]
         L.orc_block_layout.restype = C.c_size_t; L.orc_block_layout.argtypes = [C.c_int, C.c_int, C.c_size_t, C.c_void_p]
         L.orc_block_fwd.restype = C.c_int; L.orc_block_fwd.argtypes = [C.c_int] * 6 + [C.c_float, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 4
+        L.orc_block_fwd_vr.restype = C.c_int; L.orc_block_fwd_vr.argtypes = [C.c_int] * 6 + [C.c_float, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p, C.c_void_p]
         L.orc_fa8_fwd.restype = None; L.orc_fa8_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
         _lib = L
     return _lib
@@ -205,8 +206,14 @@ def fa_pack(qkv, qg, kg, nseq, S, Hh, W, nreg, Cc, rope, base=100.0):
     return qh, rq, rk, amx
 
 
-def block_fwd(bits, Cc, H, F, rope, nreg, base, P, x, nseq, S, Hh, W):
+def block_fwd(bits, Cc, H, F, rope, nreg, base, P, x, nseq, S, Hh, W, vr=0, v1=None, lam=None):
+    """vr 1: the block's V rows are written into v1 ([T][C] float32, in place); vr 2: V <- v + lam[head] (v1 - v) (src/nn_attn.cu:535-542)"""
     P = np.ascontiguousarray(P, np.float32); x = np.ascontiguousarray(x, np.float32)
     y = np.zeros_like(x)
-    assert lib().orc_block_fwd(bits, Cc, H, F, rope, nreg, base, ptr(P), ptr(x), ptr(y), nseq, S, Hh, W) == 0
+    if not vr:
+        assert lib().orc_block_fwd(bits, Cc, H, F, rope, nreg, base, ptr(P), ptr(x), ptr(y), nseq, S, Hh, W) == 0
+        return y
+    assert v1.dtype == np.float32 and v1.flags.c_contiguous and v1.size == x.size
+    lam = np.ascontiguousarray(lam if lam is not None else np.zeros(H), np.float32)
+    assert lib().orc_block_fwd_vr(bits, Cc, H, F, rope, nreg, base, ptr(P), ptr(x), ptr(y), nseq, S, Hh, W, vr, ptr(v1), ptr(lam)) == 0
     return y

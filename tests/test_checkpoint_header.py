@@ -59,7 +59,7 @@ def test_caller_side_keys_pass_through(tmp_path):
     assert rc == 0 and cfg.half_res == 1 and cfg.scan_norm == 1
 
 
-@pytest.mark.parametrize("feature", ['"lat_guide":1', '"attn_mem":4', '"lat_dec":[16,0,1]', '"film":7', '"fstem":[2,16]', '"view_P":4', '"attn_vres":1', '"l0_norm":7'])
+@pytest.mark.parametrize("feature", ['"lat_guide":1', '"attn_mem":4', '"lat_dec":[16,0,1]', '"film":7', '"fstem":[2,16]', '"view_P":4', '"attn_axis":1', '"l0_norm":7'])
 def test_refuses_architectures_it_does_not_run(tmp_path, feature):
     h = 'UFSM{"nlev":2,"widths":[32,64],%s,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":1,"extra":{}}\n' % feature
     assert read(tmp_path, h)[0] == -2

@@ -91,11 +91,56 @@ def test_block_forward(gpu, bits, rope, nreg, tol):
         assert np.linalg.norm(y - ye) / np.linalg.norm(ye) < tol
 
 
+def test_block_value_residual(gpu):
+    """at_ws.vr (src/nn_attn.cu:535-542, :609-610): vr 1 keeps the block's V rows in v1 and changes nothing else; vr 2 mixes them into a
+    later block's V by the per-head lerp; lam 0 is the plain block bit for bit."""
+    rng = np.random.default_rng(5)
+    Cc, H, F, nseq, D, nreg = 192, 4, 512, 2, 4, 3; S = nreg + D ** 3; T = nseq * S
+    P1, lay = make_block(rng, Cc, F); P2, _ = make_block(rng, Cc, F)
+    x = rng.standard_normal((T, Cc)).astype(np.float32)
+    d = at_dims(); d.C, d.H, d.F, d.rope, d.nreg, d.rope_base = Cc, H, F, 1, nreg, 100.0
+    bp = at_bp(); lib.at_block_layout(C.byref(d), C.byref(bp), 0)
+    ws = at_ws(); wsb = DevBuf(lib.at_ws_bytes(C.byref(d), T)); lib.at_ws_carve(C.byref(ws), C.byref(d), T, wsb.ptr)
+    g = at_geom(); g.nseq, g.S, g.D, g.Hh, g.W = nseq, S, D, D, D
+    dv1, down = DevBuf(T * Cc * 4), DevBuf(T * Cc * 4)
+    dx, dy = DevBuf.from_numpy(x), DevBuf(x.nbytes)
+    lib.at_set_mx(8)
+
+    def run(P, vr, lam=None, own=False):
+        dP = DevBuf.from_numpy(P); dl = DevBuf.from_numpy(np.asarray(lam if lam is not None else np.zeros(H), np.float32))
+        ws.vr = vr; ws.v1 = dv1.ptr; ws.lam = dl.ptr
+        ws.own = down.ptr if own else None
+        assert lib.at_block_fwd(C.byref(d), dP.ptr, C.byref(bp), dx.ptr, dy.ptr, C.byref(g), C.byref(ws)) == 0
+        LP.check()
+        return dy.to_numpy(np.float32, x.shape)
+
+    plain1, plain2 = run(P1, 0), run(P2, 0)
+    assert np.array_equal(run(P1, 1), plain1)                                    # keeping V changes nothing
+    v1 = dv1.to_numpy(np.float32, (T, Cc))
+    v1o = np.zeros((T, Cc), np.float32)
+    orc.block_fwd(8, Cc, H, F, 1, nreg, 100.0, P1, x, nseq, S, D, D, vr=1, v1=v1o)
+    # the value projection's rows: an MX GEMM of LayerNorm outputs both sides, last-bit differences flip an operand code now and then
+    assert np.linalg.norm(v1 - v1o) / np.linalg.norm(v1o) < 2e-3 and np.abs(v1o).max() > 0.1
+    assert np.array_equal(run(P2, 2, np.zeros(H)), plain2)                       # lam 0
+    lam = np.array([0.3, 1.0, 0.0, 0.7], np.float32)
+    got = run(P2, 2, lam, own=True)
+    want = orc.block_fwd(8, Cc, H, F, 1, nreg, 100.0, P2, x, nseq, S, D, D, vr=2, v1=v1, lam=lam)     # (from the device's v1: the mix alone is compared)
+    rel = np.linalg.norm(got - want) / np.linalg.norm(want - x)
+    assert rel < 0.02, rel
+    assert np.linalg.norm(got - plain2) / np.linalg.norm(plain2 - x) > 0.05
+    own = down.to_numpy(np.float32, (T, Cc))                                     # the block's own V rows, kept when a buffer is given
+    v2o = np.zeros((T, Cc), np.float32)
+    orc.block_fwd(8, Cc, H, F, 1, nreg, 100.0, P2, x, nseq, S, D, D, vr=1, v1=v2o)
+    assert np.linalg.norm(own - v2o) / np.linalg.norm(v2o) < 2e-3
+    assert np.array_equal(run(P2, 2, lam), got)                                  # without the buffer: the same output
+    ws.vr = 0
+
+
 def test_block_refuses_what_it_does_not_run(gpu):
     d = at_dims(); d.C, d.H, d.F = 96, 2, 128
     bp = at_bp(); lib.at_block_layout(C.byref(d), C.byref(bp), 0)
     ws = at_ws(); g = at_geom(); g.nseq, g.S = 1, 8
     d.rope = 2                                                                   # scroll-coordinate RoPE needs per-token positions
     assert lib.at_block_fwd(C.byref(d), None, C.byref(bp), None, None, C.byref(g), C.byref(ws)) == -1
-    d.rope = 0; ws.vr = 1                                                        # value residual
+    d.rope = 0; ws.vr = 1                                                        # value residual without its buffer
     assert lib.at_block_fwd(C.byref(d), None, C.byref(bp), None, None, C.byref(g), C.byref(ws)) == -1

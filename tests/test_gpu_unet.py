@@ -771,6 +771,80 @@ def test_unet_scale_cond(gpu, tmp_path, widths, cin, eb):
     assert np.array_equal(run(other), with_bias(-0.75))
 
 
+def test_unet_attention_value_residual(gpu, tmp_path):
+    """cfg.attn_vres (src/unet.h:81): every application after the first mixes the first one's V rows into its own by its block's per-head lerp
+    (tb_vr_set, src/unet.c:2699-2704; the lerps a row per block after the blocks' parameters, 0.5 from the second block on, src/unet.c:504,
+    :644). Zero lerps are the net without the residual, byte for byte; trained-like ones follow the oracle's composition of the stage."""
+    from ufsm_amd.unet import UNet, make_cfg
+    rng = np.random.default_rng(31)
+    N, D = 2, 16; widths = [32, 96]; cin, head_out, nreg, nblk, rep = 4, 2, 3, 2, 2
+    S = D ** 3; Cb = widths[-1]; Hh = Cb // 48; F = (8 * Cb // 3 + 31) // 32 * 32
+    x = rng.standard_normal((N, cin, S)).astype(np.float32); dxq = to_mx(8, x)
+    kw = dict(head_out=head_out, attn_blocks=nblk, attn_pe=1, attn_reg=nreg, attn_repeat=rep)
+    att = UNet(make_cfg(cin, widths, **kw), N, D, D, D, seed=7)
+    vr = UNet(make_cfg(cin, widths, attn_vres=1, **kw), N, D, D, D, seed=7)
+    pa, pv = att.params(), vr.params()
+    assert pv.size == pa.size + nblk * Hh and np.array_equal(pv[:pa.size], pa)
+    assert np.array_equal(pv[pa.size:], np.repeat([0, 0.5], Hh).astype(np.float32))
+    n_conv = unet_ref.param_layout(cin, widths, head_out)[1]
+    lays = []; o = n_conv + nreg * Cb
+    for _ in range(nblk):
+        bl, o = orc.block_layout(Cb, F, o); lays.append(bl)
+    assert o == pa.size
+    for lay in lays:
+        for k, n in (("wo", Cb * Cb), ("w2", Cb * F), ("bo", Cb), ("b1", 2 * F), ("bqkv", 3 * Cb)):
+            pv[lay[k]:lay[k] + n] = 0.05 * rng.standard_normal(n)
+    att.set_params(pv[:pa.size])
+
+    def run(n):
+        d = DevBuf(N * head_out * S * 4)
+        assert n.forward_x(dxq.ptr, d.ptr) == 0
+        LP.check()
+        return d.to_numpy(np.float32, (N, head_out, S))
+
+    pv[pa.size:] = 0; vr.set_params(pv)
+    ref = run(att)
+    assert np.array_equal(run(vr), ref)                                          # zero lerps: no residual
+    lam = rng.uniform(0.1, 0.9, (nblk, Hh)).astype(np.float32)
+    pv[pa.size:] = lam.ravel(); vr.set_params(pv)
+    got_l = run(vr)
+    assert not np.array_equal(got_l, ref)
+    outs = {name: (ptr, shp) for name, ptr, shp in vr.layer_outs()}
+    Sg = (D // 2) ** 3
+
+    def fetch(name):
+        ptr, shp = outs[name]; nb = lib.lp_mx8_bytes(shp[0], shp[1], Sg)
+        buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+        return orc.mx_to_f32(8, buf, N, Cb, Sg)
+
+    xb, got = fetch("enc1.c2"), fetch("attn")
+
+    def stage(with_vr):
+        tok = np.zeros((N, Sg + nreg, Cb), np.float32)
+        reg = np.ascontiguousarray(pv[n_conv:n_conv + nreg * Cb].reshape(nreg, Cb))
+        orc.lib().orc_cs_to_tok(orc.ptr(xb), orc.ptr(tok), orc.ptr(reg), N, Cb, Sg, nreg)
+        t = tok.reshape(N * (Sg + nreg), Cb); v1 = np.zeros_like(t)
+        for k in range(nblk * rep):
+            lay = lays[k % nblk]
+            t = orc.block_fwd(8, Cb, Hh, F, 1, nreg, 100.0, pv[lay["ln1g"]:lay["b2"] + Cb], t, N, Sg + nreg, D // 2, D // 2,
+                              vr=(1 if k == 0 else 2) if with_vr else 0, v1=v1, lam=lam[k % nblk])
+        want = np.zeros_like(xb)
+        orc.lib().orc_tok_to_cs(orc.ptr(t), orc.ptr(want), N, Cb, Sg, nreg)
+        return orc.mx_to_f32(8, orc.f32_to_mx(8, want, N, Cb, Sg), N, Cb, Sg)
+
+    want, without = stage(True), stage(False)
+    rel = np.linalg.norm(got - want) / np.linalg.norm(want - xb)
+    assert rel < 0.05 * rep, rel
+    assert np.linalg.norm(got - without) > 3 * np.linalg.norm(got - want)        # and the residual is what moved it
+    path = str(tmp_path / "vr.ckpt")
+    assert vr.save(path, step=5, extra="{}") == 0
+    assert b',"attn_mlp":%d,"attn_vres":1,"attn_repeat":2,' % F in open(path, "rb").readline()
+    assert att.load(path) == -1
+    other = UNet(make_cfg(cin, widths, attn_vres=1, **kw), N, D, D, D, seed=1)
+    assert other.load(path) == 5 and np.array_equal(run(other), got_l)
+    att.close(); vr.close(); other.close()
+
+
 def fma32(a, b, c):
     """fp32 fused multiply-add of arrays through float64: the product is exact there, the sum rounds to 53 bits before the 24."""
     return (np.asarray(a, np.float32).astype(np.float64) * np.asarray(b, np.float32).astype(np.float64) + np.asarray(c, np.float32).astype(np.float64)).astype(np.float32)

@@ -65,7 +65,8 @@ def test_pack_is_rms_norm_gains_rotary_and_fp16(rope):
         assert np.abs((got[0, :, :T] ** 2).sum(-1) - (want[0] ** 2).sum(-1)).max() < 0.05
 
 
-def exact_block(P, lay, x, nseq, S, H, Cc, F):
+def exact_block(P, lay, x, nseq, S, H, Cc, F, v1=None, lam=None):
+    """v1 / lam: the value residual from its definition, V <- v + lam[head] (v1 - v)"""
     P = P.astype(np.float64); x = x.astype(np.float64)
     g = lambda k, n: P[lay[k]:lay[k] + n]
     xn = ln64(x, g("ln1g", Cc), g("ln1b", Cc))
@@ -74,6 +75,8 @@ def exact_block(P, lay, x, nseq, S, H, Cc, F):
     q, k, v = (qkv[:, i * Cc:(i + 1) * Cc].reshape(T, H, 48) for i in range(3))
     q = q / np.sqrt((q ** 2).mean(-1, keepdims=True) + 1e-6) * g("qg", Cc).reshape(H, 48)
     k = k / np.sqrt((k ** 2).mean(-1, keepdims=True) + 1e-6) * g("kg", Cc).reshape(H, 48)
+    if v1 is not None:
+        v = v + np.asarray(lam, np.float64)[None, :, None] * (v1.astype(np.float64).reshape(T, H, 48) - v)
     o = np.zeros((T, Cc))
     for s in range(nseq):
         sl = slice(s * S, (s + 1) * S)
@@ -109,3 +112,43 @@ def test_block_within_reference_gate_of_exact_block(bits, tol):
     # the residual stream dominates y; the gate must also hold on what the block adds
     rel_d = np.linalg.norm((y - x) - (ye - x)) / np.linalg.norm(ye - x)
     assert rel_d < 3 * tol, rel_d
+
+
+def test_value_residual_special_cases_and_exact_block():
+    """orc_block_fwd_vr (src/nn_attn.cu:535-542, :609-610): lam 0 is the plain block bit for bit; lam 1 on one head gives that head the V rows of
+    another value projection and leaves the other heads alone (so the rows mixed are V's, head by head); a general lam stays within the
+    reference's gate of the exact fp64 block with V mixed from the definition."""
+    rng = np.random.default_rng(21)
+    Cc, H, F, nseq, D, nreg = 96, 2, 128, 2, 4, 2; S = nreg + D ** 3; T = nseq * S
+    P, lay = make_block(rng, Cc, F)
+    x = rng.standard_normal((T, Cc)).astype(np.float32)
+    run = lambda Pm, **kw: orc.block_fwd(8, Cc, H, F, 1, nreg, 100.0, Pm, x, nseq, S, D, D, **kw)
+    plain = run(P)
+    P2 = P.copy()                                                    # another value projection: the V third of wqkv / bqkv
+    P2[lay["wqkv"] + 2 * Cc * Cc:lay["wqkv"] + 3 * Cc * Cc] = 0.05 * rng.standard_normal(Cc * Cc)
+    P2[lay["bqkv"] + 2 * Cc:lay["bqkv"] + 3 * Cc] = 0.05 * rng.standard_normal(Cc)
+    v1 = np.zeros((T, Cc), np.float32)
+    assert np.array_equal(run(P2, vr=1, v1=v1), run(P2)) and np.abs(v1).max() > 0                    # keeping V changes nothing
+    v1_0 = v1.copy()
+    assert np.array_equal(run(P, vr=2, v1=v1, lam=[0, 0]), plain) and np.array_equal(v1, v1_0)
+    for head in range(H):
+        lam = np.zeros(H, np.float32); lam[head] = 1
+        P3 = P.copy()                                                # the block whose value projection of that head is P2's
+        for h_ in (head,):
+            r0 = lay["wqkv"] + (2 * Cc + h_ * 48) * Cc
+            P3[r0:r0 + 48 * Cc] = P2[r0:r0 + 48 * Cc]
+            b0 = lay["bqkv"] + 2 * Cc + h_ * 48
+            P3[b0:b0 + 48] = P2[b0:b0 + 48]
+        got, want = run(P, vr=2, v1=v1, lam=lam), run(P3)
+        assert np.linalg.norm(got - want) / np.linalg.norm(want - x) < 2e-3                           # v + (v1 - v) is v1 up to an ulp: a rare code flip downstream
+        assert np.linalg.norm(got - plain) / np.linalg.norm(plain - x) > 0.05
+    lam = np.array([0.3, 0.8], np.float32)
+    # (the exact block above has no rotary embedding and no registers: the gate is taken without them, S = D^3)
+    S0 = D ** 3; x0 = np.ascontiguousarray(x[:nseq * S0])
+    run0 = lambda Pm, **kw: orc.block_fwd(8, Cc, H, F, 0, 0, 100.0, Pm, x0, nseq, S0, D, D, **kw)
+    v1n = np.zeros((nseq * S0, Cc), np.float32); run0(P2, vr=1, v1=v1n)
+    got = run0(P, vr=2, v1=v1n, lam=lam)
+    ye = exact_block(P, lay, x0, nseq, S0, H, Cc, F, v1=v1n, lam=lam)
+    assert np.linalg.norm(got - ye) / np.linalg.norm(ye) < 0.1 and np.linalg.norm((got - x0) - (ye - x0)) / np.linalg.norm(ye - x0) < 0.3
+    ye_plain = exact_block(P, lay, x0, nseq, S0, H, Cc, F)
+    assert np.linalg.norm(got - ye_plain) > 2 * np.linalg.norm(got - ye)         # and the mix is what moved it

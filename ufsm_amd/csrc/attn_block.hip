@@ -264,13 +264,36 @@ inline int linear(const linear_t &l, long T, const float *in, float *out, const 
     return at_gemm_ex(0, 1, (int)T, l.out, l.in, in, l.w, out, 0.f, l.b, residual);
 }
 }
+// Value residual (at_ws.vr, src/nn_attn.cu:535-542, :609-610) on the V third of the qkv rows [T][3 C]: the first block of a stage (vr 1) keeps its
+// V in v1; a later one (vr 2) replaces its own V by v + lam[head] (v1 - v), one fused multiply-add, and keeps the own V when a buffer is given.
+__global__ void __launch_bounds__(256) v_keep_k(const float *__restrict__ qkv, float *__restrict__ v1, size_t n4, int C4) {
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (i >= n4) return;
+    const size_t t = i / C4; const int c = (int)(i - t * C4);
+    ((float4 *)v1)[i] = ((const float4 *)qkv)[t * 3 * C4 + 2 * C4 + c];
+}
+__global__ void __launch_bounds__(256) v_mix_k(float *__restrict__ qkv, const float *__restrict__ v1, float *__restrict__ own, const float *__restrict__ lam, size_t n4, int C4) {
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (i >= n4) return;
+    const size_t t = i / C4; const int c = (int)(i - t * C4);
+    float4 *v = (float4 *)qkv + t * 3 * C4 + 2 * C4 + c;
+    const float4 o = *v, f = ((const float4 *)v1)[i];
+    const float l = lam[c * 4 / HD];                               // (a head is 48 channels: a group of four lies in one)
+    if (own) ((float4 *)own)[i] = o;
+    *v = make_float4(fmaf(l, f.x - o.x, o.x), fmaf(l, f.y - o.y, o.y), fmaf(l, f.z - o.z, o.z), fmaf(l, f.w - o.w, o.w));
+}
 extern "C" int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, const float *x, float *y, const at_geom *g, at_ws *w) {
-    if (d->dK > 0 || g->rays || g->lens || g->pos || w->vr || d->rope > 1 || d->C != d->H * HD) return -1;
+    if (d->dK > 0 || g->rays || g->lens || g->pos || w->vr < 0 || w->vr > 2 || (w->vr && (!w->v1 || (w->vr == 2 && !w->lam))) || d->rope > 1 || d->C != d->H * HD) return -1;
     const long T = (long)g->nseq * g->S; const int C = d->C, F = d->F;
     const linear_t qkv = {P + bp->wqkv, P + bp->bqkv, 3 * C, C}, proj = {P + bp->wo, P + bp->bo, C, C}, up = {P + bp->w1, P + bp->b1, 2 * F, C}, down = {P + bp->w2, P + bp->b2, C, F};
     // attention branch
     at_ln_fwd(x, P + bp->ln1g, P + bp->ln1b, w->xn, w->m1, w->r1, T, C);
     if (int e = linear(qkv, T, w->xn, w->qkv, nullptr)) return e;
+    if (w->vr) {
+        const size_t n4 = (size_t)T * C / 4;
+        if (w->vr == 1) v_keep_k<<<nblk_(n4, 256), 256>>>(w->qkv, w->v1, n4, C / 4); else v_mix_k<<<nblk_(n4, 256), 256>>>(w->qkv, w->v1, w->own, w->lam, n4, C / 4);
+        MICK();
+    }
     at_fa_pack(w->qkv, P + bp->qg, P + bp->kg, w->qkvh, w->rq, w->rk, w->amx, g, d->nreg, C, d->rope, d->rope_base);
     if (int e = at_fa8_fwd(w->qkvh, w->o, w->lse, g, d->H, C)) return e;
     if (int e = linear(proj, T, w->o, w->x1, x)) return e;

@@ -54,6 +54,7 @@ struct unet {
     /* the attention stage on the bottleneck (src/unet.c:470-509 set-up, :2795-2835 forward) */
     int tbn; at_dims tbd; at_bp tbp[16]; size_t reg_off; at_geom tbg; at_ws tbw;
     block tb;                                                      /* its output: a2 and the statistics m2 / r2 (the level's n2 affine) */
+    float *tb_vr; size_t vr_off;                                   /* cfg.attn_vres (src/unet.h:81): the first application's V rows; the lerps' offset */
     float *tb_cs, *tb_tok; void *tb_ws;                            /* fp32 planes [n][C][Sg]; token rows, one buffer per block + 1; block scratch */
 };
 
@@ -90,7 +91,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->l0_slab && c->l0_norm != 4) return "l0_slab without l0_norm 4";
     if (c->gfilm && (!c->attn_blocks || c->nlev < 2)) return "gfilm without the attention stage (src/unet.c:517)";
     if (c->gn_ema && c->l0_norm) return "gn_ema with l0_norm (src/unet.c:551)";
-    if (c->attn_vres) return "attn_vres";
+    if (c->attn_vres && !c->attn_blocks) return "attn_vres without attention blocks";
     if (c->attn_axis) return "attn_axis";
     if (c->attn_repeat < 0 || (c->attn_repeat > 1 && (!c->attn_blocks || c->attn_blocks * c->attn_repeat > 64))) return "attn_repeat";
     if (c->attn_mem) return "attn_mem";
@@ -170,6 +171,7 @@ unet *unet_create(const unet_cfg *cfg) {
         u->reg_off = off; off += (size_t)cfg->attn_reg * C;
         for (int k = 0; k < cfg->attn_blocks; k++) off = at_block_layout(&u->tbd, &u->tbp[k], off);
         u->tbn = cfg->attn_blocks;
+        if (cfg->attn_vres) { u->vr_off = off; off += (size_t)cfg->attn_blocks * (size_t)(C / AT_HD); }      /* the value residual's per-head lerps, a row per block (src/unet.c:504) */
     }
     if (cfg->emb_lev) off = add_conv(&u->eh, dw_of(cfg, cfg->emb_lev), cfg->emb_ch, 1, off);        /* (after the attention stage, src/unet.c:511) */
     if (cfg->film) { u->film_off = off; for (int j = 0; j < 2 * L - 1; j++) off += (size_t)2 * cfg->film * film_norm(u, j)->c; }      /* (src/unet.c:513) */
@@ -234,7 +236,7 @@ static void free_acts(unet *u) {
         act_del(u->downo[i]); act_del(u->skipst[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
         u->downo[i] = u->skipst[i] = nullptr; u->dm[i] = u->dr[i] = nullptr;
     }
-    if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); u->tb.a2 = nullptr; u->tb.m2 = u->tb.r2 = nullptr; u->tb_cs = u->tb_tok = nullptr; u->tb_ws = nullptr; }
+    if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); if (u->tb_vr) mi_free(u->tb_vr); u->tb_vr = nullptr; u->tb.a2 = nullptr; u->tb.m2 = u->tb.r2 = nullptr; u->tb_cs = u->tb_tok = nullptr; u->tb_ws = nullptr; }
     for (int i = 0; i < 2; i++) { act_del(u->slab_tmp[i]); act_del(u->slab_carry[i]); u->slab_tmp[i] = u->slab_carry[i] = nullptr; }
     act_del(u->xin); u->xin = nullptr;
     mi_free(u->logits); u->logits = nullptr;
@@ -294,6 +296,7 @@ static int build_acts(unet *u, shape5 in) {
         u->tb.ys = ys; u->tb.a2 = act_new(u, ys);
         const size_t ng = (size_t)in.n * G_of(u, C);
         u->tb.m2 = f32_new(ng); u->tb.r2 = f32_new(ng);
+        if (u->cfg.attn_vres) u->tb_vr = f32_new((size_t)T * C);
         u->tb_cs = f32_new((size_t)ys.n * C * Sg); u->tb_tok = f32_new((size_t)3 * T * C);     /* the stage's input rows and two buffers the applications alternate between */
         u->tb_ws = mi_malloc(at_ws_bytes(&u->tbd, T)); at_ws_carve(&u->tbw, &u->tbd, T, u->tb_ws);
     }
@@ -419,6 +422,7 @@ void unet_init(unet *u, uint64_t seed) {
             for (size_t i = 0; i < (size_t)2 * F * C; i++) h[bp->w1 + i] = (float)(sd * gauss(&seed));
         }
         for (size_t i = 0; i < (size_t)u->tbd.nreg * C; i++) h[u->reg_off + i] = (float)(0.02 * gauss(&seed));
+        if (u->cfg.attn_vres) for (int k = 1; k < u->tbn; k++) for (int hh = 0; hh < u->tbd.H; hh++) h[u->vr_off + (size_t)k * u->tbd.H + hh] = 0.5f;      /* (src/unet.c:644) */
     }
     mi_unet_set_params(u, h);
     free(h);
@@ -517,6 +521,7 @@ static int tb_fwd(unet *u) {
     float *tin = u->tb_tok;
     for (int k = 0; k < tba; k++) {
         float *tout = u->tb_tok + (size_t)(1 + (k & 1)) * TC;
+        if (u->tb_vr) { u->tbw.vr = k ? 2 : 1; u->tbw.v1 = u->tb_vr; u->tbw.own = nullptr; u->tbw.lam = P(u, u->vr_off + (size_t)(k % u->tbn) * (size_t)u->tbd.H); }      /* (tb_vr_set, src/unet.c:2699-2704) */
         if (at_block_fwd(&u->tbd, u->params, &u->tbp[k % u->tbn], tin, tout, &u->tbg, &u->tbw)) { lp_mx_gemm_bmemo(0); fprintf(stderr, "unet: attention block forward failed\n"); return -1; }
         tin = tout;
     }
@@ -673,13 +678,13 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     cfg->ds_levels = key_int(line, "\"ds_levels\":", 0); cfg->emb_lev = key_int(line, "\"emb_lev\":", 0); cfg->emb_ch = key_int(line, "\"emb_ch\":", 0);      /* (src/unet.c:5562-5563) */
     cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
     cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
-    cfg->attn_repeat = key_int(line, "\"attn_repeat\":", 0);
+    cfg->attn_repeat = key_int(line, "\"attn_repeat\":", 0); cfg->attn_vres = key_int(line, "\"attn_vres\":", 0);      /* (src/unet.c:5690) */
     cfg->half_res = key_int(line, "\"half_res\":", 0); cfg->scan_norm = key_int(line, "\"scan_norm\":", 0);      /* (the caller's business: the graph does not use them) */
     if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
     static const char *const no[] = {"\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":",
-                                     "\"fstem\":", "\"lat_dec\":", "\"attn_vres\":", "\"attn_axis\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
+                                     "\"fstem\":", "\"lat_dec\":", "\"attn_axis\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
                                      "\"skip_empty\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
@@ -716,6 +721,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.cout != m->cout) bad = "cout";
     if (!bad && c.attn_blocks != m->attn_blocks) bad = "attn_blocks";
     if (!bad && (c.attn_repeat > 1 ? c.attn_repeat : 1) != (m->attn_repeat > 1 ? m->attn_repeat : 1)) bad = "attn_repeat";
+    if (!bad && (c.attn_vres != 0) != (m->attn_vres != 0)) bad = "attn_vres";
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";
     if (!bad && c.w4_2d != m->w4_2d) bad = "w4_2d";
     if (!bad && c.gn_ema != m->gn_ema) bad = "gn_ema";
@@ -797,6 +803,7 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     if (u->cfg.emb_lev) fprintf(f, ",\"emb_lev\":%d,\"emb_ch\":%d", u->cfg.emb_lev, u->cfg.emb_ch);
     if (u->cfg.film) fprintf(f, ",\"film\":%d", u->cfg.film);     /* (src/unet.c:5564) */
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
+    if (u->cfg.attn_vres) fprintf(f, ",\"attn_vres\":%d", u->cfg.attn_vres);      /* (src/unet.c:5569) */
     if (u->cfg.attn_blocks && u->cfg.attn_repeat > 1) fprintf(f, ",\"attn_repeat\":%d", u->cfg.attn_repeat);      /* (src/unet.c:5571) */
     if (u->cfg.l0_norm) fprintf(f, ",\"l0_norm\":%d", u->cfg.l0_norm);
     if (u->cfg.l0_norm == 4) fprintf(f, ",\"l0_slab\":%d", u->cfg.l0_slab);

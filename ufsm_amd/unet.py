@@ -87,7 +87,7 @@ def load_host():
     return L
 
 
-def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, attn_repeat=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0, gn_ema=0, dec_widths=None, dec_convs=None, enc_blocks=None, ds_levels=0, emb_lev=0, emb_ch=0, scale_cond=0, film=0, gfilm=0):
+def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, attn_repeat=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0, gn_ema=0, dec_widths=None, dec_convs=None, enc_blocks=None, ds_levels=0, emb_lev=0, emb_ch=0, scale_cond=0, film=0, gfilm=0, attn_vres=0):
     """The reference's configuration record plus, as Python attributes, what the reference keeps in process-wide switches: the activation
     storage (unet_set_act_mx4) and the compute precision policy (nn_set_prec), which UNet applies around its calls."""
     c = unet_cfg()
@@ -98,7 +98,7 @@ def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn
     c.l0_norm, c.l0_slab, c.gn_ema = l0_norm, l0_slab, gn_ema
     c.attn_repeat = attn_repeat if attn_blocks else 0
     c.ds_levels, c.emb_lev, c.emb_ch, c.scale_cond = ds_levels, emb_lev, emb_ch, scale_cond
-    c.film, c.gfilm = film, gfilm
+    c.film, c.gfilm, c.attn_vres = film, gfilm, attn_vres
     for i, d in enumerate(dec_widths or []):
         c.dec_widths[i] = d
     for i, d in enumerate(dec_convs or []):
