@@ -78,6 +78,9 @@ void at_fa_pack(const float *qkv, const float *qg, const float *kg, void *qkvh, 
 /* replace at_cs_to_tok / at_tok_to_cs (src/nn_attn.cu:748-759, :802-803): channel-major planes [n][C][Sg] <-> token rows [n][nreg + Sg][C]
    with the learned register rows reg [nreg][C] prepended (dropped on the way back) */
 void at_cs_to_tok(const float *x, float *t, const float *reg, int n, int C, long Sg, int nreg);
+/* replaces at_peg_fwd (src/attn.h:141-144, src/nn_attn.cu:688-705, :738-740): conv positional encoding, y = x + b + depthwise 3^3 conv of x on the
+   grid tokens of each sequence (zero padding), register rows copied; w [C][27], b [C]; x and y separate buffers, g->S = nreg + g->D g->Hh g->W */
+void at_peg_fwd(const float *x, float *y, const float *w, const float *b, const at_geom *g, int nreg, int C);
 void at_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg);
 /* replaces at_block_fwd (src/attn.h:..., src/nn_attn.cu:587-633) for self-attention blocks on the MX-fp8 core with MX linears:
    y = x1 + W2 swiglu(W1 LN2(x1)), x1 = x + Wo attention(pack(Wqkv LN1(x))). P: the parameter array, bp: the block's offsets; x, y fp32

@@ -994,6 +994,24 @@ void orc_cs_to_tok(const float *x, float *t, const float *reg, int n, int C, lon
         t[(size_t)r * C + c] = ts < 0 ? reg[(size_t)(r % S) * C + c] : x[((size_t)s * C + c) * Sg + ts];
     }
 }
+/* conv positional encoding (src/attn.h:141-144, src/nn_attn.cu:688-705): y = x + b + depthwise 3^3 conv of x on the grid tokens (zero padding),
+   register rows copied; each sum starts from x + b and takes the taps inside the grid in (dz, dy, dx) order, one fused multiply-add each */
+void orc_peg_fwd(const float *x, float *y, const float *w, const float *b, int nseq, int S, int D, int Hh, int W, int nreg, int C) {
+    for (long t = 0; t < (long)nseq * S; t++) for (int c = 0; c < C; c++) {
+        const int ts = (int)(t % S) - nreg;
+        const size_t i = (size_t)t * C + c;
+        if (ts < 0) { y[i] = x[i]; continue; }
+        const long g0 = t - ts;
+        const int z = ts / (Hh * W), yy = (ts / W) % Hh, xx = ts % W;
+        float a = x[i] + b[c];
+        for (int dz = -1; dz <= 1; dz++) for (int dy = -1; dy <= 1; dy++) for (int dx = -1; dx <= 1; dx++) {
+            const int zz = z + dz, y2 = yy + dy, x2 = xx + dx;
+            if (zz < 0 || zz >= D || y2 < 0 || y2 >= Hh || x2 < 0 || x2 >= W) continue;
+            a = fmaf(w[c * 27 + (dz + 1) * 9 + (dy + 1) * 3 + dx + 1], x[(size_t)(g0 + ((long)zz * Hh + y2) * W + x2) * C + c], a);
+        }
+        y[i] = a;
+    }
+}
 void orc_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg) {
     for (long s = 0; s < n; s++) for (int c = 0; c < C; c++) for (long ts = 0; ts < Sg; ts++) x[((size_t)s * C + c) * Sg + ts] = t[((size_t)s * (Sg + nreg) + nreg + ts) * C + c];
 }

@@ -23,6 +23,8 @@
  *   orc_ln_fwd, orc_glu_fwd,      pinned: textbook formulas in numpy fp64 (LayerNorm eps 1e-5, SiLU(a) b, RMS-norm eps 1e-6 times gains, rotary
  *   orc_fa_pack, orc_cs_to_tok    pairs = complex multiplication by exp(i pos base^(-f/8)), norm-preserving), fp16 rounding by numpy
  *   orc_block_fwd                 pinned: the reference's gate (tests/test_attn.c:398-424): rel. L2 against the exact fp64 block
+ *   orc_peg_fwd                   pinned: scipy's correlate (zero padding) per channel in fp64, plus bias and the token itself; register rows
+ *                                 are copies; one tap set gives the shifted tensor (tests/test_oracle_block.py)
  *   orc_block_fwd_vr              the value residual (src/nn_attn.cu:535-542, :609-610): pinned by the exact fp64 block with V mixed from the
  *                                 definition, within the same gate, and by the special cases lam 0 (the plain block, bit for bit) and
  *                                 lam 1 on one head (that head's V rows replaced by another projection's, the other heads untouched)
@@ -158,6 +160,7 @@ void orc_tok_to_cs(const float *t, float *x, int n, int C, long Sg, int nreg);
 void orc_fa_pack(const float *qkv, const float *qg, const float *kg, uint16_t *qkvh, float *rq, float *rk, float *amx, int nseq, int S, int Hh, int W, int nreg, int C, int rope, float base);
 size_t orc_block_layout(int C, int F, size_t off, size_t *o);
 int orc_block_fwd(int bits, int C, int H, int F, int rope, int nreg, float rope_base, const float *P, const float *x, float *y, int nseq, int S, int Hh, int W);
+void orc_peg_fwd(const float *x, float *y, const float *w, const float *b, int nseq, int S, int D, int Hh, int W, int nreg, int C);
 int orc_block_fwd_vr(int bits, int C, int H, int F, int rope, int nreg, float rope_base, const float *P, const float *x, float *y, int nseq, int S, int Hh, int W, int vr, float *v1, const float *lam);
 /* sliding-window prediction: sigmoid -> uint8 placement (src/nn_elem.cu:1105-1125) and the one-sided sin^2 feather blend of window borders
    (src/predict.c:282-333) */

@@ -78,6 +78,7 @@ def lib():
         L.orc_fa_pack.restype = None; L.orc_fa_pack.argtypes = [C.c_void_p] * 7 + [C.c_int] * 7 + [C.c_float]
         L.orc_block_layout.restype = C.c_size_t; L.orc_block_layout.argtypes = [C.c_int, C.c_int, C.c_size_t, C.c_void_p]
         L.orc_block_fwd.restype = C.c_int; L.orc_block_fwd.argtypes = [C.c_int] * 6 + [C.c_float, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 4
+        L.orc_peg_fwd.restype = None; L.orc_peg_fwd.argtypes = [C.c_void_p] * 4 + [C.c_int] * 7
         L.orc_block_fwd_vr.restype = C.c_int; L.orc_block_fwd_vr.argtypes = [C.c_int] * 6 + [C.c_float, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p, C.c_void_p]
         L.orc_fa8_fwd.restype = None; L.orc_fa8_fwd.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int]
         _lib = L
@@ -204,6 +205,14 @@ def fa_pack(qkv, qg, kg, nseq, S, Hh, W, nreg, Cc, rope, base=100.0):
     qh = np.zeros((3, H, T + 64, 48), np.uint16); rq = np.zeros((T, H), np.float32); rk = np.zeros((T, H), np.float32); amx = np.zeros(4, np.float32)
     lib().orc_fa_pack(ptr(qkv), ptr(qg), ptr(kg), ptr(qh), ptr(rq), ptr(rk), ptr(amx), nseq, S, Hh, W, nreg, Cc, rope, base)
     return qh, rq, rk, amx
+
+
+def peg_fwd(x, w, b, nseq, S, D, Hh, W, nreg):
+    """token rows x [nseq * S][C] -> x + b + depthwise 3^3 conv on the grid tokens; w [C][27], b [C]"""
+    x = np.ascontiguousarray(x, np.float32); w = np.ascontiguousarray(w, np.float32); b = np.ascontiguousarray(b, np.float32)
+    y = np.zeros_like(x)
+    lib().orc_peg_fwd(ptr(x), ptr(y), ptr(w), ptr(b), nseq, S, D, Hh, W, nreg, x.shape[-1])
+    return y
 
 
 def block_fwd(bits, Cc, H, F, rope, nreg, base, P, x, nseq, S, Hh, W, vr=0, v1=None, lam=None):

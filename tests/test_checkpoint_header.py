@@ -104,4 +104,6 @@ def test_reads_the_running_statistics_key(tmp_path):
 def test_rejects_foreign_files(tmp_path):
     assert read(tmp_path, "not a checkpoint\n")[0] == -1
     assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"skip_empty":[80,2,1],"nparams":1}\n')[0] == -2   # trained with masked convs
-    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":0,"attn_reg":0,"attn_mlp":256,"cin":4,"cout":1,"nparams":1}\n')[0] == -2   # PEG
+    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":3,"attn_reg":0,"attn_mlp":256,"cin":4,"cout":1,"nparams":1}\n')[0] == -2   # scroll RoPE
+    rc, cfg, n, step = read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":0,"attn_reg":0,"attn_mlp":256,"attn_vres":1,"cin":4,"cout":1,"nparams":1}\n')
+    assert rc == 0 and cfg.attn_pe == 0 and cfg.attn_vres == 1     # PEG, value residual

@@ -91,6 +91,21 @@ def test_block_forward(gpu, bits, rope, nreg, tol):
         assert np.linalg.norm(y - ye) / np.linalg.norm(ye) < tol
 
 
+@pytest.mark.parametrize("nseq,dims,nreg,Cc", [(2, (3, 4, 5), 2, 96), (1, (8, 8, 8), 0, 192), (3, (1, 1, 7), 4, 48), (1, (2, 2, 2), 1, 4)])
+def test_peg_matches_oracle_bit_for_bit(gpu, nseq, dims, nreg, Cc):
+    """at_peg_fwd (src/attn.h:141-144): x + b + depthwise 3^3 conv on the grid tokens, the taps in (dz, dy, dx) order as fused multiply-adds:
+    the same bits as the oracle's loop; register rows are copies."""
+    rng = np.random.default_rng(Cc + nreg)
+    D, Hh, W = dims; S = nreg + D * Hh * W
+    x = rng.standard_normal((nseq * S, Cc)).astype(np.float32); w = (0.3 * rng.standard_normal((Cc, 27))).astype(np.float32); b = rng.standard_normal(Cc).astype(np.float32)
+    dx, dy, dw, db = DevBuf.from_numpy(x), DevBuf(x.nbytes), DevBuf.from_numpy(w), DevBuf.from_numpy(b)
+    g = at_geom(); g.nseq, g.S, g.D, g.Hh, g.W = nseq, S, D, Hh, W
+    lib.at_peg_fwd(dx.ptr, dy.ptr, dw.ptr, db.ptr, C.byref(g), nreg, Cc); LP.check()
+    y = dy.to_numpy(np.float32, x.shape)
+    assert np.array_equal(y, orc.peg_fwd(x, w, b, nseq, S, D, Hh, W, nreg))
+    assert np.array_equal(y.reshape(nseq, S, Cc)[:, :nreg], x.reshape(nseq, S, Cc)[:, :nreg]) and np.array_equal(dx.to_numpy(np.float32, x.shape), x)
+
+
 def test_block_value_residual(gpu):
     """at_ws.vr (src/nn_attn.cu:535-542, :609-610): vr 1 keeps the block's V rows in v1 and changes nothing else; vr 2 mixes them into a
     later block's V by the per-head lerp; lam 0 is the plain block bit for bit."""

@@ -771,6 +771,80 @@ def test_unet_scale_cond(gpu, tmp_path, widths, cin, eb):
     assert np.array_equal(run(other), with_bias(-0.75))
 
 
+def test_unet_attention_peg(gpu, tmp_path):
+    """cfg.attn_pe 0 (src/unet.c:491, :2805): the conv positional encoding on the stage's token rows before the blocks (no rotary embedding in
+    them), its depthwise taps [C][27] and bias [C] before the registers in the parameter vector, zero at initialisation (then the stage is the
+    attn_pe 2 net's, byte for byte); with trained-like taps the stage's output follows the oracle's composition."""
+    from ufsm_amd.unet import UNet, make_cfg
+    rng = np.random.default_rng(41)
+    N, D = 2, 16; widths = [32, 96]; cin, head_out, nreg, nblk = 4, 2, 3, 2
+    S = D ** 3; Cb = widths[-1]; Hh = Cb // 48; F = (8 * Cb // 3 + 31) // 32 * 32
+    x = rng.standard_normal((N, cin, S)).astype(np.float32); dxq = to_mx(8, x)
+    kw = dict(head_out=head_out, attn_blocks=nblk, attn_reg=nreg)
+    nope = UNet(make_cfg(cin, widths, attn_pe=2, **kw), N, D, D, D, seed=7)
+    peg = UNet(make_cfg(cin, widths, attn_pe=0, **kw), N, D, D, D, seed=7)
+    pn, pp = nope.params(), peg.params()
+    n_conv = unet_ref.param_layout(cin, widths, head_out)[1]
+    assert pp.size == pn.size + 28 * Cb and not pp[n_conv:n_conv + 28 * Cb].any()
+    lays = []; o = n_conv + 28 * Cb + nreg * Cb
+    for _ in range(nblk):
+        bl, o = orc.block_layout(Cb, F, o); lays.append(bl)
+    assert o == pp.size
+    for lay in lays:
+        for k, n in (("wo", Cb * Cb), ("w2", Cb * F), ("bo", Cb), ("b1", 2 * F), ("bqkv", 3 * Cb)):
+            pp[lay[k]:lay[k] + n] = 0.05 * rng.standard_normal(n)
+    peg.set_params(pp)
+    nope.set_params(np.concatenate([pp[:n_conv], pp[n_conv + 28 * Cb:]]))
+
+    def run(n):
+        d = DevBuf(N * head_out * S * 4)
+        assert n.forward_x(dxq.ptr, d.ptr) == 0
+        LP.check()
+        return d.to_numpy(np.float32, (N, head_out, S))
+
+    ref = run(nope)
+    assert np.array_equal(run(peg), ref)                                         # zero taps and bias: x + 0 + 0
+    wp = (0.2 * rng.standard_normal((Cb, 27))).astype(np.float32); bpg = (0.3 * rng.standard_normal(Cb)).astype(np.float32)
+    pp[n_conv:n_conv + 27 * Cb] = wp.ravel(); pp[n_conv + 27 * Cb:n_conv + 28 * Cb] = bpg
+    peg.set_params(pp)
+    got_l = run(peg)
+    assert not np.array_equal(got_l, ref)
+    outs = {name: (ptr, shp) for name, ptr, shp in peg.layer_outs()}
+    Dg = D // 2; Sg = Dg ** 3
+
+    def fetch(name):
+        ptr, shp = outs[name]; nb = lib.lp_mx8_bytes(shp[0], shp[1], Sg)
+        buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+        return orc.mx_to_f32(8, buf, N, Cb, Sg)
+
+    xb, got = fetch("enc1.c2"), fetch("attn")
+
+    def stage(with_peg):
+        tok = np.zeros((N, Sg + nreg, Cb), np.float32)
+        reg = np.ascontiguousarray(pp[n_conv + 28 * Cb:n_conv + 28 * Cb + nreg * Cb].reshape(nreg, Cb))
+        orc.lib().orc_cs_to_tok(orc.ptr(xb), orc.ptr(tok), orc.ptr(reg), N, Cb, Sg, nreg)
+        t = tok.reshape(N * (Sg + nreg), Cb)
+        if with_peg:
+            t = orc.peg_fwd(t, wp, bpg, N, Sg + nreg, Dg, Dg, Dg, nreg)
+        for lay in lays:
+            t = orc.block_fwd(8, Cb, Hh, F, 0, nreg, 100.0, pp[lay["ln1g"]:lay["b2"] + Cb], t, N, Sg + nreg, Dg, Dg)
+        want = np.zeros_like(xb)
+        orc.lib().orc_tok_to_cs(orc.ptr(t), orc.ptr(want), N, Cb, Sg, nreg)
+        return orc.mx_to_f32(8, orc.f32_to_mx(8, want, N, Cb, Sg), N, Cb, Sg)
+
+    want, without = stage(True), stage(False)
+    rel = np.linalg.norm(got - want) / np.linalg.norm(want - xb)
+    assert rel < 0.05, rel
+    assert np.linalg.norm(got - without) > 3 * np.linalg.norm(got - want)
+    path = str(tmp_path / "peg.ckpt")
+    assert peg.save(path, step=6, extra="{}") == 0
+    assert b',"attn_blocks":2,"attn_pe":0,"attn_reg":3,' in open(path, "rb").readline()
+    assert nope.load(path) == -1
+    other = UNet(make_cfg(cin, widths, attn_pe=0, **kw), N, D, D, D, seed=1)
+    assert other.load(path) == 6 and np.array_equal(run(other), got_l)
+    nope.close(); peg.close(); other.close()
+
+
 def test_unet_attention_value_residual(gpu, tmp_path):
     """cfg.attn_vres (src/unet.h:81): every application after the first mixes the first one's V rows into its own by its block's per-head lerp
     (tb_vr_set, src/unet.c:2699-2704; the lerps a row per block after the blocks' parameters, 0.5 from the second block on, src/unet.c:504,

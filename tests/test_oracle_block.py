@@ -152,3 +152,23 @@ def test_value_residual_special_cases_and_exact_block():
     assert np.linalg.norm(got - ye) / np.linalg.norm(ye) < 0.1 and np.linalg.norm((got - x0) - (ye - x0)) / np.linalg.norm(ye - x0) < 0.3
     ye_plain = exact_block(P, lay, x0, nseq, S0, H, Cc, F)
     assert np.linalg.norm(got - ye_plain) > 2 * np.linalg.norm(got - ye)         # and the mix is what moved it
+
+
+def test_peg_is_depthwise_conv_plus_bias_plus_identity():
+    """orc_peg_fwd (src/attn.h:141-144): against scipy's zero-padded correlation per channel in fp64; a single unit tap shifts the grid."""
+    from scipy.ndimage import correlate
+    rng = np.random.default_rng(4)
+    nseq, (D, Hh, W), nreg, Cc = 2, (3, 4, 5), 2, 8
+    Sg = D * Hh * W; S = nreg + Sg
+    x = rng.standard_normal((nseq, S, Cc)).astype(np.float32); w = (0.3 * rng.standard_normal((Cc, 27))).astype(np.float32); b = rng.standard_normal(Cc).astype(np.float32)
+    y = orc.peg_fwd(x.reshape(nseq * S, Cc), w, b, nseq, S, D, Hh, W, nreg).reshape(nseq, S, Cc)
+    assert np.array_equal(y[:, :nreg], x[:, :nreg])
+    for s in range(nseq):
+        for c in range(Cc):
+            g = x[s, nreg:, c].astype(np.float64).reshape(D, Hh, W)
+            want = g + float(b[c]) + correlate(g, w[c].astype(np.float64).reshape(3, 3, 3), mode="constant", cval=0.0)
+            assert np.abs(y[s, nreg:, c].reshape(D, Hh, W) - want).max() < 1e-5
+    w1 = np.zeros((Cc, 27), np.float32); w1[:, 2 * 9 + 0 * 3 + 1] = 1      # the tap (dz, dy, dx) = (+1, -1, 0)
+    y1 = orc.peg_fwd(x.reshape(nseq * S, Cc), w1, np.zeros(Cc), nseq, S, D, Hh, W, nreg).reshape(nseq, S, Cc)
+    g = x[:, nreg:].reshape(nseq, D, Hh, W, Cc); sh = np.zeros_like(g); sh[:, :-1, 1:] = g[:, 1:, :-1]
+    assert np.array_equal(y1[:, nreg:].reshape(g.shape), g + sh)

@@ -264,6 +264,37 @@ inline int linear(const linear_t &l, long T, const float *in, float *out, const 
     return at_gemm_ex(0, 1, (int)T, l.out, l.in, in, l.w, out, 0.f, l.b, residual);
 }
 }
+// Conv positional encoding (at_peg_fwd, src/attn.h:141-144, src/nn_attn.cu:688-705): y = x + b + depthwise 3^3 conv of x over the grid tokens of a
+// sequence (zero padding: taps outside the grid add nothing), register rows copied. w [C][27] with the taps in (dz, dy, dx) order, b [C].
+// A thread takes one token's four neighbouring channels; each channel's sum starts from x + b and takes its taps in that order, one fused
+// multiply-add each, as the reference's contracted loop.
+__global__ void __launch_bounds__(256) peg_rows_k(const float *__restrict__ x, float *__restrict__ y, const float *__restrict__ w, const float *__restrict__ b,
+                                                  size_t n4, int S, int D, int Hh, int W, int nreg, int C4) {
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (i >= n4) return;
+    const size_t t = i / C4; const int c4 = (int)(i - t * C4), ts = (int)(t % S) - nreg;
+    const float4 xv = ((const float4 *)x)[i];
+    if (ts < 0) { ((float4 *)y)[i] = xv; return; }
+    const size_t row0 = t - (size_t)ts;                            // the sequence's first grid token
+    const int z = ts / (Hh * W), yy = (ts / W) % Hh, xx = ts % W;
+    const float4 bv = ((const float4 *)b)[c4];
+    float a[4] = {xv.x + bv.x, xv.y + bv.y, xv.z + bv.z, xv.w + bv.w};
+    const float *wc = w + (size_t)c4 * 4 * 27;
+    for (int dz = -1; dz <= 1; dz++) for (int dy = -1; dy <= 1; dy++) for (int dx = -1; dx <= 1; dx++) {
+        const int zz = z + dz, y2 = yy + dy, x2 = xx + dx;
+        if (zz < 0 || zz >= D || y2 < 0 || y2 >= Hh || x2 < 0 || x2 >= W) continue;
+        const float4 nv = ((const float4 *)x)[(row0 + ((size_t)zz * Hh + y2) * W + x2) * C4 + c4];
+        const int tap = (dz + 1) * 9 + (dy + 1) * 3 + dx + 1;
+        a[0] = fmaf(wc[tap], nv.x, a[0]); a[1] = fmaf(wc[27 + tap], nv.y, a[1]); a[2] = fmaf(wc[54 + tap], nv.z, a[2]); a[3] = fmaf(wc[81 + tap], nv.w, a[3]);
+    }
+    ((float4 *)y)[i] = make_float4(a[0], a[1], a[2], a[3]);
+}
+extern "C" void at_peg_fwd(const float *x, float *y, const float *w, const float *b, const at_geom *g, int nreg, int C) {
+    if (C % 4 || x == y || (long)g->D * g->Hh * g->W + nreg != g->S) mi_die("at_peg_fwd: C %d (a multiple of 4), separate buffers, S %d = nreg %d + %d x %d x %d", C, g->S, nreg, g->D, g->Hh, g->W);
+    const size_t n4 = (size_t)g->nseq * g->S * C / 4;
+    if (!n4) return;
+    peg_rows_k<<<nblk_(n4, 256), 256>>>(x, y, w, b, n4, g->S, g->D, g->Hh, g->W, nreg, C / 4); MICK();
+}
 // Value residual (at_ws.vr, src/nn_attn.cu:535-542, :609-610) on the V third of the qkv rows [T][3 C]: the first block of a stage (vr 1) keeps its
 // V in v1; a later one (vr 2) replaces its own V by v + lam[head] (v1 - v), one fused multiply-add, and keeps the own V when a buffer is given.
 __global__ void __launch_bounds__(256) v_keep_k(const float *__restrict__ qkv, float *__restrict__ v1, size_t n4, int C4) {

@@ -54,6 +54,7 @@ struct unet {
     /* the attention stage on the bottleneck (src/unet.c:470-509 set-up, :2795-2835 forward) */
     int tbn; at_dims tbd; at_bp tbp[16]; size_t reg_off; at_geom tbg; at_ws tbw;
     block tb;                                                      /* its output: a2 and the statistics m2 / r2 (the level's n2 affine) */
+    size_t peg_w, peg_b;                                           /* cfg.attn_pe 0: the conv positional encoding's parameters */
     float *tb_vr; size_t vr_off;                                   /* cfg.attn_vres (src/unet.h:81): the first application's V rows; the lerps' offset */
     float *tb_cs, *tb_tok; void *tb_ws;                            /* fp32 planes [n][C][Sg]; token rows, one buffer per block + 1; block scratch */
 };
@@ -162,12 +163,13 @@ unet *unet_create(const unet_cfg *cfg) {
     for (int j = 1; j <= cfg->ds_levels; j++) off = add_conv(&u->ds[j], dw_of(cfg, j), cfg->cout, 1, off);
     if (cfg->attn_blocks > 0) {                                   /* parameters last: registers, then the blocks (src/unet.c:490-499) */
         const int C = w[L - 1];
-        if (C % AT_HD || cfg->attn_blocks > 16 || (cfg->attn_pe != 1 && cfg->attn_pe != 2) || cfg->attn_reg < 0) {
-            fprintf(stderr, "unet_create: attention blocks need a bottleneck width that is a multiple of %d (got %d), at most 16 blocks, attn_pe 1 (RoPE) or 2 (none)\n", AT_HD, C);
+        if (C % AT_HD || cfg->attn_blocks > 16 || cfg->attn_pe < 0 || cfg->attn_pe > 2 || cfg->attn_reg < 0) {
+            fprintf(stderr, "unet_create: attention blocks need a bottleneck width that is a multiple of %d (got %d), at most 16 blocks, attn_pe 0 (PEG), 1 (RoPE) or 2 (none)\n", AT_HD, C);
             free(u); return nullptr;
         }
         const int F = cfg->attn_mlp > 0 ? cfg->attn_mlp : (8 * C / 3 + 31) / 32 * 32;
         u->tbd = (at_dims){.C = C, .H = C / AT_HD, .F = F, .rope = cfg->attn_pe == 1 ? 1 : 0, .nreg = cfg->attn_reg, .rope_base = 100.f};
+        if (cfg->attn_pe == 0) { u->peg_w = off; off += (size_t)C * 27; u->peg_b = off; off += (size_t)C; }      /* the conv positional encoding's depthwise taps and bias, before the registers (src/unet.c:491) */
         u->reg_off = off; off += (size_t)cfg->attn_reg * C;
         for (int k = 0; k < cfg->attn_blocks; k++) off = at_block_layout(&u->tbd, &u->tbp[k], off);
         u->tbn = cfg->attn_blocks;
@@ -519,6 +521,7 @@ static int tb_fwd(unet *u) {
     lp_mx_gemm_bmemo(1);                                           /* inference: the linears' weights are packed once (dropped when the weights change) */
     const int tba = u->tbn * (u->cfg.attn_repeat > 1 ? u->cfg.attn_repeat : 1);      /* application k runs block k % tbn (cfg.attn_repeat, src/unet.c:2816) */
     float *tin = u->tb_tok;
+    if (u->cfg.attn_pe == 0) { at_peg_fwd(tin, u->tb_tok + 2 * TC, P(u, u->peg_w), P(u, u->peg_b), &u->tbg, nr, C); tin = u->tb_tok + 2 * TC; }      /* (src/unet.c:2805; the first block writes the other buffer) */
     for (int k = 0; k < tba; k++) {
         float *tout = u->tb_tok + (size_t)(1 + (k & 1)) * TC;
         if (u->tb_vr) { u->tbw.vr = k ? 2 : 1; u->tbw.v1 = u->tb_vr; u->tbw.own = nullptr; u->tbw.lam = P(u, u->vr_off + (size_t)(k % u->tbn) * (size_t)u->tbd.H); }      /* (tb_vr_set, src/unet.c:2699-2704) */
@@ -701,7 +704,7 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
         if ((q = strstr(line, "\"ge_run\":["))) { q += 10; while (l0->gcnt < 8192 && *q && *q != ']') { char *e; l0->grun[l0->gcnt] = strtof(q, &e); if (e == q) break; l0->gcnt++; q = e; if (*q == ',') q++; } }
         if ((q = strstr(line, "\"l0_run\":["))) { q += 10; while (l0->cnt < 1024 && *q && *q != ']') { char *e; l0->run[l0->cnt] = strtof(q, &e); if (e == q) break; l0->cnt++; q = e; if (*q == ',') q++; } }
     }
-    if (!bad && cfg->attn_blocks && cfg->attn_pe != 1 && cfg->attn_pe != 2) bad = "\"attn_pe\": (PEG / scroll RoPE)";
+    if (!bad && cfg->attn_blocks && (cfg->attn_pe < 0 || cfg->attn_pe > 2)) bad = "\"attn_pe\": (scroll RoPE)";
     if (bad) { fprintf(stderr, "unet_peek: %s uses %s which this build does not run\n", path, bad); free(line); return -2; }
     free(line);
     return cfg->cin > 0 && cfg->cout > 0 ? 0 : -1;
@@ -720,6 +723,7 @@ int unet_load(unet *u, const char *path) {
     if (!bad && c.cin != m->cin) bad = "cin";
     if (!bad && c.cout != m->cout) bad = "cout";
     if (!bad && c.attn_blocks != m->attn_blocks) bad = "attn_blocks";
+    if (!bad && c.attn_blocks && c.attn_pe != m->attn_pe) bad = "attn_pe";      /* (RoPE and none have the same parameters and another function) */
     if (!bad && (c.attn_repeat > 1 ? c.attn_repeat : 1) != (m->attn_repeat > 1 ? m->attn_repeat : 1)) bad = "attn_repeat";
     if (!bad && (c.attn_vres != 0) != (m->attn_vres != 0)) bad = "attn_vres";
     if (!bad && c.down_norm != m->down_norm) bad = "down_norm";

@@ -153,6 +153,7 @@ _ATTN_PROTOS = {
     "at_glu_fwd": (None, [_P, _P, C.c_long, _I]),
     "at_fa_pack": (None, [_P, _P, _P, _P, _P, _P, _P, C.POINTER(at_geom), _I, _I, _I, _F]),
     "at_cs_to_tok": (None, [_P, _P, _P, _I, _I, C.c_long, _I]),
+    "at_peg_fwd": (None, [_P, _P, _P, _P, C.POINTER(at_geom), _I, _I]),
     "at_tok_to_cs": (None, [_P, _P, _I, _I, C.c_long, _I]),
     "at_block_fwd": (_I, [C.POINTER(at_dims), _P, C.POINTER(at_bp), _P, _P, C.POINTER(at_geom), C.POINTER(at_ws)]),
     "lp_mx_gemm": (_I, [_I, _I, _I, _I, _I, _I, _P, _P, _P, _F]),
