@@ -246,8 +246,8 @@ def test_checkpoint_round_trip(gpu, tmp_path):
     assert other.load(path) == -1
     open(str(tmp_path / "cut.ckpt"), "wb").write(open(path, "rb").read()[:-8])
     assert b.load(str(tmp_path / "cut.ckpt")) == -1
-    open(str(tmp_path / "film.ckpt"), "wb").write(head.replace(',"cin":', ',"film":2,"cin":').encode() + b"\0" * (8 * pa.size))
-    assert H_.unet_peek(str(tmp_path / "film.ckpt").encode(), C.byref(c2), None) == -2
+    open(str(tmp_path / "fstem.ckpt"), "wb").write(head.replace(',"cin":', ',"fstem":[2,16],"cin":').encode() + b"\0" * (8 * pa.size))
+    assert H_.unet_peek(str(tmp_path / "fstem.ckpt").encode(), C.byref(c2), None) == -2
     # the EMA copy (src/unet.h:258): a file whose second array differs loads into the EMA weights, which unet_use_ema switches the forward to
     raw = open(path, "rb").read(); hl = len(head.encode())
     ema = (pa * np.float32(0.5)).astype(np.float32)
@@ -305,7 +305,7 @@ def test_reference_signature_forwards(gpu):
     LP.check()
     assert np.array_equal(got, want)
     # a configuration field this build does not run is refused by name, not ignored
-    bad = make_cfg(4, [32, 64]); bad.film = 2
+    bad = make_cfg(4, [32, 64]); bad.fstem = 2
     assert not H_.unet_create(C.byref(bad))
     net.close()
 
