@@ -3,8 +3,8 @@
 
 value / ms_per_step (BASELINE.json configs[3], the metric's "U-Net infer voxels/s (128^3 patch, MX fp8)"): one forward of the reference-style
 U-Net (cin 4, widths 32/64/128/256, two 3x3x3 convs + GroupNorm + SiLU per level, 3x3x3 stride-2 downs, trilinear 2x fused into the decoder
-convs, skip concat, 1x1x1 head of 8 logits) over N 2 x 128^3 voxels, MX-fp8 storage and compute, the quantised input resident in HBM. A step =
-one forward; the prepared (quantised, re-laid-out) weights are memoised across forwards as an inference loop keeps them - the reference's
+convs, skip concat, 1x1x1 head of 8 logits) over N 2 x 128^3 voxels, MX-fp8 storage and compute. A step = unet_forward_ct on the two uint8 CT
+windows resident in HBM: the network input is built on the device inside the timed region (lp_pred_input_mx), then the graph runs; the prepared (quantised, re-laid-out) weights are memoised across forwards as an inference loop keeps them - the reference's
 fp8 path re-quantises them per call (src/lp_f8fwd.cu:54-71; about 15 us per layer here). `roofline`: the forward's dominant kernel (most
 total time among its conv launches, HIP events around every launch on its stream).
 conv_stack (configs[1], the metric's "3x3x3 conv % of MFMA peak"): four 3x3x3 convs 128 -> 128, N 2, 64^3, MX-fp8, bias + GroupNorm(8)
@@ -21,17 +21,30 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 METRIC = "U-Net infer voxels/s (128^3 patch, MX fp8) + 3x3x3 conv % of MFMA peak"
-TRAFFIC_BYTES_PER_LAUNCH = 183.9e6     # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, see profiles/
-# HBM bytes per launch of the U-Net's dominant conv from committed counter runs: layer -> (bytes, source); absent: not measured
-KERNEL_TRAFFIC = {"dec0.c1": (809.1e6, "profiles/conv3_row_f8_c96to32_128cube_counters.txt (the same kernel and tensor sizes on a one-segment 96-channel input)")}
 MFMA_PEAK_FP8_TFLOPS = 5033.0          # MI355X dense MXFP8 (2.5 PFLOP/s bf16 x 2)
+MFMA_PEAK_FP4_TFLOPS = 10066.0         # dense MXFP4
+# HBM bytes per launch of a kernel cannot be measured from inside the process: they come from the committed rocprofv3 --pmc runs of this very
+# command (FETCH_SIZE, then WRITE_SIZE, scaled by a copy of known size), each summary carrying one line "traffic_bytes_per_launch: <bytes>"
+TRAFFIC_PROFILES = {"dec0.c1": "profiles/conv3_row_f8_unet_dec0c1_hbm_traffic.txt", "conv_stack": "profiles/conv3_mx_f8_c128_64cube_hbm_traffic.txt"}
+
+
+def profile_traffic(key):
+    """(bytes per launch, source file) from the committed counter summary of a kernel, or (None, None) when there is none."""
+    import re
+    rel = TRAFFIC_PROFILES.get(key)
+    path = os.path.join(ROOT, rel) if rel else None
+    if not path or not os.path.exists(path):
+        return None, None
+    m = re.search(r"^traffic_bytes_per_launch:\s*([0-9.eE+]+)", open(path).read(), re.M)
+    return (float(m.group(1)), rel) if m else (None, None)
 
 
 def unet_leg(np, lib, LP, DevBuf, steps, warmup):
     """configs[3]: the reference-style U-Net forward (cin 4, widths 32/64/128/256, two 3x3x3 convs + GroupNorm + SiLU per level, 3x3x3 stride-2
     downs, trilinear 2x fused into the decoder convs, skip concat, 1x1x1 head of 8 logits), N 2 x 128^3, MX-fp8 storage and compute, random
-    init, CT-like synthetic input already quantised and resident in HBM. Two timed passes: the forwards alone (wall clock: `value`), then the
-    same number of forwards with an event pair around every conv launch (per-kernel times for the roofline; the events cost a little)."""
+    init, CT-like synthetic uint8 windows resident in HBM, the 4-channel MX input built on the device by every forward (unet_forward_ct, as the
+    reference's predict does per window). Two timed passes: the forwards alone (wall clock: `value`), then the same number of forwards with an
+    event pair around every conv launch (per-kernel times for the roofline; the events cost a little)."""
     from ufsm_amd.unet import UNet, make_cfg
     N, D, widths = 2, 128, [32, 64, 128, 256]
     S = D ** 3
@@ -41,26 +54,31 @@ def unet_leg(np, lib, LP, DevBuf, steps, warmup):
     for ax in (1, 2, 3):
         f = (np.roll(f, 1, ax) + f + np.roll(f, -1, ax)) / 3                      # smoothed field -> sheet structure
     sheet = np.sin(6 * f / f.std() + np.linspace(0, 8, D, dtype=np.float32)[None, None, None, :]) > 0
-    ct = np.clip(np.where(sheet, rng.normal(170, 20, f.shape), rng.normal(60, 20, f.shape)), 0, 255).astype(np.uint8).astype(np.float32)
-    x = np.zeros((N, 4, S), np.float32)
-    x[:, 0] = ((ct - ct.mean()) / ct.std()).reshape(N, S)
-    yy, xx = np.meshgrid(np.arange(D) - 300.0, np.arange(D) + 200.0, indexing="ij")
-    r = np.sqrt(yy * yy + xx * xx) + 1e-6
-    x[:, 2] = np.broadcast_to((yy / r)[None], (D, D, D)).reshape(1, S); x[:, 3] = np.broadcast_to((xx / r)[None], (D, D, D)).reshape(1, S)
-    dx = DevBuf.from_numpy(x)
-    dxq = DevBuf(lib.lp_mx8_bytes(N, 4, S)); lib.lp_f32_to_mx8(dx.ptr, N, 4, S, dxq.ptr)
+    ct = np.clip(np.where(sheet, rng.normal(170, 20, f.shape), rng.normal(60, 20, f.shape)), 0, 255).astype(np.uint8)
+    mean, isd = float(ct.mean()), float(1.0 / ct.std())
+    dct = DevBuf.from_numpy(ct)                                                       # [N][D][H][W] uint8, the two windows back to back
+    # per window plane the row / column offset from the scroll axis (an axis outside the window, as in a scroll volume)
+    dyo = DevBuf.from_numpy(np.full(N * D, -300.0, np.float32)); dxo = DevBuf.from_numpy(np.full(N * D, 200.0, np.float32))
+    H_ = net.L
+    xs5 = net.shape
+
+    def fwd():
+        net._mode()
+        p = H_.unet_forward_ct(net.h, dct.ptr, mean, isd, dyo.ptr, dxo.ptr, 1, xs5, 2)
+        net._unmode()
+        return p
     for _ in range(warmup):
-        assert net.forward_mx(dxq.ptr)
+        assert fwd()
     lib.mi_sync(); LP.check()
     t0 = time.perf_counter()
     for _ in range(steps):
-        net.forward_mx(dxq.ptr)                                                     # (the logits stay in the net's own device buffer)
+        fwd()                                                                       # (the logits stay in the net's own device buffer)
     lib.mi_sync(); LP.check()
     dt = (time.perf_counter() - t0) / steps
     # per-kernel: every conv launch of `steps` more forwards, grouped by kernel variant and layer position within the forward
     lib.mi_kernel_timing(1)
     for _ in range(steps):
-        net.forward_mx(dxq.ptr)
+        fwd()
     lib.mi_sync()
     nlog = lib.mi_kernel_timing_launch(-1, None, None, None, 0)
     per_fwd = nlog // steps
@@ -90,9 +108,104 @@ def unet_leg(np, lib, LP, DevBuf, steps, warmup):
     fl *= N
     net.close()
     dom = max(convs, key=lambda c: c["avg_launch_ms"])
-    return {"workload": "configs[3]: U-Net forward, N 2 x 128^3, widths 32/64/128/256, MX-fp8", "value": N * S / dt, "unit": "voxels/s", "ms_per_forward": dt * 1e3,
+    return {"workload": "configs[3]: U-Net forward from two uint8 CT windows in HBM (unet_forward_ct: input rows built on the device, then the graph), N 2 x 128^3, widths 32/64/128/256, MX-fp8", "value": N * S / dt, "unit": "voxels/s", "ms_per_forward": dt * 1e3,
             "steps": steps, "gflop_per_forward": fl / 1e9, "tflops": fl / dt / 1e12, "conv_launches": convs,
             "conv_ms_per_forward": sum(c["avg_launch_ms"] for c in convs)}, dom
+
+
+def _time_calls(lib, LP, call, steps, warmup):
+    """(wall ms per call, HIP-event ms per conv launch, kernel name) of `call` repeated back to back."""
+    for _ in range(warmup):
+        call()
+    lib.mi_sync(); LP.check()
+    lib.mi_kernel_timing(1)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        call()
+    lib.mi_sync()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    nl = C.c_long(0)
+    kms = lib.mi_kernel_timing_read(C.byref(nl)) / max(nl.value, 1)
+    lib.mi_kernel_timing(0); LP.check()
+    return wall, kms, lib.mi_last_kernel().decode(), int(nl.value)
+
+
+def c0_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, steps, warmup):
+    """configs[0]: one 3x3x3 conv 32 -> 32, N 1, 64^3, seed 0: activations N(0,1) as fp32 planes quantised to MX-fp8 while staging (bit for bit
+    lp_f32_to_mx8), Kaiming weights in MX-fp8 blocks of 32 input channels, fp32 accumulate, fp16 planes out, through lp_conv_fwd_f8. The
+    case sits at the ridge, so it reports both the MFMA fraction of the conv kernel and the HBM rate of the whole call (quantising
+    pre-pass + conv; algorithmic bytes: the fp32 planes in, the fp16 planes out, the prepared weights)."""
+    N, Cc, D = 1, 32, 64
+    S = D ** 3
+    rng = np.random.default_rng(0)
+    dx = DevBuf.from_numpy(rng.standard_normal((N, Cc, S)).astype(np.float32))
+    dw = DevBuf.from_numpy((rng.standard_normal((Cc, Cc, 27)) * np.sqrt(2.0 / (Cc * 27))).astype(np.float32))
+    dy = DevBuf(N * Cc * S * 2)
+    sp = split_t(); sp.wkey = 300
+    xs = shape5(N, Cc, D, D, D)
+    wall, kms, kernel, nl = _time_calls(lib, LP, lambda: lib.lp_conv_fwd_f8(dx.ptr, 0, xs, dw.ptr, None, Cc, dy.ptr, 2, gnp_t(), None, 0, sp), steps, warmup)
+    fl = 2.0 * 27 * Cc * Cc * N * S
+    nbytes = N * Cc * S * 4 + N * Cc * S * 2 + 28 * Cc * Cc * 33 // 32
+    lib.lp_wmemo_clear()
+    return {"workload": "configs[0]: 3x3x3 conv 32 -> 32, N 1, 64^3, fp32 planes in (quantised to MX-fp8 E4M3 per 32 channels while staging), fp16 planes out, seed 0",
+            "entry": "lp_conv_fwd_f8(x dtype 0, y dtype 2)", "kernel": kernel, "ms_per_call": wall, "conv_kernel_ms": kms, "gflop": fl / 1e9,
+            "tflops_conv_kernel": fl / kms / 1e9, "frac_of_mxfp8_peak": fl / kms / 1e9 / MFMA_PEAK_FP8_TFLOPS,
+            "algorithmic_bytes": nbytes, "GBps_whole_call": nbytes / wall / 1e6, "frac_of_hbm_peak": nbytes / wall / 1e6 / 8000.0}
+
+
+def c2a_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, steps, warmup):
+    """configs[2], the 3x3x3 part: MX-fp4 E2M1 conv 256 -> 256, N 2, 32^3, inputs uniform[-3, 3], Kaiming weights, 32-element E8M0 blocks, fp32
+    accumulate, MX-fp4 in and out, fused GroupNorm(8) statistics, through lp_conv_fwd_f4; roofline against the dense MXFP4 peak."""
+    N, Cc, D, G = 2, 256, 32, 8
+    S = D ** 3
+    rng = np.random.default_rng(0)
+    dx = DevBuf.from_numpy(rng.uniform(-3, 3, (N, Cc, S)).astype(np.float32))
+    dxq = DevBuf(lib.lp_mx4_bytes(N, Cc, S)); lib.lp_f32_to_mx4(dx.ptr, N, Cc, S, dxq.ptr)
+    dw = DevBuf.from_numpy((rng.standard_normal((Cc, Cc, 27)) * np.sqrt(2.0 / (Cc * 27))).astype(np.float32))
+    db = DevBuf.from_numpy((rng.standard_normal(Cc) * 0.1).astype(np.float32))
+    dy = DevBuf(lib.lp_mx4_bytes(N, Cc, S)); dsum = DevBuf(N * G * 2 * 24)
+    sp = split_t(); sp.wkey = 301
+    xs = shape5(N, Cc, D, D, D)
+    wall, kms, kernel, nl = _time_calls(lib, LP, lambda: lib.lp_conv_fwd_f4(dxq.ptr, 4, xs, dw.ptr, db.ptr, Cc, dy.ptr, 4, gnp_t(), dsum.ptr, G, sp), steps, warmup)
+    fl = 2.0 * 27 * Cc * Cc * N * S
+    lib.lp_wmemo_clear()
+    return {"workload": "configs[2]: MX-fp4 E2M1 3x3x3 conv 256 -> 256, N 2, 32^3, MX-fp4 in / out, GroupNorm(8) statistics fused, inputs uniform[-3, 3]",
+            "entry": "lp_conv_fwd_f4", "ms_per_call": wall,
+            "roofline": {"bound": "mfma", "kernel": kernel, "achieved": fl / kms / 1e9, "peak": MFMA_PEAK_FP4_TFLOPS, "unit": "TFLOP/s", "frac": fl / kms / 1e9 / MFMA_PEAK_FP4_TFLOPS,
+                         "launches": nl, "avg_launch_ms": kms, "flops_per_launch": fl, "algorithmic_bytes": 2 * N * (Cc // 32) * S * 17 + 28 * Cc * Cc * 17 // 32, "traffic": None}}
+
+
+def stack_fused_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, steps, warmup):
+    """configs[1] to the letter: 4 x (3x3x3 conv 128 -> 128, N 2, 64^3, MX-fp8 in / out) with bias + GroupNorm(8) affine + GELU + MX-fp8
+    re-quantisation fused into each conv's epilogue (mi_conv_fwd_fused). A GroupNorm inside the producer's epilogue needs its statistics before
+    the conv has run, so they are frozen (per (sample, group) mean / rstd fixed beforehand, as the reference's unet_gn_freeze inference mode)
+    and enter as the per-channel affine a = rstd gamma, b = beta - mean a."""
+    N, Cc, D, L = 2, 128, 64, 4
+    S = D * D * D
+    rng = np.random.default_rng(0)
+    dx = DevBuf.from_numpy(rng.standard_normal((N, Cc, S)).astype(np.float32))
+    x0 = DevBuf(lib.lp_mx8_bytes(N, Cc, S)); lib.lp_f32_to_mx8(dx.ptr, N, Cc, S, x0.ptr)
+    act = [DevBuf(lib.lp_mx8_bytes(N, Cc, S)) for _ in range(2)]
+    ws = [DevBuf.from_numpy((rng.standard_normal((Cc, Cc, 27)) * np.sqrt(2.0 / (Cc * 27))).astype(np.float32)) for _ in range(L)]
+    bs = [DevBuf.from_numpy((rng.standard_normal(Cc) * 0.1).astype(np.float32)) for _ in range(L)]
+    ea = [DevBuf.from_numpy(rng.uniform(0.8, 1.25, Cc).astype(np.float32)) for _ in range(L)]        # rstd[g] gamma[c] of the frozen statistics
+    eb = [DevBuf.from_numpy(rng.uniform(-0.1, 0.1, Cc).astype(np.float32)) for _ in range(L)]
+    xs = shape5(N, Cc, D, D, D)
+
+    def step():
+        src = x0
+        for l in range(L):
+            dst = act[l & 1]
+            sp = split_t(); sp.wkey = 310 + l
+            lib.mi_conv_fwd_fused(8, src.ptr, 3, xs, ws[l].ptr, bs[l].ptr, Cc, dst.ptr, 3, ea[l].ptr, eb[l].ptr, 2, gnp_t(), None, 0, sp)
+            src = dst
+    wall, kms, kernel, nl = _time_calls(lib, LP, step, steps, warmup)
+    fl = 2.0 * 27 * Cc * Cc * N * S
+    lib.lp_wmemo_clear()
+    return {"workload": "configs[1] to the letter: 4 x (3x3x3 conv 128->128, N 2, 64^3, MX-fp8) with bias + frozen-statistics GroupNorm(8) affine + GELU + MX-fp8 requant in the conv epilogue",
+            "entry": "mi_conv_fwd_fused(act 2)", "value": N * S / (wall * 1e-3), "unit": "voxels/s", "ms_per_step": wall, "tflops": L * fl / wall / 1e9,
+            "roofline": {"bound": "mfma", "kernel": kernel, "achieved": fl / kms / 1e9, "peak": MFMA_PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": fl / kms / 1e9 / MFMA_PEAK_FP8_TFLOPS,
+                         "launches": nl, "avg_launch_ms": kms, "flops_per_launch": fl, "algorithmic_bytes": 2 * N * (Cc // 32) * S * 33 + 28 * Cc * Cc * 33 // 32, "traffic": None}}
 
 
 def hbm_leg(np, lib, LP, DevBuf):
@@ -197,6 +310,8 @@ def main():
     ap.add_argument("--no-stack", action="store_true", help="skip the configs[1] conv-stack leg")
     ap.add_argument("--no-sliding", action="store_true", help="skip the configs[4]-geometry sliding-window leg")
     ap.add_argument("--no-hbm", action="store_true", help="skip the HBM-bound kernels leg")
+    ap.add_argument("--no-single", action="store_true", help="skip the single-conv legs (configs[0], the MX-fp4 3x3x3 conv of configs[2])")
+    ap.add_argument("--unet-only", action="store_true", help="the U-Net leg alone (what the rocprofv3 runs of the forward's kernels use)")
     ap.add_argument("--windows-per-forward", type=int, default=8, help="sliding-window leg: windows batched into one forward")
     ap.add_argument("--copy-probe", action="store_true", help="run 5 device-to-device copies of 1 GiB and exit: the known-size kernel that scales "
                     "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -245,21 +360,27 @@ def main():
                           "tflops": fl / ms / 1e9, "frac_of_mfma_peak": fl / ms / 1e9 / peak,
                           "algorithmic_bytes": int(mxb(N, Ci, S) + mxb(N, Co, S)), "GBps": (mxb(N, Ci, S) + mxb(N, Co, S)) / ms / 1e6}))
         return
+    if a.unet_only:
+        a.no_stack = a.no_sliding = a.no_hbm = a.no_single = a.no_cpu_baseline = True
     out = {"metric": METRIC, "unit": "voxels/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
            "dtype": "mxfp8 (e4m3 x e4m3 block-scaled, fp32 accumulate)", "data": "synthetic",
            "weights": "prepared (quantised, re-laid-out) once and memoised across the timed forwards, as an inference loop keeps them"}
     u, dom = unet_leg(np, lib, LP, DevBuf, a.steps, a.warmup)
     out["value"] = u["value"]; out["ms_per_step"] = u["ms_per_forward"]; out["tflops"] = u["tflops"]
     out["config"] = {"workload": u["workload"], "batch": 2, "dims": [128, 128, 128], "widths": [32, 64, 128, 256], "cin": 4, "head_out": 8, "gflop_per_forward": u["gflop_per_forward"]}
-    prof = KERNEL_TRAFFIC.get(dom["layer"])
+    prof = profile_traffic(dom["layer"])
     out["roofline"] = {"bound": "mfma", "kernel": "%s (%s)" % (dom["kernel"], dom["layer"]), "achieved": dom["tflops"], "peak": MFMA_PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
                        "frac": dom["frac_of_mxfp8_peak"], "avg_launch_ms": dom["avg_launch_ms"], "launches": a.steps, "flops_per_launch": dom["flops_per_launch"],
-                       "traffic": prof[0] if prof else None, "traffic_source": prof[1] if prof else None}
+                       "traffic": prof[0], "traffic_source": prof[1]}
     out["unet"] = u
     stack = None
     if not a.no_stack:
         stack, xq0, w_host_l0 = stack_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, max(a.steps, 20), max(a.warmup, 5))
         out["conv_stack"] = stack
+        out["conv_stack_fused"] = stack_fused_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, max(a.steps, 20), max(a.warmup, 5))
+    if not a.no_single:
+        out["c0"] = c0_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, max(a.steps, 20) * 5, max(a.warmup, 5) * 2)
+        out["c2a"] = c2a_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, max(a.steps, 20) * 5, max(a.warmup, 5) * 2)
     if not a.no_sliding:
         out["sliding_window"] = sliding_leg(np, lib, LP, DevBuf, a.windows_per_forward)
     if not a.no_hbm:
@@ -337,9 +458,7 @@ def stack_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, steps, warmup):
            "value": N * S / (ms_step * 1e-3), "unit": "voxels/s", "ms_per_step": ms_step, "steps": steps, "warmup": warmup, "tflops": L * flops_layer / (ms_step * 1e-3) / 1e12,
            "roofline": {"bound": "mfma", "kernel": kernel, "achieved": achieved, "peak": MFMA_PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_PEAK_FP8_TFLOPS,
                         "launches": nl.value, "avg_launch_ms": k_ms, "flops_per_launch": flops_layer,
-                        # HBM-side bytes per launch: not measurable from inside the process; the figure of the committed counter runs
-                        # (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000, factors from a 1 GiB copy) for this kernel at this shape
-                        "traffic": TRAFFIC_BYTES_PER_LAUNCH, "traffic_source": "profiles/conv3_mx_f8_c128_64cube_hbm_traffic.txt",
+                        "traffic": profile_traffic("conv_stack")[0], "traffic_source": profile_traffic("conv_stack")[1],
                         "algorithmic_bytes": 2 * N * (Cc // 32) * S * 33 + 28 * Cc * Cc * 33 // 32}}
     return rec, x0.to_numpy(np.uint8), w
 

@@ -184,17 +184,25 @@ double mi_kernel_timing_read(long *launches);
 /* launch i of the log kept since mi_kernel_timing(1), in launch order: its milliseconds, its algorithmic FLOPs (2 x 27 x Cin x Cout x output
    voxels, logical channels) and its kernel variant's name; returns the number of launches logged (synchronises) */
 long mi_kernel_timing_launch(long i, float *ms, double *flops, char *name, size_t name_bytes);
-/* No counterpart in the reference. lp_conv_fwd_f8 / lp_conv_fwd_f4 (bits 8 / 4) for callers that cannot allocate device memory: code under
-   HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. Same arguments, same kernels and bit-identical results, but every
-   byte of scratch (prepared weights, re-staged operands, statistics partials, the constant page) comes from one fixed device array of
-   mi_conv_static_scratch_bytes() = 64 MiB that each GPU the library runs on holds until the process ends; the call makes no hipMalloc /
-   hipFree (split_t.wkey is ignored: weights are prepared per call). A call whose scratch could exceed the array prints what it needs and
-   returns -1 with nothing launched (an input already in the compute format without GroupNorm needs only its weights: any size fits;
-   with GroupNorm or another storage format the re-staged operand must fit: e.g. 128 channels at 2 x 32^3). Calls on one GPU share the
-   array: calls that overlap on a GPU (two host threads, two streams) race; nothing in it needs clearing between calls. */
+/* No counterpart in the reference. lp_conv_fwd_f8 / lp_conv_fwd_f4 (bits 8 / 4) for callers that cannot allocate device memory: tight serving
+   loops, harnesses that forbid hipMalloc. Same arguments, same kernels and bit-identical results, but every byte of scratch (prepared weights,
+   re-staged operands, statistics partials, the constant page) comes from one fixed device array of mi_conv_static_scratch_bytes() = 64 MiB that
+   each GPU the library runs on holds until the process ends; the call makes no hipMalloc / hipFree (split_t.wkey is ignored: weights are
+   prepared per call). mi_init addresses the array on the device it selects and writes its 128-byte constant page (one synchronous copy); on a
+   device nobody passed to mi_init the first call does that itself. Like every entry of this library it launches on the null stream, so it
+   cannot be recorded into a HIP graph by stream capture. A call whose scratch could exceed the array prints what it needs and returns -1 with
+   nothing launched (an input already in the compute format without GroupNorm, or a network input of few channels on the tap-packed kernels,
+   needs only its weights: any size fits; with GroupNorm or another storage format the re-staged operand must fit: e.g. 128 channels at
+   2 x 32^3). Calls on one GPU share the array: calls that overlap on a GPU (two host threads, two streams) race; nothing in it needs clearing
+   between calls. */
 int mi_conv_fwd_static(int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp);
 size_t mi_conv_static_scratch_bytes(void);
 long mi_alloc_count(void);                     /* device allocations made by this library so far (scratch growth, memo entries, mi_malloc): diagnostics */
+/* Every fp32 bit pattern through the hardware encoder (bits 8: v_cvt_scalef32_pk_fp8_f32, 4: v_cvt_scalef32_pk_fp4_f32) at block exponent e
+   against the software encoder of x 2^-e (the reference checks its conversion instruction the same way, src/lp_mxsw.cu:45-61). out[0]: inputs
+   inside the domain the kernels use the instruction on (e4m3: |x 2^-e| <= 464 and not NaN; e2m1: not NaN), out[1]: mismatches among them (0
+   expected), out[2] / out[3]: inputs outside it and their mismatches (those blocks take the software encoder). Synchronises. 0, or -1 for bad arguments */
+int mi_cvt_sweep(int bits, int e, unsigned long long out[4]);
 /* name of the conv kernel variant the last conv call on this thread launched (diagnostics / tests), "" if none */
 const char *mi_last_kernel(void);
 #ifdef __cplusplus

@@ -1,6 +1,6 @@
 /* Host side (C23) of the MX U-Net forward: the op layer and the graph the reference keeps above its lp_* kernels, restated over
  * the C ABI of include/mi_lp.h. Names, argument meaning and error behaviour follow the reference's own declarations:
- *   nn_set_storage / nn_storage / nn_set_prec / nn_conv3d_fwd_gn_stats / nn_conv3d_fwd_x / nn_gn_stats   src/nn.h:100, :194-195, :423-433, :484
+ *   nn_set_storage / nn_storage / nn_set_prec / nn_conv3d_fwd / _gn / _gn_stats / _split / _x / nn_gn_stats   src/nn.h:100, :194-195, :399-400, :416, :423-433, :442, :484
  *   unet_cfg / unet_create / unet_init / unet_forward_x / unet_forward_ct                               src/unet.h:18-128, :141, :176, :186, :428
  * Tensors are device pointers; an activation is an MX tensor registered with nn_set_storage (dt 8 / 4), as in the reference.
  */
@@ -16,7 +16,8 @@ extern "C" {
 void nn_set_storage(const void *p, size_t bytes, int dt);      /* dt 8 MX-fp8, 4 MX-fp4, 2 fp16 planes, 0 forgets (fp32 planes) */
 int nn_storage(const void *p);                                 /* the dt of the registered range holding p, else 0 */
 void nn_storage_forget(const void *p);
-void nn_set_prec(int p);                                       /* 3: MX-fp4 compute for every conv, else the storage decides (src/nn.h:100, src/nn_bwd.cu:110-112) */
+void nn_set_prec(int p);                                       /* 3: MX-fp4 compute for every conv, else the storage decides; on tensors without MX storage 2 / 3 run the
+                                                                  fp8 / fp4 entry on the planes as they are (src/nn.h:100, src/nn_bwd.cu:97-119) */
 int nn_get_prec(void);                                         /* src/nn.h:115 */
 void nn_set_gn_stored(int on);                                 /* GroupNorm statistics of the decoded stored output (src/nn_core.cu:7; default 0) */
 size_t nn_mx8_bytes(shape5 s);
@@ -25,6 +26,18 @@ typedef struct { const float *gamma, *beta, *mean, *rstd; int G; } nn_gn_t;     
 /* y = conv3(silu(gn(x))) (G_in 0: x as is) with the GroupNorm statistics of y for G_out groups written to omean / orstd (src/nn.h:423) */
 int nn_conv3d_fwd_gn_stats(const float *x, shape5 xs, int G_in, const float *gamma, const float *beta, const float *mean, const float *rstd,
                            const float *w, const float *b, int cout, float *y, int G_out, float eps, float *omean, float *orstd);
+/* The reference's other conv entries of this path, same names and signatures (src/nn.h:399-400, :416, :442). The kernel family follows its rule
+   (conv_fwd_tc, src/nn_bwd.cu:97-119): MX storage in means MX storage of the same format out; MX-fp4 storage or precision 3 runs the fp4 kernels,
+   everything else fp8; an input of <= 8 channels runs the tap-packed fp8 stem whatever the format; a combination with no kernel prints and
+   aborts. nn_conv3d_fwd: k 1 (the head of an MX tensor), k 3 stride 1 or 2, no GroupNorm. nn_conv3d_fwd_gn: the conv of silu(gn(x)).
+   nn_conv3d_fwd_split: the conv of the channel concat [x (c_split channels), x2] under one GroupNorm of G_in groups over all xs.c channels
+   (G_in 0: none), with the output's statistics for G_out groups. */
+shape5 nn_conv3d_out_shape(shape5 xs, int cout, int k, int stride);
+void nn_conv3d_fwd(const float *x, shape5 xs, const float *w, const float *b, int cout, int k, int stride, float *y);
+int nn_conv3d_fwd_gn(const float *x, shape5 xs, int G, const float *gamma, const float *beta, const float *mean, const float *rstd,
+                     const float *w, const float *b, int cout, float *y);
+int nn_conv3d_fwd_split(const float *x, const float *x2, int c_split, shape5 xs, int G_in, const float *gamma, const float *beta, const float *mean, const float *rstd,
+                        const float *w, const float *b, int cout, float *y, int G_out, float eps, float *omean, float *orstd);
 /* input-side recompute conv: k 3 stride 1 (split / fused upsample / output statistics), k 3 stride 2, k 1 head (src/nn.h:432) */
 int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn_gn_t *gx2, int c_split, int up, shape5 xs,
                     const float *w, const float *b, int cout, int k, int stride, float *y, int G_out, float eps, float *omean, float *orstd);

@@ -57,6 +57,7 @@ def test_host_library_exports_every_declared_symbol():
     H = unet.load_host()
     names = header_functions("mi_unet.h", ("nn_", "unet_", "mi_unet_"))
     assert "unet_forward_x" in names and "nn_conv3d_fwd_x" in names and "nn_set_storage" in names and "mi_unet_predict_volume" in names
+    assert {"nn_conv3d_fwd", "nn_conv3d_fwd_gn", "nn_conv3d_fwd_gn_stats", "nn_conv3d_fwd_split", "nn_conv3d_out_shape"} <= set(names)      # src/nn.h:399-400, :416, :423, :442
     for n in names:
         assert hasattr(H, n), "libufsm_host.so does not export %s" % n
     # unet_cfg as the reference lays it out (src/unet.h:18-128): 4-byte fields in its order, three arrays of UNET_MAXLEV ints, one of 16 bytes
@@ -80,6 +81,19 @@ def test_unet_header_matches_the_cited_reference_signatures():
                  "void unet_use_ema(unet *u, int on);", "int unet_save(const unet *u, const char *path, int step, const char *extra_json);", "int unet_load(unet *u, const char *path);",
                  "int unet_peek(const char *path, unet_cfg *cfg, int *step);", "void unet_set_act_mx8(int on);", "void unet_set_act_mx4(int on);", "void unet_set_infer_slab(int planes);", "void unet_set_slab_direct(int on);", "void unet_set_scale(unet *u, double um);", "void unet_set_cond(unet *u, float c);", "void unet_set_film(unet *u, const float *codes, int k);", "size_t unet_gfilm_off(const unet *u);",
                  "const unet_cfg *unet_cfg_of(const unet *u);", "float *unet_param_ptr(unet *u);", "void unet_init(unet *u, uint64_t seed);"]:
+        assert decl in flat, decl
+
+
+def test_op_layer_header_matches_the_cited_reference_signatures():
+    """The op layer's conv entries carry the reference's parameter lists (src/nn.h:399-400, :416, :423-424, :432-433, :442-443)."""
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "mi_unet.h")).read(), flags=re.S)
+    flat = re.sub(r"\s+", " ", text)
+    for decl in ["shape5 nn_conv3d_out_shape(shape5 xs, int cout, int k, int stride);",
+                 "void nn_conv3d_fwd(const float *x, shape5 xs, const float *w, const float *b, int cout, int k, int stride, float *y);",
+                 "int nn_conv3d_fwd_gn(const float *x, shape5 xs, int G, const float *gamma, const float *beta, const float *mean, const float *rstd, const float *w, const float *b, int cout, float *y);",
+                 "int nn_conv3d_fwd_gn_stats(const float *x, shape5 xs, int G_in, const float *gamma, const float *beta, const float *mean, const float *rstd, const float *w, const float *b, int cout, float *y, int G_out, float eps, float *omean, float *orstd);",
+                 "int nn_conv3d_fwd_split(const float *x, const float *x2, int c_split, shape5 xs, int G_in, const float *gamma, const float *beta, const float *mean, const float *rstd, const float *w, const float *b, int cout, float *y, int G_out, float eps, float *omean, float *orstd);",
+                 "int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn_gn_t *gx2, int c_split, int up, shape5 xs, const float *w, const float *b, int cout, int k, int stride, float *y, int G_out, float eps, float *omean, float *orstd);"]:
         assert decl in flat, decl
 
 

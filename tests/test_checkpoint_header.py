@@ -65,6 +65,16 @@ def test_refuses_architectures_it_does_not_run(tmp_path, feature):
     assert read(tmp_path, h)[0] == -2
 
 
+@pytest.mark.parametrize("keys", ['"sparse24":1,"wq":0', '"sparse24":3,"wq":0,"muon_mom":0,"sparse24_lv":6,"sparse24_hard":1', '"sparse24":0,"wq":4', '"sparse24":0,"wq":8'])
+def test_refuses_transformed_weight_storage(tmp_path, keys):
+    """2:4-masked or packed fp8 / fp4 weights: the reference applies the masks / packs the weights after reading the same fp32 payload
+    (src/unet.c:5703-5707, :5839-5840); loading the file as dense master weights would run another function, so it is refused by name."""
+    h = 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":336129,"step":1,%s,"extra":{}}\n' % keys
+    assert read(tmp_path, h)[0] == -2
+    h0 = 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":336129,"step":1,"sparse24":0,"wq":0,"extra":{}}\n'
+    assert read(tmp_path, h0)[0] == 0
+
+
 def test_reads_the_2d_weight_scale_key(tmp_path):
     h = 'UFSM{"nlev":2,"widths":[32,64],"w4_2d":1,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":3,"extra":{}}\n'
     rc, cfg, n, step = read(tmp_path, h)

@@ -213,6 +213,56 @@ def test_unet_attention_stage(gpu, rep):
     plain.close(); att.close()
 
 
+def test_unet_init_matches_the_published_generator(gpu):
+    """unet_init(u, seed) gives the reference's initial network for the same seed (src/unet.c:584-607): splitmix64, 53-bit uniforms, one
+    Box-Muller cosine value per pair of uniforms, consumed in parameter order, Kaiming std sqrt(2 / (cin 27)), biases 0, GroupNorm 1 / 0,
+    head bias -2. The generator is restated here from its published definition, independently of the C code."""
+    import math
+    from ufsm_amd.unet import UNet, make_cfg
+    M = (1 << 64) - 1
+
+    class Gen:
+        def __init__(self, seed):
+            self.s = seed
+
+        def u(self):
+            self.s = (self.s + 0x9E3779B97F4A7C15) & M
+            z = self.s
+            z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & M
+            z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & M
+            return ((z ^ (z >> 31)) >> 11) * 2.0 ** -53
+
+        def normal(self):
+            a = self.u() + 1e-300; b = self.u()
+            return math.sqrt(-2 * math.log(a)) * math.cos(6.283185307179586 * b)
+
+    cin, widths, seed = 4, [32, 64], 12345
+    net = UNet(make_cfg(cin, widths, head_out=3), 1, 8, 8, 8, seed=seed)
+    p = net.params()
+    net.close()
+    g = Gen(seed)
+    off = 0
+
+    def conv(ci, co, k, bias):
+        nonlocal off
+        n = co * ci * k ** 3; sd = math.sqrt(2.0 / (ci * k ** 3))
+        want = np.array([np.float32(sd * g.normal()) for _ in range(n)], np.float32)
+        assert np.array_equal(p[off:off + n], want), "weights at %d" % off
+        off += n
+        assert (p[off:off + co] == np.float32(bias)).all(); off += co
+
+    def norm(c):
+        nonlocal off
+        assert (p[off:off + c] == 1).all() and (p[off + c:off + 2 * c] == 0).all(); off += 2 * c
+    # parameter order (src/unet.c:451-459): encoder blocks, downs, decoder blocks from the coarsest level, head
+    for i, w in enumerate(widths):
+        conv(cin if i == 0 else widths[i - 1], w, 3, 0); norm(w); conv(w, w, 3, 0); norm(w)
+    conv(widths[0], widths[0], 3, 0)                                   # down0 keeps the width
+    conv(widths[1] + widths[0], widths[0], 3, 0); norm(widths[0]); conv(widths[0], widths[0], 3, 0); norm(widths[0])
+    conv(widths[0], 3, 1, -2.0)
+    assert off == p.size
+
+
 def test_checkpoint_round_trip(gpu, tmp_path):
     """unet_save -> unet_peek -> unet_create -> unet_load gives the same network: identical parameters and byte-identical logits;
     a network of another architecture, a truncated payload and a checkpoint of an unsupported feature are refused (src/unet.c:5774-5800)."""

@@ -84,4 +84,10 @@ def test_static_scratch_conv_refuses_what_does_not_fit(gpu):
     assert lib.mi_conv_fwd_static(8, dx.ptr, 3, shape5(N, C, D, D, D), dw.ptr, None, C, dy.ptr, 3, gnp_t(), None, 0, split_t()) == 0
     LP.check()
     assert lib.mi_alloc_count() == n0
+    # a few-channel fp32 network input goes to the tap-packed kernel, which reads it as stored and stages nothing: a whole 2 x 128^3 window fits
+    dx4 = DevBuf(N * 4 * S * 4); w4 = DevBuf.from_numpy((rng.standard_normal((C, 4, 27)) * 0.1).astype(np.float32))
+    n1 = lib.mi_alloc_count()
+    assert lib.mi_conv_fwd_static(8, dx4.ptr, 0, shape5(N, 4, D, D, D), w4.ptr, None, C, dy.ptr, 3, gnp_t(), None, 0, split_t()) == 0
+    LP.check()
+    assert lib.mi_alloc_count() == n1 and "conv3_stem_k" in lib.mi_last_kernel().decode()
     assert lib.mi_conv_fwd_static(5, dx.ptr, 3, shape5(N, C, D, D, D), dw.ptr, None, C, dy.ptr, 3, gnp_t(), None, 0, split_t()) == -1

@@ -549,7 +549,7 @@ extern "C" int mi_conv_fwd_fused(int bits, const void *x, int xbf, shape5 xs, co
     return conv_dispatch("mi_conv_fwd_fused", bits, 1, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, ep_a, ep_b, act);
 }
 
-// ---- the stride-1 convs for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that forbid hipMalloc) ----
+// ---- the stride-1 convs for callers that cannot allocate (serving loops, harnesses that forbid hipMalloc) ----
 // Every byte of device memory the conv needs beyond its inputs and outputs - prepared weights, re-staged operands, the coarse rows of a fused
 // upsample, per-tile statistics partials, the constant page of out-of-volume rows - is carved from one file-scope device array. The array is a
 // host-side stand-in by name: its device address is taken once per device and only that address is used from then on.
@@ -559,7 +559,7 @@ static unsigned char *g_scratch_ptr[8];        // per device: the address of tha
 static std::mutex g_scratch_mu;
 extern "C" size_t mi_conv_static_scratch_bytes(void) { return MI_STATIC_SCRATCH_BYTES; }
 // an upper bound of what conv_dispatch will request from mi_ws for this call, following its choices (every request rounded up to 256 bytes)
-static size_t conv_scratch_bound(int fmt, const void *x2, int xbf, shape5 xs, int cout, gnp_t gp, const double *osum, split_t sp) {
+static size_t conv_scratch_bound(int fmt, const void *x2, int xbf, int ybf, shape5 xs, int cout, gnp_t gp, const double *osum, split_t sp) {
     auto al = [](size_t n) { return ((n + 255) & ~(size_t)255) + 256; };
     const int Ci = xs.c, Cx = x2 ? sp.c_split : Ci, C2 = Ci - Cx, N = xs.n, D = sp.Di ? sp.Di : xs.d;
     if (fmt == 4 && Ci <= 8) fmt = 8;
@@ -570,8 +570,10 @@ static size_t conv_scratch_bound(int fmt, const void *x2, int xbf, shape5 xs, in
     if (Ci <= 16 && !x2 && fmt == 8) need += al((size_t)9 * nmt_all * 2048) + al((size_t)9 * nmt_all * 256);      // the tap-packed kernels' weights
     const int nbt = (Cx + 31) / 32 + (x2 ? (C2 + 31) / 32 : 0);
     need += al(((size_t)(27 * nbt + 1) / 2 + 2 * nbt + 16) * nmt_all * 2304) + al(((size_t)(27 * nbt + 1) / 2 + 2 * nbt + 16) * nmt_all * 256);      // (at most 15 pairs per block)
+    // the tap-packed kernels read their input as stored and apply its GroupNorm while staging: nothing is re-staged (conv_dispatch's routing)
+    const bool stem = fmt == 8 && !x2 && ((xbf == 0 || xbf >= 2) && Ci <= (xbf == 0 ? 16 : 8) || (xbf >= 2 && Ci <= 16)) && (xbf == ybf || ybf >= 3);
     const bool s2g = x2 && sp.gp2.G;
-    for (int s = 0; s < (x2 ? 2 : 1); s++) {
+    for (int s = 0; s < (x2 ? 2 : 1) && !stem; s++) {
         const gnp_t g = s2g ? (s ? sp.gp2 : gp) : gp;
         const bool upseg = s == 0 && sp.up, direct = xbf == fdt && !(g.G > 0) && !upseg;
         const int C = s ? C2 : Cx;
@@ -582,20 +584,25 @@ static size_t conv_scratch_bound(int fmt, const void *x2, int xbf, shape5 xs, in
     (void)So;
     return need;
 }
+// set-up, once per device with that device current: the array's address on this device, and the constant page at its head. mi_init calls it
+// for the device it selects (a synchronous 128-byte copy: not something to meet for the first time inside a serving loop); the entry point
+// repeats the call for a device nobody initialised through mi_init
+int mi_conv_static_setup(const char *who) {
+    int dv = 0; MIRT(hipGetDevice(&dv)); dv &= 7;
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[dv]) return 0;
+    unsigned char *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) { fprintf(stderr, "%s: the fixed scratch has no address on device %d: %s\n", who, dv, hipGetErrorString(e)); return -2; }
+    uint8_t init[128]; memset(init, 0, 64); memset(init + 64, 1, 64);
+    if (hipMemcpy(ptr, init, 128, hipMemcpyHostToDevice) != hipSuccess) { fprintf(stderr, "%s: cannot initialise the fixed scratch on device %d\n", who, dv); return -2; }
+    g_scratch_ptr[dv] = ptr;
+    return 0;
+}
 static int conv_fwd_static(const char *who, int fmt, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp) {
     int dv = 0; MIRT(hipGetDevice(&dv)); dv &= 7;
-    {   // set-up, once per device with that device current: the array's address on this device, and the constant page at its head
-        std::lock_guard<std::mutex> lk(g_scratch_mu);
-        if (!g_scratch_ptr[dv]) {
-            unsigned char *ptr = nullptr;
-            const hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
-            if (e != hipSuccess || !ptr) { fprintf(stderr, "%s: the fixed scratch has no address on device %d: %s\n", who, dv, hipGetErrorString(e)); return -2; }
-            uint8_t init[128]; memset(init, 0, 64); memset(init + 64, 1, 64);
-            if (hipMemcpy(ptr, init, 128, hipMemcpyHostToDevice) != hipSuccess) { fprintf(stderr, "%s: cannot initialise the fixed scratch on device %d\n", who, dv); return -2; }
-            g_scratch_ptr[dv] = ptr;
-        }
-    }
-    const size_t need = conv_scratch_bound(fmt, sp.x2, xbf, xs, cout, gp, osum, sp);
+    if (!g_scratch_ptr[dv] && mi_conv_static_setup(who)) return -2;
+    const size_t need = conv_scratch_bound(fmt, sp.x2, xbf, ybf, xs, cout, gp, osum, sp);
     if (need > MI_STATIC_SCRATCH_BYTES) {
         fprintf(stderr, "%s: this call needs up to %zu bytes of scratch (prepared weights, re-staged operands, statistics partials); the fixed scratch holds %zu. "
                         "Use lp_conv_fwd_f8 / lp_conv_fwd_f4, which allocate, or pass an input that is already in the compute format without GroupNorm\n", who, need, (size_t)MI_STATIC_SCRATCH_BYTES);

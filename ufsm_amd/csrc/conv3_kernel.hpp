@@ -125,7 +125,19 @@ template <int FMT> struct fmt_t;
 template <> struct fmt_t<8> { static constexpr int RB = 32, NH = 2, WTILE = 2048; };
 template <> struct fmt_t<4> { static constexpr int RB = 16, NH = 1, WTILE = 1024; };
 
-__device__ __forceinline__ float gelu_erf(float x) { return 0.5f * x * (1.f + erff(x * 0.70710678f)); }
+// GELU, x Phi(x) = 0.5 x (1 + erf(x / sqrt 2)), with erf by the rational-times-Gaussian form erf z = 1 - (a1 t + ... + a5 t^5) exp(-z^2),
+// t = 1 / (1 + p z), z >= 0 (Abramowitz & Stegun 7.1.26, |error| < 1.5e-7): about 16 instructions with one reciprocal and one exponential where
+// the library's erff takes about 60; the epilogue that applies it runs alone on its SIMD, so every instruction is time. With
+// q = 0.5 |x| (a1 t + ...) exp(-z^2) the result is max(x, 0) - q for either sign. NaN stays NaN; +-inf: z^2 overflows, the exponential is 0, q = inf 0
+// would be NaN, so q takes the exponential's zero through a select
+__device__ __forceinline__ float gelu_erf(float x) {
+    const float ax = fabsf(x), z = ax * 0.70710678f;
+    const float t = __builtin_amdgcn_rcpf(fmaf(z, 0.3275911f, 1.f));
+    const float poly = t * fmaf(t, fmaf(t, fmaf(t, fmaf(t, 1.061405429f, -1.453152027f), 1.421413741f), -0.284496736f), 0.254829592f);
+    const float ex = __builtin_amdgcn_exp2f(z * z * -1.44269504f);
+    const float q = ex == 0.f ? 0.f : 0.5f * ax * poly * ex;
+    return fmaxf(x, 0.f) - q;
+}
 
 // geometry of a workgroup's halo: output tile TZ x 8 x 16, input halo HZ x HY x HX positions
 template <int FMT, int STRIDE, int TZ> struct halo_t {

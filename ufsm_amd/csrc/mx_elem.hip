@@ -92,6 +92,44 @@ extern "C" void lp_mx4_to_f32(const void *x, int N, int C, size_t S, float *y) {
     mx_to_f32_k<4><<<rows_grid(N, mx_nb(C), S), 256>>>((const uint8_t *)x, y, N, C, S); MICK();
 }
 
+// ---- every fp32 bit pattern through the hardware encoders (v_cvt_scalef32_pk_fp8_f32, v_cvt_scalef32_pk_fp4_f32) at a block exponent e,
+// against the software encoders of the scaled value x 2^-e, which equal the checker's over all 2^32 inputs (the reference checks its own
+// conversion instruction the same way, src/lp_mxsw.cu:45-61). Counts: [0] inputs inside the domain the kernels use the instruction on
+// (e4m3: |x 2^-e| <= 464, not NaN; e2m1: not NaN), [1] mismatches among them, [2] inputs outside it, [3] mismatches among those ----
+__global__ void __launch_bounds__(256) cvt_sweep_k(int bits, int e, unsigned long long *cnt) {
+    const unsigned first = (blockIdx.x * 256u + threadIdx.x) * 4096u;         // 2^20 threads x 4096 patterns
+    const float p2e = d_exp2i(e), inv = d_exp2i(-e);
+    unsigned n_in = 0, bad_in = 0, n_out = 0, bad_out = 0;
+    for (unsigned k = 0; k < 4096u; k += 2) {
+        const float a = __uint_as_float(first + k), b = __uint_as_float(first + k + 1);
+        unsigned ha, hb, sa, sb;
+        if (bits == 8) {
+            const unsigned wv = d_enc_e4m3x4_hw(a, b, a, b, p2e);
+            ha = wv & 255u; hb = (wv >> 8) & 255u;
+            sa = d_enc_e4m3(a * inv); sb = d_enc_e4m3(b * inv);
+        } else {
+            const float v8[8] = {a, b, a, b, a, b, a, b};
+            const unsigned wv = d_enc_e2m1x8_hw(v8, p2e);
+            ha = wv & 15u; hb = (wv >> 4) & 15u;
+            sa = d_enc_e2m1(a * inv); sb = d_enc_e2m1(b * inv);
+        }
+        const bool ia = bits == 8 ? fabsf(a * inv) <= 464.f : a == a, ib = bits == 8 ? fabsf(b * inv) <= 464.f : b == b;     // (NaN compares false)
+        n_in += ia + ib; n_out += !ia + !ib;
+        bad_in += (ia && ha != sa) + (ib && hb != sb); bad_out += (!ia && ha != sa) + (!ib && hb != sb);
+    }
+    atomicAdd(&cnt[0], (unsigned long long)n_in); atomicAdd(&cnt[1], (unsigned long long)bad_in);
+    atomicAdd(&cnt[2], (unsigned long long)n_out); atomicAdd(&cnt[3], (unsigned long long)bad_out);
+}
+extern "C" int mi_cvt_sweep(int bits, int e, unsigned long long out[4]) {
+    if ((bits != 8 && bits != 4) || e < -126 || e > 126) return -1;
+    unsigned long long *cnt = (unsigned long long *)mi_ws(MI_WS_MISC, 4 * sizeof(unsigned long long));
+    MIRT(hipMemsetAsync(cnt, 0, 4 * sizeof(unsigned long long), 0));
+    cvt_sweep_k<<<4096, 256>>>(bits, e, cnt);
+    MICK();
+    MIRT(hipMemcpy(out, cnt, 4 * sizeof(unsigned long long), hipMemcpyDeviceToHost));
+    return 0;
+}
+
 // ---- network input rows (src/lp_mx_cvt.cu:29-55): z-scored CT, 0, unit direction away from the axis -> one 8-wide row per voxel ----
 // Only channels 0, 2 and 3 of a row are ever non-zero, so a row is formed in registers from three values: amax over the three (integer,
 // NaN-propagating), one exponent, one packed encode. A thread owns VPT = 4 neighbouring voxels of a row of the window when W % 4 == 0
@@ -873,28 +911,40 @@ void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W
 void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int h2) { mi_restage_up_sub(x, xdt, N, C, D, H, W, gp, Cg, y, ybits, 0, D, h2); }
 
 // weights w [Co][Ci][T] rounded in place to MX-fp4 values with one E8M0 scale per Bo x Bi (output x input channel) block and tap (src/lp_mx_cvt.cu:369-395):
-// the forward's per-output-channel blocks of 32 inputs inside a 32 x 32 block then re-quantise these values exactly. One wavefront per (tap, block).
-__global__ void __launch_bounds__(256) fakeq_w4_k(float *w, int Co, int Ci, int T, int Bo, int Bi) {
-    const int nbo = (Co + Bo - 1) / Bo, nbi = (Ci + Bi - 1) / Bi, lane = threadIdx.x & 63;
-    const size_t wid = (blockIdx.x * (size_t)blockDim.x + threadIdx.x) >> 6;
-    if (wid >= (size_t)T * nbo * nbi) return;                 // (uniform per wavefront)
-    const int t = (int)(wid % T), bi = (int)((wid / T) % nbi), bo = (int)(wid / ((size_t)T * nbi));
-    const int o0 = bo * Bo, i0 = bi * Bi, no = min(Bo, Co - o0), ni = min(Bi, Ci - i0);
-    float amax = 0.f;
-    for (int e = lane; e < no * ni; e += 64) amax = fmaxf(amax, fabsf(w[((size_t)(o0 + e / ni) * Ci + i0 + e % ni) * T + t]));
-#pragma unroll
-    for (int o = 32; o; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
-    const int ex = d_mx_exp(amax, MI_INVQ4);
-    const float m = d_exp2i(-ex), sc = d_exp2i(ex);
-    for (int e = lane; e < no * ni; e += 64) {
-        float *p = w + ((size_t)(o0 + e / ni) * Ci + i0 + e % ni) * T + t;
-        *p = d_dec_e2m1(d_enc_e2m1(*p * m)) * sc;
+// the forward's per-output-channel blocks of 32 inputs inside a 32 x 32 block then re-quantise these values exactly.
+// The taps are the innermost index of the weight array, so a block's rows are runs of Bi x T contiguous floats: one workgroup takes a whole
+// block with all its taps and walks those runs with consecutive lanes on consecutive floats. First walk: every tap's maximum magnitude into
+// its LDS word (non-negative floats order as their bit patterns; NaN skipped, as fmaxf drops it); second walk: each float rounded at its
+// tap's scale and written back.
+__global__ void __launch_bounds__(256) fakeq_w4_k(float *w, int Co, int Ci, int T, int Bo, int Bi, int col_blocks) {
+    extern __shared__ unsigned tap_max[];                     // [T] bit patterns of the taps' maxima, then [T] their exponents
+    int *tap_exp = (int *)(tap_max + T);
+    const int row0 = (int)(blockIdx.x / col_blocks) * Bo, col0 = (int)(blockIdx.x % col_blocks) * Bi;
+    const int rows = min(Bo, Co - row0), run = min(Bi, Ci - col0) * T;                   // floats of the block per output row
+    float *base = w + ((size_t)row0 * Ci + col0) * T;
+    const size_t pitch = (size_t)Ci * T;
+    for (int t = threadIdx.x; t < T; t += blockDim.x) tap_max[t] = 0u;
+    __syncthreads();
+    const int total = rows * run;
+    for (int k = threadIdx.x; k < total; k += blockDim.x) {
+        const int rr = k / run, j = k - rr * run;
+        const float v = fabsf(base[rr * pitch + j]);
+        if (v == v) atomicMax(&tap_max[j % T], __float_as_uint(v));
+    }
+    __syncthreads();
+    for (int t = threadIdx.x; t < T; t += blockDim.x) tap_exp[t] = d_mx_exp(__uint_as_float(tap_max[t]), MI_INVQ4);
+    __syncthreads();
+    for (int k = threadIdx.x; k < total; k += blockDim.x) {
+        const int rr = k / run, j = k - rr * run, ex = tap_exp[j % T];
+        float *q = base + rr * pitch + j;
+        *q = d_dec_e2m1(d_enc_e2m1(*q * d_exp2i(-ex))) * d_exp2i(ex);
     }
 }
 extern "C" void lp_fakeq_w4(float *w, int Co, int Ci, int T, int Bo, int Bi) {
     if (Co <= 0 || Ci <= 0 || T <= 0 || Bo <= 0 || Bi <= 0) return;
-    const size_t nw = (size_t)T * ((Co + Bo - 1) / Bo) * ((Ci + Bi - 1) / Bi);
-    fakeq_w4_k<<<nblk_(nw * 64, 256), 256>>>(w, Co, Ci, T, Bo, Bi);
+    const int row_blocks = (Co + Bo - 1) / Bo, col_blocks = (Ci + Bi - 1) / Bi;
+    if ((size_t)row_blocks * col_blocks > 0x7fffffffu || (size_t)T * 8 > 48 * 1024 || (size_t)Bo * Bi * T > 0x7fffffffu) mi_die("lp_fakeq_w4: %d x %d weights, %d taps in blocks of %d x %d", Co, Ci, T, Bo, Bi);
+    fakeq_w4_k<<<(unsigned)(row_blocks * col_blocks), 256, (size_t)T * 8>>>(w, Co, Ci, T, Bo, Bi, col_blocks);
     MICK();
 }
 extern "C" void nn_fakeq_w4_2d(float *w, int Co, int Ci, int T, int B) { lp_fakeq_w4(w, Co, Ci, T, B, B); }      // src/nn_elem.cu:192

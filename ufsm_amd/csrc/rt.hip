@@ -26,13 +26,15 @@ extern "C" const char *lp_check(void) {
     return g_errmsg;
 }
 extern "C" int mi_device_count(void) { int n = 0; if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; } return n; }
+int mi_conv_static_setup(const char *who);      // conv3.hip
 extern "C" int mi_init(int device) {
     int n = mi_device_count();
     if (device < 0 || device >= n) { fprintf(stderr, "mi_init: no HIP device %d (%d visible): the MX kernels need a gfx950 GPU\n", device, n); return 1; }
     hipDeviceProp_t p;
     if (hipGetDeviceProperties(&p, device) != hipSuccess) return 2;
     if (strncmp(p.gcnArchName, "gfx950", 6) != 0) { fprintf(stderr, "mi_init: device %d is %s, this library is built for gfx950 only\n", device, p.gcnArchName); return 3; }
-    return hipSetDevice(device) == hipSuccess ? 0 : 4;
+    if (hipSetDevice(device) != hipSuccess) return 4;
+    return mi_conv_static_setup("mi_init") ? 5 : 0;             // the entry point that allocates nothing finds its fixed scratch addressed and its constant page written
 }
 extern "C" void *mi_malloc(size_t bytes) {
     void *p = nullptr;

@@ -388,44 +388,76 @@ void mi_unet_get_params(const unet *u, float *host) { mi_sync(); mi_d2h(host, u-
 void mi_unet_set_params(unet *u, const float *host) { mi_h2d(u->p, host, u->np * 4); mi_h2d(u->ema, host, u->np * 4); u->wm_ok = 0; lp_wmemo_clear(); }
 shape5 unet_out_shape(const unet *u, shape5 xs) { return (shape5){xs.n, u->cfg.cout, xs.d, xs.h, xs.w}; }
 
-/* splitmix64 -> uniform -> Box-Muller normal: the distribution of src/unet.c:586-593, not its generator's bits */
-static double unif(uint64_t *s) { uint64_t z = (*s += 0x9e3779b97f4a7c15ull); z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull; z = (z ^ (z >> 27)) * 0x94d049bb133111ebull; z ^= z >> 31; return (double)(z >> 11) * 0x1.0p-53; }
-static double gauss(uint64_t *s) { const double a = unif(s) + 1e-300, b = unif(s); return sqrt(-2 * log(a)) * cos(6.283185307179586 * b); }
-static void init_conv(float *h, const convp *c, uint64_t *seed, double bias) {
-    const size_t nw = (size_t)c->cout * c->cin * c->k * c->k * c->k;
-    const double std = sqrt(2.0 / ((double)c->cin * c->k * c->k * c->k));
-    for (size_t i = 0; i < nw; i++) h[c->w + i] = (float)(std * gauss(seed));
-    for (int i = 0; i < c->cout; i++) h[c->b + i] = (float)bias;
+/* ---- initial weights ----
+   Same seed, same network as the reference's unet_init, bit for bit (src/unet.c:584-644): a caller that trains or tests from unet_init(u, seed)
+   starts from identical weights in either program, which is what lets logits, checkpoints and regression baselines be compared across the two.
+   That fixes the generator (splitmix64, 53-bit uniforms, one Box-Muller cosine branch per pair of uniforms) and the order in which the
+   parameter vector consumes it; the rest is this file's: the network is first described as a list of runs (a span of the parameter vector,
+   how it is filled), then one loop fills the spans in list order. tests/test_gpu_unet.py::test_unet_init_matches_the_published_generator
+   checks the weights against an independent statement of the generator. */
+typedef struct { size_t off, n; double sd; float fill; int drop; } init_run;      /* sd > 0: N(0, sd^2) draws (drop: drawn, then stored as 0); else the constant */
+typedef struct { init_run *r; int n, cap; } init_plan;
+static void plan_add(init_plan *pl, size_t off, size_t n, double sd, float fill, int drop) {
+    if (!n) return;
+    if (pl->n == pl->cap) { pl->cap = pl->cap ? 2 * pl->cap : 128; pl->r = realloc(pl->r, (size_t)pl->cap * sizeof *pl->r); if (!pl->r) { fprintf(stderr, "unet_init: out of memory\n"); abort(); } }
+    pl->r[pl->n++] = (init_run){off, n, sd, fill, drop};
 }
-static void init_gn(float *h, const gnpar *n) { for (int i = 0; i < n->c; i++) { h[n->gamma + i] = 1.f; h[n->beta + i] = 0.f; } }
+static void plan_conv(init_plan *pl, const convp *c, float bias, int drop) {      /* Kaiming-normal weights, constant bias */
+    const size_t fan = (size_t)c->cin * c->k * c->k * c->k;
+    plan_add(pl, c->w, (size_t)c->cout * fan, sqrt(2.0 / (double)fan), 0.f, drop);
+    plan_add(pl, c->b, (size_t)c->cout, 0.0, bias, 0);
+}
+static void plan_norm(init_plan *pl, const gnpar *g) { plan_add(pl, g->gamma, (size_t)g->c, 0.0, 1.f, 0); }      /* (beta: the vector starts zeroed) */
+static uint64_t mix64(uint64_t *state) {                               /* splitmix64 */
+    uint64_t z = (*state += 0x9e3779b97f4a7c15ull);
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+static double draw_normal(uint64_t *state) {
+    const double u1 = (double)(mix64(state) >> 11) * 0x1.0p-53 + 1e-300, u2 = (double)(mix64(state) >> 11) * 0x1.0p-53;
+    return sqrt(-2 * log(u1)) * cos(6.283185307179586 * u2);
+}
 void unet_init(unet *u, uint64_t seed) {
-    float *h = calloc(u->np, 4);
-    if (!h) { fprintf(stderr, "unet_init: out of memory\n"); abort(); }
+    init_plan pl = {nullptr, 0, 0};
     const int L = u->cfg.nlev;
-    for (int i = 0; i < L; i++) { init_conv(h, &u->enc[i].c1, &seed, 0); init_gn(h, &u->enc[i].n1); init_conv(h, &u->enc[i].c2, &seed, 0); init_gn(h, &u->enc[i].n2); }
-    for (int i = 0; i < L - 1; i++) init_conv(h, &u->down[i], &seed, 0);
-    for (int i = 0; i < L - 1; i++) { init_conv(h, &u->dec[i].c1, &seed, 0); init_gn(h, &u->dec[i].n1); if (!u->dec[i].single) { init_conv(h, &u->dec[i].c2, &seed, 0); init_gn(h, &u->dec[i].n2); } }
-    init_conv(h, &u->head, &seed, -2.0);
-    for (int i = 0; i < L; i++) for (int k = 0; k < u->cfg.enc_blocks[i]; k++) {      /* residual blocks start as the identity: conv2's weights zero (src/unet.c:606-610) */
-        block *b = &u->rb[i][k];
-        init_conv(h, &b->c1, &seed, 0); init_gn(h, &b->n1); init_conv(h, &b->c2, &seed, 0); init_gn(h, &b->n2);
-        const char *nz = getenv("UFSM_RB_NONZERO");
-        if (!(nz && atoi(nz))) memset(h + b->c2.w, 0, (size_t)b->c2.cout * b->c2.cin * 27 * 4);
+    for (int i = 0; i < L; i++) { const block *b = &u->enc[i]; plan_conv(&pl, &b->c1, 0.f, 0); plan_norm(&pl, &b->n1); plan_conv(&pl, &b->c2, 0.f, 0); plan_norm(&pl, &b->n2); }
+    for (int i = 0; i + 1 < L; i++) plan_conv(&pl, &u->down[i], 0.f, 0);
+    for (int i = 0; i + 1 < L; i++) {
+        const block *b = &u->dec[i];
+        plan_conv(&pl, &b->c1, 0.f, 0); plan_norm(&pl, &b->n1);
+        if (!b->single) { plan_conv(&pl, &b->c2, 0.f, 0); plan_norm(&pl, &b->n2); }
     }
-    for (int j = 1; j <= u->cfg.ds_levels; j++) init_conv(h, &u->ds[j], &seed, -2.0);                /* as the main head (src/unet.c:611-612) */
-    if (u->cfg.emb_lev) init_conv(h, &u->eh, &seed, 0.0);
-    if (u->cfg.down_norm) for (int i = 0; i < L - 1; i++) init_gn(h, &u->dn[i]);
+    plan_conv(&pl, &u->head, -2.f, 0);
+    const char *rbnz = getenv("UFSM_RB_NONZERO");
+    const int rb_keep = rbnz && atoi(rbnz);
+    for (int i = 0; i < L; i++) for (int k = 0; k < u->cfg.enc_blocks[i]; k++) {      /* residual blocks start as the identity: conv2's weights drawn, then zero (src/unet.c:606-610) */
+        const block *b = &u->rb[i][k];
+        plan_conv(&pl, &b->c1, 0.f, 0); plan_norm(&pl, &b->n1); plan_conv(&pl, &b->c2, 0.f, !rb_keep); plan_norm(&pl, &b->n2);
+    }
+    for (int j = 1; j <= u->cfg.ds_levels; j++) plan_conv(&pl, &u->ds[j], -2.f, 0);                     /* as the main head (src/unet.c:611-612) */
+    if (u->cfg.emb_lev) plan_conv(&pl, &u->eh, 0.f, 0);
+    if (u->cfg.down_norm) for (int i = 0; i + 1 < L; i++) plan_norm(&pl, &u->dn[i]);
     if (u->tbn) {   /* LayerNorm and QK-norm gains 1, QKV and MLP-in N(0, 1 / C), out projections and biases 0 (identity blocks), registers N(0, 0.02^2) (src/unet.c:612-642) */
-        const int C = u->tbd.C, F = u->tbd.F; const double sd = 1.0 / sqrt((double)C);
+        const size_t C = (size_t)u->tbd.C, F = (size_t)u->tbd.F; const double sd = 1.0 / sqrt((double)C);
         for (int k = 0; k < u->tbn; k++) {
             const at_bp *bp = &u->tbp[k];
-            for (int c = 0; c < C; c++) h[bp->ln1g + c] = h[bp->ln2g + c] = h[bp->qg + c] = h[bp->kg + c] = 1.f;
-            for (size_t i = 0; i < (size_t)3 * C * C; i++) h[bp->wqkv + i] = (float)(sd * gauss(&seed));
-            for (size_t i = 0; i < (size_t)2 * F * C; i++) h[bp->w1 + i] = (float)(sd * gauss(&seed));
+            plan_add(&pl, bp->ln1g, C, 0.0, 1.f, 0); plan_add(&pl, bp->ln2g, C, 0.0, 1.f, 0); plan_add(&pl, bp->qg, C, 0.0, 1.f, 0); plan_add(&pl, bp->kg, C, 0.0, 1.f, 0);
+            plan_add(&pl, bp->wqkv, 3 * C * C, sd, 0.f, 0);
+            plan_add(&pl, bp->w1, 2 * F * C, sd, 0.f, 0);
         }
-        for (size_t i = 0; i < (size_t)u->tbd.nreg * C; i++) h[u->reg_off + i] = (float)(0.02 * gauss(&seed));
-        if (u->cfg.attn_vres) for (int k = 1; k < u->tbn; k++) for (int hh = 0; hh < u->tbd.H; hh++) h[u->vr_off + (size_t)k * u->tbd.H + hh] = 0.5f;      /* (src/unet.c:644) */
+        plan_add(&pl, u->reg_off, (size_t)u->tbd.nreg * C, 0.02, 0.f, 0);
+        if (u->cfg.attn_vres && u->tbn > 1) plan_add(&pl, u->vr_off + (size_t)u->tbd.H, (size_t)(u->tbn - 1) * u->tbd.H, 0.0, 0.5f, 0);      /* every application after the first (src/unet.c:644) */
     }
+    float *h = calloc(u->np, 4);
+    if (!h) { fprintf(stderr, "unet_init: out of memory\n"); abort(); }
+    for (int r = 0; r < pl.n; r++) {
+        const init_run *ir = &pl.r[r];
+        float *dst = h + ir->off;
+        if (ir->sd > 0) for (size_t i = 0; i < ir->n; i++) { const float v = (float)(ir->sd * draw_normal(&seed)); dst[i] = ir->drop ? 0.f : v; }
+        else for (size_t i = 0; i < ir->n; i++) dst[i] = ir->fill;
+    }
+    free(pl.r);
     mi_unet_set_params(u, h);
     free(h);
 }
@@ -704,6 +736,10 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
         if ((q = strstr(line, "\"ge_run\":["))) { q += 10; while (l0->gcnt < 8192 && *q && *q != ']') { char *e; l0->grun[l0->gcnt] = strtof(q, &e); if (e == q) break; l0->gcnt++; q = e; if (*q == ',') q++; } }
         if ((q = strstr(line, "\"l0_run\":["))) { q += 10; while (l0->cnt < 1024 && *q && *q != ']') { char *e; l0->run[l0->cnt] = strtof(q, &e); if (e == q) break; l0->cnt++; q = e; if (*q == ',') q++; } }
     }
+    /* weights the reference transforms after reading the same fp32 payload: 2:4 masks (unet_set_sparse24*) and packed fp8 / fp4 weight storage
+       (unet_set_wq), src/unet.c:5703-5707, :5839-5840. Loading such a file as dense fp32 master weights would run another function */
+    if (!bad && key_int(line, "\"sparse24\":", 0)) bad = "\"sparse24\": (2:4 sparse weights)";
+    if (!bad && key_int(line, "\"wq\":", 0)) bad = "\"wq\": (packed fp8 / fp4 weight storage)";
     if (!bad && cfg->attn_blocks && (cfg->attn_pe < 0 || cfg->attn_pe > 2)) bad = "\"attn_pe\": (scroll RoPE)";
     if (bad) { fprintf(stderr, "unet_peek: %s uses %s which this build does not run\n", path, bad); free(line); return -2; }
     free(line);

@@ -110,6 +110,7 @@ _PROTOS = {
     "mi_conv_fwd_static": (_I, [_I, _P, _I, shape5, _P, _P, _I, _P, _I, gnp_t, _P, _I, split_t]),
     "mi_conv_static_scratch_bytes": (_Z, []),
     "mi_alloc_count": (C.c_long, []),
+    "mi_cvt_sweep": (_I, [_I, _I, C.POINTER(C.c_ulonglong)]),
     "mi_kernel_timing": (None, [_I]),
     "mi_kernel_timing_read": (C.c_double, [C.POINTER(C.c_long)]),
     "mi_kernel_timing_launch": (C.c_long, [C.c_long, C.POINTER(C.c_float), C.POINTER(C.c_double), C.c_char_p, _Z]),

@@ -56,6 +56,12 @@ def load_host():
     L.mi_unet_set_params.restype = None; L.mi_unet_set_params.argtypes = [P, P]
     L.mi_unet_layer_out.restype = P; L.mi_unet_layer_out.argtypes = [P, _I, C.POINTER(shape5), C.POINTER(C.c_char_p)]
     L.mi_unet_layer_stats.restype = _I; L.mi_unet_layer_stats.argtypes = [P, _I, C.POINTER(P), C.POINTER(P)]
+    F = C.c_float
+    L.nn_conv3d_out_shape.restype = shape5; L.nn_conv3d_out_shape.argtypes = [shape5, _I, _I, _I]
+    L.nn_conv3d_fwd.restype = None; L.nn_conv3d_fwd.argtypes = [P, shape5, P, P, _I, _I, _I, P]
+    L.nn_conv3d_fwd_gn.restype = _I; L.nn_conv3d_fwd_gn.argtypes = [P, shape5, _I, P, P, P, P, P, P, _I, P]
+    L.nn_conv3d_fwd_gn_stats.restype = _I; L.nn_conv3d_fwd_gn_stats.argtypes = [P, shape5, _I, P, P, P, P, P, P, _I, P, _I, F, P, P]
+    L.nn_conv3d_fwd_split.restype = _I; L.nn_conv3d_fwd_split.argtypes = [P, P, _I, shape5, _I, P, P, P, P, P, P, _I, P, _I, F, P, P]
     L.nn_set_storage.restype = None; L.nn_set_storage.argtypes = [P, C.c_size_t, _I]
     L.nn_storage.restype = _I; L.nn_storage.argtypes = [P]
     L.nn_storage_forget.restype = None; L.nn_storage_forget.argtypes = [P]
