@@ -197,6 +197,46 @@ def test_exact_operand_conv(gpu, bits, N, Ci, Co, D, H, W, stride):
         assert np.array_equal(gq, wq)
 
 
+ROW1_SHAPES = [(8, 2, 32, 32, 8, 16, 32), (8, 1, 32, 32, 5, 9, 40), (8, 1, 20, 24, 7, 10, 33), (8, 2, 32, 32, 64, 64, 64),
+               (4, 1, 32, 32, 8, 12, 48), (4, 2, 32, 24, 6, 9, 34), (4, 1, 32, 32, 32, 64, 128)]
+
+
+@pytest.mark.parametrize("bits,N,Ci,Co,D,H,W", ROW1_SHAPES)
+def test_one_block_row_kernel(gpu, bits, N, Ci, Co, D, H, W):
+    """The one-input-block row kernel (17 .. 32 output channels from <= 32 input channels on volumes wider than 16 voxels; the two halves of
+    its workgroups run half a tile apart and keep their statistics per wavefront): exact operands equal the oracle in every output type, ragged
+    tiles and more tiles than workgroups included (the persistent walk's double buffer); random operands meet the conv tolerance, the statistics
+    are those of the oracle and identical run to run."""
+    rng = np.random.default_rng(Ci * 5 + Co + D + W)
+    S = D * H * W
+    xdt = 3 if bits == 8 else 4
+    x, w, b = exact_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    want, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, acc64=1)
+    got, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits)
+    assert "conv3_row1_k" in lib.mi_last_kernel().decode(), lib.mi_last_kernel().decode()
+    assert np.array_equal(got, want)
+    for ydt in (2, 3, 4):
+        wq, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=bits, acc64=1)
+        gq, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=bits)
+        assert np.array_equal(gq, wq), ydt
+    if S * N > 600000:                                            # (the large cases: exact operands only)
+        return
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    G = 8 if Co % 32 == 0 else 2                                  # (channels per group a multiple of 4, or the launch leaves this kernel)
+    want, ws = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, Go=G, want_stats=True)
+    got, gs = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, Go=G, stats=True)
+    assert "conv3_row1_k" in lib.mi_last_kernel().decode()
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-4
+    assert np.abs(gs - ws).max() / np.abs(ws).max() < 1e-5
+    gq, gs2 = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, Go=G, stats=True, stored_stats=1)
+    dec = orc.mx_to_f32(bits, gq, N, Co, S).astype(np.float64).reshape(N, G, -1)
+    assert np.allclose(gs2[:, :, 0], dec.sum(-1), rtol=1e-5, atol=1e-3) and np.allclose(gs2[:, :, 1], (dec * dec).sum(-1), rtol=1e-5)
+    gq2, gs3 = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, xdt, cbits=bits, Go=G, stats=True, stored_stats=1)
+    assert np.array_equal(gq, gq2) and np.array_equal(gs2, gs3)
+
+
 RANDOM_SHAPES = [(8, 2, 32, 16, 8, 16, 16, 1), (8, 1, 16, 24, 4, 8, 16, 1), (8, 2, 32, 32, 8, 16, 16, 1), (8, 1, 128, 128, 6, 12, 20, 1), (8, 1, 64, 64, 8, 8, 24, 1), (4, 1, 256, 256, 4, 8, 16, 1), (4, 1, 32, 32, 8, 16, 16, 1),
                  (8, 1, 64, 64, 12, 10, 14, 2), (8, 1, 80, 48, 5, 9, 18, 1),
                  # channels per group that are not a multiple of 4 on more than one channel tile: 80 / 8 = 10 (the reference's 16/32/64/80 nets)

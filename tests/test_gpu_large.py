@@ -53,7 +53,8 @@ def fetch_planes(big, N, C, S, n, itemsize=4):
 CONVS = [  # name, Ci, Co, dims, N, stride, bits, gn, kernel name part
     ("wide", 128, 128, (16, 32, 32), 2000, 1, 8, False, "conv3_wide_k"),
     ("row", 96, 32, (8, 32, 32), 5400, 1, 8, False, "conv3_row_k"),
-    ("small", 32, 32, (16, 32, 32), 8000, 1, 8, False, "conv3_small_k"),
+    ("one-block row", 32, 32, (16, 32, 32), 8000, 1, 8, False, "conv3_row1_k"),
+    ("small", 32, 32, (16, 32, 16), 16000, 1, 8, False, "conv3_small_k"),
     ("general fp4 stride 2", 64, 64, (16, 32, 32), 7800, 2, 4, False, "stride 2"),
     ("direct fp4 stride 2", 64, 64, (16, 32, 32), 7800, 2, 4, False, "conv3s2_mx_k"),
     ("restaged GroupNorm input", 64, 64, (16, 16, 32), 8000, 1, 8, True, "conv3_"),

@@ -55,7 +55,7 @@ def test_static_scratch_conv_equals_the_allocating_entry(gpu):
     names = []
     # calls in a row on the shared array, every one smaller than or unlike the one before: wide kernel with a re-staged GroupNorm input,
     # then a smaller direct input, a fused-upsample split input (coarse rows + two staged segments), the same on rows of 32 voxels and a
-    # 32 -> 32 conv (the row kernel), the small-channel kernel, the tap-packed stem, an MX-fp4 conv, and the first shape again
+    # 32 -> 32 conv (the row kernels), the small-channel kernel, the tap-packed stem, an MX-fp4 conv, and the first shape again
     names.append(run_both(rng, 8, 2, 128, 128, 16, 32, 32, gn=True))
     names.append(run_both(rng, 8, 1, 128, 128, 8, 16, 32))
     names.append(run_both(rng, 8, 1, 96, 32, 8, 16, 16, up=1, Cu=64))
@@ -65,7 +65,7 @@ def test_static_scratch_conv_equals_the_allocating_entry(gpu):
     names.append(run_both(rng, 8, 2, 4, 32, 6, 16, 16, G=8))
     names.append(run_both(rng, 4, 1, 64, 64, 4, 8, 16, gn=True))
     names.append(run_both(rng, 8, 2, 128, 128, 16, 32, 32, gn=True))
-    assert any("conv3_wide_k" in n for n in names) and any("conv3_row_k" in n for n in names) and any("conv3_small_k" in n for n in names) and any("conv3_stem_k" in n for n in names)
+    assert any("conv3_wide_k" in n for n in names) and any("conv3_row_k" in n for n in names) and any("conv3_row1_k" in n for n in names) and any("conv3_small_k" in n for n in names) and any("conv3_stem_k" in n for n in names)
 
 
 def test_static_scratch_conv_refuses_what_does_not_fit(gpu):

@@ -189,7 +189,7 @@ static void conv_stats_reduce(const char *who, const conv_args &a, int MT, split
     fin.len = (double)(a.Co / a.Go) * (double)a.Do * a.Ho * a.Wo;
     if (fin.mean && (sp.zlo || sp.zhi)) mi_die("%s: fused finalize with a z range", who);
     if (a.stat_ch) gn_part_reduce_ch_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.ncs, a.Co, a.Go, osum, fin);
-    else gn_part_reduce_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.ncs, MT, a.Co, a.Go, osum, fin);
+    else gn_part_reduce_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N) * (a.row1 ? 8 : 1), a.ncs, MT, a.Co, a.Go, osum, fin);      // (row1: eight records per tile)
     MICK();
 }
 
@@ -240,7 +240,7 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
     if (!have) conv3_stem_prep(CP, w, wq, wsc, cout, Ci, nmt_all, NP);
     a.wq = wq; a.wsc = wsc;
     a.stat_ch = osum && (cout / Go) % 4 ? 1 : 0;
-    if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * (a.stat_ch ? 32 : MT * 8) * 2 * sizeof(float));
+    if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * (a.stat_ch ? 32 : a.row1 ? 64 : MT * 8) * 2 * sizeof(float));      // (row1: a record per wavefront, eight per tile)
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     const bool ktime = g_ktime && !mi_ws_arena_on();
     if (ktime) { MIRT(hipEventCreate(&ev0)); MIRT(hipEventCreate(&ev1)); MIRT(hipEventRecord(ev0, 0)); }
@@ -427,13 +427,18 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // registers, which measures a few percent faster there (both are bound by the halo's cache misses in flight, and it loads no weights)
     static int row_env = -1;
     if (row_env < 0) row_env = getenv("MI_CONV_ROW") ? atoi(getenv("MI_CONV_ROW")) : 1;      // tuning knob: 0 keeps the other kernels for these shapes, 2 also takes one input block
-    a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && nmt_all == 1 && stride == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 ? 1 : 2) && a.nbt <= 64;
+    // ... and one input block takes the row kernel's one-block form: weights in registers, the workgroup's two halves half a tile apart so that
+    // one half's epilogue runs under the other's MFMAs (MI_CONV_ROW1=0: the small-channel kernel)
+    static int row1_env = -1;
+    if (row1_env < 0) row1_env = getenv("MI_CONV_ROW1") ? atoi(getenv("MI_CONV_ROW1")) : 1;
+    a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && nmt_all == 1 && stride == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 || row1_env ? 1 : 2) && a.nbt <= 64;
+    a.row1 = a.row && a.nbt == 1 && row1_env && row_env < 2;
     if (a.row) { a.areg = false; a.CB = a.nbt; }
     size_t smem = a.row ? (size_t)2 * 2048 * (RB + 4) : a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     if (s2d) smem = 0;
     smem = (smem + 15) & ~(size_t)15;
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);      // bias, affine a, b of the workgroup's channels
-    a.red_o = (unsigned)smem; smem += 1024;                                     // statistics scratch
+    a.red_o = (unsigned)smem; smem += a.row1 ? 3 * 2048 + 3 * 1024 : 1024;      // statistics scratch (the one-block row kernel: the weight fragments of two tap classes instead)
     if (s2d) smem += (size_t)(27 * a.nbt + 1 + 8) * sizeof(int);                // the direct stride-2 kernel's K-order table
     if (big || a.areg || a.row) {
         // rows and scale bytes of positions outside the volume: 64 zero bytes, then 64 bytes of value 1; one page per device, kept for the process
@@ -488,7 +493,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     }
     a.wq = wq; a.wsc = wsc;
     a.stat_ch = osum && (cout / Go) % 4 ? 1 : 0;
-    if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * (a.stat_ch ? 32 : MT * 8) * 2 * sizeof(float));
+    if (osum) a.part = (float *)mi_ws(MI_WS_MISC, (size_t)a.ntiles * (a.stat_ch ? 32 : a.row1 ? 64 : MT * 8) * 2 * sizeof(float));      // (row1: a record per wavefront, eight per tile)
     const bool epi = act != 0;
     const int out = ybf == 3 ? 8 : ybf == 4 ? 4 : 0;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;

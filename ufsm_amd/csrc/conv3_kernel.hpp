@@ -119,6 +119,7 @@ struct conv_args {
     bool big;                          // the wide kernel takes the launch (MT 4, or MT 2 with NT 4)
     bool areg;                         // the persistent small-channel kernel (one channel tile, one input block, weights in registers) takes the launch
     bool row;                          // the row kernel (one channel tile, any number of input blocks, 4 x 8 x 32 voxel tiles) takes the launch
+    bool row1;                         // ... its one-input-block form (weights in registers, the two halves of the workgroup half a tile apart)
 };
 
 template <int FMT> struct fmt_t;
@@ -263,7 +264,9 @@ __device__ __forceinline__ void conv_epi_consts(const conv_args &a, unsigned cha
 // NOCH: this call takes no per-channel statistics records (the caller has checked stat_ch, or never sets it): their 32 sums are not kept
 // NW: wavefronts of the workgroup (their partial statistics are summed in wave order); ROW: the row kernel's voxel mapping, lane r of tile j
 // holds voxel (oz0 + lz, oy0 + ly0 + j, ox0 + r) of a 32-voxel run along x
-template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false, bool NOCH = false, int NW = 4, bool ROW = false>
+// WPART: every wavefront writes its own statistics record (record tile NW + wave: the reduce kernel then sees NW records per tile) and the
+// epilogue has no workgroup barrier and touches no LDS scratch, so the wavefronts of a workgroup need not run it at the same time (one channel tile)
+template <int MT, int NT, int OUT, bool EPI, bool PIN = false, bool W32 = false, bool FULL = false, bool NOCH = false, int NW = 4, bool ROW = false, bool WPART = false>
 __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT][NT], unsigned char *lds, unsigned tile, int n, int cs,
                                               int oz0, int oy0, int ox0, int lz, int ly0, int tid, const long long *ovx = nullptr) {
     const int lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
@@ -402,6 +405,17 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
         });
     });
     DBG_MARK(20);
+    if constexpr (WPART) {
+        static_assert(!WPART || (MT == 1 && NOCH), "per-wavefront statistics records: one channel tile, no per-channel records");
+        if (stats) {
+            float v[8];
+#pragma unroll
+            for (int q4 = 0; q4 < 4; q4++) { v[q4 * 2] = qs[0][q4]; v[q4 * 2 + 1] = qss[0][q4]; }
+            const int idx = wave_half_reduce<8>(v, r);
+            if ((r >> 3) == 0) a.part[(((size_t)tile * NW + wave) * 8 + 4 * h + (idx >> 1)) * 2 + (idx & 1)] = v[0];
+        }
+        return;
+    }
     if (stats) __syncthreads();
     DBG_MARK(21);
     if (CH && stats && a.stat_ch) {
@@ -636,6 +650,7 @@ static void launch_conv(const conv_args &a, size_t smem) {
 #include "conv3_wide.hpp"
 #include "conv3_small.hpp"
 #include "conv3_row.hpp"
+#include "conv3_row1.hpp"
 template <int FMT, int STRIDE, int OUT, bool EPI>
 static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     switch (MT * 10 + NT) {
@@ -649,7 +664,7 @@ static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     case 22: launch_conv<FMT, STRIDE, 2, 2, OUT, EPI>(a, smem); break;
     case 32: launch_conv<FMT, STRIDE, 3, 2, OUT, EPI>(a, smem); break;
     case 42: launch_conv<FMT, STRIDE, 4, 2, OUT, EPI>(a, smem); break;
-    case 14: if constexpr (STRIDE == 1) { if (a.row) launch_row<FMT, OUT, EPI>(a, smem); else if (a.areg) launch_small<FMT, 4, OUT, EPI>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
+    case 14: if constexpr (STRIDE == 1) { if (a.row1) launch_row1<FMT, OUT, EPI>(a, smem); else if (a.row) launch_row<FMT, OUT, EPI>(a, smem); else if (a.areg) launch_small<FMT, 4, OUT, EPI>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
     case 24: if constexpr (STRIDE == 1) { if (a.big) launch_wide<FMT, OUT, EPI, 2>(a, smem); else launch_conv<FMT, 1, 2, 4, OUT, EPI>(a, smem); break; }
     default: mi_die("conv3: no kernel for MT %d NT %d stride %d", MT, NT, STRIDE);
     }

@@ -1,0 +1,206 @@
+// The row kernel for ONE input block (<= 32 channels in, 17 .. 32 out; the 32 -> 32 convs of a U-Net's level 0): runs of 32 voxels along x as in
+// conv3_row.hpp (an input fragment read from LDS once serves the three ky taps: 0.5 fragment reads per MFMA, no bank conflicts), plus what one
+// block allows:
+//   * the weight fragments of the block stay with the wavefront for the whole persistent workgroup: the 9 pairs of tap classes 0 .. 2 in registers
+//     (72 of them; the E8M0 bytes of four pairs share a register and the MFMA's op_sel picks its byte), the 6 pairs of classes 3 and 4 in 9 KiB of
+//     LDS, read one class before their turn. The K loop issues no global loads but the next halo's copies. (All 15 pairs in registers leave the
+//     epilogue a dozen registers short, and a spilled register's reload waits for every copy in flight.)
+//   * the epilogue (as long as the tile's MFMAs here) runs in the shadow of MFMAs: the workgroup's eight wavefronts form two groups of four, one
+//     wavefront per SIMD each, group 1 owning rows 4 .. 7 of the tile and running HALF A TILE BEHIND group 0. While one of a SIMD's two wavefronts
+//     multiplies, the other converts and stores. The groups meet at one workgroup barrier per phase (two per tile); nothing else synchronises
+//     them: the epilogue keeps its statistics per wavefront (no LDS scratch, no barrier inside), and every wavefront copies its share of the
+//     next tile's halo from inside its own K loop, one copy round per tap class, into the buffer both groups left at least a phase earlier.
+// Barrier 0 ends the set-up. Group 0 runs its K loop K(t) between barriers 2t and 2t + 1 and its epilogue E(t) between 2t + 1 and 2t + 2; group 1
+// runs K(t) between 2t + 1 and 2t + 2 and E(t) between 2t + 2 and 2t + 3: every wavefront passes the same 2 (tiles) + 2 barriers. Tile t lives in
+// halo buffer t & 1, read from barrier 2t to 2t + 2; the copies of tile t + 1 are issued after barrier 2t (group 0) / 2t + 1 (group 1) into the
+// buffer last read before barrier 2t, and each wavefront waits for its own before the barrier that ends its K loop (2t + 1 / 2t + 2), ahead of the
+// first reader after barrier 2t + 2.
+// Measured against the small-channel kernel on the same box (32 -> 32, N 2 x 128^3): MX-fp8 0.135 - 0.139 against 0.146 - 0.150 ms, MX-fp4 0.091 -
+// 0.094 against 0.104 - 0.105 ms. Clock stamps of one workgroup: a K loop alone on its SIMD runs its 60 MFMAs in 4.0 K cycles (96 % of the matrix
+// pipe), with the copy requests inside 7.0 K (1.2 K their address arithmetic, 1.8 K the copies' issue stalls when the memory pipeline is backed
+// up), the epilogue 4.1 - 4.7 K. What was tried and lost: all copies issued in a burst at the start of an epilogue phase (by one group or split
+// over both: the issuing wavefront stalls 5 - 9 K cycles), whole 32-byte rows per lane pair (1 KiB contiguous reads; no gain).
+#pragma once
+
+#ifdef DBG_TIMING
+#define DBG_R1(i) do { if (blockIdx.x == 8 && it == 2 && (threadIdx.x & 255) == 0) g_dbg[(threadIdx.x >> 8) * 16 + (i)] = (long long)__builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define DBG_R1(i) do { } while (0)
+#endif
+template <int FMT, int OUT, bool EPI>
+__global__ void __launch_bounds__(512, 1) conv3_row1_k(const conv_args a) {
+    constexpr int NT = 4, TZ = 4, TY = 8, TX = 32, NW = 8;
+    constexpr int HZ = TZ + 2, HY = TY + 2, HX = TX + 2, TT = HZ * HY * HX, NH = fmt_t<FMT>::NH, WTILE = fmt_t<FMT>::WTILE;
+    constexpr int NG = (TT + 63) / 64, TTP = NG * 64;           // copy groups of 64 halo positions; positions per half padded to whole groups
+    constexpr int HB = NH * TTP * 16 + TTP * 4;                 // a halo buffer: rows [half][position][16 B], then one scale word per position
+    constexpr int NC = 5, NPB = 3 * NC;                         // tap classes; weight pairs of the block
+    constexpr int NRND = NG / NW;                               // copy rounds of a tile: in a round every wavefront copies one group
+    static_assert(NG % NW == 0 && NRND <= NC - 1, "every wavefront copies a group in every round, one round per tap class");
+    extern __shared__ __align__(16) unsigned char lds[];
+    const unsigned lds0 = (unsigned)(size_t)lds;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), r = lane & 31, h = lane >> 5;
+    const int grp = wave >> 2, lz = wave & 3, ly0 = grp * NT;   // group 0: wavefronts 0 .. 3 (one per SIMD), rows 0 .. 3 of the tile; group 1: rows 4 .. 7
+    const int p00 = (lz * HY + ly0) * HX + r;
+    const unsigned ab0 = ((NH == 2 ? h * TTP : 0) + p00) * 16, sb0 = NH * TTP * 16 + p00 * 4;
+    constexpr int DCL[3] = {1, HY * HX, 0};
+    const size_t Sin = (size_t)a.D * a.H * a.W;
+
+    const unsigned per = (a.ntiles + 7u) / 8u, wg_per_xcd = gridDim.x >> 3, xcd = blockIdx.x & 7u, wix = blockIdx.x >> 3;
+    struct tile_t { unsigned tile; int n, oz0, oy0, ox0; bool ok; };
+    auto decode = [&](unsigned it) {
+        tile_t t; const unsigned k = wix + it * wg_per_xcd;
+        t.ok = k < per && xcd * per + k < a.ntiles;
+        t.tile = t.ok ? xcd * per + k : 0u;
+        int tt = (int)t.tile;
+        const int tx = tt % a.ntx; tt /= a.ntx;
+        const int ty = tt % a.nty; tt /= a.nty;
+        const int tz = tt % a.ntz; t.n = tt / a.ntz;
+        t.ox0 = tx * TX; t.oy0 = ty * TY; t.oz0 = tz * TZ;
+        return t;
+    };
+    tile_t cur = decode(0);
+    if (!cur.ok) return;                                        // (uniform over the workgroup)
+
+    // copy round rd of tile t into the buffer at byte offset bo: this wavefront's group of 64 halo positions, the two row halves back to back and
+    // the scale bytes; positions outside the volume or past the halo read the constant page. No branch: `on` false reads the constant page
+    auto request = [&](const tile_t &t, unsigned bo, int g, bool on) {
+        const int z0 = t.oz0 - 1 + a.zi0, y0 = t.oy0 - 1, x0 = t.ox0 - 1;
+        int ln = lane;
+        asm volatile("" : "+v"(ln));                            // (opaque: the coordinates are formed per request, not kept in registers across the K loop)
+        const int pos = g * 64 + ln, pz = pos / (HY * HX), rem = pos - pz * (HY * HX), py = rem / HX, px = rem - py * HX;
+        const int gz = z0 + pz, gy = y0 + py, gx = x0 + px;
+        const bool in = on & (pos < TT) & ((unsigned)gz < (unsigned)a.D) & ((unsigned)gy < (unsigned)a.H) & ((unsigned)gx < (unsigned)a.W);
+        const int sp = (gz * a.H + gy) * a.W + gx;              // (garbage where !in: unused)
+        const size_t vox = (size_t)t.n * a.nbs[0] * Sin + (size_t)(in ? sp : 0);
+        const uint8_t *row = in ? a.xq[0] + vox * (16 * NH) : a.zpage, *sc = in ? a.xsc[0] + vox : a.zpage + 64;
+        dma16(row, lds0 + bo + (unsigned)g * 1024u);
+        if constexpr (NH == 2) dma16(row + 16, lds0 + bo + (unsigned)TTP * 16u + (unsigned)g * 1024u);
+        dma1(sc, lds0 + bo + (unsigned)(NH * TTP * 16) + (unsigned)g * 256u);
+    };
+    conv_epi_consts<1, EPI>(a, lds, 0, tid);
+    for (int rd = 0; rd < NRND; rd++) request(cur, 0u, NW * rd + wave, true);
+
+    // the block's weights: pair c 3 + ky of the prepared order (class c, ky), lane-ordered codes; the scale bytes of four pairs per register.
+    // Classes 0 .. 2 stay in registers. Classes 3 and 4 wait in LDS (3 x 2 KiB and, the second unit of class 4's pairs being the zero padding
+    // unit, 3 x 1 KiB) and are read one class before their turn: 36 registers that are then free while the epilogue runs, which is where the
+    // registers run out (a spilled register's reload waits for every copy in flight)
+    constexpr int NPR = 3 * (NC - 2);
+    v4i wlo[NPR], whi[FMT == 8 ? NPR : 1]; int wsb[(NPB + 3) / 4];
+    const unsigned w3_o = a.red_o, w4_o = a.red_o + 3 * 2048;   // (the statistics scratch: this kernel's epilogue keeps its sums per wavefront)
+    {
+        const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 256;
+        int sw[NPB];
+#pragma unroll
+        for (int p = 0; p < NPB; p++) {
+            const uint8_t *wp = a.wq + (size_t)p * wq_ps + lane * 16;
+            if (p < NPR) { wlo[p] = *(const v4i *)wp; if (FMT == 8) whi[p] = *(const v4i *)(wp + 1024); }
+            else if (p < NPR + 3) {                             // class 3: wavefronts 0 .. 5 copy its six 1 KiB pieces (uniform per wavefront)
+                if (wave == 2 * (p - NPR)) dma16(wp, lds0 + w3_o + (unsigned)(p - NPR) * 2048u);
+                if (FMT == 8 && wave == 2 * (p - NPR) + 1) dma16(wp + 1024, lds0 + w3_o + (unsigned)(p - NPR) * 2048u + 1024u);
+            } else if (wave == p - NPR - 3) dma16(wp, lds0 + w4_o + (unsigned)(p - NPR - 3) * 1024u);
+            sw[p] = *(const int *)(a.wsc + (size_t)p * wsc_ps + lane * 4);
+        }
+#pragma unroll
+        for (int q = 0; q < (NPB + 3) / 4; q++) {
+            wsb[q] = 0;
+#pragma unroll
+            for (int k = 0; k < 4; k++) if (4 * q + k < NPB) wsb[q] |= (sw[4 * q + k] & 255) << (8 * k);
+        }
+    }
+    wait_vm<0>();
+    __syncthreads();                                            // barrier 0: the first halo and the epilogue's constants are in LDS
+    if (grp) __syncthreads();                                   // group 1 starts half a tile later (barrier 1)
+
+    for (unsigned it = 0;; it++) {
+        const tile_t nxt = decode(it + 1);
+        const unsigned hb = (it & 1u) * (unsigned)HB;
+        const unsigned abt = hb + ab0, sbt = hb + sb0;
+        unsigned abh[3], sbh[3];
+#pragma unroll
+        for (int k = 0; k < 3; k++) { abh[k] = abt + (h ? DCL[k] * 16 : 0); sbh[k] = sbt + (h ? DCL[k] * 4 : 0); }
+        struct frag { v4i lo, hi; int sb; };
+        auto fetch = [&](auto C, auto S) {
+            constexpr int c = decltype(C)::value, s = decltype(S)::value;
+            constexpr int kzA = c < 3 ? c : c == 3 ? 0 : 2, kxA = c < 3 ? 0 : 2, dk = c < 3 ? 0 : c == 3 ? 1 : 2;
+            constexpr int pA = (kzA * HY + s) * HX + kxA, pB = pA + DCL[dk];
+            frag f;
+            if constexpr (FMT == 8) { f.lo = *(const v4i *)(lds + abt + pA * 16); f.hi = *(const v4i *)(lds + abt + pB * 16); }
+            else { f.lo = *(const v4i *)(lds + abh[dk] + pA * 16); f.hi = (v4i){0, 0, 0, 0}; }
+            f.sb = *(const int *)(lds + sbh[dk] + pA * 4);
+            return f;
+        };
+        // ---- K loop: NC x (NT + 2) row visits as one basic block; visit (c, s) requests the fragment two visits ahead and multiplies its own by
+        // the ky weights of the rows it reaches (j = s - ky); the next tile's copy rounds are issued at fixed visits ----
+        DBG_R1(0);
+        v16f acc[1][NT];
+        constexpr int NR = NT + 2, NV = NC * NR, PF = 2;
+        {
+            frag fr[PF + 1];
+            v4i w3lo[3], w3hi[3], w4[3];                        // the weight fragments of classes 3 and 4, read from LDS one class ahead
+            static_for<PF>([&](auto V) { constexpr int v = decltype(V)::value; fr[v] = fetch(std::integral_constant<int, v / NR>{}, std::integral_constant<int, v % NR>{}); });
+            static_for<NV>([&](auto V) {
+                constexpr int v = decltype(V)::value, c = v / NR, s = v % NR, set = v % (PF + 1);
+                if constexpr (v + PF < NV) fr[(v + PF) % (PF + 1)] = fetch(std::integral_constant<int, (v + PF) / NR>{}, std::integral_constant<int, (v + PF) % NR>{});
+                if constexpr (c == NC - 3 && s == 2) {
+#pragma unroll
+                    for (int k = 0; k < 3; k++) { w3lo[k] = *(const v4i *)(lds + w3_o + k * 2048 + lane * 16); if (FMT == 8) w3hi[k] = *(const v4i *)(lds + w3_o + k * 2048 + 1024 + lane * 16); }
+                }
+                if constexpr (c == NC - 2 && s == 2) {
+#pragma unroll
+                    for (int k = 0; k < 3; k++) w4[k] = *(const v4i *)(lds + w4_o + k * 1024 + lane * 16);
+                }
+                if constexpr (s == 1 && c < NRND) request(nxt, (unsigned)HB - hb, NW * c + wave, nxt.ok);
+                const v8i fb = FMT == 8 ? (v8i){fr[set].lo[0], fr[set].lo[1], fr[set].lo[2], fr[set].lo[3], fr[set].hi[0], fr[set].hi[1], fr[set].hi[2], fr[set].hi[3]}
+                                        : (v8i){fr[set].lo[0], fr[set].lo[1], fr[set].lo[2], fr[set].lo[3], 0, 0, 0, 0};
+                static_for<3>([&](auto KY) {
+                    constexpr int ky = decltype(KY)::value, j = s - ky, p = c * 3 + ky;
+                    if constexpr (j >= 0 && j < NT) {
+                        const v16f c0 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                        // (row j's first product is class 0's: visit (0, j + ky) with ky = 0 comes first for j = s)
+                        v8i wa;
+                        if constexpr (p < NPR) wa = FMT == 8 ? (v8i){wlo[p][0], wlo[p][1], wlo[p][2], wlo[p][3], whi[FMT == 8 ? p : 0][0], whi[FMT == 8 ? p : 0][1], whi[FMT == 8 ? p : 0][2], whi[FMT == 8 ? p : 0][3]}
+                                                             : (v8i){wlo[p][0], wlo[p][1], wlo[p][2], wlo[p][3], 0, 0, 0, 0};
+                        else if constexpr (p < NPR + 3) wa = FMT == 8 ? (v8i){w3lo[p - NPR][0], w3lo[p - NPR][1], w3lo[p - NPR][2], w3lo[p - NPR][3], w3hi[p - NPR][0], w3hi[p - NPR][1], w3hi[p - NPR][2], w3hi[p - NPR][3]}
+                                                                          : (v8i){w3lo[p - NPR][0], w3lo[p - NPR][1], w3lo[p - NPR][2], w3lo[p - NPR][3], 0, 0, 0, 0};
+                        else wa = (v8i){w4[p - NPR - 3][0], w4[p - NPR - 3][1], w4[p - NPR - 3][2], w4[p - NPR - 3][3], 0, 0, 0, 0};
+                        acc[0][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(wa, fb, (c == 0 && ky == 0) ? c0 : acc[0][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4,
+                                                                                    p % 4, wsb[p / 4], 0, fr[set].sb);
+                    }
+                });
+                static_for<3>([&](auto KY) { constexpr int j = s - decltype(KY)::value; if constexpr (j >= 0 && j < NT) row_pin(acc[0][j]); });
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        }
+        DBG_R1(1);
+        wait_vm<0>();                                           // this wavefront's copies of the next tile's halo have landed
+        DBG_R1(2);
+        __syncthreads();                                        // end of this group's K phase (barrier 2 it + 1 for group 0, 2 it + 2 for group 1)
+        DBG_R1(3);
+        if (cur.oz0 + TZ <= a.Do && cur.oy0 + TY <= a.Ho && cur.ox0 + TX <= a.Wo && a.zs0 <= cur.oz0 && a.zs1 >= cur.oz0 + TZ)      // (uniform)
+            conv_epilogue<1, NT, OUT, EPI, false, true, true, true, NW, true, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+        else conv_epilogue<1, NT, OUT, EPI, false, true, false, true, NW, true, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+        DBG_R1(4);
+        __syncthreads();                                        // end of this group's epilogue phase (barrier 2 it + 2 / 2 it + 3)
+        DBG_R1(5);
+        if (!nxt.ok) break;
+        cur = nxt;
+    }
+    if (!grp) __syncthreads();                                  // group 0 waits out group 1's last epilogue phase: every wavefront has passed the same barriers
+}
+
+template <int FMT, int OUT, bool EPI>
+static void launch_row1(const conv_args &a, size_t smem) {
+    static bool attr[8]; static int ncu[8];
+    int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
+    if (!attr[d]) {
+        MIRT(hipFuncSetAttribute((const void *)conv3_row1_k<FMT, OUT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        hipDeviceProp_t pr; MIRT(hipGetDeviceProperties(&pr, d));
+        ncu[d] = pr.multiProcessorCount > 8 ? pr.multiProcessorCount & ~7 : 8;
+        attr[d] = true;
+    }
+    const unsigned per = (a.ntiles + 7u) / 8u;            // tiles per XCD; one persistent workgroup per CU, a multiple of 8 in all
+    const unsigned nwg = per * 8u < (unsigned)ncu[d] ? per * 8u : (unsigned)ncu[d];
+    conv3_row1_k<FMT, OUT, EPI><<<nwg, 512, smem>>>(a);
+    MICK();
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row1_k<fmt %d, out %d, epi %d> tiles %u wgs %u", FMT, OUT, (int)EPI, a.ntiles, nwg);
+}
