@@ -440,6 +440,11 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);      // bias, affine a, b of the workgroup's channels
     a.red_o = (unsigned)smem; smem += a.row1 ? 3 * 2048 + 3 * 1024 : 1024;      // statistics scratch (the one-block row kernel: the weight fragments of two tap classes instead)
     if (s2d) smem += (size_t)(27 * a.nbt + 1 + 8) * sizeof(int);                // the direct stride-2 kernel's K-order table
+    // the row kernel in e2m1: the prepared weights of up to four input blocks stay in LDS (MI_CONV_ROW_WL=0: loaded from global memory per tap class)
+    static int wl_env = -1;
+    if (wl_env < 0) wl_env = getenv("MI_CONV_ROW_WL") ? atoi(getenv("MI_CONV_ROW_WL")) : 1;
+    a.wl_o = 0;
+    if (a.row && !a.row1 && fmt == 4 && wl_env && smem + (size_t)a.nbt * 15 * 1280 <= 160 * 1024) { a.wl_o = (unsigned)smem; smem += (size_t)a.nbt * 15 * 1280; }
     if (big || a.areg || a.row) {
         // rows and scale bytes of positions outside the volume: 64 zero bytes, then 64 bytes of value 1; one page per device, kept for the process
         // (the entry point that must not allocate keeps its own at the head of its fixed scratch)

@@ -109,6 +109,7 @@ struct conv_args {
     const float *ep_a, *ep_b; int act;
     unsigned epi_o;                    // LDS byte offset of the epilogue's per-channel constants: bias, then ep_a, ep_b (MT x 32 floats each)
     unsigned red_o;                    // LDS byte offset of the statistics scratch (1 KiB)
+    unsigned wl_o;                     // row kernel, weights resident in LDS: byte offset of their image (per pair 1 KiB of codes + 64 scale words; 0: loaded from global memory)
     const uint8_t *zpage;              // device memory: 64 zero bytes, then 64 bytes of value 1 (rows and scale bytes of positions outside the volume)
     int ntx, nty, ntz, ncs; unsigned ntiles;
     // tap-packed stem only: the input as stored (0 fp32 planes, 2 fp16 planes, 3 MX-fp8, 4 MX-fp4: one row of 8 channels per voxel) and its GroupNorm
@@ -664,7 +665,7 @@ static void launch_mt(int MT, int NT, const conv_args &a, size_t smem) {
     case 22: launch_conv<FMT, STRIDE, 2, 2, OUT, EPI>(a, smem); break;
     case 32: launch_conv<FMT, STRIDE, 3, 2, OUT, EPI>(a, smem); break;
     case 42: launch_conv<FMT, STRIDE, 4, 2, OUT, EPI>(a, smem); break;
-    case 14: if constexpr (STRIDE == 1) { if (a.row1) launch_row1<FMT, OUT, EPI>(a, smem); else if (a.row) launch_row<FMT, OUT, EPI>(a, smem); else if (a.areg) launch_small<FMT, 4, OUT, EPI>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
+    case 14: if constexpr (STRIDE == 1) { if (a.row1) launch_row1<FMT, OUT, EPI>(a, smem); else if (a.row) { if constexpr (FMT == 4) { if (a.wl_o) { launch_row<FMT, OUT, EPI, true>(a, smem); break; } } launch_row<FMT, OUT, EPI, false>(a, smem); } else if (a.areg) launch_small<FMT, 4, OUT, EPI>(a, smem); else launch_conv<FMT, 1, 1, 4, OUT, EPI>(a, smem); break; }
     case 24: if constexpr (STRIDE == 1) { if (a.big) launch_wide<FMT, OUT, EPI, 2>(a, smem); else launch_conv<FMT, 1, 2, 4, OUT, EPI>(a, smem); break; }
     default: mi_die("conv3: no kernel for MT %d NT %d stride %d", MT, NT, STRIDE);
     }

@@ -21,8 +21,11 @@
 
 __device__ __forceinline__ void row_pin(v16f &x) { asm volatile("" : "+v"(x)::"memory"); }
 
-template <int FMT, int OUT, bool EPI>
+// WL (MX-fp4 only): the prepared weights of all input blocks are copied into LDS once per workgroup (19 200 bytes per block: an e2m1 fragment is half
+// an e4m3 one, and the halo buffers are half as large) and the K loop reads its fragments from there: no global loads but the halo's copies
+template <int FMT, int OUT, bool EPI, bool WL = false>
 __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
+    static_assert(!WL || FMT == 4, "weights resident in LDS: the e2m1 form");
     constexpr int NT = 4, TZ = 4, TY = 8, TX = 32, NW = 8;
     constexpr int HZ = TZ + 2, HY = TY + 2, HX = TX + 2, TT = HZ * HY * HX, NH = fmt_t<FMT>::NH, WTILE = fmt_t<FMT>::WTILE;
     constexpr int NG = (TT + 63) / 64, TTP = NG * 64;           // copy groups of 64 halo positions; positions per half padded to whole groups
@@ -88,8 +91,27 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
 
     // the weight fragments of one tap class of input block b: three pairs (ky 0, 1, 2), lane-ordered codes and the lane's scale word
     struct wcl { v8i f[3]; int s[3]; };
+    constexpr int WPB = 1024 + 256;                             // (WL) bytes of a pair in LDS: the lanes' 16 bytes of codes, then their scale words
+    if constexpr (WL) {                                         // every pair of every block: 80 16-byte pieces, copied by the whole workgroup
+        const size_t wq_ps0 = (size_t)a.nmt_all * WTILE, wsc_ps0 = (size_t)a.nmt_all * 256;
+        for (int i = tid; i < a.nbt * NPB * (WPB / 16); i += NW * 64) {
+            const int p = i / (WPB / 16), k = i - p * (WPB / 16);
+            const v4i v = k < 64 ? *(const v4i *)(a.wq + (size_t)p * wq_ps0 + k * 16) : *(const v4i *)(a.wsc + (size_t)p * wsc_ps0 + (k - 64) * 16);
+            *(v4i *)(lds + a.wl_o + p * WPB + k * 16) = v;
+        }
+    }
     auto wload = [&](int b, int c) {
         wcl w;
+        if constexpr (WL) {
+            const unsigned o = a.wl_o + (unsigned)((b * NPB + c * 3) * WPB);
+#pragma unroll
+            for (int ky = 0; ky < 3; ky++) {
+                const v4i lo = *(const v4i *)(lds + o + ky * WPB + lane * 16);
+                w.f[ky] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+                w.s[ky] = *(const int *)(lds + o + ky * WPB + 1024 + lane * 4);
+            }
+            return w;
+        }
         const uint8_t *wp = a.wq + ((size_t)b * NPB + c * 3) * wq_ps + lane * 16, *sp = a.wsc + ((size_t)b * NPB + c * 3) * wsc_ps + lane * 4;
 #pragma unroll
         for (int ky = 0; ky < 3; ky++) {
@@ -104,6 +126,7 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
     // step's classes 0 and 1) loads into the set class c - 1 has just left; the next step's first two classes land in sets 2 and 0 and are moved
     // to their places (0 and 1) at the step's end
     wcl ws[3];
+    if constexpr (WL) { wait_vm<0>(); __syncthreads(); }        // (the weights' image is complete before anyone reads it)
     ws[0] = wload(0, 0);
     ws[1] = wload(0, 1);
     wait_vm<0>();
@@ -186,19 +209,19 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
     }
 }
 
-template <int FMT, int OUT, bool EPI>
+template <int FMT, int OUT, bool EPI, bool WL>
 static void launch_row(const conv_args &a, size_t smem) {
     static bool attr[8]; static int ncu[8];
     int d = 0; MIRT(hipGetDevice(&d)); d &= 7;
     if (!attr[d]) {
-        MIRT(hipFuncSetAttribute((const void *)conv3_row_k<FMT, OUT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        MIRT(hipFuncSetAttribute((const void *)conv3_row_k<FMT, OUT, EPI, WL>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         hipDeviceProp_t pr; MIRT(hipGetDeviceProperties(&pr, d));
         ncu[d] = pr.multiProcessorCount > 8 ? pr.multiProcessorCount & ~7 : 8;
         attr[d] = true;
     }
     const unsigned per = (a.ntiles + 7u) / 8u;            // tiles per XCD; one persistent workgroup per CU, a multiple of 8 in all
     const unsigned nwg = per * 8u < (unsigned)ncu[d] ? per * 8u : (unsigned)ncu[d];
-    conv3_row_k<FMT, OUT, EPI><<<nwg, 512, smem>>>(a);
+    conv3_row_k<FMT, OUT, EPI, WL><<<nwg, 512, smem>>>(a);
     MICK();
-    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row_k<fmt %d, out %d, epi %d> blocks %d tiles %u wgs %u", FMT, OUT, (int)EPI, a.nbt, a.ntiles, nwg);
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row_k<fmt %d, out %d, epi %d%s> blocks %d tiles %u wgs %u", FMT, OUT, (int)EPI, WL ? ", weights in LDS" : "", a.nbt, a.ntiles, nwg);
 }
