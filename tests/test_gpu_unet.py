@@ -614,6 +614,28 @@ def test_unet_l0_norm_slab(gpu, tmp_path, bits, widths, dims, N, slab, infer):
     net.close()
 
 
+def test_unet_l0_norm_slab_single_slab_is_plain_groupnorm(gpu):
+    """cfg.l0_norm 4 on a window of at most one statistics slab's depth: ceil(depth / slab) = 1 slab, which is the sample, so nothing is
+    registered and level 0 runs ordinary GroupNorm on the convs' own statistics (src/unet.c:1004, :2336, :2364): the logits of the plain
+    net, byte for byte - for a window shallower than the slab, and for one exactly as deep."""
+    from ufsm_amd.unet import UNet, make_cfg
+    rng = np.random.default_rng(77)
+    cin, widths, head_out, N = 4, [32, 64], 2, 1
+    for D, slab in ((16, 64), (16, 16)):
+        H = W = 16
+        S = D * H * W
+        x = rng.standard_normal((N, cin, S)).astype(np.float32)
+        dxq = to_mx(8, x)
+        plain = UNet(make_cfg(cin, widths, head_out=head_out), N, D, H, W, seed=5)
+        slabn = UNet(make_cfg(cin, widths, head_out=head_out, l0_norm=4, l0_slab=slab), N, D, H, W, seed=5)
+        assert np.array_equal(plain.params(), slabn.params())
+        d0, d1 = DevBuf(N * head_out * S * 4), DevBuf(N * head_out * S * 4)
+        assert plain.forward_x(dxq.ptr, d0.ptr) == 0 and slabn.forward_x(dxq.ptr, d1.ptr) == 0
+        LP.check()
+        assert np.array_equal(d0.to_numpy(np.uint8), d1.to_numpy(np.uint8))
+        plain.close(); slabn.close()
+
+
 def ws_f64(w, gain, eps=1e-5):
     """scaled weight standardisation per output channel over its fan-in (src/nn_l0norm.cu:45-63), numpy fp64"""
     w2 = w.reshape(w.shape[0], -1).astype(np.float64)
@@ -1208,6 +1230,22 @@ def test_unet_gn_ema(gpu, tmp_path, widths, dn, attn):
     assert net.save(path, step=5, extra="{}") == 0
     head2 = open(path, "rb").readline().decode()
     assert ',"ge_n":7,"ge_warm":500,' in head2 and ("%.9g" % runs[1][-1]) in head2
+    # a value that is not finite in one copy is taken from the other copy; one that is finite in neither drops the statistics
+    def with_runs(a, b):
+        txt = ",".join(("%.9g" % v) if np.isfinite(v) else "inf" for v in np.concatenate([a, b]))
+        open(path, "wb").write((head[:i0] + ',"ge_n":7,"ge_warm":500,"ge_mom":0.01,"ge_run":[' + txt + "]" + head[i1:]).encode() + raw[len(head.encode()):])
+    hurt = [r.copy() for r in runs]; hurt[0][3] = np.inf; hurt[1][ns - 2] = np.inf
+    with_runs(*hurt)
+    assert net.load(path) == 4 and H0.unet_gn_ema_updates(net.h) == 7
+    assert net.save(path, step=6, extra="{}") == 0
+    h3 = open(path, "rb").readline().decode(); a3 = h3.index('"ge_run":[') + 10
+    back = np.array([float(t) for t in h3[a3:h3.index("]", a3)].split(",")], np.float32)
+    mend = [r.copy() for r in runs]; mend[0][3] = runs[1][3]; mend[1][ns - 2] = runs[0][ns - 2]
+    assert np.array_equal(back, np.concatenate(mend))
+    hurt[1][3] = np.inf
+    with_runs(*hurt)
+    assert net.load(path) == 4 and H0.unet_gn_ema_updates(net.h) == 0
+    assert np.array_equal(run(net), ref)                            # no statistics: the window's own
     plain.close(); net.close()
 
 

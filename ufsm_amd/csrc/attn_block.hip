@@ -277,8 +277,8 @@ __global__ void __launch_bounds__(256) peg_rows_k(const float *__restrict__ x, f
     if (ts < 0) { ((float4 *)y)[i] = xv; return; }
     const size_t row0 = t - (size_t)ts;                            // the sequence's first grid token
     const int z = ts / (Hh * W), yy = (ts / W) % Hh, xx = ts % W;
-    const float4 bv = ((const float4 *)b)[c4];
-    float a[4] = {xv.x + bv.x, xv.y + bv.y, xv.z + bv.z, xv.w + bv.w};
+    const float *bc = b + (size_t)c4 * 4;                          // (scalar loads: the bias sits at any float offset of the parameter vector, not at a multiple of 16 bytes)
+    float a[4] = {xv.x + bc[0], xv.y + bc[1], xv.z + bc[2], xv.w + bc[3]};
     const float *wc = w + (size_t)c4 * 4 * 27;
     for (int dz = -1; dz <= 1; dz++) for (int dy = -1; dy <= 1; dy++) for (int dx = -1; dx <= 1; dx++) {
         const int zz = z + dz, y2 = yy + dy, x2 = xx + dx;

@@ -100,7 +100,8 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
             *(v4i *)(lds + a.wl_o + p * WPB + k * 16) = v;
         }
     }
-    auto wload = [&](int b, int c) {
+    auto wload = [&](int b, auto C) {
+        constexpr int c = decltype(C)::value;
         wcl w;
         if constexpr (WL) {
             const unsigned o = a.wl_o + (unsigned)((b * NPB + c * 3) * WPB);
@@ -116,7 +117,8 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
 #pragma unroll
         for (int ky = 0; ky < 3; ky++) {
             const v4i lo = *(const v4i *)(wp + ky * wq_ps);
-            if (FMT == 8) { const v4i hi = *(const v4i *)(wp + ky * wq_ps + 1024); w.f[ky] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; }
+            // (e4m3: the pair's second unit; class 4's is the zero padding unit and is not loaded)
+            if (FMT == 8 && c != NC - 1) { const v4i hi = *(const v4i *)(wp + ky * wq_ps + 1024); w.f[ky] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; }
             else w.f[ky] = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
             w.s[ky] = *(const int *)(sp + ky * wsc_ps);
         }
@@ -127,8 +129,8 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
     // to their places (0 and 1) at the step's end
     wcl ws[3];
     if constexpr (WL) { wait_vm<0>(); __syncthreads(); }        // (the weights' image is complete before anyone reads it)
-    ws[0] = wload(0, 0);
-    ws[1] = wload(0, 1);
+    ws[0] = wload(0, std::integral_constant<int, 0>{});
+    ws[1] = wload(0, std::integral_constant<int, 1>{});
     wait_vm<0>();
     __syncthreads();
 
@@ -172,7 +174,7 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
                 constexpr int v = decltype(V)::value, c = v / NR, s = v % NR, set = v % (PF + 1);
                 if constexpr (v + PF < NV) fr[(v + PF) % (PF + 1)] = fetch(std::integral_constant<int, (v + PF) / NR>{}, std::integral_constant<int, (v + PF) % NR>{});
                 if constexpr (s == 0) {                          // the weights two classes ahead (past the last step: block 0 again, unused)
-                    if constexpr (c + 2 < NC) ws[CSET[c + 2]] = wload(b, c + 2); else ws[c + 2 == NC ? 2 : 0] = wload(nb, c + 2 - NC);
+                    if constexpr (c + 2 < NC) ws[CSET[c + 2]] = wload(b, std::integral_constant<int, (c + 2) % NC>{}); else ws[c + 2 == NC ? 2 : 0] = wload(nb, std::integral_constant<int, (c + 2) % NC>{});
                 }
                 if constexpr (s == 1 && c < NRND) request(nxt, nb, (unsigned)HB - hb, c, more);
                 const v8i fb = FMT == 8 ? (v8i){fr[set].lo[0], fr[set].lo[1], fr[set].lo[2], fr[set].lo[3], fr[set].hi[0], fr[set].hi[1], fr[set].hi[2], fr[set].hi[3]}

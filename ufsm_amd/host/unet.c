@@ -250,12 +250,15 @@ static int build_acts(unet *u, shape5 in) {
     if (in.n < 1 || in.c != cfg->cin || in.d < 1 || in.h < 1 || in.w < 1) { fprintf(stderr, "unet: input shape %d x %d x %d x %d x %d does not fit a net of %d input channels\n", in.n, in.c, in.d, in.h, in.w, cfg->cin); return -1; }
     if ((in.d | in.h | in.w) & ((1 << (L - 1)) - 1)) { fprintf(stderr, "unet: spatial size %dx%dx%d must be divisible by %d\n", in.d, in.h, in.w, 1 << (L - 1)); abort(); }   /* (src/unet.c:2875) */
     if (!unet_act_mx()) { fprintf(stderr, "unet: this build stores activations as MX-fp8 or MX-fp4 only (unet_set_act_mx8 / unet_set_act_mx4)\n"); return -1; }
-    if (cfg->l0_norm == 4 && in.d % (cfg->l0_slab > 0 ? cfg->l0_slab : 64)) { fprintf(stderr, "unet: l0_norm 4 needs a depth (%d) that is a multiple of the %d planes of a statistics slab\n", in.d, cfg->l0_slab > 0 ? cfg->l0_slab : 64); return -1; }
+    /* cfg.l0_norm 4: ceil(depth / slab) statistics slabs (src/unet.c:1004). Several slabs must be uniform; a window of at most one slab's depth has a
+       single slab, which is the sample: nothing is registered and level 0 runs ordinary GroupNorm on the convs' own statistics (src/unet.c:2336, :2364) */
+    const int l0_S = cfg->l0_norm == 4 ? (cfg->l0_slab > 0 ? cfg->l0_slab : 64) : 0, l0_ns = l0_S ? (in.d + l0_S - 1) / l0_S : 0;
+    if (l0_ns > 1 && in.d % l0_S) { fprintf(stderr, "unet: l0_norm 4 needs a depth (%d) that is a multiple of the %d planes of a statistics slab (or at most one slab)\n", in.d, l0_S); return -1; }
     free_acts(u);
     u->in = in; u->act_dt = act_dt_now(); u->prec = nn_get_prec();
     /* cfg.l0_norm 4 (src/unet.h:52-59; the kernel path of src/unet.c:992-1003): the four GroupNorms of level 0 take their statistics per z-slab of
        l0_slab planes (0: 64). The statistics arrays hold [n][slab][G] and are registered with their geometry, which every reader's gnp_t then carries */
-    u->l0s_zs = cfg->l0_norm == 4 ? (cfg->l0_slab > 0 ? cfg->l0_slab : 64) : 0; u->l0s_ns = u->l0s_zs ? in.d / u->l0s_zs : 0;
+    u->l0s_ns = l0_ns > 1 ? l0_ns : 0; u->l0s_zs = u->l0s_ns ? l0_S : 0;
     u->slab_ip = slab_inplace_now(u); u->slab_nl = u->slab_ip ? slab_levels(u) : 0; u->slab_s = u->slab_ip ? g_infer_slab : 0;
     /* (a level shares one buffer only if its decoder block has the encoder's width and two convs: the reference's slab_w_ok / any_single
        conditions, src/unet.c:1163; the levels that do not qualify run the direct form) */
@@ -801,9 +804,22 @@ int unet_load(unet *u, const char *path) {
         if (l0.cnt == n) { mi_h2d(u->l0run, l0.run, (size_t)n * 4); u->l0_n = l0.n; u->l0_warm = l0.warm; u->l0_mom = l0.mom; }
         else { mi_zero(u->l0run, (size_t)n * 4); u->l0_n = 0; }
     }
-    if (rc >= 0 && u->cfg.gn_ema) {                                /* a checkpoint without the statistics, or with non-finite ones: live statistics until a trainer has made some (src/unet.c:5846-5860) */
+    if (rc >= 0 && u->cfg.gn_ema) {
+        /* The file holds two copies of the running statistics, the live weights' and the EMA weights'. A value that is not finite in one copy is
+           taken from the other; only when some value is finite in neither, or the count does not fit the net, the statistics are dropped and the
+           sites read the window's own until a trainer has made new ones (src/unet.c:5846-5860) */
         int ok = l0.gcnt == (int)(2 * u->ge_ns);
-        for (int i = 0; ok && i < l0.gcnt; i++) ok = isfinite(l0.grun[i]);
+        if (ok) {
+            const size_t ns = u->ge_ns; size_t bad = 0, mended = 0;
+            for (size_t i = 0; i < ns; i++) {
+                float *live = &l0.grun[i], *avg = &l0.grun[ns + i];
+                const int fl = isfinite(*live), fa = isfinite(*avg);
+                bad += !fl + !fa;
+                if (!fl && fa) { *live = *avg; mended++; } else if (fl && !fa) { *avg = *live; mended++; }
+            }
+            if (bad) fprintf(stderr, "unet_load: gn_ema: %zu running statistics of %s are not finite, %zu taken from the other copy%s\n", bad, path, mended, mended < bad ? ": statistics dropped" : "");
+            ok = mended == bad;
+        }
         if (ok) { mi_h2d(u->ge_run, l0.grun, (size_t)l0.gcnt * 4); u->ge_n = l0.gn; u->ge_warm = l0.gwarm; u->ge_mom = l0.gmom; }
         else { mi_zero(u->ge_run, 2 * u->ge_ns * 4); u->ge_n = 0; }
     }
@@ -850,12 +866,11 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     if (u->cfg.gfilm) fputs(",\"gfilm\":1", f);                    /* (src/unet.c:5588) */
     if (u->cfg.gn_ema) {                                           /* every site's running statistics and their state (src/unet.c:5587-5592; written after l0_norm's keys there too) */
         float *r = malloc(2 * u->ge_ns * 4);
-        if (r) {
-            mi_d2h(r, u->ge_run, 2 * u->ge_ns * 4);
-            fprintf(f, ",\"gn_ema\":1,\"ge_n\":%ld,\"ge_warm\":%d,\"ge_mom\":%.9g,\"ge_run\":[", u->ge_n, u->ge_warm, (double)u->ge_mom);
-            for (size_t i = 0; i < 2 * u->ge_ns; i++) fprintf(f, "%s%.9g", i ? "," : "", (double)r[i]);
-            fputc(']', f); free(r);
-        }
+        if (!r) { fprintf(stderr, "unet_save: out of memory for the running statistics: %s not written\n", path); fclose(f); remove(tmp); free(h); free(he); return -1; }      /* (a file without them would load as a fresh warm-up) */
+        mi_d2h(r, u->ge_run, 2 * u->ge_ns * 4);
+        fprintf(f, ",\"gn_ema\":1,\"ge_n\":%ld,\"ge_warm\":%d,\"ge_mom\":%.9g,\"ge_run\":[", u->ge_n, u->ge_warm, (double)u->ge_mom);
+        for (size_t i = 0; i < 2 * u->ge_ns; i++) fprintf(f, "%s%.9g", i ? "," : "", (double)r[i]);
+        fputc(']', f); free(r);
     }
     if (u->cfg.l0_norm == 2) {                                     /* the running statistics and their state (src/unet.c:5579-5584) */
         const int n = 16 * G_of(u, u->cfg.widths[0]); float r[1024];
