@@ -436,6 +436,32 @@ def test_nonfinite_input_propagates(gpu):
     assert np.array_equal(bad, exp)
 
 
+def test_config0_full_size_against_oracle(gpu):
+    """The reference's CPU-runnable case at its full size: one 3x3x3 conv 32 -> 32, N 1, 64^3, seed 0, activations N(0, 1) as fp32 planes
+    (quantised to MX-fp8 per 32 channels while staging), Kaiming weights, no bias, fp16 planes out, through lp_conv_fwd_f8 - the call the
+    benchmark's c0 record times. Against the oracle's fp32-accumulated conv of the same operands: the north-star tolerance of 1e-3 max-abs-rel
+    on the binary16 result (whose own rounding is 4.9e-4 relative per value), and at most one binary16 step between any two values."""
+    N, Cc, D = 1, 32, 64
+    S = D ** 3
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((N, Cc, S)).astype(np.float32)
+    w = (rng.standard_normal((Cc, Cc, 27)) * np.sqrt(2.0 / (Cc * 27))).astype(np.float32)
+    want, _ = orc.conv3(x, 0, N, Cc, D, D, D, w, None, Cc, 2, cbits=8)
+    got, _ = gpu_conv(x, 0, N, Cc, D, D, D, w, None, Cc, 2, cbits=8)
+    assert "conv3_row1_k<fmt 8, out 0" in lib.mi_last_kernel().decode(), lib.mi_last_kernel().decode()
+    g = got.view(np.float16).astype(np.float32).reshape(N, Cc, S); q = want.view(np.float16).astype(np.float32).reshape(N, Cc, S)
+    assert np.isfinite(g).all()
+    assert np.abs(g - q).max() / np.abs(q).max() < 1e-3
+    # two roundings of nearly equal fp32 sums: the same binary16 value or its neighbour, and the neighbour rarely
+    gi = got.view(np.int16).astype(np.int32).ravel(); qi = want.view(np.int16).astype(np.int32).ravel()
+    ordg = np.where(gi < 0, -(gi & 0x7fff), gi); ordq = np.where(qi < 0, -(qi & 0x7fff), qi)
+    step = np.abs(ordg - ordq)
+    assert step.max() <= 1 and (step != 0).mean() < 0.02, (step.max(), (step != 0).mean())
+    # the same operands as stored MX-fp8 give the same bytes: the staging pass quantises exactly as lp_f32_to_mx8 does
+    got2, _ = gpu_conv(orc.f32_to_mx(8, x, N, Cc, S), 3, N, Cc, D, D, D, w, None, Cc, 2, cbits=8)
+    assert np.array_equal(got, got2)
+
+
 @pytest.mark.parametrize("bits", [8, 4])
 def test_full_size_properties(gpu, bits):
     """BASELINE-size layer (128 -> 128, 64^3, N 2; fp4: 256 -> 256, 32^3, N 2): exact-operand output compared on sampled planes with the
