@@ -434,7 +434,7 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && nmt_all == 1 && stride == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 || row1_env ? 1 : 2) && a.nbt <= 64;
     a.row1 = a.row && a.nbt == 1 && row1_env && row_env < 2;
     if (a.row) { a.areg = false; a.CB = a.nbt; }
-    size_t smem = a.row ? (size_t)2 * 2048 * (RB + 4) : a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
+    size_t smem = a.row1 ? (size_t)10 * 352 * (RB + 4) : a.row ? (size_t)2 * 2048 * (RB + 4) : a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     if (s2d) smem = 0;
     smem = (smem + 15) & ~(size_t)15;
     a.epi_o = (unsigned)smem; smem += (size_t)3 * MT * 32 * sizeof(float);      // bias, affine a, b of the workgroup's channels
