@@ -8,8 +8,8 @@
 // src/lp_common.cuh:1575-1597), or, for a fused call, set the slots and finalize mean / rstd from them right away (src/nn_elem.cu:5-11), which saves
 // the zeroing and finalize launches around the conv
 struct gn_fin_t { float *mean, *rstd; double len; float eps; };
-__device__ __forceinline__ void gn_part_finish(double *osum, double s, double ss, gn_fin_t fin) {
-    const size_t i = 2 * (size_t)blockIdx.x;
+__device__ __forceinline__ void gn_part_finish(double *osum, double s, double ss, gn_fin_t fin, unsigned ng) {
+    const size_t i = 2 * (size_t)ng;
     if (!fin.mean) { gn_acc_add(osum, i, s); gn_acc_add(osum, i + 1, ss); return; }
     unsigned long long *w = (unsigned long long *)osum + 3 * i;
     double v[2] = {s, ss}, got[2];
@@ -22,19 +22,24 @@ __device__ __forceinline__ void gn_part_finish(double *osum, double s, double ss
         got[k] = (double)(long long)f + (double)lo * 5.42101086242752217e-20;
     }
     const double m = got[0] / fin.len, var = got[1] / fin.len - m * m;
-    fin.mean[blockIdx.x] = (float)m;
-    fin.rstd[blockIdx.x] = (float)(1.0 / sqrt((var > 0 ? var : 0) + (double)fin.eps));
+    fin.mean[ng] = (float)m;
+    fin.rstd[ng] = (float)(1.0 / sqrt((var > 0 ? var : 0) + (double)fin.eps));
 }
 
-// (sum, sum of squares) partials of the tiles -> exact GroupNorm sum slots: one block per (sample, group), double accumulation over
-// the sample's tiles in index order, a fixed tree over the block, one slot add per sum (src/lp_common.cuh:1575-1597 does the same with
-// one fixed-point atomic per block and channel)
-__global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum, gn_fin_t fin) {
+// (sum, sum of squares) partials of the tiles -> exact GroupNorm sum slots: nsplit blocks per (sample, group), each a contiguous range of the
+// sample's records in index order, double accumulation, a fixed tree over the block, one slot add per sum (src/lp_common.cuh:1575-1597 does the
+// same with one fixed-point atomic per block and channel). nsplit > 1 (many records: the level-0 layers): every block leaves its pair of doubles
+// in scr and takes a ticket of its (sample, group); the block that draws the last one adds the nsplit pairs in index order, so the result does
+// not depend on which block that is, and puts the ticket counter back to zero for the next launch
+struct gn_split_t { int nsplit; double *scr; unsigned *cnt; };
+__global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum, gn_fin_t fin, gn_split_t sp) {
     // the group's channel quads are consecutive: quad Q = co / 4 lives in channel slice Q / (8 MT), slot Q % (8 MT) of its tile's record
-    const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, qpg = Co / Go / 4, nq = MT * 8, nst = tiles_per_n / ncs;
+    const unsigned ng = blockIdx.x / (unsigned)sp.nsplit, part_i = blockIdx.x % (unsigned)sp.nsplit;
+    const int n = (int)ng / Go, gidx = (int)ng % Go, qpg = Co / Go / 4, nq = MT * 8, nst = tiles_per_n / ncs;
+    const int total = nst * qpg, per = (total + sp.nsplit - 1) / sp.nsplit, i0 = (int)part_i * per, i1 = min(total, i0 + per);
     double s = 0.0, ss = 0.0;
 #pragma unroll 8
-    for (int i = threadIdx.x; i < nst * qpg; i += 256) {                   // (unrolled: the records' loads of several rounds are in flight together)
+    for (int i = i0 + (int)threadIdx.x; i < i1; i += 256) {                 // (unrolled: the records' loads of several rounds are in flight together)
         const int st = i / qpg, Q = gidx * qpg + i % qpg, cs = Q / nq, qd = Q - cs * nq;
         const float2 p = part[(size_t)(n * tiles_per_n + st * ncs + cs) * nq + qd];
         s += (double)p.x; ss += (double)p.y;
@@ -43,7 +48,20 @@ __global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int 
     r1[threadIdx.x] = s; r2[threadIdx.x] = ss;
     __syncthreads();
     for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) { r1[threadIdx.x] += r1[threadIdx.x + st]; r2[threadIdx.x] += r2[threadIdx.x + st]; } __syncthreads(); }
-    if (threadIdx.x == 0) gn_part_finish(osum, r1[0], r2[0], fin);
+    if (threadIdx.x) return;
+    if (sp.nsplit == 1) { gn_part_finish(osum, r1[0], r2[0], fin, ng); return; }
+    double *mine = sp.scr + 2 * (size_t)blockIdx.x;
+    __hip_atomic_store(mine, r1[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); __hip_atomic_store(mine + 1, r2[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __threadfence();                                                        // the pair is visible device-wide before the ticket is
+    if (atomicAdd(sp.cnt + ng, 1u) != (unsigned)sp.nsplit - 1u) return;
+    __threadfence();                                                        // the last block: every other block's pair is visible
+    s = 0.0; ss = 0.0;
+    for (int k = 0; k < sp.nsplit; k++) {
+        s += __hip_atomic_load(sp.scr + 2 * ((size_t)ng * sp.nsplit + k), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ss += __hip_atomic_load(sp.scr + 2 * ((size_t)ng * sp.nsplit + k) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __hip_atomic_store(sp.cnt + ng, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    gn_part_finish(osum, s, ss, fin, ng);
 }
 
 // the same from per-channel records (32 per tile: launches whose channels per group are not a multiple of 4 run one channel tile per workgroup,
@@ -60,7 +78,7 @@ __global__ void __launch_bounds__(256) gn_part_reduce_ch_k(const float2 *part, i
     r1[threadIdx.x] = s; r2[threadIdx.x] = ss;
     __syncthreads();
     for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) { r1[threadIdx.x] += r1[threadIdx.x + st]; r2[threadIdx.x] += r2[threadIdx.x + st]; } __syncthreads(); }
-    if (threadIdx.x == 0) gn_part_finish(osum, r1[0], r2[0], fin);
+    if (threadIdx.x == 0) gn_part_finish(osum, r1[0], r2[0], fin, blockIdx.x);
 }
 
 // ---- weights: fp32 w[co][ci][27] -> per (chunk, unit pair, 32-row channel tile) fragment-ordered codes + scale bytes ----
@@ -188,8 +206,24 @@ static void conv_stats_reduce(const char *who, const conv_args &a, int MT, split
     gn_fin_t fin = g_fin;
     fin.len = (double)(a.Co / a.Go) * (double)a.Do * a.Ho * a.Wo;
     if (fin.mean && (sp.zlo || sp.zhi)) mi_die("%s: fused finalize with a z range", who);
-    if (a.stat_ch) gn_part_reduce_ch_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.ncs, a.Co, a.Go, osum, fin);
-    else gn_part_reduce_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N) * (a.row1 ? 8 : 1), a.ncs, MT, a.Co, a.Go, osum, fin);      // (row1: eight records per tile)
+    if (a.stat_ch) { gn_part_reduce_ch_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.ncs, a.Co, a.Go, osum, fin); MICK(); return; }
+    const int tiles_per_n = (int)(a.ntiles / a.N) * (a.row1 ? 8 : 1);      // (row1: eight records per tile)
+    // many records per (sample, group): several blocks each, folded by the last one done. The pairs and ticket counters live in a small buffer
+    // per device, allocated on first use and left zeroed by every launch (the entry point that must not allocate keeps one block per group)
+    const long recs = (long)(tiles_per_n / a.ncs) * (a.Co / a.Go / 4);
+    gn_split_t gs = {1, nullptr, nullptr};
+    constexpr int MAXNG = 4096, MAXSPLIT = 16;
+    if (recs >= 4096 && a.N * a.Go <= MAXNG && !mi_ws_arena_on()) {
+        static double *scr[8]; static unsigned *cnt[8];
+        int dv = 0; MIRT(hipGetDevice(&dv)); dv &= 7;
+        if (!scr[dv]) {
+            MIRT(hipMalloc((void **)&scr[dv], (size_t)MAXNG * MAXSPLIT * 2 * sizeof(double))); MIRT(hipMalloc((void **)&cnt[dv], MAXNG * sizeof(unsigned))); mi_count_alloc(); mi_count_alloc();
+            if (!scr[dv] || !cnt[dv]) mi_die("%s: no device memory for the statistics fold", who);
+            MIRT(hipMemset(cnt[dv], 0, MAXNG * sizeof(unsigned)));
+        }
+        gs.nsplit = (int)((recs + 2047) / 2048 < MAXSPLIT ? (recs + 2047) / 2048 : MAXSPLIT); gs.scr = scr[dv]; gs.cnt = cnt[dv];
+    }
+    gn_part_reduce_k<<<a.N * a.Go * gs.nsplit, 256>>>((const float2 *)a.part, tiles_per_n, a.ncs, MT, a.Co, a.Go, osum, fin, gs);
     MICK();
 }
 
