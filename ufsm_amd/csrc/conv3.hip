@@ -26,20 +26,64 @@ __device__ __forceinline__ void gn_part_finish(double *osum, double s, double ss
     fin.rstd[ng] = (float)(1.0 / sqrt((var > 0 ? var : 0) + (double)fin.eps));
 }
 
-// (sum, sum of squares) partials of the tiles -> exact GroupNorm sum slots: nsplit blocks per (sample, group), each a contiguous range of the
-// sample's records in index order, double accumulation, a fixed tree over the block, one slot add per sum (src/lp_common.cuh:1575-1597 does the
-// same with one fixed-point atomic per block and channel). nsplit > 1 (many records: the level-0 layers): every block leaves its pair of doubles
-// in scr and takes a ticket of its (sample, group); the block that draws the last one adds the nsplit pairs in index order, so the result does
-// not depend on which block that is, and puts the ticket counter back to zero for the next launch
+// (sum, sum of squares) partials of the tiles -> exact GroupNorm sum slots (src/lp_common.cuh:1575-1597 does the same with one fixed-point atomic
+// per block and channel). A spatial tile's record is Q = Co / 4 (padded to whole channel slices) consecutive float2, one per channel quad; quad
+// Q = co / 4 lives in channel slice Q / (8 MT), slot Q % (8 MT). A block takes one sample's tiles [t0, t1) with ALL their quads: thread (j, q) adds
+// quad q of tiles t0 + j, t0 + j + J, ... in double (consecutive threads read consecutive records: every fetched line is used whole), then thread
+// g adds its group's quads over the J rows in a fixed order. nsplit > 1 (thousands of tiles: the level-0 layers): every block leaves its Go pairs
+// in scr and takes a ticket of its sample; the block that draws the last one adds the nsplit pairs of every group in index order - the result
+// does not depend on which block that is - and puts the ticket counter back to zero for the next launch
 struct gn_split_t { int nsplit; double *scr; unsigned *cnt; };
 __global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum, gn_fin_t fin, gn_split_t sp) {
-    // the group's channel quads are consecutive: quad Q = co / 4 lives in channel slice Q / (8 MT), slot Q % (8 MT) of its tile's record
-    const unsigned ng = blockIdx.x / (unsigned)sp.nsplit, part_i = blockIdx.x % (unsigned)sp.nsplit;
-    const int n = (int)ng / Go, gidx = (int)ng % Go, qpg = Co / Go / 4, nq = MT * 8, nst = tiles_per_n / ncs;
-    const int total = nst * qpg, per = (total + sp.nsplit - 1) / sp.nsplit, i0 = (int)part_i * per, i1 = min(total, i0 + per);
+    const int n = (int)blockIdx.x / sp.nsplit, pi = (int)blockIdx.x % sp.nsplit, tid = (int)threadIdx.x;
+    const int Q = ncs * MT * 8, nst = tiles_per_n / ncs, qpg = Co / Go / 4, J = 256 / Q;
+    const int per = (nst + sp.nsplit - 1) / sp.nsplit, t0 = pi * per, t1 = min(nst, t0 + per);
+    const int q = tid % Q, j = tid / Q;
+    const float2 *rec = part + (size_t)n * tiles_per_n * (MT * 8) + q;
+    double s = 0.0, ss = 0.0;
+    if (j < J) {
+#pragma unroll 8
+        for (int st = t0 + j; st < t1; st += J) {                            // (unrolled: the records' loads of several rounds are in flight together)
+            const float2 p = rec[(size_t)st * Q];
+            s += (double)p.x; ss += (double)p.y;
+        }
+    }
+    __shared__ double r1[256], r2[256];
+    __shared__ unsigned ticket;
+    r1[tid] = s; r2[tid] = ss;
+    __syncthreads();
+    s = 0.0; ss = 0.0;
+    if (tid < Go)
+        for (int k = 0; k < qpg; k++)
+            for (int jj = 0; jj < J; jj++) { s += r1[jj * Q + tid * qpg + k]; ss += r2[jj * Q + tid * qpg + k]; }
+    if (sp.nsplit == 1) { if (tid < Go) gn_part_finish(osum, s, ss, fin, (unsigned)(n * Go + tid)); return; }
+    if (tid < Go) {
+        double *mine = sp.scr + 2 * ((size_t)blockIdx.x * Go + tid);
+        __hip_atomic_store(mine, s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); __hip_atomic_store(mine + 1, ss, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __threadfence();                                                    // the pairs are visible device-wide before the ticket is
+    }
+    __syncthreads();
+    if (tid == 0) ticket = atomicAdd(sp.cnt + n, 1u);
+    __syncthreads();
+    if (ticket != (unsigned)sp.nsplit - 1u) return;                         // (uniform over the block)
+    __threadfence();                                                        // the last block of the sample: every other block's pairs are visible
+    if (tid == 0) __hip_atomic_store(sp.cnt + n, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid < sp.nsplit * Go) {                                             // (nsplit Go <= 256) all pairs of the sample at once, then added in index order
+        const double *theirs = sp.scr + 2 * ((size_t)n * sp.nsplit * Go + tid);
+        r1[tid] = __hip_atomic_load(theirs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); r2[tid] = __hip_atomic_load(theirs + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (tid >= Go) return;
+    s = 0.0; ss = 0.0;
+    for (int k = 0; k < sp.nsplit; k++) { s += r1[k * Go + tid]; ss += r2[k * Go + tid]; }
+    gn_part_finish(osum, s, ss, fin, (unsigned)(n * Go + tid));
+}
+// the same with one block per (sample, group), for records wider than a block (more than 1024 channels) or more than 256 groups
+__global__ void __launch_bounds__(256) gn_part_reduce_g_k(const float2 *part, int tiles_per_n, int ncs, int MT, int Co, int Go, double *osum, gn_fin_t fin) {
+    const int n = blockIdx.x / Go, gidx = blockIdx.x % Go, qpg = Co / Go / 4, nq = MT * 8, nst = tiles_per_n / ncs;
     double s = 0.0, ss = 0.0;
 #pragma unroll 8
-    for (int i = i0 + (int)threadIdx.x; i < i1; i += 256) {                 // (unrolled: the records' loads of several rounds are in flight together)
+    for (int i = threadIdx.x; i < nst * qpg; i += 256) {
         const int st = i / qpg, Q = gidx * qpg + i % qpg, cs = Q / nq, qd = Q - cs * nq;
         const float2 p = part[(size_t)(n * tiles_per_n + st * ncs + cs) * nq + qd];
         s += (double)p.x; ss += (double)p.y;
@@ -48,20 +92,7 @@ __global__ void __launch_bounds__(256) gn_part_reduce_k(const float2 *part, int 
     r1[threadIdx.x] = s; r2[threadIdx.x] = ss;
     __syncthreads();
     for (int st = 128; st > 0; st >>= 1) { if ((int)threadIdx.x < st) { r1[threadIdx.x] += r1[threadIdx.x + st]; r2[threadIdx.x] += r2[threadIdx.x + st]; } __syncthreads(); }
-    if (threadIdx.x) return;
-    if (sp.nsplit == 1) { gn_part_finish(osum, r1[0], r2[0], fin, ng); return; }
-    double *mine = sp.scr + 2 * (size_t)blockIdx.x;
-    __hip_atomic_store(mine, r1[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); __hip_atomic_store(mine + 1, r2[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __threadfence();                                                        // the pair is visible device-wide before the ticket is
-    if (atomicAdd(sp.cnt + ng, 1u) != (unsigned)sp.nsplit - 1u) return;
-    __threadfence();                                                        // the last block: every other block's pair is visible
-    s = 0.0; ss = 0.0;
-    for (int k = 0; k < sp.nsplit; k++) {
-        s += __hip_atomic_load(sp.scr + 2 * ((size_t)ng * sp.nsplit + k), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ss += __hip_atomic_load(sp.scr + 2 * ((size_t)ng * sp.nsplit + k) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __hip_atomic_store(sp.cnt + ng, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    gn_part_finish(osum, s, ss, fin, ng);
+    if (threadIdx.x == 0) gn_part_finish(osum, r1[0], r2[0], fin, blockIdx.x);
 }
 
 // the same from per-channel records (32 per tile: launches whose channels per group are not a multiple of 4 run one channel tile per workgroup,
@@ -208,22 +239,27 @@ static void conv_stats_reduce(const char *who, const conv_args &a, int MT, split
     if (fin.mean && (sp.zlo || sp.zhi)) mi_die("%s: fused finalize with a z range", who);
     if (a.stat_ch) { gn_part_reduce_ch_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, (int)(a.ntiles / a.N), a.ncs, a.Co, a.Go, osum, fin); MICK(); return; }
     const int tiles_per_n = (int)(a.ntiles / a.N) * (a.row1 ? 8 : 1);      // (row1: eight records per tile)
-    // many records per (sample, group): several blocks each, folded by the last one done. The pairs and ticket counters live in a small buffer
-    // per device, allocated on first use and left zeroed by every launch (the entry point that must not allocate keeps one block per group)
-    const long recs = (long)(tiles_per_n / a.ncs) * (a.Co / a.Go / 4);
+    const int Q = a.ncs * MT * 8, nst = tiles_per_n / a.ncs;
+    if (Q > 256 || a.Go > 256) { gn_part_reduce_g_k<<<a.N * a.Go, 256>>>((const float2 *)a.part, tiles_per_n, a.ncs, MT, a.Co, a.Go, osum, fin); MICK(); return; }
+    // thousands of tiles per sample: several blocks each (512 tiles or more per block), folded by the last one done. The pairs and ticket
+    // counters live in a small buffer per device, allocated on first use and left zeroed by every launch (the entry point that must not
+    // allocate keeps one block per sample)
     gn_split_t gs = {1, nullptr, nullptr};
-    constexpr int MAXNG = 4096, MAXSPLIT = 16;
-    if (recs >= 4096 && a.N * a.Go <= MAXNG && !mi_ws_arena_on()) {
+    constexpr int MAXN = 4096, SCR = 1 << 17;                  // samples with a ticket counter; doubles of scratch
+    int want = nst < 4096 ? 1 : nst / 512 < 32 ? nst / 512 : 32;          // (the ticket and the fold cost 2 - 3 us: a single pass is faster below a few thousand tiles)
+    if (want * a.Go > 256) want = 256 / a.Go;
+    while (want > 1 && (size_t)a.N * want * a.Go * 2 > (size_t)SCR) want >>= 1;
+    if (want > 1 && a.N <= MAXN && !mi_ws_arena_on()) {
         static double *scr[8]; static unsigned *cnt[8];
         int dv = 0; MIRT(hipGetDevice(&dv)); dv &= 7;
         if (!scr[dv]) {
-            MIRT(hipMalloc((void **)&scr[dv], (size_t)MAXNG * MAXSPLIT * 2 * sizeof(double))); MIRT(hipMalloc((void **)&cnt[dv], MAXNG * sizeof(unsigned))); mi_count_alloc(); mi_count_alloc();
+            MIRT(hipMalloc((void **)&scr[dv], (size_t)SCR * sizeof(double))); MIRT(hipMalloc((void **)&cnt[dv], MAXN * sizeof(unsigned))); mi_count_alloc(); mi_count_alloc();
             if (!scr[dv] || !cnt[dv]) mi_die("%s: no device memory for the statistics fold", who);
-            MIRT(hipMemset(cnt[dv], 0, MAXNG * sizeof(unsigned)));
+            MIRT(hipMemset(cnt[dv], 0, MAXN * sizeof(unsigned)));
         }
-        gs.nsplit = (int)((recs + 2047) / 2048 < MAXSPLIT ? (recs + 2047) / 2048 : MAXSPLIT); gs.scr = scr[dv]; gs.cnt = cnt[dv];
+        gs.nsplit = want; gs.scr = scr[dv]; gs.cnt = cnt[dv];
     }
-    gn_part_reduce_k<<<a.N * a.Go * gs.nsplit, 256>>>((const float2 *)a.part, tiles_per_n, a.ncs, MT, a.Co, a.Go, osum, fin, gs);
+    gn_part_reduce_k<<<a.N * gs.nsplit, 256>>>((const float2 *)a.part, tiles_per_n, a.ncs, MT, a.Co, a.Go, osum, fin, gs);
     MICK();
 }
 
