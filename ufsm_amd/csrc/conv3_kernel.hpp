@@ -129,15 +129,16 @@ template <> struct fmt_t<4> { static constexpr int RB = 16, NH = 1, WTILE = 1024
 
 // GELU, x Phi(x) = 0.5 x (1 + erf(x / sqrt 2)), with erf by the rational-times-Gaussian form erf z = 1 - (a1 t + ... + a5 t^5) exp(-z^2),
 // t = 1 / (1 + p z), z >= 0 (Abramowitz & Stegun 7.1.26, |error| < 1.5e-7): about 16 instructions with one reciprocal and one exponential where
-// the library's erff takes about 60; the epilogue that applies it runs alone on its SIMD, so every instruction is time. With
+// the library's erff takes about 60 (14 here); the epilogue that applies it runs alone on its SIMD, so every instruction is time. With
 // q = 0.5 |x| (a1 t + ...) exp(-z^2) the result is max(x, 0) - q for either sign. NaN stays NaN; +-inf: z^2 overflows, the exponential is 0, q = inf 0
 // would be NaN, so q takes the exponential's zero through a select
 __device__ __forceinline__ float gelu_erf(float x) {
-    const float ax = fabsf(x), z = ax * 0.70710678f;
-    const float t = __builtin_amdgcn_rcpf(fmaf(z, 0.3275911f, 1.f));
-    const float poly = t * fmaf(t, fmaf(t, fmaf(t, fmaf(t, 1.061405429f, -1.453152027f), 1.421413741f), -0.284496736f), 0.254829592f);
-    const float ex = __builtin_amdgcn_exp2f(z * z * -1.44269504f);
-    const float q = ex == 0.f ? 0.f : 0.5f * ax * poly * ex;
+    // (z never formed: p z = |x| p / sqrt 2, -z^2 log2 e = -x^2 log2 e / 2, and the factor 0.5 sits in the coefficients)
+    const float ax = fabsf(x);
+    const float t = __builtin_amdgcn_rcpf(fmaf(ax, 0.23164189f, 1.f));
+    const float poly = t * fmaf(t, fmaf(t, fmaf(t, fmaf(t, 0.5307027145f, -0.7265760135f), 0.7107068705f), -0.142248368f), 0.127414796f);
+    const float ex = __builtin_amdgcn_exp2f(ax * ax * -0.72134752f);
+    const float q = ex == 0.f ? 0.f : ax * poly * ex;
     return fmaxf(x, 0.f) - q;
 }
 
