@@ -555,7 +555,13 @@ extern "C" int lp_gn_sums_mx(const void *x, int xdt, int N, int C, int G, size_t
 
 // ---- 1x1x1 head (src/lp_mx_conv1.cu:5-21): y[n][co][v] = b[co] + sum_ci w[co][ci] act(x[ci][v]), fp32 FMA in ci order ----
 // Thread per voxel; weights, bias and the GN coefficients of the sample staged in LDS once per block; CO outputs per pass in registers.
-template <int B, int CO, typename YT>
+// MF (CO 8, whole 32-channel blocks): the 8 x 32 products of a voxel go through the matrix pipe as batched 4 x 4 outer products
+// (v_mfma_f32_4x4x1: 16 blocks of four lanes; a lane supplies its voxel's activation as column j = lane % 4 of its block and output channel
+// lane % 4 (+ 4) of the weights as row, and receives the four channels of its own voxel). One product is added per step, in ci order, so the
+// sums are those of the fused multiply-add chain; what moves is 256 of a voxel's vector instructions, into a pipe the sigmoids do not use.
+// Every lane of a wavefront must take part: a voxel past the range computes on voxel 0's row and stores nothing.
+typedef float v4f __attribute__((ext_vector_type(4)));
+template <int B, int CO, typename YT, bool MF = false>
 __global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const float *w, const float *b, YT *y, int N, int Ci, size_t S, gnp_t gp, int Co, int co0,
                                                   size_t vb, size_t nv, size_t ly) {
     extern __shared__ __align__(16) float c1s[];          // [Ci][CO] weights (input-channel major: a channel's CO weights are one or two 16-byte reads at an
@@ -571,8 +577,9 @@ __global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const flo
     }
     __syncthreads();
     const size_t vi = blockIdx.x * (size_t)256 + threadIdx.x;
-    if (vi >= nv) return;
-    const size_t v = vb + vi;
+    const bool live = vi < nv;
+    if (!MF && !live) return;
+    const size_t v = vb + (live ? vi : 0);
     float acc[CO];
 #pragma unroll
     for (int co = 0; co < CO; co++) acc[co] = sb[co];
@@ -589,6 +596,19 @@ __global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const flo
                     r[4 * k4] = d_act_ab(r[4 * k4], ta.x, tb.x); r[4 * k4 + 1] = d_act_ab(r[4 * k4 + 1], ta.y, tb.y);
                     r[4 * k4 + 2] = d_act_ab(r[4 * k4 + 2], ta.z, tb.z); r[4 * k4 + 3] = d_act_ab(r[4 * k4 + 3], ta.w, tb.w);
                 }
+            }
+            if constexpr (MF) {
+                static_assert(!MF || CO == 8, "matrix-pipe head: eight output channels");
+                const float *wl = swb + (threadIdx.x & 3);       // the lane's row of its block's two weight tiles: channels lane % 4 and 4 + lane % 4
+                v4f lo = {acc[0], acc[1], acc[2], acc[3]}, hi = {acc[4], acc[5], acc[6], acc[7]};
+#pragma unroll
+                for (int k = 0; k < 32; k++) {
+                    lo = __builtin_amdgcn_mfma_f32_4x4x1f32(wl[k * 8], r[k], lo, 0, 0, 0);
+                    hi = __builtin_amdgcn_mfma_f32_4x4x1f32(wl[k * 8 + 4], r[k], hi, 0, 0, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) { acc[i] = lo[i]; acc[4 + i] = hi[i]; }
+                continue;
             }
 #pragma unroll
             for (int k = 0; k < 32; k++) {
@@ -624,6 +644,7 @@ __global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const flo
             }
         }
     }
+    if (!live) return;
 #pragma unroll
     for (int co = 0; co < CO; co++) if (co0 + co < Co) {
         const size_t o = ((size_t)n * Co + co0 + co) * ly + vi;
@@ -655,6 +676,13 @@ static void conv1_launch_row(const void *x, int xdt, shape5 xs, const float *w, 
         const int rem = cout - co0;
         const size_t sm = ((size_t)8 * xs.c + 8 + 2 * (size_t)((xs.c + 3) & ~3)) * sizeof(float);
 #define C1(B, CO) conv1_mx_k<B, CO, YT><<<grid, 256, sm>>>(xq, w, b, y, xs.n, xs.c, S, gp, cout, co0, vb, nv, ly)
+        static int mf_env = -1;
+        if (mf_env < 0) mf_env = getenv("MI_HEAD_MFMA") ? atoi(getenv("MI_HEAD_MFMA")) : 1;     // tuning knob: 0 keeps the products on the vector ALUs
+        if (mf_env && rem >= 8 && xs.c % 32 == 0) {
+            if (xdt == 4) conv1_mx_k<4, 8, YT, true><<<grid, 256, sm>>>(xq, w, b, y, xs.n, xs.c, S, gp, cout, co0, vb, nv, ly);
+            else conv1_mx_k<8, 8, YT, true><<<grid, 256, sm>>>(xq, w, b, y, xs.n, xs.c, S, gp, cout, co0, vb, nv, ly);
+            continue;
+        }
         if (xdt == 4) { if (rem >= 8) C1(4, 8); else if (rem >= 4) { C1(4, 4); co0 -= 4; } else if (rem >= 2) { C1(4, 2); co0 -= 6; } else { C1(4, 1); co0 -= 7; } }
         else { if (rem >= 8) C1(8, 8); else if (rem >= 4) { C1(8, 4); co0 -= 4; } else if (rem >= 2) { C1(8, 2); co0 -= 6; } else { C1(8, 1); co0 -= 7; } }
 #undef C1
