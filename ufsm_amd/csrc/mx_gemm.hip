@@ -104,16 +104,25 @@ __global__ void __launch_bounds__(256) mx_gemm_k(const uint8_t *__restrict__ Aq,
             const int col = n0 + 32 * j + r;
             if (col >= N) continue;
             const float bv = bias ? bias[col] : 0.f;
+            // the tile's 16 residual and 16 old values are read first, then everything is stored: C and res may be the same array, so a load
+            // written after a store could not be moved above it, and 64 dependent round trips to memory were most of this kernel's time
+            float add[16];
+#pragma unroll
+            for (int q = 0; q < 16; q++) add[q] = bv;
+            if (res && !split) {                                // (uniform)
+#pragma unroll
+                for (int q = 0; q < 16; q++) add[q] += res[(size_t)min(m0 + 32 * i + (q & 3) + 4 * h + 8 * (q >> 2), M - 1) * N + col];
+            }
+            if (beta != 0.f && !split) {                        // (uniform)
+#pragma unroll
+                for (int q = 0; q < 16; q++) add[q] += beta * C[(size_t)min(m0 + 32 * i + (q & 3) + 4 * h + 8 * (q >> 2), M - 1) * N + col];
+            }
 #pragma unroll
             for (int q = 0; q < 16; q++) {
                 const int row = m0 + 32 * i + (q & 3) + 4 * h + 8 * (q >> 2);
                 if (row >= M) continue;
                 float *p = C + (size_t)row * N + col;
-                if (split) { atomicAdd(p, acc[i][j][q]); continue; }
-                float v = acc[i][j][q] + bv;
-                if (res) v += res[(size_t)row * N + col];
-                if (beta != 0.f) v += beta * *p;
-                *p = v;
+                if (split) atomicAdd(p, acc[i][j][q]); else *p = acc[i][j][q] + add[q];
             }
         }
 }
