@@ -93,6 +93,10 @@ void mi_conv_split(int tiles);
    straight from the stored tensor when the launch has enough output voxels to fill the device, else the general kernel (staged halo);
    0: always the general kernel; 1: the direct kernel whenever its operands allow it. The results are the same conv either way. */
 void mi_conv_s2_direct(int mode);
+/* 1x1x1 head with eight outputs on whole 32-channel blocks: where its 8 x 32 products per voxel run. mode 1: the matrix pipe (batched 4 x 4 x 1
+   fp32 outer products, one product per accumulator and step, in channel order), 0: fused multiply-adds on the vector ALUs, -1: the default
+   (1, or the environment's MI_HEAD_MFMA). The two give the same bits; the setting is the calling thread's. No counterpart in the reference. */
+void mi_conv1_matrix(int mode);
 /* no counterpart in the reference (its convs transform their input while staging, every time): GroupNorm + SiLU of x and re-quantisation to
    MX-fp8 / MX-fp4 (ybits 8 / 4) once, for a tensor several convs read; they then take y with no GroupNorm. s.c a multiple of 32. In a split
    input, gp2.G = -1 says "x2 carries no GroupNorm, gp is x's own" (gp2.G = 0 keeps the reference's meaning: gp spans both segments). */

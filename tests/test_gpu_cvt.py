@@ -281,6 +281,38 @@ def test_gn_sums_and_finalize(gpu, bits, Cc, G):
     assert (dd.to_numpy(np.float64) == 0).all()
 
 
+def test_head_matrix_pipe_gives_the_vector_form_s_bits(gpu):
+    """The head's products through the matrix pipe (v_mfma_f32_4x4x1: one product per accumulator and step, in channel order) against the same
+    products as fused multiply-adds on the vector ALUs: equal bit for bit, with GroupNorm + SiLU on the input, two channel blocks, denormal
+    products, a voxel count that leaves lanes of the last wavefront without a voxel, fp32 and fp16 outputs, MX-fp8 and MX-fp4 inputs."""
+    rng = np.random.default_rng(77)
+    N, Ci, Co, D, H, W, G = 2, 64, 8, 7, 9, 11, 8
+    S = D * H * W
+    x = rng.standard_normal((N, Ci, S)).astype(np.float32)
+    x[0, :, :40] *= 1e-30
+    w = rng.standard_normal((Co, Ci)).astype(np.float32) * 0.3; b = rng.standard_normal(Co).astype(np.float32)
+    gam = rng.uniform(0.5, 1.5, Ci).astype(np.float32); bet = rng.uniform(-.5, .5, Ci).astype(np.float32)
+    mean = rng.uniform(-.2, .2, N * G).astype(np.float32); rstd = rng.uniform(.8, 1.2, N * G).astype(np.float32)
+    dw = DevBuf.from_numpy(w); db = DevBuf.from_numpy(b)
+    xs = shape5(N, Ci, D, H, W)
+    try:
+        for bits in (8, 4):
+            dq = to_mx(bits, x)
+            for gn in (False, True):
+                g = dev_gn(gam, bet, mean, rstd, G) if gn else gnp_t()
+                for h16 in (False, True):
+                    out = []
+                    for mode in (0, 1):
+                        lib.mi_conv1_matrix(mode)
+                        dy = DevBuf(N * Co * S * (2 if h16 else 4))
+                        (lib.lp_conv1_fwd_mx_h16 if h16 else lib.lp_conv1_fwd_mx)(dq.ptr, 3 if bits == 8 else 4, xs, dw.ptr, db.ptr, Co, dy.ptr, g)
+                        out.append(dy.to_numpy(np.uint16 if h16 else np.uint32, (N, Co, S)))
+                    assert np.array_equal(out[0], out[1]), (bits, gn, h16)
+    finally:
+        lib.mi_conv1_matrix(-1)
+    LP.check()
+
+
 # (34 and 70 input channels: a whole 32-channel block, which takes the kernel's straight-line form, followed by a ragged one, with channel counts that
 # are not multiples of 4 and output groups of 2 and 1 channels)
 @pytest.mark.parametrize("bits,Ci,Co,gn,h16", [(8, 16, 1, False, False), (8, 32, 8, True, False), (4, 32, 11, True, False), (8, 64, 8, False, True), (8, 32, 20, True, False),

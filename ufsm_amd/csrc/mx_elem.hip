@@ -651,6 +651,8 @@ __global__ void __launch_bounds__(256, 4) conv1_mx_k(const uint8_t *x, const flo
         if (sizeof(YT) == 2) ((__half *)y)[o] = __float2half(acc[co]); else ((float *)y)[o] = acc[co];
     }
 }
+static thread_local int g_conv1_matrix = -1;      // mi_conv1_matrix: the calling thread's choice of where the head's products run (-1: the default)
+extern "C" void mi_conv1_matrix(int mode) { g_conv1_matrix = mode; }
 template <typename YT>
 static void conv1_launch_row(const void *x, int xdt, shape5 xs, const float *w, const float *b, int cout, YT *y, gnp_t gp, size_t vb, size_t nv, size_t ly, const char *who);
 // voxels [vb, vb + nv) of every sample; with slab-local GroupNorm statistics one launch per slab the range meets (its voxels, its statistics row)
@@ -678,7 +680,7 @@ static void conv1_launch_row(const void *x, int xdt, shape5 xs, const float *w, 
 #define C1(B, CO) conv1_mx_k<B, CO, YT><<<grid, 256, sm>>>(xq, w, b, y, xs.n, xs.c, S, gp, cout, co0, vb, nv, ly)
         static int mf_env = -1;
         if (mf_env < 0) mf_env = getenv("MI_HEAD_MFMA") ? atoi(getenv("MI_HEAD_MFMA")) : 1;     // tuning knob: 0 keeps the products on the vector ALUs
-        if (mf_env && rem >= 8 && xs.c % 32 == 0) {
+        if ((g_conv1_matrix < 0 ? mf_env : g_conv1_matrix) && rem >= 8 && xs.c % 32 == 0) {
             if (xdt == 4) conv1_mx_k<4, 8, YT, true><<<grid, 256, sm>>>(xq, w, b, y, xs.n, xs.c, S, gp, cout, co0, vb, nv, ly);
             else conv1_mx_k<8, 8, YT, true><<<grid, 256, sm>>>(xq, w, b, y, xs.n, xs.c, S, gp, cout, co0, vb, nv, ly);
             continue;

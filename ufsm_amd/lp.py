@@ -46,6 +46,7 @@ _PROTOS = {
     "mi_conv_stem_zc": (None, [C.c_int]),
     "mi_conv_split": (None, [C.c_int]),
     "mi_conv_s2_direct": (None, [C.c_int]),
+    "mi_conv1_matrix": (None, [C.c_int]),
     "mi_conv_prestage": (_I, [_P, _I, shape5, gnp_t, _P, _I]),
     "gnp_mk": (gnp_t, [_P, _P, _P, _P, _I]),
     "lp_gn_slab_any": (_I, []),
