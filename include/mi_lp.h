@@ -121,6 +121,9 @@ void lp_pred_input_mx(const uint8_t *ct, int W, float mean, float isd, const flo
 void lp_pred_input_mx8(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd);
 /* the same into sample n of an N-sample input tensor (windows batched for one forward; the reference's entry is N 1, n 0: src/lp_mx_cvt.cu:42-55) */
 void mi_pred_input_mx_n(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits, int N, int n);
+/* the same for samples n0 .. n0 + nw - 1 from nw windows in one launch (ct, dyo, dxo: host arrays of nw device pointers) */
+void mi_pred_input_mx_batch(const uint8_t *const *ct, int W, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, int z0, int nz, void *y, int hd, int bits,
+                            int N, int n0, int nw);
 
 /* ---- MX elementwise ops (src/nn_lp.h:134-137, :175-176) ---- */
 void lp_gn_silu_apply_mx(const void *x, int xdt, shape5 s, int G, const float *gamma, const float *beta, const float *mean, const float *rstd, void *y, int ydt);

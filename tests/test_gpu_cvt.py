@@ -123,6 +123,30 @@ def _pred_input_case(bits, W):
         assert np.array_equal(got, want), (z0, nz, hd, axis, (got != want).mean())
 
 
+@pytest.mark.parametrize("bits,W", [(8, 16), (4, 16), (8, 10)])
+def test_pred_input_batch_equals_the_windows_one_by_one(gpu, bits, W):
+    """Eighteen windows (more than one launch carries) into samples 1 .. 18 of a 20-sample tensor: the bytes mi_pred_input_mx_n writes window by window."""
+    import ctypes as C
+    rng = np.random.default_rng(6)
+    N, n0, nw, D = 20, 1, 18, W
+    S = D * W * W
+    ct = rng.integers(0, 256, (nw, D, W, W)).astype(np.uint8)
+    dyo = rng.uniform(-30, 30, (nw, D)).astype(np.float32); dxo = rng.uniform(-30, 30, (nw, D)).astype(np.float32)
+    dct, ddy, ddx = DevBuf.from_numpy(ct), DevBuf.from_numpy(dyo), DevBuf.from_numpy(dxo)
+    nbytes = mx_bytes(bits, N, 4, S)
+    dy = DevBuf(nbytes); d1 = DevBuf(nbytes)
+    lib.mi_zero(dy.ptr, nbytes); lib.mi_zero(d1.ptr, nbytes)
+    order = rng.permutation(nw)                                # window k of the call is window order[k] of the arrays
+    cts = (C.c_void_p * nw)(*[dct.ptr + int(j) * S for j in order])
+    dys = (C.c_void_p * nw)(*[ddy.ptr + int(j) * 4 * D for j in order]); dxs = (C.c_void_p * nw)(*[ddx.ptr + int(j) * 4 * D for j in order])
+    lib.mi_pred_input_mx_batch(cts, W, 120.0, 1 / 50.0, dys, dxs, 1, 0, D, dy.ptr, 2, bits, N, n0, nw)
+    for k, j in enumerate(order):
+        lib.mi_pred_input_mx_n(dct.ptr + int(j) * S, W, 120.0, 1 / 50.0, ddy.ptr + int(j) * 4 * D, ddx.ptr + int(j) * 4 * D, 1, 0, D, d1.ptr, 2, bits, N, n0 + k)
+    LP.check()
+    got = dy.to_numpy(np.uint8)
+    assert np.array_equal(got, d1.to_numpy(np.uint8)) and got.any()
+
+
 @pytest.mark.parametrize("xdt,yb,Cc", [(3, 8, 64), (4, 4, 64), (3, 4, 64), (4, 8, 64), (3, 8, 48), (4, 4, 80), (3, 8, 16), (4, 4, 12), (3, 4, 8), (0, 8, 64), (2, 8, 40), (1, 4, 16), (0, 4, 5)])
 def test_gn_silu_apply(gpu, xdt, yb, Cc):
     """MX rows of every block width and fp32 / fp16 / bf16 planes in, either MX format out, ragged last blocks."""

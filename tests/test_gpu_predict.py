@@ -81,6 +81,55 @@ def test_ct_window_gather(gpu, W):
     assert da.to_numpy(np.uint32)[0] == 0
 
 
+@pytest.mark.parametrize("W,n", [(24, 3), (32, 18)])     # 18: more windows than one launch carries
+def test_ct_windows_and_flags_equal_the_single_window_calls(gpu, W, n):
+    rng = np.random.default_rng(19)
+    Z, Y, X = 40, 33, 48
+    vol = (rng.integers(0, 256, (Z, Y, X)) * (rng.random((Z, Y, X)) < 0.002)).astype(np.uint8)       # sparse material: some windows are air
+    vol[:, :, :24] = 0; vol[:16] = 0                            # and whole cells of air
+    dv = DevBuf.from_numpy(vol)
+    halo = 4
+    org = np.stack([rng.integers(-W, Z, n), rng.integers(-W, Y, n), rng.integers(-W, X, n)], 1).astype(np.int64)
+    dw = DevBuf(n * W ** 3); da = DevBuf(4 * n); lib.mi_zero(da.ptr, 4 * n)
+    lib.mi_ct_windows(dv.ptr, Z, Y, X, org.ctypes.data_as(C.POINTER(C.c_int64)), n, W, dw.ptr, 3, halo, da.ptr)
+    LP.check()
+    got = dw.to_numpy(np.uint8, (n, W, W, W)); flags = da.to_numpy(np.uint32)
+    d1 = DevBuf(W ** 3); a1 = DevBuf(4)
+    for j in range(n):
+        lib.mi_zero(a1.ptr, 4)
+        lib.mi_ct_window(dv.ptr, Z, Y, X, int(org[j, 0]), int(org[j, 1]), int(org[j, 2]), W, d1.ptr, 3, halo, a1.ptr)
+        assert np.array_equal(got[j], d1.to_numpy(np.uint8, (W, W, W))) and (flags[j] != 0) == (a1.to_numpy(np.uint32)[0] != 0)
+    assert 0 < (flags != 0).sum() < n
+    # the flags of a whole sliding grid in one pass: cell (a, b, c) is the interior of the window at (a, b, c) S - halo
+    for S, sub in [(W - 2 * halo, (Z, Y, X)), (16, (Z, Y, X)), (16, (37, 30, 41))]:      # 16-voxel cells on 48-voxel rows take the 16-byte loads
+        sv = np.ascontiguousarray(vol[:sub[0], :sub[1], :sub[2]]); dsv = DevBuf.from_numpy(sv)
+        nss = np.array([(d + S - 1) // S for d in sub], np.int64); tot = int(nss.prod())
+        df = DevBuf(4 * tot); lib.mi_zero(df.ptr, 4 * tot)
+        lib.mi_ct_flags(dsv.ptr, sub[0], sub[1], sub[2], S, nss.ctypes.data_as(C.POINTER(C.c_int64)), 3, df.ptr)
+        LP.check()
+        want = np.array([(sv[a * S:a * S + S, b * S:b * S + S, c * S:c * S + S] >= 3).any() for a, b, c in np.ndindex(*nss)])
+        assert np.array_equal(df.to_numpy(np.uint32) != 0, want) and 0 < want.sum() < tot
+
+
+def test_pred_place_n_equals_the_single_window_calls(gpu):
+    rng = np.random.default_rng(23)
+    W, halo, n, En = 24, 6, 18, 16
+    lg = (rng.standard_normal((n, 2, W, W, W)) * 3).astype(np.float32)          # (a second, unused logit plane per window: lstride != W^3)
+    ct = rng.integers(0, 4, (n, W, W, W)).astype(np.uint8)
+    dl = DevBuf.from_numpy(lg); dc = DevBuf.from_numpy(ct)
+    order = rng.permutation(n + 2)[:n].astype(np.int64) * En ** 3                # targets in any order, with gaps
+    dE = DevBuf((n + 2) * En ** 3); lib.mi_zero(dE.ptr, (n + 2) * En ** 3)
+    lib.mi_pred_place_n(dl.ptr, 2 * W ** 3, dc.ptr, W ** 3, n, order.ctypes.data_as(C.POINTER(C.c_int64)), W, W, halo - 4, halo - 4, -halo, -halo, -halo, En, En, En, En, dE.ptr)
+    LP.check()
+    got = dE.to_numpy(np.uint8, (n + 2, En, En, En))
+    d1 = DevBuf(En ** 3)
+    for j in range(n):
+        lib.mi_zero(d1.ptr, En ** 3)
+        lib.nn_pred_place(dl.ptr + j * 2 * W ** 3 * 4, dc.ptr + j * W ** 3, W, halo - 4, -halo, -halo, -halo, En, En, En, En, d1.ptr)
+        assert np.array_equal(got[order[j] // En ** 3], d1.to_numpy(np.uint8, (En, En, En)))
+    assert got.any() and not got[[k for k in range(n + 2) if k * En ** 3 not in set(order.tolist())]].any()
+
+
 def test_predict_volume_equals_windows_run_one_by_one(gpu):
     """The driver against its own parts: every window gathered, run and placed separately through the C ABI, blended by the oracle.
     Also the reference's checks: core voxels and the first window equal the unfeathered run byte for byte; shells differ."""

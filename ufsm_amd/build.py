@@ -11,6 +11,14 @@ ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
 HIP_SOURCES = ["rt.hip", "mx_elem.hip", "mx_gemm.hip", "attn8.hip", "attn_block.hip", "predict.hip", "conv3.hip", "conv3_stem.hip", "conv2.hip", "conv2_f8.hip", "conv2_f4.hip"] + ["conv3_f%d_o%d.hip" % (f, o) for f in (8, 4) for o in (8, 4, 0)]
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wno-unused-value",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# per-file additions. attn8.hip: the attention core rescales its output accumulators on the vector pipe between two matrix products of every key
+# tile; with the accumulators in ordinary vector registers (the kernel has room: one wavefront per SIMD) that is one multiply each instead of a
+# read from and a write back to the accumulation registers around it
+HIPCC_FILE_FLAGS = {"attn8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
+def hipcc_cmd(src, obj):
+    return ["hipcc"] + HIPCC_FLAGS + HIPCC_FILE_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj]
 
 
 def _run(cmd, cwd=None):
@@ -26,7 +34,7 @@ def build_hip(verbose=False):
     procs = []
     for src in HIP_SOURCES:
         obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-        cmd = ["hipcc"] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = hipcc_cmd(src, obj)
         procs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(obj)
     for cmd, p in procs:

@@ -136,15 +136,21 @@ __global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, 
         if (!d1ok) vf1 = (v8i){0, 0, 0, 0, 0, 0, 0, 0};
         // ---- logits in base-2 units, keys past S masked (only the last tile can hold them) ----
         const bool full = kb + FT <= S;
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) s[b][i] *= sl2;
+        if (!full) {                                       // (uniform: no per-element key test on the tiles before the last)
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) { const int key = kb + 32 * b + (i & 3) + 4 * h + 8 * (i >> 2); if (key >= S) s[b][i] = -INFINITY; }
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int b = 0; b < 2; b++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const int key = kb + 32 * b + (i & 3) + 4 * h + 8 * (i >> 2);
-                const float v = full || key < S ? s[b][i] * sl2 : -INFINITY;
-                s[b][i] = v; mx = fmaxf(mx, v);
-            }
+            for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[b][i]);
         mx = fmaxf(mx, a8_xor32f(mx, h));
         const float mn = fmaxf(m, mx), corr = __builtin_amdgcn_exp2f(m - mn);
         m = mn; l *= corr;

@@ -24,6 +24,13 @@ __device__ __forceinline__ float d_exp2i(int e) { return __uint_as_float((unsign
 __device__ __forceinline__ float d_mx_scale(unsigned sbyte) { return __uint_as_float((sbyte & 255u) << 23); }   // 0xFF -> +inf
 
 // NaN-propagating |v| max on the bit patterns (src/lp_common.cuh:487)
+// the value of lane ^ M (M 1 or 2: inside the lane's group of four) through the vector pipe's lane permute: no LDS round trip. Every lane
+// of the group must be active
+template <int M> __device__ __forceinline__ unsigned d_quad_xor_u(unsigned x) {
+    static_assert(M == 1 || M == 2, "d_quad_xor_u: lanes of one group of four");
+    return (unsigned)__builtin_amdgcn_mov_dpp((int)x, M == 1 ? 0xB1 : 0x4E, 0xF, 0xF, true);        // quad_perm [1, 0, 3, 2] / [2, 3, 0, 1]
+}
+template <int M> __device__ __forceinline__ float d_quad_xor_f(float x) { return __uint_as_float(d_quad_xor_u<M>(__float_as_uint(x))); }
 __device__ __forceinline__ unsigned d_amax_u(unsigned a, float v) { const unsigned b = __float_as_uint(v) & 0x7fffffffu; return b > a ? b : a; }
 
 // e4m3 (OCP FN: max 448, 0x7f NaN), round to nearest even, saturating. For |x| < 448 the value is rounded to a multiple of the

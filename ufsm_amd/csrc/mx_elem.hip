@@ -139,11 +139,16 @@ template <int HD> __device__ __forceinline__ float in_round(float v) {          
     if (HD == 1) { unsigned u = __float_as_uint(v); if ((u & 0x7fffffffu) > 0x7f800000u) return v; u += 0x7fffu + ((u >> 16) & 1u); return __uint_as_float(u & 0xffff0000u); }
     return v;
 }
+constexpr int PRED_BATCH = 16;                     // windows of one launch (their pointers travel in the kernel arguments)
+struct pred_src_t { const uint8_t *ct[PRED_BATCH]; const float *dyo[PRED_BATCH], *dxo[PRED_BATCH]; };
 template <int B, int HD, int VPT>
-__global__ void __launch_bounds__(256) pred_rows_k(const uint8_t *__restrict__ ct, int W, float mean, float isd, const float *__restrict__ dyo, const float *__restrict__ dxo, int axis, int z0, size_t S,
-                                                   uint8_t *__restrict__ yrows, uint8_t *__restrict__ ysc) {
+__global__ void __launch_bounds__(256) pred_rows_k(pred_src_t src_of, int W, float mean, float isd, int axis, int z0, size_t S,
+                                                   uint8_t *__restrict__ yrows0, uint8_t *__restrict__ ysc0) {
     const size_t v0 = (blockIdx.x * (size_t)256 + threadIdx.x) * VPT;         // first voxel of the thread, relative to plane z0
     if (v0 >= S) return;
+    // blockIdx.y: the window of the launch, i.e. the sample of the tensor counted from the launch's first
+    const uint8_t *__restrict__ ct = src_of.ct[blockIdx.y]; const float *__restrict__ dyo = src_of.dyo[blockIdx.y], *__restrict__ dxo = src_of.dxo[blockIdx.y];
+    uint8_t *__restrict__ yrows = yrows0 + blockIdx.y * S * (B == 8 ? 8 : 4), *__restrict__ ysc = ysc0 + blockIdx.y * S;
     const unsigned row = (unsigned)(v0 / (unsigned)W), xx0 = (unsigned)(v0 - (size_t)row * W), yy = row % (unsigned)W, z = (unsigned)z0 + row / (unsigned)W;
     const uint8_t *src = ct + ((size_t)z * W + yy) * W + xx0;
     unsigned cw;
@@ -179,19 +184,34 @@ __global__ void __launch_bounds__(256) pred_rows_k(const uint8_t *__restrict__ c
         ysc[v0] = (uint8_t)sb;
     }
 }
+// samples n0 .. n0 + nw - 1 of an N-sample input tensor from nw windows (ct, dyo, dxo: host arrays of nw device pointers)
+extern "C" void mi_pred_input_mx_batch(const uint8_t *const *ct, int W, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, int z0, int nz, void *y, int hd, int bits,
+                                       int N, int n0, int nw) {
+    const size_t S = (size_t)nz * W * W; if (!S || nw <= 0) return;
+    if (N < 1 || n0 < 0 || n0 + nw > N) mi_die("mi_pred_input_mx_batch: samples %d .. %d of %d", n0, n0 + nw - 1, N);
+    const int rb = bits == 4 ? 4 : 8;                                           // bytes of an 8-channel row
+    for (int j0 = 0; j0 < nw; j0 += PRED_BATCH) {
+        const int nb = nw - j0 < PRED_BATCH ? nw - j0 : PRED_BATCH, n = n0 + j0;
+        uint8_t *yrows = (uint8_t *)y + (size_t)n * S * rb, *ysc = (uint8_t *)y + (size_t)N * S * rb + (size_t)n * S;      // sample n's rows; the tensor's scale plane follows all rows
+        pred_src_t src;
+        bool v4 = W % 4 == 0 && ((uintptr_t)ysc & 3) == 0 && ((uintptr_t)yrows & 15) == 0;
+        for (int j = 0; j < PRED_BATCH; j++) {
+            const int k = j0 + (j < nb ? j : 0);
+            src.ct[j] = ct[k]; src.dyo[j] = dyo[k]; src.dxo[j] = dxo[k];
+            v4 = v4 && ((uintptr_t)ct[k] & 3) == 0;
+        }
+#define PIN(B, HD) do { if (v4) pred_rows_k<B, HD, 4><<<dim3(nblk_(S / 4, 256), nb), 256>>>(src, W, mean, isd, axis, z0, S, yrows, ysc); \
+                        else pred_rows_k<B, HD, 1><<<dim3(nblk_(S, 256), nb), 256>>>(src, W, mean, isd, axis, z0, S, yrows, ysc); } while (0)
+        if (bits == 4) { if (hd == 2) PIN(4, 2); else if (hd == 1) PIN(4, 1); else PIN(4, 0); }
+        else { if (hd == 2) PIN(8, 2); else if (hd == 1) PIN(8, 1); else PIN(8, 0); }
+#undef PIN
+    }
+    MICK();
+}
 // sample n of an N-sample input tensor (the reference's entry is one window: N 1, n 0)
 extern "C" void mi_pred_input_mx_n(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits, int N, int n) {
-    const size_t S = (size_t)nz * W * W; if (!S) return;
     if (N < 1 || n < 0 || n >= N) mi_die("mi_pred_input_mx_n: sample %d of %d", n, N);
-    const int rb = bits == 4 ? 4 : 8;                                           // bytes of an 8-channel row
-    uint8_t *yrows = (uint8_t *)y + (size_t)n * S * rb, *ysc = (uint8_t *)y + (size_t)N * S * rb + (size_t)n * S;      // sample n's rows; the tensor's scale plane follows all rows
-    const bool v4 = W % 4 == 0 && ((uintptr_t)ct & 3) == 0 && ((uintptr_t)ysc & 3) == 0 && ((uintptr_t)yrows & 15) == 0;
-#define PIN(B, HD) do { if (v4) pred_rows_k<B, HD, 4><<<nblk_(S / 4, 256), 256>>>(ct, W, mean, isd, dyo, dxo, axis, z0, S, yrows, ysc); \
-                        else pred_rows_k<B, HD, 1><<<nblk_(S, 256), 256>>>(ct, W, mean, isd, dyo, dxo, axis, z0, S, yrows, ysc); } while (0)
-    if (bits == 4) { if (hd == 2) PIN(4, 2); else if (hd == 1) PIN(4, 1); else PIN(4, 0); }
-    else { if (hd == 2) PIN(8, 2); else if (hd == 1) PIN(8, 1); else PIN(8, 0); }
-#undef PIN
-    MICK();
+    mi_pred_input_mx_batch(&ct, W, mean, isd, &dyo, &dxo, axis, z0, nz, y, hd, bits, N, n, 1);
 }
 extern "C" void lp_pred_input_mx(const uint8_t *ct, int W, float mean, float isd, const float *dyo, const float *dxo, int axis, int z0, int nz, void *y, int hd, int bits) {
     mi_pred_input_mx_n(ct, W, mean, isd, dyo, dxo, axis, z0, nz, y, hd, bits, 1, 0);
@@ -828,6 +848,7 @@ void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg
 // threads of a cell meet for the row amax through lane exchanges. Each coarse row is decoded once per cell instead of once per fine voxel.
 // H2: the fp4 entry's blend (stage_up_smem_h2, src/lp_common.cuh:674-712): binary16 weights relative to the largest of the cell's 8 scale bytes,
 // binary16 fused multiply-adds in the same z, y, x order (an e4m3 code is a binary16 value), the sum widened and scaled by 2^e_max.
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 template <int BY, bool H2>
 __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y, int N, int nbo, int D, int H, int W, int zlo, int zhi, int clo, int Dcs, int mz0, int ncz_) {
     // fine planes [zlo, zhi) of the depth-D result, written at their place in the depth-D tensor y; xc holds the coarse planes [clo, clo + Dcs)
@@ -844,13 +865,19 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
     const int mx = (int)(cc - cyi * ncx) - 1, my = (int)cyi - 1, mz = (int)blockIdx.z + mz0;
     const int cz[2] = {max(mz, 0), min(mz + 1, Dc - 1)}, cy[2] = {max(my, 0), min(my + 1, Hc - 1)}, cx[2] = {max(mx, 0), min(mx + 1, Wc - 1)};
     const uint8_t *xs = xc + (size_t)N * nbo * Sc * 32;
-    float f[8][8], sc[8];
+    float f[H2 ? 1 : 8][8], sc[8];
+    __half2 hf[H2 ? 8 : 1][4];                                // H2: the rows' values as binary16 pairs (an e4m3 value is one exactly), formed once per cell
     unsigned sb[8], em = 0u;
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         const size_t row = (size_t)nbk * Sc + ((size_t)(cz[k >> 2] - clo) * Hc + cy[(k >> 1) & 1]) * Wc + cx[k & 1];
         const uint2 w = *(const uint2 *)(xc + row * 32 + q * 8);
-        d_dec4_e4m3(w.x, f[k]); d_dec4_e4m3(w.y, f[k] + 4);
+        if constexpr (H2) {
+            hf[k][0] = __builtin_bit_cast(__half2, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.x, 1.f, false));
+            hf[k][1] = __builtin_bit_cast(__half2, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.x, 1.f, true));
+            hf[k][2] = __builtin_bit_cast(__half2, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.y, 1.f, false));
+            hf[k][3] = __builtin_bit_cast(__half2, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.y, 1.f, true));
+        } else { d_dec4_e4m3(w.x, f[k]); d_dec4_e4m3(w.y, f[k] + 4); }
         sb[k] = xs[row]; em = max(em, sb[k]);
         sc[k] = d_mx_scale(sb[k]);
     }
@@ -859,21 +886,36 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
         for (int k = 0; k < 8; k++) { const int de = (int)sb[k] - (int)em; sc[k] = de >= -126 ? __uint_as_float((unsigned)(127 + de) << 23) : 0.f; }     // 2^(e_row - e_max)
     }
     const float smax = d_mx_scale(em);
-    uint8_t *ys = y + (size_t)N * nbo * S * (BY * 4);
-    __half2 hf[H2 ? 8 : 1][4];                                // H2: the rows' values as binary16 pairs (an e4m3 value is one exactly), formed once per cell
-    if constexpr (H2) {
+    // the blend weight of coarse row k for a fine voxel that is `far` axes away from it: (3/4)^(3 - far) (1/4)^far times the row's scale
+    // (the products of .75 and .25 are exact, so this is the value of the reference's ((wz wy) wx) s). 32 per cell, shared by its 8 fine voxels
+    const float cw[4] = {0.421875f, 0.140625f, 0.046875f, 0.015625f};
+    float w32[H2 ? 1 : 8][4];
+    __half2 w16[H2 ? 8 : 1][4];
 #pragma unroll
-        for (int k = 0; k < 8; k++)
+    for (int k = 0; k < 8; k++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) hf[k][i] = __floats2half2_rn(f[k][2 * i], f[k][2 * i + 1]);
-    }
+        for (int far = 0; far < 4; far++) {
+            if constexpr (H2) w16[k][far] = __half2half2(__float2half_rn(cw[far] * sc[k])); else w32[k][far] = cw[far] * sc[k];
+        }
+    // output rows: fine voxel p = (pz, py, px) of the cell is voxel (2 mz + 1 + pz, 2 my + 1 + py, 2 mx + 1 + px); row0 is p = 0's row in the
+    // tensor (outside it for cells on the low borders, whose p = 0 is not stored)
+    constexpr int RB = BY * 4;                                                    // bytes of a 32-channel row
+    const long long row0 = (long long)nbk * (long long)S + ((long long)(2 * mz + 1) * H + (2 * my + 1)) * W + (2 * mx + 1);
+    uint8_t *ys = y + (size_t)N * nbo * S * RB;
+    const bool okz[2] = {2 * mz + 1 >= zlo && 2 * mz + 1 < zhi, 2 * mz + 2 >= zlo && 2 * mz + 2 < zhi};
+    const bool oky[2] = {my >= 0, 2 * my + 2 < H}, okx[2] = {live && mx >= 0, live && 2 * mx + 2 < W};
+    // the binary16 form can encode straight from the binary16 sums when widening them (x 2^e_max) is exact, i.e. no product leaves the
+    // normal binary32 range: 2^-24 2^(e_max - 127) >= 2^-126 and 65504 2^(e_max - 127) < 2^128. Decided per wavefront
+    const bool direct = H2 && BY == 4 && __builtin_amdgcn_ballot_w64(em < 25u || em > 238u) == 0ull;
+    const float am_direct = __uint_as_float((em - 9u) << 23);                    // 2^-9 of the cell's scale: block maxima below it take the widened form (binary16 subnormals)
+    int eq[4];                                                                     // the exponents of the four voxels of a z layer of the cell, for their scale bytes
 #pragma unroll
     for (int p = 0; p < 8; p++) {
-        const int pz = p >> 2, py = (p >> 1) & 1, px = p & 1;                     // fine voxel 2m + 1 + p: p = 0 has its own coarse row at m, p = 1 at m + 1
-        const int gz = 2 * mz + 1 + pz, gy = 2 * my + 1 + py, gx = 2 * mx + 1 + px;
-        float acc[8];
+        const int pz = p >> 2, py = (p >> 1) & 1, px = p & 1;                     // p = 0 has its own coarse row at m, p = 1 at m + 1
+        float acc[8], am;
+        __half2 hacc[4];
         if constexpr (H2) {
-            __half2 hacc[4];                                  // two channels per packed fused multiply-add: each half rounds once, as the scalar form
+            // two channels per packed fused multiply-add: each half rounds once, as the scalar form
 #pragma unroll
             for (int i = 0; i < 4; i++) hacc[i] = __floats2half2_rn(0.f, 0.f);
 #pragma unroll
@@ -883,39 +925,71 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
 #pragma unroll
                     for (int c = 0; c < 2; c++) {
                         const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);
-                        const __half2 w3 = __half2half2(__float2half_rn((a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f) * sc[k]));
 #pragma unroll
-                        for (int i = 0; i < 4; i++) hacc[i] = __hfma2(w3, hf[k][i], hacc[i]);
+                        for (int i = 0; i < 4; i++) hacc[i] = __hfma2(w16[k][a + b + c], hf[k][i], hacc[i]);
                     }
+            // max |sum| 2^e_max: the widening is monotone, so the largest sum gives the largest product (NaN sums are skipped, as fmaxf skips
+            // them below; a product that is NaN - 0 x inf - counts as 0 there too)
+            h2_t m = __builtin_elementwise_abs(__builtin_bit_cast(h2_t, hacc[0]));
 #pragma unroll
-            for (int i = 0; i < 4; i++) { acc[2 * i] = __low2float(hacc[i]) * smax; acc[2 * i + 1] = __high2float(hacc[i]) * smax; }
+            for (int i = 1; i < 4; i++) m = __builtin_elementwise_max(m, __builtin_elementwise_abs(__builtin_bit_cast(h2_t, hacc[i])));
+            am = fmaxf(0.f, fmaxf((float)m.x, (float)m.y) * smax);
         } else {
 #pragma unroll
-        for (int i = 0; i < 8; i++) acc[i] = 0.f;
+            for (int i = 0; i < 8; i++) acc[i] = 0.f;
 #pragma unroll
-        for (int a = 0; a < 2; a++)
+            for (int a = 0; a < 2; a++)
 #pragma unroll
-            for (int b = 0; b < 2; b++)
+                for (int b = 0; b < 2; b++)
 #pragma unroll
-                for (int c = 0; c < 2; c++) {
-                    const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);   // a = 0: the voxel's own coarse row, a = 1: its neighbour
-                    const float w3 = (a ? 0.25f : 0.75f) * (b ? 0.25f : 0.75f) * (c ? 0.25f : 0.75f) * sc[k];
+                    for (int c = 0; c < 2; c++) {
+                        const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);   // a = 0: the voxel's own coarse row, a = 1: its neighbour
 #pragma unroll
-                    for (int i = 0; i < 8; i++) acc[i] = fmaf(w3, f[k][i], acc[i]);
-                }
+                        for (int i = 0; i < 8; i++) acc[i] = fmaf(w32[k][a + b + c], f[k][i], acc[i]);
+                    }
+            am = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) am = fmaxf(am, fabsf(acc[i]));
         }
-        float am = 0.f;
-#pragma unroll
-        for (int i = 0; i < 8; i++) am = fmaxf(am, fabsf(acc[i]));
-        am = fmaxf(am, __shfl_xor(am, 1)); am = fmaxf(am, __shfl_xor(am, 2));
+        {   // the four threads of the cell hold the row's 32 channels; am is a non-negative number (no NaN, no -0): it orders as its bit pattern
+            unsigned au = __float_as_uint(am);
+            au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
+            am = __uint_as_float(au);
+        }
         const int e = d_mx_exp(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
-        if (!live || gz < zlo || gz >= zhi || gy < 0 || gy >= H || gx < 0 || gx >= W) continue;
-        const size_t row = (size_t)nbk * S + ((size_t)gz * H + gy) * W + gx;
-        if (BY == 8) {
-            uint2 o; o.x = d_enc4_e4m3(acc[0], acc[1], acc[2], acc[3], e); o.y = d_enc4_e4m3(acc[4], acc[5], acc[6], acc[7], e);
-            *(uint2 *)(y + row * 32 + q * 8) = o;
-        } else *(unsigned *)(y + row * 16 + q * 4) = d_enc8_e2m1(acc, e);
-        if (!q) ys[row] = (uint8_t)(e + 127);
+        eq[p & 3] = e;
+        const bool ok = okz[pz] && oky[py] && okx[px];
+        uint8_t *dst = y + (row0 + ((long long)pz * H + py) * W + px) * RB + q * (RB / 4);
+        bool done = false;
+        if constexpr (H2 && BY == 4) {
+            if (direct && __builtin_amdgcn_ballot_w64(!(am >= am_direct) || e == 128) == 0ull) {
+                // (sum 2^(e_max - 127)) / 2^e = sum / 2^(e - e_max + 127): the same quotient, rounded once by the conversion either way
+                const float ds = d_exp2i(e - (int)em + 127);
+                unsigned w = 0u;
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, __builtin_bit_cast(h2_t, hacc[0]), ds, 0);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, __builtin_bit_cast(h2_t, hacc[1]), ds, 1);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, __builtin_bit_cast(h2_t, hacc[2]), ds, 2);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, __builtin_bit_cast(h2_t, hacc[3]), ds, 3);
+                if (ok) *(unsigned *)dst = w;
+                done = true;
+            }
+        }
+        if (!done) {
+            if constexpr (H2) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) { acc[2 * i] = __low2float(hacc[i]) * smax; acc[2 * i + 1] = __high2float(hacc[i]) * smax; }
+            }
+            if (BY == 8) {
+                uint2 o; o.x = d_enc4_e4m3(acc[0], acc[1], acc[2], acc[3], e); o.y = d_enc4_e4m3(acc[4], acc[5], acc[6], acc[7], e);
+                if (ok) *(uint2 *)dst = o;
+            } else { const unsigned o = d_enc8_e2m1(acc, e); if (ok) *(unsigned *)dst = o; }
+        }
+        if ((p & 3) == 3) {
+            // the scale bytes of the layer's four voxels in one store: thread q writes voxel (pz, q >> 1, q & 1)
+            const int ev = q == 0 ? eq[0] : q == 1 ? eq[1] : q == 2 ? eq[2] : eq[3];
+            const bool oks = okz[pz] && (q & 2 ? oky[1] : oky[0]) && (q & 1 ? okx[1] : okx[0]);
+            if (oks) ys[row0 + ((long long)pz * H + (q >> 1)) * W + (q & 1)] = (uint8_t)(ev + 127);
+        }
     }
 }
 // fine planes [zlo, zhi) of the upsampled depth-D tensor, written at their place in the depth-D MX tensor y

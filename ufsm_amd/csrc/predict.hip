@@ -13,10 +13,13 @@ extern "C" int nn_get_pred_iso(void) { return g_pred_iso; }
 // contiguous reads, its bytes one contiguous write), the runs of a row are neighbouring threads ----
 constexpr int PLACE_RUN = 8;
 struct place_rows_t { int z0, y0, x0, ny, nx, nrun; };
-__global__ void __launch_bounds__(256) place_rows_k(const float *__restrict__ lg, const uint8_t *__restrict__ ct, place_rows_t P, size_t nthreads, int W, int oz, int oy, int ox, int shard,
-                                                    uint8_t *__restrict__ dsh, int iso) {
+constexpr int PRED_BATCH = 16;                     // windows of one launch (their offsets travel in the kernel arguments)
+struct place_dst_t { long long off[PRED_BATCH]; };      // window j (blockIdx.y) writes from dsh + off[j]
+__global__ void __launch_bounds__(256) place_rows_k(const float *__restrict__ lg0, size_t lstride, const uint8_t *__restrict__ ct0, size_t cstride, place_rows_t P, size_t nthreads, int W,
+                                                    int oz, int oy, int ox, int shard, uint8_t *__restrict__ dsh0, place_dst_t dst, int iso) {
     const size_t t = blockIdx.x * (size_t)256 + threadIdx.x;
     if (t >= nthreads) return;
+    const float *lg = lg0 + blockIdx.y * lstride; const uint8_t *ct = ct0 + blockIdx.y * cstride; uint8_t *dsh = dsh0 + dst.off[blockIdx.y];
     const size_t row = t / (unsigned)P.nrun;
     const int run = (int)(t - row * P.nrun), y = P.y0 + (int)(row % (unsigned)P.ny), z = P.z0 + (int)(row / (unsigned)P.ny), x = P.x0 + run * PLACE_RUN;
     const int n = min(PLACE_RUN, P.x0 + P.nx - x);
@@ -28,25 +31,40 @@ __global__ void __launch_bounds__(256) place_rows_k(const float *__restrict__ lg
 #pragma unroll
     for (int i = 0; i < PLACE_RUN; i++) if (i < n) o[i] = m[i] >= iso ? (uint8_t)(255.f / (1.f + expf(-v[i])) + 0.5f) : (uint8_t)0;
 }
-extern "C" void nn_pred_place_d(const float *lg, const uint8_t *ct, int D, int W, int hz, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, uint8_t *dsh) {
+// n windows of one geometry: window j's logits at lg + j lstride (floats), its CT at ct + j cstride, its target dsh + doff[j] (doff on the host)
+extern "C" void mi_pred_place_n(const float *lg, size_t lstride, const uint8_t *ct, size_t cstride, int n, const int64_t *doff, int D, int W, int hz, int halo, int oz, int oy, int ox,
+                                int ez, int ey, int ex, int shard, uint8_t *dsh) {
     // window voxel v lands at o + v of the target; kept: v inside the interior [h, dim - h) of its axis and o + v inside [0, e)
     const int lo[3] = {max(hz, -oz), max(halo, -oy), max(halo, -ox)}, hi[3] = {min(D - hz, ez - oz), min(W - halo, ey - oy), min(W - halo, ex - ox)};
     if (hi[0] <= lo[0] || hi[1] <= lo[1] || hi[2] <= lo[2]) return;
     place_rows_t P = {lo[0], lo[1], lo[2], hi[1] - lo[1], hi[2] - lo[2], (hi[2] - lo[2] + PLACE_RUN - 1) / PLACE_RUN};
     const size_t nthreads = (size_t)(hi[0] - lo[0]) * P.ny * P.nrun;
-    place_rows_k<<<nblk_(nthreads, 256), 256>>>(lg, ct, P, nthreads, W, oz, oy, ox, shard, dsh, g_pred_iso);
+    for (int j0 = 0; j0 < n; j0 += PRED_BATCH) {
+        const int nb = min(PRED_BATCH, n - j0);
+        place_dst_t dst;
+        for (int j = 0; j < PRED_BATCH; j++) dst.off[j] = j < nb ? (doff ? doff[j0 + j] : 0) : 0;
+        place_rows_k<<<dim3(nblk_(nthreads, 256), nb), 256>>>(lg + (size_t)j0 * lstride, lstride, ct + (size_t)j0 * cstride, cstride, P, nthreads, W, oz, oy, ox, shard, dsh, dst, g_pred_iso);
+    }
     MICK();
+}
+extern "C" void nn_pred_place_d(const float *lg, const uint8_t *ct, int D, int W, int hz, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, uint8_t *dsh) {
+    mi_pred_place_n(lg, 0, ct, 0, 1, nullptr, D, W, hz, halo, oz, oy, ox, ez, ey, ex, shard, dsh);
 }
 extern "C" void nn_pred_place(const float *lg, const uint8_t *ct, int W, int halo, int oz, int oy, int ox, int ez, int ey, int ex, int shard, uint8_t *dsh) {
     nn_pred_place_d(lg, ct, W, W, halo, halo, oz, oy, ox, ez, ey, ex, shard, dsh);
 }
 
-// a thread moves 16 consecutive x of one window row: one 16-byte store, byte loads on the volume side (window origins are not aligned)
-__global__ void __launch_bounds__(256) ct_window_k(const uint8_t *__restrict__ vol, long long Z, long long Y, long long X, long long oz, long long oy, long long ox,
-                                                   int W, uint8_t *__restrict__ win, int iso, int halo, unsigned *any) {
+// a thread moves 16 consecutive x of one window row: one 16-byte store, byte loads on the volume side (window origins are not aligned).
+// blockIdx.y is the window of the launch: its origin from the kernel arguments, its bytes at win + y W^3, its flag at any + y
+struct ctw_org_t { long long o[PRED_BATCH][3]; };
+__global__ void __launch_bounds__(256) ct_window_k(const uint8_t *__restrict__ vol, long long Z, long long Y, long long X, ctw_org_t org,
+                                                   int W, uint8_t *__restrict__ win0, int iso, int halo, unsigned *any0) {
     const int W16 = (W + 15) >> 4;
     const size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x;
     if (i >= (size_t)W * W * W16) return;
+    const long long oz = org.o[blockIdx.y][0], oy = org.o[blockIdx.y][1], ox = org.o[blockIdx.y][2];
+    uint8_t *win = win0 + blockIdx.y * ((size_t)W * W * W);
+    unsigned *any = any0 ? any0 + blockIdx.y : nullptr;
     const int xc = (int)(i % W16), y = (int)((i / W16) % W), z = (int)(i / ((size_t)W16 * W));
     const long long gz = oz + z, gy = oy + y;
     const bool rowin = gz >= 0 && gz < Z && gy >= 0 && gy < Y;
@@ -71,10 +89,56 @@ __global__ void __launch_bounds__(256) ct_window_k(const uint8_t *__restrict__ v
         if ((threadIdx.x & 63) == __builtin_ctzll(__builtin_amdgcn_ballot_w64(true)) && *(volatile unsigned *)any == 0u) atomicOr(any, 1u);
     }
 }
+// n windows: window j's origin org[3 j .. 3 j + 2] (host), its bytes at win + j W^3, its flag any + j (any may be null)
+extern "C" void mi_ct_windows(const uint8_t *vol, int64_t Z, int64_t Y, int64_t X, const int64_t *org, int n, int W, uint8_t *win, int iso, int halo, unsigned *any) {
+    if (W <= 0 || n <= 0) return;
+    const size_t nt = (size_t)W * W * ((W + 15) >> 4), w3 = (size_t)W * W * W;
+    for (int j0 = 0; j0 < n; j0 += PRED_BATCH) {
+        const int nb = min(PRED_BATCH, n - j0);
+        ctw_org_t o;
+        for (int j = 0; j < PRED_BATCH; j++) for (int d = 0; d < 3; d++) o.o[j][d] = j < nb ? org[3 * (j0 + j) + d] : 0;
+        ct_window_k<<<dim3(nblk_(nt, 256), nb), 256>>>(vol, Z, Y, X, o, W, win + (size_t)j0 * w3, iso, halo, any ? any + j0 : nullptr);
+    }
+    MICK();
+}
 extern "C" void mi_ct_window(const uint8_t *vol, int64_t Z, int64_t Y, int64_t X, int64_t oz, int64_t oy, int64_t ox, int W, uint8_t *win, int iso, int halo, unsigned *any) {
-    if (W <= 0) return;
-    const size_t n = (size_t)W * W * ((W + 15) >> 4);
-    ct_window_k<<<nblk_(n, 256), 256>>>(vol, Z, Y, X, oz, oy, ox, W, win, iso, halo, any);
+    const int64_t org[3] = {oz, oy, ox};
+    mi_ct_windows(vol, Z, Y, X, org, 1, W, win, iso, halo, any);
+}
+
+// "holds a voxel >= iso" of every cell of a grid over the volume: cell (a, b, c) of nss[3] is [a S, a S + S) x [b S, ..) x [c S, ..) clipped to the
+// volume, i.e. the interior of the sliding window with that index. The cells tile the volume, so this is one read of it. A thread tests 16
+// consecutive x of a cell row (one 16-byte load where the row start allows, else bytes); a workgroup's rows belong to one cell
+__global__ void __launch_bounds__(256) ct_flags_k(const uint8_t *__restrict__ vol, long long Z, long long Y, long long X, int S, int n1, int n2, int iso, unsigned *__restrict__ any, int vec) {
+    const int S16 = (S + 15) >> 4;
+    const unsigned cell = blockIdx.x, c = cell % (unsigned)n2, b = (cell / (unsigned)n2) % (unsigned)n1, a = cell / ((unsigned)n2 * (unsigned)n1);
+    const size_t i = blockIdx.y * (size_t)256 + threadIdx.x;
+    unsigned found = 0u;
+    if (i < (size_t)S * S * S16) {
+        const int xc = (int)(i % S16), y = (int)((i / S16) % S), z = (int)(i / ((size_t)S16 * S));
+        const long long gz = (long long)a * S + z, gy = (long long)b * S + y, gx0 = (long long)c * S + xc * 16;
+        if (gz < Z && gy < Y && gx0 < X) {
+            const uint8_t *src = vol + ((size_t)gz * Y + gy) * X + gx0;
+            const int nx = (int)min((long long)min(16, S - xc * 16), X - gx0);
+            if (vec && nx == 16) {
+                const uint4 q = *(const uint4 *)src;
+                const unsigned w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                for (int k = 0; k < 16; k++) found |= (int)((w[k >> 2] >> (8 * (k & 3))) & 255u) >= iso;
+            } else for (int k = 0; k < nx; k++) found |= (int)src[k] >= iso;
+        }
+    }
+    if (__builtin_amdgcn_ballot_w64(found != 0u) != 0ull) {
+        if ((threadIdx.x & 63) == __builtin_ctzll(__builtin_amdgcn_ballot_w64(true)) && *(volatile unsigned *)(any + cell) == 0u) atomicOr(any + cell, 1u);
+    }
+}
+extern "C" void mi_ct_flags(const uint8_t *vol, int64_t Z, int64_t Y, int64_t X, int S, const int64_t nss[3], int iso, unsigned *any) {
+    const int64_t total = nss[0] * nss[1] * nss[2];
+    if (S <= 0 || total <= 0) return;
+    const size_t nt = (size_t)S * S * ((S + 15) >> 4);
+    if (total > 0x7fffffff || nblk_(nt, 256) > 65535u) mi_die("mi_ct_flags: %lld cells of %d^3 do not fit one launch", (long long)total, S);
+    const int vec = S % 16 == 0 && X % 16 == 0 && ((uintptr_t)vol & 15) == 0;
+    ct_flags_k<<<dim3((unsigned)total, nblk_(nt, 256)), 256>>>(vol, Z, Y, X, S, (int)nss[1], (int)nss[2], iso, any, vec);
     MICK();
 }
 

@@ -32,9 +32,9 @@ int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, 
      * of pass 2 are then enqueued back to back and the GPU never waits for the host. */
     if (!rc) {
         mi_zero(dany, (size_t)total * sizeof(unsigned));
+        mi_ct_flags(vol, dims[0], dims[1], dims[2], S, nss, iso, dany);       /* (a window's interior is cell (a, b, c) of the S grid: one read of the volume) */
         for (int64_t a = 0; a < nss[0]; a++) for (int64_t b = 0; b < nss[1]; b++) for (int64_t c = 0; c < nss[2]; c++) {
-            const int64_t id = (a * nss[1] + b) * nss[2] + c, oz = a * S - halo, oy = b * S - halo, ox = c * S - halo;
-            mi_ct_window(vol, dims[0], dims[1], dims[2], oz, oy, ox, W, ctw, iso, halo, dany + id);
+            const int64_t id = (a * nss[1] + b) * nss[2] + c, oy = b * S - halo, ox = c * S - halo;
             float *ho = hoff + (size_t)id * 2 * W;
             for (int z = 0; z < W; z++) { ho[z] = (float)oy - cy; ho[W + z] = (float)ox - cx; }
         }
@@ -47,20 +47,20 @@ int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, 
     if (!list) rc = -1;
     for (int64_t id = 0; id < total && !rc; id++) if (hany[id]) list[np++] = id;
     for (int64_t k = 0; k < np && !rc; k += in.n) {
-        const uint8_t *cts[16]; const float *dyos[16], *dxos[16]; int64_t ids[16];
+        const uint8_t *cts[16]; const float *dyos[16], *dxos[16]; int64_t org[16 * 3], eoff[16];
+        const int nreal = (int)(np - k < in.n ? np - k : in.n);
         for (int j = 0; j < in.n; j++) {
             const int64_t id = list[k + j < np ? k + j : np - 1], a = id / (nss[1] * nss[2]), b = (id / nss[2]) % nss[1], c = id % nss[2];
-            ids[j] = id;
-            mi_ct_window(vol, dims[0], dims[1], dims[2], a * S - halo, b * S - halo, c * S - halo, W, ctw + (size_t)j * w3, iso, halo, NULL);
+            org[3 * j] = a * S - halo; org[3 * j + 1] = b * S - halo; org[3 * j + 2] = c * S - halo;
+            eoff[j] = id * (int64_t)e3;
             cts[j] = ctw + (size_t)j * w3; dyos[j] = doff + (size_t)id * 2 * W; dxos[j] = dyos[j] + W;
         }
+        mi_ct_windows(vol, dims[0], dims[1], dims[2], org, in.n, W, ctw, iso, halo, NULL);
         const float *lg = mi_unet_forward_ct_n(u, cts, mean, isd, dyos, dxos, axis, in, 2);      /* (fp16-rounded input values, as predict) */
         if (!lg) { rc = -1; break; }
-        for (int j = 0; j < in.n && k + j < np; j++) {
-            /* E: the interior and B voxels of the upper halo, window coordinates [halo, halo + S + B) -> [0, S + B) (src/predict.c:3426-3427) */
-            nn_pred_place(lg + (size_t)j * lgn, cts[j], W, halo - B, -halo, -halo, -halo, En, En, En, En, E + (size_t)ids[j] * e3);
-            present[ids[j]] = 1; done++;
-        }
+        /* E: the interior and B voxels of the upper halo, window coordinates [halo, halo + S + B) -> [0, S + B) (src/predict.c:3426-3427) */
+        mi_pred_place_n(lg, lgn, ctw, w3, nreal, eoff, W, W, halo - B, halo - B, -halo, -halo, -halo, En, En, En, En, E);
+        for (int j = 0; j < nreal; j++) { present[list[k + j]] = 1; done++; }
     }
     free(list);
     if (!rc) {

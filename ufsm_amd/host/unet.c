@@ -657,8 +657,7 @@ const float *unet_forward(unet *u, const float *x, shape5 xs, int train) { retur
 const float *mi_unet_forward_ct_n(unet *u, const uint8_t *const *ct, float mean, float isd, const float *const *dyo, const float *const *dxo, int axis, shape5 xs, int h16) {
     if (xs.c != 4 || u->cfg.cin != 4 || xs.h != xs.w) { fprintf(stderr, "unet_forward_ct: needs square windows of 4 input channels\n"); return nullptr; }
     if (ensure_built(u, xs)) return nullptr;
-    for (int n = 0; n < xs.n; n++)
-        mi_pred_input_mx_n(ct[n], xs.w, mean, isd, dyo[n], dxo[n], axis, 0, xs.d, u->xin, h16, u->act_dt == 4 ? 4 : 8, xs.n, n);
+    mi_pred_input_mx_batch(ct, xs.w, mean, isd, dyo, dxo, axis, 0, xs.d, u->xin, h16, u->act_dt == 4 ? 4 : 8, xs.n, 0, xs.n);
     return mi_unet_forward_mx(u, u->xin, xs);
 }
 const float *unet_forward_ct(unet *u, const uint8_t *ct, float mean, float isd, const float *dyo, const float *dxo, int axis, shape5 xs, int h16) {

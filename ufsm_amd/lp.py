@@ -66,6 +66,7 @@ _PROTOS = {
     "lp_pred_input_mx": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I, _I]),
     "lp_pred_input_mx8": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I]),
     "mi_pred_input_mx_n": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I]),
+    "mi_pred_input_mx_batch": (None, [_P, _I, _F, _F, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I]),
     "lp_gn_silu_apply_mx": (None, [_P, _I, shape5, _I, _P, _P, _P, _P, _P, _I]),
     "lp_add_mx": (None, [_P, _P, shape5, _I, C.c_uint]),
     "lp_up2_fwd_mx": (None, [_P, _I, shape5, _P, _I, gnp_t]),
@@ -171,6 +172,9 @@ _PRED_PROTOS = {
     "nn_pred_place_d": (None, [_P, _P] + [_I] * 11 + [_P]),
     "nn_pred_place": (None, [_P, _P] + [_I] * 9 + [_P]),
     "mi_ct_window": (None, [_P] + [C.c_int64] * 6 + [_I, _P, _I, _I, _P]),
+    "mi_ct_windows": (None, [_P] + [C.c_int64] * 3 + [C.POINTER(C.c_int64), _I, _I, _P, _I, _I, _P]),
+    "mi_ct_flags": (None, [_P] + [C.c_int64] * 3 + [_I, C.POINTER(C.c_int64), _I, _P]),
+    "mi_pred_place_n": (None, [_P, C.c_size_t, _P, C.c_size_t, _I, C.POINTER(C.c_int64)] + [_I] * 11 + [_P]),
     "mi_feather_blend": (_I, [_P, _P, _I, _I, C.POINTER(C.c_int64), C.POINTER(C.c_int64), _P]),
 }
 PRED_EXPORTS = tuple(_PRED_PROTOS)
