@@ -40,6 +40,10 @@ int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, const float *A,
    32 keys inside each tile of 64 keys. o: fp32 [nseq S][C], head h in columns h 48 ... ; lse: fp32 [nseq][H][S], base-2 logarithm of the
    softmax denominator plus the maximum logit in base-2 units. C must equal 48 H. Returns 0, or -1 when scratch cannot be allocated. */
 int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom *g, int H, int C);
+/* (no counterpart: a tuning knob for tests) wavefronts per workgroup of at_fa8_fwd's kernel: 1 or 4, anything else = chosen from the launch
+   size. With 4, a sequence's last 32-query tile, when it is the only one of its workgroup, is worked on by all four wavefronts (a range of the
+   keys each, merged in wavefront order): the same probabilities and codes as with 1, their sums added in another order (~1e-7 relative) */
+void at_fa8_waves(int nw);
 
 /* ---- the attention block around those two (forward, self-attention path; src/attn.h:26-81, src/nn_attn.cu) ---- */
 #define AT_DFM_NLV (AT_DFM_MAXL + 1)

@@ -133,6 +133,33 @@ def test_attention_full_size_of_the_window_bottleneck(gpu):
     assert np.isfinite(o).all() and np.isfinite(lse).all()
 
 
+@pytest.mark.parametrize("nseq,S,H", [(2, 4 + 8 ** 3, 2), (1, 128 * 3 + 1, 1), (3, 5, 1), (1, 250, 2)])
+def test_attention_four_wavefront_workgroups_and_the_shared_last_tile(gpu, nseq, S, H):
+    """Workgroups of four wavefronts (the launch the window bottleneck's eight sequences get). 4 + 8^3 and 385 tokens leave a last 32-query tile
+    alone in its workgroup: its keys are shared among the four wavefronts and merged. Those rows are the same probabilities summed in another
+    order (the other rows' bits do not change); 5 tokens: the only tile is such a tile and three wavefronts hold no keys; 250: no shared tile."""
+    rng = np.random.default_rng(nseq * S + H + 1)
+    qk = normed_qkv(rng, nseq, S, H)
+    lib.at_fa8_waves(1)
+    o1, l1 = gpu_attention(qk, nseq, S, H)
+    lib.at_fa8_waves(4)
+    try:
+        o4, l4 = gpu_attention(qk, nseq, S, H)
+    finally:
+        lib.at_fa8_waves(0)
+    shared = ((S + 31) // 32) % 4 == 1
+    first = (S - 1) // 32 * 32 if shared else S                  # first token of the shared tile
+    o1s, o4s = o1.reshape(nseq, S, -1), o4.reshape(nseq, S, -1)
+    assert np.array_equal(o1s[:, :first], o4s[:, :first]) and np.array_equal(l1[:, :, :first], l4[:, :, :first])
+    wo, wl = orc.fa8_fwd(qk, nseq, S, H)
+    rows = np.abs(o4 - wo).max(1) / np.abs(wo).max()
+    assert np.median(rows) < 1e-4 and rows.max() < 2e-2 and np.linalg.norm(o4 - wo) <= 3e-3 * np.linalg.norm(wo)
+    assert np.abs(l4 - wl).max() < 1e-4 * max(1.0, np.abs(wl).max())
+    if shared:                                                    # the same probabilities and codes, summed in another order
+        d = np.abs(o4s[:, first:] - o1s[:, first:]).max() / np.abs(wo).max()
+        assert d < 1e-5 and np.abs(l4[:, :, first:] - l1[:, :, first:]).max() < 1e-5 and np.isfinite(o4).all() and np.isfinite(l4).all()
+
+
 def test_attention_closed_forms(gpu):
     """q = 0: o is the mean of the quantised V over the S valid keys and lse = log2 S, exactly as on the oracle; rows of another
     sequence or of the padding must not leak in."""

@@ -89,8 +89,15 @@ __global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, 
                                                 const uint8_t *__restrict__ Vt, const uint8_t *__restrict__ Vts, float *__restrict__ o, float *__restrict__ lse,
                                                 int S, int Sp, int H, int C, long long R, float sl2) {
     const int seq = blockIdx.z, hd = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
-    const int q0 = (blockIdx.x * (blockDim.x >> 6) + wave) * 32;      // wavefronts are independent: any number per workgroup
-    if (q0 >= S) return;                                   // (no barriers: a wavefront without queries leaves)
+    const int nwv = blockDim.x >> 6, tq = blockIdx.x * nwv;
+    // A four-wavefront workgroup whose first wavefront alone has queries (the sequence's last 32-query tile: the few tokens past a multiple
+    // of 128) shares that tile's keys among its wavefronts, a range of the key tiles each, and wavefront 0 merges the four partial
+    // softmaxes: the tile costs a third of a wavefront's full pass instead of one that the rest of the GPU waits for. Each wavefront starts
+    // from the running maximum of the tiles before its range, so the probabilities and their e4m3 codes are those of the one-wavefront
+    // pass; only the order in which the partial sums are added differs
+    const bool split = nwv == 4 && (tq + 1) * 32 >= S;
+    const int q0 = (split ? tq : tq + wave) * 32;
+    if (q0 >= S) return;                                   // (no barriers outside a split workgroup: a wavefront without queries leaves)
     const long long rb = (long long)hd * R + (long long)seq * Sp;          // the sequence's first row in the row-quantised tensors
     const long long c0 = (long long)seq * Sp;                              // its first column in the transposed one
     const v8i qf = a8_frag(Q8 + (rb + q0 + r) * 64 + 16 * h);
@@ -107,6 +114,9 @@ __global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, 
 #pragma unroll
         for (int i = 0; i < 16; i++) oa[t][i] = 0.f;
     const int nt = (S + FT - 1) / FT;
+    // (split: later ranges are shorter, since their wavefronts first look through the earlier tiles for the running maximum)
+    const int cut[5] = {0, nt * 34 / 100, nt * 61 / 100, nt * 83 / 100, nt};
+    const int it0 = split ? cut[wave] : 0, it1 = split ? cut[wave + 1] : nt;
     // The K and V fragments of tile it + 1 are requested before tile it is worked on: with one or a few wavefronts per SIMD nothing else hides
     // the L2 latency of a tile's loads. (The last iteration re-requests its own tile.)
     v8i kfn[2], vfn[2]; int ksn[2], evn[2];
@@ -117,8 +127,36 @@ __global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, 
         vfn[0] = a8_frag(vp0 + kb); vfn[1] = a8_frag(vp1 + kb);
         evn[0] = vs0[kb / 32]; evn[1] = vs1[kb / 32];
     };
-    request(0);
-    for (int it = 0; it < nt; it++) {
+    if (split && it0 > 0) {
+        // the running maximum the single-wavefront pass holds when it reaches tile it0: the logits of the tiles before it (the two products
+        // and the scaling of the main loop, nothing else), so that every probability of this range is the value that pass computes
+        v8i kq[2]; int kqs[2];
+        auto reqk = [&](int it) {
+#pragma unroll
+            for (int b = 0; b < 2; b++) { kq[b] = a8_frag(kp + (size_t)(it * FT + 32 * b) * 64); kqs[b] = ksp[(size_t)(it * FT + 32 * b) * 2]; }
+        };
+        reqk(0);
+        float mx = -INFINITY;
+        for (int it = 0; it < it0; it++) {
+            const v8i kf[2] = {kq[0], kq[1]}; const int ks[2] = {kqs[0], kqs[1]};
+            reqk(min(it + 1, it0 - 1));
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                v16f z;
+#pragma unroll
+                for (int i = 0; i < 16; i++) z[i] = 0.f;
+                const v16f sb = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(kf[b], qf, z, 0, 0, 0, ks[b], 0, qs);
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int key = it * FT + 32 * b + (i & 3) + 4 * h + 8 * (i >> 2);
+                    mx = fmaxf(mx, key < S ? sb[i] * sl2 : -INFINITY);
+                }
+            }
+        }
+        m = fmaxf(mx, a8_xor32f(mx, h));
+    }
+    request(min(it0, nt - 1));
+    for (int it = it0; it < it1; it++) {
         const int kb = it * FT;
         const v8i kf[2] = {kfn[0], kfn[1]}; const int ks[2] = {ksn[0], ksn[1]};
         v8i vf0 = vfn[0], vf1 = vfn[1];
@@ -180,6 +218,39 @@ __global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, 
         oa[1] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vf1, pf, oa[1], 0, 0, 0, e1v, 0, ps);
     }
     l += a8_xor32f(l, h);
+    if (split) {
+        // partial (m, l, O^T) of the four key ranges -> LDS [wavefront][value][lane]; wavefront 0 adds them in wavefront order at the common
+        // maximum (a wavefront without keys holds m = -inf, l = 0, O = 0: its factor is 0)
+        extern __shared__ float cmb[];
+        float *mine = cmb + (size_t)wave * 34 * 64 + lane;
+        mine[0] = m; mine[64] = l;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int k = 0; k < 16; k++) mine[(2 + 16 * t + k) * 64] = oa[t][k];
+        __syncthreads();
+        if (wave) return;
+        float mm = m;
+#pragma unroll
+        for (int w = 1; w < 4; w++) mm = fmaxf(mm, cmb[(size_t)w * 34 * 64 + lane]);
+        float ls = 0.f;
+        v16f os[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int k = 0; k < 16; k++) os[t][k] = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float *pw = cmb + (size_t)w * 34 * 64 + lane;
+            const float f = __builtin_amdgcn_exp2f(pw[0] - mm);
+            ls = fmaf(pw[64], f, ls);
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int k = 0; k < 16; k++) os[t][k] = fmaf(pw[(2 + 16 * t + k) * 64], f, os[t][k]);
+        }
+        m = mm; l = ls; oa[0] = os[0]; oa[1] = os[1];
+    }
     const int i = q0 + r;
     if (i >= S) return;
     const float il = 1.f / l;
@@ -194,6 +265,8 @@ __global__ void __launch_bounds__(256) a8_fwd_k(const uint8_t *__restrict__ Q8, 
     if (!h) lse[((size_t)seq * H + hd) * S + i] = m + __log2f(l);
 }
 
+static int g_a8_waves = 0;
+extern "C" void at_fa8_waves(int nw) { g_a8_waves = nw == 1 || nw == 4 ? nw : 0; }
 extern "C" int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom *g, int H, int C) {
     if (!g || g->nseq <= 0 || g->S <= 0 || H <= 0) return 0;
     if (C != H * HD) mi_die("at_fa8_fwd: C %d is not %d heads of %d", C, H, HD);
@@ -209,9 +282,9 @@ extern "C" int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom 
     a8_rows_k<<<dim3(nblk_((size_t)H * R * 4, 256), 2), 256>>>(Qh, q8, qs, H, g->nseq, g->S, Sp, Tp, (size_t)(Kh - Qh), (size_t)(k8 - q8), (size_t)(ks - qs));
     a8_vt_k<<<nblk_((size_t)H * (R / 32), 4), 256>>>(Vh, vt, vts, H, g->nseq, g->S, Sp, Tp);
     // few query tiles (a 16^3 bottleneck: 129 per head): one wavefront per workgroup, so that every CU gets some
-    const int nw = (size_t)((g->S + 127) / 128) * H * g->nseq >= 512 ? 4 : 1;
+    const int nw = g_a8_waves ? g_a8_waves : (size_t)((g->S + 127) / 128) * H * g->nseq >= 512 ? 4 : 1;
     const dim3 grid((unsigned)((g->S + 32 * nw - 1) / (32 * nw)), (unsigned)H, (unsigned)g->nseq);
-    a8_fwd_k<<<grid, 64 * nw>>>(q8, qs, k8, ks, vt, vts, o, lse, g->S, Sp, H, C, R, 1.4426950408889634f / sqrtf((float)HD));
+    a8_fwd_k<<<grid, 64 * nw, nw == 4 ? 4 * 34 * 64 * sizeof(float) : 0>>>(q8, qs, k8, ks, vt, vts, o, lse, g->S, Sp, H, C, R, 1.4426950408889634f / sqrtf((float)HD));
     MICK();
     return 0;
 }
