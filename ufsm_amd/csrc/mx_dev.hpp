@@ -20,6 +20,13 @@ __device__ __forceinline__ int d_mx_exp(float amax, float inv_qmax) {
     const int ec = e < -126 ? -126 : e > 126 ? 126 : e;
     return u >= 0x7f800000u ? 128 : ec;
 }
+// d_mx_exp(amax, inv_qmax) + 127, i.e. the E8M0 byte itself, of a finite amax >= 0 (not NaN, not -0): adding 0x7fffff to the bits carries into
+// the exponent field exactly when the mantissa is not zero
+__device__ __forceinline__ int d_mx_expb_fin(float amax, float inv_qmax) {
+    const unsigned u = __float_as_uint(amax * inv_qmax);
+    const int eb = (int)((u + 0x7fffffu) >> 23);
+    return eb < 1 ? 1 : eb > 253 ? 253 : eb;
+}
 __device__ __forceinline__ float d_exp2i(int e) { return __uint_as_float((unsigned)(127 + e) << 23); }   // e = -128: the bits of -inf, as the reference (src/lp_common.cuh:501)
 __device__ __forceinline__ float d_mx_scale(unsigned sbyte) { return __uint_as_float((sbyte & 255u) << 23); }   // 0xFF -> +inf
 

@@ -866,17 +866,17 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
     const int cz[2] = {max(mz, 0), min(mz + 1, Dc - 1)}, cy[2] = {max(my, 0), min(my + 1, Hc - 1)}, cx[2] = {max(mx, 0), min(mx + 1, Wc - 1)};
     const uint8_t *xs = xc + (size_t)N * nbo * Sc * 32;
     float f[H2 ? 1 : 8][8], sc[8];
-    __half2 hf[H2 ? 8 : 1][4];                                // H2: the rows' values as binary16 pairs (an e4m3 value is one exactly), formed once per cell
+    h2_t hf[H2 ? 8 : 1][4];                                   // H2: the rows' values as binary16 pairs (an e4m3 value is one exactly), formed once per cell
     unsigned sb[8], em = 0u;
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         const size_t row = (size_t)nbk * Sc + ((size_t)(cz[k >> 2] - clo) * Hc + cy[(k >> 1) & 1]) * Wc + cx[k & 1];
         const uint2 w = *(const uint2 *)(xc + row * 32 + q * 8);
         if constexpr (H2) {
-            hf[k][0] = __builtin_bit_cast(__half2, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.x, 1.f, false));
-            hf[k][1] = __builtin_bit_cast(__half2, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.x, 1.f, true));
-            hf[k][2] = __builtin_bit_cast(__half2, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.y, 1.f, false));
-            hf[k][3] = __builtin_bit_cast(__half2, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.y, 1.f, true));
+            hf[k][0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.x, 1.f, false);
+            hf[k][1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.x, 1.f, true);
+            hf[k][2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.y, 1.f, false);
+            hf[k][3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.y, 1.f, true);
         } else { d_dec4_e4m3(w.x, f[k]); d_dec4_e4m3(w.y, f[k] + 4); }
         sb[k] = xs[row]; em = max(em, sb[k]);
         sc[k] = d_mx_scale(sb[k]);
@@ -890,12 +890,12 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
     // (the products of .75 and .25 are exact, so this is the value of the reference's ((wz wy) wx) s). 32 per cell, shared by its 8 fine voxels
     const float cw[4] = {0.421875f, 0.140625f, 0.046875f, 0.015625f};
     float w32[H2 ? 1 : 8][4];
-    __half2 w16[H2 ? 8 : 1][4];
+    _Float16 w16[H2 ? 8 : 1][4];                              // (the packed multiply-add takes one half as the multiplier of both products)
 #pragma unroll
     for (int k = 0; k < 8; k++)
 #pragma unroll
         for (int far = 0; far < 4; far++) {
-            if constexpr (H2) w16[k][far] = __half2half2(__float2half_rn(cw[far] * sc[k])); else w32[k][far] = cw[far] * sc[k];
+            if constexpr (H2) w16[k][far] = (_Float16)(cw[far] * sc[k]); else w32[k][far] = cw[far] * sc[k];      // (round to nearest even)
         }
     // output rows: fine voxel p = (pz, py, px) of the cell is voxel (2 mz + 1 + pz, 2 my + 1 + py, 2 mx + 1 + px); row0 is p = 0's row in the
     // tensor (outside it for cells on the low borders, whose p = 0 is not stored)
@@ -908,16 +908,16 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
     // normal binary32 range: 2^-24 2^(e_max - 127) >= 2^-126 and 65504 2^(e_max - 127) < 2^128. Decided per wavefront
     const bool direct = H2 && BY == 4 && __builtin_amdgcn_ballot_w64(em < 25u || em > 238u) == 0ull;
     const float am_direct = __uint_as_float((em - 9u) << 23);                    // 2^-9 of the cell's scale: block maxima below it take the widened form (binary16 subnormals)
-    int eq[4];                                                                     // the exponents of the four voxels of a z layer of the cell, for their scale bytes
+    int eq[4];                                                                     // the scale bytes of the four voxels of a z layer of the cell
 #pragma unroll
     for (int p = 0; p < 8; p++) {
         const int pz = p >> 2, py = (p >> 1) & 1, px = p & 1;                     // p = 0 has its own coarse row at m, p = 1 at m + 1
         float acc[8], am;
-        __half2 hacc[4];
+        h2_t hacc[4];
         if constexpr (H2) {
             // two channels per packed fused multiply-add: each half rounds once, as the scalar form
 #pragma unroll
-            for (int i = 0; i < 4; i++) hacc[i] = __floats2half2_rn(0.f, 0.f);
+            for (int i = 0; i < 4; i++) hacc[i] = (h2_t){(_Float16)0.f, (_Float16)0.f};
 #pragma unroll
             for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -926,13 +926,13 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
                     for (int c = 0; c < 2; c++) {
                         const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);
 #pragma unroll
-                        for (int i = 0; i < 4; i++) hacc[i] = __hfma2(w16[k][a + b + c], hf[k][i], hacc[i]);
+                        for (int i = 0; i < 4; i++) hacc[i] = __builtin_elementwise_fma((h2_t){w16[k][a + b + c], w16[k][a + b + c]}, hf[k][i], hacc[i]);
                     }
             // max |sum| 2^e_max: the widening is monotone, so the largest sum gives the largest product (NaN sums are skipped, as fmaxf skips
             // them below; a product that is NaN - 0 x inf - counts as 0 there too)
-            h2_t m = __builtin_elementwise_abs(__builtin_bit_cast(h2_t, hacc[0]));
+            h2_t m = __builtin_elementwise_abs(hacc[0]);
 #pragma unroll
-            for (int i = 1; i < 4; i++) m = __builtin_elementwise_max(m, __builtin_elementwise_abs(__builtin_bit_cast(h2_t, hacc[i])));
+            for (int i = 1; i < 4; i++) m = __builtin_elementwise_max(m, __builtin_elementwise_abs(hacc[i]));
             am = fmaxf(0.f, fmaxf((float)m.x, (float)m.y) * smax);
         } else {
 #pragma unroll
@@ -956,28 +956,30 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
             au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
             am = __uint_as_float(au);
         }
-        const int e = d_mx_exp(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
-        eq[p & 3] = e;
+        // the block's E8M0 byte; 255 for a block with an infinity (am is never NaN here)
+        const bool inf = __float_as_uint(am) >= 0x7f800000u;
+        const int eb = inf ? 255 : d_mx_expb_fin(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
+        eq[p & 3] = eb;
         const bool ok = okz[pz] && oky[py] && okx[px];
         uint8_t *dst = y + (row0 + ((long long)pz * H + py) * W + px) * RB + q * (RB / 4);
-        bool done = false;
-        if constexpr (H2 && BY == 4) {
-            if (direct && __builtin_amdgcn_ballot_w64(!(am >= am_direct) || e == 128) == 0ull) {
+        bool widen = true;                                                          // (uniform)
+        if constexpr (H2 && BY == 4) widen = !direct || __builtin_amdgcn_ballot_w64(!(am >= am_direct) || inf) != 0ull;
+        if (!widen) {
+            if constexpr (H2 && BY == 4) {
                 // (sum 2^(e_max - 127)) / 2^e = sum / 2^(e - e_max + 127): the same quotient, rounded once by the conversion either way
-                const float ds = d_exp2i(e - (int)em + 127);
+                const float ds = __uint_as_float((unsigned)(eb - (int)em + 127) << 23);
                 unsigned w = 0u;
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, __builtin_bit_cast(h2_t, hacc[0]), ds, 0);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, __builtin_bit_cast(h2_t, hacc[1]), ds, 1);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, __builtin_bit_cast(h2_t, hacc[2]), ds, 2);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, __builtin_bit_cast(h2_t, hacc[3]), ds, 3);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, hacc[0], ds, 0);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, hacc[1], ds, 1);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, hacc[2], ds, 2);
+                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, hacc[3], ds, 3);
                 if (ok) *(unsigned *)dst = w;
-                done = true;
             }
-        }
-        if (!done) {
+        } else {
+            const int e = eb - 127;
             if constexpr (H2) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) { acc[2 * i] = __low2float(hacc[i]) * smax; acc[2 * i + 1] = __high2float(hacc[i]) * smax; }
+                for (int i = 0; i < 4; i++) { acc[2 * i] = (float)hacc[i].x * smax; acc[2 * i + 1] = (float)hacc[i].y * smax; }
             }
             if (BY == 8) {
                 uint2 o; o.x = d_enc4_e4m3(acc[0], acc[1], acc[2], acc[3], e); o.y = d_enc4_e4m3(acc[4], acc[5], acc[6], acc[7], e);
@@ -988,7 +990,7 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
             // the scale bytes of the layer's four voxels in one store: thread q writes voxel (pz, q >> 1, q & 1)
             const int ev = q == 0 ? eq[0] : q == 1 ? eq[1] : q == 2 ? eq[2] : eq[3];
             const bool oks = okz[pz] && (q & 2 ? oky[1] : oky[0]) && (q & 1 ? okx[1] : okx[0]);
-            if (oks) ys[row0 + ((long long)pz * H + (q >> 1)) * W + (q & 1)] = (uint8_t)(ev + 127);
+            if (oks) ys[row0 + ((long long)pz * H + (q >> 1)) * W + (q & 1)] = (uint8_t)ev;
         }
     }
 }
