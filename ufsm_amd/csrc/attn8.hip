@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(256) a8_rows_k(const __half *__restrict__ src_
     float am = 0.f;
 #pragma unroll
     for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(v[k]));
-    am = fmaxf(am, __shfl_xor(am, 1));                             // quarters (0, 1) and (2, 3) are the two blocks
+    am = __uint_as_float(max(__float_as_uint(am), d_quad_xor_u<1>(__float_as_uint(am))));       // quarters (0, 1) and (2, 3) are the two blocks (am >= 0, never NaN: it orders as its bits; the four lanes of a row leave together)
     const int e = d_mx_exp(am, MI_INVQ8);
     *(uint4 *)(dst + (size_t)hr * 64 + 16 * qt) = make_uint4(d_enc4_e4m3(v[0], v[1], v[2], v[3], e), d_enc4_e4m3(v[4], v[5], v[6], v[7], e), d_enc4_e4m3(v[8], v[9], v[10], v[11], e), d_enc4_e4m3(v[12], v[13], v[14], v[15], e));
     if (!(qt & 1)) sc[(size_t)hr * 2 + (qt >> 1)] = (uint8_t)(e + 127);

@@ -807,7 +807,7 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
         float am = 0.f;
 #pragma unroll
         for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(r[k]));
-        am = fmaxf(am, __shfl_xor(am, 1));
+        am = __uint_as_float(max(__float_as_uint(am), d_quad_xor_u<1>(__float_as_uint(am))));       // (a non-negative number, never NaN: it orders as its bits)
         const int e = d_mx_exp(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
         if (BY == 8) {
             uint4 o;
