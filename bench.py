@@ -269,7 +269,7 @@ def hbm_leg(np, lib, LP, DevBuf):
     return rows
 
 
-def sliding_leg(np, lib, LP, DevBuf, nbatch=8):
+def sliding_leg(np, lib, LP, DevBuf, nbatch=64):
     """configs[4]: a 512 x 1024 x 1024 uint8 volume resident in HBM, 128^3 windows with 16 voxels of halo (stride 96), per window a U-Net of
     widths 32/64/128/192 with MX-fp4 weights over MX-fp8 activations (prec 3) and two transformer blocks (MX-fp8 attention core, MX-fp8
     linears, 4 heads of 48, axial RoPE, 4 register tokens) on the 16^3 = 4096 bottleneck tokens, one head channel, sigmoid -> uint8
@@ -291,13 +291,20 @@ def sliding_leg(np, lib, LP, DevBuf, nbatch=8):
     t0 = time.perf_counter()
     rc, nw, ndone = net.predict_volume(dv.ptr, dims, halo, B, 115.0, 1 / 40.0, 1, 400.0, -300.0, dout.ptr)
     lib.mi_sync(); LP.check()
+    dt_first = time.perf_counter() - t0
+    assert rc == 0
+    # the driver evens the windows out over its forwards, so the first prediction of a volume builds the graph for that sample count (activation
+    # buffers, scratch): the second prediction of the same volume is the steady state the other legs' warm-up steps give them
+    t0 = time.perf_counter()
+    rc, nw, ndone = net.predict_volume(dv.ptr, dims, halo, B, 115.0, 1 / 40.0, 1, 400.0, -300.0, dout.ptr)
+    lib.mi_sync(); LP.check()
     dt = time.perf_counter() - t0
     assert rc == 0
     head = dout.to_numpy(np.uint8)[:1 << 20]
     net.close()
     nvox = float(dims[0]) * dims[1] * dims[2]
-    return {"workload": "configs[4]: 512x1024x1024 uint8 in HBM, 128^3 windows, halo 16, feather 16, U-Net 32/64/128/192, MX-fp4 weights over MX-fp8 activations, 2 attention blocks on 16^3 tokens (MX-fp8 core), %d windows per forward" % nbatch,
-            "value": nvox / dt, "unit": "voxels/s", "seconds": dt, "windows": int(nw), "windows_computed": int(ndone), "output_mean_first_mib": float(head.mean())}
+    return {"workload": "configs[4]: 512x1024x1024 uint8 in HBM, 128^3 windows, halo 16, feather 16, U-Net 32/64/128/192, MX-fp4 weights over MX-fp8 activations, 2 attention blocks on 16^3 tokens (MX-fp8 core), up to %d windows per forward" % nbatch,
+            "value": nvox / dt, "unit": "voxels/s", "seconds": dt, "seconds_first_call": dt_first, "windows": int(nw), "windows_computed": int(ndone), "output_mean_first_mib": float(head.mean())}
 
 
 def main():
@@ -312,7 +319,7 @@ def main():
     ap.add_argument("--no-hbm", action="store_true", help="skip the HBM-bound kernels leg")
     ap.add_argument("--no-single", action="store_true", help="skip the single-conv legs (configs[0], the MX-fp4 3x3x3 conv of configs[2])")
     ap.add_argument("--unet-only", action="store_true", help="the U-Net leg alone (what the rocprofv3 runs of the forward's kernels use)")
-    ap.add_argument("--windows-per-forward", type=int, default=8, help="sliding-window leg: windows batched into one forward")
+    ap.add_argument("--windows-per-forward", type=int, default=64, help="sliding-window leg: the most windows batched into one forward (the driver evens them out over its forwards)")
     ap.add_argument("--copy-probe", action="store_true", help="run 5 device-to-device copies of 1 GiB and exit: the known-size kernel that scales "
                     "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--conv-probe", default="", metavar="Ci,Co,N,D,bits", help="time one 3x3x3 conv shape (MX in / out of the compute format, fused statistics) "

@@ -166,7 +166,8 @@ int mi_unet_layer_stats(const unet *u, int k, const float **mean, const float **
 int mi_unet_infer_slab(void);                                  /* unet_set_infer_slab's current value */
 size_t mi_unet_peek_nparams(const char *path);                 /* the header's "nparams" (0: unreadable) */
 /* ---- sliding-window prediction of a volume resident in device memory (src/predict.c: the --feather single pass, :282-333, :2538-2545,
-   :3420-3436). vol: uint8 CT [dims0][dims1][dims2]; cubic windows of `window` voxels, `nbatch` (1 .. 16) per forward, with
+   :3420-3436). vol: uint8 CT [dims0][dims1][dims2]; cubic windows of `window` voxels, up to `nbatch` (1 .. 64) per forward (the windows that hold material are
+   spread evenly over the forwards that many need: 726 windows at up to 64 are 12 forwards of 61; the graph is rebuilt for that sample count if it was built for another), with
    `halo` voxels of context per side tile the volume at stride window - 2 halo in z-y-x order; each runs as a sample of unet_forward_ct (z-score mean / isd; axis, cy, cx: the scroll axis
    sign and its centre in volume y / x, axis 0: no direction channels) and places uint8(255 sigmoid(logit 0) + .5) where CT >= the
    prediction iso over its interior plus `feather` voxels of its upper halo; the window borders are then blended over `feather` voxels

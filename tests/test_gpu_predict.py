@@ -180,8 +180,8 @@ def test_predict_volume_equals_windows_run_one_by_one(gpu):
 @pytest.mark.gpu
 @pytest.mark.parametrize("attn", [0, 1])
 def test_predict_volume_batched_windows_equal_single(gpu, attn):
-    """A graph created for two (three) samples runs that many windows per forward: samples are independent, so the prediction is the
-    one-window graph's byte for byte, with an odd number of windows (11: the last batch is incomplete) and with an attention stage."""
+    """A graph created for two (three, eight) samples runs up to that many windows per forward: samples are independent, so the prediction is
+    the one-window graph's byte for byte, with an odd number of windows (11: the last batch is incomplete) and with an attention stage."""
     from ufsm_amd.unet import UNet, make_cfg
     rng = np.random.default_rng(9)
     W, halo, B = 32, 8, 8; S = W - 2 * halo
@@ -193,7 +193,7 @@ def test_predict_volume_batched_windows_equal_single(gpu, attn):
     kw = dict(attn_blocks=1, attn_pe=1, attn_reg=2) if attn else {}
     widths = [16, 192] if attn else [16, 32]
     outs = []
-    for nb in (1, 2, 3):
+    for nb in (1, 2, 3, 8):                                                 # 8: the driver evens 11 windows out over two forwards of 6 (and rebuilds the graph for 6)
         net = UNet(make_cfg(4, widths, G=8, head_out=1, act_dt=8, **kw), nb, W, W, W, seed=5)
         p = net.params(); p[-1] = 0.0; net.set_params(p)
         dout = DevBuf(vol.size)
@@ -202,7 +202,7 @@ def test_predict_volume_batched_windows_equal_single(gpu, attn):
         outs.append(dout.to_numpy(np.uint8, dims))
         net.close()
     assert outs[0].max() > 0 and outs[0].std() > 0
-    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2]) and np.array_equal(outs[0], outs[3])
 
 
 @pytest.mark.gpu

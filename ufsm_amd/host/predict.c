@@ -7,10 +7,10 @@
 
 int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, const int64_t dims[3], int halo, int feather, float mean, float isd,
                            int axis, float cy, float cx, uint8_t *out, int64_t nwin[2]) {
-    const shape5 in = {nbatch, 4, window, window, window};
+    shape5 in = {nbatch, 4, window, window, window};
     const int W = in.w, S = W - 2 * halo, B = feather, En = S + B;
-    if (in.n < 1 || in.n > 16 || in.d != W || in.h != W || halo < 0 || S <= 0 || B < 0 || B > halo || B > S || B > 1024) {
-        fprintf(stderr, "mi_unet_predict_volume: needs cubic windows (1 .. 16 per forward), 0 <= feather <= halo, window - 2 halo > 0 and feather <= it (window %d x %d x %d, halo %d, feather %d)\n",
+    if (in.n < 1 || in.n > 64 || in.d != W || in.h != W || halo < 0 || S <= 0 || B < 0 || B > halo || B > S || B > 1024) {
+        fprintf(stderr, "mi_unet_predict_volume: needs cubic windows (1 .. 64 per forward), 0 <= feather <= halo, window - 2 halo > 0 and feather <= it (window %d x %d x %d, halo %d, feather %d)\n",
                 in.d, in.h, in.w, halo, feather);
         return -1;
     }
@@ -46,8 +46,11 @@ int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, 
     int64_t *list = malloc((size_t)(total ? total : 1) * sizeof(int64_t)), np = 0;
     if (!list) rc = -1;
     for (int64_t id = 0; id < total && !rc; id++) if (hany[id]) list[np++] = id;
+    /* the windows are spread evenly over the forwards that nbatch windows per forward need: 726 windows at up to 64 per forward are 12 forwards
+     * of 61 (6 samples repeat a window), not 11 of 64 and one of 22 padded to 64. The graph is (re)built for that sample count by the first forward */
+    if (np > 0) { const int64_t nf = (np + in.n - 1) / in.n; in.n = (int)((np + nf - 1) / nf); }
     for (int64_t k = 0; k < np && !rc; k += in.n) {
-        const uint8_t *cts[16]; const float *dyos[16], *dxos[16]; int64_t org[16 * 3], eoff[16];
+        const uint8_t *cts[64]; const float *dyos[64], *dxos[64]; int64_t org[64 * 3], eoff[64];
         const int nreal = (int)(np - k < in.n ? np - k : in.n);
         for (int j = 0; j < in.n; j++) {
             const int64_t id = list[k + j < np ? k + j : np - 1], a = id / (nss[1] * nss[2]), b = (id / nss[2]) % nss[1], c = id % nss[2];
