@@ -62,12 +62,12 @@ extern "C" void at_ln_fwd(const float *x, const float *g, const float *b, float 
     MICK();
 }
 // ---- SwiGLU (src/nn_attn.cu:438-455): gg[t][f] = silu(h[t][f]) h[t][F + f]; four features per thread, 16-byte accesses ----
-__global__ void __launch_bounds__(256) glu_rows_k(const float4 *__restrict__ h, float4 *__restrict__ gg, int F4) {
-    const int f = blockIdx.x * 256 + threadIdx.x;                  // grid: x over the row's float4 chunks, y over the tokens
-    if (f >= F4) return;
-    const size_t t = blockIdx.y + (size_t)blockIdx.z * 65535u;
+__global__ void __launch_bounds__(256) glu_rows_k(const float4 *__restrict__ h, float4 *__restrict__ gg, size_t n4, unsigned F4) {
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;      // one float4 chunk of one token's output row: any token count, full workgroups
+    if (i >= n4) return;
+    const size_t t = i / F4; const unsigned f = (unsigned)(i - t * F4);
     const float4 a = h[t * 2 * F4 + f], b = h[t * 2 * F4 + F4 + f];
-    gg[t * F4 + f] = make_float4(a.x / (1.f + expf(-a.x)) * b.x, a.y / (1.f + expf(-a.y)) * b.y, a.z / (1.f + expf(-a.z)) * b.z, a.w / (1.f + expf(-a.w)) * b.w);
+    gg[i] = make_float4(a.x / (1.f + expf(-a.x)) * b.x, a.y / (1.f + expf(-a.y)) * b.y, a.z / (1.f + expf(-a.z)) * b.z, a.w / (1.f + expf(-a.w)) * b.w);
 }
 __global__ void __launch_bounds__(256) glu_any_k(const float *__restrict__ h, float *__restrict__ gg, size_t n, int F) {       // widths that are not a multiple of 4
     const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
@@ -79,9 +79,8 @@ __global__ void __launch_bounds__(256) glu_any_k(const float *__restrict__ h, fl
 extern "C" void at_glu_fwd(const float *h, float *gg, long T, int F) {
     if (T <= 0 || F <= 0) return;
     if ((F & 3) == 0 && !(((uintptr_t)h | (uintptr_t)gg) & 15)) {
-        const unsigned ty = (unsigned)(T < 65535 ? T : 65535), tz = (unsigned)((T + 65534) / 65535);
-        if ((long)ty * tz != T) { glu_any_k<<<nblk_((size_t)T * F, 256), 256>>>(h, gg, (size_t)T * F, F); MICK(); return; }      // (a token count the 2-D grid does not tile)
-        glu_rows_k<<<dim3(nblk_((size_t)F / 4, 256), ty, tz), 256>>>((const float4 *)h, (float4 *)gg, F / 4);
+        const size_t n4 = (size_t)T * (F / 4);
+        glu_rows_k<<<nblk_(n4, 256), 256>>>((const float4 *)h, (float4 *)gg, n4, (unsigned)(F / 4));
     } else glu_any_k<<<nblk_((size_t)T * F, 256), 256>>>(h, gg, (size_t)T * F, F);
     MICK();
 }
