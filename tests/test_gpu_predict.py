@@ -208,7 +208,7 @@ def test_predict_volume_batched_windows_equal_single(gpu, attn):
 @pytest.mark.gpu
 def test_config4_full_volume_prediction_properties(gpu):
     """The whole 512 x 1024 x 1024 volume of the sliding-window configuration (128^3 windows, halo 16, feather 16: 6 x 11 x 11 = 726 windows,
-    eight per forward; widths 32/64/128/192, MX-fp4 weights over MX-fp8 activations, two attention blocks) through the driver, checked by what
+    up to 64 per forward, i.e. 12 forwards of 61; widths 32/64/128/192, MX-fp4 weights over MX-fp8 activations, two attention blocks) through the driver, checked by what
     does not depend on the size (tests/test_predict_feather.c:108-121): core voxels and the first window equal the unfeathered prediction byte
     for byte, blended shells differ; windows at the far corner and in the middle, gathered, run alone on a one-window graph and placed through
     the C ABI, equal the unfeathered prediction of their region (offsets past 2^29 voxels, the incomplete last batch); a second run is identical."""
@@ -223,7 +223,7 @@ def test_config4_full_volume_prediction_properties(gpu):
     vol = np.clip(vol, 1, 255).astype(np.uint8)
     del r
     cfgk = dict(G=8, head_out=1, act_dt=8, prec=3, attn_blocks=2, attn_pe=1, attn_reg=4)
-    net = UNet(make_cfg(4, [32, 64, 128, 192], **cfgk), 8, W, W, W, seed=1)
+    net = UNet(make_cfg(4, [32, 64, 128, 192], **cfgk), 64, W, W, W, seed=1)
     p = net.params()
     dv = DevBuf.from_numpy(vol); dout = DevBuf(vol.size); dplain = DevBuf(vol.size)
     args = (115.0, 1 / 40.0, 1, 400.0, -300.0)
