@@ -762,12 +762,6 @@ template <int BX, int BY>
 __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, size_t Ss, size_t v0) {
     const int nb = C / 32, blk = blockIdx.y, n = blockIdx.z;
     __shared__ float sa[32], sb[32];
-    if (threadIdx.x < 32) {
-        float a = 1.f, b = 0.f;
-        if (gp.G) { const int c = cg0 + blk * 32 + threadIdx.x, ng = d_gn_row(gp, n) * gp.G + c / (Cg / gp.G); a = gp.rstd[ng] * gp.gamma[c]; b = fmaf(-gp.mean[ng], a, gp.beta[c]); }
-        sa[threadIdx.x] = a; sb[threadIdx.x] = b;
-    }
-    __syncthreads();
     // A workgroup moves RS32_R x 128 consecutive voxels of the block, a thread one 16-channel half of RS32_R rows 128 voxels apart: the rows are
     // requested together (one memory round trip per thread instead of one per row) and the coefficients' set-up is paid once per RS32_R rows
     constexpr int IB = BX * 2, OB = BY * 2;                        // bytes of a 16-channel half row
@@ -785,6 +779,13 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
         else { const uint2 q = *(const uint2 *)(x + row * 16 + hf * 8); w[i][0] = q.x; w[i][1] = q.y; }
         sby[i] = xs[row];
     }
+    // (the rows are requested before the block's coefficients are formed: the two chains of dependent loads overlap)
+    if (threadIdx.x < 32) {
+        float a = 1.f, b = 0.f;
+        if (gp.G) { const int c = cg0 + blk * 32 + threadIdx.x, ng = d_gn_row(gp, n) * gp.G + c / (Cg / gp.G); a = gp.rstd[ng] * gp.gamma[c]; b = fmaf(-gp.mean[ng], a, gp.beta[c]); }
+        sa[threadIdx.x] = a; sb[threadIdx.x] = b;
+    }
+    __syncthreads();
     float ca[16], cb[16];
 #pragma unroll
     for (int k = 0; k < 16; k++) { ca[k] = sa[hf * 16 + k]; cb[k] = sb[hf * 16 + k]; }
