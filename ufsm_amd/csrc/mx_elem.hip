@@ -850,35 +850,43 @@ void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg
 // H2: the fp4 entry's blend (stage_up_smem_h2, src/lp_common.cuh:674-712): binary16 weights relative to the largest of the cell's 8 scale bytes,
 // binary16 fused multiply-adds in the same z, y, x order (an e4m3 code is a binary16 value), the sum widened and scaled by 2^e_max.
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-template <int BY, bool H2>
+// CH: channels of the block per thread, 8 (four threads per cell) for the fp32 blend and 16 (two threads per cell) for the binary16 blend: what
+// a fine voxel costs beside its multiply-adds (block maximum, exponent, scale, stores) is then paid by two lanes instead of four (0.52 -> 0.40 ms
+// at 8 x 64 channels 64^3 -> 128^3). The fp32 blend with 16 holds 128 row values and 190 registers, two wavefronts per SIMD: measured no faster
+template <int BY, bool H2, int CH = H2 ? 16 : 8>
 __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y, int N, int nbo, int D, int H, int W, int zlo, int zhi, int clo, int Dcs, int mz0, int ncz_) {
     // fine planes [zlo, zhi) of the depth-D result, written at their place in the depth-D tensor y; xc holds the coarse planes [clo, clo + Dcs)
     // compactly; cells mz0 .. mz0 + ncz_ - 1 along z (the whole tensor: zlo 0, zhi D, clo 0, Dcs D / 2, mz0 -1, ncz_ D / 2 + 1)
+    static_assert(CH == 8 || CH == 16, "8 or 16 channels per thread");
+    constexpr int QP = 32 / CH, NP = CH / 2;                                      // threads per cell; binary16 pairs per thread
     const int Dc = D >> 1, Hc = H >> 1, Wc = W >> 1;
     const size_t S = (size_t)D * H * W, Sc = (size_t)Dcs * Hc * Wc;
     const int nbk = blockIdx.y;                                                   // (n, blk)
-    // grid: x over the (my, mx) cells of one z layer of cells (four threads each), y = (n, blk), z = the layer: one 32-bit division per thread
+    // grid: x over the (my, mx) cells of one z layer of cells (QP threads each), y = (n, blk), z = the layer: one 32-bit division per thread
     const unsigned t = blockIdx.x * 256u + threadIdx.x;
-    const int q = (int)(t & 3u);
-    const unsigned cell = t >> 2, ncx = (unsigned)Wc + 1u, ncy = (unsigned)Hc + 1u;
+    const int q = (int)(t & (unsigned)(QP - 1));
+    const unsigned cell = t / (unsigned)QP, ncx = (unsigned)Wc + 1u, ncy = (unsigned)Hc + 1u;
     const bool live = cell < ncx * ncy;
     const unsigned cc = live ? cell : 0u, cyi = cc / ncx;
     const int mx = (int)(cc - cyi * ncx) - 1, my = (int)cyi - 1, mz = (int)blockIdx.z + mz0;
     const int cz[2] = {max(mz, 0), min(mz + 1, Dc - 1)}, cy[2] = {max(my, 0), min(my + 1, Hc - 1)}, cx[2] = {max(mx, 0), min(mx + 1, Wc - 1)};
     const uint8_t *xs = xc + (size_t)N * nbo * Sc * 32;
-    float f[H2 ? 1 : 8][8], sc[8];
-    h2_t hf[H2 ? 8 : 1][4];                                   // H2: the rows' values as binary16 pairs (an e4m3 value is one exactly), formed once per cell
+    float f[H2 ? 1 : 8][H2 ? 1 : CH], sc[8];
+    h2_t hf[H2 ? 8 : 1][H2 ? NP : 1];                         // H2: the rows' values as binary16 pairs (an e4m3 value is one exactly), formed once per cell
     unsigned sb[8], em = 0u;
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         const size_t row = (size_t)nbk * Sc + ((size_t)(cz[k >> 2] - clo) * Hc + cy[(k >> 1) & 1]) * Wc + cx[k & 1];
-        const uint2 w = *(const uint2 *)(xc + row * 32 + q * 8);
-        if constexpr (H2) {
-            hf[k][0] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.x, 1.f, false);
-            hf[k][1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.x, 1.f, true);
-            hf[k][2] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.y, 1.f, false);
-            hf[k][3] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w.y, 1.f, true);
-        } else { d_dec4_e4m3(w.x, f[k]); d_dec4_e4m3(w.y, f[k] + 4); }
+        unsigned w[CH / 4];
+        if constexpr (CH == 8) { const uint2 v = *(const uint2 *)(xc + row * 32 + q * 8); w[0] = v.x; w[1] = v.y; }
+        else { const uint4 v = *(const uint4 *)(xc + row * 32 + q * 16); w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w; }
+#pragma unroll
+        for (int j = 0; j < CH / 4; j++) {
+            if constexpr (H2) {
+                hf[k][2 * j] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[j], 1.f, false);
+                hf[k][2 * j + 1] = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w[j], 1.f, true);
+            } else d_dec4_e4m3(w[j], f[k] + 4 * j);
+        }
         sb[k] = xs[row]; em = max(em, sb[k]);
         sc[k] = d_mx_scale(sb[k]);
     }
@@ -913,12 +921,12 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
 #pragma unroll
     for (int p = 0; p < 8; p++) {
         const int pz = p >> 2, py = (p >> 1) & 1, px = p & 1;                     // p = 0 has its own coarse row at m, p = 1 at m + 1
-        float acc[8], am;
-        h2_t hacc[4];
+        float acc[CH], am;
+        h2_t hacc[H2 ? NP : 1];
         if constexpr (H2) {
             // two channels per packed fused multiply-add: each half rounds once, as the scalar form
 #pragma unroll
-            for (int i = 0; i < 4; i++) hacc[i] = (h2_t){(_Float16)0.f, (_Float16)0.f};
+            for (int i = 0; i < NP; i++) hacc[i] = (h2_t){(_Float16)0.f, (_Float16)0.f};
 #pragma unroll
             for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -927,17 +935,17 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
                     for (int c = 0; c < 2; c++) {
                         const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);
 #pragma unroll
-                        for (int i = 0; i < 4; i++) hacc[i] = __builtin_elementwise_fma((h2_t){w16[k][a + b + c], w16[k][a + b + c]}, hf[k][i], hacc[i]);
+                        for (int i = 0; i < NP; i++) hacc[i] = __builtin_elementwise_fma((h2_t){w16[k][a + b + c], w16[k][a + b + c]}, hf[k][i], hacc[i]);
                     }
             // max |sum| 2^e_max: the widening is monotone, so the largest sum gives the largest product (NaN sums are skipped, as fmaxf skips
             // them below; a product that is NaN - 0 x inf - counts as 0 there too)
             h2_t m = __builtin_elementwise_abs(hacc[0]);
 #pragma unroll
-            for (int i = 1; i < 4; i++) m = __builtin_elementwise_max(m, __builtin_elementwise_abs(hacc[i]));
+            for (int i = 1; i < NP; i++) m = __builtin_elementwise_max(m, __builtin_elementwise_abs(hacc[i]));
             am = fmaxf(0.f, fmaxf((float)m.x, (float)m.y) * smax);
         } else {
 #pragma unroll
-            for (int i = 0; i < 8; i++) acc[i] = 0.f;
+            for (int i = 0; i < CH; i++) acc[i] = 0.f;
 #pragma unroll
             for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -946,15 +954,16 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
                     for (int c = 0; c < 2; c++) {
                         const int k = ((a ^ pz) << 2) | ((b ^ py) << 1) | (c ^ px);   // a = 0: the voxel's own coarse row, a = 1: its neighbour
 #pragma unroll
-                        for (int i = 0; i < 8; i++) acc[i] = fmaf(w32[k][a + b + c], f[k][i], acc[i]);
+                        for (int i = 0; i < CH; i++) acc[i] = fmaf(w32[k][a + b + c], f[k][i], acc[i]);
                     }
             am = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) am = fmaxf(am, fabsf(acc[i]));
+            for (int i = 0; i < CH; i++) am = fmaxf(am, fabsf(acc[i]));
         }
-        {   // the four threads of the cell hold the row's 32 channels; am is a non-negative number (no NaN, no -0): it orders as its bit pattern
+        {   // the QP threads of the cell hold the row's 32 channels; am is a non-negative number (no NaN, no -0): it orders as its bit pattern
             unsigned au = __float_as_uint(am);
-            au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
+            au = max(au, d_quad_xor_u<1>(au));
+            if constexpr (QP == 4) au = max(au, d_quad_xor_u<2>(au));
             am = __uint_as_float(au);
         }
         // the block's E8M0 byte; 255 for a block with an infinity (am is never NaN here)
@@ -962,36 +971,55 @@ __global__ void __launch_bounds__(256) up_blend_k(const uint8_t *xc, uint8_t *y,
         const int eb = inf ? 255 : d_mx_expb_fin(am, BY == 8 ? MI_INVQ8 : MI_INVQ4);
         eq[p & 3] = eb;
         const bool ok = okz[pz] && oky[py] && okx[px];
-        uint8_t *dst = y + (row0 + ((long long)pz * H + py) * W + px) * RB + q * (RB / 4);
+        uint8_t *dst = y + (row0 + ((long long)pz * H + py) * W + px) * RB + q * (RB / QP);
         bool widen = true;                                                          // (uniform)
         if constexpr (H2 && BY == 4) widen = !direct || __builtin_amdgcn_ballot_w64(!(am >= am_direct) || inf) != 0ull;
         if (!widen) {
             if constexpr (H2 && BY == 4) {
                 // (sum 2^(e_max - 127)) / 2^e = sum / 2^(e - e_max + 127): the same quotient, rounded once by the conversion either way
                 const float ds = __uint_as_float((unsigned)(eb - (int)em + 127) << 23);
-                unsigned w = 0u;
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, hacc[0], ds, 0);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, hacc[1], ds, 1);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, hacc[2], ds, 2);
-                w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w, hacc[3], ds, 3);
-                if (ok) *(unsigned *)dst = w;
+                unsigned w[NP / 4];
+#pragma unroll
+                for (int j = 0; j < NP / 4; j++) {
+                    w[j] = 0u;
+                    w[j] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w[j], hacc[4 * j], ds, 0);
+                    w[j] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w[j], hacc[4 * j + 1], ds, 1);
+                    w[j] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w[j], hacc[4 * j + 2], ds, 2);
+                    w[j] = __builtin_amdgcn_cvt_scalef32_pk_fp4_f16(w[j], hacc[4 * j + 3], ds, 3);
+                }
+                if (ok) { if constexpr (CH == 8) *(unsigned *)dst = w[0]; else *(uint2 *)dst = make_uint2(w[0], w[NP / 4 - 1]); }
             }
         } else {
             const int e = eb - 127;
             if constexpr (H2) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) { acc[2 * i] = (float)hacc[i].x * smax; acc[2 * i + 1] = (float)hacc[i].y * smax; }
+                for (int i = 0; i < NP; i++) { acc[2 * i] = (float)hacc[i].x * smax; acc[2 * i + 1] = (float)hacc[i].y * smax; }
             }
             if (BY == 8) {
-                uint2 o; o.x = d_enc4_e4m3(acc[0], acc[1], acc[2], acc[3], e); o.y = d_enc4_e4m3(acc[4], acc[5], acc[6], acc[7], e);
-                if (ok) *(uint2 *)dst = o;
-            } else { const unsigned o = d_enc8_e2m1(acc, e); if (ok) *(unsigned *)dst = o; }
+                unsigned o[CH / 4];
+#pragma unroll
+                for (int j = 0; j < CH / 4; j++) o[j] = d_enc4_e4m3(acc[4 * j], acc[4 * j + 1], acc[4 * j + 2], acc[4 * j + 3], e);
+                if (ok) { if constexpr (CH == 8) *(uint2 *)dst = make_uint2(o[0], o[1]); else *(uint4 *)dst = make_uint4(o[0], o[1], o[CH / 4 - 2], o[CH / 4 - 1]); }
+            } else {
+                unsigned o[CH / 8];
+#pragma unroll
+                for (int j = 0; j < CH / 8; j++) o[j] = d_enc8_e2m1(acc + 8 * j, e);
+                if (ok) { if constexpr (CH == 8) *(unsigned *)dst = o[0]; else *(uint2 *)dst = make_uint2(o[0], o[CH / 8 - 1]); }
+            }
         }
         if ((p & 3) == 3) {
-            // the scale bytes of the layer's four voxels in one store: thread q writes voxel (pz, q >> 1, q & 1)
-            const int ev = q == 0 ? eq[0] : q == 1 ? eq[1] : q == 2 ? eq[2] : eq[3];
-            const bool oks = okz[pz] && (q & 2 ? oky[1] : oky[0]) && (q & 1 ? okx[1] : okx[0]);
-            if (oks) ys[row0 + ((long long)pz * H + (q >> 1)) * W + (q & 1)] = (uint8_t)ev;
+            // the scale bytes of the layer's four voxels: four threads per cell: thread q writes voxel (pz, q >> 1, q & 1); two: thread q the two of row q
+            if constexpr (QP == 4) {
+                const int ev = q == 0 ? eq[0] : q == 1 ? eq[1] : q == 2 ? eq[2] : eq[3];
+                const bool oks = okz[pz] && (q & 2 ? oky[1] : oky[0]) && (q & 1 ? okx[1] : okx[0]);
+                if (oks) ys[row0 + ((long long)pz * H + (q >> 1)) * W + (q & 1)] = (uint8_t)ev;
+            } else {
+                const int e0 = q ? eq[2] : eq[0], e1 = q ? eq[3] : eq[1];
+                const bool oky_q = okz[pz] && (q ? oky[1] : oky[0]);
+                uint8_t *yq = ys + row0 + ((long long)pz * H + q) * W;
+                if (oky_q && okx[0]) yq[0] = (uint8_t)e0;
+                if (oky_q && okx[1]) yq[1] = (uint8_t)e1;
+            }
         }
     }
 }
@@ -1009,7 +1037,7 @@ void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W
     mi_restage_sub(x, xdt, N, C, (size_t)Dcs * Scp, gp, Cg, 0, xc, 8, (size_t)Dc * Scp, (size_t)clo * Scp);
     const size_t cells = (size_t)(H / 2 + 1) * (W / 2 + 1);                                   // per z layer of cells
     if ((size_t)N * nbo > 65535 || ncz > 65535) mi_die("fused upsample: launch grid (%d x %d blocks, %d cell layers)", N, nbo, ncz);
-    const dim3 grid(nblk_(cells * 4, 256), (unsigned)(N * nbo), (unsigned)ncz);
+    const dim3 grid(nblk_(cells * (h2 ? 2 : 4), 256), (unsigned)(N * nbo), (unsigned)ncz);      // (threads per cell: two in the binary16 blend, four in the fp32 one)
 #define UB(BY, H2) up_blend_k<BY, H2><<<grid, 256>>>(xc, (uint8_t *)y, N, nbo, D, H, W, zlo, zhi, 0, Dc, mz0, ncz)
     if (ybits == 4) { if (h2) UB(4, true); else UB(4, false); } else { if (h2) UB(8, true); else UB(8, false); }
 #undef UB
