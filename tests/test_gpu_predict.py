@@ -205,6 +205,24 @@ def test_predict_volume_batched_windows_equal_single(gpu, attn):
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2]) and np.array_equal(outs[0], outs[3])
 
 
+def test_predict_volume_of_air_computes_nothing(gpu):
+    """No window holds a voxel >= iso: no forward runs (the graph is not rebuilt for zero samples), the output is zero, the counts say so;
+    and a volume smaller than one window's interior in every axis is one window."""
+    from ufsm_amd.unet import UNet, make_cfg
+    W, halo, B = 32, 8, 8
+    net = UNet(make_cfg(4, [16, 32], G=8, head_out=1, act_dt=8), 4, W, W, W, seed=5)
+    dims = (40, 32, 24)
+    dv = DevBuf.from_numpy(np.zeros(dims, np.uint8)); dout = DevBuf.from_numpy(np.full(dims, 7, np.uint8))
+    rc, nw, ndone = net.predict_volume(dv.ptr, dims, halo, B, 100.0, 1 / 50.0, 1, 40.0, -20.0, dout.ptr)
+    assert rc == 0 and nw == 12 and ndone == 0 and not dout.to_numpy(np.uint8, dims).any()
+    small = (10, 12, 9)
+    vol = np.random.default_rng(3).integers(60, 200, small).astype(np.uint8)
+    dv = DevBuf.from_numpy(vol); dout = DevBuf(vol.size)
+    rc, nw, ndone = net.predict_volume(dv.ptr, small, halo, B, 100.0, 1 / 50.0, 1, 40.0, -20.0, dout.ptr)
+    assert rc == 0 and nw == 1 and ndone == 1
+    net.close()
+
+
 @pytest.mark.gpu
 def test_config4_full_volume_prediction_properties(gpu):
     """The whole 512 x 1024 x 1024 volume of the sliding-window configuration (128^3 windows, halo 16, feather 16: 6 x 11 x 11 = 726 windows,
