@@ -44,6 +44,10 @@ int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom *g, int H, 
    size. With 4, a sequence's last 32-query tile, when it is the only one of its workgroup, is worked on by all four wavefronts (a range of the
    keys each, merged in wavefront order): the same probabilities and codes as with 1, their sums added in another order (~1e-7 relative) */
 void at_fa8_waves(int nw);
+/* (no counterpart: a knob for tests) 0: at_block_fwd writes the fp32 rows of its LayerNorms and its SwiGLU (at_ws.xn, .xn2, .gg) and the GEMMs
+   pack them; 1 (default): with e4m3 linears and C, F multiples of 64 those kernels write the GEMMs' packed operands themselves and the three
+   fp32 buffers are left untouched (a forward never reads them again). The block's output has the same bits either way */
+void at_fuse_pack(int on);
 
 /* ---- the attention block around those two (forward, self-attention path; src/attn.h:26-81, src/nn_attn.cu) ---- */
 #define AT_DFM_NLV (AT_DFM_MAXL + 1)

@@ -91,6 +91,23 @@ def test_block_forward(gpu, bits, rope, nreg, tol):
         assert np.linalg.norm(y - ye) / np.linalg.norm(ye) < tol
 
 
+def test_block_with_packed_operands_from_the_producers_has_the_same_bits(gpu):
+    """The LayerNorms and the SwiGLU write the GEMMs' packed MX-fp8 operands themselves (default) or fp32 rows that the GEMMs pack: the same
+    values quantised the same way, so the block's output is equal bit for bit (C 192 = three 64-channel groups per row, a token count that is not
+    a multiple of the four rows of a workgroup)."""
+    rng = np.random.default_rng(11)
+    Cc, H, F, nseq, D, nreg = 192, 4, 512, 3, 5, 2; S = nreg + D ** 3
+    P, lay = make_block(rng, Cc, F)
+    x = (rng.standard_normal((nseq * S, Cc)) * np.exp(rng.uniform(-2, 2, (nseq * S, 1)))).astype(np.float32)
+    lib.at_fuse_pack(0)
+    try:
+        rc0, y0 = run_block(8, Cc, H, F, 1, nreg, P, lay, x, nseq, S, D)
+    finally:
+        lib.at_fuse_pack(1)
+    rc1, y1 = run_block(8, Cc, H, F, 1, nreg, P, lay, x, nseq, S, D)
+    assert rc0 == 0 and rc1 == 0 and np.isfinite(y1).all() and np.array_equal(y0, y1)
+
+
 @pytest.mark.parametrize("nseq,dims,nreg,Cc", [(2, (3, 4, 5), 2, 96), (1, (8, 8, 8), 0, 192), (3, (1, 1, 7), 4, 48), (1, (2, 2, 2), 1, 4)])
 def test_peg_matches_oracle_bit_for_bit(gpu, nseq, dims, nreg, Cc):
     """at_peg_fwd (src/attn.h:141-144): x + b + depthwise 3^3 conv on the grid tokens, the taps in (dz, dy, dx) order as fused multiply-adds:

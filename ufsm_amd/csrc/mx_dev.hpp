@@ -266,6 +266,9 @@ __device__ __forceinline__ void gn_acc_add(double *b, size_t i, double v) {
 // ---- host-side shared declarations of the library's units ----
 void mi_restage(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits);
 void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int h2);    // h2: the binary16 blend
+// the MX GEMM with A's rows quantised by the kernel that produces them (csrc/mx_gemm.hip): where to write them, then the product
+bool mi_mx_gemm_abuf(int bits, int M, int N, int K, uint8_t **Aq, uint8_t **As);
+int mi_mx_gemm_apacked(int bits, int tb, int M, int N, int K, const float *B, float *C, float beta, const float *bias, const float *res);
 void mi_restage_sub(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits, size_t Ss, size_t v0);     // only voxels [v0, v0 + S) of tensors of Ss voxels
 void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int zlo, int zhi, int h2);   // only fine planes [zlo, zhi)
 void mi_post_error(hipError_t e, const char *file, int line);

@@ -140,16 +140,36 @@ void mx_gemm_memo_clear(void) {
     g_bmemo.clear();
 }
 
-extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res) {
-    if (bits != 4 && bits != 8) return -1;
-    if (M <= 0 || N <= 0) return 0;
-    if (K < 0) K = 0;
+// the workspace of one product: packed rows and scales of both operands (the same carving for every call of one shape)
+struct gemm_ws_t { uint8_t *Aq, *Bq, *As, *Bs; int nkb; };
+static bool gemm_ws(int bits, int M, int N, int K, gemm_ws_t *w) {
     const int nkb = (K + 63) / 64 * 2, BPB = bits == 8 ? 32 : 16;         // 32-K blocks of the packed rows (K rounded up to 64)
     const size_t qa = (size_t)M * nkb * BPB, qb = (size_t)N * nkb * BPB, sa = (size_t)M * nkb, sb = (size_t)N * nkb;
     auto al = [](size_t n) { return (n + 255) & ~(size_t)255; };
     uint8_t *base = (uint8_t *)mi_ws(MI_WS_GEMM, al(qa) + al(qb) + al(sa) + al(sb) + 256);
-    if (!base) return -1;
-    uint8_t *Aq = base, *Bq = Aq + al(qa), *As = Bq + al(qb), *Bs = As + al(sa);
+    if (!base) return false;
+    w->Aq = base; w->Bq = w->Aq + al(qa); w->As = w->Bq + al(qb); w->Bs = w->As + al(sa); w->nkb = nkb;
+    return true;
+}
+// (internal) where a kernel that produces A's rows quantises them itself, instead of writing fp32 rows for mx_pack_k to read back: the packed
+// rows of A of the product (M, N, K) that mi_mx_gemm_apacked then runs, in mx_pack_k<bits, 0>'s layout: codes [M][K / 32][32 (e4m3) or 16 (e2m1)
+// bytes], scales [M][K / 32]. K must be a multiple of 64 (no padding blocks)
+bool mi_mx_gemm_abuf(int bits, int M, int N, int K, uint8_t **Aq, uint8_t **As) {
+    gemm_ws_t w;
+    if ((bits != 4 && bits != 8) || M <= 0 || N <= 0 || K <= 0 || K % 64 || !gemm_ws(bits, M, N, K, &w)) return false;
+    *Aq = w.Aq; *As = w.As;
+    return true;
+}
+static int gemm_impl(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res, bool apacked) {
+    if (bits != 4 && bits != 8) return -1;
+    if (M <= 0 || N <= 0) return 0;
+    if (K < 0) K = 0;
+    gemm_ws_t ws;
+    if (!gemm_ws(bits, M, N, K, &ws)) return -1;
+    const int nkb = ws.nkb, BPB = bits == 8 ? 32 : 16;
+    const size_t qb = (size_t)N * nkb * BPB, sb = (size_t)N * nkb;
+    auto al = [](size_t n) { return (n + 255) & ~(size_t)255; };
+    uint8_t *Aq = ws.Aq, *Bq = ws.Bq, *As = ws.As, *Bs = ws.Bs;
     const int lda = ta ? M : K, ldb = tb ? K : N;
     bool bhave = false;
     if (g_bmemo_on && nkb) {
@@ -165,10 +185,10 @@ extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, cons
     if (nkb) {
         const unsigned ga = nblk_((size_t)M * nkb, 256), gb = nblk_((size_t)N * nkb, 256);
         if (bits == 8) {
-            if (ta) mx_pack_k<8, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<8, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
+            if (apacked) {} else if (ta) mx_pack_k<8, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<8, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
             if (bhave) {} else if (tb) mx_pack_k<8, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<8, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
         } else {
-            if (ta) mx_pack_k<4, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<4, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
+            if (apacked) {} else if (ta) mx_pack_k<4, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<4, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
             if (bhave) {} else if (tb) mx_pack_k<4, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<4, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
         }
     }
@@ -186,6 +206,14 @@ extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, cons
     else mx_gemm_k<4><<<grid, 64 * wn>>>(Aq, As, Bq, Bs, C, M, N, nkb, beta, bias, res, sper);
     MICK();
     return 0;
+}
+extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res) {
+    return gemm_impl(bits, ta, tb, M, N, K, A, B, C, beta, bias, res, false);
+}
+// (internal) lp_mx_gemm_ex with A's rows already packed where mi_mx_gemm_abuf said
+int mi_mx_gemm_apacked(int bits, int tb, int M, int N, int K, const float *B, float *C, float beta, const float *bias, const float *res) {
+    if (K <= 0 || K % 64) return -1;
+    return gemm_impl(bits, 0, tb, M, N, K, nullptr, B, C, beta, bias, res, true);
 }
 extern "C" int lp_mx_gemm(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta) {
     return lp_mx_gemm_ex(bits, ta, tb, M, N, K, A, B, C, beta, nullptr, nullptr);

@@ -164,6 +164,7 @@ _ATTN_PROTOS = {
     "lp_mx_gemm_ex": (_I, [_I, _I, _I, _I, _I, _I, _P, _P, _P, _F, _P, _P]),
     "at_fa8_fwd": (_I, [_P, _P, _P, C.POINTER(at_geom), _I, _I]),
     "at_fa8_waves": (None, [_I]),
+    "at_fuse_pack": (None, [_I]),
 }
 ATTN_EXPORTS = tuple(_ATTN_PROTOS)
 # include/mi_predict.h
