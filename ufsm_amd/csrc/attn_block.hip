@@ -107,24 +107,21 @@ __global__ void __launch_bounds__(256) glu_any_k(const float *__restrict__ h, fl
     const float a = h[t * 2 * F + f];
     gg[i] = a / (1.f + expf(-a)) * h[t * 2 * F + F + f];
 }
-// at_glu_fwd with the result written as the packed MX-fp8 A operand of the GEMM that follows: a thread takes one token's block of 32 features
-// (the same expression per value as glu_rows_k, then mx_pack_k<8, 0>'s quantisation of the block). F a multiple of 64
-__global__ void __launch_bounds__(256) glu_pack_k(const float *__restrict__ h, long long nblk, int nkb, uint8_t *__restrict__ pq, uint8_t *__restrict__ ps) {
-    const long long i = blockIdx.x * 256ll + threadIdx.x;
-    if (i >= nblk) return;
-    const long long t = i / nkb; const int kb = (int)(i - t * nkb), F = nkb * 32;
-    const float4 *pa = (const float4 *)(h + (size_t)t * 2 * F + kb * 32), *pb = (const float4 *)(h + (size_t)t * 2 * F + F + kb * 32);
-    float v[32];
-#pragma unroll
-    for (int j = 0; j < 8; j++) {
-        const float4 a = pa[j], b = pb[j];
-        v[4 * j] = a.x / (1.f + expf(-a.x)) * b.x; v[4 * j + 1] = a.y / (1.f + expf(-a.y)) * b.y; v[4 * j + 2] = a.z / (1.f + expf(-a.z)) * b.z; v[4 * j + 3] = a.w / (1.f + expf(-a.w)) * b.w;
-    }
-    unsigned codes[8];
-    const unsigned sb = d_quant_row<8, false>(v, 32, codes);
-    uint8_t *o = pq + (size_t)i * 32;
-    *(uint4 *)o = make_uint4(codes[0], codes[1], codes[2], codes[3]); *(uint4 *)(o + 16) = make_uint4(codes[4], codes[5], codes[6], codes[7]);
-    ps[i] = (uint8_t)sb;
+// at_glu_fwd with the result written as the packed MX-fp8 A operand of the GEMM that follows: glu_rows_k's thread (one float4 chunk of a token's
+// row, the same expression per value: contiguous 16-byte reads across a wavefront), then mx_pack_k<8, 0>'s quantisation of the block of 32
+// features that eight neighbouring lanes hold (their maxima meet through three lane exchanges). F a multiple of 64
+__global__ void __launch_bounds__(256) glu_pack_k(const float4 *__restrict__ h, size_t n4, unsigned F4, uint8_t *__restrict__ pq, uint8_t *__restrict__ ps) {
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (i >= n4) return;                                   // (n4 is a multiple of 8: the lanes of a group of eight leave together)
+    const size_t t = i / F4; const unsigned f = (unsigned)(i - t * F4);
+    const float4 a = h[t * 2 * F4 + f], b = h[t * 2 * F4 + F4 + f];
+    const float4 o = make_float4(a.x / (1.f + expf(-a.x)) * b.x, a.y / (1.f + expf(-a.y)) * b.y, a.z / (1.f + expf(-a.z)) * b.z, a.w / (1.f + expf(-a.w)) * b.w);
+    unsigned au = __float_as_uint(fmaxf(fmaxf(fabsf(o.x), fabsf(o.y)), fmaxf(fabsf(o.z), fabsf(o.w))));       // (fmaxf drops NaN; a non-negative number orders as its bits)
+    au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
+    au = max(au, (unsigned)__builtin_amdgcn_mov_dpp((int)au, 0x141, 0xF, 0xF, true));          // row_half_mirror: lane 7 - i of the group of eight
+    const int e = d_mx_exp(__uint_as_float(au), MI_INVQ8);
+    *(unsigned *)(pq + i * 4) = d_enc4_e4m3(o.x, o.y, o.z, o.w, e);            // (block (t, f / 8) lies at ((t F4 + f) / 8) 32 bytes: the chunks' codes are consecutive)
+    if (!(f & 7)) ps[i >> 3] = (uint8_t)(e + 127);
 }
 extern "C" void at_glu_fwd(const float *h, float *gg, long T, int F) {
     if (T <= 0 || F <= 0) return;
@@ -398,8 +395,8 @@ extern "C" int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, c
         if (int e = linear(up, T, w->xn2, w->h, nullptr)) return e;
     }
     if (fuse && mi_mx_gemm_abuf(8, (int)T, C, F, &aq, &as)) {
-        const long long nb = (long long)T * (F / 32);
-        glu_pack_k<<<nblk_((size_t)nb, 256), 256>>>(w->h, nb, F / 32, aq, as); MICK();
+        const size_t n4 = (size_t)T * (F / 4);
+        glu_pack_k<<<nblk_(n4, 256), 256>>>((const float4 *)w->h, n4, (unsigned)(F / 4), aq, as); MICK();
         return mi_mx_gemm_apacked(8, 1, (int)T, C, F, down.w, y, 0.f, down.b, w->x1);
     }
     at_glu_fwd(w->h, w->gg, T, F);

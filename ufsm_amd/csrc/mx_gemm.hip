@@ -37,6 +37,22 @@ __global__ void __launch_bounds__(256) mx_pack_k(const float *__restrict__ X, in
     }
 }
 
+// mx_pack_k<8, 0> for a row-major operand whose K is a multiple of 64 and whose rows start on 16 bytes: a thread takes one float4 of a row (a
+// wavefront reads 1 KiB contiguous instead of 64 runs of 128 bytes), the block of 32 values is eight neighbouring lanes' and their maxima meet
+// through three lane exchanges; the same maximum, exponent and codes
+__global__ void __launch_bounds__(256) mx_pack8_rows_k(const float4 *__restrict__ X, int ld4, size_t n4, unsigned K4, uint8_t *__restrict__ q, uint8_t *__restrict__ sc) {
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (i >= n4) return;                                   // (n4 is a multiple of 8: the lanes of a group of eight leave together)
+    const size_t r = i / K4; const unsigned k = (unsigned)(i - r * K4);
+    const float4 o = X[r * ld4 + k];
+    unsigned au = __float_as_uint(fmaxf(fmaxf(fabsf(o.x), fabsf(o.y)), fmaxf(fabsf(o.z), fabsf(o.w))));       // (fmaxf drops NaN; a non-negative number orders as its bits)
+    au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
+    au = max(au, (unsigned)__builtin_amdgcn_mov_dpp((int)au, 0x141, 0xF, 0xF, true));          // row_half_mirror: lane 7 - i of the group of eight
+    const int e = d_mx_exp(__uint_as_float(au), MI_INVQ8);
+    *(unsigned *)(q + i * 4) = d_enc4_e4m3(o.x, o.y, o.z, o.w, e);
+    if (!(k & 7)) sc[i >> 3] = (uint8_t)(e + 127);
+}
+
 __global__ void gemm_zero_k(float *c, size_t n) {
     for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) c[i] = 0.f;
 }
@@ -185,7 +201,10 @@ static int gemm_impl(int bits, int ta, int tb, int M, int N, int K, const float 
     if (nkb) {
         const unsigned ga = nblk_((size_t)M * nkb, 256), gb = nblk_((size_t)N * nkb, 256);
         if (bits == 8) {
-            if (apacked) {} else if (ta) mx_pack_k<8, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<8, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
+            if (apacked) {}
+            else if (ta) mx_pack_k<8, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
+            else if (K % 64 == 0 && (lda & 3) == 0 && ((size_t)A & 15) == 0) { const size_t n4 = (size_t)M * (K / 4); mx_pack8_rows_k<<<nblk_(n4, 256), 256>>>((const float4 *)A, lda / 4, n4, (unsigned)(K / 4), Aq, As); }
+            else mx_pack_k<8, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
             if (bhave) {} else if (tb) mx_pack_k<8, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<8, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
         } else {
             if (apacked) {} else if (ta) mx_pack_k<4, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<4, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
