@@ -45,8 +45,9 @@ int at_fa8_fwd(const void *qkvh, float *o, float *lse, const at_geom *g, int H, 
    keys each, merged in wavefront order): the same probabilities and codes as with 1, their sums added in another order (~1e-7 relative) */
 void at_fa8_waves(int nw);
 /* (no counterpart: a knob for tests) 0: at_block_fwd writes the fp32 rows of its LayerNorms and its SwiGLU (at_ws.xn, .xn2, .gg) and the GEMMs
-   pack them; 1 (default): with e4m3 linears and C, F multiples of 64 those kernels write the GEMMs' packed operands themselves and the three
-   fp32 buffers are left untouched (a forward never reads them again). The block's output has the same bits either way */
+   pack them; 1: with e4m3 linears and C, F multiples of 64 those kernels write the GEMMs' packed operands themselves and the three fp32 buffers
+   are left untouched (a forward never reads them again); 2 (default): also, for C <= 256, the up projection forms the SwiGLU in its epilogue and
+   writes the down projection's packed operand, and at_ws.h is left untouched too. The block's output has the same bits in all three */
 void at_fuse_pack(int on);
 
 /* ---- the attention block around those two (forward, self-attention path; src/attn.h:26-81, src/nn_attn.cu) ---- */

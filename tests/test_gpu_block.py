@@ -99,13 +99,16 @@ def test_block_with_packed_operands_from_the_producers_has_the_same_bits(gpu):
     Cc, H, F, nseq, D, nreg = 192, 4, 512, 3, 5, 2; S = nreg + D ** 3
     P, lay = make_block(rng, Cc, F)
     x = (rng.standard_normal((nseq * S, Cc)) * np.exp(rng.uniform(-2, 2, (nseq * S, 1)))).astype(np.float32)
-    lib.at_fuse_pack(0)
+    ys = []
     try:
-        rc0, y0 = run_block(8, Cc, H, F, 1, nreg, P, lay, x, nseq, S, D)
+        for mode in (0, 1, 2):                                   # 2: the up projection also forms the SwiGLU and packs it for the down projection
+            lib.at_fuse_pack(mode)
+            rc, y = run_block(8, Cc, H, F, 1, nreg, P, lay, x, nseq, S, D)
+            assert rc == 0 and np.isfinite(y).all()
+            ys.append(y)
     finally:
-        lib.at_fuse_pack(1)
-    rc1, y1 = run_block(8, Cc, H, F, 1, nreg, P, lay, x, nseq, S, D)
-    assert rc0 == 0 and rc1 == 0 and np.isfinite(y1).all() and np.array_equal(y0, y1)
+        lib.at_fuse_pack(2)
+    assert np.array_equal(ys[0], ys[1]) and np.array_equal(ys[0], ys[2])
 
 
 @pytest.mark.parametrize("nseq,dims,nreg,Cc", [(2, (3, 4, 5), 2, 96), (1, (8, 8, 8), 0, 192), (3, (1, 1, 7), 4, 48), (1, (2, 2, 2), 1, 4)])

@@ -359,8 +359,8 @@ __global__ void __launch_bounds__(256) v_mix_k(float *__restrict__ qkv, const fl
     if (own) ((float4 *)own)[i] = o;
     *v = make_float4(fmaf(l, f.x - o.x, o.x), fmaf(l, f.y - o.y, o.y), fmaf(l, f.z - o.z, o.z), fmaf(l, f.w - o.w, o.w));
 }
-static int g_fuse_pack = 1;
-extern "C" void at_fuse_pack(int on) { g_fuse_pack = on != 0; }
+static int g_fuse_pack = 2;
+extern "C" void at_fuse_pack(int on) { g_fuse_pack = on < 0 ? 0 : on > 2 ? 2 : on; }
 extern "C" int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, const float *x, float *y, const at_geom *g, at_ws *w) {
     if (d->dK > 0 || g->rays || g->lens || g->pos || w->vr < 0 || w->vr > 2 || (w->vr && (!w->v1 || (w->vr == 2 && !w->lam))) || d->rope > 1 || d->C != d->H * HD) return -1;
     const long T = (long)g->nseq * g->S; const int C = d->C, F = d->F;
@@ -389,6 +389,13 @@ extern "C" int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, c
     // MLP branch
     if (fuse && mi_mx_gemm_abuf(8, (int)T, 2 * F, C, &aq, &as)) {
         ln_pack_fwd(w->x1, P + bp->ln2g, P + bp->ln2b, w->m2, w->r2, T, C, aq, as);
+        if (g_fuse_pack > 1 && C <= 256) {
+            // ... and the up projection forms the SwiGLU in its epilogue and writes the down projection's packed operand: h is not stored either
+            const size_t nb = (size_t)T * (F / 32);
+            uint8_t *gq = (uint8_t *)mi_ws(MI_WS_GEMM2, nb * 32 + ((nb + 255) & ~(size_t)255) + 256), *gs = gq + nb * 32;
+            if (int e = mi_mx_gemm_glu((int)T, F, C, up.w, up.b, gq, gs)) return e;
+            return mi_mx_gemm_apacked_at(8, 1, (int)T, C, F, gq, gs, down.w, y, 0.f, down.b, w->x1);
+        }
         if (int e = mi_mx_gemm_apacked(8, 1, (int)T, 2 * F, C, up.w, w->h, 0.f, up.b, nullptr)) return e;
     } else {
         at_ln_fwd(w->x1, P + bp->ln2g, P + bp->ln2b, w->xn2, w->m2, w->r2, T, C);

@@ -269,6 +269,11 @@ void mi_restage_up(const void *x, int xdt, int N, int C, int D, int H, int W, gn
 // the MX GEMM with A's rows quantised by the kernel that produces them (csrc/mx_gemm.hip): where to write them, then the product
 bool mi_mx_gemm_abuf(int bits, int M, int N, int K, uint8_t **Aq, uint8_t **As);
 int mi_mx_gemm_apacked(int bits, int tb, int M, int N, int K, const float *B, float *C, float beta, const float *bias, const float *res);
+// the same with A's packed rows and scales anywhere in device memory
+int mi_mx_gemm_apacked_at(int bits, int tb, int M, int N, int K, const uint8_t *Aq, const uint8_t *As, const float *B, float *C, float beta, const float *bias, const float *res);
+// the up projection and the SwiGLU in one kernel (e4m3): g[t][f] = silu(h[t][f]) h[t][F + f], h = x W^T + b with x's packed rows where
+// mi_mx_gemm_abuf(8, T, 2 F, C) said and W [2 F][C] row-major, written as the packed A operand (gq, gs) of the down projection; h is not stored
+int mi_mx_gemm_glu(int T, int F, int C, const float *W, const float *bias, uint8_t *gq, uint8_t *gs);
 void mi_restage_sub(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits, size_t Ss, size_t v0);     // only voxels [v0, v0 + S) of tensors of Ss voxels
 void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int zlo, int zhi, int h2);   // only fine planes [zlo, zhi)
 void mi_post_error(hipError_t e, const char *file, int line);
@@ -278,7 +283,7 @@ void *mi_ws(int slot, size_t bytes);        // per-device grow-on-demand scratch
 void mi_ws_arena(void *base, size_t cap);   // the calling thread's scratch requests come from this fixed region until mi_ws_arena(nullptr, 0)
 bool mi_ws_arena_on(void);
 void mi_count_alloc(void);                  // bookkeeping: one more device allocation made by the library
-enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_UPCOARSE = 5, MI_WS_GEMM = 6, MI_WS_ATTN = 7, MI_WS_NSLOTS = 8 };
+enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_UPCOARSE = 5, MI_WS_GEMM = 6, MI_WS_ATTN = 7, MI_WS_GEMM2 = 8, MI_WS_NSLOTS = 9 };
 static inline unsigned nblk_(size_t n, unsigned b) { return (unsigned)((n + b - 1) / b); }
 [[noreturn]] void mi_die(const char *fmt, ...);
 // ---- slab-local GroupNorm statistics (gnp_t.ns > 0: src/nn_lp.h:15-18, src/lp_slab.cuh:7-12): the statistics hold one row per (sample,

@@ -176,17 +176,13 @@ bool mi_mx_gemm_abuf(int bits, int M, int N, int K, uint8_t **Aq, uint8_t **As) 
     *Aq = w.Aq; *As = w.As;
     return true;
 }
-static int gemm_impl(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res, bool apacked) {
-    if (bits != 4 && bits != 8) return -1;
-    if (M <= 0 || N <= 0) return 0;
-    if (K < 0) K = 0;
-    gemm_ws_t ws;
-    if (!gemm_ws(bits, M, N, K, &ws)) return -1;
-    const int nkb = ws.nkb, BPB = bits == 8 ? 32 : 16;
+// B's packed rows and scales for a product (M, N, K): the memoised copy when the memo is on (packed on its first use), else packed into the
+// call's workspace
+static void gemm_b_operand(int bits, int tb, int N, int K, const float *B, const gemm_ws_t &ws, uint8_t **Bq_, uint8_t **Bs_) {
+    const int nkb = ws.nkb, BPB = bits == 8 ? 32 : 16, ldb = tb ? K : N;
     const size_t qb = (size_t)N * nkb * BPB, sb = (size_t)N * nkb;
     auto al = [](size_t n) { return (n + 255) & ~(size_t)255; };
-    uint8_t *Aq = ws.Aq, *Bq = ws.Bq, *As = ws.As, *Bs = ws.Bs;
-    const int lda = ta ? M : K, ldb = tb ? K : N;
+    uint8_t *Bq = ws.Bq, *Bs = ws.Bs;
     bool bhave = false;
     if (g_bmemo_on && nkb) {
         int dev = 0; MIRT(hipGetDevice(&dev));
@@ -198,18 +194,32 @@ static int gemm_impl(int bits, int ta, int tb, int M, int N, int K, const float 
             if (q && sc) { g_bmemo.push_back(bmemo_t{B, bits, tb, N, K, dev, q, sc}); Bq = q; Bs = sc; }     // (packed below, found by the next call)
         }
     }
-    if (nkb) {
-        const unsigned ga = nblk_((size_t)M * nkb, 256), gb = nblk_((size_t)N * nkb, 256);
+    if (nkb && !bhave) {
+        const unsigned gb = nblk_((size_t)N * nkb, 256);
+        if (bits == 8) { if (tb) mx_pack_k<8, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<8, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); }
+        else { if (tb) mx_pack_k<4, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<4, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); }
+    }
+    *Bq_ = Bq; *Bs_ = Bs;
+}
+static int gemm_impl(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta, const float *bias, const float *res, bool apacked,
+                     const uint8_t *Aq_at = nullptr, const uint8_t *As_at = nullptr) {
+    if (bits != 4 && bits != 8) return -1;
+    if (M <= 0 || N <= 0) return 0;
+    if (K < 0) K = 0;
+    gemm_ws_t ws;
+    if (!gemm_ws(bits, M, N, K, &ws)) return -1;
+    const int nkb = ws.nkb;
+    const uint8_t *Aq = Aq_at ? Aq_at : ws.Aq, *As = As_at ? As_at : ws.As;
+    uint8_t *Bq, *Bs;
+    const int lda = ta ? M : K;
+    gemm_b_operand(bits, tb, N, K, B, ws, &Bq, &Bs);
+    if (nkb && !apacked) {
+        const unsigned ga = nblk_((size_t)M * nkb, 256);
         if (bits == 8) {
-            if (apacked) {}
-            else if (ta) mx_pack_k<8, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
-            else if (K % 64 == 0 && (lda & 3) == 0 && ((size_t)A & 15) == 0) { const size_t n4 = (size_t)M * (K / 4); mx_pack8_rows_k<<<nblk_(n4, 256), 256>>>((const float4 *)A, lda / 4, n4, (unsigned)(K / 4), Aq, As); }
-            else mx_pack_k<8, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
-            if (bhave) {} else if (tb) mx_pack_k<8, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<8, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
-        } else {
-            if (apacked) {} else if (ta) mx_pack_k<4, 1><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As); else mx_pack_k<4, 0><<<ga, 256>>>(A, lda, M, K, nkb, Aq, As);
-            if (bhave) {} else if (tb) mx_pack_k<4, 0><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs); else mx_pack_k<4, 1><<<gb, 256>>>(B, ldb, N, K, nkb, Bq, Bs);
-        }
+            if (ta) mx_pack_k<8, 1><<<ga, 256>>>(A, lda, M, K, nkb, ws.Aq, ws.As);
+            else if (K % 64 == 0 && (lda & 3) == 0 && ((size_t)A & 15) == 0) { const size_t n4 = (size_t)M * (K / 4); mx_pack8_rows_k<<<nblk_(n4, 256), 256>>>((const float4 *)A, lda / 4, n4, (unsigned)(K / 4), ws.Aq, ws.As); }
+            else mx_pack_k<8, 0><<<ga, 256>>>(A, lda, M, K, nkb, ws.Aq, ws.As);
+        } else { if (ta) mx_pack_k<4, 1><<<ga, 256>>>(A, lda, M, K, nkb, ws.Aq, ws.As); else mx_pack_k<4, 0><<<ga, 256>>>(A, lda, M, K, nkb, ws.Aq, ws.As); }
     }
     // few output tiles and a long K (the weight-gradient shape, src/lp_mxgemm.cu:259-265): split K so the GPU's 256 CUs have work
     const int tiles = ((N + 127) / 128) * ((M + 127) / 128), nst = nkb / 2;
@@ -233,6 +243,100 @@ extern "C" int lp_mx_gemm_ex(int bits, int ta, int tb, int M, int N, int K, cons
 int mi_mx_gemm_apacked(int bits, int tb, int M, int N, int K, const float *B, float *C, float beta, const float *bias, const float *res) {
     if (K <= 0 || K % 64) return -1;
     return gemm_impl(bits, 0, tb, M, N, K, nullptr, B, C, beta, bias, res, true);
+}
+int mi_mx_gemm_apacked_at(int bits, int tb, int M, int N, int K, const uint8_t *Aq, const uint8_t *As, const float *B, float *C, float beta, const float *bias, const float *res) {
+    if (K <= 0 || K % 64 || !Aq || !As) return -1;
+    return gemm_impl(bits, 0, tb, M, N, K, nullptr, B, C, beta, bias, res, true, Aq, As);
+}
+// ---- the MLP's up projection with the SwiGLU in its epilogue (e4m3 operands): g[t][f] = silu(h[t][f]) h[t][F + f], h = x W^T + b ----
+// The product is formed transposed, h^T = W x^T, so a token is a COLUMN of the accumulators: lane (r, h) holds, for token r of its wavefront's 32,
+// features (q & 3) + 4 h + 8 (q >> 2) of a 32-feature tile in element q - of the gate rows W[f] and of the value rows W[F + f] in two accumulators.
+// gate and value of one (token, feature) then sit in the same element of the same lane, the block of 32 features that the down projection's
+// operand quantises together is the lane's 16 values and its partner lane's (r, h ^ 1) 16: one lane exchange for the maximum, two for handing
+// each lane a contiguous half of the block's 32 codes. The 1 GB of h that a 61-window forward wrote and read back is never stored.
+// A wavefront keeps its tokens' operand fragments in registers (NST steps of 64 channels) and walks feature tiles; the weights' fragments come from
+// L2 (196 KB for 1024 x 192). The same MFMA steps in the same order on the same operand bytes as mx_gemm_k's, bias added and SwiGLU formed by the
+// expressions of the separate kernels.
+template <int NST>
+__global__ void __launch_bounds__(256) glu_gemm_k(const uint8_t *__restrict__ Xq, const uint8_t *__restrict__ Xs, const uint8_t *__restrict__ Wq, const uint8_t *__restrict__ Ws,
+                                                  const float *__restrict__ bias, uint8_t *__restrict__ gq, uint8_t *__restrict__ gs, int T, int F, int tiles_per_y) {
+    extern __shared__ __align__(16) float sbias[];           // [2 F]: the bias vector sits at an arbitrary offset of the parameter array; LDS reads are 16-byte ones
+    constexpr int nkb = 2 * NST;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
+    for (int i = tid; i < 2 * F; i += 256) sbias[i] = bias ? bias[i] : 0.f;
+    __syncthreads();
+    const int t0 = (blockIdx.x * 4 + wave) * 32;
+    if (t0 >= T) return;                                   // (no barrier below)
+    const size_t tr = (size_t)min(t0 + r, T - 1);          // (tokens past the end repeat the last one and store nothing)
+    auto frag = [&](const uint8_t *p) {
+        const v4i lo = *(const v4i *)p, hi = *(const v4i *)(p + 32);
+        return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    };
+    v8i fx[NST]; int ex[NST];
+#pragma unroll
+    for (int s = 0; s < NST; s++) { fx[s] = frag(Xq + tr * nkb * 32 + s * 64 + 16 * h); ex[s] = Xs[tr * nkb + 2 * s + h]; }
+    const int nft = F / 32, ft0 = blockIdx.y * tiles_per_y, ft1 = min(nft, ft0 + tiles_per_y);
+    for (int ft = ft0; ft < ft1; ft++) {
+        const int f0 = ft * 32;
+        const uint8_t *pa = Wq + (size_t)(f0 + r) * nkb * 32 + 16 * h, *pb = Wq + (size_t)(F + f0 + r) * nkb * 32 + 16 * h;
+        const uint8_t *sa = Ws + (size_t)(f0 + r) * nkb + h, *sb = Ws + (size_t)(F + f0 + r) * nkb + h;
+        v8i fa[NST], fb[NST]; int ea[NST], eb[NST];
+#pragma unroll
+        for (int s = 0; s < NST; s++) { fa[s] = frag(pa + s * 64); ea[s] = sa[2 * s]; fb[s] = frag(pb + s * 64); eb[s] = sb[2 * s]; }
+        v16f ca, cb;
+#pragma unroll
+        for (int q = 0; q < 16; q++) { ca[q] = 0.f; cb[q] = 0.f; }
+#pragma unroll
+        for (int s = 0; s < NST; s++) {
+            ca = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[s], fx[s], ca, 0, 0, 0, ea[s], 0, ex[s]);
+            cb = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[s], fx[s], cb, 0, 0, 0, eb[s], 0, ex[s]);
+        }
+        float v[16], am = 0.f;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float4 ba = *(const float4 *)(sbias + f0 + 8 * g + 4 * h), bb = *(const float4 *)(sbias + F + f0 + 8 * g + 4 * h);
+            const float a4[4] = {ca[4 * g] + ba.x, ca[4 * g + 1] + ba.y, ca[4 * g + 2] + ba.z, ca[4 * g + 3] + ba.w};
+            const float b4[4] = {cb[4 * g] + bb.x, cb[4 * g + 1] + bb.y, cb[4 * g + 2] + bb.z, cb[4 * g + 3] + bb.w};
+#pragma unroll
+            for (int c = 0; c < 4; c++) { const float a = a4[c]; v[4 * g + c] = a / (1.f + expf(-a)) * b4[c]; am = fmaxf(am, fabsf(v[4 * g + c])); }
+        }
+        {   // the other half of the block is the partner lane's (am is a non-negative number: it orders as its bits)
+            const unsigned u = __float_as_uint(am);
+            const auto r2 = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+            am = __uint_as_float(max(r2[0], r2[1]));
+        }
+        const int e = d_mx_exp(am, MI_INVQ8);
+        unsigned d[4];
+#pragma unroll
+        for (int g = 0; g < 4; g++) d[g] = d_enc4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], e);
+        // word g of half h is word 2 g + h of the block's eight: half 0 keeps its words 0, 1 and takes the partner's, half 1 keeps its words 2, 3
+        const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false), s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+        if (t0 + r < T) {
+            *(uint4 *)(gq + (tr * nft + ft) * 32 + 16 * h) = make_uint4(s02[0], s02[1], s13[0], s13[1]);
+            if (!h) gs[tr * nft + ft] = (uint8_t)(e + 127);
+        }
+    }
+}
+int mi_mx_gemm_glu(int T, int F, int C, const float *W, const float *bias, uint8_t *gq, uint8_t *gs) {
+    if (T <= 0 || F <= 0 || C <= 0 || C % 64 || C > 256 || F % 32 || !gq || !gs) return -1;
+    gemm_ws_t ws;
+    if (!gemm_ws(8, T, 2 * F, C, &ws)) return -1;          // (x's packed rows lie where mi_mx_gemm_abuf(8, T, 2 F, C) said)
+    uint8_t *Wq, *Wsc;
+    gemm_b_operand(8, 1, 2 * F, C, W, ws, &Wq, &Wsc);
+    // feature tiles per workgroup row: all of them when the token tiles alone fill the GPU, else split so that about 2 048 wavefronts run
+    const int nft = F / 32, ntt = (T + 127) / 128;
+    int ny = 1; while (ny < nft && (size_t)ntt * 4 * ny < 2048) ny *= 2;
+    const int tpy = (nft + ny - 1) / ny;
+    const dim3 grid((unsigned)ntt, (unsigned)((nft + tpy - 1) / tpy));
+    const size_t sm = (size_t)2 * F * sizeof(float);
+    switch (C / 64) {
+        case 1: glu_gemm_k<1><<<grid, 256, sm>>>(ws.Aq, ws.As, Wq, Wsc, bias, gq, gs, T, F, tpy); break;
+        case 2: glu_gemm_k<2><<<grid, 256, sm>>>(ws.Aq, ws.As, Wq, Wsc, bias, gq, gs, T, F, tpy); break;
+        case 3: glu_gemm_k<3><<<grid, 256, sm>>>(ws.Aq, ws.As, Wq, Wsc, bias, gq, gs, T, F, tpy); break;
+        default: glu_gemm_k<4><<<grid, 256, sm>>>(ws.Aq, ws.As, Wq, Wsc, bias, gq, gs, T, F, tpy); break;
+    }
+    MICK();
+    return 0;
 }
 extern "C" int lp_mx_gemm(int bits, int ta, int tb, int M, int N, int K, const float *A, const float *B, float *C, float beta) {
     return lp_mx_gemm_ex(bits, ta, tb, M, N, K, A, B, C, beta, nullptr, nullptr);
