@@ -28,7 +28,7 @@ def test_layernorm_glu_token_layout(gpu):
     dh, dgg = DevBuf.from_numpy(h), DevBuf(T * F * 4)
     lib.at_glu_fwd(dh.ptr, dgg.ptr, T, F)
     gg = np.zeros((T, F), np.float32); orc.lib().orc_glu_fwd(orc.ptr(h), orc.ptr(gg), T, F)
-    assert np.abs(dgg.to_numpy(np.float32, (T, F)) - gg).max() < 1e-6
+    assert np.abs(dgg.to_numpy(np.float32, (T, F)) - gg).max() < 2e-6 * max(1.0, np.abs(gg).max())      # (hardware exp2 and reciprocal: a few ulp of the largest values)
     n, Sg, nreg = 2, 125, 4
     xc = rng.standard_normal((n, Cc, Sg)).astype(np.float32); reg = rng.standard_normal((nreg, Cc)).astype(np.float32)
     dxc, dreg, dtok, dback = DevBuf.from_numpy(xc), DevBuf.from_numpy(reg), DevBuf(n * (Sg + nreg) * Cc * 4), DevBuf(xc.nbytes)

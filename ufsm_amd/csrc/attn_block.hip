@@ -92,20 +92,22 @@ static void ln_pack_fwd(const float *x, const float *g, const float *b, float *m
 #undef LN
     MICK();
 }
-// ---- SwiGLU (src/nn_attn.cu:438-455): gg[t][f] = silu(h[t][f]) h[t][F + f]; four features per thread, 16-byte accesses ----
+// ---- SwiGLU (src/nn_attn.cu:438-455): gg[t][f] = silu(h[t][f]) h[t][F + f]; four features per thread, 16-byte accesses. silu(a) = a rcp(1 +
+// exp2(-a log2 e)) on the hardware's exp2 and reciprocal, the form the reference's device fast-math build gives a / (1.f + expf(-a)) (approximate
+// exponential and division) and the one the conv path's SiLU has ----
 __global__ void __launch_bounds__(256) glu_rows_k(const float4 *__restrict__ h, float4 *__restrict__ gg, size_t n4, unsigned F4) {
     const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;      // one float4 chunk of one token's output row: any token count, full workgroups
     if (i >= n4) return;
     const size_t t = i / F4; const unsigned f = (unsigned)(i - t * F4);
     const float4 a = h[t * 2 * F4 + f], b = h[t * 2 * F4 + F4 + f];
-    gg[i] = make_float4(a.x / (1.f + expf(-a.x)) * b.x, a.y / (1.f + expf(-a.y)) * b.y, a.z / (1.f + expf(-a.z)) * b.z, a.w / (1.f + expf(-a.w)) * b.w);
+    gg[i] = make_float4(d_silu(a.x) * b.x, d_silu(a.y) * b.y, d_silu(a.z) * b.z, d_silu(a.w) * b.w);
 }
 __global__ void __launch_bounds__(256) glu_any_k(const float *__restrict__ h, float *__restrict__ gg, size_t n, int F) {       // widths that are not a multiple of 4
     const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
     if (i >= n) return;
     const size_t t = i / (unsigned)F; const int f = (int)(i - t * F);
     const float a = h[t * 2 * F + f];
-    gg[i] = a / (1.f + expf(-a)) * h[t * 2 * F + F + f];
+    gg[i] = d_silu(a) * h[t * 2 * F + F + f];
 }
 // at_glu_fwd with the result written as the packed MX-fp8 A operand of the GEMM that follows: glu_rows_k's thread (one float4 chunk of a token's
 // row, the same expression per value: contiguous 16-byte reads across a wavefront), then mx_pack_k<8, 0>'s quantisation of the block of 32
@@ -115,7 +117,7 @@ __global__ void __launch_bounds__(256) glu_pack_k(const float4 *__restrict__ h, 
     if (i >= n4) return;                                   // (n4 is a multiple of 8: the lanes of a group of eight leave together)
     const size_t t = i / F4; const unsigned f = (unsigned)(i - t * F4);
     const float4 a = h[t * 2 * F4 + f], b = h[t * 2 * F4 + F4 + f];
-    const float4 o = make_float4(a.x / (1.f + expf(-a.x)) * b.x, a.y / (1.f + expf(-a.y)) * b.y, a.z / (1.f + expf(-a.z)) * b.z, a.w / (1.f + expf(-a.w)) * b.w);
+    const float4 o = make_float4(d_silu(a.x) * b.x, d_silu(a.y) * b.y, d_silu(a.z) * b.z, d_silu(a.w) * b.w);
     unsigned au = __float_as_uint(fmaxf(fmaxf(fabsf(o.x), fabsf(o.y)), fmaxf(fabsf(o.z), fabsf(o.w))));       // (fmaxf drops NaN; a non-negative number orders as its bits)
     au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
     au = max(au, (unsigned)__builtin_amdgcn_mov_dpp((int)au, 0x141, 0xF, 0xF, true));          // row_half_mirror: lane 7 - i of the group of eight

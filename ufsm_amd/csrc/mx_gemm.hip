@@ -298,7 +298,7 @@ __global__ void __launch_bounds__(256) glu_gemm_k(const uint8_t *__restrict__ Xq
             const float a4[4] = {ca[4 * g] + ba.x, ca[4 * g + 1] + ba.y, ca[4 * g + 2] + ba.z, ca[4 * g + 3] + ba.w};
             const float b4[4] = {cb[4 * g] + bb.x, cb[4 * g + 1] + bb.y, cb[4 * g + 2] + bb.z, cb[4 * g + 3] + bb.w};
 #pragma unroll
-            for (int c = 0; c < 4; c++) { const float a = a4[c]; v[4 * g + c] = a / (1.f + expf(-a)) * b4[c]; am = fmaxf(am, fabsf(v[4 * g + c])); }
+            for (int c = 0; c < 4; c++) { v[4 * g + c] = d_silu(a4[c]) * b4[c]; am = fmaxf(am, fabsf(v[4 * g + c])); }
         }
         {   // the other half of the block is the partner lane's (am is a non-negative number: it orders as its bits)
             const unsigned u = __float_as_uint(am);
