@@ -62,7 +62,7 @@ __global__ void __launch_bounds__(256) ln_row_k(const float4 *__restrict__ x, co
             float am = on ? fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fabsf(v[i].z), fabsf(v[i].w))) : 0.f;       // (fmaxf drops NaN, as the pack kernel's)
             unsigned au = __float_as_uint(am);                                 // (non-negative, never NaN: orders as its bits)
             au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
-            au = max(au, (unsigned)__builtin_amdgcn_mov_dpp((int)au, 0x141, 0xF, 0xF, true));      // row_half_mirror: lane 7 - i of the group of eight
+            au = max(au, d_oct_mirror_u(au));
             const int e = d_mx_exp(__uint_as_float(au), MI_INVQ8);
             const unsigned code = d_enc4_e4m3(v[i].x, v[i].y, v[i].z, v[i].w, e);
             if (on) {
@@ -120,7 +120,7 @@ __global__ void __launch_bounds__(256) glu_pack_k(const float4 *__restrict__ h, 
     const float4 o = make_float4(d_silu(a.x) * b.x, d_silu(a.y) * b.y, d_silu(a.z) * b.z, d_silu(a.w) * b.w);
     unsigned au = __float_as_uint(fmaxf(fmaxf(fabsf(o.x), fabsf(o.y)), fmaxf(fabsf(o.z), fabsf(o.w))));       // (fmaxf drops NaN; a non-negative number orders as its bits)
     au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
-    au = max(au, (unsigned)__builtin_amdgcn_mov_dpp((int)au, 0x141, 0xF, 0xF, true));          // row_half_mirror: lane 7 - i of the group of eight
+    au = max(au, d_oct_mirror_u(au));
     const int e = d_mx_exp(__uint_as_float(au), MI_INVQ8);
     *(unsigned *)(pq + i * 4) = d_enc4_e4m3(o.x, o.y, o.z, o.w, e);            // (block (t, f / 8) lies at ((t F4 + f) / 8) 32 bytes: the chunks' codes are consecutive)
     if (!(f & 7)) ps[i >> 3] = (uint8_t)(e + 127);
@@ -220,7 +220,7 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
                 float ss = 0.f;
 #pragma unroll
                 for (int i = 0; i < 8; i++) ss = fmaf(v[i], v[i], ss);
-                ss += __shfl_xor(ss, 1); ss += __shfl_xor(ss, 2); ss += __shfl_xor(ss, 4);
+                ss += d_quad_xor_f<1>(ss); ss += d_quad_xor_f<2>(ss); ss += d_oct_mirror_f(ss);      // (the unit's eight lanes: the same sums as the xor butterfly's, no LDS round trips)
                 const float r = 1.f / sqrtf(ss / HD + 1e-6f);
                 if (j == 0) (p ? rk : rq)[t * H + h] = r;
                 if (j < 6) {
@@ -246,7 +246,7 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
                 float m = 0.f;
 #pragma unroll
                 for (int i = 0; i < 8; i++) m = fmaxf(m, fabsf(v[i]));
-                m = fmaxf(m, __shfl_xor(m, 1)); m = fmaxf(m, __shfl_xor(m, 2)); m = fmaxf(m, __shfl_xor(m, 4));
+                m = fmaxf(m, d_quad_xor_f<1>(m)); m = fmaxf(m, d_quad_xor_f<2>(m)); m = fmaxf(m, d_oct_mirror_f(m));
                 if (j == 0) atomicMax(&bmax, __float_as_uint(m));               // (non-negative floats order as their bit patterns)
             }
             if (j < 6) {

@@ -38,6 +38,10 @@ template <int M> __device__ __forceinline__ unsigned d_quad_xor_u(unsigned x) {
     return (unsigned)__builtin_amdgcn_mov_dpp((int)x, M == 1 ? 0xB1 : 0x4E, 0xF, 0xF, true);        // quad_perm [1, 0, 3, 2] / [2, 3, 0, 1]
 }
 template <int M> __device__ __forceinline__ float d_quad_xor_f(float x) { return __uint_as_float(d_quad_xor_u<M>(__float_as_uint(x))); }
+// the value of lane 7 - i of the lane's group of eight (row_half_mirror): after the two exchanges inside the groups of four, every lane of a
+// group of four holds the same partial result, and this brings the other group's - the third step of a reduction over eight lanes
+__device__ __forceinline__ unsigned d_oct_mirror_u(unsigned x) { return (unsigned)__builtin_amdgcn_mov_dpp((int)x, 0x141, 0xF, 0xF, true); }
+__device__ __forceinline__ float d_oct_mirror_f(float x) { return __uint_as_float(d_oct_mirror_u(__float_as_uint(x))); }
 __device__ __forceinline__ unsigned d_amax_u(unsigned a, float v) { const unsigned b = __float_as_uint(v) & 0x7fffffffu; return b > a ? b : a; }
 
 // e4m3 (OCP FN: max 448, 0x7f NaN), round to nearest even, saturating. For |x| < 448 the value is rounded to a multiple of the

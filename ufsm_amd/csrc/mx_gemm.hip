@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(256) mx_pack8_rows_k(const float4 *__restrict_
     const float4 o = X[r * ld4 + k];
     unsigned au = __float_as_uint(fmaxf(fmaxf(fabsf(o.x), fabsf(o.y)), fmaxf(fabsf(o.z), fabsf(o.w))));       // (fmaxf drops NaN; a non-negative number orders as its bits)
     au = max(au, d_quad_xor_u<1>(au)); au = max(au, d_quad_xor_u<2>(au));
-    au = max(au, (unsigned)__builtin_amdgcn_mov_dpp((int)au, 0x141, 0xF, 0xF, true));          // row_half_mirror: lane 7 - i of the group of eight
+    au = max(au, d_oct_mirror_u(au));
     const int e = d_mx_exp(__uint_as_float(au), MI_INVQ8);
     *(unsigned *)(q + i * 4) = d_enc4_e4m3(o.x, o.y, o.z, o.w, e);
     if (!(k & 7)) sc[i >> 3] = (uint8_t)(e + 127);
