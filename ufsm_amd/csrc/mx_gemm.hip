@@ -276,13 +276,22 @@ __global__ void __launch_bounds__(256) glu_gemm_k(const uint8_t *__restrict__ Xq
 #pragma unroll
     for (int s = 0; s < NST; s++) { fx[s] = frag(Xq + tr * nkb * 32 + s * 64 + 16 * h); ex[s] = Xs[tr * nkb + 2 * s + h]; }
     const int nft = F / 32, ft0 = blockIdx.y * tiles_per_y, ft1 = min(nft, ft0 + tiles_per_y);
-    for (int ft = ft0; ft < ft1; ft++) {
+    // the weight fragments of tile ft + 1 are requested before tile ft is multiplied (they come from L2: nothing else hides that latency)
+    v8i fan[NST], fbn[NST]; int ean[NST], ebn[NST];
+    auto request = [&](int ft) {
         const int f0 = ft * 32;
         const uint8_t *pa = Wq + (size_t)(f0 + r) * nkb * 32 + 16 * h, *pb = Wq + (size_t)(F + f0 + r) * nkb * 32 + 16 * h;
         const uint8_t *sa = Ws + (size_t)(f0 + r) * nkb + h, *sb = Ws + (size_t)(F + f0 + r) * nkb + h;
+#pragma unroll
+        for (int s = 0; s < NST; s++) { fan[s] = frag(pa + s * 64); ean[s] = sa[2 * s]; fbn[s] = frag(pb + s * 64); ebn[s] = sb[2 * s]; }
+    };
+    if (ft0 < ft1) request(ft0);
+    for (int ft = ft0; ft < ft1; ft++) {
+        const int f0 = ft * 32;
         v8i fa[NST], fb[NST]; int ea[NST], eb[NST];
 #pragma unroll
-        for (int s = 0; s < NST; s++) { fa[s] = frag(pa + s * 64); ea[s] = sa[2 * s]; fb[s] = frag(pb + s * 64); eb[s] = sb[2 * s]; }
+        for (int s = 0; s < NST; s++) { fa[s] = fan[s]; ea[s] = ean[s]; fb[s] = fbn[s]; eb[s] = ebn[s]; }
+        request(min(ft + 1, ft1 - 1));                     // (the last tile requests itself again)
         v16f ca, cb;
 #pragma unroll
         for (int q = 0; q < 16; q++) { ca[q] = 0.f; cb[q] = 0.f; }
