@@ -254,75 +254,77 @@ int mi_mx_gemm_apacked_at(int bits, int tb, int M, int N, int K, const uint8_t *
 // gate and value of one (token, feature) then sit in the same element of the same lane, the block of 32 features that the down projection's
 // operand quantises together is the lane's 16 values and its partner lane's (r, h ^ 1) 16: one lane exchange for the maximum, two for handing
 // each lane a contiguous half of the block's 32 codes. The 1 GB of h that a 61-window forward wrote and read back is never stored.
-// A wavefront keeps its tokens' operand fragments in registers (NST steps of 64 channels) and walks feature tiles; the weights' fragments come from
-// L2 (196 KB for 1024 x 192). The same MFMA steps in the same order on the same operand bytes as mx_gemm_k's, bias added and SwiGLU formed by the
+// A wavefront keeps the operand fragments of its 64 tokens in registers (NST steps of 64 channels) and walks feature tiles; the weights' fragments
+// come from L2 (196 KB for 1024 x 192), each serving both token tiles (with one token tile per wavefront the launch was bound by that traffic). The same MFMA steps in the same order on the same operand bytes as mx_gemm_k's, bias added and SwiGLU formed by the
 // expressions of the separate kernels.
 template <int NST>
 __global__ void __launch_bounds__(256) glu_gemm_k(const uint8_t *__restrict__ Xq, const uint8_t *__restrict__ Xs, const uint8_t *__restrict__ Wq, const uint8_t *__restrict__ Ws,
                                                   const float *__restrict__ bias, uint8_t *__restrict__ gq, uint8_t *__restrict__ gs, int T, int F, int tiles_per_y) {
     extern __shared__ __align__(16) float sbias[];           // [2 F]: the bias vector sits at an arbitrary offset of the parameter array; LDS reads are 16-byte ones
-    constexpr int nkb = 2 * NST;
+    constexpr int nkb = 2 * NST, TT = 2;                     // TT: token tiles of 32 per wavefront (a weight fragment fetched from L2 serves both)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, h = lane >> 5;
     for (int i = tid; i < 2 * F; i += 256) sbias[i] = bias ? bias[i] : 0.f;
     __syncthreads();
-    const int t0 = (blockIdx.x * 4 + wave) * 32;
+    const int t0 = (blockIdx.x * 4 + wave) * 32 * TT;
     if (t0 >= T) return;                                   // (no barrier below)
-    const size_t tr = (size_t)min(t0 + r, T - 1);          // (tokens past the end repeat the last one and store nothing)
     auto frag = [&](const uint8_t *p) {
         const v4i lo = *(const v4i *)p, hi = *(const v4i *)(p + 32);
         return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
-    v8i fx[NST]; int ex[NST];
+    size_t tr[TT];                                         // (tokens past the end repeat the last one and store nothing)
+    v8i fx[TT][NST]; int ex[TT][NST];
 #pragma unroll
-    for (int s = 0; s < NST; s++) { fx[s] = frag(Xq + tr * nkb * 32 + s * 64 + 16 * h); ex[s] = Xs[tr * nkb + 2 * s + h]; }
+    for (int u = 0; u < TT; u++) {
+        tr[u] = (size_t)min(t0 + 32 * u + r, T - 1);
+#pragma unroll
+        for (int s = 0; s < NST; s++) { fx[u][s] = frag(Xq + tr[u] * nkb * 32 + s * 64 + 16 * h); ex[u][s] = Xs[tr[u] * nkb + 2 * s + h]; }
+    }
     const int nft = F / 32, ft0 = blockIdx.y * tiles_per_y, ft1 = min(nft, ft0 + tiles_per_y);
-    // the weight fragments of tile ft + 1 are requested before tile ft is multiplied (they come from L2: nothing else hides that latency)
-    v8i fan[NST], fbn[NST]; int ean[NST], ebn[NST];
-    auto request = [&](int ft) {
+    for (int ft = ft0; ft < ft1; ft++) {
         const int f0 = ft * 32;
         const uint8_t *pa = Wq + (size_t)(f0 + r) * nkb * 32 + 16 * h, *pb = Wq + (size_t)(F + f0 + r) * nkb * 32 + 16 * h;
         const uint8_t *sa = Ws + (size_t)(f0 + r) * nkb + h, *sb = Ws + (size_t)(F + f0 + r) * nkb + h;
-#pragma unroll
-        for (int s = 0; s < NST; s++) { fan[s] = frag(pa + s * 64); ean[s] = sa[2 * s]; fbn[s] = frag(pb + s * 64); ebn[s] = sb[2 * s]; }
-    };
-    if (ft0 < ft1) request(ft0);
-    for (int ft = ft0; ft < ft1; ft++) {
-        const int f0 = ft * 32;
         v8i fa[NST], fb[NST]; int ea[NST], eb[NST];
 #pragma unroll
-        for (int s = 0; s < NST; s++) { fa[s] = fan[s]; ea[s] = ean[s]; fb[s] = fbn[s]; eb[s] = ebn[s]; }
-        request(min(ft + 1, ft1 - 1));                     // (the last tile requests itself again)
-        v16f ca, cb;
+        for (int s = 0; s < NST; s++) { fa[s] = frag(pa + s * 64); ea[s] = sa[2 * s]; fb[s] = frag(pb + s * 64); eb[s] = sb[2 * s]; }
+        v16f ca[TT], cb[TT];
 #pragma unroll
-        for (int q = 0; q < 16; q++) { ca[q] = 0.f; cb[q] = 0.f; }
+        for (int u = 0; u < TT; u++)
 #pragma unroll
-        for (int s = 0; s < NST; s++) {
-            ca = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[s], fx[s], ca, 0, 0, 0, ea[s], 0, ex[s]);
-            cb = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[s], fx[s], cb, 0, 0, 0, eb[s], 0, ex[s]);
-        }
-        float v[16], am = 0.f;
+            for (int q = 0; q < 16; q++) { ca[u][q] = 0.f; cb[u][q] = 0.f; }
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const float4 ba = *(const float4 *)(sbias + f0 + 8 * g + 4 * h), bb = *(const float4 *)(sbias + F + f0 + 8 * g + 4 * h);
-            const float a4[4] = {ca[4 * g] + ba.x, ca[4 * g + 1] + ba.y, ca[4 * g + 2] + ba.z, ca[4 * g + 3] + ba.w};
-            const float b4[4] = {cb[4 * g] + bb.x, cb[4 * g + 1] + bb.y, cb[4 * g + 2] + bb.z, cb[4 * g + 3] + bb.w};
+        for (int s = 0; s < NST; s++)
 #pragma unroll
-            for (int c = 0; c < 4; c++) { v[4 * g + c] = d_silu(a4[c]) * b4[c]; am = fmaxf(am, fabsf(v[4 * g + c])); }
-        }
-        {   // the other half of the block is the partner lane's (am is a non-negative number: it orders as its bits)
-            const unsigned u = __float_as_uint(am);
-            const auto r2 = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-            am = __uint_as_float(max(r2[0], r2[1]));
-        }
-        const int e = d_mx_exp(am, MI_INVQ8);
-        unsigned d[4];
+            for (int u = 0; u < TT; u++) {
+                ca[u] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[s], fx[u][s], ca[u], 0, 0, 0, ea[s], 0, ex[u][s]);
+                cb[u] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[s], fx[u][s], cb[u], 0, 0, 0, eb[s], 0, ex[u][s]);
+            }
 #pragma unroll
-        for (int g = 0; g < 4; g++) d[g] = d_enc4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], e);
-        // word g of half h is word 2 g + h of the block's eight: half 0 keeps its words 0, 1 and takes the partner's, half 1 keeps its words 2, 3
-        const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false), s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-        if (t0 + r < T) {
-            *(uint4 *)(gq + (tr * nft + ft) * 32 + 16 * h) = make_uint4(s02[0], s02[1], s13[0], s13[1]);
-            if (!h) gs[tr * nft + ft] = (uint8_t)(e + 127);
+        for (int u = 0; u < TT; u++) {
+            float v[16], am = 0.f;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const float4 ba = *(const float4 *)(sbias + f0 + 8 * g + 4 * h), bb = *(const float4 *)(sbias + F + f0 + 8 * g + 4 * h);
+                const float a4[4] = {ca[u][4 * g] + ba.x, ca[u][4 * g + 1] + ba.y, ca[u][4 * g + 2] + ba.z, ca[u][4 * g + 3] + ba.w};
+                const float b4[4] = {cb[u][4 * g] + bb.x, cb[u][4 * g + 1] + bb.y, cb[u][4 * g + 2] + bb.z, cb[u][4 * g + 3] + bb.w};
+#pragma unroll
+                for (int c = 0; c < 4; c++) { v[4 * g + c] = d_silu(a4[c]) * b4[c]; am = fmaxf(am, fabsf(v[4 * g + c])); }
+            }
+            {   // the other half of the block is the partner lane's (am is a non-negative number: it orders as its bits)
+                const unsigned w = __float_as_uint(am);
+                const auto r2 = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+                am = __uint_as_float(max(r2[0], r2[1]));
+            }
+            const int e = d_mx_exp(am, MI_INVQ8);
+            unsigned d[4];
+#pragma unroll
+            for (int g = 0; g < 4; g++) d[g] = d_enc4_e4m3(v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3], e);
+            // word g of half h is word 2 g + h of the block's eight: half 0 keeps its words 0, 1 and takes the partner's, half 1 keeps its words 2, 3
+            const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false), s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+            if (t0 + 32 * u + r < T) {
+                *(uint4 *)(gq + (tr[u] * nft + ft) * 32 + 16 * h) = make_uint4(s02[0], s02[1], s13[0], s13[1]);
+                if (!h) gs[tr[u] * nft + ft] = (uint8_t)(e + 127);
+            }
         }
     }
 }
@@ -333,7 +335,7 @@ int mi_mx_gemm_glu(int T, int F, int C, const float *W, const float *bias, uint8
     uint8_t *Wq, *Wsc;
     gemm_b_operand(8, 1, 2 * F, C, W, ws, &Wq, &Wsc);
     // feature tiles per workgroup row: all of them when the token tiles alone fill the GPU, else split so that about 2 048 wavefronts run
-    const int nft = F / 32, ntt = (T + 127) / 128;
+    const int nft = F / 32, ntt = (T + 255) / 256;         // (a workgroup: four wavefronts of 64 tokens)
     int ny = 1; while (ny < nft && (size_t)ntt * 4 * ny < 2048) ny *= 2;
     const int tpy = (nft + ny - 1) / ny;
     const dim3 grid((unsigned)ntt, (unsigned)((nft + tpy - 1) / tpy));
