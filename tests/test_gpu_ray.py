@@ -1,0 +1,205 @@
+"""Radial attention and scroll RoPE on the device (include/mi_attn.h: at_rays_setup, at_ray_gather / _scatter, at_scroll_pos, at_fa_fwd, at_fa_pack
+with coordinates, at_block_fwd with rays) against the double-precision oracle (oracle/ray_oracle.py), with the gates of the reference's
+tests/test_attn_ray.c: max |gpu - ref| / rms(ref) < 2e-3 per tensor for the maps and the fp16 core (the block's MX linears: test_attn.c's MX gate)."""
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+import ray_oracle as ro  # noqa: E402
+from gpuutil import DevBuf, LP, lib  # noqa: E402
+from ufsm_amd import at_geom, at_dims, at_bp, at_ws, at_rays  # noqa: E402
+from test_oracle_block import make_block  # noqa: E402
+from test_oracle_ray import make_axr  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+
+def rel(a, b):
+    return np.abs(a - b).max() / max(np.sqrt((b.astype(np.float64) ** 2).mean()), 1e-30)
+
+
+class DevRays:
+    """a ray set on the device, planned by the library, with the oracle's tables beside it"""
+
+    def __init__(self, n, D, Hh, W, mult, axr):
+        self.o = ro.make_rays(n, D, Hh, W, mult, axr)
+        q, nt, nr = C.c_int(), C.c_int(), C.c_int()
+        lib.at_rays_dims(D, Hh, W, C.c_float(mult), C.byref(q), C.byref(nt), C.byref(nr))
+        Q, Nt, Nr = q.value, nt.value, nr.value; P = max(D, Hh, W)
+        assert (Q, Nt, Nr) == (self.o["Q"], self.o["Nt"], self.o["Nr"])
+        ray = np.zeros((n, Q, 8), np.float32); lens = np.zeros((n, Q), np.int32); ad = np.zeros(n, np.int32); cen = np.zeros((n, P, 4), np.float32)
+        lib.at_rays_plan(n, D, Hh, W, C.c_float(mult), axr.ctypes.data, ray.ctypes.data, lens.ctypes.data, ad.ctypes.data, cen.ctypes.data)
+        self.ray_h, self.lens_h, self.cen_h = ray, lens, cen
+        self.Tr, self.Tg = n * Q * Nr, n * D * Hh * W
+        self.bufs = dict(ray=DevBuf.from_numpy(ray), lens=DevBuf.from_numpy(lens), ad=DevBuf.from_numpy(ad), cen=DevBuf.from_numpy(cen),
+                         pos=DevBuf.from_numpy(np.full(self.Tr * 3, np.nan, np.float32)), wsum=DevBuf.from_numpy(np.full(self.Tg, np.nan, np.float32)))
+        R = at_rays(); R.n, R.Q, R.Nt, R.Nr, R.D, R.Hh, R.W = n, Q, Nt, Nr, D, Hh, W
+        R.ad, R.ray, R.lens, R.pos, R.wsum = (self.bufs[k].ptr for k in ("ad", "ray", "lens", "pos", "wsum"))
+        self.R = R
+        lib.at_rays_setup(C.byref(R)); LP.check()
+
+
+@pytest.mark.parametrize("D,Hh,W,mult", [(6, 5, 7, 2.0), (8, 8, 8, 2.0)])
+def test_ray_maps(gpu, D, Hh, W, mult):
+    n = 3; axr = make_axr(n, D, Hh, W, (0, 1, 2), (0, 1, 2))
+    t = DevRays(n, D, Hh, W, mult, axr); o = t.o
+    pos = t.bufs["pos"].to_numpy(np.float32, (t.Tr, 3)); ws = t.bufs["wsum"].to_numpy(np.float32, (t.Tg,))
+    assert np.abs(pos - o["pos"]).max() < 1e-5                                     # (r0 + i, arc, k) as the table says
+    assert rel(ws, o["winv"]) < 1e-5 and ((ws > 0) == (o["winv"] > 0)).all()
+    rng = np.random.default_rng(0); Cc = 8
+    x = rng.standard_normal((t.Tg, Cc)).astype(np.float32); y = rng.standard_normal((t.Tr, Cc)).astype(np.float32)
+    dx, dy, dg, ds = DevBuf.from_numpy(x), DevBuf.from_numpy(y), DevBuf.from_numpy(np.full((t.Tr, Cc), np.nan, np.float32)), DevBuf.from_numpy(np.full((t.Tg, Cc), np.nan, np.float32))
+    for norm in (0, 1):
+        lib.at_ray_gather(C.byref(t.R), dx.ptr, dg.ptr, Cc, norm); lib.at_ray_scatter(C.byref(t.R), dy.ptr, ds.ptr, Cc, norm); LP.check()
+        G, S = dg.to_numpy(np.float32, (t.Tr, Cc)), ds.to_numpy(np.float32, (t.Tg, Cc))
+        winv = o["winv"] if norm else None
+        wg, wsx = ro.gather(x.astype(np.float64), o["rows"], o["w"], winv), ro.scatter(y.astype(np.float64), o["rows"], o["w"], t.Tg, winv)
+        assert rel(G, wg) < 1e-5 and rel(S, wsx) < 1e-5
+        a, b = (G.astype(np.float64) * y).sum(), (x * S.astype(np.float64)).sum()  # <G x, y> = <x, S y> on the device's own results
+        assert abs(a - b) < 1e-5 * np.abs(G.astype(np.float64) * y).sum()
+    # slots past a ray's length gather zero rows
+    lens = np.repeat(t.ray_h[..., 6].reshape(-1).astype(np.int64), o["Nr"]); slot = np.tile(np.arange(o["Nr"]), n * o["Q"])
+    assert (G[slot >= lens] == 0).all()
+
+
+def test_scroll_pos_on_the_device(gpu):
+    D, Hh, W, n, nreg = 5, 6, 4, 3, 2
+    axr = make_axr(n, D, Hh, W, (1, 0, 2), (0, 1, 2))
+    t = DevRays(n, D, Hh, W, 2.0, axr)
+    S = nreg + D * Hh * W; dp = DevBuf.from_numpy(np.full((n * S, 3), np.nan, np.float32))
+    lib.at_scroll_pos(n, nreg, D, Hh, W, t.bufs["ad"].ptr, t.bufs["cen"].ptr, dp.ptr); LP.check()
+    want = ro.scroll_pos(n, nreg, D, Hh, W, t.o["ad"], t.cen_h)
+    got = dp.to_numpy(np.float32, (n * S, 3))
+    assert np.abs(got - want).max() < 1e-4
+
+
+def pack(qkv, qg, kg, g, nreg, Cc, rope):
+    T = g.nseq * g.S; H = Cc // 48
+    dq, dqg, dkg = DevBuf.from_numpy(qkv), DevBuf.from_numpy(qg), DevBuf.from_numpy(kg)
+    dqh = DevBuf.from_numpy(np.full(3 * H * (T + 64) * 48, 0x7e00, np.uint16)); drq, drk, damx = DevBuf(T * H * 4), DevBuf(T * H * 4), DevBuf(16)
+    lib.at_fa_pack(dq.ptr, dqg.ptr, dkg.ptr, dqh.ptr, drq.ptr, drk.ptr, damx.ptr, C.byref(g), nreg, Cc, rope, 100.0); LP.check()
+    return dqh
+
+
+def test_pack_with_coordinates_and_the_length_masked_core(gpu):
+    rng = np.random.default_rng(5)
+    nseq, S, Cc, H = 37, 23, 96, 2; T = nseq * S
+    qkv = rng.standard_normal((T, 3 * Cc)).astype(np.float32); qg = (1 + 0.2 * rng.standard_normal(Cc)).astype(np.float32); kg = (1 + 0.2 * rng.standard_normal(Cc)).astype(np.float32)
+    pos = rng.uniform(-4, 12, (T, 3)).astype(np.float32); lens = rng.integers(0, S + 1, nseq).astype(np.int32); lens[:3] = (0, 1, S)
+    dpos, dlens = DevBuf.from_numpy(pos), DevBuf.from_numpy(lens)
+    g = at_geom(); g.nseq, g.S, g.D, g.Hh, g.W = nseq, S, 1, 1, S; g.pos = dpos.ptr
+    dqh = pack(qkv, qg, kg, g, 0, Cc, 2)
+    got = dqh.to_numpy(np.uint16, (3, H, T + 64, 48)).view(np.float16).astype(np.float64)
+    q, k, v = (qkv[:, i * Cc:(i + 1) * Cc].astype(np.float64).reshape(T, H, 48) for i in range(3))
+    q = q / np.sqrt((q ** 2).mean(-1, keepdims=True) + 1e-6) * qg.astype(np.float64).reshape(H, 48)
+    k = k / np.sqrt((k ** 2).mean(-1, keepdims=True) + 1e-6) * kg.astype(np.float64).reshape(H, 48)
+    qr, kr = ro.rope(q, pos.astype(np.float64), 100.0), ro.rope(k, pos.astype(np.float64), 100.0)
+    for i, want in enumerate((qr, kr, v)):
+        assert np.abs(got[i, :, :T].transpose(1, 0, 2) - want).max() < 1.5e-3 * np.abs(want).max()          # fp16 storage (and fp32 angles up to 12 x 1)
+    assert (got[:, :, T:] == 0).all()
+    # the core on exactly these fp16 rows, keys masked past each sequence's length
+    g.lens = dlens.ptr
+    do, dl = DevBuf.from_numpy(np.full((T, Cc), np.nan, np.float32)), DevBuf.from_numpy(np.full((nseq, H, S), np.nan, np.float32))
+    lib.at_fa_fwd(dqh.ptr, do.ptr, dl.ptr, C.byref(g), H, Cc); LP.check()
+    o = do.to_numpy(np.float32, (T, Cc)); lse = dl.to_numpy(np.float32, (nseq, H, S))
+    qh, kh, vh = (got[i, :, :T].transpose(1, 0, 2) for i in range(3))
+    want = ro.attend(qh, kh, vh, nseq, S, lens)
+    assert rel(o, want) < 2e-3                                                     # (probabilities rounded to fp16 before they meet v)
+    assert (o[:S] == 0).all() and (lse[0] == 0).all()                              # a length of 0: zero output
+    assert np.abs(o[S:2 * S] - vh[S].reshape(-1)).max() < 1e-6                     # a length of 1: the one key's value for every query
+    s = 2; lg = np.einsum("ihd,jhd->hij", qh[s * S:(s + 1) * S], kh[s * S:(s + 1) * S]) / np.sqrt(48.0)
+    assert np.abs(lse[s] - np.log2(np.exp(lg).sum(-1))).max() < 1e-4
+    # without lengths every key counts
+    g.lens = None
+    lib.at_fa_fwd(dqh.ptr, do.ptr, dl.ptr, C.byref(g), H, Cc); LP.check()
+    assert rel(do.to_numpy(np.float32, (T, Cc)), ro.attend(qh, kh, vh, nseq, S, None)) < 2e-3
+
+
+def test_core_on_sequences_longer_than_a_wavefront(gpu):
+    rng = np.random.default_rng(6)
+    nseq, S, Cc, H = 3, 150, 48, 1; T = nseq * S
+    qkv = rng.standard_normal((T, 3 * Cc)).astype(np.float32); ones = np.ones(Cc, np.float32)
+    lens = np.array([150, 97, 64], np.int32); dlens = DevBuf.from_numpy(lens)
+    g = at_geom(); g.nseq, g.S, g.D, g.Hh, g.W = nseq, S, 1, 1, S
+    dqh = pack(qkv, ones, ones, g, 0, Cc, 0)
+    got = dqh.to_numpy(np.uint16, (3, H, T + 64, 48)).view(np.float16).astype(np.float64)
+    g.lens = dlens.ptr
+    do, dl = DevBuf(T * Cc * 4), DevBuf(nseq * H * S * 4)
+    lib.at_fa_fwd(dqh.ptr, do.ptr, dl.ptr, C.byref(g), H, Cc); LP.check()
+    qh, kh, vh = (got[i, :, :T].transpose(1, 0, 2) for i in range(3))
+    assert rel(do.to_numpy(np.float32, (T, Cc)), ro.attend(qh, kh, vh, nseq, S, lens)) < 2e-3
+
+
+def run_block(P, lay, x, d, g, Tr=0):
+    bp = at_bp(); assert lib.at_block_layout(C.byref(d), C.byref(bp), 0) == P.size
+    T = x.shape[0]
+    ws = at_ws(); wsb = DevBuf(lib.at_ws_bytes_r(C.byref(d), T, Tr)); lib.at_ws_carve_r(C.byref(ws), C.byref(d), T, Tr, wsb.ptr)
+    assert (ws.qkvr is not None) == (Tr > 0) and lib.at_ws_bytes_r(C.byref(d), T, 0) == lib.at_ws_bytes(C.byref(d), T)
+    dP, dx, dy = DevBuf.from_numpy(P), DevBuf.from_numpy(x), DevBuf.from_numpy(np.full(x.shape, np.nan, np.float32))
+    rc = lib.at_block_fwd(C.byref(d), dP.ptr, C.byref(bp), dx.ptr, dy.ptr, C.byref(g), C.byref(ws)); LP.check()
+    lib.mi_sync()
+    qkv, o = np.empty((T, 3 * d.C), np.float32), np.empty((T, d.C), np.float32)    # the block's own projected rows and its attention output
+    lib.mi_d2h(qkv.ctypes.data, ws.qkv, qkv.nbytes); lib.mi_d2h(o.ctypes.data, ws.o, o.nbytes)
+    return rc, dy.to_numpy(np.float32, x.shape), qkv, o
+
+
+def attention_of(P, lay, qkv, **kw):
+    Cc = kw["Cc"]
+    """the oracle's attention branch on the device's own qkv rows: what the block's attention output must be, without the MX linears' noise"""
+    return ro.attention(qkv.astype(np.float64), P[lay["qg"]:lay["qg"] + Cc].astype(np.float64), P[lay["kg"]:lay["kg"] + Cc].astype(np.float64), **kw)
+
+
+@pytest.mark.parametrize("rope", [2, 1, 0])
+def test_block_with_radial_attention(gpu, rope):
+    """samples with the axis inside the grid, outside it and without one (tests/test_attn_ray.c:340-372's cases), one block each way"""
+    rng = np.random.default_rng(7 + rope)
+    D, Hh, W, Cc, H, F, n = 6, 5, 7, 192, 4, 512, 3; S = D * Hh * W; T = n * S
+    axr = make_axr(n, D, Hh, W, (0, 1, 2), (0, 1, 2))
+    t = DevRays(n, D, Hh, W, 2.0, axr)
+    P, lay = make_block(rng, Cc, F)
+    x = rng.standard_normal((T, Cc)).astype(np.float32)
+    d = at_dims(); d.C, d.H, d.F, d.rope, d.nreg, d.rope_base = Cc, H, F, rope, 0, 100.0
+    g = at_geom(); g.nseq, g.S, g.D, g.Hh, g.W = n, S, D, Hh, W; g.rays = C.addressof(t.R)
+    rc, y, qkv, o = run_block(P, lay, x, d, g, t.Tr)
+    assert rc == 0 and np.isfinite(y).all()
+    # gather, QK-norm, RoPE on the ray positions, length-masked attention per ray (fp16 q / k / v), normalised scatter: the reference's gate for
+    # the fp16 core is 6e-3 of the tensor's rms (tests/test_attn_ray.c:13)
+    assert rel(o, attention_of(P, lay, qkv, nseq=n, S=S, H=H, Cc=Cc, rope_mode=rope, rays=t.o)) < 6e-3
+    want = ro.block(P, lay, x, n, S, H, Cc, F, rope_mode=rope, rays=t.o)
+    # the linears are MX-fp8 GEMMs: the reference's gate for them against the exact block is 0.1 (tests/test_attn.c)
+    assert np.linalg.norm(y - want) / np.linalg.norm(want) < 0.05
+    # and the radial attention is what ran: full attention over the grid is further away
+    full = ro.block(P, lay, x, n, S, H, Cc, F, rope_mode=0)
+    assert np.linalg.norm(y - full) > 2 * np.linalg.norm(y - want)
+    d.nreg = 1                                                                     # rays take no register tokens
+    assert run_block(P, lay, x, d, g, t.Tr)[0] == -1
+
+
+def test_block_with_scroll_rope_over_the_grid(gpu):
+    rng = np.random.default_rng(11)
+    D, Hh, W, Cc, H, F, n, nreg = 5, 6, 4, 192, 4, 512, 3, 2; S = nreg + D * Hh * W; T = n * S
+    axr = make_axr(n, D, Hh, W, (1, 0, 2), (0, 1, 2))
+    t = DevRays(n, D, Hh, W, 2.0, axr)
+    dp = DevBuf(T * 12)
+    lib.at_scroll_pos(n, nreg, D, Hh, W, t.bufs["ad"].ptr, t.bufs["cen"].ptr, dp.ptr); LP.check()
+    pos = dp.to_numpy(np.float32, (T, 3)).astype(np.float64)                       # (the device's own coordinates: their parity is the test above)
+    P, lay = make_block(rng, Cc, F)
+    x = rng.standard_normal((T, Cc)).astype(np.float32)
+    d = at_dims(); d.C, d.H, d.F, d.rope, d.nreg, d.rope_base = Cc, H, F, 2, nreg, 100.0
+    g = at_geom(); g.nseq, g.S, g.D, g.Hh, g.W = n, S, D, Hh, W; g.pos = dp.ptr
+    rc, y, qkv, o = run_block(P, lay, x, d, g)
+    assert rc == 0
+    # the MX-fp8 core with rotations by the scroll coordinates: the core's own gate (tests/test_gpu_gemm_attn.py) on the block's attention output
+    wo = attention_of(P, lay, qkv, nseq=n, S=S, H=H, Cc=Cc, rope_mode=2, pos=pos, nreg=nreg)
+    assert np.linalg.norm(o - wo) / np.linalg.norm(wo) < 0.05
+    want = ro.block(P, lay, x, n, S, H, Cc, F, rope_mode=2, pos=pos, nreg=nreg)
+    assert np.linalg.norm(y - want) / np.linalg.norm(want) < 0.05
+    grid = ro.block(P, lay, x, n, S, H, Cc, F, rope_mode=1, grid=(D, Hh, W), nreg=nreg)
+    assert np.linalg.norm(y - grid) > 2 * np.linalg.norm(y - want)                 # not the grid-index rotation
+    g.pos = None                                                                   # scroll RoPE without coordinates is refused
+    assert run_block(P, lay, x, d, g)[0] == -1

@@ -8,7 +8,7 @@ CSRC = os.path.join(ROOT, "ufsm_amd", "csrc")
 LIB = os.path.join(ROOT, "ufsm_amd", "libufsm_lp.so")
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "liboracle.so")
-HIP_SOURCES = ["rt.hip", "mx_elem.hip", "mx_gemm.hip", "attn8.hip", "attn_block.hip", "predict.hip", "conv3.hip", "conv3_stem.hip", "conv2.hip", "conv2_f8.hip", "conv2_f4.hip"] + ["conv3_f%d_o%d.hip" % (f, o) for f in (8, 4) for o in (8, 4, 0)]
+HIP_SOURCES = ["rt.hip", "mx_elem.hip", "mx_gemm.hip", "attn8.hip", "attn_block.hip", "attn_ray.hip", "predict.hip", "conv3.hip", "conv3_stem.hip", "conv2.hip", "conv2_f8.hip", "conv2_f4.hip"] + ["conv3_f%d_o%d.hip" % (f, o) for f in (8, 4) for o in (8, 4, 0)]
 HIPCC_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wno-unused-value",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # per-file additions. attn8.hip: the attention core rescales its output accumulators on the vector pipe between two matrix products of every key

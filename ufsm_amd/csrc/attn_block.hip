@@ -177,19 +177,21 @@ extern "C" void at_tok_to_cs(const float *t, float *x, int n, int C, long Sg, in
 }
 
 // ---- QKV pack (src/nn_attn_tc.cu:99-136): per (token, head) the 48 q and k dims are RMS-normalised (eps 1e-6) and scaled by their learned
-// gains, grid tokens rotated by the axial 3-D rotary embedding (16 dims per axis: pair f of axis a turns by pos_a base^(-f / 8)), v passes
+// gains, grid tokens rotated by the 3-D rotary embedding (16 dims per coordinate: pair f of coordinate a turns by pos_a base^(-f / 8); pos = the
+// token's grid indices, or its row of a coordinate array: src/nn_attn.cu:272-289), v passes
 // through; all three go to the fp16 head-major layout [3][H][T + 64][48] the attention core reads (64 zero rows of padding).
 // A unit = one (token, part, head) = 48 values = six 8-dim slices; eight neighbouring lanes own a unit (two idle), each slice is two 16-byte
 // loads and one 16-byte store of eight halves. The sum of squares meets over the unit's lanes; a rotary pair never leaves its lane
 // (slice j covers pairs 4 (j & 1) .. + 3 of axis j / 2). ----
 __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv, const float *__restrict__ qg, const float *__restrict__ kg, __half *__restrict__ out,
-                                                  float *__restrict__ rq, float *__restrict__ rk, float *__restrict__ amx, long long T, int H, int S, int Hh, int W, int nreg, int rope, float lbase) {
+                                                  float *__restrict__ rq, float *__restrict__ rk, float *__restrict__ amx, long long T, int H, int S, int Hh, int W, int nreg, int rope, float lbase,
+                                                  const float *__restrict__ gpos) {
     // the rotary angles take few values - position along an axis x frequency - and a sine / cosine pair costs far more than the rest of a unit:
     // a block forms the table once (the same expression the per-value form evaluates, so the same bits), positions up to RP per axis
     constexpr int RP = 64;
     __shared__ float2 rtab[RP * 8];
     const int pmax = max(max(S / (Hh * W), Hh), W);         // positions along an axis: < pmax (registers included in S: an upper bound)
-    const bool tab = rope && pmax <= RP;
+    const bool tab = rope && !gpos && pmax <= RP;            // (gpos: per-token coordinates, real numbers: every angle is evaluated)
     if (tab) {
         for (int i = threadIdx.x; i < pmax * 8; i += 256) { float sn, cs; sincosf((float)(i >> 3) * exp2f(-lbase * (float)(i & 7) / 8.f), &sn, &cs); rtab[i] = make_float2(sn, cs); }
         __syncthreads();
@@ -230,7 +232,7 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
                     const int ts = (int)(t % S) - nreg;
                     if (rope && ts >= 0) {
                         const int ax = j >> 1;
-                        const float pos = ax == 0 ? (float)(ts / (Hh * W)) : ax == 1 ? (float)((ts / W) % Hh) : (float)(ts % W);
+                        const float pos = gpos ? gpos[3 * t + ax] : ax == 0 ? (float)(ts / (Hh * W)) : ax == 1 ? (float)((ts / W) % Hh) : (float)(ts % W);
 #pragma unroll
                         for (int i = 0; i < 4; i++) {
                             const int fi = 4 * (j & 1) + i;
@@ -262,11 +264,10 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
 }
 __global__ void at_zero4_k(float *p) { if (threadIdx.x < 4) p[threadIdx.x] = 0.f; }
 extern "C" void at_fa_pack(const float *qkv, const float *qg, const float *kg, void *qkvh, float *rq, float *rk, float *amx, const at_geom *g, int nreg, int C, int rope, float base) {
-    if (g->pos) mi_die("at_fa_pack: per-token rotary positions are not supported");
     if (C % HD || (C & 3)) mi_die("at_fa_pack: C %d is not a whole number of heads of %d", C, HD);
     const long long T = (long long)g->nseq * g->S, Tp = T + FT; const int H = C / HD;
     at_zero4_k<<<1, 64>>>(amx);
-    qkv_pack_k<<<nblk_((size_t)Tp * H * 3 * 8, 256), 256>>>(qkv, qg, kg, (__half *)qkvh, rq, rk, amx, T, H, g->S, g->Hh, g->W, nreg, rope, log2f(base));
+    qkv_pack_k<<<nblk_((size_t)Tp * H * 3 * 8, 256), 256>>>(qkv, qg, kg, (__half *)qkvh, rq, rk, amx, T, H, g->S, g->Hh, g->W, nreg, rope, log2f(base), rope ? g->pos : nullptr);
     MICK();
 }
 
@@ -282,19 +283,22 @@ extern "C" size_t at_block_layout(const at_dims *d, at_bp *bp, size_t off) {
     return off;
 }
 extern "C" size_t at_block_nparams(const at_dims *d) { at_bp bp; return at_block_layout(d, &bp, 0); }
-static size_t ws_walk(at_ws *w, const at_dims *d, long T, float *base) {      // pieces of whole 256 bytes; base null: sizes only
-    const size_t C = d->C, F = d->F, H = d->H, t = (size_t)T;
+static size_t ws_walk(at_ws *w, const at_dims *d, long T, long Tr, float *base) {      // pieces of whole 256 bytes; base null: sizes only. Tr: ray tokens (0: none)
+    const size_t C = d->C, F = d->F, H = d->H, t = (size_t)T, ta = Tr > 0 ? (size_t)Tr : t;   // ta: the tokens the attention itself runs on
     size_t n = 0;
     auto take = [&](float *&f, size_t m) { f = base ? base + n : nullptr; n += (m + 63) & ~(size_t)63; };
     at_ws tmp; if (!w) w = &tmp;
     *w = at_ws{};
     take(w->xn, t * C); take(w->o, t * C); take(w->x1, t * C); take(w->xn2, t * C); take(w->qkv, t * 3 * C); take(w->h, t * 2 * F); take(w->gg, t * F);
-    take(w->m1, t); take(w->r1, t); take(w->m2, t); take(w->r2, t); take(w->rq, t * H); take(w->rk, t * H); take(w->lse, t * H);
-    take(w->qkvh, 3 * C * (t + FT) / 2); take(w->amx, 4);
+    take(w->m1, t); take(w->r1, t); take(w->m2, t); take(w->r2, t); take(w->rq, ta * H); take(w->rk, ta * H); take(w->lse, ta * H);
+    take(w->qkvh, 3 * C * (ta + FT) / 2); take(w->amx, 4);
+    if (Tr > 0) { take(w->qkvr, ta * 3 * C); take(w->orr, ta * C); }
     return n;
 }
-extern "C" size_t at_ws_bytes(const at_dims *d, long T) { return ws_walk(nullptr, d, T, nullptr) * sizeof(float); }
-extern "C" void at_ws_carve(at_ws *w, const at_dims *d, long T, void *base) { ws_walk(w, d, T, (float *)base); }
+extern "C" size_t at_ws_bytes(const at_dims *d, long T) { return ws_walk(nullptr, d, T, 0, nullptr) * sizeof(float); }
+extern "C" void at_ws_carve(at_ws *w, const at_dims *d, long T, void *base) { ws_walk(w, d, T, 0, (float *)base); }
+extern "C" size_t at_ws_bytes_r(const at_dims *d, long T, long Tr) { return ws_walk(nullptr, d, T, Tr, nullptr) * sizeof(float); }
+extern "C" void at_ws_carve_r(at_ws *w, const at_dims *d, long T, long Tr, void *base) { ws_walk(w, d, T, Tr, (float *)base); }
 
 static thread_local int g_at_mx = 8;
 extern "C" void at_set_mx(int bits) { g_at_mx = bits; }
@@ -364,8 +368,15 @@ __global__ void __launch_bounds__(256) v_mix_k(float *__restrict__ qkv, const fl
 static int g_fuse_pack = 2;
 extern "C" void at_fuse_pack(int on) { g_fuse_pack = on < 0 ? 0 : on > 2 ? 2 : on; }
 extern "C" int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, const float *x, float *y, const at_geom *g, at_ws *w) {
-    if (d->dK > 0 || g->rays || g->lens || g->pos || w->vr < 0 || w->vr > 2 || (w->vr && (!w->v1 || (w->vr == 2 && !w->lam))) || d->rope > 1 || d->C != d->H * HD) return -1;
+    const at_rays *R = g->rays;
+    if (d->dK > 0 || w->vr < 0 || w->vr > 2 || (w->vr && (!w->v1 || (w->vr == 2 && !w->lam))) || d->rope < 0 || d->rope > 2 || d->C != d->H * HD) return -1;
+    if (R ? d->nreg != 0 || !w->qkvr || !w->orr || !R->lens || !R->wsum || (d->rope == 2 && !R->pos) || (long)R->n * R->D * R->Hh * R->W != (long)g->nseq * g->S
+          : g->lens != nullptr || (d->rope == 2 && !g->pos)) return -1;      // (sequence lengths belong to the ray path; scroll RoPE needs its coordinates)
     const long T = (long)g->nseq * g->S; const int C = d->C, F = d->F;
+    // the attention's own geometry: the grid's, or (radial attention) the rays' - R->n Q sequences of Nr slots, their lengths and positions (src/nn_attn.cu:576-581)
+    at_geom ga = *g;
+    if (R) { ga = at_geom{}; ga.nseq = R->n * R->Q; ga.S = R->Nr; ga.D = 1; ga.Hh = 1; ga.W = R->Nr; ga.lens = R->lens; ga.pos = d->rope == 2 ? R->pos : nullptr; }
+    else if (d->rope != 2) ga.pos = nullptr;
     const linear_t qkv = {P + bp->wqkv, P + bp->bqkv, 3 * C, C}, proj = {P + bp->wo, P + bp->bo, C, C}, up = {P + bp->w1, P + bp->b1, 2 * F, C}, down = {P + bp->w2, P + bp->b2, C, F};
     // The rows a LayerNorm or the SwiGLU produces are read by one GEMM only: with e4m3 linears and widths that are multiples of 64 they are
     // written as that GEMM's packed operand directly and the fp32 rows (xn, xn2, gg of the scratch record, which only a backward pass would
@@ -385,8 +396,15 @@ extern "C" int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, c
         if (w->vr == 1) v_keep_k<<<nblk_(n4, 256), 256>>>(w->qkv, w->v1, n4, C / 4); else v_mix_k<<<nblk_(n4, 256), 256>>>(w->qkv, w->v1, w->own, w->lam, n4, C / 4);
         MICK();
     }
-    at_fa_pack(w->qkv, P + bp->qg, P + bp->kg, w->qkvh, w->rq, w->rk, w->amx, g, d->nreg, C, d->rope, d->rope_base);
-    if (int e = at_fa8_fwd(w->qkvh, w->o, w->lse, g, d->H, C)) return e;
+    if (R) {
+        at_ray_gather(R, w->qkv, w->qkvr, 3 * C, 0);
+        at_fa_pack(w->qkvr, P + bp->qg, P + bp->kg, w->qkvh, w->rq, w->rk, w->amx, &ga, 0, C, d->rope, d->rope_base);
+        at_fa_fwd(w->qkvh, w->orr, w->lse, &ga, d->H, C);
+        at_ray_scatter(R, w->orr, w->o, C, 1);
+    } else {
+        at_fa_pack(w->qkv, P + bp->qg, P + bp->kg, w->qkvh, w->rq, w->rk, w->amx, &ga, d->nreg, C, d->rope, d->rope_base);
+        if (int e = at_fa8_fwd(w->qkvh, w->o, w->lse, &ga, d->H, C)) return e;
+    }
     if (int e = linear(proj, T, w->o, w->x1, x)) return e;
     // MLP branch
     if (fuse && mi_mx_gemm_abuf(8, (int)T, 2 * F, C, &aq, &as)) {

@@ -126,6 +126,10 @@ class at_geom(C.Structure):  # src/attn.h:81
                 ("lens", C.c_void_p), ("pos", C.c_void_p), ("rays", C.c_void_p), ("dfx", C.c_void_p * 3), ("dfr", C.c_void_p)]
 
 
+class at_rays(C.Structure):  # src/attn.h:93-100
+    _fields_ = [(n, C.c_int) for n in ("n", "Q", "Nt", "Nr", "D", "Hh", "W")] + [(n, C.c_void_p) for n in ("ad", "ray", "lens", "pos", "wsum")]
+
+
 class at_dims(C.Structure):  # src/attn.h:33
     _fields_ = [("C", C.c_int), ("H", C.c_int), ("F", C.c_int), ("rope", C.c_int), ("nreg", C.c_int), ("rope_base", C.c_float),
                 ("dK", C.c_int), ("dL", C.c_int), ("dC", C.c_int * 3), ("dCo", C.c_int), ("dInit", C.c_int)]
@@ -165,6 +169,15 @@ _ATTN_PROTOS = {
     "at_fa8_fwd": (_I, [_P, _P, _P, C.POINTER(at_geom), _I, _I]),
     "at_fa8_waves": (None, [_I]),
     "at_fuse_pack": (None, [_I]),
+    "at_ws_bytes_r": (_Z, [C.POINTER(at_dims), C.c_long, C.c_long]),
+    "at_ws_carve_r": (None, [C.POINTER(at_ws), C.POINTER(at_dims), C.c_long, C.c_long, _P]),
+    "at_rays_dims": (None, [_I, _I, _I, _F, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "at_rays_plan": (None, [_I, _I, _I, _I, _F, _P, _P, _P, _P, _P]),
+    "at_rays_setup": (None, [C.POINTER(at_rays)]),
+    "at_ray_gather": (None, [C.POINTER(at_rays), _P, _P, _I, _I]),
+    "at_ray_scatter": (None, [C.POINTER(at_rays), _P, _P, _I, _I]),
+    "at_scroll_pos": (None, [_I, _I, _I, _I, _I, _P, _P, _P]),
+    "at_fa_fwd": (None, [_P, _P, _P, C.POINTER(at_geom), _I, _I]),
 }
 ATTN_EXPORTS = tuple(_ATTN_PROTOS)
 # include/mi_predict.h
