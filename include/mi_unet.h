@@ -55,7 +55,7 @@ const char *nn_check(void);                                    /* src/nn.h:28 */
 #define UNET_MAXLEV 8
 /* The reference's configuration record, field for field (src/unet.h:18-128): the layout is part of the boundary. This build runs the plain
    U-Net (+ down_norm, + self-attention blocks with RoPE / no positional encoding and register tokens). Fields it honours: nlev, widths, cin,
-   cout, G, down_norm, attn_blocks, attn_pe (1 or 2), attn_reg, attn_mlp, dec_widths (0: the encoder's width), dec_convs (1: one-conv decoder block),
+   cout, G, down_norm, attn_blocks, attn_pe (0 PEG, 1 RoPE, 2 none, 3 scroll RoPE), attn_axis (1: radial attention), attn_reg, attn_mlp, dec_widths (0: the encoder's width), dec_convs (1: one-conv decoder block),
    enc_blocks (residual blocks after encoder levels >= 1), w4_2d, l0_norm (0 .. 4) with l0_slab, gn_ema; half_res and scan_norm concern the caller only. Any other field must be 0: unet_create prints which one is not and returns NULL. */
 typedef struct {
     int nlev;
@@ -145,6 +145,15 @@ void unet_set_film(unet *u, const float *codes, int k);        /* cfg.film nets:
 size_t unet_gfilm_off(const unet *u);                          /* cfg.gfilm: the offset of its first scale / shift pair in the parameter vector (src/unet.h:160) */
 const float *mi_unet_gfilm_codes(const unet *u);               /* cfg.gfilm: the pooled codes of the last forward, widths[nlev-1] device floats (no counterpart in the reference's interface: its tests freeze them through the environment) */
 size_t mi_unet_film_off(const unet *u);                        /* cfg.film: the same for its pairs (no counterpart in the reference's interface: its tests print the offset) */
+/* cfg.attn_axis 1 / attn_pe 3 (src/unet.h:13-16, :470-474): the scroll axis of every sample of the following forwards. n records of stride floats
+   (host memory, copied): ad (the window dim of the scroll axis: 0 z, 1 y, 2 x), valid (0: no axis), np (window planes along ad), div (window
+   voxels per network input voxel), then per window plane along ad the axis centre (u, v) on the other two window dims in order, in window
+   voxels (voxel centres at integers; may lie outside the window). n 0 / null, a record count other than the forward's sample count, or a plane
+   count that does not fit the net's bottleneck grid: no axis (rays along the grid rows, grid-index coordinates) */
+#define UNET_AXR(np) (4 + 2 * (np))
+void unet_set_attn_axis(unet *u, const float *rec, int n, int stride);
+/* radial attention's ray set after a forward (src/unet.h:475-477): rays per sample, slots per ray, the share of grid tokens a sample touches; -1 without */
+int unet_attn_rays(const unet *u, int *Q, int *Nr, double *coverage);
 void unet_set_cond(unet *u, float c);                          /* ... or the code c itself (src/unet.h:146-147) */
 void unet_gn_ema_live(unet *u, int on);                        /* cfg.gn_ema: 1 = forwards normalise with the window's own statistics instead of the running ones (src/unet.h:172) */
 long unet_gn_ema_updates(const unet *u);                       /* cfg.gn_ema: updates the loaded running statistics have seen (src/unet.h:288); 0: live statistics */

@@ -59,7 +59,7 @@ def test_caller_side_keys_pass_through(tmp_path):
     assert rc == 0 and cfg.half_res == 1 and cfg.scan_norm == 1
 
 
-@pytest.mark.parametrize("feature", ['"lat_guide":1', '"attn_mem":4', '"lat_dec":[16,0,1]', '"film":7', '"fstem":[2,16]', '"view_P":4', '"attn_axis":1', '"l0_norm":7'])
+@pytest.mark.parametrize("feature", ['"lat_guide":1', '"attn_mem":4', '"lat_dec":[16,0,1]', '"film":7', '"fstem":[2,16]', '"view_P":4', '"attn_deform":4', '"l0_norm":7'])
 def test_refuses_architectures_it_does_not_run(tmp_path, feature):
     h = 'UFSM{"nlev":2,"widths":[32,64],%s,"cin":4,"cout":1,"G":8,"down_norm":1,"scale_cond":0,"nparams":10,"step":1,"extra":{}}\n' % feature
     assert read(tmp_path, h)[0] == -2
@@ -114,6 +114,9 @@ def test_reads_the_running_statistics_key(tmp_path):
 def test_rejects_foreign_files(tmp_path):
     assert read(tmp_path, "not a checkpoint\n")[0] == -1
     assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,64],"cin":4,"cout":1,"skip_empty":[80,2,1],"nparams":1}\n')[0] == -2   # trained with masked convs
-    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":3,"attn_reg":0,"attn_mlp":256,"cin":4,"cout":1,"nparams":1}\n')[0] == -2   # scroll RoPE
+    rc, cfg, n, step = read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":3,"attn_reg":0,"attn_mlp":256,"attn_axis":1,"cin":4,"cout":1,"nparams":1}\n')
+    assert rc == 0 and cfg.attn_pe == 3 and cfg.attn_axis == 1     # scroll RoPE, radial attention (src/unet.c:5691)
+    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":4,"attn_reg":0,"attn_mlp":256,"cin":4,"cout":1,"nparams":1}\n')[0] == -2
+    assert read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":1,"attn_reg":0,"attn_mlp":256,"attn_axis":2,"cin":4,"cout":1,"nparams":1}\n')[0] == -2
     rc, cfg, n, step = read(tmp_path, 'UFSM{"nlev":2,"widths":[32,96],"attn_blocks":1,"attn_pe":0,"attn_reg":0,"attn_mlp":256,"attn_vres":1,"cin":4,"cout":1,"nparams":1}\n')
     assert rc == 0 and cfg.attn_pe == 0 and cfg.attn_vres == 1     # PEG, value residual

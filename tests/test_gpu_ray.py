@@ -203,3 +203,170 @@ def test_block_with_scroll_rope_over_the_grid(gpu):
     assert np.linalg.norm(y - grid) > 2 * np.linalg.norm(y - want)                 # not the grid-index rotation
     g.pos = None                                                                   # scroll RoPE without coordinates is refused
     assert run_block(P, lay, x, d, g)[0] == -1
+
+
+def window_axis_records(N, D, kinds):
+    """unet_set_attn_axis records (window voxels, the axis along window z) and the same axes at the bottleneck of a two-level net (F = 2 window planes
+    per grid plane; a voxel centre c of the window is (c + 0.5) / F - 0.5 on the grid): kind 0 inside the window, 1 outside, 2 none"""
+    np_ = D; rec = np.zeros((N, 4 + 2 * np_), np.float32); F = 2; Dg = D // F; axr = np.zeros((N, ro.axr_len(Dg)), np.float32)
+    for b in range(N):
+        rec[b, :4] = (0, kinds[b] != 2, np_, 1)
+        for z in range(np_):
+            rec[b, 4 + 2 * z], rec[b, 5 + 2 * z] = (0.41 * D + 0.11 * z, 0.57 * D - 0.07 * z) if kinds[b] == 0 else (-3.2 - 0.05 * z, 1.3 * D + 0.04 * z)
+        axr[b, :2] = (0, kinds[b] != 2)
+        c = rec[b, 4:].astype(np.float64).reshape(Dg, F, 2).mean(1)
+        axr[b, 2:] = ((c + 0.5) / F - 0.5).reshape(-1)
+    return rec, axr
+
+
+@pytest.mark.parametrize("radial", [1, 0])
+def test_unet_attention_stage_on_the_scroll_geometry(gpu, tmp_path, radial):
+    """cfg.attn_axis 1 (radial attention) and cfg.attn_pe 3 (scroll RoPE) in the graph: the axis records of unet_set_attn_axis reach the stage at the
+    bottleneck's resolution, the stage's output follows the double-precision blocks on that geometry, no records = rays along the grid rows /
+    grid-index coordinates, and the checkpoint header carries the two fields (src/unet.h:77-83, src/unet.c:2732-2782, :5570)."""
+    import orc
+    import unet_ref
+    from gpuutil import to_mx
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    rng = np.random.default_rng(50 + radial)
+    N, D = 2, 16; widths = [32, 96]; cin, head_out, nblk = 4, 2, 2; nreg = 0 if radial else 2
+    S = D ** 3; Cb = widths[-1]; Hh = Cb // 48; F = (8 * Cb // 3 + 31) // 32 * 32; Dg = D // 2; Sg = Dg ** 3
+    x = rng.standard_normal((N, cin, S)).astype(np.float32); dxq = to_mx(8, x)
+    kw = dict(head_out=head_out, attn_blocks=nblk, attn_reg=nreg)
+    net = UNet(make_cfg(cin, widths, attn_pe=3, attn_axis=radial, **kw), N, D, D, D, seed=7)
+    plain = UNet(make_cfg(cin, widths, attn_pe=2, **kw), N, D, D, D, seed=7)
+    pp = net.params()
+    assert pp.size == plain.params().size                                          # neither field has parameters of its own
+    n_conv = unet_ref.param_layout(cin, widths, head_out)[1]
+    lays = []; o = n_conv + nreg * Cb
+    for _ in range(nblk):
+        bl, o = orc.block_layout(Cb, F, o); lays.append(bl)
+    assert o == pp.size
+    for lay in lays:
+        for k, n in (("wo", Cb * Cb), ("w2", Cb * F), ("bo", Cb), ("b1", 2 * F), ("bqkv", 3 * Cb)):
+            pp[lay[k]:lay[k] + n] = 0.05 * rng.standard_normal(n)
+    net.set_params(pp)
+    H0 = load_host()
+
+    def run(rec):
+        if rec is None:
+            H0.unet_set_attn_axis(net.h, None, 0, 0)
+        else:
+            H0.unet_set_attn_axis(net.h, rec.ctypes.data, rec.shape[0], rec.shape[1])
+        d = DevBuf(N * head_out * S * 4)
+        assert net.forward_x(dxq.ptr, d.ptr) == 0
+        LP.check()
+        outs = {name: (ptr, shp) for name, ptr, shp in net.layer_outs()}
+
+        def fetch(name):
+            ptr, shp = outs[name]; nb = lib.lp_mx8_bytes(shp[0], shp[1], Sg)
+            buf = np.empty(nb, np.uint8); lib.mi_d2h(buf.ctypes.data, ptr, nb)
+            return orc.mx_to_f32(8, buf, N, Cb, Sg)
+        return d.to_numpy(np.float32, (N, head_out, S)), fetch("enc1.c2"), fetch("attn")
+
+    def stage(xb, axr):
+        tok = np.zeros((N, Sg + nreg, Cb), np.float32)
+        reg = np.ascontiguousarray(pp[n_conv:n_conv + nreg * Cb].reshape(nreg, Cb)) if nreg else np.zeros((1, Cb), np.float32)
+        orc.lib().orc_cs_to_tok(orc.ptr(xb), orc.ptr(tok), orc.ptr(reg), N, Cb, Sg, nreg)
+        t = tok.reshape(N * (Sg + nreg), Cb).astype(np.float64)
+        R = ro.make_rays(N, Dg, Dg, Dg, 2.0, axr)
+        geo = dict(rays=R) if radial else dict(pos=ro.scroll_pos(N, nreg, Dg, Dg, Dg, R["ad"], R["cen"]), nreg=nreg)
+        for lay in lays:
+            t = ro.block(pp, lay, t, N, Sg + nreg, Hh, Cb, F, rope_mode=2, **geo)
+        t = np.ascontiguousarray(t, np.float32); want = np.zeros_like(xb)
+        orc.lib().orc_tok_to_cs(orc.ptr(t), orc.ptr(want), N, Cb, Sg, nreg)
+        return orc.mx_to_f32(8, orc.f32_to_mx(8, want, N, Cb, Sg), N, Cb, Sg)      # (the stage's output is stored as MX-fp8)
+
+    rec, axr = window_axis_records(N, D, (0, 1))
+    _, axr_none = window_axis_records(N, D, (2, 2))
+    lg, xb, got = run(rec)
+    want, other = stage(xb, axr), stage(xb, axr_none)
+    # two blocks of MX-fp8 linears against exact ones, then the MX-fp8 storage of the result; the reference's gate for an MX block is 0.1
+    # (measured 0.065: e4m3 storage of both results alone is 0.05; the other geometry is 7 x further away)
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 0.1
+    far = 3 if radial else 1.2                                                     # (rotations by other coordinates change the stage less than other rays do: 1.36 x measured)
+    assert np.linalg.norm(got - other) > far * np.linalg.norm(got - want)          # the axis is what the stage used
+    lg0, xb0, got0 = run(None)                                                      # no records: the grid rows / the grid indices
+    assert np.array_equal(xb0, xb) and not np.array_equal(got0, got)
+    assert np.linalg.norm(got0 - other) / np.linalg.norm(other) < 0.1 and np.linalg.norm(got0 - want) > far * np.linalg.norm(got0 - other)
+    bad = rec.copy(); bad[:, 2] = D // 2                                            # records of another plane count do not describe this grid: no axis
+    assert np.array_equal(run(bad[:, :4 + D])[2], got0)
+    assert np.array_equal(run(rec)[0], lg)                                          # and the records again: the first result, bit for bit
+    q, nr, cov = C.c_int(), C.c_int(), C.c_double()
+    if radial:
+        assert H0.unet_attn_rays(net.h, C.byref(q), C.byref(nr), C.byref(cov)) == 0
+        assert (q.value, nr.value) == ro.rays_dims(Dg, Dg, Dg, 2.0)[::2] and 0.8 < cov.value <= 1
+    else:
+        assert H0.unet_attn_rays(net.h, C.byref(q), C.byref(nr), C.byref(cov)) == -1
+    path = str(tmp_path / "scroll.ckpt")
+    assert net.save(path, step=4, extra="{}") == 0
+    head = open(path, "rb").readline()
+    assert b'"attn_pe":3,' in head and (b',"attn_axis":1' in head) == bool(radial)
+    c2 = type(net.cfg)(); st = C.c_int()
+    assert H0.unet_peek(path.encode(), C.byref(c2), C.byref(st)) == 0 and (c2.attn_pe, c2.attn_axis, st.value) == (3, radial, 4)
+    twin = UNet(make_cfg(cin, widths, attn_pe=3, attn_axis=radial, **kw), N, D, D, D, seed=1)
+    assert twin.load(path) == 4
+    H0.unet_set_attn_axis(twin.h, rec.ctypes.data, N, rec.shape[1])
+    d = DevBuf(N * head_out * S * 4)
+    assert twin.forward_x(dxq.ptr, d.ptr) == 0
+    assert np.array_equal(d.to_numpy(np.float32, (N, head_out, S)), lg)
+    assert plain.load(path) == -1                                                   # another positional encoding: another function
+    net.close(); plain.close(); twin.close()
+
+
+@pytest.mark.parametrize("radial", [1, 0])
+def test_predict_volume_hands_every_window_its_axis(gpu, radial):
+    """The sliding-window driver gives a net whose attention stage reads the scroll axis each window's record (pred_axis, src/predict.c:1128-1141):
+    windows run alone on a one-window graph with the record written by hand give the bytes of their region; a prediction does not depend on the
+    windows per forward (the ray sums are order-independent); and with another axis the prediction is another."""
+    from ufsm_amd.unet import UNet, make_cfg, load_host
+    rng = np.random.default_rng(9)
+    W, halo = 32, 8; S = W - 2 * halo
+    dims = (40, 32, 24)
+    z, y, x = np.meshgrid(np.arange(dims[0]), np.arange(dims[1]), np.arange(dims[2]), indexing="ij")
+    vol = np.clip(70 + 0.6 * z + 0.7 * y + 35 * np.sin(0.25 * x + 0.3 * y) * np.cos(0.2 * z) + rng.integers(0, 16, dims), 0, 255).astype(np.uint8)
+    dv = DevBuf.from_numpy(vol)
+    import orc
+    import unet_ref
+    nreg = 0 if radial else 2
+    kw = dict(G=8, head_out=1, act_dt=8, attn_blocks=2, attn_pe=3, attn_axis=radial, attn_reg=nreg)
+    args = (100.0, 1 / 50.0, 1, 11.5, 20.25)                                     # mean, 1 / sd, axis on, the axis at (y, x) = (11.5, 20.25): inside some windows, outside others
+    outs = {}
+    for nb in (1, 5):
+        net = UNet(make_cfg(4, [16, 96], **kw), nb, W, W, W, seed=5)
+        q = net.params(); r2 = np.random.default_rng(1)
+        o = unet_ref.param_layout(4, [16, 96], 1)[1] + nreg * 96                  # (the zero-initialised out projections made trained-like: the stage acts)
+        for _ in range(2):
+            lay, o = orc.block_layout(96, 256, o)
+            for k, n in (("wo", 96 * 96), ("w2", 96 * 256), ("bo", 96), ("b1", 512), ("bqkv", 288)):
+                q[lay[k]:lay[k] + n] = 0.05 * r2.standard_normal(n)
+        assert o == q.size
+        net.set_params(q)
+        dout = DevBuf(vol.size)
+        rc, nw, ndone = net.predict_volume(dv.ptr, dims, halo, 0, *args, dout.ptr)
+        assert rc == 0 and nw == 12 and ndone == 12
+        outs[nb] = dout.to_numpy(np.uint8, dims)
+        if nb == 5:
+            rc, _, _ = net.predict_volume(dv.ptr, dims, halo, 0, args[0], args[1], 1, 300.0, -200.0, dout.ptr)
+            assert rc == 0
+            outs["far"] = dout.to_numpy(np.uint8, dims)
+        net.close()
+    assert outs[1].std() > 0 and np.array_equal(outs[1], outs[5])
+    assert not np.array_equal(outs[5], outs["far"])
+    one = UNet(make_cfg(4, [16, 96], **kw), 1, W, W, W, seed=2); one.set_params(q)
+    H0 = load_host()
+    dlg = DevBuf(W ** 3 * 4); dw = DevBuf(W ** 3); dE = DevBuf(S ** 3)
+    for a, b, c in ((0, 0, 0), (1, 1, 1), (2, 0, 1)):
+        o = (a * S - halo, b * S - halo, c * S - halo)
+        lib.mi_ct_window(dv.ptr, dims[0], dims[1], dims[2], o[0], o[1], o[2], W, dw.ptr, 1, halo, None)
+        off = DevBuf.from_numpy(np.concatenate([np.full(W, o[1] - args[3], np.float32), np.full(W, o[2] - args[4], np.float32)]))
+        rec = np.zeros(4 + 2 * W, np.float32); rec[:4] = (0, 1, W, 1); rec[4::2] = args[3] - o[1]; rec[5::2] = args[4] - o[2]
+        H0.unet_set_attn_axis(one.h, rec.ctypes.data, 1, rec.size)
+        assert one.forward_ct(dw.ptr, args[0], args[1], off.ptr, off.ptr + 4 * W, args[2], dlg.ptr) == 0
+        lib.mi_zero(dE.ptr, S ** 3)
+        lib.nn_pred_place(dlg.ptr, dw.ptr, W, halo, -halo, -halo, -halo, S, S, S, S, dE.ptr)
+        LP.check()
+        E = dE.to_numpy(np.uint8, (S, S, S))
+        reg = outs[1][a * S:(a + 1) * S, b * S:(b + 1) * S, c * S:(c + 1) * S]
+        assert np.array_equal(E[:reg.shape[0], :reg.shape[1], :reg.shape[2]], reg), (a, b, c)
+    one.close()

@@ -143,20 +143,26 @@ __global__ void __launch_bounds__(256) ray_pos_k(const float *__restrict__ ray, 
     const float *rr = ray + (s / Nr) * AT_RAY_F;
     pos[3 * s] = rr[4] + (float)(s % Nr); pos[3 * s + 1] = rr[5]; pos[3 * s + 2] = rr[7];
 }
-__global__ void __launch_bounds__(256) ray_zero_k(float *__restrict__ p, size_t n) {
+// Sums that several ray slots add into one grid token go through 64-bit fixed-point integers (units of 2^-32): integer atomic adds commute, so
+// the result does not depend on the order in which the slots arrive and a forward gives the same bits every time it runs (floating-point
+// atomics, which the reference uses, do not). Weights lie in [0, 1] and attention outputs are convex combinations of value rows, far inside
+// the +-2^31 range; what is below 2^-33 in magnitude is dropped.
+__device__ __forceinline__ void fx_add(long long *acc, float v) { atomicAdd((unsigned long long *)acc, (unsigned long long)__float2ll_rn(v * 4294967296.f)); }
+__device__ __forceinline__ float fx_get(long long a) { return (float)((double)a * (1.0 / 4294967296.0)); }
+__global__ void __launch_bounds__(256) ray_zero64_k(long long *__restrict__ p, size_t n) {
     const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
-    if (i < n) p[i] = 0.f;
+    if (i < n) p[i] = 0;
 }
-__global__ void __launch_bounds__(256) ray_wsum_k(ray_geo G, const float *__restrict__ ray, const int *__restrict__ ad, long long n, float *acc) {
+__global__ void __launch_bounds__(256) ray_wsum_k(ray_geo G, const float *__restrict__ ray, const int *__restrict__ ad, long long n, long long *acc) {
     const long long s = blockIdx.x * 256ll + threadIdx.x;
     if (s >= n) return;
     long long row[4]; float w[4];
     const int nc = slot_stencil(G, ray, ad, s, row, w);
-    for (int c = 0; c < nc; c++) if (w[c] != 0.f) unsafeAtomicAdd(acc + row[c], w[c]);
+    for (int c = 0; c < nc; c++) if (w[c] != 0.f) fx_add(acc + row[c], w[c]);
 }
-__global__ void __launch_bounds__(256) ray_winv_k(float *acc, long long n) {
+__global__ void __launch_bounds__(256) ray_winv_k(const long long *__restrict__ acc, float *__restrict__ winv, long long n) {
     const long long i = blockIdx.x * 256ll + threadIdx.x;
-    if (i < n) { const float a = acc[i]; acc[i] = a > 1e-6f ? 1.f / a : 0.f; }
+    if (i < n) { const float a = fx_get(acc[i]); winv[i] = a > 1e-6f ? 1.f / a : 0.f; }
 }
 // grid rows -> ray rows: a thread forms four neighbouring channels of one slot. NORM: each corner's weight times the token's 1 / weight sum
 template <bool NORM>
@@ -176,10 +182,10 @@ __global__ void __launch_bounds__(256) ray_gather_k(ray_geo G, const float *__re
     }
     y[i] = a;
 }
-// ray rows -> grid rows (zeroed before): the adjoint, floating-point atomic adds (their order, so the last bits of a sum, is not fixed)
-template <bool NORM>
-__global__ void __launch_bounds__(256) ray_scatter_k(ray_geo G, const float *__restrict__ ray, const int *__restrict__ ad, const float *__restrict__ wsum,
-                                                     long long n, int C4, const float4 *__restrict__ y, float *x) {
+// ray rows -> grid rows: the adjoint. The slots' contributions w y meet in the fixed-point sums (zeroed before); a second kernel turns a token's
+// sum into its fp32 row, times the token's 1 / weight sum in the normalised form (the reference scales every contribution instead: the same
+// number up to rounding)
+__global__ void __launch_bounds__(256) ray_scatter_k(ray_geo G, const float *__restrict__ ray, const int *__restrict__ ad, long long n, int C4, const float4 *__restrict__ y, long long *acc) {
     const long long i = blockIdx.x * 256ll + threadIdx.x;
     if (i >= n * C4) return;
     const long long s = i / C4; const int c4 = (int)(i - s * C4);
@@ -188,11 +194,18 @@ __global__ void __launch_bounds__(256) ray_scatter_k(ray_geo G, const float *__r
     if (!nc) return;
     const float4 v = y[i];
     for (int c = 0; c < nc; c++) {
-        const float wc = NORM ? w[c] * wsum[row[c]] : w[c];
-        if (wc == 0.f) continue;
-        float *d = x + (row[c] * C4 + c4) * 4;
-        unsafeAtomicAdd(d, wc * v.x); unsafeAtomicAdd(d + 1, wc * v.y); unsafeAtomicAdd(d + 2, wc * v.z); unsafeAtomicAdd(d + 3, wc * v.w);
+        if (w[c] == 0.f) continue;
+        long long *d = acc + (row[c] * C4 + c4) * 4;
+        fx_add(d, w[c] * v.x); fx_add(d + 1, w[c] * v.y); fx_add(d + 2, w[c] * v.z); fx_add(d + 3, w[c] * v.w);
     }
+}
+template <bool NORM>
+__global__ void __launch_bounds__(256) ray_scatter_out_k(const long long *__restrict__ acc, const float *__restrict__ wsum, size_t n4, int C4, float4 *__restrict__ x) {
+    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
+    if (i >= n4) return;
+    const long long *a = acc + i * 4;
+    const float s = NORM ? wsum[i / C4] : 1.f;
+    x[i] = make_float4(fx_get(a[0]) * s, fx_get(a[1]) * s, fx_get(a[2]) * s, fx_get(a[3]) * s);
 }
 // the grid tokens' scroll coordinates (src/nn_attn_ray.cu:174-188): (r, arc, k) around the plane's centre, the angle unwrapped around the
 // plane's reference angle; registers (0, 0, 0); without an axis (cen's radius < 0) the grid indices (v, u, k)
@@ -284,9 +297,10 @@ extern "C" void at_rays_setup(const at_rays *R) {
     const ray_geo G = geo_of(R); const long long Tr = (long long)R->n * R->Q * R->Nr, Tg = (long long)R->n * G.Sg;
     if (!Tr) return;
     ray_pos_k<<<nblk_((size_t)Tr, 256), 256>>>(R->ray, R->Nr, Tr, (float *)R->pos);
-    ray_zero_k<<<nblk_((size_t)Tg, 256), 256>>>((float *)R->wsum, (size_t)Tg);       // (a fill kernel, not a memset: the sequence may be captured)
-    ray_wsum_k<<<nblk_((size_t)Tr, 256), 256>>>(G, R->ray, R->ad, Tr, (float *)R->wsum);
-    ray_winv_k<<<nblk_((size_t)Tg, 256), 256>>>((float *)R->wsum, Tg);
+    long long *acc = (long long *)mi_ws(MI_WS_RAY, (size_t)Tg * sizeof(long long));
+    ray_zero64_k<<<nblk_((size_t)Tg, 256), 256>>>(acc, (size_t)Tg);                   // (a fill kernel, not a memset: the sequence may be captured)
+    ray_wsum_k<<<nblk_((size_t)Tr, 256), 256>>>(G, R->ray, R->ad, Tr, acc);
+    ray_winv_k<<<nblk_((size_t)Tg, 256), 256>>>(acc, (float *)R->wsum, Tg);
     MICK();
 }
 extern "C" void at_ray_gather(const at_rays *R, const float *x, float *y, int Cc, int norm) {
@@ -304,9 +318,11 @@ extern "C" void at_ray_scatter(const at_rays *R, const float *y, float *x, int C
     const ray_geo G = geo_of(R); const long long Tr = (long long)R->n * R->Q * R->Nr; const int C4 = Cc / 4;
     const size_t ng = (size_t)R->n * G.Sg * Cc;
     if (!ng) return;
-    ray_zero_k<<<nblk_(ng, 256), 256>>>(x, ng);
-    if (norm) ray_scatter_k<true><<<nblk_((size_t)Tr * C4, 256), 256>>>(G, R->ray, R->ad, R->wsum, Tr, C4, (const float4 *)y, x);
-    else ray_scatter_k<false><<<nblk_((size_t)Tr * C4, 256), 256>>>(G, R->ray, R->ad, R->wsum, Tr, C4, (const float4 *)y, x);
+    long long *acc = (long long *)mi_ws(MI_WS_RAY, ng * sizeof(long long));
+    ray_zero64_k<<<nblk_(ng, 256), 256>>>(acc, ng);
+    ray_scatter_k<<<nblk_((size_t)Tr * C4, 256), 256>>>(G, R->ray, R->ad, Tr, C4, (const float4 *)y, acc);
+    if (norm) ray_scatter_out_k<true><<<nblk_(ng / 4, 256), 256>>>(acc, R->wsum, ng / 4, C4, (float4 *)x);
+    else ray_scatter_out_k<false><<<nblk_(ng / 4, 256), 256>>>(acc, R->wsum, ng / 4, C4, (float4 *)x);
     MICK();
 }
 extern "C" void at_scroll_pos(int n, int nreg, int D, int Hh, int W, const int *ad, const float *cen, float *pos) {

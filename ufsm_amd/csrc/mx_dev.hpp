@@ -287,7 +287,7 @@ void *mi_ws(int slot, size_t bytes);        // per-device grow-on-demand scratch
 void mi_ws_arena(void *base, size_t cap);   // the calling thread's scratch requests come from this fixed region until mi_ws_arena(nullptr, 0)
 bool mi_ws_arena_on(void);
 void mi_count_alloc(void);                  // bookkeeping: one more device allocation made by the library
-enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_UPCOARSE = 5, MI_WS_GEMM = 6, MI_WS_ATTN = 7, MI_WS_GEMM2 = 8, MI_WS_NSLOTS = 9 };
+enum { MI_WS_WQ = 0, MI_WS_WSC = 1, MI_WS_XSTAGE = 2, MI_WS_X2STAGE = 3, MI_WS_MISC = 4, MI_WS_UPCOARSE = 5, MI_WS_GEMM = 6, MI_WS_ATTN = 7, MI_WS_GEMM2 = 8, MI_WS_RAY = 9, MI_WS_NSLOTS = 10 };
 static inline unsigned nblk_(size_t n, unsigned b) { return (unsigned)((n + b - 1) / b); }
 [[noreturn]] void mi_die(const char *fmt, ...);
 // ---- slab-local GroupNorm statistics (gnp_t.ns > 0: src/nn_lp.h:15-18, src/lp_slab.cuh:7-12): the statistics hold one row per (sample,

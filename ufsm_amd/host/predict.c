@@ -44,7 +44,12 @@ int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, 
     /* Pass 2: the windows that hold material, in z-y-x order, in.n per forward (window j of a batch -> sample j; samples are independent, so a
      * window's prediction does not depend on its batch; a last, incomplete batch repeats its last window and places it once) */
     int64_t *list = malloc((size_t)(total ? total : 1) * sizeof(int64_t)), np = 0;
-    if (!list) rc = -1;
+    /* a net whose attention stage reads the scroll axis (cfg.attn_axis radial / attn_pe scroll) gets every forward's windows' axis records:
+     * the axis along window z, its centre per window plane = the negated row / column offsets (pred_axis, src/predict.c:1128-1141) */
+    const unet_cfg *cf = unet_cfg_of(u);
+    const int wants_axis = cf->attn_blocks > 0 && (cf->attn_axis == 1 || cf->attn_pe == 3);
+    float *axrec = wants_axis ? malloc((size_t)64 * UNET_AXR(W) * sizeof(float)) : NULL;
+    if (!list || (wants_axis && !axrec)) rc = -1;
     for (int64_t id = 0; id < total && !rc; id++) if (hany[id]) list[np++] = id;
     /* the windows are spread evenly over the forwards that nbatch windows per forward need: 726 windows at up to 64 per forward are 12 forwards
      * of 61 (6 samples repeat a window), not 11 of 64 and one of 22 padded to 64. The graph is (re)built for that sample count by the first forward */
@@ -58,6 +63,14 @@ int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, 
             eoff[j] = id * (int64_t)e3;
             cts[j] = ctw + (size_t)j * w3; dyos[j] = doff + (size_t)id * 2 * W; dxos[j] = dyos[j] + W;
         }
+        if (wants_axis) {
+            for (int j = 0; j < in.n; j++) {
+                float *r = axrec + (size_t)j * UNET_AXR(W);
+                r[0] = 0.f; r[1] = axis ? 1.f : 0.f; r[2] = (float)W; r[3] = 1.f;
+                for (int z = 0; z < W; z++) { r[4 + 2 * z] = cy - (float)org[3 * j + 1]; r[5 + 2 * z] = cx - (float)org[3 * j + 2]; }
+            }
+            unet_set_attn_axis(u, axrec, in.n, UNET_AXR(W));
+        }
         mi_ct_windows(vol, dims[0], dims[1], dims[2], org, in.n, W, ctw, iso, halo, NULL);
         const float *lg = mi_unet_forward_ct_n(u, cts, mean, isd, dyos, dxos, axis, in, 2);      /* (fp16-rounded input values, as predict) */
         if (!lg) { rc = -1; break; }
@@ -65,7 +78,7 @@ int mi_unet_predict_volume(unet *u, int window, int nbatch, const uint8_t *vol, 
         mi_pred_place_n(lg, lgn, ctw, w3, nreal, eoff, W, W, halo - B, halo - B, -halo, -halo, -halo, En, En, En, En, E);
         for (int j = 0; j < nreal; j++) { present[list[k + j]] = 1; done++; }
     }
-    free(list);
+    free(list); free(axrec);
     if (!rc) {
         mi_h2d(dpres, present, (size_t)total);
         rc = mi_feather_blend(E, dpres, S, B, nss, dims, out);

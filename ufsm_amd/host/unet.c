@@ -57,6 +57,10 @@ struct unet {
     size_t peg_w, peg_b;                                           /* cfg.attn_pe 0: the conv positional encoding's parameters */
     float *tb_vr; size_t vr_off;                                   /* cfg.attn_vres (src/unet.h:81): the first application's V rows; the lerps' offset */
     float *tb_cs, *tb_tok; void *tb_ws;                            /* fp32 planes [n][C][Sg]; token rows, one buffer per block + 1; block scratch */
+    /* cfg.attn_axis 1 / attn_pe 3: the scroll geometry (src/unet.c:280-282). One device buffer tb_rb holds the ray table, lengths, axis dims, ray
+       positions, stencil weight sums, the grid tokens' scroll coordinates and the per-plane frames; the host side of a plan; the axis records */
+    at_rays tbr; float *tb_rb, *tb_gpos, *tb_cen, *tb_rayh, *tb_cenh, *tb_axb, *tb_axh; int *tb_lensh, *tb_adh;
+    int tb_Q, tb_Nt, tb_Nr, tb_axn, tb_axs, tb_axdirty, tb_axwarn, tb_noax;
 };
 
 /* activation storage of the nets built from now on (src/unet.c:700-706): MX-fp8 unless MX-fp4 is asked for */
@@ -76,6 +80,17 @@ static void *act_new(const unet *u, shape5 s) { const size_t b = act_bytes(u, s)
 static void act_del(void *p) { if (p) { nn_storage_forget(p); mi_free(p); } }
 static float *f32_new(size_t n) { float *p = mi_malloc(n * 4); mi_zero(p, n * 4); return p; }
 
+/* the attention stage reads the scroll axis (unet_cfg_axis, src/unet.h): radial attention or the scroll rotary embedding */
+static int cfg_axis(const unet_cfg *c) { return c->attn_blocks > 0 && (c->attn_axis == 1 || c->attn_pe == 3); }
+/* radial attention: rays per axis-normal plane / the grid's largest dim (the reference's environment knob UFSM_ATTN_RAY_MULT, default 2; src/unet.c:692-694) */
+static float attn_ray_mult(void) { static float m = 0; if (m <= 0) { const char *e = getenv("UFSM_ATTN_RAY_MULT"); m = e && atof(e) > 0 ? (float)atof(e) : 2.f; } return m; }
+static void tb_geom_free(unet *u) {
+    if (u->tb_rb) mi_free(u->tb_rb);
+    free(u->tb_rayh); free(u->tb_cenh); free(u->tb_lensh); free(u->tb_adh); free(u->tb_axb);
+    u->tb_rb = u->tb_gpos = u->tb_cen = u->tb_rayh = u->tb_cenh = u->tb_axb = nullptr; u->tb_lensh = u->tb_adh = nullptr;
+    u->tbr = (at_rays){0}; u->tbg.rays = nullptr; u->tbg.pos = nullptr;
+}
+
 /* a field of the reference's configuration this build's graph does not run: named, so the caller knows which */
 static const char *cfg_unsupported(const unet_cfg *c) {
     for (int i = 0; i < UNET_MAXLEV; i++) {
@@ -93,7 +108,7 @@ static const char *cfg_unsupported(const unet_cfg *c) {
     if (c->gfilm && (!c->attn_blocks || c->nlev < 2)) return "gfilm without the attention stage (src/unet.c:517)";
     if (c->gn_ema && c->l0_norm) return "gn_ema with l0_norm (src/unet.c:551)";
     if (c->attn_vres && !c->attn_blocks) return "attn_vres without attention blocks";
-    if (c->attn_axis) return "attn_axis";
+    if (c->attn_axis < 0 || c->attn_axis > 1 || (c->attn_axis && (!c->attn_blocks || c->attn_reg))) return "attn_axis (0 or 1; radial attention takes no register tokens, src/unet.c:471-472)";
     if (c->attn_repeat < 0 || (c->attn_repeat > 1 && (!c->attn_blocks || c->attn_blocks * c->attn_repeat > 64))) return "attn_repeat";
     if (c->attn_mem) return "attn_mem";
     if (c->view_P || c->view_patch) return "view_P";
@@ -163,12 +178,12 @@ unet *unet_create(const unet_cfg *cfg) {
     for (int j = 1; j <= cfg->ds_levels; j++) off = add_conv(&u->ds[j], dw_of(cfg, j), cfg->cout, 1, off);
     if (cfg->attn_blocks > 0) {                                   /* parameters last: registers, then the blocks (src/unet.c:490-499) */
         const int C = w[L - 1];
-        if (C % AT_HD || cfg->attn_blocks > 16 || cfg->attn_pe < 0 || cfg->attn_pe > 2 || cfg->attn_reg < 0) {
-            fprintf(stderr, "unet_create: attention blocks need a bottleneck width that is a multiple of %d (got %d), at most 16 blocks, attn_pe 0 (PEG), 1 (RoPE) or 2 (none)\n", AT_HD, C);
+        if (C % AT_HD || cfg->attn_blocks > 16 || cfg->attn_pe < 0 || cfg->attn_pe > 3 || cfg->attn_reg < 0) {
+            fprintf(stderr, "unet_create: attention blocks need a bottleneck width that is a multiple of %d (got %d), at most 16 blocks, attn_pe 0 (PEG), 1 (RoPE), 2 (none) or 3 (scroll RoPE)\n", AT_HD, C);
             free(u); return nullptr;
         }
         const int F = cfg->attn_mlp > 0 ? cfg->attn_mlp : (8 * C / 3 + 31) / 32 * 32;
-        u->tbd = (at_dims){.C = C, .H = C / AT_HD, .F = F, .rope = cfg->attn_pe == 1 ? 1 : 0, .nreg = cfg->attn_reg, .rope_base = 100.f};
+        u->tbd = (at_dims){.C = C, .H = C / AT_HD, .F = F, .rope = cfg->attn_pe == 1 ? 1 : cfg->attn_pe == 3 ? 2 : 0, .nreg = cfg->attn_reg, .rope_base = 100.f};
         if (cfg->attn_pe == 0) { u->peg_w = off; off += (size_t)C * 27; u->peg_b = off; off += (size_t)C; }      /* the conv positional encoding's depthwise taps and bias, before the registers (src/unet.c:491) */
         u->reg_off = off; off += (size_t)cfg->attn_reg * C;
         for (int k = 0; k < cfg->attn_blocks; k++) off = at_block_layout(&u->tbd, &u->tbp[k], off);
@@ -238,7 +253,7 @@ static void free_acts(unet *u) {
         act_del(u->downo[i]); act_del(u->skipst[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
         u->downo[i] = u->skipst[i] = nullptr; u->dm[i] = u->dr[i] = nullptr;
     }
-    if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); if (u->tb_vr) mi_free(u->tb_vr); u->tb_vr = nullptr; u->tb.a2 = nullptr; u->tb.m2 = u->tb.r2 = nullptr; u->tb_cs = u->tb_tok = nullptr; u->tb_ws = nullptr; }
+    if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); if (u->tb_vr) mi_free(u->tb_vr); u->tb_vr = nullptr; tb_geom_free(u); u->tb.a2 = nullptr; u->tb.m2 = u->tb.r2 = nullptr; u->tb_cs = u->tb_tok = nullptr; u->tb_ws = nullptr; }
     for (int i = 0; i < 2; i++) { act_del(u->slab_tmp[i]); act_del(u->slab_carry[i]); u->slab_tmp[i] = u->slab_carry[i] = nullptr; }
     act_del(u->xin); u->xin = nullptr;
     mi_free(u->logits); u->logits = nullptr;
@@ -303,7 +318,27 @@ static int build_acts(unet *u, shape5 in) {
         u->tb.m2 = f32_new(ng); u->tb.r2 = f32_new(ng);
         if (u->cfg.attn_vres) u->tb_vr = f32_new((size_t)T * C);
         u->tb_cs = f32_new((size_t)ys.n * C * Sg); u->tb_tok = f32_new((size_t)3 * T * C);     /* the stage's input rows and two buffers the applications alternate between */
-        u->tb_ws = mi_malloc(at_ws_bytes(&u->tbd, T)); at_ws_carve(&u->tbw, &u->tbd, T, u->tb_ws);
+        long Tr = 0;
+        if (cfg_axis(&u->cfg)) {                                  /* the scroll geometry's buffers; tb_geom fills them per forward (src/unet.c:1354-1375) */
+            at_rays_dims(ys.d, ys.h, ys.w, attn_ray_mult(), &u->tb_Q, &u->tb_Nt, &u->tb_Nr);
+            const int Pm = ys.d > ys.h ? (ys.d > ys.w ? ys.d : ys.w) : (ys.h > ys.w ? ys.h : ys.w);
+            Tr = u->cfg.attn_axis == 1 ? (long)ys.n * u->tb_Q * u->tb_Nr : 0;
+            const size_t nq = (size_t)ys.n * u->tb_Q, al = 64;
+#define UP(v) (((size_t)(v) + al - 1) / al * al)
+            const size_t o_ray = 0, o_len = o_ray + UP(nq * AT_RAY_F), o_ad = o_len + UP(nq), o_pos = o_ad + UP(ys.n), o_ws = o_pos + UP((size_t)Tr * 3),
+                         o_gp = o_ws + UP((size_t)ys.n * Sg), o_cen = o_gp + UP((size_t)T * 3), o_end = o_cen + UP((size_t)ys.n * Pm * 4);
+#undef UP
+            u->tb_rb = f32_new(o_end);
+            u->tbr = (at_rays){.n = ys.n, .Q = u->tb_Q, .Nt = u->tb_Nt, .Nr = u->tb_Nr, .D = ys.d, .Hh = ys.h, .W = ys.w, .ad = (const int *)(u->tb_rb + o_ad), .ray = u->tb_rb + o_ray,
+                               .lens = (const int *)(u->tb_rb + o_len), .pos = u->tb_rb + o_pos, .wsum = u->tb_rb + o_ws};
+            u->tb_gpos = u->tb_rb + o_gp; u->tb_cen = u->tb_rb + o_cen;
+            u->tb_rayh = malloc(nq * AT_RAY_F * sizeof(float)); u->tb_cenh = malloc((size_t)ys.n * Pm * 4 * sizeof(float));
+            u->tb_lensh = malloc(nq * sizeof(int)); u->tb_adh = malloc((size_t)ys.n * sizeof(int)); u->tb_axb = malloc((size_t)ys.n * AT_AXR(Pm) * sizeof(float));
+            if (!u->tb_rayh || !u->tb_cenh || !u->tb_lensh || !u->tb_adh || !u->tb_axb) { fprintf(stderr, "unet: no host memory for the ray plan\n"); abort(); }
+            u->tb_axdirty = 1;
+            if (u->cfg.attn_axis == 1) u->tbg.rays = &u->tbr; else u->tbg.pos = u->tb_gpos;
+        }
+        u->tb_ws = mi_malloc(at_ws_bytes_r(&u->tbd, T, Tr)); at_ws_carve_r(&u->tbw, &u->tbd, T, Tr, u->tb_ws);
     }
     u->built = 1;
     return 0;
@@ -320,6 +355,7 @@ void unet_free(unet *u) {
     mi_free(u->p); mi_free(u->ema); if (u->wm) mi_free(u->wm); if (u->l0run) mi_free(u->l0run); if (u->ge_run) mi_free(u->ge_run);
     for (int i = 0; i < UNET_MAXLEV; i++) { free(u->rb[i]); free(u->rbn[i]); }
     if (u->stem_b) mi_free(u->stem_b);
+    free(u->tb_axh);
     if (u->gf_g) { mi_free(u->gf_g); mi_free(u->gf_g1); }
     lp_wmemo_clear();
     free(u);
@@ -545,6 +581,68 @@ static int block_fwd(unet *u, block *b, int level, const void *x, const nn_gn_t 
     }
     return r;
 }
+/* replaces unet_set_attn_axis (src/unet.h:470-474, src/unet.c:2732-2737): the scroll axis of every sample of the following forwards, n records of
+   stride floats (UNET_AXR, host memory, copied); n 0 or a null pointer: no axis (rays along the grid rows, grid-index coordinates) */
+void unet_set_attn_axis(unet *u, const float *rec, int n, int stride) {
+    if (n <= 0 || stride < 4 || !rec) { u->tb_axn = 0; u->tb_axdirty = 1; return; }
+    if ((size_t)n * stride > (size_t)u->tb_axn * u->tb_axs || !u->tb_axh) {
+        free(u->tb_axh); u->tb_axh = malloc((size_t)n * stride * sizeof(float));
+        if (!u->tb_axh) { fprintf(stderr, "unet: no memory for axis records\n"); abort(); }
+    }
+    memcpy(u->tb_axh, rec, (size_t)n * stride * sizeof(float));
+    u->tb_axn = n; u->tb_axs = stride; u->tb_axdirty = 1;
+}
+/* the scroll geometry of this forward from the axis records (tb_geom, src/unet.c:2738-2782): each sample's window axis centres averaged over the
+   window planes of a bottleneck plane and expressed in bottleneck voxels, then the ray plan, its device tables and the ray positions and
+   stencil weight sums (radial attention) or the grid tokens' scroll coordinates (full attention). A record that does not describe this grid
+   (another plane count) or says "no axis" leaves its sample without one */
+static void tb_geom(unet *u) {
+    if (!u->tb_rb || !u->tb_axdirty) return;
+    const shape5 ys = u->tb.ys; const int n = ys.n, D = ys.d, Hh = ys.h, W = ys.w, Pm = D > Hh ? (D > W ? D : W) : (Hh > W ? Hh : W);
+    const int fp = 1 << (u->cfg.nlev - 1), have = u->tb_axh && u->tb_axn == n;
+    u->tb_noax = 0;
+    if (!have && !u->tb_axwarn) { fprintf(stderr, "unet: the attention stage has no scroll axis records for %d samples (unet_set_attn_axis): rays along the grid rows\n", n); u->tb_axwarn = 1; }
+    for (int b = 0; b < n; b++) {
+        float *o = u->tb_axb + (size_t)b * AT_AXR(Pm);
+        memset(o, 0, AT_AXR(Pm) * sizeof *o);
+        if (!have) continue;
+        const float *r = u->tb_axh + (size_t)b * u->tb_axs;
+        const int ad = (int)r[0], np = (int)r[2], div = (int)r[3] > 0 ? (int)r[3] : 1, F = div * fp;
+        if (ad < 0 || ad > 2) continue;
+        const int Np = ad == 0 ? D : ad == 1 ? Hh : W;
+        o[0] = (float)ad;
+        if (r[1] == 0.f || np != Np * F || u->tb_axs < UNET_AXR(np)) { u->tb_noax++; continue; }
+        o[1] = 1.f;
+        for (int k = 0; k < Np; k++) {
+            double su = 0, sv = 0;
+            for (int z = k * F; z < (k + 1) * F; z++) { su += r[4 + 2 * z]; sv += r[5 + 2 * z]; }
+            o[2 + 2 * k] = (float)((su / F + 0.5) / F - 0.5); o[3 + 2 * k] = (float)((sv / F + 0.5) / F - 0.5);      /* voxel centres at integers on both grids */
+        }
+    }
+    at_rays_plan(n, D, Hh, W, attn_ray_mult(), u->tb_axb, u->tb_rayh, u->tb_lensh, u->tb_adh, u->tb_cenh);
+    mi_h2d((void *)u->tbr.ray, u->tb_rayh, (size_t)n * u->tb_Q * AT_RAY_F * sizeof(float));
+    mi_h2d((void *)u->tbr.lens, u->tb_lensh, (size_t)n * u->tb_Q * sizeof(int));
+    mi_h2d((void *)u->tbr.ad, u->tb_adh, (size_t)n * sizeof(int));
+    mi_h2d(u->tb_cen, u->tb_cenh, (size_t)n * Pm * 4 * sizeof(float));
+    if (u->cfg.attn_axis == 1) at_rays_setup(&u->tbr);
+    else at_scroll_pos(n, u->tbd.nreg, D, Hh, W, u->tbr.ad, u->tb_cen, u->tb_gpos);
+    u->tb_axdirty = 0;
+}
+/* replaces unet_attn_rays (src/unet.c:2783-2796): the ray set's sizes and, when asked, the share of grid tokens a ray sample touches; -1 without
+   radial attention or before the first forward built the graph */
+int unet_attn_rays(const unet *u, int *Q, int *Nr, double *coverage) {
+    if (!u->tb_rb || u->cfg.attn_axis != 1) return -1;
+    if (Q) *Q = u->tb_Q;
+    if (Nr) *Nr = u->tb_Nr;
+    if (coverage) {
+        const size_t ng = (size_t)u->tbr.n * u->tbr.D * u->tbr.Hh * u->tbr.W; float *w = malloc(ng * sizeof *w); size_t c = 0;
+        if (!w) return -1;
+        mi_sync(); mi_d2h(w, u->tbr.wsum, ng * sizeof *w);
+        for (size_t i = 0; i < ng; i++) c += w[i] > 0.f;
+        *coverage = (double)c / (double)ng; free(w);
+    }
+    return 0;
+}
 /* the bottleneck's raw output -> fp32 planes -> token rows with the registers prepended -> blocks -> planes -> a new MX tensor with its
    GroupNorm statistics: the level's output for the decoder (src/unet.c:2795-2835; no PEG, memory, view or deformable paths) */
 static int tb_fwd(unet *u) {
@@ -552,6 +650,7 @@ static int tb_fwd(unet *u) {
     const shape5 ys = b->ys; const int C = u->tbd.C, nr = u->tbd.nreg; const size_t Sg = (size_t)ys.d * ys.h * ys.w, TC = (size_t)u->tbg.nseq * u->tbg.S * C;
     if (u->act_dt == 4) lp_mx4_to_f32(x->a2, ys.n, C, Sg, u->tb_cs); else lp_mx8_to_f32(x->a2, ys.n, C, Sg, u->tb_cs);
     at_cs_to_tok(u->tb_cs, u->tb_tok, P(u, u->reg_off), ys.n, C, (long)Sg, nr);
+    tb_geom(u);
     at_set_mx(8);
     lp_mx_gemm_bmemo(1);                                           /* inference: the linears' weights are packed once (dropped when the weights change) */
     const int tba = u->tbn * (u->cfg.attn_repeat > 1 ? u->cfg.attn_repeat : 1);      /* application k runs block k % tbn (cfg.attn_repeat, src/unet.c:2816) */
@@ -716,12 +815,13 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
     cfg->attn_blocks = key_int(line, "\"attn_blocks\":", 0); cfg->attn_pe = key_int(line, "\"attn_pe\":", 0);
     cfg->attn_reg = key_int(line, "\"attn_reg\":", 0); cfg->attn_mlp = key_int(line, "\"attn_mlp\":", 0);
     cfg->attn_repeat = key_int(line, "\"attn_repeat\":", 0); cfg->attn_vres = key_int(line, "\"attn_vres\":", 0);      /* (src/unet.c:5690) */
+    cfg->attn_axis = key_int(line, "\"attn_axis\":", 0);                                                                  /* (src/unet.c:5691) */
     cfg->half_res = key_int(line, "\"half_res\":", 0); cfg->scan_norm = key_int(line, "\"scan_norm\":", 0);      /* (the caller's business: the graph does not use them) */
     if (nparams) { const char *q = strstr(line, "\"nparams\":"); *nparams = q ? (size_t)strtoull(q + 10, nullptr, 10) : 0; }
     if (step) *step = key_int(line, "\"step\":", 0);
     /* architecture features this build's graph does not have */
     static const char *const no[] = {"\"lat_guide\":", "\"lat_sub\":", "\"lat_c\":",
-                                     "\"fstem\":", "\"lat_dec\":", "\"attn_axis\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
+                                     "\"fstem\":", "\"lat_dec\":", "\"attn_mem\":", "\"view_P\":", "\"attn_deform\":",
                                      "\"skip_empty\":"};
     const char *bad = nullptr;
     for (size_t k = 0; k < sizeof no / sizeof *no && !bad; k++) if (strstr(line, no[k])) bad = no[k];
@@ -742,7 +842,8 @@ static int read_header(const char *path, unet_cfg *cfg, size_t *nparams, int *st
        (unet_set_wq), src/unet.c:5703-5707, :5839-5840. Loading such a file as dense fp32 master weights would run another function */
     if (!bad && key_int(line, "\"sparse24\":", 0)) bad = "\"sparse24\": (2:4 sparse weights)";
     if (!bad && key_int(line, "\"wq\":", 0)) bad = "\"wq\": (packed fp8 / fp4 weight storage)";
-    if (!bad && cfg->attn_blocks && (cfg->attn_pe < 0 || cfg->attn_pe > 2)) bad = "\"attn_pe\": (scroll RoPE)";
+    if (!bad && cfg->attn_blocks && (cfg->attn_pe < 0 || cfg->attn_pe > 3)) bad = "\"attn_pe\":";
+    if (!bad && cfg->attn_blocks && (cfg->attn_axis < 0 || cfg->attn_axis > 1)) bad = "\"attn_axis\":";
     if (bad) { fprintf(stderr, "unet_peek: %s uses %s which this build does not run\n", path, bad); free(line); return -2; }
     free(line);
     return cfg->cin > 0 && cfg->cout > 0 ? 0 : -1;
@@ -859,6 +960,7 @@ int unet_save(const unet *u, const char *path, int step, const char *extra) {
     if (u->cfg.film) fprintf(f, ",\"film\":%d", u->cfg.film);     /* (src/unet.c:5564) */
     if (u->cfg.attn_blocks) fprintf(f, ",\"attn_blocks\":%d,\"attn_pe\":%d,\"attn_reg\":%d,\"attn_mlp\":%d", u->cfg.attn_blocks, u->cfg.attn_pe, u->cfg.attn_reg, u->tbd.F);
     if (u->cfg.attn_vres) fprintf(f, ",\"attn_vres\":%d", u->cfg.attn_vres);      /* (src/unet.c:5569) */
+    if (u->cfg.attn_blocks && u->cfg.attn_axis) fprintf(f, ",\"attn_axis\":%d", u->cfg.attn_axis);      /* (src/unet.c:5570) */
     if (u->cfg.attn_blocks && u->cfg.attn_repeat > 1) fprintf(f, ",\"attn_repeat\":%d", u->cfg.attn_repeat);      /* (src/unet.c:5571) */
     if (u->cfg.l0_norm) fprintf(f, ",\"l0_norm\":%d", u->cfg.l0_norm);
     if (u->cfg.l0_norm == 4) fprintf(f, ",\"l0_slab\":%d", u->cfg.l0_slab);

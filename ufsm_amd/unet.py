@@ -76,6 +76,8 @@ def load_host():
     L.unet_gn_ema_live.restype = None; L.unet_gn_ema_live.argtypes = [C.c_void_p, _I]
     L.unet_set_scale.restype = None; L.unet_set_scale.argtypes = [C.c_void_p, C.c_double]
     L.unet_set_cond.restype = None; L.unet_set_cond.argtypes = [C.c_void_p, C.c_float]
+    L.unet_set_attn_axis.restype = None; L.unet_set_attn_axis.argtypes = [C.c_void_p, C.c_void_p, _I, _I]
+    L.unet_attn_rays.restype = _I; L.unet_attn_rays.argtypes = [C.c_void_p, C.POINTER(_I), C.POINTER(_I), C.POINTER(C.c_double)]
     L.unet_set_film.restype = None; L.unet_set_film.argtypes = [C.c_void_p, C.POINTER(C.c_float), _I]
     L.unet_gfilm_off.restype = C.c_size_t; L.unet_gfilm_off.argtypes = [C.c_void_p]
     L.mi_unet_film_off.restype = C.c_size_t; L.mi_unet_film_off.argtypes = [C.c_void_p]
@@ -93,7 +95,7 @@ def load_host():
     return L
 
 
-def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, attn_repeat=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0, gn_ema=0, dec_widths=None, dec_convs=None, enc_blocks=None, ds_levels=0, emb_lev=0, emb_ch=0, scale_cond=0, film=0, gfilm=0, attn_vres=0):
+def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn_pe=2, attn_reg=0, attn_mlp=0, attn_repeat=0, down_norm=0, w4_2d=0, l0_norm=0, l0_slab=0, gn_ema=0, dec_widths=None, dec_convs=None, enc_blocks=None, ds_levels=0, emb_lev=0, emb_ch=0, scale_cond=0, film=0, gfilm=0, attn_vres=0, attn_axis=0):
     """The reference's configuration record plus, as Python attributes, what the reference keeps in process-wide switches: the activation
     storage (unet_set_act_mx4) and the compute precision policy (nn_set_prec), which UNet applies around its calls."""
     c = unet_cfg()
@@ -105,6 +107,7 @@ def make_cfg(cin, widths, G=8, head_out=8, act_dt=8, prec=0, attn_blocks=0, attn
     c.attn_repeat = attn_repeat if attn_blocks else 0
     c.ds_levels, c.emb_lev, c.emb_ch, c.scale_cond = ds_levels, emb_lev, emb_ch, scale_cond
     c.film, c.gfilm, c.attn_vres = film, gfilm, attn_vres
+    c.attn_axis = attn_axis if attn_blocks else 0
     for i, d in enumerate(dec_widths or []):
         c.dec_widths[i] = d
     for i, d in enumerate(dec_convs or []):
