@@ -269,11 +269,13 @@ def hbm_leg(np, lib, LP, DevBuf):
     return rows
 
 
-def sliding_leg(np, lib, LP, DevBuf, nbatch=64):
+def sliding_leg(np, lib, LP, DevBuf, nbatch=64, radial=False):
     """configs[4]: a 512 x 1024 x 1024 uint8 volume resident in HBM, 128^3 windows with 16 voxels of halo (stride 96), per window a U-Net of
     widths 32/64/128/192 with MX-fp4 weights over MX-fp8 activations (prec 3) and two transformer blocks (MX-fp8 attention core, MX-fp8
     linears, 4 heads of 48, axial RoPE, 4 register tokens) on the 16^3 = 4096 bottleneck tokens, one head channel, sigmoid -> uint8
-    placement and the 16-voxel feather blend of the window borders; end-to-end output voxels per second including gather, placement and blend."""
+    placement and the 16-voxel feather blend of the window borders; end-to-end output voxels per second including gather, placement and blend.
+    radial: the attention of the reference's production fine-tune instead (attn_axis 1, attn_pe 3: each block attends along the rays of the scroll
+    coordinates, rotary embedding on (r, arc, z), no register tokens; the driver plans every forward's rays from its windows' axis records)."""
     from ufsm_amd.unet import UNet, make_cfg
     dims, W, halo, B = (512, 1024, 1024), 128, 16, 16
     rng = np.random.default_rng(7)
@@ -282,7 +284,8 @@ def sliding_leg(np, lib, LP, DevBuf, nbatch=64):
     vol = (115 + 55 * np.sin(r * 0.35 + 0.02 * z)).astype(np.float32)
     vol += rng.integers(-20, 21, (1, dims[1], dims[2])).astype(np.float32) + rng.integers(-10, 11, (dims[0], 1, 1)).astype(np.float32)
     vol = np.clip(vol, 1, 255).astype(np.uint8)
-    net = UNet(make_cfg(4, [32, 64, 128, 192], G=8, head_out=1, act_dt=8, prec=3, attn_blocks=2, attn_pe=1, attn_reg=4), nbatch, W, W, W, seed=1)  # nbatch windows per forward
+    akw = dict(attn_pe=3, attn_axis=1, attn_reg=0) if radial else dict(attn_pe=1, attn_reg=4)
+    net = UNet(make_cfg(4, [32, 64, 128, 192], G=8, head_out=1, act_dt=8, prec=3, attn_blocks=2, **akw), nbatch, W, W, W, seed=1)  # nbatch windows per forward
     dv = DevBuf.from_numpy(vol); dout = DevBuf(vol.size, zero=False)
     small = (W, W, W)                                                                 # warm-up: one window (weights prepared, scratch grown)
     rc, _, _ = net.predict_volume(dv.ptr, small, halo, B, 115.0, 1 / 40.0, 1, 400.0, -300.0, dout.ptr)
@@ -303,7 +306,7 @@ def sliding_leg(np, lib, LP, DevBuf, nbatch=64):
     head = dout.to_numpy(np.uint8)[:1 << 20]
     net.close()
     nvox = float(dims[0]) * dims[1] * dims[2]
-    return {"workload": "configs[4]: 512x1024x1024 uint8 in HBM, 128^3 windows, halo 16, feather 16, U-Net 32/64/128/192, MX-fp4 weights over MX-fp8 activations, 2 attention blocks on 16^3 tokens (MX-fp8 core), up to %d windows per forward" % nbatch,
+    return {"workload": "configs[4]: 512x1024x1024 uint8 in HBM, 128^3 windows, halo 16, feather 16, U-Net 32/64/128/192, MX-fp4 weights over MX-fp8 activations, 2 attention blocks on 16^3 tokens (%s), up to %d windows per forward" % ("radial: 512 rays of 24 slots per window, fp16 core, scroll RoPE" if radial else "MX-fp8 core", nbatch),
             "value": nvox / dt, "unit": "voxels/s", "seconds": dt, "seconds_first_call": dt_first, "windows": int(nw), "windows_computed": int(ndone), "output_mean_first_mib": float(head.mean())}
 
 
@@ -319,6 +322,7 @@ def main():
     ap.add_argument("--no-hbm", action="store_true", help="skip the HBM-bound kernels leg")
     ap.add_argument("--no-single", action="store_true", help="skip the single-conv legs (configs[0], the MX-fp4 3x3x3 conv of configs[2])")
     ap.add_argument("--unet-only", action="store_true", help="the U-Net leg alone (what the rocprofv3 runs of the forward's kernels use)")
+    ap.add_argument("--sliding-radial", action="store_true", help="also run the sliding-window leg with radial attention and scroll RoPE (sub-record sliding_window_radial)")
     ap.add_argument("--windows-per-forward", type=int, default=64, help="sliding-window leg: the most windows batched into one forward (the driver evens them out over its forwards)")
     ap.add_argument("--copy-probe", action="store_true", help="run 5 device-to-device copies of 1 GiB and exit: the known-size kernel that scales "
                     "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
@@ -390,6 +394,8 @@ def main():
         out["c2a"] = c2a_leg(np, lib, LP, DevBuf, shape5, gnp_t, split_t, max(a.steps, 20) * 5, max(a.warmup, 5) * 2)
     if not a.no_sliding:
         out["sliding_window"] = sliding_leg(np, lib, LP, DevBuf, a.windows_per_forward)
+        if a.sliding_radial:
+            out["sliding_window_radial"] = sliding_leg(np, lib, LP, DevBuf, a.windows_per_forward, radial=True)
     if not a.no_hbm:
         out["hbm_kernels"] = hbm_leg(np, lib, LP, DevBuf)
     if not a.no_cpu_baseline:

@@ -81,9 +81,9 @@ void at_rays_plan(int n, int D, int Hh, int W, float mult, const float *axr, flo
 void at_rays_setup(const at_rays *R);
 /* replace at_ray_gather / at_ray_scatter (src/attn.h:111-113; src/nn_attn_ray.cu:145-173): grid rows x [n D Hh W][Cc] -> ray rows y [Tr][Cc]
    (norm: each corner's weight x wsum of its token, the adjoint of the normalised scatter), and ray rows -> grid rows (zeroed first; x wsum with
-   norm). Cc a multiple of 4, rows 16-byte aligned. The scatter's sums (and at_rays_setup's weight sums) are formed in 64-bit fixed point
-   (units of 2^-32, integer atomics): the same bits on every run, where the reference's floating-point atomics leave the last bits to the
-   order of arrival; their scratch (8 bytes per grid value) is the library's and grows on demand */
+   norm). Cc a multiple of 4, rows 16-byte aligned. The scatter (and at_rays_setup's weight sums) walk, per grid token, the list of ray samples
+   that touch it in (ray, sample) order: the same bits on every run, where the reference's floating-point atomics leave the last bits to
+   the order of arrival; the lists (5 Nt pairs per token) are library scratch that grows on demand */
 void at_ray_gather(const at_rays *R, const float *x, float *y, int Cc, int norm);
 void at_ray_scatter(const at_rays *R, const float *y, float *x, int Cc, int norm);
 /* replaces at_scroll_pos (src/attn.h:116; src/nn_attn_ray.cu:174-192): the scroll coordinates of the grid tokens for full attention with

@@ -143,26 +143,39 @@ __global__ void __launch_bounds__(256) ray_pos_k(const float *__restrict__ ray, 
     const float *rr = ray + (s / Nr) * AT_RAY_F;
     pos[3 * s] = rr[4] + (float)(s % Nr); pos[3 * s + 1] = rr[5]; pos[3 * s + 2] = rr[7];
 }
-// Sums that several ray slots add into one grid token go through 64-bit fixed-point integers (units of 2^-32): integer atomic adds commute, so
-// the result does not depend on the order in which the slots arrive and a forward gives the same bits every time it runs (floating-point
-// atomics, which the reference uses, do not). Weights lie in [0, 1] and attention outputs are convex combinations of value rows, far inside
-// the +-2^31 range; what is below 2^-33 in magnitude is dropped.
-__device__ __forceinline__ void fx_add(long long *acc, float v) { atomicAdd((unsigned long long *)acc, (unsigned long long)__float2ll_rn(v * 4294967296.f)); }
-__device__ __forceinline__ float fx_get(long long a) { return (float)((double)a * (1.0 / 4294967296.0)); }
-__global__ void __launch_bounds__(256) ray_zero64_k(long long *__restrict__ p, size_t n) {
-    const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
-    if (i < n) p[i] = 0;
-}
-__global__ void __launch_bounds__(256) ray_wsum_k(ray_geo G, const float *__restrict__ ray, const int *__restrict__ ad, long long n, long long *acc) {
-    const long long s = blockIdx.x * 256ll + threadIdx.x;
-    if (s >= n) return;
-    long long row[4]; float w[4];
-    const int nc = slot_stencil(G, ray, ad, s, row, w);
-    for (int c = 0; c < nc; c++) if (w[c] != 0.f) fx_add(acc + row[c], w[c]);
-}
-__global__ void __launch_bounds__(256) ray_winv_k(const long long *__restrict__ acc, float *__restrict__ winv, long long n) {
-    const long long i = blockIdx.x * 256ll + threadIdx.x;
-    if (i < n) { const float a = fx_get(acc[i]); winv[i] = a > 1e-6f ? 1.f / a : 0.f; }
+// The inverse of the slots' stencils, per grid token: which ray samples touch it and with what weight. A token of plane k can only be touched by
+// the rays of that plane (Nt of them), and on a ray only by the samples within 1.5 voxels of it in both plane coordinates (a sample's corners are
+// at most one voxel from its clamped position, clamping moves a sample by at most half a voxel): at most five consecutive samples around the
+// token's projection on the ray. Those candidates are run through the very stencil function the gather uses, so the two maps are exact
+// adjoints. A thread lists its token's (slot, weight) pairs in (ray, sample) order: sums over the list have a fixed order, so the scatter and
+// the weight sums give the same bits on every run (the reference adds with floating-point atomics in the order of arrival), and no atomics run.
+struct ray_ent { int slot; float w; };
+__global__ void __launch_bounds__(256) ray_inverse_k(ray_geo G, const float *__restrict__ ray, const int *__restrict__ ad, long long Tg, int Nt, int cap,
+                                                     ray_ent *__restrict__ tab, int *__restrict__ cnt, float *__restrict__ winv) {
+    const long long t = blockIdx.x * 256ll + threadIdx.x;
+    if (t >= Tg) return;
+    const int b = (int)(t / G.Sg); const long long ts = t - (long long)b * G.Sg;
+    const int z = (int)(ts / ((long long)G.Hh * G.W)), y = (int)(ts / G.W % G.Hh), x = (int)(ts % G.W), axd = ad[b];
+    const int k = axd == 0 ? z : axd == 1 ? y : x, ua = axd == 0 ? y : z, vb = axd == 2 ? y : x;
+    int n = 0; float sum = 0.f;
+    for (int j = 0; j < Nt; j++) {
+        const long long rq = (long long)b * G.Q + (long long)k * Nt + j;
+        const float *rr = ray + rq * AT_RAY_F;
+        const int L = min((int)rr[6], G.Nr);
+        if (L <= 0) continue;
+        const float ist = ((float)ua - rr[0]) * rr[2] + ((float)vb - rr[1]) * rr[3];      // the token's projection on the ray, in samples
+        const int i0 = max(0, (int)ceilf(ist - 2.2f)), i1 = min(L - 1, (int)floorf(ist + 2.2f));
+        for (int i = i0; i <= i1; i++) {
+            long long row[4]; float w[4];
+            const long long sl = rq * G.Nr + i;
+            const int nc = slot_stencil(G, ray, ad, sl, row, w);
+            float ws = 0.f;
+            for (int c = 0; c < nc; c++) if (row[c] == t) ws += w[c];
+            if (ws != 0.f && n < cap) { if (tab) tab[t * cap + n] = ray_ent{(int)sl, ws}; n++; sum += ws; }
+        }
+    }
+    if (cnt) cnt[t] = n;
+    if (winv) winv[t] = sum > 1e-6f ? 1.f / sum : 0.f;
 }
 // grid rows -> ray rows: a thread forms four neighbouring channels of one slot. NORM: each corner's weight times the token's 1 / weight sum
 template <bool NORM>
@@ -182,30 +195,22 @@ __global__ void __launch_bounds__(256) ray_gather_k(ray_geo G, const float *__re
     }
     y[i] = a;
 }
-// ray rows -> grid rows: the adjoint. The slots' contributions w y meet in the fixed-point sums (zeroed before); a second kernel turns a token's
-// sum into its fp32 row, times the token's 1 / weight sum in the normalised form (the reference scales every contribution instead: the same
-// number up to rounding)
-__global__ void __launch_bounds__(256) ray_scatter_k(ray_geo G, const float *__restrict__ ray, const int *__restrict__ ad, long long n, int C4, const float4 *__restrict__ y, long long *acc) {
-    const long long i = blockIdx.x * 256ll + threadIdx.x;
-    if (i >= n * C4) return;
-    const long long s = i / C4; const int c4 = (int)(i - s * C4);
-    long long row[4]; float w[4];
-    const int nc = slot_stencil(G, ray, ad, s, row, w);
-    if (!nc) return;
-    const float4 v = y[i];
-    for (int c = 0; c < nc; c++) {
-        if (w[c] == 0.f) continue;
-        long long *d = acc + (row[c] * C4 + c4) * 4;
-        fx_add(d, w[c] * v.x); fx_add(d + 1, w[c] * v.y); fx_add(d + 2, w[c] * v.z); fx_add(d + 3, w[c] * v.w);
-    }
-}
+// ray rows -> grid rows: the adjoint, in gather form over the token's list. NORM: each weight times the token's 1 / weight sum
 template <bool NORM>
-__global__ void __launch_bounds__(256) ray_scatter_out_k(const long long *__restrict__ acc, const float *__restrict__ wsum, size_t n4, int C4, float4 *__restrict__ x) {
+__global__ void __launch_bounds__(256) ray_scatter_k(const ray_ent *__restrict__ tab, const int *__restrict__ cnt, int cap, const float *__restrict__ wsum, size_t n4, int C4,
+                                                     const float4 *__restrict__ y, float4 *__restrict__ x) {
     const size_t i = blockIdx.x * (size_t)256 + threadIdx.x;
     if (i >= n4) return;
-    const long long *a = acc + i * 4;
-    const float s = NORM ? wsum[i / C4] : 1.f;
-    x[i] = make_float4(fx_get(a[0]) * s, fx_get(a[1]) * s, fx_get(a[2]) * s, fx_get(a[3]) * s);
+    const size_t t = i / C4; const int c4 = (int)(i - t * C4), n = cnt[t];
+    const float sc = NORM ? wsum[t] : 1.f;
+    const ray_ent *e = tab + t * cap;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int q = 0; q < n; q++) {
+        const float wc = e[q].w * sc;
+        const float4 v = y[(size_t)e[q].slot * C4 + c4];
+        a.x = fmaf(wc, v.x, a.x); a.y = fmaf(wc, v.y, a.y); a.z = fmaf(wc, v.z, a.z); a.w = fmaf(wc, v.w, a.w);
+    }
+    x[i] = a;
 }
 // the grid tokens' scroll coordinates (src/nn_attn_ray.cu:174-188): (r, arc, k) around the plane's centre, the angle unwrapped around the
 // plane's reference angle; registers (0, 0, 0); without an axis (cen's radius < 0) the grid indices (v, u, k)
@@ -297,10 +302,7 @@ extern "C" void at_rays_setup(const at_rays *R) {
     const ray_geo G = geo_of(R); const long long Tr = (long long)R->n * R->Q * R->Nr, Tg = (long long)R->n * G.Sg;
     if (!Tr) return;
     ray_pos_k<<<nblk_((size_t)Tr, 256), 256>>>(R->ray, R->Nr, Tr, (float *)R->pos);
-    long long *acc = (long long *)mi_ws(MI_WS_RAY, (size_t)Tg * sizeof(long long));
-    ray_zero64_k<<<nblk_((size_t)Tg, 256), 256>>>(acc, (size_t)Tg);                   // (a fill kernel, not a memset: the sequence may be captured)
-    ray_wsum_k<<<nblk_((size_t)Tr, 256), 256>>>(G, R->ray, R->ad, Tr, acc);
-    ray_winv_k<<<nblk_((size_t)Tg, 256), 256>>>(acc, (float *)R->wsum, Tg);
+    ray_inverse_k<<<nblk_((size_t)Tg, 256), 256>>>(G, R->ray, R->ad, Tg, R->Nt, 5 * R->Nt, nullptr, nullptr, (float *)R->wsum);
     MICK();
 }
 extern "C" void at_ray_gather(const at_rays *R, const float *x, float *y, int Cc, int norm) {
@@ -318,11 +320,15 @@ extern "C" void at_ray_scatter(const at_rays *R, const float *y, float *x, int C
     const ray_geo G = geo_of(R); const long long Tr = (long long)R->n * R->Q * R->Nr; const int C4 = Cc / 4;
     const size_t ng = (size_t)R->n * G.Sg * Cc;
     if (!ng) return;
-    long long *acc = (long long *)mi_ws(MI_WS_RAY, ng * sizeof(long long));
-    ray_zero64_k<<<nblk_(ng, 256), 256>>>(acc, ng);
-    ray_scatter_k<<<nblk_((size_t)Tr * C4, 256), 256>>>(G, R->ray, R->ad, Tr, C4, (const float4 *)y, acc);
-    if (norm) ray_scatter_out_k<true><<<nblk_(ng / 4, 256), 256>>>(acc, R->wsum, ng / 4, C4, (float4 *)x);
-    else ray_scatter_out_k<false><<<nblk_(ng / 4, 256), 256>>>(acc, R->wsum, ng / 4, C4, (float4 *)x);
+    if ((long long)R->n * R->Q * R->Nr > 0x7fffffffll) mi_die("at_ray_scatter: %lld ray slots", (long long)R->n * R->Q * R->Nr);
+    // the tokens' lists are rebuilt from the ray table on every call (a few microseconds per million tokens: cheaper than proving a cached
+    // one current), into library scratch: 5 Nt (slot, weight) pairs and a count per token
+    const size_t Tg = (size_t)R->n * G.Sg; const int cap = 5 * R->Nt;
+    int *cnt = (int *)mi_ws(MI_WS_RAY, Tg * ((size_t)cap * sizeof(ray_ent) + sizeof(int)) + 256);
+    ray_ent *tab = (ray_ent *)(cnt + ((Tg + 63) & ~(size_t)63));
+    ray_inverse_k<<<nblk_(Tg, 256), 256>>>(G, R->ray, R->ad, (long long)Tg, R->Nt, cap, tab, cnt, nullptr);
+    if (norm) ray_scatter_k<true><<<nblk_(ng / 4, 256), 256>>>(tab, cnt, cap, R->wsum, ng / 4, C4, (const float4 *)y, (float4 *)x);
+    else ray_scatter_k<false><<<nblk_(ng / 4, 256), 256>>>(tab, cnt, cap, R->wsum, ng / 4, C4, (const float4 *)y, (float4 *)x);
     MICK();
 }
 extern "C" void at_scroll_pos(int n, int nreg, int D, int Hh, int W, const int *ad, const float *cen, float *pos) {
