@@ -4,6 +4,7 @@
 #include <hip/hip_fp16.h>
 #include "mx_dev.hpp"
 #include "../../include/mi_attn.h"
+#include "attn_ray.hpp"
 
 #define HD AT_HD
 #define FT 64
@@ -183,9 +184,10 @@ extern "C" void at_tok_to_cs(const float *t, float *x, int n, int C, long Sg, in
 // A unit = one (token, part, head) = 48 values = six 8-dim slices; eight neighbouring lanes own a unit (two idle), each slice is two 16-byte
 // loads and one 16-byte store of eight halves. The sum of squares meets over the unit's lanes; a rotary pair never leaves its lane
 // (slice j covers pairs 4 (j & 1) .. + 3 of axis j / 2). ----
+struct ray_src { ray_geo G; const float *ray; const int *ad; };      // ray: null = the rows are the tokens' own
 __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv, const float *__restrict__ qg, const float *__restrict__ kg, __half *__restrict__ out,
                                                   float *__restrict__ rq, float *__restrict__ rk, float *__restrict__ amx, long long T, int H, int S, int Hh, int W, int nreg, int rope, float lbase,
-                                                  const float *__restrict__ gpos) {
+                                                  const float *__restrict__ gpos, ray_src rs) {
     // the rotary angles take few values - position along an axis x frequency - and a sine / cosine pair costs far more than the rest of a unit:
     // a block forms the table once (the same expression the per-value form evaluates, so the same bits), positions up to RP per axis
     constexpr int RP = 64;
@@ -210,7 +212,21 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
         if (t >= T) { if (j < 6) *(uint4 *)dst = make_uint4(0u, 0u, 0u, 0u); }
         else {
             float v[8];
-            if (j < 6) {
+            if (j < 6 && rs.ray) {
+                // radial attention: token t is a ray slot, its row the bilinear mix of the grid rows under it (at_ray_gather's arithmetic, corner by
+                // corner in its order), formed here instead of in a [slots][3 C] array that this kernel would read back
+                long long row[4]; float w[4];
+                const int nc = slot_stencil(rs.G, rs.ray, rs.ad, t, row, w);
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = 0.f;
+                for (int c = 0; c < nc; c++) {
+                    if (w[c] == 0.f) continue;
+                    const float4 *xs = (const float4 *)(qkv + row[c] * 3 * C + p * C + h * HD + 8 * j);
+                    const float4 a = xs[0], b = xs[1];
+                    v[0] = fmaf(w[c], a.x, v[0]); v[1] = fmaf(w[c], a.y, v[1]); v[2] = fmaf(w[c], a.z, v[2]); v[3] = fmaf(w[c], a.w, v[3]);
+                    v[4] = fmaf(w[c], b.x, v[4]); v[5] = fmaf(w[c], b.y, v[5]); v[6] = fmaf(w[c], b.z, v[6]); v[7] = fmaf(w[c], b.w, v[7]);
+                }
+            } else if (j < 6) {
                 const float4 *xs = (const float4 *)(qkv + t * 3 * C + p * C + h * HD + 8 * j);
                 const float4 a = xs[0], b = xs[1];
                 v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
@@ -263,12 +279,17 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
     if (threadIdx.x == 0 && bmax > *(volatile unsigned *)((unsigned *)amx + 1)) atomicMax((unsigned *)amx + 1, bmax);
 }
 __global__ void at_zero4_k(float *p) { if (threadIdx.x < 4) p[threadIdx.x] = 0.f; }
-extern "C" void at_fa_pack(const float *qkv, const float *qg, const float *kg, void *qkvh, float *rq, float *rk, float *amx, const at_geom *g, int nreg, int C, int rope, float base) {
+static void fa_pack(const float *qkv, const float *qg, const float *kg, void *qkvh, float *rq, float *rk, float *amx, const at_geom *g, int nreg, int C, int rope, float base, const at_rays *R) {
     if (C % HD || (C & 3)) mi_die("at_fa_pack: C %d is not a whole number of heads of %d", C, HD);
     const long long T = (long long)g->nseq * g->S, Tp = T + FT; const int H = C / HD;
+    ray_src rs = {};
+    if (R) { rs.G = geo_of(R); rs.ray = R->ray; rs.ad = R->ad; }
     at_zero4_k<<<1, 64>>>(amx);
-    qkv_pack_k<<<nblk_((size_t)Tp * H * 3 * 8, 256), 256>>>(qkv, qg, kg, (__half *)qkvh, rq, rk, amx, T, H, g->S, g->Hh, g->W, nreg, rope, log2f(base), rope ? g->pos : nullptr);
+    qkv_pack_k<<<nblk_((size_t)Tp * H * 3 * 8, 256), 256>>>(qkv, qg, kg, (__half *)qkvh, rq, rk, amx, T, H, g->S, g->Hh, g->W, nreg, rope, log2f(base), rope ? g->pos : nullptr, rs);
     MICK();
+}
+extern "C" void at_fa_pack(const float *qkv, const float *qg, const float *kg, void *qkvh, float *rq, float *rk, float *amx, const at_geom *g, int nreg, int C, int rope, float base) {
+    fa_pack(qkv, qg, kg, qkvh, rq, rk, amx, g, nreg, C, rope, base, nullptr);
 }
 
 // ---- parameters and scratch ----
@@ -397,8 +418,8 @@ extern "C" int at_block_fwd(const at_dims *d, const float *P, const at_bp *bp, c
         MICK();
     }
     if (R) {
-        at_ray_gather(R, w->qkv, w->qkvr, 3 * C, 0);
-        at_fa_pack(w->qkvr, P + bp->qg, P + bp->kg, w->qkvh, w->rq, w->rk, w->amx, &ga, 0, C, d->rope, d->rope_base);
+        // (the pack reads the grid's rows through the rays' stencils: at_ray_gather's rows without their round trip through w->qkvr, which stays unwritten)
+        fa_pack(w->qkv, P + bp->qg, P + bp->kg, w->qkvh, w->rq, w->rk, w->amx, &ga, 0, C, d->rope, d->rope_base, R);
         at_fa_fwd(w->qkvh, w->orr, w->lse, &ga, d->H, C);
         at_ray_scatter(R, w->orr, w->o, C, 1);
     } else {

@@ -9,17 +9,12 @@
 #include <string.h>
 #include "mx_dev.hpp"
 #include "../../include/mi_attn.h"
+#include "attn_ray.hpp"
 
 #define HD AT_HD
 #define FT 64
 
 namespace {
-struct plane_t { int Np, Nu, Nv; };                                 // planes along the axis dim, and the plane's two dims (u before v in z, y, x order)
-__host__ __device__ inline plane_t ray_plane(int ad, int D, int Hh, int W) { return plane_t{ad == 0 ? D : ad == 1 ? Hh : W, ad == 0 ? Hh : D, ad == 2 ? Hh : W}; }
-__host__ __device__ inline long long ray_token(int ad, int k, int a, int b, int Hh, int W) {      // grid token of in-plane (a, b) of plane k (src/attn.h:130-133)
-    const int z = ad == 0 ? k : a, y = ad == 0 ? a : ad == 1 ? k : b, x = ad == 2 ? k : b;
-    return ((long long)z * Hh + y) * W + x;
-}
 inline int max3(int a, int b, int c) { return a > b ? (a > c ? a : c) : (b > c ? b : c); }
 
 // One ray record: the half line from (cu, cv) at angle th, clipped to the plane's rectangle [-0.5, Nu - 0.5] x [-0.5, Nv - 0.5]; L = floor(chord)
@@ -118,25 +113,6 @@ extern "C" void at_rays_plan(int n, int D, int Hh, int W, float mult, const floa
 
 // ---- device ----
 namespace {
-struct ray_geo { int Q, Nr, D, Hh, W; long long Sg; };
-inline ray_geo geo_of(const at_rays *R) { return ray_geo{R->Q, R->Nr, R->D, R->Hh, R->W, (long long)R->D * R->Hh * R->W}; }
-// the up to four grid rows under ray slot s and their bilinear weights (src/attn.h:118-128); 0 past the ray's length
-__device__ __forceinline__ int slot_stencil(const ray_geo &G, const float *__restrict__ ray, const int *__restrict__ ad, long long s, long long *row, float *w) {
-    const long long rq = s / G.Nr; const int i = (int)(s - rq * G.Nr), b = (int)(rq / G.Q);
-    const float *rr = ray + rq * AT_RAY_F;
-    if (i >= (int)rr[6]) return 0;
-    const int axd = ad[b], k = (int)rr[7];
-    const plane_t pl = ray_plane(axd, G.D, G.Hh, G.W);
-    const float pu = fminf(fmaxf(fmaf((float)i, rr[2], rr[0]), 0.f), (float)(pl.Nu - 1)), pv = fminf(fmaxf(fmaf((float)i, rr[3], rr[1]), 0.f), (float)(pl.Nv - 1));
-    const int a0 = max(min((int)pu, pl.Nu - 2), 0), b0 = max(min((int)pv, pl.Nv - 2), 0), a1 = min(a0 + 1, pl.Nu - 1), b1 = min(b0 + 1, pl.Nv - 1);
-    const float fu = pu - (float)a0, fv = pv - (float)b0;
-    const long long base = (long long)b * G.Sg;
-    row[0] = base + ray_token(axd, k, a0, b0, G.Hh, G.W); w[0] = (1.f - fu) * (1.f - fv);
-    row[1] = base + ray_token(axd, k, a1, b0, G.Hh, G.W); w[1] = fu * (1.f - fv);
-    row[2] = base + ray_token(axd, k, a0, b1, G.Hh, G.W); w[2] = (1.f - fu) * fv;
-    row[3] = base + ray_token(axd, k, a1, b1, G.Hh, G.W); w[3] = fu * fv;
-    return 4;
-}
 __global__ void __launch_bounds__(256) ray_pos_k(const float *__restrict__ ray, int Nr, long long n, float *__restrict__ pos) {
     const long long s = blockIdx.x * 256ll + threadIdx.x;
     if (s >= n) return;
@@ -235,15 +211,21 @@ __global__ void __launch_bounds__(256) scroll_pos_k(long long n, long long S, in
 // multiply-adds as scalar operands (no LDS, no lane exchange). Probabilities are rounded to fp16 before they meet v, the denominator adds the
 // unrounded ones: the rounding points of the fp16 tensor-core kernel this replaces. Ray sequences are 20 - 50 slots long: the arithmetic is
 // a few percent of a block's and the kernel is latency-bound.
+// QL: queries per (sequence, head) unit, 64 or - for sequences of at most 32 tokens - 32, two units per wavefront: a ray of 24 slots fills 75 % of
+// the lanes instead of 37 % (the keys' rows are per-lane addresses either way; the walk runs to the longer of the two units' lengths)
+template <int QL>
 __global__ void __launch_bounds__(256) fa16_rows_k(const __half *__restrict__ Qh, const __half *__restrict__ Kh, const __half *__restrict__ Vh, float *__restrict__ o, float *__restrict__ lse,
                                                    int S, int H, int C, long long Tp, int nseq, float sl2, const int *__restrict__ lens) {
-    const int nqt = (S + 63) / 64;
-    const long long wv = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4u + (threadIdx.x >> 6)));
-    if (wv >= (long long)nseq * H * nqt) return;
-    const int qt = (int)(wv % nqt), h = (int)(wv / nqt % H), seq = (int)(wv / nqt / H), lane = threadIdx.x & 63;
+    const int nqt = (S + QL - 1) / QL, lane = threadIdx.x & 63;
+    const long long nun = (long long)nseq * H * nqt;
+    long long un = ((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / QL) + lane / QL;
+    const bool live = un < nun;
+    if (!live) un = nun - 1;                                       // (an idle half: the last unit's rows, nothing stored)
+    const int qt = (int)(un % nqt), h = (int)(un / nqt % H), seq = (int)(un / nqt / H);
     const size_t base = ((size_t)h * Tp + (size_t)seq * S) * HD;
-    const int SK = lens ? min(lens[seq], S) : S;
-    const int i = qt * 64 + lane;
+    const int SK = !live ? 0 : lens ? min(lens[seq], S) : S;
+    const int SKw = QL == 64 ? SK : max(SK, __shfl_xor(SK, 32));   // how far this wavefront walks
+    const int i = qt * QL + lane % QL;
     float q[HD], acc[HD];
     {
         const uint4 *qr = (const uint4 *)(Qh + base + (size_t)i * HD);      // (rows past the sequence's end are other rows of the padded array: read, never stored)
@@ -258,7 +240,8 @@ __global__ void __launch_bounds__(256) fa16_rows_k(const __half *__restrict__ Qh
     for (int d = 0; d < HD; d++) acc[d] = 0.f;
     float m = -INFINITY, l = 0.f;
     const __half *K = Kh + base, *V = Vh + base;
-    for (int j0 = 0; j0 < SK; j0 += 8) {
+    for (int j0 = 0; j0 < SKw; j0 += 8) {
+        if (j0 >= SK) continue;                                    // (the other unit of the wavefront is longer)
         float s[8];
 #pragma unroll
         for (int jj = 0; jj < 8; jj++) {
@@ -284,7 +267,7 @@ __global__ void __launch_bounds__(256) fa16_rows_k(const __half *__restrict__ Qh
             for (int d = 0; d < HD; d++) acc[d] = fmaf(ph, __half2float(vr[d]), acc[d]);
         }
     }
-    if (i >= S) return;
+    if (i >= S || !live) return;
     const float il = l > 0.f ? 1.f / l : 0.f;
     float4 *orow = (float4 *)(o + ((size_t)seq * S + i) * C + h * HD);
 #pragma unroll
@@ -293,6 +276,27 @@ __global__ void __launch_bounds__(256) fa16_rows_k(const __half *__restrict__ Qh
 }
 }
 
+// The tokens' sample lists live in library scratch: 5 Nt (slot, weight) pairs and a count per grid token. at_rays_setup builds them with the weight
+// sums; a scatter whose ray set is the one last set up on this thread (same table pointer, same sizes, the scratch still where it was) reuses them,
+// any other builds its own first (0.2 ms per 250 000 tokens) - a ray table changed in place needs a new at_rays_setup for its weight sums anyway.
+namespace {
+struct inv_key {
+    const float *ray; const int *ad; const void *ws; int n, Q, Nt, Nr, D, Hh, W;
+    bool operator==(const inv_key &o) const { return ray == o.ray && ad == o.ad && ws == o.ws && n == o.n && Q == o.Q && Nt == o.Nt && Nr == o.Nr && D == o.D && Hh == o.Hh && W == o.W; }
+};
+thread_local inv_key g_inv = {};
+struct inv_tab { int *cnt; ray_ent *tab; int cap; };
+inv_tab inverse_table(const at_rays *R, float *winv) {
+    const ray_geo G = geo_of(R); const size_t Tg = (size_t)R->n * G.Sg; const int cap = 5 * R->Nt;
+    int *cnt = (int *)mi_ws(MI_WS_RAY, Tg * ((size_t)cap * sizeof(ray_ent) + sizeof(int)) + 256);
+    const inv_tab t = {cnt, (ray_ent *)(cnt + ((Tg + 63) & ~(size_t)63)), cap};
+    const inv_key k = {R->ray, R->ad, cnt, R->n, R->Q, R->Nt, R->Nr, R->D, R->Hh, R->W};
+    if (!winv && k == g_inv) return t;
+    ray_inverse_k<<<nblk_(Tg, 256), 256>>>(G, R->ray, R->ad, (long long)Tg, R->Nt, cap, t.tab, t.cnt, winv);
+    g_inv = k;
+    return t;
+}
+}
 static void rays_check(const at_rays *R, const char *who) {
     if (!R || R->n < 0 || R->Q <= 0 || R->Nr <= 0 || R->D <= 0 || R->Hh <= 0 || R->W <= 0 || !R->ad || !R->ray) mi_die("%s: an incomplete ray set", who);
 }
@@ -302,7 +306,8 @@ extern "C" void at_rays_setup(const at_rays *R) {
     const ray_geo G = geo_of(R); const long long Tr = (long long)R->n * R->Q * R->Nr, Tg = (long long)R->n * G.Sg;
     if (!Tr) return;
     ray_pos_k<<<nblk_((size_t)Tr, 256), 256>>>(R->ray, R->Nr, Tr, (float *)R->pos);
-    ray_inverse_k<<<nblk_((size_t)Tg, 256), 256>>>(G, R->ray, R->ad, Tg, R->Nt, 5 * R->Nt, nullptr, nullptr, (float *)R->wsum);
+    if (Tr > 0x7fffffffll) mi_die("at_rays_setup: %lld ray slots", Tr);
+    inverse_table(R, (float *)R->wsum);
     MICK();
 }
 extern "C" void at_ray_gather(const at_rays *R, const float *x, float *y, int Cc, int norm) {
@@ -321,12 +326,8 @@ extern "C" void at_ray_scatter(const at_rays *R, const float *y, float *x, int C
     const size_t ng = (size_t)R->n * G.Sg * Cc;
     if (!ng) return;
     if ((long long)R->n * R->Q * R->Nr > 0x7fffffffll) mi_die("at_ray_scatter: %lld ray slots", (long long)R->n * R->Q * R->Nr);
-    // the tokens' lists are rebuilt from the ray table on every call (a few microseconds per million tokens: cheaper than proving a cached
-    // one current), into library scratch: 5 Nt (slot, weight) pairs and a count per token
-    const size_t Tg = (size_t)R->n * G.Sg; const int cap = 5 * R->Nt;
-    int *cnt = (int *)mi_ws(MI_WS_RAY, Tg * ((size_t)cap * sizeof(ray_ent) + sizeof(int)) + 256);
-    ray_ent *tab = (ray_ent *)(cnt + ((Tg + 63) & ~(size_t)63));
-    ray_inverse_k<<<nblk_(Tg, 256), 256>>>(G, R->ray, R->ad, (long long)Tg, R->Nt, cap, tab, cnt, nullptr);
+    const inv_tab it = inverse_table(R, nullptr);
+    const ray_ent *tab = it.tab; const int *cnt = it.cnt; const int cap = it.cap;
     if (norm) ray_scatter_k<true><<<nblk_(ng / 4, 256), 256>>>(tab, cnt, cap, R->wsum, ng / 4, C4, (const float4 *)y, (float4 *)x);
     else ray_scatter_k<false><<<nblk_(ng / 4, 256), 256>>>(tab, cnt, cap, R->wsum, ng / 4, C4, (const float4 *)y, (float4 *)x);
     MICK();
@@ -342,8 +343,11 @@ extern "C" void at_fa_fwd(const void *qkvh, float *o, float *lse, const at_geom 
     const long long T = (long long)g->nseq * g->S, Tp = T + FT;
     if (!T) return;
     const __half *Qh = (const __half *)qkvh, *Kh = Qh + (size_t)H * Tp * HD, *Vh = Kh + (size_t)H * Tp * HD;
-    const long long nw = (long long)g->nseq * H * ((g->S + 63) / 64);
-    if (nw > 0x7fffffffll) mi_die("at_fa_fwd: %lld (sequence, head, query tile) units", nw);
-    fa16_rows_k<<<nblk_((size_t)nw, 4), 256>>>(Qh, Kh, Vh, o, lse, g->S, H, C, Tp, g->nseq, 1.4426950408889634f / sqrtf((float)HD), g->lens);
+    const int QL = g->S <= 32 ? 32 : 64;
+    const long long nw = ((long long)g->nseq * H * ((g->S + QL - 1) / QL) + 64 / QL - 1) / (64 / QL);      // wavefronts
+    if (nw > 0x7fffffffll) mi_die("at_fa_fwd: %lld wavefronts", nw);
+    const float sl2 = 1.4426950408889634f / sqrtf((float)HD);
+    if (QL == 32) fa16_rows_k<32><<<nblk_((size_t)nw, 4), 256>>>(Qh, Kh, Vh, o, lse, g->S, H, C, Tp, g->nseq, sl2, g->lens);
+    else fa16_rows_k<64><<<nblk_((size_t)nw, 4), 256>>>(Qh, Kh, Vh, o, lse, g->S, H, C, Tp, g->nseq, sl2, g->lens);
     MICK();
 }
