@@ -101,6 +101,11 @@ void mi_conv1_matrix(int mode);
    MX-fp8 / MX-fp4 (ybits 8 / 4) once, for a tensor several convs read; they then take y with no GroupNorm. s.c a multiple of 32. In a split
    input, gp2.G = -1 says "x2 carries no GroupNorm, gp is x's own" (gp2.G = 0 keeps the reference's meaning: gp spans both segments). */
 int mi_conv_prestage(const void *x, int xdt, shape5 s, gnp_t gp, void *y, int ybits);
+/* the same from an MX-fp8 tensor into both formats at once (y8 MX-fp8, y4 MX-fp4: the bytes of the two single calls from one read and one
+   evaluation): a tensor whose readers compute in different formats. mi_conv_x2_dt(4) before a conv entry says that the calling thread's next
+   split conv's second segment is stored as MX-fp4 although x is MX-fp8 (3: MX-fp8 beside an MX-fp4 x; the descriptor carries one format) */
+int mi_conv_prestage2(const void *x, shape5 s, gnp_t gp, void *y8, void *y4);
+void mi_conv_x2_dt(int dt);
 gnp_t gnp_mk(const float *gamma, const float *beta, const float *mean, const float *rstd, int G);   /* src/nn_lp.h:19 */
 int lp_gn_slab_any(void);                                                                         /* src/nn_lp.h:20: any statistics array registered */
 /* the statistics array `mean` holds one row per (sample, z-slab) with this geometry: every gnp_t gnp_mk builds from it (and lp_gn_silu_apply_mx,

@@ -757,3 +757,32 @@ def test_fused_upsample_blend_modes(gpu, cbits, up):
         other, _ = orc.conv3(qa, 3, N, Cu + Cs, D, H, W, w, None, Co, 0, cbits=4, x2=qb, c_split=Cu, up=5 - up, acc64=1)
         d = np.abs(got - other).max() / np.abs(want).max()
         assert d > 1e-4, d
+
+
+@pytest.mark.gpu
+def test_prestage_in_both_formats_and_a_split_conv_on_the_fp4_rows(gpu):
+    """mi_conv_prestage2: one read and one evaluation write the MX-fp8 and the MX-fp4 form of silu(gn(x)), the bytes of the two single calls; an
+    MX-fp4 conv whose second segment is those fp4 rows (mi_conv_x2_dt(4), no GroupNorm left on it) beside an upsampled MX-fp8 first segment gives
+    the bytes of the conv that transforms the MX-fp8 skip itself."""
+    from ufsm_amd import gnp_t
+    rng = np.random.default_rng(91)
+    N, Cu, Cs, Co, (D, H, W), G = 2, 64, 32, 32, (8, 16, 32), 8
+    S = D * H * W
+    xs_ = rng.standard_normal((N, Cs, S)).astype(np.float32); xu = rng.standard_normal((N, Cu, S // 8)).astype(np.float32)
+    qs, qu = orc.f32_to_mx(8, xs_, N, Cs, S), orc.f32_to_mx(8, xu, N, Cu, S // 8)
+    par = lambda C: (rng.uniform(.5, 1.5, C).astype(np.float32), rng.uniform(-.3, .3, C).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.7, 1.4, N * G).astype(np.float32))
+    p1, p2 = par(Cu), par(Cs)
+    g2 = dev_gn(*p2, G)
+    dq = DevBuf.from_numpy(qs); y8, y4, s8, s4 = (DevBuf(orc.mx_bytes(b, N, Cs, S)) for b in (8, 4, 8, 4))
+    assert lib.mi_conv_prestage2(dq.ptr, shape5(N, Cs, D, H, W), g2, y8.ptr, y4.ptr) == 0
+    assert lib.mi_conv_prestage(dq.ptr, 3, shape5(N, Cs, D, H, W), g2, s8.ptr, 8) == 0 and lib.mi_conv_prestage(dq.ptr, 3, shape5(N, Cs, D, H, W), g2, s4.ptr, 4) == 0
+    LP.check()
+    assert np.array_equal(y8.to_numpy(np.uint8), s8.to_numpy(np.uint8)) and np.array_equal(y4.to_numpy(np.uint8), s4.to_numpy(np.uint8))
+    w = (rng.standard_normal((Co, Cu + Cs, 27)) * np.sqrt(2.0 / ((Cu + Cs) * 27))).astype(np.float32)
+    own, _ = gpu_conv(qu, 3, N, Cu + Cs, D, H, W, w, None, Co, 3, cbits=4, x2=qs, c_split=Cu, up=1, gp=dev_gn(*p1, G), gp2=g2)
+    none = gnp_t(); none.G = -1
+    lib.mi_conv_x2_dt(4)
+    pre, _ = gpu_conv(qu, 3, N, Cu + Cs, D, H, W, w, None, Co, 3, cbits=4, x2=y4.to_numpy(np.uint8), c_split=Cu, up=1, gp=dev_gn(*p1, G), gp2=none)
+    assert np.array_equal(pre, own)
+    again, _ = gpu_conv(qu, 3, N, Cu + Cs, D, H, W, w, None, Co, 3, cbits=4, x2=qs, c_split=Cu, up=1, gp=dev_gn(*p1, G), gp2=g2)      # the setting held for one call
+    assert np.array_equal(again, own)

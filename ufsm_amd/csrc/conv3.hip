@@ -323,6 +323,10 @@ static int conv_stem(const char *who, const void *x, int xbf, shape5 xs, const f
 static thread_local const uint8_t *g_static_zpage = nullptr;     // the constant page of the calling thread's conv when it runs on the fixed scratch
 static thread_local int g_split = -1;       // mi_conv_split: the calling thread's tile count below which 128-channel slices are halved (-1: the default)
 extern "C" void mi_conv_split(int tiles) { g_split = tiles; }
+// storage format of the calling thread's next split conv's second segment when it differs from the first's (3 MX-fp8, 4 MX-fp4; the descriptor
+// carries one format for both); 0 = the same
+static thread_local int g_x2_dt = 0;
+extern "C" void mi_conv_x2_dt(int dt) { g_x2_dt = dt == 3 || dt == 4 ? dt : 0; }
 static thread_local int g_s2d = -1;         // mi_conv_s2_direct: the calling thread's choice of stride-2 kernel (-1: by launch size)
 extern "C" void mi_conv_s2_direct(int mode) { g_s2d = mode; }
 static int split_s2_env() { static int v = -1; if (v < 0) v = getenv("MI_CONV_SPLIT_S2") ? atoi(getenv("MI_CONV_SPLIT_S2")) : 1; return v; }      // tuning knob: 0 keeps four channel tiles
@@ -371,10 +375,13 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     const bool s2g = sp.x2 && sp.gp2.G;
     if (sp.gp2.G < 0) sp.gp2 = gnp_mk(nullptr, nullptr, nullptr, nullptr, 0);
     const void *segx[2] = {x, sp.x2}; const int segC[2] = {Cx, C2};
+    const int segbf[2] = {xbf, sp.x2 && g_x2_dt ? g_x2_dt : xbf};
+    g_x2_dt = 0;
     for (int s = 0; s < (sp.x2 ? 2 : 1); s++) {
         const gnp_t g = s2g ? (s ? sp.gp2 : gp) : gp;
         const int Cg = s2g ? segC[s] : Ci, cg0 = s2g ? 0 : (s ? Cx : 0);
         const bool upseg = s == 0 && sp.up;
+        const int xbf = segbf[s];                                 // (this segment's storage format)
         const bool direct = xbf == fdt && !g.G && !upseg;
         const int nbp = (segC[s] + 31) / 32;
         if (direct) {
@@ -591,6 +598,12 @@ extern "C" int mi_conv_prestage(const void *x, int xdt, shape5 s, gnp_t gp, void
     if ((ybits != 8 && ybits != 4) || s.c % 32 || xdt < 0 || xdt > 4 || (gp.G > 0 && s.c % gp.G)) return -1;
     const size_t hw = (size_t)s.h * s.w;
     gn_for_slabs("mi_conv_prestage", gp, s.h * s.w, 0, s.d, [&](int z0, int z1, gnp_t gs) { mi_restage_sub(x, xdt, s.n, s.c, (size_t)(z1 - z0) * hw, gs, s.c, 0, y, ybits, (size_t)s.d * hw, (size_t)z0 * hw); });
+    return 0;
+}
+extern "C" int mi_conv_prestage2(const void *x, shape5 s, gnp_t gp, void *y8, void *y4) {
+    if (s.c % 32 || (gp.G > 0 && s.c % gp.G) || !y8 || !y4) return -1;
+    const size_t hw = (size_t)s.h * s.w;
+    gn_for_slabs("mi_conv_prestage2", gp, s.h * s.w, 0, s.d, [&](int z0, int z1, gnp_t gs) { mi_restage_sub2(x, s.n, s.c, (size_t)(z1 - z0) * hw, gs, y8, y4, (size_t)s.d * hw, (size_t)z0 * hw); });
     return 0;
 }
 extern "C" int lp_conv_fwd_f8(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp) {

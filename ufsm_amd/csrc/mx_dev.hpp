@@ -279,6 +279,7 @@ int mi_mx_gemm_apacked_at(int bits, int tb, int M, int N, int K, const uint8_t *
 // mi_mx_gemm_abuf(8, T, 2 F, C) said and W [2 F][C] row-major, written as the packed A operand (gq, gs) of the down projection; h is not stored
 int mi_mx_gemm_glu(int T, int F, int C, const float *W, const float *bias, uint8_t *gq, uint8_t *gs);
 void mi_restage_sub(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits, size_t Ss, size_t v0);     // only voxels [v0, v0 + S) of tensors of Ss voxels
+void mi_restage_sub2(const void *x, int N, int C, size_t S, gnp_t gp, void *y8, void *y4, size_t Ss, size_t v0);      // MX-fp8 source, 32-wide blocks: both formats from one read
 void mi_restage_up_sub(const void *x, int xdt, int N, int C, int D, int H, int W, gnp_t gp, int Cg, void *y, int ybits, int zlo, int zhi, int h2);   // only fine planes [zlo, zhi)
 void mi_post_error(hipError_t e, const char *file, int line);
 #define MICK() do { hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) mi_post_error(e_, __FILE__, __LINE__); } while (0)

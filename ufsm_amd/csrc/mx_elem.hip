@@ -758,8 +758,10 @@ __global__ void __launch_bounds__(256) restage_k(const void *xv, uint8_t *y, int
 // 16 or 8 out), so a wavefront reads and writes contiguous memory; the halves' amaxes meet through one lane exchange. The (a, b)
 // coefficients of the block's 32 channels are formed once per workgroup in LDS. HBM-bound: (bits_in + bits_out) / 8 + 2/32 bytes per element.
 constexpr int RS32_R = 4;                                          // rows per thread of restage32_k
-template <int BX, int BY>
-__global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, size_t Ss, size_t v0) {
+// BY2 (4, with BY 8): the same values also leave as a second tensor y2 in MX-fp4 - a skip tensor whose two readers compute in different
+// formats (the stride-2 down conv in e4m3, the decoder's conv in e2m1) is read and transformed once
+template <int BX, int BY, int BY2 = 0>
+__global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, size_t Ss, size_t v0, uint8_t *y2 = nullptr) {
     const int nb = C / 32, blk = blockIdx.y, n = blockIdx.z;
     __shared__ float sa[32], sb[32];
     // A workgroup moves RS32_R x 128 consecutive voxels of the block, a thread one 16-channel half of RS32_R rows 128 voxels apart: the rows are
@@ -820,7 +822,19 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
             if (v < S) *(uint2 *)(y + row * 16 + hf * 8) = o;
         }
         if (!hf && v < S) ys[row] = (uint8_t)(e + 127);
+        if (BY2 == 4) {
+            const int e2 = d_mx_exp(am, MI_INVQ4);
+            uint2 o; o.x = d_enc8_e2m1(r, e2); o.y = d_enc8_e2m1(r + 8, e2);
+            if (v < S) { *(uint2 *)(y2 + row * 16 + hf * 8) = o; if (!hf) (y2 + (size_t)N * nb * Ss * 16)[row] = (uint8_t)(e2 + 127); }
+        }
     }
+}
+// MX-fp8 source with 32-wide blocks -> the transformed rows in both formats from one read (y8 MX-fp8, y4 MX-fp4), the bytes of the two single calls
+void mi_restage_sub2(const void *x, int N, int C, size_t S, gnp_t gp, void *y8, void *y4, size_t Ss, size_t v0) {
+    if (!N || !S) return;
+    const dim3 grid(nblk_(S, 128 * RS32_R), (unsigned)(C / 32), (unsigned)N);
+    restage32_k<8, 8, 4><<<grid, 256>>>((const uint8_t *)x, (uint8_t *)y8, N, C, S, gp, C, 0, Ss, v0, (uint8_t *)y4);
+    MICK();
 }
 // voxels [v0, v0 + S) of tensors holding Ss voxels per (sample, channel / block): the result has the source's geometry, only that range is written
 void mi_restage_sub(const void *x, int xdt, int N, int C, size_t S, gnp_t gp, int Cg, int cg0, void *y, int ybits, size_t Ss, size_t v0) {

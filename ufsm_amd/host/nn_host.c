@@ -64,7 +64,9 @@ static int conv_family(const char *who, int xdt, int ydt, int x2dt, int has_x2, 
         if (xdt == 2 && ydt >= 3 && cin <= 8 && !has_x2) return 8;
         if (xdt >= 3 && ydt >= 3 && xdt != ydt && (cin <= 8 || (xdt == 3 && ydt == 4)) && !has_x2 && !up) return 8;
         if (xdt == 4 && ydt == 0) return 4;
-        if (xdt < 3 || ydt != xdt || (has_x2 && x2dt != xdt)) {
+        /* (one extension to the reference's one-format rule: under precision 3 an MX-fp8 conv may take its second segment as MX-fp4 rows - a skip the
+           graph transformed once for two readers of different compute formats; the conv entry is told through mi_conv_x2_dt) */
+        if (xdt < 3 || ydt != xdt || (has_x2 && x2dt != xdt && !(xdt == 3 && x2dt == 4 && g_prec == 3))) {
             fprintf(stderr, "%s: MX storage needs MX inputs and outputs of one format (x %d y %d x2 %d, %dx%d ch)\n", who, xdt, ydt, has_x2 ? x2dt : -1, cin, cout);
             abort();
         }
@@ -85,6 +87,7 @@ static int conv_s1(const char *who, const float *x, shape5 xs, const float *w, c
     const int fam = conv_family(who, xdt, ydt, x2dt, sp.x2 != nullptr, xs.c, cout, sp.up);
     int (*const conv)(const void *, int, shape5, const float *, const float *, int, void *, int, gnp_t, double *, int, split_t) = fam == 4 ? lp_conv_fwd_f4 : lp_conv_fwd_f8;
     sp.wkey = (unsigned)((uintptr_t)w >> 4) | 1u;                   /* inference: weights are prepared once per conv (keyed by the weight pointer) */
+    if (sp.x2 && x2dt >= 3 && x2dt != xdt) mi_conv_x2_dt(x2dt);
     if (G_out > cout) G_out = cout;                                 /* GroupNorm uses min(G, C) groups (src/nn_wgrad.cu:105) */
     const int want = G_out > 0 && omean && orstd;
     const int fused = gn_fused_stored(ydt, cout);
@@ -111,7 +114,7 @@ static int conv_s1(const char *who, const float *x, shape5 xs, const float *w, c
 int nn_conv3d_fwd_x(const float *x, const nn_gn_t *gx, const float *x2, const nn_gn_t *gx2, int c_split, int up, shape5 xs,
                     const float *w, const float *b, int cout, int k, int stride, float *y, int G_out, float eps, float *omean, float *orstd) {
     const int xdt = lp_dt(x), ydt = lp_dt(y);
-    if (x2 && lp_dt(x2) != xdt) { fprintf(stderr, "nn_conv3d_fwd_x: x and x2 differ in storage\n"); return -1; }
+    if (x2 && lp_dt(x2) != xdt && !(xdt == 3 && lp_dt(x2) == 4 && g_prec == 3)) { fprintf(stderr, "nn_conv3d_fwd_x: x and x2 differ in storage\n"); return -1; }      /* (the exception: conv_family) */
     gnp_t gp = gx ? gnp_mk(gx->gamma, gx->beta, gx->mean, gx->rstd, gx->G) : gnp_mk(nullptr, nullptr, nullptr, nullptr, 0);
     if (k == 1) {                                                   /* the head: MX input, fp32 (or registered fp16) planes out (src/nn_fusedgn.cu:57-62) */
         if (xdt < 3 || x2 || stride != 1 || G_out) return -1;

@@ -45,6 +45,8 @@ struct unet {
     convp ds[UNET_MAXLEV], eh;         /* cfg.ds_levels / cfg.emb_lev: the deep-supervision heads of decoder levels 1 .. ds_levels and the distillation head: training-time outputs, here only their place in the parameter vector (src/unet.c:467, :511) */
     void *downo[UNET_MAXLEV];
     void *skipst[UNET_MAXLEV];         /* silu(gn(enc[i].a2)) in the compute format, formed once for its two readers (down conv, decoder conv1); null: each reader transforms it */
+    void *skipst4[UNET_MAXLEV];        /* precision 3 over MX-fp8 storage: the two readers compute in different formats (the stride-2 conv in e4m3, the decoder's in e2m1);
+                                          the same pass writes the MX-fp4 rows here beside the MX-fp8 ones in skipst */
     gnpar dn[UNET_MAXLEV]; float *dm[UNET_MAXLEV], *dr[UNET_MAXLEV];   /* down_norm: GroupNorm after down[i], its statistics */
     size_t np; float *p, *ema, *params;                            /* device: live weights, EMA copy, the one the forward reads */
     float *src, *wm; int wm_ok;                                    /* cfg.w4_2d: the selected weights (p or ema), their forward copy with the fp4 convs' weights rounded per 32 x 32 block, whether it is current */
@@ -250,8 +252,8 @@ static void free_acts(unet *u) {
             act_del(b->a1); act_del(b->a2); mi_free(b->m1); mi_free(b->r1); mi_free(b->m2); mi_free(b->r2);
             b->a1 = b->a2 = nullptr; b->m1 = b->r1 = b->m2 = b->r2 = nullptr;
         }
-        act_del(u->downo[i]); act_del(u->skipst[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
-        u->downo[i] = u->skipst[i] = nullptr; u->dm[i] = u->dr[i] = nullptr;
+        act_del(u->downo[i]); act_del(u->skipst[i]); act_del(u->skipst4[i]); mi_free(u->dm[i]); mi_free(u->dr[i]);
+        u->downo[i] = u->skipst[i] = u->skipst4[i] = nullptr; u->dm[i] = u->dr[i] = nullptr;
     }
     if (u->tbn) { act_del(u->tb.a2); mi_free(u->tb.m2); mi_free(u->tb.r2); mi_free(u->tb_cs); mi_free(u->tb_tok); mi_free(u->tb_ws); if (u->tb_vr) mi_free(u->tb_vr); u->tb_vr = nullptr; tb_geom_free(u); u->tb.a2 = nullptr; u->tb.m2 = u->tb.r2 = nullptr; u->tb_cs = u->tb_tok = nullptr; u->tb_ws = nullptr; }
     for (int i = 0; i < 2; i++) { act_del(u->slab_tmp[i]); act_del(u->slab_carry[i]); u->slab_tmp[i] = u->slab_carry[i] = nullptr; }
@@ -300,7 +302,12 @@ static int build_acts(unet *u, shape5 in) {
         if (i < L - 1) {
             shape5 ds = u->ls[i + 1]; ds.c = w[i]; u->downo[i] = act_new(u, ds);
             /* both readers of the skip compute in e4m3 from MX-fp8 storage: one shared pre-stage (any other combination: the readers' formats differ) */
-            if (u->act_dt == 8 && u->prec != 3 && w[i] % 32 == 0 && i >= u->slab_nl) u->skipst[i] = act_new(u, u->enc[i].ys);
+            static int skip2 = -1;                                 /* tuning knob MI_UNET_SKIP2=0: under precision 3 each reader transforms the skip itself */
+            if (skip2 < 0) skip2 = getenv("MI_UNET_SKIP2") ? atoi(getenv("MI_UNET_SKIP2")) : 1;
+            if (u->act_dt == 8 && (u->prec != 3 || skip2) && w[i] % 32 == 0 && i >= u->slab_nl) {
+                u->skipst[i] = act_new(u, u->enc[i].ys);
+                if (u->prec == 3) { const size_t b4 = nn_mx4_bytes(u->enc[i].ys); u->skipst4[i] = mi_malloc(b4); mi_zero(u->skipst4[i], b4); nn_set_storage(u->skipst4[i], b4, 4); }
+            }
             if (cfg->down_norm) { const size_t ng = (size_t)in.n * G_of(u, w[i]); u->dm[i] = f32_new(ng); u->dr[i] = f32_new(ng); }
         }
     }
@@ -709,7 +716,8 @@ static int graph_fwd(unet *u, const void *x) {
             const block *so = stage_out(u, i);
             const nn_gn_t g = gn_out(u, so);
             const int pre = u->skipst[i] != nullptr;
-            if (pre && mi_conv_prestage(so->a2, 3, so->ys, gnp_mk(g.gamma, g.beta, g.mean, g.rstd, g.G), u->skipst[i], 8)) return -1;
+            if (pre && (u->skipst4[i] ? mi_conv_prestage2(so->a2, so->ys, gnp_mk(g.gamma, g.beta, g.mean, g.rstd, g.G), u->skipst[i], u->skipst4[i])
+                                      : mi_conv_prestage(so->a2, 3, so->ys, gnp_mk(g.gamma, g.beta, g.mean, g.rstd, g.G), u->skipst[i], 8))) return -1;
             if (nn_conv3d_fwd_x(pre ? u->skipst[i] : so->a2, pre ? nullptr : &g, nullptr, nullptr, 0, 0, so->ys, P(u, u->down[i].w), P(u, u->down[i].b), u->cfg.widths[i], 3, 2, u->downo[i], 0, 0.f, nullptr, nullptr)) return -1;
             shape5 ds = u->ls[i + 1]; ds.c = u->cfg.widths[i];
             if (u->cfg.down_norm) {                                /* statistics of the stored down-conv output now, the transform in the next conv1's staging (src/unet.c:2974-2979) */
@@ -725,7 +733,8 @@ static int graph_fwd(unet *u, const void *x) {
         nn_gn_t gc = gn_out(u, coarse); const nn_gn_t gs = gn_out(u, skip);
         if (i == L - 2 && u->tbn) { coarse = &u->tb; gc.mean = u->tb.m2; gc.rstd = u->tb.r2; }      /* the stage's output under the level's n2 affine (src/unet.c:508) */
         static const nn_gn_t none = {nullptr, nullptr, nullptr, nullptr, -1};          /* the pre-staged skip: no GroupNorm left to apply */
-        if (block_fwd(u, &u->dec[i], i, u->skipst[i] ? u->skipst[i] : skip->a2, u->skipst[i] ? &none : &gs, coarse->a2, &gc, coarse->ys.c, dn1[i], dn2[i])) return -1;
+        const void *sk = u->skipst4[i] ? u->skipst4[i] : u->skipst[i];      /* (the decoder's conv computes in e2m1 under precision 3: its rows) */
+        if (block_fwd(u, &u->dec[i], i, sk ? sk : skip->a2, sk ? &none : &gs, coarse->a2, &gc, coarse->ys.c, dn1[i], dn2[i])) return -1;
     }
     const block *last = L > 1 ? &u->dec[0] : &u->enc[0];
     const nn_gn_t g = gn_out(u, last);

@@ -48,6 +48,8 @@ _PROTOS = {
     "mi_conv_s2_direct": (None, [C.c_int]),
     "mi_conv1_matrix": (None, [C.c_int]),
     "mi_conv_prestage": (_I, [_P, _I, shape5, gnp_t, _P, _I]),
+    "mi_conv_prestage2": (_I, [_P, shape5, gnp_t, _P, _P]),
+    "mi_conv_x2_dt": (None, [_I]),
     "gnp_mk": (gnp_t, [_P, _P, _P, _P, _I]),
     "lp_gn_slab_any": (_I, []),
     "lp_gn_slab_reg": (None, [_P, _I, _I, _I, _I]),
