@@ -254,6 +254,7 @@ __global__ void __launch_bounds__(256) qkv_pack_k(const float *__restrict__ qkv,
                             const int fi = 4 * (j & 1) + i;
                             float sn, cs;
                             if (tab) { const float2 sc2 = rtab[(int)pos * 8 + fi]; sn = sc2.x; cs = sc2.y; }
+                            else if (gpos) { const float ang = pos * exp2f(-lbase * (float)fi / 8.f); sn = __sinf(ang); cs = __cosf(ang); }      // (real coordinates: the hardware sine / cosine, as the reference's fast-math build)
                             else sincosf(pos * exp2f(-lbase * (float)fi / 8.f), &sn, &cs);
                             const float a = v[2 * i], b = v[2 * i + 1];
                             v[2 * i] = a * cs - b * sn; v[2 * i + 1] = a * sn + b * cs;
