@@ -156,6 +156,15 @@ void *mi_malloc(size_t bytes);                 /* device memory; aborts with a m
 void mi_free(void *p);
 void mi_zero(void *p, size_t bytes);
 void mi_h2d(void *dst, const void *src, size_t bytes);
+/* pinned host memory, a copy from it in stream order that the host does not wait for, and a fence: set in stream order, waited for by the host
+   (before it rewrites the source of such a copy) */
+void *mi_host_alloc(size_t bytes);
+void mi_host_free(void *p);
+void mi_h2d_async(void *dst, const void *src, size_t bytes);
+void *mi_fence_new(void);
+void mi_fence_set(void *f);
+void mi_fence_wait(void *f);
+void mi_fence_free(void *f);
 void mi_d2h(void *dst, const void *src, size_t bytes);
 void mi_d2d(void *dst, const void *src, size_t bytes);
 void mi_d2d_rows(void *dst, size_t dpitch, const void *src, size_t spitch, size_t width, size_t rows);   /* rows runs of width bytes at the two pitches, in stream order */

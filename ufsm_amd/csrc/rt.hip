@@ -46,6 +46,14 @@ extern "C" void mi_free(void *p) { if (p) MIRT(hipFree(p)); }
 __global__ void fill_u32_k(unsigned *p, size_t n, unsigned v) { size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; if (i < n) p[i] = v; }
 extern "C" void mi_zero(void *p, size_t bytes) { MIRT(hipMemsetAsync(p, 0, bytes, 0)); }
 extern "C" void mi_h2d(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice)); }
+// pinned host memory and a copy from it in stream order (the host does not wait), with a fence the host can wait on before it rewrites the source
+extern "C" void *mi_host_alloc(size_t bytes) { void *p = nullptr; hipError_t e = hipHostMalloc(&p, bytes ? bytes : 1); if (e != hipSuccess) mi_die("mi_host_alloc: %zu bytes: %s", bytes, hipGetErrorString(e)); return p; }
+extern "C" void mi_host_free(void *p) { if (p) MIRT(hipHostFree(p)); }
+extern "C" void mi_h2d_async(void *dst, const void *src, size_t bytes) { if (bytes) MIRT(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, 0)); }
+extern "C" void *mi_fence_new(void) { hipEvent_t e; MIRT(hipEventCreateWithFlags(&e, hipEventDisableTiming)); return (void *)e; }
+extern "C" void mi_fence_set(void *f) { MIRT(hipEventRecord((hipEvent_t)f, 0)); }
+extern "C" void mi_fence_wait(void *f) { MIRT(hipEventSynchronize((hipEvent_t)f)); }
+extern "C" void mi_fence_free(void *f) { if (f) MIRT(hipEventDestroy((hipEvent_t)f)); }
 extern "C" void mi_d2h(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpy(dst, src, bytes, hipMemcpyDeviceToHost)); }
 extern "C" void mi_d2d(void *dst, const void *src, size_t bytes) { MIRT(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, 0)); }
 // `rows` runs of `width` bytes, run r at dst + r * dpitch from src + r * spitch (a range of planes of every channel block of an MX tensor)

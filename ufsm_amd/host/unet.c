@@ -62,6 +62,7 @@ struct unet {
     /* cfg.attn_axis 1 / attn_pe 3: the scroll geometry (src/unet.c:280-282). One device buffer tb_rb holds the ray table, lengths, axis dims, ray
        positions, stencil weight sums, the grid tokens' scroll coordinates and the per-plane frames; the host side of a plan; the axis records */
     at_rays tbr; float *tb_rb, *tb_gpos, *tb_cen, *tb_rayh, *tb_cenh, *tb_axb, *tb_axh; int *tb_lensh, *tb_adh;
+    void *tb_pin[2], *tb_fence[2]; int tb_set;                     /* the plan's host tables: two pinned sets copied in stream order, each rewritten only after its copy ran */
     int tb_Q, tb_Nt, tb_Nr, tb_axn, tb_axs, tb_axdirty, tb_axwarn, tb_noax;
 };
 
@@ -88,7 +89,8 @@ static int cfg_axis(const unet_cfg *c) { return c->attn_blocks > 0 && (c->attn_a
 static float attn_ray_mult(void) { static float m = 0; if (m <= 0) { const char *e = getenv("UFSM_ATTN_RAY_MULT"); m = e && atof(e) > 0 ? (float)atof(e) : 2.f; } return m; }
 static void tb_geom_free(unet *u) {
     if (u->tb_rb) mi_free(u->tb_rb);
-    free(u->tb_rayh); free(u->tb_cenh); free(u->tb_lensh); free(u->tb_adh); free(u->tb_axb);
+    for (int k = 0; k < 2; k++) { if (u->tb_fence[k]) { mi_fence_wait(u->tb_fence[k]); mi_fence_free(u->tb_fence[k]); } if (u->tb_pin[k]) mi_host_free(u->tb_pin[k]); u->tb_pin[k] = u->tb_fence[k] = nullptr; }
+    free(u->tb_axb);
     u->tb_rb = u->tb_gpos = u->tb_cen = u->tb_rayh = u->tb_cenh = u->tb_axb = nullptr; u->tb_lensh = u->tb_adh = nullptr;
     u->tbr = (at_rays){0}; u->tbg.rays = nullptr; u->tbg.pos = nullptr;
 }
@@ -339,9 +341,10 @@ static int build_acts(unet *u, shape5 in) {
             u->tbr = (at_rays){.n = ys.n, .Q = u->tb_Q, .Nt = u->tb_Nt, .Nr = u->tb_Nr, .D = ys.d, .Hh = ys.h, .W = ys.w, .ad = (const int *)(u->tb_rb + o_ad), .ray = u->tb_rb + o_ray,
                                .lens = (const int *)(u->tb_rb + o_len), .pos = u->tb_rb + o_pos, .wsum = u->tb_rb + o_ws};
             u->tb_gpos = u->tb_rb + o_gp; u->tb_cen = u->tb_rb + o_cen;
-            u->tb_rayh = malloc(nq * AT_RAY_F * sizeof(float)); u->tb_cenh = malloc((size_t)ys.n * Pm * 4 * sizeof(float));
-            u->tb_lensh = malloc(nq * sizeof(int)); u->tb_adh = malloc((size_t)ys.n * sizeof(int)); u->tb_axb = malloc((size_t)ys.n * AT_AXR(Pm) * sizeof(float));
-            if (!u->tb_rayh || !u->tb_cenh || !u->tb_lensh || !u->tb_adh || !u->tb_axb) { fprintf(stderr, "unet: no host memory for the ray plan\n"); abort(); }
+            for (int k = 0; k < 2; k++) { u->tb_pin[k] = mi_host_alloc((nq * AT_RAY_F + nq + (size_t)ys.n + (size_t)ys.n * Pm * 4) * 4); u->tb_fence[k] = mi_fence_new(); mi_fence_set(u->tb_fence[k]); }
+            u->tb_set = 0;
+            u->tb_axb = malloc((size_t)ys.n * AT_AXR(Pm) * sizeof(float));
+            if (!u->tb_axb) { fprintf(stderr, "unet: no host memory for the ray plan\n"); abort(); }
             u->tb_axdirty = 1;
             if (u->cfg.attn_axis == 1) u->tbg.rays = &u->tbr; else u->tbg.pos = u->tb_gpos;
         }
@@ -626,11 +629,17 @@ static void tb_geom(unet *u) {
             o[2 + 2 * k] = (float)((su / F + 0.5) / F - 0.5); o[3 + 2 * k] = (float)((sv / F + 0.5) / F - 0.5);      /* voxel centres at integers on both grids */
         }
     }
+    /* the tables go to the device in stream order from pinned memory: the host does not wait for the forwards still queued (a synchronous copy
+       would, and the device would then idle while the next forward is enqueued); a set is rewritten only once its own copy has run */
+    const size_t nq = (size_t)n * u->tb_Q; const int set = u->tb_set; u->tb_set ^= 1;
+    mi_fence_wait(u->tb_fence[set]);
+    u->tb_rayh = u->tb_pin[set]; u->tb_lensh = (int *)(u->tb_rayh + nq * AT_RAY_F); u->tb_adh = u->tb_lensh + nq; u->tb_cenh = (float *)(u->tb_adh + n);
     at_rays_plan(n, D, Hh, W, attn_ray_mult(), u->tb_axb, u->tb_rayh, u->tb_lensh, u->tb_adh, u->tb_cenh);
-    mi_h2d((void *)u->tbr.ray, u->tb_rayh, (size_t)n * u->tb_Q * AT_RAY_F * sizeof(float));
-    mi_h2d((void *)u->tbr.lens, u->tb_lensh, (size_t)n * u->tb_Q * sizeof(int));
-    mi_h2d((void *)u->tbr.ad, u->tb_adh, (size_t)n * sizeof(int));
-    mi_h2d(u->tb_cen, u->tb_cenh, (size_t)n * Pm * 4 * sizeof(float));
+    mi_h2d_async((void *)u->tbr.ray, u->tb_rayh, nq * AT_RAY_F * sizeof(float));
+    mi_h2d_async((void *)u->tbr.lens, u->tb_lensh, nq * sizeof(int));
+    mi_h2d_async((void *)u->tbr.ad, u->tb_adh, (size_t)n * sizeof(int));
+    mi_h2d_async(u->tb_cen, u->tb_cenh, (size_t)n * Pm * 4 * sizeof(float));
+    mi_fence_set(u->tb_fence[set]);
     if (u->cfg.attn_axis == 1) at_rays_setup(&u->tbr);
     else at_scroll_pos(n, u->tbd.nreg, D, Hh, W, u->tbr.ad, u->tb_cen, u->tb_gpos);
     u->tb_axdirty = 0;

@@ -86,6 +86,13 @@ _PROTOS = {
     "mi_free": (None, [_P]),
     "mi_zero": (None, [_P, _Z]),
     "mi_h2d": (None, [_P, _P, _Z]),
+    "mi_host_alloc": (_P, [_Z]),
+    "mi_host_free": (None, [_P]),
+    "mi_h2d_async": (None, [_P, _P, _Z]),
+    "mi_fence_new": (_P, []),
+    "mi_fence_set": (None, [_P]),
+    "mi_fence_wait": (None, [_P]),
+    "mi_fence_free": (None, [_P]),
     "mi_d2h": (None, [_P, _P, _Z]),
     "mi_d2d": (None, [_P, _P, _Z]),
     "mi_d2d_rows": (None, [_P, _Z, _P, _Z, _Z, _Z]),
