@@ -805,8 +805,10 @@ __global__ void __launch_bounds__(256) restage32_k(const uint8_t *x, uint8_t *y,
 #pragma unroll
             for (int k = 0; k < 16; k++) r[k] *= sc;
         }
+        if (gp.G) {                                               // (one uniform branch around sixteen independent chains: a select per value made sixteen blocks of one dependent chain each)
 #pragma unroll
-        for (int k = 0; k < 16; k++) r[k] = gp.G ? d_act_ab(r[k], ca[k], cb[k]) : r[k];
+            for (int k = 0; k < 16; k++) r[k] = d_act_ab(r[k], ca[k], cb[k]);
+        }
         float am = 0.f;
 #pragma unroll
         for (int k = 0; k < 16; k++) am = fmaxf(am, fabsf(r[k]));
