@@ -120,11 +120,14 @@ def test_pack_with_coordinates_and_the_length_masked_core(gpu):
     assert rel(do.to_numpy(np.float32, (T, Cc)), ro.attend(qh, kh, vh, nseq, S, None)) < 2e-3
 
 
-def test_core_on_sequences_longer_than_a_wavefront(gpu):
-    rng = np.random.default_rng(6)
-    nseq, S, Cc, H = 3, 150, 48, 1; T = nseq * S
+@pytest.mark.parametrize("nseq,S,lens", [(3, 150, (150, 97, 64)), (5, 17, (17, 3, 0, 9, 16)), (1, 32, (32,)), (7, 33, (33, 1, 32, 20, 0, 33, 7))])
+def test_core_on_other_sequence_lengths(gpu, nseq, S, lens):
+    """sequences longer than a wavefront's 64 queries, an odd number of half-wavefront units (the last wavefront's second half idles), the widths at
+    which the kernel changes from two units per wavefront to one"""
+    rng = np.random.default_rng(6 + S)
+    Cc, H = 48, 1; T = nseq * S
     qkv = rng.standard_normal((T, 3 * Cc)).astype(np.float32); ones = np.ones(Cc, np.float32)
-    lens = np.array([150, 97, 64], np.int32); dlens = DevBuf.from_numpy(lens)
+    lens = np.array(lens, np.int32); dlens = DevBuf.from_numpy(lens)
     g = at_geom(); g.nseq, g.S, g.D, g.Hh, g.W = nseq, S, 1, 1, S
     dqh = pack(qkv, ones, ones, g, 0, Cc, 0)
     got = dqh.to_numpy(np.uint16, (3, H, T + 64, 48)).view(np.float16).astype(np.float64)
