@@ -39,83 +39,93 @@ __global__ void __launch_bounds__(256, 2) conv2_mx_k(const conv_args a) {
     }
     const uint8_t *xq = a.xq[0] + (size_t)n * nb * Sin * RB, *xsc = a.xsc[0] + (size_t)n * nb * Sin;
     // the activation fragment of tile j for the K pair (block b0 at voxel offset o0 | block b1 at o1; ok1: the second unit exists)
-    struct bfrag { v8i f; int sb; };
+    struct bfrag { v4i lo, hi; int sb; };
     auto fetch = [&](int j, int b0, size_t o0, int b1, size_t o1, bool ok1) {
         bfrag q;
         const size_t v0 = (size_t)b0 * Sin + iv0[j] + o0, v1 = (size_t)b1 * Sin + iv0[j] + o1;
+        const v4i z4 = {0, 0, 0, 0};
         if constexpr (FMT == 8) {
-            const v4i lo = *(const v4i *)(xq + v0 * RB + 16 * h);
-            v4i hi = {0, 0, 0, 0};
-            if (ok1) hi = *(const v4i *)(xq + v1 * RB + 16 * h);
-            q.f = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            q.lo = *(const v4i *)(xq + v0 * RB + 16 * h);
+            q.hi = *(const v4i *)(xq + v1 * RB + 16 * h);    // (ok1 false: v1 is v0's row again, its codes dropped)
+            q.hi = ok1 ? q.hi : z4;
         } else {
-            v4i lo = {0, 0, 0, 0};
-            if (!h || ok1) lo = *(const v4i *)(xq + (h ? v1 : v0) * RB);
-            q.f = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+            q.lo = *(const v4i *)(xq + (h ? v1 : v0) * RB);
+            q.lo = (!h || ok1) ? q.lo : z4; q.hi = z4;
         }
         q.sb = h ? (ok1 ? (int)xsc[v1] : 127) : (int)xsc[v0];
         return q;
     };
-    struct afrag { v8i f; int s; };
+    struct afrag { v4i lo, hi; int s; };
     auto wfetch = [&](int gp, int m) {
         afrag q;
         const size_t t = (size_t)gp * a.nmt_all + cs * MT + m;
-        const v4i lo = *(const v4i *)(a.wq + t * WTILE + lane * 16);
-        if constexpr (FMT == 8) { const v4i hi = *(const v4i *)(a.wq + t * WTILE + 1024 + lane * 16); q.f = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]}; }
-        else q.f = (v8i){lo[0], lo[1], lo[2], lo[3], 0, 0, 0, 0};
+        q.lo = *(const v4i *)(a.wq + t * WTILE + lane * 16);
+        if constexpr (FMT == 8) q.hi = *(const v4i *)(a.wq + t * WTILE + 1024 + lane * 16); else q.hi = (v4i){0, 0, 0, 0};
         q.s = *(const int *)(a.wsc + (t * 64 + lane) * 4);
         return q;
     };
     v16f acc[MT][NT];
-    auto clear = [&]() {
+#pragma unroll
+    for (int m = 0; m < MT; m++)
+#pragma unroll
+        for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
+    // register rings: the weights of pair p + 1 (cache hits) and the rows of pairs p + 1 .. p + AR - 1 (HBM) are in flight while pair p is multiplied.
+    // A wavefront has two MFMAs per channel tile and pair to hide a load's latency behind, so the launch runs at bytes in flight / latency: an
+    // e2m1 row set is 10 registers, and four of them fit beside the accumulators
+    constexpr int AR = FMT == 4 ? 4 : 2;
+    bfrag fb[AR][NT]; afrag fa[2][MT];
+    const int t_up = UP ? (int)(blockIdx.y / (unsigned)a.ncs) : 0, npt = (nb + 1) >> 1;      // up: one tap per workgroup (eight times the workgroups, the rows re-read through the L2)
+    const int np = UP ? npt : 4 * nb;                        // down: 8 taps x nb blocks, in pairs, tap-major
+    auto request_rows = [&](int p, auto SET) {
+        constexpr int set = decltype(SET)::value;
+        if constexpr (UP) {
+            const bool ok1 = 2 * p + 1 < nb;
+#pragma unroll
+            for (int j = 0; j < NT; j++) fb[set][j] = fetch(j, 2 * p, 0, ok1 ? 2 * p + 1 : 2 * p, 0, ok1);
+        } else {
+            const int u0 = 2 * p, u1 = u0 + 1, t0 = u0 / nb, b0 = u0 - t0 * nb, t1 = u1 / nb, b1 = u1 - t1 * nb;
+            const size_t o0 = ((size_t)(t0 >> 2) * a.H + ((t0 >> 1) & 1)) * a.W + (t0 & 1), o1 = ((size_t)(t1 >> 2) * a.H + ((t1 >> 1) & 1)) * a.W + (t1 & 1);
+#pragma unroll
+            for (int j = 0; j < NT; j++) fb[set][j] = fetch(j, b0, o0, b1, o1, true);
+        }
+    };
+    auto request_weights = [&](int p, auto SET) {
+        constexpr int set = decltype(SET)::value;
+#pragma unroll
+        for (int m = 0; m < MT; m++) fa[set][m] = wfetch(UP ? t_up * npt + p : p, m);
+    };
+    auto multiply = [&](auto BS, auto AS) {
+        constexpr int bs = decltype(BS)::value, as = decltype(AS)::value;
 #pragma unroll
         for (int m = 0; m < MT; m++)
 #pragma unroll
-            for (int j = 0; j < NT; j++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) acc[m][j][i] = 0.f;
-    };
-    auto step = [&](int gp, const bfrag (&fb)[NT]) {
-#pragma unroll
-        for (int m = 0; m < MT; m++) {
-            const afrag fa = wfetch(gp, m);
-#pragma unroll
-            for (int j = 0; j < NT; j++)
-                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa.f, fb[j].f, acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, fa.s, 0, fb[j].sb);
-        }
-    };
-    long long ovx[NT];
-    if constexpr (!UP) {
-        clear();
-        const int np = 4 * nb;                               // 8 taps x nb blocks, in pairs
-        for (int p = 0; p < np; p++) {
-            const int u0 = 2 * p, u1 = u0 + 1, t0 = u0 / nb, b0 = u0 - t0 * nb, t1 = u1 / nb, b1 = u1 - t1 * nb;
-            const size_t o0 = ((size_t)(t0 >> 2) * a.H + ((t0 >> 1) & 1)) * a.W + (t0 & 1), o1 = ((size_t)(t1 >> 2) * a.H + ((t1 >> 1) & 1)) * a.W + (t1 & 1);
-            bfrag fb[NT];
-#pragma unroll
-            for (int j = 0; j < NT; j++) fb[j] = fetch(j, b0, o0, b1, o1, true);
-            step(p, fb);
-        }
-#pragma unroll
-        for (int j = 0; j < NT; j++) ovx[j] = cok[j] ? (ct0 + j) * 32 + r : -1;
-        conv_epilogue<MT, NT, OUT, false, false, false, false, true, 4, true>(a, acc, lds, 0u, n, cs, 0, 0, 0, 0, 0, tid, ovx);
-    } else {
-        const int npt = (nb + 1) >> 1;
-        {
-            const int t = (int)(blockIdx.y / (unsigned)a.ncs);   // one tap per workgroup: eight times the workgroups, the rows re-read through the L2
-            clear();
-            for (int pp = 0; pp < npt; pp++) {
-                bfrag fb[NT];
-#pragma unroll
-                for (int j = 0; j < NT; j++) fb[j] = fetch(j, 2 * pp, 0, 2 * pp + 1 < nb ? 2 * pp + 1 : 2 * pp, 0, 2 * pp + 1 < nb);
-                step(t * npt + pp, fb);
+            for (int j = 0; j < NT; j++) {
+                const v8i A = {fa[as][m].lo[0], fa[as][m].lo[1], fa[as][m].lo[2], fa[as][m].lo[3], fa[as][m].hi[0], fa[as][m].hi[1], fa[as][m].hi[2], fa[as][m].hi[3]};
+                const v8i B = {fb[bs][j].lo[0], fb[bs][j].lo[1], fb[bs][j].lo[2], fb[bs][j].lo[3], fb[bs][j].hi[0], fb[bs][j].hi[1], fb[bs][j].hi[2], fb[bs][j].hi[3]};
+                acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A, B, acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, fa[as][m].s, 0, fb[bs][j].sb);
             }
-#pragma unroll
-            for (int j = 0; j < NT; j++)
-                ovx[j] = cok[j] ? ((long long)(2 * c0[j] + (t >> 2)) * a.Ho + 2 * c1[j] + ((t >> 1) & 1)) * a.Wo + 2 * c2[j] + (t & 1) : -1;
-            conv_epilogue<MT, NT, OUT, false, false, false, false, true, 4, true>(a, acc, lds, 0u, n, cs, 0, 0, 0, 0, 0, tid, ovx);
-        }
+    };
+    static_for<AR - 1>([&](auto I) { if (decltype(I)::value < np) request_rows(decltype(I)::value, I); });
+    request_weights(0, std::integral_constant<int, 0>{});
+    for (int p = 0; p < np; p += AR) {                       // (uniform branches)
+        static_for<AR>([&](auto I) {
+            constexpr int i = decltype(I)::value;
+            if (p + i < np) {
+                if (p + i + AR - 1 < np) request_rows(p + i + AR - 1, std::integral_constant<int, (i + AR - 1) % AR>{});
+                if (p + i + 1 < np) request_weights(p + i + 1, std::integral_constant<int, (i + 1) % 2>{});
+                multiply(I, std::integral_constant<int, i % 2>{});
+            }
+        });
     }
+    long long ovx[NT];
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+        if constexpr (UP) ovx[j] = cok[j] ? ((long long)(2 * c0[j] + (t_up >> 2)) * a.Ho + 2 * c1[j] + ((t_up >> 1) & 1)) * a.Wo + 2 * c2[j] + (t_up & 1) : -1;
+        else ovx[j] = cok[j] ? (ct0 + j) * 32 + r : -1;
+    }
+    conv_epilogue<MT, NT, OUT, false, false, false, false, true, 4, true>(a, acc, lds, 0u, n, cs, 0, 0, 0, 0, 0, tid, ovx);
 }
 
 // ---- the 3x3x3 stride-2 conv (src/lp_s2.cu:4-9) read the same way: no LDS staging, every tap's rows straight from the stored tensor ----
