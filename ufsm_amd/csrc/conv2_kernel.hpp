@@ -107,14 +107,15 @@ __global__ void __launch_bounds__(256, 2) conv2_mx_k(const conv_args a) {
                 acc[m][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(A, B, acc[m][j], FMT == 8 ? 0 : 4, FMT == 8 ? 0 : 4, 0, fa[as][m].s, 0, fb[bs][j].sb);
             }
     };
-    static_for<AR - 1>([&](auto I) { if (decltype(I)::value < np) request_rows(decltype(I)::value, I); });
     request_weights(0, std::integral_constant<int, 0>{});
+    static_for<AR - 1>([&](auto I) { if (decltype(I)::value < np) request_rows(decltype(I)::value, I); });
     for (int p = 0; p < np; p += AR) {                       // (uniform branches)
         static_for<AR>([&](auto I) {
             constexpr int i = decltype(I)::value;
             if (p + i < np) {
-                if (p + i + AR - 1 < np) request_rows(p + i + AR - 1, std::integral_constant<int, (i + AR - 1) % AR>{});
+                // (the weights first: loads return in order, so waiting for the next pair's weights also waits for everything requested before them)
                 if (p + i + 1 < np) request_weights(p + i + 1, std::integral_constant<int, (i + 1) % 2>{});
+                if (p + i + AR - 1 < np) request_rows(p + i + AR - 1, std::integral_constant<int, (i + AR - 1) % AR>{});
                 multiply(I, std::integral_constant<int, i % 2>{});
             }
         });
