@@ -245,14 +245,15 @@ def hbm_leg(np, lib, LP, DevBuf):
         ("up2_mx_k (trilinear 2x, 64 ch, 64^3 -> 128^3)", mx(Cc, Sc) + mx(Cc, S), lambda: lib.lp_up2_fwd_mx(qc.ptr, 3, shape5(N, Cc, D // 2, D // 2, D // 2), qu.ptr, 3, gnp_t())),
         ("conv3_stem_k (3x3x3 stem 4 -> 32, MX-fp8 in / out)", mx(4, S) + mx(C, S), lambda: lib.lp_conv_fwd_f8(q4.ptr, 3, shape5(N, 4, D, D, D), ws.ptr, bs.ptr, C, q2.ptr, 3, gnp_t(), None, 0, sp)),
     ]
-    # configs[2]'s stride-2 layers in MX-fp4 (N 2): 2x2x2 down conv 128 -> 256 from 64^3 and 2x2x2 transposed conv 256 -> 128 from 32^3 (weights prepared per call)
+    # configs[2]'s stride-2 layers in MX-fp4 (N 2): 2x2x2 down conv 128 -> 256 from 64^3 and 2x2x2 transposed conv 256 -> 128 from 32^3 (weights prepared once
+    # under a memo id, as an inference loop keeps them: mi_conv_s2_wkey)
     mx4 = lambda c, s: N * ((c + 31) // 32) * s * 17
     xd = DevBuf.from_numpy(rng.uniform(-3, 3, (N, 128, 64 ** 3)).astype(np.float32)); qd = DevBuf(lib.lp_mx4_bytes(N, 128, 64 ** 3)); lib.lp_f32_to_mx4(xd.ptr, N, 128, 64 ** 3, qd.ptr)
     yd = DevBuf(lib.lp_mx4_bytes(N, 256, 32 ** 3)); yu = DevBuf(lib.lp_mx4_bytes(N, 128, 64 ** 3))
     wd = DevBuf.from_numpy((rng.standard_normal((256, 128, 8)) * 0.04).astype(np.float32))
     cases += [
-        ("conv2_mx_k (2x2x2 stride-2 down conv 128 -> 256, 64^3 in, MX-fp4)", mx4(128, 64 ** 3) + mx4(256, 32 ** 3), lambda: lib.mi_conv_down2_fwd(4, qd.ptr, 4, shape5(N, 128, 64, 64, 64), wd.ptr, None, 256, yd.ptr, 4, gnp_t())),
-        ("conv2_mx_k (2x2x2 stride-2 transposed conv 256 -> 128, 32^3 in, MX-fp4)", mx4(256, 32 ** 3) + mx4(128, 64 ** 3), lambda: lib.mi_convt_up2_fwd(4, yd.ptr, 4, shape5(N, 256, 32, 32, 32), wd.ptr, None, 128, yu.ptr, 4, gnp_t())),
+        ("conv2_mx_k (2x2x2 stride-2 down conv 128 -> 256, 64^3 in, MX-fp4)", mx4(128, 64 ** 3) + mx4(256, 32 ** 3), lambda: (lib.mi_conv_s2_wkey(902), lib.mi_conv_down2_fwd(4, qd.ptr, 4, shape5(N, 128, 64, 64, 64), wd.ptr, None, 256, yd.ptr, 4, gnp_t()))),
+        ("conv2_mx_k (2x2x2 stride-2 transposed conv 256 -> 128, 32^3 in, MX-fp4)", mx4(256, 32 ** 3) + mx4(128, 64 ** 3), lambda: (lib.mi_conv_s2_wkey(903), lib.mi_convt_up2_fwd(4, yd.ptr, 4, shape5(N, 256, 32, 32, 32), wd.ptr, None, 128, yu.ptr, 4, gnp_t()))),
     ]
     rows = []
     for name, nbytes, call in cases:

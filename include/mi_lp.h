@@ -79,7 +79,8 @@ void nn_gfilm_pool(const float *x, int C, long S, float *g);
 void nn_gfilm_fwd(const float *p, float *fw, size_t gam, size_t bet, size_t fo, int C, int K, const float *gv, float *g1);
 void nn_ws_fwd(float *wh, const float *w, int cout, int n, float gain, float eps);
 /* no counterpart in the reference (its stride-2 entry carries no split_t and prepares the weights per call): memo id of the calling thread's
-   next lp_conv_fwd_s2_f8, as split_t.wkey for the stride-1 entries; consumed by that call. For inference loops with constant weights. */
+   next lp_conv_fwd_s2_f8, mi_conv_down2_fwd or mi_convt_up2_fwd, as split_t.wkey for the stride-1 entries; consumed by that call. For inference
+   loops with constant weights (lp_wmemo_step / lp_wmemo_clear drop the prepared images as for the other convs). */
 void mi_conv_s2_wkey(unsigned wkey);
 /* Tuning knob of the tap-packed kernel for <= 4 input channels: consecutive z tiles a workgroup walks (weights and constants set up once,
  * the next tile's input in flight during this tile's MFMAs). 0 (default) = chosen from the launch size. Results do not depend on it.

@@ -91,6 +91,43 @@ def test_config2_layers_at_full_size(gpu):
         assert (gq != wq).mean() < 1e-4, (up, (gq != wq).mean())
 
 
+@pytest.mark.parametrize("up", [0, 1])
+def test_weight_memo(gpu, up):
+    """mi_conv_s2_wkey: the prepared weights are kept under the caller's id (no second preparation, no further allocation), give the bytes of the
+    per-call preparation, are told apart by direction, and are dropped by a new weight step."""
+    rng = np.random.default_rng(81 + up)
+    N, Ci, Co, D, H, W = 1, 64, 64, 4, 4, 8
+    S = D * H * W
+    x = rng.standard_normal((N, Ci, S)).astype(np.float32)
+    w = (rng.standard_normal((Ci, Co, 8) if up else (Co, Ci, 8)) * 0.1).astype(np.float32)
+    xq = orc.f32_to_mx(8, x, N, Ci, S)
+    So = 8 * S if up else S // 8
+    dx, dw, dy = DevBuf.from_numpy(xq), DevBuf.from_numpy(w), DevBuf(mx_bytes(8, N, Co, So))
+    f = lib.mi_convt_up2_fwd if up else lib.mi_conv_down2_fwd
+
+    def run(key):
+        if key:
+            lib.mi_conv_s2_wkey(key)
+        assert f(8, dx.ptr, 3, shape5(N, Ci, D, H, W), dw.ptr, None, Co, dy.ptr, 3, gnp_t()) == 0
+        LP.check()
+        return dy.to_numpy(np.uint8).copy()
+
+    lib.lp_wmemo_clear()
+    plain = run(0)
+    first = run(777)
+    allocs = lib.mi_alloc_count()
+    second = run(777)
+    assert lib.mi_alloc_count() == allocs
+    assert np.array_equal(plain, first) and np.array_equal(plain, second)
+    w2 = np.ascontiguousarray(-2 * w)
+    lib.mi_h2d(dw.ptr, w2.ctypes.data, w2.nbytes)
+    assert np.array_equal(run(777), plain)                        # (the kept image: the caller said the weights are constant)
+    assert np.array_equal(run(0), run(0)) and not np.array_equal(run(0), plain)      # the id was consumed by its call: these prepare per call
+    lib.lp_wmemo_step(12345)                                      # weights changed: a new step drops the memo (src/nn_lp.h:56)
+    assert np.array_equal(run(777), run(0))
+    lib.lp_wmemo_clear(); lib.lp_wmemo_step(0)
+
+
 def test_refusals(gpu):
     x = DevBuf(1 << 16); w = DevBuf(1 << 16); y = DevBuf(1 << 20)
     assert lib.mi_conv_down2_fwd(8, x.ptr, 3, shape5(1, 32, 3, 4, 4), w.ptr, None, 32, y.ptr, 3, gnp_t()) == -1      # odd depth

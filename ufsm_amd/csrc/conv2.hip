@@ -2,6 +2,9 @@
 #include "conv2_kernel.hpp"
 #include "../../include/mi_lp.h"
 
+bool mi_wmemo_other(unsigned key, const float *w, int fmt, int Co, int Ci, int nmt_all, int lay, size_t wq_bytes, size_t wsc_bytes, uint8_t **wq, uint8_t **wsc);     // conv3.hip
+unsigned mi_take_s2_wkey(void);
+
 // weights -> the MFMA's lane order, one tile per (K pair, channel tile) as the 3x3x3 kernels read them. down: w [Co][Ci][8], pair gp = units 2 gp,
 // 2 gp + 1 of the tap-major (tap, block) order; up: w [Ci][Co][8], pair gp = (tap gp / npt, blocks 2 (gp % npt), + 1), a missing second block = zeros
 template <int FMT>
@@ -52,11 +55,18 @@ static int conv2_dispatch(const char *who, int up, int bits, const void *x, int 
     a.Do = up ? 2 * D : D / 2; a.Ho = up ? 2 * H : H / 2; a.Wo = up ? 2 * W : W / 2;
     const int nmt_all = (cout + 31) / 32, npairs = up ? 8 * ((nbp + 1) / 2) : 4 * nbp;
     const int MT = nmt_all % 4 == 0 ? 4 : nmt_all % 2 == 0 ? 2 : 1;
-    uint8_t *wq = (uint8_t *)mi_ws(MI_WS_WQ, (size_t)npairs * nmt_all * WTILE), *wsc = (uint8_t *)mi_ws(MI_WS_WSC, (size_t)npairs * nmt_all * 256);
-    const size_t nt = (size_t)npairs * nmt_all * 32;
-    if (fmt == 8) prep_w2_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, nbp, nmt_all, npairs, up);
-    else prep_w2_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, nbp, nmt_all, npairs, up);
-    MICK();
+    // prepared weights: per call into the scratch, or once under the memo id the calling thread set for this call (mi_conv_s2_wkey)
+    const size_t wq_bytes = (size_t)npairs * nmt_all * WTILE, wsc_bytes = (size_t)npairs * nmt_all * 256;
+    const unsigned wkey = mi_take_s2_wkey();
+    uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
+    if (wkey && !mi_ws_arena_on()) have = mi_wmemo_other(wkey, w, fmt, cout, Ci, nmt_all, up ? 2 : 1, wq_bytes, wsc_bytes, &wq, &wsc);
+    else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
+    if (!have) {
+        const size_t nt = (size_t)npairs * nmt_all * 32;
+        if (fmt == 8) prep_w2_k<8><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, nbp, nmt_all, npairs, up);
+        else prep_w2_k<4><<<nblk_(nt, 128), 128>>>(w, wq, (unsigned *)wsc, cout, Ci, nbp, nmt_all, npairs, up);
+        MICK();
+    }
     a.wq = wq; a.wsc = wsc; a.nmt_all = nmt_all; a.ncs = nmt_all / MT;
     a.bias = b; a.Co = cout; a.y = y; a.ydt = ybf;
     a.zs0 = 0; a.zs1 = a.Do;

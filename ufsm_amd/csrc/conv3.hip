@@ -184,6 +184,18 @@ static int g_w2d = -1;
 static int g_w2d_on(void) { if (g_w2d < 0) g_w2d = getenv("UFSM_W4_2D") ? atoi(getenv("UFSM_W4_2D")) : 0; return g_w2d; }
 extern "C" void lp_set_w4_2d(int on) { g_w2d = on ? 1 : 0; lp_wmemo_clear(); }
 extern "C" void lp_wmemo_step(unsigned step) { if (step != g_wstep) { g_wstep = step; lp_wmemo_clear(); } }
+// memo entries of the layouts other source files prepare (the 2x2x2 stride-2 convs: nbt = -100, lay = down / up): the image's buffers for
+// (key, weights, format, shape, lay) on the current device, allocated on first use; returns whether they already hold the prepared image
+bool mi_wmemo_other(unsigned key, const float *w, int fmt, int Co, int Ci, int nmt_all, int lay, size_t wq_bytes, size_t wsc_bytes, uint8_t **wq, uint8_t **wsc) {
+    int dev = 0; MIRT(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_wmemo_mu);
+    for (auto &m : g_wmemo)
+        if (m.key == key && m.w == w && m.fmt == fmt && m.Co == Co && m.Ci == Ci && m.nbt == -100 && m.nmt_all == nmt_all && m.dev == dev && m.lay == lay) { *wq = m.wq; *wsc = m.wsc; return true; }
+    MIRT(hipMalloc((void **)wq, wq_bytes)); MIRT(hipMalloc((void **)wsc, wsc_bytes)); mi_count_alloc(); mi_count_alloc();
+    if (!*wq || !*wsc) mi_die("no device memory for the prepared weights of a 2x2x2 conv");
+    g_wmemo.push_back(wmemo_t{key, w, fmt, Co, Ci, Ci, -100, 0, nmt_all, dev, lay, *wq, *wsc});
+    return false;
+}
 
 thread_local char g_last_kernel[128] = "";
 
@@ -612,9 +624,10 @@ extern "C" int lp_conv_fwd_f8(const void *x, int xbf, shape5 xs, const float *w,
 extern "C" int lp_conv_fwd_f4(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp, double *osum, int Go, split_t sp) {
     return conv_dispatch("lp_conv_fwd_f4", 4, 1, x, xbf, xs, w, b, cout, y, ybf, gp, osum, Go, sp, nullptr, nullptr, 0);
 }
-// prepared-weight memo id of the calling thread's next stride-2 conv (its signature carries no split_t): 0 = prepare per call
+// prepared-weight memo id of the calling thread's next stride-2 conv, 3x3x3 or 2x2x2 (their signatures carry no split_t): 0 = prepare per call
 static thread_local unsigned g_s2_wkey = 0;
 extern "C" void mi_conv_s2_wkey(unsigned wkey) { g_s2_wkey = wkey; }
+unsigned mi_take_s2_wkey(void) { const unsigned k = g_s2_wkey; g_s2_wkey = 0; return k; }      // (the 2x2x2 entries consume it too)
 extern "C" void mi_conv_stem_zc(int zc) { g_stem_zc = zc; }
 extern "C" int lp_conv_fwd_s2_f8(const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, shape5 ys, gnp_t gp) {
     const int Do = (xs.d - 1) / 2 + 1, Ho = (xs.h - 1) / 2 + 1, Wo = (xs.w - 1) / 2 + 1;
