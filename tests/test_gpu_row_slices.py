@@ -1,0 +1,41 @@
+"""The row kernel with two channel slices (33 .. 64 output channels from two or more input blocks): one slice per workgroup."""
+import numpy as np
+import pytest
+
+from ufsm_amd import lib
+import orc
+from test_gpu_conv import exact_case, rand_case, gpu_conv
+
+pytestmark = pytest.mark.gpu
+
+ROW_CS_SHAPES = [(8, 1, 64, 64, 8, 12, 20), (8, 2, 64, 64, 16, 16, 64), (8, 1, 96, 48, 5, 9, 40), (4, 1, 64, 64, 8, 12, 48), (4, 2, 96, 64, 6, 9, 34),
+                 (8, 2, 64, 64, 64, 64, 64), (4, 3, 64, 40, 12, 64, 128)]
+
+
+@pytest.mark.parametrize("bits,N,Ci,Co,D,H,W", ROW_CS_SHAPES)
+def test_row_kernel_two_channel_slices(gpu, bits, N, Ci, Co, D, H, W):
+    rng = np.random.default_rng(Ci * 5 + Co + D + W)
+    S = D * H * W
+    xdt = 3 if bits == 8 else 4
+    x, w, b = exact_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    want, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, acc64=1)
+    got, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits)
+    assert "two channel slices" in lib.mi_last_kernel().decode(), lib.mi_last_kernel().decode()
+    assert np.array_equal(got, want)
+    for ydt in (2, 3, 4):
+        wq, _ = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=bits, acc64=1)
+        gq, _ = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, ydt, cbits=bits)
+        assert np.array_equal(gq, wq), ydt
+    if S * N > 600000:                                            # (the large cases: exact operands only)
+        return
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    xq = orc.f32_to_mx(bits, x, N, Ci, S)
+    G = 8 if Co % 32 == 0 else 2                                  # (channels per group a multiple of 4, or the launch leaves this kernel)
+    want, ws = orc.conv3(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, Go=G, want_stats=True)
+    got, gs = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, Go=G, stats=True)
+    assert "two channel slices" in lib.mi_last_kernel().decode()
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-4
+    assert np.abs(gs - ws).max() / np.abs(ws).max() < 1e-5
+    got2, gs2 = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, Go=G, stats=True)
+    assert np.array_equal(got, got2) and np.array_equal(gs, gs2)

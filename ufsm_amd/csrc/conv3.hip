@@ -520,8 +520,13 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // one half's epilogue runs under the other's MFMAs (MI_CONV_ROW1=0: the small-channel kernel)
     static int row1_env = -1;
     if (row1_env < 0) row1_env = getenv("MI_CONV_ROW1") ? atoi(getenv("MI_CONV_ROW1")) : 1;
-    a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && nmt_all == 1 && stride == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 || row1_env ? 1 : 2) && a.nbt <= 64;
+    // ... and 33 .. 64 output channels from two or more input blocks run it as two channel slices, one per workgroup (MI_CONV_ROW_CS=0: the general kernel)
+    static int rowcs_env = -1;
+    if (rowcs_env < 0) rowcs_env = getenv("MI_CONV_ROW_CS") ? atoi(getenv("MI_CONV_ROW_CS")) : 1;
+    const bool row_cs = rowcs_env && nmt_all == 2 && MT == 2 && a.nbt >= 2;
+    a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && (nmt_all == 1 || row_cs) && stride == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 || row1_env ? 1 : 2) && a.nbt <= 64;
     a.row1 = a.row && a.nbt == 1 && row1_env && row_env < 2;
+    if (a.row && nmt_all == 2) MT = 1;
     if (a.row) { a.areg = false; a.CB = a.nbt; }
     size_t smem = a.row1 ? (size_t)10 * 352 * (RB + 4) : a.row ? (size_t)2 * 2048 * (RB + 4) : a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     if (s2d) smem = 0;

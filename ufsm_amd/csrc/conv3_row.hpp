@@ -47,11 +47,15 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
     const size_t wq_ps = (size_t)a.nmt_all * WTILE, wsc_ps = (size_t)a.nmt_all * 256;
 
     // XCD-aware persistent tile walk: workgroup ids go round robin over the 8 XCDs, each XCD owns a contiguous range of tiles
-    const unsigned per = (a.ntiles + 7u) / 8u, wg_per_xcd = gridDim.x >> 3, xcd = blockIdx.x & 7u, wix = blockIdx.x >> 3;
+    // Two channel tiles (33 .. 64 output channels): a workgroup keeps ONE of them for its whole walk (bias, weights and statistics records of
+    // slice cs), and neighbouring workgroups of an XCD take the same spatial tiles in the other slice, so the halo's second read finds the L2
+    const unsigned ncs = (unsigned)a.ncs, nsp = a.ntiles / ncs;                      // channel slices; spatial tiles
+    const int cs = __builtin_amdgcn_readfirstlane((int)((blockIdx.x >> 3) % ncs));
+    const unsigned per = (nsp + 7u) / 8u, wg_per_xcd = (gridDim.x >> 3) / ncs, xcd = blockIdx.x & 7u, wix = (blockIdx.x >> 3) / ncs;
     struct tile_t { unsigned tile; int n, oz0, oy0, ox0; bool ok; };
     auto decode = [&](unsigned it) {
         tile_t t; const unsigned k = wix + it * wg_per_xcd;
-        t.ok = k < per && xcd * per + k < a.ntiles;
+        t.ok = k < per && xcd * per + k < nsp;
         t.tile = t.ok ? xcd * per + k : 0u;
         int tt = (int)t.tile;
         const int tx = tt % a.ntx; tt /= a.ntx;
@@ -85,7 +89,7 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
         if constexpr (NH == 2) dma16(row + 16, lds0 + bo + (unsigned)TTP * 16u + (unsigned)g * 1024u);
         dma1(sc, lds0 + bo + (unsigned)(NH * TTP * 16) + (unsigned)g * 256u);
     };
-    conv_epi_consts<1, EPI>(a, lds, 0, tid);
+    conv_epi_consts<1, EPI>(a, lds, cs, tid);
 #pragma unroll
     for (int rd = 0; rd < NRND; rd++) request(cur, 0, 0u, rd, true);
 
@@ -96,7 +100,7 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
         const size_t wq_ps0 = (size_t)a.nmt_all * WTILE, wsc_ps0 = (size_t)a.nmt_all * 256;
         for (int i = tid; i < a.nbt * NPB * (WPB / 16); i += NW * 64) {
             const int p = i / (WPB / 16), k = i - p * (WPB / 16);
-            const v4i v = k < 64 ? *(const v4i *)(a.wq + (size_t)p * wq_ps0 + k * 16) : *(const v4i *)(a.wsc + (size_t)p * wsc_ps0 + (k - 64) * 16);
+            const v4i v = k < 64 ? *(const v4i *)(a.wq + (size_t)p * wq_ps0 + (size_t)cs * WTILE + k * 16) : *(const v4i *)(a.wsc + (size_t)p * wsc_ps0 + (size_t)cs * 256 + (k - 64) * 16);
             *(v4i *)(lds + a.wl_o + p * WPB + k * 16) = v;
         }
     }
@@ -113,7 +117,7 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
             }
             return w;
         }
-        const uint8_t *wp = a.wq + ((size_t)b * NPB + c * 3) * wq_ps + lane * 16, *sp = a.wsc + ((size_t)b * NPB + c * 3) * wsc_ps + lane * 4;
+        const uint8_t *wp = a.wq + ((size_t)b * NPB + c * 3) * wq_ps + (size_t)cs * WTILE + lane * 16, *sp = a.wsc + ((size_t)b * NPB + c * 3) * wsc_ps + (size_t)cs * 256 + lane * 4;
 #pragma unroll
         for (int ky = 0; ky < 3; ky++) {
             const v4i lo = *(const v4i *)(wp + ky * wq_ps);
@@ -197,8 +201,8 @@ __global__ void __launch_bounds__(512, 1) conv3_row_k(const conv_args a) {
         ws[1] = ws[0]; ws[0] = ws[2];                           // the next step's classes 1 and 0
         if (last_b) {
             if (cur.oz0 + TZ <= a.Do && cur.oy0 + TY <= a.Ho && cur.ox0 + TX <= a.Wo && a.zs0 <= cur.oz0 && a.zs1 >= cur.oz0 + TZ)      // (uniform)
-                conv_epilogue<1, NT, OUT, EPI, false, true, true, true, NW, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
-            else conv_epilogue<1, NT, OUT, EPI, false, true, false, true, NW, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+                conv_epilogue<1, NT, OUT, EPI, false, true, true, true, NW, true>(a, acc, lds, cur.tile * ncs + cs, cur.n, cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+            else conv_epilogue<1, NT, OUT, EPI, false, true, false, true, NW, true>(a, acc, lds, cur.tile * ncs + cs, cur.n, cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
             if (!nxt.ok) break;
             cur = nxt; it++;
 #pragma unroll
@@ -221,9 +225,9 @@ static void launch_row(const conv_args &a, size_t smem) {
         ncu[d] = pr.multiProcessorCount > 8 ? pr.multiProcessorCount & ~7 : 8;
         attr[d] = true;
     }
-    const unsigned per = (a.ntiles + 7u) / 8u;            // tiles per XCD; one persistent workgroup per CU, a multiple of 8 in all
-    const unsigned nwg = per * 8u < (unsigned)ncu[d] ? per * 8u : (unsigned)ncu[d];
+    const unsigned ncs = (unsigned)a.ncs, per = (a.ntiles / ncs + 7u) / 8u;            // spatial tiles per XCD; one persistent workgroup per CU, a multiple of 8 x slices in all
+    const unsigned cap = (unsigned)ncu[d] / (8u * ncs) * (8u * ncs), nwg = per * 8u * ncs < cap ? per * 8u * ncs : cap;
     conv3_row_k<FMT, OUT, EPI, WL><<<nwg, 512, smem>>>(a);
     MICK();
-    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row_k<fmt %d, out %d, epi %d%s> blocks %d tiles %u wgs %u", FMT, OUT, (int)EPI, WL ? ", weights in LDS" : "", a.nbt, a.ntiles, nwg);
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row_k<fmt %d, out %d, epi %d%s> blocks %d tiles %u%s wgs %u", FMT, OUT, (int)EPI, WL ? ", weights in LDS" : "", a.nbt, a.ntiles, ncs > 1 ? " (two channel slices)" : "", nwg);
 }
