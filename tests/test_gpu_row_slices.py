@@ -1,4 +1,6 @@
-"""The row kernel with two channel slices (33 .. 64 output channels from two or more input blocks): one slice per workgroup."""
+"""The row kernels with two channel slices (33 .. 64 output channels from one to three input blocks: one slice per workgroup, the one-block
+kernel for a single input block): exact operands equal the oracle in every output type, random operands meet the conv tolerance, the statistics
+are the oracle's and identical run to run."""
 import numpy as np
 import pytest
 
@@ -8,7 +10,8 @@ from test_gpu_conv import exact_case, rand_case, gpu_conv
 
 pytestmark = pytest.mark.gpu
 
-ROW_CS_SHAPES = [(8, 1, 64, 64, 8, 12, 20), (8, 2, 64, 64, 16, 16, 64), (8, 1, 96, 48, 5, 9, 40), (4, 1, 64, 64, 8, 12, 48), (4, 2, 96, 64, 6, 9, 34),
+ROW_CS_SHAPES = [(8, 2, 32, 64, 8, 16, 32), (8, 1, 32, 48, 5, 9, 40), (4, 1, 32, 64, 8, 12, 48), (8, 2, 32, 64, 64, 64, 64), (8, 3, 32, 64, 12, 64, 128), (4, 2, 20, 40, 6, 9, 34),
+                 (8, 1, 64, 64, 8, 12, 20), (8, 2, 64, 64, 16, 16, 64), (8, 1, 96, 48, 5, 9, 40), (4, 1, 64, 64, 8, 12, 48), (4, 2, 96, 64, 6, 9, 34),
                  (8, 2, 64, 64, 64, 64, 64), (4, 3, 64, 40, 12, 64, 128)]
 
 

@@ -520,10 +520,12 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // one half's epilogue runs under the other's MFMAs (MI_CONV_ROW1=0: the small-channel kernel)
     static int row1_env = -1;
     if (row1_env < 0) row1_env = getenv("MI_CONV_ROW1") ? atoi(getenv("MI_CONV_ROW1")) : 1;
-    // ... and 33 .. 64 output channels from two or more input blocks run it as two channel slices, one per workgroup (MI_CONV_ROW_CS=0: the general kernel)
+    // ... and 33 .. 64 output channels from one to three input blocks run the two row kernels as two channel slices, one per workgroup (MI_CONV_ROW_CS=0:
+    // the general kernel). Measured at 2 x 64^3 in e4m3: 32 -> 64 0.046 -> 0.039 ms, 64 -> 64 0.073 -> 0.067 ms, 96 -> 64 0.100 -> 0.095 ms; from four
+    // blocks on the wide kernel keeps these layers
     static int rowcs_env = -1;
     if (rowcs_env < 0) rowcs_env = getenv("MI_CONV_ROW_CS") ? atoi(getenv("MI_CONV_ROW_CS")) : 1;
-    const bool row_cs = rowcs_env && nmt_all == 2 && MT == 2 && a.nbt >= 2;
+    const bool row_cs = rowcs_env && nmt_all == 2 && MT == 2;
     a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && (nmt_all == 1 || row_cs) && stride == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 || row1_env ? 1 : 2) && a.nbt <= 64;
     a.row1 = a.row && a.nbt == 1 && row1_env && row_env < 2;
     if (a.row && nmt_all == 2) MT = 1;

@@ -414,7 +414,8 @@ __device__ __forceinline__ void conv_epilogue(const conv_args &a, v16f (&acc)[MT
 #pragma unroll
             for (int q4 = 0; q4 < 4; q4++) { v[q4 * 2] = qs[0][q4]; v[q4 * 2 + 1] = qss[0][q4]; }
             const int idx = wave_half_reduce<8>(v, r);
-            if ((r >> 3) == 0) a.part[(((size_t)tile * NW + wave) * 8 + 4 * h + (idx >> 1)) * 2 + (idx & 1)] = v[0];
+            // (record (tile NW + wave) of slice cs: with channel slices the records of a (tile, wavefront) lie slice by slice, as a tile's do)
+            if ((r >> 3) == 0) a.part[((((size_t)tile * NW + wave) * a.ncs + cs) * 8 + 4 * h + (idx >> 1)) * 2 + (idx & 1)] = v[0];
         }
         return;
     }

@@ -58,9 +58,13 @@ __global__ void __launch_bounds__(512, 1) conv3_row1_k(const conv_args a) {
 
     // XCD-aware persistent walk: the tiles in column order (z fastest), an XCD owns a contiguous range of them and each of its workgroups a
     // contiguous piece of that range, so a workgroup's consecutive tiles are z neighbours of one (sample, y, x) column until the column ends
-    const unsigned per = (a.ntiles + 7u) / 8u, wg_per_xcd = gridDim.x >> 3, xcd = blockIdx.x & 7u, wix = blockIdx.x >> 3;
+    // Two channel tiles (33 .. 64 output channels): a workgroup keeps ONE of them for its whole walk, and neighbouring workgroups of an XCD
+    // walk the same tiles in the other slice (the halo's second read finds the L2)
+    const unsigned ncs = (unsigned)a.ncs, nsp = a.ntiles / ncs;                      // channel slices; spatial tiles
+    const int cs = __builtin_amdgcn_readfirstlane((int)((blockIdx.x >> 3) % ncs));
+    const unsigned per = (nsp + 7u) / 8u, wg_per_xcd = (gridDim.x >> 3) / ncs, xcd = blockIdx.x & 7u, wix = (blockIdx.x >> 3) / ncs;
     const unsigned cpw = (per + wg_per_xcd - 1u) / wg_per_xcd, k0 = xcd * per + wix * cpw;
-    const unsigned kx_ = xcd * per + per, ky_ = k0 + cpw, k1 = min(min(kx_, ky_), a.ntiles);
+    const unsigned kx_ = xcd * per + per, ky_ = k0 + cpw, k1 = min(min(kx_, ky_), nsp);
     struct tile_t { unsigned tile, col; int n, oz0, oy0, ox0; bool ok; };
     auto decode = [&](unsigned it) {
         tile_t t; const unsigned k = k0 + it;
@@ -101,7 +105,7 @@ __global__ void __launch_bounds__(512, 1) conv3_row1_k(const conv_args a) {
         for (int g = wi; g < GF; g += nw) { unsigned rg = g0 + (unsigned)g; rg -= rg >= (unsigned)NGR ? (unsigned)NGR : 0u; request(t, t.oz0 - 1 + a.zi0, g, rg, true); }
     };
     int s0 = 0;                                                 // ring slot of the current tile's first plane (even)
-    conv_epi_consts<1, EPI>(a, lds, 0, tid);
+    conv_epi_consts<1, EPI>(a, lds, cs, tid);
     load_column_start(cur, 0, NW, wave);
 
     // the block's weights: pair c 3 + ky of the prepared order (class c, ky), lane-ordered codes; the scale bytes of four pairs per register.
@@ -116,13 +120,13 @@ __global__ void __launch_bounds__(512, 1) conv3_row1_k(const conv_args a) {
         int sw[NPB];
 #pragma unroll
         for (int p = 0; p < NPB; p++) {
-            const uint8_t *wp = a.wq + (size_t)p * wq_ps + lane * 16;
+            const uint8_t *wp = a.wq + (size_t)p * wq_ps + (size_t)cs * WTILE + lane * 16;
             if (p < NPR) { wlo[p] = *(const v4i *)wp; if (FMT == 8) whi[p] = *(const v4i *)(wp + 1024); }
             else if (p < NPR + 3) {                             // class 3: wavefronts 0 .. 5 copy its six 1 KiB pieces (uniform per wavefront)
                 if (wave == 2 * (p - NPR)) dma16(wp, lds0 + w3_o + (unsigned)(p - NPR) * 2048u);
                 if (FMT == 8 && wave == 2 * (p - NPR) + 1) dma16(wp + 1024, lds0 + w3_o + (unsigned)(p - NPR) * 2048u + 1024u);
             } else if (wave == p - NPR - 3) dma16(wp, lds0 + w4_o + (unsigned)(p - NPR - 3) * 1024u);
-            sw[p] = *(const int *)(a.wsc + (size_t)p * wsc_ps + lane * 4);
+            sw[p] = *(const int *)(a.wsc + (size_t)p * wsc_ps + (size_t)cs * 256 + lane * 4);
         }
 #pragma unroll
         for (int q = 0; q < (NPB + 3) / 4; q++) {
@@ -220,8 +224,8 @@ __global__ void __launch_bounds__(512, 1) conv3_row1_k(const conv_args a) {
         __syncthreads();                                        // end of this group's K phase (barrier 2 it + 1 for group 0, 2 it + 2 for group 1)
         DBG_R1(3);
         if (cur.oz0 + TZ <= a.Do && cur.oy0 + TY <= a.Ho && cur.ox0 + TX <= a.Wo && a.zs0 <= cur.oz0 && a.zs1 >= cur.oz0 + TZ)      // (uniform)
-            conv_epilogue<1, NT, OUT, EPI, false, true, true, true, NW, true, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
-        else conv_epilogue<1, NT, OUT, EPI, false, true, false, true, NW, true, true>(a, acc, lds, cur.tile, cur.n, 0, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+            conv_epilogue<1, NT, OUT, EPI, false, true, true, true, NW, true, true>(a, acc, lds, cur.tile, cur.n, cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
+        else conv_epilogue<1, NT, OUT, EPI, false, true, false, true, NW, true, true>(a, acc, lds, cur.tile, cur.n, cs, cur.oz0, cur.oy0, cur.ox0, lz, ly0, tid);
         DBG_R1(4);
         __syncthreads();                                        // end of this group's epilogue phase (barrier 2 it + 2 / 2 it + 3)
         DBG_R1(5);
@@ -249,9 +253,9 @@ static void launch_row1(const conv_args &a, size_t smem) {
         ncu[d] = pr.multiProcessorCount > 8 ? pr.multiProcessorCount & ~7 : 8;
         attr[d] = true;
     }
-    const unsigned per = (a.ntiles + 7u) / 8u;            // tiles per XCD; one persistent workgroup per CU, a multiple of 8 in all
-    const unsigned nwg = per * 8u < (unsigned)ncu[d] ? per * 8u : (unsigned)ncu[d];
+    const unsigned ncs = (unsigned)a.ncs, per = (a.ntiles / ncs + 7u) / 8u;            // spatial tiles per XCD; one persistent workgroup per CU, a multiple of 8 x slices in all
+    const unsigned cap = (unsigned)ncu[d] / (8u * ncs) * (8u * ncs), nwg = per * 8u * ncs < cap ? per * 8u * ncs : cap;
     conv3_row1_k<FMT, OUT, EPI><<<nwg, 512, smem>>>(a);
     MICK();
-    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row1_k<fmt %d, out %d, epi %d> tiles %u wgs %u", FMT, OUT, (int)EPI, a.ntiles, nwg);
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row1_k<fmt %d, out %d, epi %d> tiles %u%s wgs %u", FMT, OUT, (int)EPI, a.ntiles, ncs > 1 ? " (two channel slices)" : "", nwg);
 }
