@@ -521,7 +521,7 @@ def test_fused_statistics_finalize(gpu, bits, Ci, Co, dims):
         assert np.array_equal(u, v)
 
 
-@pytest.mark.parametrize("case", ["general32", "wide128", "stem4", "decoder_up", "fp4_64", "gn_input"])
+@pytest.mark.parametrize("case", ["general32", "wide128", "stem4", "decoder_up", "fp4_64", "gn_input", "row_slices64", "row1_slices64", "row_slices_fp4"])
 def test_z_range_slabs_equal_whole(gpu, case):
     """split_t's z-range (zi0 / Di: output plane z reads input plane z + zi0 of a depth-Di input) with direct slab outputs (yzo / yD), the
     reference's in-place slab inference (src/nn_lp.h:36-40, src/nn_bwd.cu:33-46): the conv computed slab by slab into the full-depth output,
@@ -534,6 +534,9 @@ def test_z_range_slabs_equal_whole(gpu, case):
     elif case == "stem4": N, Ci, Co, D, H, W, slabs = 2, 4, 32, 10, 16, 16, (4, 6)
     elif case == "decoder_up": N, Ci, Co, D, H, W, slabs, up, gn, Cu = 1, 96, 32, 16, 16, 16, (4, 4, 8), 1, True, 64
     elif case == "fp4_64": N, Ci, Co, D, H, W, slabs, bits, xdt = 1, 64, 64, 12, 8, 16, (8, 4), 4, 4
+    elif case == "row_slices64": N, Ci, Co, D, H, W, slabs, gn = 2, 64, 64, 12, 16, 32, (4, 8), True          # the row kernels' two channel slices
+    elif case == "row1_slices64": N, Ci, Co, D, H, W, slabs = 2, 32, 64, 12, 16, 64, (8, 4)
+    elif case == "row_slices_fp4": N, Ci, Co, D, H, W, slabs, bits, xdt = 1, 96, 64, 12, 8, 32, (4, 4, 4), 4, 4
     else: N, Ci, Co, D, H, W, slabs, gn = 2, 64, 64, 8, 16, 16, (4, 4), True
     S = D * H * W
     G = 8
@@ -569,6 +572,7 @@ def test_z_range_slabs_equal_whole(gpu, case):
         z0 += sk
     assert z0 == D
     LP.check()
+    assert ("two channel slices" in kernel) == case.startswith("row"), kernel
     assert np.array_equal(ywhole.to_numpy(np.uint8), yslab.to_numpy(np.uint8)), kernel
     a, c = np.zeros((N, G, 2), np.float64), np.zeros((N, G, 2), np.float64)
     da, dc = DevBuf(a.nbytes), DevBuf(c.nbytes)

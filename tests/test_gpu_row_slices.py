@@ -6,7 +6,7 @@ import pytest
 
 from ufsm_amd import lib
 import orc
-from test_gpu_conv import exact_case, rand_case, gpu_conv
+from test_gpu_conv import exact_case, rand_case, gpu_conv, code_mismatch_fraction
 
 pytestmark = pytest.mark.gpu
 
@@ -42,3 +42,23 @@ def test_row_kernel_two_channel_slices(gpu, bits, N, Ci, Co, D, H, W):
     assert np.abs(gs - ws).max() / np.abs(ws).max() < 1e-5
     got2, gs2 = gpu_conv(xq, xdt, N, Ci, D, H, W, w, b, Co, 0, cbits=bits, Go=G, stats=True)
     assert np.array_equal(got, got2) and np.array_equal(gs, gs2)
+
+
+@pytest.mark.parametrize("Ci", [32, 64])
+def test_fused_activation_epilogue_on_the_sliced_kernels(gpu, Ci):
+    """mi_conv_fwd_fused on 64 output channels: each slice's workgroups take their own 32 affine pairs and biases."""
+    rng = np.random.default_rng(61 + Ci)
+    N, Co, D, H, W = 2, 64, 8, 16, 32
+    S = D * H * W
+    x, w, b = rand_case(rng, N, Ci, Co, S)
+    ea = rng.uniform(0.5, 1.5, Co).astype(np.float32); eb = rng.uniform(-.5, .5, Co).astype(np.float32)
+    xq = orc.f32_to_mx(8, x, N, Ci, S)
+    for act in (1, 2, 3):
+        want, _ = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 0, fused_act=act, ep_a=ea, ep_b=eb)
+        got, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 0, fused=(act, ea, eb))
+        assert "two channel slices" in lib.mi_last_kernel().decode(), lib.mi_last_kernel().decode()
+        assert np.abs(got - want).max() / np.abs(want).max() < 1e-4
+        wq, _ = orc.conv3(xq, 3, N, Ci, D, H, W, w, b, Co, 3, fused_act=act, ep_a=ea, ep_b=eb)
+        gq, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 3, fused=(act, ea, eb))
+        frac, near = code_mismatch_fraction(8, gq, wq, N, Co, S)
+        assert frac < 5e-3 and near
