@@ -473,7 +473,13 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     if (big_env < 0) big_env = getenv("MI_CONV_WIDE") ? atoi(getenv("MI_CONV_WIDE")) : 1;      // tuning knob: 0 keeps the 8-accumulator kernel, 2 sends every 64-channel layer to the wide kernel too
     // (64 output channels: two channel tiles per workgroup; it pays from four input blocks on: 192 -> 64 at 2 x 64^3 0.190 -> 0.178 ms, 64 -> 64 the same
     // as the general kernel. MI_CONV_WIDE=2 sends every such layer there)
-    bool big = !coarse && big_env && stride == 1 && (MT == 4 || (MT == 2 && (big_env > 1 || a.nbt >= 4 || halved))) && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
+    static int rowcs4_env = -1;
+    if (rowcs4_env < 0) rowcs4_env = getenv("MI_CONV_ROW_CS4") ? atoi(getenv("MI_CONV_ROW_CS4")) : 1;      // tuning knob: input blocks up to which 65 .. 128 output channels run the row kernels as three or four slices (0: never).
+    // Measured: 32 -> 128 at 2 x 64^3 0.079 -> 0.064 ms on the one-block kernel; from two blocks on the wide kernel is as fast (64 -> 128 and 128 -> 128 at 2 x 32^3)
+    // or faster (e2m1 at 32 x 32^3: 0.151 against 0.164 ms), hence 1
+    const bool row_cs4 = rowcs4_env > 0 && g_split < 0 && (nmt_all == 3 || nmt_all == 4) && a.nbt <= rowcs4_env && stride == 1 && !coarse && a.wide && Wo > 16 && Do >= 4 && !(osum && (cout / Go) % 4);
+    if (row_cs4) { MT = 1; NT = 4; halved = false; }
+    bool big = !row_cs4 && !coarse && big_env && stride == 1 && (MT == 4 || (MT == 2 && (big_env > 1 || a.nbt >= 4 || halved))) && Do >= 3 && a.wide && a.nbt <= 12;            // (its per-tile pair table must fit LDS)
     if (big) {
         // The wide kernel streams input block b >= 2 of a tile into LDS while the tile's earlier blocks are multiplied, one copy round per
         // stage of two pairs, NRND rounds per block, a block starting once block b - 3 has been read for the last time (pair (27 (b - 3) + 26) / 2).
@@ -525,10 +531,10 @@ static int conv_dispatch(const char *who, int fmt, int stride, const void *x, in
     // blocks on the wide kernel keeps these layers
     static int rowcs_env = -1;
     if (rowcs_env < 0) rowcs_env = getenv("MI_CONV_ROW_CS") ? atoi(getenv("MI_CONV_ROW_CS")) : 1;
-    const bool row_cs = rowcs_env && nmt_all == 2 && MT == 2;
+    const bool row_cs = (rowcs_env && nmt_all == 2 && MT == 2) || row_cs4;
     a.row = row_env && !big && !s2d && !(osum && (cout / Go) % 4) && cout > 16 && (nmt_all == 1 || row_cs) && stride == 1 && NT == 4 && a.wide && Wo > 16 && a.nbt >= (row_env > 1 || row1_env ? 1 : 2) && a.nbt <= 64;
     a.row1 = a.row && a.nbt == 1 && row1_env && row_env < 2;
-    if (a.row && nmt_all == 2) MT = 1;
+    if (a.row && nmt_all >= 2) MT = 1;
     if (a.row) { a.areg = false; a.CB = a.nbt; }
     size_t smem = a.row1 ? (size_t)10 * 352 * (RB + 4) : a.row ? (size_t)2 * 2048 * (RB + 4) : a.areg ? (size_t)2 * ((TT + 63) / 64 * 64) * (RB + 4) : big ? (size_t)4 * MT * (WTILE + 256) + (size_t)3 * ((TT + 63) / 64 * 64) * (RB + 4) + (size_t)(((27 * a.nbt + 1) >> 1) + 2) * 32 : lds_bytes(a.CB);
     if (s2d) smem = 0;

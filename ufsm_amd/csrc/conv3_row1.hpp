@@ -257,5 +257,5 @@ static void launch_row1(const conv_args &a, size_t smem) {
     const unsigned cap = (unsigned)ncu[d] / (8u * ncs) * (8u * ncs), nwg = per * 8u * ncs < cap ? per * 8u * ncs : cap;
     conv3_row1_k<FMT, OUT, EPI><<<nwg, 512, smem>>>(a);
     MICK();
-    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row1_k<fmt %d, out %d, epi %d> tiles %u%s wgs %u", FMT, OUT, (int)EPI, a.ntiles, ncs > 1 ? " (two channel slices)" : "", nwg);
+    snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row1_k<fmt %d, out %d, epi %d> tiles %u%s wgs %u", FMT, OUT, (int)EPI, a.ntiles, ncs == 2 ? " (two channel slices)" : ncs > 2 ? " (channel slices)" : "", nwg);
 }
