@@ -226,7 +226,7 @@ static void launch_row(const conv_args &a, size_t smem) {
         attr[d] = true;
     }
     const unsigned ncs = (unsigned)a.ncs, per = (a.ntiles / ncs + 7u) / 8u;            // spatial tiles per XCD; one persistent workgroup per CU, a multiple of 8 x slices in all
-    const unsigned cap = (unsigned)ncu[d] / (8u * ncs) * (8u * ncs), nwg = per * 8u * ncs < cap ? per * 8u * ncs : cap;
+    const unsigned cap0 = (unsigned)ncu[d] / (8u * ncs) * (8u * ncs), cap = cap0 ? cap0 : 8u * ncs, nwg = per * 8u * ncs < cap ? per * 8u * ncs : cap;      // (fewer CUs than 8 x slices: the walk works for any grid)
     conv3_row_k<FMT, OUT, EPI, WL><<<nwg, 512, smem>>>(a);
     MICK();
     snprintf(g_last_kernel, sizeof g_last_kernel, "conv3_row_k<fmt %d, out %d, epi %d%s> blocks %d tiles %u%s wgs %u", FMT, OUT, (int)EPI, WL ? ", weights in LDS" : "", a.nbt, a.ntiles, ncs == 2 ? " (two channel slices)" : ncs > 2 ? " (channel slices)" : "", nwg);
