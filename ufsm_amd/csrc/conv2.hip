@@ -31,6 +31,7 @@ __global__ void __launch_bounds__(128) prep_w2_k(const float *__restrict__ w, ui
 }
 
 static int conv2_dispatch(const char *who, int up, int bits, const void *x, int xbf, shape5 xs, const float *w, const float *b, int cout, void *y, int ybf, gnp_t gp) {
+    const unsigned wkey = mi_take_s2_wkey();                 // (consumed by this call, whatever becomes of it)
     if (bits != 8 && bits != 4) { fprintf(stderr, "%s: compute format %d (8 or 4)\n", who, bits); return -1; }
     if (xbf != 3 && xbf != 4) { fprintf(stderr, "%s: the input must be an MX tensor (dtype %d)\n", who, xbf); return -1; }
     if (ybf != 0 && ybf != 2 && ybf != 3 && ybf != 4) { fprintf(stderr, "%s: output dtype %d\n", who, ybf); return -1; }
@@ -57,7 +58,6 @@ static int conv2_dispatch(const char *who, int up, int bits, const void *x, int 
     const int MT = nmt_all % 4 == 0 ? 4 : nmt_all % 2 == 0 ? 2 : 1;
     // prepared weights: per call into the scratch, or once under the memo id the calling thread set for this call (mi_conv_s2_wkey)
     const size_t wq_bytes = (size_t)npairs * nmt_all * WTILE, wsc_bytes = (size_t)npairs * nmt_all * 256;
-    const unsigned wkey = mi_take_s2_wkey();
     uint8_t *wq = nullptr, *wsc = nullptr; bool have = false;
     if (wkey && !mi_ws_arena_on()) have = mi_wmemo_other(wkey, w, fmt, cout, Ci, nmt_all, up ? 2 : 1, wq_bytes, wsc_bytes, &wq, &wsc);
     else { wq = (uint8_t *)mi_ws(MI_WS_WQ, wq_bytes); wsc = (uint8_t *)mi_ws(MI_WS_WSC, wsc_bytes); }
