@@ -63,3 +63,26 @@ def test_fused_activation_epilogue_on_the_sliced_kernels(gpu, Ci):
         gq, _ = gpu_conv(xq, 3, N, Ci, D, H, W, w, b, Co, 3, fused=(act, ea, eb))
         frac, near = code_mismatch_fraction(8, gq, wq, N, Co, S)
         assert frac < 5e-3 and near
+
+
+@pytest.mark.parametrize("gn", [False, True])
+def test_decoder_conv_with_split_input_on_the_sliced_kernel(gpu, gn):
+    """A decoder conv1 with 64 output channels, [up2(silu(gn(coarse 32))) | silu(gn(skip 64))] -> 64: three input blocks in two segments, the upsampled
+    one blended by the pre-pass, each channel slice on its own workgroups (exact operands without the GroupNorm, the conv tolerance with it)."""
+    import refnp
+    from gpuutil import dev_gn
+    rng = np.random.default_rng(77)
+    Cu, Cs, Co, D, H, W = 32, 64, 64, 8, 16, 32
+    N, S, Sc, G = 2, D * H * W, (D // 2) * (H // 2) * (W // 2), 8
+    exact = not gn
+    xa = refnp.gen_exact(rng, (N, Cu, Sc)) if exact else rng.standard_normal((N, Cu, Sc)).astype(np.float32)
+    xb = refnp.gen_exact(rng, (N, Cs, S)) if exact else rng.standard_normal((N, Cs, S)).astype(np.float32)
+    w = refnp.gen_exact(rng, (Co, Cu + Cs, 27)) if exact else (rng.standard_normal((Co, Cu + Cs, 27)) * 0.05).astype(np.float32)
+    qa, qb = orc.f32_to_mx(8, xa, N, Cu, Sc), orc.f32_to_mx(8, xb, N, Cs, S)
+    p = [rng.uniform(0.5, 1.5, Cu).astype(np.float32), rng.uniform(-.5, .5, Cu).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    p2 = [rng.uniform(0.5, 1.5, Cs).astype(np.float32), rng.uniform(-.5, .5, Cs).astype(np.float32), rng.uniform(-.2, .2, N * G).astype(np.float32), rng.uniform(.8, 1.2, N * G).astype(np.float32)]
+    want, _ = orc.conv3(qa, 3, N, Cu + Cs, D, H, W, w, None, Co, 0, x2=qb, c_split=Cu, up=1, gp=orc.gn(*p, G) if gn else None, gp2=orc.gn(*p2, G) if gn else None)
+    got, _ = gpu_conv(qa, 3, N, Cu + Cs, D, H, W, w, None, Co, 0, x2=qb, c_split=Cu, up=1, gp=dev_gn(*p, G) if gn else None, gp2=dev_gn(*p2, G) if gn else None)
+    assert "conv3_row_k" in lib.mi_last_kernel().decode() and "two channel slices" in lib.mi_last_kernel().decode(), lib.mi_last_kernel().decode()
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err < (1e-5 if exact else 3e-3)
